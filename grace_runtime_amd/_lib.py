@@ -1,0 +1,106 @@
+"""ctypes binding of libgrace_hip.so (the C ABI declared in include/grace_hip.h).
+
+The library is loaded from this package directory (built in-tree by grace_runtime_amd/csrc/Makefile).  There is no
+fallback: without the library, or without a GPU, every compute entry point raises."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libgrace_hip.so")
+
+GR_OK, GR_INVALID, GR_ERROR, GR_NOMEM = 0, 1, 2, 3
+FLAG_ENERGY_ONLY, FLAG_EATOM = 1, 2
+
+# every symbol include/grace_hip.h declares (checked by the CPU test-suite against the header and the library)
+SYMBOLS = [
+    "gr_last_error", "gr_abi_version", "gr_device_count", "gr_device_arch", "gr_model_load", "gr_model_get_info",
+    "gr_model_element_name", "gr_model_free", "gr_engine_create", "gr_engine_free", "gr_engine_cutoff",
+    "gr_compute_csr", "gr_engine_upload", "gr_engine_run", "gr_engine_sync", "gr_engine_fetch",
+    "gr_engine_edge_count", "gr_engine_set_profile", "gr_engine_stage_count", "gr_engine_stage_get",
+    "gr_engine_debug_radial", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
+    "gr_nlist_free", "gr_compute",
+]
+
+
+class ModelInfo(C.Structure):
+    _fields_ = [("layers", C.c_int), ("n_elements", C.c_int), ("lmax", C.c_int), ("n_radial", C.c_int),
+                ("n_radbase", C.c_int), ("max_order", C.c_int), ("rcut", C.c_double)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises RuntimeError when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(f"{LIB_PATH} is missing: build it with `make -C grace_runtime_amd/csrc` "
+                           "(there is no CPU fallback in this package)")
+    L = C.CDLL(LIB_PATH)
+    vp, i32, i64, dbl, u32 = C.c_void_p, C.c_int, C.c_int64, C.c_double, C.c_uint
+    L.gr_last_error.restype = C.c_char_p
+    L.gr_abi_version.restype = i32
+    L.gr_device_count.restype = i32
+    L.gr_device_arch.argtypes = [i32, C.c_char_p, i32]
+    L.gr_model_load.argtypes = [C.c_char_p, C.POINTER(vp)]
+    L.gr_model_get_info.argtypes = [vp, C.POINTER(ModelInfo)]
+    L.gr_model_element_name.restype = C.c_char_p
+    L.gr_model_element_name.argtypes = [vp, i32]
+    L.gr_model_free.argtypes = [vp]
+    L.gr_engine_create.argtypes = [vp, i32, vp, i32, i32, C.POINTER(vp)]
+    L.gr_engine_free.argtypes = [vp]
+    L.gr_engine_cutoff.restype = dbl
+    L.gr_engine_cutoff.argtypes = [vp, i32, i32]
+    L.gr_compute_csr.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, u32, vp, vp, vp, vp]
+    L.gr_engine_upload.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp, vp, i64]
+    L.gr_engine_run.argtypes = [vp, u32]
+    L.gr_engine_sync.argtypes = [vp]
+    L.gr_engine_fetch.argtypes = [vp, vp, vp, vp, vp]
+    L.gr_engine_edge_count.restype = i64
+    L.gr_engine_edge_count.argtypes = [vp]
+    L.gr_engine_set_profile.argtypes = [vp, i32]
+    L.gr_engine_stage_count.argtypes = [vp]
+    L.gr_engine_stage_get.argtypes = [vp, i32, C.c_char_p, i32, C.POINTER(dbl), C.POINTER(i32)]
+    L.gr_engine_debug_radial.argtypes = [vp, i32, vp, vp, vp, vp]
+    L.gr_neighbor_build.argtypes = [i64, vp, vp, vp, dbl, i32, C.POINTER(vp)]
+    L.gr_nlist_nbonds.restype = i64
+    L.gr_nlist_nbonds.argtypes = [vp]
+    L.gr_nlist_nimages.restype = i64
+    L.gr_nlist_nimages.argtypes = [vp]
+    L.gr_nlist_get.argtypes = [vp, vp, vp, vp, vp, vp]
+    L.gr_nlist_free.argtypes = [vp]
+    L.gr_compute.argtypes = [vp, i32, vp, vp, vp, vp, u32, vp, vp, vp, vp]
+    _lib = L
+    return L
+
+
+def check(status):
+    """Status code -> exception, as the reference binding maps them (python/kk/kk_module.cpp: invalid_argument ->
+    ValueError, everything else RuntimeError; allocation failure -> MemoryError)."""
+    if status == GR_OK:
+        return
+    msg = lib().gr_last_error().decode(errors="replace")
+    if status == GR_INVALID:
+        raise ValueError(msg)
+    if status == GR_NOMEM:
+        raise MemoryError(msg)
+    raise RuntimeError(msg)
+
+
+def ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def as_array(a, dtype, shape_last=None):
+    if a is None:
+        return None
+    a = np.ascontiguousarray(a, dtype=dtype)
+    if shape_last is not None and (a.ndim != 2 or a.shape[1] != shape_last):
+        raise ValueError(f"expected an array of shape (n, {shape_last})")
+    return a

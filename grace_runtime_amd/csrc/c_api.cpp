@@ -1,0 +1,334 @@
+// extern "C" layer of libgrace_hip.so (declarations and the reference interfaces they replace: include/grace_hip.h).
+// Exceptions never cross the ABI: they become a status code and a thread-local message.
+#include "../../include/grace_hip.h"
+
+#include "engine.hpp"
+#include "neighbors.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+#include <memory>
+#include <new>
+#include <string>
+
+struct gr_model {
+  grhip::ModelKind kind;
+  std::shared_ptr<grhip::Model1L> m1;
+  std::string path;
+};
+struct gr_engine {
+  std::unique_ptr<grhip::Engine> eng;
+  std::vector<grhip::StageTime> times;
+};
+struct gr_nlist {
+  grhip::NeighborList nl;
+};
+
+namespace {
+thread_local std::string g_err;
+
+template<class F> int guarded(F &&f)
+{
+  try {
+    f();
+    g_err.clear();
+    return GR_OK;
+  } catch (const grhip::InvalidArgument &e) {
+    g_err = e.what();
+    return GR_INVALID;
+  } catch (const std::invalid_argument &e) {
+    g_err = e.what();
+    return GR_INVALID;
+  } catch (const std::bad_alloc &) {
+    g_err = "out of memory";
+    return GR_NOMEM;
+  } catch (const std::exception &e) {
+    g_err = e.what();
+    return GR_ERROR;
+  } catch (...) {
+    g_err = "unknown error";
+    return GR_ERROR;
+  }
+}
+
+grhip::CsrInput make_input(int n, const int *types, const int64_t *offset, const int *j, const double *rij,
+                           const double *positions, const int *image, const double *shifts, int64_t nimages)
+{
+  if (n > 0 && (!types || !offset)) throw grhip::InvalidArgument("types and offset are required");
+  grhip::CsrInput in;
+  in.n = n;
+  in.types = types;
+  in.offset = offset;
+  in.j = j;
+  in.rij = rij;
+  in.x = positions;
+  in.image = image;
+  in.shifts = shifts;
+  in.nimages = nimages;
+  return in;
+}
+}    // namespace
+
+extern "C" {
+
+const char *gr_last_error(void) { return g_err.c_str(); }
+int gr_abi_version(void) { return 7; }
+
+int gr_device_count(void)
+{
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void) hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+int gr_device_arch(int device, char *buf, int len)
+{
+  if (buf && len > 0) buf[0] = 0;
+  return guarded([&] {
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, device) != hipSuccess) {
+      (void) hipGetLastError();
+      throw grhip::Error("no such HIP device");
+    }
+    if (buf && len > 0) {
+      std::strncpy(buf, p.gcnArchName, (size_t) len - 1);
+      buf[len - 1] = 0;
+    }
+  });
+}
+
+int gr_model_load(const char *npz_path, gr_model **out)
+{
+  return guarded([&] {
+    if (!npz_path || !out) throw grhip::InvalidArgument("null argument");
+    *out = nullptr;
+    const grhip::Npz z = grhip::npz_load(npz_path);
+    auto m = std::make_unique<gr_model>();
+    m->path = npz_path;
+    m->kind = grhip::model_kind(z, npz_path);
+    if (m->kind == grhip::ModelKind::Grace1L) {
+      m->m1 = std::make_shared<grhip::Model1L>();
+      m->m1->load(z);
+    } else {
+      throw grhip::InvalidArgument(std::string("unsupported model: this build of the GPU engine implements GRACE-1L; the file holds a GRACE-") +
+                                   (m->kind == grhip::ModelKind::Grace2L ? "2L" : "3L") + " model");
+    }
+    *out = m.release();
+  });
+}
+
+int gr_model_get_info(const gr_model *m, gr_model_info *info)
+{
+  return guarded([&] {
+    if (!m || !info) throw grhip::InvalidArgument("null argument");
+    std::memset(info, 0, sizeof(*info));
+    info->layers = (int) m->kind;
+    if (m->m1) {
+      info->n_elements = m->m1->n_elements;
+      info->lmax = m->m1->lmax;
+      info->n_radial = m->m1->nradmax;
+      info->n_radbase = m->m1->nradbase;
+      info->max_order = m->m1->max_order;
+      double rc = 0.0;
+      for (double c : m->m1->bond_cutoff_map) rc = std::max(rc, c);
+      info->rcut = m->m1->has_bond_specific_cutoff ? rc : m->m1->rcut;
+    }
+  });
+}
+
+const char *gr_model_element_name(const gr_model *m, int k)
+{
+  if (!m || !m->m1 || k < 0 || k >= (int) m->m1->element_names.size()) return "";
+  return m->m1->element_names[k].c_str();
+}
+
+void gr_model_free(gr_model *m) { delete m; }
+
+int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int precision, int device, gr_engine **out)
+{
+  return guarded([&] {
+    if (!m || !type2mu || !out) throw grhip::InvalidArgument("null argument");
+    *out = nullptr;
+    if (ntypes < 1) throw grhip::InvalidArgument("ntypes must be positive");
+    std::vector<int> t(type2mu, type2mu + ntypes + 1);
+    auto e = std::make_unique<gr_engine>();
+    e->eng = grhip::make_engine_1l(m->m1, ntypes, t, precision, device);
+    *out = e.release();
+  });
+}
+
+void gr_engine_free(gr_engine *e) { delete e; }
+
+double gr_engine_cutoff(const gr_engine *e, int t1, int t2) { return e ? e->eng->cutoff(t1, t2) : 0.0; }
+
+int gr_engine_upload(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
+                     const double *positions, const int *image, const double *shifts, int64_t nimages)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->upload(make_input(n, types, offset, j, rij, positions, image, shifts, nimages));
+  });
+}
+
+int gr_engine_run(gr_engine *e, unsigned flags)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0;
+    e->eng->run(fl);
+  });
+}
+
+int gr_engine_sync(gr_engine *e)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->synchronize();
+  });
+}
+
+int gr_engine_fetch(gr_engine *e, double *energy, double *forces, double *virial, double *eatom)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->fetch(energy, forces, virial, eatom);
+  });
+}
+
+int64_t gr_engine_edge_count(gr_engine *e)
+{
+  int64_t r = -1;
+  guarded([&] { r = e->eng->last_edge_count(); });
+  return r;
+}
+
+int gr_compute_csr(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
+                   const double *positions, const int *image, const double *shifts, int64_t nimages, unsigned flags,
+                   double *energy, double *forces, double *virial, double *eatom)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->upload(make_input(n, types, offset, j, rij, positions, image, shifts, nimages));
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    e->eng->run(fl);
+    e->eng->fetch(energy, forces, virial, eatom);
+  });
+}
+
+int gr_engine_set_profile(gr_engine *e, int on)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->set_profile(on != 0);
+  });
+}
+
+int gr_engine_stage_count(gr_engine *e)
+{
+  int n = -1;
+  guarded([&] {
+    e->times = e->eng->stage_times();
+    n = (int) e->times.size();
+  });
+  return n;
+}
+
+int gr_engine_stage_get(gr_engine *e, int k, char *name, int name_len, double *ms, int *launches)
+{
+  return guarded([&] {
+    if (!e || k < 0 || k >= (int) e->times.size()) throw grhip::InvalidArgument("no such stage");
+    if (name && name_len > 0) {
+      std::strncpy(name, e->times[k].name.c_str(), (size_t) name_len - 1);
+      name[name_len - 1] = 0;
+    }
+    if (ms) *ms = e->times[k].ms;
+    if (launches) *launches = e->times[k].launches;
+  });
+}
+
+int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->debug_radial(m, x, mu_j, Rz, dRz);
+  });
+}
+
+int gr_neighbor_build(int64_t n, const double *positions, const double *cell, const unsigned char *pbc, double cutoff,
+                      int nthreads, gr_nlist **out)
+{
+  return guarded([&] {
+    if (!out || !cell || !pbc || (n > 0 && !positions)) throw grhip::InvalidArgument("null argument");
+    *out = nullptr;
+    const bool p[3] = {pbc[0] != 0, pbc[1] != 0, pbc[2] != 0};
+    auto l = std::make_unique<gr_nlist>();
+    l->nl = grhip::neighbor_search(positions, n, cell, p, cutoff, nthreads);
+    *out = l.release();
+  });
+}
+
+int64_t gr_nlist_nbonds(const gr_nlist *l) { return l ? (int64_t) l->nl.j.size() : 0; }
+int64_t gr_nlist_nimages(const gr_nlist *l) { return l ? (int64_t) l->nl.shifts.size() / 3 : 0; }
+
+int gr_nlist_get(const gr_nlist *l, int64_t *perm, int64_t *offset, int32_t *j, int32_t *image, double *shifts)
+{
+  return guarded([&] {
+    if (!l) throw grhip::InvalidArgument("null list");
+    const auto &r = l->nl;
+    if (perm) std::memcpy(perm, r.perm.data(), r.perm.size() * sizeof(int64_t));
+    if (offset) std::memcpy(offset, r.offset.data(), r.offset.size() * sizeof(int64_t));
+    if (j) std::memcpy(j, r.j.data(), r.j.size() * sizeof(int32_t));
+    if (image) std::memcpy(image, r.image.data(), r.image.size() * sizeof(int32_t));
+    if (shifts) std::memcpy(shifts, r.shifts.data(), r.shifts.size() * sizeof(double));
+  });
+}
+
+void gr_nlist_free(gr_nlist *l) { delete l; }
+
+int gr_compute(gr_engine *e, int n, const int *types, const double *positions, const double *cell,
+               const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom)
+{
+  return guarded([&] {
+    if (!e || !cell || !pbc || (n > 0 && (!types || !positions))) throw grhip::InvalidArgument("null argument");
+    const bool p[3] = {pbc[0] != 0, pbc[1] != 0, pbc[2] != 0};
+    double rc = 0.0;
+    {
+      // largest cutoff over the types present
+      rc = e->eng->max_cutoff();
+      if (!(rc > 0.0)) throw grhip::Error("the engine has no positive cutoff");
+    }
+    grhip::NeighborList nl = grhip::neighbor_search(positions, n, cell, p, rc, 8);
+    std::vector<int> ty(n);
+    std::vector<double> x((size_t) 3 * n);
+    for (int q = 0; q < n; q++) {
+      const int64_t a = nl.perm[q];
+      ty[q] = types[a];
+      for (int d = 0; d < 3; d++) x[3 * (size_t) q + d] = positions[3 * a + d];
+    }
+    std::vector<double> dummy(3, 0.0);
+    const int64_t nimg = (int64_t) nl.shifts.size() / 3;
+    e->eng->upload(make_input(n, ty.data(), nl.offset.data(), nl.j.data(), nullptr, x.data(), nl.image.data(),
+                              nimg ? nl.shifts.data() : dummy.data(), nimg));
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    e->eng->run(fl);
+    std::vector<double> f((size_t) 3 * n), ea(fl.eatom ? n : 0);
+    e->eng->fetch(energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
+    for (int q = 0; q < n; q++) {
+      const int64_t a = nl.perm[q];
+      if (forces && !fl.energy_only)
+        for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) q + d];
+      if (fl.eatom) eatom[a] = ea[q];
+    }
+  });
+}
+}

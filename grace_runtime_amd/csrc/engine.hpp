@@ -1,0 +1,63 @@
+// Engine interface behind the C ABI: one engine = one model on one GPU for one type -> element map.
+// The call pattern mirrors the reference GPU engines (libgrace/include/grace/kk/grace_1l_kk.h:72-113: set_model /
+// setup / run) and the CSR entry of the Python module (python/src/core.cpp:292-396).
+#pragma once
+
+#include "model.hpp"
+
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <vector>
+
+namespace grhip {
+
+struct CsrInput {
+  int n = 0;
+  const int *types = nullptr;         // [n] 1-based atom types
+  const int64_t *offset = nullptr;    // [n + 1]
+  const int *j = nullptr;             // [nb]
+  const double *rij = nullptr;        // [nb][3], or null with (x, image, shifts)
+  const double *x = nullptr;          // [n][3]
+  const int *image = nullptr;         // [nb]
+  const double *shifts = nullptr;     // [nimages][3]
+  int64_t nimages = 0;
+};
+
+struct StageTime {
+  std::string name;
+  double ms = 0.0;       // summed over the launches of the stage in the last run
+  int launches = 0;
+};
+
+struct RunFlags {
+  bool energy_only = false;
+  bool eatom = false;
+};
+
+class Engine {
+ public:
+  virtual ~Engine() = default;
+  virtual int layers() const = 0;
+  virtual double cutoff(int t1, int t2) const = 0;    // atom types, 1-based
+  virtual double max_cutoff() const = 0;
+  // copy a structure to the GPU (validates types, offsets and neighbour indices)
+  virtual void upload(const CsrInput &in) = 0;
+  // one energy / forces / virial pass over the uploaded structure; results stay on the GPU
+  virtual void run(const RunFlags &fl) = 0;
+  // wait for the pass and copy results out (null pointers are skipped); forces [n][3], virial [6], eatom [n]
+  virtual void fetch(double *energy, double *forces, double *virial, double *eatom) = 0;
+  virtual void synchronize() = 0;
+  virtual void set_profile(bool on) = 0;
+  virtual const std::vector<StageTime> &stage_times() = 0;
+  virtual int64_t last_edge_count() = 0;
+  // radial functions of the device kernel for the given x = r / rc and neighbour elements: R z and dR/dx z,
+  // [m][nl][C] (tests of the MFMA kernel against the CPU restatement)
+  virtual void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) = 0;
+};
+
+// precision: 64 (network arithmetic in fp64) or 32 (fp32 network, fp64 geometry and sums)
+std::unique_ptr<Engine> make_engine_1l(std::shared_ptr<const Model1L> model, int ntypes, const std::vector<int> &type2mu,
+                                       int precision, int device);
+
+}    // namespace grhip

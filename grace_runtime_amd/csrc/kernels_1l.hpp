@@ -1,0 +1,820 @@
+// HIP kernels of the GRACE-1L energy/forces/virial pass for gfx950 (wave64, MFMA).  Included by engine_1l.hip only.
+//
+// Stage map (reference stages in libgrace/src/fused_1l.cpp:260-372 and the staged pipeline of
+// libgrace/include/grace/kk/grace_1l_kk.h:449-454):
+//   k_edge_count / k_edge_fill   bond filter r^2 < rc^2, unit vectors, x = r / rc        (bonds.h:120-162)
+//   k_radial                     Chebyshev x envelope basis + radial MLP value/tangent on MFMA, times z[mu_j]
+//                                (radial_x.h:11-60; spline tables of the CPU path replaced by the exact MLP)
+//   k_scatter_a                  A[lm][n] = sum_b Y_lm R_nl z                            (fused_cpu.h:947-982)
+//   k_fc_fwd / k_fc_bwd_*        FC                                                       (fused_cpu.h:349-364)
+//   k_prod_fwd / k_prod_bwd      channel-wise CG products                                 (fused_cpu.h:409-475)
+//   k_reduce_fwd / k_reduce_bwd  rho reduce with per-element weights                      (fused_cpu.h:637-649)
+//   k_energy                     fp64 readout MLP and its reverse                         (fused_1l.cpp:378-427)
+//   k_bond_bwd                   per-bond force, pair scatter, virial                     (fused_cpu.h:836-860,1027-1050)
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace grhip {
+
+constexpr int kKernMaxL = 6;                                // largest lmax of the kernels
+constexpr int kMaxNlm = (kKernMaxL + 1) * (kKernMaxL + 1);
+constexpr int kMaxPlm = (kKernMaxL + 1) * (kKernMaxL + 2) / 2;
+constexpr int kBondChunk = 32;                          // bonds staged per pass of the per-atom kernels
+constexpr int kMaxRadBasis = 16;                        // radial basis functions (padded to a multiple of 4)
+
+// spherical-harmonics recursion coefficients (fused_cpu.h:686-704), by index l (l + 1) / 2 + m
+struct ShCoef {
+  double a[kMaxPlm], b[kMaxPlm], c[kKernMaxL + 1], d[kKernMaxL + 1];
+  int lmax;
+};
+
+// Real spherical harmonics Y[lm] (stride ys) of the unit vector (rx, ry, rz) and, with GRAD, the gradient
+// G[lm][3] of their polynomial extension.  Same recursion as fused_cpu.h:712-798, one bond per thread, fp64.
+template<bool GRAD, class TY>
+__device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz, TY *Y, TY *G)
+{
+  double plm[kMaxPlm], dplm[kMaxPlm];
+  const int lmax = co.lmax;
+  plm[0] = 1.0;
+  dplm[0] = 0.0;
+  if (lmax > 0) {
+    const double s3 = 1.7320508075688772, s15 = -1.224744871391589;
+    plm[1] = s3 * rz; dplm[1] = s3;
+    plm[2] = s15;     dplm[2] = 0.0;
+#pragma unroll
+    for (int l = 2; l <= kKernMaxL; l++) {
+      if (l <= lmax) {
+#pragma unroll
+        for (int mm = 0; mm < l - 1; mm++) {
+          const int id = l * (l + 1) / 2 + mm, i1 = (l - 1) * l / 2 + mm, i2 = (l - 2) * (l - 1) / 2 + mm;
+          const double ca = co.a[id], cb = co.b[id];
+          plm[id] = ca * (rz * plm[i1] + cb * plm[i2]);
+          if (GRAD) dplm[id] = ca * (plm[i1] + rz * dplm[i1] + cb * dplm[i2]);
+        }
+        const int prev = (l - 1) * l / 2 + l - 1, i0 = l * (l + 1) / 2 + l - 1, i1 = l * (l + 1) / 2 + l;
+        const double sd = co.d[l], sc = co.c[l];
+        plm[i0] = sd * plm[prev] * rz;
+        plm[i1] = sc * plm[prev];
+        if (GRAD) {
+          dplm[i0] = sd * (dplm[prev] * rz + plm[prev]);
+          dplm[i1] = sc * dplm[prev];
+        }
+      }
+    }
+  }
+  const double sq2 = 1.4142135623730951;
+#pragma unroll
+  for (int l = 0; l <= kKernMaxL; l++) {
+    if (l <= lmax) {
+      const int c = l * (l + 1), p0 = l * (l + 1) / 2;
+      Y[c] = (TY) plm[p0];
+      if (GRAD) { G[3 * c] = (TY) 0; G[3 * c + 1] = (TY) 0; G[3 * c + 2] = (TY) dplm[p0]; }
+      double pr = rx, pi = ry, prx = 1.0, pry = 0.0, pix = 0.0, piy = 1.0;
+#pragma unroll
+      for (int mm = 1; mm <= l; mm++) {
+        const double sg = (mm % 2 == 0) ? sq2 : -sq2;
+        const double pv = plm[p0 + mm];
+        Y[c + mm] = (TY) (sg * pr * pv);
+        Y[c - mm] = (TY) (sg * pi * pv);
+        if (GRAD) {
+          const double dpv = dplm[p0 + mm];
+          G[3 * (c + mm)] = (TY) (sg * prx * pv);
+          G[3 * (c + mm) + 1] = (TY) (sg * pry * pv);
+          G[3 * (c + mm) + 2] = (TY) (sg * pr * dpv);
+          G[3 * (c - mm)] = (TY) (sg * pix * pv);
+          G[3 * (c - mm) + 1] = (TY) (sg * piy * pv);
+          G[3 * (c - mm) + 2] = (TY) (sg * pi * dpv);
+          const double nrx = prx * rx + pr - pix * ry, nry = pry * rx - piy * ry - pi;
+          const double nix = prx * ry + pix * rx + pi, niy = pry * ry + pr + piy * rx;
+          prx = nrx; pry = nry; pix = nix; piy = niy;
+        }
+        const double nr = pr * rx - pi * ry, ni = pr * ry + pi * rx;
+        pr = nr; pi = ni;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// bond filter
+// ---------------------------------------------------------------------------------------------------------------
+struct BondSrc {
+  const int *mu;              // [n] model element of each atom
+  const long long *offset;    // [n + 1]
+  const int *j;               // [nb]
+  const double *rij;          // [nb][3] or null
+  const double *x;            // [n][3]      (with rij null)
+  const int *image;           // [nb]
+  const double *shifts;       // [nimg][3]
+  const double *cut;          // [nel][nel] pair cutoffs
+  int nel;
+};
+
+__device__ inline void bond_vec(const BondSrc &s, int i, long long q, double &dx, double &dy, double &dz)
+{
+  if (s.rij) {
+    dx = s.rij[3 * q]; dy = s.rij[3 * q + 1]; dz = s.rij[3 * q + 2];
+  } else {    // x_j - x_i + shift, in this order (system.h:36-42)
+    const int jj = s.j[q];
+    const double *xi = s.x + 3 * (long long) i, *xj = s.x + 3 * (long long) jj, *sh = s.shifts + 3 * (long long) s.image[q];
+    dx = xj[0] - xi[0] + sh[0];
+    dy = xj[1] - xi[1] + sh[1];
+    dz = xj[2] - xi[2] + sh[2];
+  }
+}
+
+// one wave per atom: number of bonds with r^2 < rc^2; a bond of length 0 is recorded in zero_bond (i, j) and skipped
+__global__ void k_edge_count(BondSrc s, int n, int *count, int *zero_bond)
+{
+  const int lane = threadIdx.x & 63;
+  const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (i >= n) return;
+  const int mi = s.mu[i];
+  int c = 0;
+  for (long long q = s.offset[i] + lane; q < s.offset[i + 1]; q += 64) {
+    double dx, dy, dz;
+    bond_vec(s, i, q, dx, dy, dz);
+    const double rsq = dx * dx + dy * dy + dz * dz;
+    const int jj = s.j[q];
+    const double rc = s.cut[mi * s.nel + s.mu[jj]];
+    if (!(rsq < rc * rc)) continue;
+    if (rsq == 0.0) {
+      if (atomicCAS(zero_bond, -1, i) == -1) zero_bond[1] = jj;
+      continue;
+    }
+    c++;
+  }
+  for (int o = 32; o > 0; o >>= 1) c += __shfl_down(c, o, 64);
+  if (lane == 0) count[i] = c;
+}
+
+// exclusive scan of count[n] into eoff[n + 1] (single block; n up to a few million is a few passes of 1024)
+__global__ void k_scan(const int *count, int n, long long *eoff)
+{
+  __shared__ long long part[1024];
+  __shared__ long long carry;
+  if (threadIdx.x == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < n; base += 1024) {
+    const int i = base + threadIdx.x;
+    long long v = i < n ? count[i] : 0;
+    part[threadIdx.x] = v;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {
+      long long t = threadIdx.x >= o ? part[threadIdx.x - o] : 0;
+      __syncthreads();
+      part[threadIdx.x] += t;
+      __syncthreads();
+    }
+    if (i < n) eoff[i] = carry + part[threadIdx.x] - v;
+    __syncthreads();
+    if (threadIdx.x == 1023) carry += part[1023];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) eoff[n] = carry;
+}
+
+struct Edges {
+  int *ei, *ej, *emu;         // central atom, neighbour, neighbour element
+  double *rh;                 // [E][3] unit vectors
+  double *r, *x, *rc;         // length, r / rc, rc
+};
+
+// one wave per atom: in-cutoff bonds in list order -> compact edge arrays at eoff[i]
+__global__ void k_edge_fill(BondSrc s, int n, const long long *eoff, Edges e)
+{
+  const int lane = threadIdx.x & 63;
+  const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (i >= n) return;
+  const int mi = s.mu[i];
+  long long w = eoff[i];
+  const long long q0 = s.offset[i], q1 = s.offset[i + 1];
+  for (long long base = q0; base < q1; base += 64) {
+    const long long q = base + lane;
+    bool keep = false;
+    double dx = 0, dy = 0, dz = 0, rsq = 0, rc = 0;
+    int jj = 0;
+    if (q < q1) {
+      bond_vec(s, i, q, dx, dy, dz);
+      rsq = dx * dx + dy * dy + dz * dz;
+      jj = s.j[q];
+      rc = s.cut[mi * s.nel + s.mu[jj]];
+      keep = (rsq < rc * rc) && rsq != 0.0;
+    }
+    const unsigned long long m = __ballot(keep);
+    if (keep) {
+      const long long p = w + __popcll(m & ((1ull << lane) - 1ull));
+      const double r = sqrt(rsq), ir = 1.0 / r;
+      e.ei[p] = i;
+      e.ej[p] = jj;
+      e.emu[p] = s.mu[jj];
+      e.rh[3 * p] = dx * ir; e.rh[3 * p + 1] = dy * ir; e.rh[3 * p + 2] = dz * ir;
+      e.r[p] = r;
+      e.rc[p] = rc;
+      e.x[p] = r / rc;
+    }
+    w += __popcll(m);
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// radial MLP on the matrix cores
+// ---------------------------------------------------------------------------------------------------------------
+template<class T> struct Mfma;
+template<> struct Mfma<double> {
+  typedef double v4 __attribute__((ext_vector_type(4)));
+  __device__ static inline v4 mma(double a, double b, v4 c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+};
+template<> struct Mfma<float> {
+  typedef float v4 __attribute__((ext_vector_type(4)));
+  __device__ static inline v4 mma(float a, float b, v4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+};
+
+// D = A B for one wave with A[i][k], B[k][j] held as (i or j = lane % 16, k = lane / 16): every lane writes its four
+// accumulator values; the host derives which (row, column) each (lane, register) holds
+template<class T> __global__ void k_mfma_probe(const T *A, const T *B, T *D)
+{
+  const int lane = threadIdx.x;
+  typename Mfma<T>::v4 acc = {0, 0, 0, 0};
+  acc = Mfma<T>::mma(A[(lane & 15) * 4 + (lane >> 4)], B[(lane >> 4) * 16 + (lane & 15)], acc);
+  for (int v = 0; v < 4; v++) D[lane * 4 + v] = acc[v];
+}
+
+template<class T> struct RadialArgs {
+  const long long *n_edges;   // device scalar: edges of this pass are [e_begin, e_begin + count)
+  long long e_begin, e_count; // e_count < 0: take *n_edges - e_begin
+  const double *x;            // [E] r / rc
+  const int *emu;             // [E] neighbour element
+  const T *w0, *w1, *w2;      // fragment-ordered weights (norms folded in)
+  const T *z;                 // [nel][C]
+  T *Rz, *dRz;                // [E][noutp]  columns l * C + n
+  int nrb, p, ks0;            // basis functions, envelope order, k-steps of layer 0
+  int nob, noutp;             // 16-column blocks and padded width of the output
+  int C, nel, act;            // radial channels, elements, activation (0 SiLU, 1 tanh)
+  int w2_in_lds;
+  int drow[16];               // accumulator row of (lane / 16, register)
+};
+
+template<class T> __device__ inline void act_pair(int act, T &s, T &ds)
+{
+  if (act == 1) {
+    const T t = tanh(s);
+    ds = ds * ((T) 1 - t * t);
+    s = t;
+  } else {
+    const T sg = (T) 1 / ((T) 1 + exp(-s));
+    ds = sg * ((T) 1 + s * ((T) 1 - sg)) * ds;
+    s = s * sg;
+  }
+}
+
+// One wave = 16 edges.  Layers 0 and 1 run as D[feature][edge] = W^T H with the weights as the A operand, so the
+// accumulator registers of one layer are exactly the B operand of the next (no data movement between layers: the
+// k index of a step is the accumulator row held by that lane, and the weight fragments are stored in that order).
+// Layer 2 swaps the operands, D[edge][column], so that 16 lanes write 16 consecutive columns of one edge row.
+template<class T, int HB> __global__ __launch_bounds__(512) void k_radial(RadialArgs<T> a)
+{
+  typedef typename Mfma<T>::v4 v4;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T *w0s = reinterpret_cast<T *>(smem_raw);
+  T *w1s = w0s + HB * a.ks0 * 64;
+  T *w2s = w1s + HB * HB * 4 * 64;
+  {
+    const int n0 = HB * a.ks0 * 64, n1 = HB * HB * 4 * 64, n2 = a.w2_in_lds ? a.nob * HB * 4 * 64 : 0;
+    for (int q = threadIdx.x; q < n0; q += blockDim.x) w0s[q] = a.w0[q];
+    for (int q = threadIdx.x; q < n1; q += blockDim.x) w1s[q] = a.w1[q];
+    for (int q = threadIdx.x; q < n2; q += blockDim.x) w2s[q] = a.w2[q];
+  }
+  __syncthreads();
+  const T *w2p = a.w2_in_lds ? w2s : a.w2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const long long cnt = a.e_count >= 0 ? a.e_count : *a.n_edges - a.e_begin;
+  const long long ntiles = (cnt + 15) / 16;
+  const int p = a.p;
+  for (long long tile = (long long) blockIdx.x * nw + wave; tile < ntiles; tile += (long long) gridDim.x * nw) {
+    const long long eloc = tile * 16 + c;
+    const long long e = a.e_begin + eloc;
+    const double x = eloc < cnt ? a.x[e] : 0.5;
+    // basis g_k = T_k(2x - 1) fcut_p(x), k = 1..nrb, and d/dx (radial_x.h:11-26); this lane supplies k = 4 s + g
+    T h0[kMaxRadBasis / 4], dh0[kMaxRadBasis / 4];
+    {
+      const double xp = pow(x, (double) p), xp1 = xp * x, xp2 = xp1 * x;
+      const double fc = 1.0 - 0.5 * (p + 1) * (p + 2) * xp + (double) p * (p + 2) * xp1 - 0.5 * p * (p + 1) * xp2;
+      const double dfc = 0.5 * p * (p + 1) * (p + 2) * (-pow(x, (double) (p - 1)) + 2.0 * xp - xp1);
+      const double t = 2.0 * x - 1.0;
+      double Tp = 1.0, Tc = t, dTp = 0.0, dTc = 2.0;
+#pragma unroll
+      for (int s = 0; s < kMaxRadBasis / 4; s++) { h0[s] = (T) 0; dh0[s] = (T) 0; }
+      for (int k = 0; k < a.nrb; k++) {
+        const double gk = Tc * fc, dgk = dTc * fc + Tc * dfc;
+        if ((k & 3) == g) {
+#pragma unroll
+          for (int s = 0; s < kMaxRadBasis / 4; s++)
+            if (s == (k >> 2)) { h0[s] = (T) gk; dh0[s] = (T) dgk; }
+        }
+        const double Tn = 2.0 * t * Tc - Tp, dTn = 2.0 * (2.0 * Tc + t * dTc) - dTp;
+        Tp = Tc; dTp = dTc; Tc = Tn; dTc = dTn;
+      }
+    }
+    // ---- layer 0
+    v4 h1[HB], dh1[HB];
+#pragma unroll
+    for (int rb = 0; rb < HB; rb++) {
+      v4 acc = {0, 0, 0, 0}, dacc = {0, 0, 0, 0};
+#pragma unroll
+      for (int s = 0; s < kMaxRadBasis / 4; s++)
+        if (s < a.ks0) {
+          const T w = w0s[(rb * a.ks0 + s) * 64 + lane];
+          acc = Mfma<T>::mma(w, h0[s], acc);
+          dacc = Mfma<T>::mma(w, dh0[s], dacc);
+        }
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        T s_ = acc[v], d_ = dacc[v];
+        act_pair<T>(a.act, s_, d_);
+        acc[v] = s_; dacc[v] = d_;
+      }
+      h1[rb] = acc; dh1[rb] = dacc;
+    }
+    // ---- layer 1
+    v4 h2[HB], dh2[HB];
+#pragma unroll
+    for (int rb = 0; rb < HB; rb++) {
+      v4 acc = {0, 0, 0, 0}, dacc = {0, 0, 0, 0};
+#pragma unroll
+      for (int kb = 0; kb < HB; kb++)
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+          const T w = w1s[((rb * HB + kb) * 4 + s) * 64 + lane];
+          acc = Mfma<T>::mma(w, h1[kb][s], acc);
+          dacc = Mfma<T>::mma(w, dh1[kb][s], dacc);
+        }
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        T s_ = acc[v], d_ = dacc[v];
+        act_pair<T>(a.act, s_, d_);
+        acc[v] = s_; dacc[v] = d_;
+      }
+      h2[rb] = acc; dh2[rb] = dacc;
+    }
+    // ---- layer 2 (linear), operands swapped: rows = edges, columns = outputs
+    int mu_v[4];
+    long long e_v[4];
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const long long el = tile * 16 + a.drow[g * 4 + v];
+      e_v[v] = el < cnt ? a.e_begin + el : -1;
+      mu_v[v] = el < cnt ? a.emu[a.e_begin + el] : 0;
+    }
+    for (int cb = 0; cb < a.nob; cb++) {
+      v4 acc = {0, 0, 0, 0}, dacc = {0, 0, 0, 0};
+#pragma unroll
+      for (int kb = 0; kb < HB; kb++)
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+          const T w = w2p[((cb * HB + kb) * 4 + s) * 64 + lane];
+          acc = Mfma<T>::mma(h2[kb][s], w, acc);
+          dacc = Mfma<T>::mma(dh2[kb][s], w, dacc);
+        }
+      const int col = cb * 16 + c;
+      const int nch = col % a.C;
+#pragma unroll
+      for (int v = 0; v < 4; v++)
+        if (e_v[v] >= 0) {
+          const T zz = a.z[mu_v[v] * a.C + nch];
+          a.Rz[e_v[v] * a.noutp + col] = acc[v] * zz;
+          a.dRz[e_v[v] * a.noutp + col] = dacc[v] * zz;
+        }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// A basis
+// ---------------------------------------------------------------------------------------------------------------
+template<class T> struct ScatterArgs {
+  const long long *eoff;      // [n + 1]
+  const double *rh;           // [E][3]
+  const T *Rz;                // [E][noutp]
+  T *A;                       // [chunk atoms][nlm][C]
+  int a0;                     // first atom of the chunk
+  int C, nl, nlm, noutp;
+  ShCoef sh;
+};
+
+// one block per atom, thread = (l, n); Y of up to kBondChunk bonds staged in LDS per pass
+template<class T, int MAXM> __global__ void k_scatter_a(ScatterArgs<T> a)
+{
+  __shared__ T Ysh[kBondChunk][kMaxNlm];
+  const int t = threadIdx.x;
+  const int i = a.a0 + blockIdx.x;
+  const long long e0 = a.eoff[i], e1 = a.eoff[i + 1];
+  const int ncol = a.nl * a.C;
+  const int l = t < ncol ? t / a.C : 0, n = t % a.C;
+  const int nm = 2 * l + 1, lm0 = l * l;
+  T acc[MAXM];
+#pragma unroll
+  for (int m = 0; m < MAXM; m++) acc[m] = (T) 0;
+  for (long long base = e0; base < e1; base += kBondChunk) {
+    const int nb = (int) (e1 - base < kBondChunk ? e1 - base : kBondChunk);
+    __syncthreads();
+    if (t < nb) {
+      const double *u = a.rh + 3 * (base + t);
+      sh_eval<false, T>(a.sh, u[0], u[1], u[2], Ysh[t], nullptr);
+    }
+    __syncthreads();
+    if (t < ncol) {
+      for (int b = 0; b < nb; b++) {
+        const T r = a.Rz[(base + b) * a.noutp + t];
+        const T *y = Ysh[b] + lm0;
+#pragma unroll
+        for (int m = 0; m < MAXM; m++)
+          if (m < nm) acc[m] += y[m] * r;
+      }
+    }
+  }
+  if (t < ncol) {
+    T *Ai = a.A + (long long) blockIdx.x * a.nlm * a.C;
+#pragma unroll
+    for (int m = 0; m < MAXM; m++)
+      if (m < nm) Ai[(lm0 + m) * a.C + n] = acc[m];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// per-atom dense chain.  Per-atom tensors are [atom][function][channel].
+// ---------------------------------------------------------------------------------------------------------------
+template<class T> struct FcDev {
+  const T *Wl, *Wr;           // [tile][n_in][n_out], norms folded in
+  const T *WlT, *WrT;         // [tile][n_out][n_in]
+  const int *tile_l;          // [nf]
+  const T *nof;               // [nf]
+  const int *live;            // [nlive] output functions that are computed
+  const int *conn_off, *conn_from, *conn_tile;      // right connections by output function (CSR over nf)
+  const int *rlive;           // [nrlive] right-input functions that receive a gradient
+  const int *rconn_off, *rconn_to, *rconn_tile;     // right connections by right-input function (CSR over nfr)
+  int nf, nfr, nlive, nrlive, n_in_l, n_in_r, n_out;
+};
+
+// out[a][f][k] = nof[f] (sum_n Wl[tile_l f][n][k] Xl[a][f][n] + sum_{c -> f} sum_n Wr[tile c][n][k] Xr[a][from c][n])
+// grid (nlive, atom groups); block = n_out x AT threads
+template<class T> __global__ void k_fc_fwd(FcDev<T> F, const T *Xl, const T *Xr, T *out, int natoms, int nfl_stride,
+                                           int nfr_stride)
+{
+  const int k = threadIdx.x % F.n_out, al = threadIdx.x / F.n_out;
+  const int AT = blockDim.x / F.n_out;
+  const int at = blockIdx.y * AT + al;
+  if (at >= natoms || al >= AT) return;
+  const int f = F.live[blockIdx.x];
+  const T *xl = Xl + ((long long) at * nfl_stride + f) * F.n_in_l;
+  const T *wl = F.Wl + (long long) F.tile_l[f] * F.n_in_l * F.n_out + k;
+  T acc = (T) 0;
+  for (int n = 0; n < F.n_in_l; n++) acc += xl[n] * wl[(long long) n * F.n_out];
+  for (int c = F.conn_off[f]; c < F.conn_off[f + 1]; c++) {
+    const T *xr = Xr + ((long long) at * nfr_stride + F.conn_from[c]) * F.n_in_r;
+    const T *wr = F.Wr + (long long) F.conn_tile[c] * F.n_in_r * F.n_out + k;
+    for (int n = 0; n < F.n_in_r; n++) acc += xr[n] * wr[(long long) n * F.n_out];
+  }
+  out[((long long) at * nfl_stride + f) * F.n_out + k] = F.nof[f] * acc;
+}
+
+// gXl[a][f][n] += nof[f] sum_k Wl[tile_l f][n][k] g[a][f][k]     grid (nlive, atom groups); block = n_in_l x AT
+template<class T> __global__ void k_fc_bwd_left(FcDev<T> F, const T *g, T *gXl, int natoms, int nfl_stride)
+{
+  const int n = threadIdx.x % F.n_in_l, al = threadIdx.x / F.n_in_l;
+  const int AT = blockDim.x / F.n_in_l;
+  const int at = blockIdx.y * AT + al;
+  if (at >= natoms || al >= AT) return;
+  const int f = F.live[blockIdx.x];
+  const T *gg = g + ((long long) at * nfl_stride + f) * F.n_out;
+  const T *w = F.WlT + (long long) F.tile_l[f] * F.n_out * F.n_in_l + n;
+  T acc = (T) 0;
+  for (int k = 0; k < F.n_out; k++) acc += gg[k] * w[(long long) k * F.n_in_l];
+  gXl[((long long) at * nfl_stride + f) * F.n_in_l + n] += F.nof[f] * acc;
+}
+
+// gXr[a][r][n] += sum_{c: from c = r} nof[to c] sum_k Wr[tile c][n][k] g[a][to c][k]   grid (nrlive, atom groups)
+template<class T> __global__ void k_fc_bwd_right(FcDev<T> F, const T *g, T *gXr, int natoms, int nfl_stride, int nfr_stride)
+{
+  const int n = threadIdx.x % F.n_in_r, al = threadIdx.x / F.n_in_r;
+  const int AT = blockDim.x / F.n_in_r;
+  const int at = blockIdx.y * AT + al;
+  if (at >= natoms || al >= AT) return;
+  const int r = F.rlive[blockIdx.x];
+  T acc = (T) 0;
+  for (int c = F.rconn_off[r]; c < F.rconn_off[r + 1]; c++) {
+    const int to = F.rconn_to[c];
+    const T *gg = g + ((long long) at * nfl_stride + to) * F.n_out;
+    const T *w = F.WrT + (long long) F.rconn_tile[c] * F.n_out * F.n_in_r + n;
+    T s = (T) 0;
+    for (int k = 0; k < F.n_out; k++) s += gg[k] * w[(long long) k * F.n_in_r];
+    acc += F.nof[to] * s;
+  }
+  gXr[((long long) at * nfr_stride + r) * F.n_in_r + n] += acc;
+}
+
+struct ProdDev {
+  // forward: terms sorted by output (CSR off over nout; only live outputs have terms)
+  const int *off, *l, *r;
+  const double *c;
+  // reverse: terms by left operand (loff over nleft) and by right operand (roff over nright)
+  const int *loff, *l_o, *l_r;
+  const double *l_c;
+  const int *roff, *r_o, *r_l;
+  const double *r_c;
+  int nout, nleft, nright;
+};
+
+// out[a][o][k] = sum_t c_t L[a][l_t][k] R[a][r_t][k]      grid (nout, atom groups), block = C x AT
+template<class T> __global__ void k_prod_fwd(ProdDev P, const T *L, const T *R, T *out, int natoms, int C, int sl, int sr)
+{
+  const int k = threadIdx.x % C, al = threadIdx.x / C;
+  const int at = blockIdx.y * (blockDim.x / C) + al;
+  if (at >= natoms) return;
+  const int o = blockIdx.x;
+  const T *La = L + (long long) at * sl * C + k, *Ra = R + (long long) at * sr * C + k;
+  T acc = (T) 0;
+  for (int t = P.off[o]; t < P.off[o + 1]; t++) acc += (T) P.c[t] * La[(long long) P.l[t] * C] * Ra[(long long) P.r[t] * C];
+  out[((long long) at * P.nout + o) * C + k] = acc;
+}
+
+// gL[a][q][k] += sum_{t: l_t = q} c_t g[a][o_t][k] R[a][r_t][k]   (side 0), gR likewise with L (side 1)
+// grid (nleft or nright, atom groups)
+template<class T> __global__ void k_prod_bwd(ProdDev P, int side, const T *other, const T *g, T *gX, int natoms, int C, int so,
+                                             int sx)
+{
+  const int k = threadIdx.x % C, al = threadIdx.x / C;
+  const int at = blockIdx.y * (blockDim.x / C) + al;
+  if (at >= natoms) return;
+  const int q = blockIdx.x;
+  const int *off = side == 0 ? P.loff : P.roff, *oo = side == 0 ? P.l_o : P.r_o, *ot = side == 0 ? P.l_r : P.r_l;
+  const double *cc = side == 0 ? P.l_c : P.r_c;
+  if (off[q] == off[q + 1]) return;
+  const T *Oa = other + (long long) at * so * C + k, *ga = g + (long long) at * P.nout * C + k;
+  T acc = (T) 0;
+  for (int t = off[q]; t < off[q + 1]; t++) acc += (T) cc[t] * ga[(long long) oo[t] * C] * Oa[(long long) ot[t] * C];
+  gX[((long long) at * sx + q) * C + k] += acc;
+}
+
+template<class T> struct ReduceDev {
+  // per source s: collected functions fn[s][c] (unique), weights W[s][mu][c][n][kp] (norm folded, k padded to nrp)
+  const T *W[4];
+  const int *fn[4];
+  int ncol[4], nin[4], stride[4];    // collected functions, channels, functions per atom of the source tensor
+  int nsrc, nrho, nrp;
+};
+
+// rho[a][k] = sum_s sum_c sum_n W_s[mu_a][c][n][k] X_s[a][fn c][n]     one block per atom
+template<class T> __global__ void k_reduce_fwd(ReduceDev<T> R, const int *mu, int a0, const T *X0, const T *X1, const T *X2,
+                                               const T *X3, double *rho)
+{
+  __shared__ double part[4][32];
+  const int at = blockIdx.x;
+  const int m = mu[a0 + at];
+  const T *X[4] = {X0, X1, X2, X3};
+  double acc[32];
+#pragma unroll
+  for (int k = 0; k < 32; k++) acc[k] = 0.0;
+  for (int s = 0; s < R.nsrc; s++) {
+    const int nq = R.ncol[s] * R.nin[s];
+    const T *Ws = R.W[s] + (long long) m * nq * R.nrp;
+    const T *Xs = X[s] + (long long) at * R.stride[s] * R.nin[s];
+    for (int q = threadIdx.x; q < nq; q += blockDim.x) {
+      const int c = q / R.nin[s], n = q % R.nin[s];
+      const T x = Xs[(long long) R.fn[s][c] * R.nin[s] + n];
+      const T *w = Ws + (long long) q * R.nrp;
+#pragma unroll
+      for (int k = 0; k < 32; k++)
+        if (k < R.nrho) acc[k] += (double) (w[k] * x);
+    }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < 32; k++)
+    if (k < R.nrho) {
+      double v = acc[k];
+      for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
+      if (lane == 0) part[wave][k] = v;
+    }
+  __syncthreads();
+  if (threadIdx.x < R.nrho) {
+    double v = 0.0;
+    for (int w = 0; w < (int) (blockDim.x >> 6); w++) v += part[w][threadIdx.x];
+    rho[(long long) at * R.nrho + threadIdx.x] = v;
+  }
+}
+
+// gX_s[a][fn c][n] += sum_k W_s[mu_a][c][n][k] grho[a][k]            one block per atom
+template<class T> __global__ void k_reduce_bwd(ReduceDev<T> R, const int *mu, int a0, const double *grho, T *G0, T *G1, T *G2,
+                                               T *G3)
+{
+  __shared__ T gr[32];
+  const int at = blockIdx.x;
+  const int m = mu[a0 + at];
+  if (threadIdx.x < 32) gr[threadIdx.x] = threadIdx.x < R.nrho ? (T) grho[(long long) at * R.nrho + threadIdx.x] : (T) 0;
+  __syncthreads();
+  T *G[4] = {G0, G1, G2, G3};
+  for (int s = 0; s < R.nsrc; s++) {
+    const int nq = R.ncol[s] * R.nin[s];
+    const T *Ws = R.W[s] + (long long) m * nq * R.nrp;
+    T *Gs = G[s] + (long long) at * R.stride[s] * R.nin[s];
+    for (int q = threadIdx.x; q < nq; q += blockDim.x) {
+      const int c = q / R.nin[s], n = q % R.nin[s];
+      const T *w = Ws + (long long) q * R.nrp;
+      T v = (T) 0;
+#pragma unroll
+      for (int k = 0; k < 32; k++)
+        if (k < R.nrho) v += w[k] * gr[k];
+      Gs[(long long) R.fn[s][c] * R.nin[s] + n] += v;
+    }
+  }
+}
+
+struct EnergyDev {
+  const double *W[7];         // [n_in][n_out]
+  double norm[7];
+  int nin[7], nout[7];
+  int nlay, act, ln, nrho;
+  double out_scale;
+  const double *shift;        // [nel]
+};
+
+// E_i = (MLP(rho[1:]) + rho[0]) out_scale + shift[mu_i] and dE/drho, fp64, one wave per atom (fused_1l.cpp:378-427;
+// legacy RMS layer norm fused_cpu.h:666-682)
+__global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, const double *rho, double *grho, double *eatom_chunk,
+                         double *energy, int want_grad)
+{
+  __shared__ double act[8][256], pre[7][256], gbuf[2][256], x0[256];
+  const int at = blockIdx.x, lane = threadIdx.x;
+  const double *r = rho + (long long) at * M.nrho;
+  const int n0 = M.nrho - 1;
+  for (int k = lane; k < n0; k += 64) act[0][k] = r[k + 1];
+  __syncthreads();
+  double q = 0.0;
+  if (M.ln) {
+    double ms = 0.0;
+    for (int k = lane; k < n0; k += 64) { x0[k] = act[0][k]; ms += act[0][k] * act[0][k]; }
+    for (int o = 32; o > 0; o >>= 1) ms += __shfl_xor(ms, o, 64);
+    q = 1.0 / sqrt(ms / n0 + 1e-16);
+    for (int k = lane; k < n0; k += 64) act[0][k] *= q;
+    __syncthreads();
+  }
+  for (int L = 0; L < M.nlay; L++) {
+    for (int c = lane; c < M.nout[L]; c += 64) {
+      double s = 0.0;
+      for (int a = 0; a < M.nin[L]; a++) s += act[L][a] * M.W[L][(long long) a * M.nout[L] + c];
+      s *= M.norm[L];
+      pre[L][c] = s;
+      act[L + 1][c] = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+    }
+    __syncthreads();
+  }
+  const double Ei = (act[M.nlay][0] + r[0]) * M.out_scale + M.shift[mu[a0 + at]];
+  if (lane == 0) {
+    if (eatom_chunk) eatom_chunk[at] = Ei;
+    atomicAdd(energy, Ei);
+  }
+  if (!want_grad) return;
+  int cur = 0;
+  if (lane == 0) gbuf[0][0] = M.out_scale;
+  __syncthreads();
+  for (int L = M.nlay - 1; L >= 0; L--) {
+    if (L < M.nlay - 1) {
+      for (int c = lane; c < M.nout[L]; c += 64) {
+        const double v = pre[L][c];
+        if (M.act == 1) {
+          const double t = act[L + 1][c];
+          gbuf[cur][c] *= 1.0 - t * t;
+        } else {
+          const double sg = 1.0 / (1.0 + exp(-v));
+          gbuf[cur][c] *= sg * (1.0 + v * (1.0 - sg));
+        }
+      }
+      __syncthreads();
+    }
+    for (int a = lane; a < M.nin[L]; a += 64) {
+      double s = 0.0;
+      for (int c = 0; c < M.nout[L]; c++) s += gbuf[cur][c] * M.W[L][(long long) a * M.nout[L] + c];
+      gbuf[cur ^ 1][a] = s * M.norm[L];
+    }
+    cur ^= 1;
+    __syncthreads();
+  }
+  if (M.ln) {
+    double t = 0.0;
+    for (int k = lane; k < n0; k += 64) t += gbuf[cur][k] * x0[k];
+    for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
+    for (int k = lane; k < n0; k += 64) gbuf[cur][k] = q * (gbuf[cur][k] - x0[k] * t * q * q / n0);
+    __syncthreads();
+  }
+  double *g = grho + (long long) at * M.nrho;
+  if (lane == 0) g[0] = M.out_scale;
+  for (int k = lane; k < n0; k += 64) g[k + 1] = gbuf[cur][k];
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// bond backward: forces and virial
+// ---------------------------------------------------------------------------------------------------------------
+template<class T> struct BondBwdArgs {
+  const long long *eoff;
+  const int *ej;
+  const double *rh, *r, *rc;
+  const T *Rz, *dRz;          // [E][noutp]
+  const T *gA;                // [chunk atoms][nlm][C]
+  double *f;                  // [n][3]  (+=, atomics)
+  double *virial;             // [6]     (+=, atomics)
+  int a0;
+  int C, nl, nlm, noutp;
+  ShCoef sh;
+};
+
+// one block per atom, thread = (l, n).  Per bond: g_d = sum_{l n} Rz[l][n] sum_m G[lm][d] gA[lm][n],
+// dE/dx = sum_{l n} dRz[l][n] sum_m Y[lm] gA[lm][n]; fv = dEdx / rc rhat + (g - (g . rhat) rhat) / r;
+// f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv.
+template<class T, int MAXM> __global__ void k_bond_bwd(BondBwdArgs<T> a)
+{
+  __shared__ T Ysh[kBondChunk][kMaxNlm];
+  __shared__ T Gsh[kBondChunk][kMaxNlm * 3];
+  __shared__ double part[kBondChunk][16][4];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nw = blockDim.x >> 6;
+  const int i = a.a0 + blockIdx.x;
+  const long long e0 = a.eoff[i], e1 = a.eoff[i + 1];
+  const int ncol = a.nl * a.C;
+  const int l = t < ncol ? t / a.C : 0, n = t % a.C;
+  const int nm = t < ncol ? 2 * l + 1 : 0, lm0 = l * l;
+  T ga[MAXM];
+  {
+    const T *gAi = a.gA + (long long) blockIdx.x * a.nlm * a.C;
+#pragma unroll
+    for (int m = 0; m < MAXM; m++) ga[m] = m < nm ? gAi[(lm0 + m) * a.C + n] : (T) 0;
+  }
+  double fi[3] = {0, 0, 0}, vir[6] = {0, 0, 0, 0, 0, 0};
+  for (long long base = e0; base < e1; base += kBondChunk) {
+    const int nb = (int) (e1 - base < kBondChunk ? e1 - base : kBondChunk);
+    __syncthreads();
+    if (t < nb) {
+      const double *u = a.rh + 3 * (base + t);
+      sh_eval<true, T>(a.sh, u[0], u[1], u[2], Ysh[t], Gsh[t]);
+    }
+    __syncthreads();
+    for (int b = 0; b < nb; b++) {
+      double p0 = 0, p1 = 0, p2 = 0, px = 0;
+      if (t < ncol) {
+        const T rz = a.Rz[(base + b) * a.noutp + t], drz = a.dRz[(base + b) * a.noutp + t];
+        const T *y = Ysh[b] + lm0, *G = Gsh[b] + 3 * lm0;
+        T tx = 0, t0 = 0, t1 = 0, t2 = 0;
+#pragma unroll
+        for (int m = 0; m < MAXM; m++)
+          if (m < nm) {
+            tx += y[m] * ga[m];
+            t0 += G[3 * m] * ga[m];
+            t1 += G[3 * m + 1] * ga[m];
+            t2 += G[3 * m + 2] * ga[m];
+          }
+        p0 = (double) (rz * t0); p1 = (double) (rz * t1); p2 = (double) (rz * t2); px = (double) (drz * tx);
+      }
+      for (int o = 32; o > 0; o >>= 1) {
+        p0 += __shfl_down(p0, o, 64); p1 += __shfl_down(p1, o, 64);
+        p2 += __shfl_down(p2, o, 64); px += __shfl_down(px, o, 64);
+      }
+      if (lane == 0) { part[b][wave][0] = p0; part[b][wave][1] = p1; part[b][wave][2] = p2; part[b][wave][3] = px; }
+    }
+    __syncthreads();
+    if (t < nb) {
+      double gv[3] = {0, 0, 0}, dEdx = 0;
+      for (int w = 0; w < nw; w++) { gv[0] += part[t][w][0]; gv[1] += part[t][w][1]; gv[2] += part[t][w][2]; dEdx += part[t][w][3]; }
+      const long long e = base + t;
+      const double *u = a.rh + 3 * e;
+      const double r = a.r[e], rc = a.rc[e];
+      const double dEdr = dEdx / rc;
+      const double gr = gv[0] * u[0] + gv[1] * u[1] + gv[2] * u[2];
+      double fv[3];
+      for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + (gv[d] - gr * u[d]) / r;
+      const int jj = a.ej[e];
+      for (int d = 0; d < 3; d++) {
+        fi[d] += fv[d];
+        atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
+      }
+      const double dx = -u[0] * r, dy = -u[1] * r, dz = -u[2] * r;
+      vir[0] += dx * fv[0]; vir[1] += dy * fv[1]; vir[2] += dz * fv[2];
+      vir[3] += dx * fv[1]; vir[4] += dx * fv[2]; vir[5] += dy * fv[2];
+    }
+  }
+  // only the first kBondChunk threads carry partial sums: reduce them inside wave 0
+  if (wave == 0) {
+    double v[9] = {fi[0], fi[1], fi[2], vir[0], vir[1], vir[2], vir[3], vir[4], vir[5]};
+#pragma unroll
+    for (int k = 0; k < 9; k++)
+      for (int o = 32; o > 0; o >>= 1) v[k] += __shfl_down(v[k], o, 64);
+    if (lane == 0) {
+      for (int d = 0; d < 3; d++) atomicAdd(&a.f[3 * (long long) i + d], v[d]);
+      for (int k = 0; k < 6; k++) atomicAdd(&a.virial[k], v[3 + k]);
+    }
+  }
+}
+
+}    // namespace grhip

@@ -1,0 +1,405 @@
+"""MI355X plug-in module with the interface of the reference's GPU module `_kk_<arch>` (python/kk/kk_api.h:16-156,
+bindings python/kk/kk_module.cpp:200-275): module functions `initialize / finalize / initialized / device / arch /
+platform / blas / cublas / memory_info`, classes `Model`, `System`, `Batch`, and the plug-in attributes `ABI`,
+`PLATFORM` (python-rocm6/grace_runtime_rocm6/__init__.py:8-22).  `Engine` is the CSR-level entry
+(`_core.Model.compute`, python/src/core.cpp:292-396) and `neighbor_search` the list of `_core.neighbor_search`.
+
+All arithmetic runs in libgrace_hip.so on the GPU; there is no CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import FLAG_EATOM, FLAG_ENERGY_ONLY, as_array, check, ptr
+
+ABI = 7
+PLATFORM = "rocm"
+ROCM_MAJOR = 7
+
+_state = {"device": None}
+
+
+def archs():
+    return ["gfx950"]
+
+
+def initialize(device: int = 0):
+    """One GPU per process (python/kk/kk_core.cpp:86-98): a second call with another device is an error."""
+    L = _lib.lib()
+    if _state["device"] is not None:
+        if _state["device"] != int(device):
+            raise RuntimeError(f"already initialised on device {_state['device']}")
+        return
+    n = L.gr_device_count()
+    if n <= 0:
+        raise RuntimeError("no HIP device found")
+    if not 0 <= int(device) < n:
+        raise ValueError(f"device {device} out of range (0 .. {n - 1})")
+    _state["device"] = int(device)
+
+
+def finalize():
+    _state["device"] = None
+
+
+def initialized() -> bool:
+    return _state["device"] is not None
+
+
+def device() -> int:
+    if _state["device"] is None:
+        raise RuntimeError("not initialised")
+    return _state["device"]
+
+
+def arch() -> str:
+    return "gfx950"
+
+
+def platform() -> str:
+    return PLATFORM
+
+
+def blas() -> str:
+    return ""    # hand-written MFMA kernels, no BLAS library
+
+
+def cublas() -> bool:
+    return False
+
+
+def memory_info():
+    import torch
+    free, total = torch.cuda.mem_get_info(device())
+    return int(free), int(total)
+
+
+def _dev():
+    if _state["device"] is None:
+        initialize(0)
+    return _state["device"]
+
+
+def neighbor_search(positions, cell, pbc, cutoff, num_threads: int = 0):
+    """(perm, offset, j, image, shifts) of the Verlet list at `cutoff`; identical to the reference list
+    (python/src/neighbors.cpp:15-95)."""
+    L = _lib.lib()
+    pos = as_array(positions, np.float64, 3) if len(positions) else np.zeros((0, 3))
+    cell = np.ascontiguousarray(cell, dtype=np.float64).reshape(3, 3)
+    pb = np.ascontiguousarray([bool(p) for p in pbc], dtype=np.uint8)
+    h = C.c_void_p()
+    check(L.gr_neighbor_build(pos.shape[0], ptr(pos), ptr(cell), ptr(pb), float(cutoff), max(int(num_threads), 1) if
+                              num_threads else 8, C.byref(h)))
+    try:
+        n, nb, ni = pos.shape[0], L.gr_nlist_nbonds(h), L.gr_nlist_nimages(h)
+        perm, offset = np.zeros(n, np.int64), np.zeros(n + 1, np.int64)
+        j, image, shifts = np.zeros(nb, np.int32), np.zeros(nb, np.int32), np.zeros((ni, 3))
+        check(L.gr_nlist_get(h, ptr(perm), ptr(offset), ptr(j), ptr(image), ptr(shifts)))
+    finally:
+        L.gr_nlist_free(h)
+    return perm, offset, j, image, shifts
+
+
+class Model:
+    """A loaded kokkos.npz (host side).  `Model(path, spline=1024, asi="")`: python/kk/kk_api.h:51-64; `spline` is
+    accepted for interface compatibility (this engine evaluates the radial MLP exactly, without tables)."""
+
+    def __init__(self, path, spline: int = 1024, asi: str = ""):
+        L = _lib.lib()
+        if asi:
+            raise ValueError("PACE active-set files are not supported by this engine")
+        self._h = C.c_void_p()
+        check(L.gr_model_load(str(path).encode(), C.byref(self._h)))
+        info = _lib.ModelInfo()
+        check(L.gr_model_get_info(self._h, C.byref(info)))
+        self.path = str(path)
+        self.layers = info.layers
+        self.lmax, self.n_radial, self.rcut, self.max_order = info.lmax, info.n_radial, info.rcut, info.max_order
+        self.n_elements = info.n_elements
+        self.element_names = [L.gr_model_element_name(self._h, k).decode() for k in range(info.n_elements)]
+        self.has_uq = False
+        self.slow_notice = ""
+        self.needs_generic = False
+        self.engine_setups = 0
+
+    def validate_uq(self):
+        raise ValueError(f"GRACE-{self.layers}L: the model has no UQ head")
+
+    def type2mu(self, species):
+        """[-1, mu(species[0]), ...]; unknown element -> ValueError (python/kk/kk_core.cpp: std::invalid_argument)"""
+        out = [-1]
+        for s in species:
+            if s not in self.element_names:
+                raise ValueError(f"element {s} is not in the model (elements: {' '.join(self.element_names)})")
+            out.append(self.element_names.index(s))
+        return np.asarray(out, dtype=np.int32)
+
+    def __del__(self):
+        try:
+            if getattr(self, "_h", None):
+                _lib.lib().gr_model_free(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+class Engine:
+    """One model + species set on the GPU.  `compute` is `_core.Model.compute` on CSR bonds
+    (python/src/core.cpp:292-396); `upload / run / fetch` split it for callers that keep the structure resident."""
+
+    def __init__(self, model: Model, species, precision: int = 64):
+        L = _lib.lib()
+        self.model, self.species, self.precision = model, list(species), int(precision)
+        t2m = model.type2mu(self.species)
+        self._h = C.c_void_p()
+        check(L.gr_engine_create(model._h, len(self.species), ptr(t2m), self.precision, _dev(), C.byref(self._h)))
+        model.engine_setups += 1
+        self._n = 0
+
+    def cutoff(self, t1: int, t2: int) -> float:
+        return _lib.lib().gr_engine_cutoff(self._h, int(t1), int(t2))
+
+    def cutoff_matrix(self):
+        k = len(self.species)
+        return np.array([[self.cutoff(a + 1, b + 1) for b in range(k)] for a in range(k)])
+
+    def _csr_args(self, types, offset, j, rij, positions, image, shifts):
+        types = as_array(types, np.int32)
+        offset = as_array(offset, np.int64)
+        j = as_array(j, np.int32)
+        n = types.shape[0]
+        if offset.shape[0] != n + 1:
+            raise ValueError("offset must have len(types) + 1 entries")
+        table = positions is not None and image is not None and shifts is not None
+        if (rij is not None) == (positions is not None or image is not None or shifts is not None) or \
+                (rij is None and not table):
+            raise ValueError("give rij or positions, image and shifts")
+        rij = None if rij is None else np.ascontiguousarray(rij, dtype=np.float64).reshape(-1, 3)
+        positions = None if positions is None else np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
+        image = as_array(image, np.int32)
+        shifts = None if shifts is None else np.ascontiguousarray(shifts, dtype=np.float64).reshape(-1, 3)
+        if n and offset[-1] != j.shape[0]:
+            raise ValueError("offset[0] must be 0 and offset[-1] == len(j)")
+        if rij is not None and rij.shape[0] != j.shape[0]:
+            raise ValueError("j and rij differ in length")
+        if image is not None and image.shape[0] != j.shape[0]:
+            raise ValueError("j and image differ in length")
+        if positions is not None and positions.shape[0] != n:
+            raise ValueError("positions must have len(types) rows")
+        if shifts is not None and shifts.shape[0] == 0:
+            shifts = np.zeros((1, 3))
+            nimg = 0
+        else:
+            nimg = 0 if shifts is None else shifts.shape[0]
+        return n, (types, offset, j, rij, positions, image, shifts), nimg
+
+    def compute(self, types, offset, j, rij=None, energies=False, energy_only=False, positions=None, image=None,
+                shifts=None):
+        n, arrs, nimg = self._csr_args(types, offset, j, rij, positions, image, shifts)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
+        e = C.c_double(0.0)
+        f, v, ea = np.zeros((n, 3)), np.zeros(6), np.zeros(n)
+        check(_lib.lib().gr_compute_csr(self._h, n, *[ptr(a) for a in arrs], nimg, flags, C.addressof(e), ptr(f), ptr(v),
+                                        ptr(ea) if energies else None))
+        out = {"energy": e.value}
+        if not energy_only:
+            out["forces"], out["virial"] = f, v
+        if energies:
+            out["energies"] = ea
+        return out
+
+    def upload(self, types, offset, j, rij=None, positions=None, image=None, shifts=None):
+        n, arrs, nimg = self._csr_args(types, offset, j, rij, positions, image, shifts)
+        check(_lib.lib().gr_engine_upload(self._h, n, *[ptr(a) for a in arrs], nimg))
+        self._n = n
+
+    def run(self, energies=False, energy_only=False):
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
+        check(_lib.lib().gr_engine_run(self._h, flags))
+
+    def sync(self):
+        check(_lib.lib().gr_engine_sync(self._h))
+
+    def fetch(self, energies=False):
+        n = self._n
+        e = C.c_double(0.0)
+        f, v, ea = np.zeros((n, 3)), np.zeros(6), np.zeros(n)
+        check(_lib.lib().gr_engine_fetch(self._h, C.addressof(e), ptr(f), ptr(v), ptr(ea) if energies else None))
+        out = {"energy": e.value, "forces": f, "virial": v}
+        if energies:
+            out["energies"] = ea
+        return out
+
+    def edge_count(self) -> int:
+        return int(_lib.lib().gr_engine_edge_count(self._h))
+
+    def set_profile(self, on=True):
+        check(_lib.lib().gr_engine_set_profile(self._h, int(bool(on))))
+
+    def stage_times(self):
+        """{stage: (milliseconds, launches)} of the last run (HIP events on the engine's stream)"""
+        L = _lib.lib()
+        n = L.gr_engine_stage_count(self._h)
+        if n < 0:
+            check(_lib.GR_ERROR)
+        out = {}
+        buf = C.create_string_buffer(64)
+        for k in range(n):
+            ms, cnt = C.c_double(0.0), C.c_int(0)
+            check(L.gr_engine_stage_get(self._h, k, buf, 64, C.byref(ms), C.byref(cnt)))
+            out[buf.value.decode()] = (ms.value, cnt.value)
+        return out
+
+    def debug_radial(self, x, mu_j):
+        x = as_array(x, np.float64)
+        mu_j = as_array(mu_j, np.int32)
+        nl, Cn = self.model.lmax + 1, self.model.n_radial
+        R, dR = np.zeros((x.shape[0], nl, Cn)), np.zeros((x.shape[0], nl, Cn))
+        check(_lib.lib().gr_engine_debug_radial(self._h, x.shape[0], ptr(x), ptr(mu_j), ptr(R), ptr(dR)))
+        return R, dR
+
+    def close(self):
+        if getattr(self, "_h", None):
+            _lib.lib().gr_engine_free(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _padded_cell_arrays(cell, pos, reach, pbc=None):
+    """Zero cell vectors and the vectors of open directions replaced by vectors normal to the periodic ones, long
+    enough that no image is within reach, and the shift that puts the atoms inside that box
+    (python/grace_runtime/neighbors.py:27-47)."""
+    cell = np.array(cell, dtype=np.float64)
+    pad = [k for k in range(3) if not np.any(cell[k]) or (pbc is not None and not pbc[k])]
+    if not pad:
+        return cell, np.zeros(3)
+    given = np.array([cell[k] for k in range(3) if k not in pad]).reshape(-1, 3)
+    dirs = np.linalg.svd(given)[2][len(given):] if len(given) else np.eye(3)
+    shift = np.zeros(3)
+    for k, d in zip(pad, dirs):
+        proj = pos @ d
+        cell[k] = d * (np.ptp(proj) + 2.0 * reach + 1.0) if len(pos) else d * (2.0 * reach + 1.0)
+        if len(pos):
+            shift += d * (reach + 0.5 - proj.min())
+    return cell, shift
+
+
+class System:
+    """One structure on the device with a Verlet list at cutoff + skin, rebuilt when an atom moved more than
+    skin / 2 or the atoms / cell / pbc change (python/kk/kk_api.h:66-93, list policy python/grace_runtime/
+    neighbors.py:68-89)."""
+
+    def __init__(self, model: Model, species, skin: float = 0.5, spline: int = 1024, chunksize: int = -1,
+                 precision: int = 64):
+        skin = float(skin)
+        if not (np.isfinite(skin) and skin >= 0.0):
+            raise ValueError(f"skin must be a finite number >= 0, got {skin!r}")
+        self.engine = Engine(model, species, precision)
+        self.skin = skin
+        self.cutoff = float(self.engine.cutoff_matrix().max()) if len(species) else 0.0
+        self.rebuilds = 0
+        self.chunksize = 0
+        self._x0 = self._key = self._nl = None
+
+    def release_buffers(self):
+        self._x0 = self._key = self._nl = None
+
+    def set_dispersion(self, *a, **k):
+        raise ValueError("dispersion corrections are not part of this engine")
+
+    def compute(self, types, positions, cell, pbc, energies=False, uq=False, energy_only=False):
+        if uq:
+            raise ValueError("the model has no UQ head")
+        types = as_array(types, np.int32)
+        pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
+        cell = np.ascontiguousarray(cell, dtype=np.float64).reshape(3, 3)
+        pbc = np.asarray([bool(p) for p in pbc])
+        n = types.shape[0]
+        if pos.shape[0] != n:
+            raise ValueError("positions must have len(types) rows")
+        if n and (types.min() < 1 or types.max() > len(self.engine.species)):
+            raise ValueError("types must be 1 .. len(species)")
+        key = (cell.tobytes(), pbc.tobytes(), types.tobytes())
+        rebuild = self._x0 is None or key != self._key or len(self._x0) != n or \
+            (n > 0 and ((pos - self._x0) ** 2).sum(axis=1).max() > (0.5 * self.skin) ** 2)
+        if rebuild:
+            reach = self.cutoff + self.skin
+            pcell, shift = _padded_cell_arrays(cell, pos, reach, pbc)
+            self._nl = neighbor_search(pos + shift, pcell, pbc, reach)
+            self._key, self._x0 = key, pos.copy()
+            self.rebuilds += 1
+        perm, offset, j, image, shifts = self._nl
+        out = self.engine.compute(types[perm], offset, j, energies=energies, energy_only=energy_only,
+                                  positions=pos[perm], image=image, shifts=shifts)
+        res = {"energy": out["energy"]}
+        if not energy_only:
+            f = np.empty((n, 3))
+            f[perm] = out["forces"]
+            res["forces"], res["virial"] = f, out["virial"]
+        if energies:
+            e = np.empty(n)
+            e[perm] = out["energies"]
+            res["energies"] = e
+        return res
+
+
+class Batch:
+    """Many structures per call (python/kk/kk_api.h:116-156): energy [S], virial [S, 6], forces [N, 3] in input
+    order.  Structures are evaluated one engine pass each."""
+
+    def __init__(self, model: Model, species, spline: int = 1024, chunksize: int = -1, precision: int = 64):
+        self.engine = Engine(model, species, precision)
+        self.cutoff = float(self.engine.cutoff_matrix().max()) if len(species) else 0.0
+        self.passes = 0
+        self.keep_buffers = False
+        self.chunksize = 0
+
+    def release_buffers(self):
+        pass
+
+    def compute(self, natoms, types, positions, cells, pbc, energies=False, uq=False, energy_only=False,
+                max_nall=1 << 21, dispersion_parts=False):
+        if uq:
+            raise ValueError("the model has no UQ head")
+        natoms = np.asarray(natoms, dtype=np.int32)
+        types = as_array(types, np.int32)
+        pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
+        cells = np.ascontiguousarray(cells, dtype=np.float64).reshape(-1, 3, 3)
+        pbc = np.ascontiguousarray(pbc, dtype=bool).reshape(-1, 3)
+        S = natoms.shape[0]
+        if cells.shape[0] != S or pbc.shape[0] != S or natoms.sum() != types.shape[0] or pos.shape[0] != types.shape[0]:
+            raise ValueError("natoms, types, positions, cells and pbc do not describe the same structures")
+        if types.size and (types.min() < 1 or types.max() > len(self.engine.species)):
+            raise ValueError("types must be 1 .. len(species)")
+        N = types.shape[0]
+        out = {"energy": np.zeros(S)}
+        if not energy_only:
+            out["forces"], out["virial"] = np.zeros((N, 3)), np.zeros((S, 6))
+        if energies:
+            out["energies"] = np.zeros(N)
+        starts = np.concatenate([[0], np.cumsum(natoms)])
+        self.passes = 0
+        for k in range(S):
+            lo, hi = starts[k], starts[k + 1]
+            if hi == lo:
+                continue
+            pcell, shift = _padded_cell_arrays(cells[k], pos[lo:hi], self.cutoff, pbc[k])
+            perm, offset, j, image, shifts = neighbor_search(pos[lo:hi] + shift, pcell, pbc[k], self.cutoff)
+            r = self.engine.compute(types[lo:hi][perm], offset, j, energies=energies, energy_only=energy_only,
+                                    positions=pos[lo:hi][perm], image=image, shifts=shifts)
+            self.passes += 1
+            out["energy"][k] = r["energy"]
+            if not energy_only:
+                out["forces"][lo + perm] = r["forces"]
+                out["virial"][k] = r["virial"]
+            if energies:
+                out["energies"][lo + perm] = r["energies"]
+        return out

@@ -1,0 +1,341 @@
+"""Synthetic GRACE models (kokkos.npz layout, random-init weights) and synthetic periodic structures.
+
+The structure arrays of a kokkos.npz file (FC tiles, Clebsch-Gordan term lists, reduce collect indices) are
+normally written by the training code's exporter.  This module regenerates them from first principles so that
+benchmark and test models of any lmax can be written without that exporter:
+
+* real Gaunt coefficients by exact quadrature of products of real spherical harmonics (4 pi normalised, index
+  lm = l(l+1)+m, Y_1,+1 = sqrt(3) x), normalised so that coupling Y_l1(r) x Y_l2(r) returns exactly Y_LM(r);
+* AA functions ordered by L, then by the pair l1 >= l2 (parity-even couplings only), then by M; the symmetric
+  terms (m1, m2)/(m2, m1) of a self product l1 == l2 merged into one term with left index >= right index;
+* AAA = AA1 x A1 -> L = 0 for l1 >= l2 >= l3; AAAA = AA2 x AA2 -> L = 0 over pairs of AA groups of equal L
+  (left group >= right group); for lmax <= 4 the candidates the training code's exporter leaves out (_AAAA_SKIP,
+  read off its lmax-4 export) are skipped, for larger lmax a linearly independent set is kept (greedy numerical
+  rank test on a single channel, in output order);
+* FC: A1 one weight tile per l; AA1/AA2 one tile per (L, l1, l2) group, right input the A function (l = L, m = M);
+* rho reduce: collects the invariant (L = 0) functions of each source, one weight tile per collected function.
+
+File layout and key names follow the reference loader, libgrace/src/model_1l.cpp:18-273 (scalars as shape-(1,)
+int64/float64 arrays, weights [n_in, n_out] float64 with a separate 1/sqrt(n_in) norm scalar, index arrays int32).
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+__all__ = ["real_sh_np", "coupling_tables", "structure_1l", "random_model_1l", "save_model", "bcc_supercell",
+           "fcc_supercell", "jitter"]
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# real spherical harmonics (closed form through associated Legendre functions; used for the quadrature only)
+# ---------------------------------------------------------------------------------------------------------------
+def _legendre_no_cs(lmax, ct):
+    """P_l^m(cos t) without the Condon-Shortley phase, dict[(l, m)], m >= 0."""
+    st = np.sqrt(np.maximum(0.0, 1.0 - ct * ct))
+    P = {(0, 0): np.ones_like(ct)}
+    for m in range(1, lmax + 1):
+        P[(m, m)] = P[(m - 1, m - 1)] * (2 * m - 1) * st
+    for m in range(0, lmax):
+        P[(m + 1, m)] = ct * (2 * m + 1) * P[(m, m)]
+    for m in range(0, lmax + 1):
+        for l in range(m + 2, lmax + 1):
+            P[(l, m)] = ((2 * l - 1) * ct * P[(l - 1, m)] - (l + m - 1) * P[(l - 2, m)]) / (l - m)
+    return P
+
+
+def real_sh_np(u, lmax):
+    """Y[n, (lmax+1)^2] of unit vectors u[n, 3]: 4 pi normalised real harmonics, lm = l(l+1)+m,
+    Y(l, m>0) ~ cos(m phi), Y(l, m<0) ~ sin(|m| phi), all with positive leading sign (Y_1,1 = sqrt(3) x)."""
+    u = np.asarray(u, dtype=np.float64)
+    ct = u[:, 2]
+    phi = np.arctan2(u[:, 1], u[:, 0])
+    P = _legendre_no_cs(lmax, ct)
+    Y = np.zeros((u.shape[0], (lmax + 1) ** 2))
+    for l in range(lmax + 1):
+        c = l * (l + 1)
+        Y[:, c] = math.sqrt(2 * l + 1) * P[(l, 0)]
+        for m in range(1, l + 1):
+            N = math.sqrt(2.0 * (2 * l + 1) * math.factorial(l - m) / math.factorial(l + m))
+            Y[:, c + m] = N * P[(l, m)] * np.cos(m * phi)
+            Y[:, c - m] = N * P[(l, m)] * np.sin(m * phi)
+    return Y
+
+
+def _sphere_quadrature(deg):
+    """nodes u[n, 3] and weights (sum 1) exact for polynomials of degree <= deg on the unit sphere."""
+    nt = deg // 2 + 1
+    x, w = np.polynomial.legendre.leggauss(nt)
+    nphi = deg + 1
+    phi = 2.0 * math.pi * np.arange(nphi) / nphi
+    ct = np.repeat(x, nphi)
+    ww = np.repeat(w, nphi) / (2.0 * nphi)
+    ph = np.tile(phi, nt)
+    st = np.sqrt(1.0 - ct * ct)
+    return np.stack([st * np.cos(ph), st * np.sin(ph), ct], 1), ww
+
+
+_GAUNT_CACHE = {}
+
+
+def coupling_tables(lmax):
+    """C[(l1, l2, L)] = array [2l1+1, 2l2+1, 2L+1]: the real coupling coefficients with
+    sum_{m1 m2} C[m1, m2, M] Y_l1m1(r) Y_l2m2(r) = Y_LM(r) for every unit vector r (l1 + l2 + L even)."""
+    if lmax in _GAUNT_CACHE:
+        return _GAUNT_CACHE[lmax]
+    u, w = _sphere_quadrature(3 * lmax + 2)
+    Y = real_sh_np(u, lmax)
+    out = {}
+    for l1 in range(lmax + 1):
+        for l2 in range(lmax + 1):
+            for L in range(abs(l1 - l2), min(lmax, l1 + l2) + 1):
+                if (l1 + l2 + L) % 2:
+                    continue
+                a = Y[:, l1 * l1:(l1 + 1) ** 2]
+                b = Y[:, l2 * l2:(l2 + 1) ** 2]
+                c = Y[:, L * L:(L + 1) ** 2]
+                G = np.einsum("n,na,nb,nc->abc", w, a, b, c, optimize=True)
+                G[np.abs(G) < 1e-12] = 0.0
+                s = (G[:, :, 0] ** 2).sum()
+                out[(l1, l2, L)] = G / s
+    _GAUNT_CACHE[lmax] = out
+    return out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# structure arrays of a GRACE-1L model
+# ---------------------------------------------------------------------------------------------------------------
+def _aa_groups(lmax, Lmax):
+    groups = []
+    for L in range(Lmax + 1):
+        for l1 in range(lmax + 1):
+            for l2 in range(l1 + 1):
+                if abs(l1 - l2) <= L <= l1 + l2 and (l1 + l2 + L) % 2 == 0:
+                    groups.append((L, l1, l2))
+    return groups
+
+
+# AAAA candidates (L, (l1, l2), (l3, l4)) absent from exported lmax <= 4 models
+_AAAA_SKIP = {(1, (1, 0), (1, 0)), (2, (1, 1), (1, 1)), (2, (2, 0), (1, 1)), (2, (2, 0), (2, 0)), (2, (3, 1), (2, 0)),
+              (3, (3, 0), (2, 1)), (3, (4, 1), (2, 1)), (2, (2, 2), (2, 2)), (4, (2, 2), (2, 2)), (4, (4, 0), (2, 2)),
+              (4, (4, 2), (2, 2)), (3, (3, 0), (3, 0)), (3, (3, 2), (3, 0)), (3, (4, 1), (3, 0)), (4, (3, 3), (3, 1)),
+              (4, (4, 0), (3, 1)), (4, (4, 0), (3, 3)), (4, (4, 0), (4, 0)), (4, (4, 2), (4, 0)), (4, (4, 4), (4, 2))}
+
+
+def _prod_arrays(terms):
+    """terms: list of (out, left, right, coeff) -> sorted int32/float64 arrays."""
+    terms = sorted(terms, key=lambda t: t[4] if len(t) > 4 else (t[0], t[1], t[2]))
+    o = np.array([t[0] for t in terms], dtype=np.int32)
+    l = np.array([t[1] for t in terms], dtype=np.int32)
+    r = np.array([t[2] for t in terms], dtype=np.int32)
+    c = np.array([t[3] for t in terms], dtype=np.float64)
+    return l, r, o, c
+
+
+def structure_1l(lmax, order4=True, seed_indep=12345):
+    """Structure arrays (no weights) of a GRACE-1L model with Lmax = lmax: dict of numpy arrays keyed like the
+    kokkos.npz file, plus '_groups' (list of (L, l1, l2) of the AA tiles) for the weight generator."""
+    C = coupling_tables(lmax)
+    nl = lmax + 1
+    nlm = nl * nl
+    lm_l = np.repeat(np.arange(nl), 2 * np.arange(nl) + 1).astype(np.int32)
+    groups = _aa_groups(lmax, lmax)
+    g_first, fn_group, fn_M = [], [], []
+    for g, (L, l1, l2) in enumerate(groups):
+        g_first.append(len(fn_group))
+        for M in range(-L, L + 1):
+            fn_group.append(g)
+            fn_M.append(M)
+    nAA = len(fn_group)
+    s = {}
+    # ---- AA = A1 x A1
+    terms = []
+    for g, (L, l1, l2) in enumerate(groups):
+        T = C[(l1, l2, L)]
+        for M in range(-L, L + 1):
+            o = g_first[g] + M + L
+            acc = {}
+            for m1 in range(-l1, l1 + 1):
+                for m2 in range(-l2, l2 + 1):
+                    v = T[m1 + l1, m2 + l2, M + L]
+                    if v == 0.0:
+                        continue
+                    a, b = l1 * (l1 + 1) + m1, l2 * (l2 + 1) + m2
+                    if l1 == l2 and a < b:      # self product: (m1, m2) and (m2, m1) are the same term
+                        a, b = b, a
+                    acc[(a, b)] = acc.get((a, b), 0.0) + v
+            for (a, b), v in acc.items():
+                if abs(v) > 1e-12:    # self products keep the order of the unswapped (smaller, larger) pair
+                    terms.append((o, a, b, v, (o, b, a) if l1 == l2 else (o, a, b)))
+    l, r, o, c = _prod_arrays(terms)
+    s.update(prod_AA_left_ind=l, prod_AA_right_ind=r, prod_AA_m_sum_ind=o, prod_AA_cg_coeff=c,
+             prod_AA_n_output_funcs=np.array([nAA], np.int64), prod_AA_n_cg_terms=np.array([c.size], np.int64),
+             prod_AA_lmax=np.array([lmax], np.int64), prod_AA_Lmax=np.array([lmax], np.int64))
+    # ---- FCs
+    s.update(fc_A1_w_tile_left=lm_l.copy(), fc_A1_w_tile_right=lm_l.copy(),
+             fc_A1_collect_to=np.arange(nlm, dtype=np.int32), fc_A1_collect_from=np.arange(nlm, dtype=np.int32),
+             fc_A1_norm_out_factor=np.full((nlm, 1, 1), 1.0 / math.sqrt(2.0)))
+    frm = np.array([groups[g][0] * (groups[g][0] + 1) + M for g, M in zip(fn_group, fn_M)], dtype=np.int32)
+    for k in (["AA1", "AA2"] if order4 else ["AA1"]):
+        s.update({f"fc_{k}_w_tile_left": np.array(fn_group, np.int32), f"fc_{k}_w_tile_right": np.array(fn_group, np.int32),
+                  f"fc_{k}_collect_to": np.arange(nAA, dtype=np.int32), f"fc_{k}_collect_from": frm.copy(),
+                  f"fc_{k}_norm_out_factor": np.full((nAA, 1, 1), 1.0 / math.sqrt(2.0))})
+    # ---- AAA = AA1 x A1 -> invariants, l1 >= l2 >= l3 = L
+    gidx = {g: k for k, g in enumerate(groups)}
+    terms, nout = [], 0
+    for l1 in range(lmax + 1):
+        for l2 in range(l1 + 1):
+            for l3 in range(l2 + 1):
+                if (l3, l1, l2) not in gidx:
+                    continue
+                g = gidx[(l3, l1, l2)]
+                for M in range(-l3, l3 + 1):
+                    terms.append((nout, g_first[g] + M + l3, l3 * (l3 + 1) + M, 1.0 / (2 * l3 + 1)))
+                nout += 1
+    l, r, o, c = _prod_arrays(terms)
+    nAAA = nout
+    s.update(prod_AAA_left_ind=l, prod_AAA_right_ind=r, prod_AAA_m_sum_ind=o, prod_AAA_cg_coeff=c,
+             prod_AAA_n_output_funcs=np.array([nAAA], np.int64), prod_AAA_n_cg_terms=np.array([c.size], np.int64),
+             prod_AAA_lmax=np.array([0], np.int64), prod_AAA_Lmax=np.array([0], np.int64))
+    # ---- AAAA = AA2 x AA2 -> invariants: right group ascending in (l3, l4, L), left group >= right group in
+    # (l1, l2), equal L; linearly dependent invariants dropped (single-channel numerical rank test)
+    nAAAA = 0
+    if order4:
+        rng = np.random.default_rng(seed_indep)
+        nsamp = 400
+        Arand = rng.standard_normal((nsamp, nlm))
+        AAr = np.zeros((nsamp, nAA))
+        pl, pr, po, pc = s["prod_AA_left_ind"], s["prod_AA_right_ind"], s["prod_AA_m_sum_ind"], s["prod_AA_cg_coeff"]
+        np.add.at(AAr, (slice(None), po), pc[None, :] * Arand[:, pl] * Arand[:, pr])
+        order_r = sorted(range(len(groups)), key=lambda g: (groups[g][1], groups[g][2], groups[g][0]))
+        basis = np.zeros((nsamp, 0))
+        terms = []
+        for gr in order_r:
+            L = groups[gr][0]
+            for gl in sorted(range(len(groups)), key=lambda g: (groups[g][1], groups[g][2])):
+                if groups[gl][0] != L or (groups[gl][1], groups[gl][2]) < (groups[gr][1], groups[gr][2]):
+                    continue
+                if lmax <= 4:
+                    if (L, groups[gl][1:], groups[gr][1:]) in _AAAA_SKIP:
+                        continue
+                else:
+                    v = (AAr[:, g_first[gl]:g_first[gl] + 2 * L + 1] *
+                         AAr[:, g_first[gr]:g_first[gr] + 2 * L + 1]).sum(1)
+                    v = v / np.linalg.norm(v)
+                    trial = np.concatenate([basis, v[:, None]], 1)
+                    sv = np.linalg.svd(trial, compute_uv=False)
+                    if sv[-1] < 1e-8 * sv[0]:
+                        continue
+                    basis = trial
+                for M in range(-L, L + 1):
+                    terms.append((nAAAA, g_first[gl] + M + L, g_first[gr] + M + L, 1.0 / (2 * L + 1)))
+                nAAAA += 1
+        l, r, o, c = _prod_arrays(terms)
+        s.update(prod_AAAA_left_ind=l, prod_AAAA_right_ind=r, prod_AAAA_m_sum_ind=o, prod_AAAA_cg_coeff=c,
+                 prod_AAAA_n_output_funcs=np.array([nAAAA], np.int64),
+                 prod_AAAA_n_cg_terms=np.array([c.size], np.int64),
+                 prod_AAAA_lmax=np.array([0], np.int64), prod_AAAA_Lmax=np.array([0], np.int64))
+    # ---- rho reduce: invariants of each source
+    nL0 = sum(1 for g in groups if g[0] == 0)
+
+    def red(src, idx):
+        idx = np.asarray(idx, dtype=np.int32)
+        s[f"rho_collect_ind_{src}"] = idx
+        s[f"rho_w_l_tile_{src}"] = np.arange(idx.size, dtype=np.int32)
+        s[f"rho_total_sum_ind_{src}"] = np.zeros((idx.size, 1), np.int32)
+        s[f"rho_w_shape_{src}"] = np.array([idx.size], np.int64)
+
+    red("A", [0])
+    red("AA", np.arange(nL0))
+    red("AAA", np.arange(nAAA))
+    if order4:
+        red("AAAA", np.arange(nAAAA))
+    s["_groups"] = groups
+    return s
+
+
+def random_model_1l(*, lmax=4, n_elements=1, element_names=("W",), embedding_size=32, nradbase=8, nradmax=32,
+                    fc_width=None, hidden=64, rho_n_out=17, energy_hidden=64, rcut=6.0, radial_basis_p=16,
+                    inv_avg_n_neigh=1.0 / 58.0, order4=True, seed=20260101):
+    """A GRACE-1L-shaped model with weights W ~ N(0, 1) and norm scalars 1/sqrt(n_in) (i.e. N(0, 1/fan_in)),
+    chem_embedding ~ N(0, 1), zero shifts, output_scale 1, SiLU everywhere; returns the dict that `save_model`
+    writes as kokkos.npz."""
+    rng = np.random.default_rng(seed)
+    fc_width = nradmax if fc_width is None else fc_width
+    nl = lmax + 1
+    s = structure_1l(lmax, order4=order4)
+    groups = s.pop("_groups")
+    i64 = lambda v: np.array([v], dtype=np.int64)
+    f64 = lambda v: np.array([v], dtype=np.float64)
+    N = lambda *shape: rng.standard_normal(shape)
+    d = {"grace_model_kind": np.array([b"GRACE-1L"], dtype="|S8"), "grace_format_version": i64(1),
+         "n_elements": i64(n_elements), "element_names": np.array([n.encode() for n in element_names], dtype="|S2"),
+         "embedding_size": i64(embedding_size), "nradbase": i64(nradbase), "rcut": f64(rcut),
+         "radial_basis_p": i64(radial_basis_p), "has_bond_specific_cutoff": i64(0), "lmax": i64(lmax),
+         "nradmax": i64(nradmax), "mlp_rad_has_chem_emb": i64(0), "chem_embedding": N(n_elements, embedding_size)}
+    dims = [nradbase, hidden, hidden, nradmax * nl]
+    for i in range(3):
+        d[f"mlp_rad_W{i}"] = N(dims[i], dims[i + 1])
+        d[f"mlp_rad_norm{i}"] = f64(1.0 / math.sqrt(dims[i]))
+    d["mlp_rad_n_layers"] = i64(3)
+    d["A_inv_avg_n_neigh"] = np.array(inv_avg_n_neigh)
+    d["A_lin_transform_W"] = N(embedding_size, nradmax)
+    d["A_lin_transform_norm"] = f64(1.0 / math.sqrt(embedding_size))
+    ntile_aa = len(groups)
+    for k, n_in_left, ntile in ([("A1", nradmax, nl), ("AA1", fc_width, ntile_aa)] +
+                                ([("AA2", fc_width, ntile_aa)] if order4 else [])):
+        d[f"fc_{k}_w_left"] = N(fc_width, n_in_left, ntile)
+        d[f"fc_{k}_norm_left"] = np.array(1.0 / math.sqrt(n_in_left))
+        d[f"fc_{k}_w_right"] = N(fc_width, nradmax, ntile)
+        d[f"fc_{k}_norm_right"] = np.array(1.0 / math.sqrt(nradmax))
+        d[f"fc_{k}_n_out"] = i64(fc_width)
+        d[f"fc_{k}_left_coefs"] = i64(1)
+    for src, n_in in [("A", nradmax), ("AA", fc_width), ("AAA", fc_width)] + ([("AAAA", fc_width)] if order4 else []):
+        w_shape = int(s[f"rho_w_shape_{src}"][0])
+        d[f"rho_reduce_{src}_W"] = N(n_elements, rho_n_out, n_in, w_shape)
+        d[f"rho_reduce_{src}_norm"] = np.array(1.0 / math.sqrt(n_in))
+        d[f"rho_n_in_{src}"] = i64(n_in)
+    d["rho_n_out"] = i64(rho_n_out)
+    d["rho_is_central_atom_type_dependent"] = i64(1)
+    d["rho_number_of_atom_types"] = i64(n_elements)
+    d["rho_instruction_names"] = np.array([b"A", b"AA", b"AAA"] + ([b"AAAA"] if order4 else []), dtype="|S8")
+    d["energy_mlp_W0"] = N(rho_n_out - 1, energy_hidden)
+    d["energy_mlp_norm0"] = f64(1.0 / math.sqrt(rho_n_out - 1))
+    d["energy_mlp_W1"] = N(energy_hidden, 1)
+    d["energy_mlp_norm1"] = f64(1.0 / math.sqrt(energy_hidden))
+    d["energy_mlp_n_layers"] = i64(2)
+    d["energy_mlp_activation"] = i64(0)
+    d["shift_values"] = np.zeros(n_elements)
+    d.update(s)
+    return d
+
+
+def save_model(path, d):
+    """Uncompressed .npz, as np.savez (the reference loader rejects compressed members)."""
+    np.savez(path, **{k: v for k, v in d.items() if not k.startswith("_")})
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# structures
+# ---------------------------------------------------------------------------------------------------------------
+def _supercell(basis, a, reps):
+    reps = (reps, reps, reps) if np.isscalar(reps) else tuple(reps)
+    basis = np.asarray(basis, dtype=np.float64)
+    g = np.stack(np.meshgrid(np.arange(reps[0]), np.arange(reps[1]), np.arange(reps[2]), indexing="ij"), -1)
+    pos = (g.reshape(-1, 1, 3) + basis[None, :, :]).reshape(-1, 3) * a
+    cell = np.diag([a * reps[0], a * reps[1], a * reps[2]]).astype(np.float64)
+    return pos, cell
+
+
+def bcc_supercell(a, reps):
+    """positions [2 r^3, 3], cell [3, 3] of a cubic bcc supercell."""
+    return _supercell([[0, 0, 0], [0.5, 0.5, 0.5]], a, reps)
+
+
+def fcc_supercell(a, reps):
+    return _supercell([[0, 0, 0], [0.5, 0.5, 0], [0.5, 0, 0.5], [0, 0.5, 0.5]], a, reps)
+
+
+def jitter(pos, sigma, seed):
+    return pos + np.random.default_rng(seed).normal(0.0, sigma, pos.shape)

@@ -1,0 +1,119 @@
+/* C ABI of libgrace_hip.so: GRACE energy + forces + virial on one AMD MI355X (gfx950).
+ *
+ * Plain C types only; every call returns a status and never throws.  The entry points are what a binding of the
+ * reference would call for this path; each comment names the reference interface it stands in for (paths relative
+ * to the reference checkout).
+ *
+ * Threading: a gr_engine is not re-entrant (one call at a time per engine, as the reference's per-driver mutex,
+ * python/src/core.cpp:343-344).  gr_last_error() is thread-local.
+ */
+#ifndef GRACE_HIP_H
+#define GRACE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct gr_model gr_model;
+typedef struct gr_engine gr_engine;
+typedef struct gr_nlist gr_nlist;
+
+enum {
+  GR_OK = 0,
+  GR_INVALID = 1, /* bad argument: the Python layer raises ValueError (nb::value_error / std::invalid_argument) */
+  GR_ERROR = 2,   /* grace::Error / RuntimeError of the reference */
+  GR_NOMEM = 3    /* std::bad_alloc of the reference: the engine stays usable */
+};
+
+enum {
+  GR_FLAG_ENERGY_ONLY = 1, /* ComputeFlags::energy_only (libgrace/include/grace/system.h:118): no forces / virial */
+  GR_FLAG_EATOM = 2        /* ComputeFlags::eflag_atom (system.h:114): per-atom energies */
+};
+
+typedef struct gr_model_info {
+  int layers;     /* 1, 2, 3: GRACE-1L / 2L / 3L */
+  int n_elements;
+  int lmax;
+  int n_radial;   /* radial channels of the first layer */
+  int n_radbase;
+  int max_order;  /* 3 or 4 */
+  double rcut;    /* largest cutoff */
+} gr_model_info;
+
+/* message of the last failed call on this thread ("" if none).  grace::Error::what(). */
+const char *gr_last_error(void);
+/* library ABI version (the Python plug-in contract uses ABI = 7: python/grace_runtime/_gpu.py:18) */
+int gr_abi_version(void);
+/* number of HIP devices; gfx arch name of a device into buf ("" on failure).  _kk.arch(), _kk.initialize(device):
+ * python/kk/kk_api.h:16-27 */
+int gr_device_count(void);
+int gr_device_arch(int device, char *buf, int len);
+
+/* Load a kokkos.npz model (GRACE1LModel::load, libgrace/src/model_1l.cpp:16; kind by grace::model_kind,
+ * libgrace/include/grace/model_kind.h:19).  The same validation errors as the reference loader. */
+int gr_model_load(const char *npz_path, gr_model **out);
+int gr_model_get_info(const gr_model *m, gr_model_info *info);
+/* element name k (0 <= k < n_elements), "" when the file has none: Model.element_names, python/kk/kk_api.h:56 */
+const char *gr_model_element_name(const gr_model *m, int k);
+void gr_model_free(gr_model *m);
+
+/* An engine for one type map: type2mu has ntypes + 1 entries, types are 1-based, type2mu[t] = model element or -1.
+ * Grace1LFused(model, settings, log) + setup_types(ntypes, type2mu): libgrace/include/grace/fused_1l.h:28-31;
+ * Grace1LKK::set_model / setup: libgrace/include/grace/kk/grace_1l_kk.h:72-79.
+ * precision 64: network arithmetic in fp64; 32: fp32 network, fp64 geometry and sums (docs/advanced.md:37-38). */
+int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int precision, int device, gr_engine **out);
+void gr_engine_free(gr_engine *e);
+/* Grace1LFused::cutoff(t1, t2): fused_1l.h:32 */
+double gr_engine_cutoff(const gr_engine *e, int t1, int t2);
+
+/* One call on caller-supplied CSR bonds = _core.Model.compute (python/src/core.cpp:292-396) =
+ * Grace1LFused::compute<CsrBonds>(n, nullptr, n, n, src, out, flags, nthreads) (fused_1l.h:41):
+ * bonds of atom i are [offset[i], offset[i+1]); give rij [nb][3] or (positions [n][3], image [nb], shifts [nimages][3]).
+ * types are 1-based.  Outputs are OVERWRITTEN (not accumulated): energy, forces [n][3], virial[6] = xx yy zz xy xz yz,
+ * eatom [n] (with GR_FLAG_EATOM); null outputs are skipped.  Same argument errors as the reference binding. */
+int gr_compute_csr(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
+                   const double *positions, const int *image, const double *shifts, int64_t nimages, unsigned flags,
+                   double *energy, double *forces, double *virial, double *eatom);
+
+/* The same call in three steps, for callers that keep the structure on the GPU between passes (System.compute
+ * without a list rebuild, python/kk/kk_core.cpp:802-958): upload copies the CSR structure to the device, run
+ * queues one pass on the engine's stream, fetch waits and copies results out. */
+int gr_engine_upload(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
+                     const double *positions, const int *image, const double *shifts, int64_t nimages);
+int gr_engine_run(gr_engine *e, unsigned flags);
+int gr_engine_sync(gr_engine *e);
+int gr_engine_fetch(gr_engine *e, double *energy, double *forces, double *virial, double *eatom);
+/* in-cutoff bonds of the last pass */
+int64_t gr_engine_edge_count(gr_engine *e);
+
+/* Per-stage GPU times (HIP events on the engine's stream) of the last gr_engine_run, when profiling is on.
+ * The reference's counterpart is the G2LF_PROF category table (libgrace/include/grace/fused_cpu.h:171-213). */
+int gr_engine_set_profile(gr_engine *e, int on);
+int gr_engine_stage_count(gr_engine *e);
+int gr_engine_stage_get(gr_engine *e, int k, char *name, int name_len, double *ms, int *launches);
+
+/* Radial functions of the GPU kernel: Rz, dRz [m][lmax+1][n_radial] = R_nl(x) z[mu_j][n] and d/dx, for x = r / rc.
+ * Test hook for the radial-MLP kernel (the reference's counterpart is radial_x.h:29-60 evaluated on the host). */
+int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz);
+
+/* Neighbour list at `cutoff`, the exact list of grace_runtime::neighbor_search (python/src/neighbors.cpp:15-95):
+ * perm [n] (new -> original index), offset [n+1], j [nb] (new indices), image [nb], shifts [nimages][3]. */
+int gr_neighbor_build(int64_t n, const double *positions, const double *cell, const unsigned char *pbc, double cutoff,
+                      int nthreads, gr_nlist **out);
+int64_t gr_nlist_nbonds(const gr_nlist *l);
+int64_t gr_nlist_nimages(const gr_nlist *l);
+int gr_nlist_get(const gr_nlist *l, int64_t *perm, int64_t *offset, int32_t *j, int32_t *image, double *shifts);
+void gr_nlist_free(gr_nlist *l);
+
+/* Energy, forces (caller's atom order), virial of a periodic structure: neighbour list at the engine's largest
+ * cutoff, permutation to bin order, one pass, forces permuted back.  The engine part of GRACERuntimeCalculator.
+ * calculate -> _CpuEngine.compute (python/grace_runtime/calculator.py:204-224) without the Verlet skin. */
+int gr_compute(gr_engine *e, int n, const int *types, const double *positions, const double *cell,
+               const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
