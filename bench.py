@@ -1,0 +1,162 @@
+#!/usr/bin/env python3
+"""Benchmark of the GRACE energy + forces + virial pass on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--precision 64|32] [--no-cpu]
+
+Workload (BASELINE.json configs[1]): GRACE-1L-shaped random-init model (lmax 4, 32 radial channels, 8 Chebyshev
+functions, radial MLP 8-64-64-160, SiLU) on a bcc W 16x16x16 supercell (8192 atoms, a = 3.165 A, N(0, 0.05 A) jitter,
+r_cut 6 A, 475 136 directed edges), fp64.  A step is one full pass (bond filter, radial MLP, A basis, dense chain,
+readout, reverse pass, forces, virial) over the structure, which is uploaded to HBM before the timed region.
+
+Prints one JSON line: the metric (us/atom per call), the roofline of the dominant kernel (duration from HIP events
+on the engine's stream, algorithmic flops/bytes of that stage) and the reference CPU path timed on this host.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+PEAK = {64: 78.6, 32: 157.3}      # dense matrix TFLOP/s of MI355X (fp64, fp32)
+HBM_PEAK = 8000.0                 # GB/s
+
+
+def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops):
+    """Roofline entry of one stage: algorithmic work / measured time."""
+    if name == "radial_mlp":
+        # value + tangent through the 3 layers: 2 * 2 * E * sum n_in n_out
+        fl = 59392.0 * E
+        return {"bound": "mfma", "achieved": fl / (ms * 1e-3) / 1e12, "peak": PEAK[prec], "unit": "TFLOP/s", "work": fl}
+    if name == "scatter_A":
+        by = E * (s * C * nl + 4 + 24) + N * s * C * nlm
+        return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
+    if name == "bond_bwd":
+        by = E * (2 * s * C * nl + 28 + 24) + N * (s * C * nlm + 24)
+        return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
+    if name in dense_flops:
+        fl = dense_flops[name]
+        return {"bound": "mfma", "achieved": fl / (ms * 1e-3) / 1e12, "peak": PEAK[prec], "unit": "TFLOP/s", "work": fl}
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--precision", type=int, default=64, choices=[64, 32])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--reps", type=int, default=16, help="bcc supercell repetitions (16 = the benchmark config)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU (no collectives in the path); run with --gpus 1")
+
+    import torch
+
+    import cases
+    from grace_runtime_amd import kk, synth
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    tmp = tempfile.mkdtemp()
+    mpath = cases.write_model("config1", tmp)
+    pos, cell = synth.bcc_supercell(3.165, a.reps)
+    pos = synth.jitter(pos, 0.05, 2)
+    pbc = [True, True, True]
+    N = len(pos)
+    types = np.ones(N, np.int32)
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 6.0)
+    model = kk.Model(mpath)
+    eng = kk.Engine(model, ["W"], precision=a.precision)
+    eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
+
+    for _ in range(a.warmup):
+        eng.run()
+    eng.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        eng.run()
+    eng.sync()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    out = eng.fetch()
+    E = eng.edge_count()
+
+    # per-stage durations: HIP events around every launch on the engine's stream, averaged over the same K steps
+    eng.set_profile(True)
+    acc = {}
+    for _ in range(a.steps):
+        eng.run()
+        for k, (ms, cnt) in eng.stage_times().items():
+            acc[k] = acc.get(k, 0.0) + ms
+    eng.set_profile(False)
+    stages = {k: v / a.steps for k, v in acc.items()}
+
+    C, nl, nlm, s = 32, 5, 25, a.precision // 8
+    # FC flops (forward: left + right mat-vec per live function; reverse the same), fp64 FMAs on the vector/matrix pipes
+    nA1, nAA1, nAA2 = 25, 44, 141       # informational; exact live counts are the engine's
+    dense_flops = {}
+    roof = {}
+    for k, ms in stages.items():
+        r = stage_model(k, ms, E, N, C, nl, nlm, s, a.precision, dense_flops)
+        if r:
+            r["ms"] = ms
+            r["frac"] = r["achieved"] / r["peak"]
+            roof[k] = r
+    total_ms = sum(stages.values())
+    modelled = {k: v for k, v in roof.items()}
+    dom = max(modelled, key=lambda k: modelled[k]["ms"])
+    d = modelled[dom]
+    roofline = {"kernel": dom, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"],
+                "unit": d["unit"], "frac": round(d["frac"], 4), "traffic": None, "avg_ms": round(d["ms"], 4),
+                "algorithmic_work": d["work"]}
+
+    cpu = None
+    if not a.no_cpu:
+        from oracle import ref_lib      # the compiled reference CPU path: the checker, timed here as the baseline
+        if ref_lib.available():
+            nth = len(os.sched_getaffinity(0))
+            ref = ref_lib.RefModel(mpath, [0])
+            args = dict(positions=pos[perm], image=image, shifts=shifts, nthreads=nth)
+            ref.compute(types[perm], offset, j, **args)
+            ts = []
+            t_end = time.perf_counter() + 20.0
+            while len(ts) < 3 or (time.perf_counter() < t_end and len(ts) < 25):
+                t1 = time.perf_counter()
+                r = ref.compute(types[perm], offset, j, **args)
+                ts.append(time.perf_counter() - t1)
+            tm = float(np.median(ts))
+            cpu = {"value": round(tm / N * 1e6, 4), "unit": "us/atom", "cores": nth, "kind": "reference",
+                   "sample": f"{len(ts)} full calls of the compiled reference Grace1LFused (fp32 + spline tables) on the same "
+                             f"{N}-atom structure, median",
+                   "dE_per_atom_vs_gpu": abs(r["energy"] - out["energy"]) / N,
+                   "max_dF_vs_gpu": float(np.abs(r["forces"] - out["forces"]).max())}
+
+    res = {
+        "metric": "us_per_atom_EFS_call", "value": round(dt / N * 1e6, 5), "unit": "us/atom", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f64" if a.precision == 64 else "f32", "data": "synthetic",
+        "config": {"workload": f"GRACE-1L-shaped random-init model (lmax 4, 32 ch, MLP 8-64-64-160) on bcc W "
+                               f"{a.reps}x{a.reps}x{a.reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[1])",
+                   "atoms": N, "edges": int(E)},
+        "atoms_steps_per_s": round(N / dt, 1),
+        "roofline": roofline,
+        "stages_ms": {k: round(v, 4) for k, v in stages.items()},
+        "stages_roofline": {k: {"bound": v["bound"], "achieved": round(v["achieved"], 2), "unit": v["unit"],
+                                "frac": round(v["frac"], 4)} for k, v in roof.items()},
+        "sum_stage_ms": round(total_ms, 4),
+        "cpu_baseline": cpu,
+        "energy": out["energy"],
+    }
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

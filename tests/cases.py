@@ -1,0 +1,98 @@
+"""Deterministic synthetic test cases (models and structures) shared by the golden-vector generator
+(tests/golden/make_golden.py) and the tests.  Everything derives from fixed numpy Generator seeds."""
+from __future__ import annotations
+
+import os
+
+import numpy as np
+
+from grace_runtime_amd import synth
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLDEN = os.path.join(HERE, "golden")
+REF_FIXTURES = os.path.join(GOLDEN, "ref_fixtures")
+
+
+def model_config1():
+    """GRACE-1L-shaped benchmark model: lmax 4, 32 channels, 8 Chebyshev functions, MLP 8-64-64-160, 1 species."""
+    return synth.random_model_1l(seed=20260101)
+
+
+def model_mix2():
+    """two elements, lmax 3, A width 20 != FC width 40, 10 radial basis functions, with the AAAA stage"""
+    return synth.random_model_1l(lmax=3, n_elements=2, element_names=("Mo", "W"), embedding_size=16, nradbase=10,
+                                 nradmax=20, fc_width=40, hidden=64, rho_n_out=9, energy_hidden=32, rcut=5.0,
+                                 inv_avg_n_neigh=1.0 / 26.0, seed=7)
+
+
+def model_cut2():
+    """two elements with pair-specific cutoffs, lmax 2, max_order 3"""
+    d = synth.random_model_1l(lmax=2, n_elements=2, element_names=("Al", "Ni"), embedding_size=8, nradbase=8,
+                              nradmax=16, hidden=32, rho_n_out=5, energy_hidden=16, rcut=5.5, order4=False,
+                              inv_avg_n_neigh=1.0 / 30.0, seed=11)
+    d["has_bond_specific_cutoff"] = np.array([1], dtype=np.int64)
+    d["bond_cutoff_map"] = np.array([[5.5, 4.75], [4.75, 4.0]])
+    return d
+
+
+MODELS = {"config1": model_config1, "mix2": model_mix2, "cut2": model_cut2}
+
+
+def write_model(name, directory):
+    path = os.path.join(directory, f"{name}.npz")
+    if not os.path.exists(path):
+        synth.save_model(path, MODELS[name]())
+    return path
+
+
+def structure_config1():
+    pos, cell = synth.bcc_supercell(3.165, 4)
+    return synth.jitter(pos, 0.05, 1), cell, np.array([True, True, True]), np.ones(128, np.int32)
+
+
+def structure_config2():
+    pos, cell = synth.bcc_supercell(3.165, 16)
+    return synth.jitter(pos, 0.05, 2), cell, np.array([True, True, True]), np.ones(8192, np.int32)
+
+
+def structure_alloy54(seed=3):
+    pos, cell = synth.bcc_supercell(3.0, 3)
+    rng = np.random.default_rng(seed)
+    types = rng.integers(1, 3, size=len(pos)).astype(np.int32)
+    return synth.jitter(pos, 0.1, seed + 100), cell, np.array([True, True, True]), types
+
+
+def structure_triclinic(seed=5):
+    rng = np.random.default_rng(seed)
+    cell = np.array([[5.5, 0.0, 0.0], [-0.9, 5.2, 0.0], [1.1, -1.3, 6.1]])
+    frac = rng.uniform(-0.5, 1.5, (24, 3))        # also outside the cell: images of the atoms themselves
+    types = rng.integers(1, 3, size=24).astype(np.int32)
+    return frac @ cell, cell, np.array([True, True, True]), types
+
+
+def structure_slab(seed=6):
+    rng = np.random.default_rng(seed)
+    cell = np.diag([9.0, 8.0, 25.0])
+    pos = rng.uniform(0, 1, (40, 3)) * np.array([9.0, 8.0, 7.0])
+    types = rng.integers(1, 3, size=40).astype(np.int32)
+    return pos, cell, np.array([True, True, False]), types
+
+
+def structure_molecule(seed=8):
+    rng = np.random.default_rng(seed)
+    pos = rng.uniform(0, 6, (17, 3))
+    types = rng.integers(1, 3, size=17).astype(np.int32)
+    return pos, np.zeros((3, 3)), np.array([False, False, False]), types
+
+
+STRUCTURES = {"config1": structure_config1, "alloy54": structure_alloy54, "triclinic": structure_triclinic,
+              "slab": structure_slab, "molecule": structure_molecule}
+
+# (model, structure, list cutoff or None for the model cutoff): the end-to-end golden cases
+E2E_CASES = [("config1", "config1", None), ("mix2", "alloy54", 5.5), ("mix2", "triclinic", None),
+             ("cut2", "alloy54", None), ("cut2", "slab", 6.0), ("mix2", "molecule", None)]
+
+
+def bond_vectors(pos, perm, offset, j, image, shifts):
+    x = pos[perm]
+    return x[j] - np.repeat(x, np.diff(offset), axis=0) + (shifts[image] if len(shifts) else 0.0)

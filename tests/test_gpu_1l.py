@@ -1,0 +1,250 @@
+"""Parity of the HIP GRACE-1L path (through the C ABI, grace_runtime_amd.kk -> libgrace_hip.so) with the CPU oracle
+and the golden vectors.  Needs an MI355X: run with -m gpu.
+
+Tolerances.  fp64 engine vs oracle / TF fp64 goldens: the north-star bounds are 1e-6 eV/atom, 1e-5 eV/A,
+1e-6 eV/A^3; the tests hold it to 1e-10 eV/atom, 1e-9 eV/A, 1e-10 eV per atom energy (summation order only).
+fp32 engine and compiled-reference goldens (fp32 + spline tables): the reference's own fp32-vs-fp64 gate,
+1e-6 eV/atom, 2e-5 eV/A, 1e-5 eV per-atom, 1e-5 relative stress (python/tests/test_ref_tf.py:22-23)."""
+import os
+
+import numpy as np
+import pytest
+
+import cases
+from conftest import fixture_cell
+from grace_runtime_amd import kk
+from oracle import grace_oracle as go
+
+pytestmark = pytest.mark.gpu
+
+F64 = {"energy": 1e-10, "forces": 1e-9, "energies": 1e-10, "virial": 1e-9}
+F32 = {"energy": 1e-6, "forces": 2e-5, "energies": 1e-5, "virial": 1e-5}
+
+
+def _check(out, ref, n, tol, vscale=None):
+    assert abs(out["energy"] - ref["energy"]) / n < tol["energy"]
+    assert np.abs(out["forces"] - ref["forces"]).max() < tol["forces"]
+    if "energies" in out and "energies" in ref:
+        assert np.abs(out["energies"] - ref["energies"]).max() < tol["energies"]
+    vs = max(1.0, np.abs(ref["virial"]).max()) if vscale is None else vscale
+    assert np.abs(out["virial"] - ref["virial"]).max() < tol["virial"] * vs
+
+
+@pytest.fixture(scope="module")
+def engines(model_dir):
+    cache = {}
+
+    def get(name, species, precision=64, fixture=False):
+        key = (name, tuple(species), precision)
+        if key not in cache:
+            path = os.path.join(cases.REF_FIXTURES if fixture else model_dir, name + ".npz")
+            cache[key] = kk.Engine(kk.Model(path), species, precision)
+        return cache[key]
+    return get
+
+
+def test_device_is_gfx950():
+    import ctypes as C
+    from grace_runtime_amd import _lib
+    buf = C.create_string_buffer(64)
+    assert _lib.lib().gr_device_count() >= 1
+    assert _lib.lib().gr_device_arch(0, buf, 64) == 0 and buf.value.decode().startswith("gfx950")
+
+
+@pytest.mark.parametrize("precision", [64, 32])
+@pytest.mark.parametrize("name,fixture,species", [("grace_1l_order3", True, ["Mo", "W"]), ("legacy_1l_order3", True, ["Mo", "W"]),
+                                                  ("config1", False, ["W"]), ("mix2", False, ["Mo", "W"])])
+def test_radial_mfma_kernel_matches_oracle(engines, model_dir, name, fixture, species, precision):
+    """R_nl(x) z[mu_j] and d/dx of the MFMA kernel against radial_x.h restated in numpy (also ragged tile counts)"""
+    eng = engines(name, species, precision, fixture)
+    om = go.Model1L(os.path.join(cases.REF_FIXTURES if fixture else model_dir, name + ".npz"))
+    for m in (1, 15, 16, 17, 1000):
+        x = np.linspace(0.02, 0.9995, m) if m > 1 else np.array([0.37])
+        mu = (np.arange(m) * 7) % om.n_elements
+        R, dR = eng.debug_radial(x, mu)
+        Ro, dRo = om.radial(x)
+        z = om.z[mu]
+        Ro, dRo = np.transpose(Ro * z[:, :, None], (0, 2, 1)), np.transpose(dRo * z[:, :, None], (0, 2, 1))
+        tol = 1e-12 if precision == 64 else 2e-6
+        assert np.abs(R - Ro).max() < tol * max(1.0, np.abs(Ro).max())
+        assert np.abs(dR - dRo).max() < tol * max(1.0, np.abs(dRo).max())
+
+
+@pytest.mark.parametrize("precision", [64, 32])
+@pytest.mark.parametrize("cell", ["W54", "WMo54", "W2tri"])
+@pytest.mark.parametrize("name", ["grace_1l_order3", "legacy_1l_order3"])
+def test_matches_tf_fp64_goldens(engines, tf_gold, name, cell, precision):
+    eng = engines(name, ["Mo", "W"], precision, True)
+    types, offset, j, rij, vol = fixture_cell(cell)
+    out = eng.compute(types, offset, j, rij, energies=True)
+    k = f"{name}/{cell}"
+    n = len(types)
+    tol = F64 if precision == 64 else F32
+    assert abs(out["energy"] - tf_gold[k + "/energy"]) / n < max(tol["energy"], 0)
+    assert np.abs(out["forces"] - tf_gold[k + "/forces"]).max() < tol["forces"]
+    assert np.abs(out["energies"] - tf_gold[k + "/energies"]).max() < tol["energies"]
+    stress = go.virial_to_stress(out["virial"], vol)
+    if precision == 64:
+        assert np.abs(stress - tf_gold[k + "/stress"]).max() < 1e-10          # eV/A^3 (north star: 1e-6)
+    else:
+        assert np.abs(stress - tf_gold[k + "/stress"]).max() / np.abs(tf_gold[k + "/stress"]).max() < 1e-5
+
+
+@pytest.mark.parametrize("precision", [64, 32])
+@pytest.mark.parametrize("model,struct,rc", cases.E2E_CASES)
+def test_matches_oracle_and_compiled_reference(engines, model_dir, gold, model, struct, rc, precision):
+    om = go.Model1L(os.path.join(model_dir, model + ".npz"))
+    species = om.names
+    eng = engines(model, species, precision)
+    pos, cell, pbc, types = cases.STRUCTURES[struct]()
+    types = np.minimum(types, om.n_elements).astype(np.int32)
+    tag = f"e2e/{model}/{struct}"
+    rcl = float(gold[tag + "/rc_list"])
+    pcell, shift = kk._padded_cell_arrays(cell, pos, rcl, pbc)
+    perm, offset, j, image, shifts = kk.neighbor_search(pos + shift, pcell, pbc, rcl)
+    n = len(types)
+    # positions + image + shifts path, and the rij path: same bits in, same results
+    out = eng.compute(types[perm], offset, j, energies=True, positions=pos[perm], image=image, shifts=shifts)
+    rij = cases.bond_vectors(pos, perm, offset, j, image, shifts)
+    out2 = eng.compute(types[perm], offset, j, rij, energies=True)
+    assert abs(out["energy"] - out2["energy"]) < 1e-9 and np.abs(out["forces"] - out2["forces"]).max() < 1e-9
+    ref = go.compute_1l(om, types[perm] - 1, offset, j, rij)
+    _check(out, ref, n, F64 if precision == 64 else F32)
+    # the compiled reference (fp32 + spline tables) on the same list
+    g = {k: gold[f"{tag}/{k}"] for k in ("energy", "energies", "forces", "virial")}
+    _check(out, g, n, F32)
+    assert np.abs(out["forces"].sum(0)).max() < 1e-9
+
+
+def test_config2_size_properties(engines):
+    """the benchmark structure (8192 atoms, ~475 k edges): size-independent properties at full size"""
+    eng = engines("config1", ["W"], 64)
+    pos, cell, pbc, types = cases.structure_config2()
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 6.0)
+    out = eng.compute(types[perm], offset, j, energies=True, positions=pos[perm], image=image, shifts=shifts)
+    assert eng.edge_count() == len(j) == 475136
+    assert abs(out["energies"].sum() - out["energy"]) < 1e-8                      # checksum of per-atom energies
+    assert np.abs(out["forces"].sum(0)).max() < 1e-9                               # Newton's third law
+    # translation of all atoms and a relabelling of the atoms leave E and (permuted) F unchanged
+    p2 = pos + np.array([0.37, -1.21, 2.5])
+    perm2, offset2, j2, image2, shifts2 = kk.neighbor_search(p2, cell, pbc, 6.0)
+    out2 = eng.compute(types[perm2], offset2, j2, positions=p2[perm2], image=image2, shifts=shifts2)
+    f1, f2 = np.empty_like(pos), np.empty_like(pos)
+    f1[perm], f2[perm2] = out["forces"], out2["forces"]
+    assert abs(out["energy"] - out2["energy"]) < 1e-8 and np.abs(f1 - f2).max() < 1e-9
+    # a list with a 0.5 A skin filtered on the device gives the same result as the exact list
+    perm3, offset3, j3, image3, shifts3 = kk.neighbor_search(pos, cell, pbc, 6.5)
+    out3 = eng.compute(types[perm3], offset3, j3, positions=pos[perm3], image=image3, shifts=shifts3)
+    f3 = np.empty_like(pos)
+    f3[perm3] = out3["forces"]
+    assert eng.edge_count() == 475136 and len(j3) > len(j)
+    assert abs(out["energy"] - out3["energy"]) < 1e-8 and np.abs(f1 - f3).max() < 1e-9
+    assert np.abs(out["virial"] - out3["virial"]).max() < 1e-8
+    # a sample of atoms against the oracle on their own neighbourhoods is covered at config-1 size; here compare the
+    # two precisions with each other
+    eng32 = engines("config1", ["W"], 32)
+    o32 = eng32.compute(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
+    assert abs(o32["energy"] - out["energy"]) / len(pos) < 1e-6 and np.abs(o32["forces"] - out["forces"]).max() < 2e-5
+
+
+def test_finite_differences_on_gpu(engines):
+    eng = engines("mix2", ["Mo", "W"], 64)
+    pos, cell, pbc, types = cases.structure_triclinic()
+    sysm = kk.System(eng.model, ["Mo", "W"], skin=0.0)
+
+    def energy(p):
+        return sysm.compute(types, p, cell, pbc, energy_only=True)["energy"]
+    r = sysm.compute(types, pos, cell, pbc)
+    h = 1e-5
+    for a, d in [(0, 0), (5, 1), (9, 2)]:
+        p1, p2 = pos.copy(), pos.copy()
+        p1[a, d] += h
+        p2[a, d] -= h
+        assert abs(-(energy(p1) - energy(p2)) / (2 * h) - r["forces"][a, d]) < 1e-7
+
+
+def test_edge_cases(engines):
+    eng = engines("mix2", ["Mo", "W"], 64)
+    om = eng.model
+    # empty structure
+    out = eng.compute(np.zeros(0, np.int32), np.zeros(1, np.int64), np.zeros(0, np.int32), np.zeros((0, 3)))
+    assert out["energy"] == 0.0 and out["forces"].shape == (0, 3)
+    # isolated atoms: E = shift, F = 0 (tests/test_driver.cpp:432-440 of the reference)
+    out = eng.compute(np.array([1, 2], np.int32), np.zeros(3, np.int64), np.zeros(0, np.int32), np.zeros((0, 3)), energies=True)
+    assert abs(out["energy"]) < 1e-14 and np.all(out["forces"] == 0) and np.all(out["virial"] == 0)
+    # ragged rows: atoms without bonds between atoms with bonds; bonds beyond the cutoff are dropped
+    types = np.array([1, 2, 1, 2], np.int32)
+    offset = np.array([0, 2, 2, 3, 3], np.int64)
+    j = np.array([2, 1, 0], np.int32)
+    rij = np.array([[1.5, 0.3, -0.2], [9.0, 0, 0], [-1.5, -0.3, 0.2]])
+    out = eng.compute(types, offset, j, rij, energies=True)
+    assert eng.edge_count() == 2
+    ref = go.compute_1l(go.Model1L(om.path), types - 1, offset, j, rij)
+    _check(out, ref, 4, F64)
+    assert out["forces"][1].tolist() == [0, 0, 0] and out["forces"][3].tolist() == [0, 0, 0]
+    # energy_only: no forces, same energy
+    eo = eng.compute(types, offset, j, rij, energy_only=True)
+    assert abs(eo["energy"] - out["energy"]) < 1e-12 and "forces" not in eo
+    # a bond of length zero is an error, and the engine works afterwards (bonds.h:49-62 of the reference)
+    with pytest.raises(RuntimeError, match="two atoms at the same position"):
+        eng.compute(np.array([1, 1], np.int32), np.array([0, 1, 2], np.int64), np.array([1, 0], np.int32), np.zeros((2, 3)))
+    again = eng.compute(types, offset, j, rij)
+    assert abs(again["energy"] - out["energy"]) < 1e-12
+
+
+def test_argument_errors(engines):
+    eng = engines("mix2", ["Mo", "W"], 64)
+    t, o, j, r = np.array([1, 2], np.int32), np.array([0, 1, 2], np.int64), np.array([1, 0], np.int32), np.array([[1.0, 0, 0], [-1.0, 0, 0]])
+    with pytest.raises(ValueError, match="types must be 1"):
+        eng.compute(np.array([0, 2], np.int32), o, j, r)
+    with pytest.raises(ValueError, match="types must be 1"):
+        eng.compute(np.array([1, 3], np.int32), o, j, r)
+    with pytest.raises(ValueError, match="offset must have"):
+        eng.compute(t, o[:2], j, r)
+    with pytest.raises(ValueError, match="j must index"):
+        eng.compute(t, o, np.array([1, 5], np.int32), r)
+    with pytest.raises(ValueError, match="give rij or positions"):
+        eng.compute(t, o, j)
+    with pytest.raises(ValueError, match="give rij or positions"):
+        eng.compute(t, o, j, r, positions=np.zeros((2, 3)), image=np.zeros(2, np.int32), shifts=np.zeros((1, 3)))
+    with pytest.raises(ValueError, match="image must index"):
+        eng.compute(t, o, j, positions=np.zeros((2, 3)), image=np.array([0, 4], np.int32), shifts=np.zeros((1, 3)))
+    with pytest.raises(ValueError, match="not in the model"):
+        kk.Engine(eng.model, ["W", "Fe"])
+    # species in another order than the model's elements: types follow the species list
+    e2 = kk.Engine(eng.model, ["W", "Mo"])
+    a = eng.compute(t, o, j, r)
+    b = e2.compute(np.array([2, 1], np.int32), o, j, r)
+    assert abs(a["energy"] - b["energy"]) < 1e-13 and np.abs(a["forces"] - b["forces"]).max() < 1e-13
+
+
+def test_system_verlet_list_and_batch(engines):
+    eng = engines("mix2", ["Mo", "W"], 64)
+    pos, cell, pbc, types = cases.structure_alloy54()
+    s = kk.System(eng.model, ["Mo", "W"], skin=0.5)
+    r0 = s.compute(types, pos, cell, pbc, energies=True)
+    rng = np.random.default_rng(0)
+    p1 = pos + rng.uniform(-0.1, 0.1, pos.shape)      # below skin / 2: the list is kept
+    r1 = s.compute(types, p1, cell, pbc)
+    assert s.rebuilds == 1
+    s2 = kk.System(eng.model, ["Mo", "W"], skin=0.0)
+    r1x = s2.compute(types, p1, cell, pbc)
+    assert abs(r1["energy"] - r1x["energy"]) < 1e-10 and np.abs(r1["forces"] - r1x["forces"]).max() < 1e-10
+    p2 = p1.copy()
+    p2[3] += 0.4                                          # above skin / 2: rebuilt
+    s.compute(types, p2, cell, pbc)
+    assert s.rebuilds == 2
+    # batch of three structures = the structures one by one
+    structs = [cases.structure_alloy54(), cases.structure_triclinic(), cases.structure_slab()]
+    natoms = [len(x[0]) for x in structs]
+    b = kk.Batch(eng.model, ["Mo", "W"])
+    out = b.compute(natoms, np.concatenate([x[3] for x in structs]), np.concatenate([x[0] for x in structs]),
+                    np.stack([x[1] for x in structs]), np.stack([x[2] for x in structs]), energies=True)
+    lo = 0
+    for k, (p, c, pb, t) in enumerate(structs):
+        one = kk.System(eng.model, ["Mo", "W"], skin=0.0).compute(t, p, c, pb, energies=True)
+        assert abs(out["energy"][k] - one["energy"]) < 1e-10
+        assert np.abs(out["forces"][lo:lo + len(p)] - one["forces"]).max() < 1e-10
+        assert np.abs(out["virial"][k] - one["virial"]).max() < 1e-9
+        lo += len(p)
+    assert abs(r0["energies"].sum() - r0["energy"]) < 1e-10

@@ -1,0 +1,170 @@
+"""Host side of libgrace_hip.so without a GPU: the library loads and exports exactly the symbols the header declares,
+the model loader accepts the reference's fixture files and rejects malformed ones the way the reference loader does
+(libgrace/src/model_1l.cpp, tests/test_model_shapes.cpp of the reference), and the neighbour list equals the reference
+list (tests/golden/reference_outputs.npz, written by the compiled reference) and a brute-force O(N^2) search."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import cases
+from grace_runtime_amd import _lib, kk, synth
+
+
+def test_header_symbols_are_exported():
+    hdr = open(os.path.join(os.path.dirname(cases.HERE), "include", "grace_hip.h")).read()
+    declared = set(re.findall(r"\b(gr_[a-z_0-9]+)\s*\(", hdr))
+    assert declared == set(_lib.SYMBOLS)
+    L = _lib.lib()
+    for s in declared:
+        assert getattr(L, s) is not None
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], capture_output=True, text=True).stdout
+    exported = set(re.findall(r"\bT (gr_[a-z_0-9]+)", out))
+    assert declared <= exported
+    assert L.gr_abi_version() == 7 == kk.ABI
+
+
+def test_product_does_not_touch_the_oracle():
+    root = os.path.dirname(cases.HERE)
+    for dp, _, files in os.walk(os.path.join(root, "grace_runtime_amd")):
+        for f in files:
+            if f.endswith((".py", ".hpp", ".cpp", ".hip", ".h")):
+                txt = open(os.path.join(dp, f)).read()
+                assert "import oracle" not in txt and "from oracle" not in txt and "oracle/" not in txt, f
+
+
+@pytest.mark.parametrize("name,lmax,C_,order", [("grace_1l_order3", 2, 16, 3), ("legacy_1l_order3", 2, 16, 3)])
+def test_loads_reference_fixture_models(name, lmax, C_, order):
+    m = kk.Model(os.path.join(cases.REF_FIXTURES, name + ".npz"))
+    assert (m.layers, m.lmax, m.n_radial, m.max_order, m.element_names) == (1, lmax, C_, order, ["Mo", "W"])
+    assert m.rcut == 5.0
+    with pytest.raises(ValueError):
+        m.type2mu(["W", "Xx"])
+    assert list(m.type2mu(["W", "Mo"])) == [-1, 1, 0]
+
+
+def test_rejects_other_model_kinds_and_missing_files(tmp_path):
+    with pytest.raises(ValueError, match="GRACE-2L"):
+        kk.Model(os.path.join(cases.REF_FIXTURES, "grace_2l_order3.npz"))
+    with pytest.raises(RuntimeError, match="cannot read the model file"):
+        kk.Model(str(tmp_path / "nope.npz"))
+    p = tmp_path / "junk.npz"
+    p.write_bytes(b"not a zip archive at all, just forty-odd bytes of text")
+    with pytest.raises(RuntimeError, match="cannot read the model file"):
+        kk.Model(str(p))
+
+
+def _mutated(tmp_path, fn):
+    d = cases.model_cut2()
+    fn(d)
+    p = str(tmp_path / "m.npz")
+    np.savez(p, **d)
+    return p
+
+
+BAD = [
+    (lambda d: d.pop("chem_embedding"), "required weight 'chem_embedding' missing"),
+    (lambda d: d.update(mlp_rad_W1=d["mlp_rad_W1"][:, :-1]), "mlp_rad_W2"),
+    (lambda d: d.update(prod_AA_left_ind=d["prod_AA_left_ind"] + 100), "prod_AA_left_ind' has"),
+    (lambda d: d.update(fc_A1_w_tile_left=d["fc_A1_w_tile_left"][:-1]), "fc_A1_w_tile_left' has 8 values, expected 9"),
+    (lambda d: d.update(rho_reduce_AA_W=d["rho_reduce_AA_W"][:, :, :, :1]), "rho_reduce_AA_W' has shape"),
+    (lambda d: d.update(A_lin_transform_W=np.asfortranarray(d["A_lin_transform_W"])), "Fortran order"),
+    (lambda d: d.update(mlp_rad_W0=np.where(np.arange(d["mlp_rad_W0"].size).reshape(d["mlp_rad_W0"].shape) == 3, np.nan, d["mlp_rad_W0"])), "non-finite"),
+    (lambda d: d.update(lmax=np.array([300])), "lmax' is 300"),
+    (lambda d: d.update(rcut=np.array([-1.0])), "cutoff"),
+    (lambda d: d.update(fc_A1_left_coefs=np.array([0])), "fc_A1_left_coefs"),
+    (lambda d: d.update(grace_model_kind=np.array([b"GRACE-9L"], dtype="|S8")), "grace_model_kind"),
+    (lambda d: d.update(prod_AAAA_left_ind=np.zeros(1, np.int32)), "AAAA stage is incomplete"),
+    (lambda d: d.update(energy_mlp_W1=d["energy_mlp_W1"].astype("U")), "unsupported dtype"),
+]
+
+
+@pytest.mark.parametrize("k", range(len(BAD)))
+def test_malformed_models_are_rejected(tmp_path, k):
+    fn, msg = BAD[k]
+    with pytest.raises((RuntimeError, ValueError), match=re.escape(msg)):
+        kk.Model(_mutated(tmp_path, fn))
+
+
+def test_compressed_archive_is_rejected(tmp_path):
+    p = str(tmp_path / "c.npz")
+    np.savez_compressed(p, **cases.model_cut2())
+    with pytest.raises(RuntimeError, match="compressed"):
+        kk.Model(p)
+
+
+def test_float32_and_integer_arrays_are_read_by_value(tmp_path):
+    def fn(d):
+        d["rcut"] = np.array([5], dtype=np.int32)                  # integer scalar where a float is expected
+        d["chem_embedding"] = d["chem_embedding"].astype(np.float32)
+        d["prod_AA_left_ind"] = d["prod_AA_left_ind"].astype(np.int64)
+    m = kk.Model(_mutated(tmp_path, fn))
+    assert m.rcut == 5.5        # bond_cutoff_map present: its maximum
+
+
+def _brute(pos, cell, pbc, rc):
+    n = len(pos)
+    rng = [range(-3, 4) if p else range(0, 1) for p in pbc]
+    s = set()
+    for a in range(n):
+        for b in range(n):
+            for s0 in rng[0]:
+                for s1 in rng[1]:
+                    for s2 in rng[2]:
+                        if a == b and (s0, s1, s2) == (0, 0, 0):
+                            continue
+                        d = pos[b] - pos[a] + s0 * cell[0] + s1 * cell[1] + s2 * cell[2]
+                        if d @ d < rc * rc:
+                            s.add((a, b, tuple(np.round(d, 9))))
+    return s
+
+
+@pytest.mark.parametrize("struct,rc", [("triclinic", 5.0), ("slab", 6.0), ("molecule", 5.0)])
+def test_neighbor_list_matches_brute_force(struct, rc):
+    pos, cell, pbc, _ = cases.STRUCTURES[struct]()
+    pcell, shift = kk._padded_cell_arrays(cell, pos, rc, pbc)
+    perm, offset, j, image, shifts = kk.neighbor_search(pos + shift, pcell, pbc, rc)
+    rij = cases.bond_vectors(pos, perm, offset, j, image, shifts)
+    i = np.repeat(np.arange(len(pos)), np.diff(offset))
+    got = {(int(perm[a]), int(perm[b]), tuple(np.round(d, 9))) for a, b, d in zip(i, j, rij)}
+    assert len(got) == len(j)
+    assert got == _brute(pos, pcell, pbc, rc)
+
+
+def test_neighbor_list_equals_reference_list(gold):
+    keys = sorted({k.split("/")[1] for k in gold if k.startswith("nl/")})
+    assert len(keys) >= 5
+    for key in keys:
+        struct, rc = key.split("@")
+        rc = float(rc)
+        pos, cell, pbc, _ = cases.STRUCTURES[struct]()
+        pcell, shift = kk._padded_cell_arrays(cell, pos, rc, pbc)
+        perm, offset, j, image, shifts = kk.neighbor_search(pos + shift, pcell, pbc, rc, num_threads=3)
+        for name, got in (("perm", perm), ("offset", offset), ("j", j), ("image", image)):
+            assert np.array_equal(got, gold[f"nl/{key}/{name}"]), (key, name)      # bit-exact, order included
+        ref = gold[f"nl/{key}/shifts"]
+        # the shift vectors S cell: equal up to the reference's own FMA contraction (its build uses -march=native)
+        assert shifts.shape == ref.shape and np.abs(shifts - ref).max() <= 4e-16 * max(1.0, np.abs(ref).max())
+
+
+def test_neighbor_list_thread_count_independent():
+    pos, cell, pbc, _ = cases.structure_config1()
+    a = kk.neighbor_search(pos, cell, pbc, 6.0, num_threads=1)
+    b = kk.neighbor_search(pos, cell, pbc, 6.0, num_threads=8)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+    assert len(a[2]) == 7424
+
+
+def test_neighbor_list_argument_errors():
+    pos = np.zeros((2, 3))
+    with pytest.raises(ValueError, match="cutoff must be positive"):
+        kk.neighbor_search(pos, np.eye(3), [1, 1, 1], 0.0)
+    with pytest.raises(ValueError, match="full-rank"):
+        kk.neighbor_search(pos, np.zeros((3, 3)), [1, 1, 1], 3.0)
+    with pytest.raises(ValueError, match="finite"):
+        kk.neighbor_search(np.full((2, 3), np.nan), np.eye(3) * 5, [1, 1, 1], 3.0)
+    perm, offset, j, image, shifts = kk.neighbor_search(np.zeros((0, 3)), np.eye(3) * 5, [1, 1, 1], 3.0)
+    assert offset.tolist() == [0] and j.size == 0
