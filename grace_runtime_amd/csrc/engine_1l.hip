@@ -120,71 +120,101 @@ struct DevProd {
   }
 };
 
-template<class T> struct DevFc {
-  DevBuf Wl, Wr, WlT, WrT, tile_l, nof, live, conn_off, conn_from, conn_tile, rlive, rconn_off, rconn_to, rconn_tile;
-  FcDev<T> d{};
-  // nfr: functions of the right-input tensor
-  void build(const FCWeights &w, const std::vector<char> &livef, int nfr)
+// weights W[K][N] (row-major) of a tile GEMM in MFMA fragment order [cb][s][lane]: lane (g, c) holds
+// W[g * (K / 4) + s][cb * 16 + c]
+template<class T> void pack_fragments(const std::vector<double> &W, int K, int N, int Kp, int Np, std::vector<T> &out)
+{
+  const int ks = Kp / 4, nb = Np / 16;
+  const size_t base = out.size();
+  out.resize(base + (size_t) nb * ks * 64, (T) 0);
+  for (int cb = 0; cb < nb; cb++)
+    for (int s = 0; s < ks; s++)
+      for (int lane = 0; lane < 64; lane++) {
+        const int g = lane >> 4, c = lane & 15, k = g * ks + s, n = cb * 16 + c;
+        if (k < K && n < N) out[base + ((size_t) cb * ks + s) * 64 + lane] = (T) W[(size_t) k * N + n];
+      }
+}
+
+template<class T> struct DevJobs {
+  DevBuf job_out, job_scale, seg_off, seg_src, seg_fn, seg_w, seg_scale;
+  GemmJobs<T> d{};
+  struct Host {
+    std::vector<int> job_out, seg_off{0}, seg_src, seg_fn, seg_w;
+    std::vector<T> job_scale, seg_scale;
+    void job(int out, double scale) { job_out.push_back(out); job_scale.push_back((T) scale); }
+    void seg(int src, int fn, int w, double scale) { seg_src.push_back(src); seg_fn.push_back(fn); seg_w.push_back(w); seg_scale.push_back((T) scale); }
+    void end_job() { seg_off.push_back((int) seg_src.size()); }
+  };
+  void build(const Host &h, const T *WF0, const T *WF1)
   {
-    const int nt = w.tiles_left, no = w.n_out, nil = w.n_in_left, nir = w.n_in_right;
-    auto pack = [&](const std::vector<double> &W, double norm, int nin, std::vector<T> &Wo, std::vector<T> &WT) {
-      Wo.assign((size_t) nt * nin * no, (T) 0);
-      WT.assign((size_t) nt * no * nin, (T) 0);
-      for (int k = 0; k < no; k++)
-        for (int n = 0; n < nin; n++)
-          for (int t = 0; t < nt; t++) {
-            const T v = (T) (norm * W[((size_t) k * nin + n) * nt + t]);
-            Wo[((size_t) t * nin + n) * no + k] = v;
-            WT[((size_t) t * no + k) * nin + n] = v;
-          }
+    upload_vec(job_out, h.job_out); upload_vec(job_scale, h.job_scale); upload_vec(seg_off, h.seg_off);
+    upload_vec(seg_src, h.seg_src); upload_vec(seg_fn, h.seg_fn); upload_vec(seg_w, h.seg_w); upload_vec(seg_scale, h.seg_scale);
+    d.job_out = job_out.as<int>(); d.job_scale = job_scale.as<T>(); d.seg_off = seg_off.as<int>();
+    d.seg_src = seg_src.as<int>(); d.seg_fn = seg_fn.as<int>(); d.seg_w = seg_w.as<int>(); d.seg_scale = seg_scale.as<T>();
+    d.WF0 = WF0; d.WF1 = WF1;
+    d.njobs = (int) h.job_out.size();
+  }
+  void set_rows(const int *drow) { for (int q = 0; q < 16; q++) d.drow[q] = drow[q]; }
+};
+
+// One FC layer as three job lists (forward, reverse into the left input, reverse into the right input) over
+// fragment-ordered weight tiles.  Widths are the padded ones (multiples of 16; padding weights are zero).
+template<class T> struct DevFc {
+  DevBuf WlF, WrF, WlTF, WrTF;
+  DevJobs<T> fwd, bwd_l, bwd_r;
+  int nil = 0, nir = 0, no = 0;    // padded widths
+  // nfr: functions of the right-input tensor; livef: outputs that are computed
+  void build(const FCWeights &w, const std::vector<char> &livef, int nfr, int nil_p, int nir_p, int no_p, const int *drow)
+  {
+    nil = nil_p; nir = nir_p; no = no_p;
+    const int nt = w.tiles_left;
+    std::vector<T> fl, fr, flt, frt;
+    std::vector<double> M, Mt;
+    auto tile_mats = [&](const std::vector<double> &W, double norm, int nin, int t) {
+      M.assign((size_t) nin * w.n_out, 0.0);     // [n][k]
+      Mt.assign((size_t) w.n_out * nin, 0.0);    // [k][n]
+      for (int k = 0; k < w.n_out; k++)
+        for (int n = 0; n < nin; n++) {
+          const double v = norm * W[((size_t) k * nin + n) * nt + t];
+          M[(size_t) n * w.n_out + k] = v;
+          Mt[(size_t) k * nin + n] = v;
+        }
     };
-    std::vector<T> a, b;
-    pack(w.w_left, w.norm_left, nil, a, b);
-    upload_vec(Wl, a); upload_vec(WlT, b);
-    pack(w.w_right, w.norm_right, nir, a, b);
-    upload_vec(Wr, a); upload_vec(WrT, b);
-    std::vector<T> nf(w.n_funcs);
-    for (int f = 0; f < w.n_funcs; f++) nf[f] = (T) w.norm_out_factor[f];
-    upload_vec(nof, nf);
-    upload_vec(tile_l, w.w_tile_left);
-    std::vector<int> lv;
-    for (int f = 0; f < w.n_funcs; f++)
-      if (livef[f]) lv.push_back(f);
-    upload_vec(live, lv);
-    // right connections by output function, and (live outputs only) by right-input function
-    std::vector<int> ord(w.n_conn);
-    std::iota(ord.begin(), ord.end(), 0);
-    std::stable_sort(ord.begin(), ord.end(), [&](int x, int y) { return w.collect_to[x] < w.collect_to[y]; });
-    std::vector<int> coff(w.n_funcs + 1, 0), cfrom, ctile;
-    for (int c : ord) {
-      cfrom.push_back(w.collect_from[c]);
-      ctile.push_back(w.w_tile_right[c]);
-      coff[w.collect_to[c] + 1]++;
+    for (int t = 0; t < nt; t++) {
+      tile_mats(w.w_left, w.norm_left, w.n_in_left, t);
+      pack_fragments<T>(M, w.n_in_left, w.n_out, nil, no, fl);
+      pack_fragments<T>(Mt, w.n_out, w.n_in_left, no, nil, flt);
+      tile_mats(w.w_right, w.norm_right, w.n_in_right, t);
+      pack_fragments<T>(M, w.n_in_right, w.n_out, nir, no, fr);
+      pack_fragments<T>(Mt, w.n_out, w.n_in_right, no, nir, frt);
     }
-    for (int f = 0; f < w.n_funcs; f++) coff[f + 1] += coff[f];
-    upload_vec(conn_off, coff); upload_vec(conn_from, cfrom); upload_vec(conn_tile, ctile);
-    std::vector<int> ord2;
-    for (int c = 0; c < w.n_conn; c++)
-      if (livef[w.collect_to[c]]) ord2.push_back(c);
-    std::stable_sort(ord2.begin(), ord2.end(), [&](int x, int y) { return w.collect_from[x] < w.collect_from[y]; });
-    std::vector<int> roff(nfr + 1, 0), rto, rtile, rl;
-    for (int c : ord2) {
-      rto.push_back(w.collect_to[c]);
-      rtile.push_back(w.w_tile_right[c]);
-      roff[w.collect_from[c] + 1]++;
+    upload_vec(WlF, fl); upload_vec(WrF, fr); upload_vec(WlTF, flt); upload_vec(WrTF, frt);
+    typename DevJobs<T>::Host hf, hl, hr;
+    std::vector<std::vector<int>> conn_of(w.n_funcs), conn_from(nfr);
+    for (int c = 0; c < w.n_conn; c++) {
+      conn_of[w.collect_to[c]].push_back(c);
+      if (livef[w.collect_to[c]]) conn_from[w.collect_from[c]].push_back(c);
     }
-    for (int f = 0; f < nfr; f++) {
-      if (roff[f + 1] > 0) rl.push_back(f);
-      roff[f + 1] += roff[f];
+    for (int f = 0; f < w.n_funcs; f++) {
+      if (!livef[f]) continue;
+      hf.job(f, w.norm_out_factor[f]);
+      hf.seg(0, f, w.w_tile_left[f], 1.0);
+      for (int c : conn_of[f]) hf.seg(1, w.collect_from[c], w.w_tile_right[c], 1.0);
+      hf.end_job();
+      hl.job(f, w.norm_out_factor[f]);
+      hl.seg(0, f, w.w_tile_left[f], 1.0);
+      hl.end_job();
     }
-    upload_vec(rconn_off, roff); upload_vec(rconn_to, rto); upload_vec(rconn_tile, rtile); upload_vec(rlive, rl);
-    d.Wl = Wl.as<T>(); d.Wr = Wr.as<T>(); d.WlT = WlT.as<T>(); d.WrT = WrT.as<T>();
-    d.tile_l = tile_l.as<int>(); d.nof = nof.as<T>(); d.live = live.as<int>();
-    d.conn_off = conn_off.as<int>(); d.conn_from = conn_from.as<int>(); d.conn_tile = conn_tile.as<int>();
-    d.rlive = rlive.as<int>(); d.rconn_off = rconn_off.as<int>(); d.rconn_to = rconn_to.as<int>();
-    d.rconn_tile = rconn_tile.as<int>();
-    d.nf = w.n_funcs; d.nfr = nfr; d.nlive = (int) lv.size(); d.nrlive = (int) rl.size();
-    d.n_in_l = nil; d.n_in_r = nir; d.n_out = no;
+    for (int r = 0; r < nfr; r++) {
+      if (conn_from[r].empty()) continue;
+      hr.job(r, 1.0);
+      for (int c : conn_from[r]) hr.seg(0, w.collect_to[c], w.w_tile_right[c], w.norm_out_factor[w.collect_to[c]]);
+      hr.end_job();
+    }
+    fwd.build(hf, WlF.as<T>(), WrF.as<T>());
+    bwd_l.build(hl, WlTF.as<T>(), WlTF.as<T>());
+    bwd_r.build(hr, WrTF.as<T>(), WrTF.as<T>());
+    fwd.set_rows(drow); bwd_l.set_rows(drow); bwd_r.set_rows(drow);
   }
 };
 
@@ -253,6 +283,7 @@ template<class T> class Engine1L final : public Engine {
   std::vector<StageTime> times_;
 
   // model dimensions
+  int CP_ = 0, CFP_ = 0;    // channel widths padded to 16 / 32 / 64: the widths of every per-atom tensor on the device
   int lmax_ = 0, nl_ = 0, nlm_ = 0, C_ = 0, CF_ = 0, nAA_ = 0, nAAA_ = 0, nAAAA_ = 0, nrho_ = 0, nel_ = 0;
   bool order4_ = true, aaa_a_ = false;
   int hb_ = 4, ks0_ = 2, nob_ = 0, noutp_ = 0, w2_in_lds_ = 1;
@@ -264,7 +295,7 @@ template<class T> class Engine1L final : public Engine {
   DevBuf cut_, z_, w0_, w1_, w2_, shift_;
   DevFc<T> fcA1_, fcAA1_, fcAA2_;
   DevProd pAA_, pAAA_, pAAAA_;
-  DevBuf redW_[4], redFn_[4];
+  DevBuf redWF_[4], redWB_[4], redFn_[4];
   ReduceDev<T> red_{};
   DevBuf eW_[7];
   EnergyDev en_{};
@@ -273,7 +304,8 @@ template<class T> class Engine1L final : public Engine {
   int n_ = 0;
   int64_t nb_ = 0;
   bool have_rij_ = false;
-  DevBuf mu_, offset_, j_, rij_, x_, image_, shifts_;
+  DevBuf mu_, offset_, j_, rij_, x_, image_, shifts_, tiles_;
+  int ntiles_ = 0;
   // pass buffers
   DevBuf count_, eoff_, zero_, ei_, ej_, emu_, rh_, r_, xr_, rc_, Rz_, dRz_;
   DevBuf A_, A1_, AA_, AA1_, AA2_, AAA_, AAAA_, gA_, gA1_, gAA_, gAA1_, gAA2_, gAAA_, gAAAA_, rho_, grho_;
@@ -291,6 +323,7 @@ template<class T> class Engine1L final : public Engine {
     HIP_CHECK(hipGetLastError());
     prof_end();
   }
+  void launch_gemm(DevJobs<T> &J, int kb0, int kb1, int nb, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo, int accumulate);
   void launch_radial(long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
                      const long long *n_edges);
 };
@@ -389,7 +422,11 @@ template<class T> void Engine1L<T>::build()
   aaa_a_ = m.AAA_right_A;
   nrho_ = m.rho_n_out;
   if (nrho_ > 32) throw Error("GRACE-1L: rho_n_out > 32 not supported by the GPU reduce kernels");
-  if (nl_ * C_ > 1024 || CF_ > 256 || C_ > 256) throw Error("GRACE-1L: channel widths beyond the GPU kernels' limits");
+  auto pad_width = [](int c) { return c <= 16 ? 16 : c <= 32 ? 32 : c <= 64 ? 64 : -1; };
+  CP_ = pad_width(C_);
+  CFP_ = pad_width(CF_);
+  // the same limit as the reference's fused GPU engines (FC widths up to 64)
+  if (CP_ < 0 || CFP_ < 0) throw Error("GRACE-1L: channel widths above 64 are not supported by the GPU kernels");
   nAA_ = m.prod_AA.n_out;
   nAAA_ = m.prod_AAA.n_out;
   nAAAA_ = order4_ ? m.prod_AAAA.n_out : 0;
@@ -413,13 +450,13 @@ template<class T> void Engine1L<T>::build()
     for (int a = 0; a < nel_; a++)
       for (int b = 0; b < nel_; b++) cut[(size_t) a * nel_ + b] = m.pair_cutoff(a, b);
     upload_vec(cut_, cut);
-    std::vector<T> z((size_t) nel_ * C_);
+    std::vector<T> z((size_t) nel_ * CP_, (T) 0);
     for (int mu = 0; mu < nel_; mu++)
       for (int n = 0; n < C_; n++) {
         double v = 0.0;
         for (int e = 0; e < m.embedding_size; e++)
           v += m.A_lin_transform_W[(size_t) e * C_ + n] * m.chem_embedding[(size_t) mu * m.embedding_size + e];
-        z[(size_t) mu * C_ + n] = (T) (v * m.A_lin_transform_norm * m.A_inv_avg_n_neigh);
+        z[(size_t) mu * CP_ + n] = (T) (v * m.A_lin_transform_norm * m.A_inv_avg_n_neigh);
       }
     upload_vec(z_, z);
     upload_vec(shift_, m.shift_values);
@@ -437,7 +474,7 @@ template<class T> void Engine1L<T>::build()
     else if (hmax <= 128) hb_ = 8;
     else throw Error("GRACE-1L: radial MLP hidden width > 128 not supported");
     ks0_ = round_up(m.nradbase, 4) / 4;
-    const int nout = C_ * nl_;
+    const int nout = CP_ * nl_;
     noutp_ = round_up(nout, 16);
     nob_ = noutp_ / 16;
     std::vector<T> w0((size_t) hb_ * ks0_ * 64, (T) 0), w1((size_t) hb_ * hb_ * 4 * 64, (T) 0),
@@ -461,8 +498,8 @@ template<class T> void Engine1L<T>::build()
         for (int s = 0; s < 4; s++)
           for (int lane = 0; lane < 64; lane++) {
             const int g = lane >> 4, cc = lane & 15, in = kb * 16 + drow_[g * 4 + s], col = cb * 16 + cc;
-            if (in < H2 && col < nout) {
-              const int l = col / C_, n = col % C_, o = n * nl_ + l;    // file order o = n nl + l (fused_1l.cpp:123)
+            const int l = col / CP_, n = col % CP_, o = n * nl_ + l;    // file order o = n nl + l (fused_1l.cpp:123)
+            if (in < H2 && col < nout && n < C_) {
               w2[(((size_t) cb * hb_ + kb) * 4 + s) * 64 + lane] = (T) (L2.norm * L2.W[(size_t) in * L2.n_out + o]);
             }
           }
@@ -499,42 +536,52 @@ template<class T> void Engine1L<T>::build()
     pAA_.build(hAA);
     pAAA_.build(hAAA);
     if (order4_) pAAAA_.build(hAAAA);
-    fcA1_.build(m.fc_A1, liveA1, nlm_);
-    fcAA1_.build(m.fc_AA1, liveAA1, nlm_);
-    if (order4_) fcAA2_.build(m.fc_AA2, liveAA2, nlm_);
+    fcA1_.build(m.fc_A1, liveA1, nlm_, CP_, CP_, CFP_, drow_);
+    fcAA1_.build(m.fc_AA1, liveAA1, nlm_, CFP_, CP_, CFP_, drow_);
+    if (order4_) fcAA2_.build(m.fc_AA2, liveAA2, nlm_, CFP_, CP_, CFP_, drow_);
   }
 
-  // ---- rho reduce: weights per collected function, W[mu][c][n][k] with k padded (fused_cpu.h:1202-1273)
+  // ---- rho reduce: weights per collected function in MFMA fragment order (fused_cpu.h:1202-1273)
   {
     const ReduceWeights *rw[4] = {&m.red_A, &m.red_AA, &m.red_AAA, &m.red_AAAA};
     const int nfun[4] = {nlm_, nAA_, nAAA_, nAAAA_};
     red_.nsrc = order4_ ? 4 : 3;
     red_.nrho = nrho_;
-    red_.nrp = nrho_;
+    red_.nbr = (nrho_ + 15) / 16;
+    red_.ksr = (nrho_ + 3) / 4;
+    for (int q = 0; q < 16; q++) red_.drow[q] = drow_[q];
+    const int krp = red_.ksr * 4;
     for (int s = 0; s < red_.nsrc; s++) {
       const ReduceWeights &w = *rw[s];
       std::vector<int> fn(w.collect_ind);
       std::sort(fn.begin(), fn.end());
       fn.erase(std::unique(fn.begin(), fn.end()), fn.end());
-      const int nc = (int) fn.size(), nin = w.n_in;
-      std::vector<T> W((size_t) nel_ * nc * nin * nrho_, (T) 0);
-      std::vector<double> acc((size_t) nel_ * nc * nin * nrho_, 0.0);
-      for (size_t c = 0; c < w.collect_ind.size(); c++) {
-        const int u = (int) (std::lower_bound(fn.begin(), fn.end(), w.collect_ind[c]) - fn.begin());
-        const int tile = w.w_l_tile[c];
-        for (int mu = 0; mu < nel_; mu++)
+      const int nc = (int) fn.size(), nin = w.n_in, ninp = s == 0 ? CP_ : CFP_;
+      std::vector<T> WF, WB;
+      std::vector<double> M((size_t) nin * nrho_), Mt((size_t) nrho_ * nin);
+      for (int mu = 0; mu < nel_; mu++)
+        for (int u = 0; u < nc; u++) {
+          std::fill(M.begin(), M.end(), 0.0);
+          for (size_t c = 0; c < w.collect_ind.size(); c++) {
+            if (w.collect_ind[c] != fn[u]) continue;
+            const int tile = w.w_l_tile[c];
+            for (int k = 0; k < nrho_; k++)
+              for (int n = 0; n < nin; n++)
+                M[(size_t) n * nrho_ + k] += w.norm * w.W[(((size_t) mu * nrho_ + k) * nin + n) * w.w_shape + tile];
+          }
           for (int k = 0; k < nrho_; k++)
-            for (int n = 0; n < nin; n++)
-              acc[(((size_t) mu * nc + u) * nin + n) * nrho_ + k] +=
-                  w.norm * w.W[(((size_t) mu * nrho_ + k) * nin + n) * w.w_shape + tile];
-      }
-      for (size_t q = 0; q < acc.size(); q++) W[q] = (T) acc[q];
-      upload_vec(redW_[s], W);
+            for (int n = 0; n < nin; n++) Mt[(size_t) k * nin + n] = M[(size_t) n * nrho_ + k];
+          pack_fragments<T>(M, nin, nrho_, ninp, red_.nbr * 16, WF);      // X[atom][n] . M[n][k]
+          pack_fragments<T>(Mt, nrho_, nin, krp, ninp, WB);               // grho[atom][k] . Mt[k][n]
+        }
+      upload_vec(redWF_[s], WF);
+      upload_vec(redWB_[s], WB);
       upload_vec(redFn_[s], fn);
-      red_.W[s] = redW_[s].template as<T>();
+      red_.WF[s] = redWF_[s].template as<T>();
+      red_.WB[s] = redWB_[s].template as<T>();
       red_.fn[s] = redFn_[s].template as<int>();
       red_.ncol[s] = nc;
-      red_.nin[s] = nin;
+      red_.nin[s] = ninp;
       red_.stride[s] = nfun[s];
     }
   }
@@ -591,6 +638,21 @@ template<class T> void Engine1L<T>::upload(const CsrInput &in)
     if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, hipMemcpyHostToDevice, stream_));
   };
   put(mu_, mu.data(), sizeof(int) * n);
+  // tiles of 16 atoms of one element, in atom order within an element
+  std::vector<int> tiles;
+  {
+    std::vector<int> ord(n);
+    std::iota(ord.begin(), ord.end(), 0);
+    std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return mu[a] < mu[b]; });
+    for (int q = 0; q < n;) {
+      int cnt = 0;
+      const int m0 = mu[ord[q]];
+      while (cnt < 16 && q < n && mu[ord[q]] == m0) { tiles.push_back(ord[q]); q++; cnt++; }
+      while (cnt < 16) { tiles.push_back(-1); cnt++; }
+    }
+  }
+  ntiles_ = (int) tiles.size() / 16;
+  put(tiles_, tiles.data(), sizeof(int) * tiles.size());
   static_assert(sizeof(long long) == sizeof(int64_t), "offset type");
   put(offset_, in.offset, sizeof(int64_t) * (n + 1));
   put(j_, in.j, sizeof(int) * nb);
@@ -602,6 +664,44 @@ template<class T> void Engine1L<T>::upload(const CsrInput &in)
   }
   HIP_CHECK(hipStreamSynchronize(stream_));    // the host copies (mu) go out of scope
   ran_ = false;
+}
+
+template<class T>
+void Engine1L<T>::launch_gemm(DevJobs<T> &J, int kb0, int kb1, int nb, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo,
+                              int accumulate)
+{
+  if (J.d.njobs == 0 || ntiles_ == 0) return;
+  const int ksm = std::max(kb0, kb1) * 4;
+  const size_t lds = (size_t) kGemmMaxSeg * nb * ksm * 64 * sizeof(T);
+  const dim3 grid(J.d.njobs, (ntiles_ + 4 * kGemmTilesPerWave - 1) / (4 * kGemmTilesPerWave));
+#define GR_GEMM(A_, B_, C_)                                                                                            \
+  {                                                                                                                    \
+    auto kern = k_gemm_jobs<T, A_, B_, C_>;                                                                            \
+    if (lds > 48 * 1024)                                                                                               \
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, J.d, X0, nf0, X1, nf1, out, nfo, tiles_.as<int>(), ntiles_, accumulate); \
+  }
+#define GR_GEMM_C(A_, B_)                                                                                              \
+  switch (nb) {                                                                                                        \
+    case 1: GR_GEMM(A_, B_, 1) break;                                                                                  \
+    case 2: GR_GEMM(A_, B_, 2) break;                                                                                  \
+    case 4: GR_GEMM(A_, B_, 4) break;                                                                                  \
+    default: throw Error("unsupported channel widths");                                                                \
+  }
+  switch (kb0 * 10 + kb1) {
+    case 11: GR_GEMM_C(1, 1) break;
+    case 12: GR_GEMM_C(1, 2) break;
+    case 14: GR_GEMM_C(1, 4) break;
+    case 21: GR_GEMM_C(2, 1) break;
+    case 22: GR_GEMM_C(2, 2) break;
+    case 24: GR_GEMM_C(2, 4) break;
+    case 41: GR_GEMM_C(4, 1) break;
+    case 42: GR_GEMM_C(4, 2) break;
+    case 44: GR_GEMM_C(4, 4) break;
+    default: throw Error("unsupported channel widths");
+  }
+#undef GR_GEMM_C
+#undef GR_GEMM
 }
 
 template<class T>
@@ -619,7 +719,7 @@ void Engine1L<T>::launch_radial(long long e_begin, long long e_count, const doub
   ra.Rz = Rz; ra.dRz = dRz;
   ra.nrb = model_->nradbase; ra.p = model_->radial_basis_p; ra.ks0 = ks0_;
   ra.nob = nob_; ra.noutp = noutp_;
-  ra.C = C_; ra.nel = nel_; ra.act = model_->radial_activation;
+  ra.C = CP_; ra.nel = nel_; ra.act = model_->radial_activation;
   ra.w2_in_lds = w2_in_lds_;
   for (int q = 0; q < 16; q++) ra.drow[q] = drow_[q];
   const int threads = hb_ == 4 ? 512 : 256;
@@ -678,57 +778,59 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     launch_radial(0, -1, xr_.as<double>(), emu_.as<int>(), Rz_.as<T>(), dRz_.as<T>(), eoff_.as<long long>() + n);
   });
 
-  // ---- per-atom tensors (whole structure in one chunk)
+  // ---- per-atom tensors (whole structure in one chunk), channel widths padded
   const size_t na = (size_t) n;
-  A_.ensure(na * nlm_ * C_ * sizeof(T));
-  A1_.ensure(na * nlm_ * CF_ * sizeof(T));
-  AA_.ensure(na * nAA_ * CF_ * sizeof(T));
-  AA1_.ensure(na * nAA_ * CF_ * sizeof(T));
-  AAA_.ensure(na * nAAA_ * CF_ * sizeof(T));
+  A_.ensure(na * nlm_ * CP_ * sizeof(T));
+  A1_.ensure(na * nlm_ * CFP_ * sizeof(T));
+  AA_.ensure(na * nAA_ * CFP_ * sizeof(T));
+  AA1_.ensure(na * nAA_ * CFP_ * sizeof(T));
+  AAA_.ensure(na * nAAA_ * CFP_ * sizeof(T));
   if (order4_) {
-    AA2_.ensure(na * nAA_ * CF_ * sizeof(T));
-    AAAA_.ensure(na * nAAAA_ * CF_ * sizeof(T));
+    AA2_.ensure(na * nAA_ * CFP_ * sizeof(T));
+    AAAA_.ensure(na * nAAAA_ * CFP_ * sizeof(T));
   }
   rho_.ensure(na * nrho_ * sizeof(double));
   grho_.ensure(na * nrho_ * sizeof(double));
 
-  const int sthreads = round_up(nl_ * C_, 64);
+  const int sthreads = round_up(nl_ * CP_, 64);
   ScatterArgs<T> sa{};
   sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz_.as<T>(); sa.A = A_.as<T>();
-  sa.a0 = 0; sa.C = C_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = noutp_; sa.sh = sh_;
+  sa.a0 = 0; sa.C = CP_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = noutp_; sa.sh = sh_;
   stage("scatter_A", [&] {
     if (lmax_ <= 4) hipLaunchKernelGGL((k_scatter_a<T, 9>), dim3(n), dim3(sthreads), 0, stream_, sa);
     else hipLaunchKernelGGL((k_scatter_a<T, 13>), dim3(n), dim3(sthreads), 0, stream_, sa);
   });
 
-  auto fc_fwd = [&](const char *name, DevFc<T> &F, const T *Xl, const T *Xr, T *out, int nfl) {
-    const int AT = std::max(1, 256 / F.d.n_out);
-    stage(name, [&] {
-      if (F.d.nlive > 0)
-        hipLaunchKernelGGL(k_fc_fwd<T>, dim3(F.d.nlive, (n + AT - 1) / AT), dim3(F.d.n_out * AT), 0, stream_, F.d, Xl, Xr, out, n, nfl, nlm_);
-    });
-  };
+  const int *tiles = tiles_.as<int>();
+  const int ka = CP_ / 16, kf = CFP_ / 16;
   auto prod_fwd = [&](const char *name, DevProd &P, const T *L, const T *R, T *out, int sl, int sr) {
-    const int AT = std::max(1, 256 / CF_);
+    const int AT = std::max(1, 256 / CFP_);
     stage(name, [&] {
-      hipLaunchKernelGGL(k_prod_fwd<T>, dim3(P.d.nout, (n + AT - 1) / AT), dim3(CF_ * AT), 0, stream_, P.d, L, R, out, n, CF_, sl, sr);
+      hipLaunchKernelGGL(k_prod_fwd<T>, dim3(P.d.nout, (n + AT - 1) / AT), dim3(CFP_ * AT), 0, stream_, P.d, L, R, out, n, CFP_, sl, sr);
     });
   };
   T *A = A_.as<T>(), *A1 = A1_.as<T>(), *AA = AA_.as<T>(), *AA1 = AA1_.as<T>(), *AA2 = AA2_.as<T>(), *AAA = AAA_.as<T>(),
     *AAAA = AAAA_.as<T>();
-  if (aaa_a_ && C_ != CF_) throw Error("GRACE-1L: AAA = AA1 x A needs equal A and FC widths");
+  if (aaa_a_ && CP_ != CFP_) throw Error("GRACE-1L: AAA = AA1 x A needs equal A and FC widths");
   const T *Ar = aaa_a_ ? A : A1;
-  fc_fwd("fc_A1", fcA1_, A, A, A1, nlm_);
+  stage("fc_A1", [&] { launch_gemm(fcA1_.fwd, ka, ka, kf, A, nlm_, A, nlm_, A1, nlm_, 0); });
   prod_fwd("prod_AA", pAA_, A1, A1, AA, nlm_, nlm_);
-  fc_fwd("fc_AA1", fcAA1_, AA, A, AA1, nAA_);
+  stage("fc_AA1", [&] { launch_gemm(fcAA1_.fwd, kf, ka, kf, AA, nAA_, A, nlm_, AA1, nAA_, 0); });
   prod_fwd("prod_AAA", pAAA_, AA1, Ar, AAA, nAA_, nlm_);
   if (order4_) {
-    fc_fwd("fc_AA2", fcAA2_, AA, A, AA2, nAA_);
+    stage("fc_AA2", [&] { launch_gemm(fcAA2_.fwd, kf, ka, kf, AA, nAA_, A, nlm_, AA2, nAA_, 0); });
     prod_fwd("prod_AAAA", pAAAA_, AA2, AA2, AAAA, nAA_, nAA_);
   }
   stage("reduce_rho", [&] {
-    hipLaunchKernelGGL(k_reduce_fwd<T>, dim3(n), dim3(256), 0, stream_, red_, mu_.as<int>(), 0, (const T *) A, (const T *) AA,
-                       (const T *) AAA, (const T *) AAAA, rho_.as<double>());
+#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(ntiles_), dim3(256), 0, stream_, red_, mu_.as<int>(), tiles, \
+                                          (const T *) A, (const T *) AA, (const T *) AAA, (const T *) AAAA, rho_.as<double>())
+    switch (ka * 10 + kf) {
+      case 11: GR_RED(1, 1); break; case 12: GR_RED(1, 2); break; case 14: GR_RED(1, 4); break;
+      case 21: GR_RED(2, 1); break; case 22: GR_RED(2, 2); break; case 24: GR_RED(2, 4); break;
+      case 41: GR_RED(4, 1); break; case 42: GR_RED(4, 2); break; case 44: GR_RED(4, 4); break;
+      default: throw Error("unsupported channel widths");
+    }
+#undef GR_RED
   });
   stage("energy_mlp", [&] {
     hipLaunchKernelGGL(k_energy, dim3(n), dim3(64), 0, stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
@@ -737,61 +839,62 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   if (fl.energy_only) return;
 
   // ---- reverse
-  gA_.ensure(na * nlm_ * C_ * sizeof(T));
-  gA1_.ensure(na * nlm_ * CF_ * sizeof(T));
-  gAA_.ensure(na * nAA_ * CF_ * sizeof(T));
-  gAA1_.ensure(na * nAA_ * CF_ * sizeof(T));
-  gAAA_.ensure(na * nAAA_ * CF_ * sizeof(T));
+  gA_.ensure(na * nlm_ * CP_ * sizeof(T));
+  gA1_.ensure(na * nlm_ * CFP_ * sizeof(T));
+  gAA_.ensure(na * nAA_ * CFP_ * sizeof(T));
+  gAA1_.ensure(na * nAA_ * CFP_ * sizeof(T));
+  gAAA_.ensure(na * nAAA_ * CFP_ * sizeof(T));
   if (order4_) {
-    gAA2_.ensure(na * nAA_ * CF_ * sizeof(T));
-    gAAAA_.ensure(na * nAAAA_ * CF_ * sizeof(T));
+    gAA2_.ensure(na * nAA_ * CFP_ * sizeof(T));
+    gAAAA_.ensure(na * nAAAA_ * CFP_ * sizeof(T));
   }
   T *gA = gA_.as<T>(), *gA1 = gA1_.as<T>(), *gAA = gAA_.as<T>(), *gAA1 = gAA1_.as<T>(), *gAA2 = gAA2_.as<T>(),
     *gAAA = gAAA_.as<T>(), *gAAAA = gAAAA_.as<T>();
   stage("zero_grads", [&] {
-    HIP_CHECK(hipMemsetAsync(gA, 0, na * nlm_ * C_ * sizeof(T), stream_));
-    HIP_CHECK(hipMemsetAsync(gA1, 0, na * nlm_ * CF_ * sizeof(T), stream_));
-    HIP_CHECK(hipMemsetAsync(gAA, 0, na * nAA_ * CF_ * sizeof(T), stream_));
-    HIP_CHECK(hipMemsetAsync(gAA1, 0, na * nAA_ * CF_ * sizeof(T), stream_));
-    HIP_CHECK(hipMemsetAsync(gAAA, 0, na * nAAA_ * CF_ * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(gA, 0, na * nlm_ * CP_ * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(gA1, 0, na * nlm_ * CFP_ * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(gAA, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(gAA1, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(gAAA, 0, na * nAAA_ * CFP_ * sizeof(T), stream_));
     if (order4_) {
-      HIP_CHECK(hipMemsetAsync(gAA2, 0, na * nAA_ * CF_ * sizeof(T), stream_));
-      HIP_CHECK(hipMemsetAsync(gAAAA, 0, na * nAAAA_ * CF_ * sizeof(T), stream_));
+      HIP_CHECK(hipMemsetAsync(gAA2, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
+      HIP_CHECK(hipMemsetAsync(gAAAA, 0, na * nAAAA_ * CFP_ * sizeof(T), stream_));
     }
   });
   stage("reduce_rho_bwd", [&] {
-    hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(n), dim3(256), 0, stream_, red_, mu_.as<int>(), 0, grho_.as<double>(), gA, gAA, gAAA, gAAAA);
+    int njobs = 0;
+    for (int s = 0; s < red_.nsrc; s++) njobs += red_.ncol[s];
+    hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, njobs), dim3(64), 0, stream_, red_, mu_.as<int>(), tiles, grho_.as<double>(), gA, gAA,
+                       gAAA, gAAAA);
   });
   auto prod_bwd = [&](const char *name, DevProd &P, const T *L, const T *R, const T *g, T *gL, T *gR, int sl, int sr) {
-    const int AT = std::max(1, 256 / CF_);
+    const int AT = std::max(1, 256 / CFP_);
     stage(name, [&] {
-      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nleft, (n + AT - 1) / AT), dim3(CF_ * AT), 0, stream_, P.d, 0, R, g, gL, n, CF_, sr, sl);
-      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nright, (n + AT - 1) / AT), dim3(CF_ * AT), 0, stream_, P.d, 1, L, g, gR, n, CF_, sl, sr);
+      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nleft, (n + AT - 1) / AT), dim3(CFP_ * AT), 0, stream_, P.d, 0, R, g, gL, n, CFP_, sr, sl);
+      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nright, (n + AT - 1) / AT), dim3(CFP_ * AT), 0, stream_, P.d, 1, L, g, gR, n, CFP_, sl, sr);
     });
   };
-  auto fc_bwd = [&](const char *name, DevFc<T> &F, const T *g, T *gXl, T *gXr, int nfl) {
+  // FC reverse: left input (same functions as the output), then right input (functions of A)
+  auto fc_bwd = [&](const char *name, DevFc<T> &F, const T *g, T *gXl, T *gXr, int nfl, int kl) {
     stage(name, [&] {
-      const int ATl = std::max(1, 256 / F.d.n_in_l), ATr = std::max(1, 256 / F.d.n_in_r);
-      if (F.d.nlive > 0)
-        hipLaunchKernelGGL(k_fc_bwd_left<T>, dim3(F.d.nlive, (n + ATl - 1) / ATl), dim3(F.d.n_in_l * ATl), 0, stream_, F.d, g, gXl, n, nfl);
-      if (F.d.nrlive > 0)
-        hipLaunchKernelGGL(k_fc_bwd_right<T>, dim3(F.d.nrlive, (n + ATr - 1) / ATr), dim3(F.d.n_in_r * ATr), 0, stream_, F.d, g, gXr, n, nfl, nlm_);
+      launch_gemm(F.bwd_l, kf, kf, kl, g, nfl, g, nfl, gXl, nfl, 1);
+      launch_gemm(F.bwd_r, kf, kf, ka, g, nfl, g, nfl, gXr, nlm_, 1);
     });
   };
   if (order4_) {
     prod_bwd("prod_AAAA_bwd", pAAAA_, AA2, AA2, gAAAA, gAA2, gAA2, nAA_, nAA_);
-    fc_bwd("fc_AA2_bwd", fcAA2_, gAA2, gAA, gA, nAA_);
+    fc_bwd("fc_AA2_bwd", fcAA2_, gAA2, gAA, gA, nAA_, kf);
   }
   prod_bwd("prod_AAA_bwd", pAAA_, AA1, Ar, gAAA, gAA1, aaa_a_ ? gA : gA1, nAA_, nlm_);
-  fc_bwd("fc_AA1_bwd", fcAA1_, gAA1, gAA, gA, nAA_);
+  fc_bwd("fc_AA1_bwd", fcAA1_, gAA1, gAA, gA, nAA_, kf);
   prod_bwd("prod_AA_bwd", pAA_, A1, A1, gAA, gA1, gA1, nlm_, nlm_);
-  fc_bwd("fc_A1_bwd", fcA1_, gA1, gA, gA, nlm_);
+  fc_bwd("fc_A1_bwd", fcA1_, gA1, gA, gA, nlm_, ka);
 
   BondBwdArgs<T> ba{};
   ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
   ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = gA;
   ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1;
-  ba.a0 = 0; ba.C = C_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;
+  ba.a0 = 0; ba.C = CP_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;
   stage("bond_bwd", [&] {
     if (lmax_ <= 4) hipLaunchKernelGGL((k_bond_bwd<T, 9>), dim3(n), dim3(sthreads), 0, stream_, ba);
     else hipLaunchKernelGGL((k_bond_bwd<T, 13>), dim3(n), dim3(sthreads), 0, stream_, ba);
@@ -838,10 +941,11 @@ template<class T> void Engine1L<T>::debug_radial(int m, const double *x, const i
   HIP_CHECK(hipMemcpy(hR.data(), dR.p, hR.size() * sizeof(T), hipMemcpyDeviceToHost));
   HIP_CHECK(hipMemcpy(hdR.data(), ddR.p, hdR.size() * sizeof(T), hipMemcpyDeviceToHost));
   for (int q = 0; q < m; q++)
-    for (int c = 0; c < nl_ * C_; c++) {
-      Rz[(size_t) q * nl_ * C_ + c] = (double) hR[(size_t) q * noutp_ + c];
-      dRz[(size_t) q * nl_ * C_ + c] = (double) hdR[(size_t) q * noutp_ + c];
-    }
+    for (int l = 0; l < nl_; l++)
+      for (int c = 0; c < C_; c++) {
+        Rz[((size_t) q * nl_ + l) * C_ + c] = (double) hR[(size_t) q * noutp_ + l * CP_ + c];
+        dRz[((size_t) q * nl_ + l) * C_ + c] = (double) hdR[(size_t) q * noutp_ + l * CP_ + c];
+      }
 }
 
 }    // namespace

@@ -6,7 +6,7 @@
 //   k_radial                     Chebyshev x envelope basis + radial MLP value/tangent on MFMA, times z[mu_j]
 //                                (radial_x.h:11-60; spline tables of the CPU path replaced by the exact MLP)
 //   k_scatter_a                  A[lm][n] = sum_b Y_lm R_nl z                            (fused_cpu.h:947-982)
-//   k_fc_fwd / k_fc_bwd_*        FC                                                       (fused_cpu.h:349-364)
+//   k_gemm_jobs                  FC forward / reverse as tile GEMMs on MFMA               (fused_cpu.h:349-364)
 //   k_prod_fwd / k_prod_bwd      channel-wise CG products                                 (fused_cpu.h:409-475)
 //   k_reduce_fwd / k_reduce_bwd  rho reduce with per-element weights                      (fused_cpu.h:637-649)
 //   k_energy                     fp64 readout MLP and its reverse                         (fused_1l.cpp:378-427)
@@ -448,73 +448,125 @@ template<class T, int MAXM> __global__ void k_scatter_a(ScatterArgs<T> a)
 // ---------------------------------------------------------------------------------------------------------------
 // per-atom dense chain.  Per-atom tensors are [atom][function][channel].
 // ---------------------------------------------------------------------------------------------------------------
-template<class T> struct FcDev {
-  const T *Wl, *Wr;           // [tile][n_in][n_out], norms folded in
-  const T *WlT, *WrT;         // [tile][n_out][n_in]
-  const int *tile_l;          // [nf]
-  const T *nof;               // [nf]
-  const int *live;            // [nlive] output functions that are computed
-  const int *conn_off, *conn_from, *conn_tile;      // right connections by output function (CSR over nf)
-  const int *rlive;           // [nrlive] right-input functions that receive a gradient
-  const int *rconn_off, *rconn_to, *rconn_tile;     // right connections by right-input function (CSR over nfr)
-  int nf, nfr, nlive, nrlive, n_in_l, n_in_r, n_out;
+// Atoms are processed in tiles of 16 (one MFMA tile): tile_atoms[tile * 16 + r] is the atom of row r, or -1.  Tiles
+// hold atoms of one element, so that element-dependent weights (rho reduce) are uniform per tile.
+//
+// Job / segment GEMM of the FC layers on the matrix cores.  Job = one output function; its value for a tile is
+//   out[atom][fo][0:N] (+)= scale_job * sum_seg  seg_scale * X_src(seg)[atom][fn(seg)][0:K] . W[wtile(seg)][0:K][0:N]
+// FC forward:        job f,  segments (Xl, f, Wl[tile_l f]) and (Xr, from c, Wr[tile c]) for every connection c -> f
+// FC reverse, left:  job f,  segment  (g, f, Wl^T[tile_l f]), accumulated into gXl
+// FC reverse, right: job r,  segments (g, to c, nof[to c] Wr^T[tile c]) for the connections c from r, accumulated
+// Rows of the A operand are the 16 atoms (lane % 16), its k index g * (K / 4) + s (g = lane / 16), so that a lane
+// reads K / 4 consecutive channels; weights are stored in that fragment order ([tile][cb][s][lane]) and staged in LDS.
+template<class T> struct GemmJobs {
+  const int *job_out;         // [njobs] output function
+  const T *job_scale;         // [njobs]
+  const int *seg_off;         // [njobs + 1]
+  const int *seg_src;         // [nseg] 0: X0 (K0 channels), 1: X1 (K1 channels)
+  const int *seg_fn;          // [nseg] function of the source tensor
+  const int *seg_w;           // [nseg] weight tile
+  const T *seg_scale;         // [nseg]
+  const T *WF0, *WF1;         // fragments of the weights used with X0 / X1
+  int njobs;
+  int drow[16];               // accumulator row of (lane / 16, register), probed on the device
 };
 
-// out[a][f][k] = nof[f] (sum_n Wl[tile_l f][n][k] Xl[a][f][n] + sum_{c -> f} sum_n Wr[tile c][n][k] Xr[a][from c][n])
-// grid (nlive, atom groups); block = n_out x AT threads
-template<class T> __global__ void k_fc_fwd(FcDev<T> F, const T *Xl, const T *Xr, T *out, int natoms, int nfl_stride,
-                                           int nfr_stride)
-{
-  const int k = threadIdx.x % F.n_out, al = threadIdx.x / F.n_out;
-  const int AT = blockDim.x / F.n_out;
-  const int at = blockIdx.y * AT + al;
-  if (at >= natoms || al >= AT) return;
-  const int f = F.live[blockIdx.x];
-  const T *xl = Xl + ((long long) at * nfl_stride + f) * F.n_in_l;
-  const T *wl = F.Wl + (long long) F.tile_l[f] * F.n_in_l * F.n_out + k;
-  T acc = (T) 0;
-  for (int n = 0; n < F.n_in_l; n++) acc += xl[n] * wl[(long long) n * F.n_out];
-  for (int c = F.conn_off[f]; c < F.conn_off[f + 1]; c++) {
-    const T *xr = Xr + ((long long) at * nfr_stride + F.conn_from[c]) * F.n_in_r;
-    const T *wr = F.Wr + (long long) F.conn_tile[c] * F.n_in_r * F.n_out + k;
-    for (int n = 0; n < F.n_in_r; n++) acc += xr[n] * wr[(long long) n * F.n_out];
-  }
-  out[((long long) at * nfl_stride + f) * F.n_out + k] = F.nof[f] * acc;
-}
+constexpr int kGemmMaxSeg = 4;      // weight tiles staged in LDS at a time
+constexpr int kGemmTilesPerWave = 2;
 
-// gXl[a][f][n] += nof[f] sum_k Wl[tile_l f][n][k] g[a][f][k]     grid (nlive, atom groups); block = n_in_l x AT
-template<class T> __global__ void k_fc_bwd_left(FcDev<T> F, const T *g, T *gXl, int natoms, int nfl_stride)
+template<class T, int KB0, int KB1, int NB>
+__global__ __launch_bounds__(256) void k_gemm_jobs(GemmJobs<T> J, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo,
+                                                   const int *tile_atoms, int ntiles, int accumulate)
 {
-  const int n = threadIdx.x % F.n_in_l, al = threadIdx.x / F.n_in_l;
-  const int AT = blockDim.x / F.n_in_l;
-  const int at = blockIdx.y * AT + al;
-  if (at >= natoms || al >= AT) return;
-  const int f = F.live[blockIdx.x];
-  const T *gg = g + ((long long) at * nfl_stride + f) * F.n_out;
-  const T *w = F.WlT + (long long) F.tile_l[f] * F.n_out * F.n_in_l + n;
-  T acc = (T) 0;
-  for (int k = 0; k < F.n_out; k++) acc += gg[k] * w[(long long) k * F.n_in_l];
-  gXl[((long long) at * nfl_stride + f) * F.n_in_l + n] += F.nof[f] * acc;
-}
-
-// gXr[a][r][n] += sum_{c: from c = r} nof[to c] sum_k Wr[tile c][n][k] g[a][to c][k]   grid (nrlive, atom groups)
-template<class T> __global__ void k_fc_bwd_right(FcDev<T> F, const T *g, T *gXr, int natoms, int nfl_stride, int nfr_stride)
-{
-  const int n = threadIdx.x % F.n_in_r, al = threadIdx.x / F.n_in_r;
-  const int AT = blockDim.x / F.n_in_r;
-  const int at = blockIdx.y * AT + al;
-  if (at >= natoms || al >= AT) return;
-  const int r = F.rlive[blockIdx.x];
-  T acc = (T) 0;
-  for (int c = F.rconn_off[r]; c < F.rconn_off[r + 1]; c++) {
-    const int to = F.rconn_to[c];
-    const T *gg = g + ((long long) at * nfl_stride + to) * F.n_out;
-    const T *w = F.WrT + (long long) F.rconn_tile[c] * F.n_out * F.n_in_r + n;
-    T s = (T) 0;
-    for (int k = 0; k < F.n_out; k++) s += gg[k] * w[(long long) k * F.n_in_r];
-    acc += F.nof[to] * s;
+  typedef typename Mfma<T>::v4 v4;
+  constexpr int KS0 = KB0 * 4, KS1 = KB1 * 4, KSM = KS0 > KS1 ? KS0 : KS1, K0 = KB0 * 16, K1 = KB1 * 16, N = NB * 16;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T *wl = reinterpret_cast<T *>(smem_raw);      // [kGemmMaxSeg][NB][KSM][64]
+  __shared__ int s_src[kGemmMaxSeg], s_fn[kGemmMaxSeg];
+  __shared__ T s_scale[kGemmMaxSeg];
+  const int job = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int sg0 = J.seg_off[job], sg1 = J.seg_off[job + 1];
+  const int fo = J.job_out[job];
+  v4 acc[kGemmTilesPerWave][NB];
+  int arow[kGemmTilesPerWave];            // atom of this lane's A row
+#pragma unroll
+  for (int i = 0; i < kGemmTilesPerWave; i++) {
+    const int tile = (blockIdx.y * 4 + wave) * kGemmTilesPerWave + i;
+    arow[i] = tile < ntiles ? tile_atoms[tile * 16 + c] : -1;
+#pragma unroll
+    for (int cb = 0; cb < NB; cb++) acc[i][cb] = v4{0, 0, 0, 0};
   }
-  gXr[((long long) at * nfr_stride + r) * F.n_in_r + n] += acc;
+  for (int sg = sg0; sg < sg1; sg += kGemmMaxSeg) {
+    const int ns = sg1 - sg < kGemmMaxSeg ? sg1 - sg : kGemmMaxSeg;
+    __syncthreads();
+    for (int q = 0; q < ns; q++) {
+      const int src = J.seg_src[sg + q];
+      const int ks = src == 0 ? KS0 : KS1;
+      const T *wf = (src == 0 ? J.WF0 : J.WF1) + (long long) J.seg_w[sg + q] * NB * ks * 64;
+      for (int e = threadIdx.x; e < NB * ks * 64; e += 256) {
+        const int cb = e / (ks * 64), rem = e % (ks * 64);
+        wl[(q * NB + cb) * KSM * 64 + rem] = wf[e];
+      }
+      if (threadIdx.x == 0) { s_src[q] = src; s_fn[q] = J.seg_fn[sg + q]; s_scale[q] = J.seg_scale[sg + q]; }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kGemmTilesPerWave; i++) {
+      for (int q = 0; q < ns; q++) {
+        const T sc = s_scale[q];
+        const T *wq = wl + q * NB * KSM * 64 + lane;
+        if (s_src[q] == 0) {
+          T x[KS0];
+          if (arow[i] >= 0) {
+            const T *xp = X0 + ((long long) arow[i] * nf0 + s_fn[q]) * K0 + g * KS0;
+#pragma unroll
+            for (int s = 0; s < KS0; s++) x[s] = xp[s] * sc;
+          } else {
+#pragma unroll
+            for (int s = 0; s < KS0; s++) x[s] = (T) 0;
+          }
+#pragma unroll
+          for (int cb = 0; cb < NB; cb++)
+#pragma unroll
+            for (int s = 0; s < KS0; s++) acc[i][cb] = Mfma<T>::mma(x[s], wq[(cb * KSM + s) * 64], acc[i][cb]);
+        } else {
+          T x[KS1];
+          if (arow[i] >= 0) {
+            const T *xp = X1 + ((long long) arow[i] * nf1 + s_fn[q]) * K1 + g * KS1;
+#pragma unroll
+            for (int s = 0; s < KS1; s++) x[s] = xp[s] * sc;
+          } else {
+#pragma unroll
+            for (int s = 0; s < KS1; s++) x[s] = (T) 0;
+          }
+#pragma unroll
+          for (int cb = 0; cb < NB; cb++)
+#pragma unroll
+            for (int s = 0; s < KS1; s++) acc[i][cb] = Mfma<T>::mma(x[s], wq[(cb * KSM + s) * 64], acc[i][cb]);
+        }
+      }
+    }
+  }
+  // accumulator (g, v) holds row drow[4 g + v] of the tile, column cb * 16 + c
+  const T js = J.job_scale[job];
+#pragma unroll
+  for (int i = 0; i < kGemmTilesPerWave; i++) {
+    const int tile = (blockIdx.y * 4 + wave) * kGemmTilesPerWave + i;
+    if (tile >= ntiles) continue;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const int at = tile_atoms[tile * 16 + J.drow[4 * g + v]];
+      if (at < 0) continue;
+      T *o = out + ((long long) at * nfo + fo) * N + c;
+#pragma unroll
+      for (int cb = 0; cb < NB; cb++) {
+        const T val = js * acc[i][cb][v];
+        o[cb * 16] = accumulate ? o[cb * 16] + val : val;
+      }
+    }
+  }
 }
 
 struct ProdDev {
@@ -561,78 +613,107 @@ template<class T> __global__ void k_prod_bwd(ProdDev P, int side, const T *other
 }
 
 template<class T> struct ReduceDev {
-  // per source s: collected functions fn[s][c] (unique), weights W[s][mu][c][n][kp] (norm folded, k padded to nrp)
-  const T *W[4];
+  // per source s: collected functions fn[s][c] (unique), weights in fragment order
+  //   forward WF[s][mu][c][cb][ks][lane]  = W_s[mu][c][n = g KS + ks][k = cb 16 + lane % 16]    (norm folded, k >= nrho zero)
+  //   reverse WB[s][mu][c][cb][ks][lane]  = W_s[mu][c][n = cb 16 + lane % 16][k = g KSR + ks]
+  const T *WF[4], *WB[4];
   const int *fn[4];
-  int ncol[4], nin[4], stride[4];    // collected functions, channels, functions per atom of the source tensor
-  int nsrc, nrho, nrp;
+  int ncol[4], nin[4], stride[4];    // collected functions, (padded) channels, functions per atom of the source
+  int nsrc, nrho, nbr, ksr;          // rho width, its 16-column blocks, k-steps of the reverse (ceil(nrho / 4))
+  int drow[16];                      // accumulator row of (lane / 16, register)
 };
 
-// rho[a][k] = sum_s sum_c sum_n W_s[mu_a][c][n][k] X_s[a][fn c][n]     one block per atom
-template<class T> __global__ void k_reduce_fwd(ReduceDev<T> R, const int *mu, int a0, const T *X0, const T *X1, const T *X2,
-                                               const T *X3, double *rho)
+// rho[atom][k] = sum_s sum_c sum_n W_s[mu][c][n][k] X_s[atom][fn c][n] on the matrix cores: one block per tile of
+// 16 atoms, its 4 waves split the (s, c) list, partial tiles summed through LDS.  KBA / KBF: 16-channel blocks of
+// source 0 (A) and of the other sources.
+template<class T, int KBA, int KBF>
+__global__ __launch_bounds__(256) void k_reduce_fwd(ReduceDev<T> R, const int *mu, const int *tile_atoms, const T *X0, const T *X1,
+                                                    const T *X2, const T *X3, double *rho)
 {
-  __shared__ double part[4][32];
-  const int at = blockIdx.x;
-  const int m = mu[a0 + at];
+  typedef typename Mfma<T>::v4 v4;
+  __shared__ double part[4][2][16][17];
+  const int tile = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int arow = tile_atoms[tile * 16 + c];
+  const int a0 = tile_atoms[tile * 16];
+  const int m = mu[a0];
   const T *X[4] = {X0, X1, X2, X3};
-  double acc[32];
-#pragma unroll
-  for (int k = 0; k < 32; k++) acc[k] = 0.0;
+  v4 acc[2] = {v4{0, 0, 0, 0}, v4{0, 0, 0, 0}};
+  int job = 0;
   for (int s = 0; s < R.nsrc; s++) {
-    const int nq = R.ncol[s] * R.nin[s];
-    const T *Ws = R.W[s] + (long long) m * nq * R.nrp;
-    const T *Xs = X[s] + (long long) at * R.stride[s] * R.nin[s];
-    for (int q = threadIdx.x; q < nq; q += blockDim.x) {
-      const int c = q / R.nin[s], n = q % R.nin[s];
-      const T x = Xs[(long long) R.fn[s][c] * R.nin[s] + n];
-      const T *w = Ws + (long long) q * R.nrp;
+    const int ks = (s == 0 ? KBA : KBF) * 4, K = ks * 4;
+    for (int cc = 0; cc < R.ncol[s]; cc++, job++) {
+      if ((job & 3) != wave) continue;
+      const T *wf = R.WF[s] + ((long long) m * R.ncol[s] + cc) * R.nbr * ks * 64 + lane;
+      T x[(KBA > KBF ? KBA : KBF) * 4];
+      if (arow >= 0) {
+        const T *xp = X[s] + ((long long) arow * R.stride[s] + R.fn[s][cc]) * K + g * ks;
 #pragma unroll
-      for (int k = 0; k < 32; k++)
-        if (k < R.nrho) acc[k] += (double) (w[k] * x);
+        for (int q = 0; q < (KBA > KBF ? KBA : KBF) * 4; q++) x[q] = q < ks ? xp[q] : (T) 0;
+      } else {
+#pragma unroll
+        for (int q = 0; q < (KBA > KBF ? KBA : KBF) * 4; q++) x[q] = (T) 0;
+      }
+#pragma unroll
+      for (int cb = 0; cb < 2; cb++)
+        if (cb < R.nbr) {
+#pragma unroll
+          for (int q = 0; q < (KBA > KBF ? KBA : KBF) * 4; q++)
+            if (q < ks) acc[cb] = Mfma<T>::mma(x[q], wf[(cb * ks + q) * 64], acc[cb]);
+        }
     }
   }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-  for (int k = 0; k < 32; k++)
-    if (k < R.nrho) {
-      double v = acc[k];
-      for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
-      if (lane == 0) part[wave][k] = v;
-    }
+  for (int cb = 0; cb < 2; cb++)
+#pragma unroll
+    for (int v = 0; v < 4; v++) part[wave][cb][R.drow[4 * g + v]][c] = (double) acc[cb][v];
   __syncthreads();
-  if (threadIdx.x < R.nrho) {
+  for (int e = threadIdx.x; e < 16 * R.nrho; e += 256) {
+    const int r = e / R.nrho, k = e % R.nrho;
+    const int at = tile_atoms[tile * 16 + r];
+    if (at < 0) continue;
     double v = 0.0;
-    for (int w = 0; w < (int) (blockDim.x >> 6); w++) v += part[w][threadIdx.x];
-    rho[(long long) at * R.nrho + threadIdx.x] = v;
+    for (int w = 0; w < 4; w++) v += part[w][k >> 4][r][k & 15];
+    rho[(long long) at * R.nrho + k] = v;
   }
 }
 
-// gX_s[a][fn c][n] += sum_k W_s[mu_a][c][n][k] grho[a][k]            one block per atom
-template<class T> __global__ void k_reduce_bwd(ReduceDev<T> R, const int *mu, int a0, const double *grho, T *G0, T *G1, T *G2,
-                                               T *G3)
+// gX_s[atom][fn c][n] += sum_k grho[atom][k] W_s[mu][c][n][k]: grid (tiles, jobs = all (s, c)), one wave per block
+template<class T>
+__global__ __launch_bounds__(64) void k_reduce_bwd(ReduceDev<T> R, const int *mu, const int *tile_atoms, const double *grho, T *G0, T *G1,
+                                                   T *G2, T *G3)
 {
-  __shared__ T gr[32];
-  const int at = blockIdx.x;
-  const int m = mu[a0 + at];
-  if (threadIdx.x < 32) gr[threadIdx.x] = threadIdx.x < R.nrho ? (T) grho[(long long) at * R.nrho + threadIdx.x] : (T) 0;
-  __syncthreads();
+  typedef typename Mfma<T>::v4 v4;
+  const int tile = blockIdx.x;
+  int job = blockIdx.y, s = 0;
+  while (job >= R.ncol[s]) { job -= R.ncol[s]; s++; }
+  const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;
+  const int arow = tile_atoms[tile * 16 + c];
+  const int m = mu[tile_atoms[tile * 16]];
   T *G[4] = {G0, G1, G2, G3};
-  for (int s = 0; s < R.nsrc; s++) {
-    const int nq = R.ncol[s] * R.nin[s];
-    const T *Ws = R.W[s] + (long long) m * nq * R.nrp;
-    T *Gs = G[s] + (long long) at * R.stride[s] * R.nin[s];
-    for (int q = threadIdx.x; q < nq; q += blockDim.x) {
-      const int c = q / R.nin[s], n = q % R.nin[s];
-      const T *w = Ws + (long long) q * R.nrp;
-      T v = (T) 0;
+  T x[8];
 #pragma unroll
-      for (int k = 0; k < 32; k++)
-        if (k < R.nrho) v += w[k] * gr[k];
-      Gs[(long long) R.fn[s][c] * R.nin[s] + n] += v;
+  for (int q = 0; q < 8; q++) {
+    const int k = g * R.ksr + q;
+    x[q] = (arow >= 0 && q < R.ksr && k < R.nrho) ? (T) grho[(long long) arow * R.nrho + k] : (T) 0;
+  }
+  const int nb = R.nin[s] / 16;
+  const T *wb = R.WB[s] + ((long long) m * R.ncol[s] + job) * nb * R.ksr * 64 + lane;
+  const int fn = R.fn[s][job];
+  for (int cb = 0; cb < nb; cb++) {
+    v4 acc = {0, 0, 0, 0};
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+      if (q < R.ksr) acc = Mfma<T>::mma(x[q], wb[(cb * R.ksr + q) * 64], acc);
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const int at = tile_atoms[tile * 16 + R.drow[4 * g + v]];
+      if (at >= 0) G[s][((long long) at * R.stride[s] + fn) * R.nin[s] + cb * 16 + c] += acc[v];
     }
   }
 }
+
 
 struct EnergyDev {
   const double *W[7];         // [n_in][n_out]
