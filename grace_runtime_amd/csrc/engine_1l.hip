@@ -895,9 +895,14 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = gA;
   ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1;
   ba.a0 = 0; ba.C = CP_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;
+  for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
   stage("bond_bwd", [&] {
-    if (lmax_ <= 4) hipLaunchKernelGGL((k_bond_bwd<T, 9>), dim3(n), dim3(sthreads), 0, stream_, ba);
-    else hipLaunchKernelGGL((k_bond_bwd<T, 13>), dim3(n), dim3(sthreads), 0, stream_, ba);
+    const size_t lds = ((size_t) nl_ * (CP_ / 4) * 64 + (size_t) 4 * 16 * nlm_ * 4) * sizeof(T);
+    switch (CP_ / 16) {
+      case 1: hipLaunchKernelGGL((k_bond_bwd<T, 1>), dim3(n), dim3(256), lds, stream_, ba); break;
+      case 2: hipLaunchKernelGGL((k_bond_bwd<T, 2>), dim3(n), dim3(256), lds, stream_, ba); break;
+      default: hipLaunchKernelGGL((k_bond_bwd<T, 4>), dim3(n), dim3(256), lds, stream_, ba); break;
+    }
   });
 }
 

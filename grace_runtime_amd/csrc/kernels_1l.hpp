@@ -810,90 +810,135 @@ template<class T> struct BondBwdArgs {
   double *virial;             // [6]     (+=, atomics)
   int a0;
   int C, nl, nlm, noutp;
+  int drow[16];               // accumulator row of (lane / 16, register)
   ShCoef sh;
 };
 
-// one block per atom, thread = (l, n).  Per bond: g_d = sum_{l n} Rz[l][n] sum_m G[lm][d] gA[lm][n],
-// dE/dx = sum_{l n} dRz[l][n] sum_m Y[lm] gA[lm][n]; fv = dEdx / rc rhat + (g - (g . rhat) rhat) / r;
-// f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv.
-template<class T, int MAXM> __global__ void k_bond_bwd(BondBwdArgs<T> a)
+// One block (4 waves) per atom; a wave takes tiles of 16 bonds.  Per tile and l two tile GEMMs on the matrix cores,
+//   P[b][m] = sum_n Rz[b][l][n] gA[l*l + m][n],   Q[b][m] = sum_n dRz[b][l][n] gA[l*l + m][n]      (K = channels)
+// with the gA^T fragments of the atom staged once in LDS, then per bond
+//   g_d = sum_lm G[b][lm][d] P[b][lm],  dE/dx = sum_lm Y[b][lm] Q[b][lm],
+//   fv = dE/dx / rc rhat + (g - (g . rhat) rhat) / r;  f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv
+// (fused_cpu.h:836-860,1027-1050; fused_1l.cpp:46-51 of the reference).  KB = channels / 16.
+template<class T, int KB> __global__ __launch_bounds__(256) void k_bond_bwd(BondBwdArgs<T> a)
 {
-  __shared__ T Ysh[kBondChunk][kMaxNlm];
-  __shared__ T Gsh[kBondChunk][kMaxNlm * 3];
-  __shared__ double part[kBondChunk][16][4];
-  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, nw = blockDim.x >> 6;
+  typedef typename Mfma<T>::v4 v4;
+  constexpr int KS = KB * 4;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  T *gAf = reinterpret_cast<T *>(smem_raw);                          // [nl][KS][64] B-operand fragments of gA^T
+  T *Ysh = gAf + a.nl * KS * 64;                                     // [4 waves][16][nlm]
+  T *Gsh = Ysh + 4 * 16 * a.nlm;                                     // [4 waves][16][3 nlm]
+  __shared__ double red[4][9];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int c = lane & 15, g = lane >> 4;
   const int i = a.a0 + blockIdx.x;
   const long long e0 = a.eoff[i], e1 = a.eoff[i + 1];
-  const int ncol = a.nl * a.C;
-  const int l = t < ncol ? t / a.C : 0, n = t % a.C;
-  const int nm = t < ncol ? 2 * l + 1 : 0, lm0 = l * l;
-  T ga[MAXM];
+  const int C = a.C;
   {
-    const T *gAi = a.gA + (long long) blockIdx.x * a.nlm * a.C;
-#pragma unroll
-    for (int m = 0; m < MAXM; m++) ga[m] = m < nm ? gAi[(lm0 + m) * a.C + n] : (T) 0;
+    // fragment (l, s, lane (g, c)) = gA[l*l + c][g KS + s] for c < 2l + 1, else 0
+    const T *gAi = a.gA + (long long) blockIdx.x * a.nlm * C;
+    for (int q = t; q < a.nl * KS * 64; q += 256) {
+      const int l = q / (KS * 64), s = (q / 64) % KS, ln = q & 63, gg = ln >> 4, cc = ln & 15;
+      gAf[q] = cc < 2 * l + 1 ? gAi[(l * l + cc) * C + gg * KS + s] : (T) 0;
+    }
   }
+  __syncthreads();
+  T *Yw = Ysh + wave * 16 * a.nlm, *Gw = Gsh + wave * 16 * 3 * a.nlm;
   double fi[3] = {0, 0, 0}, vir[6] = {0, 0, 0, 0, 0, 0};
-  for (long long base = e0; base < e1; base += kBondChunk) {
-    const int nb = (int) (e1 - base < kBondChunk ? e1 - base : kBondChunk);
-    __syncthreads();
-    if (t < nb) {
-      const double *u = a.rh + 3 * (base + t);
-      sh_eval<true, T>(a.sh, u[0], u[1], u[2], Ysh[t], Gsh[t]);
+  const int ntile = (int) ((e1 - e0 + 15) / 16);
+  for (int tile = wave; tile < ntile; tile += 4) {
+    const long long eb = e0 + (long long) tile * 16;
+    const int nb = (int) (e1 - eb < 16 ? e1 - eb : 16);
+    if (lane < nb) {
+      const double *u = a.rh + 3 * (eb + lane);
+      sh_eval<true, T>(a.sh, u[0], u[1], u[2], Yw + lane * a.nlm, Gw + lane * 3 * a.nlm);
     }
-    __syncthreads();
-    for (int b = 0; b < nb; b++) {
-      double p0 = 0, p1 = 0, p2 = 0, px = 0;
-      if (t < ncol) {
-        const T rz = a.Rz[(base + b) * a.noutp + t], drz = a.dRz[(base + b) * a.noutp + t];
-        const T *y = Ysh[b] + lm0, *G = Gsh[b] + 3 * lm0;
-        T tx = 0, t0 = 0, t1 = 0, t2 = 0;
+    // LDS writes of this wave visible to its other lanes (the Y / G region is private to the wave)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    double p0[4] = {0, 0, 0, 0}, p1[4] = {0, 0, 0, 0}, p2[4] = {0, 0, 0, 0}, px[4] = {0, 0, 0, 0};
+    const bool rowok = c < nb;                      // A operand row = bond c of the tile
+    for (int l = 0; l < a.nl; l++) {
+      T x[KS], dx[KS];
+      if (rowok) {
+        const T *rp = a.Rz + (eb + c) * a.noutp + l * C + g * KS;
+        const T *dp = a.dRz + (eb + c) * a.noutp + l * C + g * KS;
 #pragma unroll
-        for (int m = 0; m < MAXM; m++)
-          if (m < nm) {
-            tx += y[m] * ga[m];
-            t0 += G[3 * m] * ga[m];
-            t1 += G[3 * m + 1] * ga[m];
-            t2 += G[3 * m + 2] * ga[m];
+        for (int s = 0; s < KS; s++) { x[s] = rp[s]; dx[s] = dp[s]; }
+      } else {
+#pragma unroll
+        for (int s = 0; s < KS; s++) { x[s] = (T) 0; dx[s] = (T) 0; }
+      }
+      v4 aP = {0, 0, 0, 0}, aQ = {0, 0, 0, 0};
+      const T *bf = gAf + l * KS * 64 + lane;
+#pragma unroll
+      for (int s = 0; s < KS; s++) {
+        const T b = bf[s * 64];
+        aP = Mfma<T>::mma(x[s], b, aP);
+        aQ = Mfma<T>::mma(dx[s], b, aQ);
+      }
+      if (c < 2 * l + 1) {
+        const int lm = l * l + c;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+          const int row = a.drow[4 * g + v];
+          if (row < nb) {
+            const T *G = Gw + (row * a.nlm + lm) * 3;
+            px[v] += (double) (Yw[row * a.nlm + lm] * aQ[v]);
+            p0[v] += (double) (G[0] * aP[v]);
+            p1[v] += (double) (G[1] * aP[v]);
+            p2[v] += (double) (G[2] * aP[v]);
           }
-        p0 = (double) (rz * t0); p1 = (double) (rz * t1); p2 = (double) (rz * t2); px = (double) (drz * tx);
+        }
       }
-      for (int o = 32; o > 0; o >>= 1) {
-        p0 += __shfl_down(p0, o, 64); p1 += __shfl_down(p1, o, 64);
-        p2 += __shfl_down(p2, o, 64); px += __shfl_down(px, o, 64);
-      }
-      if (lane == 0) { part[b][wave][0] = p0; part[b][wave][1] = p1; part[b][wave][2] = p2; part[b][wave][3] = px; }
     }
-    __syncthreads();
-    if (t < nb) {
-      double gv[3] = {0, 0, 0}, dEdx = 0;
-      for (int w = 0; w < nw; w++) { gv[0] += part[t][w][0]; gv[1] += part[t][w][1]; gv[2] += part[t][w][2]; dEdx += part[t][w][3]; }
-      const long long e = base + t;
-      const double *u = a.rh + 3 * e;
-      const double r = a.r[e], rc = a.rc[e];
-      const double dEdr = dEdx / rc;
-      const double gr = gv[0] * u[0] + gv[1] * u[1] + gv[2] * u[2];
-      double fv[3];
-      for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + (gv[d] - gr * u[d]) / r;
-      const int jj = a.ej[e];
-      for (int d = 0; d < 3; d++) {
-        fi[d] += fv[d];
-        atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
-      }
-      const double dx = -u[0] * r, dy = -u[1] * r, dz = -u[2] * r;
-      vir[0] += dx * fv[0]; vir[1] += dy * fv[1]; vir[2] += dz * fv[2];
-      vir[3] += dx * fv[1]; vir[4] += dx * fv[2]; vir[5] += dy * fv[2];
-    }
-  }
-  // only the first kBondChunk threads carry partial sums: reduce them inside wave 0
-  if (wave == 0) {
-    double v[9] = {fi[0], fi[1], fi[2], vir[0], vir[1], vir[2], vir[3], vir[4], vir[5]};
+    // sum over the 16 lanes of a group (the m index)
 #pragma unroll
-    for (int k = 0; k < 9; k++)
-      for (int o = 32; o > 0; o >>= 1) v[k] += __shfl_down(v[k], o, 64);
-    if (lane == 0) {
-      for (int d = 0; d < 3; d++) atomicAdd(&a.f[3 * (long long) i + d], v[d]);
-      for (int k = 0; k < 6; k++) atomicAdd(&a.virial[k], v[3 + k]);
+    for (int v = 0; v < 4; v++)
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) {
+        p0[v] += __shfl_xor(p0[v], o, 64); p1[v] += __shfl_xor(p1[v], o, 64);
+        p2[v] += __shfl_xor(p2[v], o, 64); px[v] += __shfl_xor(px[v], o, 64);
+      }
+    // lane c = v of each group finishes bond drow[4 g + v]
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const int row = a.drow[4 * g + v];
+      if (c == v && row < nb) {
+        const long long e = eb + row;
+        const double *u = a.rh + 3 * e;
+        const double r = a.r[e], rc = a.rc[e];
+        const double gv[3] = {p0[v], p1[v], p2[v]};
+        const double dEdr = px[v] / rc;
+        const double gr = gv[0] * u[0] + gv[1] * u[1] + gv[2] * u[2];
+        double fv[3];
+        for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + (gv[d] - gr * u[d]) / r;
+        const int jj = a.ej[e];
+        for (int d = 0; d < 3; d++) {
+          fi[d] += fv[d];
+          atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
+        }
+        const double ddx = -u[0] * r, ddy = -u[1] * r, ddz = -u[2] * r;
+        vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
+        vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  double vsum[9] = {fi[0], fi[1], fi[2], vir[0], vir[1], vir[2], vir[3], vir[4], vir[5]};
+#pragma unroll
+  for (int k = 0; k < 9; k++)
+    for (int o = 32; o > 0; o >>= 1) vsum[k] += __shfl_xor(vsum[k], o, 64);
+  if (lane == 0)
+    for (int k = 0; k < 9; k++) red[wave][k] = vsum[k];
+  __syncthreads();
+  if (t < 9) {
+    const double s = red[0][t] + red[1][t] + red[2][t] + red[3][t];
+    if (e1 > e0) {
+      if (t < 3) atomicAdd(&a.f[3 * (long long) i + t], s);
+      else atomicAdd(&a.virial[t - 3], s);
     }
   }
 }
