@@ -75,6 +75,7 @@ def main():
     model = kk.Model(mpath)
     eng = kk.Engine(model, ["W"], precision=a.precision)
     eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
+    eng.debug_copy(1 << 30)     # k_copy_calibration over 1 GiB: scales the rocprof FETCH_SIZE / WRITE_SIZE counters
 
     for _ in range(a.warmup):
         eng.run()

@@ -21,7 +21,7 @@ SYMBOLS = [
     "gr_model_element_name", "gr_model_free", "gr_engine_create", "gr_engine_free", "gr_engine_cutoff",
     "gr_compute_csr", "gr_engine_upload", "gr_engine_run", "gr_engine_sync", "gr_engine_fetch",
     "gr_engine_edge_count", "gr_engine_set_profile", "gr_engine_stage_count", "gr_engine_stage_get",
-    "gr_engine_debug_radial", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
+    "gr_engine_debug_radial", "gr_engine_debug_copy", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
     "gr_nlist_free", "gr_compute",
 ]
 
@@ -68,6 +68,7 @@ def lib():
     L.gr_engine_stage_count.argtypes = [vp]
     L.gr_engine_stage_get.argtypes = [vp, i32, C.c_char_p, i32, C.POINTER(dbl), C.POINTER(i32)]
     L.gr_engine_debug_radial.argtypes = [vp, i32, vp, vp, vp, vp]
+    L.gr_engine_debug_copy.argtypes = [vp, i64]
     L.gr_neighbor_build.argtypes = [i64, vp, vp, vp, dbl, i32, C.POINTER(vp)]
     L.gr_nlist_nbonds.restype = i64
     L.gr_nlist_nbonds.argtypes = [vp]

@@ -262,6 +262,14 @@ int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j
   });
 }
 
+int gr_engine_debug_copy(gr_engine *e, int64_t bytes)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->debug_copy(bytes);
+  });
+}
+
 int gr_neighbor_build(int64_t n, const double *positions, const double *cell, const unsigned char *pbc, double cutoff,
                       int nthreads, gr_nlist **out)
 {

@@ -51,6 +51,8 @@ class Engine {
   virtual void set_profile(bool on) = 0;
   virtual const std::vector<StageTime> &stage_times() = 0;
   virtual int64_t last_edge_count() = 0;
+  // a plain device-to-device copy kernel over `bytes` bytes (calibration of the memory-traffic counters)
+  virtual void debug_copy(int64_t bytes) = 0;
   // radial functions of the device kernel for the given x = r / rc and neighbour elements: R z and dR/dx z,
   // [m][nl][C] (tests of the MFMA kernel against the CPU restatement)
   virtual void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) = 0;

@@ -269,6 +269,18 @@ template<class T> class Engine1L final : public Engine {
     return e;
   }
   void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) override;
+  void debug_copy(int64_t bytes) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    const long long nd = std::max<int64_t>(bytes / 8, 1);
+    DevBuf a, b;
+    a.ensure(nd * 8);
+    b.ensure(nd * 8);
+    HIP_CHECK(hipMemsetAsync(a.p, 0, nd * 8, stream_));
+    hipLaunchKernelGGL(k_copy_calibration, dim3(4096), dim3(256), 0, stream_, a.as<double>(), b.as<double>(), nd);
+    HIP_CHECK(hipGetLastError());
+    HIP_CHECK(hipStreamSynchronize(stream_));
+  }
 
  private:
   std::shared_ptr<const Model1L> model_;
@@ -806,7 +818,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   auto prod_fwd = [&](const char *name, DevProd &P, const T *L, const T *R, T *out, int sl, int sr) {
     const int AT = std::max(1, 256 / CFP_);
     stage(name, [&] {
-      hipLaunchKernelGGL(k_prod_fwd<T>, dim3(P.d.nout, (n + AT - 1) / AT), dim3(CFP_ * AT), 0, stream_, P.d, L, R, out, n, CFP_, sl, sr);
+      hipLaunchKernelGGL(k_prod_fwd<T>, dim3(P.d.nout * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(CFP_ * AT), 0, stream_, P.d, L, R, out, n, CFP_, sl, sr);
     });
   };
   T *A = A_.as<T>(), *A1 = A1_.as<T>(), *AA = AA_.as<T>(), *AA1 = AA1_.as<T>(), *AA2 = AA2_.as<T>(), *AAA = AAA_.as<T>(),
@@ -870,8 +882,8 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   auto prod_bwd = [&](const char *name, DevProd &P, const T *L, const T *R, const T *g, T *gL, T *gR, int sl, int sr) {
     const int AT = std::max(1, 256 / CFP_);
     stage(name, [&] {
-      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nleft, (n + AT - 1) / AT), dim3(CFP_ * AT), 0, stream_, P.d, 0, R, g, gL, n, CFP_, sr, sl);
-      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nright, (n + AT - 1) / AT), dim3(CFP_ * AT), 0, stream_, P.d, 1, L, g, gR, n, CFP_, sl, sr);
+      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nleft * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(CFP_ * AT), 0, stream_, P.d, 0, R, g, gL, n, CFP_, sr, sl);
+      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nright * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(CFP_ * AT), 0, stream_, P.d, 1, L, g, gR, n, CFP_, sl, sr);
     });
   };
   // FC reverse: left input (same functions as the output), then right input (functions of A)

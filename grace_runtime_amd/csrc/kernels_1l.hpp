@@ -98,6 +98,12 @@ __device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz
   }
 }
 
+// plain copy of n doubles: the calibration kernel for the HBM counters (FETCH_SIZE / WRITE_SIZE per byte moved)
+__global__ void k_copy_calibration(const double *src, double *dst, long long n)
+{
+  for (long long i = blockIdx.x * (long long) blockDim.x + threadIdx.x; i < n; i += (long long) gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // bond filter
 // ---------------------------------------------------------------------------------------------------------------
@@ -569,6 +575,16 @@ __global__ __launch_bounds__(256) void k_gemm_jobs(GemmJobs<T> J, const T *X0, i
   }
 }
 
+// Block index -> (function q, atom group) for grids of nq * 8 * ceil(groups / 8) blocks.  Workgroups go to the 8 XCDs
+// round-robin by linear index and every XCD has its own L2: the blocks of one atom group (all its functions q) are
+// given consecutive indices on ONE XCD, so that the per-atom tensors they share are fetched into one L2 once.
+__device__ inline void xcd_block(int nq, int &q, int &group)
+{
+  const int L = blockIdx.x, xcd = L & 7, rest = L >> 3;
+  q = rest % nq;
+  group = (rest / nq) * 8 + xcd;
+}
+
 struct ProdDev {
   // forward: terms sorted by output (CSR off over nout; only live outputs have terms)
   const int *off, *l, *r;
@@ -581,13 +597,14 @@ struct ProdDev {
   int nout, nleft, nright;
 };
 
-// out[a][o][k] = sum_t c_t L[a][l_t][k] R[a][r_t][k]      grid (nout, atom groups), block = C x AT
+// out[a][o][k] = sum_t c_t L[a][l_t][k] R[a][r_t][k]      grid: xcd_block over (nout, atom groups), block = C x AT
 template<class T> __global__ void k_prod_fwd(ProdDev P, const T *L, const T *R, T *out, int natoms, int C, int sl, int sr)
 {
   const int k = threadIdx.x % C, al = threadIdx.x / C;
-  const int at = blockIdx.y * (blockDim.x / C) + al;
+  int o, ag;
+  xcd_block(P.nout, o, ag);
+  const int at = ag * (blockDim.x / C) + al;
   if (at >= natoms) return;
-  const int o = blockIdx.x;
   const T *La = L + (long long) at * sl * C + k, *Ra = R + (long long) at * sr * C + k;
   T acc = (T) 0;
   for (int t = P.off[o]; t < P.off[o + 1]; t++) acc += (T) P.c[t] * La[(long long) P.l[t] * C] * Ra[(long long) P.r[t] * C];
@@ -600,9 +617,10 @@ template<class T> __global__ void k_prod_bwd(ProdDev P, int side, const T *other
                                              int sx)
 {
   const int k = threadIdx.x % C, al = threadIdx.x / C;
-  const int at = blockIdx.y * (blockDim.x / C) + al;
+  int q, ag;
+  xcd_block(side == 0 ? P.nleft : P.nright, q, ag);
+  const int at = ag * (blockDim.x / C) + al;
   if (at >= natoms) return;
-  const int q = blockIdx.x;
   const int *off = side == 0 ? P.loff : P.roff, *oo = side == 0 ? P.l_o : P.r_o, *ot = side == 0 ? P.l_r : P.r_l;
   const double *cc = side == 0 ? P.l_c : P.r_c;
   if (off[q] == off[q + 1]) return;

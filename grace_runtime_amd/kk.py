@@ -261,6 +261,9 @@ class Engine:
         check(_lib.lib().gr_engine_debug_radial(self._h, x.shape[0], ptr(x), ptr(mu_j), ptr(R), ptr(dR)))
         return R, dR
 
+    def debug_copy(self, nbytes):
+        check(_lib.lib().gr_engine_debug_copy(self._h, int(nbytes)))
+
     def close(self):
         if getattr(self, "_h", None):
             _lib.lib().gr_engine_free(self._h)

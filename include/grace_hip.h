@@ -98,6 +98,10 @@ int gr_engine_stage_get(gr_engine *e, int k, char *name, int name_len, double *m
  * Test hook for the radial-MLP kernel (the reference's counterpart is radial_x.h:29-60 evaluated on the host). */
 int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz);
 
+/* Runs a plain device-to-device copy kernel (k_copy_calibration) over `bytes` bytes: the known-size kernel that the
+ * rocprof memory counters (FETCH_SIZE, WRITE_SIZE) are scaled by.  No counterpart in the reference. */
+int gr_engine_debug_copy(gr_engine *e, int64_t bytes);
+
 /* Neighbour list at `cutoff`, the exact list of grace_runtime::neighbor_search (python/src/neighbors.cpp:15-95):
  * perm [n] (new -> original index), offset [n+1], j [nb] (new indices), image [nb], shifts [nimages][3]. */
 int gr_neighbor_build(int64_t n, const double *positions, const double *cell, const unsigned char *pbc, double cutoff,
