@@ -3,6 +3,7 @@
 // and the staged GPU pipeline of libgrace/include/grace/kk/grace_1l_kk.h:449-454; liveness pruning of FC outputs and
 // CG terms after libgrace/src/fused_1l.cpp:176-216.
 #include "engine.hpp"
+#include "jit_prod.hpp"
 #include "kernels_1l.hpp"
 
 #include <algorithm>
@@ -65,6 +66,7 @@ struct HostProd {
   std::vector<double> c;
   std::vector<int> loff, l_o, l_r, roff, r_o, r_l;
   std::vector<double> l_c, r_c;
+  std::vector<ProdTerm> terms;    // the kept terms, for the specialised kernels
   int nout = 0, nleft = 0, nright = 0;
 };
 
@@ -85,6 +87,7 @@ HostProd build_prod(const CGProduct &p, const std::vector<char> &need, int nleft
     h.r.push_back(p.right_ind[t]);
     h.c.push_back(p.cg_coeff[t]);
     h.off[p.m_sum_ind[t] + 1]++;
+    h.terms.push_back({p.left_ind[t], p.right_ind[t], p.m_sum_ind[t], p.cg_coeff[t]});
   }
   for (int o = 0; o < h.nout; o++) h.off[o + 1] += h.off[o];
   auto by_operand = [&](const std::vector<int> &key, int nkey, std::vector<int> &off, std::vector<int> &oo,
@@ -108,6 +111,9 @@ HostProd build_prod(const CGProduct &p, const std::vector<char> &need, int nleft
 struct DevProd {
   DevBuf off, l, r, c, loff, l_o, l_r, l_c, roff, r_o, r_l, r_c;
   ProdDev d{};
+  JitKernels jit;        // model-specialised kernels (jit_prod.hpp); not ok(): the table-driven kernels run
+  std::string jit_note;
+  ~DevProd() { jit.release(); }
   void build(const HostProd &h)
   {
     upload_vec(off, h.off); upload_vec(l, h.l); upload_vec(r, h.r); upload_vec(c, h.c);
@@ -230,6 +236,7 @@ template<class T> class Engine1L final : public Engine {
     if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0 && std::string(prop.gcnArchName).rfind("gfx942", 0) != 0)
       throw Error(std::string("this library is built for gfx950 (MI355X); device is ") + prop.gcnArchName);
     ncu_ = prop.multiProcessorCount;
+    arch_ = prop.gcnArchName;
     HIP_CHECK(hipStreamCreate(&stream_));
     probe_mfma();
     build();
@@ -287,6 +294,8 @@ template<class T> class Engine1L final : public Engine {
   int ntypes_;
   std::vector<int> type2mu_;
   int device_, ncu_ = 256;
+  std::string arch_;
+  bool jit_all_ = false;
   hipStream_t stream_ = nullptr;
   bool profile_ = false;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> events_;
@@ -548,6 +557,14 @@ template<class T> void Engine1L<T>::build()
     pAA_.build(hAA);
     pAAA_.build(hAAA);
     if (order4_) pAAAA_.build(hAAAA);
+    {
+      const bool f32 = sizeof(T) == 4;
+      jit_compile_product("prod_AA", hAA.terms, nlm_, nlm_, nAA_, true, CFP_, f32, arch_, pAA_.jit, pAA_.jit_note);
+      if (!(aaa_a_ && CP_ != CFP_))
+        jit_compile_product("prod_AAA", hAAA.terms, nAA_, nlm_, nAAA_, false, CFP_, f32, arch_, pAAA_.jit, pAAA_.jit_note);
+      if (order4_) jit_compile_product("prod_AAAA", hAAAA.terms, nAA_, nAA_, nAAAA_, true, CFP_, f32, arch_, pAAAA_.jit, pAAAA_.jit_note);
+      jit_all_ = pAA_.jit.ok() && pAAA_.jit.ok() && (!order4_ || pAAAA_.jit.ok());
+    }
     fcA1_.build(m.fc_A1, liveA1, nlm_, CP_, CP_, CFP_, drow_);
     fcAA1_.build(m.fc_AA1, liveAA1, nlm_, CFP_, CP_, CFP_, drow_);
     if (order4_) fcAA2_.build(m.fc_AA2, liveAA2, nlm_, CFP_, CP_, CFP_, drow_);
@@ -815,8 +832,17 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
 
   const int *tiles = tiles_.as<int>();
   const int ka = CP_ / 16, kf = CFP_ / 16;
+  auto jit_launch = [&](hipFunction_t f, std::vector<void *> args) {
+    const long long cols = (long long) n * CFP_;
+    HIP_CHECK(hipModuleLaunchKernel(f, (unsigned) ((cols + 255) / 256), 1, 1, 256, 1, 1, 0, stream_, args.data(), nullptr));
+  };
+  int one = 1, nat = n;
   auto prod_fwd = [&](const char *name, DevProd &P, const T *L, const T *R, T *out, int sl, int sr) {
     const int AT = std::max(1, 256 / CFP_);
+    if (P.jit.ok()) {
+      stage(name, [&] { jit_launch(P.jit.fwd, {(void *) &L, (void *) &R, (void *) &out, (void *) &nat, (void *) &one}); });
+      return;
+    }
     stage(name, [&] {
       hipLaunchKernelGGL(k_prod_fwd<T>, dim3(P.d.nout * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(CFP_ * AT), 0, stream_, P.d, L, R, out, n, CFP_, sl, sr);
     });
@@ -866,10 +892,11 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     HIP_CHECK(hipMemsetAsync(gA, 0, na * nlm_ * CP_ * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(gA1, 0, na * nlm_ * CFP_ * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(gAA, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
-    HIP_CHECK(hipMemsetAsync(gAA1, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
+    // with the specialised product kernels gAA1 and gAA2 are written (not accumulated) by their first producer
+    if (!jit_all_) HIP_CHECK(hipMemsetAsync(gAA1, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(gAAA, 0, na * nAAA_ * CFP_ * sizeof(T), stream_));
     if (order4_) {
-      HIP_CHECK(hipMemsetAsync(gAA2, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
+      if (!jit_all_) HIP_CHECK(hipMemsetAsync(gAA2, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
       HIP_CHECK(hipMemsetAsync(gAAAA, 0, na * nAAAA_ * CFP_ * sizeof(T), stream_));
     }
   });
@@ -879,8 +906,17 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, njobs), dim3(64), 0, stream_, red_, mu_.as<int>(), tiles, grho_.as<double>(), gA, gAA,
                        gAAA, gAAAA);
   });
-  auto prod_bwd = [&](const char *name, DevProd &P, const T *L, const T *R, const T *g, T *gL, T *gR, int sl, int sr) {
+  // accL / accR: add to the stored adjoint or overwrite it (specialised kernels; the table-driven ones always add)
+  auto prod_bwd = [&](const char *name, DevProd &P, const T *L, const T *R, const T *g, T *gL, T *gR, int sl, int sr, int accL, int accR) {
     const int AT = std::max(1, 256 / CFP_);
+    if (P.jit.ok()) {
+      if (!jit_all_) accL = accR = 1;
+      stage(name, [&] {
+        jit_launch(P.jit.bwd, {(void *) &L, (void *) &R, (void *) &g, (void *) &gL, (void *) &gR, (void *) &accL, (void *) &accR, (void *) &nat,
+                               (void *) &one});
+      });
+      return;
+    }
     stage(name, [&] {
       hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nleft * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(CFP_ * AT), 0, stream_, P.d, 0, R, g, gL, n, CFP_, sr, sl);
       hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nright * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(CFP_ * AT), 0, stream_, P.d, 1, L, g, gR, n, CFP_, sl, sr);
@@ -894,12 +930,12 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     });
   };
   if (order4_) {
-    prod_bwd("prod_AAAA_bwd", pAAAA_, AA2, AA2, gAAAA, gAA2, gAA2, nAA_, nAA_);
+    prod_bwd("prod_AAAA_bwd", pAAAA_, AA2, AA2, gAAAA, gAA2, gAA2, nAA_, nAA_, 0, 0);
     fc_bwd("fc_AA2_bwd", fcAA2_, gAA2, gAA, gA, nAA_, kf);
   }
-  prod_bwd("prod_AAA_bwd", pAAA_, AA1, Ar, gAAA, gAA1, aaa_a_ ? gA : gA1, nAA_, nlm_);
+  prod_bwd("prod_AAA_bwd", pAAA_, AA1, Ar, gAAA, gAA1, aaa_a_ ? gA : gA1, nAA_, nlm_, 0, 1);
   fc_bwd("fc_AA1_bwd", fcAA1_, gAA1, gAA, gA, nAA_, kf);
-  prod_bwd("prod_AA_bwd", pAA_, A1, A1, gAA, gA1, gA1, nlm_, nlm_);
+  prod_bwd("prod_AA_bwd", pAA_, A1, A1, gAA, gA1, gA1, nlm_, nlm_, 1, 1);
   fc_bwd("fc_A1_bwd", fcA1_, gA1, gA, gA, nlm_, ka);
 
   BondBwdArgs<T> ba{};
