@@ -752,12 +752,9 @@ void Engine1L<T>::launch_radial(long long e_begin, long long e_count, const doub
   ra.w2_in_lds = w2_in_lds_;
   for (int q = 0; q < 16; q++) ra.drow[q] = drow_[q];
   const int threads = hb_ == 4 ? 512 : 256;
-  auto kern = hb_ == 4 ? k_radial<T, 4> : k_radial<T, 8>;
-  static bool attr_set[2] = {false, false};
-  if (!attr_set[hb_ == 8]) {
-    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    attr_set[hb_ == 8] = true;
-  }
+  const int act = model_->radial_activation;
+  auto kern = hb_ == 4 ? (act == 1 ? k_radial<T, 4, 1> : k_radial<T, 4, 0>) : (act == 1 ? k_radial<T, 8, 1> : k_radial<T, 8, 0>);
+  HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
   hipLaunchKernelGGL(kern, dim3(ncu_), dim3(threads), rad_lds_, stream_, ra);
 }
 

@@ -264,24 +264,53 @@ template<class T> struct RadialArgs {
   int drow[16];               // accumulator row of (lane / 16, register)
 };
 
-template<class T> __device__ inline void act_pair(int act, T &s, T &ds)
+// reciprocal: hardware estimate + Newton steps (2 in fp64: full precision; 1 in fp32)
+__device__ inline double fast_rcp(double x)
 {
-  if (act == 1) {
+  double r = __builtin_amdgcn_rcp(x);
+  r = fma(fma(-x, r, 1.0), r, r);
+  r = fma(fma(-x, r, 1.0), r, r);
+  return r;
+}
+__device__ inline float fast_rcp(float x)
+{
+  float r = __builtin_amdgcn_rcpf(x);
+  return fmaf(fmaf(-x, r, 1.0f), r, r);
+}
+
+template<class T, int ACT> __device__ inline void act_pair(T &s, T &ds)
+{
+  if (ACT == 1) {
     const T t = tanh(s);
     ds = ds * ((T) 1 - t * t);
     s = t;
   } else {
-    const T sg = (T) 1 / ((T) 1 + exp(-s));
+    const T sg = fast_rcp((T) 1 + exp(-s));
     ds = sg * ((T) 1 + s * ((T) 1 - sg)) * ds;
     s = s * sg;
   }
+}
+
+// x^n for a non-negative integer n by squaring
+__device__ inline double ipow(double x, int n)
+{
+  double r = 1.0, b = x;
+  while (n > 0) {
+    if (n & 1) r *= b;
+    b *= b;
+    n >>= 1;
+  }
+  return r;
 }
 
 // One wave = 16 edges.  Layers 0 and 1 run as D[feature][edge] = W^T H with the weights as the A operand, so the
 // accumulator registers of one layer are exactly the B operand of the next (no data movement between layers: the
 // k index of a step is the accumulator row held by that lane, and the weight fragments are stored in that order).
 // Layer 2 swaps the operands, D[edge][column], so that 16 lanes write 16 consecutive columns of one edge row.
-template<class T, int HB> __global__ __launch_bounds__(512) void k_radial(RadialArgs<T> a)
+// Every k-step feeds all row blocks of the value and the tangent stream (2 HB independent accumulator chains).
+// ACT: 0 SiLU, 1 tanh (compile-time: the fp64 tanh is large, and both activations inlined 32 times overflow the
+// instruction cache).
+template<class T, int HB, int ACT> __global__ __launch_bounds__(512) void k_radial(RadialArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -301,6 +330,7 @@ template<class T, int HB> __global__ __launch_bounds__(512) void k_radial(Radial
   const long long cnt = a.e_count >= 0 ? a.e_count : *a.n_edges - a.e_begin;
   const long long ntiles = (cnt + 15) / 16;
   const int p = a.p;
+  const double cf0 = 0.5 * (p + 1) * (p + 2), cf1 = (double) p * (p + 2), cf2 = 0.5 * p * (p + 1), cfd = 0.5 * p * (p + 1) * (p + 2);
   for (long long tile = (long long) blockIdx.x * nw + wave; tile < ntiles; tile += (long long) gridDim.x * nw) {
     const long long eloc = tile * 16 + c;
     const long long e = a.e_begin + eloc;
@@ -308,9 +338,9 @@ template<class T, int HB> __global__ __launch_bounds__(512) void k_radial(Radial
     // basis g_k = T_k(2x - 1) fcut_p(x), k = 1..nrb, and d/dx (radial_x.h:11-26); this lane supplies k = 4 s + g
     T h0[kMaxRadBasis / 4], dh0[kMaxRadBasis / 4];
     {
-      const double xp = pow(x, (double) p), xp1 = xp * x, xp2 = xp1 * x;
-      const double fc = 1.0 - 0.5 * (p + 1) * (p + 2) * xp + (double) p * (p + 2) * xp1 - 0.5 * p * (p + 1) * xp2;
-      const double dfc = 0.5 * p * (p + 1) * (p + 2) * (-pow(x, (double) (p - 1)) + 2.0 * xp - xp1);
+      const double xpm = ipow(x, p - 1), xp = xpm * x, xp1 = xp * x, xp2 = xp1 * x;
+      const double fc = 1.0 - cf0 * xp + cf1 * xp1 - cf2 * xp2;
+      const double dfc = cfd * (-xpm + 2.0 * xp - xp1);
       const double t = 2.0 * x - 1.0;
       double Tp = 1.0, Tc = t, dTp = 0.0, dTc = 2.0;
 #pragma unroll
@@ -329,71 +359,86 @@ template<class T, int HB> __global__ __launch_bounds__(512) void k_radial(Radial
     // ---- layer 0
     v4 h1[HB], dh1[HB];
 #pragma unroll
-    for (int rb = 0; rb < HB; rb++) {
-      v4 acc = {0, 0, 0, 0}, dacc = {0, 0, 0, 0};
+    for (int rb = 0; rb < HB; rb++) { h1[rb] = v4{0, 0, 0, 0}; dh1[rb] = v4{0, 0, 0, 0}; }
 #pragma unroll
-      for (int s = 0; s < kMaxRadBasis / 4; s++)
-        if (s < a.ks0) {
+    for (int s = 0; s < kMaxRadBasis / 4; s++)
+      if (s < a.ks0) {
+#pragma unroll
+        for (int rb = 0; rb < HB; rb++) {
           const T w = w0s[(rb * a.ks0 + s) * 64 + lane];
-          acc = Mfma<T>::mma(w, h0[s], acc);
-          dacc = Mfma<T>::mma(w, dh0[s], dacc);
+          h1[rb] = Mfma<T>::mma(w, h0[s], h1[rb]);
+          dh1[rb] = Mfma<T>::mma(w, dh0[s], dh1[rb]);
         }
+      }
+#pragma unroll
+    for (int rb = 0; rb < HB; rb++)
 #pragma unroll
       for (int v = 0; v < 4; v++) {
-        T s_ = acc[v], d_ = dacc[v];
-        act_pair<T>(a.act, s_, d_);
-        acc[v] = s_; dacc[v] = d_;
+        T s_ = h1[rb][v], d_ = dh1[rb][v];
+        act_pair<T, ACT>(s_, d_);
+        h1[rb][v] = s_; dh1[rb][v] = d_;
       }
-      h1[rb] = acc; dh1[rb] = dacc;
-    }
     // ---- layer 1
     v4 h2[HB], dh2[HB];
 #pragma unroll
-    for (int rb = 0; rb < HB; rb++) {
-      v4 acc = {0, 0, 0, 0}, dacc = {0, 0, 0, 0};
+    for (int rb = 0; rb < HB; rb++) { h2[rb] = v4{0, 0, 0, 0}; dh2[rb] = v4{0, 0, 0, 0}; }
 #pragma unroll
-      for (int kb = 0; kb < HB; kb++)
+    for (int kb = 0; kb < HB; kb++)
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
+      for (int s = 0; s < 4; s++) {
+        const T b = h1[kb][s], db = dh1[kb][s];
+#pragma unroll
+        for (int rb = 0; rb < HB; rb++) {
           const T w = w1s[((rb * HB + kb) * 4 + s) * 64 + lane];
-          acc = Mfma<T>::mma(w, h1[kb][s], acc);
-          dacc = Mfma<T>::mma(w, dh1[kb][s], dacc);
+          h2[rb] = Mfma<T>::mma(w, b, h2[rb]);
+          dh2[rb] = Mfma<T>::mma(w, db, dh2[rb]);
         }
+      }
+#pragma unroll
+    for (int rb = 0; rb < HB; rb++)
 #pragma unroll
       for (int v = 0; v < 4; v++) {
-        T s_ = acc[v], d_ = dacc[v];
-        act_pair<T>(a.act, s_, d_);
-        acc[v] = s_; dacc[v] = d_;
+        T s_ = h2[rb][v], d_ = dh2[rb][v];
+        act_pair<T, ACT>(s_, d_);
+        h2[rb][v] = s_; dh2[rb][v] = d_;
       }
-      h2[rb] = acc; dh2[rb] = dacc;
-    }
-    // ---- layer 2 (linear), operands swapped: rows = edges, columns = outputs
-    int mu_v[4];
-    long long e_v[4];
+    // ---- layer 2 (linear), operands swapped: rows = edges, columns = outputs; two column blocks at a time
+    long long row_v[4];
+    const T *z_v[4];
 #pragma unroll
     for (int v = 0; v < 4; v++) {
       const long long el = tile * 16 + a.drow[g * 4 + v];
-      e_v[v] = el < cnt ? a.e_begin + el : -1;
-      mu_v[v] = el < cnt ? a.emu[a.e_begin + el] : 0;
+      row_v[v] = el < cnt ? (a.e_begin + el) * a.noutp : -1;
+      z_v[v] = a.z + (el < cnt ? a.emu[a.e_begin + el] : 0) * a.C;
     }
-    for (int cb = 0; cb < a.nob; cb++) {
-      v4 acc = {0, 0, 0, 0}, dacc = {0, 0, 0, 0};
+    for (int cb = 0; cb < a.nob; cb += 2) {
+      const bool two = cb + 1 < a.nob;
+      v4 acc0 = {0, 0, 0, 0}, dacc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0}, dacc1 = {0, 0, 0, 0};
+      const T *wa = w2p + (long long) cb * HB * 4 * 64 + lane;
+      const T *wb = two ? wa + HB * 4 * 64 : wa;
 #pragma unroll
       for (int kb = 0; kb < HB; kb++)
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-          const T w = w2p[((cb * HB + kb) * 4 + s) * 64 + lane];
-          acc = Mfma<T>::mma(h2[kb][s], w, acc);
-          dacc = Mfma<T>::mma(dh2[kb][s], w, dacc);
+          const T w0_ = wa[(kb * 4 + s) * 64], w1_ = wb[(kb * 4 + s) * 64];
+          acc0 = Mfma<T>::mma(h2[kb][s], w0_, acc0);
+          dacc0 = Mfma<T>::mma(dh2[kb][s], w0_, dacc0);
+          acc1 = Mfma<T>::mma(h2[kb][s], w1_, acc1);
+          dacc1 = Mfma<T>::mma(dh2[kb][s], w1_, dacc1);
         }
-      const int col = cb * 16 + c;
-      const int nch = col % a.C;
+      const int col0 = cb * 16 + c, col1 = col0 + 16;
+      const int n0 = col0 % a.C, n1 = col1 % a.C;
 #pragma unroll
       for (int v = 0; v < 4; v++)
-        if (e_v[v] >= 0) {
-          const T zz = a.z[mu_v[v] * a.C + nch];
-          a.Rz[e_v[v] * a.noutp + col] = acc[v] * zz;
-          a.dRz[e_v[v] * a.noutp + col] = dacc[v] * zz;
+        if (row_v[v] >= 0) {
+          const T zz0 = z_v[v][n0];
+          a.Rz[row_v[v] + col0] = acc0[v] * zz0;
+          a.dRz[row_v[v] + col0] = dacc0[v] * zz0;
+          if (two) {
+            const T zz1 = z_v[v][n1];
+            a.Rz[row_v[v] + col1] = acc1[v] * zz1;
+            a.dRz[row_v[v] + col1] = dacc1[v] * zz1;
+          }
         }
     }
   }
