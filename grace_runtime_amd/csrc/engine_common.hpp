@@ -1,0 +1,545 @@
+// Host-side building blocks shared by the engines: device buffers, the CG-product tables, MFMA fragment packing, the
+// tile-GEMM job lists of the FC layers, and the stream / profiling base of an engine.
+#pragma once
+
+#include "engine.hpp"
+#include "jit_prod.hpp"
+#include "kernels_1l.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <numeric>
+
+namespace grhip {
+
+#define HIP_CHECK(expr)                                                                                         \
+  do {                                                                                                          \
+    hipError_t e_ = (expr);                                                                                     \
+    if (e_ != hipSuccess)                                                                                       \
+      throw Error(std::string("HIP error: ") + hipGetErrorString(e_) + " in " #expr " (" __FILE__ ":" + std::to_string(__LINE__) + ")"); \
+  } while (0)
+
+// device allocation owned by the engine
+struct DevBuf {
+  void *p = nullptr;
+  size_t bytes = 0;
+  DevBuf() = default;
+  DevBuf(const DevBuf &) = delete;
+  DevBuf &operator=(const DevBuf &) = delete;
+  ~DevBuf() { release(); }
+  void release()
+  {
+    if (p) (void) hipFree(p);
+    p = nullptr;
+    bytes = 0;
+  }
+  // at least `need` bytes (grown with head room; contents are not kept)
+  void ensure(size_t need)
+  {
+    if (need <= bytes && p) return;
+    release();
+    const size_t want = std::max<size_t>(need + need / 8, 256);
+    hipError_t e = hipMalloc(&p, want);
+    if (e != hipSuccess) {
+      p = nullptr;
+      (void) hipGetLastError();
+      throw std::bad_alloc();
+    }
+    bytes = want;
+  }
+  template<class U> U *as() const { return static_cast<U *>(p); }
+};
+
+template<class U> void upload_vec(DevBuf &b, const std::vector<U> &v)
+{
+  b.ensure(std::max<size_t>(v.size(), 1) * sizeof(U));
+  if (!v.empty()) HIP_CHECK(hipMemcpy(b.p, v.data(), v.size() * sizeof(U), hipMemcpyHostToDevice));
+}
+
+inline int round_up(int a, int b) { return (a + b - 1) / b * b; }
+
+struct HostProd {
+  std::vector<int> off, l, r;
+  std::vector<double> c;
+  std::vector<int> loff, l_o, l_r, roff, r_o, r_l;
+  std::vector<double> l_c, r_c;
+  std::vector<ProdTerm> terms;    // the kept terms, for the specialised kernels
+  int nout = 0, nleft = 0, nright = 0;
+};
+
+// terms of outputs with need[o] set, sorted by output; operand-major copies for the reverse
+inline HostProd build_prod(const CGProduct &p, const std::vector<char> &need, int nleft, int nright)
+{
+  HostProd h;
+  h.nout = p.n_out;
+  h.nleft = nleft;
+  h.nright = nright;
+  std::vector<int> ord;
+  for (int t = 0; t < p.n_terms; t++)
+    if (need[p.m_sum_ind[t]]) ord.push_back(t);
+  std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return p.m_sum_ind[a] < p.m_sum_ind[b]; });
+  h.off.assign(h.nout + 1, 0);
+  for (int t : ord) {
+    h.l.push_back(p.left_ind[t]);
+    h.r.push_back(p.right_ind[t]);
+    h.c.push_back(p.cg_coeff[t]);
+    h.off[p.m_sum_ind[t] + 1]++;
+    h.terms.push_back({p.left_ind[t], p.right_ind[t], p.m_sum_ind[t], p.cg_coeff[t]});
+  }
+  for (int o = 0; o < h.nout; o++) h.off[o + 1] += h.off[o];
+  auto by_operand = [&](const std::vector<int> &key, int nkey, std::vector<int> &off, std::vector<int> &oo,
+                        std::vector<int> &other, std::vector<double> &cc, const std::vector<int> &oth) {
+    std::vector<int> o2 = ord;
+    std::stable_sort(o2.begin(), o2.end(), [&](int a, int b) { return key[a] < key[b]; });
+    off.assign(nkey + 1, 0);
+    for (int t : o2) {
+      oo.push_back(p.m_sum_ind[t]);
+      other.push_back(oth[t]);
+      cc.push_back(p.cg_coeff[t]);
+      off[key[t] + 1]++;
+    }
+    for (int q = 0; q < nkey; q++) off[q + 1] += off[q];
+  };
+  by_operand(p.left_ind, nleft, h.loff, h.l_o, h.l_r, h.l_c, p.right_ind);
+  by_operand(p.right_ind, nright, h.roff, h.r_o, h.r_l, h.r_c, p.left_ind);
+  return h;
+}
+
+struct DevProd {
+  DevBuf off, l, r, c, loff, l_o, l_r, l_c, roff, r_o, r_l, r_c;
+  ProdDev d{};
+  JitKernels jit;        // model-specialised kernels (jit_prod.hpp); not ok(): the table-driven kernels run
+  std::string jit_note;
+  ~DevProd() { jit.release(); }
+  void build(const HostProd &h)
+  {
+    upload_vec(off, h.off); upload_vec(l, h.l); upload_vec(r, h.r); upload_vec(c, h.c);
+    upload_vec(loff, h.loff); upload_vec(l_o, h.l_o); upload_vec(l_r, h.l_r); upload_vec(l_c, h.l_c);
+    upload_vec(roff, h.roff); upload_vec(r_o, h.r_o); upload_vec(r_l, h.r_l); upload_vec(r_c, h.r_c);
+    d.off = off.as<int>(); d.l = l.as<int>(); d.r = r.as<int>(); d.c = c.as<double>();
+    d.loff = loff.as<int>(); d.l_o = l_o.as<int>(); d.l_r = l_r.as<int>(); d.l_c = l_c.as<double>();
+    d.roff = roff.as<int>(); d.r_o = r_o.as<int>(); d.r_l = r_l.as<int>(); d.r_c = r_c.as<double>();
+    d.nout = h.nout; d.nleft = h.nleft; d.nright = h.nright;
+  }
+};
+
+// weights W[K][N] (row-major) of a tile GEMM in MFMA fragment order [cb][s][lane]: lane (g, c) holds
+// W[g * (K / 4) + s][cb * 16 + c]
+template<class T> void pack_fragments(const std::vector<double> &W, int K, int N, int Kp, int Np, std::vector<T> &out)
+{
+  const int ks = Kp / 4, nb = Np / 16;
+  const size_t base = out.size();
+  out.resize(base + (size_t) nb * ks * 64, (T) 0);
+  for (int cb = 0; cb < nb; cb++)
+    for (int s = 0; s < ks; s++)
+      for (int lane = 0; lane < 64; lane++) {
+        const int g = lane >> 4, c = lane & 15, k = g * ks + s, n = cb * 16 + c;
+        if (k < K && n < N) out[base + ((size_t) cb * ks + s) * 64 + lane] = (T) W[(size_t) k * N + n];
+      }
+}
+
+template<class T> struct DevJobs {
+  DevBuf job_out, job_scale, seg_off, seg_src, seg_fn, seg_w, seg_scale;
+  GemmJobs<T> d{};
+  struct Host {
+    std::vector<int> job_out, seg_off{0}, seg_src, seg_fn, seg_w;
+    std::vector<T> job_scale, seg_scale;
+    void job(int out, double scale) { job_out.push_back(out); job_scale.push_back((T) scale); }
+    void seg(int src, int fn, int w, double scale) { seg_src.push_back(src); seg_fn.push_back(fn); seg_w.push_back(w); seg_scale.push_back((T) scale); }
+    void end_job() { seg_off.push_back((int) seg_src.size()); }
+  };
+  void build(const Host &h, const T *WF0, const T *WF1)
+  {
+    upload_vec(job_out, h.job_out); upload_vec(job_scale, h.job_scale); upload_vec(seg_off, h.seg_off);
+    upload_vec(seg_src, h.seg_src); upload_vec(seg_fn, h.seg_fn); upload_vec(seg_w, h.seg_w); upload_vec(seg_scale, h.seg_scale);
+    d.job_out = job_out.as<int>(); d.job_scale = job_scale.as<T>(); d.seg_off = seg_off.as<int>();
+    d.seg_src = seg_src.as<int>(); d.seg_fn = seg_fn.as<int>(); d.seg_w = seg_w.as<int>(); d.seg_scale = seg_scale.as<T>();
+    d.WF0 = WF0; d.WF1 = WF1;
+    d.njobs = (int) h.job_out.size();
+  }
+  void set_rows(const int *drow) { for (int q = 0; q < 16; q++) d.drow[q] = drow[q]; }
+};
+
+// One FC layer as three job lists (forward, reverse into the left input, reverse into the right input) over
+// fragment-ordered weight tiles.  Widths are the padded ones (multiples of 16; padding weights are zero).
+template<class T> struct DevFc {
+  DevBuf WlF, WrF, WlTF, WrTF;
+  DevJobs<T> fwd, bwd_l, bwd_r;
+  int nil = 0, nir = 0, no = 0;    // padded widths
+  // nfr: functions of the right-input tensor; livef: outputs that are computed
+  void build(const FCWeights &w, const std::vector<char> &livef, int nfr, int nil_p, int nir_p, int no_p, const int *drow)
+  {
+    nil = nil_p; nir = nir_p; no = no_p;
+    const int nt = w.tiles_left;
+    std::vector<T> fl, fr, flt, frt;
+    std::vector<double> M, Mt;
+    auto tile_mats = [&](const std::vector<double> &W, double norm, int nin, int t) {
+      M.assign((size_t) nin * w.n_out, 0.0);     // [n][k]
+      Mt.assign((size_t) w.n_out * nin, 0.0);    // [k][n]
+      for (int k = 0; k < w.n_out; k++)
+        for (int n = 0; n < nin; n++) {
+          const double v = norm * W[((size_t) k * nin + n) * nt + t];
+          M[(size_t) n * w.n_out + k] = v;
+          Mt[(size_t) k * nin + n] = v;
+        }
+    };
+    for (int t = 0; t < nt; t++) {
+      tile_mats(w.w_left, w.norm_left, w.n_in_left, t);
+      pack_fragments<T>(M, w.n_in_left, w.n_out, nil, no, fl);
+      pack_fragments<T>(Mt, w.n_out, w.n_in_left, no, nil, flt);
+      tile_mats(w.w_right, w.norm_right, w.n_in_right, t);
+      pack_fragments<T>(M, w.n_in_right, w.n_out, nir, no, fr);
+      pack_fragments<T>(Mt, w.n_out, w.n_in_right, no, nir, frt);
+    }
+    upload_vec(WlF, fl); upload_vec(WrF, fr); upload_vec(WlTF, flt); upload_vec(WrTF, frt);
+    typename DevJobs<T>::Host hf, hl, hr;
+    std::vector<std::vector<int>> conn_of(w.n_funcs), conn_from(nfr);
+    for (int c = 0; c < w.n_conn; c++) {
+      conn_of[w.collect_to[c]].push_back(c);
+      if (livef[w.collect_to[c]]) conn_from[w.collect_from[c]].push_back(c);
+    }
+    for (int f = 0; f < w.n_funcs; f++) {
+      if (!livef[f]) continue;
+      hf.job(f, w.norm_out_factor[f]);
+      hf.seg(0, f, w.w_tile_left[f], 1.0);
+      for (int c : conn_of[f]) hf.seg(1, w.collect_from[c], w.w_tile_right[c], 1.0);
+      hf.end_job();
+      hl.job(f, w.norm_out_factor[f]);
+      hl.seg(0, f, w.w_tile_left[f], 1.0);
+      hl.end_job();
+    }
+    for (int r = 0; r < nfr; r++) {
+      if (conn_from[r].empty()) continue;
+      hr.job(r, 1.0);
+      for (int c : conn_from[r]) hr.seg(0, w.collect_to[c], w.w_tile_right[c], w.norm_out_factor[w.collect_to[c]]);
+      hr.end_job();
+    }
+    fwd.build(hf, WlF.as<T>(), WrF.as<T>());
+    bwd_l.build(hl, WlTF.as<T>(), WlTF.as<T>());
+    bwd_r.build(hr, WrTF.as<T>(), WrTF.as<T>());
+    fwd.set_rows(drow); bwd_l.set_rows(drow); bwd_r.set_rows(drow);
+  }
+};
+
+
+// A 3-layer radial MLP in MFMA fragment order and the launch of the persistent radial kernel (radial_x.h:11-60 of the
+// reference; its spline tables are replaced by the exact network).  Output column l * CP + n of an edge holds
+// R_{n,l}(x) z[mu_j][n] (file order of the last layer: o = n nl + l, libgrace/src/fused_1l.cpp:123).
+template<class T> struct DevRadial {
+  DevBuf w0, w1, w2;
+  int hb = 4, ks0 = 2, nob = 0, noutp = 0, w2_in_lds = 1, nrb = 0, p = 0, act = 0, CP = 0, nel = 0;
+  size_t lds = 0;
+  int drow[16];
+  void build(const std::vector<MLPLayer> &mlp, int nradbase, int basis_p, int activation, int C, int CP_, int nl, int nel_,
+             const int *drow_, const std::string &who)
+  {
+    if (mlp.size() != 3)
+      throw Error(who + ": the GPU radial kernel implements 3-layer radial MLPs (file has " + std::to_string(mlp.size()) + ")");
+    const MLPLayer &L0 = mlp[0], &L1 = mlp[1], &L2 = mlp[2];
+    const int H1 = L0.n_out, H2 = L1.n_out;
+    if (nradbase > kMaxRadBasis) throw Error(who + ": nradbase > 16 not supported");
+    const int hmax = std::max(H1, H2);
+    if (hmax <= 64) hb = 4;
+    else if (hmax <= 128) hb = 8;
+    else throw Error(who + ": radial MLP hidden width > 128 not supported");
+    nrb = nradbase; p = basis_p; act = activation; CP = CP_; nel = nel_;
+    for (int q = 0; q < 16; q++) drow[q] = drow_[q];
+    ks0 = round_up(nradbase, 4) / 4;
+    const int nout = CP * nl;
+    noutp = round_up(nout, 16);
+    nob = noutp / 16;
+    std::vector<T> v0((size_t) hb * ks0 * 64, (T) 0), v1((size_t) hb * hb * 4 * 64, (T) 0), v2((size_t) nob * hb * 4 * 64, (T) 0);
+    for (int rb = 0; rb < hb; rb++)
+      for (int s = 0; s < ks0; s++)
+        for (int lane = 0; lane < 64; lane++) {
+          const int g = lane >> 4, r = lane & 15, kin = 4 * s + g, out = rb * 16 + r;
+          if (kin < L0.n_in && out < H1) v0[((size_t) rb * ks0 + s) * 64 + lane] = (T) (L0.norm * L0.W[(size_t) kin * H1 + out]);
+        }
+    for (int rb = 0; rb < hb; rb++)
+      for (int kb = 0; kb < hb; kb++)
+        for (int s = 0; s < 4; s++)
+          for (int lane = 0; lane < 64; lane++) {
+            const int g = lane >> 4, r = lane & 15, in = kb * 16 + drow[g * 4 + s], out = rb * 16 + r;
+            if (in < H1 && out < H2) v1[(((size_t) rb * hb + kb) * 4 + s) * 64 + lane] = (T) (L1.norm * L1.W[(size_t) in * H2 + out]);
+          }
+    for (int cb = 0; cb < nob; cb++)
+      for (int kb = 0; kb < hb; kb++)
+        for (int s = 0; s < 4; s++)
+          for (int lane = 0; lane < 64; lane++) {
+            const int g = lane >> 4, cc = lane & 15, in = kb * 16 + drow[g * 4 + s], col = cb * 16 + cc;
+            const int l = col / CP, n = col % CP, o = n * nl + l;
+            if (in < H2 && col < nout && n < C)
+              v2[(((size_t) cb * hb + kb) * 4 + s) * 64 + lane] = (T) (L2.norm * L2.W[(size_t) in * L2.n_out + o]);
+          }
+    upload_vec(w0, v0); upload_vec(w1, v1); upload_vec(w2, v2);
+    const size_t base = (v0.size() + v1.size()) * sizeof(T);
+    w2_in_lds = base + v2.size() * sizeof(T) <= 150 * 1024;
+    lds = base + (w2_in_lds ? v2.size() * sizeof(T) : 0);
+  }
+  // z: [nel][CP] species weights of the neighbour; e_count < 0: the edge count is read from *n_edges on the device
+  void launch(hipStream_t stream, int ncu, const T *z, long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
+              const long long *n_edges)
+  {
+    RadialArgs<T> ra{};
+    ra.n_edges = n_edges;
+    ra.e_begin = e_begin;
+    ra.e_count = e_count;
+    ra.x = x;
+    ra.emu = emu;
+    ra.w0 = w0.as<T>(); ra.w1 = w1.as<T>(); ra.w2 = w2.as<T>();
+    ra.z = z;
+    ra.Rz = Rz; ra.dRz = dRz;
+    ra.nrb = nrb; ra.p = p; ra.ks0 = ks0;
+    ra.nob = nob; ra.noutp = noutp;
+    ra.C = CP; ra.nel = nel; ra.act = act;
+    ra.w2_in_lds = w2_in_lds;
+    for (int q = 0; q < 16; q++) ra.drow[q] = drow[q];
+    const int threads = hb == 4 ? 512 : 256;
+    auto kern = hb == 4 ? (act == 1 ? k_radial<T, 4, 1> : k_radial<T, 4, 0>) : (act == 1 ? k_radial<T, 8, 1> : k_radial<T, 8, 0>);
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    hipLaunchKernelGGL(kern, dim3(ncu), dim3(threads), lds, stream, ra);
+  }
+};
+
+// One source of an element-dependent reduce, as the host containers give it (weights [nel][nout][nin][w_shape])
+struct ReduceSrc {
+  const std::vector<double> *W;
+  double norm;
+  int n_in, w_shape;
+  const std::vector<int> *collect_ind, *w_l_tile, *out_fn;    // out_fn: output function per connection, or null (one function)
+  int nfun, ninp;                                            // functions of the source tensor, its padded channel width
+};
+
+// Element-dependent reduce of up to 4 sources into `nout` channels of ONE output function (fused_cpu.h:1202-1273 of the
+// reference): weights per collected function in MFMA fragment order, for k_reduce_fwd / k_reduce_bwd.
+// fo >= 0 keeps the connections whose output function is fo.
+template<class T> struct DevReduce {
+  DevBuf WF[4], WB[4], Fn[4];
+  ReduceDev<T> d{};
+  int njobs = 0;
+  void build(const std::vector<ReduceSrc> &src, int nel, int nout, int fo, int ostride, int ooff, const int *drow)
+  {
+    d.nsrc = (int) src.size();
+    d.nrho = nout;
+    d.nbr = (nout + 15) / 16;
+    d.ksr = (nout + 3) / 4;
+    d.ostride = ostride;
+    d.ooff = ooff;
+    if (nout > 32) throw Error("reduce widths above 32 are not supported by the GPU reduce kernels");
+    for (int q = 0; q < 16; q++) d.drow[q] = drow[q];
+    const int krp = d.ksr * 4;
+    njobs = 0;
+    for (int s = 0; s < d.nsrc; s++) {
+      const ReduceSrc &w = src[s];
+      std::vector<int> fn;
+      for (size_t c = 0; c < w.collect_ind->size(); c++)
+        if (fo < 0 || !w.out_fn || (*w.out_fn)[c] == fo) fn.push_back((*w.collect_ind)[c]);
+      std::sort(fn.begin(), fn.end());
+      fn.erase(std::unique(fn.begin(), fn.end()), fn.end());
+      const int nc = (int) fn.size(), nin = w.n_in;
+      std::vector<T> vF, vB;
+      std::vector<double> M((size_t) nin * nout), Mt((size_t) nout * nin);
+      for (int mu = 0; mu < nel; mu++)
+        for (int u = 0; u < nc; u++) {
+          std::fill(M.begin(), M.end(), 0.0);
+          for (size_t c = 0; c < w.collect_ind->size(); c++) {
+            if ((*w.collect_ind)[c] != fn[u]) continue;
+            if (fo >= 0 && w.out_fn && (*w.out_fn)[c] != fo) continue;
+            const int tile = (*w.w_l_tile)[c];
+            for (int k = 0; k < nout; k++)
+              for (int n = 0; n < nin; n++)
+                M[(size_t) n * nout + k] += w.norm * (*w.W)[(((size_t) mu * nout + k) * nin + n) * w.w_shape + tile];
+          }
+          for (int k = 0; k < nout; k++)
+            for (int n = 0; n < nin; n++) Mt[(size_t) k * nin + n] = M[(size_t) n * nout + k];
+          pack_fragments<T>(M, nin, nout, w.ninp, d.nbr * 16, vF);      // X[atom][n] . M[n][k]
+          pack_fragments<T>(Mt, nout, nin, krp, w.ninp, vB);             // g[atom][k] . Mt[k][n]
+        }
+      upload_vec(WF[s], vF);
+      upload_vec(WB[s], vB);
+      upload_vec(Fn[s], fn);
+      d.WF[s] = WF[s].template as<T>();
+      d.WB[s] = WB[s].template as<T>();
+      d.fn[s] = Fn[s].template as<int>();
+      d.ncol[s] = nc;
+      d.nin[s] = w.ninp;
+      d.stride[s] = w.nfun;
+      njobs += nc;
+    }
+  }
+};
+
+// Device, stream, per-stage GPU timing and the MFMA accumulator-row probe of an engine.
+class EngineBase : public Engine {
+ public:
+  void synchronize() override { check(hipSetDevice(device_), "hipSetDevice"); check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
+  void set_profile(bool on) override { profile_ = on; }
+  const std::vector<StageTime> &stage_times() override
+  {
+    synchronize();
+    times_.clear();
+    for (size_t q = 0; q < ev_used_; q++) {
+      float ms = 0.f;
+      check(hipEventElapsedTime(&ms, events_[q].first, events_[q].second), "hipEventElapsedTime");
+      auto it = std::find_if(times_.begin(), times_.end(), [&](const StageTime &s) { return s.name == ev_names_[q]; });
+      if (it == times_.end()) {
+        times_.push_back({ev_names_[q], 0.0, 0});
+        it = times_.end() - 1;
+      }
+      it->ms += ms;
+      it->launches++;
+    }
+    return times_;
+  }
+  void debug_copy(int64_t bytes) override
+  {
+    check(hipSetDevice(device_), "hipSetDevice");
+    const long long nd = std::max<int64_t>(bytes / 8, 1);
+    DevBuf a, b;
+    a.ensure(nd * 8);
+    b.ensure(nd * 8);
+    check(hipMemsetAsync(a.p, 0, nd * 8, stream_), "hipMemsetAsync");
+    hipLaunchKernelGGL(k_copy_calibration, dim3(4096), dim3(256), 0, stream_, a.as<double>(), b.as<double>(), nd);
+    check(hipGetLastError(), "copy kernel");
+    check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+  }
+
+ protected:
+  EngineBase(int device, const char *who) : device_(device)
+  {
+    check(hipSetDevice(device_), "hipSetDevice");
+    hipDeviceProp_t prop;
+    check(hipGetDeviceProperties(&prop, device_), "hipGetDeviceProperties");
+    if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0 && std::string(prop.gcnArchName).rfind("gfx942", 0) != 0)
+      throw Error(std::string(who) + ": this library is built for gfx950 (MI355X); device is " + prop.gcnArchName);
+    ncu_ = prop.multiProcessorCount;
+    arch_ = prop.gcnArchName;
+    check(hipStreamCreate(&stream_), "hipStreamCreate");
+  }
+  ~EngineBase() override
+  {
+    (void) hipSetDevice(device_);
+    for (auto &e : events_) { (void) hipEventDestroy(e.first); (void) hipEventDestroy(e.second); }
+    if (stream_) (void) hipStreamDestroy(stream_);
+  }
+  static void check(hipError_t e, const char *what)
+  {
+    if (e != hipSuccess) throw Error(std::string("HIP error: ") + hipGetErrorString(e) + " in " + what);
+  }
+  void prof_begin(const char *name)
+  {
+    if (!profile_) return;
+    if (ev_used_ == events_.size()) {
+      hipEvent_t a, b;
+      check(hipEventCreate(&a), "hipEventCreate");
+      check(hipEventCreate(&b), "hipEventCreate");
+      events_.push_back({a, b});
+      ev_names_.push_back("");
+    }
+    ev_names_[ev_used_] = name;
+    check(hipEventRecord(events_[ev_used_].first, stream_), "hipEventRecord");
+  }
+  void prof_end()
+  {
+    if (!profile_) return;
+    check(hipEventRecord(events_[ev_used_].second, stream_), "hipEventRecord");
+    ev_used_++;
+  }
+  template<class F> void stage(const char *name, F &&f)
+  {
+    prof_begin(name);
+    f();
+    check(hipGetLastError(), name);
+    prof_end();
+  }
+  // which accumulator row each (lane / 16, register) of a 16x16x4 MFMA holds; the column must be lane % 16
+  template<class T> void probe_mfma()
+  {
+    std::vector<T> A(64), B(64), D(256);
+    for (int i = 0; i < 16; i++)
+      for (int k = 0; k < 4; k++) {
+        A[i * 4 + k] = (T) (1 + i + 16 * k);
+        B[k * 16 + i] = (T) ((k == 0 ? 1 : k == 1 ? 3 : k == 2 ? 7 : 11) * (i + 1));
+      }
+    DevBuf dA, dB, dD;
+    upload_vec(dA, A);
+    upload_vec(dB, B);
+    dD.ensure(256 * sizeof(T));
+    hipLaunchKernelGGL(k_mfma_probe<T>, dim3(1), dim3(64), 0, stream_, dA.as<T>(), dB.as<T>(), dD.as<T>());
+    check(hipGetLastError(), "k_mfma_probe");
+    check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
+    check(hipMemcpy(D.data(), dD.p, 256 * sizeof(T), hipMemcpyDeviceToHost), "hipMemcpy");
+    double ref[16][16];
+    for (int i = 0; i < 16; i++)
+      for (int j = 0; j < 16; j++) {
+        double s = 0;
+        for (int k = 0; k < 4; k++) s += (double) A[i * 4 + k] * (double) B[k * 16 + j];
+        ref[i][j] = s;
+      }
+    for (int g = 0; g < 4; g++)
+      for (int v = 0; v < 4; v++) {
+        int row = -1;
+        for (int i = 0; i < 16 && row < 0; i++) {
+          bool ok = true;
+          for (int c = 0; c < 16 && ok; c++) ok = (double) D[(g * 16 + c) * 4 + v] == ref[i][c];
+          if (ok) row = i;
+        }
+        if (row < 0) throw Error("MFMA 16x16x4 accumulator layout of this device is not the one the kernels assume");
+        drow_[g * 4 + v] = row;
+      }
+    int seen = 0;    // the 16 (group, register) pairs must cover the 16 rows
+    for (int q = 0; q < 16; q++) seen |= 1 << drow_[q];
+    if (seen != 0xFFFF) throw Error("MFMA 16x16x4 accumulator layout probe failed");
+  }
+  // out[tile atoms][job output] = GEMM jobs over X0 (kb0 16-channel blocks) and X1 (kb1), nb output blocks
+  template<class T>
+  void launch_gemm(DevJobs<T> &J, int kb0, int kb1, int nb, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo, int accumulate,
+                   const int *tiles, int ntiles)
+  {
+    if (J.d.njobs == 0 || ntiles == 0) return;
+    const int ksm = std::max(kb0, kb1) * 4;
+    const size_t lds = (size_t) kGemmMaxSeg * nb * ksm * 64 * sizeof(T);
+    const dim3 grid(J.d.njobs, (ntiles + 4 * kGemmTilesPerWave - 1) / (4 * kGemmTilesPerWave));
+#define GR_GEMM(A_, B_, C_)                                                                                            \
+  {                                                                                                                    \
+    auto kern = k_gemm_jobs<T, A_, B_, C_>;                                                                            \
+    if (lds > 48 * 1024)                                                                                               \
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, J.d, X0, nf0, X1, nf1, out, nfo, tiles, ntiles, accumulate); \
+  }
+#define GR_GEMM_C(A_, B_)                                                                                              \
+  switch (nb) {                                                                                                        \
+    case 1: GR_GEMM(A_, B_, 1) break;                                                                                  \
+    case 2: GR_GEMM(A_, B_, 2) break;                                                                                  \
+    case 4: GR_GEMM(A_, B_, 4) break;                                                                                  \
+    default: throw Error("unsupported channel widths");                                                                \
+  }
+    switch (kb0 * 10 + kb1) {
+      case 11: GR_GEMM_C(1, 1) break;
+      case 12: GR_GEMM_C(1, 2) break;
+      case 14: GR_GEMM_C(1, 4) break;
+      case 21: GR_GEMM_C(2, 1) break;
+      case 22: GR_GEMM_C(2, 2) break;
+      case 24: GR_GEMM_C(2, 4) break;
+      case 41: GR_GEMM_C(4, 1) break;
+      case 42: GR_GEMM_C(4, 2) break;
+      case 44: GR_GEMM_C(4, 4) break;
+      default: throw Error("unsupported channel widths");
+    }
+#undef GR_GEMM_C
+#undef GR_GEMM
+  }
+
+  int device_, ncu_ = 256;
+  std::string arch_;
+  hipStream_t stream_ = nullptr;
+  bool profile_ = false;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> events_;
+  std::vector<std::string> ev_names_;
+  size_t ev_used_ = 0;
+  std::vector<StageTime> times_;
+  int drow_[16];
+};
+
+}    // namespace grhip

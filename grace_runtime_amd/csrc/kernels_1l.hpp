@@ -683,6 +683,7 @@ template<class T> struct ReduceDev {
   const int *fn[4];
   int ncol[4], nin[4], stride[4];    // collected functions, (padded) channels, functions per atom of the source
   int nsrc, nrho, nbr, ksr;          // rho width, its 16-column blocks, k-steps of the reverse (ceil(nrho / 4))
+  int ostride, ooff;                 // output row of an atom: rho[atom * ostride + ooff + k]
   int drow[16];                      // accumulator row of (lane / 16, register)
 };
 
@@ -738,7 +739,7 @@ __global__ __launch_bounds__(256) void k_reduce_fwd(ReduceDev<T> R, const int *m
     if (at < 0) continue;
     double v = 0.0;
     for (int w = 0; w < 4; w++) v += part[w][k >> 4][r][k & 15];
-    rho[(long long) at * R.nrho + k] = v;
+    rho[(long long) at * R.ostride + R.ooff + k] = v;
   }
 }
 
@@ -759,7 +760,7 @@ __global__ __launch_bounds__(64) void k_reduce_bwd(ReduceDev<T> R, const int *mu
 #pragma unroll
   for (int q = 0; q < 8; q++) {
     const int k = g * R.ksr + q;
-    x[q] = (arow >= 0 && q < R.ksr && k < R.nrho) ? (T) grho[(long long) arow * R.nrho + k] : (T) 0;
+    x[q] = (arow >= 0 && q < R.ksr && k < R.nrho) ? (T) grho[(long long) arow * R.ostride + R.ooff + k] : (T) 0;
   }
   const int nb = R.nin[s] / 16;
   const T *wb = R.WB[s] + ((long long) m * R.ncol[s] + job) * nb * R.ksr * 64 + lane;

@@ -1,0 +1,293 @@
+// HIP kernels of the second message-passing layer of GRACE-2L for gfx950.
+//
+//   k_sh_edges     Y_lm and the gradient of its polynomial extension for every edge, once per pass
+//   k_fill_slot    the species weights zB0[mu_j] as one more "message function" of every atom
+//   k_pair_fwd     P[slot][lm][n] = sum_b Y_lm(b) R1_l(b)[n] M_jb[slot][n]: the neighbour gather of the messages
+//                  (slots 0 .. nI-1: the equivariant message I_j; slot nI: zB0, which gives B0)
+//                  (atom_yi / atom_scatter, libgrace/include/grace/fused_cpu.h:947-1025)
+//   k_pair_bwd     its reverse: per-bond force of layer 2, dE/dI_j added to the neighbour's row
+//                  (bond_yi_bwd_g, bond_yi_commit, bond_scatter_bwd_t, bond_force: fused_cpu.h:836-942,1027-1050)
+//   k_energy_2l    readout with the two RMSNorms, fp64 (libgrace/src/fused_2l.cpp:548-615)
+//
+// The gather kernels run one block per atom with one thread per (slot, channel): a thread keeps its 2l+1 .. nlm
+// accumulators (or adjoints) in registers and walks the atom's bonds; everything that is the same for the whole block
+// (neighbour index, Y, G of the bond) is read through uniform addresses.
+#pragma once
+
+#include "kernels_1l.hpp"
+
+namespace grhip {
+
+// one thread per edge: Y[e][lm] and YG[e][lm][4] = (Y, dY/dx, dY/dy, dY/dz)
+template<class T> __global__ void k_sh_edges(ShCoef sh, const double *rh, const long long *n_edges, int nlm, T *Y, T *YG)
+{
+  const long long e = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (e >= *n_edges) return;
+  T y[kMaxNlm], g[3 * kMaxNlm];
+  const double *u = rh + 3 * e;
+  if (YG) sh_eval<true, T>(sh, u[0], u[1], u[2], y, g);
+  else sh_eval<false, T>(sh, u[0], u[1], u[2], y, nullptr);
+  for (int q = 0; q < nlm; q++) {
+    Y[e * nlm + q] = y[q];
+    if (YG) {
+      T *o = YG + (e * nlm + q) * 4;
+      o[0] = y[q]; o[1] = g[3 * q]; o[2] = g[3 * q + 1]; o[3] = g[3 * q + 2];
+    }
+  }
+}
+
+// M[atom][slot][n] = z[mu_atom][n]
+template<class T> __global__ void k_fill_slot(const int *mu, const T *z, T *M, int natoms, int nslot, int slot, int C)
+{
+  const long long q = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (q >= (long long) natoms * C) return;
+  const int at = (int) (q / C), n = (int) (q % C);
+  M[((long long) at * nslot + slot) * C + n] = z[mu[at] * C + n];
+}
+
+// grid: atoms; block: nslot * C threads (slot = t / C, n = t % C)
+template<class T, int NLM>
+__global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ Y,
+                           const T *__restrict__ R1, const T *__restrict__ M, T *__restrict__ P, int nslot, int C, int nl, int noutp)
+{
+  const int i = blockIdx.x, t = threadIdx.x;
+  const int slot = t / C, n = t % C;
+  const int nlm = nl * nl;
+  const long long e0 = eoff[i], e1 = eoff[i + 1];
+  T acc[NLM];
+#pragma unroll
+  for (int q = 0; q < NLM; q++) acc[q] = (T) 0;
+  for (long long e = e0; e < e1; e++) {
+    const int j = ej[e];
+    const T m = M[((long long) j * nslot + slot) * C + n];
+    const T *r = R1 + e * noutp + n;
+    const T *y = Y + e * nlm;
+#pragma unroll
+    for (int l = 0; l <= kKernMaxL; l++)
+      if (l * l < NLM && l < nl) {
+        const T rm = r[l * C] * m;
+#pragma unroll
+        for (int mm = 0; mm < 2 * l + 1; mm++) acc[l * l + mm] += y[l * l + mm] * rm;
+      }
+  }
+  T *o = P + ((long long) i * nslot + slot) * nlm * C + n;
+#pragma unroll
+  for (int q = 0; q < NLM; q++)
+    if (q < nlm) o[(long long) q * C] = acc[q];
+}
+
+// sums of 4 values per lane over the wave with 7 exchanges: afterwards lanes 0, 1, 2, 3 hold the totals of
+// v0, v2, v1, v3
+__device__ inline double wave_sum4(double v0, double v1, double v2, double v3, int lane)
+{
+  const bool b0 = lane & 1, b1 = lane & 2;
+  double a = b0 ? v2 : v0, b = b0 ? v3 : v1;
+  const double sa = b0 ? v0 : v2, sb = b0 ? v1 : v3;
+  a += __shfl_xor(sa, 1, 64);
+  b += __shfl_xor(sb, 1, 64);
+  double c = b1 ? b : a;
+  const double sc = b1 ? a : b;
+  c += __shfl_xor(sc, 2, 64);
+#pragma unroll
+  for (int o = 4; o < 64; o <<= 1) c += __shfl_xor(c, o, 64);
+  return c;
+}
+
+constexpr int kPairChunk = 32;    // bonds whose force sums are gathered in LDS at a time
+
+// grid: atoms; block: nslot * C threads rounded up to a wave.  gP: adjoint of P of the atom.
+//   S_l = sum_m Y_lm gP[lm],  T_l,d = sum_m G_lm,d gP[lm]                      (per thread: slot, n)
+//   dE/dI_j[slot][n] += sum_l R1_l S_l                                        (slots < nI)
+//   dE/dx = sum_{slot,n,l} S_l dR1_l M_j,   g_d = sum_{slot,n,l} T_l,d R1_l M_j
+//   fv = dE/dx / rc rhat + (g - (g . rhat) rhat) / r;  f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv
+template<class T, int NLM>
+__global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ YG,
+                           const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
+                           const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
+                           T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
+                           int noutp)
+{
+  __shared__ double bsum[kPairChunk][4];
+  __shared__ double red[16][9];
+  const int i = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6, nwave = blockDim.x >> 6;
+  const bool active = t < nslot * C;
+  const int slot = active ? t / C : 0, n = t % C;
+  const int nlm = nl * nl;
+  const long long e0 = eoff[i], e1 = eoff[i + 1];
+  T g[NLM];
+  {
+    const T *gp = gP + ((long long) i * nslot + slot) * nlm * C + n;
+#pragma unroll
+    for (int q = 0; q < NLM; q++) g[q] = (active && q < nlm) ? gp[(long long) q * C] : (T) 0;
+  }
+  double fi[3] = {0, 0, 0}, vir[6] = {0, 0, 0, 0, 0, 0};
+  for (long long base = e0; base < e1; base += kPairChunk) {
+    const int nb = (int) (e1 - base < kPairChunk ? e1 - base : kPairChunk);
+    __syncthreads();
+    if (t < kPairChunk * 4) bsum[t >> 2][t & 3] = 0.0;
+    __syncthreads();
+    for (int b = 0; b < nb; b++) {
+      const long long e = base + b;
+      const int j = ej[e];
+      const T m = active ? M[((long long) j * nslot + slot) * C + n] : (T) 0;
+      const T *r = R1 + e * noutp + n, *dr = dR1 + e * noutp + n;
+      const T *yg = YG + e * nlm * 4;
+      T sI = (T) 0, dE = (T) 0, t0 = (T) 0, t1 = (T) 0, t2 = (T) 0;
+#pragma unroll
+      for (int l = 0; l <= kKernMaxL; l++)
+        if (l * l < NLM && l < nl) {
+          T S = (T) 0, a0 = (T) 0, a1 = (T) 0, a2 = (T) 0;
+#pragma unroll
+          for (int mm = 0; mm < 2 * l + 1; mm++) {
+            const T *q = yg + (l * l + mm) * 4;
+            const T gv = g[l * l + mm];
+            S += q[0] * gv; a0 += q[1] * gv; a1 += q[2] * gv; a2 += q[3] * gv;
+          }
+          const T rl = r[l * C], drl = dr[l * C];
+          sI += rl * S;
+          dE += drl * S;
+          t0 += rl * a0; t1 += rl * a1; t2 += rl * a2;
+        }
+      if (active && slot < nI) atomicAdd(&gM[((long long) j * nI + slot) * C + n], sI);
+      const double c = wave_sum4((double) (dE * m), (double) (t0 * m), (double) (t1 * m), (double) (t2 * m), lane);
+      if (lane < 4) atomicAdd(&bsum[b][lane], c);    // lanes 0..3: dE/dx, g_y, g_x, g_z  (order v0, v2, v1, v3)
+    }
+    __syncthreads();
+    if (t < nb) {
+      const long long e = base + t;
+      const double *u = rh + 3 * e;
+      const double r = rlen[e], rc = rcut[e];
+      const double gv[3] = {bsum[t][2], bsum[t][1], bsum[t][3]};
+      const double dEdr = bsum[t][0] / rc;
+      const double gr = gv[0] * u[0] + gv[1] * u[1] + gv[2] * u[2];
+      double fv[3];
+      for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + (gv[d] - gr * u[d]) / r;
+      const int jj = ej[e];
+      for (int d = 0; d < 3; d++) {
+        fi[d] += fv[d];
+        atomicAdd(&f[3 * (long long) jj + d], -fv[d]);
+      }
+      const double ddx = -u[0] * r, ddy = -u[1] * r, ddz = -u[2] * r;
+      vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
+      vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
+    }
+  }
+  // the finishing threads t < kPairChunk sit in wave 0
+  if (wave == 0) {
+    double vsum[9] = {fi[0], fi[1], fi[2], vir[0], vir[1], vir[2], vir[3], vir[4], vir[5]};
+#pragma unroll
+    for (int k = 0; k < 9; k++)
+      for (int o = 32; o > 0; o >>= 1) vsum[k] += __shfl_xor(vsum[k], o, 64);
+    if (lane == 0 && e1 > e0) {
+      for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) i + k], vsum[k]);
+      for (int k = 0; k < 6; k++) atomicAdd(&virial[k], vsum[3 + k]);
+    }
+  }
+  (void) red; (void) nwave;
+}
+
+struct Energy2Dev {
+  const double *W[7];         // [n_in][n_out]
+  double norm[7];
+  int nin[7], nout[7];
+  int nlay, act, ln, nrho, rms;
+  double out_scale, eps;
+  const double *shift;        // [nel]
+  const double *lnI;          // [nrho - 1] scale of the only_nonlin RMSNorm of rho
+  const double *ln0;          // [nrho]     scale of the full RMSNorm of I2
+};
+
+// E_i = (MLP(x) + rho[0] + I2[0] ln0[0] / s0) out_scale + shift,  x_k = rho[k] lnI[k-1] / s1 + I2[k] ln0[k] / s0,
+// s1 = sqrt(mean rho[1:]^2 + eps), s0 = sqrt(mean I2^2 + eps); dE/drho, dE/dI2.  One wave per atom, fp64.
+__global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, const double *rho, const double *I2, double *grho, double *gI2,
+                            double *eatom, double *energy, int want_grad)
+{
+  __shared__ double act[8][256], pre[7][256], gbuf[2][256], x0[256];
+  const int at = blockIdx.x, lane = threadIdx.x;
+  const double *r = rho + (long long) at * M.nrho, *i2 = I2 + (long long) at * M.nrho;
+  const int nr = M.nrho, n0 = nr - 1;
+  double ms1 = 0.0, ms0 = 0.0;
+  for (int k = lane; k < nr; k += 64) {
+    if (k > 0) ms1 += r[k] * r[k];
+    ms0 += i2[k] * i2[k];
+  }
+  for (int o = 32; o > 0; o >>= 1) { ms1 += __shfl_xor(ms1, o, 64); ms0 += __shfl_xor(ms0, o, 64); }
+  const double s1 = M.rms ? sqrt(ms1 / n0 + M.eps) : 1.0, s0 = M.rms ? sqrt(ms0 / nr + M.eps) : 1.0;
+  for (int k = lane; k < n0; k += 64) act[0][k] = r[k + 1] / s1 * M.lnI[k] + i2[k + 1] / s0 * M.ln0[k + 1];
+  __syncthreads();
+  double q = 0.0;
+  if (M.ln) {
+    double ms = 0.0;
+    for (int k = lane; k < n0; k += 64) { x0[k] = act[0][k]; ms += act[0][k] * act[0][k]; }
+    for (int o = 32; o > 0; o >>= 1) ms += __shfl_xor(ms, o, 64);
+    q = 1.0 / sqrt(ms / n0 + 1e-16);
+    for (int k = lane; k < n0; k += 64) act[0][k] *= q;
+    __syncthreads();
+  }
+  for (int L = 0; L < M.nlay; L++) {
+    for (int c = lane; c < M.nout[L]; c += 64) {
+      double s = 0.0;
+      for (int a = 0; a < M.nin[L]; a++) s += act[L][a] * M.W[L][(long long) a * M.nout[L] + c];
+      s *= M.norm[L];
+      pre[L][c] = s;
+      act[L + 1][c] = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+    }
+    __syncthreads();
+  }
+  const double Ei = (act[M.nlay][0] + r[0] + i2[0] / s0 * M.ln0[0]) * M.out_scale + M.shift[mu[at]];
+  if (lane == 0) {
+    if (eatom) eatom[at] = Ei;
+    atomicAdd(energy, Ei);
+  }
+  if (!want_grad) return;
+  int cur = 0;
+  if (lane == 0) gbuf[0][0] = M.out_scale;
+  __syncthreads();
+  for (int L = M.nlay - 1; L >= 0; L--) {
+    if (L < M.nlay - 1) {
+      for (int c = lane; c < M.nout[L]; c += 64) {
+        const double v = pre[L][c];
+        if (M.act == 1) {
+          const double tt = act[L + 1][c];
+          gbuf[cur][c] *= 1.0 - tt * tt;
+        } else {
+          const double sg = 1.0 / (1.0 + exp(-v));
+          gbuf[cur][c] *= sg * (1.0 + v * (1.0 - sg));
+        }
+      }
+      __syncthreads();
+    }
+    for (int a = lane; a < M.nin[L]; a += 64) {
+      double s = 0.0;
+      for (int c = 0; c < M.nout[L]; c++) s += gbuf[cur][c] * M.W[L][(long long) a * M.nout[L] + c];
+      gbuf[cur ^ 1][a] = s * M.norm[L];
+    }
+    cur ^= 1;
+    __syncthreads();
+  }
+  if (M.ln) {
+    double tt = 0.0;
+    for (int k = lane; k < n0; k += 64) tt += gbuf[cur][k] * x0[k];
+    for (int o = 32; o > 0; o >>= 1) tt += __shfl_xor(tt, o, 64);
+    for (int k = lane; k < n0; k += 64) gbuf[cur][k] = q * (gbuf[cur][k] - x0[k] * tt * q * q / n0);
+    __syncthreads();
+  }
+  // gbuf[cur][k-1] = dE/dx_k; RMSNorm reverses (y_k = x_k s_k / sigma)
+  double t1 = 0.0, t0 = 0.0;
+  if (M.rms) {
+    for (int k = lane; k < nr; k += 64) {
+      const double gy = k == 0 ? M.out_scale : gbuf[cur][k - 1];
+      if (k > 0) t1 += gy * M.lnI[k - 1] * r[k];
+      t0 += gy * M.ln0[k] * i2[k];
+    }
+    for (int o = 32; o > 0; o >>= 1) { t1 += __shfl_xor(t1, o, 64); t0 += __shfl_xor(t0, o, 64); }
+  }
+  double *gr = grho + (long long) at * nr, *gi = gI2 + (long long) at * nr;
+  for (int k = lane; k < nr; k += 64) {
+    const double gy = k == 0 ? M.out_scale : gbuf[cur][k - 1];
+    gr[k] = k == 0 ? M.out_scale : gy * M.lnI[k - 1] / s1 - r[k] * t1 / (n0 * s1 * s1 * s1);
+    gi[k] = gy * M.ln0[k] / s0 - i2[k] * t0 / (nr * s0 * s0 * s0);
+  }
+}
+
+}    // namespace grhip

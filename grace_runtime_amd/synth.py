@@ -24,8 +24,8 @@ import math
 
 import numpy as np
 
-__all__ = ["real_sh_np", "coupling_tables", "structure_1l", "random_model_1l", "save_model", "bcc_supercell",
-           "fcc_supercell", "jitter"]
+__all__ = ["real_sh_np", "coupling_tables", "real_cg", "structure_1l", "structure_2l", "random_model_1l",
+           "random_model_2l", "save_model", "bcc_supercell", "fcc_supercell", "jitter"]
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -306,6 +306,317 @@ def random_model_1l(*, lmax=4, n_elements=1, element_names=("W",), embedding_siz
     d["energy_mlp_norm1"] = f64(1.0 / math.sqrt(energy_hidden))
     d["energy_mlp_n_layers"] = i64(2)
     d["energy_mlp_activation"] = i64(0)
+    d["shift_values"] = np.zeros(n_elements)
+    d.update(s)
+    return d
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# GRACE-2L: structure arrays and random models
+# ---------------------------------------------------------------------------------------------------------------
+def _rotation(rng):
+    q = rng.standard_normal(4)
+    a, b, c, d = q / np.linalg.norm(q)
+    return np.array([[a * a + b * b - c * c - d * d, 2 * (b * c - a * d), 2 * (b * d + a * c)],
+                     [2 * (b * c + a * d), a * a - b * b + c * c - d * d, 2 * (c * d - a * b)],
+                     [2 * (b * d - a * c), 2 * (c * d + a * b), a * a - b * b - c * c + d * d]])
+
+
+_CG_CACHE = {}
+
+
+def real_cg(l1, l2, L):
+    """Real Clebsch-Gordan tensor T[2l1+1, 2l2+1, 2L+1] of the real harmonics above, for any parity of l1 + l2 + L:
+    the one-dimensional space of rotation-invariant tensors, found numerically from the rotation matrices of the
+    harmonics.  Even couplings (l1 + l2 + L even) are normalised as coupling_tables (Y x Y -> Y); odd couplings to
+    sum_{m1 m2} T[m1, m2, M]^2 = 1 with the sign that makes, at m2 = +l2, the entry of the largest m1 (smallest M)
+    positive (the vector product a x b for l1 = l2 = L = 1)."""
+    key = (l1, l2, L)
+    if key in _CG_CACHE:
+        return _CG_CACHE[key]
+    if (l1 + l2 + L) % 2 == 0:
+        T = coupling_tables(max(l1, l2, L))[key]
+        _CG_CACHE[key] = T
+        return T
+    rng = np.random.default_rng(7)
+    u = rng.standard_normal((200, 3))
+    u /= np.linalg.norm(u, axis=1)[:, None]
+    n1, n2, n3 = 2 * l1 + 1, 2 * l2 + 1, 2 * L + 1
+
+    def wigner(l, R):
+        Y = real_sh_np(u, l)[:, l * l:(l + 1) ** 2]
+        YR = real_sh_np(u @ R.T, l)[:, l * l:(l + 1) ** 2]
+        return np.linalg.lstsq(Y, YR, rcond=None)[0].T
+
+    rows = []
+    for _ in range(3):
+        R = _rotation(rng)
+        K = np.einsum("am,bn,cM->abcmnM", wigner(l1, R), wigner(l2, R), wigner(L, R)).reshape(n1 * n2 * n3, -1)
+        rows.append(K - np.eye(n1 * n2 * n3))
+    sv, vt = np.linalg.svd(np.concatenate(rows, 0))[1:]
+    if not (sv[-1] < 1e-9 and sv[-2] > 1e-6):
+        raise ValueError(f"no unique coupling {key}")
+    T = vt[-1].reshape(n1, n2, n3)
+    T[np.abs(T) < 1e-10] = 0.0
+    T /= math.sqrt((T[:, :, 0] ** 2).sum())
+    for m1 in range(n1 - 1, -1, -1):
+        nz = np.nonzero(T[m1, n2 - 1, :])[0]
+        if nz.size:
+            if T[m1, n2 - 1, nz[0]] < 0:
+                T = -T
+            break
+    _CG_CACHE[key] = T
+    return T
+
+
+def structure_2l(lmax):
+    """Structure arrays of a GRACE-2L model with body order 3 per layer (no AAAA / BBBB stage) and Lmax = lmax in both
+    layers.  Irreducible pieces carry (L, parity); lists of functions are ordered by (L, parity) with odd parity
+    first, collect lists of the equivariant reduces by (parity, L).
+
+    layer 1: A, A1, AA, AA1 as structure_1l; AAA = AA1 x A -> the invariants of structure_1l followed by the vectors
+             (L = 1, odd parity) of the AA groups (l1, l2, L') x A(l3), l3 = L' +- 1, in (l1, l2, L', l3) order, without
+             the groups l2 = 0 < l1 and the stretched self couplings L' = 2 l1 (the selection read off the exported
+             lmax 2 and lmax 3 models); I1 and I carry (0, +) and (1, -): 4 functions.
+    layer 2: YI = every coupling Y_l x I_l' -> L <= lmax, both parities; B0 = the natural-parity functions;
+             B = all (L, parity) present; B1 one weight tile per piece; BB = B1 x B1 over the first piece of every L
+             (pairs l1 >= l2, every L <= lmax, vanishing antisymmetric self couplings left out);
+             BB1 takes its right input from the B piece of equal (L, parity);
+             BBB = BB1 x B -> invariants, one per unordered triple (l1, l2, L) and coupling.
+    """
+    s = structure_1l(lmax, order4=False)
+    groups = s["_groups"]
+    nl = lmax + 1
+    nlm = nl * nl
+    g_first = np.cumsum([0] + [2 * g[0] + 1 for g in groups])
+    nAA = int(g_first[-1])
+    gidx = {(g[1], g[2], g[0]): k for k, g in enumerate(groups)}         # (l1, l2, L) -> group
+    # ---- AAA vectors
+    l0, r0, o0, c0 = (s[f"prod_AAA_{k}"] for k in ("left_ind", "right_ind", "m_sum_ind", "cg_coeff"))
+    nAAA0 = int(s["prod_AAA_n_output_funcs"][0])
+    terms = [(int(o), int(l), int(r), float(c)) for o, l, r, c in zip(o0, l0, r0, c0)]
+    nout = nAAA0
+    for (l1, l2, Lp) in sorted(gidx):
+        if (l2 == 0 and l1 > 0) or (l1 == l2 and l1 > 0 and Lp == l1 + l2):
+            continue
+        g = gidx[(l1, l2, Lp)]
+        for l3 in (Lp - 1, Lp + 1):
+            if l3 < 0 or l3 > lmax:
+                continue
+            T = real_cg(Lp, l3, 1)
+            for M in range(3):
+                for a in range(2 * Lp + 1):
+                    for b in range(2 * l3 + 1):
+                        if T[a, b, M] != 0.0:
+                            terms.append((nout + M, int(g_first[g]) + a, l3 * l3 + b, float(T[a, b, M])))
+            nout += 3
+    nAAA = nout
+    l, r, o, c = _prod_arrays(terms)
+    s.update(prod_AAA_left_ind=l, prod_AAA_right_ind=r, prod_AAA_m_sum_ind=o, prod_AAA_cg_coeff=c,
+             prod_AAA_n_output_funcs=np.array([nAAA], np.int64), prod_AAA_n_cg_terms=np.array([c.size], np.int64),
+             prod_AAA_lmax=np.array([1], np.int64), prod_AAA_Lmax=np.array([1], np.int64))
+
+    def reduce_arrays(pfx, src, conns):
+        """conns: list of (collect function, output function, group key); tiles number the groups in order."""
+        tiles, t = [], -1
+        last = None
+        for _, _, key in conns:
+            if key != last:
+                t += 1
+                last = key
+            tiles.append(t)
+        s[f"{pfx}_collect_ind_{src}"] = np.array([q[0] for q in conns], np.int32)
+        s[f"{pfx}_w_l_tile_{src}"] = np.array(tiles, np.int32)
+        s[f"{pfx}_total_sum_ind_{src}"] = np.array([q[1] for q in conns], np.int32).reshape(-1, 1)
+        s[f"{pfx}_w_shape_{src}"] = np.array([t + 1], np.int64)
+
+    # ---- I1 (0, +), (1, -) from A, AA, AAA; I from I1; rho (invariants) as structure_1l
+    reduce_arrays("I1", "A", [(1 + m, 1 + m, "l1") for m in range(3)] + [(0, 0, "l0")])
+    vec = [(int(g_first[k]) + m, 1 + m, ("g", k)) for k, g in enumerate(groups) if g[0] == 1 for m in range(3)]
+    inv = [(int(g_first[k]), 0, ("g", k)) for k, g in enumerate(groups) if g[0] == 0]
+    reduce_arrays("I1", "AA", vec + inv)
+    reduce_arrays("I1", "AAA", [(q, 1 + (q - nAAA0) % 3, ("v", (q - nAAA0) // 3)) for q in range(nAAA0, nAAA)] +
+                  [(q, 0, ("i", q)) for q in range(nAAA0)])
+    reduce_arrays("I", "I1", [(1 + m, 1 + m, "l1") for m in range(3)] + [(0, 0, "l0")])
+    # ---- YI: Y_l x I_l'
+    I_pieces = [(0, +1, 0), (1, -1, 1)]                                   # (l', parity, first function)
+    yi_groups = []                                                        # (L, parity, l, l')
+    for l in range(nl):
+        for (lp, pp, _) in I_pieces:
+            for L in range(abs(l - lp), min(lmax, l + lp) + 1):
+                yi_groups.append((L, (-1) ** l * pp, l, lp))
+    yi_groups.sort(key=lambda g: (g[0], g[1], g[2], g[3]))
+    yi_first = np.cumsum([0] + [2 * g[0] + 1 for g in yi_groups])
+    lr, yo, yc = [], [], []
+    for k, (L, p, l, lp) in enumerate(yi_groups):
+        T = real_cg(l, lp, L)
+        i0 = 0 if lp == 0 else 1
+        for M in range(2 * L + 1):
+            for a in range(2 * l + 1):
+                for b in range(2 * lp + 1):
+                    if T[a, b, M] != 0.0:
+                        lr.append((l * l + a, i0 + b))
+                        yo.append(int(yi_first[k]) + M)
+                        yc.append(float(T[a, b, M]))
+    s.update(YI_lr_inds=np.array(lr, np.int32), YI_m_sum_ind=np.array(yo, np.int32), YI_cg_coeff=np.array(yc),
+             YI_n_output_funcs=np.array([int(yi_first[-1])], np.int64), YI_n_cg_terms=np.array([len(yc)], np.int64),
+             YI_Lmax=np.array([lmax], np.int64))
+    # ---- B pieces (L, parity) and the reduce from YI and B0
+    pieces = sorted({(g[0], g[1]) for g in yi_groups} | {(l, (-1) ** l) for l in range(nl)})
+    b_first = dict(zip(pieces, np.cumsum([0] + [2 * P[0] + 1 for P in pieces])[:-1]))
+    nB = sum(2 * P[0] + 1 for P in pieces)
+    order = sorted(range(len(yi_groups)), key=lambda k: (yi_groups[k][1], yi_groups[k][0], k))
+    reduce_arrays("B", "YI", [(int(yi_first[k]) + M, int(b_first[yi_groups[k][:2]]) + M, ("g", k))
+                              for k in order for M in range(2 * yi_groups[k][0] + 1)])
+    lorder = sorted(range(nl), key=lambda l: ((-1) ** l, l))
+    reduce_arrays("B", "B0", [(l * l + M, int(b_first[(l, (-1) ** l)]) + M, ("l", l)) for l in lorder
+                              for M in range(2 * l + 1)])
+    # ---- FC B1: one tile per piece
+    tile = np.concatenate([np.full(2 * P[0] + 1, k, np.int32) for k, P in enumerate(pieces)])
+    s.update(fc_B1_w_tile_left=tile, fc_B1_w_tile_right=tile.copy(), fc_B1_collect_to=np.arange(nB, dtype=np.int32),
+             fc_B1_collect_from=np.arange(nB, dtype=np.int32),
+             fc_B1_norm_out_factor=np.full((nB, 1, 1), 1.0 / math.sqrt(2.0)))
+    # ---- BB = B1 x B1 over the first piece of every L
+    first_piece = {}
+    for P in pieces:
+        first_piece.setdefault(P[0], P)
+    bb_groups = []                                                        # (L, parity, l1, l2)
+    for l1 in range(nl):
+        for l2 in range(l1 + 1):
+            for L in range(l1 - l2, min(lmax, l1 + l2) + 1):
+                if l1 == l2 and (l1 + l2 + L) % 2:
+                    continue
+                p = first_piece[l1][1] * first_piece[l2][1]
+                if (L, p) in b_first:
+                    bb_groups.append((L, p, l1, l2))
+    bb_groups.sort()
+    bb_first = np.cumsum([0] + [2 * g[0] + 1 for g in bb_groups])
+    nBB = int(bb_first[-1])
+    terms = []
+    for k, (L, p, l1, l2) in enumerate(bb_groups):
+        T = real_cg(l1, l2, L)
+        f1, f2 = int(b_first[first_piece[l1]]), int(b_first[first_piece[l2]])
+        for M in range(2 * L + 1):
+            acc = {}
+            for a in range(2 * l1 + 1):
+                for b in range(2 * l2 + 1):
+                    v = T[a, b, M]
+                    if v == 0.0:
+                        continue
+                    x, y = f1 + a, f2 + b
+                    if l1 == l2 and x < y:
+                        x, y = y, x
+                    acc[(x, y)] = acc.get((x, y), 0.0) + v
+            for (x, y), v in acc.items():
+                if abs(v) > 1e-12:
+                    o = int(bb_first[k]) + M
+                    terms.append((o, x, y, v, (o, y, x) if l1 == l2 else (o, x, y)))
+    l, r, o, c = _prod_arrays(terms)
+    s.update(prod_BB_left_ind=l, prod_BB_right_ind=r, prod_BB_m_sum_ind=o, prod_BB_cg_coeff=c,
+             prod_BB_n_output_funcs=np.array([nBB], np.int64), prod_BB_n_cg_terms=np.array([c.size], np.int64),
+             prod_BB_lmax=np.array([lmax], np.int64), prod_BB_Lmax=np.array([lmax], np.int64))
+    tile = np.concatenate([np.full(2 * g[0] + 1, k, np.int32) for k, g in enumerate(bb_groups)])
+    frm = np.concatenate([int(b_first[(g[0], g[1])]) + np.arange(2 * g[0] + 1) for g in bb_groups]).astype(np.int32)
+    s.update(fc_BB1_w_tile_left=tile, fc_BB1_w_tile_right=tile.copy(), fc_BB1_collect_to=np.arange(nBB, dtype=np.int32),
+             fc_BB1_collect_from=frm, fc_BB1_norm_out_factor=np.full((nBB, 1, 1), 1.0 / math.sqrt(2.0)))
+    # ---- BBB = BB1 x B -> invariants: one per unordered triple and coupling parity, even-parity BB groups only
+    seen, terms, nBBB = set(), [], 0
+    for k in sorted(range(len(bb_groups)), key=lambda k: (bb_groups[k][2], bb_groups[k][3], bb_groups[k][0])):
+        L, p, l1, l2 = bb_groups[k]
+        if p != 1 or (L, 1) not in b_first:
+            continue
+        key = (tuple(sorted((l1, l2, L))), (l1 + l2 + L) % 2)
+        canonical = (l1 + l2 + L) % 2 == 1 or L <= l2
+        if key in seen or not canonical:
+            continue
+        seen.add(key)
+        for M in range(2 * L + 1):
+            terms.append((nBBB, int(bb_first[k]) + M, int(b_first[(L, 1)]) + M, 1.0 / (2 * L + 1)))
+        nBBB += 1
+    l, r, o, c = _prod_arrays(terms)
+    s.update(prod_BBB_left_ind=l, prod_BBB_right_ind=r, prod_BBB_m_sum_ind=o, prod_BBB_cg_coeff=c,
+             prod_BBB_n_output_funcs=np.array([nBBB], np.int64), prod_BBB_n_cg_terms=np.array([c.size], np.int64),
+             prod_BBB_lmax=np.array([0], np.int64), prod_BBB_Lmax=np.array([0], np.int64))
+    # ---- I2: invariants of B, BB, BBB
+    reduce_arrays("I2", "B", [(0, 0, "b")])
+    reduce_arrays("I2", "BB", [(int(bb_first[k]), 0, ("g", k)) for k, g in enumerate(bb_groups) if g[0] == 0])
+    reduce_arrays("I2", "BBB", [(q, 0, ("i", q)) for q in range(nBBB)])
+    s["_groups"] = groups
+    s["_sizes"] = dict(nAA=nAA, nAAA=nAAA, nI=4, nYI=int(yi_first[-1]), nB=nB, nBB=nBB, nBBB=nBBB,
+                       nt_AA=len(groups), nt_B=len(pieces), nt_BB=len(bb_groups))
+    return s
+
+
+def random_model_2l(*, lmax=4, n_elements=4, element_names=("Al", "Co", "Ni", "Ti"), embedding_size=32, nradbase=8,
+                    c1=32, cr=32, c2=32, i1_width=16, hidden=64, rho_n_out=17, energy_hidden=64, rcut=6.0,
+                    radial_basis_p=16, inv_avg_n_neigh=1.0 / 78.0, seed=20260103):
+    """A GRACE-2L-shaped model (body order 3 per layer) with weights ~ N(0, 1) and norm scalars 1/sqrt(n_in):
+    c1 layer-1 radial / FC channels, cr layer-2 radial channels (= message width), c2 layer-2 FC channels.
+    Keys as the reference loader reads them, libgrace/src/model_2l.cpp:28-420."""
+    rng = np.random.default_rng(seed)
+    nl = lmax + 1
+    s = structure_2l(lmax)
+    s.pop("_groups")
+    z = s.pop("_sizes")
+    i64 = lambda v: np.array([v], dtype=np.int64)
+    f64 = lambda v: np.array([v], dtype=np.float64)
+    N = lambda *shape: rng.standard_normal(shape)
+    d = {"grace_model_kind": np.array([b"GRACE-2L"], dtype="|S8"), "grace_format_version": i64(1),
+         "n_elements": i64(n_elements), "element_names": np.array([n.encode() for n in element_names], dtype="|S2"),
+         "embedding_size": i64(embedding_size), "nradbase": i64(nradbase), "rcut": f64(rcut),
+         "radial_basis_p": i64(radial_basis_p), "has_bond_specific_cutoff": i64(0), "lmax": i64(lmax),
+         "chem_embedding": N(n_elements, embedding_size)}
+    for pfx, c in (("mlp_rad_R", c1), ("mlp_rad_R1", cr)):
+        dims = [nradbase, hidden, hidden, c * nl]
+        for i in range(3):
+            d[f"{pfx}_W{i}"] = N(dims[i], dims[i + 1])
+            d[f"{pfx}_norm{i}"] = f64(1.0 / math.sqrt(dims[i]))
+        d[f"{pfx}_n_layers"] = i64(3)
+        d[f"{pfx}_n_rad_max"] = i64(c)
+        d[f"{pfx}_has_chem_emb"] = i64(0)
+    for pfx, c in (("A", c1), ("B0", cr)):
+        d[f"{pfx}_inv_avg_n_neigh"] = np.array(inv_avg_n_neigh)
+        d[f"{pfx}_lin_transform_W"] = N(embedding_size, c)
+        d[f"{pfx}_lin_transform_norm"] = f64(1.0 / math.sqrt(embedding_size))
+    d["YI_inv_avg_n_neigh"] = np.array(inv_avg_n_neigh)
+    d["YI_n_rad_max"] = i64(cr)
+    for k, c, ntile in (("A1", c1, nl), ("AA1", c1, z["nt_AA"]), ("B1", c2, z["nt_B"]), ("BB1", c2, z["nt_BB"])):
+        d[f"fc_{k}_w_left"] = N(c, c, ntile)
+        d[f"fc_{k}_norm_left"] = np.array(1.0 / math.sqrt(c))
+        d[f"fc_{k}_w_right"] = N(c, c, ntile)
+        d[f"fc_{k}_norm_right"] = np.array(1.0 / math.sqrt(c))
+        d[f"fc_{k}_n_out"] = i64(c)
+        d[f"fc_{k}_left_coefs"] = i64(1)
+
+    def reduce_w(pfx, srcs, n_out, n_in, elem, nfuncs):
+        for src in srcs:
+            w_shape = int(s[f"{pfx}_w_shape_{src}"][0])
+            d[f"{pfx}_reduce_{src}_W"] = N(n_elements, n_out, n_in[src], w_shape) if elem else N(n_out, n_in[src], w_shape)
+            d[f"{pfx}_reduce_{src}_norm"] = np.array(1.0 / math.sqrt(n_in[src]))
+            d[f"{pfx}_n_in_{src}"] = i64(n_in[src])
+        d[f"{pfx}_n_out"] = i64(n_out)
+        d[f"{pfx}_n_funcs"] = i64(nfuncs)
+        d[f"{pfx}_is_central_atom_type_dependent"] = i64(1 if elem else 0)
+        d[f"{pfx}_instruction_names"] = np.array([x.encode() for x in srcs], dtype="|S8")
+
+    l1 = {"A": c1, "AA": c1, "AAA": c1}
+    reduce_w("I1", ["A", "AA", "AAA"], i1_width, l1, True, 4)
+    reduce_w("rho", ["A", "AA", "AAA"], rho_n_out, l1, True, 1)
+    reduce_w("I", ["I1"], cr, {"I1": i1_width}, False, 4)
+    reduce_w("B", ["YI", "B0"], c2, {"YI": cr, "B0": cr}, False, z["nB"])
+    reduce_w("I2", ["B", "BB", "BBB"], rho_n_out, {"B": c2, "BB": c2, "BBB": c2}, True, 1)
+    d["I_nl_LN_scale"] = 1.0 + 0.1 * N(rho_n_out - 1)
+    d["I_nl_LN_type"] = i64(1)
+    d["I_nl_LN_n_out"] = i64(rho_n_out)
+    d["I_0_LN_scale"] = 1.0 + 0.1 * N(rho_n_out)
+    d["I_0_LN_type"] = i64(0)
+    d["I_0_LN_n_out"] = i64(rho_n_out)
+    d["energy_mlp_W0"] = N(rho_n_out - 1, energy_hidden)
+    d["energy_mlp_norm0"] = f64(1.0 / math.sqrt(rho_n_out - 1))
+    d["energy_mlp_W1"] = N(energy_hidden, 1)
+    d["energy_mlp_norm1"] = f64(1.0 / math.sqrt(energy_hidden))
+    d["energy_mlp_n_layers"] = i64(2)
+    d["energy_mlp_activation"] = i64(1)
     d["shift_values"] = np.zeros(n_elements)
     d.update(s)
     return d
