@@ -15,6 +15,7 @@
 struct gr_model {
   grhip::ModelKind kind;
   std::shared_ptr<grhip::Model1L> m1;
+  std::shared_ptr<grhip::Model2L> m2;
   std::string path;
 };
 struct gr_engine {
@@ -113,9 +114,12 @@ int gr_model_load(const char *npz_path, gr_model **out)
     if (m->kind == grhip::ModelKind::Grace1L) {
       m->m1 = std::make_shared<grhip::Model1L>();
       m->m1->load(z);
+    } else if (m->kind == grhip::ModelKind::Grace2L) {
+      m->m2 = std::make_shared<grhip::Model2L>();
+      m->m2->load(z);
     } else {
-      throw grhip::InvalidArgument(std::string("unsupported model: this build of the GPU engine implements GRACE-1L; the file holds a GRACE-") +
-                                   (m->kind == grhip::ModelKind::Grace2L ? "2L" : "3L") + " model");
+      throw grhip::InvalidArgument("unsupported model: this build of the GPU engine implements GRACE-1L and GRACE-2L; the file holds a "
+                                   "GRACE-3L model");
     }
     *out = m.release();
   });
@@ -136,14 +140,24 @@ int gr_model_get_info(const gr_model *m, gr_model_info *info)
       double rc = 0.0;
       for (double c : m->m1->bond_cutoff_map) rc = std::max(rc, c);
       info->rcut = m->m1->has_bond_specific_cutoff ? rc : m->m1->rcut;
+    } else if (m->m2) {
+      info->n_elements = m->m2->n_elements;
+      info->lmax = m->m2->lmax;
+      info->n_radial = m->m2->C1;
+      info->n_radbase = m->m2->nradbase;
+      info->max_order = m->m2->max_order;
+      double rc = 0.0;
+      for (double c : m->m2->bond_cutoff_map) rc = std::max(rc, c);
+      info->rcut = m->m2->has_bond_specific_cutoff ? rc : m->m2->rcut;
     }
   });
 }
 
 const char *gr_model_element_name(const gr_model *m, int k)
 {
-  if (!m || !m->m1 || k < 0 || k >= (int) m->m1->element_names.size()) return "";
-  return m->m1->element_names[k].c_str();
+  if (!m || k < 0) return "";
+  const std::vector<std::string> &names = m->m1 ? m->m1->element_names : m->m2->element_names;
+  return k < (int) names.size() ? names[k].c_str() : "";
 }
 
 void gr_model_free(gr_model *m) { delete m; }
@@ -156,7 +170,8 @@ int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int prec
     if (ntypes < 1) throw grhip::InvalidArgument("ntypes must be positive");
     std::vector<int> t(type2mu, type2mu + ntypes + 1);
     auto e = std::make_unique<gr_engine>();
-    e->eng = grhip::make_engine_1l(m->m1, ntypes, t, precision, device);
+    if (m->m1) e->eng = grhip::make_engine_1l(m->m1, ntypes, t, precision, device);
+    else e->eng = grhip::make_engine_2l(m->m2, ntypes, t, precision, device);
     *out = e.release();
   });
 }

@@ -4,6 +4,7 @@
 #pragma once
 
 #include "model.hpp"
+#include "model_2l.hpp"
 
 #include <cstdint>
 #include <memory>
@@ -60,6 +61,10 @@ class Engine {
 
 // precision: 64 (network arithmetic in fp64) or 32 (fp32 network, fp64 geometry and sums)
 std::unique_ptr<Engine> make_engine_1l(std::shared_ptr<const Model1L> model, int ntypes, const std::vector<int> &type2mu,
+                                       int precision, int device);
+
+// GRACE-2L: network arithmetic in fp64 only (precision 64)
+std::unique_ptr<Engine> make_engine_2l(std::shared_ptr<const Model2L> model, int ntypes, const std::vector<int> &type2mu,
                                        int precision, int device);
 
 }    // namespace grhip

@@ -11,43 +11,18 @@ namespace {
 template<class T> class Engine1L final : public EngineBase {
  public:
   Engine1L(std::shared_ptr<const Model1L> m, int ntypes, const std::vector<int> &type2mu, int device) :
-      EngineBase(device, "GRACE-1L"), model_(std::move(m)), ntypes_(ntypes), type2mu_(type2mu)
+      EngineBase(device, "GRACE-1L", ntypes, type2mu, m->n_elements), model_(std::move(m))
   {
-    check_type2mu(type2mu_, ntypes_, model_->n_elements, "GRACE-1L");
     this->template probe_mfma<T>();
     build();
   }
 
   int layers() const override { return 1; }
-  double cutoff(int t1, int t2) const override
-  {
-    if (t1 < 1 || t1 > ntypes_ || t2 < 1 || t2 > ntypes_) return 0.0;
-    return model_->pair_cutoff(type2mu_[t1], type2mu_[t2]);
-  }
-  double max_cutoff() const override
-  {
-    double m = 0.0;
-    for (int a = 1; a <= ntypes_; a++)
-      for (int b = 1; b <= ntypes_; b++) m = std::max(m, cutoff(a, b));
-    return m;
-  }
-
-  void upload(const CsrInput &in) override;
   void run(const RunFlags &fl) override;
-  void fetch(double *energy, double *forces, double *virial, double *eatom) override;
-  int64_t last_edge_count() override
-  {
-    synchronize();
-    long long e = 0;
-    if (n_ > 0) HIP_CHECK(hipMemcpy(&e, eoff_.as<long long>() + n_, sizeof(e), hipMemcpyDeviceToHost));
-    return e;
-  }
   void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) override;
 
  private:
   std::shared_ptr<const Model1L> model_;
-  int ntypes_;
-  std::vector<int> type2mu_;
   bool jit_all_ = false;
 
   // model dimensions
@@ -58,7 +33,7 @@ template<class T> class Engine1L final : public EngineBase {
   ShCoef sh_{};
 
   // device tables
-  DevBuf cut_, z_, shift_;
+  DevBuf z_, shift_;
   DevRadial<T> rad_;
   DevFc<T> fcA1_, fcAA1_, fcAA2_;
   DevProd pAA_, pAAA_, pAAAA_;
@@ -66,17 +41,9 @@ template<class T> class Engine1L final : public EngineBase {
   DevBuf eW_[7];
   EnergyDev en_{};
 
-  // structure
-  int n_ = 0;
-  int64_t nb_ = 0;
-  bool have_rij_ = false;
-  DevBuf mu_, offset_, j_, rij_, x_, image_, shifts_, tiles_;
-  int ntiles_ = 0;
   // pass buffers
-  DevBuf count_, eoff_, zero_, ei_, ej_, emu_, rh_, r_, xr_, rc_, Rz_, dRz_;
+  DevBuf Rz_, dRz_;
   DevBuf A_, A1_, AA_, AA1_, AA2_, AAA_, AAAA_, gA_, gA1_, gAA_, gAA1_, gAA2_, gAAA_, gAAAA_, rho_, grho_;
-  DevBuf f_, eatom_, scal_;    // scal: energy, virial[6]
-  bool ran_ = false, ran_forces_ = false, ran_eatom_ = false;
 
   void build();
   void launch_gemm(DevJobs<T> &J, int kb0, int kb1, int nb, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo, int accumulate)
@@ -128,7 +95,7 @@ template<class T> void Engine1L<T>::build()
     std::vector<double> cut((size_t) nel_ * nel_);
     for (int a = 0; a < nel_; a++)
       for (int b = 0; b < nel_; b++) cut[(size_t) a * nel_ + b] = m.pair_cutoff(a, b);
-    upload_vec(cut_, cut);
+    set_cutoffs(cut);
     std::vector<T> z((size_t) nel_ * CP_, (T) 0);
     for (int mu = 0; mu < nel_; mu++)
       for (int n = 0; n < C_; n++) {
@@ -212,68 +179,6 @@ template<class T> void Engine1L<T>::build()
     en_.out_scale = m.output_scale;
     en_.shift = shift_.as<double>();
   }
-  scal_.ensure(8 * sizeof(double));
-  zero_.ensure(2 * sizeof(int));
-}
-
-template<class T> void Engine1L<T>::upload(const CsrInput &in)
-{
-  HIP_CHECK(hipSetDevice(device_));
-  if (in.n < 0) throw InvalidArgument("negative atom count");
-  const bool table = in.x && in.image && in.shifts;
-  if ((in.rij != nullptr) == (in.x || in.image || in.shifts) || (!in.rij && !table))
-    throw InvalidArgument("give rij or positions, image and shifts");
-  const int n = in.n;
-  std::vector<int> mu(n);
-  for (int a = 0; a < n; a++) {
-    if (in.types[a] < 1 || in.types[a] > ntypes_) throw InvalidArgument("types must be 1 .. len(species)");
-    mu[a] = type2mu_[in.types[a]];
-    if (mu[a] < 0)
-      throw Error("GRACE-1L: atom " + std::to_string(a) + " of unmapped type " + std::to_string(in.types[a]) + " in the atom list");
-  }
-  if (in.offset[0] != 0) throw InvalidArgument("offset[0] must be 0 and offset[-1] == len(j)");
-  for (int a = 0; a < n; a++)
-    if (in.offset[a + 1] < in.offset[a]) throw InvalidArgument("offset must be non-decreasing");
-  const int64_t nb = in.offset[n];
-  for (int64_t q = 0; q < nb; q++) {
-    if (in.j[q] < 0 || in.j[q] >= n) throw InvalidArgument("j must index atoms 0 .. len(types)-1");
-    if (in.image && (in.image[q] < 0 || in.image[q] >= in.nimages)) throw InvalidArgument("image must index rows of shifts");
-  }
-  HIP_CHECK(hipStreamSynchronize(stream_));
-  n_ = n;
-  nb_ = nb;
-  have_rij_ = in.rij != nullptr;
-  auto put = [&](DevBuf &b, const void *src, size_t bytes) {
-    b.ensure(std::max<size_t>(bytes, 8));
-    if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, hipMemcpyHostToDevice, stream_));
-  };
-  put(mu_, mu.data(), sizeof(int) * n);
-  // tiles of 16 atoms of one element, in atom order within an element
-  std::vector<int> tiles;
-  {
-    std::vector<int> ord(n);
-    std::iota(ord.begin(), ord.end(), 0);
-    std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return mu[a] < mu[b]; });
-    for (int q = 0; q < n;) {
-      int cnt = 0;
-      const int m0 = mu[ord[q]];
-      while (cnt < 16 && q < n && mu[ord[q]] == m0) { tiles.push_back(ord[q]); q++; cnt++; }
-      while (cnt < 16) { tiles.push_back(-1); cnt++; }
-    }
-  }
-  ntiles_ = (int) tiles.size() / 16;
-  put(tiles_, tiles.data(), sizeof(int) * tiles.size());
-  static_assert(sizeof(long long) == sizeof(int64_t), "offset type");
-  put(offset_, in.offset, sizeof(int64_t) * (n + 1));
-  put(j_, in.j, sizeof(int) * nb);
-  if (have_rij_) put(rij_, in.rij, sizeof(double) * 3 * nb);
-  else {
-    put(x_, in.x, sizeof(double) * 3 * n);
-    put(image_, in.image, sizeof(int) * nb);
-    put(shifts_, in.shifts, sizeof(double) * 3 * in.nimages);
-  }
-  HIP_CHECK(hipStreamSynchronize(stream_));    // the host copies (mu) go out of scope
-  ran_ = false;
 }
 
 template<class T>
@@ -285,41 +190,9 @@ void Engine1L<T>::launch_radial(long long e_begin, long long e_count, const doub
 
 template<class T> void Engine1L<T>::run(const RunFlags &fl)
 {
-  HIP_CHECK(hipSetDevice(device_));
-  ev_used_ = 0;
   const int n = n_;
-  // ---- outputs
-  f_.ensure(std::max<size_t>((size_t) 3 * n, 1) * sizeof(double));
-  eatom_.ensure(std::max<size_t>(n, 1) * sizeof(double));
-  HIP_CHECK(hipMemsetAsync(f_.p, 0, (size_t) 3 * n * sizeof(double), stream_));
-  HIP_CHECK(hipMemsetAsync(scal_.p, 0, 8 * sizeof(double), stream_));
-  ran_ = true;
-  ran_forces_ = !fl.energy_only;
-  ran_eatom_ = fl.eatom;
-  if (n == 0) return;
-  // ---- bond filter and compaction
-  count_.ensure(sizeof(int) * n);
-  eoff_.ensure(sizeof(long long) * (n + 1));
-  {
-    const int init[2] = {-1, -1};
-    HIP_CHECK(hipMemcpyAsync(zero_.p, init, sizeof(init), hipMemcpyHostToDevice, stream_));
-  }
-  BondSrc src{};
-  src.mu = mu_.as<int>(); src.offset = offset_.as<long long>(); src.j = j_.as<int>();
-  src.rij = have_rij_ ? rij_.as<double>() : nullptr;
-  src.x = have_rij_ ? nullptr : x_.as<double>();
-  src.image = have_rij_ ? nullptr : image_.as<int>();
-  src.shifts = have_rij_ ? nullptr : shifts_.as<double>();
-  src.cut = cut_.as<double>(); src.nel = nel_;
+  if (!begin_pass(fl)) return;
   const size_t ecap = (size_t) std::max<int64_t>(nb_, 1);
-  ei_.ensure(ecap * sizeof(int)); ej_.ensure(ecap * sizeof(int)); emu_.ensure(ecap * sizeof(int));
-  rh_.ensure(ecap * 3 * sizeof(double)); r_.ensure(ecap * sizeof(double)); xr_.ensure(ecap * sizeof(double));
-  rc_.ensure(ecap * sizeof(double));
-  Edges ed{ei_.as<int>(), ej_.as<int>(), emu_.as<int>(), rh_.as<double>(), r_.as<double>(), xr_.as<double>(), rc_.as<double>()};
-  const int wpb = 4;
-  stage("edge_count", [&] { hipLaunchKernelGGL(k_edge_count, dim3((n + wpb - 1) / wpb), dim3(64 * wpb), 0, stream_, src, n, count_.as<int>(), zero_.as<int>()); });
-  stage("edge_scan", [&] { hipLaunchKernelGGL(k_scan, dim3(1), dim3(1024), 0, stream_, count_.as<int>(), n, eoff_.as<long long>()); });
-  stage("edge_fill", [&] { hipLaunchKernelGGL(k_edge_fill, dim3((n + wpb - 1) / wpb), dim3(64 * wpb), 0, stream_, src, n, eoff_.as<long long>(), ed); });
 
   // ---- radial functions of all edges
   Rz_.ensure(ecap * noutp_ * sizeof(T));
@@ -472,27 +345,6 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
       default: hipLaunchKernelGGL((k_bond_bwd<T, 4>), dim3(n), dim3(256), lds, stream_, ba); break;
     }
   });
-}
-
-template<class T> void Engine1L<T>::fetch(double *energy, double *forces, double *virial, double *eatom)
-{
-  HIP_CHECK(hipSetDevice(device_));
-  if (!ran_) throw Error("fetch() before run()");
-  HIP_CHECK(hipStreamSynchronize(stream_));
-  if (n_ > 0) {
-    int zb[2];
-    HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
-    if (zb[0] >= 0)    // bonds.h:49-62
-      throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " +
-                  std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
-  }
-  double s[8];
-  HIP_CHECK(hipMemcpy(s, scal_.p, sizeof(s), hipMemcpyDeviceToHost));
-  if (energy) *energy = s[0];
-  if (virial && ran_forces_)
-    for (int k = 0; k < 6; k++) virial[k] = s[1 + k];
-  if (forces && ran_forces_ && n_ > 0) HIP_CHECK(hipMemcpy(forces, f_.p, sizeof(double) * 3 * n_, hipMemcpyDeviceToHost));
-  if (eatom && ran_eatom_ && n_ > 0) HIP_CHECK(hipMemcpy(eatom, eatom_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
 }
 
 template<class T> void Engine1L<T>::debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz)

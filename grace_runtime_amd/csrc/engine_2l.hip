@@ -1,0 +1,574 @@
+// GRACE-2L engine for gfx950: two message-passing layers on one GPU, whole structure resident.
+// Phases after libgrace/src/fused_2l.cpp:849-1099 of the reference (P1 layer 1 forward -> message I and rho of every
+// atom; P3 layer 2, readout, layer-2 reverse with dE/dI_j added to the neighbours; P5 layer 1 reverse), without the
+// layer-1 recompute: the layer-1 tensors of all atoms stay in device memory between P1 and P5.
+// Dense chains (FC, CG products, reduces) reuse the GRACE-1L kernels; liveness pruning after fused_2l.cpp:296-345.
+#include "engine_common.hpp"
+#include "kernels_2l.hpp"
+#include "model_2l.hpp"
+
+namespace grhip {
+
+namespace {
+
+// One dense chain X -> X1 = FC(X, X) -> XX = X1 x X1 -> XX1 = FC(XX, X) -> XXX = XX1 x X [-> XX2 = FC(XX, X) ->
+// XXXX = XX2 x XX2] of a layer (X = A or B), all tensors of one padded channel width.
+template<class T> struct Chain {
+  int nf = 0, nXX = 0, nXXX = 0, nXXXX = 0, kb = 0;    // functions of X, XX, XXX, XXXX; 16-channel blocks
+  bool order4 = false, jit_all = false;
+  DevFc<T> fc1, fc2, fc3;
+  DevProd p2, p3, p4;
+  DevBuf X1, XX, XX1, XXX, XX2, XXXX, gX, gX1, gXX, gXX1, gXXX, gXX2, gXXXX;
+  const T *src(int s, const T *X) const
+  {
+    return s == 0 ? X : s == 1 ? XX.as<T>() : s == 2 ? XXX.as<T>() : XXXX.as<T>();
+  }
+  T *gsrc(int s) const { return s == 0 ? gX.as<T>() : s == 1 ? gXX.as<T>() : s == 2 ? gXXX.as<T>() : gXXXX.as<T>(); }
+  int nfun(int s) const { return s == 0 ? nf : s == 1 ? nXX : s == 2 ? nXXX : nXXXX; }
+};
+
+template<class T> class Engine2L final : public EngineBase {
+ public:
+  Engine2L(std::shared_ptr<const Model2L> m, int ntypes, const std::vector<int> &type2mu, int device) :
+      EngineBase(device, "GRACE-2L", ntypes, type2mu, m->n_elements), model_(std::move(m))
+  {
+    this->template probe_mfma<T>();
+    build();
+  }
+  int layers() const override { return 2; }
+  void run(const RunFlags &fl) override;
+  void debug_radial(int, const double *, const int *, double *, double *) override
+  {
+    throw Error("GRACE-2L: debug_radial is available for GRACE-1L engines");
+  }
+
+ private:
+  std::shared_ptr<const Model2L> model_;
+  int lmax_ = 0, nl_ = 0, nlm_ = 0, nel_ = 0, C1P_ = 0, CRP_ = 0, C2P_ = 0, PI1_ = 0, nI1_ = 0, nI_ = 0, nslot_ = 0, nB_ = 0, nrho_ = 0;
+  bool order4_ = false;
+  ShCoef sh_{};
+  DevBuf zA_, zB0_, ones_, shift_, lnI_, ln0_, eW_[7];
+  DevRadial<T> radR_, radR1_;
+  Chain<T> c1_, c2_;
+  DevReduce<T> redrho_, redI2_;
+  std::vector<std::unique_ptr<DevReduce<T>>> redI1_;    // one per output function of I1
+  DevBuf WI_, WIT_, WB_, WBT_;
+  DevJobs<T> jI_, jIb_, jB_, jBb_;
+  Energy2Dev en_{};
+  // pass buffers
+  DevBuf Rz_, dRz_, R1_, dR1_, Y_, YG_, A_, rho_, grho_, I1_, gI1_, M_, gM_, P_, gP_, B_, I2_, gI2_;
+
+  void build();
+  void build_chain(Chain<T> &c, const char *tag, int nf, int KP, const FCWeights *fc[3], const CGProduct *pr[3],
+                   const std::vector<const ReduceEq *> reds[4]);
+  void gemm(DevJobs<T> &J, int kb0, int nb, const T *X0, int nf0, T *out, int nfo, int accumulate)
+  {
+    EngineBase::launch_gemm<T>(J, kb0, kb0, nb, X0, nf0, X0, nf0, out, nfo, accumulate, tiles_.as<int>(), ntiles_);
+  }
+  void chain_forward(Chain<T> &c, const char *tag, const T *X);
+  void chain_zero(Chain<T> &c, const char *tag);
+  void chain_backward(Chain<T> &c, const char *tag, const T *X);
+  void reduce_fwd(DevReduce<T> &R, int kb, const Chain<T> &c, const T *X, double *out);
+  void reduce_bwd(DevReduce<T> &R, const Chain<T> &c, const double *g);
+  std::string tagged(const char *tag, const char *name) { return std::string(name) + tag; }
+};
+
+template<class T>
+void Engine2L<T>::build_chain(Chain<T> &c, const char *tag, int nf, int KP, const FCWeights *fc[3], const CGProduct *pr[3],
+                              const std::vector<const ReduceEq *> reds[4])
+{
+  c.nf = nf;
+  c.kb = KP / 16;
+  c.order4 = order4_;
+  c.nXX = pr[0]->n_out;
+  c.nXXX = pr[1]->n_out;
+  c.nXXXX = order4_ ? pr[2]->n_out : 0;
+  auto collected = [&](int s, int n) {
+    std::vector<char> v(n, 0);
+    for (const ReduceEq *r : reds[s])
+      for (int q : r->collect_ind) v[q] = 1;
+    return v;
+  };
+  HostProd h3 = build_prod(*pr[1], collected(2, c.nXXX), c.nXX, nf);
+  std::vector<char> live2(c.nXX, 0), live3(c.nXX, 0), live1(nf, 0);
+  for (int q : h3.l) live2[q] = 1;
+  HostProd h4;
+  if (order4_) {
+    h4 = build_prod(*pr[2], collected(3, c.nXXXX), c.nXX, c.nXX);
+    for (int q : h4.l) live3[q] = 1;
+    for (int q : h4.r) live3[q] = 1;
+  }
+  std::vector<char> need2 = collected(1, c.nXX);
+  for (int q = 0; q < c.nXX; q++) need2[q] = need2[q] || live2[q] || live3[q];
+  HostProd h2 = build_prod(*pr[0], need2, nf, nf);
+  for (int q : h2.l) live1[q] = 1;
+  for (int q : h2.r) live1[q] = 1;
+  c.p2.build(h2);
+  c.p3.build(h3);
+  if (order4_) c.p4.build(h4);
+  const bool f32 = sizeof(T) == 4;
+  const std::string t(tag);
+  jit_compile_product(("prod2" + t).c_str(), h2.terms, nf, nf, c.nXX, true, KP, f32, arch_, c.p2.jit, c.p2.jit_note);
+  jit_compile_product(("prod3" + t).c_str(), h3.terms, c.nXX, nf, c.nXXX, false, KP, f32, arch_, c.p3.jit, c.p3.jit_note);
+  if (order4_) jit_compile_product(("prod4" + t).c_str(), h4.terms, c.nXX, c.nXX, c.nXXXX, true, KP, f32, arch_, c.p4.jit, c.p4.jit_note);
+  c.jit_all = c.p2.jit.ok() && c.p3.jit.ok() && (!order4_ || c.p4.jit.ok());
+  c.fc1.build(*fc[0], live1, nf, KP, KP, KP, drow_);
+  c.fc2.build(*fc[1], live2, nf, KP, KP, KP, drow_);
+  if (order4_) c.fc3.build(*fc[2], live3, nf, KP, KP, KP, drow_);
+}
+
+template<class T> void Engine2L<T>::build()
+{
+  const Model2L &m = *model_;
+  lmax_ = m.lmax;
+  if (lmax_ > kKernMaxL) throw Error("GRACE-2L: lmax > " + std::to_string(kKernMaxL) + " not supported");
+  nl_ = lmax_ + 1;
+  nlm_ = nl_ * nl_;
+  nel_ = m.n_elements;
+  order4_ = m.max_order == 4;
+  nrho_ = m.rho_n_out;
+  nI1_ = m.I1_n_funcs;
+  nI_ = m.I_n_funcs;
+  nslot_ = nI_ + 1;
+  nB_ = m.B_n_funcs;
+  auto pad_width = [](int c) { return c <= 16 ? 16 : c <= 32 ? 32 : c <= 64 ? 64 : -1; };
+  C1P_ = pad_width(m.C1);
+  CRP_ = pad_width(m.CR);
+  C2P_ = pad_width(m.C2);
+  PI1_ = pad_width(m.I1_n_out);
+  if (C1P_ < 0 || CRP_ < 0 || C2P_ < 0 || PI1_ < 0) throw Error("GRACE-2L: channel widths above 64 are not supported by the GPU kernels");
+  if (nrho_ > 32 || m.I1_n_out > 32) throw Error("GRACE-2L: rho_n_out or I1_n_out > 32 not supported by the GPU reduce kernels");
+  if (nslot_ * CRP_ > 1024) throw Error("GRACE-2L: (I_n_funcs + 1) x message width exceeds one block");
+
+  std::memset(&sh_, 0, sizeof(sh_));
+  sh_.lmax = lmax_;
+  for (int l = 2; l <= lmax_; l++) {
+    for (int mm = 0; mm < l - 1; mm++) {
+      const double l2 = l * l, m2 = mm * mm, lm1 = l - 1;
+      sh_.a[l * (l + 1) / 2 + mm] = std::sqrt((4.0 * l2 - 1.0) / (l2 - m2));
+      sh_.b[l * (l + 1) / 2 + mm] = -std::sqrt((lm1 * lm1 - m2) / (4.0 * lm1 * lm1 - 1.0));
+    }
+    sh_.c[l] = -std::sqrt(1.0 + 0.5 / l);
+    sh_.d[l] = std::sqrt(2.0 * l + 1.0);
+  }
+  // ---- pair cutoffs, species weights zA, zB0 (fused_2l.cpp:176-192), unit weights for the bare layer-2 radial functions
+  {
+    std::vector<double> cut((size_t) nel_ * nel_);
+    for (int a = 0; a < nel_; a++)
+      for (int b = 0; b < nel_; b++) cut[(size_t) a * nel_ + b] = m.pair_cutoff(a, b);
+    set_cutoffs(cut);
+    auto ztab = [&](const std::vector<double> &W, double norm, double inv, int C, int CP) {
+      std::vector<T> z((size_t) nel_ * CP, (T) 0);
+      for (int mu = 0; mu < nel_; mu++)
+        for (int n = 0; n < C; n++) {
+          double v = 0.0;
+          for (int e = 0; e < m.embedding_size; e++) v += W[(size_t) e * C + n] * m.chem_embedding[(size_t) mu * m.embedding_size + e];
+          z[(size_t) mu * CP + n] = (T) (v * norm * inv);
+        }
+      return z;
+    };
+    upload_vec(zA_, ztab(m.A_lin_transform_W, m.A_lin_transform_norm, m.A_inv_avg_n_neigh, m.C1, C1P_));
+    upload_vec(zB0_, ztab(m.B0_lin_transform_W, m.B0_lin_transform_norm, m.B0_inv_avg_n_neigh, m.CR, CRP_));
+    upload_vec(ones_, std::vector<T>((size_t) nel_ * CRP_, (T) 1));
+    upload_vec(shift_, m.shift_values);
+  }
+  radR_.build(m.mlp_R, m.nradbase, m.radial_basis_p, m.radial_activation, m.C1, C1P_, nl_, nel_, drow_, "GRACE-2L");
+  radR1_.build(m.mlp_R1, m.nradbase, m.radial_basis_p, m.radial_activation, m.CR, CRP_, nl_, nel_, drow_, "GRACE-2L");
+
+  // ---- the two dense chains
+  const int ns = m.nsrc();
+  {
+    const FCWeights *fc[3] = {&m.fc_A1, &m.fc_AA1, &m.fc_AA2};
+    const CGProduct *pr[3] = {&m.prod_AA, &m.prod_AAA, &m.prod_AAAA};
+    std::vector<const ReduceEq *> reds[4];
+    for (int s = 0; s < ns; s++) reds[s] = {&m.I1_red[s], &m.rho_red[s]};
+    build_chain(c1_, "_L1", nlm_, C1P_, fc, pr, reds);
+  }
+  {
+    const FCWeights *fc[3] = {&m.fc_B1, &m.fc_BB1, &m.fc_BB2};
+    const CGProduct *pr[3] = {&m.prod_BB, &m.prod_BBB, &m.prod_BBBB};
+    std::vector<const ReduceEq *> reds[4];
+    for (int s = 0; s < ns; s++) reds[s] = {&m.I2_red[s]};
+    build_chain(c2_, "_L2", nB_, C2P_, fc, pr, reds);
+  }
+  // ---- element-dependent reduces: rho, I1 (one per output function), I2
+  auto sources = [&](const ReduceEq *r, const Chain<T> &c, int KP, bool with_fo) {
+    std::vector<ReduceSrc> v;
+    for (int s = 0; s < ns; s++)
+      v.push_back({&r[s].W, r[s].norm, r[s].n_in, r[s].w_shape, &r[s].collect_ind, &r[s].w_l_tile, with_fo ? &r[s].total_sum_ind : nullptr,
+                   c.nfun(s), KP});
+    return v;
+  };
+  redrho_.build(sources(m.rho_red, c1_, C1P_, false), nel_, nrho_, -1, nrho_, 0, drow_);
+  redI2_.build(sources(m.I2_red, c2_, C2P_, false), nel_, nrho_, -1, nrho_, 0, drow_);
+  for (int fo = 0; fo < nI1_; fo++) {
+    redI1_.emplace_back(new DevReduce<T>());
+    redI1_.back()->build(sources(m.I1_red, c1_, C1P_, true), nel_, m.I1_n_out, fo, nI1_ * PI1_, fo * PI1_, drow_);
+  }
+  // ---- I from I1 and B from (YI, B0): tile-GEMM job lists (weights not element dependent).  W: [n_out][n_in][w_shape]
+  auto tile_frags = [&](const ReduceEq &r, int nout, int KinP, int NoutP, std::vector<T> &F, std::vector<T> &Ft) {
+    std::vector<double> Mx((size_t) r.n_in * nout), Mt((size_t) nout * r.n_in);
+    for (int t = 0; t < r.w_shape; t++) {
+      for (int k = 0; k < nout; k++)
+        for (int n = 0; n < r.n_in; n++) {
+          const double v = r.norm * r.W[((size_t) k * r.n_in + n) * r.w_shape + t];
+          Mx[(size_t) n * nout + k] = v;
+          Mt[(size_t) k * r.n_in + n] = v;
+        }
+      pack_fragments<T>(Mx, r.n_in, nout, KinP, NoutP, F);
+      pack_fragments<T>(Mt, nout, r.n_in, NoutP, KinP, Ft);
+    }
+  };
+  {
+    const ReduceEq &r = m.I_red;
+    std::vector<T> F, Ft;
+    tile_frags(r, m.CR, PI1_, CRP_, F, Ft);
+    upload_vec(WI_, F);
+    upload_vec(WIT_, Ft);
+    typename DevJobs<T>::Host hf, hb;
+    for (int fo = 0; fo < nI_; fo++) {
+      hf.job(fo, 1.0);
+      for (size_t c = 0; c < r.collect_ind.size(); c++)
+        if (r.total_sum_ind[c] == fo) hf.seg(0, r.collect_ind[c], r.w_l_tile[c], 1.0);
+      hf.end_job();
+    }
+    for (int fi = 0; fi < nI1_; fi++) {
+      hb.job(fi, 1.0);
+      for (size_t c = 0; c < r.collect_ind.size(); c++)
+        if (r.collect_ind[c] == fi) hb.seg(0, r.total_sum_ind[c], r.w_l_tile[c], 1.0);
+      hb.end_job();
+    }
+    jI_.build(hf, WI_.as<T>(), WI_.as<T>());
+    jIb_.build(hb, WIT_.as<T>(), WIT_.as<T>());
+    jI_.set_rows(drow_);
+    jIb_.set_rows(drow_);
+  }
+  {
+    // B[fo] = sum over YI connections c -> fo of W_YI[tile c] YI[ci c]  +  sum over B0 connections of W_B0[tile c] B0[ci c],
+    // YI[o] = inv_avg sum_t cg_t P[(I_t, y_t)] (fused_2l.cpp:228-276, 655-665) folded in: one segment per coupling term.
+    // The pair tensor P has functions slot * nlm + lm; slot nI is B0.
+    const ReduceEq &ry = m.B_red_YI, &r0 = m.B_red_B0;
+    std::vector<T> F, Ft;
+    tile_frags(ry, m.C2, CRP_, C2P_, F, Ft);
+    tile_frags(r0, m.C2, CRP_, C2P_, F, Ft);
+    upload_vec(WB_, F);
+    upload_vec(WBT_, Ft);
+    struct Seg { int fo, pair, tile; double scale; };
+    std::vector<Seg> segs;
+    for (size_t c = 0; c < ry.collect_ind.size(); c++)
+      for (int t = 0; t < m.yi.n_terms; t++)
+        if (m.yi.m_sum_ind[t] == ry.collect_ind[c])
+          segs.push_back({ry.total_sum_ind[c], m.yi.i[t] * nlm_ + m.yi.y[t], ry.w_l_tile[c], m.yi.cg_coeff[t] * m.yi.inv_avg_n_neigh});
+    for (size_t c = 0; c < r0.collect_ind.size(); c++)
+      segs.push_back({r0.total_sum_ind[c], nI_ * nlm_ + r0.collect_ind[c], ry.w_shape + r0.w_l_tile[c], 1.0});
+    typename DevJobs<T>::Host hf, hb;
+    for (int fo = 0; fo < nB_; fo++) {
+      hf.job(fo, 1.0);
+      for (const Seg &s : segs)
+        if (s.fo == fo) hf.seg(0, s.pair, s.tile, s.scale);
+      hf.end_job();
+    }
+    for (int p = 0; p < nslot_ * nlm_; p++) {
+      bool any = false;
+      for (const Seg &s : segs) any = any || s.pair == p;
+      if (!any) continue;
+      hb.job(p, 1.0);
+      for (const Seg &s : segs)
+        if (s.pair == p) hb.seg(0, s.fo, s.tile, s.scale);
+      hb.end_job();
+    }
+    jB_.build(hf, WB_.as<T>(), WB_.as<T>());
+    jBb_.build(hb, WBT_.as<T>(), WBT_.as<T>());
+    jB_.set_rows(drow_);
+    jBb_.set_rows(drow_);
+  }
+  // ---- readout
+  {
+    en_.nlay = (int) m.energy_mlp.size();
+    for (int L = 0; L < en_.nlay; L++) {
+      upload_vec(eW_[L], m.energy_mlp[L].W);
+      en_.W[L] = eW_[L].template as<double>();
+      en_.norm[L] = m.energy_mlp[L].norm;
+      en_.nin[L] = m.energy_mlp[L].n_in;
+      en_.nout[L] = m.energy_mlp[L].n_out;
+    }
+    upload_vec(lnI_, m.I_nl_LN_scale);
+    upload_vec(ln0_, m.I_0_LN_scale);
+    en_.act = m.energy_mlp_activation;
+    en_.ln = m.energy_mlp_ln;
+    en_.nrho = nrho_;
+    en_.rms = m.energy_rms_norm;
+    en_.eps = Model2L::rms_norm_eps;
+    en_.out_scale = m.output_scale;
+    en_.shift = shift_.as<double>();
+    en_.lnI = lnI_.as<double>();
+    en_.ln0 = ln0_.as<double>();
+  }
+}
+
+template<class T> void Engine2L<T>::chain_forward(Chain<T> &c, const char *tag, const T *X)
+{
+  const int n = n_, KP = c.kb * 16;
+  const size_t na = (size_t) n;
+  c.X1.ensure(na * c.nf * KP * sizeof(T));
+  c.XX.ensure(na * c.nXX * KP * sizeof(T));
+  c.XX1.ensure(na * c.nXX * KP * sizeof(T));
+  c.XXX.ensure(na * c.nXXX * KP * sizeof(T));
+  if (c.order4) {
+    c.XX2.ensure(na * c.nXX * KP * sizeof(T));
+    c.XXXX.ensure(na * std::max(c.nXXXX, 1) * KP * sizeof(T));
+  }
+  int one = 1, nat = n;
+  auto prod = [&](const std::string &name, DevProd &P, const T *L, const T *R, T *out, int sl, int sr) {
+    if (P.jit.ok()) {
+      stage(name.c_str(), [&] {
+        void *args[] = {(void *) &L, (void *) &R, (void *) &out, (void *) &nat, (void *) &one};
+        const long long cols = (long long) n * KP;
+        HIP_CHECK(hipModuleLaunchKernel(P.jit.fwd, (unsigned) ((cols + 255) / 256), 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+      });
+      return;
+    }
+    const int AT = std::max(1, 256 / KP);
+    stage(name.c_str(), [&] {
+      hipLaunchKernelGGL(k_prod_fwd<T>, dim3(P.d.nout * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, P.d, L, R, out, n, KP, sl, sr);
+    });
+  };
+  T *X1 = c.X1.template as<T>(), *XX = c.XX.template as<T>(), *XX1 = c.XX1.template as<T>(), *XXX = c.XXX.template as<T>(),
+    *XX2 = c.XX2.template as<T>(), *XXXX = c.XXXX.template as<T>();
+  stage(tagged(tag, "fc_1").c_str(), [&] { launch_gemm<T>(c.fc1.fwd, c.kb, c.kb, c.kb, X, c.nf, X, c.nf, X1, c.nf, 0, tiles_.as<int>(), ntiles_); });
+  prod(tagged(tag, "prod_2"), c.p2, X1, X1, XX, c.nf, c.nf);
+  stage(tagged(tag, "fc_2").c_str(), [&] { launch_gemm<T>(c.fc2.fwd, c.kb, c.kb, c.kb, XX, c.nXX, X, c.nf, XX1, c.nXX, 0, tiles_.as<int>(), ntiles_); });
+  prod(tagged(tag, "prod_3"), c.p3, XX1, X, XXX, c.nXX, c.nf);
+  if (c.order4) {
+    stage(tagged(tag, "fc_3").c_str(), [&] { launch_gemm<T>(c.fc3.fwd, c.kb, c.kb, c.kb, XX, c.nXX, X, c.nf, XX2, c.nXX, 0, tiles_.as<int>(), ntiles_); });
+    prod(tagged(tag, "prod_4"), c.p4, XX2, XX2, XXXX, c.nXX, c.nXX);
+  }
+}
+
+template<class T> void Engine2L<T>::chain_zero(Chain<T> &c, const char *tag)
+{
+  const size_t na = (size_t) n_, KP = c.kb * 16;
+  c.gX.ensure(na * c.nf * KP * sizeof(T));
+  c.gX1.ensure(na * c.nf * KP * sizeof(T));
+  c.gXX.ensure(na * c.nXX * KP * sizeof(T));
+  c.gXX1.ensure(na * c.nXX * KP * sizeof(T));
+  c.gXXX.ensure(na * c.nXXX * KP * sizeof(T));
+  if (c.order4) {
+    c.gXX2.ensure(na * c.nXX * KP * sizeof(T));
+    c.gXXXX.ensure(na * std::max(c.nXXXX, 1) * KP * sizeof(T));
+  }
+  stage(tagged(tag, "zero_grads").c_str(), [&] {
+    HIP_CHECK(hipMemsetAsync(c.gX.p, 0, na * c.nf * KP * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(c.gX1.p, 0, na * c.nf * KP * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(c.gXX.p, 0, na * c.nXX * KP * sizeof(T), stream_));
+    // with the specialised product kernels gXX1 and gXX2 are written (not accumulated) by their producer
+    if (!c.jit_all) HIP_CHECK(hipMemsetAsync(c.gXX1.p, 0, na * c.nXX * KP * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(c.gXXX.p, 0, na * c.nXXX * KP * sizeof(T), stream_));
+    if (c.order4) {
+      if (!c.jit_all) HIP_CHECK(hipMemsetAsync(c.gXX2.p, 0, na * c.nXX * KP * sizeof(T), stream_));
+      HIP_CHECK(hipMemsetAsync(c.gXXXX.p, 0, na * std::max(c.nXXXX, 1) * KP * sizeof(T), stream_));
+    }
+  });
+}
+
+// reverse of the chain; the reduces have added their adjoints to gX, gXX, gXXX, gXXXX.  Result in c.gX.
+template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag, const T *X)
+{
+  const int n = n_, KP = c.kb * 16;
+  int one = 1, nat = n;
+  auto prod_bwd = [&](const std::string &name, DevProd &P, const T *L, const T *R, const T *g, T *gL, T *gR, int sl, int sr, int accL, int accR) {
+    if (P.jit.ok()) {
+      if (!c.jit_all) accL = accR = 1;
+      stage(name.c_str(), [&] {
+        void *args[] = {(void *) &L, (void *) &R, (void *) &g, (void *) &gL, (void *) &gR, (void *) &accL, (void *) &accR, (void *) &nat, (void *) &one};
+        const long long cols = (long long) n * KP;
+        HIP_CHECK(hipModuleLaunchKernel(P.jit.bwd, (unsigned) ((cols + 255) / 256), 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+      });
+      return;
+    }
+    const int AT = std::max(1, 256 / KP);
+    stage(name.c_str(), [&] {
+      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nleft * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, P.d, 0, R, g, gL, n, KP, sr, sl);
+      hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nright * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, P.d, 1, L, g, gR, n, KP, sl, sr);
+    });
+  };
+  auto fc_bwd = [&](const std::string &name, DevFc<T> &F, const T *g, T *gXl, T *gXr, int nfl) {
+    stage(name.c_str(), [&] {
+      launch_gemm<T>(F.bwd_l, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXl, nfl, 1, tiles_.as<int>(), ntiles_);
+      launch_gemm<T>(F.bwd_r, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXr, c.nf, 1, tiles_.as<int>(), ntiles_);
+    });
+  };
+  const T *X1 = c.X1.template as<T>(), *XX1 = c.XX1.template as<T>(), *XX2 = c.XX2.template as<T>();
+  T *gX = c.gX.template as<T>(), *gX1 = c.gX1.template as<T>(), *gXX = c.gXX.template as<T>(), *gXX1 = c.gXX1.template as<T>(),
+    *gXXX = c.gXXX.template as<T>(), *gXX2 = c.gXX2.template as<T>(), *gXXXX = c.gXXXX.template as<T>();
+  if (c.order4) {
+    prod_bwd(tagged(tag, "prod_4_bwd"), c.p4, XX2, XX2, gXXXX, gXX2, gXX2, c.nXX, c.nXX, 0, 0);
+    fc_bwd(tagged(tag, "fc_3_bwd"), c.fc3, gXX2, gXX, gX, c.nXX);
+  }
+  prod_bwd(tagged(tag, "prod_3_bwd"), c.p3, XX1, X, gXXX, gXX1, gX, c.nXX, c.nf, 0, 1);
+  fc_bwd(tagged(tag, "fc_2_bwd"), c.fc2, gXX1, gXX, gX, c.nXX);
+  prod_bwd(tagged(tag, "prod_2_bwd"), c.p2, X1, X1, gXX, gX1, gX1, c.nf, c.nf, 1, 1);
+  fc_bwd(tagged(tag, "fc_1_bwd"), c.fc1, gX1, gX, gX, c.nf);
+}
+
+template<class T> void Engine2L<T>::reduce_fwd(DevReduce<T> &R, int kb, const Chain<T> &c, const T *X, double *out)
+{
+  const int *tiles = tiles_.as<int>();
+#define GR_RED(KA) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KA>), dim3(ntiles_), dim3(256), 0, stream_, R.d, mu_.as<int>(), tiles, \
+                                      c.src(0, X), c.src(1, X), c.src(2, X), c.src(3, X), out)
+  switch (kb) {
+    case 1: GR_RED(1); break;
+    case 2: GR_RED(2); break;
+    case 4: GR_RED(4); break;
+    default: throw Error("unsupported channel widths");
+  }
+#undef GR_RED
+}
+
+template<class T> void Engine2L<T>::reduce_bwd(DevReduce<T> &R, const Chain<T> &c, const double *g)
+{
+  if (R.njobs == 0) return;
+  hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, R.njobs), dim3(64), 0, stream_, R.d, mu_.as<int>(), tiles_.as<int>(), g, c.gsrc(0), c.gsrc(1),
+                     c.gsrc(2), c.gsrc(3));
+}
+
+template<class T> void Engine2L<T>::run(const RunFlags &fl)
+{
+  static_assert(sizeof(T) == 8, "the GRACE-2L engine computes in fp64");
+  const int n = n_;
+  if (!begin_pass(fl)) return;
+  const size_t ecap = (size_t) std::max<int64_t>(nb_, 1), na = (size_t) n;
+  const long long *n_edges = eoff_.as<long long>() + n;
+  const bool forces = !fl.energy_only;
+
+  // ---- per-edge quantities: radial functions of both layers, spherical harmonics
+  Rz_.ensure(ecap * radR_.noutp * sizeof(T));
+  dRz_.ensure(ecap * radR_.noutp * sizeof(T));
+  R1_.ensure(ecap * radR1_.noutp * sizeof(T));
+  dR1_.ensure(ecap * radR1_.noutp * sizeof(T));
+  stage("radial_R", [&] { radR_.launch(stream_, ncu_, zA_.as<T>(), 0, -1, xr_.as<double>(), emu_.as<int>(), Rz_.as<T>(), dRz_.as<T>(), n_edges); });
+  stage("radial_R1", [&] { radR1_.launch(stream_, ncu_, ones_.as<T>(), 0, -1, xr_.as<double>(), emu_.as<int>(), R1_.as<T>(), dR1_.as<T>(), n_edges); });
+  Y_.ensure(ecap * nlm_ * sizeof(T));
+  if (forces) YG_.ensure(ecap * nlm_ * 4 * sizeof(T));
+  stage("sh_edges", [&] {
+    hipLaunchKernelGGL(k_sh_edges<T>, dim3((unsigned) ((ecap + 127) / 128)), dim3(128), 0, stream_, sh_, rh_.as<double>(), n_edges, nlm_,
+                       Y_.as<T>(), forces ? YG_.as<T>() : (T *) nullptr);
+  });
+
+  // ---- P1: layer 1 forward
+  A_.ensure(na * nlm_ * C1P_ * sizeof(T));
+  T *A = A_.as<T>();
+  {
+    ScatterArgs<T> sa{};
+    sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz_.as<T>(); sa.A = A;
+    sa.a0 = 0; sa.C = C1P_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = radR_.noutp; sa.sh = sh_;
+    const int sthreads = round_up(nl_ * C1P_, 64);
+    stage("scatter_A", [&] {
+      if (lmax_ <= 4) hipLaunchKernelGGL((k_scatter_a<T, 9>), dim3(n), dim3(sthreads), 0, stream_, sa);
+      else hipLaunchKernelGGL((k_scatter_a<T, 13>), dim3(n), dim3(sthreads), 0, stream_, sa);
+    });
+  }
+  chain_forward(c1_, "_L1", A);
+  rho_.ensure(na * nrho_ * sizeof(double));
+  grho_.ensure(na * nrho_ * sizeof(double));
+  if (I1_.bytes < na * nI1_ * PI1_ * sizeof(double)) {
+    I1_.ensure(na * nI1_ * PI1_ * sizeof(double));
+    HIP_CHECK(hipMemsetAsync(I1_.p, 0, I1_.bytes, stream_));    // the padding channels stay zero
+  }
+  stage("reduce_rho", [&] { reduce_fwd(redrho_, c1_.kb, c1_, A, rho_.as<double>()); });
+  stage("reduce_I1", [&] {
+    for (auto &r : redI1_) reduce_fwd(*r, c1_.kb, c1_, A, I1_.as<double>());
+  });
+  M_.ensure(na * nslot_ * CRP_ * sizeof(T));
+  T *M = M_.as<T>();
+  stage("reduce_I", [&] {
+    gemm(jI_, PI1_ / 16, CRP_ / 16, I1_.as<T>(), nI1_, M, nslot_, 0);
+    hipLaunchKernelGGL(k_fill_slot<T>, dim3((unsigned) ((na * CRP_ + 255) / 256)), dim3(256), 0, stream_, mu_.as<int>(), zB0_.as<T>(), M, n, nslot_,
+                       nI_, CRP_);
+  });
+
+  // ---- P3: layer 2 forward
+  const int npf = nslot_ * nlm_;
+  P_.ensure(na * npf * CRP_ * sizeof(T));
+  B_.ensure(na * nB_ * C2P_ * sizeof(T));
+  T *P = P_.as<T>(), *B = B_.as<T>();
+  const int pthreads = round_up(nslot_ * CRP_, 64);
+#define GR_PAIR(K_, ...)                                                         \
+  if (nlm_ <= 9) hipLaunchKernelGGL((K_<T, 9>), __VA_ARGS__);                    \
+  else if (nlm_ <= 16) hipLaunchKernelGGL((K_<T, 16>), __VA_ARGS__);             \
+  else if (nlm_ <= 25) hipLaunchKernelGGL((K_<T, 25>), __VA_ARGS__);             \
+  else hipLaunchKernelGGL((K_<T, 49>), __VA_ARGS__)
+  stage("pair_fwd", [&] {
+    GR_PAIR(k_pair_fwd, dim3(n), dim3(nslot_ * CRP_), 0, stream_, eoff_.as<long long>(), ej_.as<int>(), Y_.as<T>(), R1_.as<T>(), (const T *) M, P,
+            nslot_, CRP_, nl_, radR1_.noutp);
+  });
+  stage("reduce_B", [&] { gemm(jB_, CRP_ / 16, C2P_ / 16, P, npf, B, nB_, 0); });
+  chain_forward(c2_, "_L2", B);
+  I2_.ensure(na * nrho_ * sizeof(double));
+  gI2_.ensure(na * nrho_ * sizeof(double));
+  stage("reduce_I2", [&] { reduce_fwd(redI2_, c2_.kb, c2_, B, I2_.as<double>()); });
+  stage("energy_mlp", [&] {
+    hipLaunchKernelGGL(k_energy_2l, dim3(n), dim3(64), 0, stream_, en_, mu_.as<int>(), n, rho_.as<double>(), I2_.as<double>(), grho_.as<double>(),
+                       gI2_.as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0);
+  });
+  if (!forces) return;
+
+  // ---- layer 2 reverse: dE/dB -> dE/dP -> bond forces of layer 2 and dE/dI of the neighbours
+  chain_zero(c2_, "_L2");
+  stage("reduce_I2_bwd", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>()); });
+  chain_backward(c2_, "_L2", B);
+  gP_.ensure(na * npf * CRP_ * sizeof(T));
+  gM_.ensure(na * nI_ * CRP_ * sizeof(T));
+  stage("reduce_B_bwd", [&] {
+    HIP_CHECK(hipMemsetAsync(gP_.p, 0, na * npf * CRP_ * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(gM_.p, 0, na * nI_ * CRP_ * sizeof(T), stream_));
+    gemm(jBb_, C2P_ / 16, CRP_ / 16, c2_.gX.template as<T>(), nB_, gP_.as<T>(), npf, 0);
+  });
+  stage("pair_bwd", [&] {
+    GR_PAIR(k_pair_bwd, dim3(n), dim3(pthreads), 0, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), dR1_.as<T>(),
+            (const T *) M, gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),
+            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp);
+  });
+#undef GR_PAIR
+
+  // ---- P5: layer 1 reverse
+  gI1_.ensure(na * nI1_ * PI1_ * sizeof(double));
+  chain_zero(c1_, "_L1");
+  stage("reduce_I_bwd", [&] {
+    HIP_CHECK(hipMemsetAsync(gI1_.p, 0, na * nI1_ * PI1_ * sizeof(double), stream_));
+    gemm(jIb_, CRP_ / 16, PI1_ / 16, gM_.as<T>(), nI_, gI1_.as<T>(), nI1_, 0);
+  });
+  stage("reduce_rho_bwd", [&] { reduce_bwd(redrho_, c1_, grho_.as<double>()); });
+  stage("reduce_I1_bwd", [&] {
+    for (auto &r : redI1_) reduce_bwd(*r, c1_, gI1_.as<double>());
+  });
+  chain_backward(c1_, "_L1", A);
+  {
+    BondBwdArgs<T> ba{};
+    ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
+    ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = c1_.gX.template as<T>();
+    ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1;
+    ba.a0 = 0; ba.C = C1P_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = radR_.noutp; ba.sh = sh_;
+    for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
+    stage("bond_bwd", [&] {
+      const size_t lds = ((size_t) nl_ * (C1P_ / 4) * 64 + (size_t) 4 * 16 * nlm_ * 4) * sizeof(T);
+      switch (C1P_ / 16) {
+        case 1: hipLaunchKernelGGL((k_bond_bwd<T, 1>), dim3(n), dim3(256), lds, stream_, ba); break;
+        case 2: hipLaunchKernelGGL((k_bond_bwd<T, 2>), dim3(n), dim3(256), lds, stream_, ba); break;
+        default: hipLaunchKernelGGL((k_bond_bwd<T, 4>), dim3(n), dim3(256), lds, stream_, ba); break;
+      }
+    });
+  }
+}
+
+}    // namespace
+
+std::unique_ptr<Engine> make_engine_2l(std::shared_ptr<const Model2L> model, int ntypes, const std::vector<int> &type2mu, int precision,
+                                       int device)
+{
+  if (precision == 64) return std::make_unique<Engine2L<double>>(std::move(model), ntypes, type2mu, device);
+  if (precision == 32) throw InvalidArgument("GRACE-2L engines compute in fp64 (precision 64)");
+  throw InvalidArgument("precision must be 64 or 32");
+}
+
+}    // namespace grhip

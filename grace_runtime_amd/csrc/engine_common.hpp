@@ -405,9 +405,157 @@ class EngineBase : public Engine {
     check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
   }
 
- protected:
-  EngineBase(int device, const char *who) : device_(device)
+  // copies a CSR structure to the device after the argument checks of the reference's CSR entry
+  // (python/src/core.cpp:292-396); atoms are grouped into tiles of 16 of one element for the tile GEMMs
+  void upload(const CsrInput &in) override
   {
+    HIP_CHECK(hipSetDevice(device_));
+    if (in.n < 0) throw InvalidArgument("negative atom count");
+    const bool table = in.x && in.image && in.shifts;
+    if ((in.rij != nullptr) == (in.x || in.image || in.shifts) || (!in.rij && !table))
+      throw InvalidArgument("give rij or positions, image and shifts");
+    const int n = in.n;
+    std::vector<int> mu(n);
+    for (int a = 0; a < n; a++) {
+      if (in.types[a] < 1 || in.types[a] > ntypes_) throw InvalidArgument("types must be 1 .. len(species)");
+      mu[a] = type2mu_[in.types[a]];
+      if (mu[a] < 0)
+        throw Error(who_ + ": atom " + std::to_string(a) + " of unmapped type " + std::to_string(in.types[a]) + " in the atom list");
+    }
+    if (in.offset[0] != 0) throw InvalidArgument("offset[0] must be 0 and offset[-1] == len(j)");
+    for (int a = 0; a < n; a++)
+      if (in.offset[a + 1] < in.offset[a]) throw InvalidArgument("offset must be non-decreasing");
+    const int64_t nb = in.offset[n];
+    for (int64_t q = 0; q < nb; q++) {
+      if (in.j[q] < 0 || in.j[q] >= n) throw InvalidArgument("j must index atoms 0 .. len(types)-1");
+      if (in.image && (in.image[q] < 0 || in.image[q] >= in.nimages)) throw InvalidArgument("image must index rows of shifts");
+    }
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    n_ = n;
+    nb_ = nb;
+    have_rij_ = in.rij != nullptr;
+    auto put = [&](DevBuf &b, const void *src, size_t bytes) {
+      b.ensure(std::max<size_t>(bytes, 8));
+      if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, hipMemcpyHostToDevice, stream_));
+    };
+    put(mu_, mu.data(), sizeof(int) * n);
+    std::vector<int> tiles;    // tiles of 16 atoms of one element, in atom order within an element
+    {
+      std::vector<int> ord(n);
+      std::iota(ord.begin(), ord.end(), 0);
+      std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return mu[a] < mu[b]; });
+      for (int q = 0; q < n;) {
+        int cnt = 0;
+        const int m0 = mu[ord[q]];
+        while (cnt < 16 && q < n && mu[ord[q]] == m0) { tiles.push_back(ord[q]); q++; cnt++; }
+        while (cnt < 16) { tiles.push_back(-1); cnt++; }
+      }
+    }
+    ntiles_ = (int) tiles.size() / 16;
+    put(tiles_, tiles.data(), sizeof(int) * tiles.size());
+    static_assert(sizeof(long long) == sizeof(int64_t), "offset type");
+    put(offset_, in.offset, sizeof(int64_t) * (n + 1));
+    put(j_, in.j, sizeof(int) * nb);
+    if (have_rij_) put(rij_, in.rij, sizeof(double) * 3 * nb);
+    else {
+      put(x_, in.x, sizeof(double) * 3 * n);
+      put(image_, in.image, sizeof(int) * nb);
+      put(shifts_, in.shifts, sizeof(double) * 3 * in.nimages);
+    }
+    HIP_CHECK(hipStreamSynchronize(stream_));    // the host copies (mu, tiles) go out of scope
+    ran_ = false;
+  }
+  void fetch(double *energy, double *forces, double *virial, double *eatom) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (!ran_) throw Error("fetch() before run()");
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    if (n_ > 0) {
+      int zb[2];
+      HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
+      if (zb[0] >= 0)    // bonds.h:49-62
+        throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " +
+                    std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
+    }
+    double s[8];
+    HIP_CHECK(hipMemcpy(s, scal_.p, sizeof(s), hipMemcpyDeviceToHost));
+    if (energy) *energy = s[0];
+    if (virial && ran_forces_)
+      for (int k = 0; k < 6; k++) virial[k] = s[1 + k];
+    if (forces && ran_forces_ && n_ > 0) HIP_CHECK(hipMemcpy(forces, f_.p, sizeof(double) * 3 * n_, hipMemcpyDeviceToHost));
+    if (eatom && ran_eatom_ && n_ > 0) HIP_CHECK(hipMemcpy(eatom, eatom_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
+  }
+  int64_t last_edge_count() override
+  {
+    synchronize();
+    long long e = 0;
+    if (n_ > 0) HIP_CHECK(hipMemcpy(&e, eoff_.as<long long>() + n_, sizeof(e), hipMemcpyDeviceToHost));
+    return e;
+  }
+  double cutoff(int t1, int t2) const override
+  {
+    if (t1 < 1 || t1 > ntypes_ || t2 < 1 || t2 > ntypes_) return 0.0;
+    const int a = type2mu_[t1], b = type2mu_[t2];
+    return (a < 0 || b < 0) ? 0.0 : cut_host_[(size_t) a * nelem_ + b];
+  }
+  double max_cutoff() const override
+  {
+    double m = 0.0;
+    for (int a = 1; a <= ntypes_; a++)
+      for (int b = 1; b <= ntypes_; b++) m = std::max(m, cutoff(a, b));
+    return m;
+  }
+
+ protected:
+  // pair cutoffs [nel][nel] of the model
+  void set_cutoffs(const std::vector<double> &cut)
+  {
+    cut_host_ = cut;
+    upload_vec(cut_, cut);
+  }
+  // start of a pass: clears the outputs, filters the bonds of the uploaded list (r^2 < rc^2, bonds.h:120-162 of the
+  // reference) into the compact edge arrays.  false: no atoms, nothing to do.
+  bool begin_pass(const RunFlags &fl)
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    ev_used_ = 0;
+    const int n = n_;
+    f_.ensure(std::max<size_t>((size_t) 3 * n, 1) * sizeof(double));
+    eatom_.ensure(std::max<size_t>(n, 1) * sizeof(double));
+    HIP_CHECK(hipMemsetAsync(f_.p, 0, (size_t) 3 * n * sizeof(double), stream_));
+    HIP_CHECK(hipMemsetAsync(scal_.p, 0, 8 * sizeof(double), stream_));
+    ran_ = true;
+    ran_forces_ = !fl.energy_only;
+    ran_eatom_ = fl.eatom;
+    if (n == 0) return false;
+    count_.ensure(sizeof(int) * n);
+    eoff_.ensure(sizeof(long long) * (n + 1));
+    {
+      const int init[2] = {-1, -1};
+      HIP_CHECK(hipMemcpyAsync(zero_.p, init, sizeof(init), hipMemcpyHostToDevice, stream_));
+    }
+    BondSrc src{};
+    src.mu = mu_.as<int>(); src.offset = offset_.as<long long>(); src.j = j_.as<int>();
+    src.rij = have_rij_ ? rij_.as<double>() : nullptr;
+    src.x = have_rij_ ? nullptr : x_.as<double>();
+    src.image = have_rij_ ? nullptr : image_.as<int>();
+    src.shifts = have_rij_ ? nullptr : shifts_.as<double>();
+    src.cut = cut_.as<double>(); src.nel = nelem_;
+    const size_t ecap = (size_t) std::max<int64_t>(nb_, 1);
+    ei_.ensure(ecap * sizeof(int)); ej_.ensure(ecap * sizeof(int)); emu_.ensure(ecap * sizeof(int));
+    rh_.ensure(ecap * 3 * sizeof(double)); r_.ensure(ecap * sizeof(double)); xr_.ensure(ecap * sizeof(double));
+    rc_.ensure(ecap * sizeof(double));
+    Edges ed{ei_.as<int>(), ej_.as<int>(), emu_.as<int>(), rh_.as<double>(), r_.as<double>(), xr_.as<double>(), rc_.as<double>()};
+    const int wpb = 4;
+    stage("edge_count", [&] { hipLaunchKernelGGL(k_edge_count, dim3((n + wpb - 1) / wpb), dim3(64 * wpb), 0, stream_, src, n, count_.as<int>(), zero_.as<int>()); });
+    stage("edge_scan", [&] { hipLaunchKernelGGL(k_scan, dim3(1), dim3(1024), 0, stream_, count_.as<int>(), n, eoff_.as<long long>()); });
+    stage("edge_fill", [&] { hipLaunchKernelGGL(k_edge_fill, dim3((n + wpb - 1) / wpb), dim3(64 * wpb), 0, stream_, src, n, eoff_.as<long long>(), ed); });
+    return true;
+  }
+  EngineBase(int device, const char *who, int ntypes, const std::vector<int> &type2mu, int n_elements) :
+      device_(device), who_(who), ntypes_(ntypes), type2mu_(type2mu), nelem_(n_elements)
+  {
+    check_type2mu(type2mu_, ntypes_, n_elements, who);
     check(hipSetDevice(device_), "hipSetDevice");
     hipDeviceProp_t prop;
     check(hipGetDeviceProperties(&prop, device_), "hipGetDeviceProperties");
@@ -416,6 +564,8 @@ class EngineBase : public Engine {
     ncu_ = prop.multiProcessorCount;
     arch_ = prop.gcnArchName;
     check(hipStreamCreate(&stream_), "hipStreamCreate");
+    scal_.ensure(8 * sizeof(double));
+    zero_.ensure(2 * sizeof(int));
   }
   ~EngineBase() override
   {
@@ -532,7 +682,20 @@ class EngineBase : public Engine {
   }
 
   int device_, ncu_ = 256;
-  std::string arch_;
+  std::string arch_, who_;
+  int ntypes_;
+  std::vector<int> type2mu_;
+  int nelem_;
+  std::vector<double> cut_host_;
+  // uploaded structure
+  int n_ = 0;
+  int64_t nb_ = 0;
+  bool have_rij_ = false;
+  DevBuf cut_, mu_, offset_, j_, rij_, x_, image_, shifts_, tiles_;
+  int ntiles_ = 0;
+  // edges of the pass and its outputs (scal: energy, virial[6])
+  DevBuf count_, eoff_, zero_, ei_, ej_, emu_, rh_, r_, xr_, rc_, f_, eatom_, scal_;
+  bool ran_ = false, ran_forces_ = false, ran_eatom_ = false;
   hipStream_t stream_ = nullptr;
   bool profile_ = false;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> events_;

@@ -99,7 +99,7 @@ __device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz
 }
 
 // plain copy of n doubles: the calibration kernel for the HBM counters (FETCH_SIZE / WRITE_SIZE per byte moved)
-__global__ void k_copy_calibration(const double *src, double *dst, long long n)
+static __global__ void k_copy_calibration(const double *src, double *dst, long long n)
 {
   for (long long i = blockIdx.x * (long long) blockDim.x + threadIdx.x; i < n; i += (long long) gridDim.x * blockDim.x) dst[i] = src[i];
 }
@@ -133,7 +133,7 @@ __device__ inline void bond_vec(const BondSrc &s, int i, long long q, double &dx
 }
 
 // one wave per atom: number of bonds with r^2 < rc^2; a bond of length 0 is recorded in zero_bond (i, j) and skipped
-__global__ void k_edge_count(BondSrc s, int n, int *count, int *zero_bond)
+static __global__ void k_edge_count(BondSrc s, int n, int *count, int *zero_bond)
 {
   const int lane = threadIdx.x & 63;
   const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -158,7 +158,7 @@ __global__ void k_edge_count(BondSrc s, int n, int *count, int *zero_bond)
 }
 
 // exclusive scan of count[n] into eoff[n + 1] (single block; n up to a few million is a few passes of 1024)
-__global__ void k_scan(const int *count, int n, long long *eoff)
+static __global__ void k_scan(const int *count, int n, long long *eoff)
 {
   __shared__ long long part[1024];
   __shared__ long long carry;
@@ -190,7 +190,7 @@ struct Edges {
 };
 
 // one wave per atom: in-cutoff bonds in list order -> compact edge arrays at eoff[i]
-__global__ void k_edge_fill(BondSrc s, int n, const long long *eoff, Edges e)
+static __global__ void k_edge_fill(BondSrc s, int n, const long long *eoff, Edges e)
 {
   const int lane = threadIdx.x & 63;
   const int i = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -790,7 +790,7 @@ struct EnergyDev {
 
 // E_i = (MLP(rho[1:]) + rho[0]) out_scale + shift[mu_i] and dE/drho, fp64, one wave per atom (fused_1l.cpp:378-427;
 // legacy RMS layer norm fused_cpu.h:666-682)
-__global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, const double *rho, double *grho, double *eatom_chunk,
+static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, const double *rho, double *grho, double *eatom_chunk,
                          double *energy, int want_grad)
 {
   __shared__ double act[8][256], pre[7][256], gbuf[2][256], x0[256];

@@ -108,8 +108,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
                            int noutp)
 {
   __shared__ double bsum[kPairChunk][4];
-  __shared__ double red[16][9];
-  const int i = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6, nwave = blockDim.x >> 6;
+  const int i = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const bool active = t < nslot * C;
   const int slot = active ? t / C : 0, n = t % C;
   const int nlm = nl * nl;
@@ -124,7 +123,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
   for (long long base = e0; base < e1; base += kPairChunk) {
     const int nb = (int) (e1 - base < kPairChunk ? e1 - base : kPairChunk);
     __syncthreads();
-    if (t < kPairChunk * 4) bsum[t >> 2][t & 3] = 0.0;
+    for (int q = t; q < kPairChunk * 4; q += blockDim.x) bsum[q >> 2][q & 3] = 0.0;
     __syncthreads();
     for (int b = 0; b < nb; b++) {
       const long long e = base + b;
@@ -183,7 +182,6 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
       for (int k = 0; k < 6; k++) atomicAdd(&virial[k], vsum[3 + k]);
     }
   }
-  (void) red; (void) nwave;
 }
 
 struct Energy2Dev {
@@ -199,7 +197,7 @@ struct Energy2Dev {
 
 // E_i = (MLP(x) + rho[0] + I2[0] ln0[0] / s0) out_scale + shift,  x_k = rho[k] lnI[k-1] / s1 + I2[k] ln0[k] / s0,
 // s1 = sqrt(mean rho[1:]^2 + eps), s0 = sqrt(mean I2^2 + eps); dE/drho, dE/dI2.  One wave per atom, fp64.
-__global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, const double *rho, const double *I2, double *grho, double *gI2,
+static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, const double *rho, const double *I2, double *grho, double *gI2,
                             double *eatom, double *energy, int want_grad)
 {
   __shared__ double act[8][256], pre[7][256], gbuf[2][256], x0[256];
