@@ -35,7 +35,24 @@ def model_cut2():
     return d
 
 
-MODELS = {"config1": model_config1, "mix2": model_mix2, "cut2": model_cut2}
+def model_config3():
+    """GRACE-2L-shaped benchmark model: two layers, lmax 4, 32 channels everywhere, radial MLPs 8-64-64-160, body
+    order 3 per layer, 4 species"""
+    return synth.random_model_2l(seed=20260103)
+
+
+def model_l2mix():
+    """GRACE-2L, two elements with pair-specific cutoffs, lmax 2, different (unpadded) widths in every stage"""
+    d = synth.random_model_2l(lmax=2, n_elements=2, element_names=("Mo", "W"), embedding_size=8, nradbase=10, c1=20, cr=12,
+                              c2=24, i1_width=10, hidden=32, rho_n_out=9, energy_hidden=16, rcut=5.0,
+                              inv_avg_n_neigh=1.0 / 26.0, seed=13)
+    d["has_bond_specific_cutoff"] = np.array([1], dtype=np.int64)
+    d["bond_cutoff_map"] = np.array([[5.0, 4.5], [4.5, 4.25]])
+    return d
+
+
+MODELS = {"config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
+LAYERS = {"config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
 
 
 def write_model(name, directory):
@@ -85,12 +102,31 @@ def structure_molecule(seed=8):
     return pos, np.zeros((3, 3)), np.array([False, False, False]), types
 
 
-STRUCTURES = {"config1": structure_config1, "alloy54": structure_alloy54, "triclinic": structure_triclinic,
+def structure_fcc108(seed=3):
+    """3 x 3 x 3 cells of the fcc alloy of the two-layer benchmark (4 species; the box is shorter than two cutoffs)"""
+    pos, cell = synth.fcc_supercell(3.6, 3)
+    rng = np.random.default_rng(seed)
+    types = rng.integers(1, 5, size=len(pos)).astype(np.int32)
+    return synth.jitter(pos, 0.08, seed), cell, np.array([True, True, True]), types
+
+
+def structure_config3():
+    pos, cell = synth.fcc_supercell(3.6, 20)
+    rng = np.random.default_rng(3)
+    types = rng.integers(1, 5, size=len(pos)).astype(np.int32)
+    return synth.jitter(pos, 0.08, 3), cell, np.array([True, True, True]), types
+
+
+STRUCTURES = {"fcc108": structure_fcc108, "config1": structure_config1, "alloy54": structure_alloy54, "triclinic": structure_triclinic,
               "slab": structure_slab, "molecule": structure_molecule}
 
 # (model, structure, list cutoff or None for the model cutoff): the end-to-end golden cases
 E2E_CASES = [("config1", "config1", None), ("mix2", "alloy54", 5.5), ("mix2", "triclinic", None),
              ("cut2", "alloy54", None), ("cut2", "slab", 6.0), ("mix2", "molecule", None)]
+E2E_CASES_2L = [("config3", "fcc108", None), ("l2mix", "alloy54", 5.5), ("l2mix", "triclinic", None), ("l2mix", "slab", None),
+                ("l2mix", "molecule", None)]
+# reference fixture models (tests/golden/ref_fixtures) on the reference's fixture cells: goldens of the compiled reference
+FIXTURE_CASES_2L = [(m, c) for m in ("grace_2l_small", "grace_2l_l3", "legacy_2l_small", "legacy_2l_wide") for c in ("W54", "WMo54")]
 
 
 def bond_vectors(pos, perm, offset, j, image, shifts):

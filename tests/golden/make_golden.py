@@ -3,7 +3,8 @@ oracle/Makefile from the reference checkout) on the synthetic cases of tests/cas
 
 * its neighbour list (perm, offset, j, image, shifts) per structure            -> pins the host / device list
 * its energy, per-atom energies, forces, virial per (model, structure) case    -> pins the oracle and the HIP path
-  on models the reference's own TF goldens do not cover (AAAA stage, A width != FC width, pair cutoffs, lmax 3/4)
+  on models the reference's own TF goldens do not cover (AAAA stage, A width != FC width, pair cutoffs, lmax 3/4,
+  GRACE-2L at lmax 4 and with unequal stage widths, the reference's 2L fixture models with the BBBB stage)
 
 Run in the build container (needs oracle/_ref):  python tests/golden/make_golden.py
 """
@@ -26,7 +27,7 @@ def main():
     out = {}
     tmp = tempfile.mkdtemp()
     lists = {}
-    for model, struct, rc_list in cases.E2E_CASES:
+    for model, struct, rc_list in cases.E2E_CASES + cases.E2E_CASES_2L:
         path = cases.write_model(model, tmp)
         d = cases.MODELS[model]()
         nel = int(d["n_elements"][0])
@@ -48,6 +49,17 @@ def main():
         for k in ("energy", "energies", "forces", "virial"):
             out[f"{tag}/{k}"] = np.asarray(r[k])
         print(tag, key, "bonds", len(nl["j"]), "E", r["energy"], "max|F|", np.abs(r["forces"]).max())
+    # the reference's own 2L fixture models without TF goldens, on its fixture cells (CSR bonds as stored there)
+    for model, cell in cases.FIXTURE_CASES_2L:
+        with np.load(os.path.join(cases.REF_FIXTURES, cell + ".npz")) as c:
+            types = np.array([2 if z == 74 else 1 for z in c["numbers"]], dtype=np.int32)
+            offset, j, rij = c["offset"], c["j"], c["rij"]
+        ref = ref_lib.RefModel(os.path.join(cases.REF_FIXTURES, model + ".npz"), [0, 1])    # species (Mo, W)
+        r = ref.compute(types, offset, j, rij=rij, nthreads=2)
+        tag = f"fixture/{model}/{cell}"
+        for k in ("energy", "energies", "forces", "virial"):
+            out[f"{tag}/{k}"] = np.asarray(r[k])
+        print(tag, "E", r["energy"], "max|F|", np.abs(r["forces"]).max())
     np.savez(os.path.join(cases.GOLDEN, "reference_outputs.npz"), **out)
 
 

@@ -46,9 +46,51 @@ def test_loads_reference_fixture_models(name, lmax, C_, order):
     assert list(m.type2mu(["W", "Mo"])) == [-1, 1, 0]
 
 
+@pytest.mark.parametrize("name,lmax,C_,order", [("grace_2l_order3", 2, 16, 3), ("legacy_2l_order3", 2, 16, 3), ("grace_2l_small", 2, 16, 4),
+                                                ("grace_2l_l3", 3, 20, 3), ("legacy_2l_wide", 1, 40, 4)])
+def test_loads_reference_2l_fixture_models(name, lmax, C_, order):
+    m = kk.Model(os.path.join(cases.REF_FIXTURES, name + ".npz"))
+    assert (m.layers, m.lmax, m.n_radial, m.max_order, m.element_names) == (2, lmax, C_, order, ["Mo", "W"])
+    assert m.rcut == 5.0
+
+
+def _mutated_2l(tmp_path, fn):
+    d = cases.model_l2mix()
+    fn(d)
+    p = str(tmp_path / "m2.npz")
+    np.savez(p, **{k: v for k, v in d.items() if not k.startswith("_")})
+    return p
+
+
+BAD_2L = [
+    (lambda d: d.pop("B0_lin_transform_W"), "required weight 'B0_lin_transform_W' missing"),
+    (lambda d: d.update(YI_lr_inds=d["YI_lr_inds"] + 7), "YI_lr_inds' has (7, 7) at 0"),
+    (lambda d: d.update(I_n_out=np.array([11])), "I_n_out"),
+    (lambda d: d.update(B_total_sum_ind_YI=d["B_total_sum_ind_YI"] + 100), "B_total_sum_ind_YI' has"),
+    (lambda d: d.update(I1_is_central_atom_type_dependent=np.array([0])), "I1_is_central_atom_type_dependent"),
+    (lambda d: d.update(I_0_LN_scale=d["I_0_LN_scale"][:-1]), "I_0_LN_scale' has 8 values, expected 9"),
+    (lambda d: d.update(I2_n_out=np.array([7])), "I2_n_out"),
+    (lambda d: d.update(prod_BBBB_n_cg_terms=np.array([1])), "prod_AAAA_n_cg_terms"),
+    (lambda d: d.update(fc_BB1_w_left=d["fc_BB1_w_left"][:, :-1]), "fc_BB1_w_left' has shape"),
+    (lambda d: d.update(mlp_rad_R1_has_chem_emb=np.array([1])), "mlp_rad_R1_has_chem_emb"),
+    (lambda d: d.update(I2_reduce_BB_W=d["I2_reduce_BB_W"][:1]), "I2_reduce_BB_W' has shape"),
+]
+
+
+@pytest.mark.parametrize("k", range(len(BAD_2L)))
+def test_malformed_2l_models_are_rejected(tmp_path, k):
+    fn, msg = BAD_2L[k]
+    with pytest.raises((RuntimeError, ValueError), match=re.escape(msg)):
+        kk.Model(_mutated_2l(tmp_path, fn))
+
+
 def test_rejects_other_model_kinds_and_missing_files(tmp_path):
-    with pytest.raises(ValueError, match="GRACE-2L"):
-        kk.Model(os.path.join(cases.REF_FIXTURES, "grace_2l_order3.npz"))
+    d = cases.model_cut2()
+    d["grace_model_kind"] = np.array([b"GRACE-3L"], dtype="|S8")
+    p3 = str(tmp_path / "m3.npz")
+    np.savez(p3, **d)
+    with pytest.raises(ValueError, match="GRACE-3L"):
+        kk.Model(p3)
     with pytest.raises(RuntimeError, match="cannot read the model file"):
         kk.Model(str(tmp_path / "nope.npz"))
     p = tmp_path / "junk.npz"
