@@ -56,7 +56,7 @@ template<class T> class Engine2L final : public EngineBase {
   DevJobs<T> jI_, jIb_, jB_, jBb_;
   Energy2Dev en_{};
   // pass buffers
-  DevBuf Rz_, dRz_, R1_, dR1_, Y_, YG_, A_, rho_, grho_, I1_, gI1_, M_, gM_, P_, gP_, B_, I2_, gI2_;
+  DevBuf sink_, Rz_, dRz_, R1_, dR1_, YG_, A_, rho_, grho_, I1_, gI1_, M_, gM_, P_, gP_, B_, I2_, gI2_;
 
   void build();
   void build_chain(Chain<T> &c, const char *tag, int nf, int KP, const FCWeights *fc[3], const CGProduct *pr[3],
@@ -172,6 +172,7 @@ template<class T> void Engine2L<T>::build()
     upload_vec(ones_, std::vector<T>((size_t) nel_ * CRP_, (T) 1));
     upload_vec(shift_, m.shift_values);
   }
+  sink_.ensure(64);
   radR_.build(m.mlp_R, m.nradbase, m.radial_basis_p, m.radial_activation, m.C1, C1P_, nl_, nel_, drow_, "GRACE-2L");
   radR1_.build(m.mlp_R1, m.nradbase, m.radial_basis_p, m.radial_activation, m.CR, CRP_, nl_, nel_, drow_, "GRACE-2L");
 
@@ -448,11 +449,14 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   dR1_.ensure(ecap * radR1_.noutp * sizeof(T));
   stage("radial_R", [&] { radR_.launch(stream_, ncu_, zA_.as<T>(), 0, -1, xr_.as<double>(), emu_.as<int>(), Rz_.as<T>(), dRz_.as<T>(), n_edges); });
   stage("radial_R1", [&] { radR1_.launch(stream_, ncu_, ones_.as<T>(), 0, -1, xr_.as<double>(), emu_.as<int>(), R1_.as<T>(), dR1_.as<T>(), n_edges); });
-  Y_.ensure(ecap * nlm_ * sizeof(T));
-  if (forces) YG_.ensure(ecap * nlm_ * 4 * sizeof(T));
+  const int yw = forces ? 4 * nlm_ : nlm_;    // row of an edge: Y[nlm] and, for forces, G[nlm][3]
+  YG_.ensure(ecap * yw * sizeof(T));
   stage("sh_edges", [&] {
-    hipLaunchKernelGGL(k_sh_edges<T>, dim3((unsigned) ((ecap + 127) / 128)), dim3(128), 0, stream_, sh_, rh_.as<double>(), n_edges, nlm_,
-                       Y_.as<T>(), forces ? YG_.as<T>() : (T *) nullptr);
+    const size_t lds = (size_t) 64 * (yw + 1) * sizeof(T);
+    auto kern = k_sh_edges<T>;
+    if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+    hipLaunchKernelGGL(kern, dim3((unsigned) ((ecap + 63) / 64)), dim3(64), lds, stream_, sh_, rh_.as<double>(), n_edges, nlm_, forces ? 1 : 0,
+                       YG_.as<T>());
   });
 
   // ---- P1: layer 1 forward
@@ -493,14 +497,27 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   B_.ensure(na * nB_ * C2P_ * sizeof(T));
   T *P = P_.as<T>(), *B = B_.as<T>();
   const int pthreads = round_up(nslot_ * CRP_, 64);
-#define GR_PAIR(K_, ...)                                                         \
-  if (nlm_ <= 9) hipLaunchKernelGGL((K_<T, 9>), __VA_ARGS__);                    \
-  else if (nlm_ <= 16) hipLaunchKernelGGL((K_<T, 16>), __VA_ARGS__);             \
-  else if (nlm_ <= 25) hipLaunchKernelGGL((K_<T, 25>), __VA_ARGS__);             \
-  else hipLaunchKernelGGL((K_<T, 49>), __VA_ARGS__)
+#define GR_PAIR1(K_, N_, grid_, block_, lds_, ...)                                                                       \
+  {                                                                                                                      \
+    auto kern = K_<T, N_>;                                                                                               \
+    if (lds_ > 48 * 1024)                                                                                                \
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_)); \
+    hipLaunchKernelGGL(kern, grid_, block_, lds_, __VA_ARGS__);                                                          \
+  }
+#define GR_PAIR(K_, ...)                                     \
+  switch (nl_) {                                             \
+    case 1: GR_PAIR1(K_, 1, __VA_ARGS__) break;              \
+    case 2: GR_PAIR1(K_, 4, __VA_ARGS__) break;              \
+    case 3: GR_PAIR1(K_, 9, __VA_ARGS__) break;              \
+    case 4: GR_PAIR1(K_, 16, __VA_ARGS__) break;             \
+    case 5: GR_PAIR1(K_, 25, __VA_ARGS__) break;             \
+    case 6: GR_PAIR1(K_, 36, __VA_ARGS__) break;             \
+    default: GR_PAIR1(K_, 49, __VA_ARGS__) break;            \
+  }
   stage("pair_fwd", [&] {
-    GR_PAIR(k_pair_fwd, dim3(n), dim3(nslot_ * CRP_), 0, stream_, eoff_.as<long long>(), ej_.as<int>(), Y_.as<T>(), R1_.as<T>(), (const T *) M, P,
-            nslot_, CRP_, nl_, radR1_.noutp);
+    const size_t lds = (size_t) kPairChunk * (nslot_ * CRP_ + radR1_.noutp) * sizeof(T);
+    GR_PAIR(k_pair_fwd, dim3(n), dim3(nslot_ * CRP_), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), (const T *) M, P,
+            nslot_, CRP_, nl_, radR1_.noutp, yw, sink_.as<T>());
   });
   stage("reduce_B", [&] { gemm(jB_, CRP_ / 16, C2P_ / 16, P, npf, B, nB_, 0); });
   chain_forward(c2_, "_L2", B);
@@ -525,11 +542,13 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     gemm(jBb_, C2P_ / 16, CRP_ / 16, c2_.gX.template as<T>(), nB_, gP_.as<T>(), npf, 0);
   });
   stage("pair_bwd", [&] {
-    GR_PAIR(k_pair_bwd, dim3(n), dim3(pthreads), 0, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), dR1_.as<T>(),
+    const size_t lds = (size_t) kPairChunk * (pthreads + 2 * radR1_.noutp) * sizeof(T);
+    GR_PAIR(k_pair_bwd, dim3(n), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), dR1_.as<T>(),
             (const T *) M, gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),
-            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp);
+            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1);
   });
 #undef GR_PAIR
+#undef GR_PAIR1
 
   // ---- P5: layer 1 reverse
   gI1_.ensure(na * nI1_ * PI1_ * sizeof(double));
