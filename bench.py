@@ -1,12 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the GRACE energy + forces + virial pass on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--precision 64|32] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--precision 64|32] [--no-cpu] [--workload config2|config3]
 
-Workload (BASELINE.json configs[1]): GRACE-1L-shaped random-init model (lmax 4, 32 radial channels, 8 Chebyshev
+Default workload (BASELINE.json configs[1], the one the metric is quoted on): GRACE-1L-shaped random-init model (lmax 4, 32 radial channels, 8 Chebyshev
 functions, radial MLP 8-64-64-160, SiLU) on a bcc W 16x16x16 supercell (8192 atoms, a = 3.165 A, N(0, 0.05 A) jitter,
 r_cut 6 A, 475 136 directed edges), fp64.  A step is one full pass (bond filter, radial MLP, A basis, dense chain,
 readout, reverse pass, forces, virial) over the structure, which is uploaded to HBM before the timed region.
+
+--workload config3 runs BASELINE.json configs[2] instead: GRACE-2L-shaped model (two layers, lmax 4, 32 channels, two radial
+MLPs 8-64-64-160, body order 3) on the 4-species fcc 20x20x20 alloy (32 000 atoms, ~2.5 M edges), fp64.
 
 Prints one JSON line: the metric (us/atom per call), the roofline of the dominant kernel (duration from HIP events
 on the engine's stream, algorithmic flops/bytes of that stage) and the reference CPU path timed on this host.
@@ -28,9 +31,22 @@ PEAK = {64: 78.6, 32: 157.3}      # dense matrix TFLOP/s of MI355X (fp64, fp32)
 HBM_PEAK = 8000.0                 # GB/s
 
 
-def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops):
+# HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs of this
+# script, counters scaled by what they read for the 1 GiB copy kernel; summaries under profiles/): (workload, kernel)
+MEASURED_TRAFFIC = {}
+
+
+def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4):
     """Roofline entry of one stage: algorithmic work / measured time."""
-    if name == "radial_mlp":
+    if name == "pair_fwd":
+        # per edge: R1 row, Y, neighbour index, the neighbour's message rows; per atom: the pair tensor written once
+        by = E * (s * C * nl + s * nlm + 4 + nslot * C * s) + N * nslot * nlm * C * s
+        return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
+    if name == "pair_bwd":
+        # per edge: R1 and dR1 rows, Y and its gradient, neighbour rows, dE/dI rows read-modify-written, geometry, forces
+        by = E * (2 * s * C * nl + 4 * s * nlm + nslot * C * s + 2 * nI * C * s + 28 + 24) + N * (nslot * nlm * C * s + 24)
+        return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
+    if name in ("radial_mlp", "radial_R", "radial_R1"):
         # value + tangent through the 3 layers: 2 * 2 * E * sum n_in n_out
         fl = 59392.0 * E
         return {"bound": "mfma", "achieved": fl / (ms * 1e-3) / 1e12, "peak": PEAK[prec], "unit": "TFLOP/s", "work": fl}
@@ -53,7 +69,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--precision", type=int, default=64, choices=[64, 32])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--reps", type=int, default=16, help="bcc supercell repetitions (16 = the benchmark config)")
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3"])
+    ap.add_argument("--reps", type=int, default=0, help="supercell repetitions (default: 16 bcc cells / 20 fcc cells per edge)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives in the path); run with --gpus 1")
@@ -65,15 +82,27 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     tmp = tempfile.mkdtemp()
-    mpath = cases.write_model("config1", tmp)
-    pos, cell = synth.bcc_supercell(3.165, a.reps)
-    pos = synth.jitter(pos, 0.05, 2)
+    two = a.workload == "config3"
+    if two and a.precision != 64:
+        sys.exit("bench.py: the GRACE-2L engine computes in fp64")
+    reps = a.reps or (20 if two else 16)
     pbc = [True, True, True]
+    if two:
+        mpath = cases.write_model("config3", tmp)
+        species = ["Al", "Co", "Ni", "Ti"]
+        pos, cell = synth.fcc_supercell(3.6, reps)
+        pos = synth.jitter(pos, 0.08, 3)
+        types = np.random.default_rng(3).integers(1, 5, size=len(pos)).astype(np.int32)
+    else:
+        mpath = cases.write_model("config1", tmp)
+        species = ["W"]
+        pos, cell = synth.bcc_supercell(3.165, reps)
+        pos = synth.jitter(pos, 0.05, 2)
+        types = np.ones(len(pos), np.int32)
     N = len(pos)
-    types = np.ones(N, np.int32)
-    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 6.0)
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 6.0, num_threads=len(os.sched_getaffinity(0)))
     model = kk.Model(mpath)
-    eng = kk.Engine(model, ["W"], precision=a.precision)
+    eng = kk.Engine(model, species, precision=a.precision)
     eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
     eng.debug_copy(1 << 30)     # k_copy_calibration over 1 GiB: scales the rocprof FETCH_SIZE / WRITE_SIZE counters
 
@@ -116,15 +145,16 @@ def main():
     dom = max(modelled, key=lambda k: modelled[k]["ms"])
     d = modelled[dom]
     roofline = {"kernel": dom, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"],
-                "unit": d["unit"], "frac": round(d["frac"], 4), "traffic": None, "avg_ms": round(d["ms"], 4),
-                "algorithmic_work": d["work"]}
+                "unit": d["unit"], "frac": round(d["frac"], 4),
+                "traffic": MEASURED_TRAFFIC.get((a.workload, dom)) if reps == (20 if two else 16) and a.precision == 64 else None,
+                "avg_ms": round(d["ms"], 4), "algorithmic_work": d["work"]}
 
     cpu = None
     if not a.no_cpu:
         from oracle import ref_lib      # the compiled reference CPU path: the checker, timed here as the baseline
         if ref_lib.available():
             nth = len(os.sched_getaffinity(0))
-            ref = ref_lib.RefModel(mpath, [0])
+            ref = ref_lib.RefModel(mpath, list(range(len(species))))
             args = dict(positions=pos[perm], image=image, shifts=shifts, nthreads=nth)
             ref.compute(types[perm], offset, j, **args)
             ts = []
@@ -135,7 +165,7 @@ def main():
                 ts.append(time.perf_counter() - t1)
             tm = float(np.median(ts))
             cpu = {"value": round(tm / N * 1e6, 4), "unit": "us/atom", "cores": nth, "kind": "reference",
-                   "sample": f"{len(ts)} full calls of the compiled reference Grace1LFused (fp32 + spline tables) on the same "
+                   "sample": f"{len(ts)} full calls of the compiled reference Grace{2 if two else 1}LFused (fp32 + spline tables) on the same "
                              f"{N}-atom structure, median",
                    "dE_per_atom_vs_gpu": abs(r["energy"] - out["energy"]) / N,
                    "max_dF_vs_gpu": float(np.abs(r["forces"] - out["forces"]).max())}
@@ -144,8 +174,10 @@ def main():
         "metric": "us_per_atom_EFS_call", "value": round(dt / N * 1e6, 5), "unit": "us/atom", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "f64" if a.precision == 64 else "f32", "data": "synthetic",
-        "config": {"workload": f"GRACE-1L-shaped random-init model (lmax 4, 32 ch, MLP 8-64-64-160) on bcc W "
-                               f"{a.reps}x{a.reps}x{a.reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[1])",
+        "config": {"workload": (f"GRACE-2L-shaped random-init model (2 layers, lmax 4, 32 ch, MLPs 8-64-64-160, body order 3) on the "
+                                f"4-species fcc alloy {reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[2])") if two else
+                               (f"GRACE-1L-shaped random-init model (lmax 4, 32 ch, MLP 8-64-64-160) on bcc W "
+                                f"{reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[1])"),
                    "atoms": N, "edges": int(E)},
         "atoms_steps_per_s": round(N / dt, 1),
         "roofline": roofline,
