@@ -22,7 +22,7 @@ SYMBOLS = [
     "gr_compute_csr", "gr_engine_upload", "gr_engine_run", "gr_engine_sync", "gr_engine_fetch",
     "gr_engine_edge_count", "gr_engine_set_profile", "gr_engine_stage_count", "gr_engine_stage_get",
     "gr_engine_debug_radial", "gr_engine_debug_copy", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
-    "gr_nlist_free", "gr_compute",
+    "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
 ]
 
 
@@ -77,6 +77,9 @@ def lib():
     L.gr_nlist_get.argtypes = [vp, vp, vp, vp, vp, vp]
     L.gr_nlist_free.argtypes = [vp]
     L.gr_compute.argtypes = [vp, i32, vp, vp, vp, vp, u32, vp, vp, vp, vp]
+    L.gr_compute_batch.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, i32, vp, vp, vp, vp]
+    L.gr_engine_upload_batch.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i32, vp]
+    L.gr_engine_fetch_batch.argtypes = [vp, i32, vp, vp, vp, vp]
     _lib = L
     return L
 

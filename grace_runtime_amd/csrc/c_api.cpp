@@ -7,6 +7,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <array>
+#include <cmath>
 #include <cstring>
 #include <memory>
 #include <new>
@@ -352,6 +354,181 @@ int gr_compute(gr_engine *e, int n, const int *types, const double *positions, c
         for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) q + d];
       if (fl.eatom) eatom[a] = ea[q];
     }
+  });
+}
+
+int gr_engine_upload_batch(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
+                           const double *positions, const int *image, const double *shifts, int64_t nimages, int nstruct,
+                           const int *struct_of_atom)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    if (n > 0 && !struct_of_atom) throw grhip::InvalidArgument("struct_of_atom is required");
+    grhip::CsrInput in = make_input(n, types, offset, j, rij, positions, image, shifts, nimages);
+    in.nstruct = nstruct;
+    in.sid = struct_of_atom;
+    e->eng->upload(in);
+  });
+}
+
+int gr_engine_fetch_batch(gr_engine *e, int nstruct, double *energy, double *forces, double *virial, double *eatom)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->fetch_batch(nstruct, energy, forces, virial, eatom);
+  });
+}
+
+namespace {
+// Cell of a structure for the cell list: zero vectors and the vectors of open directions are replaced by unit
+// directions normal to the periodic ones, long enough that no image is within reach; `shift` puts the atoms inside
+// (python/grace_runtime/neighbors.py:27-47 of the reference).
+void padded_cell(const double *cell, const unsigned char *pbc, const double *pos, int64_t n, double reach, double *out, double *shift)
+{
+  bool pad[3];
+  std::vector<std::array<double, 3>> given;
+  for (int k = 0; k < 3; k++) {
+    const double *v = cell + 3 * k;
+    pad[k] = !pbc[k] || (v[0] == 0.0 && v[1] == 0.0 && v[2] == 0.0);
+    for (int d = 0; d < 3; d++) out[3 * k + d] = v[d];
+    if (!pad[k]) given.push_back({v[0], v[1], v[2]});
+  }
+  shift[0] = shift[1] = shift[2] = 0.0;
+  if (given.size() == 3) return;
+  auto norm = [](std::array<double, 3> &a) {
+    const double l = std::sqrt(a[0] * a[0] + a[1] * a[1] + a[2] * a[2]);
+    if (!(l > 0.0)) throw grhip::InvalidArgument("the periodic cell vectors are linearly dependent");
+    for (double &c : a) c /= l;
+  };
+  auto cross = [](const std::array<double, 3> &a, const std::array<double, 3> &b) {
+    return std::array<double, 3>{a[1] * b[2] - a[2] * b[1], a[2] * b[0] - a[0] * b[2], a[0] * b[1] - a[1] * b[0]};
+  };
+  std::vector<std::array<double, 3>> dirs;
+  if (given.empty()) dirs = {{1, 0, 0}, {0, 1, 0}, {0, 0, 1}};
+  else if (given.size() == 2) {
+    auto c = cross(given[0], given[1]);
+    norm(c);
+    dirs = {c};
+  } else {
+    std::array<double, 3> a = given[0];
+    norm(a);
+    int kmin = 0;
+    for (int d = 1; d < 3; d++)
+      if (std::fabs(a[d]) < std::fabs(a[kmin])) kmin = d;
+    std::array<double, 3> ek{0, 0, 0};
+    ek[kmin] = 1.0;
+    auto b = cross(a, ek);
+    norm(b);
+    auto c = cross(a, b);
+    norm(c);
+    dirs = {b, c};
+  }
+  size_t q = 0;
+  for (int k = 0; k < 3; k++) {
+    if (!pad[k]) continue;
+    const auto &d = dirs[q++];
+    double lo = 0.0, hi = 0.0;
+    for (int64_t a = 0; a < n; a++) {
+      const double pr = pos[3 * a] * d[0] + pos[3 * a + 1] * d[1] + pos[3 * a + 2] * d[2];
+      if (a == 0 || pr < lo) lo = pr;
+      if (a == 0 || pr > hi) hi = pr;
+    }
+    const double len = (hi - lo) + 2.0 * reach + 1.0;
+    for (int c = 0; c < 3; c++) {
+      out[3 * k + c] = d[c] * len;
+      if (n > 0) shift[c] += d[c] * (reach + 0.5 - lo);
+    }
+  }
+}
+}    // namespace
+
+int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
+                     const unsigned char *pbc, unsigned flags, int nthreads, double *energy, double *forces, double *virial,
+                     double *eatom)
+{
+  return guarded([&] {
+    if (!e || nstruct < 0 || (nstruct > 0 && (!natoms || !cells || !pbc))) throw grhip::InvalidArgument("null argument");
+    if (nstruct == 0) return;
+    const double rc = e->eng->max_cutoff();
+    if (!(rc > 0.0)) throw grhip::Error("the engine has no positive cutoff");
+    std::vector<int64_t> start(nstruct + 1, 0);
+    for (int s = 0; s < nstruct; s++) {
+      if (natoms[s] < 0) throw grhip::InvalidArgument("negative atom count");
+      start[s + 1] = start[s] + natoms[s];
+    }
+    const int64_t N = start[nstruct];
+    if (N >= INT32_MAX) throw grhip::InvalidArgument("atom count out of range");
+    if (N > 0 && (!types || !positions)) throw grhip::InvalidArgument("null argument");
+    // one cell list per structure (they are independent: in parallel), then one list of all atoms
+    std::vector<grhip::NeighborList> nls(nstruct);
+    std::string err;
+    bool invalid = false;
+#pragma omp parallel for schedule(dynamic, 4) num_threads(nthreads > 0 ? nthreads : 1)
+    for (int s = 0; s < nstruct; s++) {
+      try {
+        const int64_t n = natoms[s];
+        const double *x = positions + 3 * start[s];
+        double pc[9], sh[3];
+        padded_cell(cells + 9 * (size_t) s, pbc + 3 * (size_t) s, x, n, rc, pc, sh);
+        std::vector<double> xs((size_t) 3 * n);
+        for (int64_t a = 0; a < n; a++)
+          for (int d = 0; d < 3; d++) xs[3 * a + d] = x[3 * a + d] + sh[d];
+        const bool p[3] = {pbc[3 * s] != 0, pbc[3 * s + 1] != 0, pbc[3 * s + 2] != 0};
+        nls[s] = grhip::neighbor_search(xs.data(), n, pc, p, rc, 1);
+      } catch (const grhip::InvalidArgument &ex) {
+#pragma omp critical
+        { err = ex.what(); invalid = true; }
+      } catch (const std::exception &ex) {
+#pragma omp critical
+        { if (err.empty()) err = ex.what(); }
+      }
+    }
+    if (!err.empty()) {
+      if (invalid) throw grhip::InvalidArgument(err);
+      throw grhip::Error(err);
+    }
+    std::vector<int64_t> offset(N + 1, 0), boff(nstruct + 1, 0), ioff(nstruct + 1, 0);
+    for (int s = 0; s < nstruct; s++) {
+      boff[s + 1] = boff[s] + (int64_t) nls[s].j.size();
+      ioff[s + 1] = ioff[s] + (int64_t) nls[s].shifts.size() / 3;
+    }
+    const int64_t nb = boff[nstruct], nimg = ioff[nstruct];
+    std::vector<int> ty(N), sid(N), jj(nb), img(nb);
+    std::vector<double> x((size_t) 3 * N), shifts((size_t) 3 * std::max<int64_t>(nimg, 1), 0.0);
+#pragma omp parallel for schedule(dynamic, 4) num_threads(nthreads > 0 ? nthreads : 1)
+    for (int s = 0; s < nstruct; s++) {
+      const grhip::NeighborList &nl = nls[s];
+      const int64_t n = natoms[s], a0 = start[s];
+      for (int64_t q = 0; q < n; q++) {
+        const int64_t a = a0 + nl.perm[q];
+        ty[a0 + q] = types[a];
+        sid[a0 + q] = s;
+        for (int d = 0; d < 3; d++) x[3 * (a0 + q) + d] = positions[3 * a + d];
+        offset[a0 + q + 1] = boff[s] + nl.offset[q + 1];
+      }
+      for (size_t b = 0; b < nl.j.size(); b++) {
+        jj[boff[s] + b] = (int) (a0 + nl.j[b]);
+        img[boff[s] + b] = (int) (ioff[s] + nl.image[b]);
+      }
+      std::copy(nl.shifts.begin(), nl.shifts.end(), shifts.begin() + 3 * ioff[s]);
+    }
+    grhip::CsrInput in = make_input((int) N, ty.data(), offset.data(), jj.data(), nullptr, x.data(), img.data(), shifts.data(), nimg);
+    in.nstruct = nstruct;
+    in.sid = sid.data();
+    e->eng->upload(in);
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    e->eng->run(fl);
+    std::vector<double> f((size_t) 3 * N), ea(fl.eatom ? N : 0);
+    e->eng->fetch_batch(nstruct, energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
+    for (int s = 0; s < nstruct; s++)
+      for (int64_t q = 0; q < natoms[s]; q++) {
+        const int64_t a = start[s] + nls[s].perm[q], w = start[s] + q;
+        if (forces && !fl.energy_only)
+          for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) w + d];
+        if (fl.eatom) eatom[a] = ea[w];
+      }
   });
 }
 }

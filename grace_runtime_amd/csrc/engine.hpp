@@ -23,6 +23,9 @@ struct CsrInput {
   const int *image = nullptr;         // [nb]
   const double *shifts = nullptr;     // [nimages][3]
   int64_t nimages = 0;
+  // several independent structures in one list (no bonds between them): structure of every atom, or null for one
+  int nstruct = 1;
+  const int *sid = nullptr;           // [n] in 0 .. nstruct-1
 };
 
 struct StageTime {
@@ -48,6 +51,8 @@ class Engine {
   virtual void run(const RunFlags &fl) = 0;
   // wait for the pass and copy results out (null pointers are skipped); forces [n][3], virial [6], eatom [n]
   virtual void fetch(double *energy, double *forces, double *virial, double *eatom) = 0;
+  // the same for a list of several structures: energy [nstruct], virial [nstruct][6]
+  virtual void fetch_batch(int nstruct, double *energy, double *forces, double *virial, double *eatom) = 0;
   virtual void synchronize() = 0;
   virtual void set_profile(bool on) = 0;
   virtual const std::vector<StageTime> &stage_times() = 0;

@@ -267,7 +267,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   });
   stage("energy_mlp", [&] {
     hipLaunchKernelGGL(k_energy, dim3(n), dim3(64), 0, stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
-                       fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), fl.energy_only ? 0 : 1);
+                       fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), fl.energy_only ? 0 : 1, sid_ptr());
   });
   if (fl.energy_only) return;
 
@@ -334,7 +334,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   BondBwdArgs<T> ba{};
   ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
   ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = gA;
-  ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1;
+  ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
   ba.a0 = 0; ba.C = CP_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;
   for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
   stage("bond_bwd", [&] {

@@ -526,7 +526,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   stage("reduce_I2", [&] { reduce_fwd(redI2_, c2_.kb, c2_, B, I2_.as<double>()); });
   stage("energy_mlp", [&] {
     hipLaunchKernelGGL(k_energy_2l, dim3(n), dim3(64), 0, stream_, en_, mu_.as<int>(), n, rho_.as<double>(), I2_.as<double>(), grho_.as<double>(),
-                       gI2_.as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0);
+                       gI2_.as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0, sid_ptr());
   });
   if (!forces) return;
 
@@ -545,7 +545,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     const size_t lds = (size_t) kPairChunk * (pthreads + 2 * radR1_.noutp) * sizeof(T);
     GR_PAIR(k_pair_bwd, dim3(n), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), dR1_.as<T>(),
             (const T *) M, gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),
-            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1);
+            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr());
   });
 #undef GR_PAIR
 #undef GR_PAIR1
@@ -566,7 +566,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     BondBwdArgs<T> ba{};
     ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
     ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = c1_.gX.template as<T>();
-    ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1;
+    ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
     ba.a0 = 0; ba.C = C1P_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = radR_.noutp; ba.sh = sh_;
     for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
     stage("bond_bwd", [&] {

@@ -430,15 +430,27 @@ class EngineBase : public Engine {
       if (in.j[q] < 0 || in.j[q] >= n) throw InvalidArgument("j must index atoms 0 .. len(types)-1");
       if (in.image && (in.image[q] < 0 || in.image[q] >= in.nimages)) throw InvalidArgument("image must index rows of shifts");
     }
+    if (in.nstruct < 1) throw InvalidArgument("the number of structures must be positive");
+    if (in.sid)
+      for (int a = 0; a < n; a++)
+        if (in.sid[a] < 0 || in.sid[a] >= in.nstruct) throw InvalidArgument("structure index of an atom out of range");
+    if (in.sid)
+      for (int a = 0; a < n; a++)
+        for (int64_t q = in.offset[a]; q < in.offset[a + 1]; q++)
+          if (in.sid[in.j[q]] != in.sid[a]) throw InvalidArgument("a bond joins atoms of two structures");
     HIP_CHECK(hipStreamSynchronize(stream_));
     n_ = n;
     nb_ = nb;
+    nstruct_ = in.sid ? in.nstruct : 1;
+    have_sid_ = in.sid != nullptr;
+    scal_.ensure((size_t) 8 * nstruct_ * sizeof(double));
     have_rij_ = in.rij != nullptr;
     auto put = [&](DevBuf &b, const void *src, size_t bytes) {
       b.ensure(std::max<size_t>(bytes, 8));
       if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, hipMemcpyHostToDevice, stream_));
     };
     put(mu_, mu.data(), sizeof(int) * n);
+    if (have_sid_) put(sid_, in.sid, sizeof(int) * n);
     std::vector<int> tiles;    // tiles of 16 atoms of one element, in atom order within an element
     {
       std::vector<int> ord(n);
@@ -467,8 +479,14 @@ class EngineBase : public Engine {
   }
   void fetch(double *energy, double *forces, double *virial, double *eatom) override
   {
+    if (have_sid_) throw Error("the uploaded list holds several structures: use fetch_batch()");
+    fetch_batch(1, energy, forces, virial, eatom);
+  }
+  void fetch_batch(int nstruct, double *energy, double *forces, double *virial, double *eatom) override
+  {
     HIP_CHECK(hipSetDevice(device_));
     if (!ran_) throw Error("fetch() before run()");
+    if (nstruct != nstruct_) throw InvalidArgument("fetch_batch: the uploaded list holds " + std::to_string(nstruct_) + " structures");
     HIP_CHECK(hipStreamSynchronize(stream_));
     if (n_ > 0) {
       int zb[2];
@@ -477,11 +495,13 @@ class EngineBase : public Engine {
         throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " +
                     std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
     }
-    double s[8];
-    HIP_CHECK(hipMemcpy(s, scal_.p, sizeof(s), hipMemcpyDeviceToHost));
-    if (energy) *energy = s[0];
-    if (virial && ran_forces_)
-      for (int k = 0; k < 6; k++) virial[k] = s[1 + k];
+    std::vector<double> s((size_t) 8 * nstruct_);
+    HIP_CHECK(hipMemcpy(s.data(), scal_.p, s.size() * sizeof(double), hipMemcpyDeviceToHost));
+    for (int q = 0; q < nstruct_; q++) {
+      if (energy) energy[q] = s[8 * (size_t) q];
+      if (virial && ran_forces_)
+        for (int k = 0; k < 6; k++) virial[6 * (size_t) q + k] = s[8 * (size_t) q + 1 + k];
+    }
     if (forces && ran_forces_ && n_ > 0) HIP_CHECK(hipMemcpy(forces, f_.p, sizeof(double) * 3 * n_, hipMemcpyDeviceToHost));
     if (eatom && ran_eatom_ && n_ > 0) HIP_CHECK(hipMemcpy(eatom, eatom_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
   }
@@ -523,7 +543,7 @@ class EngineBase : public Engine {
     f_.ensure(std::max<size_t>((size_t) 3 * n, 1) * sizeof(double));
     eatom_.ensure(std::max<size_t>(n, 1) * sizeof(double));
     HIP_CHECK(hipMemsetAsync(f_.p, 0, (size_t) 3 * n * sizeof(double), stream_));
-    HIP_CHECK(hipMemsetAsync(scal_.p, 0, 8 * sizeof(double), stream_));
+    HIP_CHECK(hipMemsetAsync(scal_.p, 0, (size_t) 8 * nstruct_ * sizeof(double), stream_));
     ran_ = true;
     ran_forces_ = !fl.energy_only;
     ran_eatom_ = fl.eatom;
@@ -691,8 +711,10 @@ class EngineBase : public Engine {
   int n_ = 0;
   int64_t nb_ = 0;
   bool have_rij_ = false;
-  DevBuf cut_, mu_, offset_, j_, rij_, x_, image_, shifts_, tiles_;
-  int ntiles_ = 0;
+  DevBuf cut_, mu_, sid_, offset_, j_, rij_, x_, image_, shifts_, tiles_;
+  int ntiles_ = 0, nstruct_ = 1;
+  bool have_sid_ = false;
+  const int *sid_ptr() const { return have_sid_ ? sid_.as<int>() : nullptr; }
   // edges of the pass and its outputs (scal: energy, virial[6])
   DevBuf count_, eoff_, zero_, ei_, ej_, emu_, rh_, r_, xr_, rc_, f_, eatom_, scal_;
   bool ran_ = false, ran_forces_ = false, ran_eatom_ = false;

@@ -791,7 +791,7 @@ struct EnergyDev {
 // E_i = (MLP(rho[1:]) + rho[0]) out_scale + shift[mu_i] and dE/drho, fp64, one wave per atom (fused_1l.cpp:378-427;
 // legacy RMS layer norm fused_cpu.h:666-682)
 static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, const double *rho, double *grho, double *eatom_chunk,
-                         double *energy, int want_grad)
+                         double *energy, int want_grad, const int *sid)
 {
   __shared__ double act[8][256], pre[7][256], gbuf[2][256], x0[256];
   const int at = blockIdx.x, lane = threadIdx.x;
@@ -821,7 +821,7 @@ static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, 
   const double Ei = (act[M.nlay][0] + r[0]) * M.out_scale + M.shift[mu[a0 + at]];
   if (lane == 0) {
     if (eatom_chunk) eatom_chunk[at] = Ei;
-    atomicAdd(energy, Ei);
+    atomicAdd(energy + (sid ? 8 * sid[a0 + at] : 0), Ei);    // one (energy, virial[6]) record of 8 doubles per structure
   }
   if (!want_grad) return;
   int cur = 0;
@@ -871,7 +871,8 @@ template<class T> struct BondBwdArgs {
   const T *Rz, *dRz;          // [E][noutp]
   const T *gA;                // [chunk atoms][nlm][C]
   double *f;                  // [n][3]  (+=, atomics)
-  double *virial;             // [6]     (+=, atomics)
+  double *virial;             // [6]     (+=, atomics); with sid: record 8 sid[i] of the atom's structure
+  const int *sid;             // [n] structure of each atom, or null
   int a0;
   int C, nl, nlm, noutp;
   int drow[16];               // accumulator row of (lane / 16, register)
@@ -1002,7 +1003,7 @@ template<class T, int KB> __global__ __launch_bounds__(256) void k_bond_bwd(Bond
     const double s = red[0][t] + red[1][t] + red[2][t] + red[3][t];
     if (e1 > e0) {
       if (t < 3) atomicAdd(&a.f[3 * (long long) i + t], s);
-      else atomicAdd(&a.virial[t - 3], s);
+      else atomicAdd(&a.virial[(a.sid ? 8 * a.sid[i] : 0) + t - 3], s);
     }
   }
 }

@@ -149,7 +149,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
                            const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
                            const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
                            T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
-                           int noutp, T *__restrict__ sink, int one)
+                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   __shared__ double bsum[kPairChunk][4];
@@ -228,7 +228,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
       for (int o = 32; o > 0; o >>= 1) vsum[k] += __shfl_xor(vsum[k], o, 64);
     if (lane == 0 && e1 > e0) {
       for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) i + k], vsum[k]);
-      for (int k = 0; k < 6; k++) atomicAdd(&virial[k], vsum[3 + k]);
+      for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[i] : 0) + k], vsum[3 + k]);
     }
   }
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
@@ -248,7 +248,7 @@ struct Energy2Dev {
 // E_i = (MLP(x) + rho[0] + I2[0] ln0[0] / s0) out_scale + shift,  x_k = rho[k] lnI[k-1] / s1 + I2[k] ln0[k] / s0,
 // s1 = sqrt(mean rho[1:]^2 + eps), s0 = sqrt(mean I2^2 + eps); dE/drho, dE/dI2.  One wave per atom, fp64.
 static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, const double *rho, const double *I2, double *grho, double *gI2,
-                            double *eatom, double *energy, int want_grad)
+                            double *eatom, double *energy, int want_grad, const int *sid)
 {
   __shared__ double act[8][256], pre[7][256], gbuf[2][256], x0[256];
   const int at = blockIdx.x, lane = threadIdx.x;
@@ -285,7 +285,7 @@ static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, cons
   const double Ei = (act[M.nlay][0] + r[0] + i2[0] / s0 * M.ln0[0]) * M.out_scale + M.shift[mu[at]];
   if (lane == 0) {
     if (eatom) eatom[at] = Ei;
-    atomicAdd(energy, Ei);
+    atomicAdd(energy + (sid ? 8 * sid[at] : 0), Ei);
   }
   if (!want_grad) return;
   int cur = 0;

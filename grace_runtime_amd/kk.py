@@ -9,6 +9,7 @@ All arithmetic runs in libgrace_hip.so on the GPU; there is no CPU fallback.
 from __future__ import annotations
 
 import ctypes as C
+import os
 
 import numpy as np
 
@@ -356,7 +357,7 @@ class System:
 
 class Batch:
     """Many structures per call (python/kk/kk_api.h:116-156): energy [S], virial [S, 6], forces [N, 3] in input
-    order.  Structures are evaluated one engine pass each."""
+    order.  All structures are packed into one atom list and evaluated in one engine pass."""
 
     def __init__(self, model: Model, species, spline: int = 1024, chunksize: int = -1, precision: int = 64):
         self.engine = Engine(model, species, precision)
@@ -384,25 +385,17 @@ class Batch:
             raise ValueError("types must be 1 .. len(species)")
         N = types.shape[0]
         out = {"energy": np.zeros(S)}
+        f, v = np.zeros((N, 3)), np.zeros((S, 6))
+        ea = np.zeros(N) if energies else None
+        pb = np.ascontiguousarray(pbc, dtype=np.uint8)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
+        nth = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else 1
+        # every structure's list is built on the host (in parallel), all structures go through the GPU in ONE pass
+        check(_lib.lib().gr_compute_batch(self.engine._h, S, ptr(natoms), ptr(types), ptr(pos), ptr(cells), ptr(pb), flags, min(nth, 16),
+                                          ptr(out["energy"]), ptr(f), ptr(v), ptr(ea) if energies else None))
+        self.passes = 1 if N else 0
         if not energy_only:
-            out["forces"], out["virial"] = np.zeros((N, 3)), np.zeros((S, 6))
+            out["forces"], out["virial"] = f, v
         if energies:
-            out["energies"] = np.zeros(N)
-        starts = np.concatenate([[0], np.cumsum(natoms)])
-        self.passes = 0
-        for k in range(S):
-            lo, hi = starts[k], starts[k + 1]
-            if hi == lo:
-                continue
-            pcell, shift = _padded_cell_arrays(cells[k], pos[lo:hi], self.cutoff, pbc[k])
-            perm, offset, j, image, shifts = neighbor_search(pos[lo:hi] + shift, pcell, pbc[k], self.cutoff)
-            r = self.engine.compute(types[lo:hi][perm], offset, j, energies=energies, energy_only=energy_only,
-                                    positions=pos[lo:hi][perm], image=image, shifts=shifts)
-            self.passes += 1
-            out["energy"][k] = r["energy"]
-            if not energy_only:
-                out["forces"][lo + perm] = r["forces"]
-                out["virial"][k] = r["virial"]
-            if energies:
-                out["energies"][lo + perm] = r["energies"]
+            out["energies"] = ea
         return out

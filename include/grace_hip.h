@@ -117,6 +117,22 @@ void gr_nlist_free(gr_nlist *l);
 int gr_compute(gr_engine *e, int n, const int *types, const double *positions, const double *cell,
                const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom);
 
+/* Several independent structures in one pass (the batched small-structure workload).  Replaces Batch::compute of the
+ * reference GPU module (python/kk/kk_api.h:116-156, python/kk/kk_core.cpp:960-1160: structures packed into one atom
+ * list, one engine pass, per-structure energies and virials).
+ * gr_compute_batch: natoms [nstruct], types / positions of all atoms structure after structure, cells [nstruct][3][3],
+ * pbc [nstruct][3]; per structure the list of gr_compute (open directions padded), all lists built on `nthreads` host
+ * threads; energy [nstruct], virial [nstruct][6], forces [N][3] and eatom [N] in the caller's atom order.
+ * gr_engine_upload_batch / gr_engine_fetch_batch: the resident form for a caller with its own lists: one CSR list over
+ * all atoms (no bond may join two structures) and the structure of every atom. */
+int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
+                     const unsigned char *pbc, unsigned flags, int nthreads, double *energy, double *forces, double *virial,
+                     double *eatom);
+int gr_engine_upload_batch(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
+                           const double *positions, const int *image, const double *shifts, int64_t nimages, int nstruct,
+                           const int *struct_of_atom);
+int gr_engine_fetch_batch(gr_engine *e, int nstruct, double *energy, double *forces, double *virial, double *eatom);
+
 #ifdef __cplusplus
 }
 #endif

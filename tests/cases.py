@@ -51,8 +51,13 @@ def model_l2mix():
     return d
 
 
-MODELS = {"config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
-LAYERS = {"config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
+def model_config5():
+    """the GRACE-2L-shaped benchmark model with 3 species (batched small-structure workload)"""
+    return synth.random_model_2l(n_elements=3, element_names=("Al", "Ni", "Ti"), inv_avg_n_neigh=1.0 / 60.0, seed=20260105)
+
+
+MODELS = {"config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
+LAYERS = {"config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
 
 
 def write_model(name, directory):
@@ -115,6 +120,37 @@ def structure_config3():
     rng = np.random.default_rng(3)
     types = rng.integers(1, 5, size=len(pos)).astype(np.int32)
     return synth.jitter(pos, 0.08, 3), cell, np.array([True, True, True]), types
+
+
+def structures_config5(nstruct=512, seed=5):
+    """Independent periodic cells of 32 .. 128 atoms: random bcc / fcc / hcp lattice with lattice constant U(2.8, 4.0) A,
+    cell strain U(-3 %, 3 %), N(0, 0.1 A) jitter, 3 species drawn uniformly; atoms removed at random from the smallest
+    supercell that holds the drawn size.  Returns lists (positions, cell, types) and pbc = True."""
+    rng = np.random.default_rng(seed)
+    s3 = np.sqrt(3.0)
+    lattices = {
+        "bcc": (np.eye(3), np.array([[0, 0, 0], [0.5, 0.5, 0.5]])),
+        "fcc": (np.eye(3), np.array([[0, 0, 0], [0.5, 0.5, 0], [0.5, 0, 0.5], [0, 0.5, 0.5]])),
+        "hcp": (np.diag([1.0, s3, np.sqrt(8.0 / 3.0)]), np.array([[0, 0, 0], [0.5, 0.5, 0], [0.5, 5.0 / 6.0, 0.5], [0, 1.0 / 3.0, 0.5]])),
+    }
+    out = []
+    for _ in range(nstruct):
+        n = int(rng.integers(32, 129))
+        unit, basis = lattices[["bcc", "fcc", "hcp"][int(rng.integers(0, 3))]]
+        a = rng.uniform(2.8, 4.0)
+        reps = [1, 1, 1]
+        while reps[0] * reps[1] * reps[2] * len(basis) < n:
+            reps[int(np.argmin([reps[k] * unit[k, k] for k in range(3)]))] += 1
+        g = np.stack(np.meshgrid(*[np.arange(r) for r in reps], indexing="ij"), -1).reshape(-1, 1, 3)
+        frac = (g + basis[None]).reshape(-1, 3)
+        keep = np.sort(rng.permutation(len(frac))[:n])
+        cell = np.diag([reps[k] * unit[k, k] * a for k in range(3)])
+        pos = frac[keep] * np.array([unit[k, k] * a for k in range(3)])
+        eps = rng.uniform(-0.03, 0.03, (3, 3))
+        F = np.eye(3) + 0.5 * (eps + eps.T)
+        pos = pos @ F.T + rng.normal(0.0, 0.1, (n, 3))
+        out.append((pos, cell @ F.T, rng.integers(1, 4, n).astype(np.int32)))
+    return out
 
 
 STRUCTURES = {"fcc108": structure_fcc108, "config1": structure_config1, "alloy54": structure_alloy54, "triclinic": structure_triclinic,

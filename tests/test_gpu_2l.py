@@ -192,3 +192,33 @@ def test_system_and_batch(engines):
         assert abs(out["energy"][k] - one["energy"]) < 1e-9
         assert np.abs(out["forces"][lo:lo + len(p)] - one["forces"]).max() < 1e-9 * max(1.0, np.abs(one["forces"]).max())
         lo += len(p)
+
+
+def test_batched_small_structures(engines):
+    """48 cells of the batched benchmark workload (32 .. 128 atoms, bcc / fcc / hcp, strained, 3 species): one engine pass
+    over all of them = the structures one by one; per-structure energies are the sums of their atoms' energies"""
+    eng = engines("config5", ["Al", "Ni", "Ti"])
+    structs = cases.structures_config5(48)
+    natoms = [len(x[0]) for x in structs]
+    assert min(natoms) >= 32 and max(natoms) <= 128 and len(set(natoms)) > 20
+    b = kk.Batch(eng.model, ["Al", "Ni", "Ti"])
+    pbc = np.ones((len(structs), 3), bool)
+    out = b.compute(natoms, np.concatenate([x[2] for x in structs]), np.concatenate([x[0] for x in structs]),
+                    np.stack([x[1] for x in structs]), pbc, energies=True)
+    assert b.passes == 1
+    one = kk.System(eng.model, ["Al", "Ni", "Ti"], skin=0.0)
+    lo = 0
+    for k, (p, c, t) in enumerate(structs):
+        r = one.compute(t, p, c, [True, True, True], energies=True)
+        fs = max(1.0, np.abs(r["forces"]).max())
+        assert abs(out["energy"][k] - r["energy"]) < 1e-9 * max(1.0, abs(r["energy"]))
+        assert np.abs(out["forces"][lo:lo + len(p)] - r["forces"]).max() < 1e-9 * fs
+        assert np.abs(out["virial"][k] - r["virial"]).max() < 1e-9 * max(1.0, np.abs(r["virial"]).max())
+        assert abs(out["energies"][lo:lo + len(p)].sum() - out["energy"][k]) < 1e-9 * max(1.0, abs(r["energy"]))
+        lo += len(p)
+    eo = b.compute(natoms, np.concatenate([x[2] for x in structs]), np.concatenate([x[0] for x in structs]),
+                   np.stack([x[1] for x in structs]), pbc, energy_only=True)
+    assert np.abs(eo["energy"] - out["energy"]).max() < 1e-9 * np.abs(out["energy"]).max() and "forces" not in eo
+    with pytest.raises(ValueError, match="do not describe"):
+        b.compute(natoms[:-1], np.concatenate([x[2] for x in structs]), np.concatenate([x[0] for x in structs]),
+                  np.stack([x[1] for x in structs]), pbc)
