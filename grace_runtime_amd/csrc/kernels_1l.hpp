@@ -457,10 +457,29 @@ template<class T> struct ScatterArgs {
   ShCoef sh;
 };
 
-// one block per atom, thread = (l, n); Y of up to kBondChunk bonds staged in LDS per pass
+// One block per atom, thread = (l, n).  The harmonics of up to kScatterBonds bonds are computed by all threads into LDS,
+// then the radial rows stream through registers in groups of kScatterGroup bonds, the loads of the next group in flight
+// while the current one is accumulated.
+constexpr int kScatterBonds = 64, kScatterGroup = 16;
+
+template<class T, int MAXM> __device__ inline void scatter_group(const T *Ysh, int b0, int nb, int lm0, int nm, const T *r, T *acc)
+{
+#pragma unroll
+  for (int u = 0; u < kScatterGroup; u++)
+    if (b0 + u < nb) {
+      // no branch per m (the lanes of a wave hold two values of l): entries beyond 2l+1 read a valid address and add 0
+      const T *y = Ysh + (b0 + u) * kMaxNlm + lm0;
+      T yv[MAXM];
+#pragma unroll
+      for (int m = 0; m < MAXM; m++) yv[m] = y[m < nm ? m : 0];
+#pragma unroll
+      for (int m = 0; m < MAXM; m++) acc[m] += (m < nm ? yv[m] : (T) 0) * r[u];
+    }
+}
+
 template<class T, int MAXM> __global__ void k_scatter_a(ScatterArgs<T> a)
 {
-  __shared__ T Ysh[kBondChunk][kMaxNlm];
+  __shared__ T Ysh[kScatterBonds * kMaxNlm];
   const int t = threadIdx.x;
   const int i = a.a0 + blockIdx.x;
   const long long e0 = a.eoff[i], e1 = a.eoff[i + 1];
@@ -470,22 +489,26 @@ template<class T, int MAXM> __global__ void k_scatter_a(ScatterArgs<T> a)
   T acc[MAXM];
 #pragma unroll
   for (int m = 0; m < MAXM; m++) acc[m] = (T) 0;
-  for (long long base = e0; base < e1; base += kBondChunk) {
-    const int nb = (int) (e1 - base < kBondChunk ? e1 - base : kBondChunk);
+  for (long long base = e0; base < e1; base += kScatterBonds) {
+    const int nb = (int) (e1 - base < kScatterBonds ? e1 - base : kScatterBonds);
+    const T *rp = a.Rz + base * a.noutp + (t < ncol ? t : 0);
+    T r0[kScatterGroup], r1[kScatterGroup];
+#pragma unroll
+    for (int u = 0; u < kScatterGroup; u++) r0[u] = rp[(long long) (u < nb ? u : 0) * a.noutp];
     __syncthreads();
-    if (t < nb) {
-      const double *u = a.rh + 3 * (base + t);
-      sh_eval<false, T>(a.sh, u[0], u[1], u[2], Ysh[t], nullptr);
+    for (int b = t; b < nb; b += blockDim.x) {
+      const double *u = a.rh + 3 * (base + b);
+      sh_eval<false, T>(a.sh, u[0], u[1], u[2], Ysh + b * kMaxNlm, nullptr);
     }
     __syncthreads();
-    if (t < ncol) {
-      for (int b = 0; b < nb; b++) {
-        const T r = a.Rz[(base + b) * a.noutp + t];
-        const T *y = Ysh[b] + lm0;
+    for (int b0 = 0; b0 < nb; b0 += 2 * kScatterGroup) {
+      const int b1 = b0 + kScatterGroup, b2 = b1 + kScatterGroup;
 #pragma unroll
-        for (int m = 0; m < MAXM; m++)
-          if (m < nm) acc[m] += y[m] * r;
-      }
+      for (int u = 0; u < kScatterGroup; u++) r1[u] = rp[(long long) (b1 + u < nb ? b1 + u : 0) * a.noutp];
+      scatter_group<T, MAXM>(Ysh, b0, nb, lm0, nm, r0, acc);
+#pragma unroll
+      for (int u = 0; u < kScatterGroup; u++) r0[u] = rp[(long long) (b2 + u < nb ? b2 + u : 0) * a.noutp];
+      scatter_group<T, MAXM>(Ysh, b1, nb, lm0, nm, r1, acc);
     }
   }
   if (t < ncol) {
