@@ -216,14 +216,10 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   rho_.ensure(na * nrho_ * sizeof(double));
   grho_.ensure(na * nrho_ * sizeof(double));
 
-  const int sthreads = round_up(nl_ * CP_, 64);
   ScatterArgs<T> sa{};
   sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz_.as<T>(); sa.A = A_.as<T>();
   sa.a0 = 0; sa.C = CP_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = noutp_; sa.sh = sh_;
-  stage("scatter_A", [&] {
-    if (lmax_ <= 4) hipLaunchKernelGGL((k_scatter_a<T, 9>), dim3(n), dim3(sthreads), 0, stream_, sa);
-    else hipLaunchKernelGGL((k_scatter_a<T, 13>), dim3(n), dim3(sthreads), 0, stream_, sa);
-  });
+  stage("scatter_A", [&] { launch_scatter<T>(sa, n, lmax_); });
 
   const int *tiles = tiles_.as<int>();
   const int ka = CP_ / 16, kf = CFP_ / 16;

@@ -466,11 +466,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     ScatterArgs<T> sa{};
     sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz_.as<T>(); sa.A = A;
     sa.a0 = 0; sa.C = C1P_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = radR_.noutp; sa.sh = sh_;
-    const int sthreads = round_up(nl_ * C1P_, 64);
-    stage("scatter_A", [&] {
-      if (lmax_ <= 4) hipLaunchKernelGGL((k_scatter_a<T, 9>), dim3(n), dim3(sthreads), 0, stream_, sa);
-      else hipLaunchKernelGGL((k_scatter_a<T, 13>), dim3(n), dim3(sthreads), 0, stream_, sa);
-    });
+    stage("scatter_A", [&] { launch_scatter<T>(sa, n, lmax_); });
   }
   chain_forward(c1_, "_L1", A);
   rho_.ensure(na * nrho_ * sizeof(double));

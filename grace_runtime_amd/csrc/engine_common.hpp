@@ -662,6 +662,29 @@ class EngineBase : public Engine {
     for (int q = 0; q < 16; q++) seen |= 1 << drow_[q];
     if (seen != 0xFFFF) throw Error("MFMA 16x16x4 accumulator layout probe failed");
   }
+  // A[atom][lm][n] = sum over the atom's edges of Y_lm Rz_l[n]: on the matrix cores where the register tiles fit
+  template<class T> void launch_scatter(ScatterArgs<T> sa, int n, int lmax)
+  {
+    sa.natoms = n;
+    for (int q = 0; q < 16; q++) sa.drow[q] = drow_[q];
+    const int kb = sa.C / 16;
+    const size_t lds = (size_t) 4 * 16 * sa.nlm * sizeof(T);
+    const dim3 grid((n + 3) / 4), block(256);
+#define GR_SCAT(NL_, KB_) hipLaunchKernelGGL((k_scatter_a_mfma<T, NL_, KB_>), grid, block, lds, stream_, sa)
+    const int key = sa.nl * 10 + kb;    // register tiles of the kernel: nl * kb <= 10
+    if (key == 11) GR_SCAT(1, 1); else if (key == 12) GR_SCAT(1, 2); else if (key == 14) GR_SCAT(1, 4);
+    else if (key == 21) GR_SCAT(2, 1); else if (key == 22) GR_SCAT(2, 2); else if (key == 24) GR_SCAT(2, 4);
+    else if (key == 31) GR_SCAT(3, 1); else if (key == 32) GR_SCAT(3, 2);
+    else if (key == 41) GR_SCAT(4, 1); else if (key == 42) GR_SCAT(4, 2);
+    else if (key == 51) GR_SCAT(5, 1); else if (key == 52) GR_SCAT(5, 2);
+    else if (key == 61) GR_SCAT(6, 1); else if (key == 71) GR_SCAT(7, 1);
+#undef GR_SCAT
+    else {
+      const int sthreads = round_up(sa.nl * sa.C, 64);
+      if (lmax <= 4) hipLaunchKernelGGL((k_scatter_a<T, 9>), dim3(n), dim3(sthreads), 0, stream_, sa);
+      else hipLaunchKernelGGL((k_scatter_a<T, 13>), dim3(n), dim3(sthreads), 0, stream_, sa);
+    }
+  }
   // out[tile atoms][job output] = GEMM jobs over X0 (kb0 16-channel blocks) and X1 (kb1), nb output blocks
   template<class T>
   void launch_gemm(DevJobs<T> &J, int kb0, int kb1, int nb, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo, int accumulate,
