@@ -176,6 +176,8 @@ template<class T> void Engine1L<T>::build()
     en_.act = m.energy_mlp_activation;
     en_.ln = m.energy_mlp_ln;
     en_.nrho = nrho_;
+    en_.width = nrho_;
+    for (int L = 0; L < en_.nlay; L++) en_.width = std::max({en_.width, en_.nin[L], en_.nout[L]});
     en_.out_scale = m.output_scale;
     en_.shift = shift_.as<double>();
   }
@@ -262,7 +264,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
 #undef GR_RED
   });
   stage("energy_mlp", [&] {
-    hipLaunchKernelGGL(k_energy, dim3(n), dim3(64), 0, stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
+    hipLaunchKernelGGL(k_energy, dim3(n), dim3(64), (size_t) (2 * en_.nlay + 4) * en_.width * sizeof(double), stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
                        fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), fl.energy_only ? 0 : 1, sid_ptr());
   });
   if (fl.energy_only) return;
@@ -332,15 +334,8 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = gA;
   ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
   ba.a0 = 0; ba.C = CP_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;
-  for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
-  stage("bond_bwd", [&] {
-    const size_t lds = ((size_t) nl_ * (CP_ / 4) * 64 + (size_t) 4 * 16 * nlm_ * 4) * sizeof(T);
-    switch (CP_ / 16) {
-      case 1: hipLaunchKernelGGL((k_bond_bwd<T, 1>), dim3(n), dim3(256), lds, stream_, ba); break;
-      case 2: hipLaunchKernelGGL((k_bond_bwd<T, 2>), dim3(n), dim3(256), lds, stream_, ba); break;
-      default: hipLaunchKernelGGL((k_bond_bwd<T, 4>), dim3(n), dim3(256), lds, stream_, ba); break;
-    }
-  });
+  stage("bond_bwd", [&] { launch_bond_bwd<T>(ba, n); });
+
 }
 
 template<class T> void Engine1L<T>::debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz)

@@ -298,6 +298,8 @@ template<class T> void Engine2L<T>::build()
     en_.act = m.energy_mlp_activation;
     en_.ln = m.energy_mlp_ln;
     en_.nrho = nrho_;
+    en_.width = nrho_;
+    for (int L = 0; L < en_.nlay; L++) en_.width = std::max({en_.width, en_.nin[L], en_.nout[L]});
     en_.rms = m.energy_rms_norm;
     en_.eps = Model2L::rms_norm_eps;
     en_.out_scale = m.output_scale;
@@ -521,7 +523,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   gI2_.ensure(na * nrho_ * sizeof(double));
   stage("reduce_I2", [&] { reduce_fwd(redI2_, c2_.kb, c2_, B, I2_.as<double>()); });
   stage("energy_mlp", [&] {
-    hipLaunchKernelGGL(k_energy_2l, dim3(n), dim3(64), 0, stream_, en_, mu_.as<int>(), n, rho_.as<double>(), I2_.as<double>(), grho_.as<double>(),
+    hipLaunchKernelGGL(k_energy_2l, dim3(n), dim3(64), (size_t) (2 * en_.nlay + 4) * en_.width * sizeof(double), stream_, en_, mu_.as<int>(), n, rho_.as<double>(), I2_.as<double>(), grho_.as<double>(),
                        gI2_.as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0, sid_ptr());
   });
   if (!forces) return;
@@ -564,15 +566,8 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = c1_.gX.template as<T>();
     ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
     ba.a0 = 0; ba.C = C1P_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = radR_.noutp; ba.sh = sh_;
-    for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
-    stage("bond_bwd", [&] {
-      const size_t lds = ((size_t) nl_ * (C1P_ / 4) * 64 + (size_t) 4 * 16 * nlm_ * 4) * sizeof(T);
-      switch (C1P_ / 16) {
-        case 1: hipLaunchKernelGGL((k_bond_bwd<T, 1>), dim3(n), dim3(256), lds, stream_, ba); break;
-        case 2: hipLaunchKernelGGL((k_bond_bwd<T, 2>), dim3(n), dim3(256), lds, stream_, ba); break;
-        default: hipLaunchKernelGGL((k_bond_bwd<T, 4>), dim3(n), dim3(256), lds, stream_, ba); break;
-      }
-    });
+      stage("bond_bwd", [&] { launch_bond_bwd<T>(ba, n); });
+
   }
 }
 

@@ -685,6 +685,18 @@ class EngineBase : public Engine {
       else hipLaunchKernelGGL((k_scatter_a<T, 13>), dim3(n), dim3(sthreads), 0, stream_, sa);
     }
   }
+  // per-bond forces of a layer from the adjoint of its A basis (k_bond_bwd); ba.drow is filled here
+  template<class T> void launch_bond_bwd(BondBwdArgs<T> ba, int n)
+  {
+    for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
+    const int kb = ba.C / 16;
+    const size_t lds = ((size_t) ba.nl * (ba.C / 4) * 64 + (size_t) 4 * 16 * ba.nlm * 4) * sizeof(T);
+    switch (kb) {
+      case 1: hipLaunchKernelGGL((k_bond_bwd<T, 1>), dim3(n), dim3(256), lds, stream_, ba); break;
+      case 2: hipLaunchKernelGGL((k_bond_bwd<T, 2>), dim3(n), dim3(256), lds, stream_, ba); break;
+      default: hipLaunchKernelGGL((k_bond_bwd<T, 4>), dim3(n), dim3(256), lds, stream_, ba); break;
+    }
+  }
   // out[tile atoms][job output] = GEMM jobs over X0 (kb0 16-channel blocks) and X1 (kb1), nb output blocks
   template<class T>
   void launch_gemm(DevJobs<T> &J, int kb0, int kb1, int nb, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo, int accumulate,

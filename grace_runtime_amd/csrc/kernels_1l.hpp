@@ -880,7 +880,7 @@ struct EnergyDev {
   const double *W[7];         // [n_in][n_out]
   double norm[7];
   int nin[7], nout[7];
-  int nlay, act, ln, nrho;
+  int nlay, act, ln, nrho, width;    // width: largest layer width (LDS row of the kernel)
   double out_scale;
   const double *shift;        // [nel]
 };
@@ -890,72 +890,81 @@ struct EnergyDev {
 static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, const double *rho, double *grho, double *eatom_chunk,
                          double *energy, int want_grad, const int *sid)
 {
-  __shared__ double act[8][256], pre[7][256], gbuf[2][256], x0[256];
+  // LDS rows of W = M.width values: nlay + 1 activations, nlay pre-activations, 2 adjoint buffers, x0
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int W = M.width;
+  double *act_ = reinterpret_cast<double *>(smem_raw), *pre_ = act_ + (M.nlay + 1) * W, *gbuf_ = pre_ + M.nlay * W, *x0 = gbuf_ + 2 * W;
+#define act(L_, k_) act_[(L_) * W + (k_)]
+#define pre(L_, k_) pre_[(L_) * W + (k_)]
+#define gbuf(L_, k_) gbuf_[(L_) * W + (k_)]
   const int at = blockIdx.x, lane = threadIdx.x;
   const double *r = rho + (long long) at * M.nrho;
   const int n0 = M.nrho - 1;
-  for (int k = lane; k < n0; k += 64) act[0][k] = r[k + 1];
+  for (int k = lane; k < n0; k += 64) act(0, k) = r[k + 1];
   __syncthreads();
   double q = 0.0;
   if (M.ln) {
     double ms = 0.0;
-    for (int k = lane; k < n0; k += 64) { x0[k] = act[0][k]; ms += act[0][k] * act[0][k]; }
+    for (int k = lane; k < n0; k += 64) { x0[k] = act(0, k); ms += act(0, k) * act(0, k); }
     for (int o = 32; o > 0; o >>= 1) ms += __shfl_xor(ms, o, 64);
     q = 1.0 / sqrt(ms / n0 + 1e-16);
-    for (int k = lane; k < n0; k += 64) act[0][k] *= q;
+    for (int k = lane; k < n0; k += 64) act(0, k) *= q;
     __syncthreads();
   }
   for (int L = 0; L < M.nlay; L++) {
     for (int c = lane; c < M.nout[L]; c += 64) {
       double s = 0.0;
-      for (int a = 0; a < M.nin[L]; a++) s += act[L][a] * M.W[L][(long long) a * M.nout[L] + c];
+      for (int a = 0; a < M.nin[L]; a++) s += act(L, a) * M.W[L][(long long) a * M.nout[L] + c];
       s *= M.norm[L];
-      pre[L][c] = s;
-      act[L + 1][c] = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+      pre(L, c) = s;
+      act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
     }
     __syncthreads();
   }
-  const double Ei = (act[M.nlay][0] + r[0]) * M.out_scale + M.shift[mu[a0 + at]];
+  const double Ei = (act(M.nlay, 0) + r[0]) * M.out_scale + M.shift[mu[a0 + at]];
   if (lane == 0) {
     if (eatom_chunk) eatom_chunk[at] = Ei;
     atomicAdd(energy + (sid ? 8 * sid[a0 + at] : 0), Ei);    // one (energy, virial[6]) record of 8 doubles per structure
   }
   if (!want_grad) return;
   int cur = 0;
-  if (lane == 0) gbuf[0][0] = M.out_scale;
+  if (lane == 0) gbuf(0, 0) = M.out_scale;
   __syncthreads();
   for (int L = M.nlay - 1; L >= 0; L--) {
     if (L < M.nlay - 1) {
       for (int c = lane; c < M.nout[L]; c += 64) {
-        const double v = pre[L][c];
+        const double v = pre(L, c);
         if (M.act == 1) {
-          const double t = act[L + 1][c];
-          gbuf[cur][c] *= 1.0 - t * t;
+          const double t = act(L + 1, c);
+          gbuf(cur, c) *= 1.0 - t * t;
         } else {
           const double sg = 1.0 / (1.0 + exp(-v));
-          gbuf[cur][c] *= sg * (1.0 + v * (1.0 - sg));
+          gbuf(cur, c) *= sg * (1.0 + v * (1.0 - sg));
         }
       }
       __syncthreads();
     }
     for (int a = lane; a < M.nin[L]; a += 64) {
       double s = 0.0;
-      for (int c = 0; c < M.nout[L]; c++) s += gbuf[cur][c] * M.W[L][(long long) a * M.nout[L] + c];
-      gbuf[cur ^ 1][a] = s * M.norm[L];
+      for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * M.W[L][(long long) a * M.nout[L] + c];
+      gbuf(cur ^ 1, a) = s * M.norm[L];
     }
     cur ^= 1;
     __syncthreads();
   }
   if (M.ln) {
     double t = 0.0;
-    for (int k = lane; k < n0; k += 64) t += gbuf[cur][k] * x0[k];
+    for (int k = lane; k < n0; k += 64) t += gbuf(cur, k) * x0[k];
     for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
-    for (int k = lane; k < n0; k += 64) gbuf[cur][k] = q * (gbuf[cur][k] - x0[k] * t * q * q / n0);
+    for (int k = lane; k < n0; k += 64) gbuf(cur, k) = q * (gbuf(cur, k) - x0[k] * t * q * q / n0);
     __syncthreads();
   }
   double *g = grho + (long long) at * M.nrho;
   if (lane == 0) g[0] = M.out_scale;
-  for (int k = lane; k < n0; k += 64) g[k + 1] = gbuf[cur][k];
+  for (int k = lane; k < n0; k += 64) g[k + 1] = gbuf(cur, k);
+#undef act
+#undef pre
+#undef gbuf
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -238,7 +238,7 @@ struct Energy2Dev {
   const double *W[7];         // [n_in][n_out]
   double norm[7];
   int nin[7], nout[7];
-  int nlay, act, ln, nrho, rms;
+  int nlay, act, ln, nrho, rms, width;    // width: largest layer width (LDS row of the kernel)
   double out_scale, eps;
   const double *shift;        // [nel]
   const double *lnI;          // [nrho - 1] scale of the only_nonlin RMSNorm of rho
@@ -250,7 +250,13 @@ struct Energy2Dev {
 static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, const double *rho, const double *I2, double *grho, double *gI2,
                             double *eatom, double *energy, int want_grad, const int *sid)
 {
-  __shared__ double act[8][256], pre[7][256], gbuf[2][256], x0[256];
+  // LDS rows of W = M.width values: nlay + 1 activations, nlay pre-activations, 2 adjoint buffers, x0
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int W = M.width;
+  double *act_ = reinterpret_cast<double *>(smem_raw), *pre_ = act_ + (M.nlay + 1) * W, *gbuf_ = pre_ + M.nlay * W, *x0 = gbuf_ + 2 * W;
+#define act(L_, k_) act_[(L_) * W + (k_)]
+#define pre(L_, k_) pre_[(L_) * W + (k_)]
+#define gbuf(L_, k_) gbuf_[(L_) * W + (k_)]
   const int at = blockIdx.x, lane = threadIdx.x;
   const double *r = rho + (long long) at * M.nrho, *i2 = I2 + (long long) at * M.nrho;
   const int nr = M.nrho, n0 = nr - 1;
@@ -261,70 +267,70 @@ static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, cons
   }
   for (int o = 32; o > 0; o >>= 1) { ms1 += __shfl_xor(ms1, o, 64); ms0 += __shfl_xor(ms0, o, 64); }
   const double s1 = M.rms ? sqrt(ms1 / n0 + M.eps) : 1.0, s0 = M.rms ? sqrt(ms0 / nr + M.eps) : 1.0;
-  for (int k = lane; k < n0; k += 64) act[0][k] = r[k + 1] / s1 * M.lnI[k] + i2[k + 1] / s0 * M.ln0[k + 1];
+  for (int k = lane; k < n0; k += 64) act(0, k) = r[k + 1] / s1 * M.lnI[k] + i2[k + 1] / s0 * M.ln0[k + 1];
   __syncthreads();
   double q = 0.0;
   if (M.ln) {
     double ms = 0.0;
-    for (int k = lane; k < n0; k += 64) { x0[k] = act[0][k]; ms += act[0][k] * act[0][k]; }
+    for (int k = lane; k < n0; k += 64) { x0[k] = act(0, k); ms += act(0, k) * act(0, k); }
     for (int o = 32; o > 0; o >>= 1) ms += __shfl_xor(ms, o, 64);
     q = 1.0 / sqrt(ms / n0 + 1e-16);
-    for (int k = lane; k < n0; k += 64) act[0][k] *= q;
+    for (int k = lane; k < n0; k += 64) act(0, k) *= q;
     __syncthreads();
   }
   for (int L = 0; L < M.nlay; L++) {
     for (int c = lane; c < M.nout[L]; c += 64) {
       double s = 0.0;
-      for (int a = 0; a < M.nin[L]; a++) s += act[L][a] * M.W[L][(long long) a * M.nout[L] + c];
+      for (int a = 0; a < M.nin[L]; a++) s += act(L, a) * M.W[L][(long long) a * M.nout[L] + c];
       s *= M.norm[L];
-      pre[L][c] = s;
-      act[L + 1][c] = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+      pre(L, c) = s;
+      act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
     }
     __syncthreads();
   }
-  const double Ei = (act[M.nlay][0] + r[0] + i2[0] / s0 * M.ln0[0]) * M.out_scale + M.shift[mu[at]];
+  const double Ei = (act(M.nlay, 0) + r[0] + i2[0] / s0 * M.ln0[0]) * M.out_scale + M.shift[mu[at]];
   if (lane == 0) {
     if (eatom) eatom[at] = Ei;
     atomicAdd(energy + (sid ? 8 * sid[at] : 0), Ei);
   }
   if (!want_grad) return;
   int cur = 0;
-  if (lane == 0) gbuf[0][0] = M.out_scale;
+  if (lane == 0) gbuf(0, 0) = M.out_scale;
   __syncthreads();
   for (int L = M.nlay - 1; L >= 0; L--) {
     if (L < M.nlay - 1) {
       for (int c = lane; c < M.nout[L]; c += 64) {
-        const double v = pre[L][c];
+        const double v = pre(L, c);
         if (M.act == 1) {
-          const double tt = act[L + 1][c];
-          gbuf[cur][c] *= 1.0 - tt * tt;
+          const double tt = act(L + 1, c);
+          gbuf(cur, c) *= 1.0 - tt * tt;
         } else {
           const double sg = 1.0 / (1.0 + exp(-v));
-          gbuf[cur][c] *= sg * (1.0 + v * (1.0 - sg));
+          gbuf(cur, c) *= sg * (1.0 + v * (1.0 - sg));
         }
       }
       __syncthreads();
     }
     for (int a = lane; a < M.nin[L]; a += 64) {
       double s = 0.0;
-      for (int c = 0; c < M.nout[L]; c++) s += gbuf[cur][c] * M.W[L][(long long) a * M.nout[L] + c];
-      gbuf[cur ^ 1][a] = s * M.norm[L];
+      for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * M.W[L][(long long) a * M.nout[L] + c];
+      gbuf(cur ^ 1, a) = s * M.norm[L];
     }
     cur ^= 1;
     __syncthreads();
   }
   if (M.ln) {
     double tt = 0.0;
-    for (int k = lane; k < n0; k += 64) tt += gbuf[cur][k] * x0[k];
+    for (int k = lane; k < n0; k += 64) tt += gbuf(cur, k) * x0[k];
     for (int o = 32; o > 0; o >>= 1) tt += __shfl_xor(tt, o, 64);
-    for (int k = lane; k < n0; k += 64) gbuf[cur][k] = q * (gbuf[cur][k] - x0[k] * tt * q * q / n0);
+    for (int k = lane; k < n0; k += 64) gbuf(cur, k) = q * (gbuf(cur, k) - x0[k] * tt * q * q / n0);
     __syncthreads();
   }
-  // gbuf[cur][k-1] = dE/dx_k; RMSNorm reverses (y_k = x_k s_k / sigma)
+  // gbuf(cur, k-1) = dE/dx_k; RMSNorm reverses (y_k = x_k s_k / sigma)
   double t1 = 0.0, t0 = 0.0;
   if (M.rms) {
     for (int k = lane; k < nr; k += 64) {
-      const double gy = k == 0 ? M.out_scale : gbuf[cur][k - 1];
+      const double gy = k == 0 ? M.out_scale : gbuf(cur, k - 1);
       if (k > 0) t1 += gy * M.lnI[k - 1] * r[k];
       t0 += gy * M.ln0[k] * i2[k];
     }
@@ -332,10 +338,13 @@ static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, cons
   }
   double *gr = grho + (long long) at * nr, *gi = gI2 + (long long) at * nr;
   for (int k = lane; k < nr; k += 64) {
-    const double gy = k == 0 ? M.out_scale : gbuf[cur][k - 1];
+    const double gy = k == 0 ? M.out_scale : gbuf(cur, k - 1);
     gr[k] = k == 0 ? M.out_scale : gy * M.lnI[k - 1] / s1 - r[k] * t1 / (n0 * s1 * s1 * s1);
     gi[k] = gy * M.ln0[k] / s0 - i2[k] * t0 / (nr * s0 * s0 * s0);
   }
+#undef act
+#undef pre
+#undef gbuf
 }
 
 }    // namespace grhip
