@@ -53,10 +53,11 @@ constexpr int kPairChunk = 8;    // bonds staged in LDS at a time by the pair ke
 
 // Stages what a chunk of nb bonds (edges base .. base + nb) needs into LDS with all loads in flight at once: the
 // neighbour rows M_j[slot][n] of this thread, the radial rows (contiguous in memory), and touches the harmonics of the
-// chunk so that the uniform (scalar) reads of the bond loop find them in the L2.
+// chunk (the first yuse values of every row of ylen) so that the uniform (scalar) reads of the bond loop find them in
+// the L2.
 template<class T>
 __device__ inline T pair_stage(const int *__restrict__ ej, const T *__restrict__ M, const T *__restrict__ R1, const T *__restrict__ dR1,
-                               const T *__restrict__ Yu, int ylen, long long base, int nb, int nslot, int C, int nrow, bool active, int slot,
+                               const T *__restrict__ Yu, int ylen, int yuse, long long base, int nb, int nslot, int C, int nrow, bool active, int slot,
                                int n, T *Msh, T *Rsh, T *dRsh, int NT)
 {
   const int t = threadIdx.x;
@@ -73,7 +74,8 @@ __device__ inline T pair_stage(const int *__restrict__ ej, const T *__restrict__
   }
   T touch = (T) 0;
   const T *yu = Yu + base * ylen;
-  for (int q = t * 8; q < nb * ylen; q += blockDim.x * 8) touch += yu[q];
+  const int per = (yuse + 7) / 8;    // 64-byte pieces of a row that the bond loop reads
+  for (int q = t; q < nb * per; q += blockDim.x) touch += yu[(q / per) * ylen + (q % per) * 8];
 #pragma unroll
   for (int b = 0; b < kPairChunk; b++) Msh[b * NT + t] = mv[b];
   return touch;
@@ -99,7 +101,7 @@ __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__rest
   for (long long base = e0; base < e1; base += kPairChunk) {
     const int nb = (int) (e1 - base < kPairChunk ? e1 - base : kPairChunk);
     __syncthreads();
-    touch += pair_stage<T>(ej, M, R1, nullptr, Y, ystride, base, nb, nslot, C, noutp, true, slot, n, Msh, Rsh, nullptr, NT);
+    touch += pair_stage<T>(ej, M, R1, nullptr, Y, ystride, nlm, base, nb, nslot, C, noutp, true, slot, n, Msh, Rsh, nullptr, NT);
     __syncthreads();
     for (int b = 0; b < nb; b++) {
       const T m = Msh[b * NT + t];
@@ -170,7 +172,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
   for (long long base = e0; base < e1; base += kPairChunk) {
     const int nb = (int) (e1 - base < kPairChunk ? e1 - base : kPairChunk);
     __syncthreads();
-    touch += pair_stage<T>(ej, M, R1, dR1, YG, nlm * 4, base, nb, nslot, C, noutp, active, slot, n, Msh, Rsh, dRsh, NT);
+    touch += pair_stage<T>(ej, M, R1, dR1, YG, nlm * 4, nlm * 4, base, nb, nslot, C, noutp, active, slot, n, Msh, Rsh, dRsh, NT);
     if (t < kPairChunk * 4) bsum[t >> 2][t & 3] = 0.0;
     __syncthreads();
     for (int b = 0; b < nb; b++) {
