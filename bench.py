@@ -33,7 +33,10 @@ HBM_PEAK = 8000.0                 # GB/s
 
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs of this
 # script, counters scaled by what they read for the 1 GiB copy kernel; summaries under profiles/): (workload, kernel)
-MEASURED_TRAFFIC = {}
+MEASURED_TRAFFIC = {
+    ("config2", "radial_mlp"): 366.7e6 + 1241.0e6,      # fetch + write of k_radial<double,4,0>
+    ("config3", "pair_bwd"): 11902.3e6 + 2822.2e6,      # fetch + write of k_pair_bwd<double,25>
+}
 
 
 def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4):
@@ -118,6 +121,14 @@ def main():
     dt = (time.perf_counter() - t0) / a.steps
     out = eng.fetch()
     E = eng.edge_count()
+    # the same pass through the one-call entry point: host buffers in (PCIe), pass, results out; reported beside, never as `value`
+    th = []
+    for _ in range(4):
+        t1 = time.perf_counter()
+        eng.compute(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
+        th.append(time.perf_counter() - t1)
+    host_ms = float(np.median(th[1:])) * 1e3
+    eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
 
     # per-stage durations: HIP events around every launch on the engine's stream, averaged over the same K steps
     eng.set_profile(True)
@@ -180,6 +191,7 @@ def main():
                                 f"{reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[1])"),
                    "atoms": N, "edges": int(E)},
         "atoms_steps_per_s": round(N / dt, 1),
+        "ms_per_call_host_buffers": round(host_ms, 3),
         "roofline": roofline,
         "stages_ms": {k: round(v, 4) for k, v in stages.items()},
         "stages_roofline": {k: {"bound": v["bound"], "achieved": round(v["achieved"], 2), "unit": v["unit"],
