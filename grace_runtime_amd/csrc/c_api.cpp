@@ -18,6 +18,7 @@ struct gr_model {
   grhip::ModelKind kind;
   std::shared_ptr<grhip::Model1L> m1;
   std::shared_ptr<grhip::Model2L> m2;
+  std::shared_ptr<grhip::Model3L> m3;
   std::string path;
 };
 struct gr_engine {
@@ -120,8 +121,8 @@ int gr_model_load(const char *npz_path, gr_model **out)
       m->m2 = std::make_shared<grhip::Model2L>();
       m->m2->load(z);
     } else {
-      throw grhip::InvalidArgument("unsupported model: this build of the GPU engine implements GRACE-1L and GRACE-2L; the file holds a "
-                                   "GRACE-3L model");
+      m->m3 = std::make_shared<grhip::Model3L>();
+      m->m3->load(z);
     }
     *out = m.release();
   });
@@ -151,6 +152,15 @@ int gr_model_get_info(const gr_model *m, gr_model_info *info)
       double rc = 0.0;
       for (double c : m->m2->bond_cutoff_map) rc = std::max(rc, c);
       info->rcut = m->m2->has_bond_specific_cutoff ? rc : m->m2->rcut;
+    } else if (m->m3) {
+      info->n_elements = m->m3->n_elements;
+      info->lmax = m->m3->lmax;
+      info->n_radial = m->m3->spbf.empty() ? 0 : m->m3->spbf[0].n_rad_max;
+      info->n_radbase = m->m3->nradbase;
+      info->max_order = 4;
+      double rc = 0.0;
+      for (double c : m->m3->bond_cutoff_map) rc = std::max(rc, c);
+      info->rcut = m->m3->has_bond_specific_cutoff ? rc : m->m3->rcut;
     }
   });
 }
@@ -158,7 +168,7 @@ int gr_model_get_info(const gr_model *m, gr_model_info *info)
 const char *gr_model_element_name(const gr_model *m, int k)
 {
   if (!m || k < 0) return "";
-  const std::vector<std::string> &names = m->m1 ? m->m1->element_names : m->m2->element_names;
+  const std::vector<std::string> &names = m->m1 ? m->m1->element_names : m->m2 ? m->m2->element_names : m->m3->element_names;
   return k < (int) names.size() ? names[k].c_str() : "";
 }
 
@@ -173,7 +183,8 @@ int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int prec
     std::vector<int> t(type2mu, type2mu + ntypes + 1);
     auto e = std::make_unique<gr_engine>();
     if (m->m1) e->eng = grhip::make_engine_1l(m->m1, ntypes, t, precision, device);
-    else e->eng = grhip::make_engine_2l(m->m2, ntypes, t, precision, device);
+    else if (m->m2) e->eng = grhip::make_engine_2l(m->m2, ntypes, t, precision, device);
+    else e->eng = grhip::make_engine_3l(m->m3, ntypes, t, precision, device);
     *out = e.release();
   });
 }

@@ -5,6 +5,7 @@
 
 #include "model.hpp"
 #include "model_2l.hpp"
+#include "model_3l.hpp"
 
 #include <cstdint>
 #include <memory>
@@ -70,6 +71,10 @@ std::unique_ptr<Engine> make_engine_1l(std::shared_ptr<const Model1L> model, int
 
 // GRACE-2L: network arithmetic in fp64 only (precision 64)
 std::unique_ptr<Engine> make_engine_2l(std::shared_ptr<const Model2L> model, int ntypes, const std::vector<int> &type2mu,
+                                       int precision, int device);
+
+// GRACE-3L: network arithmetic in fp64 only (precision 64)
+std::unique_ptr<Engine> make_engine_3l(std::shared_ptr<const Model3L> model, int ntypes, const std::vector<int> &type2mu,
                                        int precision, int device);
 
 }    // namespace grhip

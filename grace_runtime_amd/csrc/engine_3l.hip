@@ -1,0 +1,762 @@
+// GRACE-3L engine for gfx950: three message-passing layers on one GPU, whole structure resident.
+// Dataflow after libgrace/src/fused_3l.cpp:1550-1637 of the reference (layer 1, 2, 3 forward with the normalised
+// messages I1, I2 of every atom kept; readout; layer 3, 2, 1 reverse with dE/dI_j added to the neighbours), without
+// the recompute of layers 1-2: the forward tensors the reverse reads stay in device memory.
+//
+// Per layer (names of libgrace/src/model_3l.cpp:28-36):
+//   radial functions  R[e][l][n] = MLP([T_k(2x-1), emb_i, emb_j]) env(x) fac[mu_j][n]          k_radial, species form
+//   SPBF              layer 1: X[lm][n] = sum_b Y_lm R_l                                       k_scatter_a*
+//                     layers 2-3: P[li][ly][n] = sum_b Y_ly R_l(ly) M_j[li][n],               k_pair_fwd
+//                     A = cg_W^T P (sparse), X = reduce(A)                                     k_lincomb, job GEMM
+//   cp_l product q    Lp = U[g] XL, Rp = V[g] XR (job GEMMs), P = sum cg Lp Rp (product kernel), R_q = reduce(P) (job GEMM)
+//   FCRight2Left      out[f] = nof[f] (left[f] + W[t] right[from])                             k_scale_rows + job GEMM
+//   eq / rho          reduces of (X, R2, R3, R4); EquivariantRMSNorm -> message; rho -> readout kernel
+// Every dense contraction over (source function, destination function, weight tile) connections is one list of tile
+// GEMM jobs on the matrix cores (k_gemm_jobs), forward by destination and reverse by source.
+#include "engine_common.hpp"
+#include "kernels_3l.hpp"
+#include "model_3l.hpp"
+
+namespace grhip {
+
+namespace {
+
+inline int pad_width(int c) { return c <= 16 ? 16 : c <= 32 ? 32 : c <= 64 ? 64 : -1; }
+
+// out[dst][k] (+)= dscale[dst] sum over connections (src, dst, tile) of sum_n W[tile][n][k] in[src][n]; reverse:
+// gin[src][n] += sum over its connections of dscale[dst] sum_k W[tile][n][k] gout[dst][k]   (fused_3l_cpu.h:84-221)
+template<class T> struct DevContract {
+  struct Conn {
+    int src, dst, tile;
+  };
+  DevBuf WF, WT;
+  DevJobs<T> fwd, bwd;
+  int kin = 0, kout = 0, nsrc = 0, ndst = 0;    // padded widths, functions of the source and destination tensors
+  template<class WGet>
+  void build(int nin, int nout, int nt, const std::vector<Conn> &conns, WGet wget, const std::vector<double> &dscale, int nsrc_, int ndst_,
+             const int *drow, const std::string &what)
+  {
+    kin = pad_width(nin);
+    kout = pad_width(nout);
+    nsrc = nsrc_;
+    ndst = ndst_;
+    if (kin < 0 || kout < 0) throw Error("GRACE-3L: " + what + ": channel widths above 64 are not supported by the GPU kernels");
+    std::vector<T> F, Ft;
+    std::vector<double> M((size_t) nin * nout), Mt((size_t) nout * nin);
+    for (int t = 0; t < nt; t++) {
+      for (int n = 0; n < nin; n++)
+        for (int k = 0; k < nout; k++) {
+          const double v = wget(t, n, k);
+          M[(size_t) n * nout + k] = v;
+          Mt[(size_t) k * nin + n] = v;
+        }
+      pack_fragments<T>(M, nin, nout, kin, kout, F);
+      pack_fragments<T>(Mt, nout, nin, kout, kin, Ft);
+    }
+    upload_vec(WF, F);
+    upload_vec(WT, Ft);
+    std::vector<std::vector<int>> by_dst(ndst), by_src(nsrc);
+    for (size_t c = 0; c < conns.size(); c++) {
+      if (conns[c].src < 0 || conns[c].src >= nsrc || conns[c].dst < 0 || conns[c].dst >= ndst || conns[c].tile < 0 || conns[c].tile >= nt)
+        throw Error("GRACE-3L: " + what + ": connection index out of range");
+      by_dst[conns[c].dst].push_back((int) c);
+      by_src[conns[c].src].push_back((int) c);
+    }
+    auto sc = [&](int d) { return dscale.empty() ? 1.0 : dscale[d]; };
+    typename DevJobs<T>::Host hf, hb;
+    for (int d = 0; d < ndst; d++) {
+      if (by_dst[d].empty()) continue;
+      hf.job(d, sc(d));
+      for (int c : by_dst[d]) hf.seg(0, conns[c].src, conns[c].tile, 1.0);
+      hf.end_job();
+    }
+    for (int s = 0; s < nsrc; s++) {
+      if (by_src[s].empty()) continue;
+      hb.job(s, 1.0);
+      for (int c : by_src[s]) hb.seg(0, conns[c].dst, conns[c].tile, sc(conns[c].dst));
+      hb.end_job();
+    }
+    fwd.build(hf, WF.as<T>(), WF.as<T>());
+    bwd.build(hb, WT.as<T>(), WT.as<T>());
+    fwd.set_rows(drow);
+    bwd.set_rows(drow);
+  }
+};
+
+// sparse matrix in CSR form on the device (k_lincomb)
+struct DevCsr {
+  DevBuf off, idx, val;
+  int nrow = 0, ncol = 0;
+  void build(int nrow_, int ncol_, const std::vector<int> &row, const std::vector<int> &col, const std::vector<double> &v)
+  {
+    nrow = nrow_;
+    ncol = ncol_;
+    std::vector<int> o(nrow + 1, 0), ix(row.size());
+    std::vector<double> vv(row.size());
+    for (int r : row) o[r + 1]++;
+    for (int r = 0; r < nrow; r++) o[r + 1] += o[r];
+    std::vector<int> pos(o.begin(), o.end() - 1);
+    for (size_t t = 0; t < row.size(); t++) {
+      const int q = pos[row[t]]++;
+      ix[q] = col[t];
+      vv[q] = v[t];
+    }
+    if (ix.empty()) { ix.push_back(0); vv.push_back(0.0); }
+    upload_vec(off, o);
+    upload_vec(idx, ix);
+    upload_vec(val, vv);
+  }
+};
+
+// a per-atom tensor [atom][nf][w]
+struct Ten {
+  DevBuf buf;
+  int nf = 0, w = 0;
+  size_t bytes(size_t na, size_t s) const { return na * nf * w * s; }
+};
+
+template<class T> struct ProdStage {
+  DevContract<T> U, V, red;
+  DevProd cp;
+  int nfunc = 0, rankP = 0;
+  bool jit = false;
+};
+
+template<class T> struct FcStage {
+  DevContract<T> right;
+  DevBuf nof;
+  int nf = 0;
+};
+
+template<class T> struct Layer3 {
+  bool equiv = false, has_eq = false;
+  int C = 0, CP = 0;                  // radial channels and their padded width
+  DevRadial<T> rad;
+  DevBuf fac;
+  // equivariant SPBF
+  int nlmi = 0, nfA = 0;
+  DevBuf zproj, mask;
+  DevCsr cg, cgt;                     // A = cg P (rows: A functions), gP = cgt gA (rows: pair functions slot * nlm + lm)
+  DevContract<T> redA;
+  ProdStage<T> p2, p3, p4;
+  FcStage<T> fa, fb;
+  std::vector<std::unique_ptr<DevContract<T>>> eq;    // sources X, R2, R3, R4
+  DevBuf eq_dw, eq_mask, eq_aff, eq_grp;
+  EqNormDev eqn{};
+  DevReduce<T> rho;
+  // forward tensors kept for the reverse
+  DevBuf R, dR;
+  Ten X, L2, R2p, L3, R3p, L4, R4p, EQ, I;
+  DevBuf rho_raw, grho;
+  int nR2 = 0, nR3 = 0, nR4 = 0, wR = 0;    // functions of the product reduces, their common padded width
+};
+
+template<class T> class Engine3L final : public EngineBase {
+ public:
+  Engine3L(std::shared_ptr<const Model3L> m, int ntypes, const std::vector<int> &type2mu, int device) :
+      EngineBase(device, "GRACE-3L", ntypes, type2mu, m->n_elements), model_(std::move(m))
+  {
+    this->template probe_mfma<T>();
+    build();
+  }
+  int layers() const override { return 3; }
+  void run(const RunFlags &fl) override;
+  void debug_radial(int, const double *, const int *, double *, double *) override
+  {
+    throw Error("GRACE-3L: debug_radial is available for GRACE-1L engines");
+  }
+
+ private:
+  std::shared_ptr<const Model3L> model_;
+  int lmax_ = 0, nl_ = 0, nlm_ = 0, nel_ = 0, nrho_ = 0;
+  ShCoef sh_{};
+  Layer3<T> L_[3];
+  DevBuf shift_, eW0_, eW1_, escale_[3], sink_, emi_, YG_;
+  Energy3Dev en_{};
+  // scratch shared by the layers (largest size over the layers): temporaries of the forward pass and all adjoints
+  DevBuf M_, gM_, pairP_, gpairP_, A_, gA_, P_, gP_, R2_, R3_, R4_, FA_, FB_, gX_, gR2_, gR3_, gR4_, gFA_, gFB_, gLp_, gRp_, gEQ_;
+
+  void build();
+  void build_layer(int k);
+  void gemm(DevJobs<T> &J, int kin, int kout, const T *X, int nfx, T *out, int nfo, int accumulate)
+  {
+    EngineBase::launch_gemm<T>(J, kin / 16, kin / 16, kout / 16, X, nfx, X, nfx, out, nfo, accumulate, tiles_.as<int>(), ntiles_);
+  }
+  void cfwd(DevContract<T> &c, const T *X, T *out, int accumulate) { gemm(c.fwd, c.kin, c.kout, X, c.nsrc, out, c.ndst, accumulate); }
+  void cbwd(DevContract<T> &c, const T *gout, T *gX, int accumulate) { gemm(c.bwd, c.kout, c.kin, gout, c.ndst, gX, c.nsrc, accumulate); }
+  void zero(void *p, size_t bytes) { if (bytes) HIP_CHECK(hipMemsetAsync(p, 0, bytes, stream_)); }
+  void couple_fwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, T *out);
+  void couple_bwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, const T *g, T *gL, T *gR);
+  void scale_rows(const T *in, const DevBuf &s, T *out, int nf, int w, int accumulate)
+  {
+    const long long tot = (long long) n_ * nf * w;
+    if (tot == 0) return;
+    hipLaunchKernelGGL(k_scale_rows<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, in, s.as<T>(), out, n_, nf, w, accumulate);
+  }
+  void layer_forward(int k, bool forces, int yw);
+  void layer_backward(int k, int yw);
+  std::string tg(int k, const char *name) { return std::string(name) + "_L" + std::to_string(k + 1); }
+};
+
+template<class T> void Engine3L<T>::build()
+{
+  const Model3L &m = *model_;
+  lmax_ = m.lmax;
+  if (lmax_ > kKernMaxL) throw Error("GRACE-3L: lmax > " + std::to_string(kKernMaxL) + " not supported");
+  nl_ = lmax_ + 1;
+  nlm_ = nl_ * nl_;
+  nel_ = m.n_elements;
+  nrho_ = m.rho_width;
+  std::memset(&sh_, 0, sizeof(sh_));
+  sh_.lmax = lmax_;
+  for (int l = 2; l <= lmax_; l++) {
+    for (int mm = 0; mm < l - 1; mm++) {
+      const double l2 = l * l, m2 = mm * mm, lm1 = l - 1;
+      sh_.a[l * (l + 1) / 2 + mm] = std::sqrt((4.0 * l2 - 1.0) / (l2 - m2));
+      sh_.b[l * (l + 1) / 2 + mm] = -std::sqrt((lm1 * lm1 - m2) / (4.0 * lm1 * lm1 - 1.0));
+    }
+    sh_.c[l] = -std::sqrt(1.0 + 0.5 / l);
+    sh_.d[l] = std::sqrt(2.0 * l + 1.0);
+  }
+  {
+    std::vector<double> cut((size_t) nel_ * nel_);
+    for (int a = 0; a < nel_; a++)
+      for (int b = 0; b < nel_; b++) cut[(size_t) a * nel_ + b] = m.pair_cutoff(a, b);
+    set_cutoffs(cut);
+  }
+  upload_vec(shift_, m.shift_values);
+  sink_.ensure(64);
+  for (int k = 0; k < 3; k++) build_layer(k);
+  for (int k = 0; k < 2; k++) {
+    const Layer3<T> &a = L_[k], &b = L_[k + 1];
+    if (a.I.nf != b.nlmi || a.eqn.Creal != b.C) throw Error("GRACE-3L: the message of layer " + std::to_string(k + 1) + " does not fit the next SPBF");
+  }
+  // ---- readout: 2-layer MLP on the summed normalised densities (fused_3l.cpp:833-843)
+  const auto &e = m.energy_mlp.layers;
+  if (e.size() != 2 || e[0].n_in != nrho_ - 1 || e[1].n_out != 1)
+    throw Error("GRACE-3L: the GPU readout implements a 2-layer energy MLP on rho[1:]");
+  for (const auto &b : m.energy_mlp.bias)
+    if (!b.empty()) throw Error("GRACE-3L: a bias in the energy MLP is not supported");
+  if (nrho_ > 256 || e[0].n_out > 1024) throw Error("GRACE-3L: energy MLP too wide for the readout kernel");
+  upload_vec(eW0_, e[0].W);
+  upload_vec(eW1_, e[1].W);
+  en_.W0 = eW0_.as<double>();
+  en_.W1 = eW1_.as<double>();
+  en_.norm0 = e[0].norm;
+  en_.norm1 = e[1].norm;
+  en_.nin = e[0].n_in;
+  en_.nh = e[0].n_out;
+  en_.act = m.energy_mlp_activation;
+  en_.nrho = nrho_;
+  en_.out_scale = m.output_scale;
+  en_.eps = Model3L::rms_norm_eps;
+  en_.shift = shift_.as<double>();
+  for (int k = 0; k < 3; k++) {
+    const auto &r = Model3L::by_name(m.rmsnorm, "rho" + std::to_string(k + 1) + "_norm");
+    upload_vec(escale_[k], r.scale);
+    en_.scale[k] = escale_[k].as<double>();
+    en_.type[k] = r.type;
+  }
+}
+
+template<class T> void Engine3L<T>::build_layer(int k)
+{
+  const Model3L &m = *model_;
+  Layer3<T> &L = L_[k];
+  const std::string ks = std::to_string(k + 1), K = "A" + ks;
+  const Model3L::Spbf &sp = Model3L::by_name(m.spbf, K);
+  L.equiv = sp.equivariant;
+  L.C = sp.n_rad_max;
+  L.CP = pad_width(L.C);
+  if (L.CP < 0) throw Error("GRACE-3L: more than 64 radial channels are not supported by the GPU kernels");
+  for (int lm = 0; lm < nlm_; lm++) {
+    int l = 0;
+    while ((l + 1) * (l + 1) <= lm) l++;
+    if (sp.l_tile[lm] != l) throw Error("GRACE-3L: " + K + "_l_tile is not the l of each (l, m) function; not supported by the GPU kernels");
+  }
+  // ---- radial MLP; fac[mu_j][n] = inv_avg (z_tr[mu_j][n] in layer 1): fused_3l.cpp:441-460
+  const int ne = m.embedding_size;
+  L.rad.build_species(sp.mlp.layers, sp.mlp.bias, m.chem_embedding, ne, m.nradbase, sp.p, L.C, L.CP, nl_, nel_, drow_, "GRACE-3L");
+  auto species_table = [&](const std::vector<double> &W, double norm) {
+    std::vector<double> z((size_t) nel_ * L.C);
+    for (int mu = 0; mu < nel_; mu++)
+      for (int n = 0; n < L.C; n++) {
+        double v = 0.0;
+        for (int e = 0; e < ne; e++) v += m.chem_embedding[(size_t) mu * ne + e] * W[(size_t) e * L.C + n];
+        z[(size_t) mu * L.C + n] = v * norm;
+      }
+    return z;
+  };
+  {
+    std::vector<T> fac((size_t) nel_ * L.CP, (T) 0);
+    std::vector<double> ztr;
+    if (!L.equiv) ztr = species_table(sp.lin_transform_W, sp.lin_transform_norm);
+    for (int mu = 0; mu < nel_; mu++)
+      for (int n = 0; n < L.C; n++) fac[(size_t) mu * L.CP + n] = (T) (sp.inv_avg_n_neigh * (L.equiv ? 1.0 : ztr[(size_t) mu * L.C + n]));
+    upload_vec(L.fac, fac);
+  }
+  typedef typename DevContract<T>::Conn Conn;
+  // a reduce instruction as a contraction; W: [n_out][n_in][w_shape], not element dependent
+  auto instr_contract = [&](DevContract<T> &c, const Model3L::Reduce &r, const Model3L::Instr &ins, int nsrc, const std::string &what) {
+    if (r.elem_dep) throw Error("GRACE-3L: " + what + ": element-dependent weights are supported for the rho reduces only");
+    std::vector<Conn> conns;
+    for (size_t q = 0; q < ins.collect_ind.size(); q++) conns.push_back({ins.collect_ind[q], r.only_invar ? 0 : ins.total_sum_ind[q], ins.w_l_tile[q]});
+    c.build(ins.n_in, r.n_out, ins.w_shape, conns,
+            [&](int t, int n, int kk) { return ins.norm * ins.W[((size_t) kk * ins.n_in + n) * ins.w_shape + t]; }, r.norm_map, nsrc, r.nfo(), drow_, what);
+  };
+  L.X.nf = nlm_;
+  if (L.equiv) {
+    L.nlmi = sp.n_lm_ind;
+    L.nfA = sp.nfunc;
+    {
+      const std::vector<double> zp = species_table(sp.chem_linear_W, sp.chem_linear_norm);
+      std::vector<T> z((size_t) nel_ * L.CP, (T) 0), mk(sp.chem_l0_mask.begin(), sp.chem_l0_mask.end());
+      for (int mu = 0; mu < nel_; mu++)
+        for (int n = 0; n < L.C; n++) z[(size_t) mu * L.CP + n] = (T) zp[(size_t) mu * L.C + n];
+      upload_vec(L.zproj, z);
+      upload_vec(L.mask, mk);
+    }
+    // cg_W rows p = ly * nlmi + li (fused_3l.cpp:523-549); the pair tensor of k_pair_fwd has functions li * nlm + ly
+    std::vector<int> rf, cf;
+    std::vector<double> vv;
+    const int np = nlm_ * L.nlmi;
+    for (int p = 0; p < np; p++)
+      for (int f = 0; f < L.nfA; f++) {
+        const double v = sp.cg_W[(size_t) p * L.nfA + f];
+        if (v == 0.0) continue;
+        const int ly = p / L.nlmi, li = p % L.nlmi;
+        rf.push_back(f);
+        cf.push_back(li * nlm_ + ly);
+        vv.push_back(v);
+      }
+    L.cg.build(L.nfA, np, rf, cf, vv);
+    L.cgt.build(np, L.nfA, cf, rf, vv);
+    const Model3L::Reduce &r = Model3L::by_name(m.reduce, K + "_red");
+    if (r.instr.size() != 1 || r.only_invar) throw Error("GRACE-3L: " + K + "_red must be one instruction on " + K);
+    instr_contract(L.redA, r, r.instr[0], L.nfA, K + "_red");
+    L.X.nf = r.nfo();
+    L.X.w = L.redA.kout;
+  } else
+    L.X.w = L.CP;
+  const int nX = L.X.nf;
+  // ---- cp_l products with their reduces
+  auto build_prod = [&](ProdStage<T> &P, const std::string &q, int nfl, int wl, int nfr, int wr, Ten &Lp, Ten &Rp, int &nfred) {
+    const Model3L::Cpl &c = Model3L::by_name(m.prod, K + "_" + q);
+    const Model3L::Reduce &r = Model3L::by_name(m.reduce, K + "_" + q + "_red");
+    if (r.instr.size() != 1 || r.only_invar) throw Error("GRACE-3L: " + r.name + " must be one instruction on the product");
+    if (pad_width(c.n_left) != wl || pad_width(c.n_right) != wr) throw Error("GRACE-3L: " + c.name + ": input widths");
+    std::vector<Conn> cl, cr;
+    for (int f = 0; f < nfl; f++) cl.push_back({f, f, c.group_left[f]});
+    for (int f = 0; f < nfr; f++) cr.push_back({f, f, c.group_right[f]});
+    P.U.build(c.n_left, c.rank, c.n_groups_left, cl, [&](int t, int n, int kk) { return c.norm_u * c.U[((size_t) t * c.rank + kk) * c.n_left + n]; }, {}, nfl,
+              nfl, drow_, c.name + "_U");
+    P.V.build(c.n_right, c.rank, c.n_groups_right, cr, [&](int t, int n, int kk) { return c.norm_v * c.V[((size_t) t * c.rank + kk) * c.n_right + n]; }, {},
+              nfr, nfr, drow_, c.name + "_V");
+    P.nfunc = c.nfunc;
+    P.rankP = P.U.kout;
+    const HostProd h = grhip::build_prod(c.cg, std::vector<char>(c.nfunc, 1), nfl, nfr);
+    P.cp.build(h);
+    // the specialised straight-line kernels pay off (and compile in seconds) for the shorter term lists
+    if (h.terms.size() <= 1500)
+      jit_compile_product((c.name + "_cp").c_str(), h.terms, nfl, nfr, c.nfunc, false, P.rankP, sizeof(T) == 4, arch_, P.cp.jit, P.cp.jit_note);
+    P.jit = P.cp.jit.ok();
+    instr_contract(P.red, r, r.instr[0], c.nfunc, r.name);
+    Lp.nf = nfl;
+    Rp.nf = nfr;
+    Lp.w = Rp.w = P.rankP;
+    nfred = r.nfo();
+    if (L.wR == 0) L.wR = P.red.kout;
+    if (P.red.kout != L.wR) throw Error("GRACE-3L: the product reduces of a layer must have one channel width");
+  };
+  auto build_fc = [&](FcStage<T> &F, const std::string &name) {
+    const Model3L::Fc &f = Model3L::by_name(m.fc, name);
+    if (f.n_funcs_left != L.nR2 || pad_width(f.n_out) != L.wR || pad_width(f.n_in_right) != L.X.w) throw Error("GRACE-3L: FC " + name + ": shapes");
+    std::vector<Conn> conns;
+    for (size_t q = 0; q < f.collect_from.size(); q++) conns.push_back({f.collect_from[q], f.collect_to[q], f.w_tile_right[q]});
+    F.right.build(f.n_in_right, f.n_out, f.w_shape_right, conns,
+                  [&](int t, int n, int kk) { return f.norm_right * f.w_right[((size_t) kk * f.n_in_right + n) * f.w_shape_right + t]; }, f.norm_out_factor,
+                  nX, f.n_funcs_left, drow_, "fc_" + name);
+    F.nf = f.n_funcs_left;
+    upload_vec(F.nof, std::vector<T>(f.norm_out_factor.begin(), f.norm_out_factor.end()));
+  };
+  build_prod(L.p2, "2", nX, L.X.w, nX, L.X.w, L.L2, L.R2p, L.nR2);
+  build_fc(L.fa, K + "_2a");
+  build_prod(L.p3, "3", L.nR2, L.wR, nX, L.X.w, L.L3, L.R3p, L.nR3);
+  build_fc(L.fb, K + "_2b");
+  build_prod(L.p4, "4", L.nR2, L.wR, L.nR2, L.wR, L.L4, L.R4p, L.nR4);
+  // ---- eq (layers 1-2) and rho reduces of (X, R2, R3, R4)
+  const std::string xname = L.equiv ? K + "_red" : K;
+  const std::string srcs[4] = {xname, K + "_2_red", K + "_3_red", K + "_4_red"};
+  const int src_nf[4] = {nX, L.nR2, L.nR3, L.nR4};
+  L.has_eq = k < 2;
+  if (L.has_eq) {
+    const Model3L::Reduce &r = Model3L::by_name(m.reduce, "eq" + ks);
+    if (r.only_invar) throw Error("GRACE-3L: eq" + ks + " is marked invariant");
+    for (int s = 0; s < 4; s++) {
+      L.eq.emplace_back(new DevContract<T>());
+      instr_contract(*L.eq.back(), r, Model3L::by_name(r.instr, srcs[s]), src_nf[s], "eq" + ks);
+    }
+    const Model3L::EqNorm &e = Model3L::by_name(m.eqnorm, "eq" + ks + "_norm");
+    L.EQ.nf = L.I.nf = e.M;
+    L.EQ.w = L.I.w = L.eq[0]->kout;
+    upload_vec(L.eq_dw, e.degree_weights);
+    upload_vec(L.eq_mask, e.l0_mask);
+    upload_vec(L.eq_grp, e.expand_index);
+    std::vector<double> aff((size_t) e.n_groups * L.EQ.w, 0.0);
+    for (int g = 0; g < e.n_groups; g++)
+      for (int n = 0; n < e.n_out; n++) aff[(size_t) g * L.EQ.w + n] = e.affine_weight[(size_t) g * e.n_out + n];
+    upload_vec(L.eq_aff, aff);
+    L.eqn.dw = L.eq_dw.template as<double>();
+    L.eqn.mask = L.eq_mask.template as<double>();
+    L.eqn.aff = L.eq_aff.template as<double>();
+    L.eqn.grp = L.eq_grp.template as<int>();
+    L.eqn.M = e.M;
+    L.eqn.C = L.EQ.w;
+    L.eqn.Creal = e.n_out;
+    L.eqn.center = e.center_l0 ? 1 : 0;
+    L.eqn.eps = e.eps;
+  }
+  {
+    const Model3L::Reduce &r = Model3L::by_name(m.reduce, "rho" + ks);
+    if (!r.only_invar) throw Error("GRACE-3L: rho" + ks + " must be an invariant reduce");
+    if (r.n_out != nrho_) throw Error("GRACE-3L: rho widths differ between the layers");
+    // element-independent weights are replicated per element for the reduce kernel
+    std::vector<std::vector<double>> Wrep(4);
+    std::vector<ReduceSrc> v;
+    for (int s = 0; s < 4; s++) {
+      const Model3L::Instr &ins = Model3L::by_name(r.instr, srcs[s]);
+      const std::vector<double> *W = &ins.W;
+      if (!r.elem_dep) {
+        for (int mu = 0; mu < nel_; mu++) Wrep[s].insert(Wrep[s].end(), ins.W.begin(), ins.W.end());
+        W = &Wrep[s];
+      }
+      v.push_back({W, ins.norm, ins.n_in, ins.w_shape, &ins.collect_ind, &ins.w_l_tile, nullptr, src_nf[s], s == 0 ? L.X.w : L.wR});
+    }
+    L.rho.build(v, nel_, nrho_, -1, nrho_, 0, drow_);
+  }
+}
+
+template<class T> void Engine3L<T>::couple_fwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, T *out)
+{
+  const int n = n_, KP = p.rankP;
+  int one = 1, nat = n;
+  if (p.jit) {
+    void *args[] = {(void *) &Lp, (void *) &Rp, (void *) &out, (void *) &nat, (void *) &one};
+    const long long cols = (long long) n * KP;
+    HIP_CHECK(hipModuleLaunchKernel(p.cp.jit.fwd, (unsigned) ((cols + 255) / 256), 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+    return;
+  }
+  const int AT = std::max(1, 256 / KP);
+  hipLaunchKernelGGL(k_prod_fwd<T>, dim3(p.cp.d.nout * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, p.cp.d, Lp, Rp, out, n, KP, nfl, nfr);
+}
+
+// gL, gR are accumulated into (zeroed by the caller)
+template<class T> void Engine3L<T>::couple_bwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, const T *g, T *gL, T *gR)
+{
+  const int n = n_, KP = p.rankP;
+  int one = 1, nat = n, acc = 1;
+  if (p.jit) {
+    void *args[] = {(void *) &Lp, (void *) &Rp, (void *) &g, (void *) &gL, (void *) &gR, (void *) &acc, (void *) &acc, (void *) &nat, (void *) &one};
+    const long long cols = (long long) n * KP;
+    HIP_CHECK(hipModuleLaunchKernel(p.cp.jit.bwd, (unsigned) ((cols + 255) / 256), 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+    return;
+  }
+  const int AT = std::max(1, 256 / KP);
+  hipLaunchKernelGGL(k_prod_bwd<T>, dim3(p.cp.d.nleft * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, p.cp.d, 0, Rp, g, gL, n, KP, nfr, nfl);
+  hipLaunchKernelGGL(k_prod_bwd<T>, dim3(p.cp.d.nright * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, p.cp.d, 1, Lp, g, gR, n, KP, nfl, nfr);
+}
+
+#define GR_PAIR1(K_, N_, grid_, block_, lds_, ...)                                                                       \
+  {                                                                                                                      \
+    auto kern = K_<T, N_>;                                                                                               \
+    if (lds_ > 48 * 1024)                                                                                                \
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_)); \
+    hipLaunchKernelGGL(kern, grid_, block_, lds_, __VA_ARGS__);                                                          \
+  }
+#define GR_PAIR(K_, ...)                                     \
+  switch (nl_) {                                             \
+    case 1: GR_PAIR1(K_, 1, __VA_ARGS__) break;              \
+    case 2: GR_PAIR1(K_, 4, __VA_ARGS__) break;              \
+    case 3: GR_PAIR1(K_, 9, __VA_ARGS__) break;              \
+    case 4: GR_PAIR1(K_, 16, __VA_ARGS__) break;             \
+    case 5: GR_PAIR1(K_, 25, __VA_ARGS__) break;             \
+    case 6: GR_PAIR1(K_, 36, __VA_ARGS__) break;             \
+    default: GR_PAIR1(K_, 49, __VA_ARGS__) break;            \
+  }
+
+template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
+{
+  Layer3<T> &L = L_[k];
+  const int n = n_;
+  const size_t na = (size_t) n, ecap = (size_t) std::max<int64_t>(nb_, 1), s = sizeof(T);
+  const long long *n_edges = eoff_.as<long long>() + n;
+  L.R.ensure(ecap * L.rad.noutp * s);
+  L.dR.ensure(ecap * L.rad.noutp * s);
+  stage(tg(k, "radial").c_str(), [&] {
+    L.rad.launch(stream_, ncu_, L.fac.template as<T>(), 0, -1, xr_.as<double>(), emu_.as<int>(), L.R.template as<T>(), L.dR.template as<T>(), n_edges,
+                 emi_.as<int>());
+  });
+  L.X.buf.ensure(L.X.bytes(na, s));
+  T *X = L.X.buf.template as<T>();
+  if (!L.equiv) {
+    ScatterArgs<T> sa{};
+    sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = L.R.template as<T>(); sa.A = X;
+    sa.a0 = 0; sa.C = L.CP; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = L.rad.noutp; sa.sh = sh_;
+    stage(tg(k, "scatter_A").c_str(), [&] { launch_scatter<T>(sa, n, lmax_); });
+  } else {
+    const Layer3<T> &Lm = L_[k - 1];
+    const int npf = L.nlmi * nlm_;
+    M_.ensure(na * L.nlmi * L.CP * s);
+    pairP_.ensure(na * npf * L.CP * s);
+    A_.ensure(na * L.nfA * L.CP * s);
+    stage(tg(k, "message").c_str(), [&] {
+      const long long tot = (long long) n * L.nlmi * L.CP;
+      hipLaunchKernelGGL(k_message<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, Lm.I.buf.template as<T>(), mu_.as<int>(),
+                         L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n, L.nlmi, L.CP);
+    });
+    const int spb = std::max(1, std::min(L.nlmi, 1024 / L.CP)), ngrp = (L.nlmi + spb - 1) / spb;
+    stage(tg(k, "pair_fwd").c_str(), [&] {
+      const size_t lds = (size_t) kPairChunk * (spb * L.CP + L.rad.noutp) * s;
+      GR_PAIR(k_pair_fwd, dim3(n, ngrp), dim3(spb * L.CP), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), L.R.template as<T>(),
+              (const T *) M_.as<T>(), pairP_.as<T>(), L.nlmi, L.CP, nl_, L.rad.noutp, yw, sink_.as<T>());
+    });
+    stage(tg(k, "couple_YI").c_str(), [&] {
+      hipLaunchKernelGGL(k_lincomb<T>, dim3(n, (L.nfA * L.CP + 255) / 256), dim3(256), 0, stream_, L.cg.off.template as<int>(), L.cg.idx.template as<int>(),
+                         L.cg.val.template as<double>(), (const T *) pairP_.as<T>(), A_.as<T>(), npf, L.nfA, L.CP);
+    });
+    stage(tg(k, "reduce_A").c_str(), [&] {
+      zero(X, L.X.bytes(na, s));
+      cfwd(L.redA, A_.as<T>(), X, 1);
+    });
+  }
+  // ---- chain (fused_3l.cpp:970-990)
+  const int nX = L.X.nf, wX = L.X.w, wR = L.wR;
+  size_t maxP = 0;
+  for (ProdStage<T> *p : {&L.p2, &L.p3, &L.p4}) maxP = std::max(maxP, (size_t) p->nfunc * p->rankP);
+  P_.ensure(na * maxP * s);
+  R2_.ensure(na * L.nR2 * wR * s);
+  R3_.ensure(na * L.nR3 * wR * s);
+  R4_.ensure(na * L.nR4 * wR * s);
+  FA_.ensure(na * L.nR2 * wR * s);
+  FB_.ensure(na * L.nR2 * wR * s);
+  for (Ten *t : {&L.L2, &L.R2p, &L.L3, &L.R3p, &L.L4, &L.R4p}) t->buf.ensure(t->bytes(na, s));
+  T *P = P_.as<T>(), *R2 = R2_.as<T>(), *R3 = R3_.as<T>(), *R4 = R4_.as<T>(), *FA = FA_.as<T>(), *FB = FB_.as<T>();
+  auto prod = [&](const char *name, ProdStage<T> &p, const T *XL, const T *XR, Ten &Lp, Ten &Rp, T *Rout, int nfred) {
+    T *lp = Lp.buf.template as<T>(), *rp = Rp.buf.template as<T>();
+    stage(tg(k, (std::string("proj_") + name).c_str()).c_str(), [&] {
+      cfwd(p.U, XL, lp, 0);
+      cfwd(p.V, XR, rp, 0);
+    });
+    stage(tg(k, (std::string("couple_") + name).c_str()).c_str(), [&] { couple_fwd(p, lp, Lp.nf, rp, Rp.nf, P); });
+    stage(tg(k, (std::string("reduce_") + name).c_str()).c_str(), [&] {
+      zero(Rout, na * nfred * wR * s);
+      cfwd(p.red, P, Rout, 1);
+    });
+  };
+  auto fc = [&](const char *name, FcStage<T> &F, T *out) {
+    stage(tg(k, name).c_str(), [&] {
+      scale_rows(R2, F.nof, out, F.nf, wR, 0);
+      cfwd(F.right, X, out, 1);
+    });
+  };
+  prod("2", L.p2, X, X, L.L2, L.R2p, R2, L.nR2);
+  fc("fc_2a", L.fa, FA);
+  prod("3", L.p3, FA, X, L.L3, L.R3p, R3, L.nR3);
+  fc("fc_2b", L.fb, FB);
+  prod("4", L.p4, FB, FB, L.L4, L.R4p, R4, L.nR4);
+  const T *srcs[4] = {X, R2, R3, R4};
+  if (L.has_eq) {
+    L.EQ.buf.ensure(L.EQ.bytes(na, s));
+    L.I.buf.ensure(L.I.bytes(na, s));
+    stage(tg(k, "reduce_eq").c_str(), [&] {
+      zero(L.EQ.buf.p, L.EQ.bytes(na, s));
+      for (int q = 0; q < 4; q++) cfwd(*L.eq[q], srcs[q], L.EQ.buf.template as<T>(), 1);
+    });
+    stage(tg(k, "eqnorm").c_str(), [&] {
+      hipLaunchKernelGGL(k_eqnorm<T>, dim3(n), dim3(256), (size_t) L.eqn.M * sizeof(double), stream_, L.eqn, (const T *) L.EQ.buf.template as<T>(),
+                         L.I.buf.template as<T>(), (const T *) nullptr, (T *) nullptr, 0);
+    });
+  }
+  L.rho_raw.ensure(na * nrho_ * sizeof(double));
+  L.grho.ensure(na * nrho_ * sizeof(double));
+  (void) nX;
+  stage(tg(k, "reduce_rho").c_str(), [&] {
+    const int *tiles = tiles_.as<int>();
+#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(ntiles_), dim3(256), 0, stream_, L.rho.d, mu_.as<int>(), tiles, srcs[0], srcs[1], \
+                                          srcs[2], srcs[3], L.rho_raw.template as<double>())
+    switch ((wX / 16) * 10 + wR / 16) {
+      case 11: GR_RED(1, 1); break;
+      case 12: GR_RED(1, 2); break;
+      case 14: GR_RED(1, 4); break;
+      case 21: GR_RED(2, 1); break;
+      case 22: GR_RED(2, 2); break;
+      case 24: GR_RED(2, 4); break;
+      case 41: GR_RED(4, 1); break;
+      case 42: GR_RED(4, 2); break;
+      case 44: GR_RED(4, 4); break;
+      default: throw Error("unsupported channel widths");
+    }
+#undef GR_RED
+  });
+  (void) forces;
+}
+
+// Reverse of layer k.  In: L.grho (adjoint of the raw density) and, for layers 1-2, gM_ (adjoint of the message this
+// layer sent: dE/dI, accumulated by the pair kernel of the layer above).  Out: forces of the layer's bonds and, for
+// layers 2-3, gM_ overwritten with the adjoint of the message of the layer below.
+template<class T> void Engine3L<T>::layer_backward(int k, int yw)
+{
+  Layer3<T> &L = L_[k];
+  const int n = n_;
+  const size_t na = (size_t) n, s = sizeof(T);
+  const int nX = L.X.nf, wX = L.X.w, wR = L.wR;
+
+  size_t maxP = 0, maxLp = 0;
+  for (ProdStage<T> *p : {&L.p2, &L.p3, &L.p4}) maxP = std::max(maxP, (size_t) p->nfunc * p->rankP);
+  for (Ten *t : {&L.L2, &L.R2p, &L.L3, &L.R3p, &L.L4, &L.R4p}) maxLp = std::max(maxLp, (size_t) t->nf * t->w);
+  gP_.ensure(na * maxP * s);
+  gLp_.ensure(na * maxLp * s);
+  gRp_.ensure(na * maxLp * s);
+  gX_.ensure(na * nX * wX * s);
+  gR2_.ensure(na * L.nR2 * wR * s);
+  gR3_.ensure(na * L.nR3 * wR * s);
+  gR4_.ensure(na * L.nR4 * wR * s);
+  gFA_.ensure(na * L.nR2 * wR * s);
+  gFB_.ensure(na * L.nR2 * wR * s);
+  T *gP = gP_.as<T>(), *gLp = gLp_.as<T>(), *gRp = gRp_.as<T>(), *gX = gX_.as<T>(), *gR2 = gR2_.as<T>(), *gR3 = gR3_.as<T>(), *gR4 = gR4_.as<T>(),
+    *gFA = gFA_.as<T>(), *gFB = gFB_.as<T>();
+  T *gsrc[4] = {gX, gR2, gR3, gR4};
+  stage(tg(k, "zero_grads").c_str(), [&] {
+    zero(gX, na * nX * wX * s);
+    zero(gR2, na * L.nR2 * wR * s);
+    zero(gR3, na * L.nR3 * wR * s);
+    zero(gR4, na * L.nR4 * wR * s);
+    zero(gFA, na * L.nR2 * wR * s);
+    zero(gFB, na * L.nR2 * wR * s);
+  });
+  if (L.has_eq) {
+    gEQ_.ensure(L.EQ.bytes(na, s));
+    stage(tg(k, "eqnorm_bwd").c_str(), [&] {
+      hipLaunchKernelGGL(k_eqnorm<T>, dim3(n), dim3(256), (size_t) L.eqn.M * sizeof(double), stream_, L.eqn, (const T *) L.EQ.buf.template as<T>(), (T *) nullptr,
+                         (const T *) gM_.as<T>(), gEQ_.as<T>(), 0);
+    });
+    stage(tg(k, "reduce_eq_bwd").c_str(), [&] {
+      for (int q = 0; q < 4; q++) cbwd(*L.eq[q], gEQ_.as<T>(), gsrc[q], 1);
+    });
+  }
+  stage(tg(k, "reduce_rho_bwd").c_str(), [&] {
+    if (L.rho.njobs)
+      hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, L.rho.njobs), dim3(64), 0, stream_, L.rho.d, mu_.as<int>(), tiles_.as<int>(),
+                         (const double *) L.grho.template as<double>(), gX, gR2, gR3, gR4);
+  });
+  // gXL / gXR: where the adjoints of the product's inputs are added
+  auto prod_bwd = [&](const char *name, ProdStage<T> &p, Ten &Lp, Ten &Rp, const T *gR, T *gXL, T *gXR) {
+    const T *lp = Lp.buf.template as<T>(), *rp = Rp.buf.template as<T>();
+    stage(tg(k, (std::string("reduce_") + name + "_bwd").c_str()).c_str(), [&] {
+      zero(gP, na * p.nfunc * p.rankP * s);
+      cbwd(p.red, gR, gP, 1);
+    });
+    stage(tg(k, (std::string("couple_") + name + "_bwd").c_str()).c_str(), [&] {
+      zero(gLp, Lp.bytes(na, s));
+      zero(gRp, Rp.bytes(na, s));
+      couple_bwd(p, lp, Lp.nf, rp, Rp.nf, gP, gLp, gRp);
+    });
+    stage(tg(k, (std::string("proj_") + name + "_bwd").c_str()).c_str(), [&] {
+      cbwd(p.U, gLp, gXL, 1);
+      cbwd(p.V, gRp, gXR, 1);
+    });
+  };
+  auto fc_bwd = [&](const char *name, FcStage<T> &F, const T *gout) {
+    stage(tg(k, name).c_str(), [&] {
+      scale_rows(gout, F.nof, gR2, F.nf, wR, 1);
+      cbwd(F.right, gout, gX, 1);
+    });
+  };
+  prod_bwd("4", L.p4, L.L4, L.R4p, gR4, gFB, gFB);
+  fc_bwd("fc_2b_bwd", L.fb, gFB);
+  prod_bwd("3", L.p3, L.L3, L.R3p, gR3, gFA, gX);
+  fc_bwd("fc_2a_bwd", L.fa, gFA);
+  prod_bwd("2", L.p2, L.L2, L.R2p, gR2, gX, gX);
+  if (!L.equiv) {
+    BondBwdArgs<T> ba{};
+    ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
+    ba.Rz = L.R.template as<T>(); ba.dRz = L.dR.template as<T>(); ba.gA = gX;
+    ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
+    ba.a0 = 0; ba.C = L.CP; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = L.rad.noutp; ba.sh = sh_;
+    stage(tg(k, "bond_bwd").c_str(), [&] { launch_bond_bwd<T>(ba, n); });
+    return;
+  }
+  const Layer3<T> &Lm = L_[k - 1];
+  const int npf = L.nlmi * nlm_;
+  gA_.ensure(na * L.nfA * L.CP * s);
+  gpairP_.ensure(na * npf * L.CP * s);
+  M_.ensure(na * L.nlmi * L.CP * s);
+  gM_.ensure(na * L.nlmi * L.CP * s);
+  stage(tg(k, "reduce_A_bwd").c_str(), [&] {
+    zero(gA_.p, na * L.nfA * L.CP * s);
+    cbwd(L.redA, gX, gA_.as<T>(), 1);
+  });
+  stage(tg(k, "couple_YI_bwd").c_str(), [&] {
+    hipLaunchKernelGGL(k_lincomb<T>, dim3(n, (npf * L.CP + 255) / 256), dim3(256), 0, stream_, L.cgt.off.template as<int>(), L.cgt.idx.template as<int>(),
+                       L.cgt.val.template as<double>(), (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP);
+  });
+  stage(tg(k, "message_bwd").c_str(), [&] {
+    const long long tot = (long long) n * L.nlmi * L.CP;
+    hipLaunchKernelGGL(k_message<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, Lm.I.buf.template as<T>(), mu_.as<int>(),
+                       L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n, L.nlmi, L.CP);
+    zero(gM_.p, na * L.nlmi * L.CP * s);
+  });
+  const int spb = std::max(1, std::min(L.nlmi, 1024 / L.CP)), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
+  stage(tg(k, "pair_bwd").c_str(), [&] {
+    const size_t lds = (size_t) kPairChunk * (pthreads + 2 * L.rad.noutp) * s;
+    GR_PAIR(k_pair_bwd, dim3(n, ngrp), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), L.R.template as<T>(),
+            L.dR.template as<T>(), (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(),
+            f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb);
+  });
+  (void) yw;
+}
+
+template<class T> void Engine3L<T>::run(const RunFlags &fl)
+{
+  static_assert(sizeof(T) == 8, "the GRACE-3L engine computes in fp64");
+  const int n = n_;
+  if (!begin_pass(fl)) return;
+  const size_t ecap = (size_t) std::max<int64_t>(nb_, 1);
+  const long long *n_edges = eoff_.as<long long>() + n;
+  const bool forces = !fl.energy_only;
+  emi_.ensure(ecap * sizeof(int));
+  stage("edge_center", [&] { hipLaunchKernelGGL(k_edge_center, dim3(n), dim3(64), 0, stream_, eoff_.as<long long>(), mu_.as<int>(), emi_.as<int>()); });
+  const int yw = forces ? 4 * nlm_ : nlm_;    // row of an edge: Y[nlm] and, for forces, G[nlm][3]
+  YG_.ensure(ecap * yw * sizeof(T));
+  stage("sh_edges", [&] {
+    const size_t lds = (size_t) 64 * (yw + 1) * sizeof(T);
+    auto kern = k_sh_edges<T>;
+    if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+    hipLaunchKernelGGL(kern, dim3((unsigned) ((ecap + 63) / 64)), dim3(64), lds, stream_, sh_, rh_.as<double>(), n_edges, nlm_, forces ? 1 : 0,
+                       YG_.as<T>());
+  });
+  for (int k = 0; k < 3; k++) layer_forward(k, forces, yw);
+  stage("energy_mlp", [&] {
+    hipLaunchKernelGGL(k_energy_3l, dim3(n), dim3(64), (size_t) (nrho_ + 2 * en_.nh) * sizeof(double), stream_, en_, mu_.as<int>(),
+                       (const double *) L_[0].rho_raw.template as<double>(), (const double *) L_[1].rho_raw.template as<double>(),
+                       (const double *) L_[2].rho_raw.template as<double>(), L_[0].grho.template as<double>(), L_[1].grho.template as<double>(),
+                       L_[2].grho.template as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0, sid_ptr());
+  });
+  if (!forces) return;
+  for (int k = 2; k >= 0; k--) layer_backward(k, yw);
+}
+
+#undef GR_PAIR
+#undef GR_PAIR1
+
+}    // namespace
+
+std::unique_ptr<Engine> make_engine_3l(std::shared_ptr<const Model3L> model, int ntypes, const std::vector<int> &type2mu, int precision,
+                                       int device)
+{
+  if (precision == 64) return std::make_unique<Engine3L<double>>(std::move(model), ntypes, type2mu, device);
+  if (precision == 32) throw InvalidArgument("GRACE-3L engines compute in fp64 (precision 64)");
+  throw InvalidArgument("precision must be 64 or 32");
+}
+
+}    // namespace grhip

@@ -227,7 +227,8 @@ template<class T> struct DevFc {
 // reference; its spline tables are replaced by the exact network).  Output column l * CP + n of an edge holds
 // R_{n,l}(x) z[mu_j][n] (file order of the last layer: o = n nl + l, libgrace/src/fused_1l.cpp:123).
 template<class T> struct DevRadial {
-  DevBuf w0, w1, w2;
+  DevBuf w0, w1, w2, bias_i, bias_j, bias1;
+  int mode = 0;    // 1: species form (build_species)
   int hb = 4, ks0 = 2, nob = 0, noutp = 0, w2_in_lds = 1, nrb = 0, p = 0, act = 0, CP = 0, nel = 0;
   size_t lds = 0;
   int drow[16];
@@ -277,9 +278,42 @@ template<class T> struct DevRadial {
     w2_in_lds = base + v2.size() * sizeof(T) <= 150 * 1024;
     lds = base + (w2_in_lds ? v2.size() * sizeof(T) : 0);
   }
-  // z: [nel][CP] species weights of the neighbour; e_count < 0: the edge count is read from *n_edges on the device
+  // Species form of GRACE-3L (libgrace/src/fused_3l.cpp:299-346, :462-493): the MLP input is [T_1..T_nrb(2x - 1),
+  // emb(mu_i), emb(mu_j)], hidden layers carry a bias, and the envelope multiplies the output.  The embedding rows of
+  // layer 0 become per-element tables added to its pre-activation: tab_i[mu] = norm0 (b0 + emb[mu] W0[nrb : nrb + ne]),
+  // tab_j[mu] = norm0 emb[mu] W0[nrb + ne : nrb + 2 ne].
+  void build_species(const std::vector<MLPLayer> &mlp, const std::vector<std::vector<double>> &bias, const std::vector<double> &emb, int ne,
+                     int nradbase, int basis_p, int C, int CP_, int nl, int nel_, const int *drow_, const std::string &who)
+  {
+    if (mlp.size() != 3)
+      throw Error(who + ": the GPU radial kernel implements 3-layer radial MLPs (file has " + std::to_string(mlp.size()) + ")");
+    std::vector<MLPLayer> cut = mlp;
+    const int H1 = mlp[0].n_out, H2 = mlp[1].n_out;
+    cut[0].n_in = nradbase;
+    cut[0].W.assign(mlp[0].W.begin(), mlp[0].W.begin() + (size_t) nradbase * H1);
+    build(cut, nradbase, basis_p, 0, C, CP_, nl, nel_, drow_, who);
+    mode = 1;
+    const int HP = hb * 16;
+    std::vector<T> ti((size_t) nel_ * HP, (T) 0), tj((size_t) nel_ * HP, (T) 0), t1((size_t) HP, (T) 0);
+    for (int mu = 0; mu < nel_; mu++)
+      for (int o = 0; o < H1; o++) {
+        double vi = bias.size() > 0 && !bias[0].empty() ? bias[0][o] : 0.0, vj = 0.0;
+        for (int e = 0; e < ne; e++) {
+          const double zz = emb[(size_t) mu * ne + e];
+          vi += zz * mlp[0].W[(size_t) (nradbase + e) * H1 + o];
+          vj += zz * mlp[0].W[(size_t) (nradbase + ne + e) * H1 + o];
+        }
+        ti[(size_t) mu * HP + o] = (T) (mlp[0].norm * vi);
+        tj[(size_t) mu * HP + o] = (T) (mlp[0].norm * vj);
+      }
+    for (int o = 0; o < H2; o++) t1[o] = (T) (bias.size() > 1 && !bias[1].empty() ? mlp[1].norm * bias[1][o] : 0.0);
+    if (bias.size() > 2 && !bias[2].empty()) throw Error(who + ": a bias on the output layer of the radial MLP is not supported");
+    upload_vec(bias_i, ti); upload_vec(bias_j, tj); upload_vec(bias1, t1);
+  }
+  // z: [nel][CP] species weights of the neighbour; e_count < 0: the edge count is read from *n_edges on the device;
+  // emi: element of the central atom of every edge (species form only)
   void launch(hipStream_t stream, int ncu, const T *z, long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
-              const long long *n_edges)
+              const long long *n_edges, const int *emi = nullptr)
   {
     RadialArgs<T> ra{};
     ra.n_edges = n_edges;
@@ -295,8 +329,11 @@ template<class T> struct DevRadial {
     ra.C = CP; ra.nel = nel; ra.act = act;
     ra.w2_in_lds = w2_in_lds;
     for (int q = 0; q < 16; q++) ra.drow[q] = drow[q];
+    ra.emi = emi; ra.bias_i = bias_i.as<T>(); ra.bias_j = bias_j.as<T>(); ra.bias1 = bias1.as<T>();
+    if (mode == 1 && !emi) throw Error("radial kernel: the species form needs the central element of every edge");
     const int threads = hb == 4 ? 512 : 256;
-    auto kern = hb == 4 ? (act == 1 ? k_radial<T, 4, 1> : k_radial<T, 4, 0>) : (act == 1 ? k_radial<T, 8, 1> : k_radial<T, 8, 0>);
+    auto kern = mode == 1 ? (hb == 4 ? k_radial<T, 4, 0, 1> : k_radial<T, 8, 0, 1>)
+                          : hb == 4 ? (act == 1 ? k_radial<T, 4, 1> : k_radial<T, 4, 0>) : (act == 1 ? k_radial<T, 8, 1> : k_radial<T, 8, 0>);
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     hipLaunchKernelGGL(kern, dim3(ncu), dim3(threads), lds, stream, ra);
   }

@@ -262,6 +262,11 @@ template<class T> struct RadialArgs {
   int C, nel, act;            // radial channels, elements, activation (0 SiLU, 1 tanh)
   int w2_in_lds;
   int drow[16];               // accumulator row of (lane / 16, register)
+  // species form (MODE 1 of k_radial): the basis is the bare T_k(2x - 1); layer 0 adds bias_i[element of the central
+  // atom] + bias_j[element of the neighbour], layer 1 adds bias1, and the envelope multiplies the output
+  const int *emi;             // [E] element of the central atom
+  const T *bias_i, *bias_j;   // [nel][HB * 16]
+  const T *bias1;             // [HB * 16]
 };
 
 // reciprocal: hardware estimate + Newton steps (2 in fp64: full precision; 1 in fp32)
@@ -310,7 +315,7 @@ __device__ inline double ipow(double x, int n)
 // Every k-step feeds all row blocks of the value and the tangent stream (2 HB independent accumulator chains).
 // ACT: 0 SiLU, 1 tanh (compile-time: the fp64 tanh is large, and both activations inlined 32 times overflow the
 // instruction cache).
-template<class T, int HB, int ACT> __global__ __launch_bounds__(512) void k_radial(RadialArgs<T> a)
+template<class T, int HB, int ACT, int MODE = 0> __global__ __launch_bounds__(HB <= 4 ? 512 : 256) void k_radial(RadialArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -346,7 +351,7 @@ template<class T, int HB, int ACT> __global__ __launch_bounds__(512) void k_radi
 #pragma unroll
       for (int s = 0; s < kMaxRadBasis / 4; s++) { h0[s] = (T) 0; dh0[s] = (T) 0; }
       for (int k = 0; k < a.nrb; k++) {
-        const double gk = Tc * fc, dgk = dTc * fc + Tc * dfc;
+        const double gk = MODE == 1 ? Tc : Tc * fc, dgk = MODE == 1 ? dTc : dTc * fc + Tc * dfc;
         if ((k & 3) == g) {
 #pragma unroll
           for (int s = 0; s < kMaxRadBasis / 4; s++)
@@ -370,6 +375,14 @@ template<class T, int HB, int ACT> __global__ __launch_bounds__(512) void k_radi
           dh1[rb] = Mfma<T>::mma(w, dh0[s], dh1[rb]);
         }
       }
+    if (MODE == 1) {
+      const long long ee = eloc < cnt ? e : a.e_begin;
+      const T *bi = a.bias_i + (long long) a.emi[ee] * (HB * 16), *bj = a.bias_j + (long long) a.emu[ee] * (HB * 16);
+#pragma unroll
+      for (int rb = 0; rb < HB; rb++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) h1[rb][v] += bi[rb * 16 + a.drow[g * 4 + v]] + bj[rb * 16 + a.drow[g * 4 + v]];
+    }
 #pragma unroll
     for (int rb = 0; rb < HB; rb++)
 #pragma unroll
@@ -394,6 +407,12 @@ template<class T, int HB, int ACT> __global__ __launch_bounds__(512) void k_radi
           dh2[rb] = Mfma<T>::mma(w, db, dh2[rb]);
         }
       }
+    if (MODE == 1) {
+#pragma unroll
+      for (int rb = 0; rb < HB; rb++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) h2[rb][v] += a.bias1[rb * 16 + a.drow[g * 4 + v]];
+    }
 #pragma unroll
     for (int rb = 0; rb < HB; rb++)
 #pragma unroll
@@ -405,11 +424,18 @@ template<class T, int HB, int ACT> __global__ __launch_bounds__(512) void k_radi
     // ---- layer 2 (linear), operands swapped: rows = edges, columns = outputs; two column blocks at a time
     long long row_v[4];
     const T *z_v[4];
+    T env_v[4], denv_v[4];
 #pragma unroll
     for (int v = 0; v < 4; v++) {
       const long long el = tile * 16 + a.drow[g * 4 + v];
       row_v[v] = el < cnt ? (a.e_begin + el) * a.noutp : -1;
       z_v[v] = a.z + (el < cnt ? a.emu[a.e_begin + el] : 0) * a.C;
+      if (MODE == 1) {
+        const double xv = el < cnt ? a.x[a.e_begin + el] : 0.5;
+        const double xpm = ipow(xv, p - 1), xp = xpm * xv, xp1 = xp * xv, xp2 = xp1 * xv;
+        env_v[v] = (T) (1.0 - cf0 * xp + cf1 * xp1 - cf2 * xp2);
+        denv_v[v] = (T) (cfd * (-xpm + 2.0 * xp - xp1));
+      }
     }
     for (int cb = 0; cb < a.nob; cb += 2) {
       const bool two = cb + 1 < a.nob;
@@ -432,12 +458,22 @@ template<class T, int HB, int ACT> __global__ __launch_bounds__(512) void k_radi
       for (int v = 0; v < 4; v++)
         if (row_v[v] >= 0) {
           const T zz0 = z_v[v][n0];
-          a.Rz[row_v[v] + col0] = acc0[v] * zz0;
-          a.dRz[row_v[v] + col0] = dacc0[v] * zz0;
+          if (MODE == 1) {
+            a.Rz[row_v[v] + col0] = acc0[v] * env_v[v] * zz0;
+            a.dRz[row_v[v] + col0] = (dacc0[v] * env_v[v] + acc0[v] * denv_v[v]) * zz0;
+          } else {
+            a.Rz[row_v[v] + col0] = acc0[v] * zz0;
+            a.dRz[row_v[v] + col0] = dacc0[v] * zz0;
+          }
           if (two) {
             const T zz1 = z_v[v][n1];
-            a.Rz[row_v[v] + col1] = acc1[v] * zz1;
-            a.dRz[row_v[v] + col1] = dacc1[v] * zz1;
+            if (MODE == 1) {
+              a.Rz[row_v[v] + col1] = acc1[v] * env_v[v] * zz1;
+              a.dRz[row_v[v] + col1] = (dacc1[v] * env_v[v] + acc1[v] * denv_v[v]) * zz1;
+            } else {
+              a.Rz[row_v[v] + col1] = acc1[v] * zz1;
+              a.dRz[row_v[v] + col1] = dacc1[v] * zz1;
+            }
           }
         }
     }

@@ -81,8 +81,8 @@ __device__ inline T pair_stage(const int *__restrict__ ej, const T *__restrict__
   return touch;
 }
 
-// grid: atoms; block: nslot * C threads (slot = t / C, n = t % C); dynamic LDS: kPairChunk * (NT + nl * C) values.
-// NLM = nl * nl exactly.
+// grid: (atoms, slot groups); block: spb * C threads, spb slots per block (slot = blockIdx.y * spb + t / C, n = t % C);
+// dynamic LDS: kPairChunk * (NT + nl * C) values.  NLM = nl * nl exactly.
 template<class T, int NLM>
 __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ Y,
                            const T *__restrict__ R1, const T *__restrict__ M, T *__restrict__ P, int nslot, int C, int nl, int noutp,
@@ -91,7 +91,9 @@ __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__rest
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const int i = blockIdx.x, t = threadIdx.x, NT = blockDim.x;
   T *Msh = reinterpret_cast<T *>(smem_raw), *Rsh = Msh + kPairChunk * NT;
-  const int slot = t / C, n = t % C;
+  const int slot_raw = blockIdx.y * (NT / C) + t / C, n = t % C;
+  const bool active = slot_raw < nslot;
+  const int slot = active ? slot_raw : 0;
   const int nlm = nl * nl;
   const long long e0 = eoff[i], e1 = eoff[i + 1];
   T acc[NLM];
@@ -101,7 +103,7 @@ __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__rest
   for (long long base = e0; base < e1; base += kPairChunk) {
     const int nb = (int) (e1 - base < kPairChunk ? e1 - base : kPairChunk);
     __syncthreads();
-    touch += pair_stage<T>(ej, M, R1, nullptr, Y, ystride, nlm, base, nb, nslot, C, noutp, true, slot, n, Msh, Rsh, nullptr, NT);
+    touch += pair_stage<T>(ej, M, R1, nullptr, Y, ystride, nlm, base, nb, nslot, C, noutp, active, slot, n, Msh, Rsh, nullptr, NT);
     __syncthreads();
     for (int b = 0; b < nb; b++) {
       const T m = Msh[b * NT + t];
@@ -119,7 +121,7 @@ __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__rest
   T *o = P + ((long long) i * nslot + slot) * nlm * C + n;
 #pragma unroll
   for (int q = 0; q < NLM; q++)
-    if (q < nlm) o[(long long) q * C] = acc[q];
+    if (active && q < nlm) o[(long long) q * C] = acc[q];
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
 }
 
@@ -140,7 +142,8 @@ __device__ inline double wave_sum4(double v0, double v1, double v2, double v3, i
   return c;
 }
 
-// grid: atoms; block: nslot * C threads rounded up to a wave; dynamic LDS: kPairChunk * (NT + 2 nl C) values.
+// grid: (atoms, slot groups); block: spb * C threads rounded up to a wave, spb slots per block (a kernel argument);
+// dynamic LDS: kPairChunk * (NT + 2 nl C) values.  Every block adds the force of its slots to the bond's two atoms.
 // gP: adjoint of P of the atom.
 //   S_l = sum_m Y_lm gP[lm],  T_l,d = sum_m G_lm,d gP[lm]                      (per thread: slot, n)
 //   dE/dI_j[slot][n] += sum_l R1_l S_l                                        (slots < nI)
@@ -151,14 +154,15 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
                            const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
                            const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
                            T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
-                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid)
+                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   __shared__ double bsum[kPairChunk][4];
   const int i = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6, NT = blockDim.x;
   T *Msh = reinterpret_cast<T *>(smem_raw), *Rsh = Msh + kPairChunk * NT, *dRsh = Rsh + kPairChunk * noutp;
-  const bool active = t < nslot * C;
-  const int slot = active ? t / C : 0, n = t % C;
+  const int slot_raw = blockIdx.y * spb + t / C;
+  const bool active = t < spb * C && slot_raw < nslot;
+  const int slot = active ? slot_raw : 0, n = t % C;
   const int nlm = nl * nl;
   const long long e0 = eoff[i], e1 = eoff[i + 1];
   T g[NLM];

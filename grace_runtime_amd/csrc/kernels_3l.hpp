@@ -1,0 +1,235 @@
+// HIP kernels of the GRACE-3L layers for gfx950 that the GRACE-1L / 2L kernels do not already provide.
+//
+//   k_edge_center      element of the central atom of every edge (input of the species form of the radial kernel)
+//   k_message          M[atom][li][n] = I[atom][li][n] + chem_l0_mask[li] zproj[mu_atom][n]: what a neighbour contributes to
+//                      the equivariant SPBF (bond_vectors, libgrace/src/fused_3l.cpp:1049-1083)
+//   k_lincomb          out[atom][f][n] = sum_t v_t in[atom][p_t][n]: the sparse Clebsch-Gordan matrix cg_W of the equivariant
+//                      SPBF and its transpose (fused_3l.cpp:1266-1272, :1443-1449)
+//   k_scale_rows       out[atom][f][n] (+)= s[f] in[atom][f][n]: the left input of an FCRight2Left layer (fused_3l.cpp:955-969)
+//   k_eqnorm_fwd/bwd   EquivariantRMSNorm (libgrace/include/grace/fused_3l_cpu.h:335-414)
+//   k_energy_3l        InvariantLayerRMSNorm of the three densities, their sum, fp64 readout MLP and the reverse of all of it
+//                      (fused_3l_cpu.h:416-444, fused_3l.cpp:1300-1360)
+#pragma once
+
+#include "kernels_2l.hpp"
+
+namespace grhip {
+
+// grid: atoms; block: 64
+static __global__ void k_edge_center(const long long *eoff, const int *mu, int *emi)
+{
+  const int i = blockIdx.x;
+  const int m = mu[i];
+  for (long long e = eoff[i] + threadIdx.x; e < eoff[i + 1]; e += blockDim.x) emi[e] = m;
+}
+
+// grid: ceil(natoms * nf * C / 256)
+template<class T>
+__global__ void k_message(const T *I, const int *mu, const T *zproj, const T *mask, T *M, int natoms, int nf, int C)
+{
+  const long long q = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (q >= (long long) natoms * nf * C) return;
+  const int n = (int) (q % C), f = (int) ((q / C) % nf), at = (int) (q / ((long long) C * nf));
+  M[q] = I[q] + mask[f] * zproj[(long long) mu[at] * C + n];
+}
+
+// CSR by output function: terms [off[f], off[f + 1]) with source function idx[t] and value val[t].
+// grid: (atoms, ceil(nout * C / 256)); block 256.  Rows of `in` have nin functions.
+template<class T>
+__global__ void k_lincomb(const int *__restrict__ off, const int *__restrict__ idx, const double *__restrict__ val, const T *__restrict__ in,
+                          T *__restrict__ out, int nin, int nout, int C)
+{
+  const int at = blockIdx.x, q = blockIdx.y * blockDim.x + threadIdx.x;
+  if (q >= nout * C) return;
+  const int f = q / C, n = q % C;
+  const T *src = in + (long long) at * nin * C + n;
+  T acc = (T) 0;
+  for (int t = off[f]; t < off[f + 1]; t++) acc += (T) val[t] * src[(long long) idx[t] * C];
+  out[((long long) at * nout + f) * C + n] = acc;
+}
+
+// grid: ceil(natoms * nf * C / 256)
+template<class T> __global__ void k_scale_rows(const T *in, const T *s, T *out, int natoms, int nf, int C, int accumulate)
+{
+  const long long q = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (q >= (long long) natoms * nf * C) return;
+  const int f = (int) ((q / C) % nf);
+  const T v = s[f] * in[q];
+  out[q] = accumulate ? out[q] + v : v;
+}
+
+struct EqNormDev {
+  const double *dw, *mask, *aff;    // [M], [M], [groups][C] (C = padded channel width, padding columns zero)
+  const int *grp;                   // [M]
+  int M, C, Creal, center;
+  double eps;
+};
+
+__device__ inline double block_sum(double v, double *red)
+{
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  double s = 0.0;
+  for (int w = 0; w < nw; w++) s += red[w];
+  return s;
+}
+
+// xc = x - l0_mask mean_n x;  r = 1 / sqrt(mean_n sum_f dw[f] xc^2 + eps);  y = xc r aff[e(f)][n].
+// One block of 256 threads per atom; a wave per function row for the means.  With gy != nullptr also the reverse:
+// gx[f][n] = r g - r^3 / C (sum g xc) dw[f] xc, minus its channel mean on the centred rows, g = gy aff.
+template<class T>
+__global__ void k_eqnorm(EqNormDev E, const T *X, T *Y, const T *gY, T *gX, int accumulate)
+{
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  double *mean = reinterpret_cast<double *>(smem_raw);    // [M]
+  __shared__ double red[16];
+  const int at = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6, nw = blockDim.x >> 6;
+  const int M = E.M, C = E.C, Cr = E.Creal;
+  const T *x = X + (long long) at * M * C;
+  for (int f = wave; f < M; f += nw) {
+    double m = 0.0;
+    if (E.center && E.mask[f] != 0.0) {
+      for (int n = lane; n < Cr; n += 64) m += (double) x[(long long) f * C + n];
+      for (int o = 32; o > 0; o >>= 1) m += __shfl_xor(m, o, 64);
+      m = m / Cr * E.mask[f];
+    }
+    if (lane == 0) mean[f] = m;
+  }
+  __syncthreads();
+  double s = 0.0;
+  for (int q = t; q < M * C; q += blockDim.x) {
+    const int f = q / C, n = q % C;
+    if (n < Cr) {
+      const double c = (double) x[q] - mean[f];
+      s += E.dw[f] * c * c;
+    }
+  }
+  const double S = block_sum(s, red);
+  const double r = 1.0 / sqrt(S / Cr + E.eps);
+  if (!gY) {
+    T *y = Y + (long long) at * M * C;
+    for (int q = t; q < M * C; q += blockDim.x) {
+      const int f = q / C, n = q % C;
+      y[q] = n < Cr ? (T) (((double) x[q] - mean[f]) * r * E.aff[(long long) E.grp[f] * C + n]) : (T) 0;
+    }
+    return;
+  }
+  const T *gy = gY + (long long) at * M * C;
+  double gx = 0.0;
+  for (int q = t; q < M * C; q += blockDim.x) {
+    const int f = q / C, n = q % C;
+    if (n < Cr) gx += (double) gy[q] * E.aff[(long long) E.grp[f] * C + n] * ((double) x[q] - mean[f]);
+  }
+  const double k3 = r * r * r * block_sum(gx, red) / Cr;
+  T *go = gX + (long long) at * M * C;
+  for (int f = wave; f < M; f += nw) {
+    const double kf = k3 * E.dw[f];
+    const bool cen = E.center && E.mask[f] != 0.0;
+    double vsum = 0.0;
+    for (int n = lane; n < Cr; n += 64) {
+      const long long q = (long long) f * C + n;
+      vsum += r * (double) gy[q] * E.aff[(long long) E.grp[f] * C + n] - kf * ((double) x[q] - mean[f]);
+    }
+    for (int o = 32; o > 0; o >>= 1) vsum += __shfl_xor(vsum, o, 64);
+    const double mg = cen ? vsum / Cr * E.mask[f] : 0.0;
+    for (int n = lane; n < Cr; n += 64) {
+      const long long q = (long long) f * C + n;
+      const double v = r * (double) gy[q] * E.aff[(long long) E.grp[f] * C + n] - kf * ((double) x[q] - mean[f]) - mg;
+      go[q] = accumulate ? go[q] + (T) v : (T) v;
+    }
+  }
+}
+
+struct Energy3Dev {
+  const double *W0, *W1;      // [nin][nh], [nh]
+  double norm0, norm1, out_scale, eps;
+  int nin, nh, act, nrho;
+  const double *shift;        // [nel]
+  const double *scale[3];     // RMSNorm scales of rho1, rho2, rho3: [nrho - type]
+  int type[3];                // 1: only_nonlin (channel 0 passes)
+};
+
+// rho_k -> y_k = RMSNorm_k(rho_k), h = y_1 + y_2 + y_3, E_i = (MLP(h[1:]) + h[0]) out_scale + shift[mu_i]; with want_grad
+// the adjoints grho_k of the raw densities.  One wave per atom, fp64.  Dynamic LDS: (nrho + 2 nh) doubles.
+static __global__ void k_energy_3l(Energy3Dev M, const int *mu, const double *rho1, const double *rho2, const double *rho3, double *g1, double *g2,
+                                   double *g3, double *eatom, double *energy, int want_grad, const int *sid)
+{
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  double *h = reinterpret_cast<double *>(smem_raw), *pre = h + M.nrho, *gs = pre + M.nh;
+  const int at = blockIdx.x, lane = threadIdx.x, nr = M.nrho;
+  const double *rho[3] = {rho1 + (long long) at * nr, rho2 + (long long) at * nr, rho3 + (long long) at * nr};
+  double rinv[3];
+  for (int k = 0; k < 3; k++) {
+    const int n0 = M.type[k];
+    double s = 0.0;
+    for (int n = n0 + lane; n < nr; n += 64) s += rho[k][n] * rho[k][n];
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    rinv[k] = 1.0 / sqrt(s / (nr - n0) + M.eps);
+  }
+  for (int n = lane; n < nr; n += 64) {
+    double v = 0.0;
+    for (int k = 0; k < 3; k++) v += n < M.type[k] ? rho[k][n] : rho[k][n] * rinv[k] * M.scale[k][n - M.type[k]];
+    h[n] = v;
+  }
+  __syncthreads();
+  double e = 0.0;
+  for (int j = lane; j < M.nh; j += 64) {
+    double s = 0.0;
+    for (int c = 0; c < M.nin; c++) s += h[c + 1] * M.W0[(long long) c * M.nh + j];
+    s *= M.norm0;
+    pre[j] = s;
+    e += M.W1[j] * (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s)));
+  }
+  for (int o = 32; o > 0; o >>= 1) e += __shfl_xor(e, o, 64);
+  const double Ei = (e * M.norm1 + h[0]) * M.out_scale + M.shift[mu[at]];
+  if (lane == 0) {
+    if (eatom) eatom[at] = Ei;
+    atomicAdd(energy + (sid ? 8 * sid[at] : 0), Ei);
+  }
+  if (!want_grad) return;
+  for (int j = lane; j < M.nh; j += 64) {
+    const double s = pre[j];
+    double da;
+    if (M.act == 1) {
+      const double tt = tanh(s);
+      da = 1.0 - tt * tt;
+    } else {
+      const double sg = 1.0 / (1.0 + exp(-s));
+      da = sg * (1.0 + s * (1.0 - sg));
+    }
+    gs[j] = M.out_scale * M.norm1 * M.W1[j] * da * M.norm0;
+  }
+  __syncthreads();
+  // dE/dh: channel 0 the linear skip, channels 1.. through the MLP; kept in `pre` is no longer needed -> reuse h for dE/dh
+  double gh_mine[4];    // nrho <= 256: up to 4 channels per lane
+  for (int q = 0; q < 4; q++) {
+    const int n = lane + 64 * q;
+    double v = 0.0;
+    if (n == 0) v = M.out_scale;
+    else if (n < nr) {
+      for (int j = 0; j < M.nh; j++) v += M.W0[(long long) (n - 1) * M.nh + j] * gs[j];
+    }
+    gh_mine[q] = v;
+  }
+  double *gout[3] = {g1 + (long long) at * nr, g2 + (long long) at * nr, g3 + (long long) at * nr};
+  for (int k = 0; k < 3; k++) {
+    const int n0 = M.type[k], nn = nr - n0;
+    double gx = 0.0;
+    for (int q = 0; q < 4; q++) {
+      const int n = lane + 64 * q;
+      if (n >= n0 && n < nr) gx += gh_mine[q] * M.scale[k][n - n0] * rho[k][n];
+    }
+    for (int o = 32; o > 0; o >>= 1) gx += __shfl_xor(gx, o, 64);
+    const double r = rinv[k], kk = r * r * r * gx / nn;
+    for (int q = 0; q < 4; q++) {
+      const int n = lane + 64 * q;
+      if (n >= nr) continue;
+      gout[k][n] = n < n0 ? gh_mine[q] : r * gh_mine[q] * M.scale[k][n - n0] - kk * rho[k][n];
+    }
+  }
+}
+
+}    // namespace grhip

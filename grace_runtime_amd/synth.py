@@ -25,7 +25,7 @@ import math
 import numpy as np
 
 __all__ = ["real_sh_np", "coupling_tables", "real_cg", "structure_1l", "structure_2l", "random_model_1l",
-           "random_model_2l", "save_model", "bcc_supercell", "fcc_supercell", "jitter"]
+           "random_model_2l", "structure_3l", "random_model_3l", "save_model", "bcc_supercell", "fcc_supercell", "jitter"]
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -618,6 +618,314 @@ def random_model_2l(*, lmax=4, n_elements=4, element_names=("Al", "Co", "Ni", "T
     d["energy_mlp_n_layers"] = i64(2)
     d["energy_mlp_activation"] = i64(1)
     d["shift_values"] = np.zeros(n_elements)
+    d.update(s)
+    return d
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# GRACE-3L: structure arrays and random weights
+# ---------------------------------------------------------------------------------------------------------------
+def _irrep_offsets(irreps):
+    return np.concatenate([[0], np.cumsum([2 * l + 1 for l, _ in irreps])]).astype(np.int64)
+
+
+def _couplings(left, right, out, self_product):
+    """Coupling paths (ia, ib, ic) of irreps (l, s) (s = 1: pseudo-tensor): triangle rule, and the product is a
+    pseudo-tensor when exactly one of {one factor pseudo, l_a + l_b + l_c odd} holds twice over, i.e.
+    s_c = s_a xor s_b xor parity(l_a + l_b + l_c).  A self product keeps ia >= ib."""
+    paths = []
+    for ia, (la, sa) in enumerate(left):
+        for ib, (lb, sb) in enumerate(right):
+            if self_product and ib > ia:
+                continue
+            for ic, (lc, sc) in enumerate(out):
+                if abs(la - lb) <= lc <= la + lb and sc == (sa ^ sb ^ ((la + lb + lc) & 1)):
+                    paths.append((ia, ib, ic))
+    return paths
+
+
+def _coupled_functions(left, right, out, paths):
+    """Functions (path, M) in path order, their CG terms (left fn, right fn, fn, value) and destination (irrep
+    function of `out`)."""
+    lo, ro, oo = _irrep_offsets(left), _irrep_offsets(right), _irrep_offsets(out)
+    terms, fn_path, fn_dst, fn_l = [], [], [], []
+    for ip, (ia, ib, ic) in enumerate(paths):
+        la, lb, lc = left[ia][0], right[ib][0], out[ic][0]
+        T = real_cg(la, lb, lc)
+        for M in range(2 * lc + 1):
+            f = len(fn_path)
+            fn_path.append(ip)
+            fn_dst.append(int(oo[ic]) + M)
+            fn_l.append(lc)
+            for m1, m2 in zip(*np.nonzero(T[:, :, M])):
+                terms.append((int(lo[ia]) + int(m1), int(ro[ib]) + int(m2), f, float(T[m1, m2, M])))
+    return terms, np.array(fn_path, np.int32), np.array(fn_dst, np.int32), np.array(fn_l, np.int32)
+
+
+def structure_3l(lmax, lmsg=None, pseudo_message=True):
+    """Structure arrays (no weights) of a GRACE-3L model, keys as libgrace/src/model_3l.cpp:165-464 reads them.
+
+    Irreps are (l, s), s = 1 for pseudo-tensors.  Per layer K = A1, A2, A3 the lm features X are the natural irreps
+    l <= lmax (the scalar SPBF in layer 1, the reduce K_red of the equivariant SPBF in layers 2-3); the product
+    reduces K_2_red, K_3_red, K_4_red carry the natural irreps l <= lmax and, in layer 2 when `pseudo_message`, the
+    pseudo irreps too; the message eq1 holds the natural irreps l <= lmsg, eq2 those and (pseudo_message) their
+    pseudo partners.  Every coupling the triangle and parity rules allow is one path with its own weight tile.
+    Returns the arrays and '_sizes'."""
+    lmsg = lmax if lmsg is None else lmsg
+    nl = lmax + 1
+    nlm = nl * nl
+    X = [(l, 0) for l in range(nl)]
+    nat_msg = [(l, 0) for l in range(lmsg + 1)]
+    s, sizes = {}, {}
+    i64 = lambda v: np.array([v], dtype=np.int64)
+    i32a = lambda v: np.asarray(v, dtype=np.int32)
+    lm_l = np.repeat(np.arange(nl), 2 * np.arange(nl) + 1).astype(np.int32)
+
+    def cpl(name, left, right, out, self_product):
+        paths = _couplings(left, right, out, self_product)
+        terms, fn_path, fn_dst, fn_l = _coupled_functions(left, right, out, paths)
+        s[f"{name}_nfunc"] = i64(len(fn_path))
+        s[f"{name}_n_groups_left"] = i64(len(left))
+        s[f"{name}_n_groups_right"] = i64(len(right))
+        s[f"{name}_group_left"] = i32a(np.repeat(np.arange(len(left)), [2 * l + 1 for l, _ in left]))
+        s[f"{name}_group_right"] = i32a(np.repeat(np.arange(len(right)), [2 * l + 1 for l, _ in right]))
+        s[f"{name}_left_ind"] = i32a([t[0] for t in terms])
+        s[f"{name}_right_ind"] = i32a([t[1] for t in terms])
+        s[f"{name}_m_sum_ind"] = i32a([t[2] for t in terms])
+        s[f"{name}_cg"] = np.array([t[3] for t in terms], dtype=np.float64)
+        s[f"{name}_out_l"] = fn_l
+        sizes[name] = dict(nfunc=len(fn_path), npaths=len(paths), ngl=len(left), ngr=len(right), nterms=len(terms))
+        return paths, fn_path, fn_dst
+
+    def reduce_instr(red, src, collect, tile, dst, w_shape):
+        s[f"{red}_collect_ind_{src}"] = i32a(collect)
+        s[f"{red}_w_l_tile_{src}"] = i32a(tile)
+        s[f"{red}_total_sum_ind_{src}"] = i32a(dst).reshape(-1, 1)
+        s[f"{red}_w_shape_{src}"] = i64(max(int(w_shape), 1))
+
+    def product_reduce(red, prod, paths, fn_path, fn_dst, out):
+        nfo = int(_irrep_offsets(out)[-1])
+        reduce_instr(red, prod, np.arange(len(fn_path)), fn_path, fn_dst, len(paths))
+        cnt = np.zeros(nfo)
+        np.add.at(cnt, fn_dst, 1.0)
+        s[f"{red}_norm_map"] = 1.0 / np.sqrt(np.maximum(cnt, 1.0))
+        s[f"{red}_n_funcs"] = i64(nfo)
+        s[f"{red}_only_invar"] = i64(0)
+        s[f"{red}_is_central_atom_type_dependent"] = i64(0)
+        s[f"{red}_instruction_names"] = np.array([prod.encode()], dtype="|S8")
+        sizes[red] = dict(nfunc=nfo, w_shape={prod: max(len(paths), 1)})
+
+    def fc(name, left):
+        """out[f] = nof[f] (left[f] + W[l] X[lm]) for the natural functions f of `left`; the others pass."""
+        lo = _irrep_offsets(left)
+        nleft = int(lo[-1])
+        frm, to, tile = [], [], []
+        for i, (l, sp) in enumerate(left):
+            if sp == 0 and l <= lmax:
+                for M in range(2 * l + 1):
+                    frm.append(l * l + M)
+                    to.append(int(lo[i]) + M)
+                    tile.append(l)
+        nof = np.ones(nleft)
+        nof[to] = 1.0 / math.sqrt(2.0)
+        s[f"fc_{name}_w_tile_left"] = np.zeros(nleft, np.int32)
+        s[f"fc_{name}_w_tile_right"] = i32a(tile)
+        s[f"fc_{name}_collect_from"] = i32a(frm)
+        s[f"fc_{name}_collect_to"] = i32a(to)
+        s[f"fc_{name}_norm_out_factor"] = nof.reshape(-1, 1, 1)
+        s[f"fc_{name}_left_coefs"] = i64(0)
+
+    def collect_reduce(red, sources, out, invariant, elem):
+        """eq / rho: from each source the functions whose irrep is in `out` (the invariants for rho), one weight tile
+        per source irrep."""
+        oo = _irrep_offsets(out)
+        names = []
+        for src, irr in sources:
+            so = _irrep_offsets(irr)
+            col, tile, dst = [], [], []
+            for i, ir in enumerate(irr):
+                if ir in out:
+                    k = out.index(ir)
+                    for M in range(2 * ir[0] + 1):
+                        col.append(int(so[i]) + M)
+                        tile.append(i)
+                        dst.append(0 if invariant else int(oo[k]) + M)
+            reduce_instr(red, src, col, tile, dst, len(irr))
+            names.append(src)
+            sizes.setdefault(red, dict(w_shape={}))["w_shape"][src] = len(irr)
+        nfo = int(oo[-1])
+        s[f"{red}_n_funcs"] = i64(nfo)
+        s[f"{red}_only_invar"] = i64(1 if invariant else 0)
+        s[f"{red}_is_central_atom_type_dependent"] = i64(1 if elem else 0)
+        s[f"{red}_instruction_names"] = np.array([n.encode() for n in names], dtype="|S8")
+        if not invariant:
+            s[f"{red}_norm_map"] = np.full(nfo, 0.5)
+        sizes[red]["nfunc"] = 1 if invariant else nfo
+
+    message = None
+    spbf, prods, reds, fcs, eqn, rmsn = [], [], [], [], [], []
+    for k in (1, 2, 3):
+        K = f"A{k}"
+        spbf.append(K)
+        s[f"{K}_equivariant"] = i64(0 if k == 1 else 1)
+        s[f"{K}_lmax"] = i64(lmax)
+        s[f"{K}_Lmax"] = i64(lmax)
+        s[f"{K}_l_tile"] = lm_l.copy()
+        Xn = K
+        if k > 1:
+            ylm = [(l, 0) for l in range(nl)]
+            paths = _couplings(ylm, message, X, False)
+            terms, fn_path, fn_dst, _ = _coupled_functions(ylm, message, X, paths)
+            nlmi = int(_irrep_offsets(message)[-1])
+            W = np.zeros((nlm * nlmi, len(fn_path)))
+            for a, b, f, v in terms:
+                W[a * nlmi + b, f] = v
+            s[f"{K}_cg_W"] = W
+            s[f"{K}_nfunc"] = i64(len(fn_path))
+            s[f"{K}_n_lm_ind"] = i64(nlmi)
+            mo = _irrep_offsets(message)
+            mask = np.zeros(nlmi)
+            mask[int(mo[message.index((0, 0))])] = 1.0
+            s[f"{K}_chem_l0_mask"] = mask
+            sizes[K] = dict(nfunc=len(fn_path), npaths=len(paths), nlmi=nlmi)
+            red = K + "_red"
+            reduce_instr(red, K, np.arange(len(fn_path)), fn_path, fn_dst, len(paths))
+            cnt = np.zeros(nlm)
+            np.add.at(cnt, fn_dst, 1.0)
+            s[f"{red}_norm_map"] = 1.0 / np.sqrt(np.maximum(cnt, 1.0))
+            s[f"{red}_n_funcs"] = i64(nlm)
+            s[f"{red}_only_invar"] = i64(0)
+            s[f"{red}_is_central_atom_type_dependent"] = i64(0)
+            s[f"{red}_instruction_names"] = np.array([K.encode()], dtype="|S8")
+            sizes[red] = dict(nfunc=nlm, w_shape={K: len(paths)})
+            reds.append(red)
+            Xn = red
+        else:
+            sizes[K] = dict(nfunc=nlm)
+        T = list(X) + ([(l, 1) for l in range(nl)] if (k == 2 and pseudo_message) else [])
+        p2 = cpl(K + "_2", X, X, T, True)
+        product_reduce(K + "_2_red", K + "_2", *p2, T)
+        fc(K + "_2a", T)
+        p3 = cpl(K + "_3", T, X, T, False)
+        product_reduce(K + "_3_red", K + "_3", *p3, T)
+        fc(K + "_2b", T)
+        p4 = cpl(K + "_4", T, T, T, True)
+        product_reduce(K + "_4_red", K + "_4", *p4, T)
+        prods += [K + "_2", K + "_3", K + "_4"]
+        reds += [K + "_2_red", K + "_3_red", K + "_4_red"]
+        fcs += [K + "_2a", K + "_2b"]
+        sources = [(Xn, X), (K + "_2_red", T), (K + "_3_red", T), (K + "_4_red", T)]
+        if k < 3:
+            message = list(nat_msg) + ([(l, 1) for l in range(lmsg + 1)] if (k == 2 and pseudo_message) else [])
+            collect_reduce(f"eq{k}", sources, message, False, False)
+            reds.append(f"eq{k}")
+            mo = _irrep_offsets(message)
+            M = int(mo[-1])
+            e = f"eq{k}_norm"
+            s[f"{e}_expand_index"] = i32a(np.repeat(np.arange(len(message)), [2 * l + 1 for l, _ in message]))
+            s[f"{e}_degree_weights"] = np.repeat([1.0 / ((2 * l + 1) * len(message)) for l, _ in message],
+                                                 [2 * l + 1 for l, _ in message])
+            mask = np.zeros(M)
+            mask[int(mo[message.index((0, 0))])] = 1.0
+            s[f"{e}_l0_mask"] = mask
+            s[f"{e}_eps"] = np.array([1e-8])
+            s[f"{e}_center_l0"] = i64(1)
+            eqn.append(e)
+            sizes[e] = dict(n_groups=len(message), M=M)
+        collect_reduce(f"rho{k}", sources, [(0, 0)], True, True)
+        reds.append(f"rho{k}")
+        rmsn.append(f"rho{k}_norm")
+    enc = lambda names: np.array([n.encode() for n in names], dtype="|S12")
+    s.update(spbf_names=enc(spbf), prod_names=enc(prods), reduce_names=enc(reds), fc_names=enc(fcs),
+             eqnorm_names=enc(eqn), rmsnorm_names=enc(rmsn), out1_origins=enc(rmsn))
+    s["_sizes"] = sizes
+    return s
+
+
+def random_model_3l(*, lmax=4, lmsg=None, pseudo_message=True, n_elements=8, element_names=None, embedding_size=32,
+                    nradbase=8, channels=64, hidden=128, rho_n_out=32, energy_hidden=64, rcut=6.0, p=5,
+                    inv_avg_n_neigh=1.0 / 72.0, rms_type=1, seed=20260104):
+    """A GRACE-3L-shaped model (three layers: scalar SPBF, then two equivariant SPBFs coupling the normalised
+    message of the layer before; cp_l products up to body order 4 per layer) with weights ~ N(0, 1) and norm
+    scalars 1/sqrt(n_in).  `channels` = radial channels = cp_l rank of every layer.  Keys as the reference loader
+    reads them, libgrace/src/model_3l.cpp:165-464."""
+    rng = np.random.default_rng(seed)
+    nl = lmax + 1
+    s = structure_3l(lmax, lmsg, pseudo_message)
+    z = s.pop("_sizes")
+    C = channels
+    i64 = lambda v: np.array([v], dtype=np.int64)
+    f64 = lambda v: np.array([v], dtype=np.float64)
+    N = lambda *shape: rng.standard_normal(shape)
+    if element_names is None:
+        table = ("H He Li Be B C N O F Ne Na Mg Al Si P S Cl Ar K Ca Sc Ti V Cr Mn Fe Co Ni Cu Zn Ga Ge As Se Br Kr Rb Sr "
+                 "Y Zr Nb Mo Tc Ru Rh Pd Ag Cd In Sn Sb Te I Xe Cs Ba La Ce Pr Nd Pm Sm Eu Gd Tb Dy Ho Er Tm Yb Lu Hf Ta "
+                 "W Re Os Ir Pt Au Hg Tl Pb Bi Ac Th Pa U Np Pu").split()
+        element_names = table[:n_elements]
+    d = {"grace_model_kind": np.array([b"GRACE-3L"], dtype="|S8"), "grace_format_version": i64(1),
+         "n_elements": i64(n_elements), "element_names": np.array([n.encode() for n in element_names], dtype="|S2"),
+         "embedding_size": i64(embedding_size), "nradbase": i64(nradbase), "rcut": f64(rcut),
+         "has_bond_specific_cutoff": i64(0), "chem_embedding": N(n_elements, embedding_size),
+         "shift_values": np.zeros(n_elements), "output_scale": f64(1.0)}
+    for k in (1, 2, 3):
+        K = f"A{k}"
+        d[f"{K}_n_rad_max"] = i64(C)
+        d[f"{K}_n_rad_basis"] = i64(nradbase)
+        d[f"{K}_p"] = i64(p)
+        d[f"{K}_rcut"] = f64(rcut)
+        d[f"{K}_inv_avg_n_neigh"] = f64(inv_avg_n_neigh)
+        dims = [nradbase + 2 * embedding_size, hidden, hidden, C * nl]
+        for i in range(3):
+            d[f"{K}_mlp_W{i}"] = N(dims[i], dims[i + 1])
+            d[f"{K}_mlp_norm{i}"] = f64(1.0 / math.sqrt(dims[i]))
+            if i < 2:
+                d[f"{K}_mlp_b{i}"] = N(dims[i + 1])
+        d[f"{K}_mlp_n_layers"] = i64(3)
+        if k == 1:
+            d[f"{K}_lin_transform_W"] = N(embedding_size, C)
+            d[f"{K}_lin_transform_norm"] = f64(1.0 / math.sqrt(embedding_size))
+        else:
+            d[f"{K}_chem_linear_W"] = N(embedding_size, C)
+            d[f"{K}_chem_linear_norm"] = f64(1.0 / math.sqrt(embedding_size))
+        for q in ("2", "3", "4"):
+            P = f"{K}_{q}"
+            d[f"{P}_rank"] = i64(C)
+            d[f"{P}_n_left"] = i64(C)
+            d[f"{P}_n_right"] = i64(C)
+            d[f"{P}_U"] = N(z[P]["ngl"], C, C)
+            d[f"{P}_V"] = N(z[P]["ngr"], C, C)
+            d[f"{P}_norm_u"] = f64(1.0 / math.sqrt(C))
+            d[f"{P}_norm_v"] = f64(1.0 / math.sqrt(C))
+        for f in ("2a", "2b"):
+            d[f"fc_{K}_{f}_n_out"] = i64(C)
+            d[f"fc_{K}_{f}_w_right"] = N(C, C, nl)
+            d[f"fc_{K}_{f}_norm_right"] = f64(1.0 / math.sqrt(C))
+    for red, info in z.items():
+        if "w_shape" not in info:
+            continue
+        elem = red.startswith("rho")
+        n_out = rho_n_out if elem else C
+        for src, w_shape in info["w_shape"].items():
+            d[f"{red}_reduce_{src}_W"] = N(n_elements, n_out, C, w_shape) if elem else N(n_out, C, w_shape)
+            d[f"{red}_reduce_{src}_norm"] = f64(1.0 / math.sqrt(C))
+            d[f"{red}_n_in_{src}"] = i64(C)
+        d[f"{red}_n_out"] = i64(n_out)
+    for k in (1, 2):
+        e = f"eq{k}_norm"
+        d[f"{e}_affine_weight"] = 1.0 + 0.1 * N(z[e]["n_groups"], C)
+    for k in (1, 2, 3):
+        r = f"rho{k}_norm"
+        d[f"{r}_scale"] = 1.0 + 0.1 * N(rho_n_out - rms_type)
+        d[f"{r}_type"] = i64(rms_type)
+        d[f"{r}_n_out"] = i64(rho_n_out)
+    d["energy_mlp_origin_n_out"] = i64(rho_n_out)
+    d["energy_mlp_n_origins"] = i64(3)
+    d["energy_mlp_W0"] = N(rho_n_out - 1, energy_hidden)
+    d["energy_mlp_norm0"] = f64(1.0 / math.sqrt(rho_n_out - 1))
+    d["energy_mlp_W1"] = N(energy_hidden, 1)
+    d["energy_mlp_norm1"] = f64(1.0 / math.sqrt(energy_hidden))
+    d["energy_mlp_n_layers"] = i64(2)
+    d["energy_mlp_activation"] = i64(0)
     d.update(s)
     return d
 

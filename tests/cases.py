@@ -56,8 +56,41 @@ def model_config5():
     return synth.random_model_2l(n_elements=3, element_names=("Al", "Ni", "Ti"), inv_avg_n_neigh=1.0 / 60.0, seed=20260105)
 
 
-MODELS = {"config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
-LAYERS = {"config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
+def model_l3mix():
+    """GRACE-3L, two elements with pair-specific cutoffs, lmax 2, messages with both parities"""
+    d = synth.random_model_3l(lmax=2, n_elements=2, element_names=("Mo", "W"), embedding_size=8, nradbase=10, channels=16,
+                              hidden=32, rho_n_out=9, energy_hidden=16, rcut=5.0, inv_avg_n_neigh=1.0 / 26.0, seed=21)
+    d["has_bond_specific_cutoff"] = np.array([1], dtype=np.int64)
+    d["bond_cutoff_map"] = np.array([[5.0, 4.5], [4.5, 4.25]])
+    return d
+
+
+def model_l3wide():
+    """GRACE-3L, four elements, lmax 3 with messages up to l = 2, channel and hidden widths that need padding
+    (20 -> 32, 48 -> 64), full RMSNorm of the densities, tanh readout"""
+    d = synth.random_model_3l(lmax=3, lmsg=2, n_elements=4, element_names=("Al", "Co", "Ni", "Ti"), embedding_size=6, nradbase=8,
+                              channels=20, hidden=48, rho_n_out=12, energy_hidden=24, rcut=5.5, p=6,
+                              inv_avg_n_neigh=1.0 / 30.0, rms_type=0, seed=22)
+    d["energy_mlp_activation"] = np.array([1], dtype=np.int64)
+    return d
+
+
+def model_l3nat():
+    """GRACE-3L with natural-parity messages only, one element, lmax 2"""
+    return synth.random_model_3l(lmax=2, pseudo_message=False, n_elements=1, element_names=("W",), embedding_size=4, nradbase=8,
+                                 channels=16, hidden=16, rho_n_out=8, energy_hidden=16, rcut=5.0, inv_avg_n_neigh=1.0 / 26.0,
+                                 seed=23)
+
+
+def model_config4():
+    """GRACE-3L-shaped benchmark model: three layers, lmax 5, 64 radial channels, radial MLPs (8 + 2 x 32)-128-128-384,
+    an embedding table of 89 species"""
+    return synth.random_model_3l(lmax=5, n_elements=89, embedding_size=32, nradbase=8, channels=64, hidden=128, rho_n_out=32,
+                                 energy_hidden=64, rcut=6.0, inv_avg_n_neigh=1.0 / 72.0, seed=20260104)
+
+
+MODELS = {"l3mix": model_l3mix, "l3wide": model_l3wide, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
+LAYERS = {"l3mix": 3, "l3wide": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
 
 
 def write_model(name, directory):
@@ -122,6 +155,49 @@ def structure_config3():
     return synth.jitter(pos, 0.08, 3), cell, np.array([True, True, True]), types
 
 
+CONFIG4_SPECIES = (6, 8, 13, 14, 22, 26, 28, 74)    # 1-based types = model element + 1: C O Al Si Ti Fe Ni W
+
+
+def structure_config4(natoms=10000, density=0.08, dmin=1.8, seed=4):
+    """Amorphous periodic cube: random sequential packing of `natoms` atoms at `density` atoms / A^3 with a minimum
+    distance `dmin`; 8 species of the 89-element table drawn uniformly."""
+    rng = np.random.default_rng(seed)
+    side = (natoms / density) ** (1.0 / 3.0)
+    nc = max(1, int(side / dmin))
+    w = side / nc
+    grid = {}
+    pos = np.zeros((natoms, 3))
+    k = 0
+    while k < natoms:
+        cand = rng.uniform(0.0, side, (4 * (natoms - k) + 64, 3))
+        for x in cand:
+            c = tuple((x / w).astype(int) % nc)
+            ok = True
+            for dx in (-1, 0, 1):
+                for dy in (-1, 0, 1):
+                    for dz in (-1, 0, 1):
+                        for q in grid.get(((c[0] + dx) % nc, (c[1] + dy) % nc, (c[2] + dz) % nc), ()):
+                            d = x - pos[q]
+                            d -= side * np.round(d / side)
+                            if d @ d < dmin * dmin:
+                                ok = False
+                                break
+                        if not ok:
+                            break
+                    if not ok:
+                        break
+                if not ok:
+                    break
+            if ok:
+                pos[k] = x
+                grid.setdefault(c, []).append(k)
+                k += 1
+                if k == natoms:
+                    break
+    types = np.array(CONFIG4_SPECIES, dtype=np.int32)[rng.integers(0, 8, natoms)]
+    return pos, np.eye(3) * side, np.array([True, True, True]), types
+
+
 def structures_config5(nstruct=512, seed=5):
     """Independent periodic cells of 32 .. 128 atoms: random bcc / fcc / hcp lattice with lattice constant U(2.8, 4.0) A,
     cell strain U(-3 %, 3 %), N(0, 0.1 A) jitter, 3 species drawn uniformly; atoms removed at random from the smallest
@@ -162,6 +238,8 @@ E2E_CASES = [("config1", "config1", None), ("mix2", "alloy54", 5.5), ("mix2", "t
 E2E_CASES_2L = [("config3", "fcc108", None), ("l2mix", "alloy54", 5.5), ("l2mix", "triclinic", None), ("l2mix", "slab", None),
                 ("l2mix", "molecule", None)]
 # reference fixture models (tests/golden/ref_fixtures) on the reference's fixture cells: goldens of the compiled reference
+E2E_CASES_3L = [("l3mix", "alloy54", 5.5), ("l3mix", "triclinic", None), ("l3mix", "slab", None), ("l3mix", "molecule", None),
+                ("l3wide", "fcc108", None), ("l3nat", "config1", None)]
 FIXTURE_CASES_2L = [(m, c) for m in ("grace_2l_small", "grace_2l_l3", "legacy_2l_small", "legacy_2l_wide") for c in ("W54", "WMo54")]
 
 
