@@ -39,8 +39,16 @@ MEASURED_TRAFFIC = {
 }
 
 
-def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4):
+def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4, radial_flops=59392.0, slots=None):
     """Roofline entry of one stage: algorithmic work / measured time."""
+    base = name.rsplit("_L", 1)[0] if slots else name     # GRACE-3L stages carry their layer: pair_fwd_L2, radial_L1 ...
+    if slots and base in ("pair_fwd", "pair_bwd"):
+        nslot = nI = slots[name[-1]]
+        name = base
+    elif slots and base in ("scatter_A", "bond_bwd"):
+        name = base
+    elif slots and base == "radial":
+        name = "radial_mlp"
     if name == "pair_fwd":
         # per edge: R1 row, Y, neighbour index, the neighbour's message rows; per atom: the pair tensor written once
         by = E * (s * C * nl + s * nlm + 4 + nslot * C * s) + N * nslot * nlm * C * s
@@ -51,7 +59,7 @@ def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4)
         return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
     if name in ("radial_mlp", "radial_R", "radial_R1"):
         # value + tangent through the 3 layers: 2 * 2 * E * sum n_in n_out
-        fl = 59392.0 * E
+        fl = radial_flops * E
         return {"bound": "mfma", "achieved": fl / (ms * 1e-3) / 1e12, "peak": PEAK[prec], "unit": "TFLOP/s", "work": fl}
     if name == "scatter_A":
         by = E * (s * C * nl + 4 + 24) + N * s * C * nlm
@@ -72,8 +80,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--precision", type=int, default=64, choices=[64, 32])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3"])
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4"])
     ap.add_argument("--reps", type=int, default=0, help="supercell repetitions (default: 16 bcc cells / 20 fcc cells per edge)")
+    ap.add_argument("--atoms", type=int, default=10000, help="atoms of the amorphous cube of config4")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives in the path); run with --gpus 1")
@@ -86,11 +95,20 @@ def main():
         sys.exit("bench.py: no GPU visible")
     tmp = tempfile.mkdtemp()
     two = a.workload == "config3"
-    if two and a.precision != 64:
-        sys.exit("bench.py: the GRACE-2L engine computes in fp64")
+    three = a.workload == "config4"
+    if (two or three) and a.precision != 64:
+        sys.exit("bench.py: the GRACE-2L and GRACE-3L engines compute in fp64")
     reps = a.reps or (20 if two else 16)
     pbc = [True, True, True]
-    if two:
+    if three:
+        mpath = cases.write_model("config4", tmp)
+        with np.load(mpath) as z:
+            names = [x.decode() for x in z["element_names"]]
+        pos, cell, _, t89 = cases.structure_config4(natoms=a.atoms)
+        # the 8 species present become atom types 1..8 of the engine (as a LAMMPS pair_coeff line would map them)
+        species = [names[t - 1] for t in cases.CONFIG4_SPECIES]
+        types = (np.searchsorted(np.array(cases.CONFIG4_SPECIES), t89) + 1).astype(np.int32)
+    elif two:
         mpath = cases.write_model("config3", tmp)
         species = ["Al", "Co", "Ni", "Ti"]
         pos, cell = synth.fcc_supercell(3.6, reps)
@@ -140,13 +158,15 @@ def main():
     eng.set_profile(False)
     stages = {k: v / a.steps for k, v in acc.items()}
 
-    C, nl, nlm, s = 32, 5, 25, a.precision // 8
+    C, nl, nlm, s = (64, 6, 36, 8) if three else (32, 5, 25, a.precision // 8)
+    # GRACE-3L: message functions gathered by the pair kernels of layers 2 and 3; radial MLP 8-128-128-384, value + tangent
+    extra = dict(radial_flops=4.0 * (8 * 128 + 128 * 128 + 128 * 384), slots={"2": 36, "3": 72}) if three else {}
     # FC flops (forward: left + right mat-vec per live function; reverse the same), fp64 FMAs on the vector/matrix pipes
     nA1, nAA1, nAA2 = 25, 44, 141       # informational; exact live counts are the engine's
     dense_flops = {}
     roof = {}
     for k, ms in stages.items():
-        r = stage_model(k, ms, E, N, C, nl, nlm, s, a.precision, dense_flops)
+        r = stage_model(k, ms, E, N, C, nl, nlm, s, a.precision, dense_flops, **extra)
         if r:
             r["ms"] = ms
             r["frac"] = r["achieved"] / r["peak"]
@@ -157,7 +177,7 @@ def main():
     d = modelled[dom]
     roofline = {"kernel": dom, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"],
                 "unit": d["unit"], "frac": round(d["frac"], 4),
-                "traffic": MEASURED_TRAFFIC.get((a.workload, dom)) if reps == (20 if two else 16) and a.precision == 64 else None,
+                "traffic": MEASURED_TRAFFIC.get((a.workload, dom)) if reps == (20 if two else 16) and a.atoms == 10000 and a.precision == 64 else None,
                 "avg_ms": round(d["ms"], 4), "algorithmic_work": d["work"]}
 
     cpu = None
@@ -165,7 +185,7 @@ def main():
         from oracle import ref_lib      # the compiled reference CPU path: the checker, timed here as the baseline
         if ref_lib.available():
             nth = len(os.sched_getaffinity(0))
-            ref = ref_lib.RefModel(mpath, list(range(len(species))))
+            ref = ref_lib.RefModel(mpath, [names.index(x) for x in species] if three else list(range(len(species))))
             args = dict(positions=pos[perm], image=image, shifts=shifts, nthreads=nth)
             ref.compute(types[perm], offset, j, **args)
             ts = []
@@ -176,7 +196,7 @@ def main():
                 ts.append(time.perf_counter() - t1)
             tm = float(np.median(ts))
             cpu = {"value": round(tm / N * 1e6, 4), "unit": "us/atom", "cores": nth, "kind": "reference",
-                   "sample": f"{len(ts)} full calls of the compiled reference Grace{2 if two else 1}LFused (fp32 + spline tables) on the same "
+                   "sample": f"{len(ts)} full calls of the compiled reference Grace{3 if three else 2 if two else 1}LFused (fp32 + spline tables) on the same "
                              f"{N}-atom structure, median",
                    "dE_per_atom_vs_gpu": abs(r["energy"] - out["energy"]) / N,
                    "max_dF_vs_gpu": float(np.abs(r["forces"] - out["forces"]).max())}
@@ -185,7 +205,10 @@ def main():
         "metric": "us_per_atom_EFS_call", "value": round(dt / N * 1e6, 5), "unit": "us/atom", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "f64" if a.precision == 64 else "f32", "data": "synthetic",
-        "config": {"workload": (f"GRACE-2L-shaped random-init model (2 layers, lmax 4, 32 ch, MLPs 8-64-64-160, body order 3) on the "
+        "config": {"workload": (f"GRACE-3L-shaped random-init model (3 layers, lmax 5, 64 ch, radial MLPs (8 + 2 x 32)-128-128-384, 89-species "
+                                f"embedding table, 8 species present) on an amorphous cube of {N} atoms at 0.08 / A^3, {E} edges, rc 6 A "
+                                f"(BASELINE configs[3])") if three else
+                               (f"GRACE-2L-shaped random-init model (2 layers, lmax 4, 32 ch, MLPs 8-64-64-160, body order 3) on the "
                                 f"4-species fcc alloy {reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[2])") if two else
                                (f"GRACE-1L-shaped random-init model (lmax 4, 32 ch, MLP 8-64-64-160) on bcc W "
                                 f"{reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[1])"),
