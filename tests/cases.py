@@ -66,13 +66,21 @@ def model_l3mix():
 
 
 def model_l3wide():
-    """GRACE-3L, four elements, lmax 3 with messages up to l = 2, channel and hidden widths that need padding
-    (20 -> 32, 48 -> 64), full RMSNorm of the densities, tanh readout"""
+    """GRACE-3L, four elements, lmax 3 with messages up to l = 2, a hidden width that needs padding (48 -> 64), full
+    RMSNorm of the densities, tanh readout"""
     d = synth.random_model_3l(lmax=3, lmsg=2, n_elements=4, element_names=("Al", "Co", "Ni", "Ti"), embedding_size=6, nradbase=8,
-                              channels=20, hidden=48, rho_n_out=12, energy_hidden=24, rcut=5.5, p=6,
+                              channels=32, hidden=48, rho_n_out=12, energy_hidden=24, rcut=5.5, p=6,
                               inv_avg_n_neigh=1.0 / 30.0, rms_type=0, seed=22)
     d["energy_mlp_activation"] = np.array([1], dtype=np.int64)
     return d
+
+
+def model_l3pad():
+    """GRACE-3L with 20 channels (padded to 32 on the GPU; the reference's CPU engine wants multiples of 16, so this
+    model is checked against the oracle only)"""
+    return synth.random_model_3l(lmax=2, lmsg=1, n_elements=2, element_names=("Mo", "W"), embedding_size=5, nradbase=6,
+                                 channels=20, hidden=24, rho_n_out=7, energy_hidden=12, rcut=5.0, inv_avg_n_neigh=1.0 / 26.0,
+                                 seed=24)
 
 
 def model_l3nat():
@@ -89,8 +97,8 @@ def model_config4():
                                  energy_hidden=64, rcut=6.0, inv_avg_n_neigh=1.0 / 72.0, seed=20260104)
 
 
-MODELS = {"l3mix": model_l3mix, "l3wide": model_l3wide, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
-LAYERS = {"l3mix": 3, "l3wide": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
+MODELS = {"l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
+LAYERS = {"l3mix": 3, "l3wide": 3, "l3pad": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
 
 
 def write_model(name, directory):

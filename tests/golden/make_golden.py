@@ -4,9 +4,12 @@ oracle/Makefile from the reference checkout) on the synthetic cases of tests/cas
 * its neighbour list (perm, offset, j, image, shifts) per structure            -> pins the host / device list
 * its energy, per-atom energies, forces, virial per (model, structure) case    -> pins the oracle and the HIP path
   on models the reference's own TF goldens do not cover (AAAA stage, A width != FC width, pair cutoffs, lmax 3/4,
-  GRACE-2L at lmax 4 and with unequal stage widths, the reference's 2L fixture models with the BBBB stage)
+  GRACE-2L at lmax 4 and with unequal stage widths, the reference's 2L fixture models with the BBBB stage, and every
+  GRACE-3L case: the reference checkout holds no 3L model file, so its compiled drivers on generated models are the
+  only reference outputs there are)
 
-Run in the build container (needs oracle/_ref):  python tests/golden/make_golden.py
+Run in the build container (needs oracle/_ref):  python tests/golden/make_golden.py [--all]
+Cases already in the file are kept as they are unless --all is given.
 """
 import os
 import sys
@@ -25,9 +28,15 @@ from oracle import ref_lib  # noqa: E402
 
 def main():
     out = {}
+    target = os.path.join(cases.GOLDEN, "reference_outputs.npz")
+    if "--all" not in sys.argv and os.path.exists(target):
+        with np.load(target) as z:
+            out = {k: z[k] for k in z.files}
     tmp = tempfile.mkdtemp()
     lists = {}
-    for model, struct, rc_list in cases.E2E_CASES + cases.E2E_CASES_2L:
+    for model, struct, rc_list in cases.E2E_CASES + cases.E2E_CASES_2L + cases.E2E_CASES_3L:
+        if f"e2e/{model}/{struct}/energy" in out:
+            continue
         path = cases.write_model(model, tmp)
         d = cases.MODELS[model]()
         nel = int(d["n_elements"][0])
@@ -41,7 +50,7 @@ def main():
         if key not in lists:
             lists[key] = nl
             for k, v in nl.items():
-                out[f"nl/{key}/{k}"] = v
+                out.setdefault(f"nl/{key}/{k}", v)
         r = ref.compute(types[nl["perm"]], nl["offset"], nl["j"], positions=pos[nl["perm"]], image=nl["image"],
                         shifts=nl["shifts"] if len(nl["shifts"]) else np.zeros((1, 3)), nthreads=2)
         tag = f"e2e/{model}/{struct}"
@@ -51,6 +60,8 @@ def main():
         print(tag, key, "bonds", len(nl["j"]), "E", r["energy"], "max|F|", np.abs(r["forces"]).max())
     # the reference's own 2L fixture models without TF goldens, on its fixture cells (CSR bonds as stored there)
     for model, cell in cases.FIXTURE_CASES_2L:
+        if f"fixture/{model}/{cell}/energy" in out:
+            continue
         with np.load(os.path.join(cases.REF_FIXTURES, cell + ".npz")) as c:
             types = np.array([2 if z == 74 else 1 for z in c["numbers"]], dtype=np.int32)
             offset, j, rij = c["offset"], c["j"], c["rij"]
@@ -60,7 +71,7 @@ def main():
         for k in ("energy", "energies", "forces", "virial"):
             out[f"{tag}/{k}"] = np.asarray(r[k])
         print(tag, "E", r["energy"], "max|F|", np.abs(r["forces"]).max())
-    np.savez(os.path.join(cases.GOLDEN, "reference_outputs.npz"), **out)
+    np.savez(target, **out)
 
 
 if __name__ == "__main__":

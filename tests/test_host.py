@@ -84,12 +84,62 @@ def test_malformed_2l_models_are_rejected(tmp_path, k):
         kk.Model(_mutated_2l(tmp_path, fn))
 
 
+def _mutated_3l(tmp_path, fn):
+    d = cases.model_l3mix()
+    fn(d)
+    p = str(tmp_path / "m3.npz")
+    np.savez(p, **{k: v for k, v in d.items() if not k.startswith("_")})
+    return p
+
+
+def test_3l_model_loads(tmp_path):
+    m = kk.Model(_mutated_3l(tmp_path, lambda d: None))
+    assert m.layers == 3 and m.element_names == ["Mo", "W"] and m.rcut == 5.0
+
+
+def _drop_name(d, key, name):
+    d[key] = np.array([x for x in d[key] if x != name.encode()], dtype=d[key].dtype)
+
+
+BAD_3L = [
+    (lambda d: d.pop("A2_cg_W"), "required weight 'A2_cg_W' missing"),
+    (lambda d: d.update(A2_cg_W=d["A2_cg_W"][:-1]), "A2_cg_W' has shape"),
+    (lambda d: d.update(A1_mlp_W0=d["A1_mlp_W0"][:-1]), "A1_mlp_W0"),
+    (lambda d: d.update(A1_mlp_b0=d["A1_mlp_b0"][:-1]), "A1_mlp_b0' has 31 values, expected 32"),
+    (lambda d: d.update(A3_equivariant=np.array([0]), A3_lin_transform_W=d["A1_lin_transform_W"]), "A3_equivariant' is 0, expected 1"),
+    (lambda d: d.update(A1_equivariant=np.array([1])), "A1_"),
+    (lambda d: _drop_name(d, "prod_names", "A2_3"), "prod_names' has no 'A2_3'"),
+    (lambda d: d.update(prod_names=np.concatenate([d["prod_names"], np.array([b"A1_2"], dtype=d["prod_names"].dtype)])), "lists 'A1_2' twice"),
+    (lambda d: _drop_name(d, "reduce_names", "eq1"), "reduce_names' has no 'eq1'"),
+    (lambda d: d.update(A1_2_left_ind=d["A1_2_left_ind"] + 1000), "A1_2_left_ind' has"),
+    (lambda d: d.update(A1_2_group_left=d["A1_2_group_left"][:-1]), "A1_2_left_ind' has 8 at"),
+    (lambda d: d.update(A2_3_U=d["A2_3_U"][:, :, :-1]), "A2_3_U' has shape"),
+    (lambda d: d.update(fc_A1_2a_left_coefs=np.array([1])), "fc_A1_2a_left_coefs"),
+    (lambda d: d.update(fc_A1_2a_collect_from=d["fc_A1_2a_collect_from"] + 100), "fc_A1_2a_collect_from' has"),
+    (lambda d: d.update(eq1_instruction_names=d["eq1_instruction_names"][:-1]), "eq1_instruction_names"),
+    (lambda d: d.update(eq1_norm_l0_mask=d["eq1_norm_l0_mask"][:-1]), "eq1_norm_l0_mask' has 8 values, expected 9"),
+    (lambda d: d.update(rho2_norm_scale=d["rho2_norm_scale"][:-1]), "rho2_norm_scale' has 7 values, expected 8"),
+    (lambda d: d.update(out1_origins=d["out1_origins"][:2], energy_mlp_n_origins=np.array([2])), "out1_origins"),
+    (lambda d: d.update(energy_mlp_W0=d["energy_mlp_W0"][:-1]), "energy_mlp_W0"),
+    (lambda d: d.update(A2_p=np.array([6])), "A2_p' is 6, the envelope order of A1 is 5"),
+    (lambda d: d.update(radial_activation=np.array([0])), "radial_activation' is a legacy GRACE-1L/2L key"),
+    (lambda d: d.update(A2_n_lm_ind=np.array([5])), "A2_"),
+]
+
+
+@pytest.mark.parametrize("k", range(len(BAD_3L)))
+def test_malformed_3l_models_are_rejected(tmp_path, k):
+    fn, msg = BAD_3L[k]
+    with pytest.raises((RuntimeError, ValueError), match=re.escape(msg)):
+        kk.Model(_mutated_3l(tmp_path, fn))
+
+
 def test_rejects_other_model_kinds_and_missing_files(tmp_path):
     d = cases.model_cut2()
     d["grace_model_kind"] = np.array([b"GRACE-3L"], dtype="|S8")
     p3 = str(tmp_path / "m3.npz")
     np.savez(p3, **d)
-    with pytest.raises(ValueError, match="GRACE-3L"):
+    with pytest.raises(RuntimeError, match="n_elements|spbf_names|A1_"):     # a 1L file labelled 3L: no 3L component is found
         kk.Model(p3)
     with pytest.raises(RuntimeError, match="cannot read the model file"):
         kk.Model(str(tmp_path / "nope.npz"))

@@ -121,3 +121,78 @@ def test_random_model_2l_file_layout(tmp_path):
         assert int(z["B_n_funcs"][0]) == 49 and int(z["prod_BB_n_output_funcs"][0]) == 197
         assert z["B_reduce_YI_W"].shape[:2] == (32, 32) and z["I_reduce_I1_W"].shape == (32, 16, 2)
         assert "prod_AAAA_n_cg_terms" not in z.files and "prod_BBBB_n_cg_terms" not in z.files
+
+
+def test_structure_3l_shares_the_couplings_of_the_exported_1l_models(sref):
+    """The first cp_l product of a GRACE-3L layer couples X with itself exactly as the AA product of GRACE-1L does: the
+    same (l1 >= l2) -> L paths with the same coefficients.  Compared with the reference's lmax-4 export, term by term
+    as a set of (left, right, coefficient) triples per (L, l1, l2, M)."""
+    s = synth.structure_3l(4, pseudo_message=False)
+    li, ri, oi, cg = s["A1_2_left_ind"], s["A1_2_right_ind"], s["A1_2_m_sum_ind"], s["A1_2_cg"]
+    assert int(s["A1_2_nfunc"][0]) == int(sref["grace_1l_w48/prod_AA_n_output_funcs"][0]) == 141
+    lm_l = np.repeat(np.arange(5), 2 * np.arange(5) + 1)
+    out_l = s["A1_2_out_l"]
+
+    def table(l, r, o, c, ol):
+        # function o of a path (L, l1, l2) -> its M by counting within the run of equal (L, l1, l2)
+        t = {}
+        first = {}
+        for a, b, f, v in zip(l, r, o, c):
+            key = (int(ol[f]), int(lm_l[a]), int(lm_l[b]))
+            first.setdefault(key, int(f))
+            first[key] = min(first[key], int(f))
+        for a, b, f, v in zip(l, r, o, c):
+            key = (int(ol[f]), int(lm_l[a]), int(lm_l[b]))
+            t.setdefault(key + (int(f) - first[key],), {})
+            pair = (int(a), int(b)) if a >= b or lm_l[a] != lm_l[b] else (int(b), int(a))
+            t[key + (int(f) - first[key],)][pair] = t[key + (int(f) - first[key],)].get(pair, 0.0) + float(v)
+        return t
+    rl, rr, ro, rc = (sref[f"grace_1l_w48/prod_AA_{k}"] for k in ("left_ind", "right_ind", "m_sum_ind", "cg_coeff"))
+    # l of each AA function of the export: from the L = 0..4 block structure of its FC tiles
+    ref_ol = np.zeros(141, int)
+    groups = synth._aa_groups(4, 4)
+    f = 0
+    for (L, l1, l2) in groups:
+        ref_ol[f:f + 2 * L + 1] = L
+        f += 2 * L + 1
+    a, b = table(li, ri, oi, cg, out_l), table(rl, rr, ro, rc, ref_ol)
+    assert set(a) == set(b)
+    for key in a:
+        assert set(a[key]) == set(b[key]), key
+        for pair in a[key]:
+            assert abs(a[key][pair] - b[key][pair]) < 2e-7, (key, pair)
+
+
+@pytest.mark.parametrize("lmax,pseudo", [(2, True), (3, False)])
+def test_structure_3l_index_ranges(lmax, pseudo):
+    s = synth.structure_3l(lmax, pseudo_message=pseudo)
+    z = s["_sizes"]
+    nlm = (lmax + 1) ** 2
+    for k in (1, 2, 3):
+        K = f"A{k}"
+        for q in ("2", "3", "4"):
+            P = f"{K}_{q}"
+            assert s[P + "_m_sum_ind"].max() == z[P]["nfunc"] - 1
+            assert s[P + "_left_ind"].max() < len(s[P + "_group_left"]) and s[P + "_right_ind"].max() < len(s[P + "_group_right"])
+            R = P + "_red"
+            assert len(s[f"{R}_collect_ind_{P}"]) == z[P]["nfunc"]
+            assert s[f"{R}_w_l_tile_{P}"].max() == z[P]["npaths"] - 1
+            assert s[f"{R}_total_sum_ind_{P}"].max() < int(s[R + "_n_funcs"][0])
+        if k > 1:
+            W = s[K + "_cg_W"]
+            assert W.shape == (nlm * int(s[K + "_n_lm_ind"][0]), int(s[K + "_nfunc"][0]))
+            assert (np.abs(W).sum(0) > 0).all()              # every coupled function has terms
+    assert int(s["A2_n_lm_ind"][0]) == (lmax + 1) ** 2
+    assert int(s["A3_n_lm_ind"][0]) == (2 if pseudo else 1) * (lmax + 1) ** 2
+
+
+def test_random_model_3l_file_layout(tmp_path):
+    d = cases.model_l3mix()
+    p = str(tmp_path / "m.npz")
+    synth.save_model(p, d)
+    with np.load(p) as zf:
+        assert [x.decode() for x in zf["spbf_names"]] == ["A1", "A2", "A3"]
+        assert len(zf["prod_names"]) == 9 and len(zf["fc_names"]) == 6 and len(zf["reduce_names"]) == 16
+        assert zf["A1_mlp_W0"].shape == (10 + 2 * 8, 32) and zf["A1_mlp_W2"].shape == (32, 16 * 3)
+        assert zf["rho1_reduce_A1_W"].shape[0] == 2 and zf["eq1_reduce_A1_W"].ndim == 3
+        assert not any(k.startswith("_") for k in zf.files)
