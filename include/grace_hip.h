@@ -51,8 +51,9 @@ int gr_abi_version(void);
 int gr_device_count(void);
 int gr_device_arch(int device, char *buf, int len);
 
-/* Load a kokkos.npz model (GRACE1LModel::load, libgrace/src/model_1l.cpp:16; kind by grace::model_kind,
- * libgrace/include/grace/model_kind.h:19).  The same validation errors as the reference loader. */
+/* Load a kokkos.npz model: GRACE1LModel::load (libgrace/src/model_1l.cpp:16), GRACE2LModel::load
+ * (libgrace/src/model_2l.cpp:26), GRACE3LModel::load (libgrace/src/model_3l.cpp:163); kind by grace::model_kind,
+ * libgrace/include/grace/model_kind.h:19.  The same validation errors as the reference loaders. */
 int gr_model_load(const char *npz_path, gr_model **out);
 int gr_model_get_info(const gr_model *m, gr_model_info *info);
 /* element name k (0 <= k < n_elements), "" when the file has none: Model.element_names, python/kk/kk_api.h:56 */
@@ -60,9 +61,11 @@ const char *gr_model_element_name(const gr_model *m, int k);
 void gr_model_free(gr_model *m);
 
 /* An engine for one type map: type2mu has ntypes + 1 entries, types are 1-based, type2mu[t] = model element or -1.
- * Grace1LFused(model, settings, log) + setup_types(ntypes, type2mu): libgrace/include/grace/fused_1l.h:28-31;
- * Grace1LKK::set_model / setup: libgrace/include/grace/kk/grace_1l_kk.h:72-79.
- * precision 64: network arithmetic in fp64; 32: fp32 network, fp64 geometry and sums (docs/advanced.md:37-38). */
+ * Grace1LFused(model, settings, log) + setup_types(ntypes, type2mu): libgrace/include/grace/fused_1l.h:28-31, likewise
+ * Grace2LFused (fused_2l.h:32-39) and Grace3LFused (fused_3l.h:26-34); Grace1LKK::set_model / setup:
+ * libgrace/include/grace/kk/grace_1l_kk.h:72-79.
+ * precision 64: network arithmetic in fp64; 32: fp32 network, fp64 geometry and sums (docs/advanced.md:37-38; GRACE-1L
+ * only, GR_INVALID for GRACE-2L / 3L models). */
 int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int precision, int device, gr_engine **out);
 void gr_engine_free(gr_engine *e);
 /* Grace1LFused::cutoff(t1, t2): fused_1l.h:32 */
