@@ -22,6 +22,7 @@ namespace grhip {
 namespace {
 
 inline int pad_width(int c) { return c <= 16 ? 16 : c <= 32 ? 32 : c <= 64 ? 64 : -1; }
+constexpr size_t kCoupleLdsMax = 158 * 1024;    // projections of one atom staged in LDS by the couple kernels
 
 // out[dst][k] (+)= dscale[dst] sum over connections (src, dst, tile) of sum_n W[tile][n][k] in[src][n]; reverse:
 // gin[src][n] += sum over its connections of dscale[dst] sum_k W[tile][n][k] gout[dst][k]   (fused_3l_cpu.h:84-221)
@@ -32,6 +33,7 @@ template<class T> struct DevContract {
   DevBuf WF, WT;
   DevJobs<T> fwd, bwd;
   int kin = 0, kout = 0, nsrc = 0, ndst = 0;    // padded widths, functions of the source and destination tensors
+  bool all_dst = false, all_src = false;        // every destination / source function has a connection
   template<class WGet>
   void build(int nin, int nout, int nt, const std::vector<Conn> &conns, WGet wget, const std::vector<double> &dscale, int nsrc_, int ndst_,
              const int *drow, const std::string &what)
@@ -62,6 +64,9 @@ template<class T> struct DevContract {
       by_dst[conns[c].dst].push_back((int) c);
       by_src[conns[c].src].push_back((int) c);
     }
+    all_dst = all_src = true;
+    for (const auto &v : by_dst) all_dst = all_dst && !v.empty();
+    for (const auto &v : by_src) all_src = all_src && !v.empty();
     auto sc = [&](int d) { return dscale.empty() ? 1.0 : dscale[d]; };
     typename DevJobs<T>::Host hf, hb;
     for (int d = 0; d < ndst; d++) {
@@ -118,6 +123,8 @@ struct Ten {
 template<class T> struct ProdStage {
   DevContract<T> U, V, red;
   DevProd cp;
+  DevBuf tl, tr, to, tc;    // the terms sorted by output, for the LDS couple kernels
+  CoupleDev cd{};
   int nfunc = 0, rankP = 0;
   bool jit = false;
 };
@@ -185,6 +192,17 @@ template<class T> class Engine3L final : public EngineBase {
   void cfwd(DevContract<T> &c, const T *X, T *out, int accumulate) { gemm(c.fwd, c.kin, c.kout, X, c.nsrc, out, c.ndst, accumulate); }
   void cbwd(DevContract<T> &c, const T *gout, T *gX, int accumulate) { gemm(c.bwd, c.kout, c.kin, gout, c.ndst, gX, c.nsrc, accumulate); }
   void zero(void *p, size_t bytes) { if (bytes) HIP_CHECK(hipMemsetAsync(p, 0, bytes, stream_)); }
+  // out = contraction (not accumulated): functions without a connection are cleared
+  void cfwd_set(DevContract<T> &c, const T *X, T *out)
+  {
+    if (!c.all_dst) zero(out, (size_t) n_ * c.ndst * c.kout * sizeof(T));
+    cfwd(c, X, out, c.all_dst ? 0 : 1);
+  }
+  void cbwd_set(DevContract<T> &c, const T *gout, T *gX)
+  {
+    if (!c.all_src) zero(gX, (size_t) n_ * c.nsrc * c.kin * sizeof(T));
+    cbwd(c, gout, gX, c.all_src ? 0 : 1);
+  }
   void couple_fwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, T *out);
   void couple_bwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, const T *g, T *gL, T *gR);
   void scale_rows(const T *in, const DevBuf &s, T *out, int nf, int w, int accumulate)
@@ -360,6 +378,17 @@ template<class T> void Engine3L<T>::build_layer(int k)
     if (h.terms.size() <= 1500)
       jit_compile_product((c.name + "_cp").c_str(), h.terms, nfl, nfr, c.nfunc, false, P.rankP, sizeof(T) == 4, arch_, P.cp.jit, P.cp.jit_note);
     P.jit = P.cp.jit.ok();
+    {
+      std::vector<int> tl, tr, to;
+      std::vector<double> tc;
+      for (const ProdTerm &t : h.terms) { tl.push_back(t.l); tr.push_back(t.r); to.push_back(t.o); tc.push_back(t.c); }
+      if (tl.empty()) { tl.push_back(0); tr.push_back(0); to.push_back(0); tc.push_back(0.0); }
+      upload_vec(P.tl, tl); upload_vec(P.tr, tr); upload_vec(P.to, to); upload_vec(P.tc, tc);
+      P.cd.l = P.tl.template as<int>(); P.cd.r = P.tr.template as<int>(); P.cd.o = P.to.template as<int>(); P.cd.c = P.tc.template as<double>();
+      P.cd.off = P.cp.off.template as<int>();
+      P.cd.nout = c.nfunc;
+      P.cd.nterms = (int) h.terms.size();
+    }
     instr_contract(P.red, r, r.instr[0], c.nfunc, r.name);
     Lp.nf = nfl;
     Rp.nf = nfr;
@@ -446,6 +475,14 @@ template<class T> void Engine3L<T>::couple_fwd(ProdStage<T> &p, const T *Lp, int
     HIP_CHECK(hipModuleLaunchKernel(p.cp.jit.fwd, (unsigned) ((cols + 255) / 256), 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
     return;
   }
+  const int ATl = 64 / KP;
+  const size_t lds = (size_t) ATl * (nfl + nfr) * KP * sizeof(T);
+  if (lds <= kCoupleLdsMax && p.cd.nterms > 0) {
+    auto kern = k_couple_fwd_lds<T>;
+    if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+    hipLaunchKernelGGL(kern, dim3((n + ATl - 1) / ATl), dim3(p.cd.nout >= 256 ? 1024 : 256), lds, stream_, p.cd, Lp, Rp, out, KP, nfl, nfr, n);
+    return;
+  }
   const int AT = std::max(1, 256 / KP);
   hipLaunchKernelGGL(k_prod_fwd<T>, dim3(p.cp.d.nout * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, p.cp.d, Lp, Rp, out, n, KP, nfl, nfr);
 }
@@ -459,6 +496,14 @@ template<class T> void Engine3L<T>::couple_bwd(ProdStage<T> &p, const T *Lp, int
     void *args[] = {(void *) &Lp, (void *) &Rp, (void *) &g, (void *) &gL, (void *) &gR, (void *) &acc, (void *) &acc, (void *) &nat, (void *) &one};
     const long long cols = (long long) n * KP;
     HIP_CHECK(hipModuleLaunchKernel(p.cp.jit.bwd, (unsigned) ((cols + 255) / 256), 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+    return;
+  }
+  const int ATl = 64 / KP;
+  const size_t lds = (size_t) 2 * ATl * (nfl + nfr) * KP * sizeof(T);
+  if (lds <= kCoupleLdsMax && p.cd.nterms > 0) {
+    auto kern = k_couple_bwd_lds<T>;
+    if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+    hipLaunchKernelGGL(kern, dim3((n + ATl - 1) / ATl), dim3(p.cd.nout >= 256 ? 1024 : 256), lds, stream_, p.cd, Lp, Rp, g, gL, gR, KP, nfl, nfr, n);
     return;
   }
   const int AT = std::max(1, 256 / KP);
@@ -524,10 +569,7 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
       hipLaunchKernelGGL(k_lincomb<T>, dim3(n, (L.nfA * L.CP + 255) / 256), dim3(256), 0, stream_, L.cg.off.template as<int>(), L.cg.idx.template as<int>(),
                          L.cg.val.template as<double>(), (const T *) pairP_.as<T>(), A_.as<T>(), npf, L.nfA, L.CP);
     });
-    stage(tg(k, "reduce_A").c_str(), [&] {
-      zero(X, L.X.bytes(na, s));
-      cfwd(L.redA, A_.as<T>(), X, 1);
-    });
+    stage(tg(k, "reduce_A").c_str(), [&] { cfwd_set(L.redA, A_.as<T>(), X); });
   }
   // ---- chain (fused_3l.cpp:970-990)
   const int nX = L.X.nf, wX = L.X.w, wR = L.wR;
@@ -542,16 +584,14 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
   for (Ten *t : {&L.L2, &L.R2p, &L.L3, &L.R3p, &L.L4, &L.R4p}) t->buf.ensure(t->bytes(na, s));
   T *P = P_.as<T>(), *R2 = R2_.as<T>(), *R3 = R3_.as<T>(), *R4 = R4_.as<T>(), *FA = FA_.as<T>(), *FB = FB_.as<T>();
   auto prod = [&](const char *name, ProdStage<T> &p, const T *XL, const T *XR, Ten &Lp, Ten &Rp, T *Rout, int nfred) {
+    (void) nfred;
     T *lp = Lp.buf.template as<T>(), *rp = Rp.buf.template as<T>();
     stage(tg(k, (std::string("proj_") + name).c_str()).c_str(), [&] {
       cfwd(p.U, XL, lp, 0);
       cfwd(p.V, XR, rp, 0);
     });
     stage(tg(k, (std::string("couple_") + name).c_str()).c_str(), [&] { couple_fwd(p, lp, Lp.nf, rp, Rp.nf, P); });
-    stage(tg(k, (std::string("reduce_") + name).c_str()).c_str(), [&] {
-      zero(Rout, na * nfred * wR * s);
-      cfwd(p.red, P, Rout, 1);
-    });
+    stage(tg(k, (std::string("reduce_") + name).c_str()).c_str(), [&] { cfwd_set(p.red, P, Rout); });
   };
   auto fc = [&](const char *name, FcStage<T> &F, T *out) {
     stage(tg(k, name).c_str(), [&] {
@@ -652,10 +692,7 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   // gXL / gXR: where the adjoints of the product's inputs are added
   auto prod_bwd = [&](const char *name, ProdStage<T> &p, Ten &Lp, Ten &Rp, const T *gR, T *gXL, T *gXR) {
     const T *lp = Lp.buf.template as<T>(), *rp = Rp.buf.template as<T>();
-    stage(tg(k, (std::string("reduce_") + name + "_bwd").c_str()).c_str(), [&] {
-      zero(gP, na * p.nfunc * p.rankP * s);
-      cbwd(p.red, gR, gP, 1);
-    });
+    stage(tg(k, (std::string("reduce_") + name + "_bwd").c_str()).c_str(), [&] { cbwd_set(p.red, gR, gP); });
     stage(tg(k, (std::string("couple_") + name + "_bwd").c_str()).c_str(), [&] {
       zero(gLp, Lp.bytes(na, s));
       zero(gRp, Rp.bytes(na, s));
@@ -692,10 +729,7 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   gpairP_.ensure(na * npf * L.CP * s);
   M_.ensure(na * L.nlmi * L.CP * s);
   gM_.ensure(na * L.nlmi * L.CP * s);
-  stage(tg(k, "reduce_A_bwd").c_str(), [&] {
-    zero(gA_.p, na * L.nfA * L.CP * s);
-    cbwd(L.redA, gX, gA_.as<T>(), 1);
-  });
+  stage(tg(k, "reduce_A_bwd").c_str(), [&] { cbwd_set(L.redA, gX, gA_.as<T>()); });
   stage(tg(k, "couple_YI_bwd").c_str(), [&] {
     hipLaunchKernelGGL(k_lincomb<T>, dim3(n, (npf * L.CP + 255) / 256), dim3(256), 0, stream_, L.cgt.off.template as<int>(), L.cgt.idx.template as<int>(),
                        L.cgt.val.template as<double>(), (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP);

@@ -157,6 +157,8 @@ template<class T> struct DevJobs {
     d.seg_src = seg_src.as<int>(); d.seg_fn = seg_fn.as<int>(); d.seg_w = seg_w.as<int>(); d.seg_scale = seg_scale.as<T>();
     d.WF0 = WF0; d.WF1 = WF1;
     d.njobs = (int) h.job_out.size();
+    d.max_seg = 0;
+    for (size_t q = 0; q + 1 < h.seg_off.size(); q++) d.max_seg = std::max(d.max_seg, h.seg_off[q + 1] - h.seg_off[q]);
   }
   void set_rows(const int *drow) { for (int q = 0; q < 16; q++) d.drow[q] = drow[q]; }
 };
@@ -742,13 +744,16 @@ class EngineBase : public Engine {
     if (J.d.njobs == 0 || ntiles == 0) return;
     const int ksm = std::max(kb0, kb1) * 4;
     const size_t lds = (size_t) kGemmMaxSeg * nb * ksm * 64 * sizeof(T);
-    const dim3 grid(J.d.njobs, (ntiles + 4 * kGemmTilesPerWave - 1) / (4 * kGemmTilesPerWave));
+    // jobs whose weight tiles fit one staging walk several groups of atom tiles per block (less re-staging)
+    const int groups = (ntiles + 4 * kGemmTilesPerWave - 1) / (4 * kGemmTilesPerWave);
+    const int reps = J.d.max_seg <= kGemmMaxSeg ? std::max(1, std::min(8, (int) ((long long) J.d.njobs * groups / 2048))) : 1;
+    const dim3 grid(J.d.njobs, (groups + reps - 1) / reps);
 #define GR_GEMM(A_, B_, C_)                                                                                            \
   {                                                                                                                    \
     auto kern = k_gemm_jobs<T, A_, B_, C_>;                                                                            \
     if (lds > 48 * 1024)                                                                                               \
       HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, J.d, X0, nf0, X1, nf1, out, nfo, tiles, ntiles, accumulate); \
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, J.d, X0, nf0, X1, nf1, out, nfo, tiles, ntiles, accumulate, reps); \
   }
 #define GR_GEMM_C(A_, B_)                                                                                              \
   switch (nb) {                                                                                                        \

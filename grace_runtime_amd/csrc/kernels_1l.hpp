@@ -652,6 +652,7 @@ template<class T> struct GemmJobs {
   const T *seg_scale;         // [nseg]
   const T *WF0, *WF1;         // fragments of the weights used with X0 / X1
   int njobs;
+  int max_seg;                // most segments of one job
   int drow[16];               // accumulator row of (lane / 16, register), probed on the device
 };
 
@@ -660,8 +661,10 @@ constexpr int kGemmTilesPerWave = 2;
 
 template<class T, int KB0, int KB1, int NB>
 __global__ __launch_bounds__(256) void k_gemm_jobs(GemmJobs<T> J, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo,
-                                                   const int *tile_atoms, int ntiles, int accumulate)
+                                                   const int *tile_atoms, int ntiles, int accumulate, int reps)
 {
+  // reps > 1 (only when every job has at most kGemmMaxSeg segments): the block stages its weight tiles once and walks
+  // `reps` groups of atom tiles with them
   typedef typename Mfma<T>::v4 v4;
   constexpr int KS0 = KB0 * 4, KS1 = KB1 * 4, KSM = KS0 > KS1 ? KS0 : KS1, K0 = KB0 * 16, K1 = KB1 * 16, N = NB * 16;
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -673,81 +676,87 @@ __global__ __launch_bounds__(256) void k_gemm_jobs(GemmJobs<T> J, const T *X0, i
   const int c = lane & 15, g = lane >> 4;
   const int sg0 = J.seg_off[job], sg1 = J.seg_off[job + 1];
   const int fo = J.job_out[job];
-  v4 acc[kGemmTilesPerWave][NB];
-  int arow[kGemmTilesPerWave];            // atom of this lane's A row
-#pragma unroll
-  for (int i = 0; i < kGemmTilesPerWave; i++) {
-    const int tile = (blockIdx.y * 4 + wave) * kGemmTilesPerWave + i;
-    arow[i] = tile < ntiles ? tile_atoms[tile * 16 + c] : -1;
-#pragma unroll
-    for (int cb = 0; cb < NB; cb++) acc[i][cb] = v4{0, 0, 0, 0};
-  }
-  for (int sg = sg0; sg < sg1; sg += kGemmMaxSeg) {
-    const int ns = sg1 - sg < kGemmMaxSeg ? sg1 - sg : kGemmMaxSeg;
-    __syncthreads();
-    for (int q = 0; q < ns; q++) {
-      const int src = J.seg_src[sg + q];
-      const int ks = src == 0 ? KS0 : KS1;
-      const T *wf = (src == 0 ? J.WF0 : J.WF1) + (long long) J.seg_w[sg + q] * NB * ks * 64;
-      for (int e = threadIdx.x; e < NB * ks * 64; e += 256) {
-        const int cb = e / (ks * 64), rem = e % (ks * 64);
-        wl[(q * NB + cb) * KSM * 64 + rem] = wf[e];
-      }
-      if (threadIdx.x == 0) { s_src[q] = src; s_fn[q] = J.seg_fn[sg + q]; s_scale[q] = J.seg_scale[sg + q]; }
-    }
-    __syncthreads();
+  const T js = J.job_scale[job];
+  for (int rep = 0; rep < reps; rep++) {
+    const int tile0 = ((blockIdx.y * reps + rep) * 4 + wave) * kGemmTilesPerWave;
+    if (rep > 0 && (blockIdx.y * reps + rep) * 4 * kGemmTilesPerWave >= ntiles) break;    // uniform over the block
+    v4 acc[kGemmTilesPerWave][NB];
+    int arow[kGemmTilesPerWave];            // atom of this lane's A row
 #pragma unroll
     for (int i = 0; i < kGemmTilesPerWave; i++) {
-      for (int q = 0; q < ns; q++) {
-        const T sc = s_scale[q];
-        const T *wq = wl + q * NB * KSM * 64 + lane;
-        if (s_src[q] == 0) {
-          T x[KS0];
-          if (arow[i] >= 0) {
-            const T *xp = X0 + ((long long) arow[i] * nf0 + s_fn[q]) * K0 + g * KS0;
+      const int tile = tile0 + i;
+      arow[i] = tile < ntiles ? tile_atoms[tile * 16 + c] : -1;
 #pragma unroll
-            for (int s = 0; s < KS0; s++) x[s] = xp[s] * sc;
-          } else {
-#pragma unroll
-            for (int s = 0; s < KS0; s++) x[s] = (T) 0;
+      for (int cb = 0; cb < NB; cb++) acc[i][cb] = v4{0, 0, 0, 0};
+    }
+    for (int sg = sg0; sg < sg1; sg += kGemmMaxSeg) {
+      const int ns = sg1 - sg < kGemmMaxSeg ? sg1 - sg : kGemmMaxSeg;
+      if (rep == 0) {
+        __syncthreads();
+        for (int q = 0; q < ns; q++) {
+          const int src = J.seg_src[sg + q];
+          const int ks = src == 0 ? KS0 : KS1;
+          const T *wf = (src == 0 ? J.WF0 : J.WF1) + (long long) J.seg_w[sg + q] * NB * ks * 64;
+          for (int e = threadIdx.x; e < NB * ks * 64; e += 256) {
+            const int cb = e / (ks * 64), rem = e % (ks * 64);
+            wl[(q * NB + cb) * KSM * 64 + rem] = wf[e];
           }
+          if (threadIdx.x == 0) { s_src[q] = src; s_fn[q] = J.seg_fn[sg + q]; s_scale[q] = J.seg_scale[sg + q]; }
+        }
+        __syncthreads();
+      }
 #pragma unroll
-          for (int cb = 0; cb < NB; cb++)
+      for (int i = 0; i < kGemmTilesPerWave; i++) {
+        for (int q = 0; q < ns; q++) {
+          const T sc = s_scale[q];
+          const T *wq = wl + q * NB * KSM * 64 + lane;
+          if (s_src[q] == 0) {
+            T x[KS0];
+            if (arow[i] >= 0) {
+              const T *xp = X0 + ((long long) arow[i] * nf0 + s_fn[q]) * K0 + g * KS0;
 #pragma unroll
-            for (int s = 0; s < KS0; s++) acc[i][cb] = Mfma<T>::mma(x[s], wq[(cb * KSM + s) * 64], acc[i][cb]);
-        } else {
-          T x[KS1];
-          if (arow[i] >= 0) {
-            const T *xp = X1 + ((long long) arow[i] * nf1 + s_fn[q]) * K1 + g * KS1;
+              for (int s = 0; s < KS0; s++) x[s] = xp[s] * sc;
+            } else {
 #pragma unroll
-            for (int s = 0; s < KS1; s++) x[s] = xp[s] * sc;
+              for (int s = 0; s < KS0; s++) x[s] = (T) 0;
+            }
+#pragma unroll
+            for (int cb = 0; cb < NB; cb++)
+#pragma unroll
+              for (int s = 0; s < KS0; s++) acc[i][cb] = Mfma<T>::mma(x[s], wq[(cb * KSM + s) * 64], acc[i][cb]);
           } else {
+            T x[KS1];
+            if (arow[i] >= 0) {
+              const T *xp = X1 + ((long long) arow[i] * nf1 + s_fn[q]) * K1 + g * KS1;
 #pragma unroll
-            for (int s = 0; s < KS1; s++) x[s] = (T) 0;
+              for (int s = 0; s < KS1; s++) x[s] = xp[s] * sc;
+            } else {
+#pragma unroll
+              for (int s = 0; s < KS1; s++) x[s] = (T) 0;
+            }
+#pragma unroll
+            for (int cb = 0; cb < NB; cb++)
+#pragma unroll
+              for (int s = 0; s < KS1; s++) acc[i][cb] = Mfma<T>::mma(x[s], wq[(cb * KSM + s) * 64], acc[i][cb]);
           }
-#pragma unroll
-          for (int cb = 0; cb < NB; cb++)
-#pragma unroll
-            for (int s = 0; s < KS1; s++) acc[i][cb] = Mfma<T>::mma(x[s], wq[(cb * KSM + s) * 64], acc[i][cb]);
         }
       }
     }
-  }
-  // accumulator (g, v) holds row drow[4 g + v] of the tile, column cb * 16 + c
-  const T js = J.job_scale[job];
+    // accumulator (g, v) holds row drow[4 g + v] of the tile, column cb * 16 + c
 #pragma unroll
-  for (int i = 0; i < kGemmTilesPerWave; i++) {
-    const int tile = (blockIdx.y * 4 + wave) * kGemmTilesPerWave + i;
-    if (tile >= ntiles) continue;
+    for (int i = 0; i < kGemmTilesPerWave; i++) {
+      const int tile = tile0 + i;
+      if (tile >= ntiles) continue;
 #pragma unroll
-    for (int v = 0; v < 4; v++) {
-      const int at = tile_atoms[tile * 16 + J.drow[4 * g + v]];
-      if (at < 0) continue;
-      T *o = out + ((long long) at * nfo + fo) * N + c;
+      for (int v = 0; v < 4; v++) {
+        const int at = tile_atoms[tile * 16 + J.drow[4 * g + v]];
+        if (at < 0) continue;
+        T *o = out + ((long long) at * nfo + fo) * N + c;
 #pragma unroll
-      for (int cb = 0; cb < NB; cb++) {
-        const T val = js * acc[i][cb][v];
-        o[cb * 16] = accumulate ? o[cb * 16] + val : val;
+        for (int cb = 0; cb < NB; cb++) {
+          const T val = js * acc[i][cb][v];
+          o[cb * 16] = accumulate ? o[cb * 16] + val : val;
+        }
       }
     }
   }

@@ -6,7 +6,8 @@
 //   k_lincomb          out[atom][f][n] = sum_t v_t in[atom][p_t][n]: the sparse Clebsch-Gordan matrix cg_W of the equivariant
 //                      SPBF and its transpose (fused_3l.cpp:1266-1272, :1443-1449)
 //   k_scale_rows       out[atom][f][n] (+)= s[f] in[atom][f][n]: the left input of an FCRight2Left layer (fused_3l.cpp:955-969)
-//   k_eqnorm_fwd/bwd   EquivariantRMSNorm (libgrace/include/grace/fused_3l_cpu.h:335-414)
+//   k_couple_*_lds     cp_l couple and its reverse with the atom's projections in LDS (fused_3l_cpu.h:223-276)
+//   k_eqnorm           EquivariantRMSNorm and its reverse (libgrace/include/grace/fused_3l_cpu.h:335-414)
 //   k_energy_3l        InvariantLayerRMSNorm of the three densities, their sum, fp64 readout MLP and the reverse of all of it
 //                      (fused_3l_cpu.h:416-444, fused_3l.cpp:1300-1360)
 #pragma once
@@ -56,6 +57,127 @@ template<class T> __global__ void k_scale_rows(const T *in, const T *s, T *out, 
   const int f = (int) ((q / C) % nf);
   const T v = s[f] * in[q];
   out[q] = accumulate ? out[q] + v : v;
+}
+
+// Term list of a cp_l couple sorted by output function: left, right, output function and coefficient of every term.
+struct CoupleDev {
+  const int *l, *r, *o;
+  const double *c;
+  const int *off;             // [nout + 1] terms of output o are [off[o], off[o + 1])
+  int nout, nterms;
+};
+
+__device__ inline double readlane_f64(double v, int k)
+{
+  const int lo = __builtin_amdgcn_readlane(__double2loint(v), k), hi = __builtin_amdgcn_readlane(__double2hiint(v), k);
+  return __hiloint2double(hi, lo);
+}
+
+// cp_l couple with the projections staged in LDS: out[o][n] = sum_t c_t Lp[l_t][n] Rp[r_t][n]
+// (couple_row_fwd, libgrace/include/grace/fused_3l_cpu.h:232-255).  A block works on AT = 64 / C atoms (a wave spans the
+// channels of AT atoms); wave w takes the outputs [w nout / nw, (w + 1) nout / nw).  The terms of a wave are read 64 at
+// a time, one per lane, and then walked with lane reads, so that no memory access sits between two terms but the LDS
+// reads of the operands.  grid: ceil(atoms / AT); dynamic LDS: AT (nfl + nfr) C values.
+template<class T>
+__global__ __launch_bounds__(1024) void k_couple_fwd_lds(CoupleDev P, const T *__restrict__ L, const T *__restrict__ R, T *__restrict__ out, int C,
+                                                         int nfl, int nfr, int natoms)
+{
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int AT = 64 / C, t = threadIdx.x, lane = t & 63, wave = t >> 6, nw = blockDim.x >> 6;
+  T *Ls = reinterpret_cast<T *>(smem_raw), *Rs = Ls + AT * nfl * C;
+  const int a0 = blockIdx.x * AT, na = natoms - a0 < AT ? natoms - a0 : AT;
+  {
+    const T *La = L + (long long) a0 * nfl * C, *Ra = R + (long long) a0 * nfr * C;
+    for (int q = t; q < na * nfl * C; q += blockDim.x) Ls[q] = La[q];
+    for (int q = t; q < na * nfr * C; q += blockDim.x) Rs[q] = Ra[q];
+  }
+  __syncthreads();
+  const int sub = lane / C, n = lane % C;
+  const bool live = sub < na;
+  const T *Lm = Ls + sub * nfl * C + n, *Rm = Rs + sub * nfr * C + n;
+  T *om = out + (long long) (a0 + (live ? sub : 0)) * P.nout * C + n;
+  const int o0 = (int) ((long long) wave * P.nout / nw), o1 = (int) ((long long) (wave + 1) * P.nout / nw);
+  const int t0 = P.off[o0], t1 = P.off[o1];
+  for (int o = o0; o < o1; o++)                       // outputs without terms
+    if (live && P.off[o] == P.off[o + 1]) om[(long long) o * C] = (T) 0;
+  int cur = -1;
+  T acc = (T) 0;
+  for (int base = t0; base < t1; base += 64) {
+    const int idx = base + lane < t1 ? base + lane : t1 - 1;
+    const int lv = P.l[idx], rv = P.r[idx], ov = P.o[idx];
+    const double cv = P.c[idx];
+    const int cnt = t1 - base < 64 ? t1 - base : 64;
+    for (int k = 0; k < cnt; k++) {
+      const int o = __builtin_amdgcn_readlane(ov, k);
+      if (o != cur) {
+        if (cur >= 0 && live) om[(long long) cur * C] = acc;
+        acc = (T) 0;
+        cur = o;
+      }
+      const int l = __builtin_amdgcn_readlane(lv, k), r = __builtin_amdgcn_readlane(rv, k);
+      acc += (T) readlane_f64(cv, k) * Lm[l * C] * Rm[r * C];
+    }
+  }
+  if (cur >= 0 && live) om[(long long) cur * C] = acc;
+}
+
+// Its reverse in scatter form: for every term gLp[l][n] += c g[o][n] Rp[r][n], gRp[r][n] += c g[o][n] Lp[l][n]
+// (couple_row_bwd, fused_3l_cpu.h:258-276), the two adjoints accumulated in LDS with LDS atomics (the waves of a block
+// share them) and added to gL / gR at the end; g is read once, row by row.  Same grid; dynamic LDS: 2 AT (nfl + nfr) C.
+template<class T>
+__global__ __launch_bounds__(1024) void k_couple_bwd_lds(CoupleDev P, const T *__restrict__ L, const T *__restrict__ R, const T *__restrict__ g,
+                                                         T *__restrict__ gL, T *__restrict__ gR, int C, int nfl, int nfr, int natoms)
+{
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int AT = 64 / C, t = threadIdx.x, lane = t & 63, wave = t >> 6, nw = blockDim.x >> 6;
+  T *Ls = reinterpret_cast<T *>(smem_raw), *Rs = Ls + AT * nfl * C, *gLs = Rs + AT * nfr * C, *gRs = gLs + AT * nfl * C;
+  const int a0 = blockIdx.x * AT, na = natoms - a0 < AT ? natoms - a0 : AT;
+  {
+    const T *La = L + (long long) a0 * nfl * C, *Ra = R + (long long) a0 * nfr * C;
+    for (int q = t; q < AT * nfl * C; q += blockDim.x) {
+      Ls[q] = q < na * nfl * C ? La[q] : (T) 0;
+      gLs[q] = (T) 0;
+    }
+    for (int q = t; q < AT * nfr * C; q += blockDim.x) {
+      Rs[q] = q < na * nfr * C ? Ra[q] : (T) 0;
+      gRs[q] = (T) 0;
+    }
+  }
+  __syncthreads();
+  const int sub = lane / C, n = lane % C;
+  const bool live = sub < na;
+  const int lo = sub * nfl * C + n, ro = sub * nfr * C + n;
+  const T *gm = g + (long long) (a0 + (live ? sub : 0)) * P.nout * C + n;
+  const int o0 = (int) ((long long) wave * P.nout / nw), o1 = (int) ((long long) (wave + 1) * P.nout / nw);
+  const int t0 = P.off[o0], t1 = P.off[o1];
+  int cur = -1;
+  T gcur = (T) 0, gnext = (T) 0;
+  int onext = -1;
+  for (int base = t0; base < t1; base += 64) {
+    const int idx = base + lane < t1 ? base + lane : t1 - 1;
+    const int lv = P.l[idx], rv = P.r[idx], ov = P.o[idx];
+    const double cv = P.c[idx];
+    const int cnt = t1 - base < 64 ? t1 - base : 64;
+    for (int k = 0; k < cnt; k++) {
+      const int o = __builtin_amdgcn_readlane(ov, k);
+      if (o != cur) {
+        gcur = o == onext ? gnext : (live ? gm[(long long) o * C] : (T) 0);
+        onext = o + 1 < o1 ? o + 1 : o;
+        gnext = live ? gm[(long long) onext * C] : (T) 0;    // the row of the next output, in flight during this one
+        cur = o;
+      }
+      const int l = __builtin_amdgcn_readlane(lv, k), r = __builtin_amdgcn_readlane(rv, k);
+      const T cg = (T) readlane_f64(cv, k) * gcur;
+      atomicAdd(&gLs[lo + l * C], cg * Rs[ro + r * C]);
+      atomicAdd(&gRs[ro + r * C], cg * Ls[lo + l * C]);
+    }
+  }
+  __syncthreads();
+  {
+    T *ga = gL + (long long) a0 * nfl * C, *gb = gR + (long long) a0 * nfr * C;
+    for (int q = t; q < na * nfl * C; q += blockDim.x) ga[q] += gLs[q];
+    for (int q = t; q < na * nfr * C; q += blockDim.x) gb[q] += gRs[q];
+  }
 }
 
 struct EqNormDev {
@@ -203,7 +325,7 @@ static __global__ void k_energy_3l(Energy3Dev M, const int *mu, const double *rh
     gs[j] = M.out_scale * M.norm1 * M.W1[j] * da * M.norm0;
   }
   __syncthreads();
-  // dE/dh: channel 0 the linear skip, channels 1.. through the MLP; kept in `pre` is no longer needed -> reuse h for dE/dh
+  // dE/dh: channel 0 the linear skip, channels 1.. through the MLP
   double gh_mine[4];    // nrho <= 256: up to 4 channels per lane
   for (int q = 0; q < 4; q++) {
     const int n = lane + 64 * q;
