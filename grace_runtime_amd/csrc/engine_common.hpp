@@ -744,9 +744,10 @@ class EngineBase : public Engine {
     if (J.d.njobs == 0 || ntiles == 0) return;
     const int ksm = std::max(kb0, kb1) * 4;
     const size_t lds = (size_t) kGemmMaxSeg * nb * ksm * 64 * sizeof(T);
-    // jobs whose weight tiles fit one staging walk several groups of atom tiles per block (less re-staging)
+    // single-segment jobs (one weight tile each: projections, reverse of the product reduces) walk several groups of
+    // atom tiles per block when the grid is large: the staging of the tile is what they spend their time on
     const int groups = (ntiles + 4 * kGemmTilesPerWave - 1) / (4 * kGemmTilesPerWave);
-    const int reps = J.d.max_seg <= kGemmMaxSeg ? std::max(1, std::min(8, (int) ((long long) J.d.njobs * groups / 2048))) : 1;
+    const int reps = J.d.max_seg == 1 ? std::max(1, std::min(8, (int) ((long long) J.d.njobs * groups / 8192))) : 1;
     const dim3 grid(J.d.njobs, (groups + reps - 1) / reps);
 #define GR_GEMM(A_, B_, C_)                                                                                            \
   {                                                                                                                    \
