@@ -146,6 +146,19 @@ def main():
         eng.compute(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
         th.append(time.perf_counter() - t1)
     host_ms = float(np.median(th[1:])) * 1e3
+    # the calculator's call (kk.System.compute: positions, cell, types in; host neighbour list, pass, results out), with
+    # the list rebuilt on every call (skin 0) and with the list kept (skin 0.5 A, unmoved atoms)
+    list_ms = {}
+    for label, skin in (("rebuilt", 0.0), ("kept", 0.5)):
+        sysm = kk.System(model, species, skin=skin, precision=a.precision)
+        tl = []
+        for k in range(3):
+            t1 = time.perf_counter()
+            sysm.compute(types, pos + (1e-9 * k if skin == 0.0 else 0.0), cell, pbc)     # any displacement rebuilds a skin-0 list
+            tl.append(time.perf_counter() - t1)
+        assert sysm.rebuilds == (3 if skin == 0.0 else 1)
+        list_ms[label] = float(np.median(tl[1:])) * 1e3
+        del sysm
     eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
 
     # per-stage durations: HIP events around every launch on the engine's stream, averaged over the same K steps
@@ -215,6 +228,7 @@ def main():
                    "atoms": N, "edges": int(E)},
         "atoms_steps_per_s": round(N / dt, 1),
         "ms_per_call_host_buffers": round(host_ms, 3),
+        "ms_per_calculator_call": {"neighbour_list_rebuilt": round(list_ms["rebuilt"], 3), "neighbour_list_kept": round(list_ms["kept"], 3)},
         "roofline": roofline,
         "stages_ms": {k: round(v, 4) for k, v in stages.items()},
         "stages_roofline": {k: {"bound": v["bound"], "achieved": round(v["achieved"], 2), "unit": v["unit"],
