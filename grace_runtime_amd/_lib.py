@@ -23,6 +23,8 @@ SYMBOLS = [
     "gr_engine_edge_count", "gr_engine_set_profile", "gr_engine_stage_count", "gr_engine_stage_get",
     "gr_engine_debug_radial", "gr_engine_debug_copy", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
+    "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
+    "gr_system_list_sizes", "gr_system_list_get",
 ]
 
 
@@ -80,6 +82,13 @@ def lib():
     L.gr_compute_batch.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, i32, vp, vp, vp, vp]
     L.gr_engine_upload_batch.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i32, vp]
     L.gr_engine_fetch_batch.argtypes = [vp, i32, vp, vp, vp, vp]
+    L.gr_system_create.argtypes = [vp, dbl, C.POINTER(vp)]
+    L.gr_system_free.argtypes = [vp]
+    L.gr_system_compute.argtypes = [vp, i32, vp, vp, vp, vp, u32, vp, vp, vp, vp]
+    L.gr_system_rebuilds.argtypes = [vp]
+    L.gr_system_list_on_device.argtypes = [vp]
+    L.gr_system_list_sizes.argtypes = [vp, C.POINTER(i64), C.POINTER(i64)]
+    L.gr_system_list_get.argtypes = [vp, vp, vp, vp, vp, vp]
     _lib = L
     return L
 

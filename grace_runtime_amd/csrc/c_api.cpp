@@ -4,6 +4,7 @@
 
 #include "engine.hpp"
 #include "neighbors.hpp"
+#include "neighbors_dev.hpp"
 
 #include <hip/hip_runtime_api.h>
 
@@ -28,8 +29,30 @@ struct gr_engine {
 struct gr_nlist {
   grhip::NeighborList nl;
 };
+// One structure resident on the device with a Verlet list at cutoff + skin (System of the reference's GPU module,
+// python/kk/kk_api.h:66-93): the pair search of a rebuild runs on the device, calls between rebuilds send positions only.
+struct gr_system {
+  gr_engine *eng = nullptr;
+  double skin = 0.0, cutoff = 0.0;
+  int rebuilds = 0;
+  bool have = false, on_device = false;
+  int n = 0;
+  std::vector<int> types;
+  std::vector<double> x0, cell;
+  unsigned char pbc[3] = {0, 0, 0};
+  std::vector<int64_t> perm;
+  grhip::DeviceNeighbors nl;
+  grhip::NeighborList host_nl;    // the list when the device search declined the structure
+  grhip::DevBuf pos_dev, x_dev;
+  hipStream_t stream = nullptr;
+  ~gr_system()
+  {
+    if (stream) (void) hipStreamDestroy(stream);
+  }
+};
 
 namespace {
+void padded_cell(const double *cell, const unsigned char *pbc, const double *pos, int64_t n, double reach, double *out, double *shift);
 thread_local std::string g_err;
 
 template<class F> int guarded(F &&f)
@@ -364,6 +387,150 @@ int gr_compute(gr_engine *e, int n, const int *types, const double *positions, c
       if (forces && !fl.energy_only)
         for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) q + d];
       if (fl.eatom) eatom[a] = ea[q];
+    }
+  });
+}
+
+int gr_system_create(gr_engine *e, double skin, gr_system **out)
+{
+  return guarded([&] {
+    if (!e || !out) throw grhip::InvalidArgument("null argument");
+    *out = nullptr;
+    if (!(std::isfinite(skin) && skin >= 0.0)) throw grhip::InvalidArgument("skin must be a finite number >= 0");
+    auto s = std::make_unique<gr_system>();
+    s->eng = e;
+    s->skin = skin;
+    s->cutoff = e->eng->max_cutoff();
+    if (hipSetDevice(e->eng->device_index()) != hipSuccess || hipStreamCreate(&s->stream) != hipSuccess)
+      throw grhip::Error("gr_system_create: cannot create a stream on the engine's device");
+    *out = s.release();
+  });
+}
+
+void gr_system_free(gr_system *s) { delete s; }
+int gr_system_rebuilds(const gr_system *s) { return s ? s->rebuilds : 0; }
+int gr_system_list_on_device(const gr_system *s) { return s && s->have && s->on_device ? 1 : 0; }
+
+int gr_system_compute(gr_system *s, int n, const int *types, const double *positions, const double *cell, const unsigned char *pbc,
+                      unsigned flags, double *energy, double *forces, double *virial, double *eatom)
+{
+  return guarded([&] {
+    if (!s || !cell || !pbc || (n > 0 && (!types || !positions))) throw grhip::InvalidArgument("null argument");
+    if (n < 0) throw grhip::InvalidArgument("negative atom count");
+    if (!(s->cutoff > 0.0)) throw grhip::Error("the engine has no positive cutoff");
+    grhip::Engine &eng = *s->eng->eng;
+    if (hipSetDevice(eng.device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
+    // list policy of the reference (python/grace_runtime/neighbors.py:68-89): rebuild when the atoms, the cell or the
+    // boundary conditions change or an atom moved more than skin / 2 since the last build
+    bool rebuild = !s->have || n != s->n || std::memcmp(pbc, s->pbc, 3) != 0 || std::memcmp(cell, s->cell.data(), 9 * sizeof(double)) != 0 ||
+                   (n > 0 && std::memcmp(types, s->types.data(), sizeof(int) * (size_t) n) != 0);
+    if (!rebuild) {
+      const double lim = 0.25 * s->skin * s->skin;
+      for (int a = 0; a < n && !rebuild; a++) {
+        const double dx = positions[3 * a] - s->x0[3 * (size_t) a], dy = positions[3 * a + 1] - s->x0[3 * (size_t) a + 1],
+                     dz = positions[3 * a + 2] - s->x0[3 * (size_t) a + 2];
+        rebuild = dx * dx + dy * dy + dz * dz > lim;
+      }
+    }
+    std::vector<double> x((size_t) 3 * n);
+    if (rebuild) {
+      s->have = false;
+      const double reach = s->cutoff + s->skin;
+      double pc[9], sh[3];
+      padded_cell(cell, pbc, positions, n, reach, pc, sh);
+      std::vector<double> xs((size_t) 3 * n);
+      for (int a = 0; a < n; a++)
+        for (int d = 0; d < 3; d++) xs[3 * (size_t) a + d] = positions[3 * a + d] + sh[d];
+      const bool p[3] = {pbc[0] != 0, pbc[1] != 0, pbc[2] != 0};
+      s->on_device = s->nl.build(xs.data(), n, pc, p, reach, s->stream);
+      if (!s->on_device) s->host_nl = grhip::neighbor_search(xs.data(), n, pc, p, reach, 8);
+      s->perm = s->on_device ? s->nl.perm : s->host_nl.perm;
+      std::vector<int> ty(n);
+      for (int q = 0; q < n; q++) {
+        const int64_t a = s->perm[q];
+        ty[q] = types[a];
+        for (int d = 0; d < 3; d++) x[3 * (size_t) q + d] = positions[3 * a + d];
+      }
+      const std::vector<double> dummy(3, 0.0);
+      if (s->on_device) {
+        s->x_dev.ensure(std::max<size_t>(sizeof(double) * 3 * (size_t) n, 8));
+        if (n > 0 && hipMemcpy(s->x_dev.p, x.data(), sizeof(double) * 3 * (size_t) n, hipMemcpyHostToDevice) != hipSuccess)
+          throw grhip::Error("copy of the positions to the device failed");
+        grhip::DeviceCsr in;
+        in.n = n;
+        in.types = ty.data();
+        in.nb = s->nl.nb;
+        in.offset = s->nl.offset.as<int64_t>();
+        in.j = s->nl.j.as<int>();
+        in.image = s->nl.image.as<int>();
+        in.x = s->x_dev.as<double>();
+        in.nimages = (int64_t) s->nl.shifts.size() / 3;
+        in.shifts = in.nimages ? s->nl.shifts.data() : dummy.data();
+        eng.upload_device(in);
+      } else {
+        const grhip::NeighborList &nl = s->host_nl;
+        const int64_t nimg = (int64_t) nl.shifts.size() / 3;
+        eng.upload(make_input(n, ty.data(), nl.offset.data(), nl.j.data(), nullptr, x.data(), nl.image.data(), nimg ? nl.shifts.data() : dummy.data(), nimg));
+      }
+      s->n = n;
+      s->types.assign(types, types + n);
+      s->x0.assign(positions, positions + 3 * (size_t) n);
+      s->cell.assign(cell, cell + 9);
+      std::memcpy(s->pbc, pbc, 3);
+      s->have = true;
+      s->rebuilds++;
+    } else {
+      for (int q = 0; q < n; q++) {
+        const int64_t a = s->perm[q];
+        for (int d = 0; d < 3; d++) x[3 * (size_t) q + d] = positions[3 * a + d];
+      }
+      eng.update_positions(x.data());
+    }
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    eng.run(fl);
+    std::vector<double> f((size_t) 3 * n), ea(fl.eatom ? n : 0);
+    eng.fetch(energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
+    for (int q = 0; q < n; q++) {
+      const int64_t a = s->perm[q];
+      if (forces && !fl.energy_only)
+        for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) q + d];
+      if (fl.eatom) eatom[a] = ea[q];
+    }
+  });
+}
+
+// the list of the last rebuild: sizes, then the arrays (perm [n], offset [n + 1], j [nb], image [nb], shifts [nimages][3])
+int gr_system_list_sizes(gr_system *s, int64_t *nbonds, int64_t *nimages)
+{
+  return guarded([&] {
+    if (!s || !s->have) throw grhip::Error("gr_system_list_sizes: no list has been built");
+    if (nbonds) *nbonds = s->on_device ? s->nl.nb : (int64_t) s->host_nl.j.size();
+    if (nimages) *nimages = (int64_t) (s->on_device ? s->nl.shifts.size() : s->host_nl.shifts.size()) / 3;
+  });
+}
+
+int gr_system_list_get(gr_system *s, int64_t *perm, int64_t *offset, int32_t *j, int32_t *image, double *shifts)
+{
+  return guarded([&] {
+    if (!s || !s->have) throw grhip::Error("gr_system_list_get: no list has been built");
+    std::memcpy(perm, s->perm.data(), sizeof(int64_t) * s->perm.size());
+    if (s->on_device) {
+      if (hipSetDevice(s->eng->eng->device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
+      bool ok = hipMemcpy(offset, s->nl.offset.p, sizeof(int64_t) * (size_t) (s->n + 1), hipMemcpyDeviceToHost) == hipSuccess;
+      if (s->nl.nb > 0) {
+        ok = ok && hipMemcpy(j, s->nl.j.p, sizeof(int32_t) * (size_t) s->nl.nb, hipMemcpyDeviceToHost) == hipSuccess;
+        ok = ok && hipMemcpy(image, s->nl.image.p, sizeof(int32_t) * (size_t) s->nl.nb, hipMemcpyDeviceToHost) == hipSuccess;
+      }
+      if (!ok) throw grhip::Error("copy of the neighbour list from the device failed");
+      std::memcpy(shifts, s->nl.shifts.data(), sizeof(double) * s->nl.shifts.size());
+    } else {
+      const grhip::NeighborList &nl = s->host_nl;
+      std::memcpy(offset, nl.offset.data(), sizeof(int64_t) * nl.offset.size());
+      std::memcpy(j, nl.j.data(), sizeof(int32_t) * nl.j.size());
+      std::memcpy(image, nl.image.data(), sizeof(int32_t) * nl.image.size());
+      std::memcpy(shifts, nl.shifts.data(), sizeof(double) * nl.shifts.size());
     }
   });
 }

@@ -29,6 +29,19 @@ struct CsrInput {
   const int *sid = nullptr;           // [n] in 0 .. nstruct-1
 };
 
+// A structure whose neighbour list is already in device memory: the engine copies it into its own buffers.
+struct DeviceCsr {
+  int n = 0;
+  const int *types = nullptr;         // host [n] 1-based atom types, in the order of the list
+  int64_t nb = 0;
+  const int64_t *offset = nullptr;    // device [n + 1]
+  const int *j = nullptr;             // device [nb]
+  const int *image = nullptr;         // device [nb]
+  const double *x = nullptr;          // device [n][3]
+  const double *shifts = nullptr;     // host [nimages][3]
+  int64_t nimages = 0;
+};
+
 struct StageTime {
   std::string name;
   double ms = 0.0;       // summed over the launches of the stage in the last run
@@ -48,6 +61,11 @@ class Engine {
   virtual double max_cutoff() const = 0;
   // copy a structure to the GPU (validates types, offsets and neighbour indices)
   virtual void upload(const CsrInput &in) = 0;
+  // the same from a list in device memory (indices are trusted: the list comes from the library's own search)
+  virtual void upload_device(const DeviceCsr &in) = 0;
+  // new positions [n][3] (host) for the uploaded list (a list given as positions + image + shifts)
+  virtual void update_positions(const double *x) = 0;
+  virtual int device_index() const = 0;
   // one energy / forces / virial pass over the uploaded structure; results stay on the GPU
   virtual void run(const RunFlags &fl) = 0;
   // wait for the pass and copy results out (null pointers are skipped); forces [n][3], virial [6], eatom [n]

@@ -490,18 +490,7 @@ class EngineBase : public Engine {
     };
     put(mu_, mu.data(), sizeof(int) * n);
     if (have_sid_) put(sid_, in.sid, sizeof(int) * n);
-    std::vector<int> tiles;    // tiles of 16 atoms of one element, in atom order within an element
-    {
-      std::vector<int> ord(n);
-      std::iota(ord.begin(), ord.end(), 0);
-      std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return mu[a] < mu[b]; });
-      for (int q = 0; q < n;) {
-        int cnt = 0;
-        const int m0 = mu[ord[q]];
-        while (cnt < 16 && q < n && mu[ord[q]] == m0) { tiles.push_back(ord[q]); q++; cnt++; }
-        while (cnt < 16) { tiles.push_back(-1); cnt++; }
-      }
-    }
+    const std::vector<int> tiles = element_tiles(mu);
     ntiles_ = (int) tiles.size() / 16;
     put(tiles_, tiles.data(), sizeof(int) * tiles.size());
     static_assert(sizeof(long long) == sizeof(int64_t), "offset type");
@@ -515,6 +504,66 @@ class EngineBase : public Engine {
     }
     HIP_CHECK(hipStreamSynchronize(stream_));    // the host copies (mu, tiles) go out of scope
     ran_ = false;
+  }
+  void upload_device(const DeviceCsr &in) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (in.n < 0) throw InvalidArgument("negative atom count");
+    const int n = in.n;
+    std::vector<int> mu(n);
+    for (int a = 0; a < n; a++) {
+      if (in.types[a] < 1 || in.types[a] > ntypes_) throw InvalidArgument("types must be 1 .. len(species)");
+      mu[a] = type2mu_[in.types[a]];
+      if (mu[a] < 0)
+        throw Error(who_ + ": atom " + std::to_string(a) + " of unmapped type " + std::to_string(in.types[a]) + " in the atom list");
+    }
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    n_ = n;
+    nb_ = in.nb;
+    nstruct_ = 1;
+    have_sid_ = false;
+    have_rij_ = false;
+    scal_.ensure(8 * sizeof(double));
+    auto put = [&](DevBuf &b, const void *src, size_t bytes, hipMemcpyKind kind) {
+      b.ensure(std::max<size_t>(bytes, 8));
+      if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, kind, stream_));
+    };
+    put(mu_, mu.data(), sizeof(int) * n, hipMemcpyHostToDevice);
+    const std::vector<int> tiles = element_tiles(mu);
+    ntiles_ = (int) tiles.size() / 16;
+    put(tiles_, tiles.data(), sizeof(int) * tiles.size(), hipMemcpyHostToDevice);
+    put(offset_, in.offset, sizeof(int64_t) * (n + 1), hipMemcpyDeviceToDevice);
+    put(j_, in.j, sizeof(int) * in.nb, hipMemcpyDeviceToDevice);
+    put(image_, in.image, sizeof(int) * in.nb, hipMemcpyDeviceToDevice);
+    put(x_, in.x, sizeof(double) * 3 * n, hipMemcpyDeviceToDevice);
+    put(shifts_, in.shifts, sizeof(double) * 3 * in.nimages, hipMemcpyHostToDevice);
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    ran_ = false;
+  }
+  void update_positions(const double *x) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (have_rij_) throw Error("update_positions: the uploaded list holds bond vectors, not positions");
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    if (n_ > 0) HIP_CHECK(hipMemcpyAsync(x_.p, x, sizeof(double) * 3 * n_, hipMemcpyHostToDevice, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    ran_ = false;
+  }
+  int device_index() const override { return device_; }
+  // tiles of 16 atoms of one element (-1 padded), in atom order within an element
+  static std::vector<int> element_tiles(const std::vector<int> &mu)
+  {
+    const int n = (int) mu.size();
+    std::vector<int> tiles, ord(n);
+    std::iota(ord.begin(), ord.end(), 0);
+    std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return mu[a] < mu[b]; });
+    for (int q = 0; q < n;) {
+      int cnt = 0;
+      const int m0 = mu[ord[q]];
+      while (cnt < 16 && q < n && mu[ord[q]] == m0) { tiles.push_back(ord[q]); q++; cnt++; }
+      while (cnt < 16) { tiles.push_back(-1); cnt++; }
+    }
+    return tiles;
   }
   void fetch(double *energy, double *forces, double *virial, double *eatom) override
   {

@@ -299,7 +299,8 @@ def _padded_cell_arrays(cell, pos, reach, pbc=None):
 class System:
     """One structure on the device with a Verlet list at cutoff + skin, rebuilt when an atom moved more than
     skin / 2 or the atoms / cell / pbc change (python/kk/kk_api.h:66-93, list policy python/grace_runtime/
-    neighbors.py:68-89)."""
+    neighbors.py:68-89).  The list lives on the device (gr_system_*): its pair search runs there, and calls between
+    rebuilds send positions only."""
 
     def __init__(self, model: Model, species, skin: float = 0.5, spline: int = 1024, chunksize: int = -1,
                  precision: int = 64):
@@ -309,15 +310,40 @@ class System:
         self.engine = Engine(model, species, precision)
         self.skin = skin
         self.cutoff = float(self.engine.cutoff_matrix().max()) if len(species) else 0.0
-        self.rebuilds = 0
         self.chunksize = 0
-        self._x0 = self._key = self._nl = None
+        self._h = C.c_void_p()
+        check(_lib.lib().gr_system_create(self.engine._h, skin, C.byref(self._h)))
+
+    def __del__(self):
+        if getattr(self, "_h", None) is not None and self._h.value:
+            _lib.lib().gr_system_free(self._h)
+            self._h = C.c_void_p()
+
+    @property
+    def rebuilds(self) -> int:
+        return int(_lib.lib().gr_system_rebuilds(self._h))
+
+    @property
+    def list_on_device(self) -> bool:
+        """True when the list of the last rebuild was searched on the device."""
+        return bool(_lib.lib().gr_system_list_on_device(self._h))
 
     def release_buffers(self):
-        self._x0 = self._key = self._nl = None
+        pass
 
     def set_dispersion(self, *a, **k):
         raise ValueError("dispersion corrections are not part of this engine")
+
+    def neighbor_list(self):
+        """(perm, offset, j, image, shifts) of the last rebuild, as neighbor_search returns them."""
+        nb, nimg = C.c_int64(), C.c_int64()
+        check(_lib.lib().gr_system_list_sizes(self._h, C.byref(nb), C.byref(nimg)))
+        n = self._n
+        perm, offset = np.empty(n, np.int64), np.empty(n + 1, np.int64)
+        j, image = np.empty(nb.value, np.int32), np.empty(nb.value, np.int32)
+        shifts = np.empty((nimg.value, 3))
+        check(_lib.lib().gr_system_list_get(self._h, ptr(perm), ptr(offset), ptr(j), ptr(image), ptr(shifts)))
+        return perm, offset, j, image, shifts
 
     def compute(self, types, positions, cell, pbc, energies=False, uq=False, energy_only=False):
         if uq:
@@ -325,33 +351,26 @@ class System:
         types = as_array(types, np.int32)
         pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
         cell = np.ascontiguousarray(cell, dtype=np.float64).reshape(3, 3)
-        pbc = np.asarray([bool(p) for p in pbc])
+        pb = np.ascontiguousarray([1 if p else 0 for p in pbc], dtype=np.uint8)
         n = types.shape[0]
         if pos.shape[0] != n:
             raise ValueError("positions must have len(types) rows")
         if n and (types.min() < 1 or types.max() > len(self.engine.species)):
             raise ValueError("types must be 1 .. len(species)")
-        key = (cell.tobytes(), pbc.tobytes(), types.tobytes())
-        rebuild = self._x0 is None or key != self._key or len(self._x0) != n or \
-            (n > 0 and ((pos - self._x0) ** 2).sum(axis=1).max() > (0.5 * self.skin) ** 2)
-        if rebuild:
-            reach = self.cutoff + self.skin
-            pcell, shift = _padded_cell_arrays(cell, pos, reach, pbc)
-            self._nl = neighbor_search(pos + shift, pcell, pbc, reach)
-            self._key, self._x0 = key, pos.copy()
-            self.rebuilds += 1
-        perm, offset, j, image, shifts = self._nl
-        out = self.engine.compute(types[perm], offset, j, energies=energies, energy_only=energy_only,
-                                  positions=pos[perm], image=image, shifts=shifts)
-        res = {"energy": out["energy"]}
+        self._n = n
+        e = C.c_double()
+        forces = None if energy_only else np.empty((n, 3))
+        virial = None if energy_only else np.empty(6)
+        eat = np.empty(n) if energies else None
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
+        check(_lib.lib().gr_system_compute(self._h, n, ptr(types), ptr(pos), ptr(cell), ptr(pb), flags, C.byref(e),
+                                      ptr(forces) if forces is not None else None, ptr(virial) if virial is not None else None,
+                                      ptr(eat) if eat is not None else None))
+        res = {"energy": e.value}
         if not energy_only:
-            f = np.empty((n, 3))
-            f[perm] = out["forces"]
-            res["forces"], res["virial"] = f, out["virial"]
+            res["forces"], res["virial"] = forces, virial
         if energies:
-            e = np.empty(n)
-            e[perm] = out["energies"]
-            res["energies"] = e
+            res["energies"] = eat
         return res
 
 

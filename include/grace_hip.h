@@ -19,6 +19,7 @@ extern "C" {
 typedef struct gr_model gr_model;
 typedef struct gr_engine gr_engine;
 typedef struct gr_nlist gr_nlist;
+typedef struct gr_system gr_system;
 
 enum {
   GR_OK = 0,
@@ -119,6 +120,24 @@ void gr_nlist_free(gr_nlist *l);
  * calculate -> _CpuEngine.compute (python/grace_runtime/calculator.py:204-224) without the Verlet skin. */
 int gr_compute(gr_engine *e, int n, const int *types, const double *positions, const double *cell,
                const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom);
+
+/* One structure resident on the device with a Verlet list at cutoff + skin: System of the reference's GPU module
+ * (python/kk/kk_api.h:66-93, System::compute python/kk/kk_core.cpp:802-958; list policy python/grace_runtime/
+ * neighbors.py:68-89: rebuild when types, cell or pbc change or an atom moved more than skin / 2).  The pair search of
+ * a rebuild runs on the device (the reference's device list: libgrace/include/grace/kk/neighbors_kk.h) and gives the
+ * list of gr_neighbor_build bond for bond; between rebuilds a call sends the positions only.  Results in the caller's
+ * atom order, as gr_compute.  The engine must outlive the system and serves one system at a time.
+ * gr_system_list_*: the list of the last rebuild (perm [n], offset [n + 1], j [nb], image [nb], shifts [nimages][3]);
+ * gr_system_list_on_device: 1 when that list was searched on the device, 0 when the structure was handed to the host
+ * search (atoms many thousands of cells apart). */
+int gr_system_create(gr_engine *e, double skin, gr_system **out);
+void gr_system_free(gr_system *s);
+int gr_system_compute(gr_system *s, int n, const int *types, const double *positions, const double *cell, const unsigned char *pbc,
+                      unsigned flags, double *energy, double *forces, double *virial, double *eatom);
+int gr_system_rebuilds(const gr_system *s);
+int gr_system_list_on_device(const gr_system *s);
+int gr_system_list_sizes(gr_system *s, int64_t *nbonds, int64_t *nimages);
+int gr_system_list_get(gr_system *s, int64_t *perm, int64_t *offset, int32_t *j, int32_t *image, double *shifts);
 
 /* Several independent structures in one pass (the batched small-structure workload).  Replaces Batch::compute of the
  * reference GPU module (python/kk/kk_api.h:116-156, python/kk/kk_core.cpp:960-1160: structures packed into one atom
