@@ -90,13 +90,13 @@ template<class T> struct DevContract {
 
 // sparse matrix in CSR form on the device (k_lincomb)
 struct DevCsr {
-  DevBuf off, idx, val;
+  DevBuf off, idx, rowof, val;
   int nrow = 0, ncol = 0;
   void build(int nrow_, int ncol_, const std::vector<int> &row, const std::vector<int> &col, const std::vector<double> &v)
   {
     nrow = nrow_;
     ncol = ncol_;
-    std::vector<int> o(nrow + 1, 0), ix(row.size());
+    std::vector<int> o(nrow + 1, 0), ix(row.size()), rw(row.size());
     std::vector<double> vv(row.size());
     for (int r : row) o[r + 1]++;
     for (int r = 0; r < nrow; r++) o[r + 1] += o[r];
@@ -104,11 +104,13 @@ struct DevCsr {
     for (size_t t = 0; t < row.size(); t++) {
       const int q = pos[row[t]]++;
       ix[q] = col[t];
+      rw[q] = row[t];
       vv[q] = v[t];
     }
-    if (ix.empty()) { ix.push_back(0); vv.push_back(0.0); }
+    if (ix.empty()) { ix.push_back(0); rw.push_back(0); vv.push_back(0.0); }
     upload_vec(off, o);
     upload_vec(idx, ix);
+    upload_vec(rowof, rw);
     upload_vec(val, vv);
   }
 };
@@ -566,8 +568,10 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
               (const T *) M_.as<T>(), pairP_.as<T>(), L.nlmi, L.CP, nl_, L.rad.noutp, yw, sink_.as<T>());
     });
     stage(tg(k, "couple_YI").c_str(), [&] {
-      hipLaunchKernelGGL(k_lincomb<T>, dim3(n, (L.nfA * L.CP + 255) / 256), dim3(256), 0, stream_, L.cg.off.template as<int>(), L.cg.idx.template as<int>(),
-                         L.cg.val.template as<double>(), (const T *) pairP_.as<T>(), A_.as<T>(), npf, L.nfA, L.CP);
+      const int AT = 64 / L.CP;
+      hipLaunchKernelGGL(k_lincomb<T>, dim3((n + AT - 1) / AT, (L.nfA + 4 * kLincombRows - 1) / (4 * kLincombRows)), dim3(256), 0, stream_,
+                         L.cg.off.template as<int>(), L.cg.idx.template as<int>(), L.cg.rowof.template as<int>(), L.cg.val.template as<double>(),
+                         (const T *) pairP_.as<T>(), A_.as<T>(), npf, L.nfA, L.CP, n);
     });
     stage(tg(k, "reduce_A").c_str(), [&] { cfwd_set(L.redA, A_.as<T>(), X); });
   }
@@ -731,8 +735,10 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   gM_.ensure(na * L.nlmi * L.CP * s);
   stage(tg(k, "reduce_A_bwd").c_str(), [&] { cbwd_set(L.redA, gX, gA_.as<T>()); });
   stage(tg(k, "couple_YI_bwd").c_str(), [&] {
-    hipLaunchKernelGGL(k_lincomb<T>, dim3(n, (npf * L.CP + 255) / 256), dim3(256), 0, stream_, L.cgt.off.template as<int>(), L.cgt.idx.template as<int>(),
-                       L.cgt.val.template as<double>(), (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP);
+    const int AT = 64 / L.CP;
+    hipLaunchKernelGGL(k_lincomb<T>, dim3((n + AT - 1) / AT, (npf + 4 * kLincombRows - 1) / (4 * kLincombRows)), dim3(256), 0, stream_,
+                       L.cgt.off.template as<int>(), L.cgt.idx.template as<int>(), L.cgt.rowof.template as<int>(), L.cgt.val.template as<double>(),
+                       (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP, n);
   });
   stage(tg(k, "message_bwd").c_str(), [&] {
     const long long tot = (long long) n * L.nlmi * L.CP;

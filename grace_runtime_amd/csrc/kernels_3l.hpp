@@ -16,6 +16,12 @@
 
 namespace grhip {
 
+__device__ inline double readlane_f64(double v, int k)
+{
+  const int lo = __builtin_amdgcn_readlane(__double2loint(v), k), hi = __builtin_amdgcn_readlane(__double2hiint(v), k);
+  return __hiloint2double(hi, lo);
+}
+
 // grid: atoms; block: 64
 static __global__ void k_edge_center(const long long *eoff, const int *mu, int *emi)
 {
@@ -34,19 +40,56 @@ __global__ void k_message(const T *I, const int *mu, const T *zproj, const T *ma
   M[q] = I[q] + mask[f] * zproj[(long long) mu[at] * C + n];
 }
 
-// CSR by output function: terms [off[f], off[f + 1]) with source function idx[t] and value val[t].
-// grid: (atoms, ceil(nout * C / 256)); block 256.  Rows of `in` have nin functions.
+// Sparse matrix times the per-atom tensor: out[atom][f][n] = sum_{t in row f} val[t] in[atom][idx[t]][n].  CSR by output
+// row: terms [off[f], off[f + 1]), row[t] = f.  A wave spans the channels of AT = 64 / C atoms and takes kLincombRows
+// consecutive output rows; it reads its terms 64 at a time, one per lane, and walks them with lane reads, the source
+// rows of 8 terms requested before the first is used.  grid: (ceil(atoms / AT), ceil(nout / (4 kLincombRows))); block 256.
+constexpr int kLincombRows = 8;
 template<class T>
-__global__ void k_lincomb(const int *__restrict__ off, const int *__restrict__ idx, const double *__restrict__ val, const T *__restrict__ in,
-                          T *__restrict__ out, int nin, int nout, int C)
+__global__ __launch_bounds__(256) void k_lincomb(const int *__restrict__ off, const int *__restrict__ idx, const int *__restrict__ row,
+                                                 const double *__restrict__ val, const T *__restrict__ in, T *__restrict__ out, int nin, int nout,
+                                                 int C, int natoms)
 {
-  const int at = blockIdx.x, q = blockIdx.y * blockDim.x + threadIdx.x;
-  if (q >= nout * C) return;
-  const int f = q / C, n = q % C;
-  const T *src = in + (long long) at * nin * C + n;
+  const int AT = 64 / C, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int a0 = blockIdx.x * AT, sub = lane / C, n = lane % C;
+  const bool live = a0 + sub < natoms;
+  const int r0 = (blockIdx.y * 4 + wave) * kLincombRows, r1 = r0 + kLincombRows < nout ? r0 + kLincombRows : nout;
+  if (r0 >= nout) return;
+  const T *src = in + (long long) (a0 + (live ? sub : 0)) * nin * C + n;
+  T *dst = out + (long long) (a0 + (live ? sub : 0)) * nout * C + n;
+  const int t0 = off[r0], t1 = off[r1];
+  for (int f = r0; f < r1; f++)                        // rows without terms
+    if (live && off[f] == off[f + 1]) dst[(long long) f * C] = (T) 0;
+  int cur = -1;
   T acc = (T) 0;
-  for (int t = off[f]; t < off[f + 1]; t++) acc += (T) val[t] * src[(long long) idx[t] * C];
-  out[((long long) at * nout + f) * C + n] = acc;
+  for (int base = t0; base < t1; base += 64) {
+    const int q = base + lane < t1 ? base + lane : t1 - 1;
+    const int iv = idx[q], rv = row[q];
+    const double cv = val[q];
+    const int cnt = t1 - base < 64 ? t1 - base : 64;
+    for (int k0 = 0; k0 < cnt; k0 += 8) {
+      T x[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int k = k0 + u < cnt ? k0 + u : cnt - 1;
+        x[u] = src[(long long) __builtin_amdgcn_readlane(iv, k) * C];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const int k = k0 + u;
+        if (k < cnt) {
+          const int f = __builtin_amdgcn_readlane(rv, k);
+          if (f != cur) {
+            if (cur >= 0 && live) dst[(long long) cur * C] = acc;
+            acc = (T) 0;
+            cur = f;
+          }
+          acc += (T) readlane_f64(cv, k) * x[u];
+        }
+      }
+    }
+  }
+  if (cur >= 0 && live) dst[(long long) cur * C] = acc;
 }
 
 // grid: ceil(natoms * nf * C / 256)
@@ -66,12 +109,6 @@ struct CoupleDev {
   const int *off;             // [nout + 1] terms of output o are [off[o], off[o + 1])
   int nout, nterms;
 };
-
-__device__ inline double readlane_f64(double v, int k)
-{
-  const int lo = __builtin_amdgcn_readlane(__double2loint(v), k), hi = __builtin_amdgcn_readlane(__double2hiint(v), k);
-  return __hiloint2double(hi, lo);
-}
 
 // cp_l couple with the projections staged in LDS: out[o][n] = sum_t c_t Lp[l_t][n] Rp[r_t][n]
 // (couple_row_fwd, libgrace/include/grace/fused_3l_cpu.h:232-255).  A block works on AT = 64 / C atoms (a wave spans the
