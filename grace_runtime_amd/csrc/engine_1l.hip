@@ -178,6 +178,9 @@ template<class T> void Engine1L<T>::build()
     en_.nrho = nrho_;
     en_.width = nrho_;
     for (int L = 0; L < en_.nlay; L++) en_.width = std::max({en_.width, en_.nin[L], en_.nout[L]});
+    en_.wlds = 0;
+    for (int L = 0; L < en_.nlay; L++) en_.wlds += 2 * en_.nin[L] * en_.nout[L];
+    if (en_.wlds > 4096) en_.wlds = 0;    // 32 kB: larger networks read their weights from global memory
     en_.out_scale = m.output_scale;
     en_.shift = shift_.as<double>();
   }
@@ -264,7 +267,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
 #undef GR_RED
   });
   stage("energy_mlp", [&] {
-    hipLaunchKernelGGL(k_energy, dim3(n), dim3(64), (size_t) (2 * en_.nlay + 4) * en_.width * sizeof(double), stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
+    hipLaunchKernelGGL(k_energy, dim3(n), dim3(64), (size_t) ((2 * en_.nlay + 4) * en_.width + en_.wlds) * sizeof(double), stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
                        fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), fl.energy_only ? 0 : 1, sid_ptr());
   });
   if (fl.energy_only) return;

@@ -926,6 +926,7 @@ struct EnergyDev {
   double norm[7];
   int nin[7], nout[7];
   int nlay, act, ln, nrho, width;    // width: largest layer width (LDS row of the kernel)
+  int wlds;                   // weights staged in LDS (sum of n_in n_out values, twice: as stored and transposed), or 0
   double out_scale;
   const double *shift;        // [nel]
 };
@@ -945,6 +946,28 @@ static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, 
   const int at = blockIdx.x, lane = threadIdx.x;
   const double *r = rho + (long long) at * M.nrho;
   const int n0 = M.nrho - 1;
+  // the weights of a small network go to LDS first, as stored [a][c] for the forward pass and transposed [c][a] for the
+  // reverse: one round of coalesced loads instead of a dependent chain of them per layer
+  const double *wf[7], *wt[7];
+  {
+    double *wl = x0 + W;
+    for (int L = 0; L < M.nlay; L++) {
+      const int sz = M.nin[L] * M.nout[L];
+      if (M.wlds) {
+        for (int e = lane; e < sz; e += 64) {
+          const double v = M.W[L][e];
+          wl[e] = v;
+          wl[sz + (e % M.nout[L]) * M.nin[L] + e / M.nout[L]] = v;
+        }
+        wf[L] = wl;
+        wt[L] = wl + sz;
+        wl += 2 * sz;
+      } else {
+        wf[L] = M.W[L];
+        wt[L] = nullptr;
+      }
+    }
+  }
   for (int k = lane; k < n0; k += 64) act(0, k) = r[k + 1];
   __syncthreads();
   double q = 0.0;
@@ -959,7 +982,7 @@ static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, 
   for (int L = 0; L < M.nlay; L++) {
     for (int c = lane; c < M.nout[L]; c += 64) {
       double s = 0.0;
-      for (int a = 0; a < M.nin[L]; a++) s += act(L, a) * M.W[L][(long long) a * M.nout[L] + c];
+      for (int a = 0; a < M.nin[L]; a++) s += act(L, a) * wf[L][a * M.nout[L] + c];
       s *= M.norm[L];
       pre(L, c) = s;
       act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
@@ -991,7 +1014,10 @@ static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, 
     }
     for (int a = lane; a < M.nin[L]; a += 64) {
       double s = 0.0;
-      for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * M.W[L][(long long) a * M.nout[L] + c];
+      if (wt[L])
+        for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * wt[L][c * M.nin[L] + a];
+      else
+        for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * wf[L][(long long) a * M.nout[L] + c];
       gbuf(cur ^ 1, a) = s * M.norm[L];
     }
     cur ^= 1;
