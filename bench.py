@@ -36,7 +36,7 @@ HBM_PEAK = 8000.0                 # GB/s
 MEASURED_TRAFFIC = {
     ("config2", "radial_mlp"): 366.7e6 + 1241.0e6,      # fetch + write of k_radial<double,4,0>
     ("config3", "pair_bwd"): 11883.6e6 + 2822.1e6,      # fetch + write of k_pair_bwd<double,25>
-    ("config4", "pair_bwd_L3"): 49855.3e6 + 23865.9e6,  # k_pair_bwd<double,36>: average of its layer-2 and layer-3 launches
+    ("config4", "pair_bwd_L3"): 64600e6 + 31459e6,      # the layer-3 launches of k_pair_bwd<double,36> (layer 2: 35.2 + 16.3 GB)
 }
 
 
