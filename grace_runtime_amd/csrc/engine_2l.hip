@@ -515,7 +515,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   stage("pair_fwd", [&] {
     const size_t lds = (size_t) kPairChunk * (nslot_ * CRP_ + radR1_.noutp) * sizeof(T);
     GR_PAIR(k_pair_fwd, dim3(n), dim3(nslot_ * CRP_), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), (const T *) M, P,
-            nslot_, CRP_, nl_, radR1_.noutp, yw, sink_.as<T>());
+            nslot_, CRP_, nl_, radR1_.noutp, yw, sink_.as<T>(), 0, n);
   });
   stage("reduce_B", [&] { gemm(jB_, CRP_ / 16, C2P_ / 16, P, npf, B, nB_, 0); });
   chain_forward(c2_, "_L2", B);
@@ -543,7 +543,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     const size_t lds = (size_t) kPairChunk * (pthreads + 2 * radR1_.noutp) * sizeof(T);
     GR_PAIR(k_pair_bwd, dim3(n), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), dR1_.as<T>(),
             (const T *) M, gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),
-            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_);
+            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_, 0, n);
   });
 #undef GR_PAIR
 #undef GR_PAIR1

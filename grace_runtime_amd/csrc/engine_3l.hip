@@ -564,8 +564,8 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
     const int spb = std::max(1, std::min(L.nlmi, 1024 / L.CP)), ngrp = (L.nlmi + spb - 1) / spb;
     stage(tg(k, "pair_fwd").c_str(), [&] {
       const size_t lds = (size_t) kPairChunk * (spb * L.CP + L.rad.noutp) * s;
-      GR_PAIR(k_pair_fwd, dim3(n, ngrp), dim3(spb * L.CP), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), L.R.template as<T>(),
-              (const T *) M_.as<T>(), pairP_.as<T>(), L.nlmi, L.CP, nl_, L.rad.noutp, yw, sink_.as<T>());
+      GR_PAIR(k_pair_fwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(spb * L.CP), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), L.R.template as<T>(),
+              (const T *) M_.as<T>(), pairP_.as<T>(), L.nlmi, L.CP, nl_, L.rad.noutp, yw, sink_.as<T>(), ngrp, n);
     });
     stage(tg(k, "couple_YI").c_str(), [&] {
       const int AT = 64 / L.CP;
@@ -749,9 +749,9 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   const int spb = std::max(1, std::min(L.nlmi, 1024 / L.CP)), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
   stage(tg(k, "pair_bwd").c_str(), [&] {
     const size_t lds = (size_t) kPairChunk * (pthreads + 2 * L.rad.noutp) * s;
-    GR_PAIR(k_pair_bwd, dim3(n, ngrp), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), L.R.template as<T>(),
+    GR_PAIR(k_pair_bwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), L.R.template as<T>(),
             L.dR.template as<T>(), (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(),
-            f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb);
+            f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n);
   });
   (void) yw;
 }

@@ -51,6 +51,22 @@ template<class T> __global__ void k_fill_slot(const int *mu, const T *z, T *M, i
 
 constexpr int kPairChunk = 8;    // bonds staged in LDS at a time by the pair kernels
 
+// Block -> (atom, slot group).  ngrp == 0: a (atoms, groups) grid.  ngrp > 0: a 1-d grid of 8 ceil(atoms / 8) ngrp
+// blocks laid out so that the groups of one atom are blocks b, b + 8, b + 16 ...: workgroups go to the 8 XCDs in turn,
+// so those blocks run on ONE XCD shortly after each other and find the atom's radial rows and harmonics in its L2.
+__device__ inline bool pair_block(int ngrp, int natoms, int &atom, int &grp)
+{
+  if (ngrp == 0) {
+    atom = blockIdx.x;
+    grp = blockIdx.y;
+    return true;
+  }
+  const int b = blockIdx.x, q = b >> 3;
+  grp = q % ngrp;
+  atom = (q / ngrp) * 8 + (b & 7);
+  return atom < natoms;
+}
+
 // Stages what a chunk of nb bonds (edges base .. base + nb) needs into LDS with all loads in flight at once: the
 // neighbour rows M_j[slot][n] of this thread, the radial rows (contiguous in memory), and touches the harmonics of the
 // chunk (the first yuse values of every row of ylen) so that the uniform (scalar) reads of the bond loop find them in
@@ -86,12 +102,14 @@ __device__ inline T pair_stage(const int *__restrict__ ej, const T *__restrict__
 template<class T, int NLM>
 __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ Y,
                            const T *__restrict__ R1, const T *__restrict__ M, T *__restrict__ P, int nslot, int C, int nl, int noutp,
-                           int ystride, T *__restrict__ sink)
+                           int ystride, T *__restrict__ sink, int ngrp, int natoms)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  const int i = blockIdx.x, t = threadIdx.x, NT = blockDim.x;
+  int i, grp;
+  if (!pair_block(ngrp, natoms, i, grp)) return;
+  const int t = threadIdx.x, NT = blockDim.x;
   T *Msh = reinterpret_cast<T *>(smem_raw), *Rsh = Msh + kPairChunk * NT;
-  const int slot_raw = blockIdx.y * (NT / C) + t / C, n = t % C;
+  const int slot_raw = grp * (NT / C) + t / C, n = t % C;
   const bool active = slot_raw < nslot;
   const int slot = active ? slot_raw : 0;
   const int nlm = nl * nl;
@@ -154,13 +172,15 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
                            const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
                            const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
                            T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
-                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb)
+                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   __shared__ double bsum[kPairChunk][4];
-  const int i = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6, NT = blockDim.x;
+  int i, grp;
+  if (!pair_block(ngrp, natoms, i, grp)) return;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, NT = blockDim.x;
   T *Msh = reinterpret_cast<T *>(smem_raw), *Rsh = Msh + kPairChunk * NT, *dRsh = Rsh + kPairChunk * noutp;
-  const int slot_raw = blockIdx.y * spb + t / C;
+  const int slot_raw = grp * spb + t / C;
   const bool active = t < spb * C && slot_raw < nslot;
   const int slot = active ? slot_raw : 0, n = t % C;
   const int nlm = nl * nl;
