@@ -1,15 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the GRACE energy + forces + virial pass on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--precision 64|32] [--no-cpu] [--workload config2|config3]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--precision 64|32] [--no-cpu] [--workload config2|config3|config4]
 
-Default workload (BASELINE.json configs[1], the one the metric is quoted on): GRACE-1L-shaped random-init model (lmax 4, 32 radial channels, 8 Chebyshev
+Default workload (the second benchmark configuration, the one the metric is quoted on): GRACE-1L-shaped random-init model (lmax 4, 32 radial channels, 8 Chebyshev
 functions, radial MLP 8-64-64-160, SiLU) on a bcc W 16x16x16 supercell (8192 atoms, a = 3.165 A, N(0, 0.05 A) jitter,
 r_cut 6 A, 475 136 directed edges), fp64.  A step is one full pass (bond filter, radial MLP, A basis, dense chain,
 readout, reverse pass, forces, virial) over the structure, which is uploaded to HBM before the timed region.
 
---workload config3 runs BASELINE.json configs[2] instead: GRACE-2L-shaped model (two layers, lmax 4, 32 channels, two radial
+--workload config3 runs the third configuration instead: GRACE-2L-shaped model (two layers, lmax 4, 32 channels, two radial
 MLPs 8-64-64-160, body order 3) on the 4-species fcc 20x20x20 alloy (32 000 atoms, ~2.5 M edges), fp64.
+--workload config4 the fourth: GRACE-3L-shaped model (three layers, lmax 5, 64 channels, radial MLPs (8 + 2 x 32)-128-128-384,
+89-species embedding table) on an amorphous cube of 10 000 atoms with 8 species (~0.72 M edges), fp64.
 
 Prints one JSON line: the metric (us/atom per call), the roofline of the dominant kernel (duration from HIP events
 on the engine's stream, algorithmic flops/bytes of that stage) and the reference CPU path timed on this host.
@@ -221,11 +223,11 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "f64" if a.precision == 64 else "f32", "data": "synthetic",
         "config": {"workload": (f"GRACE-3L-shaped random-init model (3 layers, lmax 5, 64 ch, radial MLPs (8 + 2 x 32)-128-128-384, 89-species "
                                 f"embedding table, 8 species present) on an amorphous cube of {N} atoms at 0.08 / A^3, {E} edges, rc 6 A "
-                                f"(BASELINE configs[3])") if three else
+                                f"(benchmark configuration 4)") if three else
                                (f"GRACE-2L-shaped random-init model (2 layers, lmax 4, 32 ch, MLPs 8-64-64-160, body order 3) on the "
-                                f"4-species fcc alloy {reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[2])") if two else
+                                f"4-species fcc alloy {reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (benchmark configuration 3)") if two else
                                (f"GRACE-1L-shaped random-init model (lmax 4, 32 ch, MLP 8-64-64-160) on bcc W "
-                                f"{reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (BASELINE configs[1])"),
+                                f"{reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (benchmark configuration 2)"),
                    "atoms": N, "edges": int(E)},
         "atoms_steps_per_s": round(N / dt, 1),
         "ms_per_call_host_buffers": round(host_ms, 3),
