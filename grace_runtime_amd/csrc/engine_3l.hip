@@ -32,12 +32,15 @@ template<class T> struct DevContract {
   };
   DevBuf WF, WT;
   DevJobs<T> fwd, bwd;
+  int nel = 1;                                  // weight sets: 1, or one per element (wget(el * nt + t, n, k))
+  size_t wstride = 0, wtstride = 0;             // values of one weight set, forward / transposed
   int kin = 0, kout = 0, nsrc = 0, ndst = 0;    // padded widths, functions of the source and destination tensors
   bool all_dst = false, all_src = false;        // every destination / source function has a connection
   template<class WGet>
   void build(int nin, int nout, int nt, const std::vector<Conn> &conns, WGet wget, const std::vector<double> &dscale, int nsrc_, int ndst_,
-             const int *drow, const std::string &what)
+             const int *drow, const std::string &what, int nel_ = 1)
   {
+    nel = nel_;
     kin = pad_width(nin);
     kout = pad_width(nout);
     nsrc = nsrc_;
@@ -45,7 +48,8 @@ template<class T> struct DevContract {
     if (kin < 0 || kout < 0) throw Error("GRACE-3L: " + what + ": channel widths above 64 are not supported by the GPU kernels");
     std::vector<T> F, Ft;
     std::vector<double> M((size_t) nin * nout), Mt((size_t) nout * nin);
-    for (int t = 0; t < nt; t++) {
+    for (int t = 0; t < nel * nt; t++) {
+      if (t == nt) { wstride = F.size(); wtstride = Ft.size(); }
       for (int n = 0; n < nin; n++)
         for (int k = 0; k < nout; k++) {
           const double v = wget(t, n, k);
@@ -191,8 +195,23 @@ template<class T> class Engine3L final : public EngineBase {
   {
     EngineBase::launch_gemm<T>(J, kin / 16, kin / 16, kout / 16, X, nfx, X, nfx, out, nfo, accumulate, tiles_.as<int>(), ntiles_);
   }
-  void cfwd(DevContract<T> &c, const T *X, T *out, int accumulate) { gemm(c.fwd, c.kin, c.kout, X, c.nsrc, out, c.ndst, accumulate); }
-  void cbwd(DevContract<T> &c, const T *gout, T *gX, int accumulate) { gemm(c.bwd, c.kout, c.kin, gout, c.ndst, gX, c.nsrc, accumulate); }
+  // element-dependent weights: one launch per element over its tiles (tiles hold atoms of one element, elements in order)
+  void gemm_el(DevJobs<T> &J, size_t wstride, int nel, int kin, int kout, const T *X, int nfx, T *out, int nfo, int accumulate)
+  {
+    if (nel == 1) return gemm(J, kin, kout, X, nfx, out, nfo, accumulate);
+    const T *w0 = J.d.WF0, *w1 = J.d.WF1;
+    for (int e = 0; e < nel; e++) {
+      const int t0 = tile_el_[e], nt = tile_el_[e + 1] - t0;
+      if (nt == 0) continue;
+      J.d.WF0 = w0 + e * wstride;
+      J.d.WF1 = w1 + e * wstride;
+      EngineBase::launch_gemm<T>(J, kin / 16, kin / 16, kout / 16, X, nfx, X, nfx, out, nfo, accumulate, tiles_.as<int>() + (size_t) 16 * t0, nt);
+    }
+    J.d.WF0 = w0;
+    J.d.WF1 = w1;
+  }
+  void cfwd(DevContract<T> &c, const T *X, T *out, int accumulate) { gemm_el(c.fwd, c.wstride, c.nel, c.kin, c.kout, X, c.nsrc, out, c.ndst, accumulate); }
+  void cbwd(DevContract<T> &c, const T *gout, T *gX, int accumulate) { gemm_el(c.bwd, c.wtstride, c.nel, c.kout, c.kin, gout, c.ndst, gX, c.nsrc, accumulate); }
   void zero(void *p, size_t bytes) { if (bytes) HIP_CHECK(hipMemsetAsync(p, 0, bytes, stream_)); }
   // out = contraction (not accumulated): functions without a connection are cleared
   void cfwd_set(DevContract<T> &c, const T *X, T *out)
@@ -316,13 +335,17 @@ template<class T> void Engine3L<T>::build_layer(int k)
     upload_vec(L.fac, fac);
   }
   typedef typename DevContract<T>::Conn Conn;
-  // a reduce instruction as a contraction; W: [n_out][n_in][w_shape], not element dependent
+  // a reduce instruction as a contraction; W: [n_elements |] [n_out][n_in][w_shape]
   auto instr_contract = [&](DevContract<T> &c, const Model3L::Reduce &r, const Model3L::Instr &ins, int nsrc, const std::string &what) {
-    if (r.elem_dep) throw Error("GRACE-3L: " + what + ": element-dependent weights are supported for the rho reduces only");
     std::vector<Conn> conns;
     for (size_t q = 0; q < ins.collect_ind.size(); q++) conns.push_back({ins.collect_ind[q], r.only_invar ? 0 : ins.total_sum_ind[q], ins.w_l_tile[q]});
+    const size_t per = (size_t) r.n_out * ins.n_in * ins.w_shape;
     c.build(ins.n_in, r.n_out, ins.w_shape, conns,
-            [&](int t, int n, int kk) { return ins.norm * ins.W[((size_t) kk * ins.n_in + n) * ins.w_shape + t]; }, r.norm_map, nsrc, r.nfo(), drow_, what);
+            [&](int t, int n, int kk) {
+              const int el = t / ins.w_shape, tt = t % ins.w_shape;
+              return ins.norm * ins.W[el * per + ((size_t) kk * ins.n_in + n) * ins.w_shape + tt];
+            },
+            r.norm_map, nsrc, r.nfo(), drow_, what, r.elem_dep ? nel_ : 1);
   };
   L.X.nf = nlm_;
   if (L.equiv) {

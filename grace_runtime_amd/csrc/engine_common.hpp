@@ -490,7 +490,7 @@ class EngineBase : public Engine {
     };
     put(mu_, mu.data(), sizeof(int) * n);
     if (have_sid_) put(sid_, in.sid, sizeof(int) * n);
-    const std::vector<int> tiles = element_tiles(mu);
+    const std::vector<int> tiles = element_tiles(mu, nelem_, tile_el_);
     ntiles_ = (int) tiles.size() / 16;
     put(tiles_, tiles.data(), sizeof(int) * tiles.size());
     static_assert(sizeof(long long) == sizeof(int64_t), "offset type");
@@ -529,7 +529,7 @@ class EngineBase : public Engine {
       if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, kind, stream_));
     };
     put(mu_, mu.data(), sizeof(int) * n, hipMemcpyHostToDevice);
-    const std::vector<int> tiles = element_tiles(mu);
+    const std::vector<int> tiles = element_tiles(mu, nelem_, tile_el_);
     ntiles_ = (int) tiles.size() / 16;
     put(tiles_, tiles.data(), sizeof(int) * tiles.size(), hipMemcpyHostToDevice);
     put(offset_, in.offset, sizeof(int64_t) * (n + 1), hipMemcpyDeviceToDevice);
@@ -550,19 +550,23 @@ class EngineBase : public Engine {
     ran_ = false;
   }
   int device_index() const override { return device_; }
-  // tiles of 16 atoms of one element (-1 padded), in atom order within an element
-  static std::vector<int> element_tiles(const std::vector<int> &mu)
+  // tiles of 16 atoms of one element (-1 padded), in atom order within an element, elements ascending;
+  // el_off[e] .. el_off[e + 1]: the tiles of element e
+  static std::vector<int> element_tiles(const std::vector<int> &mu, int nel, std::vector<int> &el_off)
   {
     const int n = (int) mu.size();
     std::vector<int> tiles, ord(n);
     std::iota(ord.begin(), ord.end(), 0);
     std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return mu[a] < mu[b]; });
+    el_off.assign(nel + 1, 0);
     for (int q = 0; q < n;) {
       int cnt = 0;
       const int m0 = mu[ord[q]];
       while (cnt < 16 && q < n && mu[ord[q]] == m0) { tiles.push_back(ord[q]); q++; cnt++; }
       while (cnt < 16) { tiles.push_back(-1); cnt++; }
+      el_off[m0 + 1]++;
     }
+    for (int e = 0; e < nel; e++) el_off[e + 1] += el_off[e];
     return tiles;
   }
   void fetch(double *energy, double *forces, double *virial, double *eatom) override
@@ -840,6 +844,7 @@ class EngineBase : public Engine {
   bool have_rij_ = false;
   DevBuf cut_, mu_, sid_, offset_, j_, rij_, x_, image_, shifts_, tiles_;
   int ntiles_ = 0, nstruct_ = 1;
+  std::vector<int> tile_el_;    // [nel + 1] tile range of every element
   bool have_sid_ = false;
   const int *sid_ptr() const { return have_sid_ ? sid_.as<int>() : nullptr; }
   // edges of the pass and its outputs (scal: energy, virial[6])

@@ -662,7 +662,7 @@ def _coupled_functions(left, right, out, paths):
     return terms, np.array(fn_path, np.int32), np.array(fn_dst, np.int32), np.array(fn_l, np.int32)
 
 
-def structure_3l(lmax, lmsg=None, pseudo_message=True):
+def structure_3l(lmax, lmsg=None, pseudo_message=True, elem_dep=False):
     """Structure arrays (no weights) of a GRACE-3L model, keys as libgrace/src/model_3l.cpp:165-464 reads them.
 
     Irreps are (l, s), s = 1 for pseudo-tensors.  Per layer K = A1, A2, A3 the lm features X are the natural irreps
@@ -670,7 +670,8 @@ def structure_3l(lmax, lmsg=None, pseudo_message=True):
     reduces K_2_red, K_3_red, K_4_red carry the natural irreps l <= lmax and, in layer 2 when `pseudo_message`, the
     pseudo irreps too; the message eq1 holds the natural irreps l <= lmsg, eq2 those and (pseudo_message) their
     pseudo partners.  Every coupling the triangle and parity rules allow is one path with its own weight tile.
-    Returns the arrays and '_sizes'."""
+    `elem_dep`: the eq reduces and the reduces of the equivariant SPBFs carry one weight set per element of the
+    central atom (the rho reduces always do).  Returns the arrays and '_sizes'."""
     lmsg = lmax if lmsg is None else lmsg
     nl = lmax + 1
     nlm = nl * nl
@@ -795,7 +796,7 @@ def structure_3l(lmax, lmsg=None, pseudo_message=True):
             s[f"{red}_norm_map"] = 1.0 / np.sqrt(np.maximum(cnt, 1.0))
             s[f"{red}_n_funcs"] = i64(nlm)
             s[f"{red}_only_invar"] = i64(0)
-            s[f"{red}_is_central_atom_type_dependent"] = i64(0)
+            s[f"{red}_is_central_atom_type_dependent"] = i64(1 if elem_dep else 0)
             s[f"{red}_instruction_names"] = np.array([K.encode()], dtype="|S8")
             sizes[red] = dict(nfunc=nlm, w_shape={K: len(paths)})
             reds.append(red)
@@ -817,7 +818,7 @@ def structure_3l(lmax, lmsg=None, pseudo_message=True):
         sources = [(Xn, X), (K + "_2_red", T), (K + "_3_red", T), (K + "_4_red", T)]
         if k < 3:
             message = list(nat_msg) + ([(l, 1) for l in range(lmsg + 1)] if (k == 2 and pseudo_message) else [])
-            collect_reduce(f"eq{k}", sources, message, False, False)
+            collect_reduce(f"eq{k}", sources, message, False, elem_dep)
             reds.append(f"eq{k}")
             mo = _irrep_offsets(message)
             M = int(mo[-1])
@@ -842,7 +843,7 @@ def structure_3l(lmax, lmsg=None, pseudo_message=True):
     return s
 
 
-def random_model_3l(*, lmax=4, lmsg=None, pseudo_message=True, n_elements=8, element_names=None, embedding_size=32,
+def random_model_3l(*, lmax=4, lmsg=None, pseudo_message=True, elem_dep=False, n_elements=8, element_names=None, embedding_size=32,
                     nradbase=8, channels=64, hidden=128, rho_n_out=32, energy_hidden=64, rcut=6.0, p=5,
                     inv_avg_n_neigh=1.0 / 72.0, rms_type=1, seed=20260104):
     """A GRACE-3L-shaped model (three layers: scalar SPBF, then two equivariant SPBFs coupling the normalised
@@ -851,7 +852,7 @@ def random_model_3l(*, lmax=4, lmsg=None, pseudo_message=True, n_elements=8, ele
     reads them, libgrace/src/model_3l.cpp:165-464."""
     rng = np.random.default_rng(seed)
     nl = lmax + 1
-    s = structure_3l(lmax, lmsg, pseudo_message)
+    s = structure_3l(lmax, lmsg, pseudo_message, elem_dep)
     z = s.pop("_sizes")
     C = channels
     i64 = lambda v: np.array([v], dtype=np.int64)
@@ -903,8 +904,8 @@ def random_model_3l(*, lmax=4, lmsg=None, pseudo_message=True, n_elements=8, ele
     for red, info in z.items():
         if "w_shape" not in info:
             continue
-        elem = red.startswith("rho")
-        n_out = rho_n_out if elem else C
+        elem = bool(int(s[f"{red}_is_central_atom_type_dependent"][0]))
+        n_out = rho_n_out if red.startswith("rho") else C
         for src, w_shape in info["w_shape"].items():
             d[f"{red}_reduce_{src}_W"] = N(n_elements, n_out, C, w_shape) if elem else N(n_out, C, w_shape)
             d[f"{red}_reduce_{src}_norm"] = f64(1.0 / math.sqrt(C))

@@ -83,6 +83,13 @@ def model_l3pad():
                                  seed=24)
 
 
+def model_l3el():
+    """GRACE-3L whose eq reduces and SPBF reduces carry one weight set per element of the central atom"""
+    return synth.random_model_3l(lmax=2, lmsg=1, elem_dep=True, n_elements=2, element_names=("Mo", "W"), embedding_size=6,
+                                 nradbase=8, channels=16, hidden=32, rho_n_out=8, energy_hidden=16, rcut=5.0,
+                                 inv_avg_n_neigh=1.0 / 26.0, seed=25)
+
+
 def model_l3nat():
     """GRACE-3L with natural-parity messages only, one element, lmax 2"""
     return synth.random_model_3l(lmax=2, pseudo_message=False, n_elements=1, element_names=("W",), embedding_size=4, nradbase=8,
@@ -97,8 +104,8 @@ def model_config4():
                                  energy_hidden=64, rcut=6.0, inv_avg_n_neigh=1.0 / 72.0, seed=20260104)
 
 
-MODELS = {"l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
-LAYERS = {"l3mix": 3, "l3wide": 3, "l3pad": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
+MODELS = {"l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3el": model_l3el, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
+LAYERS = {"l3mix": 3, "l3wide": 3, "l3pad": 3, "l3el": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
 
 
 def write_model(name, directory):
@@ -247,7 +254,7 @@ E2E_CASES_2L = [("config3", "fcc108", None), ("l2mix", "alloy54", 5.5), ("l2mix"
                 ("l2mix", "molecule", None)]
 # reference fixture models (tests/golden/ref_fixtures) on the reference's fixture cells: goldens of the compiled reference
 E2E_CASES_3L = [("l3mix", "alloy54", 5.5), ("l3mix", "triclinic", None), ("l3mix", "slab", None), ("l3mix", "molecule", None),
-                ("l3wide", "fcc108", None), ("l3nat", "config1", None)]
+                ("l3wide", "fcc108", None), ("l3nat", "config1", None), ("l3el", "alloy54", None)]
 FIXTURE_CASES_2L = [(m, c) for m in ("grace_2l_small", "grace_2l_l3", "legacy_2l_small", "legacy_2l_wide") for c in ("W54", "WMo54")]
 
 
