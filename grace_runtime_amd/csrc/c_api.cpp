@@ -391,6 +391,75 @@ int gr_compute(gr_engine *e, int n, const int *types, const double *positions, c
   });
 }
 
+int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const double *x, int inum, const int *ilist, const int *numneigh,
+                      const int *const *firstneigh, int neighmask, const int *owner, unsigned flags, double *energy, double *f,
+                      double *virial, double *eatom)
+{
+  return guarded([&] {
+    if (!e || (nall > 0 && (!type || !x)) || (inum > 0 && (!ilist || !numneigh || !firstneigh))) throw grhip::InvalidArgument("null argument");
+    if (nlocal < 0 || nall < nlocal || inum < 0) throw grhip::InvalidArgument("atom counts out of range");
+    grhip::Engine &eng = *e->eng;
+    // atoms of types the engine has no element for take no part (pair_style hybrid): neither central atoms nor neighbours
+    auto mapped = [&](int a) { return eng.cutoff(type[a], type[a]) > 0.0; };
+    std::vector<int> idx(nlocal, -1), atom;
+    std::vector<char> central(nlocal, 0);
+    for (int q = 0; q < inum; q++) {
+      const int i = ilist[q];
+      if (i < 0 || i >= nlocal) throw grhip::InvalidArgument("ilist must index owned atoms");
+      if (!mapped(i)) throw grhip::Error("atom " + std::to_string(i) + " of unmapped type " + std::to_string(type[i]) + " in the atom list");
+      central[i] = 1;
+    }
+    for (int i = 0; i < nlocal; i++) {
+      if (!mapped(i)) continue;
+      if (!central[i]) throw grhip::InvalidArgument("every owned atom of a mapped type must be in ilist (sub-lists are not supported)");
+      idx[i] = (int) atom.size();
+      atom.push_back(i);
+    }
+    const int n = (int) atom.size();
+    std::vector<int> ty(n), jj;
+    std::vector<int64_t> offset(n + 1, 0);
+    std::vector<double> rij;
+    for (int q = 0; q < n; q++) {
+      const int i = atom[q];
+      ty[q] = type[i];
+      const int *nb = firstneigh[i];
+      for (int k = 0; k < numneigh[i]; k++) {
+        const int j = nb[k] & neighmask;
+        if (j < 0 || j >= nall) throw grhip::InvalidArgument("neighbour index outside the owned and ghost atoms");
+        if (!mapped(j)) continue;
+        int o = j;
+        if (j >= nlocal) {
+          if (!owner) throw grhip::InvalidArgument("ghost neighbours need the owner map (the owned atom each ghost is an image of)");
+          o = owner[j];
+        }
+        if (o < 0 || o >= nlocal || idx[o] < 0 || type[o] != type[j])
+          throw grhip::InvalidArgument("owner of ghost atom " + std::to_string(j) + " is not an owned atom of the same type");
+        jj.push_back(idx[o]);
+        for (int d = 0; d < 3; d++) rij.push_back(x[3 * (size_t) j + d] - x[3 * (size_t) i + d]);
+      }
+      offset[q + 1] = (int64_t) jj.size();
+    }
+    const std::vector<double> dummy(3, 0.0);
+    eng.upload(make_input(n, ty.data(), offset.data(), jj.data(), rij.empty() ? dummy.data() : rij.data(), nullptr, nullptr, nullptr, 0));
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    eng.run(fl);
+    std::vector<double> fo((size_t) 3 * n), ea(fl.eatom ? n : 0);
+    double en = 0.0, vir[6] = {0, 0, 0, 0, 0, 0};
+    eng.fetch(&en, f ? fo.data() : nullptr, vir, fl.eatom ? ea.data() : nullptr);
+    if (energy) *energy = en;
+    if (virial && !fl.energy_only)
+      for (int k = 0; k < 6; k++) virial[k] = vir[k];
+    for (int q = 0; q < n; q++) {
+      const int i = atom[q];
+      if (f && !fl.energy_only)
+        for (int d = 0; d < 3; d++) f[3 * (size_t) i + d] += fo[3 * (size_t) q + d];
+      if (fl.eatom) eatom[i] += ea[q];
+    }
+  });
+}
+
 int gr_system_create(gr_engine *e, double skin, gr_system **out)
 {
   return guarded([&] {

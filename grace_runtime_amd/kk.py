@@ -130,9 +130,13 @@ class Model:
         raise ValueError(f"GRACE-{self.layers}L: the model has no UQ head")
 
     def type2mu(self, species):
-        """[-1, mu(species[0]), ...]; unknown element -> ValueError (python/kk/kk_core.cpp: std::invalid_argument)"""
+        """[-1, mu(species[0]), ...]; unknown element -> ValueError (python/kk/kk_core.cpp: std::invalid_argument);
+        None leaves the atom type unmapped (-1), the NULL of a LAMMPS pair_coeff line"""
         out = [-1]
         for s in species:
+            if s is None:
+                out.append(-1)
+                continue
             if s not in self.element_names:
                 raise ValueError(f"element {s} is not in the model (elements: {' '.join(self.element_names)})")
             out.append(self.element_names.index(s))
@@ -196,6 +200,33 @@ class Engine:
         else:
             nimg = 0 if shifts is None else shifts.shape[0]
         return n, (types, offset, j, rij, positions, image, shifts), nimg
+
+    def compute_lammps(self, nlocal, types, x, ilist, numneigh, firstneigh, owner=None, neighmask=0x1FFFFFFF, energies=False,
+                       energy_only=False, forces=None, eatom=None):
+        """The call of a LAMMPS pair style (gr_compute_lammps): owned + ghost atoms `x[nall, 3]`, `types[nall]`, the full
+        neighbour list as `numneigh[nlocal]` and a list of index arrays `firstneigh[i]`, `owner[nall]` the owned atom of every
+        ghost.  Forces are ADDED to `forces[nall, 3]` (zeros when not given), per-atom energies to `eatom[nall]`."""
+        types = as_array(types, np.int32)
+        x = as_array(x, np.float64, 3)
+        nall = types.shape[0]
+        ilist = as_array(ilist, np.int32)
+        numneigh = as_array(numneigh, np.int32)
+        rows = [np.ascontiguousarray(r, dtype=np.int32) for r in firstneigh]
+        fn = (C.c_void_p * max(len(rows), 1))(*[r.ctypes.data if r.size else None for r in rows])
+        own = as_array(owner, np.int32) if owner is not None else None
+        f = np.zeros((nall, 3)) if forces is None else forces
+        ea = (np.zeros(nall) if eatom is None else eatom) if energies else None
+        e, v = C.c_double(), np.zeros(6)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
+        check(_lib.lib().gr_compute_lammps(self._h, int(nlocal), nall, ptr(types), ptr(x), ilist.shape[0], ptr(ilist), ptr(numneigh), fn,
+                                           int(neighmask), ptr(own) if own is not None else None, flags, C.byref(e),
+                                           None if energy_only else ptr(f), ptr(v), ptr(ea) if ea is not None else None))
+        out = {"energy": e.value}
+        if not energy_only:
+            out["forces"], out["virial"] = f, v
+        if energies:
+            out["energies"] = ea
+        return out
 
     def compute(self, types, offset, j, rij=None, energies=False, energy_only=False, positions=None, image=None,
                 shifts=None):

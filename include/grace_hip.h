@@ -121,6 +121,21 @@ void gr_nlist_free(gr_nlist *l);
 int gr_compute(gr_engine *e, int n, const int *types, const double *positions, const double *cell,
                const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom);
 
+/* The call of a LAMMPS pair style on one MPI rank: owned and ghost atoms with LAMMPS' full neighbour list.  Replaces
+ * Grace{1,2,3}LFused::compute<LammpsBonds>(inum, ilist, n_nodes, nmax_nodes, LammpsBonds{x, type, numneigh, firstneigh,
+ * neighmask}, Exchange&, Outputs&, flags, nthreads) (libgrace/include/grace/system.h:14-20, fused_1l.h:41, fused_2l.h:49,
+ * fused_3l.h:44) and the RunInput / RunOutput of the reference's GPU engines (kk/grace_1l_kk.h:80-113).
+ * x [nall][3], type [nall] (1-based); neighbour indices are masked with neighmask (0x1FFFFFFF in LAMMPS); atoms of types
+ * without a model element take no part.  owner [nall]: for a ghost atom the owned atom it is a periodic image of (LAMMPS:
+ * atom->map(tag[j])); it stands in for the Exchange of the reference: the message of a ghost is its owner's, and what
+ * the reference leaves on the ghosts for the reverse communication (forces, message adjoints) is added to the owner here.
+ * May be NULL when no neighbour is a ghost.  Ghosts owned by another rank are not supported (one GPU, one rank).
+ * As the reference's Outputs (system.h:66-75): forces are ADDED to f [nall][3], per-atom energies to eatom [nall];
+ * energy and virial (xx yy zz xy xz yz) are returned.  ilist must hold every owned atom of a mapped type. */
+int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const double *x, int inum, const int *ilist, const int *numneigh,
+                      const int *const *firstneigh, int neighmask, const int *owner, unsigned flags, double *energy, double *f,
+                      double *virial, double *eatom);
+
 /* One structure resident on the device with a Verlet list at cutoff + skin: System of the reference's GPU module
  * (python/kk/kk_api.h:66-93, System::compute python/kk/kk_core.cpp:802-958; list policy python/grace_runtime/
  * neighbors.py:68-89: rebuild when types, cell or pbc change or an atom moved more than skin / 2).  The pair search of
