@@ -24,7 +24,7 @@ SYMBOLS = [
     "gr_engine_debug_radial", "gr_engine_debug_copy", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
-    "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps",
+    "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device",
 ]
 
 
@@ -44,6 +44,13 @@ def lib():
     if not os.path.exists(LIB_PATH):
         raise RuntimeError(f"{LIB_PATH} is missing: build it with `make -C grace_runtime_amd/csrc` "
                            "(there is no CPU fallback in this package)")
+    # One HIP runtime per process.  PyTorch ships a copy of its own: when PyTorch is installed it is imported BEFORE
+    # the library is opened, so that the library binds to the runtime PyTorch uses and device arrays can be shared
+    # (Batch.compute_device).  With the library opened first, PyTorch would bring up a second runtime and find no GPU.
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(LIB_PATH)
     vp, i32, i64, dbl, u32 = C.c_void_p, C.c_int, C.c_int64, C.c_double, C.c_uint
     L.gr_last_error.restype = C.c_char_p
@@ -82,6 +89,7 @@ def lib():
     L.gr_compute_batch.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, i32, vp, vp, vp, vp]
     L.gr_engine_upload_batch.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i32, vp]
     L.gr_engine_fetch_batch.argtypes = [vp, i32, vp, vp, vp, vp]
+    L.gr_compute_batch_device.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, vp, vp, vp, vp]
     L.gr_compute_lammps.argtypes = [vp, i32, i32, vp, vp, i32, vp, vp, vp, i32, vp, u32, vp, vp, vp, vp]
     L.gr_system_create.argtypes = [vp, dbl, C.POINTER(vp)]
     L.gr_system_free.argtypes = [vp]

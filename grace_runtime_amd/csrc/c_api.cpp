@@ -5,6 +5,7 @@
 #include "engine.hpp"
 #include "neighbors.hpp"
 #include "neighbors_dev.hpp"
+#include "neighbors_batch_dev.hpp"
 
 #include <hip/hip_runtime_api.h>
 
@@ -25,6 +26,12 @@ struct gr_model {
 struct gr_engine {
   std::unique_ptr<grhip::Engine> eng;
   std::vector<grhip::StageTime> times;
+  std::unique_ptr<grhip::BatchDeviceNeighbors> bnl;    // lists of gr_compute_batch_device (buffers kept between calls)
+  hipStream_t bnl_stream = nullptr;
+  ~gr_engine()
+  {
+    if (bnl_stream) (void) hipStreamDestroy(bnl_stream);
+  }
 };
 struct gr_nlist {
   grhip::NeighborList nl;
@@ -776,6 +783,68 @@ int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *ty
           for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) w + d];
         if (fl.eatom) eatom[a] = ea[w];
       }
+  });
+}
+
+int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
+                            const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom)
+{
+  return guarded([&] {
+    if (!e || nstruct < 0 || (nstruct > 0 && (!natoms || !cells || !pbc))) throw grhip::InvalidArgument("null argument");
+    if (nstruct == 0) return;
+    const double rc = e->eng->max_cutoff();
+    if (!(rc > 0.0)) throw grhip::Error("the engine has no positive cutoff");
+    int64_t N = 0;
+    for (int s = 0; s < nstruct; s++) {
+      if (natoms[s] < 0) throw grhip::InvalidArgument("negative atom count");
+      N += natoms[s];
+    }
+    if (N >= INT32_MAX) throw grhip::InvalidArgument("atom count out of range");
+    if (N > 0 && (!types || !positions)) throw grhip::InvalidArgument("null argument");
+    if (hipSetDevice(e->eng->device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
+    // the pointers must be memory of the engine's GPU: a host pointer here would fault in the kernels
+    auto on_device = [&](const void *p, const char *name) {
+      if (!p) return;
+      hipPointerAttribute_t at;
+      if (hipPointerGetAttributes(&at, p) != hipSuccess || at.type != hipMemoryTypeDevice || at.device != e->eng->device_index()) {
+        (void) hipGetLastError();
+        throw grhip::InvalidArgument(std::string(name) + " must be memory of the engine's GPU");
+      }
+    };
+    on_device(types, "types");
+    on_device(positions, "positions");
+    on_device(energy, "energy");
+    on_device(forces, "forces");
+    on_device(virial, "virial");
+    on_device(eatom, "energies");
+    if (!e->bnl) {
+      e->bnl = std::make_unique<grhip::BatchDeviceNeighbors>();
+      if (hipStreamCreateWithFlags(&e->bnl_stream, hipStreamNonBlocking) != hipSuccess) throw grhip::Error("hipStreamCreate failed");
+    }
+    // work queued by the caller on the default stream (the tensors that hold the inputs) is finished first
+    if (hipDeviceSynchronize() != hipSuccess) throw grhip::Error("hipDeviceSynchronize failed");
+    grhip::BatchDeviceNeighbors &nl = *e->bnl;
+    nl.build(nstruct, natoms, positions, cells, pbc, rc, e->bnl_stream);
+    // atom types: 4 bytes per atom to the host, where the element tiles of the tile GEMMs are laid out
+    std::vector<int> ty((size_t) N);
+    if (N > 0 && hipMemcpyAsync(ty.data(), types, sizeof(int) * (size_t) N, hipMemcpyDeviceToHost, e->bnl_stream) != hipSuccess)
+      throw grhip::Error("copy of the atom types failed");
+    if (hipStreamSynchronize(e->bnl_stream) != hipSuccess) throw grhip::Error("the device neighbour search failed");
+    grhip::DeviceCsr in;
+    in.n = (int) N;
+    in.types = ty.data();
+    in.nb = nl.nb;
+    in.offset = nl.offset.as<int64_t>();
+    in.j = nl.j.as<int>();
+    in.rij = nl.rij.as<double>();
+    in.nstruct = nstruct;
+    in.sid = nl.sid.data();
+    e->eng->upload_device(in);
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    e->eng->run(fl);
+    e->eng->fetch_batch_device(nstruct, energy, forces, virial, fl.eatom ? eatom : nullptr);
   });
 }
 }

@@ -40,6 +40,9 @@ struct DeviceCsr {
   const double *x = nullptr;          // device [n][3]
   const double *shifts = nullptr;     // host [nimages][3]
   int64_t nimages = 0;
+  const double *rij = nullptr;        // device [nb][3] bond vectors, in place of (image, x, shifts)
+  int nstruct = 1;                    // several independent structures in one list:
+  const int *sid = nullptr;           // host [n] structure of every atom, or null for one structure
 };
 
 struct StageTime {
@@ -72,6 +75,8 @@ class Engine {
   virtual void fetch(double *energy, double *forces, double *virial, double *eatom) = 0;
   // the same for a list of several structures: energy [nstruct], virial [nstruct][6]
   virtual void fetch_batch(int nstruct, double *energy, double *forces, double *virial, double *eatom) = 0;
+  // the same with every output in device memory (the engine's GPU); null pointers are skipped
+  virtual void fetch_batch_device(int nstruct, double *energy, double *forces, double *virial, double *eatom) = 0;
   virtual void synchronize() = 0;
   virtual void set_profile(bool on) = 0;
   virtual const std::vector<StageTime> &stage_times() = 0;

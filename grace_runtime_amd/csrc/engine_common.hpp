@@ -518,12 +518,16 @@ class EngineBase : public Engine {
         throw Error(who_ + ": atom " + std::to_string(a) + " of unmapped type " + std::to_string(in.types[a]) + " in the atom list");
     }
     HIP_CHECK(hipStreamSynchronize(stream_));
+    if (in.nstruct < 1) throw InvalidArgument("the number of structures must be positive");
+    if (in.sid)
+      for (int a = 0; a < n; a++)
+        if (in.sid[a] < 0 || in.sid[a] >= in.nstruct) throw InvalidArgument("structure index of an atom out of range");
     n_ = n;
     nb_ = in.nb;
-    nstruct_ = 1;
-    have_sid_ = false;
-    have_rij_ = false;
-    scal_.ensure(8 * sizeof(double));
+    nstruct_ = in.sid ? in.nstruct : 1;
+    have_sid_ = in.sid != nullptr;
+    have_rij_ = in.rij != nullptr;
+    scal_.ensure((size_t) 8 * nstruct_ * sizeof(double));
     auto put = [&](DevBuf &b, const void *src, size_t bytes, hipMemcpyKind kind) {
       b.ensure(std::max<size_t>(bytes, 8));
       if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, kind, stream_));
@@ -534,9 +538,13 @@ class EngineBase : public Engine {
     put(tiles_, tiles.data(), sizeof(int) * tiles.size(), hipMemcpyHostToDevice);
     put(offset_, in.offset, sizeof(int64_t) * (n + 1), hipMemcpyDeviceToDevice);
     put(j_, in.j, sizeof(int) * in.nb, hipMemcpyDeviceToDevice);
-    put(image_, in.image, sizeof(int) * in.nb, hipMemcpyDeviceToDevice);
-    put(x_, in.x, sizeof(double) * 3 * n, hipMemcpyDeviceToDevice);
-    put(shifts_, in.shifts, sizeof(double) * 3 * in.nimages, hipMemcpyHostToDevice);
+    if (have_sid_) put(sid_, in.sid, sizeof(int) * n, hipMemcpyHostToDevice);
+    if (have_rij_) put(rij_, in.rij, sizeof(double) * 3 * in.nb, hipMemcpyDeviceToDevice);
+    else {
+      put(image_, in.image, sizeof(int) * in.nb, hipMemcpyDeviceToDevice);
+      put(x_, in.x, sizeof(double) * 3 * n, hipMemcpyDeviceToDevice);
+      put(shifts_, in.shifts, sizeof(double) * 3 * in.nimages, hipMemcpyHostToDevice);
+    }
     HIP_CHECK(hipStreamSynchronize(stream_));
     ran_ = false;
   }
@@ -596,6 +604,24 @@ class EngineBase : public Engine {
     }
     if (forces && ran_forces_ && n_ > 0) HIP_CHECK(hipMemcpy(forces, f_.p, sizeof(double) * 3 * n_, hipMemcpyDeviceToHost));
     if (eatom && ran_eatom_ && n_ > 0) HIP_CHECK(hipMemcpy(eatom, eatom_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
+  }
+  void fetch_batch_device(int nstruct, double *energy, double *forces, double *virial, double *eatom) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (!ran_) throw Error("fetch() before run()");
+    if (nstruct != nstruct_) throw InvalidArgument("fetch_batch: the uploaded list holds " + std::to_string(nstruct_) + " structures");
+    hipLaunchKernelGGL(k_unpack_records, dim3((unsigned) ((nstruct_ + 255) / 256)), dim3(256), 0, stream_, scal_.as<double>(), nstruct_, energy,
+                       ran_forces_ ? virial : nullptr);
+    if (forces && ran_forces_ && n_ > 0) HIP_CHECK(hipMemcpyAsync(forces, f_.p, sizeof(double) * 3 * n_, hipMemcpyDeviceToDevice, stream_));
+    if (eatom && ran_eatom_ && n_ > 0) HIP_CHECK(hipMemcpyAsync(eatom, eatom_.p, sizeof(double) * n_, hipMemcpyDeviceToDevice, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    if (n_ > 0) {
+      int zb[2];
+      HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
+      if (zb[0] >= 0)    // bonds.h:49-62
+        throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " +
+                    std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
+    }
   }
   int64_t last_edge_count() override
   {

@@ -183,6 +183,16 @@ static __global__ void k_scan(const int *count, int n, long long *eoff)
   if (threadIdx.x == 0) eoff[n] = carry;
 }
 
+// (energy, virial[6], unused) records of the structures -> energy [nstruct], virial [nstruct][6] (null: skipped)
+static __global__ void k_unpack_records(const double *rec, int nstruct, double *energy, double *virial)
+{
+  const int s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= nstruct) return;
+  if (energy) energy[s] = rec[8 * (long long) s];
+  if (virial)
+    for (int k = 0; k < 6; k++) virial[6 * (long long) s + k] = rec[8 * (long long) s + 1 + k];
+}
+
 struct Edges {
   int *ei, *ej, *emu;         // central atom, neighbour, neighbour element
   double *rh;                 // [E][3] unit vectors

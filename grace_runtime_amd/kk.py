@@ -449,3 +449,51 @@ class Batch:
         if energies:
             out["energies"] = ea
         return out
+
+    def compute_device(self, natoms, types, positions, cells, pbc, energy, forces=None, virial=None, energies=None,
+                       gamma=None, atomic_sigma=None, gmm_cluster=None, energy_only=False, max_nall=1 << 21):
+        """`Batch.compute_device` of the reference module (python/kk/kk_module.cpp:142-193): `types` int32 [N],
+        `positions` float64 [N, 3] and the outputs `energy` [S], `forces` [N, 3], `virial` [S, 6], `energies` [N] are
+        arrays ON the module's GPU (torch tensors, or anything with `__cuda_array_interface__` such as CuPy arrays),
+        read and written in place; `natoms`, `cells`, `pbc` are host arrays.  The neighbour lists are built on the
+        device; positions, forces and energies never visit the host."""
+        if gamma is not None or atomic_sigma is not None or gmm_cluster is not None:
+            raise ValueError("the model has no UQ head")
+        natoms = np.ascontiguousarray(natoms, dtype=np.int32)
+        cells = np.ascontiguousarray(cells, dtype=np.float64).reshape(-1, 3, 3)
+        pb = np.ascontiguousarray(np.asarray(pbc, dtype=bool).reshape(-1, 3), dtype=np.uint8)
+        S, N = natoms.shape[0], int(natoms.sum())
+        if cells.shape[0] != S or pb.shape[0] != S:
+            raise ValueError("natoms, cells and pbc differ in length")
+        p_types = _device_pointer(types, "types", (N,), "int32")
+        p_pos = _device_pointer(positions, "positions", (N, 3), "float64")
+        p_e = _device_pointer(energy, "energy", (S,), "float64")
+        p_f = _device_pointer(forces, "forces", (N, 3), "float64") if forces is not None else None
+        p_v = _device_pointer(virial, "virial", (S, 6), "float64") if virial is not None else None
+        p_ea = _device_pointer(energies, "energies", (N,), "float64") if energies is not None else None
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies is not None else 0)
+        check(_lib.lib().gr_compute_batch_device(self.engine._h, S, ptr(natoms), p_types, p_pos, ptr(cells), ptr(pb), flags, p_e, p_f,
+                                                 p_v, p_ea))
+        self.passes = 1 if N else 0
+
+
+_CAI_TYPES = {"int32": "<i4", "float64": "<f8"}
+
+
+def _device_pointer(a, name, shape, dtype):
+    """Address of a C-contiguous device array of the given shape and dtype on the module's GPU (torch tensor or
+    `__cuda_array_interface__`); ValueError otherwise, with the reference's messages (python/kk/kk_module.cpp:129-134)."""
+    where = f"{name} must be on the module's GPU ({PLATFORM}:{_dev()})"
+    if hasattr(a, "data_ptr") and hasattr(a, "is_contiguous"):    # torch
+        if a.device.type != "cuda" or (a.device.index or 0) != _dev():
+            raise ValueError(where)
+        if str(a.dtype).split(".")[-1] != dtype or tuple(a.shape) != tuple(shape) or not a.is_contiguous():
+            raise ValueError(f"{name}: expected a contiguous {dtype} array of shape {tuple(shape)}")
+        return C.c_void_p(a.data_ptr() if a.numel() else 0)
+    cai = getattr(a, "__cuda_array_interface__", None)
+    if cai is None:
+        raise ValueError(where)
+    if cai["typestr"] != _CAI_TYPES[dtype] or tuple(cai["shape"]) != tuple(shape) or cai.get("strides") is not None:
+        raise ValueError(f"{name}: expected a contiguous {dtype} array of shape {tuple(shape)}")
+    return C.c_void_p(cai["data"][0])
+

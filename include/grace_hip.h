@@ -165,6 +165,17 @@ int gr_system_list_get(gr_system *s, int64_t *perm, int64_t *offset, int32_t *j,
 int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
                      const unsigned char *pbc, unsigned flags, int nthreads, double *energy, double *forces, double *virial,
                      double *eatom);
+/* The same pass with the atoms and the results in device memory: replaces Batch::compute_device of the reference GPU
+ * module (python/kk/kk_api.h:107-120,141-146; binding python/kk/kk_module.cpp:142-193, which hands over DLPack arrays of
+ * the module's GPU).  types [N] (int32) and positions [N][3] are DEVICE pointers of the engine's GPU, as are the outputs
+ * energy [nstruct], forces [N][3], virial [nstruct][6], eatom [N] (NULL: not wanted); natoms, cells, pbc are host arrays
+ * as in gr_compute_batch.  A direction is periodic when its flag is set and its cell vector is not zero.  The neighbour
+ * lists are built on the device (the reference: kk/neighbors_kk.h BatchNeighborListKK); positions, forces and per-atom
+ * energies never visit the host (the atom types do, 4 bytes per atom, for the layout of the element tiles).  Results in
+ * the caller's atom order.  The call waits for work queued on the device before it reads the inputs and returns when
+ * the outputs are written.  A pointer that is not memory of the engine's GPU gives GR_INVALID. */
+int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
+                            const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom);
 int gr_engine_upload_batch(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
                            const double *positions, const int *image, const double *shifts, int64_t nimages, int nstruct,
                            const int *struct_of_atom);

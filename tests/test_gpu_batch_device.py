@@ -1,0 +1,120 @@
+"""`Batch.compute_device` (gr_compute_batch_device through the C ABI): atoms and results in device memory, neighbour
+lists built on the device.  Checked against `Batch.compute` (host lists, the reference's list order) on the same
+structures: periodic, triclinic with atoms outside the cell, slab, molecule, and the small cells of the batched
+workload.  The two paths sum the same bonds in different orders: 1e-9 relative.  Needs an MI355X: run with -m gpu."""
+import os
+
+import numpy as np
+import pytest
+
+import cases
+from grace_runtime_amd import kk
+
+pytestmark = pytest.mark.gpu
+
+
+def _engine(model_dir, name, species):
+    return kk.Engine(kk.Model(os.path.join(model_dir, name + ".npz")), species, 64)
+
+
+def _pack(structs):
+    natoms = np.array([len(s[0]) for s in structs], np.int32)
+    pos = np.concatenate([s[0] for s in structs])
+    cells = np.stack([s[1] for s in structs])
+    pbc = np.stack([np.asarray(s[2], bool) for s in structs])
+    types = np.concatenate([s[3] for s in structs]).astype(np.int32)
+    return natoms, types, pos, cells, pbc
+
+
+def _device_run(b, natoms, types, pos, cells, pbc, energy_only=False, energies=True):
+    import torch
+    dev = torch.device("cuda", kk.device() if kk.initialized() else 0)
+    S, N = len(natoms), len(types)
+    t = torch.as_tensor(types, device=dev)
+    x = torch.as_tensor(pos, device=dev)
+    e = torch.full((S,), 7.0, dtype=torch.float64, device=dev)
+    f = None if energy_only else torch.full((N, 3), 7.0, dtype=torch.float64, device=dev)
+    v = None if energy_only else torch.full((S, 6), 7.0, dtype=torch.float64, device=dev)
+    ea = torch.full((N,), 7.0, dtype=torch.float64, device=dev) if energies else None
+    b.compute_device(natoms, t, x, cells, pbc, e, forces=f, virial=v, energies=ea, energy_only=energy_only)
+    out = {"energy": e.cpu().numpy()}
+    if f is not None:
+        out["forces"], out["virial"] = f.cpu().numpy(), v.cpu().numpy()
+    if ea is not None:
+        out["energies"] = ea.cpu().numpy()
+    return out
+
+
+def _compare(out, ref):
+    fs = max(1.0, np.abs(ref["forces"]).max())
+    assert np.abs(out["energy"] - ref["energy"]).max() < 1e-9 * max(1.0, np.abs(ref["energy"]).max())
+    assert np.abs(out["forces"] - ref["forces"]).max() < 1e-9 * fs
+    assert np.abs(out["virial"] - ref["virial"]).max() < 1e-9 * max(1.0, np.abs(ref["virial"]).max())
+    assert np.abs(out["energies"] - ref["energies"]).max() < 1e-9 * fs
+
+
+@pytest.mark.parametrize("name", ["mix2", "l2mix", "l3mix"])
+def test_device_batch_equals_host_batch(model_dir, name):
+    eng = _engine(model_dir, name, ["Mo", "W"])
+    mol = cases.structure_molecule()
+    structs = [cases.structure_alloy54(), cases.structure_triclinic(), cases.structure_slab(),
+               (mol[0], np.zeros((3, 3)), mol[2], mol[3])]
+    natoms, types, pos, cells, pbc = _pack(structs)
+    b = kk.Batch(eng.model, ["Mo", "W"])
+    ref = b.compute(natoms, types, pos, cells, pbc, energies=True)
+    out = _device_run(b, natoms, types, pos, cells, pbc)
+    assert b.passes == 1
+    _compare(out, ref)
+    eo = _device_run(b, natoms, types, pos, cells, pbc, energy_only=True, energies=False)
+    assert np.abs(eo["energy"] - ref["energy"]).max() < 1e-9 * max(1.0, np.abs(ref["energy"]).max())
+    # a second call with fewer structures reuses the buffers
+    sub = _pack(structs[1:3])
+    out2 = _device_run(b, *sub)
+    ref2 = b.compute(*sub, energies=True)
+    _compare(out2, ref2)
+
+
+def test_small_cells_with_several_images_per_direction(model_dir):
+    """cells shorter than the cutoff: every atom sees several images of itself and of each neighbour"""
+    eng = _engine(model_dir, "config5", ["Al", "Ni", "Ti"])
+    structs = [(p, c, [True, True, True], t) for p, c, t in cases.structures_config5(24)]
+    rng = np.random.default_rng(11)
+    tiny = np.array([[2.9, 0.0, 0.0], [0.3, 3.1, 0.0], [-0.2, 0.4, 3.3]])
+    structs.append((rng.uniform(-1, 2, (2, 3)) @ tiny * 0.5 + np.array([[0, 0, 0], [1.4, 1.5, 1.6]]), tiny, [True, True, True],
+                    np.array([1, 3], np.int32)))
+    structs.append((np.array([[0.1, 0.2, 0.3]]), np.diag([3.0, 3.2, 2.8]), [True, True, True], np.array([2], np.int32)))
+    natoms, types, pos, cells, pbc = _pack(structs)
+    b = kk.Batch(eng.model, ["Al", "Ni", "Ti"])
+    ref = b.compute(natoms, types, pos, cells, pbc, energies=True)
+    out = _device_run(b, natoms, types, pos, cells, pbc)
+    _compare(out, ref)
+
+
+def test_argument_errors(model_dir):
+    import torch
+    eng = _engine(model_dir, "mix2", ["Mo", "W"])
+    b = kk.Batch(eng.model, ["Mo", "W"])
+    p, c, pb, t = cases.structure_alloy54()
+    dev = torch.device("cuda", 0)
+    x, ty = torch.as_tensor(p, device=dev), torch.as_tensor(t, device=dev)
+    e = torch.zeros(1, dtype=torch.float64, device=dev)
+    with pytest.raises(ValueError, match="must be on the module's GPU"):
+        b.compute_device([len(p)], ty, torch.as_tensor(p), c[None], pb[None], e)
+    with pytest.raises(ValueError, match="must be on the module's GPU"):
+        b.compute_device([len(p)], t, x, c[None], pb[None], e)
+    with pytest.raises(ValueError, match="positions: expected"):
+        b.compute_device([len(p)], ty, x.float(), c[None], pb[None], e)
+    with pytest.raises(ValueError, match="forces: expected"):
+        b.compute_device([len(p)], ty, x, c[None], pb[None], e, forces=torch.zeros(len(p) - 1, 3, dtype=torch.float64, device=dev))
+    with pytest.raises(ValueError, match="differ in length"):
+        b.compute_device([len(p)], ty, x, np.stack([c, c]), pb[None], e)
+    with pytest.raises(ValueError, match="no UQ head"):
+        b.compute_device([len(p)], ty, x, c[None], pb[None], e, gamma=torch.zeros(len(p), dtype=torch.float64, device=dev))
+    bad = ty.clone()
+    bad[3] = 3
+    with pytest.raises(ValueError, match="types must be 1"):
+        b.compute_device([len(p)], bad, x, c[None], pb[None], e)
+    # no atoms at all: nothing to do, energies of empty structures are 0
+    e2 = torch.full((2,), 5.0, dtype=torch.float64, device=dev)
+    b.compute_device([0, 0], ty[:0], x[:0], np.stack([c, c]), np.stack([pb, pb]), e2)
+    assert e2.tolist() == [0.0, 0.0]
