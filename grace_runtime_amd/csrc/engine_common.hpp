@@ -808,12 +808,16 @@ class EngineBase : public Engine {
   {
     for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
     const int kb = ba.C / 16;
-    const size_t lds = ((size_t) ba.nl * (ba.C / 4) * 64 + (size_t) 4 * 16 * ba.nlm * 4) * sizeof(T);
-    switch (kb) {
-      case 1: hipLaunchKernelGGL((k_bond_bwd<T, 1>), dim3(n), dim3(256), lds, stream_, ba); break;
-      case 2: hipLaunchKernelGGL((k_bond_bwd<T, 2>), dim3(n), dim3(256), lds, stream_, ba); break;
-      default: hipLaunchKernelGGL((k_bond_bwd<T, 4>), dim3(n), dim3(256), lds, stream_, ba); break;
+    const size_t lds = ((size_t) ba.nlm * (ba.C + 2) + (size_t) 4 * 16 * ba.nlm * 4) * sizeof(T);
+    if (kb != 1 && kb != 2 && kb != 4) throw Error("bond backward: channel width must be 16, 32 or 64");
+#define GR_BB(KB, NL) hipLaunchKernelGGL((k_bond_bwd<T, KB, NL>), dim3(n), dim3(256), lds, stream_, ba)
+#define GR_BB_NL(NL) case NL: if (kb == 1) GR_BB(1, NL); else if (kb == 2) GR_BB(2, NL); else GR_BB(4, NL); break
+    switch (ba.nl) {
+      GR_BB_NL(1); GR_BB_NL(2); GR_BB_NL(3); GR_BB_NL(4); GR_BB_NL(5); GR_BB_NL(6); GR_BB_NL(7);
+      default: throw Error("bond backward: lmax above " + std::to_string(kKernMaxL));
     }
+#undef GR_BB_NL
+#undef GR_BB
   }
   // out[tile atoms][job output] = GEMM jobs over X0 (kb0 16-channel blocks) and X1 (kb1), nb output blocks
   template<class T>

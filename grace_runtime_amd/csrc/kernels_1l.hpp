@@ -33,19 +33,20 @@ struct ShCoef {
 
 // Real spherical harmonics Y[lm] (stride ys) of the unit vector (rx, ry, rz) and, with GRAD, the gradient
 // G[lm][3] of their polynomial extension.  Same recursion as fused_cpu.h:712-798, one bond per thread, fp64.
-template<bool GRAD, class TY>
+// LMAX: compile-time bound of co.lmax (the register arrays of the recursion are sized by it).
+template<bool GRAD, class TY, int LMAX = kKernMaxL>
 __device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz, TY *Y, TY *G)
 {
-  double plm[kMaxPlm], dplm[kMaxPlm];
-  const int lmax = co.lmax;
+  double plm[(LMAX + 1) * (LMAX + 2) / 2], dplm[(LMAX + 1) * (LMAX + 2) / 2];
+  const int lmax = co.lmax < LMAX ? co.lmax : LMAX;
   plm[0] = 1.0;
   dplm[0] = 0.0;
-  if (lmax > 0) {
+  if (LMAX > 0 && lmax > 0) {
     const double s3 = 1.7320508075688772, s15 = -1.224744871391589;
-    plm[1] = s3 * rz; dplm[1] = s3;
-    plm[2] = s15;     dplm[2] = 0.0;
+    plm[LMAX > 0 ? 1 : 0] = s3 * rz; dplm[LMAX > 0 ? 1 : 0] = s3;
+    plm[LMAX > 0 ? 2 : 0] = s15;     dplm[LMAX > 0 ? 2 : 0] = 0.0;
 #pragma unroll
-    for (int l = 2; l <= kKernMaxL; l++) {
+    for (int l = 2; l <= LMAX; l++) {
       if (l <= lmax) {
 #pragma unroll
         for (int mm = 0; mm < l - 1; mm++) {
@@ -67,7 +68,7 @@ __device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz
   }
   const double sq2 = 1.4142135623730951;
 #pragma unroll
-  for (int l = 0; l <= kKernMaxL; l++) {
+  for (int l = 0; l <= LMAX; l++) {
     if (l <= lmax) {
       const int c = l * (l + 1), p0 = l * (l + 1) / 2;
       Y[c] = (TY) plm[p0];
@@ -606,7 +607,7 @@ template<class T, int NL, int KB> __global__ __launch_bounds__(256) void k_scatt
     if (lane < 16) {
       if (lane < nb) {
         const double *u = a.rh + 3 * (eb + lane);
-        sh_eval<false, T>(a.sh, u[0], u[1], u[2], Yw + lane * a.nlm, nullptr);
+        sh_eval<false, T, NL - 1>(a.sh, u[0], u[1], u[2], Yw + lane * a.nlm, nullptr);
       } else {
         for (int q = 0; q < a.nlm; q++) Yw[lane * a.nlm + q] = (T) 0;
       }
@@ -1067,114 +1068,106 @@ template<class T> struct BondBwdArgs {
 };
 
 // One block (4 waves) per atom; a wave takes tiles of 16 bonds.  Per tile and l two tile GEMMs on the matrix cores,
-//   P[b][m] = sum_n Rz[b][l][n] gA[l*l + m][n],   Q[b][m] = sum_n dRz[b][l][n] gA[l*l + m][n]      (K = channels)
-// with the gA^T fragments of the atom staged once in LDS, then per bond
-//   g_d = sum_lm G[b][lm][d] P[b][lm],  dE/dx = sum_lm Y[b][lm] Q[b][lm],
+//   P[m][b] = sum_n gA[l*l + m][n] Rz[b][l][n],   Q[m][b] = sum_n gA[l*l + m][n] dRz[b][l][n]      (K = channels)
+// with the bonds as columns: lane (g, c) of the wave ends up with the rows m = drow[4 g + v] of bond c, so the sums over
+// m are four terms in the lane and two exchanges between the lane groups, and lane c < 16 -- the lane that evaluated
+// the harmonics of bond c and holds its geometry in registers -- finishes the bond:
+//   g_d = sum_lm G[b][lm][d] P[lm][b],  dE/dx = sum_lm Y[b][lm] Q[lm][b],
 //   fv = dE/dx / rc rhat + (g - (g . rhat) rhat) / r;  f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv
-// (fused_cpu.h:836-860,1027-1050; fused_1l.cpp:46-51 of the reference).  KB = channels / 16.
-template<class T, int KB> __global__ __launch_bounds__(256) void k_bond_bwd(BondBwdArgs<T> a)
+// (fused_cpu.h:836-860,1027-1050; fused_1l.cpp:46-51 of the reference).  gA of the atom sits in LDS as [lm][C + 2]
+// (the pad spreads the rows over the banks); the radial rows of l + 1 are requested before the products of l.
+// KB = channels / 16, NL = lmax + 1.  dynamic LDS: nlm (C + 2) + 4 waves x 16 bonds x 4 nlm values.
+template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_bwd(BondBwdArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
-  constexpr int KS = KB * 4;
+  constexpr int KS = KB * 4, C = KB * 16, CS = C + 2, NLM = NL * NL;
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  T *gAf = reinterpret_cast<T *>(smem_raw);                          // [nl][KS][64] B-operand fragments of gA^T
-  T *Ysh = gAf + a.nl * KS * 64;                                     // [4 waves][16][nlm]
-  T *Gsh = Ysh + 4 * 16 * a.nlm;                                     // [4 waves][16][3 nlm]
+  T *gAl = reinterpret_cast<T *>(smem_raw);                          // [NLM][CS]
+  T *Ysh = gAl + NLM * CS;                                           // [4 waves][16][NLM]
+  T *Gsh = Ysh + 4 * 16 * NLM;                                       // [4 waves][16][NLM][3]
   __shared__ double red[4][9];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int i = a.a0 + blockIdx.x;
   const long long e0 = a.eoff[i], e1 = a.eoff[i + 1];
-  const int C = a.C;
   {
-    // fragment (l, s, lane (g, c)) = gA[l*l + c][g KS + s] for c < 2l + 1, else 0
-    const T *gAi = a.gA + (long long) blockIdx.x * a.nlm * C;
-    for (int q = t; q < a.nl * KS * 64; q += 256) {
-      const int l = q / (KS * 64), s = (q / 64) % KS, ln = q & 63, gg = ln >> 4, cc = ln & 15;
-      gAf[q] = cc < 2 * l + 1 ? gAi[(l * l + cc) * C + gg * KS + s] : (T) 0;
-    }
+    const T *gAi = a.gA + (long long) blockIdx.x * NLM * C;
+    for (int q = t; q < NLM * C; q += 256) gAl[(q / C) * CS + q % C] = gAi[q];
   }
   __syncthreads();
-  T *Yw = Ysh + wave * 16 * a.nlm, *Gw = Gsh + wave * 16 * 3 * a.nlm;
+  T *Yw = Ysh + wave * 16 * NLM, *Gw = Gsh + wave * 16 * 3 * NLM;
+  int mrow[4];
+#pragma unroll
+  for (int v = 0; v < 4; v++) mrow[v] = a.drow[4 * g + v];
   double fi[3] = {0, 0, 0}, vir[6] = {0, 0, 0, 0, 0, 0};
   const int ntile = (int) ((e1 - e0 + 15) / 16);
   for (int tile = wave; tile < ntile; tile += 4) {
     const long long eb = e0 + (long long) tile * 16;
     const int nb = (int) (e1 - eb < 16 ? e1 - eb : 16);
+    const bool colok = c < nb;                      // B operand column = bond c of the tile
+    const T *rp = a.Rz + (eb + (colok ? c : 0)) * a.noutp + g * KS;
+    const T *dp = a.dRz + (eb + (colok ? c : 0)) * a.noutp + g * KS;
+    T x[2][KS], dx[2][KS];
+#pragma unroll
+    for (int s = 0; s < KS; s++) { x[0][s] = rp[s]; dx[0][s] = dp[s]; }
+    // geometry of bond `lane` (lanes below nb), kept for the end of the tile
+    double u0 = 0, u1 = 0, u2 = 1, br = 1, brc = 1;
+    int jj = 0;
     if (lane < nb) {
-      const double *u = a.rh + 3 * (eb + lane);
-      sh_eval<true, T>(a.sh, u[0], u[1], u[2], Yw + lane * a.nlm, Gw + lane * 3 * a.nlm);
+      const long long e = eb + lane;
+      u0 = a.rh[3 * e]; u1 = a.rh[3 * e + 1]; u2 = a.rh[3 * e + 2];
+      br = a.r[e]; brc = a.rc[e]; jj = a.ej[e];
+      sh_eval<true, T, NL - 1>(a.sh, u0, u1, u2, Yw + lane * NLM, Gw + lane * 3 * NLM);
     }
     // LDS writes of this wave visible to its other lanes (the Y / G region is private to the wave)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    double p0[4] = {0, 0, 0, 0}, p1[4] = {0, 0, 0, 0}, p2[4] = {0, 0, 0, 0}, px[4] = {0, 0, 0, 0};
-    const bool rowok = c < nb;                      // A operand row = bond c of the tile
-    for (int l = 0; l < a.nl; l++) {
-      T x[KS], dx[KS];
-      if (rowok) {
-        const T *rp = a.Rz + (eb + c) * a.noutp + l * C + g * KS;
-        const T *dp = a.dRz + (eb + c) * a.noutp + l * C + g * KS;
+    double px = 0, p0 = 0, p1 = 0, p2 = 0;
 #pragma unroll
-        for (int s = 0; s < KS; s++) { x[s] = rp[s]; dx[s] = dp[s]; }
-      } else {
+    for (int l = 0; l < NL; l++) {
+      const int cur = l & 1, nxt = cur ^ 1;
+      if (l + 1 < NL) {
 #pragma unroll
-        for (int s = 0; s < KS; s++) { x[s] = (T) 0; dx[s] = (T) 0; }
+        for (int s = 0; s < KS; s++) { x[nxt][s] = rp[(l + 1) * C + s]; dx[nxt][s] = dp[(l + 1) * C + s]; }
       }
       v4 aP = {0, 0, 0, 0}, aQ = {0, 0, 0, 0};
-      const T *bf = gAf + l * KS * 64 + lane;
+      // A operand: row m = c of gA_l^T, k = g KS + s
+      const T *ga = gAl + (l * l + (c < 2 * l + 1 ? c : 0)) * CS + g * KS;
 #pragma unroll
       for (int s = 0; s < KS; s++) {
-        const T b = bf[s * 64];
-        aP = Mfma<T>::mma(x[s], b, aP);
-        aQ = Mfma<T>::mma(dx[s], b, aQ);
+        const T w = c < 2 * l + 1 ? ga[s] : (T) 0;
+        aP = Mfma<T>::mma(w, x[cur][s], aP);
+        aQ = Mfma<T>::mma(w, dx[cur][s], aQ);
       }
-      if (c < 2 * l + 1) {
-        const int lm = l * l + c;
+      if (colok) {
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-          const int row = a.drow[4 * g + v];
-          if (row < nb) {
-            const T *G = Gw + (row * a.nlm + lm) * 3;
-            px[v] += (double) (Yw[row * a.nlm + lm] * aQ[v]);
-            p0[v] += (double) (G[0] * aP[v]);
-            p1[v] += (double) (G[1] * aP[v]);
-            p2[v] += (double) (G[2] * aP[v]);
+          if (mrow[v] < 2 * l + 1) {
+            const int lm = l * l + mrow[v];
+            const T *G = Gw + (c * NLM + lm) * 3;
+            px += (double) (Yw[c * NLM + lm] * aQ[v]);
+            p0 += (double) (G[0] * aP[v]);
+            p1 += (double) (G[1] * aP[v]);
+            p2 += (double) (G[2] * aP[v]);
           }
         }
       }
     }
-    // sum over the 16 lanes of a group (the m index)
-#pragma unroll
-    for (int v = 0; v < 4; v++)
-#pragma unroll
-      for (int o = 8; o > 0; o >>= 1) {
-        p0[v] += __shfl_xor(p0[v], o, 64); p1[v] += __shfl_xor(p1[v], o, 64);
-        p2[v] += __shfl_xor(p2[v], o, 64); px[v] += __shfl_xor(px[v], o, 64);
+    // sum over the four lane groups (the rows m of a bond are spread over them)
+    px += __shfl_xor(px, 16, 64); p0 += __shfl_xor(p0, 16, 64); p1 += __shfl_xor(p1, 16, 64); p2 += __shfl_xor(p2, 16, 64);
+    px += __shfl_xor(px, 32, 64); p0 += __shfl_xor(p0, 32, 64); p1 += __shfl_xor(p1, 32, 64); p2 += __shfl_xor(p2, 32, 64);
+    if (lane < nb) {
+      const double dEdr = px / brc;
+      const double gr = p0 * u0 + p1 * u1 + p2 * u2;
+      const double fv[3] = {dEdr * u0 + (p0 - gr * u0) / br, dEdr * u1 + (p1 - gr * u1) / br, dEdr * u2 + (p2 - gr * u2) / br};
+      for (int d = 0; d < 3; d++) {
+        fi[d] += fv[d];
+        atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
       }
-    // lane c = v of each group finishes bond drow[4 g + v]
-#pragma unroll
-    for (int v = 0; v < 4; v++) {
-      const int row = a.drow[4 * g + v];
-      if (c == v && row < nb) {
-        const long long e = eb + row;
-        const double *u = a.rh + 3 * e;
-        const double r = a.r[e], rc = a.rc[e];
-        const double gv[3] = {p0[v], p1[v], p2[v]};
-        const double dEdr = px[v] / rc;
-        const double gr = gv[0] * u[0] + gv[1] * u[1] + gv[2] * u[2];
-        double fv[3];
-        for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + (gv[d] - gr * u[d]) / r;
-        const int jj = a.ej[e];
-        for (int d = 0; d < 3; d++) {
-          fi[d] += fv[d];
-          atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
-        }
-        const double ddx = -u[0] * r, ddy = -u[1] * r, ddz = -u[2] * r;
-        vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
-        vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
-      }
+      const double ddx = -u0 * br, ddy = -u1 * br, ddz = -u2 * br;
+      vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
+      vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
