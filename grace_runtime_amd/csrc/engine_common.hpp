@@ -252,7 +252,7 @@ template<class T> struct DevRadial {
     const int nout = CP * nl;
     noutp = round_up(nout, 16);
     nob = noutp / 16;
-    std::vector<T> v0((size_t) hb * ks0 * 64, (T) 0), v1((size_t) hb * hb * 4 * 64, (T) 0), v2((size_t) nob * hb * 4 * 64, (T) 0);
+    std::vector<T> v0((size_t) hb * ks0 * 64, (T) 0), v1((size_t) hb * hb * 4 * 64, (T) 0), v2(((size_t) nob * hb * 4 + kRadialPrefetch) * 64, (T) 0);
     for (int rb = 0; rb < hb; rb++)
       for (int s = 0; s < ks0; s++)
         for (int lane = 0; lane < 64; lane++) {
@@ -334,8 +334,16 @@ template<class T> struct DevRadial {
     ra.emi = emi; ra.bias_i = bias_i.as<T>(); ra.bias_j = bias_j.as<T>(); ra.bias1 = bias1.as<T>();
     if (mode == 1 && !emi) throw Error("radial kernel: the species form needs the central element of every edge");
     const int threads = hb == 4 ? 512 : 256;
-    auto kern = mode == 1 ? (hb == 4 ? k_radial<T, 4, 0, 1> : k_radial<T, 8, 0, 1>)
-                          : hb == 4 ? (act == 1 ? k_radial<T, 4, 1> : k_radial<T, 4, 0>) : (act == 1 ? k_radial<T, 8, 1> : k_radial<T, 8, 0>);
+    // <T, 16-row blocks of the hidden width, activation, species form, layer-2 weights in LDS>
+    void (*kern)(RadialArgs<T>);
+    if (w2_in_lds)
+      kern = mode == 1 ? (hb == 4 ? k_radial<T, 4, 0, 1, true> : k_radial<T, 8, 0, 1, true>)
+                       : hb == 4 ? (act == 1 ? k_radial<T, 4, 1, 0, true> : k_radial<T, 4, 0, 0, true>)
+                                 : (act == 1 ? k_radial<T, 8, 1, 0, true> : k_radial<T, 8, 0, 0, true>);
+    else
+      kern = mode == 1 ? (hb == 4 ? k_radial<T, 4, 0, 1, false> : k_radial<T, 8, 0, 1, false>)
+                       : hb == 4 ? (act == 1 ? k_radial<T, 4, 1, 0, false> : k_radial<T, 4, 0, 0, false>)
+                                 : (act == 1 ? k_radial<T, 8, 1, 0, false> : k_radial<T, 8, 0, 0, false>);
     HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     hipLaunchKernelGGL(kern, dim3(ncu), dim3(threads), lds, stream, ra);
   }

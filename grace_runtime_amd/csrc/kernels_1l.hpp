@@ -23,7 +23,8 @@ constexpr int kKernMaxL = 6;                                // largest lmax of t
 constexpr int kMaxNlm = (kKernMaxL + 1) * (kKernMaxL + 1);
 constexpr int kMaxPlm = (kKernMaxL + 1) * (kKernMaxL + 2) / 2;
 constexpr int kBondChunk = 32;                          // bonds staged per pass of the per-atom kernels
-constexpr int kMaxRadBasis = 16;                        // radial basis functions (padded to a multiple of 4)
+constexpr int kMaxRadBasis = 16;
+constexpr int kRadialPrefetch = 16;                     // weight fragments the radial kernel reads ahead: padding of the layer-2 weights                        // radial basis functions (padded to a multiple of 4)
 
 // spherical-harmonics recursion coefficients (fused_cpu.h:686-704), by index l (l + 1) / 2 + m
 struct ShCoef {
@@ -326,7 +327,7 @@ __device__ inline double ipow(double x, int n)
 // Every k-step feeds all row blocks of the value and the tangent stream (2 HB independent accumulator chains).
 // ACT: 0 SiLU, 1 tanh (compile-time: the fp64 tanh is large, and both activations inlined 32 times overflow the
 // instruction cache).
-template<class T, int HB, int ACT, int MODE = 0> __global__ __launch_bounds__(HB <= 4 ? 512 : 256) void k_radial(RadialArgs<T> a)
+template<class T, int HB, int ACT, int MODE, bool W2L> __global__ __launch_bounds__(HB <= 4 ? 512 : 256) void k_radial(RadialArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -334,23 +335,45 @@ template<class T, int HB, int ACT, int MODE = 0> __global__ __launch_bounds__(HB
   T *w1s = w0s + HB * a.ks0 * 64;
   T *w2s = w1s + HB * HB * 4 * 64;
   {
-    const int n0 = HB * a.ks0 * 64, n1 = HB * HB * 4 * 64, n2 = a.w2_in_lds ? a.nob * HB * 4 * 64 : 0;
+    const int n0 = HB * a.ks0 * 64, n1 = HB * HB * 4 * 64, n2 = W2L ? (a.nob * HB * 4 + kRadialPrefetch) * 64 : 0;
     for (int q = threadIdx.x; q < n0; q += blockDim.x) w0s[q] = a.w0[q];
     for (int q = threadIdx.x; q < n1; q += blockDim.x) w1s[q] = a.w1[q];
     for (int q = threadIdx.x; q < n2; q += blockDim.x) w2s[q] = a.w2[q];
   }
   __syncthreads();
-  const T *w2p = a.w2_in_lds ? w2s : a.w2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const long long cnt = a.e_count >= 0 ? a.e_count : *a.n_edges - a.e_begin;
   const long long ntiles = (cnt + 15) / 16;
   const int p = a.p;
   const double cf0 = 0.5 * (p + 1) * (p + 2), cf1 = (double) p * (p + 2), cf2 = 0.5 * p * (p + 1), cfd = 0.5 * p * (p + 1) * (p + 2);
-  for (long long tile = (long long) blockIdx.x * nw + wave; tile < ntiles; tile += (long long) gridDim.x * nw) {
+  // The memory counter of a wave retires loads and stores in order: a load issued behind a store waits for that store
+  // to complete.  The per-edge inputs of the NEXT tile (x of this lane's column, element and x of this lane's four
+  // output rows) are therefore requested before the first store of the current tile.
+  const int KZ = a.C >> 4;                        // distinct columns n = (16 cb + c) mod C of a lane: c + 16 k, k < KZ <= 4
+  const long long tstep = (long long) gridDim.x * nw;
+  long long tile = (long long) blockIdx.x * nw + wave;
+  double x_n = 0.5, xv_n[4] = {0.5, 0.5, 0.5, 0.5};
+  int emu_n[4] = {0, 0, 0, 0};
+  auto fetch_edge_inputs = [&](long long tl) {
+    const long long el = tl * 16 + c;
+    x_n = (tl < ntiles && el < cnt) ? a.x[a.e_begin + el] : 0.5;
+#pragma unroll
+    for (int v = 0; v < 4; v++) {
+      const long long er = tl * 16 + a.drow[g * 4 + v];
+      const bool ok = tl < ntiles && er < cnt;
+      emu_n[v] = ok ? a.emu[a.e_begin + er] : 0;
+      if (MODE == 1) xv_n[v] = ok ? a.x[a.e_begin + er] : 0.5;
+    }
+  };
+  fetch_edge_inputs(tile);
+  for (; tile < ntiles; tile += tstep) {
     const long long eloc = tile * 16 + c;
     const long long e = a.e_begin + eloc;
-    const double x = eloc < cnt ? a.x[e] : 0.5;
+    const double x = x_n;
+    double xv[4];
+#pragma unroll
+    for (int v = 0; v < 4; v++) xv[v] = xv_n[v];
     // basis g_k = T_k(2x - 1) fcut_p(x), k = 1..nrb, and d/dx (radial_x.h:11-26); this lane supplies k = 4 s + g
     T h0[kMaxRadBasis / 4], dh0[kMaxRadBasis / 4];
     {
@@ -403,21 +426,29 @@ template<class T, int HB, int ACT, int MODE = 0> __global__ __launch_bounds__(HB
         h1[rb][v] = s_; dh1[rb][v] = d_;
       }
     // ---- layer 1
+    // An fp64 MFMA holds its wave for the 64 cycles it runs, and nothing else of the wave issues meanwhile: what hides
+    // the latency of a weight fragment is to request it a few steps (2 MFMAs each) before its use.  The scheduling
+    // barriers keep the compiler from moving the request back next to the use.
     v4 h2[HB], dh2[HB];
 #pragma unroll
     for (int rb = 0; rb < HB; rb++) { h2[rb] = v4{0, 0, 0, 0}; dh2[rb] = v4{0, 0, 0, 0}; }
+    {
+      constexpr int NS = HB * 4 * HB;
+      // step q = (kb, s, rb): fragment ((rb HB + kb) 4 + s) of w1
+      auto frag = [&](int q) { return w1s[(((q % HB) * HB + q / (4 * HB)) * 4 + (q / HB) % 4) * 64 + lane]; };
+      T wa_ = frag(0), wb_ = frag(1);
 #pragma unroll
-    for (int kb = 0; kb < HB; kb++)
-#pragma unroll
-      for (int s = 0; s < 4; s++) {
-        const T b = h1[kb][s], db = dh1[kb][s];
-#pragma unroll
-        for (int rb = 0; rb < HB; rb++) {
-          const T w = w1s[((rb * HB + kb) * 4 + s) * 64 + lane];
-          h2[rb] = Mfma<T>::mma(w, b, h2[rb]);
-          dh2[rb] = Mfma<T>::mma(w, db, dh2[rb]);
-        }
+      for (int q = 0; q < NS; q++) {
+        const int kb = q / (4 * HB), s_ = (q / HB) % 4, rb = q % HB;
+        const T w = wa_;
+        wa_ = wb_;
+        if (q + 2 < NS) wb_ = frag(q + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        h2[rb] = Mfma<T>::mma(w, h1[kb][s_], h2[rb]);
+        dh2[rb] = Mfma<T>::mma(w, dh1[kb][s_], dh2[rb]);
+        __builtin_amdgcn_sched_barrier(0);
       }
+    }
     if (MODE == 1) {
 #pragma unroll
       for (int rb = 0; rb < HB; rb++)
@@ -432,61 +463,66 @@ template<class T, int HB, int ACT, int MODE = 0> __global__ __launch_bounds__(HB
         act_pair<T, ACT>(s_, d_);
         h2[rb][v] = s_; dh2[rb][v] = d_;
       }
-    // ---- layer 2 (linear), operands swapped: rows = edges, columns = outputs; two column blocks at a time
+    // ---- layer 2 (linear), operands swapped: rows = edges, columns = outputs; one block of 16 columns at a time (a
+    // single dependent accumulator chain keeps the matrix pipe full, and one block's weights are all that is in flight)
+    // The z values of a column block are requested one block ahead and the inputs of the next tile before the first
+    // store of this one: no load is issued behind a store whose completion it would then wait for.
+    const T *zrow[4];
     long long row_v[4];
-    const T *z_v[4];
-    T env_v[4], denv_v[4];
+    T env_v[4], denv_v[4], zc[4];
 #pragma unroll
     for (int v = 0; v < 4; v++) {
       const long long el = tile * 16 + a.drow[g * 4 + v];
       row_v[v] = el < cnt ? (a.e_begin + el) * a.noutp : -1;
-      z_v[v] = a.z + (el < cnt ? a.emu[a.e_begin + el] : 0) * a.C;
+      zrow[v] = a.z + emu_n[v] * a.C + c;
+      zc[v] = zrow[v][0];
       if (MODE == 1) {
-        const double xv = el < cnt ? a.x[a.e_begin + el] : 0.5;
-        const double xpm = ipow(xv, p - 1), xp = xpm * xv, xp1 = xp * xv, xp2 = xp1 * xv;
+        const double xpm = ipow(xv[v], p - 1), xp = xpm * xv[v], xp1 = xp * xv[v], xp2 = xp1 * xv[v];
         env_v[v] = (T) (1.0 - cf0 * xp + cf1 * xp1 - cf2 * xp2);
         denv_v[v] = (T) (cfd * (-xpm + 2.0 * xp - xp1));
       }
     }
-    for (int cb = 0; cb < a.nob; cb += 2) {
-      const bool two = cb + 1 < a.nob;
-      v4 acc0 = {0, 0, 0, 0}, dacc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0}, dacc1 = {0, 0, 0, 0};
-      const T *wa = w2p + (long long) cb * HB * 4 * 64 + lane;
-      const T *wb = two ? wa + HB * 4 * 64 : wa;
+    fetch_edge_inputs(tile + tstep);
+    // weight fragments of layer 2 run PF steps ahead of their use, across the column blocks (the fragments of
+    // consecutive steps are consecutive in memory): LDS when they fit, else global memory, hence the depth
+    constexpr int PF = W2L ? 2 : 16, NQ = HB * 4;
+    static_assert(PF <= kRadialPrefetch, "padding of the layer-2 weights");
+    // two separate pointers: one pointer that may be either would make every read a flat load, which waits for the
+    // stores of the block before it
+    const T *wl = (W2L ? (const T *) w2s : a.w2) + lane;
+    T wq[PF];
 #pragma unroll
-      for (int kb = 0; kb < HB; kb++)
+    for (int i = 0; i < PF; i++) wq[i] = wl[i * 64];
+    for (int cb = 0; cb < a.nob; cb++) {
+      T zn[4];
+      const int kn = ((cb + 1) & (KZ - 1)) * 16;       // column n = c + 16 k of z in the next block
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-          const T w0_ = wa[(kb * 4 + s) * 64], w1_ = wb[(kb * 4 + s) * 64];
-          acc0 = Mfma<T>::mma(h2[kb][s], w0_, acc0);
-          dacc0 = Mfma<T>::mma(dh2[kb][s], w0_, dacc0);
-          acc1 = Mfma<T>::mma(h2[kb][s], w1_, acc1);
-          dacc1 = Mfma<T>::mma(dh2[kb][s], w1_, dacc1);
-        }
-      const int col0 = cb * 16 + c, col1 = col0 + 16;
-      const int n0 = col0 % a.C, n1 = col1 % a.C;
+      for (int v = 0; v < 4; v++) zn[v] = zrow[v][kn];
+      v4 acc = {0, 0, 0, 0}, dacc = {0, 0, 0, 0};
+      const T *wc = wl + (long long) cb * NQ * 64;
 #pragma unroll
-      for (int v = 0; v < 4; v++)
+      for (int q = 0; q < NQ; q++) {
+        const T w_ = wq[q % PF];
+        wq[q % PF] = wc[(q + PF) * 64];               // beyond the last block: the zero padding of the weights
+        __builtin_amdgcn_sched_barrier(0);
+        acc = Mfma<T>::mma(h2[q / 4][q % 4], w_, acc);
+        dacc = Mfma<T>::mma(dh2[q / 4][q % 4], w_, dacc);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      const int col = cb * 16 + c;
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
         if (row_v[v] >= 0) {
-          const T zz0 = z_v[v][n0];
           if (MODE == 1) {
-            a.Rz[row_v[v] + col0] = acc0[v] * env_v[v] * zz0;
-            a.dRz[row_v[v] + col0] = (dacc0[v] * env_v[v] + acc0[v] * denv_v[v]) * zz0;
+            a.Rz[row_v[v] + col] = acc[v] * env_v[v] * zc[v];
+            a.dRz[row_v[v] + col] = (dacc[v] * env_v[v] + acc[v] * denv_v[v]) * zc[v];
           } else {
-            a.Rz[row_v[v] + col0] = acc0[v] * zz0;
-            a.dRz[row_v[v] + col0] = dacc0[v] * zz0;
-          }
-          if (two) {
-            const T zz1 = z_v[v][n1];
-            if (MODE == 1) {
-              a.Rz[row_v[v] + col1] = acc1[v] * env_v[v] * zz1;
-              a.dRz[row_v[v] + col1] = (dacc1[v] * env_v[v] + acc1[v] * denv_v[v]) * zz1;
-            } else {
-              a.Rz[row_v[v] + col1] = acc1[v] * zz1;
-              a.dRz[row_v[v] + col1] = dacc1[v] * zz1;
-            }
+            a.Rz[row_v[v] + col] = acc[v] * zc[v];
+            a.dRz[row_v[v] + col] = dacc[v] * zc[v];
           }
         }
+        zc[v] = zn[v];
+      }
     }
   }
 }
