@@ -36,6 +36,7 @@ template<class T> class Engine1L final : public EngineBase {
   DevBuf z_, shift_;
   DevRadial<T> rad_;
   DevFc<T> fcA1_, fcAA1_, fcAA2_;
+  DevFcPairBwd<T> fcAA12_;    // reverse of fc_AA1 and fc_AA2 in one pass over their shared inputs (models with the AAAA stage)
   DevProd pAA_, pAAA_, pAAAA_;
   DevReduce<T> redrho_;
   DevBuf eW_[7];
@@ -149,7 +150,10 @@ template<class T> void Engine1L<T>::build()
     }
     fcA1_.build(m.fc_A1, liveA1, nlm_, CP_, CP_, CFP_, drow_);
     fcAA1_.build(m.fc_AA1, liveAA1, nlm_, CFP_, CP_, CFP_, drow_);
-    if (order4_) fcAA2_.build(m.fc_AA2, liveAA2, nlm_, CFP_, CP_, CFP_, drow_);
+    if (order4_) {
+      fcAA2_.build(m.fc_AA2, liveAA2, nlm_, CFP_, CP_, CFP_, drow_);
+      fcAA12_.build(m.fc_AA1, liveAA1, fcAA1_, m.fc_AA2, liveAA2, fcAA2_, nlm_, drow_);
+    }
   }
 
   // ---- rho reduce: weights per collected function in MFMA fragment order (fused_cpu.h:1202-1273)
@@ -323,12 +327,17 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
       launch_gemm(F.bwd_r, kf, kf, ka, g, nfl, g, nfl, gXr, nlm_, 1);
     });
   };
-  if (order4_) {
-    prod_bwd("prod_AAAA_bwd", pAAAA_, AA2, AA2, gAAAA, gAA2, gAA2, nAA_, nAA_, 0, 0);
-    fc_bwd("fc_AA2_bwd", fcAA2_, gAA2, gAA, gA, nAA_, kf);
-  }
+  if (order4_) prod_bwd("prod_AAAA_bwd", pAAAA_, AA2, AA2, gAAAA, gAA2, gAA2, nAA_, nAA_, 0, 0);
   prod_bwd("prod_AAA_bwd", pAAA_, AA1, Ar, gAAA, gAA1, aaa_a_ ? gA : gA1, nAA_, nlm_, 0, 1);
-  fc_bwd("fc_AA1_bwd", fcAA1_, gAA1, gAA, gA, nAA_, kf);
+  if (order4_) {
+    // fc_AA1 and fc_AA2 share their inputs: one pass over gAA and gA for both
+    stage("fc_AA12_bwd", [&] {
+      launch_gemm(fcAA12_.bwd_l, kf, kf, kf, gAA1, nAA_, gAA2, nAA_, gAA, nAA_, 1);
+      launch_gemm(fcAA12_.bwd_r, kf, kf, ka, gAA1, nAA_, gAA2, nAA_, gA, nlm_, 1);
+    });
+  } else {
+    fc_bwd("fc_AA1_bwd", fcAA1_, gAA1, gAA, gA, nAA_, kf);
+  }
   prod_bwd("prod_AA_bwd", pAA_, A1, A1, gAA, gA1, gA1, nlm_, nlm_, 1, 1);
   fc_bwd("fc_A1_bwd", fcA1_, gA1, gA, gA, nlm_, ka);
 

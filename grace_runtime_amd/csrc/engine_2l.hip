@@ -17,6 +17,7 @@ template<class T> struct Chain {
   int nf = 0, nXX = 0, nXXX = 0, nXXXX = 0, kb = 0;    // functions of X, XX, XXX, XXXX; 16-channel blocks
   bool order4 = false, jit_all = false;
   DevFc<T> fc1, fc2, fc3;
+  DevFcPairBwd<T> fc23;    // reverse of fc2 and fc3 in one pass over their shared inputs (order 4)
   DevProd p2, p3, p4;
   DevBuf X1, XX, XX1, XXX, XX2, XXXX, gX, gX1, gXX, gXX1, gXXX, gXX2, gXXXX;
   const T *src(int s, const T *X) const
@@ -114,7 +115,10 @@ void Engine2L<T>::build_chain(Chain<T> &c, const char *tag, int nf, int KP, cons
   c.jit_all = c.p2.jit.ok() && c.p3.jit.ok() && (!order4_ || c.p4.jit.ok());
   c.fc1.build(*fc[0], live1, nf, KP, KP, KP, drow_);
   c.fc2.build(*fc[1], live2, nf, KP, KP, KP, drow_);
-  if (order4_) c.fc3.build(*fc[2], live3, nf, KP, KP, KP, drow_);
+  if (order4_) {
+    c.fc3.build(*fc[2], live3, nf, KP, KP, KP, drow_);
+    c.fc23.build(*fc[1], live2, c.fc2, *fc[2], live3, c.fc3, nf, drow_);
+  }
 }
 
 template<class T> void Engine2L<T>::build()
@@ -404,12 +408,17 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
   const T *X1 = c.X1.template as<T>(), *XX1 = c.XX1.template as<T>(), *XX2 = c.XX2.template as<T>();
   T *gX = c.gX.template as<T>(), *gX1 = c.gX1.template as<T>(), *gXX = c.gXX.template as<T>(), *gXX1 = c.gXX1.template as<T>(),
     *gXXX = c.gXXX.template as<T>(), *gXX2 = c.gXX2.template as<T>(), *gXXXX = c.gXXXX.template as<T>();
-  if (c.order4) {
-    prod_bwd(tagged(tag, "prod_4_bwd"), c.p4, XX2, XX2, gXXXX, gXX2, gXX2, c.nXX, c.nXX, 0, 0);
-    fc_bwd(tagged(tag, "fc_3_bwd"), c.fc3, gXX2, gXX, gX, c.nXX);
-  }
+  if (c.order4) prod_bwd(tagged(tag, "prod_4_bwd"), c.p4, XX2, XX2, gXXXX, gXX2, gXX2, c.nXX, c.nXX, 0, 0);
   prod_bwd(tagged(tag, "prod_3_bwd"), c.p3, XX1, X, gXXX, gXX1, gX, c.nXX, c.nf, 0, 1);
-  fc_bwd(tagged(tag, "fc_2_bwd"), c.fc2, gXX1, gXX, gX, c.nXX);
+  if (c.order4) {
+    // fc2 and fc3 share their inputs: one pass over gXX and gX for both
+    stage(tagged(tag, "fc_23_bwd").c_str(), [&] {
+      launch_gemm<T>(c.fc23.bwd_l, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gXX, c.nXX, 1, tiles_.as<int>(), ntiles_);
+      launch_gemm<T>(c.fc23.bwd_r, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gX, c.nf, 1, tiles_.as<int>(), ntiles_);
+    });
+  } else {
+    fc_bwd(tagged(tag, "fc_2_bwd"), c.fc2, gXX1, gXX, gX, c.nXX);
+  }
   prod_bwd(tagged(tag, "prod_2_bwd"), c.p2, X1, X1, gXX, gX1, gX1, c.nf, c.nf, 1, 1);
   fc_bwd(tagged(tag, "fc_1_bwd"), c.fc1, gX1, gX, gX, c.nf);
 }

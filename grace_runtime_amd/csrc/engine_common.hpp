@@ -224,6 +224,44 @@ template<class T> struct DevFc {
   }
 };
 
+// The reverse of two FC layers that read the same two inputs (AA1 = FC1(AA, A), AA2 = FC2(AA, A)) as ONE pair of job
+// lists: the adjoint of the shared left input is read, added to and written once instead of twice, and so is the
+// adjoint of the right input.  Source 0 of a segment is the output adjoint of the first layer, source 1 of the second.
+template<class T> struct DevFcPairBwd {
+  DevJobs<T> bwd_l, bwd_r;
+  void build(const FCWeights &w1, const std::vector<char> &live1, const DevFc<T> &F1, const FCWeights &w2, const std::vector<char> &live2,
+             const DevFc<T> &F2, int nfr, const int *drow)
+  {
+    if (w1.n_funcs != w2.n_funcs || F1.nil != F2.nil || F1.nir != F2.nir || F1.no != F2.no) throw Error("FC pair: the two layers differ in shape");
+    typename DevJobs<T>::Host hl, hr;
+    for (int f = 0; f < w1.n_funcs; f++) {
+      if (!live1[f] && !live2[f]) continue;
+      hl.job(f, 1.0);
+      if (live1[f]) hl.seg(0, f, w1.w_tile_left[f], w1.norm_out_factor[f]);
+      if (live2[f]) hl.seg(1, f, w2.w_tile_left[f], w2.norm_out_factor[f]);
+      hl.end_job();
+    }
+    std::vector<std::vector<std::pair<int, int>>> from(nfr);    // (layer, connection)
+    for (int c = 0; c < w1.n_conn; c++)
+      if (live1[w1.collect_to[c]]) from[w1.collect_from[c]].push_back({0, c});
+    for (int c = 0; c < w2.n_conn; c++)
+      if (live2[w2.collect_to[c]]) from[w2.collect_from[c]].push_back({1, c});
+    for (int r = 0; r < nfr; r++) {
+      if (from[r].empty()) continue;
+      hr.job(r, 1.0);
+      for (const auto &lc : from[r]) {
+        const FCWeights &w = lc.first ? w2 : w1;
+        const int c = lc.second;
+        hr.seg(lc.first, w.collect_to[c], w.w_tile_right[c], w.norm_out_factor[w.collect_to[c]]);
+      }
+      hr.end_job();
+    }
+    bwd_l.build(hl, F1.WlTF.template as<T>(), F2.WlTF.template as<T>());
+    bwd_r.build(hr, F1.WrTF.template as<T>(), F2.WrTF.template as<T>());
+    bwd_l.set_rows(drow); bwd_r.set_rows(drow);
+  }
+};
+
 
 // A 3-layer radial MLP in MFMA fragment order and the launch of the persistent radial kernel (radial_x.h:11-60 of the
 // reference; its spline tables are replaced by the exact network).  Output column l * CP + n of an edge holds
