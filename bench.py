@@ -36,7 +36,7 @@ HBM_PEAK = 8000.0                 # GB/s
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs of this
 # script, counters scaled by what they read for the 1 GiB copy kernel; summaries under profiles/): (workload, kernel)
 MEASURED_TRAFFIC = {
-    ("config2", "radial_mlp"): 366.7e6 + 1241.0e6,      # fetch + write of k_radial<double,4,0>
+    ("config2", "radial_mlp"): 7.0e6 + 1216.3e6,        # fetch + write of k_radial<double,4,0,0,true>
     ("config3", "pair_bwd"): 11883.6e6 + 2822.1e6,      # fetch + write of k_pair_bwd<double,25>
     ("config4", "pair_bwd_L3"): 64600e6 + 31459e6,      # the layer-3 launches of k_pair_bwd<double,36> (layer 2: 35.2 + 16.3 GB)
 }
