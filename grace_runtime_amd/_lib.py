@@ -89,7 +89,7 @@ def lib():
     L.gr_compute_batch.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, i32, vp, vp, vp, vp]
     L.gr_engine_upload_batch.argtypes = [vp, i32, vp, vp, vp, vp, vp, vp, vp, i64, i32, vp]
     L.gr_engine_fetch_batch.argtypes = [vp, i32, vp, vp, vp, vp]
-    L.gr_compute_batch_device.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, vp, vp, vp, vp]
+    L.gr_compute_batch_device.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, i64, vp, vp, vp, vp, vp]
     L.gr_compute_lammps.argtypes = [vp, i32, i32, vp, vp, i32, vp, vp, vp, i32, vp, u32, vp, vp, vp, vp]
     L.gr_system_create.argtypes = [vp, dbl, C.POINTER(vp)]
     L.gr_system_free.argtypes = [vp]

@@ -787,20 +787,25 @@ int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *ty
 }
 
 int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
-                            const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom)
+                            const unsigned char *pbc, unsigned flags, int64_t max_atoms, double *energy, double *forces, double *virial,
+                            double *eatom, int *passes)
 {
   return guarded([&] {
+    if (passes) *passes = 0;
     if (!e || nstruct < 0 || (nstruct > 0 && (!natoms || !cells || !pbc))) throw grhip::InvalidArgument("null argument");
+    if (max_atoms < 0) throw grhip::InvalidArgument("max_atoms must be >= 0");
     if (nstruct == 0) return;
     const double rc = e->eng->max_cutoff();
     if (!(rc > 0.0)) throw grhip::Error("the engine has no positive cutoff");
-    int64_t N = 0;
+    std::vector<int64_t> start((size_t) nstruct + 1, 0);
     for (int s = 0; s < nstruct; s++) {
       if (natoms[s] < 0) throw grhip::InvalidArgument("negative atom count");
-      N += natoms[s];
+      start[s + 1] = start[s] + natoms[s];
     }
+    const int64_t N = start[nstruct];
     if (N >= INT32_MAX) throw grhip::InvalidArgument("atom count out of range");
     if (N > 0 && (!types || !positions)) throw grhip::InvalidArgument("null argument");
+    if (!energy) throw grhip::InvalidArgument("the energy output is required");
     if (hipSetDevice(e->eng->device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
     // the pointers must be memory of the engine's GPU: a host pointer here would fault in the kernels
     auto on_device = [&](const void *p, const char *name) {
@@ -824,27 +829,37 @@ int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const 
     // work queued by the caller on the default stream (the tensors that hold the inputs) is finished first
     if (hipDeviceSynchronize() != hipSuccess) throw grhip::Error("hipDeviceSynchronize failed");
     grhip::BatchDeviceNeighbors &nl = *e->bnl;
-    nl.build(nstruct, natoms, positions, cells, pbc, rc, e->bnl_stream);
-    // atom types: 4 bytes per atom to the host, where the element tiles of the tile GEMMs are laid out
-    std::vector<int> ty((size_t) N);
-    if (N > 0 && hipMemcpyAsync(ty.data(), types, sizeof(int) * (size_t) N, hipMemcpyDeviceToHost, e->bnl_stream) != hipSuccess)
-      throw grhip::Error("copy of the atom types failed");
-    if (hipStreamSynchronize(e->bnl_stream) != hipSuccess) throw grhip::Error("the device neighbour search failed");
-    grhip::DeviceCsr in;
-    in.n = (int) N;
-    in.types = ty.data();
-    in.nb = nl.nb;
-    in.offset = nl.offset.as<int64_t>();
-    in.j = nl.j.as<int>();
-    in.rij = nl.rij.as<double>();
-    in.nstruct = nstruct;
-    in.sid = nl.sid.data();
-    e->eng->upload_device(in);
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
-    e->eng->run(fl);
-    e->eng->fetch_batch_device(nstruct, energy, forces, virial, fl.eatom ? eatom : nullptr);
+    // passes of whole structures with at most max_atoms atoms (at least one structure each)
+    for (int g0 = 0; g0 < nstruct;) {
+      int g1 = g0 + 1;
+      while (g1 < nstruct && (max_atoms == 0 || start[g1 + 1] - start[g0] <= max_atoms)) g1++;
+      const int ns = g1 - g0;
+      const int64_t a0 = start[g0], na = start[g1] - a0;
+      nl.build(ns, natoms + g0, positions + 3 * a0, cells + 9 * (size_t) g0, pbc + 3 * (size_t) g0, rc, e->bnl_stream);
+      // atom types: 4 bytes per atom to the host, where the element tiles of the tile GEMMs are laid out
+      std::vector<int> ty((size_t) na);
+      if (na > 0 && hipMemcpyAsync(ty.data(), types + a0, sizeof(int) * (size_t) na, hipMemcpyDeviceToHost, e->bnl_stream) != hipSuccess)
+        throw grhip::Error("copy of the atom types failed");
+      if (hipStreamSynchronize(e->bnl_stream) != hipSuccess) throw grhip::Error("the device neighbour search failed");
+      grhip::DeviceCsr in;
+      in.n = (int) na;
+      in.types = ty.data();
+      in.nb = nl.nb;
+      in.offset = nl.offset.as<int64_t>();
+      in.j = nl.j.as<int>();
+      in.rij = nl.rij.as<double>();
+      in.nstruct = ns;
+      in.sid = nl.sid.data();
+      e->eng->upload_device(in);
+      e->eng->run(fl);
+      e->eng->fetch_batch_device(ns, energy + g0, forces ? forces + 3 * a0 : nullptr, virial ? virial + 6 * (size_t) g0 : nullptr,
+                                 fl.eatom ? eatom + a0 : nullptr);
+      if (passes) ++*passes;
+      g0 = g1;
+    }
   });
 }
 }

@@ -433,6 +433,8 @@ class Batch:
             raise ValueError("natoms, types, positions, cells and pbc do not describe the same structures")
         if types.size and (types.min() < 1 or types.max() > len(self.engine.species)):
             raise ValueError("types must be 1 .. len(species)")
+        if int(max_nall) < 1:
+            raise ValueError("max_nall must be >= 1")
         N = types.shape[0]
         out = {"energy": np.zeros(S)}
         f, v = np.zeros((N, 3)), np.zeros((S, 6))
@@ -440,10 +442,20 @@ class Batch:
         pb = np.ascontiguousarray(pbc, dtype=np.uint8)
         flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
         nth = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else 1
-        # every structure's list is built on the host (in parallel), all structures go through the GPU in ONE pass
-        check(_lib.lib().gr_compute_batch(self.engine._h, S, ptr(natoms), ptr(types), ptr(pos), ptr(cells), ptr(pb), flags, min(nth, 16),
-                                          ptr(out["energy"]), ptr(f), ptr(v), ptr(ea) if energies else None))
-        self.passes = 1 if N else 0
+        # every structure's list is built on the host (in parallel); the structures go through the GPU in passes of whole
+        # structures with at most max_nall atoms (python/kk/kk_core.cpp:1311-1347: ONE pass unless the batch is larger)
+        start = np.concatenate([[0], np.cumsum(natoms, dtype=np.int64)])
+        self.passes, g0 = 0, 0
+        while g0 < S:
+            g1 = g0 + 1
+            while g1 < S and start[g1 + 1] - start[g0] <= int(max_nall):
+                g1 += 1
+            a0, a1 = int(start[g0]), int(start[g1])
+            check(_lib.lib().gr_compute_batch(self.engine._h, g1 - g0, ptr(natoms[g0:g1]), ptr(types[a0:a1]), ptr(pos[a0:a1]), ptr(cells[g0:g1]),
+                                              ptr(pb[g0:g1]), flags, min(nth, 16), ptr(out["energy"][g0:g1]), ptr(f[a0:a1]), ptr(v[g0:g1]),
+                                              ptr(ea[a0:a1]) if energies else None))
+            self.passes += 1 if a1 > a0 else 0
+            g0 = g1
         if not energy_only:
             out["forces"], out["virial"] = f, v
         if energies:
@@ -456,7 +468,8 @@ class Batch:
         `positions` float64 [N, 3] and the outputs `energy` [S], `forces` [N, 3], `virial` [S, 6], `energies` [N] are
         arrays ON the module's GPU (torch tensors, or anything with `__cuda_array_interface__` such as CuPy arrays),
         read and written in place; `natoms`, `cells`, `pbc` are host arrays.  The neighbour lists are built on the
-        device; positions, forces and energies never visit the host."""
+        device; positions, forces and energies never visit the host.  `max_nall`: atoms per engine pass (whole
+        structures, at least one per pass); `passes` holds the number of passes made."""
         if gamma is not None or atomic_sigma is not None or gmm_cluster is not None:
             raise ValueError("the model has no UQ head")
         natoms = np.ascontiguousarray(natoms, dtype=np.int32)
@@ -472,9 +485,12 @@ class Batch:
         p_v = _device_pointer(virial, "virial", (S, 6), "float64") if virial is not None else None
         p_ea = _device_pointer(energies, "energies", (N,), "float64") if energies is not None else None
         flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies is not None else 0)
-        check(_lib.lib().gr_compute_batch_device(self.engine._h, S, ptr(natoms), p_types, p_pos, ptr(cells), ptr(pb), flags, p_e, p_f,
-                                                 p_v, p_ea))
-        self.passes = 1 if N else 0
+        if int(max_nall) < 1:
+            raise ValueError("max_nall must be >= 1")
+        passes = C.c_int(0)
+        check(_lib.lib().gr_compute_batch_device(self.engine._h, S, ptr(natoms), p_types, p_pos, ptr(cells), ptr(pb), flags, int(max_nall),
+                                                 p_e, p_f, p_v, p_ea, C.byref(passes)))
+        self.passes = passes.value if N else 0
 
 
 _CAI_TYPES = {"int32": "<i4", "float64": "<f8"}
@@ -491,6 +507,12 @@ def _device_pointer(a, name, shape, dtype):
             raise ValueError(f"{name}: expected a contiguous {dtype} array of shape {tuple(shape)}")
         return C.c_void_p(a.data_ptr() if a.numel() else 0)
     cai = getattr(a, "__cuda_array_interface__", None)
+    if cai is None and hasattr(a, "__dlpack__"):    # any other DLPack exporter: through torch, without a copy
+        try:
+            import torch
+            return _device_pointer(torch.from_dlpack(a), name, shape, dtype)
+        except ImportError:
+            pass
     if cai is None:
         raise ValueError(where)
     if cai["typestr"] != _CAI_TYPES[dtype] or tuple(cai["shape"]) != tuple(shape) or cai.get("strides") is not None:

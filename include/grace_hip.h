@@ -173,9 +173,14 @@ int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *ty
  * lists are built on the device (the reference: kk/neighbors_kk.h BatchNeighborListKK); positions, forces and per-atom
  * energies never visit the host (the atom types do, 4 bytes per atom, for the layout of the element tiles).  Results in
  * the caller's atom order.  The call waits for work queued on the device before it reads the inputs and returns when
- * the outputs are written.  A pointer that is not memory of the engine's GPU gives GR_INVALID. */
+ * the outputs are written.  A pointer that is not memory of the engine's GPU gives GR_INVALID.
+ * max_atoms: the structures go through the engine in passes of whole structures with at most max_atoms atoms (at least
+ * one structure per pass), which bounds the engine's device memory as max_nall does in the reference
+ * (python/kk/kk_core.cpp:1311-1347; this list holds no ghost images, so atoms stand for the reference's atoms + images);
+ * 0: one pass.  *passes (may be NULL): engine passes made. */
 int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
-                            const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom);
+                            const unsigned char *pbc, unsigned flags, int64_t max_atoms, double *energy, double *forces, double *virial,
+                            double *eatom, int *passes);
 int gr_engine_upload_batch(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
                            const double *positions, const int *image, const double *shifts, int64_t nimages, int nstruct,
                            const int *struct_of_atom);

@@ -26,7 +26,7 @@ def _pack(structs):
     return natoms, types, pos, cells, pbc
 
 
-def _device_run(b, natoms, types, pos, cells, pbc, energy_only=False, energies=True):
+def _device_run(b, natoms, types, pos, cells, pbc, energy_only=False, energies=True, **kw):
     import torch
     dev = torch.device("cuda", kk.device() if kk.initialized() else 0)
     S, N = len(natoms), len(types)
@@ -36,7 +36,7 @@ def _device_run(b, natoms, types, pos, cells, pbc, energy_only=False, energies=T
     f = None if energy_only else torch.full((N, 3), 7.0, dtype=torch.float64, device=dev)
     v = None if energy_only else torch.full((S, 6), 7.0, dtype=torch.float64, device=dev)
     ea = torch.full((N,), 7.0, dtype=torch.float64, device=dev) if energies else None
-    b.compute_device(natoms, t, x, cells, pbc, e, forces=f, virial=v, energies=ea, energy_only=energy_only)
+    b.compute_device(natoms, t, x, cells, pbc, e, forces=f, virial=v, energies=ea, energy_only=energy_only, **kw)
     out = {"energy": e.cpu().numpy()}
     if f is not None:
         out["forces"], out["virial"] = f.cpu().numpy(), v.cpu().numpy()
@@ -87,7 +87,24 @@ def test_small_cells_with_several_images_per_direction(model_dir):
     b = kk.Batch(eng.model, ["Al", "Ni", "Ti"])
     ref = b.compute(natoms, types, pos, cells, pbc, energies=True)
     out = _device_run(b, natoms, types, pos, cells, pbc)
+    assert b.passes == 1
     _compare(out, ref)
+    # the same batch in passes of at most 300 atoms (whole structures; a structure above the limit is a pass of its own)
+    out = _device_run(b, natoms, types, pos, cells, pbc, max_nall=300)
+    start = np.concatenate([[0], np.cumsum(natoms)])
+    want, g0 = 0, 0
+    while g0 < len(natoms):
+        g1 = g0 + 1
+        while g1 < len(natoms) and start[g1 + 1] - start[g0] <= 300:
+            g1 += 1
+        want, g0 = want + 1, g1
+    assert b.passes == want and want > 3
+    _compare(out, ref)
+    host = b.compute(natoms, types, pos, cells, pbc, energies=True, max_nall=300)
+    assert b.passes == want
+    _compare(host, ref)
+    with pytest.raises(ValueError, match="max_nall"):
+        b.compute(natoms, types, pos, cells, pbc, max_nall=0)
 
 
 def test_argument_errors(model_dir):
