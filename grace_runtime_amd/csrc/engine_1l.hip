@@ -271,7 +271,12 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
 #undef GR_RED
   });
   stage("energy_mlp", [&] {
-    hipLaunchKernelGGL(k_energy, dim3(n), dim3(64), (size_t) ((2 * en_.nlay + 4) * en_.width + en_.wlds) * sizeof(double), stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
+    const size_t lds = (size_t) (4 * (2 * en_.nlay + 4) * en_.width + en_.wlds) * sizeof(double);
+    const dim3 grid((unsigned) ((n + kEnergyAtomsPerBlock - 1) / kEnergyAtomsPerBlock));
+    auto kern = en_.wlds > 0 ? k_energy<true> : k_energy<false>;
+    if (lds > 48 * 1024)
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
                        fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), fl.energy_only ? 0 : 1, sid_ptr());
   });
   if (fl.energy_only) return;

@@ -978,30 +978,42 @@ struct EnergyDev {
   const double *shift;        // [nel]
 };
 
+constexpr int kEnergyAtomsPerBlock = 16;    // atoms of one block of k_energy (4 waves, 4 atoms each)
+
 // E_i = (MLP(rho[1:]) + rho[0]) out_scale + shift[mu_i] and dE/drho, fp64, one wave per atom (fused_1l.cpp:378-427;
-// legacy RMS layer norm fused_cpu.h:666-682)
-static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, const double *rho, double *grho, double *eatom_chunk,
-                         double *energy, int want_grad, const int *sid)
+// legacy RMS layer norm fused_cpu.h:666-682).  A block of 4 waves shares the staged weights and walks
+// kEnergyAtomsPerBlock atoms; WLDS: the weights of the network sit in LDS (as stored and transposed), else they are
+// read from global memory.  dynamic LDS: M.wlds + 4 x (2 nlay + 4) x width doubles.
+template<bool WLDS>
+static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *mu, int a0, int natoms, const double *rho, double *grho,
+                                                         double *eatom_chunk, double *energy, int want_grad, const int *sid)
 {
-  // LDS rows of W = M.width values: nlay + 1 activations, nlay pre-activations, 2 adjoint buffers, x0
+  // LDS rows of W = M.width values per wave: nlay + 1 activations, nlay pre-activations, 2 adjoint buffers, x0
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const int W = M.width;
-  double *act_ = reinterpret_cast<double *>(smem_raw), *pre_ = act_ + (M.nlay + 1) * W, *gbuf_ = pre_ + M.nlay * W, *x0 = gbuf_ + 2 * W;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  double *wl0 = reinterpret_cast<double *>(smem_raw);
+  double *act_ = wl0 + (WLDS ? M.wlds : 0) + wave * (2 * M.nlay + 4) * W, *pre_ = act_ + (M.nlay + 1) * W, *gbuf_ = pre_ + M.nlay * W,
+         *x0 = gbuf_ + 2 * W;
 #define act(L_, k_) act_[(L_) * W + (k_)]
 #define pre(L_, k_) pre_[(L_) * W + (k_)]
 #define gbuf(L_, k_) gbuf_[(L_) * W + (k_)]
-  const int at = blockIdx.x, lane = threadIdx.x;
-  const double *r = rho + (long long) at * M.nrho;
-  const int n0 = M.nrho - 1;
-  // the weights of a small network go to LDS first, as stored [a][c] for the forward pass and transposed [c][a] for the
-  // reverse: one round of coalesced loads instead of a dependent chain of them per layer
+  // the rows of a wave are its own: a wave-level barrier orders its LDS writes before the reads of its other lanes
+#define GR_WAVE_SYNC()                                        \
+  do {                                                        \
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");    \
+    __builtin_amdgcn_wave_barrier();                          \
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");    \
+  } while (0)
+  // as stored [a][c] for the forward pass and transposed [c][a] for the reverse: one round of coalesced loads per block
+  // instead of a dependent chain of them per layer and atom
   const double *wf[7], *wt[7];
   {
-    double *wl = x0 + W;
+    double *wl = wl0;
     for (int L = 0; L < M.nlay; L++) {
       const int sz = M.nin[L] * M.nout[L];
-      if (M.wlds) {
-        for (int e = lane; e < sz; e += 64) {
+      if (WLDS) {
+        for (int e = threadIdx.x; e < sz; e += 256) {
           const double v = M.W[L][e];
           wl[e] = v;
           wl[sz + (e % M.nout[L]) * M.nin[L] + e / M.nout[L]] = v;
@@ -1015,71 +1027,80 @@ static __global__ void k_energy(EnergyDev M, const int *mu, int a0, int natoms, 
       }
     }
   }
-  for (int k = lane; k < n0; k += 64) act(0, k) = r[k + 1];
   __syncthreads();
-  double q = 0.0;
-  if (M.ln) {
-    double ms = 0.0;
-    for (int k = lane; k < n0; k += 64) { x0[k] = act(0, k); ms += act(0, k) * act(0, k); }
-    for (int o = 32; o > 0; o >>= 1) ms += __shfl_xor(ms, o, 64);
-    q = 1.0 / sqrt(ms / n0 + 1e-16);
-    for (int k = lane; k < n0; k += 64) act(0, k) *= q;
-    __syncthreads();
-  }
-  for (int L = 0; L < M.nlay; L++) {
-    for (int c = lane; c < M.nout[L]; c += 64) {
-      double s = 0.0;
-      for (int a = 0; a < M.nin[L]; a++) s += act(L, a) * wf[L][a * M.nout[L] + c];
-      s *= M.norm[L];
-      pre(L, c) = s;
-      act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+  const int n0 = M.nrho - 1;
+  for (int k4 = 0; k4 < kEnergyAtomsPerBlock / 4; k4++) {
+    const int at = blockIdx.x * kEnergyAtomsPerBlock + k4 * 4 + wave;
+    if (at >= natoms) break;                        // uniform over the wave; no block barrier below
+    const double *r = rho + (long long) at * M.nrho;
+    GR_WAVE_SYNC();                                 // the rows of the previous atom are no longer read
+    for (int k = lane; k < n0; k += 64) act(0, k) = r[k + 1];
+    GR_WAVE_SYNC();
+    double q = 0.0;
+    if (M.ln) {
+      double ms = 0.0;
+      for (int k = lane; k < n0; k += 64) { x0[k] = act(0, k); ms += act(0, k) * act(0, k); }
+      for (int o = 32; o > 0; o >>= 1) ms += __shfl_xor(ms, o, 64);
+      q = 1.0 / sqrt(ms / n0 + 1e-16);
+      for (int k = lane; k < n0; k += 64) act(0, k) *= q;
+      GR_WAVE_SYNC();
     }
-    __syncthreads();
-  }
-  const double Ei = (act(M.nlay, 0) + r[0]) * M.out_scale + M.shift[mu[a0 + at]];
-  if (lane == 0) {
-    if (eatom_chunk) eatom_chunk[at] = Ei;
-    atomicAdd(energy + (sid ? 8 * sid[a0 + at] : 0), Ei);    // one (energy, virial[6]) record of 8 doubles per structure
-  }
-  if (!want_grad) return;
-  int cur = 0;
-  if (lane == 0) gbuf(0, 0) = M.out_scale;
-  __syncthreads();
-  for (int L = M.nlay - 1; L >= 0; L--) {
-    if (L < M.nlay - 1) {
+    for (int L = 0; L < M.nlay; L++) {
       for (int c = lane; c < M.nout[L]; c += 64) {
-        const double v = pre(L, c);
-        if (M.act == 1) {
-          const double t = act(L + 1, c);
-          gbuf(cur, c) *= 1.0 - t * t;
-        } else {
-          const double sg = 1.0 / (1.0 + exp(-v));
-          gbuf(cur, c) *= sg * (1.0 + v * (1.0 - sg));
-        }
+        double s = 0.0;
+        for (int a = 0; a < M.nin[L]; a++) s += act(L, a) * wf[L][a * M.nout[L] + c];
+        s *= M.norm[L];
+        pre(L, c) = s;
+        act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
       }
-      __syncthreads();
+      GR_WAVE_SYNC();
     }
-    for (int a = lane; a < M.nin[L]; a += 64) {
-      double s = 0.0;
-      if (wt[L])
-        for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * wt[L][c * M.nin[L] + a];
-      else
-        for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * wf[L][(long long) a * M.nout[L] + c];
-      gbuf(cur ^ 1, a) = s * M.norm[L];
+    const double Ei = (act(M.nlay, 0) + r[0]) * M.out_scale + M.shift[mu[a0 + at]];
+    if (lane == 0) {
+      if (eatom_chunk) eatom_chunk[at] = Ei;
+      atomicAdd(energy + (sid ? 8 * sid[a0 + at] : 0), Ei);    // one (energy, virial[6]) record of 8 doubles per structure
     }
-    cur ^= 1;
-    __syncthreads();
+    if (!want_grad) continue;
+    int cur = 0;
+    if (lane == 0) gbuf(0, 0) = M.out_scale;
+    GR_WAVE_SYNC();
+    for (int L = M.nlay - 1; L >= 0; L--) {
+      if (L < M.nlay - 1) {
+        for (int c = lane; c < M.nout[L]; c += 64) {
+          const double v = pre(L, c);
+          if (M.act == 1) {
+            const double t = act(L + 1, c);
+            gbuf(cur, c) *= 1.0 - t * t;
+          } else {
+            const double sg = 1.0 / (1.0 + exp(-v));
+            gbuf(cur, c) *= sg * (1.0 + v * (1.0 - sg));
+          }
+        }
+        GR_WAVE_SYNC();
+      }
+      for (int a = lane; a < M.nin[L]; a += 64) {
+        double s = 0.0;
+        if (WLDS)
+          for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * wt[L][c * M.nin[L] + a];
+        else
+          for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * wf[L][(long long) a * M.nout[L] + c];
+        gbuf(cur ^ 1, a) = s * M.norm[L];
+      }
+      cur ^= 1;
+      GR_WAVE_SYNC();
+    }
+    if (M.ln) {
+      double t = 0.0;
+      for (int k = lane; k < n0; k += 64) t += gbuf(cur, k) * x0[k];
+      for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
+      for (int k = lane; k < n0; k += 64) gbuf(cur, k) = q * (gbuf(cur, k) - x0[k] * t * q * q / n0);
+      GR_WAVE_SYNC();
+    }
+    double *g = grho + (long long) at * M.nrho;
+    if (lane == 0) g[0] = M.out_scale;
+    for (int k = lane; k < n0; k += 64) g[k + 1] = gbuf(cur, k);
   }
-  if (M.ln) {
-    double t = 0.0;
-    for (int k = lane; k < n0; k += 64) t += gbuf(cur, k) * x0[k];
-    for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
-    for (int k = lane; k < n0; k += 64) gbuf(cur, k) = q * (gbuf(cur, k) - x0[k] * t * q * q / n0);
-    __syncthreads();
-  }
-  double *g = grho + (long long) at * M.nrho;
-  if (lane == 0) g[0] = M.out_scale;
-  for (int k = lane; k < n0; k += 64) g[k + 1] = gbuf(cur, k);
+#undef GR_WAVE_SYNC
 #undef act
 #undef pre
 #undef gbuf
