@@ -6,6 +6,7 @@
 #include "neighbors.hpp"
 #include "neighbors_dev.hpp"
 #include "neighbors_batch_dev.hpp"
+#include "lammps_dev.hpp"
 
 #include <hip/hip_runtime_api.h>
 
@@ -27,7 +28,8 @@ struct gr_engine {
   std::unique_ptr<grhip::Engine> eng;
   std::vector<grhip::StageTime> times;
   std::unique_ptr<grhip::BatchDeviceNeighbors> bnl;    // lists of gr_compute_batch_device (buffers kept between calls)
-  hipStream_t bnl_stream = nullptr;
+  std::unique_ptr<grhip::LammpsDeviceList> lmp;       // converted list of gr_compute_lammps_device
+  hipStream_t bnl_stream = nullptr;                    // stream of the list builds of the device entry points
   ~gr_engine()
   {
     if (bnl_stream) (void) hipStreamDestroy(bnl_stream);
@@ -467,6 +469,110 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
   });
 }
 
+int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, const int *type, const double *x, int inum, const int *ilist,
+                             const int *numneigh, const int *neighbors, int64_t stride_i, int64_t stride_k, int neighmask, const int *owner,
+                             unsigned flags, double *energy, double *f, double *virial, double *eatom)
+{
+  return guarded([&] {
+    if (!e || (nall > 0 && (!type || !x)) || (inum > 0 && (!ilist || !numneigh || !neighbors))) throw grhip::InvalidArgument("null argument");
+    if (nlocal < 0 || nall < nlocal || inum < 0 || ntypes < 0) throw grhip::InvalidArgument("atom counts out of range");
+    grhip::Engine &eng = *e->eng;
+    if (hipSetDevice(eng.device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
+    auto on_device = [&](const void *p, const char *name) {
+      if (!p) return;
+      hipPointerAttribute_t at;
+      if (hipPointerGetAttributes(&at, p) != hipSuccess || at.type != hipMemoryTypeDevice || at.device != eng.device_index()) {
+        (void) hipGetLastError();
+        throw grhip::InvalidArgument(std::string(name) + " must be memory of the engine's GPU");
+      }
+    };
+    on_device(type, "type"); on_device(x, "x"); on_device(ilist, "ilist"); on_device(numneigh, "numneigh");
+    on_device(neighbors, "neighbors"); on_device(owner, "owner"); on_device(f, "f"); on_device(eatom, "eatom");
+    if (!e->bnl_stream && hipStreamCreateWithFlags(&e->bnl_stream, hipStreamNonBlocking) != hipSuccess) throw grhip::Error("hipStreamCreate failed");
+    if (!e->lmp) e->lmp = std::make_unique<grhip::LammpsDeviceList>();
+    grhip::LammpsDeviceList &W = *e->lmp;
+    hipStream_t st = e->bnl_stream;
+    // work queued by the caller on other streams (the arrays that hold the inputs) is finished first
+    if (hipDeviceSynchronize() != hipSuccess) throw grhip::Error("hipDeviceSynchronize failed");
+    // atom types and the atom list: 4 bytes per atom to the host, where the rows of the engine and its element tiles are laid out
+    std::vector<int> ty((size_t) nall), il((size_t) inum);
+    if (nall > 0 && hipMemcpy(ty.data(), type, sizeof(int) * (size_t) nall, hipMemcpyDeviceToHost) != hipSuccess) throw grhip::Error("copy of the atom types failed");
+    if (inum > 0 && hipMemcpy(il.data(), ilist, sizeof(int) * (size_t) inum, hipMemcpyDeviceToHost) != hipSuccess) throw grhip::Error("copy of ilist failed");
+    std::vector<unsigned char> mapped((size_t) ntypes + 1, 0);
+    for (int t = 1; t <= ntypes; t++) mapped[t] = eng.cutoff(t, t) > 0.0;
+    for (int a = 0; a < nall; a++)
+      if (ty[a] < 1 || ty[a] > ntypes) throw grhip::InvalidArgument("types must be 1 .. ntypes");
+    std::vector<int> idx((size_t) nlocal, -1), atom, tq;
+    std::vector<char> central((size_t) nlocal, 0);
+    for (int q = 0; q < inum; q++) {
+      const int i = il[q];
+      if (i < 0 || i >= nlocal) throw grhip::InvalidArgument("ilist must index owned atoms");
+      if (!mapped[ty[i]]) throw grhip::Error("atom " + std::to_string(i) + " of unmapped type " + std::to_string(ty[i]) + " in the atom list");
+      central[i] = 1;
+    }
+    for (int i = 0; i < nlocal; i++) {
+      if (!mapped[ty[i]]) continue;
+      if (!central[i]) throw grhip::InvalidArgument("every owned atom of a mapped type must be in ilist (sub-lists are not supported)");
+      idx[i] = (int) atom.size();
+      atom.push_back(i);
+      tq.push_back(ty[i]);
+    }
+    const int n = (int) atom.size();
+    auto put = [&](grhip::DevBuf &b, const void *src, size_t bytes) {
+      b.ensure(std::max<size_t>(bytes, 8));
+      if (bytes && hipMemcpyAsync(b.p, src, bytes, hipMemcpyHostToDevice, st) != hipSuccess) throw grhip::Error("copy to the device failed");
+    };
+    put(W.idx, idx.data(), sizeof(int) * (size_t) nlocal);
+    put(W.atom, atom.data(), sizeof(int) * (size_t) n);
+    put(W.mapped, mapped.data(), mapped.size());
+    const int zero = 0;
+    put(W.err, &zero, sizeof(int));
+    W.count.ensure(sizeof(int) * (size_t) std::max(n, 1));
+    W.offset.ensure(sizeof(long long) * (size_t) (n + 1));
+    grhip::LmpListDev L{};
+    L.type = type; L.x = x; L.numneigh = numneigh; L.neighbors = neighbors; L.stride_i = stride_i; L.stride_k = stride_k;
+    L.owner = owner; L.idx = W.idx.as<int>(); L.atom = W.atom.as<int>(); L.mapped = W.mapped.as<unsigned char>();
+    L.n = n; L.nlocal = nlocal; L.nall = nall; L.neighmask = neighmask;
+    W.nb = 0;
+    if (n > 0) {
+      const dim3 grid((unsigned) ((n + 127) / 128)), block(128);
+      hipLaunchKernelGGL(grhip::k_lmp_rows<false>, grid, block, 0, st, L, W.count.as<int>(), W.err.as<int>(), (const long long *) nullptr, (int *) nullptr,
+                         (double *) nullptr);
+      hipLaunchKernelGGL(grhip::k_scan, dim3(1), dim3(1024), 0, st, W.count.as<int>(), n, W.offset.as<long long>());
+      long long total = 0;
+      int err = 0;
+      if (hipMemcpyAsync(&total, W.offset.as<long long>() + n, sizeof(total), hipMemcpyDeviceToHost, st) != hipSuccess ||
+          hipMemcpyAsync(&err, W.err.p, sizeof(err), hipMemcpyDeviceToHost, st) != hipSuccess || hipStreamSynchronize(st) != hipSuccess)
+        throw grhip::Error("the conversion of the neighbour list failed");
+      if (err == 1) throw grhip::InvalidArgument("neighbour index outside the owned and ghost atoms");
+      if (err == 2) throw grhip::InvalidArgument(owner ? "the owner of a ghost atom is not an owned atom of the same type"
+                                                       : "ghost neighbours need the owner map (the owned atom each ghost is an image of)");
+      W.nb = total;
+      W.j.ensure(sizeof(int) * (size_t) std::max<int64_t>(W.nb, 1));
+      W.rij.ensure(sizeof(double) * 3 * (size_t) std::max<int64_t>(W.nb, 1));
+      hipLaunchKernelGGL(grhip::k_lmp_rows<true>, grid, block, 0, st, L, (int *) nullptr, (int *) nullptr, (const long long *) W.offset.as<long long>(),
+                         W.j.as<int>(), W.rij.as<double>());
+    } else {
+      const long long z = 0;
+      put(W.offset, &z, sizeof(z));
+    }
+    if (hipStreamSynchronize(st) != hipSuccess) throw grhip::Error("the conversion of the neighbour list failed");
+    grhip::DeviceCsr in;
+    in.n = n;
+    in.types = tq.data();
+    in.nb = W.nb;
+    in.offset = W.offset.as<int64_t>();
+    in.j = W.j.as<int>();
+    in.rij = W.rij.as<double>();
+    eng.upload_device(in);
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    eng.run(fl);
+    eng.fetch_add_device(W.atom.as<int>(), energy, f, virial, fl.eatom ? eatom : nullptr);
+  });
+}
+
 int gr_system_create(gr_engine *e, double skin, gr_system **out)
 {
   return guarded([&] {
@@ -822,10 +928,8 @@ int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const 
     on_device(forces, "forces");
     on_device(virial, "virial");
     on_device(eatom, "energies");
-    if (!e->bnl) {
-      e->bnl = std::make_unique<grhip::BatchDeviceNeighbors>();
-      if (hipStreamCreateWithFlags(&e->bnl_stream, hipStreamNonBlocking) != hipSuccess) throw grhip::Error("hipStreamCreate failed");
-    }
+    if (!e->bnl) e->bnl = std::make_unique<grhip::BatchDeviceNeighbors>();
+    if (!e->bnl_stream && hipStreamCreateWithFlags(&e->bnl_stream, hipStreamNonBlocking) != hipSuccess) throw grhip::Error("hipStreamCreate failed");
     // work queued by the caller on the default stream (the tensors that hold the inputs) is finished first
     if (hipDeviceSynchronize() != hipSuccess) throw grhip::Error("hipDeviceSynchronize failed");
     grhip::BatchDeviceNeighbors &nl = *e->bnl;

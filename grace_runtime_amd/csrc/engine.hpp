@@ -77,6 +77,9 @@ class Engine {
   virtual void fetch_batch(int nstruct, double *energy, double *forces, double *virial, double *eatom) = 0;
   // the same with every output in device memory (the engine's GPU); null pointers are skipped
   virtual void fetch_batch_device(int nstruct, double *energy, double *forces, double *virial, double *eatom) = 0;
+  // one structure: energy and virial [6] to the host; forces and per-atom energies ADDED to device arrays of the
+  // caller, row q of the engine to row atom[q] (atom: device [n]); null pointers are skipped
+  virtual void fetch_add_device(const int *atom, double *energy, double *forces, double *virial, double *eatom) = 0;
   virtual void synchronize() = 0;
   virtual void set_profile(bool on) = 0;
   virtual const std::vector<StageTime> &stage_times() = 0;

@@ -669,6 +669,30 @@ class EngineBase : public Engine {
                     std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
     }
   }
+  void fetch_add_device(const int *atom, double *energy, double *forces, double *virial, double *eatom) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (!ran_) throw Error("fetch() before run()");
+    if (have_sid_) throw Error("the uploaded list holds several structures: use fetch_batch()");
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    if (n_ > 0) {    // before anything is added to the caller's arrays
+      int zb[2];
+      HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
+      if (zb[0] >= 0)    // bonds.h:49-62
+        throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " +
+                    std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
+    }
+    const bool wf = forces && ran_forces_, we = eatom && ran_eatom_;
+    if (n_ > 0 && (wf || we))
+      hipLaunchKernelGGL(k_add_results, dim3((unsigned) ((n_ + 255) / 256)), dim3(256), 0, stream_, atom, n_, f_.as<double>(), wf ? forces : nullptr,
+                         eatom_.as<double>(), we ? eatom : nullptr);
+    double s[8];
+    HIP_CHECK(hipMemcpyAsync(s, scal_.p, sizeof(s), hipMemcpyDeviceToHost, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    if (energy) *energy = s[0];
+    if (virial && ran_forces_)
+      for (int k = 0; k < 6; k++) virial[k] = s[1 + k];
+  }
   int64_t last_edge_count() override
   {
     synchronize();

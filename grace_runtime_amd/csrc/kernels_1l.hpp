@@ -195,6 +195,20 @@ static __global__ void k_unpack_records(const double *rec, int nstruct, double *
     for (int k = 0; k < 6; k++) virial[6 * (long long) s + k] = rec[8 * (long long) s + 1 + k];
 }
 
+// f[atom[q]] += fe[q], eatom[atom[q]] += ee[q] for the n rows of the engine (null pointers are skipped)
+static __global__ void k_add_results(const int *atom, int n, const double *fe, double *f, const double *ee, double *eatom)
+{
+  const int q = blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= n) return;
+  const long long i = atom[q];
+  if (f) {
+    f[3 * i] += fe[3 * (long long) q];
+    f[3 * i + 1] += fe[3 * (long long) q + 1];
+    f[3 * i + 2] += fe[3 * (long long) q + 2];
+  }
+  if (eatom) eatom[i] += ee[q];
+}
+
 struct Edges {
   int *ei, *ej, *emu;         // central atom, neighbour, neighbour element
   double *rh;                 // [E][3] unit vectors

@@ -228,6 +228,33 @@ class Engine:
             out["energies"] = ea
         return out
 
+    def compute_lammps_device(self, nlocal, types, x, ilist, numneigh, neighbors, owner=None, neighmask=0x1FFFFFFF, energy_only=False,
+                              forces=None, eatom=None):
+        """The call of a KOKKOS pair style (gr_compute_lammps_device): every array is a device array of the module's GPU
+        (torch tensors): `types[nall]` int32, `x[nall, 3]`, `ilist[inum]`, `numneigh[nlocal]`, the 2-d neighbour view
+        `neighbors[nlocal, maxneigh]` in either layout, `owner[nall]`.  Forces are ADDED to `forces[nall, 3]` and per-atom
+        energies to `eatom[nall]` in place; energy and virial come back on the host."""
+        nall, inum = int(types.shape[0]), int(ilist.shape[0])
+        p_t = _device_pointer(types, "types", (nall,), "int32")
+        p_x = _device_pointer(x, "x", (nall, 3), "float64")
+        p_il = _device_pointer(ilist, "ilist", (inum,), "int32")
+        p_nn = _device_pointer(numneigh, "numneigh", (int(numneigh.shape[0]),), "int32")
+        if numneigh.shape[0] < nlocal or neighbors.dim() != 2 or neighbors.shape[0] < nlocal or str(neighbors.dtype) != "torch.int32" or \
+                neighbors.device != types.device:
+            raise ValueError("neighbors: expected an int32 device array [nlocal, maxneigh]")
+        p_own = _device_pointer(owner, "owner", (nall,), "int32") if owner is not None else None
+        p_f = _device_pointer(forces, "forces", (nall, 3), "float64") if forces is not None else None
+        p_ea = _device_pointer(eatom, "eatom", (nall,), "float64") if eatom is not None else None
+        e, v = C.c_double(), np.zeros(6)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if eatom is not None else 0)
+        check(_lib.lib().gr_compute_lammps_device(self._h, int(nlocal), nall, len(self.species), p_t, p_x, inum, p_il, p_nn,
+                                                  C.c_void_p(neighbors.data_ptr()), int(neighbors.stride(0)), int(neighbors.stride(1)),
+                                                  int(neighmask), p_own, flags, C.byref(e), None if energy_only else p_f, ptr(v), p_ea))
+        out = {"energy": e.value}
+        if not energy_only:
+            out["virial"] = v
+        return out
+
     def compute(self, types, offset, j, rij=None, energies=False, energy_only=False, positions=None, image=None,
                 shifts=None):
         n, arrs, nimg = self._csr_args(types, offset, j, rij, positions, image, shifts)

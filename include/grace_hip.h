@@ -136,6 +136,19 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
                       const int *const *firstneigh, int neighmask, const int *owner, unsigned flags, double *energy, double *f,
                       double *virial, double *eatom);
 
+/* The same call with every per-atom array in DEVICE memory of the engine's GPU: the RunInput / RunOutput of the
+ * reference's GPU engines (libgrace/include/grace/kk/grace_1l_kk.h:80-103, grace_2l_kk.h:81-157, grace_3l_kk.h:232-324),
+ * i.e. what a KOKKOS pair style holds.  type [nall], x [nall][3], ilist [inum], numneigh [nlocal] (by atom), owner [nall]
+ * (or NULL), f [nall][3] and eatom [nall] (added to) are device pointers; the neighbour list is the 2-d view of the KOKKOS
+ * list, element (i, k) at neighbors[i * stride_i + k * stride_k] (either layout).  ntypes: atom types of the run (the
+ * engine's type map covers 1 .. ntypes).  The list is converted to the engine's rows on the device; the atom types and
+ * ilist make one 4-byte-per-atom trip to the host for the layout of the rows.  energy and virial [6] are returned to the
+ * host, as RunOutput.  The call waits for work queued on the device before it reads the inputs.  Same restrictions as
+ * gr_compute_lammps. */
+int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, const int *type, const double *x, int inum, const int *ilist,
+                             const int *numneigh, const int *neighbors, int64_t stride_i, int64_t stride_k, int neighmask, const int *owner,
+                             unsigned flags, double *energy, double *f, double *virial, double *eatom);
+
 /* One structure resident on the device with a Verlet list at cutoff + skin: System of the reference's GPU module
  * (python/kk/kk_api.h:66-93, System::compute python/kk/kk_core.cpp:802-958; list policy python/grace_runtime/
  * neighbors.py:68-89: rebuild when types, cell or pbc change or an atom moved more than skin / 2).  The pair search of

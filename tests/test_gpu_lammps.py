@@ -65,6 +65,49 @@ def test_lammps_call_equals_csr_call(model_dir, model, species, struct):
     assert abs(eo["energy"] - ref["energy"]) < 1e-10 * max(1.0, abs(ref["energy"])) and "forces" not in eo
 
 
+@pytest.mark.parametrize("layout", ["right", "left"])
+@pytest.mark.parametrize("model,species,struct", [("mix2", ["Mo", "W"], "alloy54"), ("l2mix", ["Mo", "W"], "triclinic")])
+def test_device_arrays_equal_host_arrays(model_dir, model, species, struct, layout):
+    """the KOKKOS form of the call (every array on the device, the 2-d neighbour view in either layout) = the host form"""
+    import torch
+    eng = kk.Engine(kk.Model(os.path.join(model_dir, model + ".npz")), species, 64)
+    pos, cell, pbc, types = cases.STRUCTURES[struct]()
+    n = len(pos)
+    rc = max(eng.cutoff(a, b) for a in (1, 2) for b in (1, 2))
+    x, t, owner, rows = lammps_inputs(pos, cell, types, rc + 0.7)
+    f0 = np.random.default_rng(1).standard_normal((len(x), 3))
+    ref = eng.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows, owner=owner, energies=True, forces=f0.copy())
+    dev = torch.device("cuda", 0)
+    maxn = max(len(r) for r in rows) + 3
+    nbh = np.full((n, maxn), -7, np.int32)                                  # entries beyond numneigh are never read
+    for i, r in enumerate(rows):
+        nbh[i, :len(r)] = r
+    nb = torch.as_tensor(nbh, device=dev)
+    if layout == "left":
+        nb = nb.t().contiguous().t()                                        # column-major storage, same shape
+        assert nb.stride(0) == 1
+    td, xd, od = torch.as_tensor(t, device=dev), torch.as_tensor(x, device=dev), torch.as_tensor(owner, device=dev)
+    il = torch.arange(n, dtype=torch.int32, device=dev)
+    nn = torch.as_tensor(np.array([len(r) for r in rows], np.int32), device=dev)
+    f, ea = torch.as_tensor(f0.copy(), device=dev), torch.zeros(len(x), dtype=torch.float64, device=dev)
+    out = eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=od, forces=f, eatom=ea)
+    fs = max(1.0, np.abs(ref["forces"]).max())
+    assert abs(out["energy"] - ref["energy"]) < 1e-10 * max(1.0, abs(ref["energy"]))
+    assert np.abs(f.cpu().numpy() - ref["forces"]).max() < 1e-9 * fs
+    assert np.abs(out["virial"] - ref["virial"]).max() < 1e-9 * max(1.0, np.abs(ref["virial"]).max())
+    assert np.abs(ea.cpu().numpy() - ref["energies"]).max() < 1e-10 * fs
+    eo = eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=od, energy_only=True)
+    assert abs(eo["energy"] - ref["energy"]) < 1e-10 * max(1.0, abs(ref["energy"]))
+    with pytest.raises(ValueError, match="owner"):
+        eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=None, forces=f)
+    bad = od.clone()
+    bad[n:] = n + 5
+    with pytest.raises(ValueError, match="owner of a ghost"):
+        eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=bad, forces=f)
+    with pytest.raises(ValueError, match="must be on the module's GPU"):
+        eng.compute_lammps_device(n, td, torch.as_tensor(x), il, nn, nb, owner=od, forces=f)
+
+
 def test_unmapped_types_take_no_part_and_argument_errors(model_dir):
     """pair_style hybrid: atoms of a type without a model element are neither central atoms nor neighbours"""
     model = kk.Model(os.path.join(model_dir, "mix2.npz"))
