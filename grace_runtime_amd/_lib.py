@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgrace_hip.so")
 
 GR_OK, GR_INVALID, GR_ERROR, GR_NOMEM = 0, 1, 2, 3
-FLAG_ENERGY_ONLY, FLAG_EATOM = 1, 2
+FLAG_ENERGY_ONLY, FLAG_EATOM, FLAG_UQ = 1, 2, 4
 
 # every symbol include/grace_hip.h declares (checked by the CPU test-suite against the header and the library)
 SYMBOLS = [
@@ -24,7 +24,8 @@ SYMBOLS = [
     "gr_engine_debug_radial", "gr_engine_debug_copy", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
-    "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_lammps_device",
+    "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
+    "gr_system_fetch_uq",
 ]
 
 
@@ -91,6 +92,10 @@ def lib():
     L.gr_engine_fetch_batch.argtypes = [vp, i32, vp, vp, vp, vp]
     L.gr_compute_batch_device.argtypes = [vp, i32, vp, vp, vp, vp, vp, u32, i64, vp, vp, vp, vp, vp]
     L.gr_compute_lammps_device.argtypes = [vp, i32, i32, i32, vp, vp, i32, vp, vp, vp, i64, i64, i32, vp, u32, vp, vp, vp, vp]
+    L.gr_model_has_uq.argtypes = [vp]
+    L.gr_model_validate_uq.argtypes = [vp]
+    L.gr_engine_fetch_uq.argtypes = [vp, vp, vp, vp]
+    L.gr_system_fetch_uq.argtypes = [vp, vp, vp, vp]
     L.gr_compute_lammps.argtypes = [vp, i32, i32, vp, vp, i32, vp, vp, vp, i32, vp, u32, vp, vp, vp, vp]
     L.gr_system_create.argtypes = [vp, dbl, C.POINTER(vp)]
     L.gr_system_free.argtypes = [vp]

@@ -241,7 +241,31 @@ int gr_engine_run(gr_engine *e, unsigned flags)
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0;
+    fl.uq = (flags & GR_FLAG_UQ) != 0;
     e->eng->run(fl);
+  });
+}
+
+int gr_engine_fetch_uq(gr_engine *e, double *gamma, double *sigma, double *cluster)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->eng->fetch_uq(gamma, sigma, cluster);
+  });
+}
+
+int gr_model_has_uq(const gr_model *m) { return m && m->m1 && m->m1->uq.has_uq ? 1 : 0; }
+
+int gr_model_validate_uq(const gr_model *m)
+{
+  return guarded([&] {
+    if (!m) throw grhip::InvalidArgument("null model");
+    if (!m->m1) throw grhip::InvalidArgument("the UQ head is evaluated for GRACE-1L models only");
+    try {
+      m->m1->validate_uq();
+    } catch (const grhip::Error &e) {
+      throw grhip::InvalidArgument(e.what());    // python/kk/kk_core.cpp: std::invalid_argument (unsupported model)
+    }
   });
 }
 
@@ -671,6 +695,7 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.uq = (flags & GR_FLAG_UQ) != 0;
     eng.run(fl);
     std::vector<double> f((size_t) 3 * n), ea(fl.eatom ? n : 0);
     eng.fetch(energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
@@ -679,6 +704,22 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
       if (forces && !fl.energy_only)
         for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) q + d];
       if (fl.eatom) eatom[a] = ea[q];
+    }
+  });
+}
+
+int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *cluster)
+{
+  return guarded([&] {
+    if (!s || !s->have) throw grhip::Error("gr_system_fetch_uq: no structure has been computed");
+    const int n = s->n;
+    std::vector<double> g((size_t) n), sg((size_t) n), cl((size_t) n);
+    s->eng->eng->fetch_uq(g.data(), sg.data(), cl.data());
+    for (int q = 0; q < n; q++) {
+      const int64_t a = s->perm[q];
+      if (gamma) gamma[a] = g[q];
+      if (sigma) sigma[a] = sg[q];
+      if (cluster) cluster[a] = cl[q];
     }
   });
 }

@@ -54,6 +54,7 @@ struct StageTime {
 struct RunFlags {
   bool energy_only = false;
   bool eatom = false;
+  bool uq = false;    // UQ head (ComputeFlags::uq, libgrace/include/grace/system.h:117): gamma, sigma, cluster per atom
 };
 
 class Engine {
@@ -80,6 +81,8 @@ class Engine {
   // one structure: energy and virial [6] to the host; forces and per-atom energies ADDED to device arrays of the
   // caller, row q of the engine to row atom[q] (atom: device [n]); null pointers are skipped
   virtual void fetch_add_device(const int *atom, double *energy, double *forces, double *virial, double *eatom) = 0;
+  // UQ outputs of the last run with RunFlags::uq, [n] each in the order of the uploaded list (null pointers are skipped)
+  virtual void fetch_uq(double *gamma, double *sigma, double *cluster) = 0;
   virtual void synchronize() = 0;
   virtual void set_profile(bool on) = 0;
   virtual const std::vector<StageTime> &stage_times() = 0;

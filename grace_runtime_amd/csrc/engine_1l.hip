@@ -39,6 +39,8 @@ template<class T> class Engine1L final : public EngineBase {
   DevFcPairBwd<T> fcAA12_;    // reverse of fc_AA1 and fc_AA2 in one pass over their shared inputs (models with the AAAA stage)
   DevProd pAA_, pAAA_, pAAAA_;
   DevReduce<T> redrho_;
+  UqDev<T> uq_{};             // UQ head (models that carry a valid one)
+  DevBuf uqR_, uqCen_, uqIcov_, uqNcl_, uqThr_, uqCi_[4];
   DevBuf eW_[7];
   EnergyDev en_{};
 
@@ -167,6 +169,41 @@ template<class T> void Engine1L<T>::build()
     redrho_.build(src, nel_, nrho_, -1, nrho_, 0, drow_);
   }
 
+  // ---- UQ head: a head that does not validate leaves the model usable without UQ (libgrace/src/model_1l.cpp:216-271)
+  if (m.uq.has_uq) {
+    try {
+      m.validate_uq();
+      if (m.uq.rp_dim > 256 || m.uq.feature_dim > 256) throw Error("GRACE-1L UQ: feature widths above 256 are not supported");
+      const ReduceWeights *rw[4] = {&m.red_A, &m.red_AA, &m.red_AAA, &m.red_AAAA};
+      const int nfun[4] = {nlm_, nAA_, nAAA_, nAAAA_};
+      uq_.nsrc = order4_ ? 4 : 3;
+      int off = 0;
+      for (int s = 0; s < uq_.nsrc; s++) {
+        upload_vec(uqCi_[s], rw[s]->collect_ind);
+        uq_.ci[s] = uqCi_[s].template as<int>();
+        uq_.nfun[s] = nfun[s];
+        uq_.cpad[s] = s == 0 ? CP_ : CFP_;
+        uq_.nin[s] = rw[s]->n_in;
+        uq_.nc[s] = (int) rw[s]->collect_ind.size();
+        uq_.off[s] = off;
+        off += uq_.nin[s] * uq_.nc[s];
+      }
+      uq_.d_basis = off;
+      uq_.rp = m.uq.rp_dim; uq_.D = m.uq.feature_dim; uq_.K = m.uq.max_clusters;
+      uq_.density_scale = m.uq.density_scale;
+      upload_vec(uqR_, m.uq.rp_matrix); upload_vec(uqCen_, m.uq.centroids); upload_vec(uqIcov_, m.uq.inv_cov);
+      upload_vec(uqNcl_, m.uq.n_clusters); upload_vec(uqThr_, m.uq.interp_thresholds);
+      uq_.R = uqR_.template as<double>(); uq_.cen = uqCen_.template as<double>(); uq_.icov = uqIcov_.template as<double>();
+      uq_.ncl = uqNcl_.template as<int>(); uq_.thr = uqThr_.template as<double>();
+      if ((size_t) (uq_.d_basis + 4 * uq_.rp + 2 * uq_.D) * sizeof(double) > 150 * 1024) throw Error("GRACE-1L UQ: the basis does not fit the kernel's LDS");
+      has_uq_head_ = true;
+    } catch (const std::exception &e) {
+      uq_why_ = e.what();
+    }
+  } else {
+    uq_why_ = "the model file carries none";
+  }
+
   // ---- energy MLP
   {
     en_.nlay = (int) m.energy_mlp.size();
@@ -279,6 +316,20 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
                        fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), fl.energy_only ? 0 : 1, sid_ptr());
   });
+  if (fl.uq) {
+    uq_gamma_.ensure(na * sizeof(double)); uq_sigma_.ensure(na * sizeof(double)); uq_cluster_.ensure(na * sizeof(double));
+    stage("uq", [&] {
+      UqDev<T> u = uq_;
+      u.X[0] = A; u.X[1] = AA; u.X[2] = AAA; u.X[3] = AAAA;
+      const size_t lds = (size_t) (u.d_basis + 4 * u.rp + 2 * u.D) * sizeof(double);
+      auto kern = k_uq<T>;
+      if (lds > 48 * 1024)
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+      hipLaunchKernelGGL(kern, dim3(n), dim3(256), lds, stream_, u, mu_.as<int>(), n, uq_gamma_.as<double>(), uq_sigma_.as<double>(),
+                         uq_cluster_.as<double>());
+    });
+    ran_uq_ = true;
+  }
   if (fl.energy_only) return;
 
   // ---- reverse

@@ -693,6 +693,16 @@ class EngineBase : public Engine {
     if (virial && ran_forces_)
       for (int k = 0; k < 6; k++) virial[k] = s[1 + k];
   }
+  void fetch_uq(double *gamma, double *sigma, double *cluster) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (!ran_ || !ran_uq_) throw Error("fetch_uq() needs a run with the UQ flag");
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    if (n_ == 0) return;
+    if (gamma) HIP_CHECK(hipMemcpy(gamma, uq_gamma_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
+    if (sigma) HIP_CHECK(hipMemcpy(sigma, uq_sigma_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
+    if (cluster) HIP_CHECK(hipMemcpy(cluster, uq_cluster_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
+  }
   int64_t last_edge_count() override
   {
     synchronize();
@@ -735,6 +745,8 @@ class EngineBase : public Engine {
     ran_ = true;
     ran_forces_ = !fl.energy_only;
     ran_eatom_ = fl.eatom;
+    ran_uq_ = false;    // set by the engine that evaluates a UQ head
+    if (fl.uq && !has_uq_head_) throw InvalidArgument(who_ + ": the model has no usable UQ head (" + uq_why_ + ")");
     if (n == 0) return false;
     count_.ensure(sizeof(int) * n);
     eoff_.ensure(sizeof(long long) * (n + 1));
@@ -949,7 +961,10 @@ class EngineBase : public Engine {
   const int *sid_ptr() const { return have_sid_ ? sid_.as<int>() : nullptr; }
   // edges of the pass and its outputs (scal: energy, virial[6])
   DevBuf count_, eoff_, zero_, ei_, ej_, emu_, rh_, r_, xr_, rc_, f_, eatom_, scal_;
-  bool ran_ = false, ran_forces_ = false, ran_eatom_ = false;
+  bool ran_ = false, ran_forces_ = false, ran_eatom_ = false, ran_uq_ = false;
+  bool has_uq_head_ = false;      // set by an engine whose model carries a valid UQ head
+  std::string uq_why_ = "this engine evaluates none";
+  DevBuf uq_gamma_, uq_sigma_, uq_cluster_;
   hipStream_t stream_ = nullptr;
   bool profile_ = false;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> events_;

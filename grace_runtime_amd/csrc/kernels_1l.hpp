@@ -1121,6 +1121,112 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// UQ head (uqv6, gamma only)
+// ---------------------------------------------------------------------------------------------------------------
+template<class T> struct UqDev {
+  const T *X[4];              // per-atom tensors of the reduce's sources [atom][function][channel]
+  const int *ci[4];           // collected functions of each source
+  int nfun[4], cpad[4], nin[4], nc[4], off[4];    // functions per atom, padded / real channels, collected, first basis index
+  int nsrc, d_basis, rp, D, K;
+  double density_scale;
+  const double *R;            // [d_basis][rp]
+  const double *cen;          // [nel][K][D]
+  const double *icov;         // [nel][K][D][D]
+  const int *ncl;             // [nel]
+  const double *thr;          // [nel][K]
+};
+
+// gamma, sigma, cluster of one atom per block (libgrace/include/grace/fused_cpu.h:1290-1312 basis, :1375-1412 GMM;
+// libgrace/src/fused_1l.cpp:616-636): basis B = the collected functions of the rho reduce's sources, n-outer and
+// c-inner per source; phi = ((B / |B|) R, log |B| scale, ...); nearest centroid of the atom's element, Mahalanobis
+// distance over the cluster's threshold.  fp64 throughout.  block: 256 threads; dynamic LDS: d_basis + 4 rp + 2 D doubles.
+template<class T>
+__global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natoms, double *gamma, double *sigma, double *cluster)
+{
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  double *Bsh = reinterpret_cast<double *>(smem_raw);       // [d_basis]
+  double *Zp = Bsh + U.d_basis;                             // [4][rp] partial projections
+  double *f = Zp + 4 * U.rp;                                // [D]
+  double *dl = f + U.D;                                     // [D]
+  __shared__ double wsum[4];
+  __shared__ int kstar;
+  const int at = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  if (at >= natoms) return;
+  // ---- basis and its norm
+  double n2 = 0.0;
+  for (int s = 0; s < U.nsrc; s++) {
+    const T *x = U.X[s] + (long long) at * U.nfun[s] * U.cpad[s];
+    const int w = U.nin[s] * U.nc[s];
+    for (int r = t; r < w; r += 256) {
+      const int n = r / U.nc[s], c = r % U.nc[s];
+      const double v = (double) x[U.ci[s][c] * U.cpad[s] + n];
+      Bsh[U.off[s] + r] = v;
+      n2 += v * v;
+    }
+  }
+  for (int o = 32; o > 0; o >>= 1) n2 += __shfl_xor(n2, o, 64);
+  if (lane == 0) wsum[wave] = n2;
+  __syncthreads();
+  const double nrm = sqrt(wsum[0] + wsum[1] + wsum[2] + wsum[3]);
+  // ---- projection Z = B R: column d = t mod rp, rows split over the 256 / rp (at most 4 used) thread groups
+  {
+    const int ng = 256 / U.rp > 4 ? 4 : 256 / U.rp, gq = t / U.rp, d = t % U.rp;
+    if (gq < ng) {
+      double z = 0.0;
+      for (int b = gq; b < U.d_basis; b += ng) z += Bsh[b] * U.R[(long long) b * U.rp + d];
+      Zp[gq * U.rp + d] = z;
+    }
+    __syncthreads();
+    if (t < U.D) {
+      if (t < U.rp) {
+        double z = 0.0;
+        for (int q = 0; q < ng; q++) z += Zp[q * U.rp + t];
+        f[t] = z / (nrm + 1.0e-12);
+      } else {
+        f[t] = log(nrm + 1.0e-12) * U.density_scale;
+      }
+    }
+    __syncthreads();
+  }
+  // ---- nearest centroid of the element (the first of equal distances)
+  const int m = mu[at];
+  if (t == 0) {
+    int kb = 0;
+    double best = 1.0e300;
+    for (int q = 0; q < U.ncl[m]; q++) {
+      const double *c = U.cen + ((long long) m * U.K + q) * U.D;
+      double d2 = 0.0;
+      for (int p = 0; p < U.D; p++) d2 += (f[p] - c[p]) * (f[p] - c[p]);
+      if (d2 < best) { best = d2; kb = q; }
+    }
+    kstar = kb;
+  }
+  __syncthreads();
+  const int kq = kstar;
+  for (int p = t; p < U.D; p += 256) dl[p] = f[p] - U.cen[((long long) m * U.K + kq) * U.D + p];
+  __syncthreads();
+  // ---- sigma^2 = delta^T S delta
+  const double *S = U.icov + ((long long) m * U.K + kq) * U.D * U.D;
+  double part = 0.0;
+  for (int p = t; p < U.D; p += 256) {
+    double y = 0.0;
+    for (int q = 0; q < U.D; q++) y += S[(long long) p * U.D + q] * dl[q];
+    part += dl[p] * y;
+  }
+  for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+  __syncthreads();
+  if (lane == 0) wsum[wave] = part;
+  __syncthreads();
+  if (t == 0) {
+    const double sg = sqrt(wsum[0] + wsum[1] + wsum[2] + wsum[3] + 1.0e-8);
+    const double th = U.thr[(long long) m * U.K + kq];
+    sigma[at] = sg;
+    gamma[at] = sg / (th > 1.0e-10 ? th : 1.0e-10);
+    cluster[at] = (double) kq;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
 // bond backward: forces and virial
 // ---------------------------------------------------------------------------------------------------------------
 template<class T> struct BondBwdArgs {

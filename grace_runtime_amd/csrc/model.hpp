@@ -78,6 +78,72 @@ inline std::vector<MLPLayer> load_mlp(const NpzView &v, const std::string &pfx, 
   return layers;
 }
 
+// The uqv6 UQ head of a model file (libgrace/include/grace/uq_head.h, loader libgrace/src/uq_head.cpp:11-76): the GMM
+// feature of an atom is phi = concat((B / |B|) R, n_density log-norm channels), B the invariant basis of the energy
+// path (the raw l = 0 inputs of the rho reduce), R the stored random projection; gamma = Mahalanobis distance to the
+// nearest centroid of the atom's element over the cluster's interpolation threshold.
+struct UqHead {
+  bool has_uq = false;
+  int schema = 0, n_elements = 0, max_clusters = 0, feature_dim = 0, rp_dim = 0, n_density = 0, normalize = 0, d_basis = 0;
+  double density_scale = 1.0;
+  std::vector<double> centroids;            // [E][Kmax][D]
+  std::vector<double> inv_cov;              // [E][Kmax][D][D]
+  std::vector<int> n_clusters;              // [E]
+  std::vector<double> interp_thresholds;    // [E][Kmax]
+  std::vector<double> rp_matrix;            // [d_basis][rp_dim]
+  std::string error;                        // what is wrong with the head (reported by validate_uq; the model stays usable)
+
+  // who: "GRACE-1L/KK"; checks and messages of uq_head.cpp:11-76
+  void load(const NpzView &v, int model_elements, const std::string &who)
+  {
+    *this = UqHead();
+    schema = v.int_scalar("uq_schema_version", 0);
+    has_uq = schema != 0;
+    if (schema != 6) return;
+    const std::string pre = who + " UQ: ";
+    try {
+      n_elements = v.int_scalar("uq_n_elements", model_elements);
+      require_eq("uq_n_elements", n_elements, model_elements, "n_elements");
+      max_clusters = v.int_in("uq_max_clusters", 0, 1, kMaxDim);
+      rp_dim = v.int_in("uq_rp_dim", 0, 1, kMaxDim);
+      feature_dim = v.int_in("uq_feature_dim", 0, rp_dim, kMaxDim);
+      normalize = v.int_scalar("uq_rp_normalize", 0);
+      const int add_density = v.int_scalar("uq_rp_add_density_channel", 0);
+      density_scale = v.double_scalar("uq_rp_density_scale", 1.0);
+      const int transform = v.int_scalar("uq_feature_transform", 0);
+      centroids = v.require_doubles("uq_centroids");
+      inv_cov = v.require_doubles("uq_inv_cov");
+      n_clusters = v.require_ints("uq_n_clusters");
+      interp_thresholds = v.require_doubles("uq_interp_thresholds");
+      rp_matrix = v.require_doubles("uq_rp_matrix");
+      if (normalize != 1 || add_density != 1 || transform != 0)
+        throw Error("schema v6 expects normalize=1, add_density_channel=1, feature_transform=0 (identity); got normalize=" +
+                    std::to_string(normalize) + ", add_density=" + std::to_string(add_density) + ", transform=" + std::to_string(transform) +
+                    ". Artifact mislabeled or unsupported variant.");
+      n_density = feature_dim - rp_dim;
+      const auto rs = v.shape_rank("uq_rp_matrix", 2);
+      require_eq("uq_rp_matrix", (int64_t) rs[1], rp_dim, "uq_rp_dim", "columns");
+      d_basis = (int) rs[0];
+      const size_t E = (size_t) n_elements, K = (size_t) max_clusters, D = (size_t) feature_dim;
+      require_size("uq_centroids", centroids, E * K * D);
+      require_size("uq_inv_cov", inv_cov, E * K * D * D);
+      require_size("uq_n_clusters", n_clusters, E);
+      require_size("uq_interp_thresholds", interp_thresholds, E * K);
+      for (size_t e = 0; e < n_clusters.size(); e++) {
+        if (n_clusters[e] <= 0)
+          throw Error("element index " + std::to_string(e) + " has no GMM clusters; uqv6 artifacts must cover all elements. Re-export the "
+                      "UQ artifacts with a current grace_utils.");
+        if (n_clusters[e] > max_clusters)
+          throw Error("element index " + std::to_string(e) + " has " + std::to_string(n_clusters[e]) + " GMM clusters, more than uq_max_clusters = " +
+                      std::to_string(max_clusters));
+      }
+    } catch (const std::exception &e) {
+      error = e.what();
+      if (error.rfind(pre, 0) != 0) error = pre + error;
+    }
+  }
+};
+
 struct Model1L {
   int n_elements = 0, embedding_size = 0, lmax = 0, nradbase = 0, nradmax = 0, radial_basis_p = 0;
   int max_order = 4;    // 3: the file has no AAAA stage (its contribution is exactly zero, the engine skips it)
@@ -96,9 +162,34 @@ struct Model1L {
   std::vector<double> shift_values;
   double output_scale = 1.0;
   std::vector<std::string> element_names;
+  UqHead uq;
 
   int nl() const { return lmax + 1; }
   int nlm() const { return (lmax + 1) * (lmax + 1); }
+  // width of the UQ basis: the collected functions of the rho reduce's sources times their channels
+  // (libgrace/include/grace/uq.h:31-48)
+  int uq_basis_width() const
+  {
+    int w = red_A.n_in * (int) red_A.collect_ind.size() + red_AA.n_in * (int) red_AA.collect_ind.size() +
+            red_AAA.n_in * (int) red_AAA.collect_ind.size();
+    if (max_order == 4) w += red_AAAA.n_in * (int) red_AAAA.collect_ind.size();
+    return w;
+  }
+  // libgrace/src/model_1l.cpp:275-285, libgrace/src/uq.cpp:8-33
+  void validate_uq() const
+  {
+    if (!uq.has_uq) throw Error("GRACE-1L: the model has no UQ head");
+    if (max_order == 3) throw Error("GRACE-1L: UQ is not supported for max_order 3 models");
+    if (uq.schema != 6)
+      throw Error("GRACE-1L: UQ schema v" + std::to_string(uq.schema) + " unsupported (expects v6, uqv6 basis-RP normalize+density). Re-export the "
+                  "UQ artifacts at schema v6 with a current grace_utils.");
+    if (!uq.error.empty()) throw Error(uq.error);
+    if (uq_basis_width() != uq.d_basis)
+      throw Error("GRACE-1L UQ: uq_rp_matrix has " + std::to_string(uq.d_basis) + " rows, the model's invariant basis has " +
+                  std::to_string(uq_basis_width()) + "; re-export the UQ artifacts for this model");
+    if (uq.n_density != 2)
+      throw Error("GRACE-1L UQ: " + std::to_string(uq.n_density) + " density channels, expected 2 (1 + basis blocks)");
+  }
   double pair_cutoff(int mu_i, int mu_j) const    // libgrace/include/grace/type_map.h:23-28
   {
     if (mu_i < 0 || mu_j < 0) return 0.0;
@@ -265,6 +356,7 @@ struct Model1L {
     if (v.has("shift_values")) require_size("shift_values", shift_values, (size_t) n_elements);
     else shift_values.assign(n_elements, 0.0);
     output_scale = v.double_scalar("output_scale", 1.0);
+    uq.load(v, n_elements, "GRACE-1L/KK");
   }
 };
 

@@ -14,7 +14,7 @@ import os
 import numpy as np
 
 from . import _lib
-from ._lib import FLAG_EATOM, FLAG_ENERGY_ONLY, as_array, check, ptr
+from ._lib import FLAG_EATOM, FLAG_ENERGY_ONLY, FLAG_UQ, as_array, check, ptr
 
 ABI = 7
 PLATFORM = "rocm"
@@ -121,13 +121,15 @@ class Model:
         self.lmax, self.n_radial, self.rcut, self.max_order = info.lmax, info.n_radial, info.rcut, info.max_order
         self.n_elements = info.n_elements
         self.element_names = [L.gr_model_element_name(self._h, k).decode() for k in range(info.n_elements)]
-        self.has_uq = False
+        self.has_uq = bool(L.gr_model_has_uq(self._h))
         self.slow_notice = ""
         self.needs_generic = False
         self.engine_setups = 0
 
     def validate_uq(self):
-        raise ValueError(f"GRACE-{self.layers}L: the model has no UQ head")
+        """ValueError when the model's UQ head cannot be evaluated (none, another schema, sizes that do not fit):
+        python/kk/kk_api.h:51-64, libgrace/src/model_1l.cpp:275-285.  The UQ head is evaluated for GRACE-1L models."""
+        check(_lib.lib().gr_model_validate_uq(self._h))
 
     def type2mu(self, species):
         """[-1, mu(species[0]), ...]; unknown element -> ValueError (python/kk/kk_core.cpp: std::invalid_argument);
@@ -275,9 +277,16 @@ class Engine:
         check(_lib.lib().gr_engine_upload(self._h, n, *[ptr(a) for a in arrs], nimg))
         self._n = n
 
-    def run(self, energies=False, energy_only=False):
-        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
+    def run(self, energies=False, energy_only=False, uq=False):
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (FLAG_UQ if uq else 0)
         check(_lib.lib().gr_engine_run(self._h, flags))
+
+    def fetch_uq(self):
+        """gamma, atomic_sigma, gmm_cluster [n] of the last run(uq=True), in the order of the uploaded list"""
+        n = self._n
+        g, sg, cl = np.empty(n), np.empty(n), np.empty(n)
+        check(_lib.lib().gr_engine_fetch_uq(self._h, ptr(g), ptr(sg), ptr(cl)))
+        return {"gamma": g, "atomic_sigma": sg, "gmm_cluster": cl}
 
     def sync(self):
         check(_lib.lib().gr_engine_sync(self._h))
@@ -404,8 +413,8 @@ class System:
         return perm, offset, j, image, shifts
 
     def compute(self, types, positions, cell, pbc, energies=False, uq=False, energy_only=False):
-        if uq:
-            raise ValueError("the model has no UQ head")
+        """energy, forces [n, 3], virial [6], energies [n]; with `uq` also gamma, atomic_sigma, gmm_cluster [n] of the
+        model's UQ head (ValueError when the model has none that can be evaluated)."""
         types = as_array(types, np.int32)
         pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
         cell = np.ascontiguousarray(cell, dtype=np.float64).reshape(3, 3)
@@ -420,7 +429,7 @@ class System:
         forces = None if energy_only else np.empty((n, 3))
         virial = None if energy_only else np.empty(6)
         eat = np.empty(n) if energies else None
-        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (FLAG_UQ if uq else 0)
         check(_lib.lib().gr_system_compute(self._h, n, ptr(types), ptr(pos), ptr(cell), ptr(pb), flags, C.byref(e),
                                       ptr(forces) if forces is not None else None, ptr(virial) if virial is not None else None,
                                       ptr(eat) if eat is not None else None))
@@ -429,6 +438,10 @@ class System:
             res["forces"], res["virial"] = forces, virial
         if energies:
             res["energies"] = eat
+        if uq:
+            g, sg, cl = np.empty(n), np.empty(n), np.empty(n)
+            check(_lib.lib().gr_system_fetch_uq(self._h, ptr(g), ptr(sg), ptr(cl)))
+            res["gamma"], res["atomic_sigma"], res["gmm_cluster"] = g, sg, cl
         return res
 
 
@@ -449,7 +462,7 @@ class Batch:
     def compute(self, natoms, types, positions, cells, pbc, energies=False, uq=False, energy_only=False,
                 max_nall=1 << 21, dispersion_parts=False):
         if uq:
-            raise ValueError("the model has no UQ head")
+            raise ValueError("the UQ head is evaluated per structure (System.compute(uq=True)), not for batches")
         natoms = np.asarray(natoms, dtype=np.int32)
         types = as_array(types, np.int32)
         pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
@@ -498,7 +511,7 @@ class Batch:
         device; positions, forces and energies never visit the host.  `max_nall`: atoms per engine pass (whole
         structures, at least one per pass); `passes` holds the number of passes made."""
         if gamma is not None or atomic_sigma is not None or gmm_cluster is not None:
-            raise ValueError("the model has no UQ head")
+            raise ValueError("the UQ head is evaluated per structure (System.compute(uq=True)), not for batches: no UQ head here")
         natoms = np.ascontiguousarray(natoms, dtype=np.int32)
         cells = np.ascontiguousarray(cells, dtype=np.float64).reshape(-1, 3, 3)
         pb = np.ascontiguousarray(np.asarray(pbc, dtype=bool).reshape(-1, 3), dtype=np.uint8)

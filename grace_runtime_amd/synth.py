@@ -311,6 +311,36 @@ def random_model_1l(*, lmax=4, n_elements=1, element_names=("W",), embedding_siz
     return d
 
 
+def add_uq_head_1l(d, *, rp_dim=12, max_clusters=3, seed=20260111):
+    """Adds a random uqv6 UQ head to a GRACE-1L model dict (the keys libgrace/src/uq_head.cpp:11-76 reads): random
+    projection R [d_basis, rp_dim] of the invariant basis (the collected functions of the rho reduce's sources times
+    their channels, libgrace/include/grace/uq.h:31-48), per element 1 .. max_clusters GMM clusters with centroids,
+    symmetric positive definite precision matrices and interpolation thresholds over the rp_dim + 2 features."""
+    rng = np.random.default_rng(seed)
+    i64 = lambda v: np.array([v], dtype=np.int64)
+    srcs = [k for k in ("A", "AA", "AAA", "AAAA") if f"rho_collect_ind_{k}" in d]
+    d_basis = sum(int(d[f"rho_n_in_{k}"][0]) * len(d[f"rho_collect_ind_{k}"]) for k in srcs)
+    E, K, D = int(d["n_elements"][0]), max_clusters, rp_dim + 2
+    d["uq_schema_version"] = i64(6)
+    d["uq_n_elements"] = i64(E)
+    d["uq_max_clusters"] = i64(K)
+    d["uq_rp_dim"] = i64(rp_dim)
+    d["uq_feature_dim"] = i64(D)
+    d["uq_rp_normalize"] = i64(1)
+    d["uq_rp_add_density_channel"] = i64(1)
+    d["uq_rp_density_scale"] = np.array([1.0])
+    d["uq_feature_transform"] = i64(0)
+    d["uq_rp_matrix"] = rng.standard_normal((d_basis, rp_dim)) / math.sqrt(rp_dim)
+    cen = rng.standard_normal((E, K, D)) * 0.4
+    cen[:, :, rp_dim:] = rng.normal(1.0, 1.0, (E, K, 2))
+    d["uq_centroids"] = cen
+    a = rng.standard_normal((E, K, D, D))
+    d["uq_inv_cov"] = a @ np.swapaxes(a, -1, -2) / D + np.eye(D)
+    d["uq_n_clusters"] = rng.integers(1, K + 1, size=E).astype(np.int32)
+    d["uq_interp_thresholds"] = rng.uniform(0.5, 3.0, (E, K))
+    return d
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # GRACE-2L: structure arrays and random models
 # ---------------------------------------------------------------------------------------------------------------

@@ -18,6 +18,7 @@ Every function cites the reference file:line it follows (paths relative to the r
 * bond force, virial ............................ libgrace/include/grace/fused_cpu.h:1027-1050 (bond_force),
                                                   libgrace/src/fused_1l.cpp:46-51,351-371
 * dead AAAA stage of max_order-3 files .......... libgrace/src/max_order3.h:84-134 (here: the stage is skipped)
+* UQ head (uqv6: basis, projection, GMM) ........ libgrace/include/grace/fused_cpu.h:1275-1412, src/fused_1l.cpp:594-636
 
 The reference evaluates the network in fp32 with cubic-Hermite tables of the radial MLP; this restatement evaluates
 the same formulas directly in fp64 (no tables), which is what the reference's own TensorFlow fp64 goldens
@@ -27,6 +28,9 @@ Pinning status (see tests/test_oracle_*.py):
 * GRACE-1L end to end (radial basis, MLP, SH, A, FC, CG product, reduce, readout, forces, virial): pinned by the
   TF-fp64 goldens of grace_1l_order3 / legacy_1l_order3 on W54, WMo54, W2tri, by finite differences of E, and by the
   compiled reference (oracle/_ref) for the AAAA stage (grace_1l_w48) and the synthetic benchmark models.
+* UQ head of GRACE-1L (gamma, sigma, cluster): no fixture of the reference carries a UQ head; pinned by the compiled
+  reference on generated heads (its projection runs in fp32: gamma to 1e-4 relative) and by a brute-force restatement
+  of the GMM in the test.
 * GRACE-2L: see grace_oracle_2l.py.
 """
 from __future__ import annotations
@@ -293,6 +297,48 @@ class Model1L:
         self.shift = np.asarray(d["shift_values"], dtype=np.float64).ravel() if "shift_values" in d \
             else np.zeros(self.n_elements)
         self.out_scale = float(_scalar(d, "output_scale", 1.0))
+        self.has_uq = int(_scalar(d, "uq_schema_version", 0)) == 6
+        if self.has_uq:                                     # the uqv6 head: libgrace/src/uq_head.cpp:11-76
+            self.uq_rp = int(_scalar(d, "uq_rp_dim"))
+            self.uq_D = int(_scalar(d, "uq_feature_dim"))
+            self.uq_K = int(_scalar(d, "uq_max_clusters"))
+            self.uq_scale = float(_scalar(d, "uq_rp_density_scale", 1.0))
+            self.uq_R = np.asarray(d["uq_rp_matrix"], dtype=np.float64).reshape(-1, self.uq_rp)
+            self.uq_cen = np.asarray(d["uq_centroids"], dtype=np.float64).reshape(self.n_elements, self.uq_K, self.uq_D)
+            self.uq_icov = np.asarray(d["uq_inv_cov"], dtype=np.float64).reshape(self.n_elements, self.uq_K, self.uq_D, self.uq_D)
+            self.uq_ncl = np.asarray(d["uq_n_clusters"]).astype(np.int64).ravel()
+            self.uq_thr = np.asarray(d["uq_interp_thresholds"], dtype=np.float64).reshape(self.n_elements, self.uq_K)
+
+    def uq_features(self, t):
+        """phi [atoms, rp_dim + n_density] = concat((B / |B|) R, log |B| density_scale ...)."""
+        parts = []
+        for src in ["A", "AA", "AAA"] + (["AAAA"] if self.order4 else []):
+            X = t[src][:, self.red[src].ci, :]                                     # [a, c, n]
+            parts.append(np.transpose(X, (0, 2, 1)).reshape(X.shape[0], -1))
+        B = np.concatenate(parts, axis=1)
+        nrm = np.sqrt((B * B).sum(1))
+        f = np.empty((B.shape[0], self.uq_D))
+        f[:, :self.uq_rp] = (B @ self.uq_R) / (nrm + 1.0e-12)[:, None]
+        f[:, self.uq_rp:] = (np.log(nrm + 1.0e-12) * self.uq_scale)[:, None]
+        return f
+
+    def uq(self, mu, t):
+        """gamma, sigma, cluster of every atom from the forward tensors (uqv6, gamma only).
+        Basis: per source of the rho reduce, X_s[ci_s[c]][n] flattened n-outer, c-inner (fused_cpu.h:1290-1312,
+        libgrace/include/grace/uq.h:1-9); projection, normalisation, log-norm density channels, nearest centroid,
+        Mahalanobis distance: fused_cpu.h:1375-1412, src/fused_1l.cpp:616-636."""
+        f = self.uq_features(t)
+        na = f.shape[0]
+        gamma, sigma, cluster = np.zeros(na), np.zeros(na), np.zeros(na)
+        for a in range(na):
+            m = mu[a]
+            d2 = ((f[a][None, :] - self.uq_cen[m, :self.uq_ncl[m]]) ** 2).sum(1)
+            k = int(np.argmin(d2))                                                 # the first of equal distances
+            dl = f[a] - self.uq_cen[m, k]
+            sigma[a] = np.sqrt(dl @ self.uq_icov[m, k] @ dl + 1.0e-8)
+            gamma[a] = sigma[a] / max(self.uq_thr[m, k], 1.0e-10)
+            cluster[a] = k
+        return gamma, sigma, cluster
 
     # ---- per-atom dense chain -------------------------------------------------------------------------------
     def dense_forward(self, mu, A):
@@ -386,7 +432,7 @@ class ZeroBondError(ValueError):
     """bonds.h:49-62: two atoms at the same position."""
 
 
-def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=True):
+def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=True, uq=False):
     """One GRACE-1L energy + forces + virial call on a CSR bond list.
 
     mu[n]      model element of every atom (all mapped)
@@ -404,6 +450,8 @@ def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=Tru
     energies = np.zeros(n)
     forces = np.zeros((n, 3))
     virial = np.zeros(6)
+    uqv = [np.zeros(n), np.zeros(n), np.zeros(n)] if uq else None
+    feats = np.zeros((n, model.uq_D)) if uq else None
     for a0 in range(0, n, chunk):
         a1 = min(n, a0 + chunk)
         na = a1 - a0
@@ -432,6 +480,10 @@ def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=Tru
         rho, t = model.dense_forward(mu[a0:a1], A)
         E, grho = model.energy_atoms(mu[a0:a1], rho)
         energies[a0:a1] = E
+        if uq:
+            for dst, val in zip(uqv, model.uq(mu[a0:a1], t)):
+                dst[a0:a1] = val
+            feats[a0:a1] = model.uq_features(t)
         if not want_forces:
             continue
         gA = model.dense_backward(mu[a0:a1], t, grho)
@@ -452,7 +504,10 @@ def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=Tru
         dl = -rh * r[:, None]                                                    # src/fused_1l.cpp:46-51
         virial += np.array([(dl[:, 0] * fv[:, 0]).sum(), (dl[:, 1] * fv[:, 1]).sum(), (dl[:, 2] * fv[:, 2]).sum(),
                             (dl[:, 0] * fv[:, 1]).sum(), (dl[:, 0] * fv[:, 2]).sum(), (dl[:, 1] * fv[:, 2]).sum()])
-    return {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial}
+    out = {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial}
+    if uq:
+        out.update(gamma=uqv[0], atomic_sigma=uqv[1], gmm_cluster=uqv[2], uq_features=feats)
+    return out
 
 
 def virial_to_stress(virial, volume):

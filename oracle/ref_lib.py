@@ -54,6 +54,7 @@ def _load():
     L.ref_cutoff.restype = C.c_double
     L.ref_cutoff.argtypes = [C.c_void_p, C.c_int, C.c_int]
     L.ref_compute.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 7 + [C.c_int, C.c_int] + [C.c_void_p] * 4
+    L.ref_compute_uq.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 7 + [C.c_int] + [C.c_void_p] * 4
     L.ref_close.argtypes = [C.c_void_p]
     L.ref_nl_build.restype = C.c_void_p
     L.ref_nl_build.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_double, C.c_int]
@@ -108,6 +109,21 @@ class RefModel:
         if rc:
             raise RuntimeError(self._L.ref_last_error().decode())
         return {"energy": e.value, "energies": eat, "forces": f, "virial": v}
+
+    def compute_uq(self, types, offset, j, rij, nthreads=1):
+        """GRACE-1L UQ head of the reference (forward only): energy, gamma, atomic_sigma, gmm_cluster per atom."""
+        types = np.ascontiguousarray(types, dtype=np.int32)
+        offset = np.ascontiguousarray(offset, dtype=np.int64)
+        j = np.ascontiguousarray(j, dtype=np.int32)
+        rij = np.ascontiguousarray(rij, dtype=np.float64)
+        n = types.size
+        e = C.c_double(0.0)
+        g, sg, cl = np.zeros(n), np.zeros(n), np.zeros(n)
+        rc = self._L.ref_compute_uq(self._h, n, _p(types), _p(offset), _p(j), _p(rij), None, None, None, int(nthreads),
+                                    C.addressof(e), _p(g), _p(sg), _p(cl))
+        if rc:
+            raise RuntimeError(self._L.ref_last_error().decode())
+        return {"energy": e.value, "gamma": g, "atomic_sigma": sg, "gmm_cluster": cl}
 
     def close(self):
         if self._h:

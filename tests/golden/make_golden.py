@@ -71,6 +71,20 @@ def main():
         for k in ("energy", "energies", "forces", "virial"):
             out[f"{tag}/{k}"] = np.asarray(r[k])
         print(tag, "E", r["energy"], "max|F|", np.abs(r["forces"]).max())
+    # the UQ head (generated: no fixture of the reference carries one) through the compiled reference, forward only
+    for model, struct in cases.UQ_CASES:
+        if f"uq/{model}/{struct}/gamma" in out:
+            continue
+        path = cases.write_model(model, tmp)
+        pos, cell, pbc, types = cases.STRUCTURES[struct]()
+        nl = ref_lib.neighbor_search(pos, cell, pbc, 5.0, 2)
+        rij = cases.bond_vectors(pos, nl["perm"], nl["offset"], nl["j"], nl["image"], nl["shifts"])
+        r = ref_lib.RefModel(path, [0, 1]).compute_uq(types[nl["perm"]], nl["offset"], nl["j"], rij, nthreads=2)
+        tag = f"uq/{model}/{struct}"
+        for k in ("gamma", "atomic_sigma", "gmm_cluster"):
+            out[f"{tag}/{k}"] = np.asarray(r[k])
+        out[f"{tag}/perm"] = nl["perm"]
+        print(tag, "gamma", r["gamma"].min(), r["gamma"].max(), "clusters", np.unique(r["gmm_cluster"]))
     np.savez(target, **out)
 
 

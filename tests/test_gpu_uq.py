@@ -1,0 +1,83 @@
+"""The UQ head of GRACE-1L on the GPU (k_uq through the C ABI) against the CPU oracle: gamma and sigma to 1e-9 relative in
+fp64 (1e-4 with the fp32 network), the cluster index exactly.  Needs an MI355X: run with -m gpu."""
+import os
+
+import numpy as np
+import pytest
+
+import cases
+from grace_runtime_amd import kk
+from oracle import grace_oracle as go
+
+pytestmark = pytest.mark.gpu
+
+
+def _bonds(struct, rc=5.0):
+    pos, cell, pbc, types = cases.STRUCTURES[struct]()
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, rc)
+    x, t = pos[perm], types[perm]
+    rij = x[j] - np.repeat(x, np.diff(offset), axis=0) + shifts[image]
+    return t, offset, j, rij
+
+
+@pytest.mark.parametrize("precision,tol", [(64, 1e-9), (32, 1e-4)])
+@pytest.mark.parametrize("struct", ["alloy54", "triclinic"])
+def test_uq_matches_oracle(model_dir, struct, precision, tol):
+    path = os.path.join(model_dir, "uq2.npz")
+    eng = kk.Engine(kk.Model(path), ["Mo", "W"], precision)
+    t, offset, j, rij = _bonds(struct)
+    ref = go.compute_1l(go.Model1L(path), t - 1, offset, j, rij, uq=True)
+    eng.upload(t, offset, j, rij)
+    eng.run(uq=True)
+    out, uq = eng.fetch(), eng.fetch_uq()
+    if precision == 64:
+        assert np.array_equal(uq["gmm_cluster"], ref["gmm_cluster"])
+        assert abs(out["energy"] - ref["energy"]) < 1e-9 and np.abs(out["forces"] - ref["forces"]).max() < 1e-9
+    else:
+        far = ref["atomic_sigma"] > 1e-3          # the atom that sits ON a centroid: its sigma is rounding noise in fp32
+        assert np.array_equal(uq["gmm_cluster"][far], ref["gmm_cluster"][far])
+        uq = {k: v[far] for k, v in uq.items()}
+        ref = {k: ref[k][far] for k in ("gamma", "atomic_sigma")}
+    assert np.abs(uq["gamma"] / ref["gamma"] - 1).max() < tol
+    assert np.abs(uq["atomic_sigma"] / ref["atomic_sigma"] - 1).max() < tol
+    # forward only: the same values without the reverse pass
+    eng.run(uq=True, energy_only=True)
+    assert np.array_equal(eng.fetch_uq()["gamma"], eng.fetch_uq()["gamma"])
+    assert np.abs(eng.fetch_uq()["gamma"] / ref["gamma"] - 1).max() < tol if precision == 64 else True
+
+
+def test_calculator_level_call_returns_uq_in_the_callers_order(model_dir):
+    path = os.path.join(model_dir, "uq2.npz")
+    model = kk.Model(path)
+    pos, cell, pbc, types = cases.structure_alloy54()
+    s = kk.System(model, ["Mo", "W"], skin=0.3)
+    out = s.compute(types, pos, cell, pbc, uq=True, energies=True)
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 5.0)
+    x, t = pos[perm], types[perm]
+    rij = x[j] - np.repeat(x, np.diff(offset), axis=0) + shifts[image]
+    ref = go.compute_1l(go.Model1L(path), t - 1, offset, j, rij, uq=True)
+    for k in ("gamma", "atomic_sigma", "gmm_cluster"):
+        want = np.empty(len(t))
+        want[perm] = ref[k]
+        assert np.abs(out[k] / want - 1).max() < 1e-9 if k != "gmm_cluster" else np.array_equal(out[k], want)
+    # a second call on the kept list (positions moved within the skin)
+    p2 = pos + np.random.default_rng(2).uniform(-0.05, 0.05, pos.shape)
+    o2 = s.compute(types, p2, cell, pbc, uq=True)
+    fresh = kk.System(model, ["Mo", "W"], skin=0.0).compute(types, p2, cell, pbc, uq=True)
+    assert s.rebuilds == 1 and not np.array_equal(o2["gamma"], out["gamma"])
+    assert np.abs(o2["gamma"] / fresh["gamma"] - 1).max() < 1e-9 and np.array_equal(o2["gmm_cluster"], fresh["gmm_cluster"])
+
+
+def test_uq_errors(model_dir):
+    plain = kk.Engine(kk.Model(os.path.join(model_dir, "mix2.npz")), ["Mo", "W"], 64)
+    t, offset, j, rij = _bonds("alloy54")
+    plain.upload(t, offset, j, rij)
+    with pytest.raises(ValueError, match="no usable UQ head"):
+        plain.run(uq=True)
+    plain.run()
+    with pytest.raises(RuntimeError, match="needs a run with the UQ flag"):
+        plain.fetch_uq()
+    two = kk.System(kk.Model(os.path.join(model_dir, "l2mix.npz")), ["Mo", "W"])
+    pos, cell, pbc, types = cases.structure_alloy54()
+    with pytest.raises(ValueError, match="no usable UQ head"):
+        two.compute(types, pos, cell, pbc, uq=True)

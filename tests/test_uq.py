@@ -1,0 +1,129 @@
+"""The UQ head (uqv6, gamma only) of GRACE-1L: the CPU oracle against the compiled reference and against what the
+definition fixes, and the loader's checks (no GPU needed).
+
+No fixture of the reference carries a UQ head, so the head is a generated one (tests/cases.py model_uq2).  The compiled
+reference projects the basis in fp32 (libgrace/include/grace/fused_cpu.h:1275-1283: gamma within ~1e-5 of an fp64
+projection): 1e-4 relative on gamma and sigma, the cluster index exactly."""
+import os
+
+import numpy as np
+import pytest
+
+import cases
+from grace_runtime_amd import kk
+from oracle import grace_oracle as go
+from oracle import ref_lib
+
+
+def _bonds(struct, rc=5.0):
+    pos, cell, pbc, types = cases.STRUCTURES[struct]()
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, rc)
+    x, t = pos[perm], types[perm]
+    rij = x[j] - np.repeat(x, np.diff(offset), axis=0) + shifts[image]
+    return t, offset, j, rij
+
+
+@pytest.fixture(scope="module")
+def uq_model(model_dir):
+    return os.path.join(model_dir, "uq2.npz")
+
+
+@pytest.mark.skipif(not ref_lib.available(), reason="compiled reference not built")
+@pytest.mark.parametrize("struct", ["alloy54", "triclinic"])
+def test_oracle_matches_compiled_reference(uq_model, struct):
+    t, offset, j, rij = _bonds(struct)
+    o = go.compute_1l(go.Model1L(uq_model), t - 1, offset, j, rij, want_forces=False, uq=True)
+    r = ref_lib.RefModel(uq_model, [0, 1]).compute_uq(t, offset, j, rij)
+    assert np.array_equal(o["gmm_cluster"], r["gmm_cluster"])
+    if struct == "alloy54":
+        assert len(np.unique(o["gmm_cluster"][t == 1])) == 3 and len(np.unique(o["gmm_cluster"][t == 2])) == 2
+    assert np.abs(o["gamma"] / r["gamma"] - 1).max() < 1e-4
+    assert np.abs(o["atomic_sigma"] / r["atomic_sigma"] - 1).max() < 1e-4
+
+
+@pytest.mark.parametrize("model,struct", cases.UQ_CASES)
+def test_oracle_matches_golden_of_the_compiled_reference(model_dir, gold, model, struct):
+    """the committed outputs of the compiled reference (tests/golden/make_golden.py), for machines without it"""
+    t, offset, j, rij = _bonds(struct)
+    o = go.compute_1l(go.Model1L(os.path.join(model_dir, model + ".npz")), t - 1, offset, j, rij, want_forces=False, uq=True)
+    tag = f"uq/{model}/{struct}"
+    assert np.array_equal(o["gmm_cluster"], gold[tag + "/gmm_cluster"])
+    assert np.abs(o["gamma"] / gold[tag + "/gamma"] - 1).max() < 1e-4
+    assert np.abs(o["atomic_sigma"] / gold[tag + "/atomic_sigma"] - 1).max() < 1e-4
+
+
+def test_what_the_definition_fixes(uq_model):
+    """the atom whose feature vector IS a centroid has sigma = sqrt(1e-8) and gamma = sigma / threshold; the features are
+    invariants of the neighbourhood: a rotated structure gives the same gamma; gamma = sigma / threshold everywhere"""
+    m = go.Model1L(uq_model)
+    t, offset, j, rij = _bonds("alloy54")
+    o = go.compute_1l(m, t - 1, offset, j, rij, want_forces=False, uq=True)
+    thr = m.uq_thr[t - 1, o["gmm_cluster"].astype(int)]
+    assert np.abs(o["gamma"] * thr - o["atomic_sigma"]).max() < 1e-12
+    assert abs(o["atomic_sigma"].min() - 1e-4) < 1e-9 and (o["atomic_sigma"] < 2e-4).sum() == 1
+    # brute force over all clusters of the element: the chosen one is the nearest in the Euclidean sense
+    f = o["uq_features"]
+    for a in range(len(t)):
+        e = t[a] - 1
+        d2 = [((f[a] - m.uq_cen[e, k]) ** 2).sum() for k in range(m.uq_ncl[e])]
+        assert int(o["gmm_cluster"][a]) == int(np.argmin(d2))
+        dl = f[a] - m.uq_cen[e, int(np.argmin(d2))]
+        assert abs(o["atomic_sigma"][a] ** 2 - (sum(dl[p] * m.uq_icov[e, int(np.argmin(d2)), p, q] * dl[q] for p in range(len(dl))
+                                                   for q in range(len(dl))) + 1e-8)) < 1e-10
+    assert np.abs(np.linalg.norm(f[:, :m.uq_rp], axis=1)).max() < np.linalg.norm(m.uq_R, 2) + 1e-9     # |B R| / |B| <= |R|
+    assert np.abs(f[:, m.uq_rp] - f[:, m.uq_rp + 1]).max() == 0.0                                     # one basis block: equal channels
+    rot = np.linalg.qr(np.random.default_rng(4).standard_normal((3, 3)))[0]
+    o2 = go.compute_1l(m, t - 1, offset, j, rij @ rot.T, want_forces=False, uq=True)
+    assert np.abs(o2["gamma"] - o["gamma"]).max() < 1e-9 * o["gamma"].max()
+
+
+def _mutated(tmp_path, edit, name="uq2"):
+    d = cases.MODELS[name]()
+    edit(d)
+    p = str(tmp_path / "m.npz")
+    np.savez(p, **{k: v for k, v in d.items() if not k.startswith("_")})
+    return p
+
+
+BAD_UQ = [
+    (lambda d: d.update(uq_schema_version=np.array([5])), "UQ schema v5 unsupported"),
+    (lambda d: d.update(uq_rp_matrix=d["uq_rp_matrix"][:-1]), "rows, the model's invariant basis has"),
+    (lambda d: d.update(uq_rp_matrix=np.ascontiguousarray(d["uq_rp_matrix"].T)), "uq_rp_matrix"),
+    (lambda d: d.update(uq_n_clusters=np.array([3, 0], np.int32)), "element index 1 has no GMM clusters"),
+    (lambda d: d.update(uq_n_clusters=np.array([3, 4], np.int32)), "more than uq_max_clusters = 3"),
+    (lambda d: d.update(uq_centroids=d["uq_centroids"][:, :2]), "uq_centroids"),
+    (lambda d: d.update(uq_inv_cov=d["uq_inv_cov"][:, :, :, :-1]), "uq_inv_cov"),
+    (lambda d: d.update(uq_rp_normalize=np.array([0])), "schema v6 expects normalize=1"),
+    (lambda d: d.update(uq_feature_dim=np.array([15]), uq_centroids=np.zeros((2, 3, 15)), uq_inv_cov=np.zeros((2, 3, 15, 15))),
+     "3 density channels, expected 2"),
+    (lambda d: d.update(uq_n_elements=np.array([3])), "uq_n_elements"),
+    (lambda d: d.pop("uq_interp_thresholds"), "uq_interp_thresholds"),
+]
+
+
+@pytest.mark.parametrize("edit,msg", BAD_UQ)
+def test_a_broken_head_is_reported_by_validate_uq_and_leaves_the_model_usable(tmp_path, edit, msg):
+    m = kk.Model(_mutated(tmp_path, edit))                     # loads (libgrace/src/model_1l.cpp:216-271)
+    assert m.has_uq and m.layers == 1
+    with pytest.raises(ValueError, match=msg):
+        m.validate_uq()
+
+
+def test_heads_that_validate_and_models_without(tmp_path, uq_model, model_dir):
+    m = kk.Model(uq_model)
+    assert m.has_uq
+    m.validate_uq()
+    plain = kk.Model(os.path.join(model_dir, "mix2.npz"))
+    assert not plain.has_uq
+    with pytest.raises(ValueError, match="no UQ head"):
+        plain.validate_uq()
+    with pytest.raises(ValueError, match="GRACE-1L models only"):
+        kk.Model(os.path.join(model_dir, "l2mix.npz")).validate_uq()
+    o3 = kk.Model(_mutated(tmp_path, lambda d: synth_uq(d), "cut2"))          # max_order 3: refused (tests/test_driver.cpp:406-415)
+    with pytest.raises(ValueError, match="max_order 3"):
+        o3.validate_uq()
+
+
+def synth_uq(d):
+    from grace_runtime_amd import synth
+    synth.add_uq_head_1l(d, rp_dim=6, max_clusters=2)
