@@ -254,15 +254,16 @@ int gr_engine_fetch_uq(gr_engine *e, double *gamma, double *sigma, double *clust
   });
 }
 
-int gr_model_has_uq(const gr_model *m) { return m && m->m1 && m->m1->uq.has_uq ? 1 : 0; }
+int gr_model_has_uq(const gr_model *m) { return m && ((m->m1 && m->m1->uq.has_uq) || (m->m2 && m->m2->uq.has_uq)) ? 1 : 0; }
 
 int gr_model_validate_uq(const gr_model *m)
 {
   return guarded([&] {
     if (!m) throw grhip::InvalidArgument("null model");
-    if (!m->m1) throw grhip::InvalidArgument("the UQ head is evaluated for GRACE-1L models only");
+    if (!m->m1 && !m->m2) throw grhip::InvalidArgument("the UQ head is evaluated for GRACE-1L and GRACE-2L models only");
     try {
-      m->m1->validate_uq();
+      if (m->m1) m->m1->validate_uq();
+      else m->m2->validate_uq();
     } catch (const grhip::Error &e) {
       throw grhip::InvalidArgument(e.what());    // python/kk/kk_core.cpp: std::invalid_argument (unsupported model)
     }

@@ -186,9 +186,11 @@ template<class T> void Engine1L<T>::build()
         uq_.nin[s] = rw[s]->n_in;
         uq_.nc[s] = (int) rw[s]->collect_ind.size();
         uq_.off[s] = off;
+        uq_.blk[s] = 0;
         off += uq_.nin[s] * uq_.nc[s];
       }
       uq_.d_basis = off;
+      uq_.nblk = 1;
       uq_.rp = m.uq.rp_dim; uq_.D = m.uq.feature_dim; uq_.K = m.uq.max_clusters;
       uq_.density_scale = m.uq.density_scale;
       upload_vec(uqR_, m.uq.rp_matrix); upload_vec(uqCen_, m.uq.centroids); upload_vec(uqIcov_, m.uq.inv_cov);

@@ -52,6 +52,8 @@ template<class T> class Engine2L final : public EngineBase {
   DevRadial<T> radR_, radR1_;
   Chain<T> c1_, c2_;
   DevReduce<T> redrho_, redI2_;
+  UqDev<T> uq_{};             // UQ head: blocks [I2 (layer 2), rho (layer 1)]
+  DevBuf uqR_, uqCen_, uqIcov_, uqNcl_, uqThr_, uqCi_[kUqMaxSrc];
   std::vector<std::unique_ptr<DevReduce<T>>> redI1_;    // one per output function of I1
   DevBuf WI_, WIT_, WB_, WBT_;
   DevJobs<T> jI_, jIb_, jB_, jBb_;
@@ -206,6 +208,42 @@ template<class T> void Engine2L<T>::build()
   };
   redrho_.build(sources(m.rho_red, c1_, C1P_, false), nel_, nrho_, -1, nrho_, 0, drow_);
   redI2_.build(sources(m.I2_red, c2_, C2P_, false), nel_, nrho_, -1, nrho_, 0, drow_);
+  // ---- UQ head: a head that does not validate leaves the model usable without UQ (libgrace/src/model_2l.cpp:404-478)
+  if (m.uq.has_uq) {
+    try {
+      m.validate_uq();
+      if (m.uq.rp_dim > 256 || m.uq.feature_dim > 256) throw Error("GRACE-2L UQ: feature widths above 256 are not supported");
+      int off = 0, q = 0;
+      for (int b = 0; b < 2; b++) {    // block 0: I2 over (B, BB, BBB, BBBB); block 1: rho over (A, AA, AAA, AAAA)
+        const ReduceEq *r = b == 0 ? m.I2_red : m.rho_red;
+        const Chain<T> &c = b == 0 ? c2_ : c1_;
+        for (int s = 0; s < ns; s++, q++) {
+          upload_vec(uqCi_[q], r[s].collect_ind);
+          uq_.ci[q] = uqCi_[q].template as<int>();
+          uq_.nfun[q] = c.nfun(s);
+          uq_.cpad[q] = b == 0 ? C2P_ : C1P_;
+          uq_.nin[q] = r[s].n_in;
+          uq_.nc[q] = (int) r[s].collect_ind.size();
+          uq_.off[q] = off;
+          uq_.blk[q] = b;
+          off += uq_.nin[q] * uq_.nc[q];
+        }
+      }
+      uq_.nsrc = q; uq_.nblk = 2; uq_.d_basis = off;
+      uq_.rp = m.uq.rp_dim; uq_.D = m.uq.feature_dim; uq_.K = m.uq.max_clusters;
+      uq_.density_scale = m.uq.density_scale;
+      upload_vec(uqR_, m.uq.rp_matrix); upload_vec(uqCen_, m.uq.centroids); upload_vec(uqIcov_, m.uq.inv_cov);
+      upload_vec(uqNcl_, m.uq.n_clusters); upload_vec(uqThr_, m.uq.interp_thresholds);
+      uq_.R = uqR_.template as<double>(); uq_.cen = uqCen_.template as<double>(); uq_.icov = uqIcov_.template as<double>();
+      uq_.ncl = uqNcl_.template as<int>(); uq_.thr = uqThr_.template as<double>();
+      if ((size_t) (uq_.d_basis + 4 * uq_.rp + 2 * uq_.D) * sizeof(double) > 150 * 1024) throw Error("GRACE-2L UQ: the basis does not fit the kernel's LDS");
+      has_uq_head_ = true;
+    } catch (const std::exception &e) {
+      uq_why_ = e.what();
+    }
+  } else {
+    uq_why_ = "the model file carries none";
+  }
   for (int fo = 0; fo < nI1_; fo++) {
     redI1_.emplace_back(new DevReduce<T>());
     redI1_.back()->build(sources(m.I1_red, c1_, C1P_, true), nel_, m.I1_n_out, fo, nI1_ * PI1_, fo * PI1_, drow_);
@@ -531,6 +569,20 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   I2_.ensure(na * nrho_ * sizeof(double));
   gI2_.ensure(na * nrho_ * sizeof(double));
   stage("reduce_I2", [&] { reduce_fwd(redI2_, c2_.kb, c2_, B, I2_.as<double>()); });
+  if (fl.uq) {
+    uq_gamma_.ensure(na * sizeof(double)); uq_sigma_.ensure(na * sizeof(double)); uq_cluster_.ensure(na * sizeof(double));
+    stage("uq", [&] {
+      UqDev<T> u = uq_;
+      for (int q = 0; q < u.nsrc; q++) u.X[q] = u.blk[q] == 0 ? c2_.src(q, B) : c1_.src(q - u.nsrc / 2, A);
+      const size_t lds = (size_t) (u.d_basis + 4 * u.rp + 2 * u.D) * sizeof(double);
+      auto kern = k_uq<T>;
+      if (lds > 48 * 1024)
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+      hipLaunchKernelGGL(kern, dim3(n), dim3(256), lds, stream_, u, mu_.as<int>(), n, uq_gamma_.as<double>(), uq_sigma_.as<double>(),
+                         uq_cluster_.as<double>());
+    });
+    ran_uq_ = true;
+  }
   stage("energy_mlp", [&] {
     hipLaunchKernelGGL(k_energy_2l, dim3(n), dim3(64), (size_t) (2 * en_.nlay + 4) * en_.width * sizeof(double), stream_, en_, mu_.as<int>(), n, rho_.as<double>(), I2_.as<double>(), grho_.as<double>(),
                        gI2_.as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0, sid_ptr());

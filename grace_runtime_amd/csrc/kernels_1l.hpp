@@ -1123,11 +1123,13 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
 // ---------------------------------------------------------------------------------------------------------------
 // UQ head (uqv6, gamma only)
 // ---------------------------------------------------------------------------------------------------------------
+constexpr int kUqMaxSrc = 8, kUqMaxBlk = 2;
 template<class T> struct UqDev {
-  const T *X[4];              // per-atom tensors of the reduce's sources [atom][function][channel]
-  const int *ci[4];           // collected functions of each source
-  int nfun[4], cpad[4], nin[4], nc[4], off[4];    // functions per atom, padded / real channels, collected, first basis index
-  int nsrc, d_basis, rp, D, K;
+  const T *X[kUqMaxSrc];      // per-atom tensors of the reduces' sources [atom][function][channel]
+  const int *ci[kUqMaxSrc];   // collected functions of each source
+  int nfun[kUqMaxSrc], cpad[kUqMaxSrc], nin[kUqMaxSrc], nc[kUqMaxSrc], off[kUqMaxSrc];    // functions per atom, padded / real channels, collected, first basis index
+  int blk[kUqMaxSrc];         // invariant block of the source (1L: rho = 0; 2L: I2 = 0, rho = 1)
+  int nsrc, nblk, d_basis, rp, D, K;
   double density_scale;
   const double *R;            // [d_basis][rp]
   const double *cen;          // [nel][K][D]
@@ -1137,9 +1139,10 @@ template<class T> struct UqDev {
 };
 
 // gamma, sigma, cluster of one atom per block (libgrace/include/grace/fused_cpu.h:1290-1312 basis, :1375-1412 GMM;
-// libgrace/src/fused_1l.cpp:616-636): basis B = the collected functions of the rho reduce's sources, n-outer and
-// c-inner per source; phi = ((B / |B|) R, log |B| scale, ...); nearest centroid of the atom's element, Mahalanobis
-// distance over the cluster's threshold.  fp64 throughout.  block: 256 threads; dynamic LDS: d_basis + 4 rp + 2 D doubles.
+// libgrace/src/fused_1l.cpp:616-636, fused_2l.cpp:1156-1186): basis B = per invariant block the collected functions of
+// the reduce's sources, n-outer and c-inner per source; phi = ((B / |B|) R, log |B| scale, log |B_block| scale ...);
+// nearest centroid of the atom's element, Mahalanobis distance over the cluster's threshold.  fp64 throughout.
+// block: 256 threads; dynamic LDS: d_basis + 4 rp + 2 D doubles.
 template<class T>
 __global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natoms, double *gamma, double *sigma, double *cluster)
 {
@@ -1148,26 +1151,41 @@ __global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natom
   double *Zp = Bsh + U.d_basis;                             // [4][rp] partial projections
   double *f = Zp + 4 * U.rp;                                // [D]
   double *dl = f + U.D;                                     // [D]
-  __shared__ double wsum[4];
+  __shared__ double wsum[4], bsum[4][kUqMaxBlk];
   __shared__ int kstar;
   const int at = blockIdx.x, t = threadIdx.x, lane = t & 63, wave = t >> 6;
   if (at >= natoms) return;
-  // ---- basis and its norm
-  double n2 = 0.0;
+  // ---- basis and the norms of its blocks
+  double n2[kUqMaxBlk];
+#pragma unroll
+  for (int b = 0; b < kUqMaxBlk; b++) n2[b] = 0.0;
   for (int s = 0; s < U.nsrc; s++) {
     const T *x = U.X[s] + (long long) at * U.nfun[s] * U.cpad[s];
     const int w = U.nin[s] * U.nc[s];
+    double acc = 0.0;
     for (int r = t; r < w; r += 256) {
       const int n = r / U.nc[s], c = r % U.nc[s];
       const double v = (double) x[U.ci[s][c] * U.cpad[s] + n];
       Bsh[U.off[s] + r] = v;
-      n2 += v * v;
+      acc += v * v;
     }
+#pragma unroll
+    for (int b = 0; b < kUqMaxBlk; b++)
+      if (U.blk[s] == b) n2[b] += acc;
   }
-  for (int o = 32; o > 0; o >>= 1) n2 += __shfl_xor(n2, o, 64);
-  if (lane == 0) wsum[wave] = n2;
+#pragma unroll
+  for (int b = 0; b < kUqMaxBlk; b++) {
+    for (int o = 32; o > 0; o >>= 1) n2[b] += __shfl_xor(n2[b], o, 64);
+    if (lane == 0) bsum[wave][b] = n2[b];
+  }
   __syncthreads();
-  const double nrm = sqrt(wsum[0] + wsum[1] + wsum[2] + wsum[3]);
+  double nb2[kUqMaxBlk], tot = 0.0;
+#pragma unroll
+  for (int b = 0; b < kUqMaxBlk; b++) {
+    nb2[b] = bsum[0][b] + bsum[1][b] + bsum[2][b] + bsum[3][b];
+    tot += nb2[b];
+  }
+  const double nrm = sqrt(tot);
   // ---- projection Z = B R: column d = t mod rp, rows split over the 256 / rp (at most 4 used) thread groups
   {
     const int ng = 256 / U.rp > 4 ? 4 : 256 / U.rp, gq = t / U.rp, d = t % U.rp;
@@ -1182,8 +1200,13 @@ __global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natom
         double z = 0.0;
         for (int q = 0; q < ng; q++) z += Zp[q * U.rp + t];
         f[t] = z / (nrm + 1.0e-12);
-      } else {
-        f[t] = log(nrm + 1.0e-12) * U.density_scale;
+      } else {    // density channels: the whole basis, then its blocks (one block: the same norm again)
+        const int p = t - U.rp;
+        double dn = nrm;
+#pragma unroll
+        for (int b = 0; b < kUqMaxBlk; b++)
+          if (U.nblk > 1 && p == 1 + b) dn = sqrt(nb2[b]);
+        f[t] = log(dn + 1.0e-12) * U.density_scale;
       }
     }
     __syncthreads();

@@ -43,12 +43,35 @@ struct Model2L {
   int energy_mlp_activation = 1, radial_activation = 0;
   std::vector<double> shift_values;
   double output_scale = 1.0;
+  UqHead uq;    // the uqv6 UQ head: invariant blocks [I2 (B .. BBBB), rho (A .. AAAA)] (libgrace/src/model_2l.cpp:518-534)
   std::vector<std::string> element_names;
   static constexpr double rms_norm_eps = 1e-10;    // libgrace/include/grace/model_2l.h:156
 
   int nl() const { return lmax + 1; }
   int nlm() const { return (lmax + 1) * (lmax + 1); }
   int nsrc() const { return max_order == 4 ? 4 : 3; }
+  // widths of the two blocks of the UQ basis (libgrace/include/grace/uq.h:31-48)
+  int uq_block_width(const ReduceEq *r) const
+  {
+    int w = 0;
+    for (int s = 0; s < nsrc(); s++) w += r[s].n_in * (int) r[s].collect_ind.size();
+    return w;
+  }
+  // libgrace/src/model_2l.cpp:466-478, libgrace/src/uq.cpp:8-33
+  void validate_uq() const
+  {
+    if (!uq.has_uq) throw Error("GRACE-2L: the model has no UQ head");
+    if (max_order == 3) throw Error("GRACE-2L: UQ is not supported for max_order 3 models");
+    if (uq.schema != 6)
+      throw Error("GRACE-2L: UQ schema v" + std::to_string(uq.schema) + " unsupported (expects v6, uqv6 basis-RP normalize+density). Re-export the "
+                  "UQ artifacts at schema v6 with a current grace_utils.");
+    if (!uq.error.empty()) throw Error(uq.error);
+    const int total = uq_block_width(I2_red) + uq_block_width(rho_red);
+    if (total != uq.d_basis)
+      throw Error("GRACE-2L UQ: uq_rp_matrix has " + std::to_string(uq.d_basis) + " rows, the model's invariant basis has " + std::to_string(total) +
+                  "; re-export the UQ artifacts for this model");
+    if (uq.n_density != 3) throw Error("GRACE-2L UQ: " + std::to_string(uq.n_density) + " density channels, expected 3 (1 + basis blocks)");
+  }
   double pair_cutoff(int mu_i, int mu_j) const
   {
     if (mu_i < 0 || mu_j < 0) return 0.0;
@@ -289,6 +312,7 @@ struct Model2L {
     if (v.has("shift_values")) require_size("shift_values", shift_values, (size_t) n_elements);
     else shift_values.assign(n_elements, 0.0);
     output_scale = v.double_scalar("output_scale", 1.0);
+    uq.load(v, n_elements, "GRACE-2L/KK");
     element_names = v.names("element_names");
     if (v.has("element_names")) require_size("element_names", element_names, (size_t) n_elements);
   }

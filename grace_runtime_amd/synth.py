@@ -311,16 +311,20 @@ def random_model_1l(*, lmax=4, n_elements=1, element_names=("W",), embedding_siz
     return d
 
 
-def add_uq_head_1l(d, *, rp_dim=12, max_clusters=3, seed=20260111):
-    """Adds a random uqv6 UQ head to a GRACE-1L model dict (the keys libgrace/src/uq_head.cpp:11-76 reads): random
-    projection R [d_basis, rp_dim] of the invariant basis (the collected functions of the rho reduce's sources times
-    their channels, libgrace/include/grace/uq.h:31-48), per element 1 .. max_clusters GMM clusters with centroids,
-    symmetric positive definite precision matrices and interpolation thresholds over the rp_dim + 2 features."""
+def add_uq_head(d, blocks, *, rp_dim=12, max_clusters=3, seed=20260111):
+    """Adds a random uqv6 UQ head to a model dict (the keys libgrace/src/uq_head.cpp:11-76 reads): random projection
+    R [d_basis, rp_dim] of the invariant basis (per block, the collected functions of that reduce's sources times their
+    channels, libgrace/include/grace/uq.h:31-48), per element 1 .. max_clusters GMM clusters with centroids, symmetric
+    positive definite precision matrices and interpolation thresholds over the rp_dim + n_density features, n_density =
+    2 for one basis block and 1 + the number of blocks otherwise.  blocks: [(reduce prefix, source names)]."""
     rng = np.random.default_rng(seed)
     i64 = lambda v: np.array([v], dtype=np.int64)
-    srcs = [k for k in ("A", "AA", "AAA", "AAAA") if f"rho_collect_ind_{k}" in d]
-    d_basis = sum(int(d[f"rho_n_in_{k}"][0]) * len(d[f"rho_collect_ind_{k}"]) for k in srcs)
-    E, K, D = int(d["n_elements"][0]), max_clusters, rp_dim + 2
+    d_basis = 0
+    for pre, names in blocks:
+        srcs = [k for k in names if f"{pre}_collect_ind_{k}" in d]
+        d_basis += sum(int(np.asarray(d[f"{pre}_n_in_{k}"]).ravel()[0]) * len(d[f"{pre}_collect_ind_{k}"]) for k in srcs)
+    nd = 2 if len(blocks) == 1 else 1 + len(blocks)
+    E, K, D = int(np.asarray(d["n_elements"]).ravel()[0]), max_clusters, rp_dim + nd
     d["uq_schema_version"] = i64(6)
     d["uq_n_elements"] = i64(E)
     d["uq_max_clusters"] = i64(K)
@@ -332,13 +336,23 @@ def add_uq_head_1l(d, *, rp_dim=12, max_clusters=3, seed=20260111):
     d["uq_feature_transform"] = i64(0)
     d["uq_rp_matrix"] = rng.standard_normal((d_basis, rp_dim)) / math.sqrt(rp_dim)
     cen = rng.standard_normal((E, K, D)) * 0.4
-    cen[:, :, rp_dim:] = rng.normal(1.0, 1.0, (E, K, 2))
+    cen[:, :, rp_dim:] = rng.normal(1.0, 1.0, (E, K, nd))
     d["uq_centroids"] = cen
     a = rng.standard_normal((E, K, D, D))
     d["uq_inv_cov"] = a @ np.swapaxes(a, -1, -2) / D + np.eye(D)
     d["uq_n_clusters"] = rng.integers(1, K + 1, size=E).astype(np.int32)
     d["uq_interp_thresholds"] = rng.uniform(0.5, 3.0, (E, K))
     return d
+
+
+def add_uq_head_1l(d, **kw):
+    """GRACE-1L: one basis block, the sources of the rho reduce (libgrace/src/model_1l.cpp:216-271)"""
+    return add_uq_head(d, [("rho", ("A", "AA", "AAA", "AAAA"))], **kw)
+
+
+def add_uq_head_2l(d, **kw):
+    """GRACE-2L: blocks [I2 over B .. BBBB, rho over A .. AAAA] (libgrace/src/model_2l.cpp:404-478)"""
+    return add_uq_head(d, [("I2", ("B", "BB", "BBB", "BBBB")), ("rho", ("A", "AA", "AAA", "AAAA"))], **kw)
 
 
 # ---------------------------------------------------------------------------------------------------------------

@@ -15,11 +15,15 @@ Reference followed (paths relative to the reference checkout):
 * readout with the two RMSNorms .................. libgrace/src/fused_2l.cpp:548-615          (energy_atom)
 * layer 1 reverse ................................ libgrace/src/fused_2l.cpp:458-542          (layer1_backward)
 * phases P1 .. P5 ................................ libgrace/src/fused_2l.cpp:849-1099         (compute)
+* UQ head (uqv6, gamma only): keys, basis blocks .. libgrace/src/model_2l.cpp:404-478, src/fused_2l.cpp:1156-1186,
+  GMM ............................................ libgrace/include/grace/fused_cpu.h:1375-1412
 
 Pinning status: end to end (energy, per-atom energies, forces, stress) against the reference's TensorFlow fp64
 goldens of grace_2l_order3 / legacy_2l_order3 on W54, WMo54, W2tri (tests/fixtures/ref_tf/order3_tf.npz), by finite
 differences of the energy, and against the compiled reference (oracle/_ref) for models with the BBBB / AAAA stages and
-the synthetic benchmark models.
+the synthetic benchmark models.  UQ head (uq_features, uq): against the compiled reference on a generated head attached
+to the fixture model grace_2l_small (cluster indices exactly, gamma and sigma to 1e-4: its projection is fp32), live and
+as committed goldens, and by what the definition fixes (tests/test_uq.py).
 """
 from __future__ import annotations
 
@@ -121,6 +125,7 @@ class Model2L:
         self.yp_i = np.array([p[1] for p in pairs], dtype=np.int64)
         self.yp_l = np.floor(np.sqrt(self.yp_y + 1e-9)).astype(np.int64)
         self.yt_pair = np.array([pid[(int(y), int(i))] for y, i in lr], dtype=np.int64)
+        self.uq_setup(d)
         self.SYI = np.zeros((self.nYI, len(pairs)))                                 # YI[o] = sum_p SYI[o, p] YIp[p]
         np.add.at(self.SYI, (self.yi_o, self.yt_pair), self.yi_c * self.yi_inv)
         # readout
@@ -141,6 +146,53 @@ class Model2L:
         self.shift = np.asarray(d["shift_values"], dtype=np.float64).ravel() if "shift_values" in d \
             else np.zeros(self.n_elements)
         self.out_scale = float(_scalar(d, "output_scale", 1.0))
+
+    def uq_setup(self, d):
+        """the uqv6 UQ head (libgrace/src/model_2l.cpp:404-478): blocks [I2 over B .. BBBB, rho over A .. AAAA]"""
+        self.has_uq = int(_scalar(d, "uq_schema_version", 0)) == 6
+        if not self.has_uq:
+            return
+        ne = int(_scalar(d, "n_elements"))
+        self.uq_rp, self.uq_D, self.uq_K = int(_scalar(d, "uq_rp_dim")), int(_scalar(d, "uq_feature_dim")), int(_scalar(d, "uq_max_clusters"))
+        self.uq_scale = float(_scalar(d, "uq_rp_density_scale", 1.0))
+        self.uq_R = np.asarray(d["uq_rp_matrix"], dtype=np.float64).reshape(-1, self.uq_rp)
+        self.uq_cen = np.asarray(d["uq_centroids"], dtype=np.float64).reshape(ne, self.uq_K, self.uq_D)
+        self.uq_icov = np.asarray(d["uq_inv_cov"], dtype=np.float64).reshape(ne, self.uq_K, self.uq_D, self.uq_D)
+        self.uq_ncl = np.asarray(d["uq_n_clusters"]).astype(np.int64).ravel()
+        self.uq_thr = np.asarray(d["uq_interp_thresholds"], dtype=np.float64).reshape(ne, self.uq_K)
+
+    def uq_features(self, t1, t2):
+        """phi = ((B / |B|) R, log |B|, log |B_I2|, log |B_rho|) density_scale; B = [I2 block, rho block], each the collected
+        functions of its reduce's sources, n-outer and c-inner (libgrace/include/grace/uq.h:1-9, src/fused_2l.cpp:1156-1186)."""
+        blocks = []
+        for reds, t in ((self.rI2, t2), (self.rRho, t1)):
+            parts = []
+            for src, r in reds.items():
+                X = t[src][:, r.ci, :]
+                parts.append(np.transpose(X, (0, 2, 1)).reshape(X.shape[0], -1))
+            blocks.append(np.concatenate(parts, axis=1))
+        B = np.concatenate(blocks, axis=1)
+        nrm = np.sqrt((B * B).sum(1))
+        f = np.empty((B.shape[0], self.uq_D))
+        f[:, :self.uq_rp] = (B @ self.uq_R) / (nrm + 1.0e-12)[:, None]
+        f[:, self.uq_rp] = np.log(nrm + 1.0e-12) * self.uq_scale
+        for b, blk in enumerate(blocks):
+            f[:, self.uq_rp + 1 + b] = np.log(np.sqrt((blk * blk).sum(1)) + 1.0e-12) * self.uq_scale
+        return f
+
+    def uq(self, mu, f):
+        """nearest centroid of the element, Mahalanobis distance, gamma (libgrace/include/grace/fused_cpu.h:1375-1412)"""
+        na = f.shape[0]
+        gamma, sigma, cluster = np.zeros(na), np.zeros(na), np.zeros(na)
+        for a in range(na):
+            m = mu[a]
+            d2 = ((f[a][None, :] - self.uq_cen[m, :self.uq_ncl[m]]) ** 2).sum(1)
+            k = int(np.argmin(d2))
+            dl = f[a] - self.uq_cen[m, k]
+            sigma[a] = np.sqrt(dl @ self.uq_icov[m, k] @ dl + 1.0e-8)
+            gamma[a] = sigma[a] / max(self.uq_thr[m, k], 1.0e-10)
+            cluster[a] = k
+        return gamma, sigma, cluster
 
     def radial(self, which, x):
         layers, C = (self.rad1, self.C1) if which == 1 else (self.rad2, self.CR)
@@ -297,7 +349,7 @@ def _virial(rh, r, fv):
                      (dl[:, 0] * fv[:, 1]).sum(), (dl[:, 0] * fv[:, 2]).sum(), (dl[:, 1] * fv[:, 2]).sum()])
 
 
-def compute_2l(model: Model2L, mu, offset, j, rij, *, chunk=128, want_forces=True):
+def compute_2l(model: Model2L, mu, offset, j, rij, *, chunk=128, want_forces=True, uq=False):
     """One GRACE-2L energy + forces + virial call on a CSR bond list of a closed system (every j is a central atom:
     the periodic images are folded onto their owners, as the reference's CSR path does).
 
@@ -349,6 +401,7 @@ def compute_2l(model: Model2L, mu, offset, j, rij, *, chunk=128, want_forces=Tru
         rho_glob[a0:a1] = rho
         state.append(t)
     # ---- P3
+    feats = np.zeros((n, model.uq_D)) if uq else None
     gI_sum = np.zeros_like(I_glob)
     grho_glob = np.zeros_like(rho_glob)
     for a0, a1 in chunks:
@@ -365,6 +418,8 @@ def compute_2l(model: Model2L, mu, offset, j, rij, *, chunk=128, want_forces=Tru
         I2, t2 = model.layer2_forward(mu[a0:a1], YIp, B0)
         E, grho, gI2 = model.energy_atoms(mu[a0:a1], rho_glob[a0:a1], I2)
         energies[a0:a1] = E
+        if uq:
+            feats[a0:a1] = model.uq_features(state[chunks.index((a0, a1))], t2)
         if not want_forces:
             continue
         grho_glob[a0:a1] = grho
@@ -406,4 +461,8 @@ def compute_2l(model: Model2L, mu, offset, j, rij, *, chunk=128, want_forces=Tru
             np.add.at(forces, bi, fv)
             np.add.at(forces, bj, -fv)
             virial += _virial(rh, r, fv)
-    return {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial}
+    out = {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial}
+    if uq:
+        g, sg, cl = model.uq(mu, feats)
+        out.update(gamma=g, atomic_sigma=sg, gmm_cluster=cl, uq_features=feats)
+    return out

@@ -140,17 +140,18 @@ int ref_compute(void *hv, int n, const int *types, const int64_t *offset, const 
   }
 }
 
-// GRACE-1L with the UQ head (uqv6): forward only; gamma, sigma, cluster [n] per atom (Grace1LFused::enable_uq, uq_batch)
+// GRACE-1L / 2L with the UQ head (uqv6): forward only; gamma, sigma, cluster [n] per atom (Grace{1,2}LFused::enable_uq)
 int ref_compute_uq(void *hv, int n, const int *types, const int64_t *offset, const int *j, const double *rij, const double *x,
                    const int *image, const double *shifts, int nthreads, double *energy, double *gamma, double *sigma, double *cluster)
 {
   Ref *h = static_cast<Ref *>(hv);
   try {
-    if (!h->d1) {
-      g_err = "UQ: a GRACE-1L driver is required (setup_types first)";
+    if (!h->d1 && !h->d2) {
+      g_err = "UQ: a GRACE-1L or GRACE-2L driver is required (setup_types first)";
       return 1;
     }
-    h->d1->enable_uq();
+    if (h->d1) h->d1->enable_uq();
+    else h->d2->enable_uq();
     grace::CsrBonds src{types, offset, j, rij, x, image, shifts};
     grace::Outputs out;
     std::vector<double> f((size_t) 3 * n, 0.0);
@@ -161,7 +162,9 @@ int ref_compute_uq(void *hv, int n, const int *types, const int64_t *offset, con
     grace::ComputeFlags fl;
     fl.energy_only = true;
     fl.uq = true;
-    h->d1->compute(n, nullptr, n, n, src, out, fl, nthreads);
+    grace::NoExchange ex;
+    if (h->d1) h->d1->compute(n, nullptr, n, n, src, out, fl, nthreads);
+    else h->d2->compute(n, nullptr, n, n, src, ex, out, fl, nthreads);
     *energy = out.energy;
     return 0;
   } catch (const std::exception &e) {

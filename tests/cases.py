@@ -127,8 +127,31 @@ def model_uq2():
     return d
 
 
-MODELS = {"uq2": model_uq2, "l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3el": model_l3el, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
-LAYERS = {"uq2": 1, "l3mix": 3, "l3wide": 3, "l3pad": 3, "l3el": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
+def model_uq2l():
+    """the reference's fixture model grace_2l_small (max_order 4: the UQ head refuses max_order 3) with a generated uqv6 head
+    of two basis blocks whose centroids sit next to features of atoms of the alloy54 structure, one exactly on an atom"""
+    from grace_runtime_amd import kk
+    from oracle import grace_oracle_2l as go2
+    with np.load(os.path.join(REF_FIXTURES, "grace_2l_small.npz")) as z:
+        d = {k: z[k] for k in z.files}
+    synth.add_uq_head_2l(d, rp_dim=10, max_clusters=3, seed=47)
+    pos, cell, pbc, types = structure_alloy54()
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 5.0)
+    x, t = pos[perm], types[perm]
+    rij = x[j] - np.repeat(x, np.diff(offset), axis=0) + shifts[image]
+    f = go2.compute_2l(go2.Model2L(d), t - 1, offset, j, rij, want_forces=False, uq=True)["uq_features"]
+    cen = d["uq_centroids"]
+    ncl = np.array([2, 3], np.int32)
+    for e in range(2):
+        at = np.nonzero(t - 1 == e)[0]
+        for k in range(ncl[e]):
+            cen[e, k] = f[at[(k * (len(at) - 1)) // max(ncl[e] - 1, 1)]] + (0.0 if (e, k) == (0, 1) else 0.002 * (k + 1))
+    d["uq_centroids"], d["uq_n_clusters"] = cen, ncl
+    return d
+
+
+MODELS = {"uq2l": model_uq2l, "uq2": model_uq2, "l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3el": model_l3el, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
+LAYERS = {"uq2l": 2, "uq2": 1, "l3mix": 3, "l3wide": 3, "l3pad": 3, "l3el": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
 
 
 def write_model(name, directory):
@@ -278,7 +301,7 @@ E2E_CASES_2L = [("config3", "fcc108", None), ("l2mix", "alloy54", 5.5), ("l2mix"
 # reference fixture models (tests/golden/ref_fixtures) on the reference's fixture cells: goldens of the compiled reference
 E2E_CASES_3L = [("l3mix", "alloy54", 5.5), ("l3mix", "triclinic", None), ("l3mix", "slab", None), ("l3mix", "molecule", None),
                 ("l3wide", "fcc108", None), ("l3nat", "config1", None), ("l3el", "alloy54", None)]
-UQ_CASES = [("uq2", "alloy54"), ("uq2", "triclinic")]
+UQ_CASES = [("uq2", "alloy54"), ("uq2", "triclinic"), ("uq2l", "alloy54"), ("uq2l", "triclinic")]
 FIXTURE_CASES_2L = [(m, c) for m in ("grace_2l_small", "grace_2l_l3", "legacy_2l_small", "legacy_2l_wide") for c in ("W54", "WMo54")]
 
 

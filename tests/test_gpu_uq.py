@@ -1,4 +1,4 @@
-"""The UQ head of GRACE-1L on the GPU (k_uq through the C ABI) against the CPU oracle: gamma and sigma to 1e-9 relative in
+"""The UQ head of GRACE-1L and GRACE-2L on the GPU (k_uq through the C ABI) against the CPU oracle: gamma and sigma to 1e-9 relative in
 fp64 (1e-4 with the fp32 network), the cluster index exactly.  Needs an MI355X: run with -m gpu."""
 import os
 
@@ -8,6 +8,7 @@ import pytest
 import cases
 from grace_runtime_amd import kk
 from oracle import grace_oracle as go
+from oracle import grace_oracle_2l as go2
 
 pytestmark = pytest.mark.gpu
 
@@ -20,13 +21,20 @@ def _bonds(struct, rc=5.0):
     return t, offset, j, rij
 
 
-@pytest.mark.parametrize("precision,tol", [(64, 1e-9), (32, 1e-4)])
+def _oracle(path, name, t, offset, j, rij):
+    if cases.LAYERS[name] == 2:
+        return go2.compute_2l(go2.Model2L(path), t - 1, offset, j, rij, uq=True)
+    return go.compute_1l(go.Model1L(path), t - 1, offset, j, rij, uq=True)
+
+
+# GRACE-2L engines compute in fp64 only
+@pytest.mark.parametrize("name,precision,tol", [("uq2", 64, 1e-9), ("uq2", 32, 1e-4), ("uq2l", 64, 1e-9)])
 @pytest.mark.parametrize("struct", ["alloy54", "triclinic"])
-def test_uq_matches_oracle(model_dir, struct, precision, tol):
-    path = os.path.join(model_dir, "uq2.npz")
+def test_uq_matches_oracle(model_dir, name, struct, precision, tol):
+    path = os.path.join(model_dir, name + ".npz")
     eng = kk.Engine(kk.Model(path), ["Mo", "W"], precision)
     t, offset, j, rij = _bonds(struct)
-    ref = go.compute_1l(go.Model1L(path), t - 1, offset, j, rij, uq=True)
+    ref = _oracle(path, name, t, offset, j, rij)
     eng.upload(t, offset, j, rij)
     eng.run(uq=True)
     out, uq = eng.fetch(), eng.fetch_uq()
@@ -46,8 +54,9 @@ def test_uq_matches_oracle(model_dir, struct, precision, tol):
     assert np.abs(eng.fetch_uq()["gamma"] / ref["gamma"] - 1).max() < tol if precision == 64 else True
 
 
-def test_calculator_level_call_returns_uq_in_the_callers_order(model_dir):
-    path = os.path.join(model_dir, "uq2.npz")
+@pytest.mark.parametrize("name", ["uq2", "uq2l"])
+def test_calculator_level_call_returns_uq_in_the_callers_order(model_dir, name):
+    path = os.path.join(model_dir, name + ".npz")
     model = kk.Model(path)
     pos, cell, pbc, types = cases.structure_alloy54()
     s = kk.System(model, ["Mo", "W"], skin=0.3)
@@ -55,7 +64,7 @@ def test_calculator_level_call_returns_uq_in_the_callers_order(model_dir):
     perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 5.0)
     x, t = pos[perm], types[perm]
     rij = x[j] - np.repeat(x, np.diff(offset), axis=0) + shifts[image]
-    ref = go.compute_1l(go.Model1L(path), t - 1, offset, j, rij, uq=True)
+    ref = _oracle(path, name, t, offset, j, rij)
     for k in ("gamma", "atomic_sigma", "gmm_cluster"):
         want = np.empty(len(t))
         want[perm] = ref[k]

@@ -1,7 +1,8 @@
-"""The UQ head (uqv6, gamma only) of GRACE-1L: the CPU oracle against the compiled reference and against what the
+"""The UQ head (uqv6, gamma only) of GRACE-1L and GRACE-2L: the CPU oracle against the compiled reference and against what the
 definition fixes, and the loader's checks (no GPU needed).
 
-No fixture of the reference carries a UQ head, so the head is a generated one (tests/cases.py model_uq2).  The compiled
+No fixture of the reference carries a UQ head, so the head is a generated one (tests/cases.py model_uq2, and model_uq2l: the
+reference's fixture model grace_2l_small with a generated head of two basis blocks).  The compiled
 reference projects the basis in fp32 (libgrace/include/grace/fused_cpu.h:1275-1283: gamma within ~1e-5 of an fp64
 projection): 1e-4 relative on gamma and sigma, the cluster index exactly."""
 import os
@@ -12,6 +13,7 @@ import pytest
 import cases
 from grace_runtime_amd import kk
 from oracle import grace_oracle as go
+from oracle import grace_oracle_2l as go2
 from oracle import ref_lib
 
 
@@ -23,20 +25,28 @@ def _bonds(struct, rc=5.0):
     return t, offset, j, rij
 
 
+def _oracle(path, t, offset, j, rij, **kw):
+    """the oracle of the model's kind (GRACE-1L or GRACE-2L) with the UQ head evaluated"""
+    if cases.LAYERS[os.path.basename(path)[:-4]] == 2:
+        return go2.compute_2l(go2.Model2L(path), t - 1, offset, j, rij, want_forces=False, uq=True, **kw), go2.Model2L(path)
+    return go.compute_1l(go.Model1L(path), t - 1, offset, j, rij, want_forces=False, uq=True, **kw), go.Model1L(path)
+
+
 @pytest.fixture(scope="module")
 def uq_model(model_dir):
     return os.path.join(model_dir, "uq2.npz")
 
 
 @pytest.mark.skipif(not ref_lib.available(), reason="compiled reference not built")
-@pytest.mark.parametrize("struct", ["alloy54", "triclinic"])
-def test_oracle_matches_compiled_reference(uq_model, struct):
+@pytest.mark.parametrize("model,struct", cases.UQ_CASES)
+def test_oracle_matches_compiled_reference(model_dir, model, struct):
+    path = os.path.join(model_dir, model + ".npz")
     t, offset, j, rij = _bonds(struct)
-    o = go.compute_1l(go.Model1L(uq_model), t - 1, offset, j, rij, want_forces=False, uq=True)
-    r = ref_lib.RefModel(uq_model, [0, 1]).compute_uq(t, offset, j, rij)
+    o, m = _oracle(path, t, offset, j, rij)
+    r = ref_lib.RefModel(path, [0, 1]).compute_uq(t, offset, j, rij)
     assert np.array_equal(o["gmm_cluster"], r["gmm_cluster"])
-    if struct == "alloy54":
-        assert len(np.unique(o["gmm_cluster"][t == 1])) == 3 and len(np.unique(o["gmm_cluster"][t == 2])) == 2
+    if struct == "alloy54":                                           # every cluster of the head is some atom's nearest
+        assert [len(np.unique(o["gmm_cluster"][t == e + 1])) for e in range(2)] == list(m.uq_ncl)
     assert np.abs(o["gamma"] / r["gamma"] - 1).max() < 1e-4
     assert np.abs(o["atomic_sigma"] / r["atomic_sigma"] - 1).max() < 1e-4
 
@@ -45,19 +55,20 @@ def test_oracle_matches_compiled_reference(uq_model, struct):
 def test_oracle_matches_golden_of_the_compiled_reference(model_dir, gold, model, struct):
     """the committed outputs of the compiled reference (tests/golden/make_golden.py), for machines without it"""
     t, offset, j, rij = _bonds(struct)
-    o = go.compute_1l(go.Model1L(os.path.join(model_dir, model + ".npz")), t - 1, offset, j, rij, want_forces=False, uq=True)
+    o, _ = _oracle(os.path.join(model_dir, model + ".npz"), t, offset, j, rij)
     tag = f"uq/{model}/{struct}"
     assert np.array_equal(o["gmm_cluster"], gold[tag + "/gmm_cluster"])
     assert np.abs(o["gamma"] / gold[tag + "/gamma"] - 1).max() < 1e-4
     assert np.abs(o["atomic_sigma"] / gold[tag + "/atomic_sigma"] - 1).max() < 1e-4
 
 
-def test_what_the_definition_fixes(uq_model):
+@pytest.mark.parametrize("name", ["uq2", "uq2l"])
+def test_what_the_definition_fixes(model_dir, name):
     """the atom whose feature vector IS a centroid has sigma = sqrt(1e-8) and gamma = sigma / threshold; the features are
     invariants of the neighbourhood: a rotated structure gives the same gamma; gamma = sigma / threshold everywhere"""
-    m = go.Model1L(uq_model)
+    path = os.path.join(model_dir, name + ".npz")
     t, offset, j, rij = _bonds("alloy54")
-    o = go.compute_1l(m, t - 1, offset, j, rij, want_forces=False, uq=True)
+    o, m = _oracle(path, t, offset, j, rij)
     thr = m.uq_thr[t - 1, o["gmm_cluster"].astype(int)]
     assert np.abs(o["gamma"] * thr - o["atomic_sigma"]).max() < 1e-12
     assert abs(o["atomic_sigma"].min() - 1e-4) < 1e-9 and (o["atomic_sigma"] < 2e-4).sum() == 1
@@ -71,9 +82,15 @@ def test_what_the_definition_fixes(uq_model):
         assert abs(o["atomic_sigma"][a] ** 2 - (sum(dl[p] * m.uq_icov[e, int(np.argmin(d2)), p, q] * dl[q] for p in range(len(dl))
                                                    for q in range(len(dl))) + 1e-8)) < 1e-10
     assert np.abs(np.linalg.norm(f[:, :m.uq_rp], axis=1)).max() < np.linalg.norm(m.uq_R, 2) + 1e-9     # |B R| / |B| <= |R|
-    assert np.abs(f[:, m.uq_rp] - f[:, m.uq_rp + 1]).max() == 0.0                                     # one basis block: equal channels
+    if name == "uq2":
+        assert np.abs(f[:, m.uq_rp] - f[:, m.uq_rp + 1]).max() == 0.0                                 # one basis block: equal channels
+    else:                                                # two blocks: |B|^2 = |B_I2|^2 + |B_rho|^2 (the 1e-12 inside the logs: 1e-9)
+        s = m.uq_scale
+        assert m.uq_D == m.uq_rp + 3
+        assert np.abs(np.exp(2 * f[:, m.uq_rp] / s) - np.exp(2 * f[:, m.uq_rp + 1] / s) - np.exp(2 * f[:, m.uq_rp + 2] / s)).max() < \
+            1e-9 * np.exp(2 * f[:, m.uq_rp] / s).max()
     rot = np.linalg.qr(np.random.default_rng(4).standard_normal((3, 3)))[0]
-    o2 = go.compute_1l(m, t - 1, offset, j, rij @ rot.T, want_forces=False, uq=True)
+    o2, _ = _oracle(path, t, offset, j, rij @ rot.T)
     assert np.abs(o2["gamma"] - o["gamma"]).max() < 1e-9 * o["gamma"].max()
 
 
@@ -117,8 +134,13 @@ def test_heads_that_validate_and_models_without(tmp_path, uq_model, model_dir):
     assert not plain.has_uq
     with pytest.raises(ValueError, match="no UQ head"):
         plain.validate_uq()
-    with pytest.raises(ValueError, match="GRACE-1L models only"):
+    with pytest.raises(ValueError, match="no UQ head"):
         kk.Model(os.path.join(model_dir, "l2mix.npz")).validate_uq()
+    with pytest.raises(ValueError, match="GRACE-1L and GRACE-2L models only"):
+        kk.Model(os.path.join(model_dir, "l3mix.npz")).validate_uq()
+    two = kk.Model(os.path.join(model_dir, "uq2l.npz"))
+    assert two.has_uq and two.layers == 2
+    two.validate_uq()
     o3 = kk.Model(_mutated(tmp_path, lambda d: synth_uq(d), "cut2"))          # max_order 3: refused (tests/test_driver.cpp:406-415)
     with pytest.raises(ValueError, match="max_order 3"):
         o3.validate_uq()
@@ -127,3 +149,28 @@ def test_heads_that_validate_and_models_without(tmp_path, uq_model, model_dir):
 def synth_uq(d):
     from grace_runtime_amd import synth
     synth.add_uq_head_1l(d, rp_dim=6, max_clusters=2)
+
+
+BAD_UQ_2L = [
+    (lambda d: d.update(uq_rp_matrix=d["uq_rp_matrix"][:-1]), "rows, the model's invariant basis has"),
+    (lambda d: d.update(uq_feature_dim=np.array([12]), uq_centroids=np.zeros((2, 3, 12)), uq_inv_cov=np.zeros((2, 3, 12, 12))),
+     "2 density channels, expected 3"),
+    (lambda d: d.update(uq_schema_version=np.array([4])), "UQ schema v4 unsupported"),
+    (lambda d: d.update(uq_n_clusters=np.array([0, 3], np.int32)), "element index 0 has no GMM clusters"),
+]
+
+
+@pytest.mark.parametrize("edit,msg", BAD_UQ_2L)
+def test_a_broken_head_on_a_2l_model(tmp_path, edit, msg):
+    m = kk.Model(_mutated(tmp_path, edit, "uq2l"))                     # loads (libgrace/src/model_2l.cpp:404-478)
+    assert m.has_uq and m.layers == 2
+    with pytest.raises(ValueError, match=msg):
+        m.validate_uq()
+
+
+def test_max_order_3_2l_model_with_a_head_is_refused(tmp_path):
+    from grace_runtime_amd import synth
+    m = kk.Model(_mutated(tmp_path, lambda d: synth.add_uq_head_2l(d, rp_dim=6, max_clusters=2), "l2mix"))
+    assert m.has_uq
+    with pytest.raises(ValueError, match="max_order 3"):
+        m.validate_uq()
