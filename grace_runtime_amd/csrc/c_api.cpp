@@ -254,16 +254,20 @@ int gr_engine_fetch_uq(gr_engine *e, double *gamma, double *sigma, double *clust
   });
 }
 
-int gr_model_has_uq(const gr_model *m) { return m && ((m->m1 && m->m1->uq.has_uq) || (m->m2 && m->m2->uq.has_uq)) ? 1 : 0; }
+int gr_model_has_uq(const gr_model *m)
+{
+  return m && ((m->m1 && m->m1->uq.has_uq) || (m->m2 && m->m2->uq.has_uq) || (m->m3 && m->m3->uq.has_uq)) ? 1 : 0;
+}
 
 int gr_model_validate_uq(const gr_model *m)
 {
   return guarded([&] {
     if (!m) throw grhip::InvalidArgument("null model");
-    if (!m->m1 && !m->m2) throw grhip::InvalidArgument("the UQ head is evaluated for GRACE-1L and GRACE-2L models only");
     try {
       if (m->m1) m->m1->validate_uq();
-      else m->m2->validate_uq();
+      else if (m->m2) m->m2->validate_uq();
+      else if (!m->m3->uq.has_uq)    // a GRACE-3L file with a broken head does not load (libgrace/src/fused_3l.cpp:269-274)
+        throw grhip::Error("GRACE-3L: the model has no UQ head (kokkos.npz exported without UQ artifacts)");
     } catch (const grhip::Error &e) {
       throw grhip::InvalidArgument(e.what());    // python/kk/kk_core.cpp: std::invalid_argument (unsupported model)
     }

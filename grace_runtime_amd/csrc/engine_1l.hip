@@ -189,7 +189,7 @@ template<class T> void Engine1L<T>::build()
         uq_.blk[s] = 0;
         off += uq_.nin[s] * uq_.nc[s];
       }
-      uq_.d_basis = off;
+      uq_.d_basis = off; uq_.row0 = 0; uq_.carry_in = uq_.carry_out = 0;
       uq_.nblk = 1;
       uq_.rp = m.uq.rp_dim; uq_.D = m.uq.feature_dim; uq_.K = m.uq.max_clusters;
       uq_.density_scale = m.uq.density_scale;

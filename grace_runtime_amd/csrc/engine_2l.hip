@@ -229,7 +229,7 @@ template<class T> void Engine2L<T>::build()
           off += uq_.nin[q] * uq_.nc[q];
         }
       }
-      uq_.nsrc = q; uq_.nblk = 2; uq_.d_basis = off;
+      uq_.nsrc = q; uq_.nblk = 2; uq_.d_basis = off; uq_.row0 = 0; uq_.carry_in = uq_.carry_out = 0;
       uq_.rp = m.uq.rp_dim; uq_.D = m.uq.feature_dim; uq_.K = m.uq.max_clusters;
       uq_.density_scale = m.uq.density_scale;
       upload_vec(uqR_, m.uq.rp_matrix); upload_vec(uqCen_, m.uq.centroids); upload_vec(uqIcov_, m.uq.inv_cov);

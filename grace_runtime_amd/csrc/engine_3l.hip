@@ -162,6 +162,10 @@ template<class T> struct Layer3 {
   Ten X, L2, R2p, L3, R3p, L4, R4p, EQ, I;
   DevBuf rho_raw, grho;
   int nR2 = 0, nR3 = 0, nR4 = 0, wR = 0;    // functions of the product reduces, their common padded width
+  // UQ head: the rows of this layer's basis block (inputs of the rho reduce in the model's instruction order)
+  UqDev<T> uq{};
+  int uqSlot[4] = {0, 0, 0, 0};             // tensor of each instruction: 0 X, 1 R2, 2 R3, 3 R4
+  DevBuf uqCi[4];
 };
 
 template<class T> class Engine3L final : public EngineBase {
@@ -186,6 +190,8 @@ template<class T> class Engine3L final : public EngineBase {
   Layer3<T> L_[3];
   DevBuf shift_, eW0_, eW1_, escale_[3], sink_, emi_, YG_;
   Energy3Dev en_{};
+  DevBuf uqR_, uqCen_, uqIcov_, uqNcl_, uqThr_, uqZ_, uqN2_;    // UQ head arrays; raw projection and block norms carried over the layers
+  bool uq_on_ = false;
   // scratch shared by the layers (largest size over the layers): temporaries of the forward pass and all adjoints
   DevBuf M_, gM_, pairP_, gpairP_, A_, gA_, P_, gP_, R2_, R3_, R4_, FA_, FB_, gX_, gR2_, gR3_, gR4_, gFA_, gFB_, gLp_, gRp_, gEQ_;
 
@@ -266,6 +272,60 @@ template<class T> void Engine3L<T>::build()
   upload_vec(shift_, m.shift_values);
   sink_.ensure(64);
   for (int k = 0; k < 3; k++) build_layer(k);
+  // ---- UQ head (libgrace/src/fused_3l.cpp:845-866): basis = inputs of the rho1 | rho2 | rho3 reduces, one block per layer
+  if (m.uq.has_uq) {
+    try {
+      if (m.uq.rp_dim > 256 || m.uq.feature_dim > 256) throw Error("GRACE-3L UQ: feature widths above 256 are not supported");
+      upload_vec(uqR_, m.uq.rp_matrix); upload_vec(uqCen_, m.uq.centroids); upload_vec(uqIcov_, m.uq.inv_cov);
+      upload_vec(uqNcl_, m.uq.n_clusters); upload_vec(uqThr_, m.uq.interp_thresholds);
+      int off = 0;
+      for (int k = 0; k < 3; k++) {
+        Layer3<T> &L = L_[k];
+        const std::string K = "A" + std::to_string(k + 1);
+        const std::string names[4] = {L.equiv ? K + "_red" : K, K + "_2_red", K + "_3_red", K + "_4_red"};
+        const int nf[4] = {L.X.nf, L.nR2, L.nR3, L.nR4};
+        const Model3L::Reduce &r = Model3L::by_name(m.reduce, "rho" + std::to_string(k + 1));
+        if (r.instr.size() != 4) throw Error("GRACE-3L UQ: rho" + std::to_string(k + 1) + " does not have four inputs");
+        UqDev<T> &u = L.uq;
+        u = UqDev<T>{};
+        int loc = 0;
+        for (int q = 0; q < 4; q++) {
+          const Model3L::Instr &ins = r.instr[q];
+          int slot = -1;
+          for (int s = 0; s < 4; s++)
+            if (ins.name == names[s]) slot = s;
+          if (slot < 0) throw Error("GRACE-3L UQ: rho input " + ins.name + " is not a tensor of the layer");
+          for (int c : ins.collect_ind)
+            if (c < 0 || c >= nf[slot]) throw Error("GRACE-3L UQ: rho input " + ins.name + " collects a function it does not have");
+          L.uqSlot[q] = slot;
+          upload_vec(L.uqCi[q], ins.collect_ind);
+          u.ci[q] = L.uqCi[q].template as<int>();
+          u.nfun[q] = nf[slot];
+          u.cpad[q] = slot == 0 ? L.X.w : L.wR;
+          u.nin[q] = ins.n_in;
+          u.nc[q] = (int) ins.collect_ind.size();
+          u.off[q] = loc;
+          u.blk[q] = k;
+          if (u.nin[q] > u.cpad[q]) throw Error("GRACE-3L UQ: rho input " + ins.name + " is wider than its tensor");
+          loc += u.nin[q] * u.nc[q];
+        }
+        u.nsrc = 4; u.nblk = 3; u.row0 = off; u.d_basis = loc;
+        u.carry_in = k > 0 ? 1 : 0; u.carry_out = k < 2 ? 1 : 0;
+        u.rp = m.uq.rp_dim; u.D = m.uq.feature_dim; u.K = m.uq.max_clusters;
+        u.density_scale = m.uq.density_scale;
+        u.R = uqR_.template as<double>(); u.cen = uqCen_.template as<double>(); u.icov = uqIcov_.template as<double>();
+        u.ncl = uqNcl_.template as<int>(); u.thr = uqThr_.template as<double>();
+        if ((size_t) (u.d_basis + 4 * u.rp + 2 * u.D) * sizeof(double) > 150 * 1024) throw Error("GRACE-3L UQ: the basis does not fit the kernel's LDS");
+        off += loc;
+      }
+      if (off != m.uq.d_basis) throw Error("GRACE-3L UQ: basis width " + std::to_string(off) + " != uq_rp_matrix rows " + std::to_string(m.uq.d_basis));
+      has_uq_head_ = true;
+    } catch (const std::exception &e) {
+      uq_why_ = e.what();
+    }
+  } else {
+    uq_why_ = "the model file carries none";
+  }
   for (int k = 0; k < 2; k++) {
     const Layer3<T> &a = L_[k], &b = L_[k + 1];
     if (a.I.nf != b.nlmi || a.eqn.Creal != b.C) throw Error("GRACE-3L: the message of layer " + std::to_string(k + 1) + " does not fit the next SPBF");
@@ -665,6 +725,20 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
     }
 #undef GR_RED
   });
+  if (uq_on_) {    // this layer's rows of the basis while its tensors exist; the last layer finishes the GMM (fused_3l.cpp:1158-1201)
+    stage(tg(k, "uq").c_str(), [&] {
+      UqDev<T> u = L.uq;
+      for (int q = 0; q < u.nsrc; q++) u.X[q] = srcs[L.uqSlot[q]];
+      u.zacc = uqZ_.as<double>();
+      u.n2acc = uqN2_.as<double>();
+      const size_t lds = (size_t) (u.d_basis + 4 * u.rp + 2 * u.D) * sizeof(double);
+      auto kern = k_uq<T>;
+      if (lds > 48 * 1024)
+        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+      hipLaunchKernelGGL(kern, dim3(n), dim3(256), lds, stream_, u, mu_.as<int>(), n, uq_gamma_.as<double>(), uq_sigma_.as<double>(),
+                         uq_cluster_.as<double>());
+    });
+  }
   (void) forces;
 }
 
@@ -798,7 +872,15 @@ template<class T> void Engine3L<T>::run(const RunFlags &fl)
     hipLaunchKernelGGL(kern, dim3((unsigned) ((ecap + 63) / 64)), dim3(64), lds, stream_, sh_, rh_.as<double>(), n_edges, nlm_, forces ? 1 : 0,
                        YG_.as<T>());
   });
+  uq_on_ = fl.uq;
+  if (fl.uq) {
+    const size_t na = (size_t) n;
+    uq_gamma_.ensure(na * sizeof(double)); uq_sigma_.ensure(na * sizeof(double)); uq_cluster_.ensure(na * sizeof(double));
+    uqZ_.ensure(na * L_[0].uq.rp * sizeof(double));
+    uqN2_.ensure(na * kUqMaxBlk * sizeof(double));
+  }
   for (int k = 0; k < 3; k++) layer_forward(k, forces, yw);
+  if (fl.uq) ran_uq_ = true;
   stage("energy_mlp", [&] {
     hipLaunchKernelGGL(k_energy_3l, dim3(n), dim3(64), (size_t) (nrho_ + 2 * en_.nh) * sizeof(double), stream_, en_, mu_.as<int>(),
                        (const double *) L_[0].rho_raw.template as<double>(), (const double *) L_[1].rho_raw.template as<double>(),

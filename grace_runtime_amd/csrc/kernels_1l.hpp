@@ -1123,13 +1123,16 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
 // ---------------------------------------------------------------------------------------------------------------
 // UQ head (uqv6, gamma only)
 // ---------------------------------------------------------------------------------------------------------------
-constexpr int kUqMaxSrc = 8, kUqMaxBlk = 2;
+constexpr int kUqMaxSrc = 8, kUqMaxBlk = 3;
 template<class T> struct UqDev {
   const T *X[kUqMaxSrc];      // per-atom tensors of the reduces' sources [atom][function][channel]
   const int *ci[kUqMaxSrc];   // collected functions of each source
   int nfun[kUqMaxSrc], cpad[kUqMaxSrc], nin[kUqMaxSrc], nc[kUqMaxSrc], off[kUqMaxSrc];    // functions per atom, padded / real channels, collected, first basis index
-  int blk[kUqMaxSrc];         // invariant block of the source (1L: rho = 0; 2L: I2 = 0, rho = 1)
-  int nsrc, nblk, d_basis, rp, D, K;
+  int blk[kUqMaxSrc];         // invariant block of the source (1L: rho = 0; 2L: I2 = 0, rho = 1; 3L: layer)
+  int nsrc, nblk, rp, D, K;
+  int row0, d_basis;          // this launch holds rows row0 .. row0 + d_basis of the basis (off[] counts from row0)
+  int carry_in, carry_out;    // 3L, one launch per layer: add the projection and block norms kept by the earlier layers / keep them and stop
+  double *zacc, *n2acc;       // [atom][rp], [atom][kUqMaxBlk]: the kept raw projection and squared block norms
   double density_scale;
   const double *R;            // [d_basis][rp]
   const double *cen;          // [nel][K][D]
@@ -1142,6 +1145,8 @@ template<class T> struct UqDev {
 // libgrace/src/fused_1l.cpp:616-636, fused_2l.cpp:1156-1186): basis B = per invariant block the collected functions of
 // the reduce's sources, n-outer and c-inner per source; phi = ((B / |B|) R, log |B| scale, log |B_block| scale ...);
 // nearest centroid of the atom's element, Mahalanobis distance over the cluster's threshold.  fp64 throughout.
+// GRACE-3L (libgrace/src/fused_3l.cpp:1156-1201) evaluates the rows of one layer per launch, right after that layer's
+// rho reduce while its tensors exist: raw projection and squared block norms are carried in zacc / n2acc.
 // block: 256 threads; dynamic LDS: d_basis + 4 rp + 2 D doubles.
 template<class T>
 __global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natoms, double *gamma, double *sigma, double *cluster)
@@ -1183,6 +1188,7 @@ __global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natom
 #pragma unroll
   for (int b = 0; b < kUqMaxBlk; b++) {
     nb2[b] = bsum[0][b] + bsum[1][b] + bsum[2][b] + bsum[3][b];
+    if (U.carry_in) nb2[b] += U.n2acc[(long long) at * kUqMaxBlk + b];
     tot += nb2[b];
   }
   const double nrm = sqrt(tot);
@@ -1191,7 +1197,7 @@ __global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natom
     const int ng = 256 / U.rp > 4 ? 4 : 256 / U.rp, gq = t / U.rp, d = t % U.rp;
     if (gq < ng) {
       double z = 0.0;
-      for (int b = gq; b < U.d_basis; b += ng) z += Bsh[b] * U.R[(long long) b * U.rp + d];
+      for (int b = gq; b < U.d_basis; b += ng) z += Bsh[b] * U.R[(long long) (U.row0 + b) * U.rp + d];
       Zp[gq * U.rp + d] = z;
     }
     __syncthreads();
@@ -1199,15 +1205,23 @@ __global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natom
       if (t < U.rp) {
         double z = 0.0;
         for (int q = 0; q < ng; q++) z += Zp[q * U.rp + t];
+        if (U.carry_in) z += U.zacc[(long long) at * U.rp + t];
+        if (U.carry_out) U.zacc[(long long) at * U.rp + t] = z;
         f[t] = z / (nrm + 1.0e-12);
       } else {    // density channels: the whole basis, then its blocks (one block: the same norm again)
         const int p = t - U.rp;
         double dn = nrm;
 #pragma unroll
         for (int b = 0; b < kUqMaxBlk; b++)
-          if (U.nblk > 1 && p == 1 + b) dn = sqrt(nb2[b]);
+          if (p == 1 + b) dn = sqrt(nb2[b]);
         f[t] = log(dn + 1.0e-12) * U.density_scale;
       }
+    }
+    if (U.carry_out) {    // the same for every thread of the block
+#pragma unroll
+      for (int b = 0; b < kUqMaxBlk; b++)
+        if (t == b) U.n2acc[(long long) at * kUqMaxBlk + b] = nb2[b];
+      return;
     }
     __syncthreads();
   }

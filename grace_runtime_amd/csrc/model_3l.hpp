@@ -80,6 +80,7 @@ struct Model3L {
   std::vector<RmsNorm> rmsnorm;
   Mlp energy_mlp;
   int energy_mlp_activation = 0, rho_width = 0;
+  UqHead uq;    // uqv6 UQ head; a file whose head is broken does not load (libgrace/src/model_3l.cpp:453-463)
   static constexpr double rms_norm_eps = 1e-10;    // libgrace/include/grace/fused_3l_cpu.h:424
 
   int nl() const { return lmax + 1; }
@@ -307,6 +308,21 @@ struct Model3L {
     if (v.has("energy_mlp_origin_n_out")) require_eq("energy_mlp_origin_n_out", v.int_scalar("energy_mlp_origin_n_out", 0), rho_width, "the channels of out1_origins");
     load_net("energy_mlp", energy_mlp, rho_width - 1, 1, "the channels of out1_origins but the linear channel 0", "one energy per atom");
     energy_mlp_activation = v.int_in("energy_mlp_activation", 0, 0, 1);
+    // ---- UQ head (optional): the GMM feature projects the inputs of the rho1 | rho2 | rho3 reduces
+    uq.load(v, n_elements, "GRACE-3L");
+    if (uq.has_uq) {
+      if (uq.schema != 6)
+        throw Error("GRACE-3L UQ: schema v" + std::to_string(uq.schema) + " unsupported (expects v6, uqv6 basis-RP normalize+density). Re-export the "
+                    "UQ artifacts at schema v6 with a current grace_utils.");
+      if (!uq.error.empty()) throw Error(uq.error);
+      if (uq.n_density > 4)
+        throw Error("GRACE-3L UQ: uq_n_density (" + std::to_string(uq.n_density) + ") > 4, the number of density channels this model's UQ kernels "
+                    "write. Artifact has an unexpected invariant-block count.");
+      int64_t width = 0;
+      for (int k = 1; k <= 3; k++)
+        for (const auto &ins : by_name(reduce, "rho" + std::to_string(k)).instr) width += (int64_t) ins.n_in * (int64_t) ins.collect_ind.size();
+      require_eq("uq_rp_matrix", uq.d_basis, width, "the inputs of the rho1, rho2, rho3 reduces", "rows");
+    }
   }
 
  private:

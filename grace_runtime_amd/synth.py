@@ -350,6 +350,13 @@ def add_uq_head_1l(d, **kw):
     return add_uq_head(d, [("rho", ("A", "AA", "AAA", "AAAA"))], **kw)
 
 
+def add_uq_head_3l(d, **kw):
+    """GRACE-3L: one block per layer, the inputs of rho1, rho2, rho3 in their instruction order (libgrace/src/model_3l.cpp:
+    453-463); four density channels"""
+    names = lambda k: tuple(n.decode() if isinstance(n, bytes) else str(n) for n in np.asarray(d[f"rho{k}_instruction_names"]).ravel())
+    return add_uq_head(d, [(f"rho{k}", names(k)) for k in (1, 2, 3)], **kw)
+
+
 def add_uq_head_2l(d, **kw):
     """GRACE-2L: blocks [I2 over B .. BBBB, rho over A .. AAAA] (libgrace/src/model_2l.cpp:404-478)"""
     return add_uq_head(d, [("I2", ("B", "BB", "BBB", "BBBB")), ("rho", ("A", "AA", "AAA", "AAAA"))], **kw)

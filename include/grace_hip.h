@@ -122,16 +122,18 @@ void gr_nlist_free(gr_nlist *l);
 int gr_compute(gr_engine *e, int n, const int *types, const double *positions, const double *cell,
                const unsigned char *pbc, unsigned flags, double *energy, double *forces, double *virial, double *eatom);
 
-/* UQ head (uqv6, gamma only) of GRACE-1L and GRACE-2L models: replaces GRACE1LModel::has_uq / validate_uq (libgrace/src/
+/* UQ head (uqv6, gamma only) of GRACE-1L, GRACE-2L and GRACE-3L models: replaces GRACE1LModel::has_uq / validate_uq (libgrace/src/
  * model_1l.cpp:216-285) and GRACE2LModel's (libgrace/src/model_2l.cpp:404-478), Grace1LFused::enable_uq / uq_batch /
  * uq_flush (libgrace/src/fused_1l.cpp:584-636), Grace2LFused's UQ stage (libgrace/src/fused_2l.cpp:1156-1186: basis
- * blocks [I2 inputs, rho inputs], density channels total / I2 / rho) and the gamma, atomic_sigma, gmm_cluster outputs of
- * Outputs (libgrace/include/grace/system.h:72-73).  A run with GR_FLAG_UQ (gr_engine_run,
+ * blocks [I2 inputs, rho inputs], density channels total / I2 / rho), Grace3LFused::enable_uq / uq_layer (libgrace/src/
+ * fused_3l.cpp:269-274, 1156-1201: one block per layer, the inputs of rho1, rho2, rho3, evaluated layer by layer; a
+ * GRACE-3L file with a broken head does not load, libgrace/src/model_3l.cpp:453-463) and the gamma, atomic_sigma,
+ * gmm_cluster outputs of Outputs (libgrace/include/grace/system.h:72-73).  A run with GR_FLAG_UQ (gr_engine_run,
  * gr_system_compute) evaluates per atom the extrapolation grade gamma, the Mahalanobis distance sigma to the nearest GMM
  * centroid of the atom's element and that cluster's index; the fetch calls copy them out ([n] each, NULL: skipped):
  * gr_engine_fetch_uq in the order of the uploaded list, gr_system_fetch_uq in the caller's atom order.
  * gr_model_has_uq: 1 when the file carries a UQ head; gr_model_validate_uq: GR_OK when it can be evaluated, else
- * GR_INVALID with the reason (no head, max_order 3, another schema, sizes that do not fit the model, a GRACE-3L model).  A run with
+ * GR_INVALID with the reason (no head, max_order 3, another schema, sizes that do not fit the model).  A run with
  * GR_FLAG_UQ on a model without a usable head gives GR_INVALID. */
 int gr_model_has_uq(const gr_model *m);
 int gr_model_validate_uq(const gr_model *m);

@@ -18,11 +18,15 @@ Reference followed (paths relative to the reference checkout):
 * EquivariantRMSNorm, InvariantLayerRMSNorm ...... libgrace/include/grace/fused_3l_cpu.h:335-444
 * readout ........................................ libgrace/src/fused_3l.cpp:1300-1360
 * bond force from dE/dx and dE/dY, virial ........ libgrace/src/fused_3l.cpp:1030-1047, :117-123
+* UQ head (uqv6, gamma only): basis blocks ....... libgrace/src/fused_3l.cpp:845-866, :1156-1201 (uq_layer),
+  GMM ............................................ libgrace/include/grace/fused_cpu.h:1385-1416 (uq_gmm)
 
 Pinning status: there is no GRACE-3L model file, golden vector or fixture in the reference checkout (its 3L tests
 need a registry model that is downloaded), so this oracle is pinned against the COMPILED REFERENCE (oracle/_ref) on
 generated random-weight models (energy, per-atom energies, forces, virial, at the reference's fp32 + spline
-accuracy), by finite differences of the energy, and by rotation / translation / permutation invariance.
+accuracy), by finite differences of the energy, and by rotation / translation / permutation invariance.  The UQ head
+(uq_block, uq): against the compiled reference on a generated head (cluster indices exactly, gamma and sigma to 1e-4:
+the reference projects in fp32), live and as committed goldens, and by what the definition fixes (tests/test_uq.py).
 """
 from __future__ import annotations
 
@@ -191,6 +195,49 @@ class Model3L:
         nlay = int(_scalar(d, "energy_mlp_n_layers"))
         self.emlp = [(_T(d[f"energy_mlp_W{i}"]), float(_scalar(d, f"energy_mlp_norm{i}", 1.0))) for i in range(nlay)]
         self.eact = int(_scalar(d, "energy_mlp_activation", 0))
+        # the uqv6 UQ head (libgrace/src/uq_head.cpp:11-76, model_3l.cpp:453-463)
+        self.has_uq = int(_scalar(d, "uq_schema_version", 0)) == 6
+        if self.has_uq:
+            ne = self.n_elements
+            self.uq_rp, self.uq_D, self.uq_K = int(_scalar(d, "uq_rp_dim")), int(_scalar(d, "uq_feature_dim")), int(_scalar(d, "uq_max_clusters"))
+            self.uq_scale = float(_scalar(d, "uq_rp_density_scale", 1.0))
+            self.uq_R = np.asarray(d["uq_rp_matrix"], dtype=np.float64).reshape(-1, self.uq_rp)
+            self.uq_cen = np.asarray(d["uq_centroids"], dtype=np.float64).reshape(ne, self.uq_K, self.uq_D)
+            self.uq_icov = np.asarray(d["uq_inv_cov"], dtype=np.float64).reshape(ne, self.uq_K, self.uq_D, self.uq_D)
+            self.uq_ncl = np.asarray(d["uq_n_clusters"]).astype(np.int64).ravel()
+            self.uq_thr = np.asarray(d["uq_interp_thresholds"], dtype=np.float64).reshape(ne, self.uq_K)
+
+    def uq_block(self, L, T):
+        """the rows of one layer's basis block: the inputs of its rho reduce in the model's instruction order, per input
+        channel-outer and collected-function-inner (libgrace/src/fused_3l.cpp:1167-1181)"""
+        parts = []
+        for cn, c in zip(L["rho"].inputs, L["rho"].ins):
+            X = T[cn].detach().numpy()[:, np.asarray(self.d[f"{L['rho'].name}_collect_ind_{cn}"]).astype(np.int64).ravel(), :]
+            parts.append(np.transpose(X, (0, 2, 1)).reshape(X.shape[0], -1))
+        return np.concatenate(parts, axis=1)
+
+    def uq(self, mu, blocks):
+        """phi = ((B / |B|) R, log |B|, log |B_rho1|, log |B_rho2|, log |B_rho3|) density_scale (the first uq_D - uq_rp
+        density channels), nearest centroid of the element (first of equal distances), sigma = sqrt(delta^T S delta +
+        1e-8), gamma = sigma / max(threshold, 1e-10)  (fused_3l.cpp:1191-1199, fused_cpu.h:1385-1416)"""
+        B = np.concatenate(blocks, axis=1)
+        nrm = np.sqrt((B * B).sum(1))
+        dens = [nrm] + [np.sqrt((b * b).sum(1)) for b in blocks]
+        f = np.empty((B.shape[0], self.uq_D))
+        f[:, :self.uq_rp] = (B @ self.uq_R) / (nrm + 1.0e-12)[:, None]
+        for p in range(self.uq_D - self.uq_rp):
+            f[:, self.uq_rp + p] = np.log(dens[p] + 1.0e-12) * self.uq_scale
+        na = f.shape[0]
+        gamma, sigma, cluster = np.zeros(na), np.zeros(na), np.zeros(na)
+        for a in range(na):
+            m = int(mu[a])
+            d2 = ((f[a][None, :] - self.uq_cen[m, :self.uq_ncl[m]]) ** 2).sum(1)
+            k = int(np.argmin(d2))
+            dl = f[a] - self.uq_cen[m, k]
+            sigma[a] = np.sqrt(dl @ self.uq_icov[m, k] @ dl + 1.0e-8)
+            gamma[a] = sigma[a] / max(self.uq_thr[m, k], 1.0e-10)
+            cluster[a] = k
+        return gamma, sigma, cluster, f
 
     # ---- radial functions R[b, l, c] of layer k: MLP([T_1..T_nrb(2x - 1), emb_i, emb_j]) env(x) fac[mu_j]
     def radial(self, L, x, mi, mj):
@@ -247,7 +294,7 @@ class Model3L:
         return (e + lin) * self.oscale + self.shift[mu]
 
 
-def compute_3l(model: Model3L, mu, offset, j, rij, *, want_forces=True, bond_chunk=20000, debug=None):
+def compute_3l(model: Model3L, mu, offset, j, rij, *, want_forces=True, bond_chunk=20000, debug=None, uq=False):
     """One GRACE-3L energy + forces + virial call on a CSR bond list (arguments and results as compute_1l).
     Driver skeleton: src/fused_3l.cpp:1550-1637; bond filter bonds.h:120-162.  `debug`: dict that receives the
     per-layer tensors (numpy) by model name."""
@@ -275,6 +322,9 @@ def compute_3l(model: Model3L, mu, offset, j, rij, *, want_forces=True, bond_chu
     x = r / rc
     mi, mj = mu_t[bi_t], mu_t[bj_t]
     I_prev, h = None, 0.0
+    uq_blocks = []
+    if uq and not model.has_uq:
+        raise ValueError("GRACE-3L: the model has no UQ head")
     for L in model.layers:
         R = model.radial(L, x, mi, mj)                                            # [b, l, c]
         Uy = Y[:, :, None] * R[:, L["lt"], :]                                     # [b, nlm, c]
@@ -292,6 +342,8 @@ def compute_3l(model: Model3L, mu, offset, j, rij, *, want_forces=True, bond_chu
             T[L["K"] + "_red"] = L["redA"].apply(T, mu_t)
         I_prev, rn = model.chain(L, T, mu_t)
         h = h + rn
+        if uq:
+            uq_blocks.append(model.uq_block(L, T))
         if debug is not None:
             for key, v in T.items():
                 debug[key] = v.detach().numpy()
@@ -301,6 +353,8 @@ def compute_3l(model: Model3L, mu, offset, j, rij, *, want_forces=True, bond_chu
                 debug[L["K"] + "_I"] = I_prev.detach().numpy()
     E = model.readout(h, mu_t)
     out = {"energy": float(E.detach().sum()), "energies": E.detach().numpy().copy()}
+    if uq:
+        out["gamma"], out["atomic_sigma"], out["gmm_cluster"], out["uq_features"] = model.uq(mu_np, uq_blocks)
     if not want_forces:
         return out
     (g,) = torch.autograd.grad(E.sum(), d)

@@ -140,18 +140,19 @@ int ref_compute(void *hv, int n, const int *types, const int64_t *offset, const 
   }
 }
 
-// GRACE-1L / 2L with the UQ head (uqv6): forward only; gamma, sigma, cluster [n] per atom (Grace{1,2}LFused::enable_uq)
+// GRACE-1L / 2L / 3L with the UQ head (uqv6): forward only; gamma, sigma, cluster [n] per atom (Grace{1,2,3}LFused::enable_uq)
 int ref_compute_uq(void *hv, int n, const int *types, const int64_t *offset, const int *j, const double *rij, const double *x,
                    const int *image, const double *shifts, int nthreads, double *energy, double *gamma, double *sigma, double *cluster)
 {
   Ref *h = static_cast<Ref *>(hv);
   try {
-    if (!h->d1 && !h->d2) {
-      g_err = "UQ: a GRACE-1L or GRACE-2L driver is required (setup_types first)";
+    if (!h->d1 && !h->d2 && !h->d3) {
+      g_err = "UQ: setup_types first";
       return 1;
     }
     if (h->d1) h->d1->enable_uq();
-    else h->d2->enable_uq();
+    else if (h->d2) h->d2->enable_uq();
+    else h->d3->enable_uq();
     grace::CsrBonds src{types, offset, j, rij, x, image, shifts};
     grace::Outputs out;
     std::vector<double> f((size_t) 3 * n, 0.0);
@@ -164,7 +165,8 @@ int ref_compute_uq(void *hv, int n, const int *types, const int64_t *offset, con
     fl.uq = true;
     grace::NoExchange ex;
     if (h->d1) h->d1->compute(n, nullptr, n, n, src, out, fl, nthreads);
-    else h->d2->compute(n, nullptr, n, n, src, ex, out, fl, nthreads);
+    else if (h->d2) h->d2->compute(n, nullptr, n, n, src, ex, out, fl, nthreads);
+    else h->d3->compute(n, nullptr, n, n, src, ex, out, fl, nthreads);
     *energy = out.energy;
     return 0;
   } catch (const std::exception &e) {

@@ -150,8 +150,30 @@ def model_uq2l():
     return d
 
 
-MODELS = {"uq2l": model_uq2l, "uq2": model_uq2, "l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3el": model_l3el, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
-LAYERS = {"uq2l": 2, "uq2": 1, "l3mix": 3, "l3wide": 3, "l3pad": 3, "l3el": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
+def model_uq3l():
+    """model_l3mix with a generated uqv6 head of three basis blocks (the inputs of rho1, rho2, rho3) and four density
+    channels, centroids next to features of atoms of the alloy54 structure, one exactly on an atom"""
+    from grace_runtime_amd import kk
+    from oracle import grace_oracle_3l as go3
+    d = model_l3mix()
+    synth.add_uq_head_3l(d, rp_dim=9, max_clusters=3, seed=53)
+    pos, cell, pbc, types = structure_alloy54()
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 5.0)
+    x, t = pos[perm], types[perm]
+    rij = x[j] - np.repeat(x, np.diff(offset), axis=0) + shifts[image]
+    f = go3.compute_3l(go3.Model3L(d), t - 1, offset, j, rij, want_forces=False, uq=True)["uq_features"]
+    cen = d["uq_centroids"]
+    ncl = np.array([3, 3], np.int32)
+    for e in range(2):
+        at = np.nonzero(t - 1 == e)[0]
+        for k in range(ncl[e]):
+            cen[e, k] = f[at[(k * (len(at) - 1)) // max(ncl[e] - 1, 1)]] + (0.0 if (e, k) == (1, 2) else 0.002 * (k + 1))
+    d["uq_centroids"], d["uq_n_clusters"] = cen, ncl
+    return d
+
+
+MODELS = {"uq3l": model_uq3l, "uq2l": model_uq2l, "uq2": model_uq2, "l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3el": model_l3el, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
+LAYERS = {"uq3l": 3, "uq2l": 2, "uq2": 1, "l3mix": 3, "l3wide": 3, "l3pad": 3, "l3el": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
 
 
 def write_model(name, directory):
@@ -301,7 +323,7 @@ E2E_CASES_2L = [("config3", "fcc108", None), ("l2mix", "alloy54", 5.5), ("l2mix"
 # reference fixture models (tests/golden/ref_fixtures) on the reference's fixture cells: goldens of the compiled reference
 E2E_CASES_3L = [("l3mix", "alloy54", 5.5), ("l3mix", "triclinic", None), ("l3mix", "slab", None), ("l3mix", "molecule", None),
                 ("l3wide", "fcc108", None), ("l3nat", "config1", None), ("l3el", "alloy54", None)]
-UQ_CASES = [("uq2", "alloy54"), ("uq2", "triclinic"), ("uq2l", "alloy54"), ("uq2l", "triclinic")]
+UQ_CASES = [("uq2", "alloy54"), ("uq2", "triclinic"), ("uq2l", "alloy54"), ("uq2l", "triclinic"), ("uq3l", "alloy54"), ("uq3l", "triclinic")]
 FIXTURE_CASES_2L = [(m, c) for m in ("grace_2l_small", "grace_2l_l3", "legacy_2l_small", "legacy_2l_wide") for c in ("W54", "WMo54")]
 
 

@@ -1,4 +1,4 @@
-"""The UQ head of GRACE-1L and GRACE-2L on the GPU (k_uq through the C ABI) against the CPU oracle: gamma and sigma to 1e-9 relative in
+"""The UQ head of GRACE-1L, GRACE-2L and GRACE-3L on the GPU (k_uq through the C ABI) against the CPU oracle: gamma and sigma to 1e-9 relative in
 fp64 (1e-4 with the fp32 network), the cluster index exactly.  Needs an MI355X: run with -m gpu."""
 import os
 
@@ -9,6 +9,7 @@ import cases
 from grace_runtime_amd import kk
 from oracle import grace_oracle as go
 from oracle import grace_oracle_2l as go2
+from oracle import grace_oracle_3l as go3
 
 pytestmark = pytest.mark.gpu
 
@@ -22,13 +23,15 @@ def _bonds(struct, rc=5.0):
 
 
 def _oracle(path, name, t, offset, j, rij):
+    if cases.LAYERS[name] == 3:
+        return go3.compute_3l(go3.Model3L(path), t - 1, offset, j, rij, uq=True)
     if cases.LAYERS[name] == 2:
         return go2.compute_2l(go2.Model2L(path), t - 1, offset, j, rij, uq=True)
     return go.compute_1l(go.Model1L(path), t - 1, offset, j, rij, uq=True)
 
 
-# GRACE-2L engines compute in fp64 only
-@pytest.mark.parametrize("name,precision,tol", [("uq2", 64, 1e-9), ("uq2", 32, 1e-4), ("uq2l", 64, 1e-9)])
+# GRACE-2L and GRACE-3L engines compute in fp64 only
+@pytest.mark.parametrize("name,precision,tol", [("uq2", 64, 1e-9), ("uq2", 32, 1e-4), ("uq2l", 64, 1e-9), ("uq3l", 64, 1e-9)])
 @pytest.mark.parametrize("struct", ["alloy54", "triclinic"])
 def test_uq_matches_oracle(model_dir, name, struct, precision, tol):
     path = os.path.join(model_dir, name + ".npz")
@@ -54,7 +57,7 @@ def test_uq_matches_oracle(model_dir, name, struct, precision, tol):
     assert np.abs(eng.fetch_uq()["gamma"] / ref["gamma"] - 1).max() < tol if precision == 64 else True
 
 
-@pytest.mark.parametrize("name", ["uq2", "uq2l"])
+@pytest.mark.parametrize("name", ["uq2", "uq2l", "uq3l"])
 def test_calculator_level_call_returns_uq_in_the_callers_order(model_dir, name):
     path = os.path.join(model_dir, name + ".npz")
     model = kk.Model(path)

@@ -1,8 +1,8 @@
-"""The UQ head (uqv6, gamma only) of GRACE-1L and GRACE-2L: the CPU oracle against the compiled reference and against what the
+"""The UQ head (uqv6, gamma only) of GRACE-1L, GRACE-2L and GRACE-3L: the CPU oracle against the compiled reference and against what the
 definition fixes, and the loader's checks (no GPU needed).
 
 No fixture of the reference carries a UQ head, so the head is a generated one (tests/cases.py model_uq2, and model_uq2l: the
-reference's fixture model grace_2l_small with a generated head of two basis blocks).  The compiled
+reference's fixture model grace_2l_small with a generated head of two basis blocks, model_uq3l: three blocks).  The compiled
 reference projects the basis in fp32 (libgrace/include/grace/fused_cpu.h:1275-1283: gamma within ~1e-5 of an fp64
 projection): 1e-4 relative on gamma and sigma, the cluster index exactly."""
 import os
@@ -14,6 +14,7 @@ import cases
 from grace_runtime_amd import kk
 from oracle import grace_oracle as go
 from oracle import grace_oracle_2l as go2
+from oracle import grace_oracle_3l as go3
 from oracle import ref_lib
 
 
@@ -26,7 +27,9 @@ def _bonds(struct, rc=5.0):
 
 
 def _oracle(path, t, offset, j, rij, **kw):
-    """the oracle of the model's kind (GRACE-1L or GRACE-2L) with the UQ head evaluated"""
+    """the oracle of the model's kind (GRACE-1L, 2L or 3L) with the UQ head evaluated"""
+    if cases.LAYERS[os.path.basename(path)[:-4]] == 3:
+        return go3.compute_3l(go3.Model3L(path), t - 1, offset, j, rij, want_forces=False, uq=True, **kw), go3.Model3L(path)
     if cases.LAYERS[os.path.basename(path)[:-4]] == 2:
         return go2.compute_2l(go2.Model2L(path), t - 1, offset, j, rij, want_forces=False, uq=True, **kw), go2.Model2L(path)
     return go.compute_1l(go.Model1L(path), t - 1, offset, j, rij, want_forces=False, uq=True, **kw), go.Model1L(path)
@@ -62,7 +65,7 @@ def test_oracle_matches_golden_of_the_compiled_reference(model_dir, gold, model,
     assert np.abs(o["atomic_sigma"] / gold[tag + "/atomic_sigma"] - 1).max() < 1e-4
 
 
-@pytest.mark.parametrize("name", ["uq2", "uq2l"])
+@pytest.mark.parametrize("name", ["uq2", "uq2l", "uq3l"])
 def test_what_the_definition_fixes(model_dir, name):
     """the atom whose feature vector IS a centroid has sigma = sqrt(1e-8) and gamma = sigma / threshold; the features are
     invariants of the neighbourhood: a rotated structure gives the same gamma; gamma = sigma / threshold everywhere"""
@@ -84,11 +87,11 @@ def test_what_the_definition_fixes(model_dir, name):
     assert np.abs(np.linalg.norm(f[:, :m.uq_rp], axis=1)).max() < np.linalg.norm(m.uq_R, 2) + 1e-9     # |B R| / |B| <= |R|
     if name == "uq2":
         assert np.abs(f[:, m.uq_rp] - f[:, m.uq_rp + 1]).max() == 0.0                                 # one basis block: equal channels
-    else:                                                # two blocks: |B|^2 = |B_I2|^2 + |B_rho|^2 (the 1e-12 inside the logs: 1e-9)
-        s = m.uq_scale
-        assert m.uq_D == m.uq_rp + 3
-        assert np.abs(np.exp(2 * f[:, m.uq_rp] / s) - np.exp(2 * f[:, m.uq_rp + 1] / s) - np.exp(2 * f[:, m.uq_rp + 2] / s)).max() < \
-            1e-9 * np.exp(2 * f[:, m.uq_rp] / s).max()
+    else:                       # two / three blocks: |B|^2 = the sum of the blocks' |B_b|^2 (the 1e-12 inside the logs: 1e-9)
+        s, nb = m.uq_scale, cases.LAYERS[name]
+        assert m.uq_D == m.uq_rp + 1 + nb
+        n2 = np.exp(2 * f[:, m.uq_rp:] / s)
+        assert np.abs(n2[:, 0] - n2[:, 1:].sum(1)).max() < 1e-9 * n2[:, 0].max()
     rot = np.linalg.qr(np.random.default_rng(4).standard_normal((3, 3)))[0]
     o2, _ = _oracle(path, t, offset, j, rij @ rot.T)
     assert np.abs(o2["gamma"] - o["gamma"]).max() < 1e-9 * o["gamma"].max()
@@ -136,8 +139,11 @@ def test_heads_that_validate_and_models_without(tmp_path, uq_model, model_dir):
         plain.validate_uq()
     with pytest.raises(ValueError, match="no UQ head"):
         kk.Model(os.path.join(model_dir, "l2mix.npz")).validate_uq()
-    with pytest.raises(ValueError, match="GRACE-1L and GRACE-2L models only"):
+    with pytest.raises(ValueError, match="GRACE-3L: the model has no UQ head"):
         kk.Model(os.path.join(model_dir, "l3mix.npz")).validate_uq()
+    three = kk.Model(os.path.join(model_dir, "uq3l.npz"))
+    assert three.has_uq and three.layers == 3
+    three.validate_uq()
     two = kk.Model(os.path.join(model_dir, "uq2l.npz"))
     assert two.has_uq and two.layers == 2
     two.validate_uq()
@@ -174,3 +180,35 @@ def test_max_order_3_2l_model_with_a_head_is_refused(tmp_path):
     assert m.has_uq
     with pytest.raises(ValueError, match="max_order 3"):
         m.validate_uq()
+
+
+BAD_UQ_3L = [
+    (lambda d: d.update(uq_rp_matrix=d["uq_rp_matrix"][:-1]), "uq_rp_matrix"),
+    (lambda d: d.update(uq_feature_dim=np.array([14]), uq_centroids=np.zeros((2, 3, 14)), uq_inv_cov=np.zeros((2, 3, 14, 14))),
+     r"uq_n_density \(5\) > 4"),
+    (lambda d: d.update(uq_schema_version=np.array([3])), "schema v3 unsupported"),
+    (lambda d: d.update(uq_n_clusters=np.array([3, 0], np.int32)), "element index 1 has no GMM clusters"),
+    (lambda d: d.update(uq_rp_normalize=np.array([0])), "schema v6 expects normalize=1"),
+]
+
+
+@pytest.mark.parametrize("edit,msg", BAD_UQ_3L)
+def test_a_3l_file_with_a_broken_head_does_not_load(tmp_path, edit, msg):
+    """libgrace/src/model_3l.cpp:453-463: the GRACE-3L loader throws where the 1L / 2L loaders keep the model usable"""
+    with pytest.raises((ValueError, RuntimeError), match=msg):
+        kk.Model(_mutated(tmp_path, edit, "uq3l"))
+
+
+def test_a_3l_head_with_fewer_density_channels_loads(tmp_path):
+    """the reference accepts 1 .. 4 density channels for GRACE-3L and writes the first uq_n_density of (total, rho1, rho2, rho3)"""
+    def edit(d):
+        D = int(d["uq_rp_dim"][0]) + 2
+        d.update(uq_feature_dim=np.array([D]), uq_centroids=np.ascontiguousarray(d["uq_centroids"][:, :, :D]),
+                 uq_inv_cov=np.ascontiguousarray(d["uq_inv_cov"][:, :, :D, :D]))
+    p = _mutated(tmp_path, edit, "uq3l")
+    kk.Model(p).validate_uq()
+    t, offset, j, rij = _bonds("triclinic")
+    o = go3.compute_3l(go3.Model3L(p), t - 1, offset, j, rij, want_forces=False, uq=True)
+    if ref_lib.available():
+        r = ref_lib.RefModel(p, [0, 1]).compute_uq(t, offset, j, rij)
+        assert np.array_equal(o["gmm_cluster"], r["gmm_cluster"]) and np.abs(o["gamma"] / r["gamma"] - 1).max() < 1e-4
