@@ -997,7 +997,9 @@ constexpr int kEnergyAtomsPerBlock = 16;    // atoms of one block of k_energy (4
 // E_i = (MLP(rho[1:]) + rho[0]) out_scale + shift[mu_i] and dE/drho, fp64, one wave per atom (fused_1l.cpp:378-427;
 // legacy RMS layer norm fused_cpu.h:666-682).  A block of 4 waves shares the staged weights and walks
 // kEnergyAtomsPerBlock atoms; WLDS: the weights of the network sit in LDS (as stored and transposed), else they are
-// read from global memory.  dynamic LDS: M.wlds + 4 x (2 nlay + 4) x width doubles.
+// read from global memory.  A layer with fewer than 33 outputs splits each dot product over 64 / outputs lanes (the
+// last layer's single output: all 64).  Without structure records the block adds its energies to the total with one
+// atomic.  dynamic LDS: M.wlds + 4 x (2 nlay + 4) x width doubles.
 template<bool WLDS>
 static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *mu, int a0, int natoms, const double *rho, double *grho,
                                                          double *eatom_chunk, double *energy, int want_grad, const int *sid)
@@ -1043,9 +1045,16 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
   }
   __syncthreads();
   const int n0 = M.nrho - 1;
+  // lanes that share one output of a layer: the largest power of two g with outputs x g <= 64
+  auto group = [](int nout_) {
+    int g = 1;
+    while (g < 64 && nout_ * (g * 2) <= 64) g *= 2;
+    return g;
+  };
+  double esum = 0.0;                                // lane 0: energies of this wave's atoms (no structure records)
   for (int k4 = 0; k4 < kEnergyAtomsPerBlock / 4; k4++) {
     const int at = blockIdx.x * kEnergyAtomsPerBlock + k4 * 4 + wave;
-    if (at >= natoms) break;                        // uniform over the wave; no block barrier below
+    if (at >= natoms) break;                        // uniform over the wave; no block barrier inside the loop
     const double *r = rho + (long long) at * M.nrho;
     GR_WAVE_SYNC();                                 // the rows of the previous atom are no longer read
     for (int k = lane; k < n0; k += 64) act(0, k) = r[k + 1];
@@ -1060,19 +1069,28 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
       GR_WAVE_SYNC();
     }
     for (int L = 0; L < M.nlay; L++) {
-      for (int c = lane; c < M.nout[L]; c += 64) {
+      const int no = M.nout[L], ni = M.nin[L], g = group(no), p = lane % g;
+      for (int c0 = 0; c0 < no; c0 += 64 / g) {     // every lane walks the loop: the exchanges below need the whole wave
+        const int c = c0 + lane / g;
         double s = 0.0;
-        for (int a = 0; a < M.nin[L]; a++) s += act(L, a) * wf[L][a * M.nout[L] + c];
-        s *= M.norm[L];
-        pre(L, c) = s;
-        act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+        if (c < no) {
+#pragma unroll 4
+          for (int a = p; a < ni; a += g) s += act(L, a) * wf[L][a * no + c];
+        }
+        for (int o = g >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        if (c < no && p == 0) {
+          s *= M.norm[L];
+          pre(L, c) = s;
+          act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+        }
       }
       GR_WAVE_SYNC();
     }
     const double Ei = (act(M.nlay, 0) + r[0]) * M.out_scale + M.shift[mu[a0 + at]];
     if (lane == 0) {
       if (eatom_chunk) eatom_chunk[at] = Ei;
-      atomicAdd(energy + (sid ? 8 * sid[a0 + at] : 0), Ei);    // one (energy, virial[6]) record of 8 doubles per structure
+      if (sid) atomicAdd(energy + 8 * sid[a0 + at], Ei);    // one (energy, virial[6]) record of 8 doubles per structure
+      else esum += Ei;
     }
     if (!want_grad) continue;
     int cur = 0;
@@ -1092,13 +1110,23 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
         }
         GR_WAVE_SYNC();
       }
-      for (int a = lane; a < M.nin[L]; a += 64) {
-        double s = 0.0;
-        if (WLDS)
-          for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * wt[L][c * M.nin[L] + a];
-        else
-          for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * wf[L][(long long) a * M.nout[L] + c];
-        gbuf(cur ^ 1, a) = s * M.norm[L];
+      {
+        const int no = M.nout[L], ni = M.nin[L], g = group(ni), p = lane % g;
+        for (int b0 = 0; b0 < ni; b0 += 64 / g) {
+          const int a = b0 + lane / g;
+          double s = 0.0;
+          if (a < ni) {
+            if (WLDS) {
+#pragma unroll 4
+              for (int c = p; c < no; c += g) s += gbuf(cur, c) * wt[L][c * ni + a];
+            } else {
+#pragma unroll 4
+              for (int c = p; c < no; c += g) s += gbuf(cur, c) * wf[L][(long long) a * no + c];
+            }
+          }
+          for (int o = g >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+          if (a < ni && p == 0) gbuf(cur ^ 1, a) = s * M.norm[L];
+        }
       }
       cur ^= 1;
       GR_WAVE_SYNC();
@@ -1113,6 +1141,15 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
     double *g = grho + (long long) at * M.nrho;
     if (lane == 0) g[0] = M.out_scale;
     for (int k = lane; k < n0; k += 64) g[k + 1] = gbuf(cur, k);
+  }
+  if (!sid) {    // one atomic per block (every wave leaves the loop above and arrives here)
+    __shared__ double eblk[4];
+    if (lane == 0) eblk[wave] = esum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const double e = eblk[0] + eblk[1] + eblk[2] + eblk[3];
+      if (e != 0.0) atomicAdd(energy, e);
+    }
   }
 #undef GR_WAVE_SYNC
 #undef act
