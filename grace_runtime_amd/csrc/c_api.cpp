@@ -26,6 +26,28 @@ struct gr_model {
 };
 struct gr_engine {
   std::unique_ptr<grhip::Engine> eng;
+  // what the engine was made from: reset() makes a fresh one after a failed allocation left this one half grown
+  std::shared_ptr<grhip::Model1L> m1;
+  std::shared_ptr<grhip::Model2L> m2;
+  std::shared_ptr<grhip::Model3L> m3;
+  std::vector<int> type2mu;
+  int ntypes = 0, precision = 64, device = 0;
+  int generation = 0;                                  // counts reset(): holders of uploaded state (gr_system) upload again
+  int64_t nall_cap = INT64_MAX;                        // atoms per batch pass after an allocation failure (kept for later calls)
+  void make()
+  {
+    if (m1) eng = grhip::make_engine_1l(m1, ntypes, type2mu, precision, device);
+    else if (m2) eng = grhip::make_engine_2l(m2, ntypes, type2mu, precision, device);
+    else eng = grhip::make_engine_3l(m3, ntypes, type2mu, precision, device);
+  }
+  void reset()
+  {
+    bnl.reset();
+    lmp.reset();
+    eng.reset();    // frees every device buffer of the engine before the new one allocates
+    generation++;
+    make();
+  }
   std::vector<grhip::StageTime> times;
   std::unique_ptr<grhip::BatchDeviceNeighbors> bnl;    // lists of gr_compute_batch_device (buffers kept between calls)
   std::unique_ptr<grhip::LammpsDeviceList> lmp;       // converted list of gr_compute_lammps_device
@@ -43,7 +65,7 @@ struct gr_nlist {
 struct gr_system {
   gr_engine *eng = nullptr;
   double skin = 0.0, cutoff = 0.0;
-  int rebuilds = 0;
+  int rebuilds = 0, generation = 0;
   bool have = false, on_device = false;
   int n = 0;
   std::vector<int> types;
@@ -212,14 +234,25 @@ int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int prec
     if (!m || !type2mu || !out) throw grhip::InvalidArgument("null argument");
     *out = nullptr;
     if (ntypes < 1) throw grhip::InvalidArgument("ntypes must be positive");
-    std::vector<int> t(type2mu, type2mu + ntypes + 1);
     auto e = std::make_unique<gr_engine>();
-    if (m->m1) e->eng = grhip::make_engine_1l(m->m1, ntypes, t, precision, device);
-    else if (m->m2) e->eng = grhip::make_engine_2l(m->m2, ntypes, t, precision, device);
-    else e->eng = grhip::make_engine_3l(m->m3, ntypes, t, precision, device);
+    e->m1 = m->m1; e->m2 = m->m2; e->m3 = m->m3;
+    e->type2mu.assign(type2mu, type2mu + ntypes + 1);
+    e->ntypes = ntypes; e->precision = precision; e->device = device;
+    e->make();
     *out = e.release();
   });
 }
+
+int gr_engine_reset(gr_engine *e)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->reset();
+  });
+}
+
+void gr_set_memory_limit(int64_t bytes) { grhip::dev_bytes_limit().store(bytes > 0 ? bytes : 0); }
+int64_t gr_memory_in_use(void) { return grhip::dev_bytes_in_use().load(); }
 
 void gr_engine_free(gr_engine *e) { delete e; }
 
@@ -633,6 +666,10 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
     if (hipSetDevice(eng.device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
     // list policy of the reference (python/grace_runtime/neighbors.py:68-89): rebuild when the atoms, the cell or the
     // boundary conditions change or an atom moved more than skin / 2 since the last build
+    if (s->generation != s->eng->generation) {    // the engine was reset: what was uploaded is gone
+      s->have = false;
+      s->generation = s->eng->generation;
+    }
     bool rebuild = !s->have || n != s->n || std::memcmp(pbc, s->pbc, 3) != 0 || std::memcmp(cell, s->cell.data(), 9 * sizeof(double)) != 0 ||
                    (n > 0 && std::memcmp(types, s->types.data(), sizeof(int) * (size_t) n) != 0);
     if (!rebuild) {
@@ -974,41 +1011,60 @@ int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const 
     on_device(forces, "forces");
     on_device(virial, "virial");
     on_device(eatom, "energies");
-    if (!e->bnl) e->bnl = std::make_unique<grhip::BatchDeviceNeighbors>();
     if (!e->bnl_stream && hipStreamCreateWithFlags(&e->bnl_stream, hipStreamNonBlocking) != hipSuccess) throw grhip::Error("hipStreamCreate failed");
     // work queued by the caller on the default stream (the tensors that hold the inputs) is finished first
     if (hipDeviceSynchronize() != hipSuccess) throw grhip::Error("hipDeviceSynchronize failed");
-    grhip::BatchDeviceNeighbors &nl = *e->bnl;
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
-    // passes of whole structures with at most max_atoms atoms (at least one structure each)
-    for (int g0 = 0; g0 < nstruct;) {
-      int g1 = g0 + 1;
-      while (g1 < nstruct && (max_atoms == 0 || start[g1 + 1] - start[g0] <= max_atoms)) g1++;
-      const int ns = g1 - g0;
-      const int64_t a0 = start[g0], na = start[g1] - a0;
-      nl.build(ns, natoms + g0, positions + 3 * a0, cells + 9 * (size_t) g0, pbc + 3 * (size_t) g0, rc, e->bnl_stream);
-      // atom types: 4 bytes per atom to the host, where the element tiles of the tile GEMMs are laid out
-      std::vector<int> ty((size_t) na);
-      if (na > 0 && hipMemcpyAsync(ty.data(), types + a0, sizeof(int) * (size_t) na, hipMemcpyDeviceToHost, e->bnl_stream) != hipSuccess)
-        throw grhip::Error("copy of the atom types failed");
-      if (hipStreamSynchronize(e->bnl_stream) != hipSuccess) throw grhip::Error("the device neighbour search failed");
-      grhip::DeviceCsr in;
-      in.n = (int) na;
-      in.types = ty.data();
-      in.nb = nl.nb;
-      in.offset = nl.offset.as<int64_t>();
-      in.j = nl.j.as<int>();
-      in.rij = nl.rij.as<double>();
-      in.nstruct = ns;
-      in.sid = nl.sid.data();
-      e->eng->upload_device(in);
-      e->eng->run(fl);
-      e->eng->fetch_batch_device(ns, energy + g0, forces ? forces + 3 * a0 : nullptr, virial ? virial + 6 * (size_t) g0 : nullptr,
-                                 fl.eatom ? eatom + a0 : nullptr);
-      if (passes) ++*passes;
-      g0 = g1;
+    // passes of whole structures with at most `limit` atoms (at least one structure each); every pass overwrites its outputs
+    auto once = [&](int64_t limit) {
+      if (passes) *passes = 0;
+      if (!e->bnl) e->bnl = std::make_unique<grhip::BatchDeviceNeighbors>();
+      grhip::BatchDeviceNeighbors &nl = *e->bnl;
+      for (int g0 = 0; g0 < nstruct;) {
+        int g1 = g0 + 1;
+        while (g1 < nstruct && start[g1 + 1] - start[g0] <= limit) g1++;
+        const int ns = g1 - g0;
+        const int64_t a0 = start[g0], na = start[g1] - a0;
+        nl.build(ns, natoms + g0, positions + 3 * a0, cells + 9 * (size_t) g0, pbc + 3 * (size_t) g0, rc, e->bnl_stream);
+        // atom types: 4 bytes per atom to the host, where the element tiles of the tile GEMMs are laid out
+        std::vector<int> ty((size_t) na);
+        if (na > 0 && hipMemcpyAsync(ty.data(), types + a0, sizeof(int) * (size_t) na, hipMemcpyDeviceToHost, e->bnl_stream) != hipSuccess)
+          throw grhip::Error("copy of the atom types failed");
+        if (hipStreamSynchronize(e->bnl_stream) != hipSuccess) throw grhip::Error("the device neighbour search failed");
+        grhip::DeviceCsr in;
+        in.n = (int) na;
+        in.types = ty.data();
+        in.nb = nl.nb;
+        in.offset = nl.offset.as<int64_t>();
+        in.j = nl.j.as<int>();
+        in.rij = nl.rij.as<double>();
+        in.nstruct = ns;
+        in.sid = nl.sid.data();
+        e->eng->upload_device(in);
+        e->eng->run(fl);
+        e->eng->fetch_batch_device(ns, energy + g0, forces ? forces + 3 * a0 : nullptr, virial ? virial + 6 * (size_t) g0 : nullptr,
+                                   fl.eatom ? eatom + a0 : nullptr);
+        if (passes) ++*passes;
+        g0 = g1;
+      }
+    };
+    // After an allocation failure: a fresh engine (the failed one is half grown) and passes of half as many atoms, down
+    // to 16384, from the first structure again; the limit found is kept for later calls (python/kk/kk_core.cpp:1452-1484)
+    int64_t limit = std::min<int64_t>(max_atoms == 0 ? INT64_MAX : max_atoms, e->nall_cap);
+    for (;;) {
+      try {
+        once(limit);
+        return;
+      } catch (const std::bad_alloc &) {
+        const int64_t tried = std::min<int64_t>(limit, N);
+        e->reset();
+        if (tried <= 16384)
+          throw grhip::Error("the batch (" + std::to_string(N) + " atoms) does not fit the GPU memory even in passes of " + std::to_string(tried) +
+                             " atoms; use a GPU with more memory");
+        limit = e->nall_cap = std::max<int64_t>(16384, tried / 2);
+      }
     }
   });
 }

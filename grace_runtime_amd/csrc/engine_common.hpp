@@ -7,6 +7,7 @@
 #include "kernels_1l.hpp"
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstring>
 #include <numeric>
@@ -20,6 +21,20 @@ namespace grhip {
       throw Error(std::string("HIP error: ") + hipGetErrorString(e_) + " in " #expr " (" __FILE__ ":" + std::to_string(__LINE__) + ")"); \
   } while (0)
 
+// Device memory held by the library's buffers and an optional cap on it (0: none).  With a cap an allocation that would
+// pass it fails like one the device refuses (std::bad_alloc), which lets a GPU be shared by budget and lets the
+// retry paths be exercised without exhausting the device.
+inline std::atomic<long long> &dev_bytes_in_use()
+{
+  static std::atomic<long long> v{0};
+  return v;
+}
+inline std::atomic<long long> &dev_bytes_limit()
+{
+  static std::atomic<long long> v{0};
+  return v;
+}
+
 // device allocation owned by the engine
 struct DevBuf {
   void *p = nullptr;
@@ -30,7 +45,10 @@ struct DevBuf {
   ~DevBuf() { release(); }
   void release()
   {
-    if (p) (void) hipFree(p);
+    if (p) {
+      (void) hipFree(p);
+      dev_bytes_in_use() -= (long long) bytes;
+    }
     p = nullptr;
     bytes = 0;
   }
@@ -40,6 +58,8 @@ struct DevBuf {
     if (need <= bytes && p) return;
     release();
     const size_t want = std::max<size_t>(need + need / 8, 256);
+    const long long cap = dev_bytes_limit().load();
+    if (cap > 0 && dev_bytes_in_use().load() + (long long) want > cap) throw std::bad_alloc();
     hipError_t e = hipMalloc(&p, want);
     if (e != hipSuccess) {
       p = nullptr;
@@ -47,6 +67,7 @@ struct DevBuf {
       throw std::bad_alloc();
     }
     bytes = want;
+    dev_bytes_in_use() += (long long) want;
   }
   template<class U> U *as() const { return static_cast<U *>(p); }
 };

@@ -78,6 +78,17 @@ def memory_info():
     return int(free), int(total)
 
 
+def memory_in_use() -> int:
+    """bytes of device memory held by the library's buffers (all engines of the process)"""
+    return int(_lib.lib().gr_memory_in_use())
+
+
+def set_memory_limit(nbytes: int):
+    """cap on memory_in_use(): an allocation beyond it fails like one the device refuses (MemoryError, or the smaller
+    passes of Batch); 0 removes the cap"""
+    _lib.lib().gr_set_memory_limit(int(nbytes))
+
+
 def _dev():
     if _state["device"] is None:
         initialize(0)
@@ -168,6 +179,11 @@ class Engine:
 
     def cutoff(self, t1: int, t2: int) -> float:
         return _lib.lib().gr_engine_cutoff(self._h, int(t1), int(t2))
+
+    def reset(self):
+        """a fresh engine in place of this one, every device buffer dropped (after an allocation failure)"""
+        check(_lib.lib().gr_engine_reset(self._h))
+        self._n = 0
 
     def cutoff_matrix(self):
         k = len(self.species)
@@ -455,6 +471,7 @@ class Batch:
         self.passes = 0
         self.keep_buffers = False
         self.chunksize = 0
+        self._nall_cap = 1 << 62    # atoms per pass after an allocation failure (python/kk/kk_core.cpp:1461: nall_cap)
 
     def release_buffers(self):
         pass
@@ -485,17 +502,30 @@ class Batch:
         # every structure's list is built on the host (in parallel); the structures go through the GPU in passes of whole
         # structures with at most max_nall atoms (python/kk/kk_core.cpp:1311-1347: ONE pass unless the batch is larger)
         start = np.concatenate([[0], np.cumsum(natoms, dtype=np.int64)])
-        self.passes, g0 = 0, 0
-        while g0 < S:
-            g1 = g0 + 1
-            while g1 < S and start[g1 + 1] - start[g0] <= int(max_nall):
-                g1 += 1
-            a0, a1 = int(start[g0]), int(start[g1])
-            check(_lib.lib().gr_compute_batch(self.engine._h, g1 - g0, ptr(natoms[g0:g1]), ptr(types[a0:a1]), ptr(pos[a0:a1]), ptr(cells[g0:g1]),
-                                              ptr(pb[g0:g1]), flags, min(nth, 16), ptr(out["energy"][g0:g1]), ptr(f[a0:a1]), ptr(v[g0:g1]),
-                                              ptr(ea[a0:a1]) if energies else None))
-            self.passes += 1 if a1 > a0 else 0
-            g0 = g1
+        # after an allocation failure: a fresh engine and passes of half as many atoms, down to 16384, from the first
+        # structure again (every pass overwrites its outputs); python/kk/kk_core.cpp:1452-1484 compute_with_retry
+        limit = min(int(max_nall), self._nall_cap)
+        while True:
+            try:
+                self.passes, g0 = 0, 0
+                while g0 < S:
+                    g1 = g0 + 1
+                    while g1 < S and start[g1 + 1] - start[g0] <= limit:
+                        g1 += 1
+                    a0, a1 = int(start[g0]), int(start[g1])
+                    check(_lib.lib().gr_compute_batch(self.engine._h, g1 - g0, ptr(natoms[g0:g1]), ptr(types[a0:a1]), ptr(pos[a0:a1]),
+                                                      ptr(cells[g0:g1]), ptr(pb[g0:g1]), flags, min(nth, 16), ptr(out["energy"][g0:g1]),
+                                                      ptr(f[a0:a1]), ptr(v[g0:g1]), ptr(ea[a0:a1]) if energies else None))
+                    self.passes += 1 if a1 > a0 else 0
+                    g0 = g1
+                break
+            except MemoryError:
+                tried = min(limit, N)
+                self.engine.reset()
+                if tried <= 16384:
+                    raise RuntimeError(f"the batch ({N} atoms) does not fit the GPU memory even in passes of {tried} atoms; "
+                                       "use a GPU with more memory") from None
+                limit = self._nall_cap = max(16384, tried // 2)
         if not energy_only:
             out["forces"], out["virial"] = f, v
         if energies:

@@ -70,6 +70,17 @@ void gr_model_free(gr_model *m);
  * only, GR_INVALID for GRACE-2L / 3L models). */
 int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int precision, int device, gr_engine **out);
 void gr_engine_free(gr_engine *e);
+/* Drops the engine and every device buffer it holds and makes a fresh one from the same model, types, precision and
+ * device: what the reference's GPU module does with an engine that an allocation failure left half grown
+ * (python/kk/kk_core.cpp:478-497 poison / drop, the next compute attaches a fresh engine).  A structure uploaded before
+ * is gone; a gr_system on this engine notices and uploads its structure again. */
+int gr_engine_reset(gr_engine *e);
+/* Bytes of device memory the library's buffers hold (all engines of the process), and a cap on them: with a cap an
+ * allocation that would pass it fails as one the device refuses (GR_NOMEM, or the retry of gr_compute_batch_device).
+ * 0: no cap.  The part of the reference module's memory_info() / chunk-by-free-memory policy (kk/support.h:415-450) that
+ * the caller controls; it also lets the allocation-failure paths be tested without exhausting a GPU. */
+void gr_set_memory_limit(int64_t bytes);
+int64_t gr_memory_in_use(void);
 /* Grace1LFused::cutoff(t1, t2): fused_1l.h:32 */
 double gr_engine_cutoff(const gr_engine *e, int t1, int t2);
 
@@ -209,7 +220,11 @@ int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *ty
  * max_atoms: the structures go through the engine in passes of whole structures with at most max_atoms atoms (at least
  * one structure per pass), which bounds the engine's device memory as max_nall does in the reference
  * (python/kk/kk_core.cpp:1311-1347; this list holds no ghost images, so atoms stand for the reference's atoms + images);
- * 0: one pass.  *passes (may be NULL): engine passes made. */
+ * 0: one pass.  *passes (may be NULL): engine passes made.
+ * Allocation failure (python/kk/kk_core.cpp:1452-1484 compute_with_retry): the engine is reset and the batch runs again
+ * from its first structure in passes of half as many atoms, down to 16384; the limit found is kept by the engine for
+ * later calls.  When 16384 atoms per pass do not fit either: GR_ERROR "... does not fit the GPU memory ...", the engine
+ * reset and usable. */
 int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
                             const unsigned char *pbc, unsigned flags, int64_t max_atoms, double *energy, double *forces, double *virial,
                             double *eatom, int *passes);

@@ -135,3 +135,55 @@ def test_argument_errors(model_dir):
     e2 = torch.full((2,), 5.0, dtype=torch.float64, device=dev)
     b.compute_device([0, 0], ty[:0], x[:0], np.stack([c, c]), np.stack([pb, pb]), e2)
     assert e2.tolist() == [0.0, 0.0]
+
+
+def test_allocation_failure_halves_the_passes_and_keeps_the_limit(model_dir):
+    """python/kk/kk_core.cpp:1452-1484: after an allocation failure the batch runs again from its first structure in
+    passes of half as many atoms (not below 16384), on a fresh engine, and later calls start from the limit found.  The
+    failure is forced with the library's own memory cap (the GPU is never exhausted)."""
+    eng = _engine(model_dir, "config5", ["Al", "Ni", "Ti"])
+    structs = [(p, c, [True, True, True], t) for p, c, t in cases.structures_config5(440)]
+    natoms, types, pos, cells, pbc = _pack(structs)
+    N = int(natoms.sum())
+    assert 33000 < N < 65000                      # one halving reaches a pass size above the floor of 16384
+    b = kk.Batch(eng.model, ["Al", "Ni", "Ti"])
+    try:
+        ref = _device_run(b, natoms, types, pos, cells, pbc, max_nall=N // 2)
+        assert b.passes >= 2
+        held = kk.memory_in_use()
+        b.engine.reset()
+        base = kk.memory_in_use()                 # the weights of the engines alive in this process
+        assert 0 < base < held
+        # enough for passes of N / 2 atoms, not for one pass of N
+        kk.set_memory_limit(base + int(1.35 * (held - base)))
+        out = _device_run(b, natoms, types, pos, cells, pbc)
+        assert b.passes >= 2
+        _compare(out, ref)
+        p_first = b.passes
+        out = _device_run(b, natoms, types, pos, cells, pbc)        # the limit is kept: no failure this time, the same passes
+        assert b.passes == p_first
+        _compare(out, ref)
+        host = b.compute(natoms, types, pos, cells, pbc, energies=True)
+        assert b.passes >= 2
+        _compare(host, ref)
+        # nothing fits: an error that says so, and an engine that works again once the cap is lifted
+        kk.set_memory_limit(base + (held - base) // 50)
+        with pytest.raises(RuntimeError, match="does not fit the GPU memory"):
+            _device_run(b, natoms, types, pos, cells, pbc)
+        with pytest.raises(RuntimeError, match="does not fit the GPU memory"):
+            b.compute(natoms, types, pos, cells, pbc)
+        kk.set_memory_limit(0)
+        sub = _pack(structs[:20])
+        _compare(_device_run(b, *sub), b.compute(*sub, energies=True))
+    finally:
+        kk.set_memory_limit(0)
+
+
+def test_engine_reset_is_seen_by_a_system(model_dir):
+    model = kk.Model(os.path.join(model_dir, "mix2.npz"))
+    s = kk.System(model, ["Mo", "W"], skin=0.3)
+    p, c, pb, t = cases.structure_alloy54()
+    a = s.compute(t, p, c, pb)
+    s.engine.reset()
+    b = s.compute(t, p, c, pb)
+    assert s.rebuilds == 2 and abs(a["energy"] - b["energy"]) < 1e-9 and np.abs(a["forces"] - b["forces"]).max() < 1e-9
