@@ -889,6 +889,14 @@ int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *ty
                      const unsigned char *pbc, unsigned flags, int nthreads, double *energy, double *forces, double *virial,
                      double *eatom)
 {
+  return gr_compute_batch_uq(e, nstruct, natoms, types, positions, cells, pbc, flags, nthreads, energy, forces, virial, eatom, nullptr, nullptr,
+                             nullptr);
+}
+
+int gr_compute_batch_uq(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
+                        const unsigned char *pbc, unsigned flags, int nthreads, double *energy, double *forces, double *virial,
+                        double *eatom, double *gamma, double *sigma, double *cluster)
+{
   return guarded([&] {
     if (!e || nstruct < 0 || (nstruct > 0 && (!natoms || !cells || !pbc))) throw grhip::InvalidArgument("null argument");
     if (nstruct == 0) return;
@@ -962,15 +970,21 @@ int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *ty
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.uq = gamma || sigma || cluster;
     e->eng->run(fl);
     std::vector<double> f((size_t) 3 * N), ea(fl.eatom ? N : 0);
     e->eng->fetch_batch(nstruct, energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
+    std::vector<double> ug(gamma ? N : 0), us(sigma ? N : 0), uc(cluster ? N : 0);
+    if (fl.uq) e->eng->fetch_uq(gamma ? ug.data() : nullptr, sigma ? us.data() : nullptr, cluster ? uc.data() : nullptr);
     for (int s = 0; s < nstruct; s++)
       for (int64_t q = 0; q < natoms[s]; q++) {
         const int64_t a = start[s] + nls[s].perm[q], w = start[s] + q;
         if (forces && !fl.energy_only)
           for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) w + d];
         if (fl.eatom) eatom[a] = ea[w];
+        if (gamma) gamma[a] = ug[w];
+        if (sigma) sigma[a] = us[w];
+        if (cluster) cluster[a] = uc[w];
       }
   });
 }
@@ -978,6 +992,14 @@ int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *ty
 int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
                             const unsigned char *pbc, unsigned flags, int64_t max_atoms, double *energy, double *forces, double *virial,
                             double *eatom, int *passes)
+{
+  return gr_compute_batch_device_uq(e, nstruct, natoms, types, positions, cells, pbc, flags, max_atoms, energy, forces, virial, eatom, nullptr,
+                                    nullptr, nullptr, passes);
+}
+
+int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
+                               const unsigned char *pbc, unsigned flags, int64_t max_atoms, double *energy, double *forces, double *virial,
+                               double *eatom, double *gamma, double *sigma, double *cluster, int *passes)
 {
   return guarded([&] {
     if (passes) *passes = 0;
@@ -1011,12 +1033,16 @@ int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const 
     on_device(forces, "forces");
     on_device(virial, "virial");
     on_device(eatom, "energies");
+    on_device(gamma, "gamma");
+    on_device(sigma, "atomic_sigma");
+    on_device(cluster, "gmm_cluster");
     if (!e->bnl_stream && hipStreamCreateWithFlags(&e->bnl_stream, hipStreamNonBlocking) != hipSuccess) throw grhip::Error("hipStreamCreate failed");
     // work queued by the caller on the default stream (the tensors that hold the inputs) is finished first
     if (hipDeviceSynchronize() != hipSuccess) throw grhip::Error("hipDeviceSynchronize failed");
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.uq = gamma || sigma || cluster;
     // passes of whole structures with at most `limit` atoms (at least one structure each); every pass overwrites its outputs
     auto once = [&](int64_t limit) {
       if (passes) *passes = 0;
@@ -1046,6 +1072,7 @@ int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const 
         e->eng->run(fl);
         e->eng->fetch_batch_device(ns, energy + g0, forces ? forces + 3 * a0 : nullptr, virial ? virial + 6 * (size_t) g0 : nullptr,
                                    fl.eatom ? eatom + a0 : nullptr);
+        if (fl.uq) e->eng->fetch_uq(gamma ? gamma + a0 : nullptr, sigma ? sigma + a0 : nullptr, cluster ? cluster + a0 : nullptr);
         if (passes) ++*passes;
         g0 = g1;
       }

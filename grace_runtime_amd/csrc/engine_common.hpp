@@ -720,9 +720,10 @@ class EngineBase : public Engine {
     if (!ran_ || !ran_uq_) throw Error("fetch_uq() needs a run with the UQ flag");
     HIP_CHECK(hipStreamSynchronize(stream_));
     if (n_ == 0) return;
-    if (gamma) HIP_CHECK(hipMemcpy(gamma, uq_gamma_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
-    if (sigma) HIP_CHECK(hipMemcpy(sigma, uq_sigma_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
-    if (cluster) HIP_CHECK(hipMemcpy(cluster, uq_cluster_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
+    // host or device destinations (the batch call on device arrays hands in device pointers)
+    if (gamma) HIP_CHECK(hipMemcpy(gamma, uq_gamma_.p, sizeof(double) * n_, hipMemcpyDefault));
+    if (sigma) HIP_CHECK(hipMemcpy(sigma, uq_sigma_.p, sizeof(double) * n_, hipMemcpyDefault));
+    if (cluster) HIP_CHECK(hipMemcpy(cluster, uq_cluster_.p, sizeof(double) * n_, hipMemcpyDefault));
   }
   int64_t last_edge_count() override
   {

@@ -478,8 +478,8 @@ class Batch:
 
     def compute(self, natoms, types, positions, cells, pbc, energies=False, uq=False, energy_only=False,
                 max_nall=1 << 21, dispersion_parts=False):
-        if uq:
-            raise ValueError("the UQ head is evaluated per structure (System.compute(uq=True)), not for batches")
+        if uq and not self.engine.model.has_uq:
+            raise ValueError("uq=True: the model has no UQ head")
         natoms = np.asarray(natoms, dtype=np.int32)
         types = as_array(types, np.int32)
         pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
@@ -496,6 +496,7 @@ class Batch:
         out = {"energy": np.zeros(S)}
         f, v = np.zeros((N, 3)), np.zeros((S, 6))
         ea = np.zeros(N) if energies else None
+        ug, us, uc = (np.zeros(N), np.zeros(N), np.zeros(N)) if uq else (None, None, None)
         pb = np.ascontiguousarray(pbc, dtype=np.uint8)
         flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
         nth = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else 1
@@ -513,9 +514,11 @@ class Batch:
                     while g1 < S and start[g1 + 1] - start[g0] <= limit:
                         g1 += 1
                     a0, a1 = int(start[g0]), int(start[g1])
-                    check(_lib.lib().gr_compute_batch(self.engine._h, g1 - g0, ptr(natoms[g0:g1]), ptr(types[a0:a1]), ptr(pos[a0:a1]),
-                                                      ptr(cells[g0:g1]), ptr(pb[g0:g1]), flags, min(nth, 16), ptr(out["energy"][g0:g1]),
-                                                      ptr(f[a0:a1]), ptr(v[g0:g1]), ptr(ea[a0:a1]) if energies else None))
+                    check(_lib.lib().gr_compute_batch_uq(self.engine._h, g1 - g0, ptr(natoms[g0:g1]), ptr(types[a0:a1]), ptr(pos[a0:a1]),
+                                                         ptr(cells[g0:g1]), ptr(pb[g0:g1]), flags, min(nth, 16), ptr(out["energy"][g0:g1]),
+                                                         ptr(f[a0:a1]), ptr(v[g0:g1]), ptr(ea[a0:a1]) if energies else None,
+                                                         ptr(ug[a0:a1]) if uq else None, ptr(us[a0:a1]) if uq else None,
+                                                         ptr(uc[a0:a1]) if uq else None))
                     self.passes += 1 if a1 > a0 else 0
                     g0 = g1
                 break
@@ -530,6 +533,8 @@ class Batch:
             out["forces"], out["virial"] = f, v
         if energies:
             out["energies"] = ea
+        if uq:
+            out["gamma"], out["atomic_sigma"], out["gmm_cluster"] = ug, us, uc
         return out
 
     def compute_device(self, natoms, types, positions, cells, pbc, energy, forces=None, virial=None, energies=None,
@@ -537,11 +542,12 @@ class Batch:
         """`Batch.compute_device` of the reference module (python/kk/kk_module.cpp:142-193): `types` int32 [N],
         `positions` float64 [N, 3] and the outputs `energy` [S], `forces` [N, 3], `virial` [S, 6], `energies` [N] are
         arrays ON the module's GPU (torch tensors, or anything with `__cuda_array_interface__` such as CuPy arrays),
-        read and written in place; `natoms`, `cells`, `pbc` are host arrays.  The neighbour lists are built on the
+        read and written in place; `natoms`, `cells`, `pbc` are host arrays.  `gamma`, `atomic_sigma`, `gmm_cluster`
+        (float64 [N] on the GPU, each optional) receive the UQ head's outputs.  The neighbour lists are built on the
         device; positions, forces and energies never visit the host.  `max_nall`: atoms per engine pass (whole
         structures, at least one per pass); `passes` holds the number of passes made."""
-        if gamma is not None or atomic_sigma is not None or gmm_cluster is not None:
-            raise ValueError("the UQ head is evaluated per structure (System.compute(uq=True)), not for batches: no UQ head here")
+        if (gamma is not None or atomic_sigma is not None or gmm_cluster is not None) and not self.engine.model.has_uq:
+            raise ValueError("gamma / atomic_sigma / gmm_cluster: the model has no UQ head")
         natoms = np.ascontiguousarray(natoms, dtype=np.int32)
         cells = np.ascontiguousarray(cells, dtype=np.float64).reshape(-1, 3, 3)
         pb = np.ascontiguousarray(np.asarray(pbc, dtype=bool).reshape(-1, 3), dtype=np.uint8)
@@ -554,12 +560,14 @@ class Batch:
         p_f = _device_pointer(forces, "forces", (N, 3), "float64") if forces is not None else None
         p_v = _device_pointer(virial, "virial", (S, 6), "float64") if virial is not None else None
         p_ea = _device_pointer(energies, "energies", (N,), "float64") if energies is not None else None
+        p_uq = [_device_pointer(a, nm, (N,), "float64") if a is not None else None
+                for a, nm in ((gamma, "gamma"), (atomic_sigma, "atomic_sigma"), (gmm_cluster, "gmm_cluster"))]
         flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies is not None else 0)
         if int(max_nall) < 1:
             raise ValueError("max_nall must be >= 1")
         passes = C.c_int(0)
-        check(_lib.lib().gr_compute_batch_device(self.engine._h, S, ptr(natoms), p_types, p_pos, ptr(cells), ptr(pb), flags, int(max_nall),
-                                                 p_e, p_f, p_v, p_ea, C.byref(passes)))
+        check(_lib.lib().gr_compute_batch_device_uq(self.engine._h, S, ptr(natoms), p_types, p_pos, ptr(cells), ptr(pb), flags, int(max_nall),
+                                                    p_e, p_f, p_v, p_ea, p_uq[0], p_uq[1], p_uq[2], C.byref(passes)))
         self.passes = passes.value if N else 0
 
 

@@ -228,6 +228,16 @@ int gr_compute_batch(gr_engine *e, int nstruct, const int *natoms, const int *ty
 int gr_compute_batch_device(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
                             const unsigned char *pbc, unsigned flags, int64_t max_atoms, double *energy, double *forces, double *virial,
                             double *eatom, int *passes);
+/* The two batch calls with the UQ head evaluated as well (Batch.compute(uq=True) and the gamma / atomic_sigma /
+ * gmm_cluster outputs of Batch.compute_device, python/kk/kk_api.h:116-156): gamma, sigma, cluster [N] per atom in the
+ * caller's order, host arrays for gr_compute_batch_uq and arrays of the engine's GPU for gr_compute_batch_device_uq;
+ * each may be NULL, all NULL: the call without UQ.  A model without a usable head gives GR_INVALID. */
+int gr_compute_batch_uq(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
+                        const unsigned char *pbc, unsigned flags, int nthreads, double *energy, double *forces, double *virial,
+                        double *eatom, double *gamma, double *sigma, double *cluster);
+int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, const int *types, const double *positions, const double *cells,
+                               const unsigned char *pbc, unsigned flags, int64_t max_atoms, double *energy, double *forces, double *virial,
+                               double *eatom, double *gamma, double *sigma, double *cluster, int *passes);
 int gr_engine_upload_batch(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
                            const double *positions, const int *image, const double *shifts, int64_t nimages, int nstruct,
                            const int *struct_of_atom);

@@ -93,3 +93,40 @@ def test_uq_errors(model_dir):
     pos, cell, pbc, types = cases.structure_alloy54()
     with pytest.raises(ValueError, match="no usable UQ head"):
         two.compute(types, pos, cell, pbc, uq=True)
+
+
+@pytest.mark.parametrize("name", ["uq2", "uq2l", "uq3l"])
+def test_batches_return_uq_per_atom_in_the_callers_order(model_dir, name):
+    """Batch.compute(uq=True) and the gamma / atomic_sigma / gmm_cluster outputs of Batch.compute_device
+    (python/kk/kk_api.h:116-156) against one System call per structure, in one pass and in passes of one structure"""
+    import torch
+    model = kk.Model(os.path.join(model_dir, name + ".npz"))
+    structs = [cases.structure_alloy54(), cases.structure_triclinic(), cases.structure_slab()]
+    natoms = np.array([len(s[0]) for s in structs], np.int32)
+    pos = np.concatenate([s[0] for s in structs])
+    cells = np.stack([s[1] for s in structs])
+    pbc = np.stack([np.asarray(s[2], bool) for s in structs])
+    types = np.concatenate([s[3] for s in structs]).astype(np.int32)
+    one = [kk.System(model, ["Mo", "W"], skin=0.0).compute(s[3], s[0], s[1], s[2], uq=True) for s in structs]
+    want = {k: np.concatenate([o[k] for o in one]) for k in ("gamma", "atomic_sigma", "gmm_cluster")}
+    b = kk.Batch(model, ["Mo", "W"])
+    dev = torch.device("cuda", kk.device())
+    for max_nall in (1 << 21, 1):
+        out = b.compute(natoms, types, pos, cells, pbc, uq=True, max_nall=max_nall)
+        assert b.passes == (1 if max_nall > 1 else 3)
+        assert np.array_equal(out["gmm_cluster"], want["gmm_cluster"])
+        assert np.abs(out["gamma"] / want["gamma"] - 1).max() < 1e-9 and np.abs(out["atomic_sigma"] / want["atomic_sigma"] - 1).max() < 1e-9
+        assert np.abs(out["energy"] - np.array([o["energy"] for o in one])).max() < 1e-9
+        g, sg, cl = (torch.full((len(types),), 7.0, dtype=torch.float64, device=dev) for _ in range(3))
+        e = torch.zeros(3, dtype=torch.float64, device=dev)
+        b.compute_device(natoms, torch.as_tensor(types, device=dev), torch.as_tensor(pos, device=dev), cells, pbc, e, gamma=g,
+                         atomic_sigma=sg, gmm_cluster=cl, energy_only=True, max_nall=max_nall)
+        assert np.array_equal(cl.cpu().numpy(), want["gmm_cluster"])
+        assert np.abs(g.cpu().numpy() / want["gamma"] - 1).max() < 1e-9 and np.abs(sg.cpu().numpy() / want["atomic_sigma"] - 1).max() < 1e-9
+    # only one of the three outputs
+    g = torch.zeros(len(types), dtype=torch.float64, device=dev)
+    b.compute_device(natoms, torch.as_tensor(types, device=dev), torch.as_tensor(pos, device=dev), cells, pbc, e, gamma=g)
+    assert np.abs(g.cpu().numpy() / want["gamma"] - 1).max() < 1e-9
+    plain = kk.Batch(kk.Model(os.path.join(model_dir, "mix2.npz")), ["Mo", "W"])
+    with pytest.raises(ValueError, match="no UQ head"):
+        plain.compute(natoms, types, pos, cells, pbc, uq=True)
