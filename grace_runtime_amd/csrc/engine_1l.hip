@@ -154,7 +154,7 @@ template<class T> void Engine1L<T>::build()
     fcAA1_.build(m.fc_AA1, liveAA1, nlm_, CFP_, CP_, CFP_, drow_);
     if (order4_) {
       fcAA2_.build(m.fc_AA2, liveAA2, nlm_, CFP_, CP_, CFP_, drow_);
-      fcAA12_.build(m.fc_AA1, liveAA1, fcAA1_, m.fc_AA2, liveAA2, fcAA2_, nlm_, drow_);
+      fcAA12_.build(m.fc_AA1, liveAA1, fcAA1_, m.fc_AA2, liveAA2, fcAA2_, nlm_, drow_, true);
     }
   }
 
@@ -349,7 +349,9 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   stage("zero_grads", [&] {
     HIP_CHECK(hipMemsetAsync(gA, 0, na * nlm_ * CP_ * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(gA1, 0, na * nlm_ * CFP_ * sizeof(T), stream_));
-    HIP_CHECK(hipMemsetAsync(gAA, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
+    // with the AAAA stage the merged FC reverse WRITES every row of gAA (a job per function) and the rho reverse of the
+    // sources A and AA runs after it: no fill of the largest adjoint, and no read of it by the FC reverse
+    if (!order4_) HIP_CHECK(hipMemsetAsync(gAA, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
     // with the specialised product kernels gAA1 and gAA2 are written (not accumulated) by their first producer
     if (!jit_all_) HIP_CHECK(hipMemsetAsync(gAA1, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(gAAA, 0, na * nAAA_ * CFP_ * sizeof(T), stream_));
@@ -358,9 +360,12 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
       HIP_CHECK(hipMemsetAsync(gAAAA, 0, na * nAAAA_ * CFP_ * sizeof(T), stream_));
     }
   });
+  const int jobs_a_aa = redrho_.d.ncol[0] + redrho_.d.ncol[1];    // jobs of the sources A and AA (the first two)
   stage("reduce_rho_bwd", [&] {
-    hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, redrho_.njobs), dim3(64), 0, stream_, redrho_.d, mu_.as<int>(), tiles, grho_.as<double>(), gA, gAA,
-                       gAAA, gAAAA);
+    const int first = order4_ ? jobs_a_aa : 0;
+    if (redrho_.njobs > first)
+      hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, redrho_.njobs - first), dim3(64), 0, stream_, redrho_.d, mu_.as<int>(), tiles, grho_.as<double>(),
+                         gA, gAA, gAAA, gAAAA, first);
   });
   // accL / accR: add to the stored adjoint or overwrite it (specialised kernels; the table-driven ones always add)
   auto prod_bwd = [&](const char *name, DevProd &P, const T *L, const T *R, const T *g, T *gL, T *gR, int sl, int sr, int accL, int accR) {
@@ -390,8 +395,13 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   if (order4_) {
     // fc_AA1 and fc_AA2 share their inputs: one pass over gAA and gA for both
     stage("fc_AA12_bwd", [&] {
-      launch_gemm(fcAA12_.bwd_l, kf, kf, kf, gAA1, nAA_, gAA2, nAA_, gAA, nAA_, 1);
+      launch_gemm(fcAA12_.bwd_l, kf, kf, kf, gAA1, nAA_, gAA2, nAA_, gAA, nAA_, 0);
       launch_gemm(fcAA12_.bwd_r, kf, kf, ka, gAA1, nAA_, gAA2, nAA_, gA, nlm_, 1);
+    });
+    stage("reduce_rho_bwd_A_AA", [&] {
+      if (jobs_a_aa > 0)
+        hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, jobs_a_aa), dim3(64), 0, stream_, redrho_.d, mu_.as<int>(), tiles, grho_.as<double>(), gA, gAA,
+                           gAAA, gAAAA, 0);
     });
   } else {
     fc_bwd("fc_AA1_bwd", fcAA1_, gAA1, gAA, gA, nAA_, kf);

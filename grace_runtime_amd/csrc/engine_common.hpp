@@ -250,13 +250,15 @@ template<class T> struct DevFc {
 // adjoint of the right input.  Source 0 of a segment is the output adjoint of the first layer, source 1 of the second.
 template<class T> struct DevFcPairBwd {
   DevJobs<T> bwd_l, bwd_r;
+  // cover_left: the reverse into the left input has a job for EVERY function (those no live output reads get one without
+  // segments), so that a launch that overwrites instead of accumulating leaves no row of the adjoint unwritten
   void build(const FCWeights &w1, const std::vector<char> &live1, const DevFc<T> &F1, const FCWeights &w2, const std::vector<char> &live2,
-             const DevFc<T> &F2, int nfr, const int *drow)
+             const DevFc<T> &F2, int nfr, const int *drow, bool cover_left = false)
   {
     if (w1.n_funcs != w2.n_funcs || F1.nil != F2.nil || F1.nir != F2.nir || F1.no != F2.no) throw Error("FC pair: the two layers differ in shape");
     typename DevJobs<T>::Host hl, hr;
     for (int f = 0; f < w1.n_funcs; f++) {
-      if (!live1[f] && !live2[f]) continue;
+      if (!live1[f] && !live2[f] && !cover_left) continue;
       hl.job(f, 1.0);
       if (live1[f]) hl.seg(0, f, w1.w_tile_left[f], w1.norm_out_factor[f]);
       if (live2[f]) hl.seg(1, f, w2.w_tile_left[f], w2.norm_out_factor[f]);

@@ -946,14 +946,15 @@ __global__ __launch_bounds__(256) void k_reduce_fwd(ReduceDev<T> R, const int *m
   }
 }
 
-// gX_s[atom][fn c][n] += sum_k grho[atom][k] W_s[mu][c][n][k]: grid (tiles, jobs = all (s, c)), one wave per block
+// gX_s[atom][fn c][n] += sum_k grho[atom][k] W_s[mu][c][n][k]: grid (tiles, jobs), one wave per block; the jobs are all
+// (s, c) in the order of the sources, this launch takes those from job_first on
 template<class T>
 __global__ __launch_bounds__(64) void k_reduce_bwd(ReduceDev<T> R, const int *mu, const int *tile_atoms, const double *grho, T *G0, T *G1,
-                                                   T *G2, T *G3)
+                                                   T *G2, T *G3, int job_first = 0)
 {
   typedef typename Mfma<T>::v4 v4;
   const int tile = blockIdx.x;
-  int job = blockIdx.y, s = 0;
+  int job = blockIdx.y + job_first, s = 0;
   while (job >= R.ncol[s]) { job -= R.ncol[s]; s++; }
   const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;
   const int arow = tile_atoms[tile * 16 + c];

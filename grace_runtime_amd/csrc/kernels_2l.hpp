@@ -272,7 +272,8 @@ struct Energy2Dev {
 };
 
 // E_i = (MLP(x) + rho[0] + I2[0] ln0[0] / s0) out_scale + shift,  x_k = rho[k] lnI[k-1] / s1 + I2[k] ln0[k] / s0,
-// s1 = sqrt(mean rho[1:]^2 + eps), s0 = sqrt(mean I2^2 + eps); dE/drho, dE/dI2.  One wave per atom, fp64.
+// s1 = sqrt(mean rho[1:]^2 + eps), s0 = sqrt(mean I2^2 + eps); dE/drho, dE/dI2.  One wave per atom, fp64; a layer with
+// fewer than 33 outputs splits each dot product over 64 / outputs lanes.
 static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, const double *rho, const double *I2, double *grho, double *gI2,
                             double *eatom, double *energy, int want_grad, const int *sid)
 {
@@ -304,13 +305,27 @@ static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, cons
     for (int k = lane; k < n0; k += 64) act(0, k) *= q;
     __syncthreads();
   }
+  // lanes that share one output of a layer: the largest power of two g with outputs x g <= 64
+  auto group = [](int nout_) {
+    int g = 1;
+    while (g < 64 && nout_ * (g * 2) <= 64) g *= 2;
+    return g;
+  };
   for (int L = 0; L < M.nlay; L++) {
-    for (int c = lane; c < M.nout[L]; c += 64) {
+    const int no = M.nout[L], ni = M.nin[L], g = group(no), p = lane % g;
+    for (int c0 = 0; c0 < no; c0 += 64 / g) {    // every lane walks the loop: the exchanges need the whole wave
+      const int c = c0 + lane / g;
       double s = 0.0;
-      for (int a = 0; a < M.nin[L]; a++) s += act(L, a) * M.W[L][(long long) a * M.nout[L] + c];
-      s *= M.norm[L];
-      pre(L, c) = s;
-      act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+      if (c < no) {
+#pragma unroll 4
+        for (int a = p; a < ni; a += g) s += act(L, a) * M.W[L][(long long) a * no + c];
+      }
+      for (int o = g >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+      if (c < no && p == 0) {
+        s *= M.norm[L];
+        pre(L, c) = s;
+        act(L + 1, c) = (L < M.nlay - 1) ? (M.act == 1 ? tanh(s) : s / (1.0 + exp(-s))) : s;
+      }
     }
     __syncthreads();
   }
@@ -337,10 +352,18 @@ static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, cons
       }
       __syncthreads();
     }
-    for (int a = lane; a < M.nin[L]; a += 64) {
-      double s = 0.0;
-      for (int c = 0; c < M.nout[L]; c++) s += gbuf(cur, c) * M.W[L][(long long) a * M.nout[L] + c];
-      gbuf(cur ^ 1, a) = s * M.norm[L];
+    {
+      const int no = M.nout[L], ni = M.nin[L], g = group(ni), p = lane % g;
+      for (int b0 = 0; b0 < ni; b0 += 64 / g) {
+        const int a = b0 + lane / g;
+        double s = 0.0;
+        if (a < ni) {
+#pragma unroll 4
+          for (int c = p; c < no; c += g) s += gbuf(cur, c) * M.W[L][(long long) a * no + c];
+        }
+        for (int o = g >> 1; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        if (a < ni && p == 0) gbuf(cur ^ 1, a) = s * M.norm[L];
+      }
     }
     cur ^= 1;
     __syncthreads();
