@@ -70,9 +70,9 @@ template<class T> class Engine2L final : public EngineBase {
   }
   void chain_forward(Chain<T> &c, const char *tag, const T *X);
   void chain_zero(Chain<T> &c, const char *tag);
-  void chain_backward(Chain<T> &c, const char *tag, const T *X);
+  void chain_backward(Chain<T> &c, const char *tag, const T *X, const std::function<void()> &reduces_x_xx);
   void reduce_fwd(DevReduce<T> &R, int kb, const Chain<T> &c, const T *X, double *out);
-  void reduce_bwd(DevReduce<T> &R, const Chain<T> &c, const double *g);
+  void reduce_bwd(DevReduce<T> &R, const Chain<T> &c, const double *g, bool high);
   std::string tagged(const char *tag, const char *name) { return std::string(name) + tag; }
 };
 
@@ -116,10 +116,11 @@ void Engine2L<T>::build_chain(Chain<T> &c, const char *tag, int nf, int KP, cons
   if (order4_) jit_compile_product(("prod4" + t).c_str(), h4.terms, c.nXX, c.nXX, c.nXXXX, true, KP, f32, arch_, c.p4.jit, c.p4.jit_note);
   c.jit_all = c.p2.jit.ok() && c.p3.jit.ok() && (!order4_ || c.p4.jit.ok());
   c.fc1.build(*fc[0], live1, nf, KP, KP, KP, drow_);
-  c.fc2.build(*fc[1], live2, nf, KP, KP, KP, drow_);
+  // the reverse of fc2 (with the fourth-order stage: of fc2 and fc3 in one pass) WRITES the adjoint of XX: a job per function
+  c.fc2.build(*fc[1], live2, nf, KP, KP, KP, drow_, true);
   if (order4_) {
     c.fc3.build(*fc[2], live3, nf, KP, KP, KP, drow_);
-    c.fc23.build(*fc[1], live2, c.fc2, *fc[2], live3, c.fc3, nf, drow_);
+    c.fc23.build(*fc[1], live2, c.fc2, *fc[2], live3, c.fc3, nf, drow_, true);
   }
 }
 
@@ -405,7 +406,7 @@ template<class T> void Engine2L<T>::chain_zero(Chain<T> &c, const char *tag)
   stage(tagged(tag, "zero_grads").c_str(), [&] {
     HIP_CHECK(hipMemsetAsync(c.gX.p, 0, na * c.nf * KP * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(c.gX1.p, 0, na * c.nf * KP * sizeof(T), stream_));
-    HIP_CHECK(hipMemsetAsync(c.gXX.p, 0, na * c.nXX * KP * sizeof(T), stream_));
+    // gXX is not filled: the FC reverse writes every row of it, and the reduces add their XX parts afterwards
     // with the specialised product kernels gXX1 and gXX2 are written (not accumulated) by their producer
     if (!c.jit_all) HIP_CHECK(hipMemsetAsync(c.gXX1.p, 0, na * c.nXX * KP * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(c.gXXX.p, 0, na * c.nXXX * KP * sizeof(T), stream_));
@@ -416,8 +417,9 @@ template<class T> void Engine2L<T>::chain_zero(Chain<T> &c, const char *tag)
   });
 }
 
-// reverse of the chain; the reduces have added their adjoints to gX, gXX, gXXX, gXXXX.  Result in c.gX.
-template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag, const T *X)
+// reverse of the chain; the reduces have added their adjoints to gXXX and gXXXX.  The FC reverse WRITES gXX (no fill, no
+// read of the largest adjoint); reduces_x_xx then adds the reduces' adjoints of X and XX.  Result in c.gX.
+template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag, const T *X, const std::function<void()> &reduces_x_xx)
 {
   const int n = n_, KP = c.kb * 16;
   int one = 1, nat = n;
@@ -437,9 +439,9 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
       hipLaunchKernelGGL(k_prod_bwd<T>, dim3(P.d.nright * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, P.d, 1, L, g, gR, n, KP, sl, sr);
     });
   };
-  auto fc_bwd = [&](const std::string &name, DevFc<T> &F, const T *g, T *gXl, T *gXr, int nfl) {
+  auto fc_bwd = [&](const std::string &name, DevFc<T> &F, const T *g, T *gXl, T *gXr, int nfl, int acc_left) {
     stage(name.c_str(), [&] {
-      launch_gemm<T>(F.bwd_l, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXl, nfl, 1, tiles_.as<int>(), ntiles_);
+      launch_gemm<T>(F.bwd_l, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXl, nfl, acc_left, tiles_.as<int>(), ntiles_);
       launch_gemm<T>(F.bwd_r, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXr, c.nf, 1, tiles_.as<int>(), ntiles_);
     });
   };
@@ -451,14 +453,15 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
   if (c.order4) {
     // fc2 and fc3 share their inputs: one pass over gXX and gX for both
     stage(tagged(tag, "fc_23_bwd").c_str(), [&] {
-      launch_gemm<T>(c.fc23.bwd_l, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gXX, c.nXX, 1, tiles_.as<int>(), ntiles_);
+      launch_gemm<T>(c.fc23.bwd_l, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gXX, c.nXX, 0, tiles_.as<int>(), ntiles_);
       launch_gemm<T>(c.fc23.bwd_r, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gX, c.nf, 1, tiles_.as<int>(), ntiles_);
     });
   } else {
-    fc_bwd(tagged(tag, "fc_2_bwd"), c.fc2, gXX1, gXX, gX, c.nXX);
+    fc_bwd(tagged(tag, "fc_2_bwd"), c.fc2, gXX1, gXX, gX, c.nXX, 0);
   }
+  reduces_x_xx();
   prod_bwd(tagged(tag, "prod_2_bwd"), c.p2, X1, X1, gXX, gX1, gX1, c.nf, c.nf, 1, 1);
-  fc_bwd(tagged(tag, "fc_1_bwd"), c.fc1, gX1, gX, gX, c.nf);
+  fc_bwd(tagged(tag, "fc_1_bwd"), c.fc1, gX1, gX, gX, c.nf, 1);
 }
 
 template<class T> void Engine2L<T>::reduce_fwd(DevReduce<T> &R, int kb, const Chain<T> &c, const T *X, double *out)
@@ -475,11 +478,14 @@ template<class T> void Engine2L<T>::reduce_fwd(DevReduce<T> &R, int kb, const Ch
 #undef GR_RED
 }
 
-template<class T> void Engine2L<T>::reduce_bwd(DevReduce<T> &R, const Chain<T> &c, const double *g)
+// high: the sources XXX and XXXX (before the chain's reverse reads their adjoints); else X and XX (after the FC reverse
+// has written the adjoint of XX)
+template<class T> void Engine2L<T>::reduce_bwd(DevReduce<T> &R, const Chain<T> &c, const double *g, bool high)
 {
-  if (R.njobs == 0) return;
-  hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, R.njobs), dim3(64), 0, stream_, R.d, mu_.as<int>(), tiles_.as<int>(), g, c.gsrc(0), c.gsrc(1),
-                     c.gsrc(2), c.gsrc(3));
+  const int low = R.d.ncol[0] + R.d.ncol[1], first = high ? low : 0, count = high ? R.njobs - low : low;
+  if (count <= 0) return;
+  hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, count), dim3(64), 0, stream_, R.d, mu_.as<int>(), tiles_.as<int>(), g, c.gsrc(0), c.gsrc(1),
+                     c.gsrc(2), c.gsrc(3), first);
 }
 
 template<class T> void Engine2L<T>::run(const RunFlags &fl)
@@ -591,8 +597,8 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
 
   // ---- layer 2 reverse: dE/dB -> dE/dP -> bond forces of layer 2 and dE/dI of the neighbours
   chain_zero(c2_, "_L2");
-  stage("reduce_I2_bwd", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>()); });
-  chain_backward(c2_, "_L2", B);
+  stage("reduce_I2_bwd", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), true); });
+  chain_backward(c2_, "_L2", B, [&] { stage("reduce_I2_bwd_X_XX", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), false); }); });
   gP_.ensure(na * npf * CRP_ * sizeof(T));
   gM_.ensure(na * nI_ * CRP_ * sizeof(T));
   stage("reduce_B_bwd", [&] {
@@ -616,11 +622,16 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     HIP_CHECK(hipMemsetAsync(gI1_.p, 0, na * nI1_ * PI1_ * sizeof(double), stream_));
     gemm(jIb_, CRP_ / 16, PI1_ / 16, gM_.as<T>(), nI_, gI1_.as<T>(), nI1_, 0);
   });
-  stage("reduce_rho_bwd", [&] { reduce_bwd(redrho_, c1_, grho_.as<double>()); });
+  stage("reduce_rho_bwd", [&] { reduce_bwd(redrho_, c1_, grho_.as<double>(), true); });
   stage("reduce_I1_bwd", [&] {
-    for (auto &r : redI1_) reduce_bwd(*r, c1_, gI1_.as<double>());
+    for (auto &r : redI1_) reduce_bwd(*r, c1_, gI1_.as<double>(), true);
   });
-  chain_backward(c1_, "_L1", A);
+  chain_backward(c1_, "_L1", A, [&] {
+    stage("reduce_rho_bwd_X_XX", [&] { reduce_bwd(redrho_, c1_, grho_.as<double>(), false); });
+    stage("reduce_I1_bwd_X_XX", [&] {
+      for (auto &r : redI1_) reduce_bwd(*r, c1_, gI1_.as<double>(), false);
+    });
+  });
   {
     BondBwdArgs<T> ba{};
     ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();

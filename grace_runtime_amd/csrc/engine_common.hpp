@@ -8,6 +8,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <functional>
 #include <cmath>
 #include <cstring>
 #include <numeric>
@@ -190,8 +191,11 @@ template<class T> struct DevFc {
   DevBuf WlF, WrF, WlTF, WrTF;
   DevJobs<T> fwd, bwd_l, bwd_r;
   int nil = 0, nir = 0, no = 0;    // padded widths
-  // nfr: functions of the right-input tensor; livef: outputs that are computed
-  void build(const FCWeights &w, const std::vector<char> &livef, int nfr, int nil_p, int nir_p, int no_p, const int *drow)
+  // nfr: functions of the right-input tensor; livef: outputs that are computed; cover_left: the reverse into the left
+  // input has a job for EVERY function (without segments for outputs that are not computed), so that a launch that
+  // overwrites instead of accumulating leaves no row of the adjoint unwritten
+  void build(const FCWeights &w, const std::vector<char> &livef, int nfr, int nil_p, int nir_p, int no_p, const int *drow,
+             bool cover_left = false)
   {
     nil = nil_p; nir = nir_p; no = no_p;
     const int nt = w.tiles_left;
@@ -223,7 +227,10 @@ template<class T> struct DevFc {
       if (livef[w.collect_to[c]]) conn_from[w.collect_from[c]].push_back(c);
     }
     for (int f = 0; f < w.n_funcs; f++) {
-      if (!livef[f]) continue;
+      if (!livef[f]) {
+        if (cover_left) { hl.job(f, 1.0); hl.end_job(); }
+        continue;
+      }
       hf.job(f, w.norm_out_factor[f]);
       hf.seg(0, f, w.w_tile_left[f], 1.0);
       for (int c : conn_of[f]) hf.seg(1, w.collect_from[c], w.w_tile_right[c], 1.0);
