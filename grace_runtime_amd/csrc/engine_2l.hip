@@ -313,10 +313,7 @@ template<class T> void Engine2L<T>::build()
       hf.end_job();
     }
     for (int p = 0; p < nslot_ * nlm_; p++) {
-      bool any = false;
-      for (const Seg &s : segs) any = any || s.pair == p;
-      if (!any) continue;
-      hb.job(p, 1.0);
+      hb.job(p, 1.0);    // a job for every pair function, without segments when no term reads it: the launch writes all of gP
       for (const Seg &s : segs)
         if (s.pair == p) hb.seg(0, s.fo, s.tile, s.scale);
       hb.end_job();
@@ -602,8 +599,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   gP_.ensure(na * npf * CRP_ * sizeof(T));
   gM_.ensure(na * nI_ * CRP_ * sizeof(T));
   stage("reduce_B_bwd", [&] {
-    HIP_CHECK(hipMemsetAsync(gP_.p, 0, na * npf * CRP_ * sizeof(T), stream_));
-    HIP_CHECK(hipMemsetAsync(gM_.p, 0, na * nI_ * CRP_ * sizeof(T), stream_));
+    HIP_CHECK(hipMemsetAsync(gM_.p, 0, na * nI_ * CRP_ * sizeof(T), stream_));    // gP: every row is written below
     gemm(jBb_, C2P_ / 16, CRP_ / 16, c2_.gX.template as<T>(), nB_, gP_.as<T>(), npf, 0);
   });
   stage("pair_bwd", [&] {
@@ -619,7 +615,6 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   gI1_.ensure(na * nI1_ * PI1_ * sizeof(double));
   chain_zero(c1_, "_L1");
   stage("reduce_I_bwd", [&] {
-    HIP_CHECK(hipMemsetAsync(gI1_.p, 0, na * nI1_ * PI1_ * sizeof(double), stream_));
     gemm(jIb_, CRP_ / 16, PI1_ / 16, gM_.as<T>(), nI_, gI1_.as<T>(), nI1_, 0);
   });
   stage("reduce_rho_bwd", [&] { reduce_bwd(redrho_, c1_, grho_.as<double>(), true); });
