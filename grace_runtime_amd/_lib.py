@@ -24,7 +24,7 @@ SYMBOLS = [
     "gr_engine_debug_radial", "gr_engine_debug_copy", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
-    "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_batch_uq", "gr_compute_batch_device_uq", "gr_engine_reset", "gr_set_memory_limit", "gr_memory_in_use", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
+    "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_batch_uq", "gr_compute_batch_device_uq", "gr_engine_reset", "gr_engine_release_buffers", "gr_set_memory_limit", "gr_memory_in_use", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
     "gr_system_fetch_uq",
 ]
 
@@ -66,6 +66,7 @@ def lib():
     L.gr_engine_create.argtypes = [vp, i32, vp, i32, i32, C.POINTER(vp)]
     L.gr_engine_free.argtypes = [vp]
     L.gr_engine_reset.argtypes = [vp]
+    L.gr_engine_release_buffers.argtypes = [vp]
     L.gr_set_memory_limit.restype = None
     L.gr_set_memory_limit.argtypes = [i64]
     L.gr_memory_in_use.restype = i64

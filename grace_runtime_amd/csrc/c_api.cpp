@@ -243,6 +243,17 @@ int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int prec
   });
 }
 
+int gr_engine_release_buffers(gr_engine *e)
+{
+  return guarded([&] {
+    if (!e) throw grhip::InvalidArgument("null engine");
+    e->bnl.reset();
+    e->lmp.reset();
+    e->eng->release_buffers();
+    e->generation++;    // a gr_system on this engine uploads its structure again
+  });
+}
+
 int gr_engine_reset(gr_engine *e)
 {
   return guarded([&] {

@@ -83,6 +83,7 @@ class Engine {
   virtual void fetch_add_device(const int *atom, double *energy, double *forces, double *virial, double *eatom) = 0;
   // UQ outputs of the last run with RunFlags::uq, [n] each in the order of the uploaded list (null pointers are skipped)
   virtual void fetch_uq(double *gamma, double *sigma, double *cluster) = 0;
+  virtual void release_buffers() = 0;    // frees the work buffers and the uploaded structure; weights stay
   virtual void synchronize() = 0;
   virtual void set_profile(bool on) = 0;
   virtual const std::vector<StageTime> &stage_times() = 0;

@@ -15,6 +15,7 @@ template<class T> class Engine1L final : public EngineBase {
   {
     this->template probe_mfma<T>();
     build();
+    end_build();    // buffers allocated from here on are work buffers (release_buffers)
   }
 
   int layers() const override { return 1; }

@@ -35,6 +35,7 @@ template<class T> class Engine2L final : public EngineBase {
   {
     this->template probe_mfma<T>();
     build();
+    end_build();    // buffers allocated from here on are work buffers (release_buffers)
   }
   int layers() const override { return 2; }
   void run(const RunFlags &fl) override;

@@ -175,6 +175,7 @@ template<class T> class Engine3L final : public EngineBase {
   {
     this->template probe_mfma<T>();
     build();
+    end_build();    // buffers allocated from here on are work buffers (release_buffers)
   }
   int layers() const override { return 3; }
   void run(const RunFlags &fl) override;

@@ -36,14 +36,35 @@ inline std::atomic<long long> &dev_bytes_limit()
   return v;
 }
 
+// The buffers of the engine under construction on this thread register themselves here (BufRegistry below): the engine
+// can then give back the memory of its work buffers without knowing each of them.
+struct DevBuf;
+inline std::vector<DevBuf *> *&building_registry()
+{
+  static thread_local std::vector<DevBuf *> *r = nullptr;
+  return r;
+}
+
 // device allocation owned by the engine
 struct DevBuf {
   void *p = nullptr;
   size_t bytes = 0;
-  DevBuf() = default;
+  bool model_data = false;              // allocated while the engine was built (weights, tables): kept by release_work()
+  std::vector<DevBuf *> *reg = nullptr;
+  DevBuf() : reg(building_registry())
+  {
+    if (reg) reg->push_back(this);
+  }
   DevBuf(const DevBuf &) = delete;
   DevBuf &operator=(const DevBuf &) = delete;
-  ~DevBuf() { release(); }
+  ~DevBuf()
+  {
+    release();
+    if (reg) {
+      auto it = std::find(reg->begin(), reg->end(), this);
+      if (it != reg->end()) reg->erase(it);
+    }
+  }
   void release()
   {
     if (p) {
@@ -68,6 +89,7 @@ struct DevBuf {
       throw std::bad_alloc();
     }
     bytes = want;
+    model_data = building_registry() != nullptr;
     dev_bytes_in_use() += (long long) want;
   }
   template<class U> U *as() const { return static_cast<U *>(p); }
@@ -486,8 +508,38 @@ template<class T> struct DevReduce {
 };
 
 // Device, stream, per-stage GPU timing and the MFMA accumulator-row probe of an engine.
-class EngineBase : public Engine {
+// First base of an engine: from its construction until end_build() every DevBuf made on this thread (members of the
+// engine and of the structures it holds) is listed in bufs_, and what they allocate in that time is model data.
+struct BufRegistry {
+  std::vector<DevBuf *> bufs_;
+  BufRegistry() { building_registry() = &bufs_; }
+  ~BufRegistry()
+  {
+    if (building_registry() == &bufs_) building_registry() = nullptr;    // a constructor that threw
+  }
+  void end_build()
+  {
+    if (building_registry() == &bufs_) building_registry() = nullptr;
+  }
+};
+
+class EngineBase : public Engine, protected BufRegistry {
  public:
+  // Frees every buffer that was allocated after the engine was built (per-atom and per-bond work buffers, the uploaded
+  // structure); weights, tables and compiled kernels stay.  The engine then holds no structure: upload before the next
+  // run.  The reference's engines: release_buffers() (kk/grace_1l_kk.h:72-113).
+  void release_buffers() override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    for (DevBuf *b : bufs_)
+      if (!b->model_data) b->release();
+    scal_.ensure(8 * sizeof(double));    // grown by a batch upload: an empty pass still clears and reads one record
+    n_ = 0;
+    nb_ = 0;
+    nstruct_ = 1;
+    ran_ = ran_forces_ = ran_eatom_ = ran_uq_ = false;
+  }
   void synchronize() override { check(hipSetDevice(device_), "hipSetDevice"); check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
   void set_profile(bool on) override { profile_ = on; }
   const std::vector<StageTime> &stage_times() override

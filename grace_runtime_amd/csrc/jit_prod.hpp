@@ -21,6 +21,8 @@
 #include <map>
 #include <set>
 #include <sstream>
+#include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -209,29 +211,45 @@ inline bool jit_compile_product(const char *name, const std::vector<ProdTerm> &t
       std::fclose(f);
     }
   }
-  hiprtcProgram prog;
-  if (hiprtcCreateProgram(&prog, src.c_str(), name, 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
-    why = "hiprtcCreateProgram failed";
-    return false;
+  // compiled code objects of the process by (architecture, source): a second engine of the same model, or a fresh one
+  // after a reset, loads the code without compiling it again
+  static std::mutex cache_mu;
+  static std::map<std::string, std::shared_ptr<const std::vector<char>>> cache;
+  const std::string key = arch + "\n" + src;
+  std::shared_ptr<const std::vector<char>> obj;
+  {
+    std::lock_guard<std::mutex> lk(cache_mu);
+    auto it = cache.find(key);
+    if (it != cache.end()) obj = it->second;
   }
-  const std::string a = "--offload-arch=" + arch;
-  const char *opts[] = {a.c_str(), "-O3", "-ffp-contract=fast"};
-  const hiprtcResult rc = hiprtcCompileProgram(prog, 3, opts);
-  if (rc != HIPRTC_SUCCESS) {
-    size_t ls = 0;
-    hiprtcGetProgramLogSize(prog, &ls);
-    std::string log(ls, ' ');
-    if (ls) hiprtcGetProgramLog(prog, &log[0]);
-    why = "hiprtc: " + log.substr(0, 400);
+  if (!obj) {
+    hiprtcProgram prog;
+    if (hiprtcCreateProgram(&prog, src.c_str(), name, 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
+      why = "hiprtcCreateProgram failed";
+      return false;
+    }
+    const std::string a = "--offload-arch=" + arch;
+    const char *opts[] = {a.c_str(), "-O3", "-ffp-contract=fast"};
+    const hiprtcResult rc = hiprtcCompileProgram(prog, 3, opts);
+    if (rc != HIPRTC_SUCCESS) {
+      size_t ls = 0;
+      hiprtcGetProgramLogSize(prog, &ls);
+      std::string log(ls, ' ');
+      if (ls) hiprtcGetProgramLog(prog, &log[0]);
+      why = "hiprtc: " + log.substr(0, 400);
+      hiprtcDestroyProgram(&prog);
+      return false;
+    }
+    size_t cs = 0;
+    hiprtcGetCodeSize(prog, &cs);
+    std::vector<char> code(cs);
+    hiprtcGetCode(prog, code.data());
     hiprtcDestroyProgram(&prog);
-    return false;
+    obj = std::make_shared<const std::vector<char>>(std::move(code));
+    std::lock_guard<std::mutex> lk(cache_mu);
+    cache[key] = obj;
   }
-  size_t cs = 0;
-  hiprtcGetCodeSize(prog, &cs);
-  std::vector<char> code(cs);
-  hiprtcGetCode(prog, code.data());
-  hiprtcDestroyProgram(&prog);
-  if (hipModuleLoadData(&out.mod, code.data()) != hipSuccess) {
+  if (hipModuleLoadData(&out.mod, obj->data()) != hipSuccess) {
     (void) hipGetLastError();
     out.mod = nullptr;
     why = "hipModuleLoadData failed";

@@ -180,6 +180,11 @@ class Engine:
     def cutoff(self, t1: int, t2: int) -> float:
         return _lib.lib().gr_engine_cutoff(self._h, int(t1), int(t2))
 
+    def release_buffers(self):
+        """frees the work buffers and the uploaded structure; weights, tables and compiled kernels stay"""
+        check(_lib.lib().gr_engine_release_buffers(self._h))
+        self._n = 0
+
     def reset(self):
         """a fresh engine in place of this one, every device buffer dropped (after an allocation failure)"""
         check(_lib.lib().gr_engine_reset(self._h))
@@ -412,7 +417,8 @@ class System:
         return bool(_lib.lib().gr_system_list_on_device(self._h))
 
     def release_buffers(self):
-        pass
+        """frees the engine's work buffers (python/kk/kk_api.h:66-93); the next compute builds its list again"""
+        self.engine.release_buffers()
 
     def set_dispersion(self, *a, **k):
         raise ValueError("dispersion corrections are not part of this engine")
@@ -474,7 +480,14 @@ class Batch:
         self._nall_cap = 1 << 62    # atoms per pass after an allocation failure (python/kk/kk_core.cpp:1461: nall_cap)
 
     def release_buffers(self):
-        pass
+        """frees the engine's work buffers (python/kk/kk_api.h:116-156)"""
+        self.engine.release_buffers()
+
+    def _done(self):
+        # a batch is a job: its device memory goes back after the call unless keep_buffers is set (an MD loop over the
+        # same batch), python/kk/kk_core.cpp:1466-1469
+        if not self.keep_buffers:
+            self.release_buffers()
 
     def compute(self, natoms, types, positions, cells, pbc, energies=False, uq=False, energy_only=False,
                 max_nall=1 << 21, dispersion_parts=False):
@@ -529,6 +542,7 @@ class Batch:
                     raise RuntimeError(f"the batch ({N} atoms) does not fit the GPU memory even in passes of {tried} atoms; "
                                        "use a GPU with more memory") from None
                 limit = self._nall_cap = max(16384, tried // 2)
+        self._done()
         if not energy_only:
             out["forces"], out["virial"] = f, v
         if energies:
@@ -569,6 +583,7 @@ class Batch:
         check(_lib.lib().gr_compute_batch_device_uq(self.engine._h, S, ptr(natoms), p_types, p_pos, ptr(cells), ptr(pb), flags, int(max_nall),
                                                     p_e, p_f, p_v, p_ea, p_uq[0], p_uq[1], p_uq[2], C.byref(passes)))
         self.passes = passes.value if N else 0
+        self._done()
 
 
 _CAI_TYPES = {"int32": "<i4", "float64": "<f8"}

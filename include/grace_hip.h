@@ -75,6 +75,11 @@ void gr_engine_free(gr_engine *e);
  * (python/kk/kk_core.cpp:478-497 poison / drop, the next compute attaches a fresh engine).  A structure uploaded before
  * is gone; a gr_system on this engine notices and uploads its structure again. */
 int gr_engine_reset(gr_engine *e);
+/* Frees the engine's work buffers (per-atom and per-bond arrays, the uploaded structure, the lists of the device entry
+ * points); weights, tables and compiled kernels stay, the next call allocates again.  System.release_buffers() /
+ * Batch.release_buffers() of the reference's GPU module (python/kk/kk_api.h:66-156; engines: release_buffers(),
+ * kk/grace_1l_kk.h:72-113). */
+int gr_engine_release_buffers(gr_engine *e);
 /* Bytes of device memory the library's buffers hold (all engines of the process), and a cap on them: with a cap an
  * allocation that would pass it fails as one the device refuses (GR_NOMEM, or the retry of gr_compute_batch_device).
  * 0: no cap.  The part of the reference module's memory_info() / chunk-by-free-memory policy (kk/support.h:415-450) that

@@ -147,6 +147,7 @@ def test_allocation_failure_halves_the_passes_and_keeps_the_limit(model_dir):
     N = int(natoms.sum())
     assert 33000 < N < 65000                      # one halving reaches a pass size above the floor of 16384
     b = kk.Batch(eng.model, ["Al", "Ni", "Ti"])
+    b.keep_buffers = True                         # the buffers of a call stay, so that what they hold can be measured
     try:
         ref = _device_run(b, natoms, types, pos, cells, pbc, max_nall=N // 2)
         assert b.passes >= 2
@@ -187,3 +188,43 @@ def test_engine_reset_is_seen_by_a_system(model_dir):
     s.engine.reset()
     b = s.compute(t, p, c, pb)
     assert s.rebuilds == 2 and abs(a["energy"] - b["energy"]) < 1e-9 and np.abs(a["forces"] - b["forces"]).max() < 1e-9
+
+
+def test_release_buffers_gives_the_work_memory_back(model_dir):
+    """Batch.release_buffers / keep_buffers and System.release_buffers (python/kk/kk_api.h:66-156): after a release the
+    library holds what it held right after the engine was made (weights, tables), and the next call gives the same
+    results"""
+    model = kk.Model(os.path.join(model_dir, "l2mix.npz"))
+    structs = [cases.structure_alloy54(), cases.structure_triclinic(), cases.structure_slab()]
+    natoms, types, pos, cells, pbc = _pack(structs)
+    before = kk.memory_in_use()
+    b = kk.Batch(model, ["Mo", "W"])
+    built = kk.memory_in_use()
+    assert built > before
+    b.keep_buffers = True
+    ref = b.compute(natoms, types, pos, cells, pbc, energies=True)
+    grown = kk.memory_in_use()
+    assert grown > built
+    b.release_buffers()
+    assert kk.memory_in_use() <= built + 4096          # one small record is allocated again at once
+    _compare(b.compute(natoms, types, pos, cells, pbc, energies=True), ref)
+    assert kk.memory_in_use() > built
+    b.keep_buffers = False                              # the reference's default: a batch is a job
+    _compare(b.compute(natoms, types, pos, cells, pbc, energies=True), ref)
+    assert kk.memory_in_use() <= built + 4096
+    _compare(_device_run(b, natoms, types, pos, cells, pbc), ref)
+    assert kk.memory_in_use() <= built + 4096
+    # a System on a released engine builds its list again
+    s = kk.System(model, ["Mo", "W"], skin=0.3)
+    p, c, pb, t = structs[0]
+    a = s.compute(t, p, c, pb)
+    held = kk.memory_in_use()
+    s.release_buffers()
+    assert kk.memory_in_use() < held
+    a2 = s.compute(t, p, c, pb)
+    assert s.rebuilds == 2 and abs(a["energy"] - a2["energy"]) < 1e-9 and np.abs(a["forces"] - a2["forces"]).max() < 1e-9
+    # an engine with nothing uploaded after a release: an empty pass, not a fault
+    eng = _engine(model_dir, "mix2", ["Mo", "W"])
+    eng.release_buffers()
+    eng.run()
+    assert eng.fetch()["energy"] == 0.0
