@@ -99,8 +99,6 @@ def main():
     tmp = tempfile.mkdtemp()
     two = a.workload == "config3"
     three = a.workload == "config4"
-    if (two or three) and a.precision != 64:
-        sys.exit("bench.py: the GRACE-2L and GRACE-3L engines compute in fp64")
     reps = a.reps or (20 if two else 16)
     pbc = [True, True, True]
     if three:

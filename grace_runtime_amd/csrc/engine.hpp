@@ -99,11 +99,11 @@ class Engine {
 std::unique_ptr<Engine> make_engine_1l(std::shared_ptr<const Model1L> model, int ntypes, const std::vector<int> &type2mu,
                                        int precision, int device);
 
-// GRACE-2L: network arithmetic in fp64 only (precision 64)
+// GRACE-2L: the same two precisions (fp32: the scalar reduces, the two RMSNorms and the readout stay in fp64)
 std::unique_ptr<Engine> make_engine_2l(std::shared_ptr<const Model2L> model, int ntypes, const std::vector<int> &type2mu,
                                        int precision, int device);
 
-// GRACE-3L: network arithmetic in fp64 only (precision 64)
+// GRACE-3L: the same two precisions (fp32: the scalar reduces, the norms and the readout stay in fp64)
 std::unique_ptr<Engine> make_engine_3l(std::shared_ptr<const Model3L> model, int ntypes, const std::vector<int> &type2mu,
                                        int precision, int device);
 

@@ -60,7 +60,7 @@ template<class T> class Engine2L final : public EngineBase {
   DevJobs<T> jI_, jIb_, jB_, jBb_;
   Energy2Dev en_{};
   // pass buffers
-  DevBuf sink_, Rz_, dRz_, R1_, dR1_, YG_, A_, rho_, grho_, I1_, gI1_, M_, gM_, P_, gP_, B_, I2_, gI2_;
+  DevBuf sink_, Rz_, dRz_, R1_, dR1_, YG_, A_, rho_, grho_, I1_, gI1_, I1t_, gI1t_, M_, gM_, P_, gP_, B_, I2_, gI2_;
 
   void build();
   void build_chain(Chain<T> &c, const char *tag, int nf, int KP, const FCWeights *fc[3], const CGProduct *pr[3],
@@ -488,7 +488,6 @@ template<class T> void Engine2L<T>::reduce_bwd(DevReduce<T> &R, const Chain<T> &
 
 template<class T> void Engine2L<T>::run(const RunFlags &fl)
 {
-  static_assert(sizeof(T) == 8, "the GRACE-2L engine computes in fp64");
   const int n = n_;
   if (!begin_pass(fl)) return;
   const size_t ecap = (size_t) std::max<int64_t>(nb_, 1), na = (size_t) n;
@@ -534,8 +533,17 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   });
   M_.ensure(na * nslot_ * CRP_ * sizeof(T));
   T *M = M_.as<T>();
+  // I1 leaves the scalar reduce in fp64; the fp32 engine hands the GEMM a copy in fp32
+  const long long nI1v = (long long) na * nI1_ * PI1_;
+  const T *I1t = I1_.as<T>();
+  if constexpr (sizeof(T) == 4) {
+    I1t_.ensure(nI1v * sizeof(T));
+    I1t = I1t_.as<T>();
+  }
   stage("reduce_I", [&] {
-    gemm(jI_, PI1_ / 16, CRP_ / 16, I1_.as<T>(), nI1_, M, nslot_, 0);
+    if constexpr (sizeof(T) == 4)
+      hipLaunchKernelGGL((k_convert<double, T>), dim3((unsigned) ((nI1v + 255) / 256)), dim3(256), 0, stream_, I1_.as<double>(), I1t_.as<T>(), nI1v);
+    gemm(jI_, PI1_ / 16, CRP_ / 16, I1t, nI1_, M, nslot_, 0);
     hipLaunchKernelGGL(k_fill_slot<T>, dim3((unsigned) ((na * CRP_ + 255) / 256)), dim3(256), 0, stream_, mu_.as<int>(), zB0_.as<T>(), M, n, nslot_,
                        nI_, CRP_);
   });
@@ -616,7 +624,13 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   gI1_.ensure(na * nI1_ * PI1_ * sizeof(double));
   chain_zero(c1_, "_L1");
   stage("reduce_I_bwd", [&] {
-    gemm(jIb_, CRP_ / 16, PI1_ / 16, gM_.as<T>(), nI_, gI1_.as<T>(), nI1_, 0);
+    if constexpr (sizeof(T) == 4) {
+      gI1t_.ensure(nI1v * sizeof(T));
+      gemm(jIb_, CRP_ / 16, PI1_ / 16, gM_.as<T>(), nI_, gI1t_.as<T>(), nI1_, 0);
+      hipLaunchKernelGGL((k_convert<T, double>), dim3((unsigned) ((nI1v + 255) / 256)), dim3(256), 0, stream_, gI1t_.as<T>(), gI1_.as<double>(), nI1v);
+    } else {
+      gemm(jIb_, CRP_ / 16, PI1_ / 16, gM_.as<T>(), nI_, gI1_.as<T>(), nI1_, 0);
+    }
   });
   stage("reduce_rho_bwd", [&] { reduce_bwd(redrho_, c1_, grho_.as<double>(), true); });
   stage("reduce_I1_bwd", [&] {
@@ -645,7 +659,7 @@ std::unique_ptr<Engine> make_engine_2l(std::shared_ptr<const Model2L> model, int
                                        int device)
 {
   if (precision == 64) return std::make_unique<Engine2L<double>>(std::move(model), ntypes, type2mu, device);
-  if (precision == 32) throw InvalidArgument("GRACE-2L engines compute in fp64 (precision 64)");
+  if (precision == 32) return std::make_unique<Engine2L<float>>(std::move(model), ntypes, type2mu, device);
   throw InvalidArgument("precision must be 64 or 32");
 }
 

@@ -856,7 +856,6 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
 
 template<class T> void Engine3L<T>::run(const RunFlags &fl)
 {
-  static_assert(sizeof(T) == 8, "the GRACE-3L engine computes in fp64");
   const int n = n_;
   if (!begin_pass(fl)) return;
   const size_t ecap = (size_t) std::max<int64_t>(nb_, 1);
@@ -901,7 +900,7 @@ std::unique_ptr<Engine> make_engine_3l(std::shared_ptr<const Model3L> model, int
                                        int device)
 {
   if (precision == 64) return std::make_unique<Engine3L<double>>(std::move(model), ntypes, type2mu, device);
-  if (precision == 32) throw InvalidArgument("GRACE-3L engines compute in fp64 (precision 64)");
+  if (precision == 32) return std::make_unique<Engine3L<float>>(std::move(model), ntypes, type2mu, device);
   throw InvalidArgument("precision must be 64 or 32");
 }
 

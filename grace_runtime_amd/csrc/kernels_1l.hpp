@@ -619,39 +619,47 @@ template<class T, int MAXM> __global__ void k_scatter_a(ScatterArgs<T> a)
 
 // A[lm][n] = sum_b Y_lm(b) Rz[b][l][n] on the matrix cores.  One wave per atom (4 atoms per block); per tile of 16
 // bonds and per l:  D_l[m][n] += Y_l^T[m][b] . Rz_l[b][n]  with K = bonds (4 per MFMA step), rows m padded to 16.
-// The B operand (Rz) comes straight from memory, 16 lanes reading 128 consecutive bytes of one bond row; all B
-// operands of a tile are requested before the harmonics of the tile are evaluated, so that one memory latency is paid
-// per tile.  The A operand (Y) comes from the wave's LDS tile.  The accumulators of the wave are the atom's A.
+// The B operand (Rz) comes straight from memory, 16 lanes reading 128 consecutive bytes of one bond row; the B operands
+// of a tile are requested before the harmonics of the tile are evaluated, and each half of the next tile as soon as the
+// MFMAs have consumed that half of the current one.  The A operand (Y) comes from the wave's LDS tile.  The
+// accumulators of the wave are the atom's A.
+// The grid walks the atoms from the LAST to the first: the radial kernel, which runs right before, writes the edge rows
+// in ascending order, so the rows it wrote last are the ones still held by the memory-side cache.
 // NL = lmax + 1, KB = channels / 16.   dynamic LDS: 4 * 16 * nlm values.
-template<class T, int NL, int KB> __global__ __launch_bounds__(256) void k_scatter_a_mfma(ScatterArgs<T> a)
+template<class T, int NL, int KB> __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_scatter_a_mfma(ScatterArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   T *Yw = reinterpret_cast<T *>(smem_raw) + wave * 16 * a.nlm;     // [16 bonds][nlm]
-  const int ia = blockIdx.x * 4 + wave;
-  if (ia >= a.natoms) return;
+  const int ia = a.natoms - 1 - (blockIdx.x * 4 + wave);
+  if (ia < 0) return;
   const int i = a.a0 + ia;
-  const long long e0 = a.eoff[i], e1 = a.eoff[i + 1];
+  const long long w0 = a.eoff[i], w1 = a.eoff[i + 1];
   const int C = a.C;
   v4 acc[NL][KB];
 #pragma unroll
   for (int l = 0; l < NL; l++)
 #pragma unroll
     for (int cb = 0; cb < KB; cb++) acc[l][cb] = v4{0, 0, 0, 0};
-  for (long long eb = e0; eb < e1; eb += 16) {
-    const int nb = (int) (e1 - eb < 16 ? e1 - eb : 16);
-    T breg[4][NL][KB];
+  T breg[4][NL][KB];
+  auto request = [&](long long eb, int h) {
+    const int nb = (int) (w1 - eb < 16 ? w1 - eb : 16);
 #pragma unroll
-    for (int s = 0; s < 4; s++) {
+    for (int s = 2 * h; s < 2 * h + 2; s++) {
+      if (4 * s >= nb) continue;                      // a step with no bond: neither loaded nor multiplied
       const int b = 4 * s + g;                        // k index of this lane in step s = bond of the tile
-      const T *row = a.Rz + (eb + (b < nb ? b : 0)) * a.noutp + c;      // rows beyond the tile: any valid row (Y = 0 there)
+      const T *row = a.Rz + (eb + (b < nb ? b : 0)) * a.noutp + c;      // rows beyond the range: any valid row (Y = 0 there)
 #pragma unroll
       for (int l = 0; l < NL; l++)
 #pragma unroll
         for (int cb = 0; cb < KB; cb++) breg[s][l][cb] = row[l * C + cb * 16];
     }
+  };
+  if (w0 < w1) { request(w0, 0); request(w0, 1); }
+  for (long long eb = w0; eb < w1; eb += 16) {
+    const int nb = (int) (w1 - eb < 16 ? w1 - eb : 16);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     if (lane < 16) {
@@ -665,15 +673,21 @@ template<class T, int NL, int KB> __global__ __launch_bounds__(256) void k_scatt
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const bool more = eb + 16 < w1;
 #pragma unroll
-    for (int s = 0; s < 4; s++) {
-      const T *yb = Yw + (4 * s + g) * a.nlm;
+    for (int h = 0; h < 2; h++) {
 #pragma unroll
-      for (int l = 0; l < NL; l++) {
-        const T y = c < 2 * l + 1 ? yb[l * l + c] : (T) 0;       // A operand: row m = c
+      for (int s = 2 * h; s < 2 * h + 2; s++) {
+        if (4 * s >= nb) continue;
+        const T *yb = Yw + (4 * s + g) * a.nlm;
 #pragma unroll
-        for (int cb = 0; cb < KB; cb++) acc[l][cb] = Mfma<T>::mma(y, breg[s][l][cb], acc[l][cb]);
+        for (int l = 0; l < NL; l++) {
+          const T y = c < 2 * l + 1 ? yb[l * l + c] : (T) 0;       // A operand: row m = c
+#pragma unroll
+          for (int cb = 0; cb < KB; cb++) acc[l][cb] = Mfma<T>::mma(y, breg[s][l][cb], acc[l][cb]);
+        }
       }
+      if (more) request(eb + 16, h);
     }
   }
   T *Ai = a.A + (long long) ia * a.nlm * C;

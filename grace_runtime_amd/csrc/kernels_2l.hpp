@@ -49,6 +49,13 @@ template<class T> __global__ void k_fill_slot(const int *mu, const T *z, T *M, i
   M[((long long) at * nslot + slot) * C + n] = z[mu[at] * C + n];
 }
 
+// dst[q] = src[q] in another precision (the fp32 engine: the scalar reduces write and read fp64 rows, the GEMMs fp32 rows)
+template<class S, class D> __global__ void k_convert(const S *src, D *dst, long long count)
+{
+  const long long q = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (q < count) dst[q] = (D) src[q];
+}
+
 constexpr int kPairChunk = 8;    // bonds staged in LDS at a time by the pair kernels
 
 // Block -> (atom, slot group).  ngrp == 0: a (atoms, groups) grid.  ngrp > 0: a 1-d grid of 8 ceil(atoms / 8) ngrp

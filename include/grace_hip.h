@@ -66,8 +66,8 @@ void gr_model_free(gr_model *m);
  * Grace1LFused(model, settings, log) + setup_types(ntypes, type2mu): libgrace/include/grace/fused_1l.h:28-31, likewise
  * Grace2LFused (fused_2l.h:32-39) and Grace3LFused (fused_3l.h:26-34); Grace1LKK::set_model / setup:
  * libgrace/include/grace/kk/grace_1l_kk.h:72-79.
- * precision 64: network arithmetic in fp64; 32: fp32 network, fp64 geometry and sums (docs/advanced.md:37-38; GRACE-1L
- * only, GR_INVALID for GRACE-2L / 3L models). */
+ * precision 64: network arithmetic in fp64; 32: fp32 network, fp64 geometry, norms, readout and sums
+ * (docs/advanced.md:37-38), for GRACE-1L, 2L and 3L models; any other value: GR_INVALID. */
 int gr_engine_create(const gr_model *m, int ntypes, const int *type2mu, int precision, int device, gr_engine **out);
 void gr_engine_free(gr_engine *e);
 /* Drops the engine and every device buffer it holds and makes a fresh one from the same model, types, precision and
