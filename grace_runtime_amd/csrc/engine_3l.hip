@@ -585,7 +585,7 @@ template<class T> void Engine3L<T>::couple_bwd(ProdStage<T> &p, const T *Lp, int
     return;
   }
   const int ATl = 64 / KP;
-  const size_t lds = (size_t) 2 * ATl * (nfl + nfr) * KP * sizeof(T);
+  const size_t lds = (size_t) ATl * (nfl + nfr) * KP * (sizeof(T) + sizeof(double));
   if (lds <= kCoupleLdsMax && p.cd.nterms > 0) {
     auto kern = k_couple_bwd_lds<T>;
     if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));

@@ -160,24 +160,27 @@ __global__ __launch_bounds__(1024) void k_couple_fwd_lds(CoupleDev P, const T *_
 
 // Its reverse in scatter form: for every term gLp[l][n] += c g[o][n] Rp[r][n], gRp[r][n] += c g[o][n] Lp[l][n]
 // (couple_row_bwd, fused_3l_cpu.h:258-276), the two adjoints accumulated in LDS with LDS atomics (the waves of a block
-// share them) and added to gL / gR at the end; g is read once, row by row.  Same grid; dynamic LDS: 2 AT (nfl + nfr) C.
+// share them) and added to gL / gR at the end; g is read once, row by row.  The LDS accumulators are fp64 for both
+// precisions (ds_add_f32 runs several times slower than ds_add_f64 on this hardware).  Same grid; dynamic LDS:
+// AT (nfl + nfr) C (sizeof(T) + 8) bytes.
 template<class T>
 __global__ __launch_bounds__(1024) void k_couple_bwd_lds(CoupleDev P, const T *__restrict__ L, const T *__restrict__ R, const T *__restrict__ g,
                                                          T *__restrict__ gL, T *__restrict__ gR, int C, int nfl, int nfr, int natoms)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   const int AT = 64 / C, t = threadIdx.x, lane = t & 63, wave = t >> 6, nw = blockDim.x >> 6;
-  T *Ls = reinterpret_cast<T *>(smem_raw), *Rs = Ls + AT * nfl * C, *gLs = Rs + AT * nfr * C, *gRs = gLs + AT * nfl * C;
+  double *gLs = reinterpret_cast<double *>(smem_raw), *gRs = gLs + AT * nfl * C;
+  T *Ls = reinterpret_cast<T *>(gRs + AT * nfr * C), *Rs = Ls + AT * nfl * C;
   const int a0 = blockIdx.x * AT, na = natoms - a0 < AT ? natoms - a0 : AT;
   {
     const T *La = L + (long long) a0 * nfl * C, *Ra = R + (long long) a0 * nfr * C;
     for (int q = t; q < AT * nfl * C; q += blockDim.x) {
       Ls[q] = q < na * nfl * C ? La[q] : (T) 0;
-      gLs[q] = (T) 0;
+      gLs[q] = 0.0;
     }
     for (int q = t; q < AT * nfr * C; q += blockDim.x) {
       Rs[q] = q < na * nfr * C ? Ra[q] : (T) 0;
-      gRs[q] = (T) 0;
+      gRs[q] = 0.0;
     }
   }
   __syncthreads();
@@ -205,15 +208,15 @@ __global__ __launch_bounds__(1024) void k_couple_bwd_lds(CoupleDev P, const T *_
       }
       const int l = __builtin_amdgcn_readlane(lv, k), r = __builtin_amdgcn_readlane(rv, k);
       const T cg = (T) readlane_f64(cv, k) * gcur;
-      atomicAdd(&gLs[lo + l * C], cg * Rs[ro + r * C]);
-      atomicAdd(&gRs[ro + r * C], cg * Ls[lo + l * C]);
+      atomicAdd(&gLs[lo + l * C], (double) (cg * Rs[ro + r * C]));
+      atomicAdd(&gRs[ro + r * C], (double) (cg * Ls[lo + l * C]));
     }
   }
   __syncthreads();
   {
     T *ga = gL + (long long) a0 * nfl * C, *gb = gR + (long long) a0 * nfr * C;
-    for (int q = t; q < na * nfl * C; q += blockDim.x) ga[q] += gLs[q];
-    for (int q = t; q < na * nfr * C; q += blockDim.x) gb[q] += gRs[q];
+    for (int q = t; q < na * nfl * C; q += blockDim.x) ga[q] += (T) gLs[q];
+    for (int q = t; q < na * nfr * C; q += blockDim.x) gb[q] += (T) gRs[q];
   }
 }
 
