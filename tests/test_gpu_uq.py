@@ -31,7 +31,8 @@ def _oracle(path, name, t, offset, j, rij):
 
 
 # GRACE-2L and GRACE-3L engines compute in fp64 only
-@pytest.mark.parametrize("name,precision,tol", [("uq2", 64, 1e-9), ("uq2", 32, 1e-4), ("uq2l", 64, 1e-9), ("uq3l", 64, 1e-9)])
+@pytest.mark.parametrize("name,precision,tol", [("uq2", 64, 1e-9), ("uq2", 32, 1e-4), ("uq2l", 64, 1e-9), ("uq2l", 32, 1e-4), ("uq3l", 64, 1e-9),
+                                                ("uq3l", 32, 1e-4)])
 @pytest.mark.parametrize("struct", ["alloy54", "triclinic"])
 def test_uq_matches_oracle(model_dir, name, struct, precision, tol):
     path = os.path.join(model_dir, name + ".npz")
