@@ -985,24 +985,32 @@ class EngineBase : public Engine, protected BufRegistry {
 #undef GR_BB
   }
   // out[tile atoms][job output] = GEMM jobs over X0 (kb0 16-channel blocks) and X1 (kb1), nb output blocks
+  static constexpr size_t kGemmLdsBudget = 40 * 1024;
   template<class T>
   void launch_gemm(DevJobs<T> &J, int kb0, int kb1, int nb, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo, int accumulate,
                    const int *tiles, int ntiles)
   {
     if (J.d.njobs == 0 || ntiles == 0) return;
     const int ksm = std::max(kb0, kb1) * 4;
-    const size_t lds = (size_t) kGemmMaxSeg * nb * ksm * 64 * sizeof(T);
+    // weight tiles staged at a time: as many as fit kGemmLdsBudget, so that the wide tiles of 64-channel models (32 kB
+    // in fp64) leave room for several blocks per CU
+    const size_t tile_bytes = (size_t) nb * ksm * 64 * sizeof(T);
+    const int mseg = std::max(1, std::min(kGemmMaxSeg, (int) (kGemmLdsBudget / tile_bytes)));
+    const size_t lds = (size_t) mseg * tile_bytes;
     // single-segment jobs (one weight tile each: projections, reverse of the product reduces) walk several groups of
     // atom tiles per block when the grid is large: the staging of the tile is what they spend their time on
-    const int groups = (ntiles + 4 * kGemmTilesPerWave - 1) / (4 * kGemmTilesPerWave);
+    const bool widest = kb0 == 4 && kb1 == 4 && nb == 4;
+    const int tpw = widest ? 1 : 2;      // = gemm_tiles_per_wave<kb0, kb1, nb>()
+    const int nwave = widest ? 8 : 4;    // waves of a block: the widest weight tiles (32 kB in fp64) are shared by more atom tiles
+    const int groups = (ntiles + nwave * tpw - 1) / (nwave * tpw);
     const int reps = J.d.max_seg == 1 ? std::max(1, std::min(8, (int) ((long long) J.d.njobs * groups / 8192))) : 1;
     const dim3 grid(J.d.njobs, (groups + reps - 1) / reps);
 #define GR_GEMM(A_, B_, C_)                                                                                            \
   {                                                                                                                    \
-    auto kern = k_gemm_jobs<T, A_, B_, C_>;                                                                            \
+    auto kern = k_gemm_jobs<T, A_, B_, C_, gemm_tiles_per_wave<A_, B_, C_>()>;                                         \
     if (lds > 48 * 1024)                                                                                               \
       HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds)); \
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, J.d, X0, nf0, X1, nf1, out, nfo, tiles, ntiles, accumulate, reps); \
+    hipLaunchKernelGGL(kern, grid, dim3(64 * nwave), lds, stream_, J.d, X0, nf0, X1, nf1, out, nfo, tiles, ntiles, accumulate, reps, mseg); \
   }
 #define GR_GEMM_C(A_, B_)                                                                                              \
   switch (nb) {                                                                                                        \

@@ -731,48 +731,51 @@ template<class T> struct GemmJobs {
   int drow[16];               // accumulator row of (lane / 16, register), probed on the device
 };
 
-constexpr int kGemmMaxSeg = 4;      // weight tiles staged in LDS at a time
-constexpr int kGemmTilesPerWave = 2;
+constexpr int kGemmMaxSeg = 4;      // most weight tiles staged in LDS at a time (the launch passes the number, mseg)
+// atom tiles of a wave (TPW): 2, and 1 for the widest tiles (64 channels in, 64 out), whose accumulators and operands
+// of two atom tiles would leave two waves per SIMD
+template<int KB0, int KB1, int NB> constexpr int gemm_tiles_per_wave() { return KB0 == 4 && KB1 == 4 && NB == 4 ? 1 : 2; }
 
-template<class T, int KB0, int KB1, int NB>
-__global__ __launch_bounds__(256) void k_gemm_jobs(GemmJobs<T> J, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo,
-                                                   const int *tile_atoms, int ntiles, int accumulate, int reps)
+template<class T, int KB0, int KB1, int NB, int TPW>
+__global__ __launch_bounds__(512) void k_gemm_jobs(GemmJobs<T> J, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo,
+                                                   const int *tile_atoms, int ntiles, int accumulate, int reps, int mseg)
 {
-  // reps > 1 (only when every job has at most kGemmMaxSeg segments): the block stages its weight tiles once and walks
-  // `reps` groups of atom tiles with them
+  // mseg <= kGemmMaxSeg weight tiles are staged at a time (dynamic LDS: mseg tiles; wide tiles are staged fewer at a
+  // time so that several blocks fit a CU).  reps > 1 (only when every job has one segment): the block stages its
+  // weight tile once and walks `reps` groups of atom tiles with it
   typedef typename Mfma<T>::v4 v4;
   constexpr int KS0 = KB0 * 4, KS1 = KB1 * 4, KSM = KS0 > KS1 ? KS0 : KS1, K0 = KB0 * 16, K1 = KB1 * 16, N = NB * 16;
   extern __shared__ __align__(16) unsigned char smem_raw[];
-  T *wl = reinterpret_cast<T *>(smem_raw);      // [kGemmMaxSeg][NB][KSM][64]
+  T *wl = reinterpret_cast<T *>(smem_raw);      // [mseg][NB][KSM][64]
   __shared__ int s_src[kGemmMaxSeg], s_fn[kGemmMaxSeg];
   __shared__ T s_scale[kGemmMaxSeg];
   const int job = blockIdx.x;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = blockDim.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int sg0 = J.seg_off[job], sg1 = J.seg_off[job + 1];
   const int fo = J.job_out[job];
   const T js = J.job_scale[job];
   for (int rep = 0; rep < reps; rep++) {
-    const int tile0 = ((blockIdx.y * reps + rep) * 4 + wave) * kGemmTilesPerWave;
-    if (rep > 0 && (blockIdx.y * reps + rep) * 4 * kGemmTilesPerWave >= ntiles) break;    // uniform over the block
-    v4 acc[kGemmTilesPerWave][NB];
-    int arow[kGemmTilesPerWave];            // atom of this lane's A row
+    const int tile0 = ((blockIdx.y * reps + rep) * nwave + wave) * TPW;
+    if (rep > 0 && (blockIdx.y * reps + rep) * nwave * TPW >= ntiles) break;    // uniform over the block
+    v4 acc[TPW][NB];
+    int arow[TPW];            // atom of this lane's A row
 #pragma unroll
-    for (int i = 0; i < kGemmTilesPerWave; i++) {
+    for (int i = 0; i < TPW; i++) {
       const int tile = tile0 + i;
       arow[i] = tile < ntiles ? tile_atoms[tile * 16 + c] : -1;
 #pragma unroll
       for (int cb = 0; cb < NB; cb++) acc[i][cb] = v4{0, 0, 0, 0};
     }
-    for (int sg = sg0; sg < sg1; sg += kGemmMaxSeg) {
-      const int ns = sg1 - sg < kGemmMaxSeg ? sg1 - sg : kGemmMaxSeg;
+    for (int sg = sg0; sg < sg1; sg += mseg) {
+      const int ns = sg1 - sg < mseg ? sg1 - sg : mseg;
       if (rep == 0) {
         __syncthreads();
         for (int q = 0; q < ns; q++) {
           const int src = J.seg_src[sg + q];
           const int ks = src == 0 ? KS0 : KS1;
           const T *wf = (src == 0 ? J.WF0 : J.WF1) + (long long) J.seg_w[sg + q] * NB * ks * 64;
-          for (int e = threadIdx.x; e < NB * ks * 64; e += 256) {
+          for (int e = threadIdx.x; e < NB * ks * 64; e += blockDim.x) {
             const int cb = e / (ks * 64), rem = e % (ks * 64);
             wl[(q * NB + cb) * KSM * 64 + rem] = wf[e];
           }
@@ -781,7 +784,7 @@ __global__ __launch_bounds__(256) void k_gemm_jobs(GemmJobs<T> J, const T *X0, i
         __syncthreads();
       }
 #pragma unroll
-      for (int i = 0; i < kGemmTilesPerWave; i++) {
+      for (int i = 0; i < TPW; i++) {
         for (int q = 0; q < ns; q++) {
           const T sc = s_scale[q];
           const T *wq = wl + q * NB * KSM * 64 + lane;
@@ -819,7 +822,7 @@ __global__ __launch_bounds__(256) void k_gemm_jobs(GemmJobs<T> J, const T *X0, i
     }
     // accumulator (g, v) holds row drow[4 g + v] of the tile, column cb * 16 + c
 #pragma unroll
-    for (int i = 0; i < kGemmTilesPerWave; i++) {
+    for (int i = 0; i < TPW; i++) {
       const int tile = tile0 + i;
       if (tile >= ntiles) continue;
 #pragma unroll
