@@ -57,8 +57,9 @@ def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4,
         by = E * (s * C * nl + s * nlm + 4 + nslot * C * s) + N * nslot * nlm * C * s
         return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
     if name == "pair_bwd":
-        # per edge: R1 and dR1 rows, Y and its gradient, neighbour rows, dE/dI rows read-modify-written, geometry, forces
-        by = E * (2 * s * C * nl + 4 * s * nlm + nslot * C * s + 2 * nI * C * s + 28 + 24) + N * (nslot * nlm * C * s + 24)
+        # per edge: R1 and dR1 rows, Y and its two tangential gradients, neighbour rows, dE/dI rows read-modify-written,
+        # geometry, forces
+        by = E * (2 * s * C * nl + 3 * s * nlm + nslot * C * s + 2 * nI * C * s + 28 + 24) + N * (nslot * nlm * C * s + 24)
         return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
     if name in ("radial_mlp", "radial_R", "radial_R1"):
         # value + tangent through the 3 layers: 2 * 2 * E * sum n_in n_out

@@ -18,26 +18,60 @@
 
 namespace grhip {
 
-// One thread per edge: YG[e] = (Y[nlm], G[nlm][3]) (row width W = 4 nlm), or Y[nlm] alone (W = nlm, no gradients).
+// Two unit vectors that span the plane normal to the unit vector u: e1 = a x u / |a x u| with a the coordinate axis on
+// which u has its smallest component, e2 = u x e1.  A pure function of u: the kernel that stores tangential gradients
+// and the kernel that turns their adjoints into a force compute the same pair.
+__device__ inline void tangent_basis(const double *u, double *e1, double *e2)
+{
+  const double ax = fabs(u[0]), ay = fabs(u[1]), az = fabs(u[2]);
+  double a[3] = {0.0, 0.0, 0.0};
+  if (ax <= ay && ax <= az) a[0] = 1.0;
+  else if (ay <= az) a[1] = 1.0;
+  else a[2] = 1.0;
+  const double c0 = a[1] * u[2] - a[2] * u[1], c1 = a[2] * u[0] - a[0] * u[2], c2 = a[0] * u[1] - a[1] * u[0];
+  const double inv = 1.0 / sqrt(c0 * c0 + c1 * c1 + c2 * c2);
+  e1[0] = c0 * inv; e1[1] = c1 * inv; e1[2] = c2 * inv;
+  e2[0] = u[1] * e1[2] - u[2] * e1[1]; e2[1] = u[2] * e1[0] - u[0] * e1[2]; e2[2] = u[0] * e1[1] - u[1] * e1[0];
+}
+
+// One thread per edge: YG[e] = (Y[nlm], D1[nlm], D2[nlm]) (row width W = 3 nlm), or Y[nlm] alone (W = nlm, no
+// gradients).  D1 = G . e1, D2 = G . e2 are the components of the gradient G of the polynomial extension of Y along the
+// tangent vectors of the bond (tangent_basis): the bond force only uses the part of sum_lm gY_lm G_lm normal to the bond,
+// g - (g . rhat) rhat = (g . e1) e1 + (g . e2) e2, so two components per harmonic carry all of it.
 // The lanes write their rows into an LDS tile, the block copies the tile out in consecutive addresses.
-// block: 64 threads; dynamic LDS: 64 * (W + 1) values.
+// block: 64 threads; dynamic LDS: 64 * (4 nlm + 1) values with gradients, 64 * (nlm + 1) without.
 template<class T> __global__ void k_sh_edges(ShCoef sh, const double *rh, const long long *n_edges, int nlm, int grad, T *YG)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *tile = reinterpret_cast<T *>(smem_raw);
-  const int W = grad ? 4 * nlm : nlm, t = threadIdx.x;
+  const int W = grad ? 3 * nlm : nlm, WT = (grad ? 4 * nlm : nlm) + 1, t = threadIdx.x;
   const long long ne = *n_edges, e0 = blockIdx.x * 64ll, e = e0 + t;
   if (e0 >= ne) return;
   if (e < ne) {
     const double *u = rh + 3 * e;
-    T *row = tile + t * (W + 1);
-    if (grad) sh_eval<true, T>(sh, u[0], u[1], u[2], row, row + nlm);
-    else sh_eval<false, T>(sh, u[0], u[1], u[2], row, nullptr);
+    T *row = tile + t * WT;
+    if (grad) {
+      sh_eval<true, T>(sh, u[0], u[1], u[2], row, row + nlm);
+      double e1[3], e2[3];
+      tangent_basis(u, e1, e2);
+      for (int q = 0; q < nlm; q++) {      // in place: D1, D2 of harmonic q over the first two components of its G
+        T *gq = row + nlm + 3 * q;
+        const double g0 = (double) gq[0], g1 = (double) gq[1], g2 = (double) gq[2];
+        gq[0] = (T) (g0 * e1[0] + g1 * e1[1] + g2 * e1[2]);
+        gq[1] = (T) (g0 * e2[0] + g1 * e2[1] + g2 * e2[2]);
+      }
+    } else {
+      sh_eval<false, T>(sh, u[0], u[1], u[2], row, nullptr);
+    }
   }
   __syncthreads();
   const int rows = (int) (ne - e0 < 64 ? ne - e0 : 64);
   T *out = YG + e0 * W;
-  for (int q = t; q < rows * W; q += 64) out[q] = tile[(q / W) * (W + 1) + q % W];
+  for (int q = t; q < rows * W; q += 64) {
+    const int col = q % W;
+    const int src = col < nlm ? col : (col < 2 * nlm ? nlm + 3 * (col - nlm) : nlm + 3 * (col - 2 * nlm) + 1);
+    out[q] = tile[(q / W) * WT + src];
+  }
 }
 
 // M[atom][slot][n] = z[mu_atom][n]
@@ -170,10 +204,11 @@ __device__ inline double wave_sum4(double v0, double v1, double v2, double v3, i
 // grid: (atoms, slot groups); block: spb * C threads rounded up to a wave, spb slots per block (a kernel argument);
 // dynamic LDS: kPairChunk * (NT + 2 nl C) values.  Every block adds the force of its slots to the bond's two atoms.
 // gP: adjoint of P of the atom.
-//   S_l = sum_m Y_lm gP[lm],  T_l,d = sum_m G_lm,d gP[lm]                      (per thread: slot, n)
+//   S_l = sum_m Y_lm gP[lm],  T_l,k = sum_m D_k,lm gP[lm], k = 1, 2 (tangential gradients)   (per thread: slot, n)
 //   dE/dI_j[slot][n] += sum_l R1_l S_l                                        (slots < nI)
-//   dE/dx = sum_{slot,n,l} S_l dR1_l M_j,   g_d = sum_{slot,n,l} T_l,d R1_l M_j
-//   fv = dE/dx / rc rhat + (g - (g . rhat) rhat) / r;  f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv
+//   dE/dx = sum_{slot,n,l} S_l dR1_l M_j,   g_k = sum_{slot,n,l} T_l,k R1_l M_j
+//   fv = dE/dx / rc rhat + (g_1 e1 + g_2 e2) / r  (= the reference's dE/dx / rc rhat + (g - (g . rhat) rhat) / r with
+//   g the Cartesian sum);  f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv
 template<class T, int NLM>
 __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ YG,
                            const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
@@ -203,46 +238,44 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
   for (long long base = e0; base < e1; base += kPairChunk) {
     const int nb = (int) (e1 - base < kPairChunk ? e1 - base : kPairChunk);
     __syncthreads();
-    touch += pair_stage<T>(ej, M, R1, dR1, YG, nlm * 4, nlm * 4, base, nb, nslot, C, noutp, active, slot, n, Msh, Rsh, dRsh, NT);
+    touch += pair_stage<T>(ej, M, R1, dR1, YG, nlm * 3, nlm * 3, base, nb, nslot, C, noutp, active, slot, n, Msh, Rsh, dRsh, NT);
     if (t < kPairChunk * 4) bsum[t >> 2][t & 3] = 0.0;
     __syncthreads();
     for (int b = 0; b < nb; b++) {
       const long long e = base + b;
       const T m = Msh[b * NT + t];
       const T *r = Rsh + b * noutp + n, *dr = dRsh + b * noutp + n;
-      const T *yg = YG + e * nlm * 4;
-      T sI = (T) 0, dE = (T) 0, t0 = (T) 0, t1 = (T) 0, t2 = (T) 0;
+      const T *yg = YG + e * nlm * 3;
+      T sI = (T) 0, dE = (T) 0, t1 = (T) 0, t2 = (T) 0;
       // every l is the body of a loop that runs `one` (= 1, a kernel argument) times: its uniform loads then stay inside
       // it (all harmonics of a bond at once need more scalar registers than there are)
 #pragma unroll
       for (int l = 0; l <= kKernMaxL; l++)
         if (l * l < NLM) for (int it = 0; it < one; it++) {
-          T S = (T) 0, a0 = (T) 0, a1 = (T) 0, a2 = (T) 0;
+          T S = (T) 0, a1 = (T) 0, a2 = (T) 0;
 #pragma unroll
           for (int mm = 0; mm < 2 * l + 1; mm++) {
-            const T *q = yg + nlm + (l * l + mm) * 3;
             const T gv = g[l * l + mm];
-            S += yg[l * l + mm] * gv; a0 += q[0] * gv; a1 += q[1] * gv; a2 += q[2] * gv;
+            S += yg[l * l + mm] * gv; a1 += yg[nlm + l * l + mm] * gv; a2 += yg[2 * nlm + l * l + mm] * gv;
           }
           const T rl = r[l * C], drl = dr[l * C];
           sI += rl * S;
           dE += drl * S;
-          t0 += rl * a0; t1 += rl * a1; t2 += rl * a2;
+          t1 += rl * a1; t2 += rl * a2;
         }
       if (active && slot < nI) atomicAdd(&gM[((long long) ej[e] * nI + slot) * C + n], sI);
-      const double c = wave_sum4((double) (dE * m), (double) (t0 * m), (double) (t1 * m), (double) (t2 * m), lane);
-      if (lane < 4) atomicAdd(&bsum[b][lane], c);    // lanes 0..3: dE/dx, g_y, g_x, g_z  (order v0, v2, v1, v3)
+      const double c = wave_sum4((double) (dE * m), (double) (t1 * m), (double) (t2 * m), 0.0, lane);
+      if (lane < 3) atomicAdd(&bsum[b][lane], c);    // lanes 0..2: dE/dx, g . e2, g . e1  (order v0, v2, v1, v3)
     }
     __syncthreads();
     if (t < nb) {
       const long long e = base + t;
       const double *u = rh + 3 * e;
       const double r = rlen[e], rc = rcut[e];
-      const double gv[3] = {bsum[t][2], bsum[t][1], bsum[t][3]};
-      const double dEdr = bsum[t][0] / rc;
-      const double gr = gv[0] * u[0] + gv[1] * u[1] + gv[2] * u[2];
-      double fv[3];
-      for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + (gv[d] - gr * u[d]) / r;
+      const double dEdr = bsum[t][0] / rc, g1 = bsum[t][2] / r, g2 = bsum[t][1] / r;
+      double e1[3], e2[3], fv[3];
+      tangent_basis(u, e1, e2);
+      for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + g1 * e1[d] + g2 * e2[d];
       const int jj = ej[e];
       for (int d = 0; d < 3; d++) {
         fi[d] += fv[d];
