@@ -504,7 +504,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   const int yw = forces ? 3 * nlm_ : nlm_;    // row of an edge: Y[nlm] and, for forces, the two tangential gradients D1[nlm], D2[nlm]
   YG_.ensure(ecap * yw * sizeof(T));
   stage("sh_edges", [&] {
-    const size_t lds = (size_t) 64 * ((forces ? 4 * nlm_ : nlm_) + 1) * sizeof(T);
+    const size_t lds = (size_t) 64 * (yw + 1) * sizeof(T);
     auto kern = k_sh_edges<T>;
     if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
     hipLaunchKernelGGL(kern, dim3((unsigned) ((ecap + 63) / 64)), dim3(64), lds, stream_, sh_, rh_.as<double>(), n_edges, nlm_, forces ? 1 : 0,

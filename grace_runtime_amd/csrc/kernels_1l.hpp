@@ -35,9 +35,20 @@ struct ShCoef {
 // Real spherical harmonics Y[lm] (stride ys) of the unit vector (rx, ry, rz) and, with GRAD, the gradient
 // G[lm][3] of their polynomial extension.  Same recursion as fused_cpu.h:712-798, one bond per thread, fp64.
 // LMAX: compile-time bound of co.lmax (the register arrays of the recursion are sized by it).
+// With e1, e2 and D2 given, the gradient is stored as its two components along e1 and e2 instead: G[lm] = grad . e1,
+// D2[lm] = grad . e2.
 template<bool GRAD, class TY, int LMAX = kKernMaxL>
-__device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz, TY *Y, TY *G)
+__device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz, TY *Y, TY *G, const double *e1 = nullptr,
+                               const double *e2 = nullptr, TY *D2 = nullptr)
 {
+  auto put = [&](int lm, double gx, double gy, double gz) {
+    if (e1) {
+      G[lm] = (TY) (gx * e1[0] + gy * e1[1] + gz * e1[2]);
+      D2[lm] = (TY) (gx * e2[0] + gy * e2[1] + gz * e2[2]);
+    } else {
+      G[3 * lm] = (TY) gx; G[3 * lm + 1] = (TY) gy; G[3 * lm + 2] = (TY) gz;
+    }
+  };
   double plm[(LMAX + 1) * (LMAX + 2) / 2], dplm[(LMAX + 1) * (LMAX + 2) / 2];
   const int lmax = co.lmax < LMAX ? co.lmax : LMAX;
   plm[0] = 1.0;
@@ -73,7 +84,7 @@ __device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz
     if (l <= lmax) {
       const int c = l * (l + 1), p0 = l * (l + 1) / 2;
       Y[c] = (TY) plm[p0];
-      if (GRAD) { G[3 * c] = (TY) 0; G[3 * c + 1] = (TY) 0; G[3 * c + 2] = (TY) dplm[p0]; }
+      if (GRAD) put(c, 0.0, 0.0, dplm[p0]);
       double pr = rx, pi = ry, prx = 1.0, pry = 0.0, pix = 0.0, piy = 1.0;
 #pragma unroll
       for (int mm = 1; mm <= l; mm++) {
@@ -83,12 +94,8 @@ __device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz
         Y[c - mm] = (TY) (sg * pi * pv);
         if (GRAD) {
           const double dpv = dplm[p0 + mm];
-          G[3 * (c + mm)] = (TY) (sg * prx * pv);
-          G[3 * (c + mm) + 1] = (TY) (sg * pry * pv);
-          G[3 * (c + mm) + 2] = (TY) (sg * pr * dpv);
-          G[3 * (c - mm)] = (TY) (sg * pix * pv);
-          G[3 * (c - mm) + 1] = (TY) (sg * piy * pv);
-          G[3 * (c - mm) + 2] = (TY) (sg * pi * dpv);
+          put(c + mm, sg * prx * pv, sg * pry * pv, sg * pr * dpv);
+          put(c - mm, sg * pix * pv, sg * piy * pv, sg * pi * dpv);
           const double nrx = prx * rx + pr - pix * ry, nry = pry * rx - piy * ry - pi;
           const double nix = prx * ry + pix * rx + pi, niy = pry * ry + pr + piy * rx;
           prx = nrx; pry = nry; pix = nix; piy = niy;

@@ -39,27 +39,21 @@ __device__ inline void tangent_basis(const double *u, double *e1, double *e2)
 // tangent vectors of the bond (tangent_basis): the bond force only uses the part of sum_lm gY_lm G_lm normal to the bond,
 // g - (g . rhat) rhat = (g . e1) e1 + (g . e2) e2, so two components per harmonic carry all of it.
 // The lanes write their rows into an LDS tile, the block copies the tile out in consecutive addresses.
-// block: 64 threads; dynamic LDS: 64 * (4 nlm + 1) values with gradients, 64 * (nlm + 1) without.
+// block: 64 threads; dynamic LDS: 64 * (W + 1) values.
 template<class T> __global__ void k_sh_edges(ShCoef sh, const double *rh, const long long *n_edges, int nlm, int grad, T *YG)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *tile = reinterpret_cast<T *>(smem_raw);
-  const int W = grad ? 3 * nlm : nlm, WT = (grad ? 4 * nlm : nlm) + 1, t = threadIdx.x;
+  const int W = grad ? 3 * nlm : nlm, t = threadIdx.x;
   const long long ne = *n_edges, e0 = blockIdx.x * 64ll, e = e0 + t;
   if (e0 >= ne) return;
   if (e < ne) {
     const double *u = rh + 3 * e;
-    T *row = tile + t * WT;
+    T *row = tile + t * (W + 1);
     if (grad) {
-      sh_eval<true, T>(sh, u[0], u[1], u[2], row, row + nlm);
       double e1[3], e2[3];
       tangent_basis(u, e1, e2);
-      for (int q = 0; q < nlm; q++) {      // in place: D1, D2 of harmonic q over the first two components of its G
-        T *gq = row + nlm + 3 * q;
-        const double g0 = (double) gq[0], g1 = (double) gq[1], g2 = (double) gq[2];
-        gq[0] = (T) (g0 * e1[0] + g1 * e1[1] + g2 * e1[2]);
-        gq[1] = (T) (g0 * e2[0] + g1 * e2[1] + g2 * e2[2]);
-      }
+      sh_eval<true, T>(sh, u[0], u[1], u[2], row, row + nlm, e1, e2, row + 2 * nlm);
     } else {
       sh_eval<false, T>(sh, u[0], u[1], u[2], row, nullptr);
     }
@@ -67,11 +61,7 @@ template<class T> __global__ void k_sh_edges(ShCoef sh, const double *rh, const 
   __syncthreads();
   const int rows = (int) (ne - e0 < 64 ? ne - e0 : 64);
   T *out = YG + e0 * W;
-  for (int q = t; q < rows * W; q += 64) {
-    const int col = q % W;
-    const int src = col < nlm ? col : (col < 2 * nlm ? nlm + 3 * (col - nlm) : nlm + 3 * (col - 2 * nlm) + 1);
-    out[q] = tile[(q / W) * WT + src];
-  }
+  for (int q = t; q < rows * W; q += 64) out[q] = tile[(q / W) * (W + 1) + q % W];
 }
 
 // M[atom][slot][n] = z[mu_atom][n]
