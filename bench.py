@@ -37,8 +37,8 @@ HBM_PEAK = 8000.0                 # GB/s
 # script, counters scaled by what they read for the 1 GiB copy kernel; summaries under profiles/): (workload, kernel)
 MEASURED_TRAFFIC = {
     ("config2", "radial_mlp"): 7.0e6 + 1216.3e6,        # fetch + write of k_radial<double,4,0,0,true>
-    ("config3", "pair_bwd"): 11883.6e6 + 2822.1e6,      # fetch + write of k_pair_bwd<double,25>
-    ("config4", "pair_bwd_L3"): 64600e6 + 31459e6,      # the layer-3 launches of k_pair_bwd<double,36> (layer 2: 35.2 + 16.3 GB)
+    ("config3", "pair_bwd"): 11234.9e6 + 2773.0e6,      # fetch + write of k_pair_bwd<double,25>
+    ("config4", "pair_bwd_L3"): 48727e6 + 30596e6,      # the layer-3 launches of k_pair_bwd<double,36> (layer 2: 25.6 + 15.2 GB)
 }
 
 
