@@ -395,6 +395,14 @@ int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j
   });
 }
 
+int gr_engine_radial_noalloc(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz)
+{
+  return guarded([&] {
+    if (!e || !e->eng) throw grhip::InvalidArgument("null engine");
+    e->eng->radial_noalloc(m, x, mu_j, Rz, dRz);
+  });
+}
+
 int gr_engine_debug_copy(gr_engine *e, int64_t bytes)
 {
   return guarded([&] {

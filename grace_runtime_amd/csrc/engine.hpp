@@ -93,6 +93,9 @@ class Engine {
   // radial functions of the device kernel for the given x = r / rc and neighbour elements: R z and dR/dx z,
   // [m][nl][C] (tests of the MFMA kernel against the CPU restatement)
   virtual void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) = 0;
+  // the same functions for callers that must not allocate device memory: x [m], mu_j [m], Rz, dRz [m][nl][C] are device
+  // arrays of the engine's GPU, the staging rows come from a fixed device array of the library (bounded m)
+  virtual void radial_noalloc(int m, const double *x, const int *mu_j, double *Rz, double *dRz) = 0;
 };
 
 // precision: 64 (network arithmetic in fp64) or 32 (fp32 network, fp64 geometry and sums)

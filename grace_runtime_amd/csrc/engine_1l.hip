@@ -4,9 +4,68 @@
 // CG terms after libgrace/src/fused_1l.cpp:176-216.
 #include "engine_common.hpp"
 
+#include <mutex>
+
 namespace grhip {
 
 namespace {
+
+// ---------------------------------------------------------------------------------------------------------------
+// Fixed device memory of the radial call that allocates nothing (radial_noalloc): a header (error flag), the checked
+// neighbour elements and the padded rows the radial kernel writes.  Every GPU the library runs on holds its own copy
+// of the array until the process ends.  In host code the array's name is only a handle for hipGetSymbolAddress: the
+// address of a device's copy is looked up once per device (with that device current, when the first GRACE-1L engine
+// of the device is built) and kept in scratch_ptr; host code uses that pointer and never the name.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr size_t kScratchBytes = (size_t) 32 << 20;
+constexpr size_t kScratchHeader = 256;
+constexpr int kScratchMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+static void *scratch_ptr[kScratchMaxDevices] = {};
+static std::mutex scratch_mutex;
+
+// address of the current device's copy of `scratch`
+static unsigned char *scratch_of_device(int device)
+{
+  if (device < 0 || device >= kScratchMaxDevices) throw Error("device index " + std::to_string(device) + " out of range");
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[device]) {
+    void *p = nullptr;
+    HIP_CHECK(hipSetDevice(device));
+    HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) throw Error("hipGetSymbolAddress gave no address for the library's fixed device array");
+    scratch_ptr[device] = p;
+  }
+  return static_cast<unsigned char *>(scratch_ptr[device]);
+}
+
+// neighbour elements of the caller checked into the fixed array: an element outside 0 .. nel-1 is replaced by 0 (so that
+// the radial kernel stays inside its tables) and reported through *bad
+static __global__ void k_stage_elements(const int *mu, int m, int nel, int *out, int *bad)
+{
+  const int q = blockIdx.x * blockDim.x + threadIdx.x;
+  if (q >= m) return;
+  const int v = mu[q];
+  const bool ok = v >= 0 && v < nel;
+  out[q] = ok ? v : 0;
+  if (!ok) atomicMax(bad, 1);
+}
+// the flag starts at zero on every call (a fill kernel: a memset node would not survive a graph capture by the caller)
+static __global__ void k_clear_flag(int *bad)
+{
+  if (threadIdx.x == 0 && blockIdx.x == 0) *bad = 0;
+}
+// padded rows [m][noutp] (column l * CP + n) -> caller's [m][nl][C] doubles
+template<class T> static __global__ void k_unpack_radial(const T *R, const T *dR, long long total, int nl, int C, int CP, int noutp, double *oR, double *odR)
+{
+  for (long long i = blockIdx.x * (long long) blockDim.x + threadIdx.x; i < total; i += (long long) gridDim.x * blockDim.x) {
+    const long long q = i / (nl * C);
+    const int rest = (int) (i - q * (nl * C)), l = rest / C, n = rest - l * C;
+    const long long src = q * noutp + l * CP + n;
+    oR[i] = (double) R[src];
+    odR[i] = (double) dR[src];
+  }
+}
 
 template<class T> class Engine1L final : public EngineBase {
  public:
@@ -15,14 +74,17 @@ template<class T> class Engine1L final : public EngineBase {
   {
     this->template probe_mfma<T>();
     build();
+    scratch_dev_ = scratch_of_device(device);    // set-up: the device is current (EngineBase)
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
   }
 
   int layers() const override { return 1; }
   void run(const RunFlags &fl) override;
   void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) override;
+  void radial_noalloc(int m, const double *x, const int *mu_j, double *Rz, double *dRz) override;
 
  private:
+  unsigned char *scratch_dev_ = nullptr;    // this device's copy of the fixed array (hipGetSymbolAddress)
   std::shared_ptr<const Model1L> model_;
   bool jit_all_ = false;
 
@@ -443,6 +505,50 @@ template<class T> void Engine1L<T>::debug_radial(int m, const double *x, const i
         Rz[((size_t) q * nl_ + l) * C_ + c] = (double) hR[(size_t) q * noutp_ + l * CP_ + c];
         dRz[((size_t) q * nl_ + l) * C_ + c] = (double) hdR[(size_t) q * noutp_ + l * CP_ + c];
       }
+}
+
+// The radial functions of debug_radial for device arrays, without any device allocation: the staging rows live in the
+// fixed array.  Calls on one GPU share that array (also calls of different engines): they must not overlap.
+template<class T> void Engine1L<T>::radial_noalloc(int m, const double *x, const int *mu_j, double *Rz, double *dRz)
+{
+  HIP_CHECK(hipSetDevice(device_));
+  if (m < 0) throw InvalidArgument("negative number of radial arguments");
+  if (m == 0) return;
+  if (!x || !mu_j || !Rz || !dRz) throw InvalidArgument("x, mu_j, Rz and dRz are required");
+  for (const void *p : {(const void *) x, (const void *) mu_j, (const void *) Rz, (const void *) dRz}) {
+    hipPointerAttribute_t at{};
+    if (hipPointerGetAttributes(&at, p) != hipSuccess || at.type != hipMemoryTypeDevice || at.device != device_) {
+      (void) hipGetLastError();
+      throw InvalidArgument("x, mu_j, Rz and dRz must be device memory of the engine's GPU");
+    }
+  }
+  auto align = [](size_t b) { return (b + 255) / 256 * 256; };
+  const size_t mu_bytes = align((size_t) m * sizeof(int)), row_bytes = align((size_t) m * noutp_ * sizeof(T));
+  const size_t need = kScratchHeader + mu_bytes + 2 * row_bytes;
+  if (need > kScratchBytes) {
+    const size_t per = sizeof(int) + 2 * (size_t) noutp_ * sizeof(T);
+    throw InvalidArgument("radial call without allocations: " + std::to_string(m) + " arguments need " + std::to_string(need) +
+                          " bytes of the fixed " + std::to_string(kScratchBytes) + "-byte device array (at most " +
+                          std::to_string((kScratchBytes - kScratchHeader - 768) / per) + " arguments for this model and precision)");
+  }
+  unsigned char *base = scratch_dev_;
+  int *bad = reinterpret_cast<int *>(base);
+  long long *nedges = reinterpret_cast<long long *>(base + 8);    // not read: the count is passed by value
+  int *mu = reinterpret_cast<int *>(base + kScratchHeader);
+  T *R = reinterpret_cast<T *>(base + kScratchHeader + mu_bytes), *dR = reinterpret_cast<T *>(base + kScratchHeader + mu_bytes + row_bytes);
+  hipLaunchKernelGGL(k_clear_flag, dim3(1), dim3(64), 0, stream_, bad);
+  hipLaunchKernelGGL(k_stage_elements, dim3((unsigned) ((m + 255) / 256)), dim3(256), 0, stream_, mu_j, m, nel_, mu, bad);
+  HIP_CHECK(hipGetLastError());
+  launch_radial(0, m, x, mu, R, dR, nedges);
+  HIP_CHECK(hipGetLastError());
+  const long long total = (long long) m * nl_ * C_;
+  hipLaunchKernelGGL(k_unpack_radial<T>, dim3((unsigned) std::min<long long>((total + 255) / 256, 4096)), dim3(256), 0, stream_, (const T *) R,
+                     (const T *) dR, total, nl_, C_, CP_, noutp_, Rz, dRz);
+  HIP_CHECK(hipGetLastError());
+  int flag = 0;
+  HIP_CHECK(hipMemcpyAsync(&flag, bad, sizeof(int), hipMemcpyDeviceToHost, stream_));
+  HIP_CHECK(hipStreamSynchronize(stream_));
+  if (flag) throw InvalidArgument("neighbour element out of range");
 }
 
 }    // namespace

@@ -686,6 +686,10 @@ class EngineBase : public Engine, protected BufRegistry {
     ran_ = false;
   }
   int device_index() const override { return device_; }
+  void radial_noalloc(int, const double *, const int *, double *, double *) override
+  {
+    throw Error(who_ + ": the radial call without allocations is available for GRACE-1L engines");
+  }
   // tiles of 16 atoms of one element (-1 padded), in atom order within an element, elements ascending;
   // el_off[e] .. el_off[e + 1]: the tiles of element e
   static std::vector<int> element_tiles(const std::vector<int> &mu, int nel, std::vector<int> &el_off)

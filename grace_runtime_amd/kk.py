@@ -350,6 +350,16 @@ class Engine:
         check(_lib.lib().gr_engine_debug_radial(self._h, x.shape[0], ptr(x), ptr(mu_j), ptr(R), ptr(dR)))
         return R, dR
 
+    def radial_noalloc(self, x, mu_j, R, dR):
+        """debug_radial on device arrays of the module's GPU (x [m] float64, mu_j [m] int32, R and dR [m, lmax + 1,
+        n_radial] float64, written in place) through the entry point that allocates no device memory."""
+        m = int(x.shape[0])
+        nl, Cn = self.model.lmax + 1, self.model.n_radial
+        check(_lib.lib().gr_engine_radial_noalloc(self._h, m, _device_pointer(x, "x", (m,), "float64"),
+                                                  _device_pointer(mu_j, "mu_j", (m,), "int32"),
+                                                  _device_pointer(R, "R", (m, nl, Cn), "float64"),
+                                                  _device_pointer(dR, "dR", (m, nl, Cn), "float64")))
+
     def debug_copy(self, nbytes):
         check(_lib.lib().gr_engine_debug_copy(self._h, int(nbytes)))
 

@@ -119,6 +119,16 @@ int gr_engine_stage_get(gr_engine *e, int k, char *name, int name_len, double *m
  * Test hook for the radial-MLP kernel (the reference's counterpart is radial_x.h:29-60 evaluated on the host). */
 int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz);
 
+/* gr_engine_debug_radial for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  x [m], mu_j [m], Rz and dRz [m][lmax+1]
+ * [n_radial] are DEVICE arrays of the engine's GPU.  The staging rows of the radial kernel live in a fixed 32 MiB
+ * device array of the library (one per GPU, held until the process ends), so the call makes no hipMalloc / hipFree:
+ * m is bounded by 256 + 4 m + 2 m nl CP s <= 32 MiB (CP = n_radial padded to 16 / 32 / 64, s = 8 or 4 bytes; 13 000
+ * arguments for a 32-channel lmax-4 model in fp64), a larger m gives GR_INVALID with the limit in the message.
+ * GRACE-1L engines only.  The call returns when Rz and dRz are written.  All calls on one GPU share the array: calls
+ * that overlap on one GPU (two threads, two engines) race. */
+int gr_engine_radial_noalloc(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz);
+
 /* Runs a plain device-to-device copy kernel (k_copy_calibration) over `bytes` bytes: the known-size kernel that the
  * rocprof memory counters (FETCH_SIZE, WRITE_SIZE) are scaled by.  No counterpart in the reference. */
 int gr_engine_debug_copy(gr_engine *e, int64_t bytes);
