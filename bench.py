@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the GRACE energy + forces + virial pass on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--precision 64|32] [--no-cpu] [--workload config2|config3|config4]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--precision 64|32] [--no-cpu] [--workload config2|config3|config4|config5]
 
 Default workload (the second benchmark configuration, the one the metric is quoted on): GRACE-1L-shaped random-init model (lmax 4, 32 radial channels, 8 Chebyshev
 functions, radial MLP 8-64-64-160, SiLU) on a bcc W 16x16x16 supercell (8192 atoms, a = 3.165 A, N(0, 0.05 A) jitter,
@@ -12,6 +12,12 @@ readout, reverse pass, forces, virial) over the structure, which is uploaded to 
 MLPs 8-64-64-160, body order 3) on the 4-species fcc 20x20x20 alloy (32 000 atoms, ~2.5 M edges), fp64.
 --workload config4 the fourth: GRACE-3L-shaped model (three layers, lmax 5, 64 channels, radial MLPs (8 + 2 x 32)-128-128-384,
 89-species embedding table) on an amorphous cube of 10 000 atoms with 8 species (~0.72 M edges), fp64.
+--workload config5 the fifth: the GRACE-2L-shaped model with 3 species over 512 independent periodic cells of 32 .. 128 atoms
+(41 701 atoms, ~2.2 M edges) as ONE resident ragged batch; a step is one engine pass over all cells.
+
+Timing: `value` / `ms_per_step` are the mean over the K timed passes (one synchronisation before and one after the K
+passes); `median_ms_per_step` is the median of K passes timed one by one, the reference's protocol
+(docs/benchmarks.md:13: median of the calls after the first).
 
 Prints one JSON line: the metric (us/atom per call), the roofline of the dominant kernel (duration from HIP events
 on the engine's stream, algorithmic flops/bytes of that stage) and the reference CPU path timed on this host.
@@ -27,7 +33,6 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
-sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 PEAK = {64: 78.6, 32: 157.3}      # dense matrix TFLOP/s of MI355X (fp64, fp32)
 HBM_PEAK = 8000.0                 # GB/s
@@ -40,6 +45,9 @@ MEASURED_TRAFFIC = {
     ("config3", "pair_bwd"): 11234.9e6 + 2773.0e6,      # fetch + write of k_pair_bwd<double,25>
     ("config4", "pair_bwd_L3"): 48727e6 + 30596e6,      # the layer-3 launches of k_pair_bwd<double,36> (layer 2: 25.6 + 15.2 GB)
 }
+# the per-atom dense chain of configuration 2 (every FC, product, reduce and readout launch of a pass), same counters
+DENSE_TRAFFIC = {"config2": 6.5e9}
+DENSE_PREFIXES = ("fc_", "prod_", "reduce_", "energy_mlp", "zero_grads", "chain_")
 
 
 def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4, radial_flops=59392.0, slots=None):
@@ -84,7 +92,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--precision", type=int, default=64, choices=[64, 32])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4"])
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5"])
     ap.add_argument("--reps", type=int, default=0, help="supercell repetitions (default: 16 bcc cells / 20 fcc cells per edge)")
     ap.add_argument("--atoms", type=int, default=10000, help="atoms of the amorphous cube of config4")
     a = ap.parse_args()
@@ -93,40 +101,55 @@ def main():
 
     import torch
 
-    import cases
-    from grace_runtime_amd import kk, synth
+    from grace_runtime_amd import kk, synth, workloads
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
     tmp = tempfile.mkdtemp()
-    two = a.workload == "config3"
+    batch = a.workload == "config5"
+    two = a.workload == "config3" or batch
     three = a.workload == "config4"
     reps = a.reps or (20 if two else 16)
     pbc = [True, True, True]
+    structs = None
     if three:
-        mpath = cases.write_model("config4", tmp)
+        mpath = workloads.write_model("config4", tmp)
         with np.load(mpath) as z:
             names = [x.decode() for x in z["element_names"]]
-        pos, cell, _, t89 = cases.structure_config4(natoms=a.atoms)
+        pos, cell, _, t89 = workloads.structure_config4(natoms=a.atoms)
         # the 8 species present become atom types 1..8 of the engine (as a LAMMPS pair_coeff line would map them)
-        species = [names[t - 1] for t in cases.CONFIG4_SPECIES]
-        types = (np.searchsorted(np.array(cases.CONFIG4_SPECIES), t89) + 1).astype(np.int32)
+        species = workloads.config4_species(names)
+        types = workloads.config4_types(t89)
+    elif batch:
+        mpath = workloads.write_model("config5", tmp)
+        species = ["Al", "Ni", "Ti"]
+        structs = workloads.structures_config5()
+        b_natoms, types, pos, b_cells, b_pbc = workloads.batch_arrays(structs)
     elif two:
-        mpath = cases.write_model("config3", tmp)
+        mpath = workloads.write_model("config3", tmp)
         species = ["Al", "Co", "Ni", "Ti"]
         pos, cell = synth.fcc_supercell(3.6, reps)
         pos = synth.jitter(pos, 0.08, 3)
         types = np.random.default_rng(3).integers(1, 5, size=len(pos)).astype(np.int32)
     else:
-        mpath = cases.write_model("config1", tmp)
+        mpath = workloads.write_model("config1", tmp)
         species = ["W"]
         pos, cell = synth.bcc_supercell(3.165, reps)
         pos = synth.jitter(pos, 0.05, 2)
         types = np.ones(len(pos), np.int32)
     N = len(pos)
-    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 6.0, num_threads=len(os.sched_getaffinity(0)))
     model = kk.Model(mpath)
+    t1 = time.perf_counter()
     eng = kk.Engine(model, species, precision=a.precision)
-    eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
+    create_s = time.perf_counter() - t1        # includes the run-time compilation of the model-specialised product kernels
+    if batch:
+        def upload():
+            eng.upload_batch(structs, 6.0)
+    else:
+        perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 6.0, num_threads=len(os.sched_getaffinity(0)))
+
+        def upload():
+            eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
+    upload()
     eng.debug_copy(1 << 30)     # k_copy_calibration over 1 GiB: scales the rocprof FETCH_SIZE / WRITE_SIZE counters
 
     for _ in range(a.warmup):
@@ -139,29 +162,60 @@ def main():
     eng.sync()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / a.steps
-    out = eng.fetch()
-    E = eng.edge_count()
-    # the same pass through the one-call entry point: host buffers in (PCIe), pass, results out; reported beside, never as `value`
-    th = []
-    for _ in range(4):
+    one = []
+    for _ in range(a.steps):
         t1 = time.perf_counter()
-        eng.compute(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
-        th.append(time.perf_counter() - t1)
-    host_ms = float(np.median(th[1:])) * 1e3
-    # the calculator's call (kk.System.compute: positions, cell, types in; host neighbour list, pass, results out), with
-    # the list rebuilt on every call (skin 0) and with the list kept (skin 0.5 A, unmoved atoms)
-    list_ms = {}
-    for label, skin in (("rebuilt", 0.0), ("kept", 0.5)):
-        sysm = kk.System(model, species, skin=skin, precision=a.precision)
-        tl = []
-        for k in range(3):
+        eng.run()
+        eng.sync()
+        one.append(time.perf_counter() - t1)
+    median_ms = float(np.median(one)) * 1e3
+    out = eng.fetch_batch() if batch else eng.fetch()
+    E = eng.edge_count()
+    host_ms, list_ms, batch_ms = None, None, None
+    if batch:
+        # the calculator-level calls: Batch.compute (host arrays, host lists) and Batch.compute_device (device arrays,
+        # device lists), whole batch per call
+        bt = kk.Batch(model, species, precision=a.precision)
+        bt.keep_buffers = True
+        dev = torch.device("cuda", 0)
+        d_t, d_x = torch.tensor(types, device=dev), torch.tensor(pos, device=dev)
+        d_e = torch.zeros(len(structs), dtype=torch.float64, device=dev)
+        d_f = torch.zeros((N, 3), dtype=torch.float64, device=dev)
+        d_v = torch.zeros((len(structs), 6), dtype=torch.float64, device=dev)
+        th, td = [], []
+        for _ in range(3):
             t1 = time.perf_counter()
-            sysm.compute(types, pos + (1e-9 * k if skin == 0.0 else 0.0), cell, pbc)     # any displacement rebuilds a skin-0 list
-            tl.append(time.perf_counter() - t1)
-        assert sysm.rebuilds == (3 if skin == 0.0 else 1)
-        list_ms[label] = float(np.median(tl[1:])) * 1e3
-        del sysm
-    eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
+            bt.compute(b_natoms, types, pos, b_cells, b_pbc)
+            th.append(time.perf_counter() - t1)
+            t1 = time.perf_counter()
+            bt.compute_device(b_natoms, d_t, d_x, b_cells, b_pbc, d_e, forces=d_f, virial=d_v)
+            torch.cuda.synchronize()
+            td.append(time.perf_counter() - t1)
+        batch_ms = {"Batch.compute_host_arrays": round(float(np.median(th[1:])) * 1e3, 3),
+                    "Batch.compute_device": round(float(np.median(td[1:])) * 1e3, 3)}
+        del bt
+    else:
+        # the same pass through the one-call entry point: host buffers in (PCIe), pass, results out; reported beside, never as `value`
+        th = []
+        for _ in range(4):
+            t1 = time.perf_counter()
+            eng.compute(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
+            th.append(time.perf_counter() - t1)
+        host_ms = float(np.median(th[1:])) * 1e3
+        # the calculator's call (kk.System.compute: positions, cell, types in; neighbour list, pass, results out), with
+        # the list rebuilt on every call (skin 0) and with the list kept (skin 0.5 A, unmoved atoms)
+        list_ms = {}
+        for label, skin in (("rebuilt", 0.0), ("kept", 0.5)):
+            sysm = kk.System(model, species, skin=skin, precision=a.precision)
+            tl = []
+            for k in range(3):
+                t1 = time.perf_counter()
+                sysm.compute(types, pos + (1e-9 * k if skin == 0.0 else 0.0), cell, pbc)     # any displacement rebuilds a skin-0 list
+                tl.append(time.perf_counter() - t1)
+            assert sysm.rebuilds == (3 if skin == 0.0 else 1)
+            list_ms[label] = float(np.median(tl[1:])) * 1e3
+            del sysm
+    upload()
 
     # per-stage durations: HIP events around every launch on the engine's stream, averaged over the same K steps
     eng.set_profile(True)
@@ -170,15 +224,15 @@ def main():
         eng.run()
         for k, (ms, cnt) in eng.stage_times().items():
             acc[k] = acc.get(k, 0.0) + ms
+    gemm_flops = eng.stage_flops()       # tile-GEMM flops per stage (live functions only), counted by the engine
     eng.set_profile(False)
     stages = {k: v / a.steps for k, v in acc.items()}
 
     C, nl, nlm, s = (64, 6, 36, 8) if three else (32, 5, 25, a.precision // 8)
     # GRACE-3L: message functions gathered by the pair kernels of layers 2 and 3; radial MLP 8-128-128-384, value + tangent
     extra = dict(radial_flops=4.0 * (8 * 128 + 128 * 128 + 128 * 384), slots={"2": 36, "3": 72}) if three else {}
-    # FC flops (forward: left + right mat-vec per live function; reverse the same), fp64 FMAs on the vector/matrix pipes
-    nA1, nAA1, nAA2 = 25, 44, 141       # informational; exact live counts are the engine's
-    dense_flops = {}
+    # FC / reduce tile GEMMs: flops of the live functions as the engine counts them
+    dense_flops = dict(gemm_flops)
     roof = {}
     for k, ms in stages.items():
         r = stage_model(k, ms, E, N, C, nl, nlm, s, a.precision, dense_flops, **extra)
@@ -187,7 +241,15 @@ def main():
             r["frac"] = r["achieved"] / r["peak"]
             roof[k] = r
     total_ms = sum(stages.values())
-    modelled = {k: v for k, v in roof.items()}
+    # the per-atom dense chain as one entry: every FC, product, reduce and readout launch; flops = the tile GEMMs'
+    dense_ms = sum(v for k, v in stages.items() if k.startswith(DENSE_PREFIXES))
+    dense_fl = sum(v for k, v in gemm_flops.items() if k.startswith(DENSE_PREFIXES))
+    dense = {"ms": round(dense_ms, 4), "share_of_pass": round(dense_ms / total_ms, 4), "gemm_flops": dense_fl,
+             "bound": "mfma", "achieved": round(dense_fl / (dense_ms * 1e-3) / 1e12, 3) if dense_ms > 0 else 0.0, "peak": PEAK[a.precision],
+             "unit": "TFLOP/s", "frac": round(dense_fl / (dense_ms * 1e-3) / 1e12 / PEAK[a.precision], 4) if dense_ms > 0 else 0.0,
+             "traffic": DENSE_TRAFFIC.get(a.workload) if a.precision == 64 and reps == (20 if two else 16) else None,
+             "minimal_bytes": N * (2 * nlm * C * s + 2 * 8 * 32) if not (two or three) else None}
+    modelled = dict(roof)
     dom = max(modelled, key=lambda k: modelled[k]["ms"])
     d = modelled[dom]
     roofline = {"kernel": dom, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"],
@@ -198,7 +260,27 @@ def main():
     cpu = None
     if not a.no_cpu:
         from oracle import ref_lib      # the compiled reference CPU path: the checker, timed here as the baseline
-        if ref_lib.available():
+        if ref_lib.available() and batch:
+            # the reference evaluates a batch one structure at a time (python/grace_runtime/batch.py); sample: the first cells
+            nth = len(os.sched_getaffinity(0))
+            ref = ref_lib.RefModel(mpath, [0, 1, 2])
+            lists = [kk.neighbor_search(p, c, [True, True, True], 6.0) for p, c, _ in structs[:128]]
+            t_end = time.perf_counter() + 20.0
+            done, secs, de, a0 = 0, 0.0, 0.0, 0
+            for (p, c, t), (pm, of, jj, im, sh) in zip(structs[:128], lists):
+                t1 = time.perf_counter()
+                r = ref.compute(t[pm], of, jj, positions=p[pm], image=im, shifts=sh, nthreads=nth)
+                secs += time.perf_counter() - t1
+                de = max(de, abs(r["energy"] - out["energy"][done]) / len(p))
+                done += 1
+                a0 += len(p)
+                if time.perf_counter() > t_end:
+                    break
+            cpu = {"value": round(secs / a0 * 1e6, 4), "unit": "us/atom", "cores": nth, "kind": "reference",
+                   "sample": f"the first {done} cells ({a0} atoms) of the batch, one call of the compiled reference Grace2LFused (fp32 + spline "
+                             f"tables) per cell, neighbour lists not timed",
+                   "dE_per_atom_vs_gpu": de}
+        elif ref_lib.available():
             nth = len(os.sched_getaffinity(0))
             ref = ref_lib.RefModel(mpath, [names.index(x) for x in species] if three else list(range(len(species))))
             args = dict(positions=pos[perm], image=image, shifts=shifts, nthreads=nth)
@@ -220,7 +302,9 @@ def main():
         "metric": "us_per_atom_EFS_call", "value": round(dt / N * 1e6, 5), "unit": "us/atom", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "f64" if a.precision == 64 else "f32", "data": "synthetic",
-        "config": {"workload": (f"GRACE-3L-shaped random-init model (3 layers, lmax 5, 64 ch, radial MLPs (8 + 2 x 32)-128-128-384, 89-species "
+        "config": {"workload": (f"GRACE-2L-shaped random-init model (2 layers, lmax 4, 32 ch, 3 species) over {len(structs)} independent periodic "
+                                f"cells of 32-128 atoms as one ragged batch, {N} atoms, {E} edges, rc 6 A (benchmark configuration 5)") if batch else
+                               (f"GRACE-3L-shaped random-init model (3 layers, lmax 5, 64 ch, radial MLPs (8 + 2 x 32)-128-128-384, 89-species "
                                 f"embedding table, 8 species present) on an amorphous cube of {N} atoms at 0.08 / A^3, {E} edges, rc 6 A "
                                 f"(benchmark configuration 4)") if three else
                                (f"GRACE-2L-shaped random-init model (2 layers, lmax 4, 32 ch, MLPs 8-64-64-160, body order 3) on the "
@@ -229,15 +313,20 @@ def main():
                                 f"{reps}x{reps}x{reps}, {N} atoms, {E} edges, rc 6 A (benchmark configuration 2)"),
                    "atoms": N, "edges": int(E)},
         "atoms_steps_per_s": round(N / dt, 1),
-        "ms_per_call_host_buffers": round(host_ms, 3),
-        "ms_per_calculator_call": {"neighbour_list_rebuilt": round(list_ms["rebuilt"], 3), "neighbour_list_kept": round(list_ms["kept"], 3)},
+        "median_ms_per_step": round(median_ms, 4),
+        "timing": "value, ms_per_step: mean of the K passes on the resident structure; median_ms_per_step: median of K passes timed one by one",
+        "ms_per_call_host_buffers": round(host_ms, 3) if host_ms is not None else None,
+        "ms_per_calculator_call": batch_ms if batch else {"neighbour_list_rebuilt": round(list_ms["rebuilt"], 3),
+                                                          "neighbour_list_kept": round(list_ms["kept"], 3)},
+        "engine_create_s": round(create_s, 3),
         "roofline": roofline,
+        "dense_chain": dense,
         "stages_ms": {k: round(v, 4) for k, v in stages.items()},
         "stages_roofline": {k: {"bound": v["bound"], "achieved": round(v["achieved"], 2), "unit": v["unit"],
                                 "frac": round(v["frac"], 4)} for k, v in roof.items()},
         "sum_stage_ms": round(total_ms, 4),
         "cpu_baseline": cpu,
-        "energy": out["energy"],
+        "energy": float(np.sum(out["energy"])),
     }
     print(json.dumps(res))
 

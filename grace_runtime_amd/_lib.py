@@ -20,7 +20,7 @@ SYMBOLS = [
     "gr_last_error", "gr_abi_version", "gr_device_count", "gr_device_arch", "gr_model_load", "gr_model_get_info",
     "gr_model_element_name", "gr_model_free", "gr_engine_create", "gr_engine_free", "gr_engine_cutoff",
     "gr_compute_csr", "gr_engine_upload", "gr_engine_run", "gr_engine_sync", "gr_engine_fetch",
-    "gr_engine_edge_count", "gr_engine_set_profile", "gr_engine_stage_count", "gr_engine_stage_get",
+    "gr_engine_edge_count", "gr_engine_set_profile", "gr_engine_stage_count", "gr_engine_stage_get", "gr_engine_stage_flops",
     "gr_engine_debug_radial", "gr_engine_radial_noalloc", "gr_engine_debug_copy", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
@@ -84,6 +84,7 @@ def lib():
     L.gr_engine_stage_count.argtypes = [vp]
     L.gr_engine_stage_get.argtypes = [vp, i32, C.c_char_p, i32, C.POINTER(dbl), C.POINTER(i32)]
     L.gr_engine_debug_radial.argtypes = [vp, i32, vp, vp, vp, vp]
+    L.gr_engine_stage_flops.argtypes = [vp, i32, vp]
     L.gr_engine_radial_noalloc.argtypes = [vp, i32, vp, vp, vp, vp]
     L.gr_engine_debug_copy.argtypes = [vp, i64]
     L.gr_neighbor_build.argtypes = [i64, vp, vp, vp, dbl, i32, C.POINTER(vp)]

@@ -387,6 +387,14 @@ int gr_engine_stage_get(gr_engine *e, int k, char *name, int name_len, double *m
   });
 }
 
+int gr_engine_stage_flops(gr_engine *e, int k, double *flops)
+{
+  return guarded([&] {
+    if (!e || k < 0 || k >= (int) e->times.size()) throw grhip::InvalidArgument("no such stage");
+    if (flops) *flops = e->times[k].flops;
+  });
+}
+
 int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz)
 {
   return guarded([&] {

@@ -49,6 +49,7 @@ struct StageTime {
   std::string name;
   double ms = 0.0;       // summed over the launches of the stage in the last run
   int launches = 0;
+  double flops = 0.0;    // floating-point operations of the stage's tile GEMMs in the last run (2 per multiply-add; 0: not counted)
 };
 
 struct RunFlags {

@@ -186,6 +186,7 @@ template<class T> void pack_fragments(const std::vector<double> &W, int K, int N
 template<class T> struct DevJobs {
   DevBuf job_out, job_scale, seg_off, seg_src, seg_fn, seg_w, seg_scale;
   GemmJobs<T> d{};
+  long long nseg[2] = {0, 0};    // segments that read source 0 / source 1
   struct Host {
     std::vector<int> job_out, seg_off{0}, seg_src, seg_fn, seg_w;
     std::vector<T> job_scale, seg_scale;
@@ -201,6 +202,8 @@ template<class T> struct DevJobs {
     d.seg_src = seg_src.as<int>(); d.seg_fn = seg_fn.as<int>(); d.seg_w = seg_w.as<int>(); d.seg_scale = seg_scale.as<T>();
     d.WF0 = WF0; d.WF1 = WF1;
     d.njobs = (int) h.job_out.size();
+    nseg[0] = nseg[1] = 0;
+    for (int src : h.seg_src) nseg[src ? 1 : 0]++;
     d.max_seg = 0;
     for (size_t q = 0; q + 1 < h.seg_off.size(); q++) d.max_seg = std::max(d.max_seg, h.seg_off[q + 1] - h.seg_off[q]);
   }
@@ -556,6 +559,7 @@ class EngineBase : public Engine, protected BufRegistry {
       }
       it->ms += ms;
       it->launches++;
+      it->flops += ev_flops_[q];
     }
     return times_;
   }
@@ -893,7 +897,9 @@ class EngineBase : public Engine, protected BufRegistry {
       check(hipEventCreate(&b), "hipEventCreate");
       events_.push_back({a, b});
       ev_names_.push_back("");
+      ev_flops_.push_back(0.0);
     }
+    cur_flops_ = 0.0;
     ev_names_[ev_used_] = name;
     check(hipEventRecord(events_[ev_used_].first, stream_), "hipEventRecord");
   }
@@ -901,6 +907,7 @@ class EngineBase : public Engine, protected BufRegistry {
   {
     if (!profile_) return;
     check(hipEventRecord(events_[ev_used_].second, stream_), "hipEventRecord");
+    ev_flops_[ev_used_] = cur_flops_;
     ev_used_++;
   }
   template<class F> void stage(const char *name, F &&f)
@@ -995,6 +1002,8 @@ class EngineBase : public Engine, protected BufRegistry {
                    const int *tiles, int ntiles)
   {
     if (J.d.njobs == 0 || ntiles == 0) return;
+    // multiply-adds of the launch: every segment is a [16 atoms x K] . [K x N] product per atom tile
+    cur_flops_ += 2.0 * 16.0 * ntiles * (double) (nb * 16) * ((double) J.nseg[0] * kb0 * 16 + (double) J.nseg[1] * kb1 * 16);
     const int ksm = std::max(kb0, kb1) * 4;
     // weight tiles staged at a time: as many as fit kGemmLdsBudget, so that the wide tiles of 64-channel models (32 kB
     // in fp64) leave room for several blocks per CU
@@ -1064,6 +1073,8 @@ class EngineBase : public Engine, protected BufRegistry {
   bool profile_ = false;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> events_;
   std::vector<std::string> ev_names_;
+  std::vector<double> ev_flops_;
+  double cur_flops_ = 0.0;
   size_t ev_used_ = 0;
   std::vector<StageTime> times_;
   int drow_[16];

@@ -342,6 +342,45 @@ class Engine:
             out[buf.value.decode()] = (ms.value, cnt.value)
         return out
 
+    def stage_flops(self):
+        """{stage: flops of its tile GEMMs in the last run} (stages without tile GEMMs are left out)"""
+        L = _lib.lib()
+        out = {}
+        buf = C.create_string_buffer(64)
+        for k in range(max(L.gr_engine_stage_count(self._h), 0)):
+            ms, cnt, fl = C.c_double(0.0), C.c_int(0), C.c_double(0.0)
+            check(L.gr_engine_stage_get(self._h, k, buf, 64, C.byref(ms), C.byref(cnt)))
+            check(L.gr_engine_stage_flops(self._h, k, C.byref(fl)))
+            if fl.value > 0:
+                out[buf.value.decode()] = fl.value
+        return out
+
+    def upload_batch(self, structures, cutoff=None):
+        """Several independent periodic structures [(positions, cell, types), ...] as ONE resident list (host neighbour
+        lists, gr_engine_upload_batch): run() then evaluates all of them in one pass, fetch_batch() returns energy [S],
+        virial [S, 6], forces [N, 3] in the order of the uploaded lists (perm of every structure is returned)."""
+        rc = float(self.cutoff_matrix().max()) if cutoff is None else float(cutoff)
+        tt, off, jj, xx, im, sh, sid, perms = [], [np.zeros(1, np.int64)], [], [], [], [], [], []
+        a0 = b0 = s0 = 0
+        for k, (pos, cell, types) in enumerate(structures):
+            perm, offset, j, image, shifts = neighbor_search(pos, cell, [True, True, True], rc)
+            tt.append(np.asarray(types, np.int32)[perm]); xx.append(np.asarray(pos)[perm]); perms.append(perm)
+            off.append(offset[1:] + b0); jj.append(j + a0); im.append(image + s0); sh.append(shifts.reshape(-1, 3))
+            sid.append(np.full(len(perm), k, np.int32))
+            a0 += len(perm); b0 += len(j); s0 += len(shifts)
+        types, offset, j = np.concatenate(tt), np.concatenate(off), np.concatenate(jj).astype(np.int32)
+        n, arrs, nimg = self._csr_args(types, offset, j, None, np.concatenate(xx), np.concatenate(im).astype(np.int32), np.concatenate(sh))
+        sid = np.concatenate(sid)
+        check(_lib.lib().gr_engine_upload_batch(self._h, n, *[ptr(a) for a in arrs], nimg, len(structures), ptr(sid)))
+        self._n, self._nstruct = n, len(structures)
+        return perms
+
+    def fetch_batch(self):
+        n, S = self._n, self._nstruct
+        e, f, v = np.zeros(S), np.zeros((n, 3)), np.zeros((S, 6))
+        check(_lib.lib().gr_engine_fetch_batch(self._h, S, ptr(e), ptr(f), ptr(v), None))
+        return {"energy": e, "forces": f, "virial": v}
+
     def debug_radial(self, x, mu_j):
         x = as_array(x, np.float64)
         mu_j = as_array(mu_j, np.int32)

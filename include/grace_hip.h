@@ -114,6 +114,10 @@ int64_t gr_engine_edge_count(gr_engine *e);
 int gr_engine_set_profile(gr_engine *e, int on);
 int gr_engine_stage_count(gr_engine *e);
 int gr_engine_stage_get(gr_engine *e, int k, char *name, int name_len, double *ms, int *launches);
+/* floating-point operations (2 per multiply-add) of the tile GEMMs stage k launched in that run: the channel-mixing
+ * GEMMs of the FC layers and equivariant reduces over the functions the engine keeps live (the reference prunes the same
+ * functions, libgrace/src/fused_1l.cpp:176-216); 0 for stages that are not tile GEMMs */
+int gr_engine_stage_flops(gr_engine *e, int k, double *flops);
 
 /* Radial functions of the GPU kernel: Rz, dRz [m][lmax+1][n_radial] = R_nl(x) z[mu_j][n] and d/dx, for x = r / rc.
  * Test hook for the radial-MLP kernel (the reference's counterpart is radial_x.h:29-60 evaluated on the host). */

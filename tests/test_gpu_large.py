@@ -1,0 +1,143 @@
+"""The benchmark configurations at FULL size on the GPU, through the C ABI, against goldens of the compiled reference
+(tests/golden/reference_large.npz, written by tests/golden/make_golden_large.py) and against the fp64 oracle.
+
+The compiled reference computes in fp32 with spline tables, so the fp64 engine is compared with it at the reference's own
+fp32-vs-fp64 gate (python/tests/test_ref_tf.py:43-55: 1e-6 eV/atom, forces 2e-5 eV/A here scaled by the largest force,
+per-atom energies 1e-5 eV); the 1e-10 comparisons are against oracle/grace_oracle_2l.py, live and as committed outputs.
+Neighbour lists are compared bit for bit through SHA-256 digests of the reference's arrays."""
+import hashlib
+import os
+
+import numpy as np
+import pytest
+
+import cases
+from grace_runtime_amd import kk, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def large():
+    with np.load(os.path.join(cases.GOLDEN, "reference_large.npz")) as z:
+        return {k: z[k] for k in z.files}
+
+
+@pytest.fixture(scope="module")
+def bench_models(tmp_path_factory):
+    d = str(tmp_path_factory.mktemp("bench_models"))
+    return lambda name: workloads.write_model(name, d)
+
+
+def sha(a):
+    return np.frombuffer(hashlib.sha256(np.ascontiguousarray(a).tobytes()).digest(), dtype=np.uint8)
+
+
+def large_case(name, bench_models):
+    if name == "config2":
+        pos, cell, pbc, types = workloads.structure_config2()
+        return bench_models("config1"), ["W"], pos, cell, pbc, types
+    if name == "config3":
+        pos, cell, pbc, types = workloads.structure_config3()
+        return bench_models("config3"), ["Al", "Co", "Ni", "Ti"], pos, cell, pbc, types
+    pos, cell, pbc, t89 = workloads.structure_config4()
+    path = bench_models("config4")
+    return path, workloads.config4_species(kk.Model(path).element_names), pos, cell, pbc, workloads.config4_types(t89)
+
+
+@pytest.mark.parametrize("name", ["config2", "config3", "config4"])
+def test_full_size_configuration_equals_the_compiled_reference(name, large, bench_models):
+    path, species, pos, cell, pbc, types = large_case(name, bench_models)
+    n = len(pos)
+    sysm = kk.System(kk.Model(path), species, skin=0.0, precision=64)
+    out = sysm.compute(types, pos, cell, pbc, energies=True)
+    # the device list is the reference's list, bond for bond and in its order
+    perm, offset, j, image, shifts = sysm.neighbor_list()
+    assert sysm.list_on_device
+    assert len(j) == int(large[f"{name}/nbonds"])
+    for key, arr in (("perm", perm), ("offset", offset), ("j", j), ("image", image)):
+        assert np.array_equal(sha(arr), large[f"{name}/nl_sha256_{key}"]), key
+    assert np.abs(shifts - large[f"{name}/nl_shifts"]).max() < 1e-12
+    # energy, virial, sampled forces and per-atom energies at the reference's fp32 gate
+    idx = large[f"{name}/atoms"]
+    fmax = float(large[f"{name}/max_abs_force"])
+    vol = abs(np.linalg.det(cell))
+    assert abs(out["energy"] - float(large[f"{name}/energy"])) / n < 1e-6
+    assert np.abs(out["forces"][idx] - large[f"{name}/forces"]).max() < 2e-5 * max(1.0, fmax)
+    assert np.abs(out["energies"][idx] - large[f"{name}/energies"]).max() < 1e-5 * max(1.0, np.abs(large[f"{name}/energies"]).max())
+    assert np.abs(out["virial"] - large[f"{name}/virial"]).max() / vol < 1e-6          # eV/A^3 (stress)
+    # what holds at any size
+    assert abs(out["energies"].sum() - out["energy"]) < 1e-9 * max(1.0, abs(out["energy"]))
+    assert np.abs(out["forces"].sum(axis=0)).max() < 1e-8 * max(1.0, fmax) * np.sqrt(n)
+    del sysm
+
+
+def config5_batch():
+    structs = workloads.structures_config5()
+    return structs, workloads.batch_arrays(structs)
+
+
+def check_config5(out, large, natoms, cells):
+    start = np.concatenate([[0], np.cumsum(natoms)])
+    vol = np.abs(np.linalg.det(cells))
+    assert np.abs((out["energy"] - large["config5/energy"]) / natoms).max() < 1e-6
+    for k in large["config5/forces_cells"]:
+        ref = large[f"config5/forces_{k}"]
+        assert np.abs(out["forces"][start[k]:start[k + 1]] - ref).max() < 2e-5 * max(1.0, np.abs(ref).max()), k
+    assert (np.abs(out["virial"] - large["config5/virial"]).max(axis=1) / vol).max() < 1e-6      # eV/A^3 (stress)
+    # the fp64 oracle on the cells it was run on (committed outputs)
+    for k in large["config5/oracle_cells"]:
+        fs = max(1.0, np.abs(large[f"config5/oracle_forces_{k}"]).max())
+        assert abs(out["energy"][k] - float(large[f"config5/oracle_energy_{k}"])) / natoms[k] < 1e-10 * fs, k
+        assert np.abs(out["forces"][start[k]:start[k + 1]] - large[f"config5/oracle_forces_{k}"]).max() < 1e-9 * fs, k
+        assert np.abs(out["virial"][k] - large[f"config5/oracle_virial_{k}"]).max() < 1e-8 * fs, k
+
+
+def test_config5_batch_equals_the_compiled_reference_and_the_oracle(large, bench_models):
+    """all 512 cells in one Batch.compute call (host lists), against the reference cell by cell"""
+    structs, (natoms, types, pos, cells, pbc) = config5_batch()
+    assert np.array_equal(natoms, large["config5/natoms"])
+    b = kk.Batch(kk.Model(bench_models("config5")), ["Al", "Ni", "Ti"], precision=64)
+    out = b.compute(natoms, types, pos, cells, pbc)
+    assert b.passes == 1
+    check_config5(out, large, natoms, cells)
+
+
+def test_config5_device_batch_equals_the_compiled_reference_and_the_oracle(large, bench_models):
+    """the same batch with atoms and results in device memory and the lists built on the device"""
+    import torch
+    structs, (natoms, types, pos, cells, pbc) = config5_batch()
+    dev = torch.device("cuda", 0)
+    S, N = len(natoms), len(types)
+    b = kk.Batch(kk.Model(bench_models("config5")), ["Al", "Ni", "Ti"], precision=64)
+    e = torch.zeros(S, dtype=torch.float64, device=dev)
+    f = torch.zeros((N, 3), dtype=torch.float64, device=dev)
+    v = torch.zeros((S, 6), dtype=torch.float64, device=dev)
+    b.compute_device(natoms, torch.tensor(types, device=dev), torch.tensor(pos, device=dev), cells, pbc, e, forces=f, virial=v)
+    out = {"energy": e.cpu().numpy(), "forces": f.cpu().numpy(), "virial": v.cpu().numpy()}
+    check_config5(out, large, natoms, cells)
+
+
+def test_config5_cells_equal_the_live_oracle(bench_models):
+    """two cells of the batch against oracle/grace_oracle_2l.py evaluated here (1e-10 eV/atom, 1e-9 eV/A)"""
+    from oracle import grace_oracle_2l as g2
+    structs = workloads.structures_config5()
+    sizes = np.array([len(s[0]) for s in structs])
+    pick = [int(k) for k in np.argsort(sizes, kind="stable")[4:6]]     # not the cells of the committed oracle outputs
+    path = bench_models("config5")
+    om = g2.Model2L(path)
+    natoms, types, pos, cells, pbc = workloads.batch_arrays([structs[k] for k in pick])
+    b = kk.Batch(kk.Model(path), ["Al", "Ni", "Ti"], precision=64)
+    out = b.compute(natoms, types, pos, cells, pbc)
+    a0 = 0
+    for q, k in enumerate(pick):
+        p, c, t = structs[k]
+        perm, offset, j, image, shifts = kk.neighbor_search(p, c, [True, True, True], 6.0)
+        ref = g2.compute_2l(om, t[perm] - 1, offset, j, cases.bond_vectors(p, perm, offset, j, image, shifts))
+        fref = np.zeros_like(p)
+        fref[perm] = ref["forces"]
+        fs = max(1.0, np.abs(fref).max())
+        assert abs(out["energy"][q] - ref["energy"]) / len(p) < 1e-10 * fs
+        assert np.abs(out["forces"][a0:a0 + len(p)] - fref).max() < 1e-9 * fs
+        assert np.abs(out["virial"][q] - ref["virial"]).max() < 1e-8 * fs
+        a0 += len(p)
