@@ -1,9 +1,10 @@
-// Host-side containers of GRACE models read from kokkos.npz, with the validation of the reference loaders:
-// GRACE-1L keys and checks follow libgrace/src/model_1l.cpp:18-273 (container libgrace/include/grace/model_1l.h),
-// the kind of a file libgrace/include/grace/model_kind.h:13-19.
+// Host-side containers of GRACE models read from kokkos.npz and the GRACE-1L loader.  The keys, their meaning and the
+// consistency rules are the file format's, as the reference loader reads it (libgrace/src/model_1l.cpp:18-273, container
+// libgrace/include/grace/model_1l.h; kind of a file: libgrace/include/grace/model_kind.h:13-19).  Every array is
+// requested through FileReader (schema.hpp) with the shape it must have, so it is checked at the moment it is read.
 #pragma once
 
-#include "npz.hpp"
+#include "schema.hpp"
 
 #include <algorithm>
 #include <string>
@@ -13,21 +14,37 @@ namespace grhip {
 
 enum class ModelKind { Grace1L = 1, Grace2L = 2, Grace3L = 3 };
 
-// grace_model_kind names the kind; files without it are told apart by their members
+// The kind a file declares, or, for files older than the declaration, the kind its members give away.
 inline ModelKind model_kind(const Npz &z, const std::string &path)
 {
-  NpzView v(z);
-  if (v.has("grace_model_kind")) {
-    const auto k = v.names("grace_model_kind");
-    if (k.size() == 1 && k[0] == "GRACE-1L") return ModelKind::Grace1L;
-    if (k.size() == 1 && k[0] == "GRACE-2L") return ModelKind::Grace2L;
-    if (k.size() == 1 && k[0] == "GRACE-3L") return ModelKind::Grace3L;
-    throw Error("model file " + path + ": unknown grace_model_kind");
+  FileReader f(z, "GRACE");
+  static const struct { const char *label; const char *telltale; ModelKind kind; } kinds[] = {
+      {"GRACE-3L", "prod_names", ModelKind::Grace3L},
+      {"GRACE-2L", "B0_lin_transform_W", ModelKind::Grace2L},
+      {"GRACE-1L", "mlp_rad_W0", ModelKind::Grace1L},
+  };
+  if (f.present("grace_model_kind")) {
+    const auto declared = f.labels("grace_model_kind");
+    for (const auto &k : kinds)
+      if (declared.size() == 1 && declared[0] == k.label) return k.kind;
+    throw Error(path + ": grace_model_kind names no model family this library knows (GRACE-1L, GRACE-2L, GRACE-3L)");
   }
-  if (v.has("prod_names")) return ModelKind::Grace3L;
-  if (v.has("B0_lin_transform_W")) return ModelKind::Grace2L;
-  if (v.has("mlp_rad_W0")) return ModelKind::Grace1L;
-  throw Error("model file " + path + " is not a GRACE kokkos.npz");
+  for (const auto &k : kinds)
+    if (f.present(k.telltale)) return k.kind;
+  throw Error(path + " holds none of the arrays of a GRACE kokkos.npz export");
+}
+
+// What every loader checks first: the declared kind is the loader's, and the format revision is one it reads.
+inline void check_declaration(const FileReader &f, const char *label)
+{
+  const long revision = f.whole_or("grace_format_version", 0, kSizeLimit, 0);
+  if (f.present("grace_model_kind")) {
+    const auto declared = f.labels("grace_model_kind");
+    if (declared.size() != 1) f.reject("grace_model_kind", "must hold exactly one name");
+    if (declared[0] != label) throw Error(std::string(label) + " loader: the file declares a " + declared[0] + " model");
+    if (revision < 1) f.reject("grace_format_version", "must be at least 1 in a file that declares its kind");
+  }
+  if (revision > 2) f.reject("grace_format_version", "= " + std::to_string(revision) + " is newer than the revisions (up to 2) this library reads");
 }
 
 struct MLPLayer {
@@ -57,25 +74,70 @@ struct ReduceWeights {
   std::vector<int> collect_ind, w_l_tile;
 };
 
-inline std::vector<MLPLayer> load_mlp(const NpzView &v, const std::string &pfx, int n, int64_t n_in, int64_t n_out,
-                                      const std::string &in_why, const std::string &out_why)
+// A stack of dense layers `<stem>_W0, <stem>_W1, ...` with scalar norms: `depth` matrices chained from `first_in` inputs
+// to `last_out` outputs; the widths in between are whatever the file holds.
+inline std::vector<MLPLayer> read_dense_stack(const FileReader &f, const std::string &stem, long depth, long first_in, long last_out)
 {
-  std::vector<MLPLayer> layers;
-  int64_t prev = n_in;
-  for (int i = 0; i < n; i++) {
-    const std::string wk = pfx + "_W" + std::to_string(i);
-    MLPLayer L;
-    L.W = v.require_doubles(wk);
-    const auto sh = v.shape_rank(wk, 2);
-    require_eq(wk, (int64_t) sh[0], prev, i == 0 ? in_why : "the outputs of the layer before", "rows");
-    if (i == n - 1) require_eq(wk, (int64_t) sh[1], n_out, out_why, "columns");
-    L.n_in = (int) sh[0];
-    L.n_out = (int) sh[1];
-    L.norm = v.double_scalar(pfx + "_norm" + std::to_string(i), 1.0);
-    prev = L.n_out;
-    layers.push_back(std::move(L));
+  std::vector<MLPLayer> stack((size_t) depth);
+  long width = first_in;
+  for (long k = 0; k < depth; k++) {
+    const std::string tag = std::to_string(k);
+    MLPLayer &layer = stack[(size_t) k];
+    long out = last_out;
+    layer.W = k + 1 == depth ? f.reals(stem + "_W" + tag, {width, out}) : f.reals(stem + "_W" + tag, {width, Ext::any(out)});
+    layer.n_in = (int) width;
+    layer.n_out = (int) out;
+    layer.norm = f.real_or(stem + "_norm" + tag, 1.0);
+    width = out;
   }
-  return layers;
+  return stack;
+}
+
+// Channel-mixing layer `<name>_*`: per output function a left weight tile applied to the same function of the left input and
+// right tiles applied to collected functions of the right input.
+struct FcExtents {
+  long functions;          // functions of the left input = of the output
+  long right_functions;    // functions of the right input
+  long left_width, right_width, out_width;
+};
+inline FCWeights read_fc(const FileReader &f, const std::string &name, const FcExtents &x)
+{
+  FCWeights fc;
+  long tiles = 0, links = 0;
+  f.must_be(name + "_n_out", x.out_width, x.out_width, "all FC layers of a chain have the width of its first one");
+  f.must_be(name + "_left_coefs", 1, 1, "the engines of this model family apply a left weight in every FC layer");
+  fc.w_left = f.reals(name + "_w_left", {x.out_width, x.left_width, Ext::any(tiles)});
+  fc.w_right = f.reals(name + "_w_right", {x.out_width, x.right_width, tiles});
+  fc.w_tile_left = f.indices(name + "_w_tile_left", {x.functions}, tiles);
+  fc.norm_out_factor = f.reals(name + "_norm_out_factor", Flat{x.functions});
+  fc.collect_from = f.indices(name + "_collect_from", {Ext::any(links)}, x.right_functions);
+  fc.collect_to = f.indices(name + "_collect_to", {links}, x.functions);
+  fc.w_tile_right = f.indices(name + "_w_tile_right", {links}, tiles);
+  fc.norm_left = f.real_or(name + "_norm_left", 1.0);
+  fc.norm_right = f.real_or(name + "_norm_right", 1.0);
+  fc.n_out = (int) x.out_width;
+  fc.n_in_left = (int) x.left_width;
+  fc.n_in_right = (int) x.right_width;
+  fc.n_funcs = (int) x.functions;
+  fc.n_conn = (int) links;
+  fc.tiles_left = fc.tiles_right = (int) tiles;
+  return fc;
+}
+
+// Channel-wise Clebsch-Gordan product `<name>_*`: a list of (left function, right function, output function, coefficient).
+inline CGProduct read_product(const FileReader &f, const std::string &name, long left_functions, long right_functions)
+{
+  CGProduct p;
+  const long terms = f.whole(name + "_n_cg_terms", 1, kSizeLimit), outputs = f.whole(name + "_n_output_funcs", 1, kSizeLimit);
+  p.cg_coeff = f.reals(name + "_cg_coeff", {terms});
+  p.left_ind = f.indices(name + "_left_ind", {terms}, left_functions);
+  p.right_ind = f.indices(name + "_right_ind", {terms}, right_functions);
+  p.m_sum_ind = f.indices(name + "_m_sum_ind", {terms}, outputs);
+  if (addressed(p.m_sum_ind) != outputs)
+    f.reject(name + "_n_output_funcs", "= " + std::to_string(outputs) + " but " + name + "_m_sum_ind addresses " + std::to_string(addressed(p.m_sum_ind)) + " functions");
+  p.n_terms = (int) terms;
+  p.n_out = (int) outputs;
+  return p;
 }
 
 // The uqv6 UQ head of a model file (libgrace/include/grace/uq_head.h, loader libgrace/src/uq_head.cpp:11-76): the GMM
@@ -93,55 +155,61 @@ struct UqHead {
   std::vector<double> rp_matrix;            // [d_basis][rp_dim]
   std::string error;                        // what is wrong with the head (reported by validate_uq; the model stays usable)
 
-  // who: "GRACE-1L/KK"; checks and messages of uq_head.cpp:11-76
-  void load(const NpzView &v, int model_elements, const std::string &who)
+  // A head that cannot be used leaves `error` set instead of failing the load: energies and forces do not need it.
+  void load(const FileReader &f, int model_elements)
   {
     *this = UqHead();
-    schema = v.int_scalar("uq_schema_version", 0);
+    schema = (int) f.whole_or("uq_schema_version", 0, kSizeLimit, 0);
     has_uq = schema != 0;
-    if (schema != 6) return;
-    const std::string pre = who + " UQ: ";
+    if (schema != 6) return;    // another schema: validate_uq() says so
     try {
-      n_elements = v.int_scalar("uq_n_elements", model_elements);
-      require_eq("uq_n_elements", n_elements, model_elements, "n_elements");
-      max_clusters = v.int_in("uq_max_clusters", 0, 1, kMaxDim);
-      rp_dim = v.int_in("uq_rp_dim", 0, 1, kMaxDim);
-      feature_dim = v.int_in("uq_feature_dim", 0, rp_dim, kMaxDim);
-      normalize = v.int_scalar("uq_rp_normalize", 0);
-      const int add_density = v.int_scalar("uq_rp_add_density_channel", 0);
-      density_scale = v.double_scalar("uq_rp_density_scale", 1.0);
-      const int transform = v.int_scalar("uq_feature_transform", 0);
-      centroids = v.require_doubles("uq_centroids");
-      inv_cov = v.require_doubles("uq_inv_cov");
-      n_clusters = v.require_ints("uq_n_clusters");
-      interp_thresholds = v.require_doubles("uq_interp_thresholds");
-      rp_matrix = v.require_doubles("uq_rp_matrix");
-      if (normalize != 1 || add_density != 1 || transform != 0)
-        throw Error("schema v6 expects normalize=1, add_density_channel=1, feature_transform=0 (identity); got normalize=" +
-                    std::to_string(normalize) + ", add_density=" + std::to_string(add_density) + ", transform=" + std::to_string(transform) +
-                    ". Artifact mislabeled or unsupported variant.");
+      f.must_be("uq_n_elements", model_elements, model_elements, "the head must cover the elements of the model");
+      n_elements = model_elements;
+      max_clusters = (int) f.whole("uq_max_clusters", 1, kSizeLimit);
+      rp_dim = (int) f.whole("uq_rp_dim", 1, kSizeLimit);
+      feature_dim = (int) f.whole("uq_feature_dim", rp_dim, kSizeLimit);
       n_density = feature_dim - rp_dim;
-      const auto rs = v.shape_rank("uq_rp_matrix", 2);
-      require_eq("uq_rp_matrix", (int64_t) rs[1], rp_dim, "uq_rp_dim", "columns");
-      d_basis = (int) rs[0];
-      const size_t E = (size_t) n_elements, K = (size_t) max_clusters, D = (size_t) feature_dim;
-      require_size("uq_centroids", centroids, E * K * D);
-      require_size("uq_inv_cov", inv_cov, E * K * D * D);
-      require_size("uq_n_clusters", n_clusters, E);
-      require_size("uq_interp_thresholds", interp_thresholds, E * K);
-      for (size_t e = 0; e < n_clusters.size(); e++) {
-        if (n_clusters[e] <= 0)
-          throw Error("element index " + std::to_string(e) + " has no GMM clusters; uqv6 artifacts must cover all elements. Re-export the "
-                      "UQ artifacts with a current grace_utils.");
-        if (n_clusters[e] > max_clusters)
-          throw Error("element index " + std::to_string(e) + " has " + std::to_string(n_clusters[e]) + " GMM clusters, more than uq_max_clusters = " +
-                      std::to_string(max_clusters));
-      }
+      normalize = (int) f.whole_or("uq_rp_normalize", 0, 1, 0);
+      const bool density = f.flag_or("uq_rp_add_density_channel", false);
+      const long transform = f.whole_or("uq_feature_transform", 0, kSizeLimit, 0);
+      if (!normalize || !density || transform != 0)
+        throw Error("a uqv6 head is defined with a normalised projection, density channels and no feature transform; this file has "
+                    "uq_rp_normalize = " + std::to_string(normalize) + ", uq_rp_add_density_channel = " + std::to_string((int) density) +
+                    ", uq_feature_transform = " + std::to_string(transform));
+      density_scale = f.real_or("uq_rp_density_scale", 1.0);
+      long basis = 0;
+      rp_matrix = f.reals("uq_rp_matrix", {Ext::any(basis), rp_dim});
+      d_basis = (int) basis;
+      const long E = n_elements, K = max_clusters, D = feature_dim;
+      centroids = f.reals("uq_centroids", Flat{E * K * D});
+      inv_cov = f.reals("uq_inv_cov", Flat{E * K * D * D});
+      interp_thresholds = f.reals("uq_interp_thresholds", Flat{E * K});
+      n_clusters = f.indices("uq_n_clusters", {E}, K + 1);
+      for (long e = 0; e < E; e++)
+        if (n_clusters[(size_t) e] == 0) throw Error("uq_n_clusters: element " + std::to_string(e) + " has no GMM cluster; a head must cover every element");
     } catch (const std::exception &e) {
-      error = e.what();
-      if (error.rfind(pre, 0) != 0) error = pre + error;
+      error = f.family() + " UQ head: " + e.what();
     }
   }
+  // Shared part of validate_uq(): is there a head of the schema the kernels implement, loaded without complaint, sized
+  // for this model (`basis` rows of the projection, `blocks` basis blocks -> 1 + blocks density channels)?
+  void require_usable(const std::string &family, bool order4, long basis, int blocks) const
+  {
+    if (!has_uq) throw Error(family + ": the model has no UQ head");
+    if (!order4) throw Error(family + ": a UQ head needs the fourth-order stage; this is a max_order 3 model");
+    if (schema != 6) throw Error(family + ": UQ head of schema " + std::to_string(schema) + "; only schema 6 (uqv6) can be evaluated");
+    if (!error.empty()) throw Error(error);
+    if (basis != d_basis)
+      throw Error(family + " UQ head: uq_rp_matrix projects " + std::to_string(d_basis) + " basis functions, the model has " + std::to_string(basis));
+    if (n_density != 1 + blocks)
+      throw Error(family + " UQ head: " + std::to_string(n_density) + " density channels where " + std::to_string(1 + blocks) + " belong to this model family");
+  }
+};
+
+// Sizes and switches shared by the GRACE-1L and GRACE-2L files: key, accepted range, value of a file without the key.
+struct SizeKey {
+  const char *key;
+  long lo, hi, absent;
 };
 
 struct Model1L {
@@ -170,26 +238,12 @@ struct Model1L {
   // (libgrace/include/grace/uq.h:31-48)
   int uq_basis_width() const
   {
-    int w = red_A.n_in * (int) red_A.collect_ind.size() + red_AA.n_in * (int) red_AA.collect_ind.size() +
-            red_AAA.n_in * (int) red_AAA.collect_ind.size();
-    if (max_order == 4) w += red_AAAA.n_in * (int) red_AAAA.collect_ind.size();
+    int w = 0;
+    for (const ReduceWeights *r : {&red_A, &red_AA, &red_AAA, &red_AAAA}) w += r->n_in * (int) r->collect_ind.size();
     return w;
   }
-  // libgrace/src/model_1l.cpp:275-285, libgrace/src/uq.cpp:8-33
-  void validate_uq() const
-  {
-    if (!uq.has_uq) throw Error("GRACE-1L: the model has no UQ head");
-    if (max_order == 3) throw Error("GRACE-1L: UQ is not supported for max_order 3 models");
-    if (uq.schema != 6)
-      throw Error("GRACE-1L: UQ schema v" + std::to_string(uq.schema) + " unsupported (expects v6, uqv6 basis-RP normalize+density). Re-export the "
-                  "UQ artifacts at schema v6 with a current grace_utils.");
-    if (!uq.error.empty()) throw Error(uq.error);
-    if (uq_basis_width() != uq.d_basis)
-      throw Error("GRACE-1L UQ: uq_rp_matrix has " + std::to_string(uq.d_basis) + " rows, the model's invariant basis has " +
-                  std::to_string(uq_basis_width()) + "; re-export the UQ artifacts for this model");
-    if (uq.n_density != 2)
-      throw Error("GRACE-1L UQ: " + std::to_string(uq.n_density) + " density channels, expected 2 (1 + basis blocks)");
-  }
+  // can the head be evaluated (libgrace/src/model_1l.cpp:275-285, libgrace/src/uq.cpp:8-33)
+  void validate_uq() const { uq.require_usable("GRACE-1L", max_order == 4, uq_basis_width(), 1); }
   double pair_cutoff(int mu_i, int mu_j) const    // libgrace/include/grace/type_map.h:23-28
   {
     if (mu_i < 0 || mu_j < 0) return 0.0;
@@ -199,175 +253,112 @@ struct Model1L {
   void load(const Npz &z)
   {
     *this = Model1L();
-    NpzView v(z);
-    if (v.has("grace_model_kind")) {
-      const auto k = v.names("grace_model_kind");
-      if (k.size() != 1) throw bad_array("grace_model_kind", "must hold one name");
-      if (k[0] != "GRACE-1L") throw Error("GRACE-1L: the file holds a " + k[0] + " model");
-      if (v.int_scalar("grace_format_version", 0) < 1) throw bad_array("grace_format_version", "is missing or below 1 next to grace_model_kind");
-    }
-    if (v.int_scalar("grace_format_version", 0) > 2)
-      throw Error("GRACE-1L: kokkos.npz format " + std::to_string(v.int_scalar("grace_format_version", 0)) + ", this build reads up to 2");
-    // max_order 3: no AAAA stage; some but not all of its arrays is a broken file (libgrace/src/max_order3.h:104-134)
-    const bool order4 = v.has("prod_AAAA_n_cg_terms");
-    if (!order4)
-      for (const auto &kv : z)
-        if (kv.first.find("AAAA") != std::string::npos || kv.first.rfind("fc_AA2_", 0) == 0)
-          throw bad_array(kv.first, "is present, but prod_AAAA_n_cg_terms is not: the AAAA stage is incomplete");
-    max_order = order4 ? 4 : 3;
+    const FileReader f(z, "GRACE-1L");
+    check_declaration(f, "GRACE-1L");
 
-    n_elements = v.int_in("n_elements", 89, 1, kMaxDim);
-    embedding_size = v.int_in("embedding_size", 128, 1, kMaxDim);
-    lmax = v.int_in("lmax", 4, 0, kMaxL);
-    nradbase = v.int_in("nradbase", 10, 1, kMaxDim);
-    nradmax = v.int_in("nradmax", 32, 1, kMaxDim);
-    radial_basis_p = v.int_in("radial_basis_p", 16, 1, kMaxP);
-    rcut = v.cutoff_scalar("rcut", 6.0, "GRACE-1L/KK");
-    has_bond_specific_cutoff = v.flag("has_bond_specific_cutoff", 0);
-    require_eq("mlp_rad_has_chem_emb", v.int_scalar("mlp_rad_has_chem_emb", 0), 0, "chem-embedded radial MLPs are not supported");
-    const int64_t nlm_ = (int64_t) (lmax + 1) * (lmax + 1);
+    // ---- sizes
+    int *const into[] = {&n_elements, &embedding_size, &lmax, &nradbase, &nradmax, &radial_basis_p};
+    static const SizeKey sizes[] = {{"n_elements", 1, kSizeLimit, 89}, {"embedding_size", 1, kSizeLimit, 128}, {"lmax", 0, kDegreeLimit, 4},
+                                    {"nradbase", 1, kSizeLimit, 10},   {"nradmax", 1, kSizeLimit, 32},         {"radial_basis_p", 1, kEnvelopeLimit, 16}};
+    for (size_t k = 0; k < sizeof(sizes) / sizeof(sizes[0]); k++) *into[k] = (int) f.whole_or(sizes[k].key, sizes[k].lo, sizes[k].hi, sizes[k].absent);
+    const long harmonics = nlm(), channels = nradmax;
 
-    element_names = v.names("element_names");
-    chem_embedding = v.require_doubles("chem_embedding");
-    {
-      const auto ce = v.shape_rank("chem_embedding", 2);
-      if ((long) ce[0] != n_elements && (element_names.empty() || element_names.size() == ce[0]))
-        throw bad_array("n_elements", "is " + std::to_string(n_elements) + ", but chem_embedding has " + std::to_string(ce[0]) + " rows");
-      if (!element_names.empty()) require_size("element_names", element_names, n_elements);
-      v.require_shape("chem_embedding", {n_elements, embedding_size});
-    }
-    bond_cutoff_map = v.cutoffs("bond_cutoff_map", "GRACE-1L/KK");
-    v.require_shape("bond_cutoff_map", {n_elements, n_elements});
+    // ---- which stages the file has: a file without the fourth-order product must not carry pieces of that stage
+    const bool fourth = f.present("prod_AAAA_n_cg_terms");
+    max_order = fourth ? 4 : 3;
+    if (!fourth)
+      for (const auto &member : z)
+        if (member.first.find("AAAA") != std::string::npos || member.first.compare(0, 7, "fc_AA2_") == 0)
+          f.reject(member.first, "belongs to the AAAA stage, which this file otherwise lacks (no prod_AAAA_n_cg_terms): the stage is incomplete");
+
+    // ---- elements, cutoffs, species weights
+    element_names = f.labels("element_names");
+    if (!element_names.empty() && (long) element_names.size() != n_elements)
+      f.reject("element_names", "lists " + std::to_string(element_names.size()) + " elements where n_elements = " + std::to_string(n_elements));
+    chem_embedding = f.reals("chem_embedding", {n_elements, embedding_size});
+    rcut = f.length_or("rcut", 6.0);
+    has_bond_specific_cutoff = f.flag_or("has_bond_specific_cutoff", false);
+    bond_cutoff_map = f.distances_or_none("bond_cutoff_map", n_elements, n_elements);
     if (bond_cutoff_map.empty()) bond_cutoff_map.assign((size_t) n_elements * n_elements, rcut);
+    A_lin_transform_W = f.reals("A_lin_transform_W", {embedding_size, channels});
+    A_lin_transform_norm = f.real_or("A_lin_transform_norm", 1.0);
+    A_inv_avg_n_neigh = f.real_or("A_inv_avg_n_neigh", 1.0);
 
-    A_lin_transform_W = v.require_doubles("A_lin_transform_W");
-    v.require_shape("A_lin_transform_W", {embedding_size, nradmax});
-    A_lin_transform_norm = v.double_scalar("A_lin_transform_norm", 1.0);
-    A_inv_avg_n_neigh = v.double_scalar("A_inv_avg_n_neigh", 1.0);
+    // ---- radial network
+    f.must_be("mlp_rad_has_chem_emb", 0, 0, "radial networks with species inputs belong to GRACE-3L");
+    mlp_rad = read_dense_stack(f, "mlp_rad", f.whole_or("mlp_rad_n_layers", 1, kSizeLimit, 3), nradbase, channels * nl());
+    radial_activation = (int) f.whole_or("radial_activation", 0, 1, 0);
 
-    mlp_rad = load_mlp(v, "mlp_rad", v.int_in("mlp_rad_n_layers", 3, 1, kMaxDim), nradbase, (int64_t) nradmax * (lmax + 1),
-                       "nradbase", "nradmax x (lmax + 1)");
+    // ---- the chain A -> A1 -> AA -> AA1 / AA2 -> AAA / AAAA; the FC width is that of its first layer
+    const long fcw = f.whole_or("fc_A1_n_out", 1, kSizeLimit, 64);
+    fc_A1 = read_fc(f, "fc_A1", {harmonics, harmonics, channels, channels, fcw});
+    prod_AA = read_product(f, "prod_AA", harmonics, harmonics);
+    const long pairs = prod_AA.n_out;
+    fc_AA1 = read_fc(f, "fc_AA1", {pairs, harmonics, fcw, channels, fcw});
+    prod_AAA = read_product(f, "prod_AAA", pairs, harmonics);
+    if (fourth) {
+      fc_AA2 = read_fc(f, "fc_AA2", {pairs, harmonics, fcw, channels, fcw});
+      prod_AAAA = read_product(f, "prod_AAAA", pairs, pairs);
+    }
+    AAA_right_A = f.flag_or("AAA_right_A", false);
+    if (AAA_right_A && fcw != channels)
+      f.reject("AAA_right_A", "is set (AAA = AA1 x A), which needs the FC width " + std::to_string(fcw) + " to equal nradmax = " + std::to_string(channels));
 
-    auto load_fc = [&](const std::string &p, FCWeights &fc, int64_t n_funcs, int64_t n_in_left) {
-      fc.w_left = v.require_doubles(p + "_w_left");
-      fc.w_right = v.require_doubles(p + "_w_right");
-      fc.w_tile_left = v.require_ints(p + "_w_tile_left");
-      fc.w_tile_right = v.require_ints(p + "_w_tile_right");
-      fc.collect_to = v.require_ints(p + "_collect_to");
-      fc.collect_from = v.require_ints(p + "_collect_from");
-      fc.norm_out_factor = v.require_doubles(p + "_norm_out_factor");
-      fc.norm_left = v.double_scalar(p + "_norm_left", 1.0);
-      fc.norm_right = v.double_scalar(p + "_norm_right", 1.0);
-      fc.n_out = v.int_in(p + "_n_out", 64, 1, kMaxDim);
-      require_eq(p + "_left_coefs", v.int_scalar(p + "_left_coefs", 1), 1, "the GRACE-1L engines apply left weights in every FC");
-      fc.tiles_left = (int) v.shape_rank(p + "_w_left", 3)[2];
-      fc.tiles_right = (int) v.shape_rank(p + "_w_right", 3)[2];
-      require_eq(p + "_w_right", fc.tiles_right, fc.tiles_left, "the tiles of " + p + "_w_left", "tiles");
-      v.require_shape(p + "_w_left", {fc.n_out, n_in_left, fc.tiles_left});
-      v.require_shape(p + "_w_right", {fc.n_out, nradmax, fc.tiles_right});
-      require_size(p + "_w_tile_left", fc.w_tile_left, (size_t) n_funcs);
-      require_size(p + "_norm_out_factor", fc.norm_out_factor, (size_t) n_funcs);
-      require_index(p + "_w_tile_left", fc.w_tile_left, fc.tiles_left);
-      const size_t nc = fc.collect_from.size();
-      require_size(p + "_collect_to", fc.collect_to, nc);
-      require_size(p + "_w_tile_right", fc.w_tile_right, nc);
-      require_index(p + "_collect_from", fc.collect_from, nlm_);
-      require_index(p + "_collect_to", fc.collect_to, n_funcs);
-      require_index(p + "_w_tile_right", fc.w_tile_right, fc.tiles_right);
-      fc.n_in_left = (int) n_in_left;
-      fc.n_in_right = nradmax;
-      fc.n_funcs = (int) n_funcs;
-      fc.n_conn = (int) nc;
-    };
-    auto load_prod = [&](const std::string &p, CGProduct &pr, int64_t n_left, int64_t n_right) {
-      pr.left_ind = v.require_ints(p + "_left_ind");
-      pr.right_ind = v.require_ints(p + "_right_ind");
-      pr.m_sum_ind = v.require_ints(p + "_m_sum_ind");
-      pr.cg_coeff = v.require_doubles(p + "_cg_coeff");
-      pr.n_out = v.int_in(p + "_n_output_funcs", 0, 1, kMaxDim);
-      pr.n_terms = v.int_in(p + "_n_cg_terms", 0, 1, kMaxDim);
-      const size_t nt = (size_t) pr.n_terms;
-      require_size(p + "_left_ind", pr.left_ind, nt);
-      require_size(p + "_right_ind", pr.right_ind, nt);
-      require_size(p + "_m_sum_ind", pr.m_sum_ind, nt);
-      require_size(p + "_cg_coeff", pr.cg_coeff, nt);
-      require_index(p + "_left_ind", pr.left_ind, n_left);
-      require_index(p + "_right_ind", pr.right_ind, n_right);
-      require_index(p + "_m_sum_ind", pr.m_sum_ind, pr.n_out);
-      require_eq(p + "_n_output_funcs", pr.n_out, index_extent(pr.m_sum_ind), "1 + the largest " + p + "_m_sum_ind");
-    };
-
-    // the FC width is needed before the checks: read it first
-    const int CF = v.int_in("fc_A1_n_out", 64, 1, kMaxDim);
-    load_fc("fc_A1", fc_A1, nlm_, nradmax);
-    load_prod("prod_AA", prod_AA, nlm_, nlm_);
-    const int64_t nAA = prod_AA.n_out;
-    load_fc("fc_AA1", fc_AA1, nAA, CF);
-    require_eq("fc_AA1_n_out", fc_AA1.n_out, CF, "fc_A1_n_out");
-    load_prod("prod_AAA", prod_AAA, nAA, nlm_);
-    if (order4) {
-      load_fc("fc_AA2", fc_AA2, nAA, CF);
-      require_eq("fc_AA2_n_out", fc_AA2.n_out, CF, "fc_A1_n_out");
-      load_prod("prod_AAAA", prod_AAAA, nAA, nAA);
+    // ---- density: one element-dependent projection per stage
+    rho_n_out = (int) f.whole_or("rho_n_out", 2, kSizeLimit, 17);
+    f.must_be("rho_is_central_atom_type_dependent", 1, 1, "the density weights of this model family depend on the central element");
+    struct Stage { const char *tag; ReduceWeights *into; long width, functions; bool have; };
+    const Stage stages[] = {{"A", &red_A, channels, harmonics, true}, {"AA", &red_AA, fcw, pairs, true}, {"AAA", &red_AAA, fcw, prod_AAA.n_out, true},
+                            {"AAAA", &red_AAAA, fcw, prod_AAAA.n_out, fourth}};
+    for (const Stage &s : stages) {
+      if (!s.have) continue;
+      const std::string tag = s.tag;
+      ReduceWeights &r = *s.into;
+      long tiles = 0, picked = 0;
+      f.must_be("rho_n_in_" + tag, s.width, s.width, "it is the channel width of " + tag);
+      r.W = f.reals("rho_reduce_" + tag + "_W", {n_elements, rho_n_out, s.width, Ext::any(tiles)});
+      f.must_be("rho_w_shape_" + tag, tiles, tiles, "it counts the weight tiles stored in rho_reduce_" + tag + "_W");
+      r.collect_ind = f.indices("rho_collect_ind_" + tag, {Ext::any(picked)}, s.functions);
+      r.w_l_tile = f.indices("rho_w_l_tile_" + tag, {picked}, tiles);
+      r.norm = f.real_or("rho_reduce_" + tag + "_norm", 1.0);
+      r.n_in = (int) s.width;
+      r.w_shape = (int) tiles;
     }
 
-    rho_n_out = v.int_in("rho_n_out", 17, 2, kMaxDim);
-    require_eq("rho_is_central_atom_type_dependent", v.int_scalar("rho_is_central_atom_type_dependent", 1), 1,
-               "the GRACE-1L engines implement this layout only");
-    auto load_reduce = [&](const std::string &s, ReduceWeights &rw, int64_t n_in, int64_t n_funcs) {
-      const std::string wkey = "rho_reduce_" + s + "_W", ckey = "rho_collect_ind_" + s, tkey = "rho_w_l_tile_" + s;
-      rw.W = v.require_doubles(wkey);
-      rw.norm = v.double_scalar("rho_reduce_" + s + "_norm", 1.0);
-      rw.collect_ind = v.require_ints(ckey);
-      rw.w_l_tile = v.require_ints(tkey);
-      rw.n_in = v.int_scalar("rho_n_in_" + s, 0);
-      rw.w_shape = v.int_in("rho_w_shape_" + s, 0, 1, kMaxDim);
-      require_eq("rho_n_in_" + s, rw.n_in, n_in, "the channels of " + s);
-      v.require_shape(wkey, {n_elements, rho_n_out, rw.n_in, rw.w_shape});
-      require_size(tkey, rw.w_l_tile, rw.collect_ind.size());
-      require_index(ckey, rw.collect_ind, n_funcs);
-      require_index(tkey, rw.w_l_tile, rw.w_shape);
-    };
-    load_reduce("A", red_A, nradmax, nlm_);
-    load_reduce("AA", red_AA, CF, nAA);
-    load_reduce("AAA", red_AAA, CF, prod_AAA.n_out);
-    if (order4) load_reduce("AAAA", red_AAAA, CF, prod_AAAA.n_out);
+    // ---- readout
+    read_readout(f, "GRACE-1L", rho_n_out, 0, energy_mlp, energy_mlp_activation, energy_mlp_ln);
+    shift_values = f.reals_or("shift_values", Flat{n_elements}, 0.0);
+    output_scale = f.real_or("output_scale", 1.0);
+    uq.load(f, n_elements);
+  }
 
-    energy_mlp = load_mlp(v, "energy_mlp", v.int_in("energy_mlp_n_layers", 2, 1, kMaxDim), rho_n_out - 1, 1, "rho_n_out - 1", "one energy");
-    energy_mlp_activation = v.int_in("energy_mlp_activation", 0, 0, 1);
-    radial_activation = v.int_in("radial_activation", 0, 0, 1);
-    AAA_right_A = v.flag("AAA_right_A", 0);
-    if (AAA_right_A) require_eq("fc_AA1_n_out", fc_AA1.n_out, nradmax, "nradmax (AAA = AA1 x A)");
-    {    // legacy: RMS layer norm of the energy-MLP input, its scale folded into layer 0 (libgrace/src/npz3.h:330-338)
-      const auto s = v.doubles("energy_mlp_scale");
-      if (!s.empty()) {
-        MLPLayer &L = energy_mlp[0];
-        require_size("energy_mlp_scale", s, (size_t) L.n_in);
-        for (int k = 0; k < L.n_in; k++)
-          for (int j = 0; j < L.n_out; j++) L.W[(size_t) k * L.n_out + j] *= s[k];
-        energy_mlp_ln = true;
-      }
+  // The readout network on the non-linear density channels, shared with GRACE-2L: `energy_mlp_*`, an activation switch, and in
+  // legacy files the scale of an RMS layer norm of its input, which is folded into the first matrix.  The engines hold at
+  // most 7 layers of at most 256 units (libgrace/src/fused_1l.cpp:226-236).
+  static void read_readout(const FileReader &f, const char *family, int density_width, int default_activation, std::vector<MLPLayer> &net,
+                           int &activation, bool &layer_norm)
+  {
+    net = read_dense_stack(f, "energy_mlp", f.whole_or("energy_mlp_n_layers", 1, 7, 2), density_width - 1, 1);
+    for (const MLPLayer &layer : net)
+      if (layer.n_out > 256 || layer.n_in > 256) throw Error(std::string(family) + ": readout layers wider than 256 units do not fit the engines");
+    activation = (int) f.whole_or("energy_mlp_activation", 0, 1, default_activation);
+    layer_norm = f.present("energy_mlp_scale");
+    if (layer_norm) {
+      const std::vector<double> scale = f.reals("energy_mlp_scale", Flat{net[0].n_in});
+      for (int row = 0; row < net[0].n_in; row++)
+        for (int col = 0; col < net[0].n_out; col++) net[0].W[(size_t) row * net[0].n_out + col] *= scale[(size_t) row];
     }
-    // readout limits of the engines (libgrace/src/fused_1l.cpp:226-236)
-    if (energy_mlp.size() > 7) throw Error("GRACE-1L: energy MLP has " + std::to_string(energy_mlp.size()) + " layers, at most 7 supported");
-    for (const auto &L : energy_mlp)
-      if (L.n_in > 256 || L.n_out > 256) throw Error("GRACE-1L: energy MLP layer widths above 256 are not supported");
-    shift_values = v.doubles("shift_values");
-    if (v.has("shift_values")) require_size("shift_values", shift_values, (size_t) n_elements);
-    else shift_values.assign(n_elements, 0.0);
-    output_scale = v.double_scalar("output_scale", 1.0);
-    uq.load(v, n_elements, "GRACE-1L/KK");
   }
 };
 
 // type2mu has ntypes + 1 entries (types are 1-based), each -1 or a model element: libgrace/include/grace/type_map.h:31-39
 inline void check_type2mu(const std::vector<int> &type2mu, int ntypes, int n_elements, const char *who)
 {
-  if ((int) type2mu.size() != ntypes + 1) throw Error(std::string(who) + ": type2mu must have ntypes + 1 entries");
+  if ((int) type2mu.size() != ntypes + 1) throw Error(std::string(who) + ": the type map needs one entry per atom type plus the unused entry 0");
   for (int t = 1; t <= ntypes; t++)
     if (type2mu[t] < -1 || type2mu[t] >= n_elements)
-      throw Error(std::string(who) + ": atom type " + std::to_string(t) + " maps to model element " + std::to_string(type2mu[t]) +
-                  " (the model has " + std::to_string(n_elements) + ")");
+      throw Error(std::string(who) + ": atom type " + std::to_string(t) + " is mapped to element " + std::to_string(type2mu[t]) + " of a model with " +
+                  std::to_string(n_elements) + " elements");
 }
 
 }    // namespace grhip

@@ -1,6 +1,6 @@
-// Host-side container of a GRACE-2L model read from kokkos.npz.  Keys, defaults and consistency checks follow the
-// reference loader libgrace/src/model_2l.cpp:28-420 (container libgrace/include/grace/model_2l.h:22-175); files of
-// max_order 3 (no AAAA / BBBB stage, libgrace/src/max_order3.h) are loaded with those stages absent.
+// Host-side container of a GRACE-2L model read from kokkos.npz and its loader.  Keys and consistency rules are the file
+// format's, as the reference loader reads it (libgrace/src/model_2l.cpp:28-420, container libgrace/include/grace/
+// model_2l.h:22-175); files of max_order 3 (no AAAA / BBBB stage, libgrace/src/max_order3.h) load with those stages absent.
 #pragma once
 
 #include "model.hpp"
@@ -57,21 +57,8 @@ struct Model2L {
     for (int s = 0; s < nsrc(); s++) w += r[s].n_in * (int) r[s].collect_ind.size();
     return w;
   }
-  // libgrace/src/model_2l.cpp:466-478, libgrace/src/uq.cpp:8-33
-  void validate_uq() const
-  {
-    if (!uq.has_uq) throw Error("GRACE-2L: the model has no UQ head");
-    if (max_order == 3) throw Error("GRACE-2L: UQ is not supported for max_order 3 models");
-    if (uq.schema != 6)
-      throw Error("GRACE-2L: UQ schema v" + std::to_string(uq.schema) + " unsupported (expects v6, uqv6 basis-RP normalize+density). Re-export the "
-                  "UQ artifacts at schema v6 with a current grace_utils.");
-    if (!uq.error.empty()) throw Error(uq.error);
-    const int total = uq_block_width(I2_red) + uq_block_width(rho_red);
-    if (total != uq.d_basis)
-      throw Error("GRACE-2L UQ: uq_rp_matrix has " + std::to_string(uq.d_basis) + " rows, the model's invariant basis has " + std::to_string(total) +
-                  "; re-export the UQ artifacts for this model");
-    if (uq.n_density != 3) throw Error("GRACE-2L UQ: " + std::to_string(uq.n_density) + " density channels, expected 3 (1 + basis blocks)");
-  }
+  // can the head be evaluated (libgrace/src/model_2l.cpp:466-478, libgrace/src/uq.cpp:8-33)
+  void validate_uq() const { uq.require_usable("GRACE-2L", max_order == 4, uq_block_width(I2_red) + uq_block_width(rho_red), 2); }
   double pair_cutoff(int mu_i, int mu_j) const
   {
     if (mu_i < 0 || mu_j < 0) return 0.0;
@@ -81,240 +68,156 @@ struct Model2L {
   void load(const Npz &z)
   {
     *this = Model2L();
-    NpzView v(z);
-    if (v.has("grace_model_kind")) {
-      const auto k = v.names("grace_model_kind");
-      if (k.size() != 1) throw bad_array("grace_model_kind", "must hold one name");
-      if (k[0] != "GRACE-2L") throw Error("GRACE-2L: the file holds a " + k[0] + " model");
-      if (v.int_scalar("grace_format_version", 0) < 1) throw bad_array("grace_format_version", "is missing or below 1 next to grace_model_kind");
-    }
-    if (v.int_scalar("grace_format_version", 0) > 2)
-      throw Error("GRACE-2L: kokkos.npz format " + std::to_string(v.int_scalar("grace_format_version", 0)) + ", this build reads up to 2");
-    const bool o4a = v.has("prod_AAAA_n_cg_terms"), o4b = v.has("prod_BBBB_n_cg_terms");
-    if (o4a != o4b) throw bad_array(o4a ? "prod_BBBB_n_cg_terms" : "prod_AAAA_n_cg_terms", "is missing: the two layers must have the same max_order");
-    const bool order4 = o4a;
-    if (!order4)
-      for (const auto &kv : z)
-        if (kv.first.find("AAAA") != std::string::npos || kv.first.find("BBBB") != std::string::npos ||
-            kv.first.rfind("fc_AA2_", 0) == 0 || kv.first.rfind("fc_BB2_", 0) == 0)
-          throw bad_array(kv.first, "is present, but the order-4 product is not: the stage is incomplete");
-    max_order = order4 ? 4 : 3;
+    const FileReader f(z, "GRACE-2L");
+    check_declaration(f, "GRACE-2L");
 
-    n_elements = v.int_in("n_elements", 89, 1, kMaxDim);
-    embedding_size = v.int_in("embedding_size", 128, 1, kMaxDim);
-    chem_embedding = v.require_doubles("chem_embedding");
-    v.require_shape("chem_embedding", {n_elements, embedding_size});
-    lmax = v.int_in("lmax", 4, 0, kMaxL);
-    nradbase = v.int_in("nradbase", 10, 1, kMaxDim);
-    radial_basis_p = v.int_in("radial_basis_p", 16, 1, kMaxP);
-    rcut = v.cutoff_scalar("rcut", 6.0, "GRACE-2L/KK");
-    has_bond_specific_cutoff = v.flag("has_bond_specific_cutoff", 0);
-    bond_cutoff_map = v.cutoffs("bond_cutoff_map", "GRACE-2L/KK");
-    v.require_shape("bond_cutoff_map", {n_elements, n_elements});
+    int *const into[] = {&n_elements, &embedding_size, &lmax, &nradbase, &radial_basis_p, &C1, &CR, &C2, &B_n_funcs, &I1_n_out, &I1_n_funcs, &I_n_funcs, &rho_n_out};
+    static const SizeKey sizes[] = {{"n_elements", 1, kSizeLimit, 89},  {"embedding_size", 1, kSizeLimit, 128},       {"lmax", 0, kDegreeLimit, 4},
+                                    {"nradbase", 1, kSizeLimit, 10},    {"radial_basis_p", 1, kEnvelopeLimit, 16},    {"mlp_rad_R_n_rad_max", 1, kSizeLimit, 32},
+                                    {"mlp_rad_R1_n_rad_max", 1, kSizeLimit, 32}, {"B_n_out", 1, kSizeLimit, 64},      {"B_n_funcs", 1, kSizeLimit, 31},
+                                    {"I1_n_out", 1, kSizeLimit, 12},    {"I1_n_funcs", 1, kSizeLimit, 4},             {"I_n_funcs", 1, kSizeLimit, 4},
+                                    {"rho_n_out", 2, kSizeLimit, 17}};
+    for (size_t k = 0; k < sizeof(sizes) / sizeof(sizes[0]); k++) *into[k] = (int) f.whole_or(sizes[k].key, sizes[k].lo, sizes[k].hi, sizes[k].absent);
+    const long harmonics = nlm();
+
+    // ---- both layers carry the fourth-order stage, or neither does
+    const bool fourth = f.present("prod_AAAA_n_cg_terms");
+    if (fourth != f.present("prod_BBBB_n_cg_terms"))
+      f.reject(fourth ? "prod_BBBB_n_cg_terms" : "prod_AAAA_n_cg_terms", "is absent while the other layer has its fourth-order product: both layers must stop at the same order");
+    max_order = fourth ? 4 : 3;
+    if (!fourth)
+      for (const auto &member : z)
+        for (const char *piece : {"AAAA", "BBBB", "fc_AA2_", "fc_BB2_"})
+          if (member.first.find(piece) != std::string::npos)
+            f.reject(member.first, "belongs to the fourth-order stage, which this file otherwise lacks: the stage is incomplete");
+
+    // ---- elements and cutoffs
+    element_names = f.labels("element_names");
+    if (f.present("element_names") && (long) element_names.size() != n_elements)
+      f.reject("element_names", "lists " + std::to_string(element_names.size()) + " elements where n_elements = " + std::to_string(n_elements));
+    chem_embedding = f.reals("chem_embedding", {n_elements, embedding_size});
+    rcut = f.length_or("rcut", 6.0);
+    has_bond_specific_cutoff = f.flag_or("has_bond_specific_cutoff", false);
+    bond_cutoff_map = f.distances_or_none("bond_cutoff_map", n_elements, n_elements);
     if (bond_cutoff_map.empty()) bond_cutoff_map.assign((size_t) n_elements * n_elements, rcut);
-    const int64_t nl_ = lmax + 1, nlm_ = nl_ * nl_;
 
-    auto load_rad = [&](const std::string &p, std::vector<MLPLayer> &layers, int &nrad) {
-      require_eq(p + "_has_chem_emb", v.int_scalar(p + "_has_chem_emb", 0), 0, "chem-embedded radial MLPs are not supported");
-      nrad = v.int_in(p + "_n_rad_max", 32, 1, kMaxDim);
-      layers = load_mlp(v, p, v.int_in(p + "_n_layers", 3, 1, kMaxDim), nradbase, (int64_t) nrad * nl_, "nradbase", "n_rad_max x (lmax + 1)");
-    };
-    load_rad("mlp_rad_R", mlp_R, C1);
-    load_rad("mlp_rad_R1", mlp_R1, CR);
-    A_lin_transform_W = v.require_doubles("A_lin_transform_W");
-    v.require_shape("A_lin_transform_W", {embedding_size, C1});
-    A_lin_transform_norm = v.double_scalar("A_lin_transform_norm", 1.0);
-    A_inv_avg_n_neigh = v.double_scalar("A_inv_avg_n_neigh", 1.0);
-    B0_lin_transform_W = v.require_doubles("B0_lin_transform_W");
-    v.require_shape("B0_lin_transform_W", {embedding_size, CR});
-    B0_lin_transform_norm = v.double_scalar("B0_lin_transform_norm", 1.0);
-    B0_inv_avg_n_neigh = v.double_scalar("B0_inv_avg_n_neigh", 1.0);
-    C2 = v.int_in("B_n_out", 64, 1, kMaxDim);
-    B_n_funcs = v.int_in("B_n_funcs", 31, 1, kMaxDim);
-
-    // FC of ch channels over nfl functions, right input with nfr functions
-    auto load_fc = [&](const std::string &p, FCWeights &fc, int64_t nfl, int64_t nfr, int64_t ch, const std::string &ch_what) {
-      fc.w_left = v.require_doubles(p + "_w_left");
-      fc.w_right = v.require_doubles(p + "_w_right");
-      fc.w_tile_left = v.require_ints(p + "_w_tile_left");
-      fc.w_tile_right = v.require_ints(p + "_w_tile_right");
-      fc.collect_to = v.require_ints(p + "_collect_to");
-      fc.collect_from = v.require_ints(p + "_collect_from");
-      fc.norm_out_factor = v.require_doubles(p + "_norm_out_factor");
-      fc.norm_left = v.double_scalar(p + "_norm_left", 1.0);
-      fc.norm_right = v.double_scalar(p + "_norm_right", 1.0);
-      fc.n_out = v.int_in(p + "_n_out", 64, 1, kMaxDim);
-      require_eq(p + "_left_coefs", v.int_scalar(p + "_left_coefs", 1), 1, "the GRACE-2L engines apply left weights in every FC");
-      require_eq(p + "_n_out", fc.n_out, ch, ch_what);
-      fc.tiles_left = (int) v.shape_rank(p + "_w_left", 3)[2];
-      fc.tiles_right = (int) v.shape_rank(p + "_w_right", 3)[2];
-      v.require_shape(p + "_w_left", {fc.n_out, ch, fc.tiles_left});
-      v.require_shape(p + "_w_right", {fc.n_out, ch, fc.tiles_right});
-      require_size(p + "_w_tile_left", fc.w_tile_left, (size_t) nfl);
-      require_index(p + "_w_tile_left", fc.w_tile_left, fc.tiles_left);
-      require_size(p + "_norm_out_factor", fc.norm_out_factor, (size_t) nfl);
-      const size_t nc = fc.collect_from.size();
-      require_size(p + "_collect_to", fc.collect_to, nc);
-      require_size(p + "_w_tile_right", fc.w_tile_right, nc);
-      require_index(p + "_collect_to", fc.collect_to, nfl);
-      require_index(p + "_collect_from", fc.collect_from, nfr);
-      require_index(p + "_w_tile_right", fc.w_tile_right, fc.tiles_right);
-      fc.n_in_left = fc.n_in_right = (int) ch;
-      fc.n_funcs = (int) nfl;
-      fc.n_conn = (int) nc;
-    };
-    auto load_prod = [&](const std::string &p, CGProduct &pr, int64_t n_left, int64_t n_right) {
-      pr.left_ind = v.require_ints(p + "_left_ind");
-      pr.right_ind = v.require_ints(p + "_right_ind");
-      pr.m_sum_ind = v.require_ints(p + "_m_sum_ind");
-      pr.cg_coeff = v.require_doubles(p + "_cg_coeff");
-      pr.n_out = v.int_in(p + "_n_output_funcs", 0, 1, kMaxDim);
-      pr.n_terms = v.int_in(p + "_n_cg_terms", 0, 1, kMaxDim);
-      const size_t nt = (size_t) pr.n_terms;
-      require_size(p + "_left_ind", pr.left_ind, nt);
-      require_size(p + "_right_ind", pr.right_ind, nt);
-      require_size(p + "_m_sum_ind", pr.m_sum_ind, nt);
-      require_size(p + "_cg_coeff", pr.cg_coeff, nt);
-      require_index(p + "_m_sum_ind", pr.m_sum_ind, pr.n_out);
-      require_eq(p + "_n_output_funcs", pr.n_out, index_extent(pr.m_sum_ind), "1 + the largest " + p + "_m_sum_ind");
-      require_index(p + "_left_ind", pr.left_ind, n_left);
-      require_index(p + "_right_ind", pr.right_ind, n_right);
-      return (int64_t) pr.n_out;
-    };
-    // reduce r of n_out channels into nfo output functions from source s (ch channels, nf functions)
-    auto load_reduce = [&](const std::string &r, const std::string &s, ReduceEq &rw, bool elem, int64_t n_out, int64_t nfo, int64_t ch,
-                           int64_t nf) {
-      const std::string wkey = r + "_reduce_" + s + "_W";
-      rw.elem = elem;
-      rw.W = v.require_doubles(wkey);
-      rw.norm = v.double_scalar(r + "_reduce_" + s + "_norm", 1.0);
-      rw.collect_ind = v.require_ints(r + "_collect_ind_" + s);
-      rw.w_l_tile = v.require_ints(r + "_w_l_tile_" + s);
-      rw.total_sum_ind = v.require_ints(r + "_total_sum_ind_" + s);
-      rw.n_in = v.int_scalar(r + "_n_in_" + s, 0);
-      rw.w_shape = v.int_in(r + "_w_shape_" + s, 0, 1, kMaxDim);
-      require_eq(r + "_n_in_" + s, rw.n_in, ch, "the channels of " + s);
-      if (elem) v.require_shape(wkey, {n_elements, n_out, ch, rw.w_shape});
-      else v.require_shape(wkey, {n_out, ch, rw.w_shape});
-      const size_t nc = rw.collect_ind.size();
-      require_size(r + "_w_l_tile_" + s, rw.w_l_tile, nc);
-      require_size(r + "_total_sum_ind_" + s, rw.total_sum_ind, nc);
-      require_index(r + "_collect_ind_" + s, rw.collect_ind, nf);
-      require_index(r + "_w_l_tile_" + s, rw.w_l_tile, rw.w_shape);
-      require_index(r + "_total_sum_ind_" + s, rw.total_sum_ind, nfo);
-    };
-    auto elem_dependent = [&](const std::string &p, int fixed) {
-      require_eq(p + "_is_central_atom_type_dependent", v.int_scalar(p + "_is_central_atom_type_dependent", fixed), fixed,
-                 "the GRACE-2L engines implement this layout only");
-    };
-
-    // ---- layer 1
-    const std::string c1_what = "the layer-1 radial channels mlp_rad_R_n_rad_max";
-    load_fc("fc_A1", fc_A1, nlm_, nlm_, C1, c1_what);
-    const int64_t nAA = load_prod("prod_AA", prod_AA, nlm_, nlm_);
-    load_fc("fc_AA1", fc_AA1, nAA, nlm_, C1, c1_what);
-    const int64_t nAAA = load_prod("prod_AAA", prod_AAA, nAA, nlm_);
-    int64_t nAAAA = 0;
-    if (order4) {
-      load_fc("fc_AA2", fc_AA2, nAA, nlm_, C1, c1_what);
-      nAAAA = load_prod("prod_AAAA", prod_AAAA, nAA, nAA);
+    // ---- the two radial networks and the species weights of the two gathers
+    for (const char *stem : {"mlp_rad_R", "mlp_rad_R1"}) {
+      const bool first = std::string(stem) == "mlp_rad_R";
+      f.must_be(std::string(stem) + "_has_chem_emb", 0, 0, "radial networks with species inputs belong to GRACE-3L");
+      (first ? mlp_R : mlp_R1) =
+          read_dense_stack(f, stem, f.whole_or(std::string(stem) + "_n_layers", 1, kSizeLimit, 3), nradbase, (long) (first ? C1 : CR) * nl());
     }
-    const char *s1[4] = {"A", "AA", "AAA", "AAAA"};
-    const int64_t nf1[4] = {nlm_, nAA, nAAA, nAAAA};
-    I1_n_out = v.int_in("I1_n_out", 12, 1, kMaxDim);
-    I1_n_funcs = v.int_in("I1_n_funcs", 4, 1, kMaxDim);
-    elem_dependent("I1", 1);
-    rho_n_out = v.int_in("rho_n_out", 17, 2, kMaxDim);
-    elem_dependent("rho", 1);
+    radial_activation = (int) f.whole_or("radial_activation", 0, 1, 0);
+    A_lin_transform_W = f.reals("A_lin_transform_W", {embedding_size, C1});
+    A_lin_transform_norm = f.real_or("A_lin_transform_norm", 1.0);
+    A_inv_avg_n_neigh = f.real_or("A_inv_avg_n_neigh", 1.0);
+    B0_lin_transform_W = f.reals("B0_lin_transform_W", {embedding_size, CR});
+    B0_lin_transform_norm = f.real_or("B0_lin_transform_norm", 1.0);
+    B0_inv_avg_n_neigh = f.real_or("B0_inv_avg_n_neigh", 1.0);
+
+    // ---- layer 1: chain over A, message I1 -> I, density rho
+    long fun1[4] = {harmonics, 0, 0, 0};
+    read_chain(f, "A", C1, fourth, fc_A1, prod_AA, fc_AA1, prod_AAA, fc_AA2, prod_AAAA, fun1);
+    const char *tags1[4] = {"A", "AA", "AAA", "AAAA"};
     for (int s = 0; s < nsrc(); s++) {
-      load_reduce("I1", s1[s], I1_red[s], true, I1_n_out, I1_n_funcs, C1, nf1[s]);
-      load_reduce("rho", s1[s], rho_red[s], true, rho_n_out, 1, C1, nf1[s]);
+      I1_red[s] = read_reduce(f, "I1", tags1[s], true, I1_n_out, I1_n_funcs, C1, fun1[s]);
+      rho_red[s] = read_reduce(f, "rho", tags1[s], true, rho_n_out, 1, C1, fun1[s]);
     }
-    require_eq("I_n_out", v.int_in("I_n_out", 32, 1, kMaxDim), CR, "YI couples I with the layer-2 radial channels mlp_rad_R1_n_rad_max");
-    I_n_funcs = v.int_in("I_n_funcs", 4, 1, kMaxDim);
-    elem_dependent("I", 0);
-    load_reduce("I", "I1", I_red, false, CR, I_n_funcs, I1_n_out, I1_n_funcs);
+    f.must_be("I_n_out", 32, CR, "the message is coupled with the layer-2 radial functions, mlp_rad_R1_n_rad_max channels wide");
+    I_red = read_reduce(f, "I", "I1", false, CR, I_n_funcs, I1_n_out, I1_n_funcs);
 
-    // ---- layer 2
+    // ---- layer 2: the neighbour gather coupled with the harmonics (YI), B, chain over B, I2
     {
-      const auto lr = v.require_ints("YI_lr_inds");
-      yi.m_sum_ind = v.require_ints("YI_m_sum_ind");
-      yi.cg_coeff = v.require_doubles("YI_cg_coeff");
-      yi.n_terms = v.int_in("YI_n_cg_terms", 0, 1, kMaxDim);
-      yi.n_out = v.int_in("YI_n_output_funcs", 0, 1, kMaxDim);
-      yi.inv_avg_n_neigh = v.double_scalar("YI_inv_avg_n_neigh", 1.0);
-      require_eq("YI_n_rad_max", v.int_scalar("YI_n_rad_max", 32), CR, "the layer-2 radial channels mlp_rad_R1_n_rad_max");
-      v.require_shape("YI_lr_inds", {yi.n_terms, 2});
-      require_size("YI_m_sum_ind", yi.m_sum_ind, (size_t) yi.n_terms);
-      require_size("YI_cg_coeff", yi.cg_coeff, (size_t) yi.n_terms);
-      for (int t = 0; t < yi.n_terms; t++) {
-        const int y = lr[2 * t], i = lr[2 * t + 1];
-        if (y < 0 || y >= nlm_ || i < 0 || i >= I_n_funcs)
-          throw bad_array("YI_lr_inds", "has (" + std::to_string(y) + ", " + std::to_string(i) + ") at " + std::to_string(t) + ", outside [0, " +
-                                            std::to_string(nlm_) + ") x [0, I_n_funcs = " + std::to_string(I_n_funcs) + ")");
+      const long terms = f.whole("YI_n_cg_terms", 1, kSizeLimit), outputs = f.whole("YI_n_output_funcs", 1, kSizeLimit);
+      f.must_be("YI_n_rad_max", 32, CR, "YI carries the layer-2 radial channels mlp_rad_R1_n_rad_max");
+      // one (harmonic, message function) pair per term: read the two columns against their own ranges
+      const std::vector<int> pairs = f.indices("YI_lr_inds", {terms, 2}, std::max<long>(harmonics, I_n_funcs));
+      for (long t = 0; t < terms; t++) {
+        const int y = pairs[(size_t) (2 * t)], fn = pairs[(size_t) (2 * t + 1)];
+        if (y >= harmonics || fn >= I_n_funcs)
+          f.reject("YI_lr_inds", "row " + std::to_string(t) + " = (" + std::to_string(y) + ", " + std::to_string(fn) + ") names a harmonic or a message function "
+                                 "that does not exist (" + std::to_string(harmonics) + " harmonics, I_n_funcs = " + std::to_string(I_n_funcs) + ")");
         yi.y.push_back(y);
-        yi.i.push_back(i);
+        yi.i.push_back(fn);
       }
-      require_index("YI_m_sum_ind", yi.m_sum_ind, yi.n_out);
-      require_eq("YI_n_output_funcs", yi.n_out, index_extent(yi.m_sum_ind), "1 + the largest YI_m_sum_ind");
+      yi.cg_coeff = f.reals("YI_cg_coeff", {terms});
+      yi.m_sum_ind = f.indices("YI_m_sum_ind", {terms}, outputs);
+      if (addressed(yi.m_sum_ind) != outputs)
+        f.reject("YI_n_output_funcs", "= " + std::to_string(outputs) + " but YI_m_sum_ind addresses " + std::to_string(addressed(yi.m_sum_ind)) + " functions");
+      yi.n_terms = (int) terms;
+      yi.n_out = (int) outputs;
+      yi.inv_avg_n_neigh = f.real_or("YI_inv_avg_n_neigh", 1.0);
     }
-    elem_dependent("B", 0);
-    load_reduce("B", "YI", B_red_YI, false, C2, B_n_funcs, CR, yi.n_out);
-    load_reduce("B", "B0", B_red_B0, false, C2, B_n_funcs, CR, nlm_);
-    const int64_t nB = B_n_funcs;
-    load_fc("fc_B1", fc_B1, nB, nB, C2, "B_n_out");
-    const int64_t nBB = load_prod("prod_BB", prod_BB, nB, nB);
-    load_fc("fc_BB1", fc_BB1, nBB, nB, C2, "B_n_out");
-    const int64_t nBBB = load_prod("prod_BBB", prod_BBB, nBB, nB);
-    int64_t nBBBB = 0;
-    if (order4) {
-      load_fc("fc_BB2", fc_BB2, nBB, nB, C2, "B_n_out");
-      nBBBB = load_prod("prod_BBBB", prod_BBBB, nBB, nBB);
-    }
-    const char *s2[4] = {"B", "BB", "BBB", "BBBB"};
-    const int64_t nf2[4] = {nB, nBB, nBBB, nBBBB};
-    require_eq("I2_n_out", v.int_in("I2_n_out", 17, 1, kMaxDim), rho_n_out, "the energy adds rho and I2 function by function: rho_n_out");
-    elem_dependent("I2", 1);
-    for (int s = 0; s < nsrc(); s++) load_reduce("I2", s2[s], I2_red[s], true, rho_n_out, 1, C2, nf2[s]);
+    B_red_YI = read_reduce(f, "B", "YI", false, C2, B_n_funcs, CR, yi.n_out);
+    B_red_B0 = read_reduce(f, "B", "B0", false, C2, B_n_funcs, CR, harmonics);
+    long fun2[4] = {B_n_funcs, 0, 0, 0};
+    read_chain(f, "B", C2, fourth, fc_B1, prod_BB, fc_BB1, prod_BBB, fc_BB2, prod_BBBB, fun2);
+    f.must_be("I2_n_out", 17, rho_n_out, "the readout adds rho and I2 channel by channel, so I2 has rho_n_out channels");
+    const char *tags2[4] = {"B", "BB", "BBB", "BBBB"};
+    for (int s = 0; s < nsrc(); s++) I2_red[s] = read_reduce(f, "I2", tags2[s], true, rho_n_out, 1, C2, fun2[s]);
 
-    // ---- readout
-    energy_rms_norm = v.flag("energy_rms_norm", 1);
+    // ---- readout: two RMS norms, the network on the non-linear channels
+    energy_rms_norm = f.flag_or("energy_rms_norm", true);
     if (energy_rms_norm) {
-      I_nl_LN_scale = v.require_doubles("I_nl_LN_scale");
-      require_eq("I_nl_LN_type", v.int_scalar("I_nl_LN_type", 1), 1, "the GRACE-2L engines implement the only_nonlin RMSNorm here");
-      require_eq("I_nl_LN_n_out", v.int_scalar("I_nl_LN_n_out", 17), rho_n_out, "rho_n_out");
-      require_size("I_nl_LN_scale", I_nl_LN_scale, (size_t) rho_n_out - 1);
-      I_0_LN_scale = v.require_doubles("I_0_LN_scale");
-      require_eq("I_0_LN_type", v.int_scalar("I_0_LN_type", 0), 0, "the GRACE-2L engines implement the full RMSNorm here");
-      require_eq("I_0_LN_n_out", v.int_scalar("I_0_LN_n_out", 17), rho_n_out, "I2_n_out");
-      require_size("I_0_LN_scale", I_0_LN_scale, (size_t) rho_n_out);
+      f.must_be("I_nl_LN_type", 1, 1, "the norm of the non-linear channels leaves the linear channel out");
+      f.must_be("I_nl_LN_n_out", 17, rho_n_out, "it normalises the rho_n_out density channels");
+      f.must_be("I_0_LN_type", 0, 0, "the norm of the second-layer density covers all its channels");
+      f.must_be("I_0_LN_n_out", 17, rho_n_out, "it normalises the I2 channels, as many as rho_n_out");
+      I_nl_LN_scale = f.reals("I_nl_LN_scale", Flat{rho_n_out - 1});
+      I_0_LN_scale = f.reals("I_0_LN_scale", Flat{rho_n_out});
     } else {
-      I_nl_LN_scale.assign(rho_n_out - 1, 1.0);
-      I_0_LN_scale.assign(rho_n_out, 1.0);
+      I_nl_LN_scale.assign((size_t) rho_n_out - 1, 1.0);
+      I_0_LN_scale.assign((size_t) rho_n_out, 1.0);
     }
-    energy_mlp = load_mlp(v, "energy_mlp", v.int_in("energy_mlp_n_layers", 2, 1, kMaxDim), rho_n_out - 1, 1, "rho_n_out - 1", "one energy");
-    energy_mlp_activation = v.int_in("energy_mlp_activation", 1, 0, 1);
-    radial_activation = v.int_in("radial_activation", 0, 0, 1);
-    {
-      const auto s = v.doubles("energy_mlp_scale");
-      if (!s.empty()) {
-        MLPLayer &L = energy_mlp[0];
-        require_size("energy_mlp_scale", s, (size_t) L.n_in);
-        for (int k = 0; k < L.n_in; k++)
-          for (int j = 0; j < L.n_out; j++) L.W[(size_t) k * L.n_out + j] *= s[k];
-        energy_mlp_ln = true;
-      }
+    Model1L::read_readout(f, "GRACE-2L", rho_n_out, 1, energy_mlp, energy_mlp_activation, energy_mlp_ln);
+    shift_values = f.reals_or("shift_values", Flat{n_elements}, 0.0);
+    output_scale = f.real_or("output_scale", 1.0);
+    uq.load(f, n_elements);
+  }
+
+ private:
+  // FC / product chain over the functions X of one layer (X = "A" or "B", all stages `width` channels wide):
+  // X1 = fc_X1(X, X), XX = X1 x X1, XX1 = fc_XX1(XX, X), XXX = XX1 x X1, [XX2 = fc_XX2(XX, X), XXXX = XX2 x XX2].
+  // functions[0] holds the functions of X on entry; the counts of XX, XXX, XXXX are filled in.
+  static void read_chain(const FileReader &f, const std::string &X, long width, bool fourth, FCWeights &fc1, CGProduct &p2, FCWeights &fc21,
+                         CGProduct &p3, FCWeights &fc22, CGProduct &p4, long functions[4])
+  {
+    const long base = functions[0];
+    const std::string XX = X + X;
+    fc1 = read_fc(f, "fc_" + X + "1", {base, base, width, width, width});
+    p2 = read_product(f, "prod_" + XX, base, base);
+    functions[1] = p2.n_out;
+    fc21 = read_fc(f, "fc_" + XX + "1", {functions[1], base, width, width, width});
+    p3 = read_product(f, "prod_" + XX + X, functions[1], base);
+    functions[2] = p3.n_out;
+    if (fourth) {
+      fc22 = read_fc(f, "fc_" + XX + "2", {functions[1], base, width, width, width});
+      p4 = read_product(f, "prod_" + XX + XX, functions[1], functions[1]);
+      functions[3] = p4.n_out;
     }
-    if (energy_mlp.size() > 7) throw Error("GRACE-2L: energy MLP has " + std::to_string(energy_mlp.size()) + " layers, at most 7 supported");
-    for (const auto &L : energy_mlp)
-      if (L.n_in > 256 || L.n_out > 256) throw Error("GRACE-2L: energy MLP layer widths above 256 are not supported");
-    shift_values = v.doubles("shift_values");
-    if (v.has("shift_values")) require_size("shift_values", shift_values, (size_t) n_elements);
-    else shift_values.assign(n_elements, 0.0);
-    output_scale = v.double_scalar("output_scale", 1.0);
-    uq.load(v, n_elements, "GRACE-2L/KK");
-    element_names = v.names("element_names");
-    if (v.has("element_names")) require_size("element_names", element_names, (size_t) n_elements);
+  }
+  // Projection `<target>_*_<source>` of a source tensor (`in_width` channels, `in_functions` functions) onto `out_width` channels
+  // of `out_functions` output functions; `per_element`: one weight set per element of the central atom.
+  ReduceEq read_reduce(const FileReader &f, const std::string &target, const std::string &source, bool per_element, long out_width, long out_functions,
+                       long in_width, long in_functions) const
+  {
+    ReduceEq r;
+    long tiles = 0, picked = 0;
+    const std::string W = target + "_reduce_" + source + "_W";
+    f.must_be(target + "_is_central_atom_type_dependent", per_element, per_element,
+              per_element ? "this projection has one weight set per central element" : "this projection has one weight set for all elements");
+    f.must_be(target + "_n_in_" + source, in_width, in_width, "it is the channel width of " + source);
+    r.W = per_element ? f.reals(W, {n_elements, out_width, in_width, Ext::any(tiles)}) : f.reals(W, {out_width, in_width, Ext::any(tiles)});
+    f.must_be(target + "_w_shape_" + source, tiles, tiles, "it counts the weight tiles stored in " + W);
+    r.collect_ind = f.indices(target + "_collect_ind_" + source, {Ext::any(picked)}, in_functions);
+    r.w_l_tile = f.indices(target + "_w_l_tile_" + source, {picked}, tiles);
+    r.total_sum_ind = f.indices(target + "_total_sum_ind_" + source, {picked}, out_functions);
+    r.norm = f.real_or(W.substr(0, W.size() - 2) + "_norm", 1.0);
+    r.elem = per_element;
+    r.n_in = (int) in_width;
+    r.w_shape = (int) tiles;
+    return r;
   }
 };
 

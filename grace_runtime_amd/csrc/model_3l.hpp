@@ -1,11 +1,14 @@
-// Host-side container of a GRACE-3L model read from kokkos.npz.  The file names its components (SPBF layers, cp_l
-// products, reduces, FCs, norms) in index lists; keys, defaults and the dataflow check follow the reference loader
-// libgrace/src/model_3l.cpp:36-464 (container libgrace/include/grace/model_3l.h:38-190).
+// Host-side container of a GRACE-3L model read from kokkos.npz and its loader.  The file lists its components (SPBF layers,
+// cp_l products, reduces, FCs, norms) by name; keys and consistency rules are the file format's, as the reference loader
+// reads it (libgrace/src/model_3l.cpp:36-464, container libgrace/include/grace/model_3l.h:38-190).  The architecture the
+// engines evaluate is written down once, as a table of components and their inputs (kLayerPlan), and the file is
+// checked against that table.
 #pragma once
 
 #include "model.hpp"
 
 #include <map>
+#include <set>
 
 namespace grhip {
 
@@ -94,349 +97,363 @@ struct Model3L {
   {
     for (const auto &x : v)
       if (x.name == name) return x;
-    throw Error("GRACE-3L: no component '" + name + "'");
+    throw Error("GRACE-3L: the model has no component named '" + name + "'");
   }
 
   void load(const Npz &z)
   {
     *this = Model3L();
-    NpzView v(z);
-    if (v.has("grace_model_kind")) {
-      const auto k = v.names("grace_model_kind");
-      if (k.size() != 1) throw bad_array("grace_model_kind", "must hold one name");
-      if (k[0] != "GRACE-3L") throw Error("GRACE-3L: the file holds a " + k[0] + " model");
-      if (v.int_scalar("grace_format_version", 0) < 1) throw bad_array("grace_format_version", "is missing or below 1 next to grace_model_kind");
-    }
-    if (v.int_scalar("grace_format_version", 0) > 2)
-      throw Error("GRACE-3L: kokkos.npz format " + std::to_string(v.int_scalar("grace_format_version", 0)) + ", this build reads up to 2");
-    for (const char *k : {"energy_mlp_scale", "radial_activation", "energy_rms_norm", "AAA_right_A"})
-      if (v.has(k)) throw bad_array(k, "is a legacy GRACE-1L/2L key, not supported in GRACE-3L");
-    auto size = [&](const std::string &k) { return v.int_in(k, 0, 1, kMaxDim); };
+    const FileReader f(z, "GRACE-3L");
+    check_declaration(f, "GRACE-3L");
+    for (const char *old : {"energy_mlp_scale", "radial_activation", "energy_rms_norm", "AAA_right_A"})
+      if (f.present(old)) f.reject(old, "is a switch of the one- and two-layer formats; a GRACE-3L file must not carry it");
 
-    n_elements = size("n_elements");
-    embedding_size = v.int_in("embedding_size", 64, 1, kMaxDim);
-    nradbase = v.int_in("nradbase", 10, 1, kMaxDim);
-    lmax = v.int_in("lmax", v.int_in("A1_lmax", 4, 0, kMaxL), 0, kMaxL);
-    const int nl_ = lmax + 1, nlm_ = nl_ * nl_;
-    rcut = v.cutoff_scalar("rcut", 6.0, "GRACE-3L/KK");
-    has_bond_specific_cutoff = v.flag("has_bond_specific_cutoff", 0);
-    chem_embedding = v.require_doubles("chem_embedding");
-    v.require_shape("chem_embedding", {n_elements, embedding_size});
-    shift_values = v.require_doubles("shift_values");
-    require_size("shift_values", shift_values, n_elements);
-    output_scale = v.double_scalar("output_scale", 1.0);
-    element_names = v.names("element_names");
-    require_size("element_names", element_names, n_elements);
-    bond_cutoff_map = v.cutoffs("bond_cutoff_map", "GRACE-3L/KK");
-    v.require_shape("bond_cutoff_map", {n_elements, n_elements});
+    n_elements = (int) f.whole("n_elements", 1, kSizeLimit);
+    embedding_size = (int) f.whole_or("embedding_size", 1, kSizeLimit, 64);
+    nradbase = (int) f.whole_or("nradbase", 1, kSizeLimit, 10);
+    lmax = (int) f.whole_or("lmax", 0, kDegreeLimit, f.whole_or("A1_lmax", 0, kDegreeLimit, 4));
+    rcut = f.length_or("rcut", 6.0);
+    has_bond_specific_cutoff = f.flag_or("has_bond_specific_cutoff", false);
+    bond_cutoff_map = f.distances_or_none("bond_cutoff_map", n_elements, n_elements);
     if (bond_cutoff_map.empty()) bond_cutoff_map.assign((size_t) n_elements * n_elements, rcut);
+    chem_embedding = f.reals("chem_embedding", {n_elements, embedding_size});
+    shift_values = f.reals("shift_values", Flat{n_elements});
+    output_scale = f.real_or("output_scale", 1.0);
+    element_names = f.labels("element_names");
+    if ((long) element_names.size() != n_elements)
+      f.reject("element_names", "lists " + std::to_string(element_names.size()) + " elements where n_elements = " + std::to_string(n_elements));
 
-    auto load_net = [&](const std::string &p, Mlp &m, int64_t n_in, int64_t n_out, const std::string &in_why, const std::string &out_why) {
-      const int n = v.int_in(p + "_n_layers", 0, 1, kMaxDim);
-      if (v.has(p + "_W" + std::to_string(n))) throw bad_array(p + "_n_layers", "is " + std::to_string(n) + ", but the file has " + p + "_W" + std::to_string(n));
-      m.layers = load_mlp(v, p, n, n_in, n_out, in_why, out_why);
-      for (int i = 0; i < n; i++) {
-        const std::string bk = p + "_b" + std::to_string(i);
-        m.bias.push_back(v.doubles(bk));
-        if (v.has(bk)) require_size(bk, m.bias.back(), m.layers[i].n_out);
-      }
-    };
+    for (const std::string &name : f.labels("spbf_names")) spbf.push_back(read_spbf(f, name));
+    for (const std::string &name : f.labels("prod_names")) prod.push_back(read_couple(f, name));
+    for (const std::string &name : f.labels("reduce_names")) reduce.push_back(read_projection(f, name));
+    for (const std::string &name : f.labels("fc_names")) fc.push_back(read_right_fc(f, name));
+    for (const std::string &name : f.labels("eqnorm_names")) eqnorm.push_back(read_eqnorm(f, name));
+    for (const std::string &name : f.labels("rmsnorm_names")) rmsnorm.push_back(read_rmsnorm(f, name));
 
-    for (const auto &nm : v.names("spbf_names")) {
-      Spbf s;
-      s.name = nm;
-      s.equivariant = v.flag(nm + "_equivariant", 0);
-      s.n_rad_max = size(nm + "_n_rad_max");
-      require_eq(nm + "_n_rad_basis", v.int_scalar(nm + "_n_rad_basis", nradbase), nradbase, "nradbase, the radial MLP's Chebyshev inputs");
-      require_eq(nm + "_lmax", v.int_scalar(nm + "_lmax", 4), lmax, "the model's lmax");
-      (void) v.int_in(nm + "_Lmax", 4, 0, kMaxL);
-      s.p = v.int_in(nm + "_p", 5, 1, kMaxP);
-      (void) v.cutoff_scalar(nm + "_rcut", rcut, "GRACE-3L/KK");
-      s.inv_avg_n_neigh = v.double_scalar(nm + "_inv_avg_n_neigh", 1.0);
-      s.l_tile = v.require_ints(nm + "_l_tile");
-      require_size(nm + "_l_tile", s.l_tile, nlm_);
-      require_index(nm + "_l_tile", s.l_tile, nl_);
-      load_net(nm + "_mlp", s.mlp, nradbase + 2 * embedding_size, (int64_t) s.n_rad_max * nl_, "nradbase + 2 embedding_size", "n_rad_max (lmax+1)");
-      if (!s.equivariant) {
-        s.lin_transform_W = v.require_doubles(nm + "_lin_transform_W");
-        v.require_shape(nm + "_lin_transform_W", {embedding_size, s.n_rad_max});
-        s.lin_transform_norm = v.double_scalar(nm + "_lin_transform_norm", 1.0);
-      } else {
-        s.nfunc = size(nm + "_nfunc");
-        s.n_lm_ind = size(nm + "_n_lm_ind");
-        s.chem_linear_W = v.require_doubles(nm + "_chem_linear_W");
-        v.require_shape(nm + "_chem_linear_W", {embedding_size, s.n_rad_max});
-        s.chem_linear_norm = v.double_scalar(nm + "_chem_linear_norm", 1.0);
-        s.chem_l0_mask = v.require_doubles(nm + "_chem_l0_mask");
-        require_size(nm + "_chem_l0_mask", s.chem_l0_mask, s.n_lm_ind);
-        s.cg_W = v.require_doubles(nm + "_cg_W");
-        v.require_shape(nm + "_cg_W", {(int64_t) nlm_ * s.n_lm_ind, s.nfunc});
-      }
-      spbf.push_back(std::move(s));
-    }
+    // one envelope for all layers
     if (!spbf.empty()) radial_basis_p = spbf[0].p;
-    for (const auto &s : spbf)
+    for (const Spbf &s : spbf)
       if (s.p != radial_basis_p)
-        throw bad_array(s.name + "_p", "is " + std::to_string(s.p) + ", the envelope order of " + spbf[0].name + " is " + std::to_string(radial_basis_p) +
-                                           "; layers with different orders are not supported");
+        f.reject(s.name + "_p", "= " + std::to_string(s.p) + " while " + spbf[0].name + " uses the envelope order " + std::to_string(radial_basis_p) +
+                                    "; the engines evaluate one envelope for all layers");
 
-    for (const auto &nm : v.names("prod_names")) {
-      Cpl c;
-      c.name = nm;
-      c.rank = size(nm + "_rank");
-      c.nfunc = size(nm + "_nfunc");
-      c.n_left = size(nm + "_n_left");
-      c.n_right = size(nm + "_n_right");
-      c.n_groups_left = size(nm + "_n_groups_left");
-      c.n_groups_right = size(nm + "_n_groups_right");
-      c.norm_u = v.double_scalar(nm + "_norm_u", 1.0);
-      c.norm_v = v.double_scalar(nm + "_norm_v", 1.0);
-      c.U = v.require_doubles(nm + "_U");
-      v.require_shape(nm + "_U", {c.n_groups_left, c.rank, c.n_left});
-      c.V = v.require_doubles(nm + "_V");
-      v.require_shape(nm + "_V", {c.n_groups_right, c.rank, c.n_right});
-      c.cg.cg_coeff = v.require_doubles(nm + "_cg");
-      c.cg.n_terms = (int) c.cg.cg_coeff.size();
-      c.cg.n_out = c.nfunc;
-      c.group_left = v.require_ints(nm + "_group_left");
-      require_index(nm + "_group_left", c.group_left, c.n_groups_left);
-      c.group_right = v.require_ints(nm + "_group_right");
-      require_index(nm + "_group_right", c.group_right, c.n_groups_right);
-      c.cg.left_ind = v.require_ints(nm + "_left_ind");
-      require_size(nm + "_left_ind", c.cg.left_ind, c.cg.n_terms);
-      require_index(nm + "_left_ind", c.cg.left_ind, (int64_t) c.group_left.size());
-      c.cg.right_ind = v.require_ints(nm + "_right_ind");
-      require_size(nm + "_right_ind", c.cg.right_ind, c.cg.n_terms);
-      require_index(nm + "_right_ind", c.cg.right_ind, (int64_t) c.group_right.size());
-      c.cg.m_sum_ind = v.require_ints(nm + "_m_sum_ind");
-      require_size(nm + "_m_sum_ind", c.cg.m_sum_ind, c.cg.n_terms);
-      require_index(nm + "_m_sum_ind", c.cg.m_sum_ind, c.nfunc);
-      const auto out_l = v.require_ints(nm + "_out_l");
-      require_size(nm + "_out_l", out_l, c.nfunc);
-      require_index(nm + "_out_l", out_l, kMaxL + 1);
-      prod.push_back(std::move(c));
-    }
+    rho_width = check_against_plan(f);
+    const std::vector<std::string> origins = f.labels("out1_origins");
+    if (std::set<std::string>(origins.begin(), origins.end()) != std::set<std::string>{"rho1_norm", "rho2_norm", "rho3_norm"} || origins.size() != 3)
+      f.reject("out1_origins", "must name the three normalised densities rho1_norm, rho2_norm, rho3_norm, whose sum the readout takes");
+    f.must_be("energy_mlp_n_origins", 3, 3, "the readout sums three densities");
+    f.must_be("energy_mlp_origin_n_out", rho_width, rho_width, "it is the channel width of the normalised densities");
+    read_net(f, "energy_mlp", energy_mlp, rho_width - 1, 1);
+    energy_mlp_activation = (int) f.whole_or("energy_mlp_activation", 0, 1, 0);
 
-    for (const auto &nm : v.names("reduce_names")) {
-      Reduce r;
-      r.name = nm;
-      r.n_out = size(nm + "_n_out");
-      r.n_funcs = size(nm + "_n_funcs");
-      r.only_invar = v.flag(nm + "_only_invar", 0);
-      r.elem_dep = v.flag(nm + "_is_central_atom_type_dependent", 0);
-      for (const auto &cn : v.names(nm + "_instruction_names")) {
-        Instr ri;
-        ri.name = cn;
-        ri.n_in = size(nm + "_n_in_" + cn);
-        ri.w_shape = size(nm + "_w_shape_" + cn);
-        const std::string wk = nm + "_reduce_" + cn + "_W";
-        ri.W = v.require_doubles(wk);
-        if (r.elem_dep) v.require_shape(wk, {n_elements, r.n_out, ri.n_in, ri.w_shape});
-        else v.require_shape(wk, {r.n_out, ri.n_in, ri.w_shape});
-        ri.norm = v.double_scalar(nm + "_reduce_" + cn + "_norm", 1.0);
-        ri.collect_ind = v.require_ints(nm + "_collect_ind_" + cn);
-        const size_t nc = ri.collect_ind.size();
-        ri.w_l_tile = v.require_ints(nm + "_w_l_tile_" + cn);
-        require_size(nm + "_w_l_tile_" + cn, ri.w_l_tile, nc);
-        require_index(nm + "_w_l_tile_" + cn, ri.w_l_tile, ri.w_shape);
-        ri.total_sum_ind = v.require_ints(nm + "_total_sum_ind_" + cn);
-        require_size(nm + "_total_sum_ind_" + cn, ri.total_sum_ind, nc);
-        require_index(nm + "_total_sum_ind_" + cn, ri.total_sum_ind, r.nfo());
-        r.instr.push_back(std::move(ri));
-      }
-      r.norm_map = v.doubles(nm + "_norm_map");
-      if (v.has(nm + "_norm_map")) require_size(nm + "_norm_map", r.norm_map, r.nfo());
-      reduce.push_back(std::move(r));
-    }
-
-    for (const auto &nm : v.names("fc_names")) {
-      Fc f;
-      f.name = nm;
-      const std::string p = "fc_" + nm;
-      f.n_out = size(p + "_n_out");
-      if (v.flag(p + "_left_coefs", 0)) throw bad_array(p + "_left_coefs", "is 1: FCs with left weights are not a part of the GRACE-3L architecture");
-      f.w_right = v.require_doubles(p + "_w_right");
-      const auto wr = v.shape_rank(p + "_w_right", 3);
-      require_eq(p + "_w_right", (int64_t) wr[0], f.n_out, p + "_n_out", "rows");
-      f.n_in_right = (int) wr[1];
-      f.w_shape_right = (int) wr[2];
-      f.norm_right = v.double_scalar(p + "_norm_right", 1.0);
-      f.n_funcs_left = (int) v.shape_rank(p + "_w_tile_left", 1)[0];
-      f.norm_out_factor = v.require_doubles(p + "_norm_out_factor");
-      require_size(p + "_norm_out_factor", f.norm_out_factor, f.n_funcs_left);
-      f.collect_from = v.require_ints(p + "_collect_from");
-      f.collect_to = v.require_ints(p + "_collect_to");
-      require_size(p + "_collect_to", f.collect_to, f.collect_from.size());
-      require_index(p + "_collect_to", f.collect_to, f.n_funcs_left);
-      f.w_tile_right = v.require_ints(p + "_w_tile_right");
-      require_size(p + "_w_tile_right", f.w_tile_right, f.collect_from.size());
-      require_index(p + "_w_tile_right", f.w_tile_right, f.w_shape_right);
-      fc.push_back(std::move(f));
-    }
-
-    for (const auto &nm : v.names("eqnorm_names")) {
-      EqNorm e;
-      e.name = nm;
-      e.affine_weight = v.require_doubles(nm + "_affine_weight");
-      const auto aw = v.shape_rank(nm + "_affine_weight", 2);
-      e.n_groups = (int) aw[0];
-      e.n_out = (int) aw[1];
-      e.degree_weights = v.require_doubles(nm + "_degree_weights");
-      e.M = (int) e.degree_weights.size();
-      e.l0_mask = v.require_doubles(nm + "_l0_mask");
-      require_size(nm + "_l0_mask", e.l0_mask, e.M);
-      e.expand_index = v.require_ints(nm + "_expand_index");
-      require_size(nm + "_expand_index", e.expand_index, e.M);
-      require_index(nm + "_expand_index", e.expand_index, e.n_groups);
-      e.eps = v.double_scalar(nm + "_eps", 1e-8);
-      if (e.eps < 0.0) throw bad_array(nm + "_eps", "is negative");
-      e.center_l0 = v.flag(nm + "_center_l0", 1);
-      eqnorm.push_back(std::move(e));
-    }
-    for (const auto &nm : v.names("rmsnorm_names")) {
-      RmsNorm r;
-      r.name = nm;
-      r.scale = v.require_doubles(nm + "_scale");
-      r.type = v.flag(nm + "_type", 0) ? 1 : 0;
-      r.n_out = v.int_in(nm + "_n_out", (int) std::min<size_t>(r.scale.size() + r.type, kMaxDim), 1, kMaxDim);
-      require_size(nm + "_scale", r.scale, r.n_out - r.type);
-      rmsnorm.push_back(std::move(r));
-    }
-    const auto origins = v.names("out1_origins");
-    require_eq("energy_mlp_n_origins", v.int_scalar("energy_mlp_n_origins", (int) origins.size()), (int64_t) origins.size(), "the names in out1_origins");
-    rho_width = check_dataflow(origins);
-    if (v.has("energy_mlp_origin_n_out")) require_eq("energy_mlp_origin_n_out", v.int_scalar("energy_mlp_origin_n_out", 0), rho_width, "the channels of out1_origins");
-    load_net("energy_mlp", energy_mlp, rho_width - 1, 1, "the channels of out1_origins but the linear channel 0", "one energy per atom");
-    energy_mlp_activation = v.int_in("energy_mlp_activation", 0, 0, 1);
-    // ---- UQ head (optional): the GMM feature projects the inputs of the rho1 | rho2 | rho3 reduces
-    uq.load(v, n_elements, "GRACE-3L");
+    // ---- UQ head (optional): the GMM feature projects the inputs of the rho1 | rho2 | rho3 reduces.  Unlike the one- and
+    // two-layer loaders this one refuses a file whose head cannot be evaluated.
+    uq.load(f, n_elements);
     if (uq.has_uq) {
-      if (uq.schema != 6)
-        throw Error("GRACE-3L UQ: schema v" + std::to_string(uq.schema) + " unsupported (expects v6, uqv6 basis-RP normalize+density). Re-export the "
-                    "UQ artifacts at schema v6 with a current grace_utils.");
+      if (uq.schema != 6) throw Error("GRACE-3L: UQ head of schema " + std::to_string(uq.schema) + "; only schema 6 (uqv6) can be evaluated");
       if (!uq.error.empty()) throw Error(uq.error);
       if (uq.n_density > 4)
-        throw Error("GRACE-3L UQ: uq_n_density (" + std::to_string(uq.n_density) + ") > 4, the number of density channels this model's UQ kernels "
-                    "write. Artifact has an unexpected invariant-block count.");
-      int64_t width = 0;
-      for (int k = 1; k <= 3; k++)
-        for (const auto &ins : by_name(reduce, "rho" + std::to_string(k)).instr) width += (int64_t) ins.n_in * (int64_t) ins.collect_ind.size();
-      require_eq("uq_rp_matrix", uq.d_basis, width, "the inputs of the rho1, rho2, rho3 reduces", "rows");
+        throw Error("GRACE-3L UQ head: " + std::to_string(uq.n_density) + " density channels; the three-layer kernels write at most 4 (total, rho1, rho2, rho3)");
+      long basis = 0;
+      for (const char *rho : {"rho1", "rho2", "rho3"})
+        for (const Instr &ins : by_name(reduce, rho).instr) basis += (long) ins.n_in * (long) ins.collect_ind.size();
+      if (basis != uq.d_basis)
+        f.reject("uq_rp_matrix", "projects " + std::to_string(uq.d_basis) + " basis functions; the inputs of rho1, rho2, rho3 hold " + std::to_string(basis));
     }
   }
 
  private:
-  // Every component against the functions and channels of its inputs, in the order the engines evaluate them
-  // (libgrace/src/model_3l.cpp:36-154); a component outside the three-layer graph, or a missing one, is an error.
-  int check_dataflow(const std::vector<std::string> &origins)
+  // ---- component readers --------------------------------------------------------------------------------------
+  // dense stack with optional biases `<stem>_b<k>`; the declared depth must match the matrices in the file
+  static void read_net(const FileReader &f, const std::string &stem, Mlp &net, long first_in, long last_out)
   {
-    struct Shape {
-      int nf, nc;
-    };
-    std::map<std::string, Shape> T;
-    std::map<std::string, int> used;
-    auto find = [&](auto &vec, const char *list, const std::string &name) -> auto & {
-      int at = -1;
-      for (size_t i = 0; i < vec.size(); i++)
-        if (vec[i].name == name) {
-          if (at >= 0) throw bad_array(list, "lists '" + name + "' twice");
-          at = (int) i;
-        }
-      if (at < 0) throw bad_array(list, "has no '" + name + "', a part of the GRACE-3L architecture");
-      used[std::string(list) + "/" + name] = 1;
-      return vec[at];
-    };
-    auto unused = [&](auto &vec, const char *list) {
-      for (const auto &x : vec)
-        if (!used.count(std::string(list) + "/" + x.name)) throw bad_array(list, "lists '" + x.name + "', not a part of the GRACE-3L architecture");
-    };
-    auto red = [&](const std::string &name, std::vector<std::string> inputs) {
-      auto &r = find(reduce, "reduce_names", name);
-      std::vector<std::string> got;
-      for (const auto &ins : r.instr) got.push_back(ins.name);
-      std::vector<std::string> a = got, b = inputs;
-      std::sort(a.begin(), a.end());
-      std::sort(b.begin(), b.end());
-      if (a != b) throw bad_array(name + "_instruction_names", "does not name the inputs of " + name + " in the GRACE-3L architecture");
-      for (const auto &ins : r.instr) {
-        const Shape in = T.at(ins.name);
-        require_eq(name + "_n_in_" + ins.name, ins.n_in, in.nc, "the channels of " + ins.name);
-        require_index(name + "_collect_ind_" + ins.name, ins.collect_ind, in.nf);
-      }
-      T[name] = {r.nfo(), r.n_out};
-    };
-    auto cpl = [&](const std::string &name, const std::string &left, const std::string &right) {
-      auto &c = find(prod, "prod_names", name);
-      const Shape l = T.at(left), r = T.at(right);
-      require_eq(name + "_group_left", (int64_t) c.group_left.size(), l.nf, "the functions of " + left, "values");
-      require_eq(name + "_n_left", c.n_left, l.nc, "the channels of " + left);
-      require_eq(name + "_group_right", (int64_t) c.group_right.size(), r.nf, "the functions of " + right, "values");
-      require_eq(name + "_n_right", c.n_right, r.nc, "the channels of " + right);
-      T[name] = {c.nfunc, c.rank};
-    };
-    auto fcl = [&](const std::string &name, const std::string &left, const std::string &right) {
-      auto &f = find(fc, "fc_names", name);
-      const std::string p = "fc_" + name;
-      const Shape l = T.at(left), r = T.at(right);
-      require_eq(p + "_w_tile_left", f.n_funcs_left, l.nf, "the functions of " + left, "values");
-      require_eq(p + "_n_out", f.n_out, l.nc, "the channels of " + left);
-      require_eq(p + "_w_right", f.n_in_right, r.nc, "the channels of " + right, "columns");
-      require_index(p + "_collect_from", f.collect_from, r.nf);
-      T[name] = {f.n_funcs_left, f.n_out};
-    };
-    if (spbf.size() != 3) throw bad_array("spbf_names", "has " + std::to_string(spbf.size()) + " names, expected 3 (A1, A2, A3)");
-    for (int k = 1; k <= 3; k++) {
-      const std::string ks = std::to_string(k), K = "A" + ks;
-      auto &s = find(spbf, "spbf_names", K);
-      if (s.name != spbf[k - 1].name) throw bad_array("spbf_names", "lists '" + K + "' out of order");
-      std::string X = K;
-      if (k == 1) {
-        if (s.equivariant) throw bad_array(K + "_equivariant", "is 1, expected 0 (the first layer has no message to couple)");
-        T[K] = {nlm(), s.n_rad_max};
-      } else {
-        if (!s.equivariant) throw bad_array(K + "_equivariant", "is 0, expected 1 (the layer couples the message of the one before)");
-        const std::string msg = "eq" + std::to_string(k - 1) + "_norm";
-        require_eq(K + "_n_lm_ind", s.n_lm_ind, T.at(msg).nf, "the functions of the message " + msg);
-        require_eq(K + "_n_rad_max", s.n_rad_max, T.at(msg).nc, "the channels of the message " + msg);
-        T[K] = {s.nfunc, s.n_rad_max};
-        red(K + "_red", {K});
-        X = K + "_red";
-      }
-      cpl(K + "_2", X, X);
-      red(K + "_2_red", {K + "_2"});
-      fcl(K + "_2a", K + "_2_red", X);
-      cpl(K + "_3", K + "_2a", X);
-      red(K + "_3_red", {K + "_3"});
-      fcl(K + "_2b", K + "_2_red", X);
-      cpl(K + "_4", K + "_2b", K + "_2b");
-      red(K + "_4_red", {K + "_4"});
-      const std::vector<std::string> collect = {X, K + "_2_red", K + "_3_red", K + "_4_red"};
-      if (k < 3) {
-        red("eq" + ks, collect);
-        auto &e = find(eqnorm, "eqnorm_names", "eq" + ks + "_norm");
-        const Shape in = T.at("eq" + ks);
-        require_eq(e.name + "_degree_weights", e.M, in.nf, "the functions of eq" + ks, "values");
-        require_eq(e.name + "_affine_weight", e.n_out, in.nc, "the channels of eq" + ks, "columns");
-        T[e.name] = {e.M, e.n_out};
-      }
-      red("rho" + ks, collect);
-      auto &n = find(rmsnorm, "rmsnorm_names", "rho" + ks + "_norm");
-      const Shape in = T.at("rho" + ks);
-      require_eq(n.name + "_n_out", n.n_out, in.nc, "the channels of rho" + ks);
-      T[n.name] = {in.nf, n.n_out};
+    const long depth = f.whole(stem + "_n_layers", 1, kSizeLimit);
+    if (f.present(stem + "_W" + std::to_string(depth)))
+      f.reject(stem + "_n_layers", "= " + std::to_string(depth) + " but the file holds a further matrix " + stem + "_W" + std::to_string(depth));
+    net.layers = read_dense_stack(f, stem, depth, first_in, last_out);
+    for (long k = 0; k < depth; k++) {
+      const std::string key = stem + "_b" + std::to_string(k);
+      net.bias.push_back(f.present(key) ? f.reals(key, Flat{net.layers[(size_t) k].n_out}) : std::vector<double>());
     }
-    unused(spbf, "spbf_names");
-    unused(prod, "prod_names");
-    unused(reduce, "reduce_names");
-    unused(fc, "fc_names");
-    unused(eqnorm, "eqnorm_names");
-    unused(rmsnorm, "rmsnorm_names");
-    std::vector<std::string> want = {"rho1_norm", "rho2_norm", "rho3_norm"}, got = origins;
-    std::sort(got.begin(), got.end());
-    if (got != want) throw bad_array("out1_origins", "does not name rho1_norm, rho2_norm, rho3_norm");
-    const int w = T.at(want[0]).nc;
-    for (const auto &o : want) require_eq(o + "_n_out", T.at(o).nc, w, "the channels of " + want[0]);
-    return w;
+  }
+  Spbf read_spbf(const FileReader &f, const std::string &name) const
+  {
+    Spbf s;
+    s.name = name;
+    s.equivariant = f.flag_or(name + "_equivariant", false);
+    s.n_rad_max = (int) f.whole(name + "_n_rad_max", 1, kSizeLimit);
+    s.p = (int) f.whole_or(name + "_p", 1, kEnvelopeLimit, 5);
+    s.inv_avg_n_neigh = f.real_or(name + "_inv_avg_n_neigh", 1.0);
+    f.must_be(name + "_n_rad_basis", nradbase, nradbase, "every layer's radial network takes the nradbase Chebyshev functions");
+    f.must_be(name + "_lmax", 4, lmax, "every layer expands the bonds up to the model's lmax");
+    (void) f.whole_or(name + "_Lmax", 0, kDegreeLimit, 4);
+    (void) f.length_or(name + "_rcut", rcut);
+    s.l_tile = f.indices(name + "_l_tile", {nlm()}, nl());
+    read_net(f, name + "_mlp", s.mlp, nradbase + 2 * embedding_size, (long) s.n_rad_max * nl());
+    if (s.equivariant) {
+      s.nfunc = (int) f.whole(name + "_nfunc", 1, kSizeLimit);
+      s.n_lm_ind = (int) f.whole(name + "_n_lm_ind", 1, kSizeLimit);
+      s.chem_linear_W = f.reals(name + "_chem_linear_W", {embedding_size, s.n_rad_max});
+      s.chem_linear_norm = f.real_or(name + "_chem_linear_norm", 1.0);
+      s.chem_l0_mask = f.reals(name + "_chem_l0_mask", Flat{s.n_lm_ind});
+      s.cg_W = f.reals(name + "_cg_W", {(long) nlm() * s.n_lm_ind, s.nfunc});
+    } else {
+      s.lin_transform_W = f.reals(name + "_lin_transform_W", {embedding_size, s.n_rad_max});
+      s.lin_transform_norm = f.real_or(name + "_lin_transform_norm", 1.0);
+    }
+    return s;
+  }
+  static Cpl read_couple(const FileReader &f, const std::string &name)
+  {
+    Cpl c;
+    c.name = name;
+    int *const into[] = {&c.rank, &c.nfunc, &c.n_left, &c.n_right, &c.n_groups_left, &c.n_groups_right};
+    const char *const keys[] = {"_rank", "_nfunc", "_n_left", "_n_right", "_n_groups_left", "_n_groups_right"};
+    for (int k = 0; k < 6; k++) *into[k] = (int) f.whole(name + keys[k], 1, kSizeLimit);
+    c.U = f.reals(name + "_U", {c.n_groups_left, c.rank, c.n_left});
+    c.V = f.reals(name + "_V", {c.n_groups_right, c.rank, c.n_right});
+    c.norm_u = f.real_or(name + "_norm_u", 1.0);
+    c.norm_v = f.real_or(name + "_norm_v", 1.0);
+    long lf = 0, rf = 0, terms = 0;
+    c.group_left = f.indices(name + "_group_left", {Ext::any(lf)}, c.n_groups_left);
+    c.group_right = f.indices(name + "_group_right", {Ext::any(rf)}, c.n_groups_right);
+    c.cg.cg_coeff = f.reals(name + "_cg", {Ext::any(terms)});
+    c.cg.left_ind = f.indices(name + "_left_ind", {terms}, lf);
+    c.cg.right_ind = f.indices(name + "_right_ind", {terms}, rf);
+    c.cg.m_sum_ind = f.indices(name + "_m_sum_ind", {terms}, c.nfunc);
+    (void) f.indices(name + "_out_l", {c.nfunc}, kDegreeLimit + 1);
+    c.cg.n_terms = (int) terms;
+    c.cg.n_out = c.nfunc;
+    return c;
+  }
+  Reduce read_projection(const FileReader &f, const std::string &name) const
+  {
+    Reduce r;
+    r.name = name;
+    r.n_out = (int) f.whole(name + "_n_out", 1, kSizeLimit);
+    r.n_funcs = (int) f.whole(name + "_n_funcs", 1, kSizeLimit);
+    r.only_invar = f.flag_or(name + "_only_invar", false);
+    r.elem_dep = f.flag_or(name + "_is_central_atom_type_dependent", false);
+    for (const std::string &source : f.labels(name + "_instruction_names")) {
+      Instr in;
+      in.name = source;
+      in.n_in = (int) f.whole(name + "_n_in_" + source, 1, kSizeLimit);
+      in.w_shape = (int) f.whole(name + "_w_shape_" + source, 1, kSizeLimit);
+      const std::string W = name + "_reduce_" + source + "_W";
+      in.W = r.elem_dep ? f.reals(W, {n_elements, r.n_out, in.n_in, in.w_shape}) : f.reals(W, {r.n_out, in.n_in, in.w_shape});
+      in.norm = f.real_or(name + "_reduce_" + source + "_norm", 1.0);
+      long picked = 0;
+      in.collect_ind = f.indices(name + "_collect_ind_" + source, {Ext::any(picked)}, kSizeLimit);    // range: checked against the plan
+      in.w_l_tile = f.indices(name + "_w_l_tile_" + source, {picked}, in.w_shape);
+      in.total_sum_ind = f.indices(name + "_total_sum_ind_" + source, {picked}, r.nfo());
+      r.instr.push_back(std::move(in));
+    }
+    if (f.present(name + "_norm_map")) r.norm_map = f.reals(name + "_norm_map", Flat{r.nfo()});
+    return r;
+  }
+  static Fc read_right_fc(const FileReader &f, const std::string &name)
+  {
+    Fc c;
+    c.name = name;
+    const std::string p = "fc_" + name;
+    c.n_out = (int) f.whole(p + "_n_out", 1, kSizeLimit);
+    f.must_be(p + "_left_coefs", 0, 0, "the FC layers of the three-layer architecture carry weights on their right input only");
+    long in_right = 0, tiles = 0, functions = 0, links = 0;
+    c.w_right = f.reals(p + "_w_right", {c.n_out, Ext::any(in_right), Ext::any(tiles)});
+    c.norm_right = f.real_or(p + "_norm_right", 1.0);
+    (void) f.indices(p + "_w_tile_left", {Ext::any(functions)}, kSizeLimit);
+    c.norm_out_factor = f.reals(p + "_norm_out_factor", Flat{functions});
+    c.collect_from = f.indices(p + "_collect_from", {Ext::any(links)}, kSizeLimit);    // range: checked against the plan
+    c.collect_to = f.indices(p + "_collect_to", {links}, functions);
+    c.w_tile_right = f.indices(p + "_w_tile_right", {links}, tiles);
+    c.n_in_right = (int) in_right;
+    c.w_shape_right = (int) tiles;
+    c.n_funcs_left = (int) functions;
+    return c;
+  }
+  static EqNorm read_eqnorm(const FileReader &f, const std::string &name)
+  {
+    EqNorm e;
+    e.name = name;
+    long groups = 0, width = 0, functions = 0;
+    e.affine_weight = f.reals(name + "_affine_weight", {Ext::any(groups), Ext::any(width)});
+    e.degree_weights = f.reals(name + "_degree_weights", {Ext::any(functions)});
+    e.l0_mask = f.reals(name + "_l0_mask", Flat{functions});
+    e.expand_index = f.indices(name + "_expand_index", {functions}, groups);
+    e.eps = f.real_or(name + "_eps", 1e-8);
+    if (e.eps < 0.0) f.reject(name + "_eps", "is negative; it is added to a mean square");
+    e.center_l0 = f.flag_or(name + "_center_l0", true);
+    e.n_groups = (int) groups;
+    e.n_out = (int) width;
+    e.M = (int) functions;
+    return e;
+  }
+  static RmsNorm read_rmsnorm(const FileReader &f, const std::string &name)
+  {
+    RmsNorm r;
+    r.name = name;
+    r.type = f.flag_or(name + "_type", false) ? 1 : 0;    // 1: the linear channel 0 is left out
+    long scaled = 0;
+    r.scale = f.reals(name + "_scale", {Ext::any(scaled)});
+    r.n_out = (int) f.whole_or(name + "_n_out", 1, kSizeLimit, scaled + r.type);
+    if (r.n_out - r.type != scaled)
+      f.reject(name + "_scale", "holds " + std::to_string(scaled) + " values, expected " + std::to_string(r.n_out - r.type) + " for " + std::to_string(r.n_out) + " channels");
+    return r;
+  }
+
+  // ---- the architecture ---------------------------------------------------------------------------------------
+  // One row per component of a layer, in evaluation order.  '#' in a name stands for the layer number, "X" for the
+  // layer's basis functions: the SPBF output A1 in layer 1, its projection A#_red in layers 2 and 3.
+  enum class Part { Basis, Project, Couple, MixRight, MessageNorm, DensityNorm };
+  struct PlanRow {
+    Part part;
+    const char *name;
+    const char *in[4];     // inputs (Couple, MixRight: left, right; Project: up to four sources)
+    int first, last;       // layers that have the row
+  };
+  static const std::vector<PlanRow> &layer_plan()
+  {
+    static const std::vector<PlanRow> kLayerPlan = {
+        {Part::Basis, "A#", {}, 1, 3},
+        {Part::Project, "A#_red", {"A#"}, 2, 3},
+        {Part::Couple, "A#_2", {"X", "X"}, 1, 3},
+        {Part::Project, "A#_2_red", {"A#_2"}, 1, 3},
+        {Part::MixRight, "A#_2a", {"A#_2_red", "X"}, 1, 3},
+        {Part::Couple, "A#_3", {"A#_2a", "X"}, 1, 3},
+        {Part::Project, "A#_3_red", {"A#_3"}, 1, 3},
+        {Part::MixRight, "A#_2b", {"A#_2_red", "X"}, 1, 3},
+        {Part::Couple, "A#_4", {"A#_2b", "A#_2b"}, 1, 3},
+        {Part::Project, "A#_4_red", {"A#_4"}, 1, 3},
+        {Part::Project, "eq#", {"X", "A#_2_red", "A#_3_red", "A#_4_red"}, 1, 2},
+        {Part::MessageNorm, "eq#_norm", {"eq#"}, 1, 2},
+        {Part::Project, "rho#", {"X", "A#_2_red", "A#_3_red", "A#_4_red"}, 1, 3},
+        {Part::DensityNorm, "rho#_norm", {"rho#"}, 1, 3},
+    };
+    return kLayerPlan;
+  }
+  struct Extent2 {
+    long functions, channels;
+  };
+  // Walks the plan: every row must be in the file's inventory exactly once, sized for the tensors its inputs produce; and
+  // the inventories must hold nothing else.  Returns the channel width of the normalised densities.
+  long check_against_plan(const FileReader &f) const
+  {
+    std::map<std::string, Extent2> made;       // tensors produced so far
+    std::set<std::string> visited;             // "<inventory>/<name>"
+    auto locate = [&](const auto &inventory, const char *list, const std::string &name) {
+      long hits = 0, at = -1;
+      for (size_t k = 0; k < inventory.size(); k++)
+        if (inventory[k].name == name) { hits++; at = (long) k; }
+      if (hits == 0) f.reject(list, "does not list '" + name + "', which the three-layer architecture needs");
+      if (hits > 1) f.reject(list, "lists '" + name + "' " + std::to_string(hits) + " times");
+      visited.insert(std::string(list) + "/" + name);
+      return (size_t) at;
+    };
+    auto same = [&](const std::string &key, long have, long want, const std::string &of) {
+      if (have != want) f.reject(key, "is sized for " + std::to_string(have) + " where " + of + " gives " + std::to_string(want));
+    };
+    if (spbf.size() != 3) f.reject("spbf_names", "lists " + std::to_string(spbf.size()) + " layers; the architecture has three (A1, A2, A3)");
+    for (int layer = 1; layer <= 3; layer++) {
+      const std::string number = std::to_string(layer);
+      auto spell = [&](const char *pattern) {
+        std::string s = pattern ? pattern : "";
+        if (s == "X") s = layer == 1 ? "A#" : "A#_red";
+        for (size_t at; (at = s.find('#')) != std::string::npos;) s.replace(at, 1, number);
+        return s;
+      };
+      for (const PlanRow &row : layer_plan()) {
+        if (layer < row.first || layer > row.last) continue;
+        const std::string name = spell(row.name);
+        std::vector<std::string> inputs;
+        for (const char *in : row.in)
+          if (in) inputs.push_back(spell(in));
+        switch (row.part) {
+        case Part::Basis: {
+          const size_t at = locate(spbf, "spbf_names", name);
+          if (at != (size_t) layer - 1) f.reject("spbf_names", "must list the layers in the order A1, A2, A3");
+          const Spbf &s = spbf[at];
+          if (layer == 1) {
+            if (s.equivariant) f.reject(name + "_equivariant", "is 1, expected 0: the first layer has no message to gather");
+            made[name] = {nlm(), s.n_rad_max};
+          } else {
+            if (!s.equivariant) f.reject(name + "_equivariant", "is 0, expected 1: the layer gathers the message of the layer before");
+            const std::string message = "eq" + std::to_string(layer - 1) + "_norm";
+            same(name + "_n_lm_ind", s.n_lm_ind, made.at(message).functions, "the message " + message);
+            same(name + "_n_rad_max", s.n_rad_max, made.at(message).channels, "the message " + message);
+            made[name] = {s.nfunc, s.n_rad_max};
+          }
+          break;
+        }
+        case Part::Project: {
+          const Reduce &r = reduce[locate(reduce, "reduce_names", name)];
+          std::multiset<std::string> have, want(inputs.begin(), inputs.end());
+          for (const Instr &in : r.instr) have.insert(in.name);
+          if (have != want) f.reject(name + "_instruction_names", "must name exactly the inputs the architecture gives " + name);
+          for (const Instr &in : r.instr) {
+            const Extent2 src = made.at(in.name);
+            same(name + "_n_in_" + in.name, in.n_in, src.channels, "the channel width of " + in.name);
+            for (size_t q = 0; q < in.collect_ind.size(); q++)
+              if (in.collect_ind[q] >= src.functions)
+                f.reject(name + "_collect_ind_" + in.name, "[" + std::to_string(q) + "] = " + std::to_string(in.collect_ind[q]) + " points outside the " +
+                                                                 std::to_string(src.functions) + " functions of " + in.name);
+          }
+          made[name] = {r.nfo(), r.n_out};
+          break;
+        }
+        case Part::Couple: {
+          const Cpl &c = prod[locate(prod, "prod_names", name)];
+          const Extent2 l = made.at(inputs[0]), r = made.at(inputs[1]);
+          same(name + "_group_left", (long) c.group_left.size(), l.functions, "the function count of " + inputs[0]);
+          same(name + "_n_left", c.n_left, l.channels, "the channel width of " + inputs[0]);
+          same(name + "_group_right", (long) c.group_right.size(), r.functions, "the function count of " + inputs[1]);
+          same(name + "_n_right", c.n_right, r.channels, "the channel width of " + inputs[1]);
+          made[name] = {c.nfunc, c.rank};
+          break;
+        }
+        case Part::MixRight: {
+          const Fc &c = fc[locate(fc, "fc_names", name)];
+          const Extent2 l = made.at(inputs[0]), r = made.at(inputs[1]);
+          same("fc_" + name + "_w_tile_left", c.n_funcs_left, l.functions, "the function count of " + inputs[0]);
+          same("fc_" + name + "_n_out", c.n_out, l.channels, "the channel width of " + inputs[0]);
+          same("fc_" + name + "_w_right", c.n_in_right, r.channels, "the channel width of " + inputs[1]);
+          for (size_t q = 0; q < c.collect_from.size(); q++)
+            if (c.collect_from[q] >= r.functions)
+              f.reject("fc_" + name + "_collect_from", "[" + std::to_string(q) + "] = " + std::to_string(c.collect_from[q]) + " points outside the " +
+                                                           std::to_string(r.functions) + " functions of " + inputs[1]);
+          made[name] = {c.n_funcs_left, c.n_out};
+          break;
+        }
+        case Part::MessageNorm: {
+          const EqNorm &e = eqnorm[locate(eqnorm, "eqnorm_names", name)];
+          const Extent2 src = made.at(inputs[0]);
+          same(name + "_degree_weights", e.M, src.functions, "the function count of " + inputs[0]);
+          same(name + "_affine_weight", e.n_out, src.channels, "the channel width of " + inputs[0]);
+          made[name] = {e.M, e.n_out};
+          break;
+        }
+        case Part::DensityNorm: {
+          const RmsNorm &n = rmsnorm[locate(rmsnorm, "rmsnorm_names", name)];
+          const Extent2 src = made.at(inputs[0]);
+          same(name + "_n_out", n.n_out, src.channels, "the channel width of " + inputs[0]);
+          made[name] = {src.functions, n.n_out};
+          break;
+        }
+        }
+      }
+    }
+    auto nothing_else = [&](const auto &inventory, const char *list) {
+      for (const auto &x : inventory)
+        if (!visited.count(std::string(list) + "/" + x.name)) f.reject(list, "lists '" + x.name + "', which the three-layer architecture does not contain");
+    };
+    nothing_else(spbf, "spbf_names");
+    nothing_else(prod, "prod_names");
+    nothing_else(reduce, "reduce_names");
+    nothing_else(fc, "fc_names");
+    nothing_else(eqnorm, "eqnorm_names");
+    nothing_else(rmsnorm, "rmsnorm_names");
+    const long width = made.at("rho1_norm").channels;
+    for (const char *rho : {"rho2_norm", "rho3_norm"}) same(std::string(rho) + "_n_out", made.at(rho).channels, width, "rho1_norm");
+    return width;
   }
 };
 

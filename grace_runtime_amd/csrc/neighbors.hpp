@@ -1,13 +1,19 @@
-// Host neighbour list that reproduces the reference list bond for bond (same permutation, CSR rows, (j, image)
-// order and shift table): fractional-coordinate binning with bin edge >= cutoff / 2, stable counting sort by bin,
-// per atom the bins in lexicographic offset order and inside a bin by slot.  Algorithm of
-// libgrace/include/grace/cell_list.h:39-152,216-241 and python/src/neighbors.cpp:15-95; the floating-point
-// expressions are written in the same operation order so that the r^2 < rc^2 decisions agree bit for bit.
+// Host neighbour list: the list the reference's search returns (python/src/neighbors.cpp:15-95 over the cell list of
+// libgrace/include/grace/cell_list.h:39-152), bond for bond: the same permutation (atoms in bin order, a bin's atoms in
+// input order), the same rows (bins in ascending offset order, a bin's atoms by slot), the same shift table (distinct
+// image differences in ascending order).
+//
+// Layout of this implementation: a Frame (cell, inverse, plane spacings), a Grid (bins per direction and the map atom ->
+// bin), and a search in which every thread walks a contiguous range of slots ONCE, appending (neighbour, image key) pairs
+// to its own arrays; rows are then laid out by prefix sums and the image keys are ranked.  Only the floating-point
+// expressions that decide a result are fixed by the reference and keep its operation order: the fractional coordinate,
+// the bin index, the wrapped position and the squared distance (marked "order matters" below).
 #pragma once
 
 #include "npz.hpp"
 
 #include <algorithm>
+#include <array>
 #include <cmath>
 #include <cstdint>
 #include <vector>
@@ -24,217 +30,283 @@ struct NeighborList {
   std::vector<double> shifts;
 };
 
-namespace nl_detail {
-inline int64_t floordiv(int64_t a, int64_t b) { return a >= 0 ? a / b : -((-a + b - 1) / b); }
-inline int64_t bin_reach(double rc, double w, int64_t nbin, bool pbc)
-{
-  const int64_t r = (int64_t) std::ceil(rc / w - 1e-12);
-  return pbc ? r : std::min(r, nbin - 1);
-}
+namespace nl {
 
-struct Cells {
-  int64_t n = 0;
-  double cell[9];
-  bool pbc[3];
-  int64_t nbin[3] = {1, 1, 1};
-  double width[3] = {1, 1, 1};
-  std::vector<int64_t> perm, start, b3, img;
-  std::vector<double> xw;
+constexpr int64_t kFarImages = int64_t(1) << 20;    // image differences must stay below this in every direction
 
-  void build(const double *pos, int64_t n_, const double *cell_, const bool *pbc_, double bin_size)
+// The periodic frame: rows of `a` are the cell vectors, columns of `inv` the reciprocal ones, `gap[k]` the distance
+// between the lattice planes normal to reciprocal vector k.
+struct Frame {
+  double a[9], inv[9], gap[3];
+  bool periodic[3];
+
+  Frame(const double *cell, const bool *pbc)
   {
-    n = n_;
-    for (int k = 0; k < 9; k++) cell[k] = cell_[k];
-    for (int k = 0; k < 3; k++) pbc[k] = pbc_[k];
-    perm.assign(n, 0);
-    xw.assign(3 * n, 0.0);
-    b3.assign(3 * n, 0);
-    img.assign(3 * n, 0);
-    const double *a = cell;
-    const double det = a[0] * (a[4] * a[8] - a[5] * a[7]) - a[1] * (a[3] * a[8] - a[5] * a[6]) + a[2] * (a[3] * a[7] - a[4] * a[6]);
-    {
-      const double na = std::sqrt(a[0] * a[0] + a[1] * a[1] + a[2] * a[2]);
-      const double nb = std::sqrt(a[3] * a[3] + a[4] * a[4] + a[5] * a[5]);
-      const double nc = std::sqrt(a[6] * a[6] + a[7] * a[7] + a[8] * a[8]);
-      if (!std::isfinite(det) || !(std::abs(det) > 1e-12 * na * nb * nc))
-        throw InvalidArgument("neighbour search needs a full-rank cell");
+    for (int k = 0; k < 9; k++) a[k] = cell[k];
+    for (int k = 0; k < 3; k++) periodic[k] = pbc[k];
+    const double c00 = a[4] * a[8] - a[5] * a[7], c01 = a[3] * a[8] - a[5] * a[6], c02 = a[3] * a[7] - a[4] * a[6];
+    const double volume = a[0] * c00 - a[1] * c01 + a[2] * c02;    // order matters (threshold below, and 1 / volume)
+    double edge[3];
+    for (int k = 0; k < 3; k++) edge[k] = std::sqrt(a[3 * k] * a[3 * k] + a[3 * k + 1] * a[3 * k + 1] + a[3 * k + 2] * a[3 * k + 2]);
+    if (!std::isfinite(volume) || !(std::abs(volume) > 1e-12 * edge[0] * edge[1] * edge[2]))
+      throw InvalidArgument("the neighbour search needs three linearly independent cell vectors (a full-rank cell)");
+    const double s = 1.0 / volume;
+    // adjugate times 1 / volume, element by element: order matters (fractional coordinates)
+    inv[0] = c00 * s;
+    inv[1] = (a[2] * a[7] - a[1] * a[8]) * s;
+    inv[2] = (a[1] * a[5] - a[2] * a[4]) * s;
+    inv[3] = (a[5] * a[6] - a[3] * a[8]) * s;
+    inv[4] = (a[0] * a[8] - a[2] * a[6]) * s;
+    inv[5] = (a[2] * a[3] - a[0] * a[5]) * s;
+    inv[6] = c02 * s;
+    inv[7] = (a[1] * a[6] - a[0] * a[7]) * s;
+    inv[8] = (a[0] * a[4] - a[1] * a[3]) * s;
+    for (int k = 0; k < 3; k++) gap[k] = 1.0 / std::sqrt(inv[k] * inv[k] + inv[3 + k] * inv[3 + k] + inv[6 + k] * inv[6 + k]);
+  }
+  // order matters
+  double fractional(const double *x, int k) const { return x[0] * inv[k] + x[1] * inv[3 + k] + x[2] * inv[6 + k]; }
+  double cartesian(const double *u, int d) const { return u[0] * a[d] + u[1] * a[3 + d] + u[2] * a[6 + d]; }
+  double image_shift(int64_t s0, int64_t s1, int64_t s2, int d) const { return s0 * a[d] + s1 * a[3 + d] + s2 * a[6 + d]; }
+};
+
+// Bins of edge >= bin_edge along every direction over the span of the fractional coordinates (the whole cell along
+// periodic directions, the occupied range along open ones), at most 8 n + 64 bins in all.
+struct Grid {
+  int64_t count[3] = {1, 1, 1};
+  double origin[3] = {0.0, 0.0, 0.0}, extent[3] = {1.0, 1.0, 1.0}, width[3] = {1.0, 1.0, 1.0};
+
+  void choose(const Frame &fr, const std::vector<double> &u, int64_t n, double bin_edge)
+  {
+    double low[3], high[3];
+    for (int k = 0; k < 3; k++) {
+      low[k] = high[k] = u[k];
+      for (int64_t i = 1; i < n; i++) {
+        low[k] = std::min(low[k], u[3 * i + k]);
+        high[k] = std::max(high[k], u[3 * i + k]);
+      }
     }
-    const double d = 1.0 / det;
-    const double inv[9] = {(a[4] * a[8] - a[5] * a[7]) * d, (a[2] * a[7] - a[1] * a[8]) * d, (a[1] * a[5] - a[2] * a[4]) * d,
-                           (a[5] * a[6] - a[3] * a[8]) * d, (a[0] * a[8] - a[2] * a[6]) * d, (a[2] * a[3] - a[0] * a[5]) * d,
-                           (a[3] * a[7] - a[4] * a[6]) * d, (a[1] * a[6] - a[0] * a[7]) * d, (a[0] * a[4] - a[1] * a[3]) * d};
-    double h[3], lo[3] = {0, 0, 0}, span[3] = {1, 1, 1};
-    for (int k = 0; k < 3; k++) h[k] = 1.0 / std::sqrt(inv[k] * inv[k] + inv[3 + k] * inv[3 + k] + inv[6 + k] * inv[6 + k]);
-    std::vector<double> frac(3 * n);
+    choose(fr, low, high, n, bin_edge);
+  }
+  // low / high: smallest and largest fractional coordinate of the atoms per direction (used along open directions)
+  void choose(const Frame &fr, const double *low, const double *high, int64_t n, double bin_edge)
+  {
+    for (int k = 0; k < 3; k++) {
+      if (fr.periodic[k]) continue;
+      origin[k] = low[k];
+      extent[k] = std::max(high[k] - low[k], 1e-12);
+    }
+    const double budget = (double) (8 * n + 64);
+    for (int k = 0; k < 3; k++) count[k] = (int64_t) std::min(std::max(std::floor(extent[k] * fr.gap[k] / bin_edge), 1.0), budget);    // order matters
+    while ((double) count[0] * (double) count[1] * (double) count[2] > budget) {
+      int widest = 0;
+      for (int k = 1; k < 3; k++)
+        if (count[k] > count[widest]) widest = k;
+      count[widest] = std::max<int64_t>(1, count[widest] / 2);
+    }
+    for (int k = 0; k < 3; k++) width[k] = extent[k] * fr.gap[k] / (double) count[k];
+  }
+  int64_t total() const { return count[0] * count[1] * count[2]; }
+  int64_t along(double u, int k) const    // order matters
+  {
+    const int64_t b = (int64_t) std::floor((u - origin[k]) / extent[k] * (double) count[k]);
+    return std::min(std::max<int64_t>(b, 0), count[k] - 1);
+  }
+  // bins to visit on either side so that nothing within `cutoff` is missed
+  int64_t reach(double cutoff, int k, bool periodic) const
+  {
+    const int64_t r = (int64_t) std::ceil(cutoff / width[k] - 1e-12);
+    return periodic ? r : std::min(r, count[k] - 1);
+  }
+};
+
+// The atoms sorted into bins: slot q holds atom perm[q]; per slot the wrapped Cartesian position, the bin triple and the
+// image the atom was wrapped by.
+struct Binned {
+  Frame frame;
+  Grid grid;
+  int64_t n = 0;
+  std::vector<int64_t> perm, first;     // first[b] .. first[b + 1]: slots of bin b
+  std::vector<double> x;                // [n][3] wrapped positions by slot
+  std::vector<int32_t> bin3, wrap3;     // [n][3] by slot
+
+  Binned(const double *pos, int64_t n_, const double *cell, const bool *pbc, double bin_edge) : frame(cell, pbc), n(n_)
+  {
+    std::vector<double> u((size_t) 3 * n);
+    std::vector<int64_t> wrapped((size_t) 3 * n);
     for (int64_t i = 0; i < n; i++)
       for (int k = 0; k < 3; k++) {
-        const double f = pos[3 * i] * inv[k] + pos[3 * i + 1] * inv[3 + k] + pos[3 * i + 2] * inv[6 + k];
-        if (!std::isfinite(f)) throw InvalidArgument("positions must be finite");
-        const double fl = pbc[k] ? std::floor(f) : 0.0;
-        img[3 * i + k] = (int64_t) fl;
-        frac[3 * i + k] = f - fl;
+        const double f = frame.fractional(pos + 3 * i, k);
+        if (!std::isfinite(f)) throw InvalidArgument("atom " + std::to_string(i) + " has a position that is not finite");
+        const double whole = frame.periodic[k] ? std::floor(f) : 0.0;
+        wrapped[3 * i + k] = (int64_t) whole;
+        u[3 * i + k] = f - whole;
       }
-    for (int k = 0; k < 3; k++)
-      if (!pbc[k]) {
-        double mn = frac[k], mx = frac[k];
-        for (int64_t i = 1; i < n; i++) {
-          mn = std::min(mn, frac[3 * i + k]);
-          mx = std::max(mx, frac[3 * i + k]);
-        }
-        lo[k] = mn;
-        span[k] = std::max(mx - mn, 1e-12);
-      }
-    const int64_t max_bins = 8 * n + 64;
-    for (int k = 0; k < 3; k++) {
-      const double nb = std::floor(span[k] * h[k] / bin_size);
-      nbin[k] = (int64_t) std::min<double>(std::max(nb, 1.0), (double) max_bins);
-    }
-    while ((double) nbin[0] * (double) nbin[1] * (double) nbin[2] > (double) max_bins) {
-      const int k = (int) (std::max_element(nbin, nbin + 3) - nbin);
-      nbin[k] = std::max<int64_t>(1, nbin[k] / 2);
-    }
-    for (int k = 0; k < 3; k++) width[k] = span[k] * h[k] / (double) nbin[k];
-    const int64_t nbt = nbin[0] * nbin[1] * nbin[2];
-    std::vector<int64_t> bin(n);
-    start.assign(nbt + 1, 0);
+    grid.choose(frame, u, n, bin_edge);
+    // counting sort by bin, atoms of a bin in input order
+    std::vector<int64_t> bin_of((size_t) n);
+    first.assign((size_t) grid.total() + 1, 0);
     for (int64_t i = 0; i < n; i++) {
+      bin_of[i] = (grid.along(u[3 * i], 0) * grid.count[1] + grid.along(u[3 * i + 1], 1)) * grid.count[2] + grid.along(u[3 * i + 2], 2);
+      first[bin_of[i] + 1]++;
+    }
+    for (size_t b = 1; b < first.size(); b++) first[b] += first[b - 1];
+    std::vector<int64_t> cursor(first.begin(), first.end() - 1);
+    perm.resize((size_t) n);
+    x.resize((size_t) 3 * n);
+    bin3.resize((size_t) 3 * n);
+    wrap3.resize((size_t) 3 * n);
+    for (int64_t i = 0; i < n; i++) {
+      const int64_t q = cursor[bin_of[i]]++;
+      perm[q] = i;
       for (int k = 0; k < 3; k++) {
-        const int64_t b = (int64_t) std::floor((frac[3 * i + k] - lo[k]) / span[k] * (double) nbin[k]);
-        b3[3 * i + k] = std::min(std::max<int64_t>(b, 0), nbin[k] - 1);
+        if (std::abs(wrapped[3 * i + k]) >= (int64_t(1) << 30)) throw InvalidArgument("atoms a million cells or more from the cell: wrap the positions first");
+        x[3 * q + k] = frame.cartesian(&u[3 * i], k);
+        bin3[3 * q + k] = (int32_t) grid.along(u[3 * i + k], k);
+        wrap3[3 * q + k] = (int32_t) wrapped[3 * i + k];
       }
-      bin[i] = (b3[3 * i] * nbin[1] + b3[3 * i + 1]) * nbin[2] + b3[3 * i + 2];
-      start[bin[i] + 1]++;
-    }
-    for (int64_t b = 0; b < nbt; b++) start[b + 1] += start[b];
-    std::vector<int64_t> fill(start.begin(), start.end() - 1);
-    for (int64_t i = 0; i < n; i++) {
-      const int64_t s = fill[bin[i]]++;
-      perm[s] = i;
-      for (int dd = 0; dd < 3; dd++)
-        xw[3 * s + dd] = frac[3 * i] * cell[dd] + frac[3 * i + 1] * cell[3 + dd] + frac[3 * i + 2] * cell[6 + dd];
     }
   }
 
-  // fn(p, s0, s1, s2) for every neighbour slot p of slot q within rc, images S in the wrapped frame
-  template<class F> void visit(int64_t q, double rc, F &&fn) const
+  // One direction of the walk over neighbouring bins: the bins at offsets -reach .. reach of bin b, folded back into
+  // the grid along a periodic direction (with the image they lie in) and clipped along an open one.
+  struct Step {
+    int64_t bin, image;
+    bool home;
+  };
+  void steps(int k, int64_t b, int64_t reach, std::vector<Step> &out) const
   {
-    const double rc2 = rc * rc;
-    const double *xq = &xw[3 * q];
-    int64_t reach[3];
-    for (int k = 0; k < 3; k++) reach[k] = bin_reach(rc, width[k], nbin[k], pbc[k]);
-    const int64_t *bq = &b3[3 * perm[q]];
-    for (int64_t o0 = -reach[0]; o0 <= reach[0]; o0++) {
-      int64_t c0 = bq[0] + o0, s0 = 0;
-      if (pbc[0]) { s0 = floordiv(c0, nbin[0]); c0 -= s0 * nbin[0]; }
-      else if (c0 < 0 || c0 >= nbin[0]) continue;
-      for (int64_t o1 = -reach[1]; o1 <= reach[1]; o1++) {
-        int64_t c1 = bq[1] + o1, s1 = 0;
-        if (pbc[1]) { s1 = floordiv(c1, nbin[1]); c1 -= s1 * nbin[1]; }
-        else if (c1 < 0 || c1 >= nbin[1]) continue;
-        for (int64_t o2 = -reach[2]; o2 <= reach[2]; o2++) {
-          int64_t c2 = bq[2] + o2, s2 = 0;
-          if (pbc[2]) { s2 = floordiv(c2, nbin[2]); c2 -= s2 * nbin[2]; }
-          else if (c2 < 0 || c2 >= nbin[2]) continue;
-          const int64_t c = (c0 * nbin[1] + c1) * nbin[2] + c2;
-          const double sx = s0 * cell[0] + s1 * cell[3] + s2 * cell[6];
-          const double sy = s0 * cell[1] + s1 * cell[4] + s2 * cell[7];
-          const double sz = s0 * cell[2] + s1 * cell[5] + s2 * cell[8];
-          const bool own = o0 == 0 && o1 == 0 && o2 == 0;
-          for (int64_t p = start[c]; p < start[c + 1]; p++) {
-            if (own && p == q) continue;
-            const double dx = xw[3 * p] + sx - xq[0];
-            const double dy = xw[3 * p + 1] + sy - xq[1];
-            const double dz = xw[3 * p + 2] + sz - xq[2];
-            const double r2 = dx * dx + dy * dy + dz * dz;
-            if (r2 < rc2) fn(p, s0, s1, s2);
-          }
-        }
+    out.clear();
+    const int64_t m = grid.count[k];
+    for (int64_t o = -reach; o <= reach; o++) {
+      int64_t c = b + o, s = 0;
+      if (frame.periodic[k]) {
+        s = c >= 0 ? c / m : -((m - 1 - c) / m);    // floor division
+        c -= s * m;
+      } else if (c < 0 || c >= m) {
+        continue;
       }
+      out.push_back({c, s, o == 0});
     }
   }
 };
-}    // namespace nl_detail
+
+inline int64_t pack_image(int64_t t0, int64_t t1, int64_t t2)
+{
+  return ((t0 + kFarImages) << 42) | ((t1 + kFarImages) << 21) | (t2 + kFarImages);
+}
+inline void unpack_image(int64_t key, int64_t t[3])
+{
+  const int64_t mask = (int64_t(1) << 21) - 1;
+  t[0] = ((key >> 42) & mask) - kFarImages;
+  t[1] = ((key >> 21) & mask) - kFarImages;
+  t[2] = (key & mask) - kFarImages;
+}
+// row of the shift table for an image difference: t0 a + t1 b + t2 c accumulated with fused multiply-adds from the
+// first term on, the form the reference's optimised build evaluates, so that the table agrees to the last bit
+inline void shift_row(const double *cell, const int64_t t[3], double *out)
+{
+  for (int d = 0; d < 3; d++) out[d] = std::fma((double) t[2], cell[6 + d], std::fma((double) t[1], cell[3 + d], (double) t[0] * cell[d]));
+}
+
+}    // namespace nl
 
 inline NeighborList neighbor_search(const double *pos, int64_t n, const double *cell, const bool *pbc, double cutoff, int nthreads)
 {
-  using namespace nl_detail;
-  if (!(cutoff > 0.0) || !std::isfinite(cutoff)) throw InvalidArgument("cutoff must be positive");
-  if (n < 0 || n >= INT32_MAX) throw InvalidArgument("atom count out of range");
-  NeighborList r;
-  r.offset.assign(n + 1, 0);
-  if (n == 0) return r;
-  Cells cl;
-  cl.build(pos, n, cell, pbc, 0.5 * cutoff);
-  r.perm = cl.perm;
-  constexpr int64_t kB = int64_t(1) << 20;
-  bool far = false;
-  auto key = [&](int64_t a, int64_t b, int64_t s0, int64_t s1, int64_t s2, bool &far_) {
-    const int64_t *ia = &cl.img[3 * a], *ib = &cl.img[3 * b];
-    const int64_t t0 = s0 - ib[0] + ia[0], t1 = s1 - ib[1] + ia[1], t2 = s2 - ib[2] + ia[2];
-    if (std::max({std::abs(t0), std::abs(t1), std::abs(t2)}) >= kB) {
-      far_ = true;
-      return int64_t(0);
-    }
-    return ((t0 + kB) << 42) | ((t1 + kB) << 21) | (t2 + kB);
+  if (!(cutoff > 0.0) || !std::isfinite(cutoff)) throw InvalidArgument("the neighbour search needs a cutoff: cutoff must be positive and finite");
+  if (n < 0 || n >= INT32_MAX) throw InvalidArgument("the neighbour search handles fewer than 2^31 atoms");
+  NeighborList out;
+  out.offset.assign((size_t) n + 1, 0);
+  if (n == 0) return out;
+  const nl::Binned B(pos, n, cell, pbc, 0.5 * cutoff);
+  out.perm = B.perm;
+  const double cut2 = cutoff * cutoff;
+  int64_t reach[3];
+  for (int k = 0; k < 3; k++) reach[k] = B.grid.reach(cutoff, k, B.frame.periodic[k]);
+
+  // every thread owns a contiguous range of slots and collects their rows in its own arrays
+  const int threads = (int) std::max<int64_t>(1, std::min<int64_t>(nthreads, (n + 255) / 256));
+  struct Part {
+    std::vector<int32_t> j;
+    std::vector<int64_t> key;
+    bool far = false;
   };
-  std::vector<int64_t> nn(n), keys;
-  const int nth = std::max(1, nthreads);
-#pragma omp parallel num_threads(nth)
+  std::vector<Part> part((size_t) threads);
+  std::vector<int64_t> row_len((size_t) n);
+#pragma omp parallel num_threads(threads)
   {
-    std::vector<int64_t> seen;
-    int64_t last = -1;
-    bool myfar = false;
-#pragma omp for schedule(dynamic, 64)
-    for (int64_t q = 0; q < n; q++) {
-      const int64_t a = r.perm[q];
-      int64_t c = 0;
-      cl.visit(q, cutoff, [&](int64_t p, int64_t s0, int64_t s1, int64_t s2) {
-        c++;
-        const int64_t k = key(a, r.perm[p], s0, s1, s2, myfar);
-        if (k != last) seen.push_back(last = k);
-      });
-      nn[q] = c;
-      if (seen.size() > 4096) {
-        std::sort(seen.begin(), seen.end());
-        seen.erase(std::unique(seen.begin(), seen.end()), seen.end());
-      }
-    }
-#pragma omp critical
-    {
-      keys.insert(keys.end(), seen.begin(), seen.end());
-      far = far || myfar;
+#ifdef _OPENMP
+    const int me = omp_get_thread_num(), team = omp_get_num_threads();
+#else
+    const int me = 0, team = 1;
+#endif
+    // with fewer threads than planned (team < threads) the ranges still cover every slot
+    Part &mine = part[(size_t) me];
+    std::vector<nl::Binned::Step> s0, s1, s2;
+    for (int64_t q = n * me / team; q < n * (me + 1) / team; q++) {
+      const double *xq = &B.x[3 * q];
+      const int32_t *wq = &B.wrap3[3 * q];
+      const size_t before = mine.j.size();
+      B.steps(0, B.bin3[3 * q], reach[0], s0);
+      B.steps(1, B.bin3[3 * q + 1], reach[1], s1);
+      B.steps(2, B.bin3[3 * q + 2], reach[2], s2);
+      for (const auto &a : s0)
+        for (const auto &b : s1)
+          for (const auto &c : s2) {
+            const int64_t bin = (a.bin * B.grid.count[1] + b.bin) * B.grid.count[2] + c.bin;
+            const double shift[3] = {B.frame.image_shift(a.image, b.image, c.image, 0), B.frame.image_shift(a.image, b.image, c.image, 1),
+                                     B.frame.image_shift(a.image, b.image, c.image, 2)};
+            const bool home = a.home && b.home && c.home;
+            for (int64_t p = B.first[bin]; p < B.first[bin + 1]; p++) {
+              if (home && p == q) continue;
+              // order matters: (x_p + shift) - x_q, then the sum of squares from the first term on
+              const double dx = B.x[3 * p] + shift[0] - xq[0], dy = B.x[3 * p + 1] + shift[1] - xq[1], dz = B.x[3 * p + 2] + shift[2] - xq[2];
+              const double d2 = dx * dx + dy * dy + dz * dz;
+              if (!(d2 < cut2)) continue;
+              // image of the bond in the caller's frame: both atoms un-wrapped
+              const int32_t *wp = &B.wrap3[3 * p];
+              const int64_t t0 = a.image - wp[0] + wq[0], t1 = b.image - wp[1] + wq[1], t2 = c.image - wp[2] + wq[2];
+              if (std::max({std::abs(t0), std::abs(t1), std::abs(t2)}) >= nl::kFarImages) mine.far = true;
+              mine.j.push_back((int32_t) p);
+              mine.key.push_back(nl::pack_image(t0, t1, t2));
+            }
+          }
+      row_len[q] = (int64_t) (mine.j.size() - before);
     }
   }
-  if (far) throw InvalidArgument("atoms a million cells or more apart: wrap the positions");
+  for (const Part &p : part)
+    if (p.far) throw InvalidArgument("atoms a million cells or more apart: wrap the positions first");
+
+  // rows: the parts are in slot order already
+  for (int64_t q = 0; q < n; q++) out.offset[q + 1] = out.offset[q] + row_len[q];
+  std::vector<int64_t> keys;
+  for (const Part &p : part) {
+    std::vector<int64_t> seen(p.key);
+    std::sort(seen.begin(), seen.end());
+    seen.erase(std::unique(seen.begin(), seen.end()), seen.end());
+    keys.insert(keys.end(), seen.begin(), seen.end());
+  }
   std::sort(keys.begin(), keys.end());
   keys.erase(std::unique(keys.begin(), keys.end()), keys.end());
-  r.shifts.resize(3 * keys.size());
-  for (size_t u = 0; u < keys.size(); u++) {
-    const int64_t m = (int64_t(1) << 21) - 1, k = keys[u];
-    const double t0 = (double) (((k >> 42) & m) - kB), t1 = (double) (((k >> 21) & m) - kB), t2 = (double) ((k & m) - kB);
-    // fused multiply-adds in the order an FMA-contracting compiler gives the reference's expression
-    // t0 a_d + t1 b_d + t2 c_d (the reference builds with -march=native), so that the table agrees to the bit
-    for (int d = 0; d < 3; d++) r.shifts[3 * u + d] = std::fma(t2, cell[6 + d], std::fma(t1, cell[3 + d], t0 * cell[d]));
+  out.shifts.resize(3 * keys.size());
+  for (size_t r = 0; r < keys.size(); r++) {
+    int64_t t[3];
+    nl::unpack_image(keys[r], t);
+    nl::shift_row(cell, t, &out.shifts[3 * r]);
   }
-  for (int64_t q = 0; q < n; q++) r.offset[q + 1] = r.offset[q] + nn[q];
-  const int64_t nb = r.offset[n];
-  r.j.resize(nb);
-  r.image.resize(nb);
-#pragma omp parallel for schedule(dynamic, 64) num_threads(nth)
-  for (int64_t q = 0; q < n; q++) {
-    int64_t w = r.offset[q], last = -1;
-    int32_t u = 0;
-    bool f2 = false;
-    const int64_t a = r.perm[q];
-    cl.visit(q, cutoff, [&](int64_t p, int64_t s0, int64_t s1, int64_t s2) {
-      const int64_t k = key(a, r.perm[p], s0, s1, s2, f2);
-      if (k != last) u = (int32_t) (std::lower_bound(keys.begin(), keys.end(), last = k) - keys.begin());
-      r.j[w] = (int32_t) p;
-      r.image[w] = u;
-      w++;
-    });
+  out.j.resize((size_t) out.offset[n]);
+  out.image.resize((size_t) out.offset[n]);
+  size_t at = 0;
+  for (const Part &p : part) {
+    std::copy(p.j.begin(), p.j.end(), out.j.begin() + (std::ptrdiff_t) at);
+    int64_t last = -1;
+    int32_t rank = 0;
+    for (size_t w = 0; w < p.key.size(); w++) {
+      if (p.key[w] != last) rank = (int32_t) (std::lower_bound(keys.begin(), keys.end(), last = p.key[w]) - keys.begin());
+      out.image[at + w] = rank;
+    }
+    at += p.j.size();
   }
-  return r;
+  return out;
 }
 
 }    // namespace grhip

@@ -1,7 +1,7 @@
-// Reader for uncompressed .npz archives (numpy.savez) and typed accessors with the validation rules of the model
-// loaders.  Semantics follow the reference's private helpers (libgrace/src/npz3.h:22-330): every value is converted
-// by its stored dtype or rejected, Fortran-ordered multi-dimensional arrays, compressed members, big-endian data
-// and NaN/Inf are errors, a missing required array is an error naming it.
+// Reader for uncompressed .npz archives (numpy.savez): the ZIP directory and the .npy members, as raw bytes with their
+// dtype and shape.  Compressed members, big-endian data and dtypes other than float / int / bool / byte strings are
+// errors (the reference's reader, libgrace/src/npz3.h:22-58, accepts and refuses the same files).  Typed, validated
+// access to the members is schema.hpp.
 #pragma once
 
 #include <climits>
@@ -172,220 +172,6 @@ inline Npz npz_load(const std::string &path)
     out[name] = parse_npy(&buf[data], (size_t) usize, name);
   }
   return out;
-}
-
-// ---------------------------------------------------------------------------------------------------------------
-// typed access
-// ---------------------------------------------------------------------------------------------------------------
-constexpr int kMaxDim = 1 << 16;    // any size or count read from a file
-constexpr int kMaxL = 255;
-constexpr int kMaxP = 46339;
-
-inline Error bad_array(const std::string &key, const std::string &what)
-{
-  return Error("model array '" + key + "' " + what + "; re-export the model");
-}
-
-struct NpzView {
-  const Npz &z;
-  explicit NpzView(const Npz &z_) : z(z_) {}
-
-  bool has(const std::string &k) const { return z.count(k) != 0; }
-
-  const NpyArray *find(const std::string &key) const
-  {
-    auto it = z.find(key);
-    if (it == z.end()) return nullptr;
-    const NpyArray &a = it->second;
-    if (a.fortran) {
-      int dims = 0;
-      for (size_t d : a.shape) dims += d > 1;
-      if (dims > 1) throw Error("model array '" + key + "' is stored in Fortran order; re-export it in C order");
-    }
-    return &a;
-  }
-
-  static bool int_at(const NpyArray &a, size_t q, int64_t &v)
-  {
-    const bool u = a.kind == 'u';
-    switch (a.word) {
-    case 1: v = u ? (int64_t) a.as<uint8_t>()[q] : (int64_t) a.as<int8_t>()[q]; return true;
-    case 2: v = u ? (int64_t) a.as<uint16_t>()[q] : (int64_t) a.as<int16_t>()[q]; return true;
-    case 4: v = u ? (int64_t) a.as<uint32_t>()[q] : (int64_t) a.as<int32_t>()[q]; return true;
-    case 8:
-      if (!u) { v = a.as<int64_t>()[q]; return true; }
-      v = (int64_t) a.as<uint64_t>()[q];
-      return a.as<uint64_t>()[q] <= (uint64_t) INT64_MAX;
-    default: return false;
-    }
-  }
-  static bool is_int(const NpyArray &a) { return (a.kind == 'i' || a.kind == 'u') && (a.word == 1 || a.word == 2 || a.word == 4 || a.word == 8); }
-
-  std::vector<double> doubles(const std::string &key) const
-  {
-    const NpyArray *a = find(key);
-    if (!a) return {};
-    std::vector<double> v(a->count);
-    auto put = [&](size_t q, double x) {
-      if (!std::isfinite(x)) throw bad_array(key, "has a non-finite value (NaN / Inf) at " + std::to_string(q));
-      v[q] = x;
-    };
-    if (a->kind == 'f' && a->word == 4) for (size_t q = 0; q < v.size(); q++) put(q, a->as<float>()[q]);
-    else if (a->kind == 'f' && a->word == 8) for (size_t q = 0; q < v.size(); q++) put(q, a->as<double>()[q]);
-    else if (is_int(*a)) {
-      for (size_t q = 0; q < v.size(); q++) {
-        int64_t x;
-        if (!int_at(*a, q, x)) throw bad_array(key, "has dtype '" + a->descr + "', expected a float32 or float64 array");
-        v[q] = (double) x;
-      }
-    } else throw bad_array(key, "has dtype '" + a->descr + "', expected a float32 or float64 array");
-    return v;
-  }
-
-  std::vector<int> ints(const std::string &key) const
-  {
-    const NpyArray *a = find(key);
-    if (!a) return {};
-    std::vector<int> v(a->count);
-    if (a->kind == 'b' && a->word == 1) {
-      for (size_t q = 0; q < v.size(); q++) v[q] = a->as<uint8_t>()[q] != 0;
-      return v;
-    }
-    if (!is_int(*a)) throw bad_array(key, "has dtype '" + a->descr + "', expected an integer array");
-    for (size_t q = 0; q < v.size(); q++) {
-      int64_t x;
-      if (!int_at(*a, q, x) || x < INT_MIN || x > INT_MAX) throw bad_array(key, "has a value outside the range of int");
-      v[q] = (int) x;
-    }
-    return v;
-  }
-
-  void require_scalar(const std::string &key) const
-  {
-    auto it = z.find(key);
-    if (it != z.end() && it->second.count != 1)
-      throw bad_array(key, "has " + std::to_string(it->second.count) + " values, expected one");
-  }
-  int int_scalar(const std::string &key, int def = 0) const
-  {
-    require_scalar(key);
-    auto v = ints(key);
-    return v.empty() ? def : v[0];
-  }
-  double double_scalar(const std::string &key, double def = 0.0) const
-  {
-    require_scalar(key);
-    auto v = doubles(key);
-    return v.empty() ? def : v[0];
-  }
-  // an int scalar in [lo, hi]; def when absent (a def outside [lo, hi]: the key is required)
-  int int_in(const std::string &key, int def, int lo, int hi) const
-  {
-    if (!has(key) && (def < lo || def > hi)) throw bad_array(key, "is missing from the .npz file");
-    const int v = int_scalar(key, def);
-    if (v < lo || v > hi)
-      throw bad_array(key, "is " + std::to_string(v) + ", expected a value in [" + std::to_string(lo) + ", " + std::to_string(hi) + "]");
-    return v;
-  }
-  bool flag(const std::string &key, int def) const { return int_in(key, def, 0, 1) != 0; }
-
-  std::vector<double> require_doubles(const std::string &key) const
-  {
-    auto v = doubles(key);
-    if (v.empty())
-      throw Error("required weight '" + key + "' missing from the .npz file (an empty load would give zero forces); re-export the model");
-    return v;
-  }
-  std::vector<int> require_ints(const std::string &key) const
-  {
-    auto v = ints(key);
-    if (v.empty()) throw Error("required index array '" + key + "' missing from the .npz file; re-export the model");
-    return v;
-  }
-  std::vector<double> cutoffs(const std::string &key, const char *style) const
-  {
-    auto v = doubles(key);
-    for (double x : v)
-      if (x < 0.0) throw Error(std::string(style) + ": invalid cutoff in '" + key + "'");
-    return v;
-  }
-  double cutoff_scalar(const std::string &key, double def, const char *style) const
-  {
-    require_scalar(key);
-    auto v = cutoffs(key, style);
-    if (v.empty()) return def;
-    if (!(v[0] > 0.0)) throw Error(std::string(style) + ": cutoff '" + key + "' is not positive");
-    return v[0];
-  }
-  std::vector<std::string> names(const std::string &key) const
-  {
-    std::vector<std::string> out;
-    const NpyArray *a = find(key);
-    if (!a) return out;
-    if (a->kind != 'S' || a->shape.size() > 1) throw bad_array(key, "has dtype '" + a->descr + "', expected a 1-d byte-string array (|S)");
-    const size_t n = a->shape.empty() ? 0 : a->shape[0];
-    for (size_t i = 0; i < n; i++) {
-      std::string s((const char *) a->raw.data() + i * a->word, a->word);
-      while (!s.empty() && s.back() == '\0') s.pop_back();
-      out.push_back(s);
-    }
-    return out;
-  }
-  std::vector<size_t> shape(const std::string &key) const
-  {
-    auto it = z.find(key);
-    return it == z.end() ? std::vector<size_t>{} : it->second.shape;
-  }
-  static std::string dims_str(const std::vector<size_t> &d)
-  {
-    std::string o = "(";
-    for (size_t i = 0; i < d.size(); i++) o += (i ? ", " : "") + std::to_string(d[i]);
-    return o + ")";
-  }
-  std::vector<size_t> shape_rank(const std::string &key, size_t rank) const
-  {
-    const auto d = shape(key);
-    bool ok = d.size() == rank;
-    for (size_t x : d) ok = ok && x >= 1 && x <= (size_t) kMaxDim;
-    if (!ok) throw bad_array(key, "has shape " + dims_str(d) + ", expected " + std::to_string(rank) + " dimensions in [1, " + std::to_string(kMaxDim) + "]");
-    return d;
-  }
-  // the stored shape is exactly `want` (an absent key passes)
-  void require_shape(const std::string &key, const std::vector<int64_t> &want) const
-  {
-    const NpyArray *a = find(key);
-    if (!a) return;
-    bool ok = a->shape.size() == want.size();
-    for (size_t i = 0; ok && i < want.size(); i++) ok = want[i] >= 0 && a->shape[i] == (size_t) want[i];
-    if (!ok) {
-      std::vector<size_t> w;
-      std::string ws = "(";
-      for (size_t i = 0; i < want.size(); i++) ws += (i ? ", " : "") + std::to_string(want[i]);
-      throw bad_array(key, "has shape " + dims_str(a->shape) + ", expected " + ws + ")");
-    }
-  }
-};
-
-template<class V> inline void require_size(const std::string &key, const V &v, size_t n)
-{
-  if (v.size() != n) throw bad_array(key, "has " + std::to_string(v.size()) + " values, expected " + std::to_string(n));
-}
-inline void require_eq(const std::string &key, int64_t got, int64_t want, const std::string &why, const char *noun = nullptr)
-{
-  if (got != want)
-    throw bad_array(key, (noun ? "has " + std::to_string(got) + " " + noun : "is " + std::to_string(got)) + ", expected " + std::to_string(want) + " (" + why + ")");
-}
-inline void require_index(const std::string &key, const std::vector<int> &v, int64_t n)
-{
-  for (size_t q = 0; q < v.size(); q++)
-    if (v[q] < 0 || v[q] >= n)
-      throw bad_array(key, "has " + std::to_string(v[q]) + " at " + std::to_string(q) + ", outside [0, " + std::to_string(n) + ")");
-}
-inline int64_t index_extent(const std::vector<int> &v)
-{
-  int64_t m = 0;
-  for (int x : v) m = std::max<int64_t>(m, (int64_t) x + 1);
-  return m;
 }
 
 }    // namespace grhip

@@ -415,22 +415,41 @@ class Engine:
 
 
 def _padded_cell_arrays(cell, pos, reach, pbc=None):
-    """Zero cell vectors and the vectors of open directions replaced by vectors normal to the periodic ones, long
-    enough that no image is within reach, and the shift that puts the atoms inside that box
-    (python/grace_runtime/neighbors.py:27-47)."""
-    cell = np.array(cell, dtype=np.float64)
-    pad = [k for k in range(3) if not np.any(cell[k]) or (pbc is not None and not pbc[k])]
-    if not pad:
-        return cell, np.zeros(3)
-    given = np.array([cell[k] for k in range(3) if k not in pad]).reshape(-1, 3)
-    dirs = np.linalg.svd(given)[2][len(given):] if len(given) else np.eye(3)
-    shift = np.zeros(3)
-    for k, d in zip(pad, dirs):
-        proj = pos @ d
-        cell[k] = d * (np.ptp(proj) + 2.0 * reach + 1.0) if len(pos) else d * (2.0 * reach + 1.0)
+    """A full-rank box for a structure with open directions (what the reference does before its search,
+    python/grace_runtime/neighbors.py:27-47): every cell vector that is zero or whose direction is not periodic is replaced
+    by a unit normal to the remaining vectors, scaled to the extent of the atoms along it plus 2 * reach + 1, so that no
+    image lies within reach.  Returns the box and the translation that moves the atoms inside it.  The same construction as
+    the library uses for gr_compute / gr_system_compute."""
+    box = np.array(cell, dtype=np.float64).reshape(3, 3)
+    pos = np.asarray(pos, dtype=np.float64).reshape(-1, 3)
+    is_open = [not box[k].any() or (pbc is not None and not pbc[k]) for k in range(3)]
+    kept = [box[k] for k in range(3) if not is_open[k]]
+    if len(kept) == 3:
+        return box, np.zeros(3)
+
+    def unit(v):
+        length = np.sqrt(v @ v)
+        if not length > 0.0:
+            raise ValueError("the periodic cell vectors are linearly dependent")
+        return v / length
+
+    if not kept:
+        normals = list(np.eye(3))
+    elif len(kept) == 2:
+        normals = [unit(np.cross(kept[0], kept[1]))]
+    else:
+        a = unit(kept[0])
+        e = np.zeros(3)
+        e[int(np.argmin(np.abs(a)))] = 1.0        # the axis least aligned with the one periodic vector
+        b = unit(np.cross(a, e))
+        normals = [b, unit(np.cross(a, b))]
+    move = np.zeros(3)
+    for k, d in zip([k for k in range(3) if is_open[k]], normals):
+        along = pos @ d if len(pos) else np.zeros(1)
+        box[k] = d * ((along.max() - along.min()) + 2.0 * reach + 1.0)
         if len(pos):
-            shift += d * (reach + 0.5 - proj.min())
-    return cell, shift
+            move += d * (reach + 0.5 - along.min())
+    return box, move
 
 
 class System:

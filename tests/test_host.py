@@ -63,17 +63,17 @@ def _mutated_2l(tmp_path, fn):
 
 
 BAD_2L = [
-    (lambda d: d.pop("B0_lin_transform_W"), "required weight 'B0_lin_transform_W' missing"),
-    (lambda d: d.update(YI_lr_inds=d["YI_lr_inds"] + 7), "YI_lr_inds' has (7, 7) at 0"),
+    (lambda d: d.pop("B0_lin_transform_W"), "'B0_lin_transform_W' is absent or empty"),
+    (lambda d: d.update(YI_lr_inds=d["YI_lr_inds"] + 7), "'YI_lr_inds' "),
     (lambda d: d.update(I_n_out=np.array([11])), "I_n_out"),
-    (lambda d: d.update(B_total_sum_ind_YI=d["B_total_sum_ind_YI"] + 100), "B_total_sum_ind_YI' has"),
+    (lambda d: d.update(B_total_sum_ind_YI=d["B_total_sum_ind_YI"] + 100), "'B_total_sum_ind_YI' [0] = 101 points outside"),
     (lambda d: d.update(I1_is_central_atom_type_dependent=np.array([0])), "I1_is_central_atom_type_dependent"),
-    (lambda d: d.update(I_0_LN_scale=d["I_0_LN_scale"][:-1]), "I_0_LN_scale' has 8 values, expected 9"),
+    (lambda d: d.update(I_0_LN_scale=d["I_0_LN_scale"][:-1]), "'I_0_LN_scale' holds 8 values, expected 9"),
     (lambda d: d.update(I2_n_out=np.array([7])), "I2_n_out"),
     (lambda d: d.update(prod_BBBB_n_cg_terms=np.array([1])), "prod_AAAA_n_cg_terms"),
-    (lambda d: d.update(fc_BB1_w_left=d["fc_BB1_w_left"][:, :-1]), "fc_BB1_w_left' has shape"),
+    (lambda d: d.update(fc_BB1_w_left=d["fc_BB1_w_left"][:, :-1]), "'fc_BB1_w_left' is stored as 24 x 23 x 9"),
     (lambda d: d.update(mlp_rad_R1_has_chem_emb=np.array([1])), "mlp_rad_R1_has_chem_emb"),
-    (lambda d: d.update(I2_reduce_BB_W=d["I2_reduce_BB_W"][:1]), "I2_reduce_BB_W' has shape"),
+    (lambda d: d.update(I2_reduce_BB_W=d["I2_reduce_BB_W"][:1]), "'I2_reduce_BB_W' is stored as 1 x 9 x 24 x 3"),
 ]
 
 
@@ -102,27 +102,27 @@ def _drop_name(d, key, name):
 
 
 BAD_3L = [
-    (lambda d: d.pop("A2_cg_W"), "required weight 'A2_cg_W' missing"),
-    (lambda d: d.update(A2_cg_W=d["A2_cg_W"][:-1]), "A2_cg_W' has shape"),
+    (lambda d: d.pop("A2_cg_W"), "'A2_cg_W' is absent or empty"),
+    (lambda d: d.update(A2_cg_W=d["A2_cg_W"][:-1]), "'A2_cg_W' is stored as 80 x 35 where 81 x 35 is needed"),
     (lambda d: d.update(A1_mlp_W0=d["A1_mlp_W0"][:-1]), "A1_mlp_W0"),
-    (lambda d: d.update(A1_mlp_b0=d["A1_mlp_b0"][:-1]), "A1_mlp_b0' has 31 values, expected 32"),
+    (lambda d: d.update(A1_mlp_b0=d["A1_mlp_b0"][:-1]), "'A1_mlp_b0' holds 31 values, expected 32"),
     (lambda d: d.update(A3_equivariant=np.array([0]), A3_lin_transform_W=d["A1_lin_transform_W"]), "A3_equivariant' is 0, expected 1"),
     (lambda d: d.update(A1_equivariant=np.array([1])), "A1_"),
-    (lambda d: _drop_name(d, "prod_names", "A2_3"), "prod_names' has no 'A2_3'"),
-    (lambda d: d.update(prod_names=np.concatenate([d["prod_names"], np.array([b"A1_2"], dtype=d["prod_names"].dtype)])), "lists 'A1_2' twice"),
-    (lambda d: _drop_name(d, "reduce_names", "eq1"), "reduce_names' has no 'eq1'"),
-    (lambda d: d.update(A1_2_left_ind=d["A1_2_left_ind"] + 1000), "A1_2_left_ind' has"),
-    (lambda d: d.update(A1_2_group_left=d["A1_2_group_left"][:-1]), "A1_2_left_ind' has 8 at"),
-    (lambda d: d.update(A2_3_U=d["A2_3_U"][:, :, :-1]), "A2_3_U' has shape"),
+    (lambda d: _drop_name(d, "prod_names", "A2_3"), "'prod_names' does not list 'A2_3'"),
+    (lambda d: d.update(prod_names=np.concatenate([d["prod_names"], np.array([b"A1_2"], dtype=d["prod_names"].dtype)])), "lists 'A1_2' 2 times"),
+    (lambda d: _drop_name(d, "reduce_names", "eq1"), "'reduce_names' does not list 'eq1'"),
+    (lambda d: d.update(A1_2_left_ind=d["A1_2_left_ind"] + 1000), "'A1_2_left_ind' [0] = 1000 points outside"),
+    (lambda d: d.update(A1_2_group_left=d["A1_2_group_left"][:-1]), "'A1_2_left_ind' [22] = 8 points outside the 8 entries"),
+    (lambda d: d.update(A2_3_U=d["A2_3_U"][:, :, :-1]), "'A2_3_U' is stored as 6 x 16 x 15"),
     (lambda d: d.update(fc_A1_2a_left_coefs=np.array([1])), "fc_A1_2a_left_coefs"),
-    (lambda d: d.update(fc_A1_2a_collect_from=d["fc_A1_2a_collect_from"] + 100), "fc_A1_2a_collect_from' has"),
+    (lambda d: d.update(fc_A1_2a_collect_from=d["fc_A1_2a_collect_from"] + 100), "'fc_A1_2a_collect_from' [0] = 100 points outside the 9 functions of A1"),
     (lambda d: d.update(eq1_instruction_names=d["eq1_instruction_names"][:-1]), "eq1_instruction_names"),
-    (lambda d: d.update(eq1_norm_l0_mask=d["eq1_norm_l0_mask"][:-1]), "eq1_norm_l0_mask' has 8 values, expected 9"),
-    (lambda d: d.update(rho2_norm_scale=d["rho2_norm_scale"][:-1]), "rho2_norm_scale' has 7 values, expected 8"),
+    (lambda d: d.update(eq1_norm_l0_mask=d["eq1_norm_l0_mask"][:-1]), "'eq1_norm_l0_mask' holds 8 values, expected 9"),
+    (lambda d: d.update(rho2_norm_scale=d["rho2_norm_scale"][:-1]), "'rho2_norm_scale' holds 7 values, expected 8"),
     (lambda d: d.update(out1_origins=d["out1_origins"][:2], energy_mlp_n_origins=np.array([2])), "out1_origins"),
     (lambda d: d.update(energy_mlp_W0=d["energy_mlp_W0"][:-1]), "energy_mlp_W0"),
-    (lambda d: d.update(A2_p=np.array([6])), "A2_p' is 6, the envelope order of A1 is 5"),
-    (lambda d: d.update(radial_activation=np.array([0])), "radial_activation' is a legacy GRACE-1L/2L key"),
+    (lambda d: d.update(A2_p=np.array([6])), "'A2_p' = 6 while A1 uses the envelope order 5"),
+    (lambda d: d.update(radial_activation=np.array([0])), "'radial_activation' is a switch of the one- and two-layer formats"),
     (lambda d: d.update(A2_n_lm_ind=np.array([5])), "A2_"),
 ]
 
@@ -158,18 +158,18 @@ def _mutated(tmp_path, fn):
 
 
 BAD = [
-    (lambda d: d.pop("chem_embedding"), "required weight 'chem_embedding' missing"),
+    (lambda d: d.pop("chem_embedding"), "'chem_embedding' is absent or empty"),
     (lambda d: d.update(mlp_rad_W1=d["mlp_rad_W1"][:, :-1]), "mlp_rad_W2"),
-    (lambda d: d.update(prod_AA_left_ind=d["prod_AA_left_ind"] + 100), "prod_AA_left_ind' has"),
-    (lambda d: d.update(fc_A1_w_tile_left=d["fc_A1_w_tile_left"][:-1]), "fc_A1_w_tile_left' has 8 values, expected 9"),
-    (lambda d: d.update(rho_reduce_AA_W=d["rho_reduce_AA_W"][:, :, :, :1]), "rho_reduce_AA_W' has shape"),
+    (lambda d: d.update(prod_AA_left_ind=d["prod_AA_left_ind"] + 100), "'prod_AA_left_ind' [0] = 100 points outside the 9 entries"),
+    (lambda d: d.update(fc_A1_w_tile_left=d["fc_A1_w_tile_left"][:-1]), "'fc_A1_w_tile_left' holds 8 values, expected 9"),
+    (lambda d: d.update(rho_reduce_AA_W=d["rho_reduce_AA_W"][:, :, :, :1]), "rho_reduce_AA_W"),
     (lambda d: d.update(A_lin_transform_W=np.asfortranarray(d["A_lin_transform_W"])), "Fortran order"),
-    (lambda d: d.update(mlp_rad_W0=np.where(np.arange(d["mlp_rad_W0"].size).reshape(d["mlp_rad_W0"].shape) == 3, np.nan, d["mlp_rad_W0"])), "non-finite"),
-    (lambda d: d.update(lmax=np.array([300])), "lmax' is 300"),
+    (lambda d: d.update(mlp_rad_W0=np.where(np.arange(d["mlp_rad_W0"].size).reshape(d["mlp_rad_W0"].shape) == 3, np.nan, d["mlp_rad_W0"])), "is not a finite number"),
+    (lambda d: d.update(lmax=np.array([300])), "'lmax' = 300 lies outside 0 .. 255"),
     (lambda d: d.update(rcut=np.array([-1.0])), "cutoff"),
     (lambda d: d.update(fc_A1_left_coefs=np.array([0])), "fc_A1_left_coefs"),
     (lambda d: d.update(grace_model_kind=np.array([b"GRACE-9L"], dtype="|S8")), "grace_model_kind"),
-    (lambda d: d.update(prod_AAAA_left_ind=np.zeros(1, np.int32)), "AAAA stage is incomplete"),
+    (lambda d: d.update(prod_AAAA_left_ind=np.zeros(1, np.int32)), "the stage is incomplete"),
     (lambda d: d.update(energy_mlp_W1=d["energy_mlp_W1"].astype("U")), "unsupported dtype"),
 ]
 

@@ -106,16 +106,16 @@ def _mutated(tmp_path, edit, name="uq2"):
 
 
 BAD_UQ = [
-    (lambda d: d.update(uq_schema_version=np.array([5])), "UQ schema v5 unsupported"),
-    (lambda d: d.update(uq_rp_matrix=d["uq_rp_matrix"][:-1]), "rows, the model's invariant basis has"),
+    (lambda d: d.update(uq_schema_version=np.array([5])), "UQ head of schema 5; only schema 6"),
+    (lambda d: d.update(uq_rp_matrix=d["uq_rp_matrix"][:-1]), "basis functions, the model has"),
     (lambda d: d.update(uq_rp_matrix=np.ascontiguousarray(d["uq_rp_matrix"].T)), "uq_rp_matrix"),
-    (lambda d: d.update(uq_n_clusters=np.array([3, 0], np.int32)), "element index 1 has no GMM clusters"),
-    (lambda d: d.update(uq_n_clusters=np.array([3, 4], np.int32)), "more than uq_max_clusters = 3"),
+    (lambda d: d.update(uq_n_clusters=np.array([3, 0], np.int32)), "element 1 has no GMM cluster"),
+    (lambda d: d.update(uq_n_clusters=np.array([3, 4], np.int32)), "uq_n_clusters\' \\[1\\] = 4 points outside"),
     (lambda d: d.update(uq_centroids=d["uq_centroids"][:, :2]), "uq_centroids"),
     (lambda d: d.update(uq_inv_cov=d["uq_inv_cov"][:, :, :, :-1]), "uq_inv_cov"),
-    (lambda d: d.update(uq_rp_normalize=np.array([0])), "schema v6 expects normalize=1"),
+    (lambda d: d.update(uq_rp_normalize=np.array([0])), "uq_rp_normalize = 0"),
     (lambda d: d.update(uq_feature_dim=np.array([15]), uq_centroids=np.zeros((2, 3, 15)), uq_inv_cov=np.zeros((2, 3, 15, 15))),
-     "3 density channels, expected 2"),
+     "3 density channels where 2 belong"),
     (lambda d: d.update(uq_n_elements=np.array([3])), "uq_n_elements"),
     (lambda d: d.pop("uq_interp_thresholds"), "uq_interp_thresholds"),
 ]
@@ -158,11 +158,11 @@ def synth_uq(d):
 
 
 BAD_UQ_2L = [
-    (lambda d: d.update(uq_rp_matrix=d["uq_rp_matrix"][:-1]), "rows, the model's invariant basis has"),
+    (lambda d: d.update(uq_rp_matrix=d["uq_rp_matrix"][:-1]), "basis functions, the model has"),
     (lambda d: d.update(uq_feature_dim=np.array([12]), uq_centroids=np.zeros((2, 3, 12)), uq_inv_cov=np.zeros((2, 3, 12, 12))),
-     "2 density channels, expected 3"),
-    (lambda d: d.update(uq_schema_version=np.array([4])), "UQ schema v4 unsupported"),
-    (lambda d: d.update(uq_n_clusters=np.array([0, 3], np.int32)), "element index 0 has no GMM clusters"),
+     "2 density channels where 3 belong"),
+    (lambda d: d.update(uq_schema_version=np.array([4])), "UQ head of schema 4; only schema 6"),
+    (lambda d: d.update(uq_n_clusters=np.array([0, 3], np.int32)), "element 0 has no GMM cluster"),
 ]
 
 
@@ -185,10 +185,10 @@ def test_max_order_3_2l_model_with_a_head_is_refused(tmp_path):
 BAD_UQ_3L = [
     (lambda d: d.update(uq_rp_matrix=d["uq_rp_matrix"][:-1]), "uq_rp_matrix"),
     (lambda d: d.update(uq_feature_dim=np.array([14]), uq_centroids=np.zeros((2, 3, 14)), uq_inv_cov=np.zeros((2, 3, 14, 14))),
-     r"uq_n_density \(5\) > 4"),
-    (lambda d: d.update(uq_schema_version=np.array([3])), "schema v3 unsupported"),
-    (lambda d: d.update(uq_n_clusters=np.array([3, 0], np.int32)), "element index 1 has no GMM clusters"),
-    (lambda d: d.update(uq_rp_normalize=np.array([0])), "schema v6 expects normalize=1"),
+     "5 density channels; the three-layer kernels write at most 4"),
+    (lambda d: d.update(uq_schema_version=np.array([3])), "UQ head of schema 3; only schema 6"),
+    (lambda d: d.update(uq_n_clusters=np.array([3, 0], np.int32)), "element 1 has no GMM cluster"),
+    (lambda d: d.update(uq_rp_normalize=np.array([0])), "uq_rp_normalize = 0"),
 ]
 
 
