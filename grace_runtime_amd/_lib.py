@@ -25,7 +25,7 @@ SYMBOLS = [
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
     "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_batch_uq", "gr_compute_batch_device_uq", "gr_engine_reset", "gr_engine_release_buffers", "gr_set_memory_limit", "gr_memory_in_use", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
-    "gr_system_fetch_uq",
+    "gr_system_fetch_uq", "gr_engine_set_chunksize", "gr_engine_chunksize", "gr_system_set_chunksize", "gr_system_chunksize",
 ]
 
 
@@ -85,6 +85,10 @@ def lib():
     L.gr_engine_stage_get.argtypes = [vp, i32, C.c_char_p, i32, C.POINTER(dbl), C.POINTER(i32)]
     L.gr_engine_debug_radial.argtypes = [vp, i32, vp, vp, vp, vp]
     L.gr_engine_stage_flops.argtypes = [vp, i32, vp]
+    L.gr_engine_set_chunksize.argtypes = [vp, i32]
+    L.gr_engine_chunksize.argtypes = [vp]
+    L.gr_system_set_chunksize.argtypes = [vp, i32]
+    L.gr_system_chunksize.argtypes = [vp]
     L.gr_engine_radial_noalloc.argtypes = [vp, i32, vp, vp, vp, vp]
     L.gr_engine_debug_copy.argtypes = [vp, i64]
     L.gr_neighbor_build.argtypes = [i64, vp, vp, vp, dbl, i32, C.POINTER(vp)]

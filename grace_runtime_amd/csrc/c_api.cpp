@@ -67,6 +67,7 @@ struct gr_system {
   double skin = 0.0, cutoff = 0.0;
   int rebuilds = 0, generation = 0;
   bool have = false, on_device = false;
+  bool auto_chunk = true;    // the chunk is the engine's choice (and may be halved after an allocation failure)
   int n = 0;
   std::vector<int> types;
   std::vector<double> x0, cell;
@@ -83,6 +84,13 @@ struct gr_system {
 };
 
 namespace {
+// the engine behind a handle; a handle whose engine was dropped by a reset that could not build the new one says so
+grhip::Engine &live(const gr_engine *e)
+{
+  if (!e) throw grhip::InvalidArgument("null engine");
+  if (!e->eng) throw grhip::Error("the engine was lost when a reset could not allocate its replacement; call gr_engine_reset");
+  return *e->eng;
+}
 void padded_cell(const double *cell, const unsigned char *pbc, const double *pos, int64_t n, double reach, double *out, double *shift);
 thread_local std::string g_err;
 
@@ -249,7 +257,7 @@ int gr_engine_release_buffers(gr_engine *e)
     if (!e) throw grhip::InvalidArgument("null engine");
     e->bnl.reset();
     e->lmp.reset();
-    e->eng->release_buffers();
+    live(e).release_buffers();
     e->generation++;    // a gr_system on this engine uploads its structure again
   });
 }
@@ -267,14 +275,14 @@ int64_t gr_memory_in_use(void) { return grhip::dev_bytes_in_use().load(); }
 
 void gr_engine_free(gr_engine *e) { delete e; }
 
-double gr_engine_cutoff(const gr_engine *e, int t1, int t2) { return e ? e->eng->cutoff(t1, t2) : 0.0; }
+double gr_engine_cutoff(const gr_engine *e, int t1, int t2) { return e && e->eng ? e->eng->cutoff(t1, t2) : 0.0; }
 
 int gr_engine_upload(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
                      const double *positions, const int *image, const double *shifts, int64_t nimages)
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->upload(make_input(n, types, offset, j, rij, positions, image, shifts, nimages));
+    live(e).upload(make_input(n, types, offset, j, rij, positions, image, shifts, nimages));
   });
 }
 
@@ -286,7 +294,7 @@ int gr_engine_run(gr_engine *e, unsigned flags)
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0;
     fl.uq = (flags & GR_FLAG_UQ) != 0;
-    e->eng->run(fl);
+    live(e).run(fl);
   });
 }
 
@@ -294,7 +302,7 @@ int gr_engine_fetch_uq(gr_engine *e, double *gamma, double *sigma, double *clust
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->fetch_uq(gamma, sigma, cluster);
+    live(e).fetch_uq(gamma, sigma, cluster);
   });
 }
 
@@ -322,7 +330,7 @@ int gr_engine_sync(gr_engine *e)
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->synchronize();
+    live(e).synchronize();
   });
 }
 
@@ -330,14 +338,14 @@ int gr_engine_fetch(gr_engine *e, double *energy, double *forces, double *virial
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->fetch(energy, forces, virial, eatom);
+    live(e).fetch(energy, forces, virial, eatom);
   });
 }
 
 int64_t gr_engine_edge_count(gr_engine *e)
 {
   int64_t r = -1;
-  guarded([&] { r = e->eng->last_edge_count(); });
+  guarded([&] { r = live(e).last_edge_count(); });
   return r;
 }
 
@@ -347,12 +355,12 @@ int gr_compute_csr(gr_engine *e, int n, const int *types, const int64_t *offset,
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->upload(make_input(n, types, offset, j, rij, positions, image, shifts, nimages));
+    live(e).upload(make_input(n, types, offset, j, rij, positions, image, shifts, nimages));
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
-    e->eng->run(fl);
-    e->eng->fetch(energy, forces, virial, eatom);
+    live(e).run(fl);
+    live(e).fetch(energy, forces, virial, eatom);
   });
 }
 
@@ -360,7 +368,7 @@ int gr_engine_set_profile(gr_engine *e, int on)
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->set_profile(on != 0);
+    live(e).set_profile(on != 0);
   });
 }
 
@@ -368,7 +376,7 @@ int gr_engine_stage_count(gr_engine *e)
 {
   int n = -1;
   guarded([&] {
-    e->times = e->eng->stage_times();
+    e->times = live(e).stage_times();
     n = (int) e->times.size();
   });
   return n;
@@ -399,7 +407,7 @@ int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->debug_radial(m, x, mu_j, Rz, dRz);
+    live(e).debug_radial(m, x, mu_j, Rz, dRz);
   });
 }
 
@@ -407,7 +415,7 @@ int gr_engine_radial_noalloc(gr_engine *e, int m, const double *x, const int *mu
 {
   return guarded([&] {
     if (!e || !e->eng) throw grhip::InvalidArgument("null engine");
-    e->eng->radial_noalloc(m, x, mu_j, Rz, dRz);
+    live(e).radial_noalloc(m, x, mu_j, Rz, dRz);
   });
 }
 
@@ -415,7 +423,7 @@ int gr_engine_debug_copy(gr_engine *e, int64_t bytes)
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->debug_copy(bytes);
+    live(e).debug_copy(bytes);
   });
 }
 
@@ -459,7 +467,7 @@ int gr_compute(gr_engine *e, int n, const int *types, const double *positions, c
     double rc = 0.0;
     {
       // largest cutoff over the types present
-      rc = e->eng->max_cutoff();
+      rc = live(e).max_cutoff();
       if (!(rc > 0.0)) throw grhip::Error("the engine has no positive cutoff");
     }
     grhip::NeighborList nl = grhip::neighbor_search(positions, n, cell, p, rc, 8);
@@ -472,14 +480,14 @@ int gr_compute(gr_engine *e, int n, const int *types, const double *positions, c
     }
     std::vector<double> dummy(3, 0.0);
     const int64_t nimg = (int64_t) nl.shifts.size() / 3;
-    e->eng->upload(make_input(n, ty.data(), nl.offset.data(), nl.j.data(), nullptr, x.data(), nl.image.data(),
+    live(e).upload(make_input(n, ty.data(), nl.offset.data(), nl.j.data(), nullptr, x.data(), nl.image.data(),
                               nimg ? nl.shifts.data() : dummy.data(), nimg));
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
-    e->eng->run(fl);
+    live(e).run(fl);
     std::vector<double> f((size_t) 3 * n), ea(fl.eatom ? n : 0);
-    e->eng->fetch(energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
+    live(e).fetch(energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
     for (int q = 0; q < n; q++) {
       const int64_t a = nl.perm[q];
       if (forces && !fl.energy_only)
@@ -671,8 +679,8 @@ int gr_system_create(gr_engine *e, double skin, gr_system **out)
     auto s = std::make_unique<gr_system>();
     s->eng = e;
     s->skin = skin;
-    s->cutoff = e->eng->max_cutoff();
-    if (hipSetDevice(e->eng->device_index()) != hipSuccess || hipStreamCreate(&s->stream) != hipSuccess)
+    s->cutoff = live(e).max_cutoff();
+    if (hipSetDevice(live(e).device_index()) != hipSuccess || hipStreamCreate(&s->stream) != hipSuccess)
       throw grhip::Error("gr_system_create: cannot create a stream on the engine's device");
     *out = s.release();
   });
@@ -685,11 +693,12 @@ int gr_system_list_on_device(const gr_system *s) { return s && s->have && s->on_
 int gr_system_compute(gr_system *s, int n, const int *types, const double *positions, const double *cell, const unsigned char *pbc,
                       unsigned flags, double *energy, double *forces, double *virial, double *eatom)
 {
-  return guarded([&] {
+  // one attempt; an allocation failure inside leaves as std::bad_alloc
+  auto attempt = [&] {
     if (!s || !cell || !pbc || (n > 0 && (!types || !positions))) throw grhip::InvalidArgument("null argument");
     if (n < 0) throw grhip::InvalidArgument("negative atom count");
     if (!(s->cutoff > 0.0)) throw grhip::Error("the engine has no positive cutoff");
-    grhip::Engine &eng = *s->eng->eng;
+    grhip::Engine &eng = live(s->eng);
     if (hipSetDevice(eng.device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
     // list policy of the reference (python/grace_runtime/neighbors.py:68-89): rebuild when the atoms, the cell or the
     // boundary conditions change or an atom moved more than skin / 2 since the last build
@@ -774,8 +783,54 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
         for (int d = 0; d < 3; d++) forces[3 * a + d] = f[3 * (size_t) q + d];
       if (fl.eatom) eatom[a] = ea[q];
     }
+  };
+  // Allocation failure with the automatic chunk (python/kk/kk_api.h:72-75, kk_core.cpp:453-497): the work buffers go back,
+  // the chunk is halved (never below 512 atoms) and kept for later calls, and the call starts again; when 512 atoms per
+  // pass do not fit either, or the chunk was fixed by the caller, the failure is reported and the engine stays usable.
+  return guarded([&] {
+    for (;;) {
+      try {
+        attempt();
+        return;
+      } catch (const std::bad_alloc &) {
+        grhip::Engine &eng = live(s->eng);
+        const int used = eng.chunksize_used() > 0 ? eng.chunksize_used() : n;
+        s->have = false;
+        eng.release_buffers();
+        if (!s->auto_chunk || used <= 512)
+          throw grhip::Error("the structure (" + std::to_string(n) + " atoms) does not fit the GPU memory " +
+                             (s->auto_chunk ? "even in chunks of 512 atoms" : "with the chunk size that was asked for") +
+                             "; use a GPU with more memory or a smaller chunksize");
+        int next = 512;
+        while (2 * next < used) next *= 2;
+        try {
+          eng.set_chunksize(next);
+        } catch (const grhip::InvalidArgument &) {    // an engine that evaluates structures in one pass only
+          throw grhip::Error("the structure (" + std::to_string(n) + " atoms) does not fit the GPU memory in one pass, and this model kind is "
+                             "not evaluated in chunks");
+        }
+      }
+    }
   });
 }
+
+int gr_system_set_chunksize(gr_system *s, int atoms)
+{
+  return guarded([&] {
+    if (!s) throw grhip::InvalidArgument("null system");
+    live(s->eng).set_chunksize(atoms);
+    s->auto_chunk = atoms < 0;
+  });
+}
+
+int gr_system_chunksize(const gr_system *s) { return s && s->eng && s->eng->eng ? s->eng->eng->chunksize_used() : 0; }
+
+int gr_engine_set_chunksize(gr_engine *e, int atoms)
+{
+  return guarded([&] { live(e).set_chunksize(atoms); });
+}
+
+int gr_engine_chunksize(const gr_engine *e) { return e && e->eng ? e->eng->chunksize_used() : 0; }
 
 int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *cluster)
 {
@@ -783,7 +838,7 @@ int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *clust
     if (!s || !s->have) throw grhip::Error("gr_system_fetch_uq: no structure has been computed");
     const int n = s->n;
     std::vector<double> g((size_t) n), sg((size_t) n), cl((size_t) n);
-    s->eng->eng->fetch_uq(g.data(), sg.data(), cl.data());
+    live(s->eng).fetch_uq(g.data(), sg.data(), cl.data());
     for (int q = 0; q < n; q++) {
       const int64_t a = s->perm[q];
       if (gamma) gamma[a] = g[q];
@@ -809,7 +864,7 @@ int gr_system_list_get(gr_system *s, int64_t *perm, int64_t *offset, int32_t *j,
     if (!s || !s->have) throw grhip::Error("gr_system_list_get: no list has been built");
     std::memcpy(perm, s->perm.data(), sizeof(int64_t) * s->perm.size());
     if (s->on_device) {
-      if (hipSetDevice(s->eng->eng->device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
+      if (hipSetDevice(live(s->eng).device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
       bool ok = hipMemcpy(offset, s->nl.offset.p, sizeof(int64_t) * (size_t) (s->n + 1), hipMemcpyDeviceToHost) == hipSuccess;
       if (s->nl.nb > 0) {
         ok = ok && hipMemcpy(j, s->nl.j.p, sizeof(int32_t) * (size_t) s->nl.nb, hipMemcpyDeviceToHost) == hipSuccess;
@@ -837,7 +892,7 @@ int gr_engine_upload_batch(gr_engine *e, int n, const int *types, const int64_t 
     grhip::CsrInput in = make_input(n, types, offset, j, rij, positions, image, shifts, nimages);
     in.nstruct = nstruct;
     in.sid = struct_of_atom;
-    e->eng->upload(in);
+    live(e).upload(in);
   });
 }
 
@@ -845,7 +900,7 @@ int gr_engine_fetch_batch(gr_engine *e, int nstruct, double *energy, double *for
 {
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
-    e->eng->fetch_batch(nstruct, energy, forces, virial, eatom);
+    live(e).fetch_batch(nstruct, energy, forces, virial, eatom);
   });
 }
 
@@ -927,7 +982,7 @@ int gr_compute_batch_uq(gr_engine *e, int nstruct, const int *natoms, const int 
   return guarded([&] {
     if (!e || nstruct < 0 || (nstruct > 0 && (!natoms || !cells || !pbc))) throw grhip::InvalidArgument("null argument");
     if (nstruct == 0) return;
-    const double rc = e->eng->max_cutoff();
+    const double rc = live(e).max_cutoff();
     if (!(rc > 0.0)) throw grhip::Error("the engine has no positive cutoff");
     std::vector<int64_t> start(nstruct + 1, 0);
     for (int s = 0; s < nstruct; s++) {
@@ -993,16 +1048,16 @@ int gr_compute_batch_uq(gr_engine *e, int nstruct, const int *natoms, const int 
     grhip::CsrInput in = make_input((int) N, ty.data(), offset.data(), jj.data(), nullptr, x.data(), img.data(), shifts.data(), nimg);
     in.nstruct = nstruct;
     in.sid = sid.data();
-    e->eng->upload(in);
+    live(e).upload(in);
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
     fl.uq = gamma || sigma || cluster;
-    e->eng->run(fl);
+    live(e).run(fl);
     std::vector<double> f((size_t) 3 * N), ea(fl.eatom ? N : 0);
-    e->eng->fetch_batch(nstruct, energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
+    live(e).fetch_batch(nstruct, energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
     std::vector<double> ug(gamma ? N : 0), us(sigma ? N : 0), uc(cluster ? N : 0);
-    if (fl.uq) e->eng->fetch_uq(gamma ? ug.data() : nullptr, sigma ? us.data() : nullptr, cluster ? uc.data() : nullptr);
+    if (fl.uq) live(e).fetch_uq(gamma ? ug.data() : nullptr, sigma ? us.data() : nullptr, cluster ? uc.data() : nullptr);
     for (int s = 0; s < nstruct; s++)
       for (int64_t q = 0; q < natoms[s]; q++) {
         const int64_t a = start[s] + nls[s].perm[q], w = start[s] + q;
@@ -1033,7 +1088,7 @@ int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, con
     if (!e || nstruct < 0 || (nstruct > 0 && (!natoms || !cells || !pbc))) throw grhip::InvalidArgument("null argument");
     if (max_atoms < 0) throw grhip::InvalidArgument("max_atoms must be >= 0");
     if (nstruct == 0) return;
-    const double rc = e->eng->max_cutoff();
+    const double rc = live(e).max_cutoff();
     if (!(rc > 0.0)) throw grhip::Error("the engine has no positive cutoff");
     std::vector<int64_t> start((size_t) nstruct + 1, 0);
     for (int s = 0; s < nstruct; s++) {
@@ -1044,12 +1099,12 @@ int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, con
     if (N >= INT32_MAX) throw grhip::InvalidArgument("atom count out of range");
     if (N > 0 && (!types || !positions)) throw grhip::InvalidArgument("null argument");
     if (!energy) throw grhip::InvalidArgument("the energy output is required");
-    if (hipSetDevice(e->eng->device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
+    if (hipSetDevice(live(e).device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
     // the pointers must be memory of the engine's GPU: a host pointer here would fault in the kernels
     auto on_device = [&](const void *p, const char *name) {
       if (!p) return;
       hipPointerAttribute_t at;
-      if (hipPointerGetAttributes(&at, p) != hipSuccess || at.type != hipMemoryTypeDevice || at.device != e->eng->device_index()) {
+      if (hipPointerGetAttributes(&at, p) != hipSuccess || at.type != hipMemoryTypeDevice || at.device != live(e).device_index()) {
         (void) hipGetLastError();
         throw grhip::InvalidArgument(std::string(name) + " must be memory of the engine's GPU");
       }
@@ -1095,11 +1150,11 @@ int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, con
         in.rij = nl.rij.as<double>();
         in.nstruct = ns;
         in.sid = nl.sid.data();
-        e->eng->upload_device(in);
-        e->eng->run(fl);
-        e->eng->fetch_batch_device(ns, energy + g0, forces ? forces + 3 * a0 : nullptr, virial ? virial + 6 * (size_t) g0 : nullptr,
+        live(e).upload_device(in);
+        live(e).run(fl);
+        live(e).fetch_batch_device(ns, energy + g0, forces ? forces + 3 * a0 : nullptr, virial ? virial + 6 * (size_t) g0 : nullptr,
                                    fl.eatom ? eatom + a0 : nullptr);
-        if (fl.uq) e->eng->fetch_uq(gamma ? gamma + a0 : nullptr, sigma ? sigma + a0 : nullptr, cluster ? cluster + a0 : nullptr);
+        if (fl.uq) live(e).fetch_uq(gamma ? gamma + a0 : nullptr, sigma ? sigma + a0 : nullptr, cluster ? cluster + a0 : nullptr);
         if (passes) ++*passes;
         g0 = g1;
       }

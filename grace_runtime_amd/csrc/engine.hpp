@@ -84,6 +84,11 @@ class Engine {
   virtual void fetch_add_device(const int *atom, double *energy, double *forces, double *virial, double *eatom) = 0;
   // UQ outputs of the last run with RunFlags::uq, [n] each in the order of the uploaded list (null pointers are skipped)
   virtual void fetch_uq(double *gamma, double *sigma, double *cluster) = 0;
+  // atoms per engine pass (python/kk/kk_api.h:72-75): 0 all atoms in one pass, < 0 chosen from the free device memory
+  // (one pass while it fits, else the largest power of two >= 512 that fits), > 0 as given.  chunksize_used(): atoms per
+  // pass of the last run (0: one pass).  Engines that do not chunk refuse values other than 0 and -1.
+  virtual void set_chunksize(int atoms) = 0;
+  virtual int chunksize_used() const = 0;
   virtual void release_buffers() = 0;    // frees the work buffers and the uploaded structure; weights stay
   virtual void synchronize() = 0;
   virtual void set_profile(bool on) = 0;

@@ -73,6 +73,7 @@ template<class T> class Engine1L final : public EngineBase {
       EngineBase(device, "GRACE-1L", ntypes, type2mu, m->n_elements), model_(std::move(m))
   {
     this->template probe_mfma<T>();
+    chunks_ = true;
     build();
     scratch_dev_ = scratch_of_device(device);    // set-up: the device is current (EngineBase)
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
@@ -112,9 +113,13 @@ template<class T> class Engine1L final : public EngineBase {
   DevBuf A_, A1_, AA_, AA1_, AA2_, AAA_, AAAA_, gA_, gA1_, gAA_, gAA1_, gAA2_, gAAA_, gAAAA_, rho_, grho_;
 
   void build();
+  // the atom tiles of the chunk that is being evaluated (all atoms when there is one chunk)
+  const int *cur_tiles_ = nullptr;
+  int cur_ntiles_ = 0;
+  void run_chunk(const RunFlags &fl, int a0, int nc, long long e_begin, long long e_count);
   void launch_gemm(DevJobs<T> &J, int kb0, int kb1, int nb, const T *X0, int nf0, const T *X1, int nf1, T *out, int nfo, int accumulate)
   {
-    EngineBase::launch_gemm<T>(J, kb0, kb1, nb, X0, nf0, X1, nf1, out, nfo, accumulate, tiles_.as<int>(), ntiles_);
+    EngineBase::launch_gemm<T>(J, kb0, kb1, nb, X0, nf0, X1, nf1, out, nfo, accumulate, cur_tiles_, cur_ntiles_);
   }
   void launch_radial(long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
                      const long long *n_edges);
@@ -303,18 +308,27 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
 {
   const int n = n_;
   if (!begin_pass(fl)) return;
-  const size_t ecap = (size_t) std::max<int64_t>(nb_, 1);
 
-  // ---- radial functions of all edges
+  // ---- chunks of atoms: every stage after the bond filter acts on the atoms of a chunk and on their bonds only, so the
+  // radial rows and the per-atom tensors are sized for one chunk; forces, per-atom energies and the compact bonds are
+  // kept for the whole structure
+  const double bonds_per_atom = (double) std::max<int64_t>(nb_, 1) / n;
+  const double per_atom = sizeof(T) * (2.0 * nlm_ * CP_ + (double) CFP_ * (2.0 * nlm_ + (order4_ ? 6.0 : 4.0) * nAA_ + 2.0 * nAAA_ + 2.0 * nAAAA_)) +
+                          16.0 * nrho_ + bonds_per_atom * 2.0 * noutp_ * sizeof(T);
+  const int cs = plan_chunk(n, per_atom, 64.0 * bonds_per_atom + 64.0);
+  const int nchunks = (n + cs - 1) / cs;
+  chunk_used_ = nchunks > 1 ? cs : 0;
+  std::vector<long long> ebound;
+  size_t ecap = (size_t) std::max<int64_t>(nb_, 1);
+  if (nchunks > 1) {
+    layout_chunks(cs);
+    ebound = chunk_edge_bounds(cs);
+    ecap = 1;
+    for (int k = 0; k < nchunks; k++) ecap = std::max(ecap, (size_t) (ebound[(size_t) k + 1] - ebound[(size_t) k]));
+  }
+  const size_t na = (size_t) cs;
   Rz_.ensure(ecap * noutp_ * sizeof(T));
-  if (!fl.energy_only) dRz_.ensure(ecap * noutp_ * sizeof(T));
-  else dRz_.ensure(ecap * noutp_ * sizeof(T));
-  stage("radial_mlp", [&] {
-    launch_radial(0, -1, xr_.as<double>(), emu_.as<int>(), Rz_.as<T>(), dRz_.as<T>(), eoff_.as<long long>() + n);
-  });
-
-  // ---- per-atom tensors (whole structure in one chunk), channel widths padded
-  const size_t na = (size_t) n;
+  dRz_.ensure(ecap * noutp_ * sizeof(T));
   A_.ensure(na * nlm_ * CP_ * sizeof(T));
   A1_.ensure(na * nlm_ * CFP_ * sizeof(T));
   AA_.ensure(na * nAA_ * CFP_ * sizeof(T));
@@ -326,13 +340,55 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   }
   rho_.ensure(na * nrho_ * sizeof(double));
   grho_.ensure(na * nrho_ * sizeof(double));
+  if (fl.uq) {
+    uq_gamma_.ensure((size_t) n * sizeof(double)); uq_sigma_.ensure((size_t) n * sizeof(double)); uq_cluster_.ensure((size_t) n * sizeof(double));
+    ran_uq_ = true;
+  }
+  if (!fl.energy_only) {
+    gA_.ensure(na * nlm_ * CP_ * sizeof(T));
+    gA1_.ensure(na * nlm_ * CFP_ * sizeof(T));
+    gAA_.ensure(na * nAA_ * CFP_ * sizeof(T));
+    gAA1_.ensure(na * nAA_ * CFP_ * sizeof(T));
+    gAAA_.ensure(na * nAAA_ * CFP_ * sizeof(T));
+    if (order4_) {
+      gAA2_.ensure(na * nAA_ * CFP_ * sizeof(T));
+      gAAAA_.ensure(na * nAAAA_ * CFP_ * sizeof(T));
+    }
+  }
+  if (aaa_a_ && CP_ != CFP_) throw Error("GRACE-1L: AAA = AA1 x A needs equal A and FC widths");
+  for (int k = 0; k < nchunks; k++) {
+    const int a0 = k * cs, nc = std::min(n, a0 + cs) - a0;
+    if (nchunks == 1) {
+      cur_tiles_ = tiles_.as<int>();
+      cur_ntiles_ = ntiles_;
+      run_chunk(fl, 0, n, 0, -1);
+    } else {
+      cur_tiles_ = chunk_tiles_.as<int>() + (size_t) 16 * chunk_tile_off_[(size_t) k];
+      cur_ntiles_ = chunk_tile_off_[(size_t) k + 1] - chunk_tile_off_[(size_t) k];
+      run_chunk(fl, a0, nc, ebound[(size_t) k], ebound[(size_t) k + 1] - ebound[(size_t) k]);
+    }
+  }
+}
+
+// One chunk: atoms [a0, a0 + nc) and their bonds [e_begin, e_begin + e_count) (e_count < 0: all bonds, counted on the
+// device).  Per-atom tensors hold the chunk's atoms from row 0; cur_tiles_ names them by that row.
+template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc, long long e_begin, long long e_count)
+{
+  const int n = nc;
+  const int ntiles = cur_ntiles_;
+  const int *tiles = cur_tiles_;
+  const int *mu = mu_.as<int>() + a0;
+  const size_t na = (size_t) nc;
+  // the radial rows of the chunk start at row 0 of Rz_ / dRz_; the kernels index them by the bond's number in the structure
+  T *Rz = moved_back(Rz_.as<T>(), e_begin * noutp_), *dRz = moved_back(dRz_.as<T>(), e_begin * noutp_);
+
+  stage("radial_mlp", [&] { launch_radial(e_begin, e_count, xr_.as<double>(), emu_.as<int>(), Rz, dRz, eoff_.as<long long>() + n_); });
 
   ScatterArgs<T> sa{};
-  sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz_.as<T>(); sa.A = A_.as<T>();
-  sa.a0 = 0; sa.C = CP_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = noutp_; sa.sh = sh_;
+  sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz; sa.A = A_.as<T>();
+  sa.a0 = a0; sa.C = CP_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = noutp_; sa.sh = sh_;
   stage("scatter_A", [&] { launch_scatter<T>(sa, n, lmax_); });
 
-  const int *tiles = tiles_.as<int>();
   const int ka = CP_ / 16, kf = CFP_ / 16;
   auto jit_launch = [&](hipFunction_t f, std::vector<void *> args) {
     const long long cols = (long long) n * CFP_;
@@ -351,7 +407,6 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   };
   T *A = A_.as<T>(), *A1 = A1_.as<T>(), *AA = AA_.as<T>(), *AA1 = AA1_.as<T>(), *AA2 = AA2_.as<T>(), *AAA = AAA_.as<T>(),
     *AAAA = AAAA_.as<T>();
-  if (aaa_a_ && CP_ != CFP_) throw Error("GRACE-1L: AAA = AA1 x A needs equal A and FC widths");
   const T *Ar = aaa_a_ ? A : A1;
   stage("fc_A1", [&] { launch_gemm(fcA1_.fwd, ka, ka, kf, A, nlm_, A, nlm_, A1, nlm_, 0); });
   prod_fwd("prod_AA", pAA_, A1, A1, AA, nlm_, nlm_);
@@ -362,7 +417,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     prod_fwd("prod_AAAA", pAAAA_, AA2, AA2, AAAA, nAA_, nAA_);
   }
   stage("reduce_rho", [&] {
-#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(ntiles_), dim3(256), 0, stream_, redrho_.d, mu_.as<int>(), tiles, \
+#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(ntiles), dim3(256), 0, stream_, redrho_.d, mu, tiles, \
                                           (const T *) A, (const T *) AA, (const T *) AAA, (const T *) AAAA, rho_.as<double>())
     switch (ka * 10 + kf) {
       case 11: GR_RED(1, 1); break; case 12: GR_RED(1, 2); break; case 14: GR_RED(1, 4); break;
@@ -378,11 +433,10 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     auto kern = en_.wlds > 0 ? k_energy<true> : k_energy<false>;
     if (lds > 48 * 1024)
       HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, en_, mu_.as<int>(), 0, n, rho_.as<double>(), grho_.as<double>(),
-                       fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), fl.energy_only ? 0 : 1, sid_ptr());
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream_, en_, mu_.as<int>(), a0, n, rho_.as<double>(), grho_.as<double>(),
+                       fl.eatom ? eatom_.as<double>() + a0 : nullptr, scal_.as<double>(), fl.energy_only ? 0 : 1, sid_ptr());
   });
   if (fl.uq) {
-    uq_gamma_.ensure(na * sizeof(double)); uq_sigma_.ensure(na * sizeof(double)); uq_cluster_.ensure(na * sizeof(double));
     stage("uq", [&] {
       UqDev<T> u = uq_;
       u.X[0] = A; u.X[1] = AA; u.X[2] = AAA; u.X[3] = AAAA;
@@ -390,23 +444,13 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
       auto kern = k_uq<T>;
       if (lds > 48 * 1024)
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-      hipLaunchKernelGGL(kern, dim3(n), dim3(256), lds, stream_, u, mu_.as<int>(), n, uq_gamma_.as<double>(), uq_sigma_.as<double>(),
-                         uq_cluster_.as<double>());
+      hipLaunchKernelGGL(kern, dim3(n), dim3(256), lds, stream_, u, mu, n, uq_gamma_.as<double>() + a0, uq_sigma_.as<double>() + a0,
+                         uq_cluster_.as<double>() + a0);
     });
-    ran_uq_ = true;
   }
   if (fl.energy_only) return;
 
   // ---- reverse
-  gA_.ensure(na * nlm_ * CP_ * sizeof(T));
-  gA1_.ensure(na * nlm_ * CFP_ * sizeof(T));
-  gAA_.ensure(na * nAA_ * CFP_ * sizeof(T));
-  gAA1_.ensure(na * nAA_ * CFP_ * sizeof(T));
-  gAAA_.ensure(na * nAAA_ * CFP_ * sizeof(T));
-  if (order4_) {
-    gAA2_.ensure(na * nAA_ * CFP_ * sizeof(T));
-    gAAAA_.ensure(na * nAAAA_ * CFP_ * sizeof(T));
-  }
   T *gA = gA_.as<T>(), *gA1 = gA1_.as<T>(), *gAA = gAA_.as<T>(), *gAA1 = gAA1_.as<T>(), *gAA2 = gAA2_.as<T>(),
     *gAAA = gAAA_.as<T>(), *gAAAA = gAAAA_.as<T>();
   stage("zero_grads", [&] {
@@ -427,7 +471,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   stage("reduce_rho_bwd", [&] {
     const int first = order4_ ? jobs_a_aa : 0;
     if (redrho_.njobs > first)
-      hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, redrho_.njobs - first), dim3(64), 0, stream_, redrho_.d, mu_.as<int>(), tiles, grho_.as<double>(),
+      hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles, redrho_.njobs - first), dim3(64), 0, stream_, redrho_.d, mu, tiles, grho_.as<double>(),
                          gA, gAA, gAAA, gAAAA, first);
   });
   // accL / accR: add to the stored adjoint or overwrite it (specialised kernels; the table-driven ones always add)
@@ -463,7 +507,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     });
     stage("reduce_rho_bwd_A_AA", [&] {
       if (jobs_a_aa > 0)
-        hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, jobs_a_aa), dim3(64), 0, stream_, redrho_.d, mu_.as<int>(), tiles, grho_.as<double>(), gA, gAA,
+        hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles, jobs_a_aa), dim3(64), 0, stream_, redrho_.d, mu, tiles, grho_.as<double>(), gA, gAA,
                            gAAA, gAAAA, 0);
     });
   } else {
@@ -474,11 +518,10 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
 
   BondBwdArgs<T> ba{};
   ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
-  ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = gA;
+  ba.Rz = Rz; ba.dRz = dRz; ba.gA = gA;
   ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
-  ba.a0 = 0; ba.C = CP_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;
+  ba.a0 = a0; ba.C = CP_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;
   stage("bond_bwd", [&] { launch_bond_bwd<T>(ba, n); });
-
 }
 
 template<class T> void Engine1L<T>::debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz)

@@ -538,12 +538,21 @@ class EngineBase : public Engine, protected BufRegistry {
     for (DevBuf *b : bufs_)
       if (!b->model_data) b->release();
     scal_.ensure(8 * sizeof(double));    // grown by a batch upload: an empty pass still clears and reads one record
+    chunk_laid_out_ = 0;
     n_ = 0;
     nb_ = 0;
     nstruct_ = 1;
     ran_ = ran_forces_ = ran_eatom_ = ran_uq_ = false;
   }
   void synchronize() override { check(hipSetDevice(device_), "hipSetDevice"); check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
+  void set_chunksize(int atoms) override
+  {
+    if (!chunks_ && atoms > 0)
+      throw InvalidArgument(who_ + ": this engine evaluates a structure in one pass; chunksize must be 0 (one pass) or -1 (auto), got " +
+                            std::to_string(atoms));
+    chunk_request_ = atoms;
+  }
+  int chunksize_used() const override { return chunk_used_; }
   void set_profile(bool on) override { profile_ = on; }
   const std::vector<StageTime> &stage_times() override
   {
@@ -622,6 +631,8 @@ class EngineBase : public Engine, protected BufRegistry {
     };
     put(mu_, mu.data(), sizeof(int) * n);
     if (have_sid_) put(sid_, in.sid, sizeof(int) * n);
+    mu_host_ = mu;
+    chunk_laid_out_ = 0;
     const std::vector<int> tiles = element_tiles(mu, nelem_, tile_el_);
     ntiles_ = (int) tiles.size() / 16;
     put(tiles_, tiles.data(), sizeof(int) * tiles.size());
@@ -665,6 +676,8 @@ class EngineBase : public Engine, protected BufRegistry {
       if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, kind, stream_));
     };
     put(mu_, mu.data(), sizeof(int) * n, hipMemcpyHostToDevice);
+    mu_host_ = mu;
+    chunk_laid_out_ = 0;
     const std::vector<int> tiles = element_tiles(mu, nelem_, tile_el_);
     ntiles_ = (int) tiles.size() / 16;
     put(tiles_, tiles.data(), sizeof(int) * tiles.size(), hipMemcpyHostToDevice);
@@ -724,13 +737,7 @@ class EngineBase : public Engine, protected BufRegistry {
     if (!ran_) throw Error("fetch() before run()");
     if (nstruct != nstruct_) throw InvalidArgument("fetch_batch: the uploaded list holds " + std::to_string(nstruct_) + " structures");
     HIP_CHECK(hipStreamSynchronize(stream_));
-    if (n_ > 0) {
-      int zb[2];
-      HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
-      if (zb[0] >= 0)    // bonds.h:49-62
-        throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " +
-                    std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
-    }
+    check_zero_bond();
     std::vector<double> s((size_t) 8 * nstruct_);
     HIP_CHECK(hipMemcpy(s.data(), scal_.p, s.size() * sizeof(double), hipMemcpyDeviceToHost));
     for (int q = 0; q < nstruct_; q++) {
@@ -746,18 +753,23 @@ class EngineBase : public Engine, protected BufRegistry {
     HIP_CHECK(hipSetDevice(device_));
     if (!ran_) throw Error("fetch() before run()");
     if (nstruct != nstruct_) throw InvalidArgument("fetch_batch: the uploaded list holds " + std::to_string(nstruct_) + " structures");
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    check_zero_bond();    // before anything is written to the caller's arrays
     hipLaunchKernelGGL(k_unpack_records, dim3((unsigned) ((nstruct_ + 255) / 256)), dim3(256), 0, stream_, scal_.as<double>(), nstruct_, energy,
                        ran_forces_ ? virial : nullptr);
     if (forces && ran_forces_ && n_ > 0) HIP_CHECK(hipMemcpyAsync(forces, f_.p, sizeof(double) * 3 * n_, hipMemcpyDeviceToDevice, stream_));
     if (eatom && ran_eatom_ && n_ > 0) HIP_CHECK(hipMemcpyAsync(eatom, eatom_.p, sizeof(double) * n_, hipMemcpyDeviceToDevice, stream_));
     HIP_CHECK(hipStreamSynchronize(stream_));
-    if (n_ > 0) {
-      int zb[2];
-      HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
-      if (zb[0] >= 0)    // bonds.h:49-62
-        throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " +
-                    std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
-    }
+  }
+  // two atoms at one position make a bond of length 0 (bonds.h:49-62 of the reference): reported by the pass in zero_
+  void check_zero_bond()
+  {
+    if (n_ == 0) return;
+    int zb[2];
+    HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
+    if (zb[0] >= 0)
+      throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " + std::to_string(zb[1]) +
+                  " of the neighbour list): not a physical structure");
   }
   void fetch_add_device(const int *atom, double *energy, double *forces, double *virial, double *eatom) override
   {
@@ -765,13 +777,7 @@ class EngineBase : public Engine, protected BufRegistry {
     if (!ran_) throw Error("fetch() before run()");
     if (have_sid_) throw Error("the uploaded list holds several structures: use fetch_batch()");
     HIP_CHECK(hipStreamSynchronize(stream_));
-    if (n_ > 0) {    // before anything is added to the caller's arrays
-      int zb[2];
-      HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
-      if (zb[0] >= 0)    // bonds.h:49-62
-        throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " +
-                    std::to_string(zb[1]) + " of the neighbour list): not a physical structure");
-    }
+    check_zero_bond();    // before anything is added to the caller's arrays
     const bool wf = forces && ran_forces_, we = eatom && ran_eatom_;
     if (n_ > 0 && (wf || we))
       hipLaunchKernelGGL(k_add_results, dim3((unsigned) ((n_ + 255) / 256)), dim3(256), 0, stream_, atom, n_, f_.as<double>(), wf ? forces : nullptr,
@@ -1047,6 +1053,68 @@ class EngineBase : public Engine, protected BufRegistry {
 #undef GR_GEMM_C
 #undef GR_GEMM
   }
+
+  // ---- chunks of atoms ---------------------------------------------------------------------------------------
+  // Atoms per pass for a structure whose work buffers take `per_atom` bytes per atom of a chunk and `kept` bytes per atom
+  // of the structure, after the reference's policy (libgrace/include/grace/kk/support.h:425-450): everything in one pass
+  // while that fits 70 % of the memory this engine can have (the free device memory, or what the library's own cap
+  // leaves, plus what its work buffers hold already), else the largest power of two >= 512 that fits.  Returns n for one pass.
+  int plan_chunk(int n, double per_atom, double kept)
+  {
+    if (n <= 0 || chunk_request_ == 0) return n;
+    if (chunk_request_ > 0) return std::min(n, chunk_request_);
+    size_t free_b = 0, total_b = 0;
+    HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    double avail = (double) free_b;
+    const long long cap = dev_bytes_limit().load();
+    if (cap > 0) avail = std::min(avail, (double) (cap - dev_bytes_in_use().load()));
+    double held = 0.0;
+    for (const DevBuf *b : bufs_)
+      if (!b->model_data) held += (double) b->bytes;
+    const double budget = 0.7 * (avail + held);
+    if (per_atom * 1.125 * n + kept * n <= budget) return n;
+    int c = std::min(n, kChunkFloor);
+    while (2 * c < n && per_atom * 1.125 * 2.0 * c + kept * n <= budget) c *= 2;
+    return c;
+  }
+  static constexpr int kChunkFloor = 512;    // smallest chunk of the automatic choice and of the retries after a failed allocation
+  // Tiles of 16 atoms of one element for every chunk of `cs` atoms, with atom indices counted from the chunk's first atom:
+  // chunk k owns tiles [chunk_tile_off_[k], chunk_tile_off_[k + 1]) of chunk_tiles_.
+  void layout_chunks(int cs)
+  {
+    if (chunk_laid_out_ == cs) return;
+    const int n = n_, nch = (n + cs - 1) / cs;
+    std::vector<int> all, el;
+    chunk_tile_off_.assign(1, 0);
+    for (int k = 0; k < nch; k++) {
+      const int a0 = k * cs, a1 = std::min(n, a0 + cs);
+      const std::vector<int> sub(mu_host_.begin() + a0, mu_host_.begin() + a1);
+      const std::vector<int> t = element_tiles(sub, nelem_, el);
+      all.insert(all.end(), t.begin(), t.end());
+      chunk_tile_off_.push_back((int) all.size() / 16);
+    }
+    upload_vec(chunk_tiles_, all);
+    chunk_laid_out_ = cs;
+  }
+  // first edge of every chunk (and the end of the last): eoff at the chunk boundaries, read back after the bond filter
+  std::vector<long long> chunk_edge_bounds(int cs)
+  {
+    const int nch = (n_ + cs - 1) / cs;
+    std::vector<long long> b((size_t) nch + 1);
+    for (int k = 0; k <= nch; k++)
+      HIP_CHECK(hipMemcpyAsync(&b[(size_t) k], eoff_.as<long long>() + std::min(n_, k * cs), sizeof(long long), hipMemcpyDeviceToHost, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    return b;
+  }
+  // a pointer moved back by `count` elements: kernels that index a chunk's buffer with structure-wide indices (edges)
+  template<class U> static U *moved_back(U *p, long long count)
+  {
+    return reinterpret_cast<U *>(reinterpret_cast<intptr_t>(p) - (intptr_t) (count * (long long) sizeof(U)));
+  }
+  bool chunks_ = false;          // the engine can evaluate a structure in chunks of atoms
+  int chunk_request_ = -1, chunk_used_ = 0, chunk_laid_out_ = 0;
+  std::vector<int> mu_host_, chunk_tile_off_;
+  DevBuf chunk_tiles_;
 
   int device_, ncu_ = 256;
   std::string arch_, who_;

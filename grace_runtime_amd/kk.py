@@ -180,6 +180,14 @@ class Engine:
     def cutoff(self, t1: int, t2: int) -> float:
         return _lib.lib().gr_engine_cutoff(self._h, int(t1), int(t2))
 
+    def set_chunksize(self, atoms: int):
+        """atoms per engine pass: 0 one pass, < 0 automatic, > 0 as given"""
+        check(_lib.lib().gr_engine_set_chunksize(self._h, int(atoms)))
+
+    @property
+    def chunksize(self) -> int:
+        return int(_lib.lib().gr_engine_chunksize(self._h))
+
     def release_buffers(self):
         """frees the work buffers and the uploaded structure; weights, tables and compiled kernels stay"""
         check(_lib.lib().gr_engine_release_buffers(self._h))
@@ -466,9 +474,11 @@ class System:
         self.engine = Engine(model, species, precision)
         self.skin = skin
         self.cutoff = float(self.engine.cutoff_matrix().max()) if len(species) else 0.0
-        self.chunksize = 0
         self._h = C.c_void_p()
         check(_lib.lib().gr_system_create(self.engine._h, skin, C.byref(self._h)))
+        # atoms per engine pass: 0 one pass, < 0 from the free device memory, > 0 as given (ValueError for a model kind
+        # that is evaluated in one pass only)
+        check(_lib.lib().gr_system_set_chunksize(self._h, int(chunksize)))
 
     def __del__(self):
         if getattr(self, "_h", None) is not None and self._h.value:
@@ -478,6 +488,11 @@ class System:
     @property
     def rebuilds(self) -> int:
         return int(_lib.lib().gr_system_rebuilds(self._h))
+
+    @property
+    def chunksize(self) -> int:
+        """atoms per engine pass in the last compute (0: one pass), python/kk/kk_api.h:86"""
+        return int(_lib.lib().gr_system_chunksize(self._h))
 
     @property
     def list_on_device(self) -> bool:
@@ -544,8 +559,13 @@ class Batch:
         self.cutoff = float(self.engine.cutoff_matrix().max()) if len(species) else 0.0
         self.passes = 0
         self.keep_buffers = False
-        self.chunksize = 0
+        self.engine.set_chunksize(int(chunksize))    # atoms per engine pass within a batch pass (0 one pass, < 0 automatic)
         self._nall_cap = 1 << 62    # atoms per pass after an allocation failure (python/kk/kk_core.cpp:1461: nall_cap)
+
+    @property
+    def chunksize(self) -> int:
+        """atoms per engine pass in the last compute (0: one pass)"""
+        return self.engine.chunksize
 
     def release_buffers(self):
         """frees the engine's work buffers (python/kk/kk_api.h:116-156)"""

@@ -211,6 +211,17 @@ int gr_system_create(gr_engine *e, double skin, gr_system **out);
 void gr_system_free(gr_system *s);
 int gr_system_compute(gr_system *s, int n, const int *types, const double *positions, const double *cell, const unsigned char *pbc,
                       unsigned flags, double *energy, double *forces, double *virial, double *eatom);
+/* Atoms per engine pass, which bounds the device memory of a large structure (System(chunksize) and System::chunksize()
+ * of the reference's GPU module, python/kk/kk_api.h:72-75,86; the engines' chunksize, kk/grace_1l_kk.h:72-113; automatic
+ * choice libgrace/include/grace/kk/support.h:425-450).  atoms = 0: all atoms in one pass; < 0 (the default): chosen from
+ * the free device memory: one pass while the work buffers fit 70 % of it, else the largest power of two >= 512 that
+ * fits, and halved (down to 512) when an allocation still fails; > 0: as given.  gr_*_chunksize: atoms per pass of the last
+ * call, 0 for one pass.  GRACE-1L engines evaluate chunks; the GRACE-2L and GRACE-3L engines evaluate a structure in one
+ * pass and give GR_INVALID for atoms > 0. */
+int gr_engine_set_chunksize(gr_engine *e, int atoms);
+int gr_engine_chunksize(const gr_engine *e);
+int gr_system_set_chunksize(gr_system *s, int atoms);
+int gr_system_chunksize(const gr_system *s);
 int gr_system_rebuilds(const gr_system *s);
 int gr_system_list_on_device(const gr_system *s);
 int gr_system_list_sizes(gr_system *s, int64_t *nbonds, int64_t *nimages);
