@@ -13,11 +13,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgrace_hip.so")
 
 GR_OK, GR_INVALID, GR_ERROR, GR_NOMEM = 0, 1, 2, 3
-FLAG_ENERGY_ONLY, FLAG_EATOM, FLAG_UQ = 1, 2, 4
+FLAG_ENERGY_ONLY, FLAG_EATOM, FLAG_UQ, FLAG_ACCUMULATE = 1, 2, 4, 8
 
 # every symbol include/grace_hip.h declares (checked by the CPU test-suite against the header and the library)
 SYMBOLS = [
-    "gr_last_error", "gr_abi_version", "gr_device_count", "gr_device_arch", "gr_model_load", "gr_model_get_info",
+    "gr_last_error", "gr_set_logger", "gr_abi_version", "gr_device_count", "gr_device_arch", "gr_model_load", "gr_model_get_info",
     "gr_model_element_name", "gr_model_free", "gr_engine_create", "gr_engine_free", "gr_engine_cutoff",
     "gr_compute_csr", "gr_engine_upload", "gr_engine_run", "gr_engine_sync", "gr_engine_fetch",
     "gr_engine_edge_count", "gr_engine_set_profile", "gr_engine_stage_count", "gr_engine_stage_get", "gr_engine_stage_flops",
@@ -25,7 +25,7 @@ SYMBOLS = [
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
     "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_batch_uq", "gr_compute_batch_device_uq", "gr_engine_reset", "gr_engine_release_buffers", "gr_set_memory_limit", "gr_memory_in_use", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
-    "gr_system_fetch_uq", "gr_engine_set_chunksize", "gr_engine_chunksize", "gr_system_set_chunksize", "gr_system_chunksize",
+    "gr_system_fetch_uq", "gr_engine_atoms_that_fit", "gr_engine_set_chunksize", "gr_engine_chunksize", "gr_system_set_chunksize", "gr_system_chunksize",
 ]
 
 
@@ -55,6 +55,8 @@ def lib():
     L = C.CDLL(LIB_PATH)
     vp, i32, i64, dbl, u32 = C.c_void_p, C.c_int, C.c_int64, C.c_double, C.c_uint
     L.gr_last_error.restype = C.c_char_p
+    L.gr_set_logger.restype = None
+    L.gr_set_logger.argtypes = [vp, vp]
     L.gr_abi_version.restype = i32
     L.gr_device_count.restype = i32
     L.gr_device_arch.argtypes = [i32, C.c_char_p, i32]
@@ -86,6 +88,8 @@ def lib():
     L.gr_engine_debug_radial.argtypes = [vp, i32, vp, vp, vp, vp]
     L.gr_engine_stage_flops.argtypes = [vp, i32, vp]
     L.gr_engine_set_chunksize.argtypes = [vp, i32]
+    L.gr_engine_atoms_that_fit.argtypes = [vp]
+    L.gr_engine_atoms_that_fit.restype = i64
     L.gr_engine_chunksize.argtypes = [vp]
     L.gr_system_set_chunksize.argtypes = [vp, i32]
     L.gr_system_chunksize.argtypes = [vp]

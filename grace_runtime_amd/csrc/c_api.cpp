@@ -140,6 +140,11 @@ extern "C" {
 
 const char *gr_last_error(void) { return g_err.c_str(); }
 int gr_abi_version(void) { return 7; }
+void gr_set_logger(gr_log_fn fn, void *user)
+{
+  grhip::log_sink().user.store(user);
+  grhip::log_sink().fn.store(fn);
+}
 
 int gr_device_count(void)
 {
@@ -360,7 +365,19 @@ int gr_compute_csr(gr_engine *e, int n, const int *types, const int64_t *offset,
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
     live(e).run(fl);
-    live(e).fetch(energy, forces, virial, eatom);
+    if (!(flags & GR_FLAG_ACCUMULATE)) {
+      live(e).fetch(energy, forces, virial, eatom);
+      return;
+    }
+    // Outputs of the reference accumulate (libgrace/include/grace/system.h:66-75): add to what the caller's arrays hold
+    double en = 0.0, vir[6] = {0, 0, 0, 0, 0, 0};
+    std::vector<double> f(forces && !fl.energy_only ? (size_t) 3 * n : 0), ea(fl.eatom ? (size_t) n : 0);
+    live(e).fetch(&en, f.empty() ? nullptr : f.data(), vir, ea.empty() ? nullptr : ea.data());
+    if (energy) *energy += en;
+    if (virial && !fl.energy_only)
+      for (int k = 0; k < 6; k++) virial[k] += vir[k];
+    for (size_t q = 0; q < f.size(); q++) forces[q] += f[q];
+    for (size_t q = 0; q < ea.size(); q++) eatom[q] += ea[q];
   });
 }
 
@@ -803,6 +820,7 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
                              "; use a GPU with more memory or a smaller chunksize");
         int next = 512;
         while (2 * next < used) next *= 2;
+        grhip::log_message(1, "device allocation failed with " + std::to_string(used) + " atoms per pass; trying again with " + std::to_string(next));
         try {
           eng.set_chunksize(next);
         } catch (const grhip::InvalidArgument &) {    // an engine that evaluates structures in one pass only
@@ -824,6 +842,13 @@ int gr_system_set_chunksize(gr_system *s, int atoms)
 }
 
 int gr_system_chunksize(const gr_system *s) { return s && s->eng && s->eng->eng ? s->eng->eng->chunksize_used() : 0; }
+
+int64_t gr_engine_atoms_that_fit(gr_engine *e)
+{
+  int64_t r = 0;
+  guarded([&] { r = live(e).atoms_that_fit(); });
+  return r;
+}
 
 int gr_engine_set_chunksize(gr_engine *e, int atoms)
 {
@@ -1132,7 +1157,8 @@ int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, con
       grhip::BatchDeviceNeighbors &nl = *e->bnl;
       for (int g0 = 0; g0 < nstruct;) {
         int g1 = g0 + 1;
-        while (g1 < nstruct && start[g1 + 1] - start[g0] <= limit) g1++;
+        const int64_t fit = std::min<int64_t>(limit, live(e).atoms_that_fit());    // what the device memory holds, once a pass has shown it
+        while (g1 < nstruct && start[g1 + 1] - start[g0] <= fit) g1++;
         const int ns = g1 - g0;
         const int64_t a0 = start[g0], na = start[g1] - a0;
         nl.build(ns, natoms + g0, positions + 3 * a0, cells + 9 * (size_t) g0, pbc + 3 * (size_t) g0, rc, e->bnl_stream);
@@ -1173,6 +1199,7 @@ int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, con
           throw grhip::Error("the batch (" + std::to_string(N) + " atoms) does not fit the GPU memory even in passes of " + std::to_string(tried) +
                              " atoms; use a GPU with more memory");
         limit = e->nall_cap = std::max<int64_t>(16384, tried / 2);
+        grhip::log_message(1, "device allocation failed with batch passes of " + std::to_string(tried) + " atoms; trying again with " + std::to_string(limit));
       }
     }
   });

@@ -87,6 +87,10 @@ class Engine {
   // atoms per engine pass (python/kk/kk_api.h:72-75): 0 all atoms in one pass, < 0 chosen from the free device memory
   // (one pass while it fits, else the largest power of two >= 512 that fits), > 0 as given.  chunksize_used(): atoms per
   // pass of the last run (0: one pass).  Engines that do not chunk refuse values other than 0 and -1.
+  // atoms of one pass whose work buffers fit 70 % of the memory the library may use, from the bytes per atom that the
+  // buffers of the last pass hold; before the first pass: a bound by model kind.  The batch entry points size their
+  // passes with it (the reference sizes the first pass from the free memory: libgrace/include/grace/kk/support.h:425-450)
+  virtual int64_t atoms_that_fit() = 0;
   virtual void set_chunksize(int atoms) = 0;
   virtual int chunksize_used() const = 0;
   virtual void release_buffers() = 0;    // frees the work buffers and the uploaded structure; weights stay

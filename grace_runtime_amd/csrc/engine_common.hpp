@@ -22,6 +22,25 @@ namespace grhip {
       throw Error(std::string("HIP error: ") + hipGetErrorString(e_) + " in " #expr " (" __FILE__ ":" + std::to_string(__LINE__) + ")"); \
   } while (0)
 
+// Messages of the library (choice of a chunk, retries after a failed allocation, kernels that fall back to their
+// table-driven form) go to a callback the caller installs, as the reference's grace::Logger (libgrace/include/grace/
+// error.h:10-15): fn(user, level, message), level 0 information, 1 warning.  Without a callback they are dropped.
+typedef void (*LogCallback)(void *user, int level, const char *message);
+struct LogSink {
+  std::atomic<LogCallback> fn{nullptr};
+  std::atomic<void *> user{nullptr};
+};
+inline LogSink &log_sink()
+{
+  static LogSink s;
+  return s;
+}
+inline void log_message(int level, const std::string &m)
+{
+  const LogCallback f = log_sink().fn.load();
+  if (f) f(log_sink().user.load(), level, m.c_str());
+}
+
 // Device memory held by the library's buffers and an optional cap on it (0: none).  With a cap an allocation that would
 // pass it fails like one the device refuses (std::bad_alloc), which lets a GPU be shared by budget and lets the
 // retry paths be exercised without exhausting the device.
@@ -539,6 +558,7 @@ class EngineBase : public Engine, protected BufRegistry {
       if (!b->model_data) b->release();
     scal_.ensure(8 * sizeof(double));    // grown by a batch upload: an empty pass still clears and reads one record
     chunk_laid_out_ = 0;
+    n_peak_ = 0;
     n_ = 0;
     nb_ = 0;
     nstruct_ = 1;
@@ -553,6 +573,23 @@ class EngineBase : public Engine, protected BufRegistry {
     chunk_request_ = atoms;
   }
   int chunksize_used() const override { return chunk_used_; }
+  int64_t atoms_that_fit() override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (chunks_ && chunk_request_ < 0) return INT64_MAX;    // the engine splits a pass that does not fit by itself
+    if (n_peak_ <= 0 || chunk_used_ > 0) return layers() == 3 ? 16384 : layers() == 2 ? 131072 : 262144;
+    double held = 0.0;
+    for (const DevBuf *b : bufs_)
+      if (!b->model_data) held += (double) b->bytes;
+    size_t free_b = 0, total_b = 0;
+    HIP_CHECK(hipMemGetInfo(&free_b, &total_b));
+    double avail = (double) free_b;
+    const long long cap = dev_bytes_limit().load();
+    if (cap > 0) avail = std::min(avail, (double) (cap - dev_bytes_in_use().load()));
+    // the buffers grew to the largest pass since they were last released: that pass fits, and sets the bytes per atom
+    const double per_atom = std::max(held / n_peak_, 1.0);
+    return std::max<int64_t>(n_peak_, (int64_t) (0.7 * (avail + held) / per_atom));
+  }
   void set_profile(bool on) override { profile_ = on; }
   const std::vector<StageTime> &stage_times() override
   {
@@ -840,6 +877,7 @@ class EngineBase : public Engine, protected BufRegistry {
     HIP_CHECK(hipMemsetAsync(f_.p, 0, (size_t) 3 * n * sizeof(double), stream_));
     HIP_CHECK(hipMemsetAsync(scal_.p, 0, (size_t) 8 * nstruct_ * sizeof(double), stream_));
     ran_ = true;
+    n_peak_ = std::max(n_peak_, n_);
     ran_forces_ = !fl.energy_only;
     ran_eatom_ = fl.eatom;
     ran_uq_ = false;    // set by the engine that evaluates a UQ head
@@ -1075,6 +1113,10 @@ class EngineBase : public Engine, protected BufRegistry {
     if (per_atom * 1.125 * n + kept * n <= budget) return n;
     int c = std::min(n, kChunkFloor);
     while (2 * c < n && per_atom * 1.125 * 2.0 * c + kept * n <= budget) c *= 2;
+    log_message(0, who_ + ": chunksize auto: " + std::to_string(c) + " atoms per pass for " + std::to_string(n) + " atoms (" +
+                       std::to_string((long long) (per_atom * 1000 / 1048576)) + " MB of work buffers and " +
+                       std::to_string((long long) (kept * 1000 / 1048576)) + " MB kept per 1000 atoms, " + std::to_string((long long) (avail / 1048576)) +
+                       " MB of device memory available)");
     return c;
   }
   static constexpr int kChunkFloor = 512;    // smallest chunk of the automatic choice and of the retries after a failed allocation
@@ -1123,7 +1165,7 @@ class EngineBase : public Engine, protected BufRegistry {
   int nelem_;
   std::vector<double> cut_host_;
   // uploaded structure
-  int n_ = 0;
+  int n_ = 0, n_peak_ = 0;    // atoms of the uploaded structure; of the largest pass since the work buffers were released
   int64_t nb_ = 0;
   bool have_rij_ = false;
   DevBuf cut_, mu_, sid_, offset_, j_, rij_, x_, image_, shifts_, tiles_;

@@ -95,6 +95,22 @@ def _dev():
     return _state["device"]
 
 
+_LOG_FN = C.CFUNCTYPE(None, C.c_void_p, C.c_int, C.c_char_p)
+_log_keepalive = None
+
+
+def set_logger(fn):
+    """fn(level, message) receives the library's messages (level 0 information, 1 warning); None switches them off"""
+    global _log_keepalive
+    if fn is None:
+        _lib.lib().gr_set_logger(None, None)
+        _log_keepalive = None
+        return
+    cb = _LOG_FN(lambda user, level, msg: fn(int(level), msg.decode(errors="replace")))
+    _lib.lib().gr_set_logger(C.cast(cb, C.c_void_p), None)
+    _log_keepalive = cb
+
+
 def neighbor_search(positions, cell, pbc, cutoff, num_threads: int = 0):
     """(perm, offset, j, image, shifts) of the Verlet list at `cutoff`; identical to the reference list
     (python/src/neighbors.cpp:15-95)."""
@@ -287,11 +303,18 @@ class Engine:
         return out
 
     def compute(self, types, offset, j, rij=None, energies=False, energy_only=False, positions=None, image=None,
-                shifts=None):
+                shifts=None, add_to=None):
+        """add_to: a result of an earlier call (energy, forces, virial, energies) that this call's outputs are ADDED to,
+        as the reference's Outputs accumulate"""
         n, arrs, nimg = self._csr_args(types, offset, j, rij, positions, image, shifts)
         flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
         e = C.c_double(0.0)
         f, v, ea = np.zeros((n, 3)), np.zeros(6), np.zeros(n)
+        if add_to is not None:
+            flags |= _lib.FLAG_ACCUMULATE
+            e = C.c_double(float(add_to["energy"]))
+            f, v = np.array(add_to.get("forces", f), dtype=np.float64), np.array(add_to.get("virial", v), dtype=np.float64)
+            ea = np.array(add_to.get("energies", ea), dtype=np.float64)
         check(_lib.lib().gr_compute_csr(self._h, n, *[ptr(a) for a in arrs], nimg, flags, C.addressof(e), ptr(f), ptr(v),
                                         ptr(ea) if energies else None))
         out = {"energy": e.value}
@@ -612,7 +635,9 @@ class Batch:
                 self.passes, g0 = 0, 0
                 while g0 < S:
                     g1 = g0 + 1
-                    while g1 < S and start[g1 + 1] - start[g0] <= limit:
+                    # what the device memory holds, once a pass has shown the engine's bytes per atom
+                    fit = min(limit, int(_lib.lib().gr_engine_atoms_that_fit(self.engine._h)))
+                    while g1 < S and start[g1 + 1] - start[g0] <= fit:
                         g1 += 1
                     a0, a1 = int(start[g0]), int(start[g1])
                     check(_lib.lib().gr_compute_batch_uq(self.engine._h, g1 - g0, ptr(natoms[g0:g1]), ptr(types[a0:a1]), ptr(pos[a0:a1]),

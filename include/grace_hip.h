@@ -31,7 +31,9 @@ enum {
 enum {
   GR_FLAG_ENERGY_ONLY = 1, /* ComputeFlags::energy_only (libgrace/include/grace/system.h:118): no forces / virial */
   GR_FLAG_EATOM = 2,       /* ComputeFlags::eflag_atom (system.h:114): per-atom energies */
-  GR_FLAG_UQ = 4           /* ComputeFlags::uq (system.h:117): the UQ head; gr_engine_run and gr_system_compute */
+  GR_FLAG_UQ = 4,          /* ComputeFlags::uq (system.h:117): the UQ head; gr_engine_run and gr_system_compute */
+  GR_FLAG_ACCUMULATE = 8   /* gr_compute_csr: energy, forces, virial and per-atom energies are ADDED to the caller's values, as
+                              the reference's Outputs accumulate (system.h:66-75); without it they are overwritten */
 };
 
 typedef struct gr_model_info {
@@ -46,6 +48,11 @@ typedef struct gr_model_info {
 
 /* message of the last failed call on this thread ("" if none).  grace::Error::what(). */
 const char *gr_last_error(void);
+/* Messages of the library (the automatic chunk, retries after a failed allocation): fn(user, level, message) with level 0
+ * information, 1 warning -- the callback of grace::Logger (libgrace/include/grace/error.h:10-15).  NULL: dropped (default).
+ * The callback may be called from any thread that calls into the library. */
+typedef void (*gr_log_fn)(void *user, int level, const char *message);
+void gr_set_logger(gr_log_fn fn, void *user);
 /* library ABI version (the Python plug-in contract uses ABI = 7: python/grace_runtime/_gpu.py:18) */
 int gr_abi_version(void);
 /* number of HIP devices; gfx arch name of a device into buf ("" on failure).  _kk.arch(), _kk.initialize(device):
@@ -92,8 +99,8 @@ double gr_engine_cutoff(const gr_engine *e, int t1, int t2);
 /* One call on caller-supplied CSR bonds = _core.Model.compute (python/src/core.cpp:292-396) =
  * Grace1LFused::compute<CsrBonds>(n, nullptr, n, n, src, out, flags, nthreads) (fused_1l.h:41):
  * bonds of atom i are [offset[i], offset[i+1]); give rij [nb][3] or (positions [n][3], image [nb], shifts [nimages][3]).
- * types are 1-based.  Outputs are OVERWRITTEN (not accumulated): energy, forces [n][3], virial[6] = xx yy zz xy xz yz,
- * eatom [n] (with GR_FLAG_EATOM); null outputs are skipped.  Same argument errors as the reference binding. */
+ * types are 1-based.  Outputs: energy, forces [n][3], virial[6] = xx yy zz xy xz yz, eatom [n] (with GR_FLAG_EATOM);
+ * overwritten, or added to with GR_FLAG_ACCUMULATE; null outputs are skipped.  Same argument errors as the reference binding. */
 int gr_compute_csr(gr_engine *e, int n, const int *types, const int64_t *offset, const int *j, const double *rij,
                    const double *positions, const int *image, const double *shifts, int64_t nimages, unsigned flags,
                    double *energy, double *forces, double *virial, double *eatom);
@@ -218,6 +225,11 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
  * fits, and halved (down to 512) when an allocation still fails; > 0: as given.  gr_*_chunksize: atoms per pass of the last
  * call, 0 for one pass.  GRACE-1L engines evaluate chunks; the GRACE-2L and GRACE-3L engines evaluate a structure in one
  * pass and give GR_INVALID for atoms > 0. */
+/* Atoms of one pass whose work buffers fit 70 % of the device memory the library may use, from the bytes per atom the
+ * last pass held (before any pass: 262144 / 131072 / 16384 atoms for GRACE-1L / 2L / 3L).  The batch entry points bound
+ * their passes by it, as the reference sizes a batch pass from the free memory (libgrace/include/grace/kk/support.h:425-450,
+ * python/kk/kk_core.cpp:1311-1347). */
+int64_t gr_engine_atoms_that_fit(gr_engine *e);
 int gr_engine_set_chunksize(gr_engine *e, int atoms);
 int gr_engine_chunksize(const gr_engine *e);
 int gr_system_set_chunksize(gr_system *s, int atoms);

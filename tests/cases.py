@@ -157,10 +157,16 @@ LAYERS = {"uq3l": 3, "uq2l": 2, "uq2": 1, "l3mix": 3, "l3wide": 3, "l3pad": 3, "
 
 
 def write_model(name, directory):
+    """the model's kokkos.npz in `directory`, written on first use (atomically: workers of a parallel run share the directory)"""
     path = os.path.join(directory, f"{name}.npz")
     if not os.path.exists(path):
-        synth.save_model(path, MODELS[name]())
+        tmp = os.path.join(directory, f".{name}.{os.getpid()}.npz")
+        synth.save_model(tmp, MODELS[name]())
+        os.replace(tmp, path)
     return path
+
+
+model_file = lambda directory, name: write_model(name, directory)    # noqa: E731  (argument order of os.path.join)
 
 
 def structure_alloy54(seed=3):

@@ -17,11 +17,19 @@ def pytest_configure(config):
 
 
 @pytest.fixture(scope="session")
-def model_dir(tmp_path_factory):
-    """directory holding the synthetic models of tests/cases.py as kokkos.npz files"""
-    d = str(tmp_path_factory.mktemp("models"))
-    for name in cases.MODELS:
-        cases.write_model(name, d)
+def model_dir():
+    """Directory of the synthetic models of tests/cases.py as kokkos.npz files.  A model is written when a test first asks
+    for it (cases.model_file); the directory is shared by the workers of a run and by later runs as long as the
+    generators do not change (its name carries a digest of their sources)."""
+    import hashlib
+    import tempfile
+    h = hashlib.sha256()
+    for f in (os.path.join(ROOT, "grace_runtime_amd", "synth.py"), os.path.join(ROOT, "grace_runtime_amd", "workloads.py"),
+              os.path.join(ROOT, "tests", "cases.py")):
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    d = os.path.join(tempfile.gettempdir(), "grace_hip_test_models_" + h.hexdigest()[:16])
+    os.makedirs(d, exist_ok=True)
     return d
 
 

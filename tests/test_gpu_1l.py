@@ -37,7 +37,7 @@ def engines(model_dir):
     def get(name, species, precision=64, fixture=False):
         key = (name, tuple(species), precision)
         if key not in cache:
-            path = os.path.join(cases.REF_FIXTURES if fixture else model_dir, name + ".npz")
+            path = (os.path.join(cases.REF_FIXTURES, name + ".npz") if fixture else cases.model_file(model_dir, name))
             cache[key] = kk.Engine(kk.Model(path), species, precision)
         return cache[key]
     return get
@@ -57,7 +57,7 @@ def test_device_is_gfx950():
 def test_radial_mfma_kernel_matches_oracle(engines, model_dir, name, fixture, species, precision):
     """R_nl(x) z[mu_j] and d/dx of the MFMA kernel against radial_x.h restated in numpy (also ragged tile counts)"""
     eng = engines(name, species, precision, fixture)
-    om = go.Model1L(os.path.join(cases.REF_FIXTURES if fixture else model_dir, name + ".npz"))
+    om = go.Model1L((os.path.join(cases.REF_FIXTURES, name + ".npz") if fixture else cases.model_file(model_dir, name)))
     for m in (1, 15, 16, 17, 1000):
         x = np.linspace(0.02, 0.9995, m) if m > 1 else np.array([0.37])
         mu = (np.arange(m) * 7) % om.n_elements
@@ -93,7 +93,7 @@ def test_matches_tf_fp64_goldens(engines, tf_gold, name, cell, precision):
 @pytest.mark.parametrize("precision", [64, 32])
 @pytest.mark.parametrize("model,struct,rc", cases.E2E_CASES)
 def test_matches_oracle_and_compiled_reference(engines, model_dir, gold, model, struct, rc, precision):
-    om = go.Model1L(os.path.join(model_dir, model + ".npz"))
+    om = go.Model1L(cases.model_file(model_dir, model))
     species = om.names
     eng = engines(model, species, precision)
     pos, cell, pbc, types = cases.STRUCTURES[struct]()

@@ -41,7 +41,7 @@ def engines(model_dir):
     def get(name, species, fixture=False, precision=64):
         key = (name, tuple(species), precision)
         if key not in cache:
-            path = os.path.join(cases.REF_FIXTURES if fixture else model_dir, name + ".npz")
+            path = (os.path.join(cases.REF_FIXTURES, name + ".npz") if fixture else cases.model_file(model_dir, name))
             cache[key] = kk.Engine(kk.Model(path), species, precision)
         return cache[key]
     return get
@@ -82,7 +82,7 @@ def test_fixture_models_match_oracle_and_compiled_reference(engines, gold, model
 @pytest.mark.parametrize("precision", [64, 32])
 @pytest.mark.parametrize("model,struct,rc", cases.E2E_CASES_2L)
 def test_matches_oracle_and_compiled_reference(engines, model_dir, gold, model, struct, rc, precision):
-    om = g2.Model2L(os.path.join(model_dir, model + ".npz"))
+    om = g2.Model2L(cases.model_file(model_dir, model))
     eng = engines(model, om.names, False, precision)
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     types = np.minimum(types, om.n_elements).astype(np.int32)

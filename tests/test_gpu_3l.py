@@ -43,7 +43,7 @@ def engines(model_dir):
 
     def get(name, precision=64):
         if (name, precision) not in cache:
-            path = os.path.join(model_dir, name + ".npz")
+            path = cases.model_file(model_dir, name)
             om = g3.Model3L(path)
             cache[(name, precision)] = (kk.Engine(kk.Model(path), _names(om), precision), om)
         return cache[(name, precision)]

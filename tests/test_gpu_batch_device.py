@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 
 def _engine(model_dir, name, species):
-    return kk.Engine(kk.Model(os.path.join(model_dir, name + ".npz")), species, 64)
+    return kk.Engine(kk.Model(cases.model_file(model_dir, name)), species, 64)
 
 
 def _pack(structs):
@@ -167,7 +167,9 @@ def test_allocation_failure_halves_the_passes_and_keeps_the_limit(model_dir):
         host = b.compute(natoms, types, pos, cells, pbc, energies=True)
         assert b.passes >= 2
         _compare(host, ref)
-        # nothing fits: an error that says so, and an engine that works again once the cap is lifted
+        # nothing fits (the buffers of the passes that fitted are given back first): an error that says so, and an engine
+        # that works again once the cap is lifted
+        b.release_buffers()
         kk.set_memory_limit(base + (held - base) // 50)
         with pytest.raises(RuntimeError, match="does not fit the GPU memory"):
             _device_run(b, natoms, types, pos, cells, pbc)
@@ -181,7 +183,7 @@ def test_allocation_failure_halves_the_passes_and_keeps_the_limit(model_dir):
 
 
 def test_engine_reset_is_seen_by_a_system(model_dir):
-    model = kk.Model(os.path.join(model_dir, "mix2.npz"))
+    model = kk.Model(cases.model_file(model_dir, "mix2"))
     s = kk.System(model, ["Mo", "W"], skin=0.3)
     p, c, pb, t = cases.structure_alloy54()
     a = s.compute(t, p, c, pb)
@@ -194,7 +196,7 @@ def test_release_buffers_gives_the_work_memory_back(model_dir):
     """Batch.release_buffers / keep_buffers and System.release_buffers (python/kk/kk_api.h:66-156): after a release the
     library holds what it held right after the engine was made (weights, tables), and the next call gives the same
     results"""
-    model = kk.Model(os.path.join(model_dir, "l2mix.npz"))
+    model = kk.Model(cases.model_file(model_dir, "l2mix"))
     structs = [cases.structure_alloy54(), cases.structure_triclinic(), cases.structure_slab()]
     natoms, types, pos, cells, pbc = _pack(structs)
     before = kk.memory_in_use()

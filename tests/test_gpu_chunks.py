@@ -28,7 +28,7 @@ def test_chunked_pass_equals_one_pass(model_dir, model, struct, species, precisi
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     types = np.minimum(types, len(species)).astype(np.int32)
     n = len(pos)
-    m = kk.Model(os.path.join(model_dir, model + ".npz"))
+    m = kk.Model(cases.model_file(model_dir, model))
     one = kk.System(m, species, skin=0.0, chunksize=0, precision=precision)
     ref = one.compute(types, pos, cell, pbc, energies=True)
     assert one.chunksize == 0
@@ -45,7 +45,7 @@ def test_chunked_pass_equals_one_pass(model_dir, model, struct, species, precisi
 
 def test_chunked_uq_and_energy_only(model_dir):
     pos, cell, pbc, types = cases.structure_alloy54()
-    m = kk.Model(os.path.join(model_dir, "uq2.npz"))
+    m = kk.Model(cases.model_file(model_dir, "uq2"))
     ref = kk.System(m, ["Mo", "W"], skin=0.0, chunksize=0).compute(types, pos, cell, pbc, uq=True, energies=True)
     s = kk.System(m, ["Mo", "W"], skin=0.0, chunksize=13)
     out = s.compute(types, pos, cell, pbc, uq=True, energies=True)
@@ -62,7 +62,7 @@ def test_chunked_batch_equals_one_pass(model_dir):
     structs = workloads.structures_config5(6)
     natoms, types, pos, cells, pbc = workloads.batch_arrays(structs)
     types = np.minimum(types, 2).astype(np.int32)
-    m = kk.Model(os.path.join(model_dir, "mix2.npz"))
+    m = kk.Model(cases.model_file(model_dir, "mix2"))
     ref = kk.Batch(m, ["Mo", "W"], chunksize=0).compute(natoms, types, pos, cells, pbc, energies=True)
     b = kk.Batch(m, ["Mo", "W"], chunksize=50)
     out = b.compute(natoms, types, pos, cells, pbc, energies=True)
@@ -85,11 +85,14 @@ def test_automatic_chunk_follows_the_memory_the_library_may_use(tmp_path):
     assert s.chunksize == 0                              # fits: one pass
     _same(out, ref, len(pos))
     s.release_buffers()
+    said = []
+    kk.set_logger(lambda level, msg: said.append((level, msg)))
     try:
         s2 = kk.System(m, ["W"], skin=0.0)
         L.gr_set_memory_limit(L.gr_memory_in_use() + 900 * 1024 * 1024)
         out = s2.compute(types, pos, cell, pbc)
         assert s2.chunksize == 1024                      # the largest power of two whose work buffers fit 70 % of 900 MB
+        assert any(level == 0 and "chunksize auto: 1024 atoms per pass" in msg for level, msg in said)
         _same(out, ref, len(pos))
         # a fixed chunk that does not fit: reported, not retried
         s2.release_buffers()
@@ -101,18 +104,32 @@ def test_automatic_chunk_follows_the_memory_the_library_may_use(tmp_path):
         L.gr_set_memory_limit(L.gr_memory_in_use() + 60 * 1024 * 1024)
         with pytest.raises(RuntimeError, match="does not fit"):
             s2.compute(types, pos, cell, pbc)
+        assert any(level == 0 and "chunksize auto: 512 atoms per pass" in msg for level, msg in said)
     finally:
         L.gr_set_memory_limit(0)
+        kk.set_logger(None)
     out = s2.compute(types, pos, cell, pbc)              # the engine is usable again
     _same(out, ref, len(pos))
 
 
 @pytest.mark.parametrize("model", ["l2mix", "l3mix"])
 def test_model_kinds_that_run_in_one_pass_refuse_a_chunk_size(model_dir, model):
-    m = kk.Model(os.path.join(model_dir, model + ".npz"))
+    m = kk.Model(cases.model_file(model_dir, model))
     with pytest.raises(ValueError, match="one pass"):
         kk.System(m, ["Mo", "W"], chunksize=64)
     s = kk.System(m, ["Mo", "W"], chunksize=-1)
     pos, cell, pbc, types = cases.structure_alloy54()
     s.compute(types, pos, cell, pbc)
     assert s.chunksize == 0
+
+
+def test_outputs_accumulate_on_request(model_dir):
+    """GR_FLAG_ACCUMULATE: the outputs of a call are added to the caller's values (libgrace/include/grace/system.h:66-75)"""
+    pos, cell, pbc, types = cases.structure_alloy54()
+    perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 5.0)
+    eng = kk.Engine(kk.Model(cases.model_file(model_dir, "mix2")), ["Mo", "W"], 64)
+    args = dict(positions=pos[perm], image=image, shifts=shifts, energies=True)
+    one = eng.compute(types[perm], offset, j, **args)
+    two = eng.compute(types[perm], offset, j, add_to=one, **args)
+    for k in ("energy", "forces", "virial", "energies"):
+        assert np.allclose(two[k], 2.0 * np.asarray(one[k]), rtol=0, atol=1e-11 * max(1.0, np.abs(one[k]).max()))

@@ -47,7 +47,7 @@ def lammps_inputs(pos, cell, types, reach, seed=0):
 @pytest.mark.parametrize("model,species,struct", [("mix2", ["Mo", "W"], "alloy54"), ("l2mix", ["Mo", "W"], "triclinic"),
                                                   ("l3mix", ["Mo", "W"], "alloy54")])
 def test_lammps_call_equals_csr_call(model_dir, model, species, struct):
-    eng = kk.Engine(kk.Model(os.path.join(model_dir, model + ".npz")), species, 64)
+    eng = kk.Engine(kk.Model(cases.model_file(model_dir, model)), species, 64)
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     n = len(pos)
     ref = kk.System(eng.model, species, skin=0.0).compute(types, pos, cell, pbc, energies=True)
@@ -70,7 +70,7 @@ def test_lammps_call_equals_csr_call(model_dir, model, species, struct):
 def test_device_arrays_equal_host_arrays(model_dir, model, species, struct, layout):
     """the KOKKOS form of the call (every array on the device, the 2-d neighbour view in either layout) = the host form"""
     import torch
-    eng = kk.Engine(kk.Model(os.path.join(model_dir, model + ".npz")), species, 64)
+    eng = kk.Engine(kk.Model(cases.model_file(model_dir, model)), species, 64)
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     n = len(pos)
     rc = max(eng.cutoff(a, b) for a in (1, 2) for b in (1, 2))
@@ -110,7 +110,7 @@ def test_device_arrays_equal_host_arrays(model_dir, model, species, struct, layo
 
 def test_unmapped_types_take_no_part_and_argument_errors(model_dir):
     """pair_style hybrid: atoms of a type without a model element are neither central atoms nor neighbours"""
-    model = kk.Model(os.path.join(model_dir, "mix2.npz"))
+    model = kk.Model(cases.model_file(model_dir, "mix2"))
     eng2 = kk.Engine(model, ["Mo", "W"], 64)
     pos, cell, pbc, types = cases.structure_alloy54()
     n = len(pos)

@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 @pytest.fixture(scope="module")
 def model(model_dir):
-    return kk.Model(os.path.join(model_dir, "mix2.npz"))
+    return kk.Model(cases.model_file(model_dir, "mix2"))
 
 
 def test_device_list_equals_reference_list(model, gold):

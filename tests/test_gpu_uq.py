@@ -35,7 +35,7 @@ def _oracle(path, name, t, offset, j, rij):
                                                 ("uq3l", 32, 1e-4)])
 @pytest.mark.parametrize("struct", ["alloy54", "triclinic"])
 def test_uq_matches_oracle(model_dir, name, struct, precision, tol):
-    path = os.path.join(model_dir, name + ".npz")
+    path = cases.model_file(model_dir, name)
     eng = kk.Engine(kk.Model(path), ["Mo", "W"], precision)
     t, offset, j, rij = _bonds(struct)
     ref = _oracle(path, name, t, offset, j, rij)
@@ -62,7 +62,7 @@ def test_uq_matches_oracle(model_dir, name, struct, precision, tol):
 
 @pytest.mark.parametrize("name", ["uq2", "uq2l", "uq3l"])
 def test_calculator_level_call_returns_uq_in_the_callers_order(model_dir, name):
-    path = os.path.join(model_dir, name + ".npz")
+    path = cases.model_file(model_dir, name)
     model = kk.Model(path)
     pos, cell, pbc, types = cases.structure_alloy54()
     s = kk.System(model, ["Mo", "W"], skin=0.3)
@@ -84,7 +84,7 @@ def test_calculator_level_call_returns_uq_in_the_callers_order(model_dir, name):
 
 
 def test_uq_errors(model_dir):
-    plain = kk.Engine(kk.Model(os.path.join(model_dir, "mix2.npz")), ["Mo", "W"], 64)
+    plain = kk.Engine(kk.Model(cases.model_file(model_dir, "mix2")), ["Mo", "W"], 64)
     t, offset, j, rij = _bonds("alloy54")
     plain.upload(t, offset, j, rij)
     with pytest.raises(ValueError, match="no usable UQ head"):
@@ -92,7 +92,7 @@ def test_uq_errors(model_dir):
     plain.run()
     with pytest.raises(RuntimeError, match="needs a run with the UQ flag"):
         plain.fetch_uq()
-    two = kk.System(kk.Model(os.path.join(model_dir, "l2mix.npz")), ["Mo", "W"])
+    two = kk.System(kk.Model(cases.model_file(model_dir, "l2mix")), ["Mo", "W"])
     pos, cell, pbc, types = cases.structure_alloy54()
     with pytest.raises(ValueError, match="no usable UQ head"):
         two.compute(types, pos, cell, pbc, uq=True)
@@ -103,7 +103,7 @@ def test_batches_return_uq_per_atom_in_the_callers_order(model_dir, name):
     """Batch.compute(uq=True) and the gamma / atomic_sigma / gmm_cluster outputs of Batch.compute_device
     (python/kk/kk_api.h:116-156) against one System call per structure, in one pass and in passes of one structure"""
     import torch
-    model = kk.Model(os.path.join(model_dir, name + ".npz"))
+    model = kk.Model(cases.model_file(model_dir, name))
     structs = [cases.structure_alloy54(), cases.structure_triclinic(), cases.structure_slab()]
     natoms = np.array([len(s[0]) for s in structs], np.int32)
     pos = np.concatenate([s[0] for s in structs])
@@ -130,6 +130,6 @@ def test_batches_return_uq_per_atom_in_the_callers_order(model_dir, name):
     g = torch.zeros(len(types), dtype=torch.float64, device=dev)
     b.compute_device(natoms, torch.as_tensor(types, device=dev), torch.as_tensor(pos, device=dev), cells, pbc, e, gamma=g)
     assert np.abs(g.cpu().numpy() / want["gamma"] - 1).max() < 1e-9
-    plain = kk.Batch(kk.Model(os.path.join(model_dir, "mix2.npz")), ["Mo", "W"])
+    plain = kk.Batch(kk.Model(cases.model_file(model_dir, "mix2")), ["Mo", "W"])
     with pytest.raises(ValueError, match="no UQ head"):
         plain.compute(natoms, types, pos, cells, pbc, uq=True)

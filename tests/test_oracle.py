@@ -38,7 +38,7 @@ def test_oracle_matches_tf_fp64(tf_gold, name, cell):
 
 @pytest.mark.parametrize("model,struct,rc", cases.E2E_CASES)
 def test_oracle_matches_compiled_reference(model_dir, gold, model, struct, rc):
-    m = go.Model1L(os.path.join(model_dir, model + ".npz"))
+    m = go.Model1L(cases.model_file(model_dir, model))
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     types = np.minimum(types, m.n_elements)
     tag = f"e2e/{model}/{struct}"
@@ -135,7 +135,7 @@ def _w2tri_energy(m, mu, pos, cell, rc):
 
 
 def test_forces_and_virial_are_energy_derivatives(model_dir):
-    m = go.Model1L(os.path.join(model_dir, "mix2.npz"))
+    m = go.Model1L(cases.model_file(model_dir, "mix2"))
     pos, cell, pbc, types = cases.structure_triclinic()
     mu = types - 1
     E0, F, W = _w2tri_energy(m, mu, pos, cell, m.rcut)
@@ -161,7 +161,7 @@ def test_forces_and_virial_are_energy_derivatives(model_dir):
 
 
 def test_rotation_and_permutation_invariance(model_dir):
-    m = go.Model1L(os.path.join(model_dir, "mix2.npz"))
+    m = go.Model1L(cases.model_file(model_dir, "mix2"))
     pos, cell, pbc, types = cases.structure_triclinic()
     mu = types - 1
     E0, F0, _ = _w2tri_energy(m, mu, pos, cell, m.rcut)
@@ -174,7 +174,7 @@ def test_rotation_and_permutation_invariance(model_dir):
 
 
 def test_isolated_atom_and_zero_bond(model_dir):
-    m = go.Model1L(os.path.join(model_dir, "mix2.npz"))
+    m = go.Model1L(cases.model_file(model_dir, "mix2"))
     out = go.compute_1l(m, np.array([1]), np.array([0, 0]), np.zeros(0, int), np.zeros((0, 3)))
     # no bonds: A = 0, rho = 0, E = MLP(0) * scale + shift = shift (tests/test_driver.cpp:432-440 of the reference)
     assert abs(out["energy"] - m.shift[1]) < 1e-14 and np.all(out["forces"] == 0)

@@ -56,7 +56,7 @@ def test_oracle_matches_compiled_reference_on_fixture_models(gold, model, cell):
 
 @pytest.mark.parametrize("model,struct,rc", cases.E2E_CASES_2L)
 def test_oracle_matches_compiled_reference(model_dir, gold, model, struct, rc):
-    m = g2.Model2L(os.path.join(model_dir, model + ".npz"))
+    m = g2.Model2L(cases.model_file(model_dir, model))
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     types = np.minimum(types, m.n_elements)
     tag = f"e2e/{model}/{struct}"
@@ -123,7 +123,7 @@ def test_forces_and_virial_are_derivatives_of_the_energy():
 
 def test_rotation_invariance_of_a_generated_model(model_dir):
     """the structure generator's couplings (also the odd-parity ones) make an invariant energy and covariant forces"""
-    m = g2.Model2L(os.path.join(model_dir, "l2mix.npz"))
+    m = g2.Model2L(cases.model_file(model_dir, "l2mix"))
     pos, cell, mu = _tiny_system(4)
     off, jj, rij = _bonds(pos, cell, 5.0)
     out = g2.compute_2l(m, mu, off, jj, rij)

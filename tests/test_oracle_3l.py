@@ -26,7 +26,7 @@ TOL = {"energy": 1e-6, "forces": 2e-5, "energies": 1e-5, "stress": 1e-5}    # eV
 
 @pytest.mark.parametrize("model,struct,rc", cases.E2E_CASES_3L)
 def test_oracle_matches_compiled_reference(model_dir, gold, model, struct, rc):
-    m = g3.Model3L(os.path.join(model_dir, model + ".npz"))
+    m = g3.Model3L(cases.model_file(model_dir, model))
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     types = np.minimum(types, m.n_elements)
     tag = f"e2e/{model}/{struct}"
@@ -46,7 +46,7 @@ def test_oracle_matches_compiled_reference(model_dir, gold, model, struct, rc):
 
 @pytest.mark.parametrize("model", ["l3mix", "l3pad"])
 def test_forces_and_virial_are_derivatives_of_the_energy(model_dir, model):
-    m = g3.Model3L(os.path.join(model_dir, model + ".npz"))
+    m = g3.Model3L(cases.model_file(model_dir, model))
     pos, cell, mu = _tiny_system()
 
     def energy(p, c):
@@ -73,7 +73,7 @@ def test_forces_and_virial_are_derivatives_of_the_energy(model_dir, model):
 @pytest.mark.parametrize("model", ["l3mix", "l3wide"])
 def test_invariances_of_a_generated_model(model_dir, model):
     """the generator's couplings (pseudo-tensor paths included) give an invariant energy and covariant forces"""
-    m = g3.Model3L(os.path.join(model_dir, model + ".npz"))
+    m = g3.Model3L(cases.model_file(model_dir, model))
     pos, cell, mu = _tiny_system(4)
     off, jj, rij = _bonds(pos, cell, 5.0)
     out = g3.compute_3l(m, mu, off, jj, rij)
@@ -101,7 +101,7 @@ def test_invariances_of_a_generated_model(model_dir, model):
 
 
 def test_isolated_atoms_and_zero_bond(model_dir):
-    m = g3.Model3L(os.path.join(model_dir, "l3mix.npz"))
+    m = g3.Model3L(cases.model_file(model_dir, "l3mix"))
     mu = np.array([0, 1, 1])
     out = g3.compute_3l(m, mu, np.zeros(4, np.int64), np.zeros(0, np.int64), np.zeros((0, 3)))
     # no neighbours: every density is zero, rho_norm = 0, E_i = MLP(0) + 0 = 0 (no biases) plus the shift

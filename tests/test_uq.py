@@ -37,13 +37,13 @@ def _oracle(path, t, offset, j, rij, **kw):
 
 @pytest.fixture(scope="module")
 def uq_model(model_dir):
-    return os.path.join(model_dir, "uq2.npz")
+    return cases.model_file(model_dir, "uq2")
 
 
 @pytest.mark.skipif(not ref_lib.available(), reason="compiled reference not built")
 @pytest.mark.parametrize("model,struct", cases.UQ_CASES)
 def test_oracle_matches_compiled_reference(model_dir, model, struct):
-    path = os.path.join(model_dir, model + ".npz")
+    path = cases.model_file(model_dir, model)
     t, offset, j, rij = _bonds(struct)
     o, m = _oracle(path, t, offset, j, rij)
     r = ref_lib.RefModel(path, [0, 1]).compute_uq(t, offset, j, rij)
@@ -58,7 +58,7 @@ def test_oracle_matches_compiled_reference(model_dir, model, struct):
 def test_oracle_matches_golden_of_the_compiled_reference(model_dir, gold, model, struct):
     """the committed outputs of the compiled reference (tests/golden/make_golden.py), for machines without it"""
     t, offset, j, rij = _bonds(struct)
-    o, _ = _oracle(os.path.join(model_dir, model + ".npz"), t, offset, j, rij)
+    o, _ = _oracle(cases.model_file(model_dir, model), t, offset, j, rij)
     tag = f"uq/{model}/{struct}"
     assert np.array_equal(o["gmm_cluster"], gold[tag + "/gmm_cluster"])
     assert np.abs(o["gamma"] / gold[tag + "/gamma"] - 1).max() < 1e-4
@@ -69,7 +69,7 @@ def test_oracle_matches_golden_of_the_compiled_reference(model_dir, gold, model,
 def test_what_the_definition_fixes(model_dir, name):
     """the atom whose feature vector IS a centroid has sigma = sqrt(1e-8) and gamma = sigma / threshold; the features are
     invariants of the neighbourhood: a rotated structure gives the same gamma; gamma = sigma / threshold everywhere"""
-    path = os.path.join(model_dir, name + ".npz")
+    path = cases.model_file(model_dir, name)
     t, offset, j, rij = _bonds("alloy54")
     o, m = _oracle(path, t, offset, j, rij)
     thr = m.uq_thr[t - 1, o["gmm_cluster"].astype(int)]
@@ -133,18 +133,18 @@ def test_heads_that_validate_and_models_without(tmp_path, uq_model, model_dir):
     m = kk.Model(uq_model)
     assert m.has_uq
     m.validate_uq()
-    plain = kk.Model(os.path.join(model_dir, "mix2.npz"))
+    plain = kk.Model(cases.model_file(model_dir, "mix2"))
     assert not plain.has_uq
     with pytest.raises(ValueError, match="no UQ head"):
         plain.validate_uq()
     with pytest.raises(ValueError, match="no UQ head"):
-        kk.Model(os.path.join(model_dir, "l2mix.npz")).validate_uq()
+        kk.Model(cases.model_file(model_dir, "l2mix")).validate_uq()
     with pytest.raises(ValueError, match="GRACE-3L: the model has no UQ head"):
-        kk.Model(os.path.join(model_dir, "l3mix.npz")).validate_uq()
-    three = kk.Model(os.path.join(model_dir, "uq3l.npz"))
+        kk.Model(cases.model_file(model_dir, "l3mix")).validate_uq()
+    three = kk.Model(cases.model_file(model_dir, "uq3l"))
     assert three.has_uq and three.layers == 3
     three.validate_uq()
-    two = kk.Model(os.path.join(model_dir, "uq2l.npz"))
+    two = kk.Model(cases.model_file(model_dir, "uq2l"))
     assert two.has_uq and two.layers == 2
     two.validate_uq()
     o3 = kk.Model(_mutated(tmp_path, lambda d: synth_uq(d), "cut2"))          # max_order 3: refused (tests/test_driver.cpp:406-415)
