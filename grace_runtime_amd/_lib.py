@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgrace_hip.so")
 
 GR_OK, GR_INVALID, GR_ERROR, GR_NOMEM = 0, 1, 2, 3
-FLAG_ENERGY_ONLY, FLAG_EATOM, FLAG_UQ, FLAG_ACCUMULATE = 1, 2, 4, 8
+FLAG_ENERGY_ONLY, FLAG_EATOM, FLAG_UQ, FLAG_ACCUMULATE, FLAG_SAME_LIST = 1, 2, 4, 8, 16
 
 # every symbol include/grace_hip.h declares (checked by the CPU test-suite against the header and the library)
 SYMBOLS = [
@@ -25,7 +25,7 @@ SYMBOLS = [
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
     "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_batch_uq", "gr_compute_batch_device_uq", "gr_engine_reset", "gr_engine_release_buffers", "gr_set_memory_limit", "gr_memory_in_use", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
-    "gr_system_fetch_uq", "gr_engine_atoms_that_fit", "gr_engine_set_chunksize", "gr_engine_chunksize", "gr_system_set_chunksize", "gr_system_chunksize",
+    "gr_system_fetch_uq", "gr_engine_atoms_that_fit", "gr_engine_set_exchange", "gr_engine_comm_layers", "gr_engine_comm_width", "gr_engine_pack_forward", "gr_engine_unpack_forward", "gr_engine_pack_reverse", "gr_engine_unpack_reverse", "gr_engine_pack_forward_host", "gr_engine_unpack_forward_host", "gr_engine_pack_reverse_host", "gr_engine_unpack_reverse_host", "gr_engine_set_chunksize", "gr_engine_chunksize", "gr_system_set_chunksize", "gr_system_chunksize",
 ]
 
 
@@ -88,6 +88,13 @@ def lib():
     L.gr_engine_debug_radial.argtypes = [vp, i32, vp, vp, vp, vp]
     L.gr_engine_stage_flops.argtypes = [vp, i32, vp]
     L.gr_engine_set_chunksize.argtypes = [vp, i32]
+    L.gr_engine_set_exchange.argtypes = [vp, vp]
+    L.gr_engine_comm_layers.argtypes = [vp]
+    L.gr_engine_comm_width.argtypes = [vp, i32]
+    for name in ("gr_engine_pack_forward", "gr_engine_unpack_reverse", "gr_engine_pack_forward_host", "gr_engine_unpack_reverse_host"):
+        getattr(L, name).argtypes = [vp, i32, i32, vp, vp]          # engine, layer, n, sendlist, buf
+    for name in ("gr_engine_unpack_forward", "gr_engine_pack_reverse", "gr_engine_unpack_forward_host", "gr_engine_pack_reverse_host"):
+        getattr(L, name).argtypes = [vp, i32, i32, i32, vp]         # engine, layer, n, first, buf
     L.gr_engine_atoms_that_fit.argtypes = [vp]
     L.gr_engine_atoms_that_fit.restype = i64
     L.gr_engine_chunksize.argtypes = [vp]

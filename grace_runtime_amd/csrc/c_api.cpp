@@ -34,6 +34,8 @@ struct gr_engine {
   int ntypes = 0, precision = 64, device = 0;
   int generation = 0;                                  // counts reset(): holders of uploaded state (gr_system) upload again
   int64_t nall_cap = INT64_MAX;                        // atoms per batch pass after an allocation failure (kept for later calls)
+  bool has_exchange = false;                           // an exchange is installed: ghosts of the LAMMPS call stay atoms of their own
+  grhip::ExchangeCallbacks exchange;                   // kept for the engine a reset makes
   void make()
   {
     if (m1) eng = grhip::make_engine_1l(m1, ntypes, type2mu, precision, device);
@@ -47,6 +49,7 @@ struct gr_engine {
     eng.reset();    // frees every device buffer of the engine before the new one allocates
     generation++;
     make();
+    if (has_exchange) eng->set_exchange(exchange);
   }
   std::vector<grhip::StageTime> times;
   std::unique_ptr<grhip::BatchDeviceNeighbors> bnl;    // lists of gr_compute_batch_device (buffers kept between calls)
@@ -521,9 +524,54 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
   return guarded([&] {
     if (!e || (nall > 0 && (!type || !x)) || (inum > 0 && (!ilist || !numneigh || !firstneigh))) throw grhip::InvalidArgument("null argument");
     if (nlocal < 0 || nall < nlocal || inum < 0) throw grhip::InvalidArgument("atom counts out of range");
-    grhip::Engine &eng = *e->eng;
+    grhip::Engine &eng = live(e);
     // atoms of types the engine has no element for take no part (pair_style hybrid): neither central atoms nor neighbours
     auto mapped = [&](int a) { return eng.cutoff(type[a], type[a]) > 0.0; };
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    if (!owner && nall > nlocal && (e->has_exchange || eng.comm_layers() == 0)) {
+      // Ghosts stay atoms of their own (the way of the reference's drivers): bonds name them by their LAMMPS index, their
+      // message rows come through the exchange, and what the pass leaves on them (forces, adjoint rows) goes back through
+      // the reverse exchange and LAMMPS' reverse communication of f.  Every atom must have a model element here.
+      for (int a = 0; a < nall; a++)
+        if (!mapped(a)) throw grhip::InvalidArgument("with an exchange every owned and ghost atom needs a type with a model element");
+      std::vector<char> listed(nlocal, 0);
+      for (int q = 0; q < inum; q++) {
+        if (ilist[q] < 0 || ilist[q] >= nlocal) throw grhip::InvalidArgument("ilist must index owned atoms");
+        listed[ilist[q]] = 1;
+      }
+      for (int i = 0; i < nlocal; i++)
+        if (!listed[i]) throw grhip::InvalidArgument("every owned atom of a mapped type must be in ilist (sub-lists are not supported)");
+      std::vector<int64_t> offset((size_t) nlocal + 1, 0);
+      std::vector<int> jj;
+      std::vector<double> rij;
+      for (int i = 0; i < nlocal; i++) {
+        const int *nb = firstneigh[i];
+        for (int k = 0; k < numneigh[i]; k++) {
+          const int j = nb[k] & neighmask;
+          if (j < 0 || j >= nall) throw grhip::InvalidArgument("neighbour index outside the owned and ghost atoms");
+          jj.push_back(j);
+          for (int d = 0; d < 3; d++) rij.push_back(x[3 * (size_t) j + d] - x[3 * (size_t) i + d]);
+        }
+        offset[(size_t) i + 1] = (int64_t) jj.size();
+      }
+      const std::vector<double> dummy(3, 0.0);
+      grhip::CsrInput in = make_input(nlocal, type, offset.data(), jj.data(), rij.empty() ? dummy.data() : rij.data(), nullptr, nullptr, nullptr, 0);
+      in.n_nodes = nall;
+      eng.upload(in);
+      eng.run(fl);
+      std::vector<double> fo((size_t) 3 * nall), ea(fl.eatom ? nlocal : 0);
+      double en = 0.0, vir[6] = {0, 0, 0, 0, 0, 0};
+      eng.fetch(&en, f ? fo.data() : nullptr, vir, fl.eatom ? ea.data() : nullptr);
+      if (energy) *energy = en;
+      if (virial && !fl.energy_only)
+        for (int k = 0; k < 6; k++) virial[k] = vir[k];
+      if (f && !fl.energy_only)
+        for (size_t q = 0; q < fo.size(); q++) f[q] += fo[q];
+      for (int i = 0; i < (fl.eatom ? nlocal : 0); i++) eatom[i] += ea[(size_t) i];
+      return;
+    }
     std::vector<int> idx(nlocal, -1), atom;
     std::vector<char> central(nlocal, 0);
     for (int q = 0; q < inum; q++) {
@@ -552,7 +600,7 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
         if (!mapped(j)) continue;
         int o = j;
         if (j >= nlocal) {
-          if (!owner) throw grhip::InvalidArgument("ghost neighbours need the owner map (the owned atom each ghost is an image of)");
+          if (!owner) throw grhip::InvalidArgument("ghost neighbours need the owner map (the owned atom each ghost is an image of) or an exchange");
           o = owner[j];
         }
         if (o < 0 || o >= nlocal || idx[o] < 0 || type[o] != type[j])
@@ -564,9 +612,6 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
     }
     const std::vector<double> dummy(3, 0.0);
     eng.upload(make_input(n, ty.data(), offset.data(), jj.data(), rij.empty() ? dummy.data() : rij.data(), nullptr, nullptr, nullptr, 0));
-    grhip::RunFlags fl;
-    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
-    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
     eng.run(fl);
     std::vector<double> fo((size_t) 3 * n), ea(fl.eatom ? n : 0);
     double en = 0.0, vir[6] = {0, 0, 0, 0, 0, 0};
@@ -583,6 +628,66 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
   });
 }
 
+// ---- message exchange with ghost atoms (LAMMPS comm) ----------------------------------------------------------------
+int gr_engine_set_exchange(gr_engine *e, const gr_exchange *x)
+{
+  return guarded([&] {
+    grhip::ExchangeCallbacks cb;
+    if (x) {
+      cb.forward = x->forward;
+      cb.reverse = x->reverse;
+      cb.user = x->user;
+    }
+    live(e).set_exchange(cb);
+    e->has_exchange = x && (x->forward || x->reverse);
+    e->exchange = cb;
+  });
+}
+int gr_engine_comm_layers(gr_engine *e)
+{
+  int r = -1;
+  guarded([&] { r = live(e).comm_layers(); });
+  return r;
+}
+int gr_engine_comm_width(gr_engine *e, int layer)
+{
+  int r = -1;
+  guarded([&] { r = live(e).comm_width(layer); });
+  return r;
+}
+int gr_engine_pack_forward(gr_engine *e, int layer, int n, const int *sendlist, double *buf)
+{
+  return guarded([&] { live(e).comm_rows(0, layer, n, sendlist, 0, buf, false); });
+}
+int gr_engine_unpack_forward(gr_engine *e, int layer, int n, int first, const double *buf)
+{
+  return guarded([&] { live(e).comm_rows(1, layer, n, nullptr, first, const_cast<double *>(buf), false); });
+}
+int gr_engine_pack_reverse(gr_engine *e, int layer, int n, int first, double *buf)
+{
+  return guarded([&] { live(e).comm_rows(2, layer, n, nullptr, first, buf, false); });
+}
+int gr_engine_unpack_reverse(gr_engine *e, int layer, int n, const int *sendlist, const double *buf)
+{
+  return guarded([&] { live(e).comm_rows(3, layer, n, sendlist, 0, const_cast<double *>(buf), false); });
+}
+int gr_engine_pack_forward_host(gr_engine *e, int layer, int n, const int *sendlist, double *buf)
+{
+  return guarded([&] { live(e).comm_rows(0, layer, n, sendlist, 0, buf, true); });
+}
+int gr_engine_unpack_forward_host(gr_engine *e, int layer, int n, int first, const double *buf)
+{
+  return guarded([&] { live(e).comm_rows(1, layer, n, nullptr, first, const_cast<double *>(buf), true); });
+}
+int gr_engine_pack_reverse_host(gr_engine *e, int layer, int n, int first, double *buf)
+{
+  return guarded([&] { live(e).comm_rows(2, layer, n, nullptr, first, buf, true); });
+}
+int gr_engine_unpack_reverse_host(gr_engine *e, int layer, int n, const int *sendlist, const double *buf)
+{
+  return guarded([&] { live(e).comm_rows(3, layer, n, sendlist, 0, const_cast<double *>(buf), true); });
+}
+
 int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, const int *type, const double *x, int inum, const int *ilist,
                              const int *numneigh, const int *neighbors, int64_t stride_i, int64_t stride_k, int neighmask, const int *owner,
                              unsigned flags, double *energy, double *f, double *virial, double *eatom)
@@ -590,7 +695,7 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
   return guarded([&] {
     if (!e || (nall > 0 && (!type || !x)) || (inum > 0 && (!ilist || !numneigh || !neighbors))) throw grhip::InvalidArgument("null argument");
     if (nlocal < 0 || nall < nlocal || inum < 0 || ntypes < 0) throw grhip::InvalidArgument("atom counts out of range");
-    grhip::Engine &eng = *e->eng;
+    grhip::Engine &eng = live(e);
     if (hipSetDevice(eng.device_index()) != hipSuccess) throw grhip::Error("hipSetDevice failed");
     auto on_device = [&](const void *p, const char *name) {
       if (!p) return;
@@ -608,6 +713,29 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
     hipStream_t st = e->bnl_stream;
     // work queued by the caller on other streams (the arrays that hold the inputs) is finished first
     if (hipDeviceSynchronize() != hipSuccess) throw grhip::Error("hipDeviceSynchronize failed");
+    grhip::RunFlags fl;
+    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
+    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    const bool nodes = !owner && nall > nlocal && (e->has_exchange || eng.comm_layers() == 0);
+    grhip::LmpListDev L{};
+    L.type = type; L.x = x; L.numneigh = numneigh; L.neighbors = neighbors; L.stride_i = stride_i; L.stride_k = stride_k;
+    L.owner = owner; L.nlocal = nlocal; L.nall = nall; L.neighmask = neighmask; L.nodes = nodes ? 1 : 0;
+    if ((flags & GR_FLAG_SAME_LIST) && W.kept && W.serial == eng.upload_serial() && W.nlocal == nlocal && W.nall == nall && W.inum == inum &&
+        W.nodes == L.nodes && W.neighmask == neighmask && W.stride_i == stride_i && W.stride_k == stride_k && W.neighbors == neighbors &&
+        W.type == type && W.numneigh == numneigh && W.owner == owner) {
+      // the steps between two reneighbourings: same rows, same bonds, new bond vectors written into the engine's array
+      L.idx = W.idx.as<int>(); L.atom = W.atom.as<int>(); L.mapped = W.mapped.as<unsigned char>(); L.n = W.n;
+      if (W.n > 0 && W.nb > 0) {
+        double *rij = eng.bond_vectors_device();
+        hipLaunchKernelGGL(grhip::k_lmp_rows<true>, dim3((unsigned) ((W.n + 127) / 128)), dim3(128), 0, st, L, (int *) nullptr, (int *) nullptr,
+                           (const long long *) W.offset.as<long long>(), W.j.as<int>(), rij);
+        if (hipStreamSynchronize(st) != hipSuccess) throw grhip::Error("the renewal of the bond vectors failed");
+      }
+      eng.run(fl);
+      eng.fetch_add_device(nodes ? nullptr : W.atom.as<int>(), energy, f, virial, fl.eatom ? eatom : nullptr);
+      return;
+    }
+    W.kept = false;
     // atom types and the atom list: 4 bytes per atom to the host, where the rows of the engine and its element tiles are laid out
     std::vector<int> ty((size_t) nall), il((size_t) inum);
     if (nall > 0 && hipMemcpy(ty.data(), type, sizeof(int) * (size_t) nall, hipMemcpyDeviceToHost) != hipSuccess) throw grhip::Error("copy of the atom types failed");
@@ -616,6 +744,10 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
     for (int t = 1; t <= ntypes; t++) mapped[t] = eng.cutoff(t, t) > 0.0;
     for (int a = 0; a < nall; a++)
       if (ty[a] < 1 || ty[a] > ntypes) throw grhip::InvalidArgument("types must be 1 .. ntypes");
+    // ghosts as atoms of their own, as in gr_compute_lammps: the engine's rows are the owned atoms in LAMMPS order
+    if (nodes)
+      for (int a = 0; a < nall; a++)
+        if (!mapped[ty[a]]) throw grhip::InvalidArgument("with an exchange every owned and ghost atom needs a type with a model element");
     std::vector<int> idx((size_t) nlocal, -1), atom, tq;
     std::vector<char> central((size_t) nlocal, 0);
     for (int q = 0; q < inum; q++) {
@@ -632,6 +764,7 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
       tq.push_back(ty[i]);
     }
     const int n = (int) atom.size();
+    if (nodes) tq.insert(tq.end(), ty.begin() + nlocal, ty.end());    // n = nlocal here: the types of all nall atoms
     auto put = [&](grhip::DevBuf &b, const void *src, size_t bytes) {
       b.ensure(std::max<size_t>(bytes, 8));
       if (bytes && hipMemcpyAsync(b.p, src, bytes, hipMemcpyHostToDevice, st) != hipSuccess) throw grhip::Error("copy to the device failed");
@@ -643,10 +776,7 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
     put(W.err, &zero, sizeof(int));
     W.count.ensure(sizeof(int) * (size_t) std::max(n, 1));
     W.offset.ensure(sizeof(long long) * (size_t) (n + 1));
-    grhip::LmpListDev L{};
-    L.type = type; L.x = x; L.numneigh = numneigh; L.neighbors = neighbors; L.stride_i = stride_i; L.stride_k = stride_k;
-    L.owner = owner; L.idx = W.idx.as<int>(); L.atom = W.atom.as<int>(); L.mapped = W.mapped.as<unsigned char>();
-    L.n = n; L.nlocal = nlocal; L.nall = nall; L.neighmask = neighmask;
+    L.idx = W.idx.as<int>(); L.atom = W.atom.as<int>(); L.mapped = W.mapped.as<unsigned char>(); L.n = n;
     W.nb = 0;
     if (n > 0) {
       const dim3 grid((unsigned) ((n + 127) / 128)), block(128);
@@ -660,7 +790,7 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
         throw grhip::Error("the conversion of the neighbour list failed");
       if (err == 1) throw grhip::InvalidArgument("neighbour index outside the owned and ghost atoms");
       if (err == 2) throw grhip::InvalidArgument(owner ? "the owner of a ghost atom is not an owned atom of the same type"
-                                                       : "ghost neighbours need the owner map (the owned atom each ghost is an image of)");
+                                                       : "ghost neighbours need the owner map (the owned atom each ghost is an image of) or an exchange");
       W.nb = total;
       W.j.ensure(sizeof(int) * (size_t) std::max<int64_t>(W.nb, 1));
       W.rij.ensure(sizeof(double) * 3 * (size_t) std::max<int64_t>(W.nb, 1));
@@ -678,12 +808,14 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
     in.offset = W.offset.as<int64_t>();
     in.j = W.j.as<int>();
     in.rij = W.rij.as<double>();
+    in.n_nodes = nodes ? nall : 0;
     eng.upload_device(in);
-    grhip::RunFlags fl;
-    fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
-    fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    W.kept = true;
+    W.serial = eng.upload_serial();
+    W.n = n; W.nlocal = nlocal; W.nall = nall; W.inum = inum; W.nodes = L.nodes; W.neighmask = neighmask;
+    W.stride_i = stride_i; W.stride_k = stride_k; W.neighbors = neighbors; W.type = type; W.numneigh = numneigh; W.owner = owner;
     eng.run(fl);
-    eng.fetch_add_device(W.atom.as<int>(), energy, f, virial, fl.eatom ? eatom : nullptr);
+    eng.fetch_add_device(nodes ? nullptr : W.atom.as<int>(), energy, f, virial, fl.eatom ? eatom : nullptr);
   });
 }
 

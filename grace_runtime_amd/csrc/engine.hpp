@@ -27,6 +27,20 @@ struct CsrInput {
   // several independent structures in one list (no bonds between them): structure of every atom, or null for one
   int nstruct = 1;
   const int *sid = nullptr;           // [n] in 0 .. nstruct-1
+  // atoms with and without a row of bonds (a LAMMPS rank: owned atoms, then ghosts): n_nodes >= n atoms in all, the
+  // first n are central atoms; types (and positions) have n_nodes entries, j indexes 0 .. n_nodes - 1, forces are
+  // returned for all n_nodes.  0: every atom is central (n_nodes = n)
+  int n_nodes = 0;
+};
+
+// Exchange of the message rows between the central atoms and the ghost atoms of a layer, as the reference's Exchange
+// (libgrace/include/grace/system.h:53-60): forward(layer) is called when the layer's message rows of the central atoms
+// are complete and must fill the rows of the ghosts; reverse(layer) when the adjoint rows are complete and must add the
+// ghosts' rows to their owners'.  layer counts from 1.  The callbacks use Engine::comm_rows to move rows.
+struct ExchangeCallbacks {
+  void (*forward)(void *user, int layer) = nullptr;
+  void (*reverse)(void *user, int layer) = nullptr;
+  void *user = nullptr;
 };
 
 // A structure whose neighbour list is already in device memory: the engine copies it into its own buffers.
@@ -43,6 +57,7 @@ struct DeviceCsr {
   const double *rij = nullptr;        // device [nb][3] bond vectors, in place of (image, x, shifts)
   int nstruct = 1;                    // several independent structures in one list:
   const int *sid = nullptr;           // host [n] structure of every atom, or null for one structure
+  int n_nodes = 0;                    // as CsrInput::n_nodes: types has n_nodes entries, j indexes 0 .. n_nodes - 1
 };
 
 struct StageTime {
@@ -70,6 +85,11 @@ class Engine {
   virtual void upload_device(const DeviceCsr &in) = 0;
   // new positions [n][3] (host) for the uploaded list (a list given as positions + image + shifts)
   virtual void update_positions(const double *x) = 0;
+  // the device array [nb][3] that holds the bond vectors of the uploaded list (a list given with bond vectors), for a
+  // caller that writes new vectors for the same bonds; the results of the last pass are dropped
+  virtual double *bond_vectors_device() = 0;
+  // counts the uploads of this engine: tells a caller whether the list it uploaded is still the one held
+  virtual uint64_t upload_serial() const = 0;
   virtual int device_index() const = 0;
   // one energy / forces / virial pass over the uploaded structure; results stay on the GPU
   virtual void run(const RunFlags &fl) = 0;
@@ -87,6 +107,16 @@ class Engine {
   // atoms per engine pass (python/kk/kk_api.h:72-75): 0 all atoms in one pass, < 0 chosen from the free device memory
   // (one pass while it fits, else the largest power of two >= 512 that fits), > 0 as given.  chunksize_used(): atoms per
   // pass of the last run (0: one pass).  Engines that do not chunk refuse values other than 0 and -1.
+  // message exchange with ghost atoms (LAMMPS comm): the callbacks, the layers that have a message (0 for GRACE-1L, 1 for
+  // 2L, 2 for 3L), the doubles per atom of a layer's message, and the four row movers of the reference's GPU engines
+  // (libgrace/include/grace/kk/grace_2l_kk.h:141-157): mode 0 pack_forward (rows of the atoms list[0 .. n) -> buf),
+  // 1 unpack_forward (buf -> rows of atoms first .. first + n), 2 pack_reverse (adjoint rows of first .. first + n -> buf),
+  // 3 unpack_reverse (buf ADDED to the adjoint rows of list[0 .. n)); list and buf in device memory, or, with host = true,
+  // in host memory
+  virtual void set_exchange(const ExchangeCallbacks &cb) = 0;
+  virtual int comm_layers() const = 0;
+  virtual int comm_width(int layer) const = 0;
+  virtual void comm_rows(int mode, int layer, int n, const int *list, int first, double *buf, bool host) = 0;
   // atoms of one pass whose work buffers fit 70 % of the memory the library may use, from the bytes per atom that the
   // buffers of the last pass hold; before the first pass: a bound by model kind.  The batch entry points size their
   // passes with it (the reference sizes the first pass from the free memory: libgrace/include/grace/kk/support.h:425-450)

@@ -43,6 +43,15 @@ template<class T> class Engine2L final : public EngineBase {
   {
     throw Error("GRACE-2L: debug_radial is available for GRACE-1L engines");
   }
+  // one message: the functions I of layer 1 (libgrace/include/grace/kk/grace_2l_kk.h:141: I_n_funcs x I_n_out doubles per atom)
+  int comm_layers() const override { return 1; }
+  int comm_width(int layer) const override { return layer == 1 ? nI_ * model_->CR : 0; }
+  void comm_rows(int mode, int layer, int n, const int *list, int first, double *buf, bool host) override
+  {
+    if (layer != 1) throw InvalidArgument("GRACE-2L exchanges the message of layer 1 only");
+    if (mode < 2) move_rows<T>(mode, M_.as<T>(), (long long) nslot_ * CRP_, nI_, model_->CR, CRP_, n, list, first, buf, host);
+    else move_rows<T>(mode, gM_.as<T>(), (long long) nI_ * CRP_, nI_, model_->CR, CRP_, n, list, first, buf, host);
+  }
 
  private:
   std::shared_ptr<const Model2L> model_;
@@ -531,7 +540,9 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   stage("reduce_I1", [&] {
     for (auto &r : redI1_) reduce_fwd(*r, c1_.kb, c1_, A, I1_.as<double>());
   });
-  M_.ensure(na * nslot_ * CRP_ * sizeof(T));
+  // the message rows exist for the ghost atoms too: the exchange fills them, the gather reads them
+  const size_t nnodes = (size_t) n_nodes_;
+  M_.ensure(nnodes * nslot_ * CRP_ * sizeof(T));
   T *M = M_.as<T>();
   // I1 leaves the scalar reduce in fp64; the fp32 engine hands the GEMM a copy in fp32
   const long long nI1v = (long long) na * nI1_ * PI1_;
@@ -544,9 +555,10 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     if constexpr (sizeof(T) == 4)
       hipLaunchKernelGGL((k_convert<double, T>), dim3((unsigned) ((nI1v + 255) / 256)), dim3(256), 0, stream_, I1_.as<double>(), I1t_.as<T>(), nI1v);
     gemm(jI_, PI1_ / 16, CRP_ / 16, I1t, nI1_, M, nslot_, 0);
-    hipLaunchKernelGGL(k_fill_slot<T>, dim3((unsigned) ((na * CRP_ + 255) / 256)), dim3(256), 0, stream_, mu_.as<int>(), zB0_.as<T>(), M, n, nslot_,
-                       nI_, CRP_);
+    hipLaunchKernelGGL(k_fill_slot<T>, dim3((unsigned) ((nnodes * CRP_ + 255) / 256)), dim3(256), 0, stream_, mu_.as<int>(), zB0_.as<T>(), M, n_nodes_,
+                       nslot_, nI_, CRP_);
   });
+  exchange_forward(1);
 
   // ---- P3: layer 2 forward
   const int npf = nslot_ * nlm_;
@@ -606,9 +618,9 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   stage("reduce_I2_bwd", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), true); });
   chain_backward(c2_, "_L2", B, [&] { stage("reduce_I2_bwd_X_XX", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), false); }); });
   gP_.ensure(na * npf * CRP_ * sizeof(T));
-  gM_.ensure(na * nI_ * CRP_ * sizeof(T));
+  gM_.ensure(nnodes * nI_ * CRP_ * sizeof(T));
   stage("reduce_B_bwd", [&] {
-    HIP_CHECK(hipMemsetAsync(gM_.p, 0, na * nI_ * CRP_ * sizeof(T), stream_));    // gP: every row is written below
+    HIP_CHECK(hipMemsetAsync(gM_.p, 0, nnodes * nI_ * CRP_ * sizeof(T), stream_));    // gP: every row is written below
     gemm(jBb_, C2P_ / 16, CRP_ / 16, c2_.gX.template as<T>(), nB_, gP_.as<T>(), npf, 0);
   });
   stage("pair_bwd", [&] {
@@ -619,6 +631,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   });
 #undef GR_PAIR
 #undef GR_PAIR1
+  exchange_reverse(1);
 
   // ---- P5: layer 1 reverse
   gI1_.ensure(na * nI1_ * PI1_ * sizeof(double));

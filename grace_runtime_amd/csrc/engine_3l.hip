@@ -183,6 +183,21 @@ template<class T> class Engine3L final : public EngineBase {
   {
     throw Error("GRACE-3L: debug_radial is available for GRACE-1L engines");
   }
+  // two messages: the normalised equivariant outputs of layers 1 and 2 (libgrace/include/grace/kk/grace_3l_kk.h:313-324)
+  int comm_layers() const override { return 2; }
+  int comm_width(int layer) const override { return layer == 1 || layer == 2 ? L_[layer].nlmi * L_[layer].C : 0; }
+  void comm_rows(int mode, int layer, int n, const int *list, int first, double *buf, bool host) override
+  {
+    if (layer != 1 && layer != 2) throw InvalidArgument("GRACE-3L exchanges the messages of layers 1 and 2");
+    const Layer3<T> &L = L_[layer];    // the layer that gathers the message
+    if (mode < 2) {
+      move_rows<T>(mode, L_[layer - 1].I.buf.template as<T>(), (long long) L.nlmi * L.CP, L.nlmi, L.C, L.CP, n, list, first, buf, host);
+    } else {
+      // the adjoint rows live in scratch shared by the layers: they are this layer's only inside its reverse exchange
+      if (comm_reverse_layer_ != layer) throw Error("GRACE-3L: the adjoint rows of a message exist only inside its reverse exchange");
+      move_rows<T>(mode, gM_.as<T>(), (long long) L.nlmi * L.CP, L.nlmi, L.C, L.CP, n, list, first, buf, host);
+    }
+  }
 
  private:
   std::shared_ptr<const Model3L> model_;
@@ -193,6 +208,7 @@ template<class T> class Engine3L final : public EngineBase {
   Energy3Dev en_{};
   DevBuf uqR_, uqCen_, uqIcov_, uqNcl_, uqThr_, uqZ_, uqN2_;    // UQ head arrays; raw projection and block norms carried over the layers
   bool uq_on_ = false;
+  int comm_reverse_layer_ = 0;    // the message whose adjoint rows gM_ holds while its reverse exchange runs
   // scratch shared by the layers (largest size over the layers): temporaries of the forward pass and all adjoints
   DevBuf M_, gM_, pairP_, gpairP_, A_, gA_, P_, gP_, R2_, R3_, R4_, FA_, FB_, gX_, gR2_, gR3_, gR4_, gFA_, gFB_, gLp_, gRp_, gEQ_;
 
@@ -647,13 +663,14 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
   } else {
     const Layer3<T> &Lm = L_[k - 1];
     const int npf = L.nlmi * nlm_;
-    M_.ensure(na * L.nlmi * L.CP * s);
+    M_.ensure((size_t) n_nodes_ * L.nlmi * L.CP * s);
     pairP_.ensure(na * npf * L.CP * s);
     A_.ensure(na * L.nfA * L.CP * s);
+    exchange_forward(k);    // the message of layer k (counted from 1) reaches the ghost atoms
     stage(tg(k, "message").c_str(), [&] {
-      const long long tot = (long long) n * L.nlmi * L.CP;
+      const long long tot = (long long) n_nodes_ * L.nlmi * L.CP;
       hipLaunchKernelGGL(k_message<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, Lm.I.buf.template as<T>(), mu_.as<int>(),
-                         L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n, L.nlmi, L.CP);
+                         L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n_nodes_, L.nlmi, L.CP);
     });
     const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb;
     stage(tg(k, "pair_fwd").c_str(), [&] {
@@ -705,7 +722,7 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
   const T *srcs[4] = {X, R2, R3, R4};
   if (L.has_eq) {
     L.EQ.buf.ensure(L.EQ.bytes(na, s));
-    L.I.buf.ensure(L.I.bytes(na, s));
+    L.I.buf.ensure(L.I.bytes((size_t) n_nodes_, s));    // rows of the ghost atoms too: the exchange fills them
     stage(tg(k, "reduce_eq").c_str(), [&] {
       zero(L.EQ.buf.p, L.EQ.bytes(na, s));
       for (int q = 0; q < 4; q++) cfwd(*L.eq[q], srcs[q], L.EQ.buf.template as<T>(), 1);
@@ -839,8 +856,8 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   const int npf = L.nlmi * nlm_;
   gA_.ensure(na * L.nfA * L.CP * s);
   gpairP_.ensure(na * npf * L.CP * s);
-  M_.ensure(na * L.nlmi * L.CP * s);
-  gM_.ensure(na * L.nlmi * L.CP * s);
+  M_.ensure((size_t) n_nodes_ * L.nlmi * L.CP * s);
+  gM_.ensure((size_t) n_nodes_ * L.nlmi * L.CP * s);
   stage(tg(k, "reduce_A_bwd").c_str(), [&] { cbwd_set(L.redA, gX, gA_.as<T>()); });
   stage(tg(k, "couple_YI_bwd").c_str(), [&] {
     const int AT = 64 / L.CP;
@@ -849,10 +866,10 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
                        (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP, n);
   });
   stage(tg(k, "message_bwd").c_str(), [&] {
-    const long long tot = (long long) n * L.nlmi * L.CP;
+    const long long tot = (long long) n_nodes_ * L.nlmi * L.CP;
     hipLaunchKernelGGL(k_message<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, Lm.I.buf.template as<T>(), mu_.as<int>(),
-                       L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n, L.nlmi, L.CP);
-    zero(gM_.p, na * L.nlmi * L.CP * s);
+                       L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n_nodes_, L.nlmi, L.CP);
+    zero(gM_.p, (size_t) n_nodes_ * L.nlmi * L.CP * s);
   });
   const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
   stage(tg(k, "pair_bwd").c_str(), [&] {
@@ -861,6 +878,9 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
             L.dR.template as<T>(), (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(),
             f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n);
   });
+  comm_reverse_layer_ = k;
+  exchange_reverse(k);    // the ghosts' adjoint rows of the message of layer k go to their owners
+  comm_reverse_layer_ = 0;
   (void) yw;
 }
 

@@ -560,9 +560,11 @@ class EngineBase : public Engine, protected BufRegistry {
     chunk_laid_out_ = 0;
     n_peak_ = 0;
     n_ = 0;
+    n_nodes_ = 0;
     nb_ = 0;
     nstruct_ = 1;
     ran_ = ran_forces_ = ran_eatom_ = ran_uq_ = false;
+    upload_serial_++;
   }
   void synchronize() override { check(hipSetDevice(device_), "hipSetDevice"); check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
   void set_chunksize(int atoms) override
@@ -573,6 +575,10 @@ class EngineBase : public Engine, protected BufRegistry {
     chunk_request_ = atoms;
   }
   int chunksize_used() const override { return chunk_used_; }
+  void set_exchange(const ExchangeCallbacks &cb) override { exchange_ = cb; }
+  int comm_layers() const override { return 0; }
+  int comm_width(int) const override { return 0; }
+  void comm_rows(int, int, int, const int *, int, double *, bool) override { throw Error(who_ + ": this model kind has no message rows to exchange"); }
   int64_t atoms_that_fit() override
   {
     HIP_CHECK(hipSetDevice(device_));
@@ -631,9 +637,10 @@ class EngineBase : public Engine, protected BufRegistry {
     const bool table = in.x && in.image && in.shifts;
     if ((in.rij != nullptr) == (in.x || in.image || in.shifts) || (!in.rij && !table))
       throw InvalidArgument("give rij or positions, image and shifts");
-    const int n = in.n;
-    std::vector<int> mu(n);
-    for (int a = 0; a < n; a++) {
+    const int n = in.n, nn = std::max(in.n, in.n_nodes);
+    if (nn > n && (in.sid || !in.rij)) throw InvalidArgument("a list with ghost atoms holds one structure and gives its bond vectors");
+    std::vector<int> mu(nn);
+    for (int a = 0; a < nn; a++) {
       if (in.types[a] < 1 || in.types[a] > ntypes_) throw InvalidArgument("types must be 1 .. len(species)");
       mu[a] = type2mu_[in.types[a]];
       if (mu[a] < 0)
@@ -644,7 +651,7 @@ class EngineBase : public Engine, protected BufRegistry {
       if (in.offset[a + 1] < in.offset[a]) throw InvalidArgument("offset must be non-decreasing");
     const int64_t nb = in.offset[n];
     for (int64_t q = 0; q < nb; q++) {
-      if (in.j[q] < 0 || in.j[q] >= n) throw InvalidArgument("j must index atoms 0 .. len(types)-1");
+      if (in.j[q] < 0 || in.j[q] >= nn) throw InvalidArgument("j must index atoms 0 .. len(types)-1");
       if (in.image && (in.image[q] < 0 || in.image[q] >= in.nimages)) throw InvalidArgument("image must index rows of shifts");
     }
     if (in.nstruct < 1) throw InvalidArgument("the number of structures must be positive");
@@ -657,6 +664,7 @@ class EngineBase : public Engine, protected BufRegistry {
           if (in.sid[in.j[q]] != in.sid[a]) throw InvalidArgument("a bond joins atoms of two structures");
     HIP_CHECK(hipStreamSynchronize(stream_));
     n_ = n;
+    n_nodes_ = nn;
     nb_ = nb;
     nstruct_ = in.sid ? in.nstruct : 1;
     have_sid_ = in.sid != nullptr;
@@ -666,11 +674,11 @@ class EngineBase : public Engine, protected BufRegistry {
       b.ensure(std::max<size_t>(bytes, 8));
       if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, hipMemcpyHostToDevice, stream_));
     };
-    put(mu_, mu.data(), sizeof(int) * n);
+    put(mu_, mu.data(), sizeof(int) * nn);
     if (have_sid_) put(sid_, in.sid, sizeof(int) * n);
-    mu_host_ = mu;
+    mu_host_.assign(mu.begin(), mu.begin() + n);    // the central atoms: they make the element tiles
     chunk_laid_out_ = 0;
-    const std::vector<int> tiles = element_tiles(mu, nelem_, tile_el_);
+    const std::vector<int> tiles = element_tiles(mu_host_, nelem_, tile_el_);
     ntiles_ = (int) tiles.size() / 16;
     put(tiles_, tiles.data(), sizeof(int) * tiles.size());
     static_assert(sizeof(long long) == sizeof(int64_t), "offset type");
@@ -684,14 +692,16 @@ class EngineBase : public Engine, protected BufRegistry {
     }
     HIP_CHECK(hipStreamSynchronize(stream_));    // the host copies (mu, tiles) go out of scope
     ran_ = false;
+    upload_serial_++;
   }
   void upload_device(const DeviceCsr &in) override
   {
     HIP_CHECK(hipSetDevice(device_));
     if (in.n < 0) throw InvalidArgument("negative atom count");
-    const int n = in.n;
-    std::vector<int> mu(n);
-    for (int a = 0; a < n; a++) {
+    const int n = in.n, nn = std::max(in.n, in.n_nodes);
+    if (nn > n && (in.sid || !in.rij)) throw InvalidArgument("a list with ghost atoms holds one structure and gives its bond vectors");
+    std::vector<int> mu(nn);
+    for (int a = 0; a < nn; a++) {
       if (in.types[a] < 1 || in.types[a] > ntypes_) throw InvalidArgument("types must be 1 .. len(species)");
       mu[a] = type2mu_[in.types[a]];
       if (mu[a] < 0)
@@ -703,6 +713,7 @@ class EngineBase : public Engine, protected BufRegistry {
       for (int a = 0; a < n; a++)
         if (in.sid[a] < 0 || in.sid[a] >= in.nstruct) throw InvalidArgument("structure index of an atom out of range");
     n_ = n;
+    n_nodes_ = nn;
     nb_ = in.nb;
     nstruct_ = in.sid ? in.nstruct : 1;
     have_sid_ = in.sid != nullptr;
@@ -712,10 +723,10 @@ class EngineBase : public Engine, protected BufRegistry {
       b.ensure(std::max<size_t>(bytes, 8));
       if (bytes) HIP_CHECK(hipMemcpyAsync(b.p, src, bytes, kind, stream_));
     };
-    put(mu_, mu.data(), sizeof(int) * n, hipMemcpyHostToDevice);
-    mu_host_ = mu;
+    put(mu_, mu.data(), sizeof(int) * nn, hipMemcpyHostToDevice);
+    mu_host_.assign(mu.begin(), mu.begin() + n);    // the central atoms: they make the element tiles
     chunk_laid_out_ = 0;
-    const std::vector<int> tiles = element_tiles(mu, nelem_, tile_el_);
+    const std::vector<int> tiles = element_tiles(mu_host_, nelem_, tile_el_);
     ntiles_ = (int) tiles.size() / 16;
     put(tiles_, tiles.data(), sizeof(int) * tiles.size(), hipMemcpyHostToDevice);
     put(offset_, in.offset, sizeof(int64_t) * (n + 1), hipMemcpyDeviceToDevice);
@@ -729,6 +740,7 @@ class EngineBase : public Engine, protected BufRegistry {
     }
     HIP_CHECK(hipStreamSynchronize(stream_));
     ran_ = false;
+    upload_serial_++;
   }
   void update_positions(const double *x) override
   {
@@ -739,6 +751,15 @@ class EngineBase : public Engine, protected BufRegistry {
     HIP_CHECK(hipStreamSynchronize(stream_));
     ran_ = false;
   }
+  double *bond_vectors_device() override
+  {
+    if (!have_rij_) throw Error("bond_vectors_device: the uploaded list holds positions, not bond vectors");
+    HIP_CHECK(hipSetDevice(device_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    ran_ = false;
+    return rij_.as<double>();
+  }
+  uint64_t upload_serial() const override { return upload_serial_; }
   int device_index() const override { return device_; }
   void radial_noalloc(int, const double *, const int *, double *, double *) override
   {
@@ -782,7 +803,7 @@ class EngineBase : public Engine, protected BufRegistry {
       if (virial && ran_forces_)
         for (int k = 0; k < 6; k++) virial[6 * (size_t) q + k] = s[8 * (size_t) q + 1 + k];
     }
-    if (forces && ran_forces_ && n_ > 0) HIP_CHECK(hipMemcpy(forces, f_.p, sizeof(double) * 3 * n_, hipMemcpyDeviceToHost));
+    if (forces && ran_forces_ && n_nodes_ > 0) HIP_CHECK(hipMemcpy(forces, f_.p, sizeof(double) * 3 * n_nodes_, hipMemcpyDeviceToHost));
     if (eatom && ran_eatom_ && n_ > 0) HIP_CHECK(hipMemcpy(eatom, eatom_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
   }
   void fetch_batch_device(int nstruct, double *energy, double *forces, double *virial, double *eatom) override
@@ -816,9 +837,10 @@ class EngineBase : public Engine, protected BufRegistry {
     HIP_CHECK(hipStreamSynchronize(stream_));
     check_zero_bond();    // before anything is added to the caller's arrays
     const bool wf = forces && ran_forces_, we = eatom && ran_eatom_;
+    if (n_nodes_ > n_ && atom) throw Error("fetch_add_device: a list with ghost atoms keeps the caller's atom order");
     if (n_ > 0 && (wf || we))
-      hipLaunchKernelGGL(k_add_results, dim3((unsigned) ((n_ + 255) / 256)), dim3(256), 0, stream_, atom, n_, f_.as<double>(), wf ? forces : nullptr,
-                         eatom_.as<double>(), we ? eatom : nullptr);
+      hipLaunchKernelGGL(k_add_results, dim3((unsigned) ((n_nodes_ + 255) / 256)), dim3(256), 0, stream_, atom, n_nodes_, n_, f_.as<double>(),
+                         wf ? forces : nullptr, eatom_.as<double>(), we ? eatom : nullptr);
     double s[8];
     HIP_CHECK(hipMemcpyAsync(s, scal_.p, sizeof(s), hipMemcpyDeviceToHost, stream_));
     HIP_CHECK(hipStreamSynchronize(stream_));
@@ -872,9 +894,9 @@ class EngineBase : public Engine, protected BufRegistry {
     HIP_CHECK(hipSetDevice(device_));
     ev_used_ = 0;
     const int n = n_;
-    f_.ensure(std::max<size_t>((size_t) 3 * n, 1) * sizeof(double));
+    f_.ensure(std::max<size_t>((size_t) 3 * n_nodes_, 1) * sizeof(double));
     eatom_.ensure(std::max<size_t>(n, 1) * sizeof(double));
-    HIP_CHECK(hipMemsetAsync(f_.p, 0, (size_t) 3 * n * sizeof(double), stream_));
+    HIP_CHECK(hipMemsetAsync(f_.p, 0, (size_t) 3 * n_nodes_ * sizeof(double), stream_));
     HIP_CHECK(hipMemsetAsync(scal_.p, 0, (size_t) 8 * nstruct_ * sizeof(double), stream_));
     ran_ = true;
     n_peak_ = std::max(n_peak_, n_);
@@ -1092,6 +1114,56 @@ class EngineBase : public Engine, protected BufRegistry {
 #undef GR_GEMM
   }
 
+  // ---- exchange with ghost atoms ------------------------------------------------------------------------------
+  void exchange_forward(int layer)
+  {
+    if (!exchange_.forward || n_nodes_ == n_) return;
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    exchange_.forward(exchange_.user, layer);
+  }
+  void exchange_reverse(int layer)
+  {
+    if (!exchange_.reverse || n_nodes_ == n_) return;
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    exchange_.reverse(exchange_.user, layer);
+  }
+  // The four row movers on rows [atom][function][CP] of which the first nf functions and C channels travel
+  // (nf C doubles per atom); stride: elements per atom.
+  template<class T> void move_rows(int mode, T *rows, long long stride, int nf, int C, int CP, int n, const int *list, int first, double *buf, bool host)
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (n <= 0) return;
+    if (!rows) throw Error(who_ + ": the message rows do not exist yet (the exchange runs inside a pass)");
+    const bool by_list = mode == 0 || mode == 3;
+    if (by_list && !list) throw InvalidArgument("the atom list of the exchange is missing");
+    if (!buf) throw InvalidArgument("the buffer of the exchange is missing");
+    const size_t count = (size_t) n * nf * C;
+    const int *dl = list;
+    double *db = buf;
+    if (host) {
+      comm_buf_.ensure(count * sizeof(double));
+      db = comm_buf_.as<double>();
+      if (by_list) {
+        for (int k = 0; k < n; k++)
+          if (list[k] < 0 || list[k] >= n_nodes_) throw InvalidArgument("the atom list of the exchange names an atom outside the owned and ghost atoms");
+        comm_list_.ensure((size_t) n * sizeof(int));
+        HIP_CHECK(hipMemcpyAsync(comm_list_.p, list, (size_t) n * sizeof(int), hipMemcpyHostToDevice, stream_));
+        dl = comm_list_.as<int>();
+      }
+      if (mode == 1 || mode == 3) HIP_CHECK(hipMemcpyAsync(db, buf, count * sizeof(double), hipMemcpyHostToDevice, stream_));
+    }
+    if (!by_list && (first < 0 || first + n > n_nodes_)) throw InvalidArgument("the atom range of the exchange lies outside the owned and ghost atoms");
+    const dim3 grid((unsigned) ((count + 255) / 256)), block(256);
+    if (mode == 0 || mode == 2)
+      hipLaunchKernelGGL(k_comm_pack<T>, grid, block, 0, stream_, (const T *) rows, stride, nf, C, CP, by_list ? dl : nullptr, first, n, db);
+    else
+      hipLaunchKernelGGL(k_comm_unpack<T>, grid, block, 0, stream_, rows, stride, nf, C, CP, by_list ? dl : nullptr, first, n, (const double *) db,
+                         mode == 3 ? 1 : 0);
+    HIP_CHECK(hipGetLastError());
+    if (host && (mode == 0 || mode == 2)) HIP_CHECK(hipMemcpyAsync(buf, db, count * sizeof(double), hipMemcpyDeviceToHost, stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));
+  }
+
   // ---- chunks of atoms ---------------------------------------------------------------------------------------
   // Atoms per pass for a structure whose work buffers take `per_atom` bytes per atom of a chunk and `kept` bytes per atom
   // of the structure, after the reference's policy (libgrace/include/grace/kk/support.h:425-450): everything in one pass
@@ -1165,6 +1237,10 @@ class EngineBase : public Engine, protected BufRegistry {
   int nelem_;
   std::vector<double> cut_host_;
   // uploaded structure
+  int n_nodes_ = 0;           // central atoms and ghosts (= n_ without ghosts)
+  uint64_t upload_serial_ = 0;
+  ExchangeCallbacks exchange_{};
+  DevBuf comm_list_, comm_buf_;    // staging of the host forms of the row movers
   int n_ = 0, n_peak_ = 0;    // atoms of the uploaded structure; of the largest pass since the work buffers were released
   int64_t nb_ = 0;
   bool have_rij_ = false;

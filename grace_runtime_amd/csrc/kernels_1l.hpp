@@ -107,6 +107,31 @@ __device__ inline void sh_eval(const ShCoef &co, double rx, double ry, double rz
   }
 }
 
+// Message rows to and from an exchange buffer (the pack / unpack kernels of the reference's GPU engines,
+// libgrace/include/grace/kk/grace_2l_kk.h:141-157): rows[atom][function][CP], of which nf functions x C channels travel
+// as doubles; the atoms are list[0 .. n) or first .. first + n.  add: the buffer is added to the rows (reverse exchange).
+template<class T>
+__global__ void k_comm_pack(const T *rows, long long stride, int nf, int C, int CP, const int *list, int first, int n, double *buf)
+{
+  const long long e = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (e >= (long long) n * nf * C) return;
+  const int c = (int) (e % C), fn = (int) ((e / C) % nf), k = (int) (e / ((long long) C * nf));
+  const int atom = list ? list[k] : first + k;
+  buf[e] = (double) rows[atom * stride + (long long) fn * CP + c];
+}
+template<class T>
+__global__ void k_comm_unpack(T *rows, long long stride, int nf, int C, int CP, const int *list, int first, int n, const double *buf, int add)
+{
+  const long long e = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (e >= (long long) n * nf * C) return;
+  const int c = (int) (e % C), fn = (int) ((e / C) % nf), k = (int) (e / ((long long) C * nf));
+  const int atom = list ? list[k] : first + k;
+  T *dst = rows + atom * stride + (long long) fn * CP + c;
+  // several entries of a send list may name one atom (an atom with several images): atomic add
+  if (add) atomicAdd(dst, (T) buf[e]);
+  else *dst = (T) buf[e];
+}
+
 // plain copy of n doubles: the calibration kernel for the HBM counters (FETCH_SIZE / WRITE_SIZE per byte moved)
 static __global__ void k_copy_calibration(const double *src, double *dst, long long n)
 {
@@ -203,17 +228,19 @@ static __global__ void k_unpack_records(const double *rec, int nstruct, double *
 }
 
 // f[atom[q]] += fe[q], eatom[atom[q]] += ee[q] for the n rows of the engine (null pointers are skipped)
-static __global__ void k_add_results(const int *atom, int n, const double *fe, double *f, const double *ee, double *eatom)
+// adds the pass's forces (rows 0 .. nf) and atom energies (rows 0 .. ne) to the caller's arrays; atom: caller's index of row q,
+// null when the rows are in the caller's order
+static __global__ void k_add_results(const int *atom, int nf, int ne, const double *fe, double *f, const double *ee, double *eatom)
 {
   const int q = blockIdx.x * blockDim.x + threadIdx.x;
-  if (q >= n) return;
-  const long long i = atom[q];
-  if (f) {
+  if (q >= nf && q >= ne) return;
+  const long long i = atom ? atom[q] : q;
+  if (f && q < nf) {
     f[3 * i] += fe[3 * (long long) q];
     f[3 * i + 1] += fe[3 * (long long) q + 1];
     f[3 * i + 2] += fe[3 * (long long) q + 2];
   }
-  if (eatom) eatom[i] += ee[q];
+  if (eatom && q < ne) eatom[i] += ee[q];
 }
 
 struct Edges {

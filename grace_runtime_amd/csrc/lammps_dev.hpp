@@ -1,7 +1,8 @@
 // The LAMMPS pair-style call with every per-atom array in device memory (the RunInput of the reference's GPU engines,
 // libgrace/include/grace/kk/grace_1l_kk.h:80-103: x, f, type, ilist, numneigh and the 2-d neighbour view of a KOKKOS
 // pair style).  The full neighbour list is turned into the engine's CSR list with bond vectors by two kernels (count,
-// fill) without leaving the device; the owner map stands in for the exchange of the reference on one rank.
+// fill) without leaving the device; the owner map stands in for the exchange of the reference on one rank, with an
+// exchange installed the ghosts stay atoms of their own.
 #pragma once
 
 #include "engine_common.hpp"
@@ -19,6 +20,7 @@ struct LmpListDev {
   const int *atom;         // [n] owned atom of engine row q
   const unsigned char *mapped;    // [ntypes + 1] type has a model element
   int n, nlocal, nall, neighmask;
+  int nodes;               // 1: ghosts are atoms of their own (an exchange moves their rows): a neighbour keeps its index
 };
 
 // FILL = false: count[q] = bonds of row q to atoms of mapped types; *err = 1: neighbour index outside the atoms,
@@ -43,13 +45,16 @@ __global__ void k_lmp_rows(LmpListDev L, int *count, int *err, const long long *
     const int ta = L.type[a];
     if (!L.mapped[ta]) continue;
     int o = a;
-    if (a >= L.nlocal) o = L.owner ? L.owner[a] : -1;
-    if (o < 0 || o >= L.nlocal || L.idx[o] < 0 || L.type[o] != ta) {
-      if (!FILL) *err = 2;
-      continue;
+    if (!L.nodes) {
+      if (a >= L.nlocal) o = L.owner ? L.owner[a] : -1;
+      if (o < 0 || o >= L.nlocal || L.idx[o] < 0 || L.type[o] != ta) {
+        if (!FILL) *err = 2;
+        continue;
+      }
+      o = L.idx[o];
     }
     if (FILL) {
-      j[w] = L.idx[o];
+      j[w] = o;
       rij[3 * w] = L.x[3 * (long long) a] - xi0;
       rij[3 * w + 1] = L.x[3 * (long long) a + 1] - xi1;
       rij[3 * w + 2] = L.x[3 * (long long) a + 2] - xi2;
@@ -65,6 +70,12 @@ __global__ void k_lmp_rows(LmpListDev L, int *count, int *err, const long long *
 struct LammpsDeviceList {
   DevBuf idx, atom, mapped, count, err, offset, j, rij;
   int64_t nb = 0;
+  // what the kept list was made for: a call that says "same list" and matches it only renews the bond vectors
+  bool kept = false;
+  int n = 0, nlocal = 0, nall = 0, inum = 0, nodes = 0, neighmask = 0;
+  long long stride_i = 0, stride_k = 0;
+  const void *neighbors = nullptr, *type = nullptr, *numneigh = nullptr, *owner = nullptr;
+  uint64_t serial = 0;
 };
 
 }    // namespace grhip

@@ -196,6 +196,70 @@ class Engine:
     def cutoff(self, t1: int, t2: int) -> float:
         return _lib.lib().gr_engine_cutoff(self._h, int(t1), int(t2))
 
+    # ---- message exchange with ghost atoms (gr_engine_set_exchange and the row movers) ----
+    class _Exchange(C.Structure):
+        _fields_ = [("forward", C.c_void_p), ("reverse", C.c_void_p), ("user", C.c_void_p)]
+
+    def set_exchange(self, forward=None, reverse=None):
+        """forward(layer) / reverse(layer) are called inside compute_lammps when the message rows / adjoint rows of a layer
+        are complete (the Exchange of the reference's drivers); both None removes the exchange."""
+        cbt = C.CFUNCTYPE(None, C.c_void_p, C.c_int)
+        if forward is None and reverse is None:
+            check(_lib.lib().gr_engine_set_exchange(self._h, None))
+            self._exchange_keepalive = None
+            return
+        f = cbt(lambda user, layer: forward(int(layer))) if forward else None
+        r = cbt(lambda user, layer: reverse(int(layer))) if reverse else None
+        x = Engine._Exchange(C.cast(f, C.c_void_p) if f else None, C.cast(r, C.c_void_p) if r else None, None)
+        check(_lib.lib().gr_engine_set_exchange(self._h, C.byref(x)))
+        self._exchange_keepalive = (f, r)
+
+    @property
+    def comm_layers(self) -> int:
+        return int(_lib.lib().gr_engine_comm_layers(self._h))
+
+    def comm_width(self, layer: int) -> int:
+        return int(_lib.lib().gr_engine_comm_width(self._h, int(layer)))
+
+    def pack_forward_host(self, layer, sendlist):
+        sl = as_array(sendlist, np.int32)
+        buf = np.zeros((sl.shape[0], self.comm_width(layer)))
+        check(_lib.lib().gr_engine_pack_forward_host(self._h, int(layer), sl.shape[0], ptr(sl), ptr(buf)))
+        return buf
+
+    def unpack_forward_host(self, layer, first, buf):
+        buf = np.ascontiguousarray(buf, dtype=np.float64)
+        check(_lib.lib().gr_engine_unpack_forward_host(self._h, int(layer), buf.shape[0], int(first), ptr(buf)))
+
+    def pack_reverse_host(self, layer, first, n):
+        buf = np.zeros((int(n), self.comm_width(layer)))
+        check(_lib.lib().gr_engine_pack_reverse_host(self._h, int(layer), int(n), int(first), ptr(buf)))
+        return buf
+
+    def unpack_reverse_host(self, layer, sendlist, buf):
+        sl = as_array(sendlist, np.int32)
+        buf = np.ascontiguousarray(buf, dtype=np.float64)
+        check(_lib.lib().gr_engine_unpack_reverse_host(self._h, int(layer), sl.shape[0], ptr(sl), ptr(buf)))
+
+    def pack_forward(self, layer, sendlist, buf):
+        """device form: sendlist int32 [n] and buf float64 [n, comm_width] are arrays of the module's GPU"""
+        n = int(sendlist.shape[0])
+        check(_lib.lib().gr_engine_pack_forward(self._h, int(layer), n, _device_pointer(sendlist, "sendlist", (n,), "int32"),
+                                                _device_pointer(buf, "buf", (n, self.comm_width(layer)), "float64")))
+
+    def unpack_forward(self, layer, first, buf):
+        n = int(buf.shape[0])
+        check(_lib.lib().gr_engine_unpack_forward(self._h, int(layer), n, int(first), _device_pointer(buf, "buf", (n, self.comm_width(layer)), "float64")))
+
+    def pack_reverse(self, layer, first, buf):
+        n = int(buf.shape[0])
+        check(_lib.lib().gr_engine_pack_reverse(self._h, int(layer), n, int(first), _device_pointer(buf, "buf", (n, self.comm_width(layer)), "float64")))
+
+    def unpack_reverse(self, layer, sendlist, buf):
+        n = int(sendlist.shape[0])
+        check(_lib.lib().gr_engine_unpack_reverse(self._h, int(layer), n, _device_pointer(sendlist, "sendlist", (n,), "int32"),
+                                                  _device_pointer(buf, "buf", (n, self.comm_width(layer)), "float64")))
+
     def set_chunksize(self, atoms: int):
         """atoms per engine pass: 0 one pass, < 0 automatic, > 0 as given"""
         check(_lib.lib().gr_engine_set_chunksize(self._h, int(atoms)))
@@ -276,11 +340,13 @@ class Engine:
         return out
 
     def compute_lammps_device(self, nlocal, types, x, ilist, numneigh, neighbors, owner=None, neighmask=0x1FFFFFFF, energy_only=False,
-                              forces=None, eatom=None):
+                              forces=None, eatom=None, same_list=False):
         """The call of a KOKKOS pair style (gr_compute_lammps_device): every array is a device array of the module's GPU
         (torch tensors): `types[nall]` int32, `x[nall, 3]`, `ilist[inum]`, `numneigh[nlocal]`, the 2-d neighbour view
         `neighbors[nlocal, maxneigh]` in either layout, `owner[nall]`.  Forces are ADDED to `forces[nall, 3]` and per-atom
-        energies to `eatom[nall]` in place; energy and virial come back on the host."""
+        energies to `eatom[nall]` in place; energy and virial come back on the host.  `same_list`: the arrays are those
+        of the previous call and only the contents of `x` changed (the steps between two reneighbourings): the converted
+        list is kept and only its bond vectors are renewed."""
         nall, inum = int(types.shape[0]), int(ilist.shape[0])
         p_t = _device_pointer(types, "types", (nall,), "int32")
         p_x = _device_pointer(x, "x", (nall, 3), "float64")
@@ -293,7 +359,7 @@ class Engine:
         p_f = _device_pointer(forces, "forces", (nall, 3), "float64") if forces is not None else None
         p_ea = _device_pointer(eatom, "eatom", (nall,), "float64") if eatom is not None else None
         e, v = C.c_double(), np.zeros(6)
-        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if eatom is not None else 0)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if eatom is not None else 0) | (_lib.FLAG_SAME_LIST if same_list else 0)
         check(_lib.lib().gr_compute_lammps_device(self._h, int(nlocal), nall, len(self.species), p_t, p_x, inum, p_il, p_nn,
                                                   C.c_void_p(neighbors.data_ptr()), int(neighbors.stride(0)), int(neighbors.stride(1)),
                                                   int(neighmask), p_own, flags, C.byref(e), None if energy_only else p_f, ptr(v), p_ea))

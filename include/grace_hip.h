@@ -32,8 +32,13 @@ enum {
   GR_FLAG_ENERGY_ONLY = 1, /* ComputeFlags::energy_only (libgrace/include/grace/system.h:118): no forces / virial */
   GR_FLAG_EATOM = 2,       /* ComputeFlags::eflag_atom (system.h:114): per-atom energies */
   GR_FLAG_UQ = 4,          /* ComputeFlags::uq (system.h:117): the UQ head; gr_engine_run and gr_system_compute */
-  GR_FLAG_ACCUMULATE = 8   /* gr_compute_csr: energy, forces, virial and per-atom energies are ADDED to the caller's values, as
+  GR_FLAG_ACCUMULATE = 8,  /* gr_compute_csr: energy, forces, virial and per-atom energies are ADDED to the caller's values, as
                               the reference's Outputs accumulate (system.h:66-75); without it they are overwritten */
+  GR_FLAG_SAME_LIST = 16   /* gr_compute_lammps_device: atom counts, types, ilist, neighbour list and owner map are those of the
+                              previous call on this engine and only x has changed (LAMMPS: neighbor->ago > 0, the steps between
+                              two reneighbourings): the converted list is kept, only the bond vectors are renewed and no array
+                              makes a trip to the host.  The reference's engines walk the whole list in every run; this flag has
+                              no counterpart there.  A hint: when the engine no longer holds that list the call converts anew */
 };
 
 typedef struct gr_model_info {
@@ -191,6 +196,38 @@ int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *clust
 int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const double *x, int inum, const int *ilist, const int *numneigh,
                       const int *const *firstneigh, int neighmask, const int *owner, unsigned flags, double *energy, double *f,
                       double *virial, double *eatom);
+
+/* Message exchange between owned atoms and ghosts, for ghosts that are NOT images of this rank's atoms (several MPI
+ * ranks): replaces the Exchange of the reference's drivers (libgrace/include/grace/system.h:53-60) and the comm surface of
+ * its GPU engines (comm_width, pack_forward / unpack_forward / pack_reverse / unpack_reverse and their _host forms,
+ * libgrace/include/grace/kk/grace_2l_kk.h:141-157, grace_3l_kk.h:313-324).
+ * With an exchange installed (or a GRACE-1L engine, which has no message) gr_compute_lammps with owner = NULL keeps the
+ * ghosts as atoms of their own: during the call forward(user, layer) is called when the message rows of the owned atoms of
+ * `layer` (1 .. gr_engine_comm_layers: 0 for GRACE-1L, 1 for 2L, 2 for 3L) are complete -- it must fill the ghosts' rows,
+ * as LAMMPS' comm->forward_comm does through pack_forward / unpack_forward -- and reverse(user, layer) when the adjoint rows
+ * are complete -- it must add the ghosts' rows to their owners' (pack_reverse / unpack_reverse).  Forces left on ghosts
+ * are added to f [nall][3] for LAMMPS' reverse communication of f.  Every owned and ghost atom needs a mapped type.
+ * Row movers: gr_engine_comm_width doubles per atom; atoms by LAMMPS index (owned 0 .. nlocal-1, ghosts after);
+ * pack_forward: rows of sendlist[0 .. n) -> buf; unpack_forward: buf -> rows of first .. first + n; pack_reverse: adjoint
+ * rows of first .. first + n -> buf; unpack_reverse: buf ADDED to the adjoint rows of sendlist[0 .. n).  sendlist and buf
+ * are device memory of the engine's GPU, host memory for the _host forms.  They may only be called from inside the
+ * callbacks of the matching direction and layer; each returns when its copy is done. */
+typedef struct gr_exchange {
+  void (*forward)(void *user, int layer);
+  void (*reverse)(void *user, int layer);
+  void *user;
+} gr_exchange;
+int gr_engine_set_exchange(gr_engine *e, const gr_exchange *x);    /* NULL: none */
+int gr_engine_comm_layers(gr_engine *e);
+int gr_engine_comm_width(gr_engine *e, int layer);
+int gr_engine_pack_forward(gr_engine *e, int layer, int n, const int *sendlist, double *buf);
+int gr_engine_unpack_forward(gr_engine *e, int layer, int n, int first, const double *buf);
+int gr_engine_pack_reverse(gr_engine *e, int layer, int n, int first, double *buf);
+int gr_engine_unpack_reverse(gr_engine *e, int layer, int n, const int *sendlist, const double *buf);
+int gr_engine_pack_forward_host(gr_engine *e, int layer, int n, const int *sendlist, double *buf);
+int gr_engine_unpack_forward_host(gr_engine *e, int layer, int n, int first, const double *buf);
+int gr_engine_pack_reverse_host(gr_engine *e, int layer, int n, int first, double *buf);
+int gr_engine_unpack_reverse_host(gr_engine *e, int layer, int n, const int *sendlist, const double *buf);
 
 /* The same call with every per-atom array in DEVICE memory of the engine's GPU: the RunInput / RunOutput of the
  * reference's GPU engines (libgrace/include/grace/kk/grace_1l_kk.h:80-103, grace_2l_kk.h:81-157, grace_3l_kk.h:232-324),

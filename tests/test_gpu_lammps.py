@@ -98,14 +98,103 @@ def test_device_arrays_equal_host_arrays(model_dir, model, species, struct, layo
     assert np.abs(ea.cpu().numpy() - ref["energies"]).max() < 1e-10 * fs
     eo = eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=od, energy_only=True)
     assert abs(eo["energy"] - ref["energy"]) < 1e-10 * max(1.0, abs(ref["energy"]))
-    with pytest.raises(ValueError, match="owner"):
-        eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=None, forces=f)
+    if eng.comm_layers:                                                     # a message needs the map or an exchange
+        with pytest.raises(ValueError, match="owner map"):
+            eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=None, forces=f)
+    else:                                                                   # GRACE-1L: the ghosts keep what they receive
+        f2 = torch.zeros_like(f)
+        loose = eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=None, forces=f2)
+        folded = f2[:n].cpu().numpy().copy()
+        np.add.at(folded, owner[n:], f2[n:].cpu().numpy())
+        assert abs(loose["energy"] - ref["energy"]) < 1e-10 * max(1.0, abs(ref["energy"]))
+        assert np.abs(folded - (ref["forces"][:n] - f0[:n])).max() < 1e-9 * fs
     bad = od.clone()
     bad[n:] = n + 5
     with pytest.raises(ValueError, match="owner of a ghost"):
         eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=bad, forces=f)
     with pytest.raises(ValueError, match="must be on the module's GPU"):
         eng.compute_lammps_device(n, td, torch.as_tensor(x), il, nn, nb, owner=od, forces=f)
+
+
+@pytest.mark.parametrize("model,species,struct", [("mix2", ["Mo", "W"], "alloy54"), ("l3mix", ["Mo", "W"], "triclinic")])
+def test_same_list_renews_only_the_bond_vectors(model_dir, model, species, struct):
+    """the steps between two reneighbourings: the arrays stay, the positions in them move; a call with same_list gives what a
+    call that converts the list anew gives, and falls back to the conversion when the engine holds another list"""
+    import torch
+    eng = kk.Engine(kk.Model(cases.model_file(model_dir, model)), species, 64)
+    fresh = kk.Engine(eng.model, species, 64)
+    pos, cell, pbc, types = cases.STRUCTURES[struct]()
+    n = len(pos)
+    rc = max(eng.cutoff(a, b) for a in (1, 2) for b in (1, 2))
+    x, t, owner, rows = lammps_inputs(pos, cell, types, rc + 0.7)
+    dev = torch.device("cuda", 0)
+    nbh = np.zeros((n, max(len(r) for r in rows)), np.int32)
+    for i, r in enumerate(rows):
+        nbh[i, :len(r)] = r
+    td, xd, od, nb = (torch.as_tensor(a, device=dev) for a in (t, x, owner, nbh))
+    il = torch.arange(n, dtype=torch.int32, device=dev)
+    nn = torch.as_tensor(np.array([len(r) for r in rows], np.int32), device=dev)
+    rng = np.random.default_rng(5)
+
+    def call(e, same):
+        f, ea = torch.zeros((len(x), 3), dtype=torch.float64, device=dev), torch.zeros(len(x), dtype=torch.float64, device=dev)
+        out = e.compute_lammps_device(n, td, xd, il, nn, nb, owner=od, forces=f, eatom=ea, same_list=same)
+        return out["energy"], out["virial"], f.cpu().numpy(), ea.cpu().numpy()
+
+    first = call(eng, True)                                  # nothing kept yet: converts
+    e0 = first[0]
+    for step in range(3):
+        d = 0.02 * rng.standard_normal((n, 3))
+        xd += torch.as_tensor(d[owner], device=dev)          # owners and their images move together
+        got, want = call(eng, True), call(fresh, False)
+        assert abs(got[0] - want[0]) < 1e-11 * max(1.0, abs(want[0])) and abs(got[0] - e0) > 1e-6
+        for a, b in zip(got[1:], want[1:]):                  # sums by atomic adds: equal up to their order
+            assert np.abs(a - b).max() < 1e-11 * max(1.0, np.abs(b).max())
+    # another list on the engine in between: the hint is dropped and the list converted again
+    eng.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows, owner=owner)
+    got, want = call(eng, True), call(fresh, False)
+    assert abs(got[0] - want[0]) < 1e-11 * max(1.0, abs(want[0]))
+    assert all(np.abs(a - b).max() < 1e-11 * max(1.0, np.abs(b).max()) for a, b in zip(got[1:], want[1:]))
+
+
+def test_cxx_adapter_header_runs_a_pair_style_pass(model_dir, tmp_path):
+    """include/grace_hip_lammps.hpp (set_model / setup / run(RunInput) -> RunOutput, as a KOKKOS pair style would use it) from
+    a C++ program: two passes, the second with same_list on moved atoms, against the Python mirror on the same arrays"""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "tests", "build", "adapter_run")
+    if not os.path.exists(exe) or os.path.getmtime(exe) < os.path.getmtime(os.path.join(root, "include", "grace_hip_lammps.hpp")):
+        sys.path.insert(0, root)
+        import __graft_entry__
+        exe = __graft_entry__.build_adapter_driver()
+    path = cases.model_file(model_dir, "l2mix")
+    eng = kk.Engine(kk.Model(path), ["Mo", "W"], 64)
+    pos, cell, pbc, types = cases.structure_triclinic()
+    n = len(pos)
+    x, t, owner, rows = lammps_inputs(pos, cell, types, eng.cutoff(1, 2) + 0.7)
+    maxn = max(len(r) for r in rows)
+    nbh = np.zeros((n, maxn), np.int32)
+    for i, r in enumerate(rows):
+        nbh[i, :len(r)] = r
+    dx = (0.03 * np.random.default_rng(3).standard_normal((n, 3)))[owner]
+    with open(tmp_path / "in.bin", "wb") as f:
+        for a in (np.array([n, len(x), maxn, 2], np.int32), np.array(eng.model.type2mu(["Mo", "W"]), np.int32), t,
+                  np.array([len(r) for r in rows], np.int32), nbh, owner, x, dx):
+            f.write(np.ascontiguousarray(a).tobytes())
+    res = subprocess.run([exe, path, str(tmp_path / "in.bin")], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stderr
+    lines = res.stdout.strip().split("\n")
+    nall = len(x)
+    assert len(lines) == 2 * (nall + 1) + 1 and lines[-1].startswith("cutoff ") and lines[-1].endswith("layers 1")
+    for k, xs in enumerate((x, x + dx)):
+        want = eng.compute_lammps(n, t, xs, np.arange(n), [len(r) for r in rows], rows, owner=owner, energies=True)
+        head = np.array(lines[k * (nall + 1)].split(), float)
+        body = np.array([ln.split() for ln in lines[k * (nall + 1) + 1:(k + 1) * (nall + 1)]], float)
+        fs = max(1.0, np.abs(want["forces"]).max())
+        assert abs(head[0] - want["energy"]) < 1e-11 * max(1.0, abs(want["energy"]))
+        assert np.abs(head[1:] - want["virial"]).max() < 1e-10 * max(1.0, np.abs(want["virial"]).max())
+        assert np.abs(body[:, :3] - want["forces"]).max() < 1e-11 * fs and np.abs(body[:, 3] - want["energies"]).max() < 1e-11 * fs
 
 
 def test_unmapped_types_take_no_part_and_argument_errors(model_dir):
@@ -132,8 +221,16 @@ def test_unmapped_types_take_no_part_and_argument_errors(model_dir):
         assert np.abs(out["forces"][:n] - ref["forces"][:n]).max() < 1e-9 and np.all(out["forces"][n:n + 5] == 0)
         with pytest.raises(RuntimeError, match="unmapped type"):
             eng3.compute_lammps(n + 5, t3, x3, np.arange(n + 5), [len(r) for r in rows3], rows3, owner=owner3)
+    # without an owner map a GRACE-1L engine keeps the ghosts as atoms of their own (no message to exchange): the forces they
+    # receive stay on them, and folded back onto their owners they give the result of the call with the map
+    loose = eng2.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows)
+    folded = loose["forces"][:n].copy()
+    np.add.at(folded, owner[n:], loose["forces"][n:])
+    assert abs(loose["energy"] - ref["energy"]) < 1e-10 * abs(ref["energy"]) and np.abs(folded - ref["forces"][:n]).max() < 1e-9
+    # an engine with a message needs the map or an exchange
+    two = kk.Engine(kk.Model(cases.model_file(model_dir, "l2mix")), ["Mo", "W"], 64)
     with pytest.raises(ValueError, match="owner map"):
-        eng2.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows)
+        two.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows)
     with pytest.raises(ValueError, match="must be in ilist"):
         eng2.compute_lammps(n, t, x, np.arange(n - 1), [len(r) for r in rows], rows, owner=owner)
     bad = owner.copy()
