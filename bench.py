@@ -44,6 +44,7 @@ MEASURED_TRAFFIC = {
     ("config2", "radial_mlp"): 7.0e6 + 1216.3e6,        # fetch + write of k_radial<double,4,0,0,true>
     ("config3", "pair_bwd"): 11234.9e6 + 2773.0e6,      # fetch + write of k_pair_bwd<double,25>
     ("config4", "pair_bwd_L3"): 48727e6 + 30596e6,      # the layer-3 launches of k_pair_bwd<double,36> (layer 2: 25.6 + 15.2 GB)
+    ("config5", "pair_bwd"): 9811.7e6 + 2477.6e6,       # fetch + write of k_pair_bwd<double,25> over the ragged batch
 }
 # the per-atom dense chain of configuration 2 (every FC, product, reduce and readout launch of a pass), same counters
 DENSE_TRAFFIC = {"config2": 6.5e9}
@@ -151,6 +152,7 @@ def main():
             eng.upload(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)
     upload()
     eng.debug_copy(1 << 30)     # k_copy_calibration over 1 GiB: scales the rocprof FETCH_SIZE / WRITE_SIZE counters
+    copy_gbs, read_gbs = eng.stream_rates(1 << 30)      # what plain stream kernels reach on this GPU (HIP events)
 
     for _ in range(a.warmup):
         eng.run()
@@ -228,7 +230,7 @@ def main():
     eng.set_profile(False)
     stages = {k: v / a.steps for k, v in acc.items()}
 
-    C, nl, nlm, s = (64, 6, 36, 8) if three else (32, 5, 25, a.precision // 8)
+    C, nl, nlm, s = (64, 6, 36, a.precision // 8) if three else (32, 5, 25, a.precision // 8)
     # GRACE-3L: message functions gathered by the pair kernels of layers 2 and 3; radial MLP 8-128-128-384, value + tangent
     extra = dict(radial_flops=4.0 * (8 * 128 + 128 * 128 + 128 * 384), slots={"2": 36, "3": 72}) if three else {}
     # FC / reduce tile GEMMs: flops of the live functions as the engine counts them
@@ -320,6 +322,9 @@ def main():
                                                           "neighbour_list_kept": round(list_ms["kept"], 3)},
         "engine_create_s": round(create_s, 3),
         "roofline": roofline,
+        "hbm_calibration": {"copy_GBs": round(copy_gbs, 1), "read_only_GBs": round(read_gbs, 1), "bytes": 1 << 30,
+                            "note": "plain stream kernels over 1 GiB, best of 5: copy counts bytes read + written; roofline.frac "
+                                    "divides by the published 8000 GB/s, not by these"},
         "dense_chain": dense,
         "stages_ms": {k: round(v, 4) for k, v in stages.items()},
         "stages_roofline": {k: {"bound": v["bound"], "achieved": round(v["achieved"], 2), "unit": v["unit"],

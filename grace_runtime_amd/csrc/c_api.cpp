@@ -447,6 +447,14 @@ int gr_engine_debug_copy(gr_engine *e, int64_t bytes)
   });
 }
 
+int gr_engine_stream_rates(gr_engine *e, int64_t bytes, double *copy_gbs, double *read_gbs)
+{
+  return guarded([&] {
+    if (!e || bytes < 16) throw grhip::InvalidArgument("null engine or no bytes");
+    live(e).stream_rates(bytes, copy_gbs, read_gbs);
+  });
+}
+
 int gr_neighbor_build(int64_t n, const double *positions, const double *cell, const unsigned char *pbc, double cutoff,
                       int nthreads, gr_nlist **out)
 {

@@ -130,6 +130,8 @@ class Engine {
   virtual int64_t last_edge_count() = 0;
   // a plain device-to-device copy kernel over `bytes` bytes (calibration of the memory-traffic counters)
   virtual void debug_copy(int64_t bytes) = 0;
+  // measured rates (GB/s) of that copy kernel and of a read-only stream kernel: the ceilings HBM-bound kernels are compared with
+  virtual void stream_rates(int64_t bytes, double *copy_gbs, double *read_gbs) = 0;
   // radial functions of the device kernel for the given x = r / rc and neighbour elements: R z and dR/dx z,
   // [m][nl][C] (tests of the MFMA kernel against the CPU restatement)
   virtual void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) = 0;

@@ -627,6 +627,37 @@ class EngineBase : public Engine, protected BufRegistry {
     check(hipGetLastError(), "copy kernel");
     check(hipStreamSynchronize(stream_), "hipStreamSynchronize");
   }
+  // GB/s of the copy kernel (bytes read + bytes written) and of a read-only stream kernel over `bytes` bytes, best of 5
+  void stream_rates(int64_t bytes, double *copy_gbs, double *read_gbs) override
+  {
+    check(hipSetDevice(device_), "hipSetDevice");
+    const long long nd = std::max<int64_t>(bytes / 16, 1) * 2;
+    DevBuf a, b, part;
+    a.ensure(nd * 8);
+    b.ensure(nd * 8);
+    part.ensure(4096 * 8);
+    check(hipMemsetAsync(a.p, 0, nd * 8, stream_), "hipMemsetAsync");
+    check(hipMemsetAsync(part.p, 0, 4096 * 8, stream_), "hipMemsetAsync");
+    hipEvent_t e0, e1;
+    check(hipEventCreate(&e0), "hipEventCreate");
+    check(hipEventCreate(&e1), "hipEventCreate");
+    double best[2] = {1e30, 1e30};
+    for (int rep = 0; rep < 6; rep++)
+      for (int k = 0; k < 2; k++) {
+        check(hipEventRecord(e0, stream_), "hipEventRecord");
+        if (k == 0) hipLaunchKernelGGL(k_copy_calibration, dim3(4096), dim3(256), 0, stream_, a.as<double>(), b.as<double>(), nd);
+        else hipLaunchKernelGGL(k_read_calibration, dim3(4096), dim3(256), 0, stream_, a.as<double>(), part.as<double>(), nd);
+        check(hipEventRecord(e1, stream_), "hipEventRecord");
+        check(hipEventSynchronize(e1), "hipEventSynchronize");
+        float ms = 0.f;
+        check(hipEventElapsedTime(&ms, e0, e1), "hipEventElapsedTime");
+        if (rep > 0) best[k] = std::min(best[k], (double) ms);
+      }
+    (void) hipEventDestroy(e0);
+    (void) hipEventDestroy(e1);
+    if (copy_gbs) *copy_gbs = 2.0 * nd * 8 / (best[0] * 1e-3) * 1e-9;
+    if (read_gbs) *read_gbs = 1.0 * nd * 8 / (best[1] * 1e-3) * 1e-9;
+  }
 
   // copies a CSR structure to the device after the argument checks of the reference's CSR entry
   // (python/src/core.cpp:292-396); atoms are grouped into tiles of 16 of one element for the tile GEMMs

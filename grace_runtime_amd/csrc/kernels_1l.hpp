@@ -138,6 +138,20 @@ static __global__ void k_copy_calibration(const double *src, double *dst, long l
   for (long long i = blockIdx.x * (long long) blockDim.x + threadIdx.x; i < n; i += (long long) gridDim.x * blockDim.x) dst[i] = src[i];
 }
 
+// read-only stream over n doubles (16 bytes per lane and step, one partial sum written per block): what a kernel that
+// only reads can draw from HBM, next to the copy kernel's rate for one that reads and writes as much
+static __global__ void k_read_calibration(const double *src, double *partial, long long n)
+{
+  const double2 *s2 = reinterpret_cast<const double2 *>(src);
+  double acc = 0.0;
+  for (long long i = blockIdx.x * (long long) blockDim.x + threadIdx.x; i < n / 2; i += (long long) gridDim.x * blockDim.x) {
+    const double2 v = s2[i];
+    acc += v.x + v.y;
+  }
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+  if ((threadIdx.x & 63) == 0) atomicAdd(&partial[blockIdx.x], acc);
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // bond filter
 // ---------------------------------------------------------------------------------------------------------------

@@ -499,6 +499,13 @@ class Engine:
     def debug_copy(self, nbytes):
         check(_lib.lib().gr_engine_debug_copy(self._h, int(nbytes)))
 
+    def stream_rates(self, nbytes=1 << 30):
+        """(copy GB/s counting bytes read + written, read-only GB/s) of two plain stream kernels over nbytes: the HBM
+        rates this GPU shows to a kernel that moves memory and does nothing else"""
+        c, r = C.c_double(), C.c_double()
+        check(_lib.lib().gr_engine_stream_rates(self._h, int(nbytes), C.byref(c), C.byref(r)))
+        return c.value, r.value
+
     def close(self):
         if getattr(self, "_h", None):
             _lib.lib().gr_engine_free(self._h)

@@ -148,6 +148,10 @@ int gr_engine_radial_noalloc(gr_engine *e, int m, const double *x, const int *mu
 /* Runs a plain device-to-device copy kernel (k_copy_calibration) over `bytes` bytes: the known-size kernel that the
  * rocprof memory counters (FETCH_SIZE, WRITE_SIZE) are scaled by.  No counterpart in the reference. */
 int gr_engine_debug_copy(gr_engine *e, int64_t bytes);
+/* Times that copy kernel and a read-only stream kernel over `bytes` bytes with HIP events and returns their rates in
+ * GB/s (copy: bytes read + bytes written): the ceilings this GPU shows to a kernel bound by HBM, which the published peak
+ * is not.  Measurement support of bench.py; no counterpart in the reference. */
+int gr_engine_stream_rates(gr_engine *e, int64_t bytes, double *copy_gbs, double *read_gbs);
 
 /* Neighbour list at `cutoff`, the exact list of grace_runtime::neighbor_search (python/src/neighbors.cpp:15-95):
  * perm [n] (new -> original index), offset [n+1], j [nb] (new indices), image [nb], shifts [nimages][3]. */
