@@ -627,7 +627,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     const size_t lds = (size_t) kPairChunk * (pthreads + 2 * radR1_.noutp) * sizeof(T);
     GR_PAIR(k_pair_bwd, dim3(n), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), dR1_.as<T>(),
             (const T *) M, gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),
-            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_, 0, n);
+            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_, 0, n, 0);
   });
 #undef GR_PAIR
 #undef GR_PAIR1

@@ -176,6 +176,7 @@ template<class T> class Engine3L final : public EngineBase {
     this->template probe_mfma<T>();
     build();
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
+    chunks_ = true;
   }
   int layers() const override { return 3; }
   void run(const RunFlags &fl) override;
@@ -211,12 +212,20 @@ template<class T> class Engine3L final : public EngineBase {
   int comm_reverse_layer_ = 0;    // the message whose adjoint rows gM_ holds while its reverse exchange runs
   // scratch shared by the layers (largest size over the layers): temporaries of the forward pass and all adjoints
   DevBuf M_, gM_, pairP_, gpairP_, A_, gA_, P_, gP_, R2_, R3_, R4_, FA_, FB_, gX_, gR2_, gR3_, gR4_, gFA_, gFB_, gLp_, gRp_, gEQ_;
+  DevBuf gMin_;    // adjoint of the message the layer in reverse SENT (filled by the layer above); gM_: of the one it gathers
+  // the chunk of atoms the layer functions act on: atoms [a0_, a0_ + cn_), their bonds [eb_, eb_ + ecnt_) (ecnt_ < 0: all
+  // bonds), the capacities the chunk buffers are sized for, the chunk's element tiles (atoms counted from a0_)
+  int cn_ = 0, a0_ = 0;
+  size_t cap_ = 0, ecap_ = 1;
+  long long eb_ = 0, ecnt_ = -1;
+  const int *cur_tiles_ = nullptr, *cur_tile_el_ = nullptr;
+  int cur_ntiles_ = 0;
 
   void build();
   void build_layer(int k);
   void gemm(DevJobs<T> &J, int kin, int kout, const T *X, int nfx, T *out, int nfo, int accumulate)
   {
-    EngineBase::launch_gemm<T>(J, kin / 16, kin / 16, kout / 16, X, nfx, X, nfx, out, nfo, accumulate, tiles_.as<int>(), ntiles_);
+    EngineBase::launch_gemm<T>(J, kin / 16, kin / 16, kout / 16, X, nfx, X, nfx, out, nfo, accumulate, cur_tiles_, cur_ntiles_);
   }
   // element-dependent weights: one launch per element over its tiles (tiles hold atoms of one element, elements in order)
   void gemm_el(DevJobs<T> &J, size_t wstride, int nel, int kin, int kout, const T *X, int nfx, T *out, int nfo, int accumulate)
@@ -224,11 +233,11 @@ template<class T> class Engine3L final : public EngineBase {
     if (nel == 1) return gemm(J, kin, kout, X, nfx, out, nfo, accumulate);
     const T *w0 = J.d.WF0, *w1 = J.d.WF1;
     for (int e = 0; e < nel; e++) {
-      const int t0 = tile_el_[e], nt = tile_el_[e + 1] - t0;
+      const int t0 = cur_tile_el_[e], nt = cur_tile_el_[e + 1] - t0;
       if (nt == 0) continue;
       J.d.WF0 = w0 + e * wstride;
       J.d.WF1 = w1 + e * wstride;
-      EngineBase::launch_gemm<T>(J, kin / 16, kin / 16, kout / 16, X, nfx, X, nfx, out, nfo, accumulate, tiles_.as<int>() + (size_t) 16 * t0, nt);
+      EngineBase::launch_gemm<T>(J, kin / 16, kin / 16, kout / 16, X, nfx, X, nfx, out, nfo, accumulate, cur_tiles_ + (size_t) 16 * t0, nt);
     }
     J.d.WF0 = w0;
     J.d.WF1 = w1;
@@ -239,24 +248,26 @@ template<class T> class Engine3L final : public EngineBase {
   // out = contraction (not accumulated): functions without a connection are cleared
   void cfwd_set(DevContract<T> &c, const T *X, T *out)
   {
-    if (!c.all_dst) zero(out, (size_t) n_ * c.ndst * c.kout * sizeof(T));
+    if (!c.all_dst) zero(out, (size_t) cn_ * c.ndst * c.kout * sizeof(T));
     cfwd(c, X, out, c.all_dst ? 0 : 1);
   }
   void cbwd_set(DevContract<T> &c, const T *gout, T *gX)
   {
-    if (!c.all_src) zero(gX, (size_t) n_ * c.nsrc * c.kin * sizeof(T));
+    if (!c.all_src) zero(gX, (size_t) cn_ * c.nsrc * c.kin * sizeof(T));
     cbwd(c, gout, gX, c.all_src ? 0 : 1);
   }
   void couple_fwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, T *out);
   void couple_bwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, const T *g, T *gL, T *gR);
   void scale_rows(const T *in, const DevBuf &s, T *out, int nf, int w, int accumulate)
   {
-    const long long tot = (long long) n_ * nf * w;
+    const long long tot = (long long) cn_ * nf * w;
     if (tot == 0) return;
-    hipLaunchKernelGGL(k_scale_rows<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, in, s.as<T>(), out, n_, nf, w, accumulate);
+    hipLaunchKernelGGL(k_scale_rows<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, in, s.as<T>(), out, cn_, nf, w, accumulate);
   }
-  void layer_forward(int k, bool forces, int yw);
+  void layer_messages(int k);
+  void layer_forward(int k, bool forces, int yw, bool again);
   void layer_backward(int k, int yw);
+  double chunk_bytes_per_atom() const;
   std::string tg(int k, const char *name) { return std::string(name) + "_L" + std::to_string(k + 1); }
 };
 
@@ -569,7 +580,7 @@ template<class T> void Engine3L<T>::build_layer(int k)
 
 template<class T> void Engine3L<T>::couple_fwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, T *out)
 {
-  const int n = n_, KP = p.rankP;
+  const int n = cn_, KP = p.rankP;
   int one = 1, nat = n;
   if (p.jit) {
     void *args[] = {(void *) &Lp, (void *) &Rp, (void *) &out, (void *) &nat, (void *) &one};
@@ -592,7 +603,7 @@ template<class T> void Engine3L<T>::couple_fwd(ProdStage<T> &p, const T *Lp, int
 // gL, gR are accumulated into (zeroed by the caller)
 template<class T> void Engine3L<T>::couple_bwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, const T *g, T *gL, T *gR)
 {
-  const int n = n_, KP = p.rankP;
+  const int n = cn_, KP = p.rankP;
   int one = 1, nat = n, acc = 1;
   if (p.jit) {
     void *args[] = {(void *) &Lp, (void *) &Rp, (void *) &g, (void *) &gL, (void *) &gR, (void *) &acc, (void *) &acc, (void *) &nat, (void *) &one};
@@ -641,41 +652,53 @@ static int slots_per_block(int nslot, int CP)
     default: GR_PAIR1(K_, 49, __VA_ARGS__) break;            \
   }
 
-template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
+// The message layer k gathers, for every atom and ghost: the normalised output of the layer below plus the species term
+// (once per layer, before the chunks of its forward pass and again before those of its reverse: M_ is shared scratch).
+template<class T> void Engine3L<T>::layer_messages(int k)
 {
   Layer3<T> &L = L_[k];
-  const int n = n_;
-  const size_t na = (size_t) n, ecap = (size_t) std::max<int64_t>(nb_, 1), s = sizeof(T);
-  const long long *n_edges = eoff_.as<long long>() + n;
-  L.R.ensure(ecap * L.rad.noutp * s);
-  L.dR.ensure(ecap * L.rad.noutp * s);
+  const Layer3<T> &Lm = L_[k - 1];
+  M_.ensure((size_t) n_nodes_ * L.nlmi * L.CP * sizeof(T));
+  stage(tg(k, "message").c_str(), [&] {
+    const long long tot = (long long) n_nodes_ * L.nlmi * L.CP;
+    hipLaunchKernelGGL(k_message<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, Lm.I.buf.template as<T>(), mu_.as<int>(),
+                       L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n_nodes_, L.nlmi, L.CP);
+  });
+}
+
+// Forward pass of layer k over the atoms of the current chunk.  Per-atom tensors hold the chunk's atoms from row 0 and the
+// radial rows the chunk's bonds from row 0 (kernels index bonds by their number in the structure: the pointers are moved
+// back); the messages, the raw densities and their adjoints are kept for the whole structure.  again: the forward pass
+// repeated before the layer's reverse (a structure evaluated in several chunks keeps no layer tensors between the sweeps).
+template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw, bool again)
+{
+  Layer3<T> &L = L_[k];
+  const int n = cn_;
+  const size_t na = cap_, s = sizeof(T);
+  const long long *n_edges = eoff_.as<long long>() + n_;
+  const long long *eoff = eoff_.as<long long>() + a0_;
+  const int *mu = mu_.as<int>() + a0_;
+  L.R.ensure(ecap_ * L.rad.noutp * s);
+  L.dR.ensure(ecap_ * L.rad.noutp * s);
+  T *Rl = moved_back(L.R.template as<T>(), eb_ * L.rad.noutp), *dRl = moved_back(L.dR.template as<T>(), eb_ * L.rad.noutp);
   stage(tg(k, "radial").c_str(), [&] {
-    L.rad.launch(stream_, ncu_, L.fac.template as<T>(), 0, -1, xr_.as<double>(), emu_.as<int>(), L.R.template as<T>(), L.dR.template as<T>(), n_edges,
-                 emi_.as<int>());
+    L.rad.launch(stream_, ncu_, L.fac.template as<T>(), eb_, ecnt_, xr_.as<double>(), emu_.as<int>(), Rl, dRl, n_edges, emi_.as<int>());
   });
   L.X.buf.ensure(L.X.bytes(na, s));
   T *X = L.X.buf.template as<T>();
   if (!L.equiv) {
     ScatterArgs<T> sa{};
-    sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = L.R.template as<T>(); sa.A = X;
-    sa.a0 = 0; sa.C = L.CP; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = L.rad.noutp; sa.sh = sh_;
+    sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rl; sa.A = X;
+    sa.a0 = a0_; sa.C = L.CP; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = L.rad.noutp; sa.sh = sh_;
     stage(tg(k, "scatter_A").c_str(), [&] { launch_scatter<T>(sa, n, lmax_); });
   } else {
-    const Layer3<T> &Lm = L_[k - 1];
     const int npf = L.nlmi * nlm_;
-    M_.ensure((size_t) n_nodes_ * L.nlmi * L.CP * s);
     pairP_.ensure(na * npf * L.CP * s);
     A_.ensure(na * L.nfA * L.CP * s);
-    exchange_forward(k);    // the message of layer k (counted from 1) reaches the ghost atoms
-    stage(tg(k, "message").c_str(), [&] {
-      const long long tot = (long long) n_nodes_ * L.nlmi * L.CP;
-      hipLaunchKernelGGL(k_message<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, Lm.I.buf.template as<T>(), mu_.as<int>(),
-                         L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n_nodes_, L.nlmi, L.CP);
-    });
     const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb;
     stage(tg(k, "pair_fwd").c_str(), [&] {
       const size_t lds = (size_t) kPairChunk * (spb * L.CP + L.rad.noutp) * s;
-      GR_PAIR(k_pair_fwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(spb * L.CP), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), L.R.template as<T>(),
+      GR_PAIR(k_pair_fwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(spb * L.CP), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl,
               (const T *) M_.as<T>(), pairP_.as<T>(), L.nlmi, L.CP, nl_, L.rad.noutp, yw, sink_.as<T>(), ngrp, n);
     });
     stage(tg(k, "couple_YI").c_str(), [&] {
@@ -724,21 +747,23 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
     L.EQ.buf.ensure(L.EQ.bytes(na, s));
     L.I.buf.ensure(L.I.bytes((size_t) n_nodes_, s));    // rows of the ghost atoms too: the exchange fills them
     stage(tg(k, "reduce_eq").c_str(), [&] {
-      zero(L.EQ.buf.p, L.EQ.bytes(na, s));
+      zero(L.EQ.buf.p, L.EQ.bytes((size_t) n, s));
       for (int q = 0; q < 4; q++) cfwd(*L.eq[q], srcs[q], L.EQ.buf.template as<T>(), 1);
     });
-    stage(tg(k, "eqnorm").c_str(), [&] {
-      hipLaunchKernelGGL(k_eqnorm<T>, dim3(n), dim3(256), (size_t) L.eqn.M * sizeof(double), stream_, L.eqn, (const T *) L.EQ.buf.template as<T>(),
-                         L.I.buf.template as<T>(), (const T *) nullptr, (T *) nullptr, 0);
-    });
+    if (!again)    // the message rows exist already (and the layer above has read them)
+      stage(tg(k, "eqnorm").c_str(), [&] {
+        hipLaunchKernelGGL(k_eqnorm<T>, dim3(n), dim3(256), (size_t) L.eqn.M * sizeof(double), stream_, L.eqn, (const T *) L.EQ.buf.template as<T>(),
+                           L.I.buf.template as<T>() + (size_t) a0_ * L.eqn.M * L.eqn.C, (const T *) nullptr, (T *) nullptr, 0);
+      });
   }
-  L.rho_raw.ensure(na * nrho_ * sizeof(double));
-  L.grho.ensure(na * nrho_ * sizeof(double));
+  L.rho_raw.ensure((size_t) n_ * nrho_ * sizeof(double));
+  L.grho.ensure((size_t) n_ * nrho_ * sizeof(double));
   (void) nX;
+  if (again) return;    // the densities, the energy and the UQ rows come from the first forward pass
   stage(tg(k, "reduce_rho").c_str(), [&] {
-    const int *tiles = tiles_.as<int>();
-#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(ntiles_), dim3(256), 0, stream_, L.rho.d, mu_.as<int>(), tiles, srcs[0], srcs[1], \
-                                          srcs[2], srcs[3], L.rho_raw.template as<double>())
+    const int *tiles = cur_tiles_;
+#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(cur_ntiles_), dim3(256), 0, stream_, L.rho.d, mu, tiles, srcs[0], srcs[1], \
+                                          srcs[2], srcs[3], L.rho_raw.template as<double>() + (size_t) a0_ * nrho_)
     switch ((wX / 16) * 10 + wR / 16) {
       case 11: GR_RED(1, 1); break;
       case 12: GR_RED(1, 2); break;
@@ -757,27 +782,31 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw)
     stage(tg(k, "uq").c_str(), [&] {
       UqDev<T> u = L.uq;
       for (int q = 0; q < u.nsrc; q++) u.X[q] = srcs[L.uqSlot[q]];
-      u.zacc = uqZ_.as<double>();
-      u.n2acc = uqN2_.as<double>();
+      u.zacc = uqZ_.as<double>() + (size_t) a0_ * u.rp;
+      u.n2acc = uqN2_.as<double>() + (size_t) a0_ * kUqMaxBlk;
       const size_t lds = (size_t) (u.d_basis + 4 * u.rp + 2 * u.D) * sizeof(double);
       auto kern = k_uq<T>;
       if (lds > 48 * 1024)
         HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-      hipLaunchKernelGGL(kern, dim3(n), dim3(256), lds, stream_, u, mu_.as<int>(), n, uq_gamma_.as<double>(), uq_sigma_.as<double>(),
-                         uq_cluster_.as<double>());
+      hipLaunchKernelGGL(kern, dim3(n), dim3(256), lds, stream_, u, mu, n, uq_gamma_.as<double>() + a0_, uq_sigma_.as<double>() + a0_,
+                         uq_cluster_.as<double>() + a0_);
     });
   }
   (void) forces;
 }
 
-// Reverse of layer k.  In: L.grho (adjoint of the raw density) and, for layers 1-2, gM_ (adjoint of the message this
-// layer sent: dE/dI, accumulated by the pair kernel of the layer above).  Out: forces of the layer's bonds and, for
-// layers 2-3, gM_ overwritten with the adjoint of the message of the layer below.
+// Reverse of layer k over the atoms of the current chunk.  In: L.grho (adjoint of the raw density) and, for layers 1-2,
+// gMin_ (adjoint of the message this layer sent: dE/dI, accumulated by the pair kernel of the layer above).  Out: forces of
+// the layer's bonds and, for layers 2-3, the adjoint of the message of the layer below added to gM_ (cleared by the caller
+// before the first chunk).
 template<class T> void Engine3L<T>::layer_backward(int k, int yw)
 {
   Layer3<T> &L = L_[k];
-  const int n = n_;
-  const size_t na = (size_t) n, s = sizeof(T);
+  const int n = cn_;
+  const size_t na = cap_, s = sizeof(T);
+  const long long *eoff = eoff_.as<long long>() + a0_;
+  const int *mu = mu_.as<int>() + a0_;
+  T *Rl = moved_back(L.R.template as<T>(), eb_ * L.rad.noutp), *dRl = moved_back(L.dR.template as<T>(), eb_ * L.rad.noutp);
   const int nX = L.X.nf, wX = L.X.w, wR = L.wR;
 
   size_t maxP = 0, maxLp = 0;
@@ -795,19 +824,20 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   T *gP = gP_.as<T>(), *gLp = gLp_.as<T>(), *gRp = gRp_.as<T>(), *gX = gX_.as<T>(), *gR2 = gR2_.as<T>(), *gR3 = gR3_.as<T>(), *gR4 = gR4_.as<T>(),
     *gFA = gFA_.as<T>(), *gFB = gFB_.as<T>();
   T *gsrc[4] = {gX, gR2, gR3, gR4};
+  const size_t nn = (size_t) n;
   stage(tg(k, "zero_grads").c_str(), [&] {
-    zero(gX, na * nX * wX * s);
-    zero(gR2, na * L.nR2 * wR * s);
-    zero(gR3, na * L.nR3 * wR * s);
-    zero(gR4, na * L.nR4 * wR * s);
-    zero(gFA, na * L.nR2 * wR * s);
-    zero(gFB, na * L.nR2 * wR * s);
+    zero(gX, nn * nX * wX * s);
+    zero(gR2, nn * L.nR2 * wR * s);
+    zero(gR3, nn * L.nR3 * wR * s);
+    zero(gR4, nn * L.nR4 * wR * s);
+    zero(gFA, nn * L.nR2 * wR * s);
+    zero(gFB, nn * L.nR2 * wR * s);
   });
   if (L.has_eq) {
     gEQ_.ensure(L.EQ.bytes(na, s));
     stage(tg(k, "eqnorm_bwd").c_str(), [&] {
       hipLaunchKernelGGL(k_eqnorm<T>, dim3(n), dim3(256), (size_t) L.eqn.M * sizeof(double), stream_, L.eqn, (const T *) L.EQ.buf.template as<T>(), (T *) nullptr,
-                         (const T *) gM_.as<T>(), gEQ_.as<T>(), 0);
+                         (const T *) gMin_.as<T>() + (size_t) a0_ * L.eqn.M * L.eqn.C, gEQ_.as<T>(), 0);
     });
     stage(tg(k, "reduce_eq_bwd").c_str(), [&] {
       for (int q = 0; q < 4; q++) cbwd(*L.eq[q], gEQ_.as<T>(), gsrc[q], 1);
@@ -815,16 +845,16 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   }
   stage(tg(k, "reduce_rho_bwd").c_str(), [&] {
     if (L.rho.njobs)
-      hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, L.rho.njobs), dim3(64), 0, stream_, L.rho.d, mu_.as<int>(), tiles_.as<int>(),
-                         (const double *) L.grho.template as<double>(), gX, gR2, gR3, gR4);
+      hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(cur_ntiles_, L.rho.njobs), dim3(64), 0, stream_, L.rho.d, mu, cur_tiles_,
+                         (const double *) L.grho.template as<double>() + (size_t) a0_ * nrho_, gX, gR2, gR3, gR4);
   });
   // gXL / gXR: where the adjoints of the product's inputs are added
   auto prod_bwd = [&](const char *name, ProdStage<T> &p, Ten &Lp, Ten &Rp, const T *gR, T *gXL, T *gXR) {
     const T *lp = Lp.buf.template as<T>(), *rp = Rp.buf.template as<T>();
     stage(tg(k, (std::string("reduce_") + name + "_bwd").c_str()).c_str(), [&] { cbwd_set(p.red, gR, gP); });
     stage(tg(k, (std::string("couple_") + name + "_bwd").c_str()).c_str(), [&] {
-      zero(gLp, Lp.bytes(na, s));
-      zero(gRp, Rp.bytes(na, s));
+      zero(gLp, Lp.bytes(nn, s));
+      zero(gRp, Rp.bytes(nn, s));
       couple_bwd(p, lp, Lp.nf, rp, Rp.nf, gP, gLp, gRp);
     });
     stage(tg(k, (std::string("proj_") + name + "_bwd").c_str()).c_str(), [&] {
@@ -846,18 +876,15 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   if (!L.equiv) {
     BondBwdArgs<T> ba{};
     ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
-    ba.Rz = L.R.template as<T>(); ba.dRz = L.dR.template as<T>(); ba.gA = gX;
+    ba.Rz = Rl; ba.dRz = dRl; ba.gA = gX;
     ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
-    ba.a0 = 0; ba.C = L.CP; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = L.rad.noutp; ba.sh = sh_;
+    ba.a0 = a0_; ba.C = L.CP; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = L.rad.noutp; ba.sh = sh_;
     stage(tg(k, "bond_bwd").c_str(), [&] { launch_bond_bwd<T>(ba, n); });
     return;
   }
-  const Layer3<T> &Lm = L_[k - 1];
   const int npf = L.nlmi * nlm_;
   gA_.ensure(na * L.nfA * L.CP * s);
   gpairP_.ensure(na * npf * L.CP * s);
-  M_.ensure((size_t) n_nodes_ * L.nlmi * L.CP * s);
-  gM_.ensure((size_t) n_nodes_ * L.nlmi * L.CP * s);
   stage(tg(k, "reduce_A_bwd").c_str(), [&] { cbwd_set(L.redA, gX, gA_.as<T>()); });
   stage(tg(k, "couple_YI_bwd").c_str(), [&] {
     const int AT = 64 / L.CP;
@@ -865,23 +892,37 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
                        L.cgt.off.template as<int>(), L.cgt.idx.template as<int>(), L.cgt.rowof.template as<int>(), L.cgt.val.template as<double>(),
                        (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP, n);
   });
-  stage(tg(k, "message_bwd").c_str(), [&] {
-    const long long tot = (long long) n_nodes_ * L.nlmi * L.CP;
-    hipLaunchKernelGGL(k_message<T>, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, Lm.I.buf.template as<T>(), mu_.as<int>(),
-                       L.zproj.template as<T>(), L.mask.template as<T>(), M_.as<T>(), n_nodes_, L.nlmi, L.CP);
-    zero(gM_.p, (size_t) n_nodes_ * L.nlmi * L.CP * s);
-  });
   const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
   stage(tg(k, "pair_bwd").c_str(), [&] {
     const size_t lds = (size_t) kPairChunk * (pthreads + 2 * L.rad.noutp) * s;
-    GR_PAIR(k_pair_bwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), L.R.template as<T>(),
-            L.dR.template as<T>(), (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(),
-            f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n);
+    GR_PAIR(k_pair_bwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl,
+            (const T *) dRl, (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(),
+            f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_);
   });
-  comm_reverse_layer_ = k;
-  exchange_reverse(k);    // the ghosts' adjoint rows of the message of layer k go to their owners
-  comm_reverse_layer_ = 0;
   (void) yw;
+}
+
+// bytes of chunk-sized work buffers per atom of a chunk (per-atom tensors of the forward and the reverse pass and, per bond
+// of an atom, the radial rows of the three layers), largest layer
+template<class T> double Engine3L<T>::chunk_bytes_per_atom() const
+{
+  const double bonds = (double) std::max<int64_t>(nb_, 1) / std::max(n_, 1);
+  double shared = 0.0, kept = 0.0;
+  for (int k = 0; k < 3; k++) {
+    const Layer3<T> &L = L_[k];
+    double maxP = 0, maxLp = 0, proj = 0;
+    for (const ProdStage<T> *p : {&L.p2, &L.p3, &L.p4}) maxP = std::max(maxP, (double) p->nfunc * p->rankP);
+    for (const Ten *t : {&L.L2, &L.R2p, &L.L3, &L.R3p, &L.L4, &L.R4p}) {
+      maxLp = std::max(maxLp, (double) t->nf * t->w);
+      proj += (double) t->nf * t->w;
+    }
+    const double X = (double) L.X.nf * L.X.w, R = (double) (L.nR2 + L.nR3 + L.nR4) * L.wR, F = 2.0 * L.nR2 * L.wR;
+    const double spbf = L.equiv ? 2.0 * ((double) L.nlmi * nlm_ + L.nfA) * L.CP : 0.0;    // pair tensor and coupled functions, with adjoints
+    const double eq = L.has_eq ? 2.0 * L.EQ.nf * L.EQ.w : 0.0;
+    shared = std::max(shared, spbf + 2.0 * maxP + 2.0 * maxLp + X + 2.0 * R + 2.0 * F + (L.has_eq ? (double) L.EQ.nf * L.EQ.w : 0.0));
+    kept += X + proj + eq / 2.0 + 2.0 * bonds * L.rad.noutp;    // every layer keeps its own inputs of the reverse
+  }
+  return (shared + kept) * sizeof(T);
 }
 
 template<class T> void Engine3L<T>::run(const RunFlags &fl)
@@ -909,7 +950,53 @@ template<class T> void Engine3L<T>::run(const RunFlags &fl)
     uqZ_.ensure(na * L_[0].uq.rp * sizeof(double));
     uqN2_.ensure(na * kUqMaxBlk * sizeof(double));
   }
-  for (int k = 0; k < 3; k++) layer_forward(k, forces, yw);
+
+  // ---- chunks of atoms.  A layer needs the messages of ALL atoms of the layer below, so the forward pass goes layer by
+  // layer over the chunks, and so does the reverse from the top.  What is kept for the whole structure: the harmonics and
+  // the compact bonds, per layer the message, the raw density and its adjoint, and two arrays of message adjoints.  Every
+  // other tensor (the radial rows of a layer included) exists for one chunk: with more than one chunk the reverse of a
+  // layer repeats that layer's forward pass for the chunk first (the reference's store_l1 = false, libgrace/include/grace/
+  // system.h:79-80, extended to every layer).
+  const double bonds_per_atom = (double) ecap / n;
+  double kept = bonds_per_atom * (60.0 + yw * sizeof(T)) + 64.0;
+  for (int k = 0; k < 3; k++) kept += 3.0 * (double) L_[k].I.nf * L_[k].I.w * sizeof(T) + 16.0 * nrho_;
+  const int cs = plan_chunk(n, chunk_bytes_per_atom(), kept);
+  const int nchunks = (n + cs - 1) / cs;
+  chunk_used_ = nchunks > 1 ? cs : 0;
+  std::vector<long long> ebound;
+  cap_ = (size_t) cs;
+  ecap_ = ecap;
+  if (nchunks > 1) {
+    layout_chunks(cs);
+    ebound = chunk_edge_bounds(cs);
+    ecap_ = 1;
+    for (int q = 0; q < nchunks; q++) ecap_ = std::max(ecap_, (size_t) (ebound[(size_t) q + 1] - ebound[(size_t) q]));
+  }
+  auto set_chunk = [&](int q) {
+    if (nchunks == 1) {
+      a0_ = 0; cn_ = n; eb_ = 0; ecnt_ = -1;
+      cur_tiles_ = tiles_.as<int>(); cur_ntiles_ = ntiles_; cur_tile_el_ = tile_el_.data();
+      return;
+    }
+    a0_ = q * cs;
+    cn_ = std::min(n, a0_ + cs) - a0_;
+    eb_ = ebound[(size_t) q];
+    ecnt_ = ebound[(size_t) q + 1] - eb_;
+    cur_tiles_ = chunk_tiles_.as<int>() + (size_t) 16 * chunk_tile_off_[(size_t) q];
+    cur_ntiles_ = chunk_tile_off_[(size_t) q + 1] - chunk_tile_off_[(size_t) q];
+    cur_tile_el_ = chunk_tile_el_[(size_t) q].data();
+  };
+  for (int k = 0; k < 3; k++) {
+    if (L_[k].equiv) {
+      exchange_forward(k);    // the message of layer k (counted from 1) reaches the ghost atoms
+      layer_messages(k);
+    }
+    for (int q = 0; q < nchunks; q++) {
+      set_chunk(q);
+      layer_forward(k, forces, yw, false);
+    }
+  }
+  set_chunk(0);
   if (fl.uq) ran_uq_ = true;
   stage("energy_mlp", [&] {
     hipLaunchKernelGGL(k_energy_3l, dim3(n), dim3(64), (size_t) (nrho_ + 2 * en_.nh) * sizeof(double), stream_, en_, mu_.as<int>(),
@@ -918,7 +1005,27 @@ template<class T> void Engine3L<T>::run(const RunFlags &fl)
                        L_[2].grho.template as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0, sid_ptr());
   });
   if (!forces) return;
-  for (int k = 2; k >= 0; k--) layer_backward(k, yw);
+  for (int k = 2; k >= 0; k--) {
+    Layer3<T> &L = L_[k];
+    if (L.equiv) {
+      layer_messages(k);    // M_ holds the message of the layer that ran last
+      gM_.ensure((size_t) n_nodes_ * L.nlmi * L.CP * sizeof(T));
+      stage(tg(k, "message_bwd").c_str(), [&] { zero(gM_.p, (size_t) n_nodes_ * L.nlmi * L.CP * sizeof(T)); });
+    }
+    for (int q = 0; q < nchunks; q++) {
+      set_chunk(q);
+      if (nchunks > 1) layer_forward(k, forces, yw, true);
+      layer_backward(k, yw);
+    }
+    if (L.equiv) {
+      comm_reverse_layer_ = k;
+      exchange_reverse(k);    // the ghosts' adjoint rows of the message of layer k go to their owners
+      comm_reverse_layer_ = 0;
+      std::swap(gM_.p, gMin_.p);    // what this layer gathered is what the layer below sent
+      std::swap(gM_.bytes, gMin_.bytes);
+    }
+  }
+  set_chunk(0);
 }
 
 #undef GR_PAIR

@@ -1231,12 +1231,14 @@ class EngineBase : public Engine, protected BufRegistry {
     const int n = n_, nch = (n + cs - 1) / cs;
     std::vector<int> all, el;
     chunk_tile_off_.assign(1, 0);
+    chunk_tile_el_.clear();
     for (int k = 0; k < nch; k++) {
       const int a0 = k * cs, a1 = std::min(n, a0 + cs);
       const std::vector<int> sub(mu_host_.begin() + a0, mu_host_.begin() + a1);
       const std::vector<int> t = element_tiles(sub, nelem_, el);
       all.insert(all.end(), t.begin(), t.end());
       chunk_tile_off_.push_back((int) all.size() / 16);
+      chunk_tile_el_.push_back(el);    // tiles of element e within the chunk: [el[e], el[e + 1])
     }
     upload_vec(chunk_tiles_, all);
     chunk_laid_out_ = cs;
@@ -1259,6 +1261,7 @@ class EngineBase : public Engine, protected BufRegistry {
   bool chunks_ = false;          // the engine can evaluate a structure in chunks of atoms
   int chunk_request_ = -1, chunk_used_ = 0, chunk_laid_out_ = 0;
   std::vector<int> mu_host_, chunk_tile_off_;
+  std::vector<std::vector<int>> chunk_tile_el_;
   DevBuf chunk_tiles_;
 
   int device_, ncu_ = 256;

@@ -193,6 +193,8 @@ __device__ inline double wave_sum4(double v0, double v1, double v2, double v3, i
 
 // grid: (atoms, slot groups); block: spb * C threads rounded up to a wave, spb slots per block (a kernel argument);
 // dynamic LDS: kPairChunk * (NT + 2 nl C) values.  Every block adds the force of its slots to the bond's two atoms.
+// The atoms are a chunk of the structure: eoff, gP start at the chunk's first atom a0; ej, M, gM, f, sid, the harmonics
+// and the radial rows are indexed by the atom's or the bond's number in the structure.
 // gP: adjoint of P of the atom.
 //   S_l = sum_m Y_lm gP[lm],  T_l,k = sum_m D_k,lm gP[lm], k = 1, 2 (tangential gradients)   (per thread: slot, n)
 //   dE/dI_j[slot][n] += sum_l R1_l S_l                                        (slots < nI)
@@ -204,7 +206,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
                            const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
                            const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
                            T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
-                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms)
+                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms, int a0)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   __shared__ double bsum[kPairChunk][4];
@@ -283,8 +285,8 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
     for (int k = 0; k < 9; k++)
       for (int o = 32; o > 0; o >>= 1) vsum[k] += __shfl_xor(vsum[k], o, 64);
     if (lane == 0 && e1 > e0) {
-      for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) i + k], vsum[k]);
-      for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[i] : 0) + k], vsum[3 + k]);
+      for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) (a0 + i) + k], vsum[k]);
+      for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[a0 + i] : 0) + k], vsum[3 + k]);
     }
   }
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive

@@ -22,7 +22,8 @@ def _same(a, b, n, tol=1e-10):
 
 
 @pytest.mark.parametrize("precision", [64, 32])
-@pytest.mark.parametrize("model,struct,species", [("mix2", "alloy54", ["Mo", "W"]), ("cut2", "slab", ["Al", "Ni"]), ("config1", "config1", ["W"])])
+@pytest.mark.parametrize("model,struct,species", [("mix2", "alloy54", ["Mo", "W"]), ("cut2", "slab", ["Al", "Ni"]), ("config1", "config1", ["W"]),
+                                                  ("l3mix", "alloy54", ["Mo", "W"]), ("l3wide", "fcc108", ["Al", "Ni"]), ("l3el", "alloy54", ["Mo", "W"])])
 def test_chunked_pass_equals_one_pass(model_dir, model, struct, species, precision):
     """chunk sizes that split the tiles of 16 atoms of one element, a chunk of one atom, a chunk larger than the structure"""
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
@@ -43,9 +44,10 @@ def test_chunked_pass_equals_one_pass(model_dir, model, struct, species, precisi
         del s
 
 
-def test_chunked_uq_and_energy_only(model_dir):
+@pytest.mark.parametrize("model", ["uq2", "uq3l"])
+def test_chunked_uq_and_energy_only(model_dir, model):
     pos, cell, pbc, types = cases.structure_alloy54()
-    m = kk.Model(cases.model_file(model_dir, "uq2"))
+    m = kk.Model(cases.model_file(model_dir, model))
     ref = kk.System(m, ["Mo", "W"], skin=0.0, chunksize=0).compute(types, pos, cell, pbc, uq=True, energies=True)
     s = kk.System(m, ["Mo", "W"], skin=0.0, chunksize=13)
     out = s.compute(types, pos, cell, pbc, uq=True, energies=True)
@@ -57,12 +59,13 @@ def test_chunked_uq_and_energy_only(model_dir):
     assert abs(eo["energy"] - ref["energy"]) < 1e-9
 
 
-def test_chunked_batch_equals_one_pass(model_dir):
+@pytest.mark.parametrize("model", ["mix2", "l3mix"])
+def test_chunked_batch_equals_one_pass(model_dir, model):
     """several structures in one list, chunks that cut through structures"""
     structs = workloads.structures_config5(6)
     natoms, types, pos, cells, pbc = workloads.batch_arrays(structs)
     types = np.minimum(types, 2).astype(np.int32)
-    m = kk.Model(cases.model_file(model_dir, "mix2"))
+    m = kk.Model(cases.model_file(model_dir, model))
     ref = kk.Batch(m, ["Mo", "W"], chunksize=0).compute(natoms, types, pos, cells, pbc, energies=True)
     b = kk.Batch(m, ["Mo", "W"], chunksize=50)
     out = b.compute(natoms, types, pos, cells, pbc, energies=True)
@@ -112,7 +115,7 @@ def test_automatic_chunk_follows_the_memory_the_library_may_use(tmp_path):
     _same(out, ref, len(pos))
 
 
-@pytest.mark.parametrize("model", ["l2mix", "l3mix"])
+@pytest.mark.parametrize("model", ["l2mix"])
 def test_model_kinds_that_run_in_one_pass_refuse_a_chunk_size(model_dir, model):
     m = kk.Model(cases.model_file(model_dir, model))
     with pytest.raises(ValueError, match="one pass"):

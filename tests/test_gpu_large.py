@@ -72,6 +72,40 @@ def test_full_size_configuration_equals_the_compiled_reference(name, large, benc
     del sysm
 
 
+def test_config4_in_chunks_under_a_memory_cap_equals_the_one_pass_result(large, bench_models):
+    """the GRACE-3L benchmark structure (86 GB of work buffers in one fp64 pass) with the library's device memory capped at
+    24 GB: the automatic choice splits the atoms into chunks, every layer's forward pass is repeated before its reverse, and
+    the result is the one-pass result (and the compiled reference's at its gate)"""
+    from grace_runtime_amd import _lib
+    path, species, pos, cell, pbc, types = large_case("config4", bench_models)
+    n = len(pos)
+    L = _lib.lib()
+    m = kk.Model(path)
+    one = kk.System(m, species, skin=0.0, precision=64, chunksize=0)
+    ref = one.compute(types, pos, cell, pbc, energies=True)
+    one.release_buffers()
+    del one
+    said = []
+    kk.set_logger(lambda level, msg: said.append(msg))
+    try:
+        s = kk.System(m, species, skin=0.0, precision=64)          # chunksize -1: automatic
+        L.gr_set_memory_limit(L.gr_memory_in_use() + 24 * 1024 ** 3)
+        out = s.compute(types, pos, cell, pbc, energies=True)
+        assert 512 <= s.chunksize < n and any("chunksize auto" in msg for msg in said)
+        assert L.gr_memory_in_use() < 25 * 1024 ** 3
+    finally:
+        L.gr_set_memory_limit(0)
+        kk.set_logger(None)
+    fs = max(1.0, np.abs(ref["forces"]).max())
+    assert abs(out["energy"] - ref["energy"]) / n < 1e-10 * fs
+    assert np.abs(out["forces"] - ref["forces"]).max() < 1e-9 * fs
+    assert np.abs(out["energies"] - ref["energies"]).max() < 1e-10 * fs
+    assert np.abs(out["virial"] - ref["virial"]).max() < 1e-7 * fs
+    idx = large["config4/atoms"]
+    assert np.abs(out["forces"][idx] - large["config4/forces"]).max() < 2e-5 * max(1.0, float(large["config4/max_abs_force"]))
+    del s
+
+
 def config5_batch():
     structs = workloads.structures_config5()
     return structs, workloads.batch_arrays(structs)
