@@ -36,6 +36,7 @@ struct gr_engine {
   int64_t nall_cap = INT64_MAX;                        // atoms per batch pass after an allocation failure (kept for later calls)
   bool has_exchange = false;                           // an exchange is installed: ghosts of the LAMMPS call stay atoms of their own
   grhip::ExchangeCallbacks exchange;                   // kept for the engine a reset makes
+  int chunk_request = -1;                              // the caller's chunk size, kept for the engine a reset makes
   void make()
   {
     if (m1) eng = grhip::make_engine_1l(m1, ntypes, type2mu, precision, device);
@@ -50,6 +51,7 @@ struct gr_engine {
     generation++;
     make();
     if (has_exchange) eng->set_exchange(exchange);
+    eng->set_chunksize(chunk_request);
   }
   std::vector<grhip::StageTime> times;
   std::unique_ptr<grhip::BatchDeviceNeighbors> bnl;    // lists of gr_compute_batch_device (buffers kept between calls)
@@ -963,6 +965,7 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
         grhip::log_message(1, "device allocation failed with " + std::to_string(used) + " atoms per pass; trying again with " + std::to_string(next));
         try {
           eng.set_chunksize(next);
+          s->eng->chunk_request = next;
         } catch (const grhip::InvalidArgument &) {    // an engine that evaluates structures in one pass only
           throw grhip::Error("the structure (" + std::to_string(n) + " atoms) does not fit the GPU memory in one pass, and this model kind is "
                              "not evaluated in chunks");
@@ -977,6 +980,7 @@ int gr_system_set_chunksize(gr_system *s, int atoms)
   return guarded([&] {
     if (!s) throw grhip::InvalidArgument("null system");
     live(s->eng).set_chunksize(atoms);
+    s->eng->chunk_request = atoms;
     s->auto_chunk = atoms < 0;
   });
 }
@@ -992,7 +996,10 @@ int64_t gr_engine_atoms_that_fit(gr_engine *e)
 
 int gr_engine_set_chunksize(gr_engine *e, int atoms)
 {
-  return guarded([&] { live(e).set_chunksize(atoms); });
+  return guarded([&] {
+    live(e).set_chunksize(atoms);
+    e->chunk_request = atoms;
+  });
 }
 
 int gr_engine_chunksize(const gr_engine *e) { return e && e->eng ? e->eng->chunksize_used() : 0; }

@@ -36,6 +36,7 @@ template<class T> class Engine2L final : public EngineBase {
     this->template probe_mfma<T>();
     build();
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
+    chunks_ = true;
   }
   int layers() const override { return 2; }
   void run(const RunFlags &fl) override;
@@ -70,13 +71,19 @@ template<class T> class Engine2L final : public EngineBase {
   Energy2Dev en_{};
   // pass buffers
   DevBuf sink_, Rz_, dRz_, R1_, dR1_, YG_, A_, rho_, grho_, I1_, gI1_, I1t_, gI1t_, M_, gM_, P_, gP_, B_, I2_, gI2_;
+  // the chunk of atoms the chain and reduce functions act on: cn_ atoms from a0_, the chunk's element tiles (atoms counted
+  // from a0_), the capacity the chunk buffers are sized for
+  int cn_ = 0, a0_ = 0;
+  size_t cap_ = 0;
+  const int *cur_tiles_ = nullptr;
+  int cur_ntiles_ = 0;
 
   void build();
   void build_chain(Chain<T> &c, const char *tag, int nf, int KP, const FCWeights *fc[3], const CGProduct *pr[3],
                    const std::vector<const ReduceEq *> reds[4]);
   void gemm(DevJobs<T> &J, int kb0, int nb, const T *X0, int nf0, T *out, int nfo, int accumulate)
   {
-    EngineBase::launch_gemm<T>(J, kb0, kb0, nb, X0, nf0, X0, nf0, out, nfo, accumulate, tiles_.as<int>(), ntiles_);
+    EngineBase::launch_gemm<T>(J, kb0, kb0, nb, X0, nf0, X0, nf0, out, nfo, accumulate, cur_tiles_, cur_ntiles_);
   }
   void chain_forward(Chain<T> &c, const char *tag, const T *X);
   void chain_zero(Chain<T> &c, const char *tag);
@@ -361,8 +368,8 @@ template<class T> void Engine2L<T>::build()
 
 template<class T> void Engine2L<T>::chain_forward(Chain<T> &c, const char *tag, const T *X)
 {
-  const int n = n_, KP = c.kb * 16;
-  const size_t na = (size_t) n;
+  const int n = cn_, KP = c.kb * 16;
+  const size_t na = cap_;
   c.X1.ensure(na * c.nf * KP * sizeof(T));
   c.XX.ensure(na * c.nXX * KP * sizeof(T));
   c.XX1.ensure(na * c.nXX * KP * sizeof(T));
@@ -388,28 +395,29 @@ template<class T> void Engine2L<T>::chain_forward(Chain<T> &c, const char *tag, 
   };
   T *X1 = c.X1.template as<T>(), *XX = c.XX.template as<T>(), *XX1 = c.XX1.template as<T>(), *XXX = c.XXX.template as<T>(),
     *XX2 = c.XX2.template as<T>(), *XXXX = c.XXXX.template as<T>();
-  stage(tagged(tag, "fc_1").c_str(), [&] { launch_gemm<T>(c.fc1.fwd, c.kb, c.kb, c.kb, X, c.nf, X, c.nf, X1, c.nf, 0, tiles_.as<int>(), ntiles_); });
+  stage(tagged(tag, "fc_1").c_str(), [&] { launch_gemm<T>(c.fc1.fwd, c.kb, c.kb, c.kb, X, c.nf, X, c.nf, X1, c.nf, 0, cur_tiles_, cur_ntiles_); });
   prod(tagged(tag, "prod_2"), c.p2, X1, X1, XX, c.nf, c.nf);
-  stage(tagged(tag, "fc_2").c_str(), [&] { launch_gemm<T>(c.fc2.fwd, c.kb, c.kb, c.kb, XX, c.nXX, X, c.nf, XX1, c.nXX, 0, tiles_.as<int>(), ntiles_); });
+  stage(tagged(tag, "fc_2").c_str(), [&] { launch_gemm<T>(c.fc2.fwd, c.kb, c.kb, c.kb, XX, c.nXX, X, c.nf, XX1, c.nXX, 0, cur_tiles_, cur_ntiles_); });
   prod(tagged(tag, "prod_3"), c.p3, XX1, X, XXX, c.nXX, c.nf);
   if (c.order4) {
-    stage(tagged(tag, "fc_3").c_str(), [&] { launch_gemm<T>(c.fc3.fwd, c.kb, c.kb, c.kb, XX, c.nXX, X, c.nf, XX2, c.nXX, 0, tiles_.as<int>(), ntiles_); });
+    stage(tagged(tag, "fc_3").c_str(), [&] { launch_gemm<T>(c.fc3.fwd, c.kb, c.kb, c.kb, XX, c.nXX, X, c.nf, XX2, c.nXX, 0, cur_tiles_, cur_ntiles_); });
     prod(tagged(tag, "prod_4"), c.p4, XX2, XX2, XXXX, c.nXX, c.nXX);
   }
 }
 
 template<class T> void Engine2L<T>::chain_zero(Chain<T> &c, const char *tag)
 {
-  const size_t na = (size_t) n_, KP = c.kb * 16;
-  c.gX.ensure(na * c.nf * KP * sizeof(T));
-  c.gX1.ensure(na * c.nf * KP * sizeof(T));
-  c.gXX.ensure(na * c.nXX * KP * sizeof(T));
-  c.gXX1.ensure(na * c.nXX * KP * sizeof(T));
-  c.gXXX.ensure(na * c.nXXX * KP * sizeof(T));
+  const size_t nc = cap_, KP = c.kb * 16;
+  c.gX.ensure(nc * c.nf * KP * sizeof(T));
+  c.gX1.ensure(nc * c.nf * KP * sizeof(T));
+  c.gXX.ensure(nc * c.nXX * KP * sizeof(T));
+  c.gXX1.ensure(nc * c.nXX * KP * sizeof(T));
+  c.gXXX.ensure(nc * c.nXXX * KP * sizeof(T));
   if (c.order4) {
-    c.gXX2.ensure(na * c.nXX * KP * sizeof(T));
-    c.gXXXX.ensure(na * std::max(c.nXXXX, 1) * KP * sizeof(T));
+    c.gXX2.ensure(nc * c.nXX * KP * sizeof(T));
+    c.gXXXX.ensure(nc * std::max(c.nXXXX, 1) * KP * sizeof(T));
   }
+  const size_t na = (size_t) cn_;
   stage(tagged(tag, "zero_grads").c_str(), [&] {
     HIP_CHECK(hipMemsetAsync(c.gX.p, 0, na * c.nf * KP * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(c.gX1.p, 0, na * c.nf * KP * sizeof(T), stream_));
@@ -428,7 +436,7 @@ template<class T> void Engine2L<T>::chain_zero(Chain<T> &c, const char *tag)
 // read of the largest adjoint); reduces_x_xx then adds the reduces' adjoints of X and XX.  Result in c.gX.
 template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag, const T *X, const std::function<void()> &reduces_x_xx)
 {
-  const int n = n_, KP = c.kb * 16;
+  const int n = cn_, KP = c.kb * 16;
   int one = 1, nat = n;
   auto prod_bwd = [&](const std::string &name, DevProd &P, const T *L, const T *R, const T *g, T *gL, T *gR, int sl, int sr, int accL, int accR) {
     if (P.jit.ok()) {
@@ -448,8 +456,8 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
   };
   auto fc_bwd = [&](const std::string &name, DevFc<T> &F, const T *g, T *gXl, T *gXr, int nfl, int acc_left) {
     stage(name.c_str(), [&] {
-      launch_gemm<T>(F.bwd_l, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXl, nfl, acc_left, tiles_.as<int>(), ntiles_);
-      launch_gemm<T>(F.bwd_r, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXr, c.nf, 1, tiles_.as<int>(), ntiles_);
+      launch_gemm<T>(F.bwd_l, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXl, nfl, acc_left, cur_tiles_, cur_ntiles_);
+      launch_gemm<T>(F.bwd_r, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXr, c.nf, 1, cur_tiles_, cur_ntiles_);
     });
   };
   const T *X1 = c.X1.template as<T>(), *XX1 = c.XX1.template as<T>(), *XX2 = c.XX2.template as<T>();
@@ -460,8 +468,8 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
   if (c.order4) {
     // fc2 and fc3 share their inputs: one pass over gXX and gX for both
     stage(tagged(tag, "fc_23_bwd").c_str(), [&] {
-      launch_gemm<T>(c.fc23.bwd_l, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gXX, c.nXX, 0, tiles_.as<int>(), ntiles_);
-      launch_gemm<T>(c.fc23.bwd_r, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gX, c.nf, 1, tiles_.as<int>(), ntiles_);
+      launch_gemm<T>(c.fc23.bwd_l, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gXX, c.nXX, 0, cur_tiles_, cur_ntiles_);
+      launch_gemm<T>(c.fc23.bwd_r, c.kb, c.kb, c.kb, gXX1, c.nXX, gXX2, c.nXX, gX, c.nf, 1, cur_tiles_, cur_ntiles_);
     });
   } else {
     fc_bwd(tagged(tag, "fc_2_bwd"), c.fc2, gXX1, gXX, gX, c.nXX, 0);
@@ -473,8 +481,8 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
 
 template<class T> void Engine2L<T>::reduce_fwd(DevReduce<T> &R, int kb, const Chain<T> &c, const T *X, double *out)
 {
-  const int *tiles = tiles_.as<int>();
-#define GR_RED(KA) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KA>), dim3(ntiles_), dim3(256), 0, stream_, R.d, mu_.as<int>(), tiles, \
+  const int *tiles = cur_tiles_;
+#define GR_RED(KA) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KA>), dim3(cur_ntiles_), dim3(256), 0, stream_, R.d, mu_.as<int>() + a0_, tiles, \
                                       c.src(0, X), c.src(1, X), c.src(2, X), c.src(3, X), out)
   switch (kb) {
     case 1: GR_RED(1); break;
@@ -491,7 +499,7 @@ template<class T> void Engine2L<T>::reduce_bwd(DevReduce<T> &R, const Chain<T> &
 {
   const int low = R.d.ncol[0] + R.d.ncol[1], first = high ? low : 0, count = high ? R.njobs - low : low;
   if (count <= 0) return;
-  hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles_, count), dim3(64), 0, stream_, R.d, mu_.as<int>(), tiles_.as<int>(), g, c.gsrc(0), c.gsrc(1),
+  hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(cur_ntiles_, count), dim3(64), 0, stream_, R.d, mu_.as<int>() + a0_, cur_tiles_, g, c.gsrc(0), c.gsrc(1),
                      c.gsrc(2), c.gsrc(3), first);
 }
 
@@ -499,73 +507,131 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
 {
   const int n = n_;
   if (!begin_pass(fl)) return;
-  const size_t ecap = (size_t) std::max<int64_t>(nb_, 1), na = (size_t) n;
+  const size_t ecap_all = (size_t) std::max<int64_t>(nb_, 1);
   const long long *n_edges = eoff_.as<long long>() + n;
   const bool forces = !fl.energy_only;
-
-  // ---- per-edge quantities: radial functions of both layers, spherical harmonics
-  Rz_.ensure(ecap * radR_.noutp * sizeof(T));
-  dRz_.ensure(ecap * radR_.noutp * sizeof(T));
-  R1_.ensure(ecap * radR1_.noutp * sizeof(T));
-  dR1_.ensure(ecap * radR1_.noutp * sizeof(T));
-  stage("radial_R", [&] { radR_.launch(stream_, ncu_, zA_.as<T>(), 0, -1, xr_.as<double>(), emu_.as<int>(), Rz_.as<T>(), dRz_.as<T>(), n_edges); });
-  stage("radial_R1", [&] { radR1_.launch(stream_, ncu_, ones_.as<T>(), 0, -1, xr_.as<double>(), emu_.as<int>(), R1_.as<T>(), dR1_.as<T>(), n_edges); });
   const int yw = forces ? 3 * nlm_ : nlm_;    // row of an edge: Y[nlm] and, for forces, the two tangential gradients D1[nlm], D2[nlm]
-  YG_.ensure(ecap * yw * sizeof(T));
+  YG_.ensure(ecap_all * yw * sizeof(T));
   stage("sh_edges", [&] {
     const size_t lds = (size_t) 64 * (yw + 1) * sizeof(T);
     auto kern = k_sh_edges<T>;
     if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-    hipLaunchKernelGGL(kern, dim3((unsigned) ((ecap + 63) / 64)), dim3(64), lds, stream_, sh_, rh_.as<double>(), n_edges, nlm_, forces ? 1 : 0,
+    hipLaunchKernelGGL(kern, dim3((unsigned) ((ecap_all + 63) / 64)), dim3(64), lds, stream_, sh_, rh_.as<double>(), n_edges, nlm_, forces ? 1 : 0,
                        YG_.as<T>());
   });
 
-  // ---- P1: layer 1 forward
+  // ---- chunks of atoms.  Layer 2 gathers the messages of ALL atoms, so the pass is three sweeps over the chunks: layer 1
+  // forward (the message rows of the chunk's atoms); layer 2 forward, the readout and layer 2 reverse (the message
+  // adjoints, added to the rows of the neighbours); layer 1 reverse.  Kept for the whole structure: the harmonics and the
+  // compact bonds, the message and its adjoint, rho and its adjoint.  Every other tensor, the radial rows of both layers
+  // included, exists for one chunk; with more than one chunk the third sweep repeats the chunk's layer-1 forward pass
+  // first (the reference's store_l1 = false, libgrace/include/grace/system.h:79-80).
+  const double bonds_per_atom = (double) ecap_all / n;
+  auto chain_values = [](const Chain<T> &c) {    // forward tensors and adjoints of a chain, values per atom
+    return 2.0 * c.kb * 16 * (2.0 * c.nf + (c.order4 ? 3.0 : 2.0) * c.nXX + c.nXXX + (c.order4 ? std::max(c.nXXXX, 1) : 0));
+  };
+  const int npf = nslot_ * nlm_;
+  const double per_atom = sizeof(T) * (chain_values(c1_) + chain_values(c2_) + (double) nlm_ * C1P_ + 2.0 * npf * CRP_ + (double) nB_ * C2P_ +
+                                       bonds_per_atom * 2.0 * (radR_.noutp + radR1_.noutp)) +
+                          (2.0 * nI1_ * PI1_ + 2.0 * nrho_) * sizeof(double) + 2.0 * nI1_ * PI1_ * (sizeof(T) == 4 ? 4.0 : 0.0);
+  const double kept = bonds_per_atom * (60.0 + yw * sizeof(T)) + (double) (nslot_ + nI_) * CRP_ * sizeof(T) + 32.0 * nrho_ + 64.0;
+  const int cs = plan_chunk(n, per_atom, kept);
+  const int nchunks = (n + cs - 1) / cs;
+  chunk_used_ = nchunks > 1 ? cs : 0;
+  std::vector<long long> ebound;
+  size_t ecap = ecap_all;
+  cap_ = (size_t) cs;
+  if (nchunks > 1) {
+    layout_chunks(cs);
+    ebound = chunk_edge_bounds(cs);
+    ecap = 1;
+    for (int q = 0; q < nchunks; q++) ecap = std::max(ecap, (size_t) (ebound[(size_t) q + 1] - ebound[(size_t) q]));
+  }
+  long long eb = 0, ecnt = -1;
+  auto set_chunk = [&](int q) {
+    if (nchunks == 1) {
+      a0_ = 0; cn_ = n; eb = 0; ecnt = -1;
+      cur_tiles_ = tiles_.as<int>(); cur_ntiles_ = ntiles_;
+      return;
+    }
+    a0_ = q * cs;
+    cn_ = std::min(n, a0_ + cs) - a0_;
+    eb = ebound[(size_t) q];
+    ecnt = ebound[(size_t) q + 1] - eb;
+    cur_tiles_ = chunk_tiles_.as<int>() + (size_t) 16 * chunk_tile_off_[(size_t) q];
+    cur_ntiles_ = chunk_tile_off_[(size_t) q + 1] - chunk_tile_off_[(size_t) q];
+  };
+  const size_t na = cap_, nnodes = (size_t) n_nodes_;
+
+  // buffers of the whole structure
+  rho_.ensure((size_t) n * nrho_ * sizeof(double));
+  grho_.ensure((size_t) n * nrho_ * sizeof(double));
+  M_.ensure(nnodes * nslot_ * CRP_ * sizeof(T));    // the message rows exist for the ghost atoms too: the exchange fills them
+  T *M = M_.as<T>();
+  if (fl.uq) {
+    uq_gamma_.ensure((size_t) n * sizeof(double)); uq_sigma_.ensure((size_t) n * sizeof(double)); uq_cluster_.ensure((size_t) n * sizeof(double));
+  }
+  // buffers of a chunk
+  Rz_.ensure(ecap * radR_.noutp * sizeof(T));
+  dRz_.ensure(ecap * radR_.noutp * sizeof(T));
   A_.ensure(na * nlm_ * C1P_ * sizeof(T));
   T *A = A_.as<T>();
-  {
-    ScatterArgs<T> sa{};
-    sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz_.as<T>(); sa.A = A;
-    sa.a0 = 0; sa.C = C1P_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = radR_.noutp; sa.sh = sh_;
-    stage("scatter_A", [&] { launch_scatter<T>(sa, n, lmax_); });
-  }
-  chain_forward(c1_, "_L1", A);
-  rho_.ensure(na * nrho_ * sizeof(double));
-  grho_.ensure(na * nrho_ * sizeof(double));
   if (I1_.bytes < na * nI1_ * PI1_ * sizeof(double)) {
     I1_.ensure(na * nI1_ * PI1_ * sizeof(double));
     HIP_CHECK(hipMemsetAsync(I1_.p, 0, I1_.bytes, stream_));    // the padding channels stay zero
   }
-  stage("reduce_rho", [&] { reduce_fwd(redrho_, c1_.kb, c1_, A, rho_.as<double>()); });
-  stage("reduce_I1", [&] {
-    for (auto &r : redI1_) reduce_fwd(*r, c1_.kb, c1_, A, I1_.as<double>());
-  });
-  // the message rows exist for the ghost atoms too: the exchange fills them, the gather reads them
-  const size_t nnodes = (size_t) n_nodes_;
-  M_.ensure(nnodes * nslot_ * CRP_ * sizeof(T));
-  T *M = M_.as<T>();
-  // I1 leaves the scalar reduce in fp64; the fp32 engine hands the GEMM a copy in fp32
-  const long long nI1v = (long long) na * nI1_ * PI1_;
-  const T *I1t = I1_.as<T>();
-  if constexpr (sizeof(T) == 4) {
-    I1t_.ensure(nI1v * sizeof(T));
-    I1t = I1t_.as<T>();
+  if constexpr (sizeof(T) == 4) I1t_.ensure(na * nI1_ * PI1_ * sizeof(T));
+
+  // layer 1 of the current chunk up to its chain (radial rows from row 0 of Rz_ / dRz_; kernels index bonds by their number
+  // in the structure)
+  auto layer1_chain = [&] {
+    T *Rz = moved_back(Rz_.as<T>(), eb * radR_.noutp), *dRz = moved_back(dRz_.as<T>(), eb * radR_.noutp);
+    stage("radial_R", [&] { radR_.launch(stream_, ncu_, zA_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), Rz, dRz, n_edges); });
+    ScatterArgs<T> sa{};
+    sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz; sa.A = A;
+    sa.a0 = a0_; sa.C = C1P_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = radR_.noutp; sa.sh = sh_;
+    stage("scatter_A", [&] { launch_scatter<T>(sa, cn_, lmax_); });
+    chain_forward(c1_, "_L1", A);
+  };
+
+  // ---- sweep 1: layer 1 forward
+  for (int q = 0; q < nchunks; q++) {
+    set_chunk(q);
+    layer1_chain();
+    stage("reduce_rho", [&] { reduce_fwd(redrho_, c1_.kb, c1_, A, rho_.as<double>() + (size_t) a0_ * nrho_); });
+    stage("reduce_I1", [&] {
+      for (auto &r : redI1_) reduce_fwd(*r, c1_.kb, c1_, A, I1_.as<double>());
+    });
+    // I1 leaves the scalar reduce in fp64; the fp32 engine hands the GEMM a copy in fp32
+    const long long nI1v = (long long) cn_ * nI1_ * PI1_;
+    const T *I1t = I1_.as<T>();
+    if constexpr (sizeof(T) == 4) I1t = I1t_.as<T>();
+    stage("reduce_I", [&] {
+      if constexpr (sizeof(T) == 4)
+        hipLaunchKernelGGL((k_convert<double, T>), dim3((unsigned) ((nI1v + 255) / 256)), dim3(256), 0, stream_, I1_.as<double>(), I1t_.as<T>(), nI1v);
+      gemm(jI_, PI1_ / 16, CRP_ / 16, I1t, nI1_, M + (size_t) a0_ * nslot_ * CRP_, nslot_, 0);
+    });
   }
-  stage("reduce_I", [&] {
-    if constexpr (sizeof(T) == 4)
-      hipLaunchKernelGGL((k_convert<double, T>), dim3((unsigned) ((nI1v + 255) / 256)), dim3(256), 0, stream_, I1_.as<double>(), I1t_.as<T>(), nI1v);
-    gemm(jI_, PI1_ / 16, CRP_ / 16, I1t, nI1_, M, nslot_, 0);
+  stage("fill_slot", [&] {
     hipLaunchKernelGGL(k_fill_slot<T>, dim3((unsigned) ((nnodes * CRP_ + 255) / 256)), dim3(256), 0, stream_, mu_.as<int>(), zB0_.as<T>(), M, n_nodes_,
                        nslot_, nI_, CRP_);
   });
   exchange_forward(1);
 
-  // ---- P3: layer 2 forward
-  const int npf = nslot_ * nlm_;
+  // ---- sweep 2: layer 2 forward, readout, layer 2 reverse
+  R1_.ensure(ecap * radR1_.noutp * sizeof(T));
+  dR1_.ensure(ecap * radR1_.noutp * sizeof(T));
   P_.ensure(na * npf * CRP_ * sizeof(T));
   B_.ensure(na * nB_ * C2P_ * sizeof(T));
+  I2_.ensure(na * nrho_ * sizeof(double));
+  gI2_.ensure(na * nrho_ * sizeof(double));
   T *P = P_.as<T>(), *B = B_.as<T>();
   const int pthreads = round_up(nslot_ * CRP_, 64);
+  if (forces) {
+    gP_.ensure(na * npf * CRP_ * sizeof(T));
+    gM_.ensure(nnodes * nI_ * CRP_ * sizeof(T));
+    stage("zero_gM", [&] { HIP_CHECK(hipMemsetAsync(gM_.p, 0, nnodes * nI_ * CRP_ * sizeof(T), stream_)); });
+  }
 #define GR_PAIR1(K_, N_, grid_, block_, lds_, ...)                                                                       \
   {                                                                                                                      \
     auto kern = K_<T, N_>;                                                                                               \
@@ -583,87 +649,98 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     case 6: GR_PAIR1(K_, 36, __VA_ARGS__) break;             \
     default: GR_PAIR1(K_, 49, __VA_ARGS__) break;            \
   }
-  stage("pair_fwd", [&] {
-    const size_t lds = (size_t) kPairChunk * (nslot_ * CRP_ + radR1_.noutp) * sizeof(T);
-    GR_PAIR(k_pair_fwd, dim3(n), dim3(nslot_ * CRP_), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), (const T *) M, P,
-            nslot_, CRP_, nl_, radR1_.noutp, yw, sink_.as<T>(), 0, n);
-  });
-  stage("reduce_B", [&] { gemm(jB_, CRP_ / 16, C2P_ / 16, P, npf, B, nB_, 0); });
-  chain_forward(c2_, "_L2", B);
-  I2_.ensure(na * nrho_ * sizeof(double));
-  gI2_.ensure(na * nrho_ * sizeof(double));
-  stage("reduce_I2", [&] { reduce_fwd(redI2_, c2_.kb, c2_, B, I2_.as<double>()); });
-  if (fl.uq) {
-    uq_gamma_.ensure(na * sizeof(double)); uq_sigma_.ensure(na * sizeof(double)); uq_cluster_.ensure(na * sizeof(double));
-    stage("uq", [&] {
-      UqDev<T> u = uq_;
-      for (int q = 0; q < u.nsrc; q++) u.X[q] = u.blk[q] == 0 ? c2_.src(q, B) : c1_.src(q - u.nsrc / 2, A);
-      const size_t lds = (size_t) (u.d_basis + 4 * u.rp + 2 * u.D) * sizeof(double);
-      auto kern = k_uq<T>;
-      if (lds > 48 * 1024)
-        HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
-      hipLaunchKernelGGL(kern, dim3(n), dim3(256), lds, stream_, u, mu_.as<int>(), n, uq_gamma_.as<double>(), uq_sigma_.as<double>(),
-                         uq_cluster_.as<double>());
+  for (int q = 0; q < nchunks; q++) {
+    set_chunk(q);
+    const int nc = cn_;
+    const long long *eoff = eoff_.as<long long>() + a0_;
+    const int *mu = mu_.as<int>() + a0_;
+    T *R1 = moved_back(R1_.as<T>(), eb * radR1_.noutp), *dR1 = moved_back(dR1_.as<T>(), eb * radR1_.noutp);
+    stage("radial_R1", [&] { radR1_.launch(stream_, ncu_, ones_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), R1, dR1, n_edges); });
+    stage("pair_fwd", [&] {
+      const size_t lds = (size_t) kPairChunk * (nslot_ * CRP_ + radR1_.noutp) * sizeof(T);
+      GR_PAIR(k_pair_fwd, dim3(nc), dim3(nslot_ * CRP_), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) M, P, nslot_, CRP_,
+              nl_, radR1_.noutp, yw, sink_.as<T>(), 0, nc);
     });
-    ran_uq_ = true;
+    stage("reduce_B", [&] { gemm(jB_, CRP_ / 16, C2P_ / 16, P, npf, B, nB_, 0); });
+    chain_forward(c2_, "_L2", B);
+    stage("reduce_I2", [&] { reduce_fwd(redI2_, c2_.kb, c2_, B, I2_.as<double>()); });
+    if (fl.uq) {
+      if (nchunks > 1) layer1_chain();    // the head reads layer 1's tensors of these atoms as well
+      stage("uq", [&] {
+        UqDev<T> u = uq_;
+        for (int k = 0; k < u.nsrc; k++) u.X[k] = u.blk[k] == 0 ? c2_.src(k, B) : c1_.src(k - u.nsrc / 2, A);
+        const size_t lds = (size_t) (u.d_basis + 4 * u.rp + 2 * u.D) * sizeof(double);
+        auto kern = k_uq<T>;
+        if (lds > 48 * 1024)
+          HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
+        hipLaunchKernelGGL(kern, dim3(nc), dim3(256), lds, stream_, u, mu, nc, uq_gamma_.as<double>() + a0_, uq_sigma_.as<double>() + a0_,
+                           uq_cluster_.as<double>() + a0_);
+      });
+      ran_uq_ = true;
+    }
+    stage("energy_mlp", [&] {
+      hipLaunchKernelGGL(k_energy_2l, dim3(nc), dim3(64), (size_t) (2 * en_.nlay + 4) * en_.width * sizeof(double), stream_, en_, mu, nc,
+                         (const double *) rho_.as<double>() + (size_t) a0_ * nrho_, (const double *) I2_.as<double>(),
+                         grho_.as<double>() + (size_t) a0_ * nrho_, gI2_.as<double>(), fl.eatom ? eatom_.as<double>() + a0_ : nullptr,
+                         scal_.as<double>(), forces ? 1 : 0, sid_ptr() ? sid_ptr() + a0_ : nullptr);
+    });
+    if (!forces) continue;
+    // layer 2 reverse: dE/dB -> dE/dP -> bond forces of layer 2 and dE/dI of the neighbours
+    chain_zero(c2_, "_L2");
+    stage("reduce_I2_bwd", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), true); });
+    chain_backward(c2_, "_L2", B, [&] { stage("reduce_I2_bwd_X_XX", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), false); }); });
+    stage("reduce_B_bwd", [&] { gemm(jBb_, C2P_ / 16, CRP_ / 16, c2_.gX.template as<T>(), nB_, gP_.as<T>(), npf, 0); });    // gP: every row is written
+    stage("pair_bwd", [&] {
+      const size_t lds = (size_t) kPairChunk * (pthreads + 2 * radR1_.noutp) * sizeof(T);
+      GR_PAIR(k_pair_bwd, dim3(nc), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) dR1, (const T *) M,
+              (const T *) gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(), scal_.as<double>() + 1,
+              nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_, 0, nc, a0_);
+    });
   }
-  stage("energy_mlp", [&] {
-    hipLaunchKernelGGL(k_energy_2l, dim3(n), dim3(64), (size_t) (2 * en_.nlay + 4) * en_.width * sizeof(double), stream_, en_, mu_.as<int>(), n, rho_.as<double>(), I2_.as<double>(), grho_.as<double>(),
-                       gI2_.as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0, sid_ptr());
-  });
-  if (!forces) return;
-
-  // ---- layer 2 reverse: dE/dB -> dE/dP -> bond forces of layer 2 and dE/dI of the neighbours
-  chain_zero(c2_, "_L2");
-  stage("reduce_I2_bwd", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), true); });
-  chain_backward(c2_, "_L2", B, [&] { stage("reduce_I2_bwd_X_XX", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), false); }); });
-  gP_.ensure(na * npf * CRP_ * sizeof(T));
-  gM_.ensure(nnodes * nI_ * CRP_ * sizeof(T));
-  stage("reduce_B_bwd", [&] {
-    HIP_CHECK(hipMemsetAsync(gM_.p, 0, nnodes * nI_ * CRP_ * sizeof(T), stream_));    // gP: every row is written below
-    gemm(jBb_, C2P_ / 16, CRP_ / 16, c2_.gX.template as<T>(), nB_, gP_.as<T>(), npf, 0);
-  });
-  stage("pair_bwd", [&] {
-    const size_t lds = (size_t) kPairChunk * (pthreads + 2 * radR1_.noutp) * sizeof(T);
-    GR_PAIR(k_pair_bwd, dim3(n), dim3(pthreads), lds, stream_, eoff_.as<long long>(), ej_.as<int>(), YG_.as<T>(), R1_.as<T>(), dR1_.as<T>(),
-            (const T *) M, gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),
-            scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_, 0, n, 0);
-  });
 #undef GR_PAIR
 #undef GR_PAIR1
+  if (!forces) {
+    set_chunk(0);
+    return;
+  }
   exchange_reverse(1);
 
-  // ---- P5: layer 1 reverse
+  // ---- sweep 3: layer 1 reverse
   gI1_.ensure(na * nI1_ * PI1_ * sizeof(double));
-  chain_zero(c1_, "_L1");
-  stage("reduce_I_bwd", [&] {
-    if constexpr (sizeof(T) == 4) {
-      gI1t_.ensure(nI1v * sizeof(T));
-      gemm(jIb_, CRP_ / 16, PI1_ / 16, gM_.as<T>(), nI_, gI1t_.as<T>(), nI1_, 0);
-      hipLaunchKernelGGL((k_convert<T, double>), dim3((unsigned) ((nI1v + 255) / 256)), dim3(256), 0, stream_, gI1t_.as<T>(), gI1_.as<double>(), nI1v);
-    } else {
-      gemm(jIb_, CRP_ / 16, PI1_ / 16, gM_.as<T>(), nI_, gI1_.as<T>(), nI1_, 0);
-    }
-  });
-  stage("reduce_rho_bwd", [&] { reduce_bwd(redrho_, c1_, grho_.as<double>(), true); });
-  stage("reduce_I1_bwd", [&] {
-    for (auto &r : redI1_) reduce_bwd(*r, c1_, gI1_.as<double>(), true);
-  });
-  chain_backward(c1_, "_L1", A, [&] {
-    stage("reduce_rho_bwd_X_XX", [&] { reduce_bwd(redrho_, c1_, grho_.as<double>(), false); });
-    stage("reduce_I1_bwd_X_XX", [&] {
-      for (auto &r : redI1_) reduce_bwd(*r, c1_, gI1_.as<double>(), false);
+  if constexpr (sizeof(T) == 4) gI1t_.ensure(na * nI1_ * PI1_ * sizeof(T));
+  for (int q = 0; q < nchunks; q++) {
+    set_chunk(q);
+    if (nchunks > 1) layer1_chain();
+    const long long nI1v = (long long) cn_ * nI1_ * PI1_;
+    const T *gMc = gM_.as<T>() + (size_t) a0_ * nI_ * CRP_;
+    const double *grho = grho_.as<double>() + (size_t) a0_ * nrho_;
+    chain_zero(c1_, "_L1");
+    stage("reduce_I_bwd", [&] {
+      if constexpr (sizeof(T) == 4) {
+        gemm(jIb_, CRP_ / 16, PI1_ / 16, gMc, nI_, gI1t_.as<T>(), nI1_, 0);
+        hipLaunchKernelGGL((k_convert<T, double>), dim3((unsigned) ((nI1v + 255) / 256)), dim3(256), 0, stream_, gI1t_.as<T>(), gI1_.as<double>(), nI1v);
+      } else {
+        gemm(jIb_, CRP_ / 16, PI1_ / 16, gMc, nI_, gI1_.as<T>(), nI1_, 0);
+      }
     });
-  });
-  {
+    stage("reduce_rho_bwd", [&] { reduce_bwd(redrho_, c1_, grho, true); });
+    stage("reduce_I1_bwd", [&] {
+      for (auto &r : redI1_) reduce_bwd(*r, c1_, gI1_.as<double>(), true);
+    });
+    chain_backward(c1_, "_L1", A, [&] {
+      stage("reduce_rho_bwd_X_XX", [&] { reduce_bwd(redrho_, c1_, grho, false); });
+      stage("reduce_I1_bwd_X_XX", [&] {
+        for (auto &r : redI1_) reduce_bwd(*r, c1_, gI1_.as<double>(), false);
+      });
+    });
     BondBwdArgs<T> ba{};
     ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
-    ba.Rz = Rz_.as<T>(); ba.dRz = dRz_.as<T>(); ba.gA = c1_.gX.template as<T>();
+    ba.Rz = moved_back(Rz_.as<T>(), eb * radR_.noutp); ba.dRz = moved_back(dRz_.as<T>(), eb * radR_.noutp); ba.gA = c1_.gX.template as<T>();
     ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
-    ba.a0 = 0; ba.C = C1P_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = radR_.noutp; ba.sh = sh_;
-      stage("bond_bwd", [&] { launch_bond_bwd<T>(ba, n); });
-
+    ba.a0 = a0_; ba.C = C1P_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = radR_.noutp; ba.sh = sh_;
+    stage("bond_bwd", [&] { launch_bond_bwd<T>(ba, cn_); });
   }
+  set_chunk(0);
 }
 
 }    // namespace

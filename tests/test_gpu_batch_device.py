@@ -146,7 +146,7 @@ def test_allocation_failure_halves_the_passes_and_keeps_the_limit(model_dir):
     natoms, types, pos, cells, pbc = _pack(structs)
     N = int(natoms.sum())
     assert 33000 < N < 65000                      # one halving reaches a pass size above the floor of 16384
-    b = kk.Batch(eng.model, ["Al", "Ni", "Ti"])
+    b = kk.Batch(eng.model, ["Al", "Ni", "Ti"], chunksize=0)      # engine passes are not split into chunks of atoms: the batch is
     b.keep_buffers = True                         # the buffers of a call stay, so that what they hold can be measured
     try:
         ref = _device_run(b, natoms, types, pos, cells, pbc, max_nall=N // 2)
@@ -178,6 +178,14 @@ def test_allocation_failure_halves_the_passes_and_keeps_the_limit(model_dir):
         kk.set_memory_limit(0)
         sub = _pack(structs[:20])
         _compare(_device_run(b, *sub), b.compute(*sub, energies=True))
+        # with the automatic chunk size the engine splits the pass itself: one batch pass, chunks of atoms inside it
+        b.release_buffers()
+        auto = kk.Batch(eng.model, ["Al", "Ni", "Ti"])
+        auto.keep_buffers = True
+        kk.set_memory_limit(kk.memory_in_use() + int(0.6 * (held - base)))
+        out = _device_run(auto, natoms, types, pos, cells, pbc)
+        assert auto.passes == 1 and 512 <= auto.chunksize < N
+        _compare(out, ref)
     finally:
         kk.set_memory_limit(0)
 

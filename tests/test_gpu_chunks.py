@@ -1,6 +1,6 @@
 """Atom chunking of an engine pass (System(chunksize=...), python/kk/kk_api.h:72-75,86): a structure evaluated in chunks of
-atoms equals the one-pass result; the automatic choice follows the memory the library may use; an allocation failure
-halves the chunk; model kinds that run in one pass refuse a chunk size."""
+atoms equals the one-pass result for GRACE-1L, 2L and 3L; the automatic choice follows the memory the library may use; an
+allocation failure halves the chunk."""
 import os
 
 import numpy as np
@@ -23,6 +23,7 @@ def _same(a, b, n, tol=1e-10):
 
 @pytest.mark.parametrize("precision", [64, 32])
 @pytest.mark.parametrize("model,struct,species", [("mix2", "alloy54", ["Mo", "W"]), ("cut2", "slab", ["Al", "Ni"]), ("config1", "config1", ["W"]),
+                                                  ("l2mix", "alloy54", ["Mo", "W"]), ("l2mix", "slab", ["Mo", "W"]), ("config3", "fcc108", ["Al", "Co", "Ni", "Ti"]),
                                                   ("l3mix", "alloy54", ["Mo", "W"]), ("l3wide", "fcc108", ["Al", "Ni"]), ("l3el", "alloy54", ["Mo", "W"])])
 def test_chunked_pass_equals_one_pass(model_dir, model, struct, species, precision):
     """chunk sizes that split the tiles of 16 atoms of one element, a chunk of one atom, a chunk larger than the structure"""
@@ -44,7 +45,7 @@ def test_chunked_pass_equals_one_pass(model_dir, model, struct, species, precisi
         del s
 
 
-@pytest.mark.parametrize("model", ["uq2", "uq3l"])
+@pytest.mark.parametrize("model", ["uq2", "uq2l", "uq3l"])
 def test_chunked_uq_and_energy_only(model_dir, model):
     pos, cell, pbc, types = cases.structure_alloy54()
     m = kk.Model(cases.model_file(model_dir, model))
@@ -59,7 +60,7 @@ def test_chunked_uq_and_energy_only(model_dir, model):
     assert abs(eo["energy"] - ref["energy"]) < 1e-9
 
 
-@pytest.mark.parametrize("model", ["mix2", "l3mix"])
+@pytest.mark.parametrize("model", ["mix2", "l2mix", "l3mix"])
 def test_chunked_batch_equals_one_pass(model_dir, model):
     """several structures in one list, chunks that cut through structures"""
     structs = workloads.structures_config5(6)
@@ -113,17 +114,6 @@ def test_automatic_chunk_follows_the_memory_the_library_may_use(tmp_path):
         kk.set_logger(None)
     out = s2.compute(types, pos, cell, pbc)              # the engine is usable again
     _same(out, ref, len(pos))
-
-
-@pytest.mark.parametrize("model", ["l2mix"])
-def test_model_kinds_that_run_in_one_pass_refuse_a_chunk_size(model_dir, model):
-    m = kk.Model(cases.model_file(model_dir, model))
-    with pytest.raises(ValueError, match="one pass"):
-        kk.System(m, ["Mo", "W"], chunksize=64)
-    s = kk.System(m, ["Mo", "W"], chunksize=-1)
-    pos, cell, pbc, types = cases.structure_alloy54()
-    s.compute(types, pos, cell, pbc)
-    assert s.chunksize == 0
 
 
 def test_outputs_accumulate_on_request(model_dir):
