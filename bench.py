@@ -96,6 +96,8 @@ def main():
     ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5"])
     ap.add_argument("--reps", type=int, default=0, help="supercell repetitions (default: 16 bcc cells / 20 fcc cells per edge)")
     ap.add_argument("--atoms", type=int, default=10000, help="atoms of the amorphous cube of config4")
+    ap.add_argument("--chunksize", type=int, default=-1, help="atoms per engine pass: -1 chosen from the free device memory (one pass when "
+                                                              "the structure fits), 0 one pass, > 0 fixed")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives in the path); run with --gpus 1")
@@ -142,6 +144,7 @@ def main():
     t1 = time.perf_counter()
     eng = kk.Engine(model, species, precision=a.precision)
     create_s = time.perf_counter() - t1        # includes the run-time compilation of the model-specialised product kernels
+    eng.set_chunksize(a.chunksize)
     if batch:
         def upload():
             eng.upload_batch(structs, 6.0)
@@ -171,6 +174,7 @@ def main():
         eng.sync()
         one.append(time.perf_counter() - t1)
     median_ms = float(np.median(one)) * 1e3
+    mem_gb = kk.memory_in_use() / 1e9          # device memory the library holds after the timed passes (weights + work buffers)
     out = eng.fetch_batch() if batch else eng.fetch()
     E = eng.edge_count()
     host_ms, list_ms, batch_ms = None, None, None
@@ -321,6 +325,8 @@ def main():
         "ms_per_calculator_call": batch_ms if batch else {"neighbour_list_rebuilt": round(list_ms["rebuilt"], 3),
                                                           "neighbour_list_kept": round(list_ms["kept"], 3)},
         "engine_create_s": round(create_s, 3),
+        "chunksize": eng.chunksize,              # atoms per engine pass the timed steps ran with (0: the whole structure in one pass)
+        "device_memory_GB": round(mem_gb, 3),
         "roofline": roofline,
         "hbm_calibration": {"copy_GBs": round(copy_gbs, 1), "read_only_GBs": round(read_gbs, 1), "bytes": 1 << 30,
                             "note": "plain stream kernels over 1 GiB, best of 5: copy counts bytes read + written; roofline.frac "
