@@ -13,7 +13,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgrace_hip.so")
 
 GR_OK, GR_INVALID, GR_ERROR, GR_NOMEM = 0, 1, 2, 3
-FLAG_ENERGY_ONLY, FLAG_EATOM, FLAG_UQ, FLAG_ACCUMULATE, FLAG_SAME_LIST = 1, 2, 4, 8, 16
+FLAG_ENERGY_ONLY, FLAG_EATOM, FLAG_UQ, FLAG_ACCUMULATE, FLAG_SAME_LIST, FLAG_VATOM = 1, 2, 4, 8, 16, 32
 
 # every symbol include/grace_hip.h declares (checked by the CPU test-suite against the header and the library)
 SYMBOLS = [
@@ -21,7 +21,8 @@ SYMBOLS = [
     "gr_model_element_name", "gr_model_free", "gr_engine_create", "gr_engine_free", "gr_engine_cutoff",
     "gr_compute_csr", "gr_engine_upload", "gr_engine_run", "gr_engine_sync", "gr_engine_fetch",
     "gr_engine_edge_count", "gr_engine_set_profile", "gr_engine_stage_count", "gr_engine_stage_get", "gr_engine_stage_flops",
-    "gr_engine_debug_radial", "gr_engine_radial_noalloc", "gr_engine_debug_copy", "gr_engine_stream_rates", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
+    "gr_engine_debug_radial", "gr_engine_radial_noalloc", "gr_engine_debug_copy", "gr_engine_stream_rates", "gr_engine_fetch_vatom", "gr_system_fetch_vatom", "gr_lammps_add_vatom",
+    "gr_lammps_add_vatom_device", "gr_neighbor_build", "gr_nlist_nbonds", "gr_nlist_nimages", "gr_nlist_get",
     "gr_nlist_free", "gr_compute", "gr_compute_batch", "gr_engine_upload_batch", "gr_engine_fetch_batch",
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
     "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_batch_uq", "gr_compute_batch_device_uq", "gr_engine_reset", "gr_engine_release_buffers", "gr_set_memory_limit", "gr_memory_in_use", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
@@ -103,6 +104,10 @@ def lib():
     L.gr_engine_radial_noalloc.argtypes = [vp, i32, vp, vp, vp, vp]
     L.gr_engine_debug_copy.argtypes = [vp, i64]
     L.gr_engine_stream_rates.argtypes = [vp, i64, vp, vp]
+    L.gr_engine_fetch_vatom.argtypes = [vp, vp]
+    L.gr_system_fetch_vatom.argtypes = [vp, vp]
+    L.gr_lammps_add_vatom.argtypes = [vp, i32, vp]
+    L.gr_lammps_add_vatom_device.argtypes = [vp, i32, vp]
     L.gr_neighbor_build.argtypes = [i64, vp, vp, vp, dbl, i32, C.POINTER(vp)]
     L.gr_nlist_nbonds.restype = i64
     L.gr_nlist_nbonds.argtypes = [vp]

@@ -37,6 +37,10 @@ struct gr_engine {
   bool has_exchange = false;                           // an exchange is installed: ghosts of the LAMMPS call stay atoms of their own
   grhip::ExchangeCallbacks exchange;                   // kept for the engine a reset makes
   int chunk_request = -1;                              // the caller's chunk size, kept for the engine a reset makes
+  std::vector<int> lmp_rows;                           // gr_compute_lammps: LAMMPS index of engine row q (empty: rows are LAMMPS indices)
+  int lmp_nall = -1;                                   // atoms of the last gr_compute_lammps[_device] call
+  uint64_t lmp_serial = 0;                             // the engine's upload count at that call: its list is still the one held
+  bool lmp_on_device = false;                          // that call was the device form (its row map is lmp->atom)
   void make()
   {
     if (m1) eng = grhip::make_engine_1l(m1, ntypes, type2mu, precision, device);
@@ -303,6 +307,7 @@ int gr_engine_run(gr_engine *e, unsigned flags)
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0;
+    fl.vatom = (flags & GR_FLAG_VATOM) != 0;
     fl.uq = (flags & GR_FLAG_UQ) != 0;
     live(e).run(fl);
   });
@@ -313,6 +318,14 @@ int gr_engine_fetch_uq(gr_engine *e, double *gamma, double *sigma, double *clust
   return guarded([&] {
     if (!e) throw grhip::InvalidArgument("null engine");
     live(e).fetch_uq(gamma, sigma, cluster);
+  });
+}
+
+int gr_engine_fetch_vatom(gr_engine *e, double *vatom)
+{
+  return guarded([&] {
+    if (!e || !vatom) throw grhip::InvalidArgument("null argument");
+    live(e).fetch_vatom(vatom);
   });
 }
 
@@ -369,6 +382,7 @@ int gr_compute_csr(gr_engine *e, int n, const int *types, const int64_t *offset,
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.vatom = (flags & GR_FLAG_VATOM) != 0;
     live(e).run(fl);
     if (!(flags & GR_FLAG_ACCUMULATE)) {
       live(e).fetch(energy, forces, virial, eatom);
@@ -515,6 +529,7 @@ int gr_compute(gr_engine *e, int n, const int *types, const double *positions, c
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.vatom = (flags & GR_FLAG_VATOM) != 0;
     live(e).run(fl);
     std::vector<double> f((size_t) 3 * n), ea(fl.eatom ? n : 0);
     live(e).fetch(energy, forces ? f.data() : nullptr, virial, fl.eatom ? ea.data() : nullptr);
@@ -540,6 +555,7 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.vatom = (flags & GR_FLAG_VATOM) != 0;
     if (!owner && nall > nlocal && (e->has_exchange || eng.comm_layers() == 0)) {
       // Ghosts stay atoms of their own (the way of the reference's drivers): bonds name them by their LAMMPS index, their
       // message rows come through the exchange, and what the pass leaves on them (forces, adjoint rows) goes back through
@@ -571,6 +587,10 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
       in.n_nodes = nall;
       eng.upload(in);
       eng.run(fl);
+      e->lmp_rows.clear();    // rows are LAMMPS indices
+      e->lmp_nall = nall;
+      e->lmp_serial = eng.upload_serial();
+      e->lmp_on_device = false;
       std::vector<double> fo((size_t) 3 * nall), ea(fl.eatom ? nlocal : 0);
       double en = 0.0, vir[6] = {0, 0, 0, 0, 0, 0};
       eng.fetch(&en, f ? fo.data() : nullptr, vir, fl.eatom ? ea.data() : nullptr);
@@ -623,6 +643,10 @@ int gr_compute_lammps(gr_engine *e, int nlocal, int nall, const int *type, const
     const std::vector<double> dummy(3, 0.0);
     eng.upload(make_input(n, ty.data(), offset.data(), jj.data(), rij.empty() ? dummy.data() : rij.data(), nullptr, nullptr, nullptr, 0));
     eng.run(fl);
+    e->lmp_rows = atom;
+    e->lmp_nall = nall;
+    e->lmp_serial = eng.upload_serial();
+    e->lmp_on_device = false;
     std::vector<double> fo((size_t) 3 * n), ea(fl.eatom ? n : 0);
     double en = 0.0, vir[6] = {0, 0, 0, 0, 0, 0};
     eng.fetch(&en, f ? fo.data() : nullptr, vir, fl.eatom ? ea.data() : nullptr);
@@ -726,6 +750,7 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.vatom = (flags & GR_FLAG_VATOM) != 0;
     const bool nodes = !owner && nall > nlocal && (e->has_exchange || eng.comm_layers() == 0);
     grhip::LmpListDev L{};
     L.type = type; L.x = x; L.numneigh = numneigh; L.neighbors = neighbors; L.stride_i = stride_i; L.stride_k = stride_k;
@@ -743,6 +768,9 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
       }
       eng.run(fl);
       eng.fetch_add_device(nodes ? nullptr : W.atom.as<int>(), energy, f, virial, fl.eatom ? eatom : nullptr);
+      e->lmp_nall = nall;
+      e->lmp_serial = eng.upload_serial();
+      e->lmp_on_device = true;
       return;
     }
     W.kept = false;
@@ -826,6 +854,38 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
     W.stride_i = stride_i; W.stride_k = stride_k; W.neighbors = neighbors; W.type = type; W.numneigh = numneigh; W.owner = owner;
     eng.run(fl);
     eng.fetch_add_device(nodes ? nullptr : W.atom.as<int>(), energy, f, virial, fl.eatom ? eatom : nullptr);
+    e->lmp_nall = nall;
+    e->lmp_serial = eng.upload_serial();
+    e->lmp_on_device = true;
+  });
+}
+
+int gr_lammps_add_vatom(gr_engine *e, int nall, double *vatom)
+{
+  return guarded([&] {
+    if (!e || !vatom) throw grhip::InvalidArgument("null argument");
+    grhip::Engine &eng = live(e);
+    if (e->lmp_nall != nall || e->lmp_on_device || e->lmp_serial != eng.upload_serial())
+      throw grhip::Error("gr_lammps_add_vatom follows a gr_compute_lammps call with GR_FLAG_VATOM on the same atoms");
+    const bool nodes = e->lmp_rows.empty();
+    const size_t rows = nodes ? (size_t) nall : e->lmp_rows.size();
+    std::vector<double> v(6 * std::max<size_t>(rows, 1));
+    eng.fetch_vatom(v.data());
+    for (size_t q = 0; q < rows; q++) {
+      const size_t a = nodes ? q : (size_t) e->lmp_rows[q];
+      for (int k = 0; k < 6; k++) vatom[6 * a + k] += v[6 * q + k];
+    }
+  });
+}
+
+int gr_lammps_add_vatom_device(gr_engine *e, int nall, double *vatom)
+{
+  return guarded([&] {
+    if (!e || !vatom) throw grhip::InvalidArgument("null argument");
+    grhip::Engine &eng = live(e);
+    if (e->lmp_nall != nall || !e->lmp_on_device || e->lmp_serial != eng.upload_serial() || !e->lmp)
+      throw grhip::Error("gr_lammps_add_vatom_device follows a gr_compute_lammps_device call with GR_FLAG_VATOM on the same atoms");
+    eng.add_vatom_device(e->lmp->nodes ? nullptr : e->lmp->atom.as<int>(), vatom);
   });
 }
 
@@ -932,6 +992,7 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.vatom = (flags & GR_FLAG_VATOM) != 0;
     fl.uq = (flags & GR_FLAG_UQ) != 0;
     eng.run(fl);
     std::vector<double> f((size_t) 3 * n), ea(fl.eatom ? n : 0);
@@ -1017,6 +1078,19 @@ int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *clust
       if (sigma) sigma[a] = sg[q];
       if (cluster) cluster[a] = cl[q];
     }
+  });
+}
+
+int gr_system_fetch_vatom(gr_system *s, double *vatom)
+{
+  return guarded([&] {
+    if (!s || !s->have) throw grhip::Error("gr_system_fetch_vatom: no structure has been computed");
+    if (!vatom) throw grhip::InvalidArgument("null argument");
+    const int n = s->n;
+    std::vector<double> v((size_t) 6 * n);
+    live(s->eng).fetch_vatom(v.data());
+    for (int q = 0; q < n; q++)
+      for (int k = 0; k < 6; k++) vatom[6 * s->perm[q] + k] = v[6 * (size_t) q + k];
   });
 }
 
@@ -1224,6 +1298,7 @@ int gr_compute_batch_uq(gr_engine *e, int nstruct, const int *natoms, const int 
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.vatom = (flags & GR_FLAG_VATOM) != 0;
     fl.uq = gamma || sigma || cluster;
     live(e).run(fl);
     std::vector<double> f((size_t) 3 * N), ea(fl.eatom ? N : 0);
@@ -1296,6 +1371,7 @@ int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, con
     grhip::RunFlags fl;
     fl.energy_only = (flags & GR_FLAG_ENERGY_ONLY) != 0;
     fl.eatom = (flags & GR_FLAG_EATOM) != 0 && eatom;
+    fl.vatom = (flags & GR_FLAG_VATOM) != 0;
     fl.uq = gamma || sigma || cluster;
     // passes of whole structures with at most `limit` atoms (at least one structure each); every pass overwrites its outputs
     auto once = [&](int64_t limit) {

@@ -71,6 +71,7 @@ struct RunFlags {
   bool energy_only = false;
   bool eatom = false;
   bool uq = false;    // UQ head (ComputeFlags::uq, libgrace/include/grace/system.h:117): gamma, sigma, cluster per atom
+  bool vatom = false; // per-atom virials (ComputeFlags::vflag_atom, system.h:115): half of every bond's virial to each of its atoms
 };
 
 class Engine {
@@ -103,6 +104,10 @@ class Engine {
   // caller, row q of the engine to row atom[q] (atom: device [n]); null pointers are skipped
   virtual void fetch_add_device(const int *atom, double *energy, double *forces, double *virial, double *eatom) = 0;
   // UQ outputs of the last run with RunFlags::uq, [n] each in the order of the uploaded list (null pointers are skipped)
+  // per-atom virials [n_nodes][6] (xx yy zz xy xz yz) of a run with the vatom flag, in the order of the uploaded list; host memory
+  virtual void fetch_vatom(double *vatom) = 0;
+  // the same rows added to a device array: row q of the list goes to row atom[q] (null: row q) of vatom
+  virtual void add_vatom_device(const int *atom, double *vatom) = 0;
   virtual void fetch_uq(double *gamma, double *sigma, double *cluster) = 0;
   // atoms per engine pass (python/kk/kk_api.h:72-75): 0 all atoms in one pass, < 0 chosen from the free device memory
   // (one pass while it fits, else the largest power of two >= 512 that fits), > 0 as given.  chunksize_used(): atoms per

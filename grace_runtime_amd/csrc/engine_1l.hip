@@ -519,7 +519,7 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
   BondBwdArgs<T> ba{};
   ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
   ba.Rz = Rz; ba.dRz = dRz; ba.gA = gA;
-  ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
+  ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr(); ba.vatom = vatom_ptr();
   ba.a0 = a0; ba.C = CP_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;
   stage("bond_bwd", [&] { launch_bond_bwd<T>(ba, n); });
 }

@@ -694,7 +694,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
       const size_t lds = (size_t) kPairChunk * (pthreads + 2 * radR1_.noutp) * sizeof(T);
       GR_PAIR(k_pair_bwd, dim3(nc), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) dR1, (const T *) M,
               (const T *) gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(), scal_.as<double>() + 1,
-              nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_, 0, nc, a0_);
+              nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_, 0, nc, a0_, vatom_ptr());
     });
   }
 #undef GR_PAIR
@@ -736,7 +736,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     BondBwdArgs<T> ba{};
     ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
     ba.Rz = moved_back(Rz_.as<T>(), eb * radR_.noutp); ba.dRz = moved_back(dRz_.as<T>(), eb * radR_.noutp); ba.gA = c1_.gX.template as<T>();
-    ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
+    ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr(); ba.vatom = vatom_ptr();
     ba.a0 = a0_; ba.C = C1P_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = radR_.noutp; ba.sh = sh_;
     stage("bond_bwd", [&] { launch_bond_bwd<T>(ba, cn_); });
   }

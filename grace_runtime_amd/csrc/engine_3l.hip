@@ -877,7 +877,7 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
     BondBwdArgs<T> ba{};
     ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
     ba.Rz = Rl; ba.dRz = dRl; ba.gA = gX;
-    ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr();
+    ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr(); ba.vatom = vatom_ptr();
     ba.a0 = a0_; ba.C = L.CP; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = L.rad.noutp; ba.sh = sh_;
     stage(tg(k, "bond_bwd").c_str(), [&] { launch_bond_bwd<T>(ba, n); });
     return;
@@ -897,7 +897,7 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
     const size_t lds = (size_t) kPairChunk * (pthreads + 2 * L.rad.noutp) * s;
     GR_PAIR(k_pair_bwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl,
             (const T *) dRl, (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(),
-            f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_);
+            f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_, vatom_ptr());
   });
   (void) yw;
 }

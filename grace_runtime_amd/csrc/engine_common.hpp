@@ -563,7 +563,7 @@ class EngineBase : public Engine, protected BufRegistry {
     n_nodes_ = 0;
     nb_ = 0;
     nstruct_ = 1;
-    ran_ = ran_forces_ = ran_eatom_ = ran_uq_ = false;
+    ran_ = ran_forces_ = ran_eatom_ = ran_uq_ = ran_vatom_ = false;
     upload_serial_++;
   }
   void synchronize() override { check(hipSetDevice(device_), "hipSetDevice"); check(hipStreamSynchronize(stream_), "hipStreamSynchronize"); }
@@ -879,6 +879,25 @@ class EngineBase : public Engine, protected BufRegistry {
     if (virial && ran_forces_)
       for (int k = 0; k < 6; k++) virial[k] = s[1 + k];
   }
+  void fetch_vatom(double *vatom) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (!ran_ || !ran_vatom_) throw Error("fetch_vatom() needs a run with the per-atom virial flag (and forces)");
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    check_zero_bond();
+    if (vatom && n_nodes_ > 0) HIP_CHECK(hipMemcpy(vatom, vatom_.p, sizeof(double) * 6 * n_nodes_, hipMemcpyDeviceToHost));
+  }
+  void add_vatom_device(const int *atom, double *vatom) override
+  {
+    HIP_CHECK(hipSetDevice(device_));
+    if (!ran_ || !ran_vatom_) throw Error("per-atom virials need a run with the per-atom virial flag (and forces)");
+    if (n_nodes_ > n_ && atom) throw Error("add_vatom_device: a list with ghost atoms keeps the caller's atom order");
+    HIP_CHECK(hipStreamSynchronize(stream_));
+    check_zero_bond();
+    const long long tot = 6ll * n_nodes_;
+    if (tot > 0) hipLaunchKernelGGL(k_add_rows6, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, atom, n_nodes_, vatom_.as<double>(), vatom);
+    HIP_CHECK(hipStreamSynchronize(stream_));
+  }
   void fetch_uq(double *gamma, double *sigma, double *cluster) override
   {
     HIP_CHECK(hipSetDevice(device_));
@@ -932,6 +951,11 @@ class EngineBase : public Engine, protected BufRegistry {
     ran_ = true;
     n_peak_ = std::max(n_peak_, n_);
     ran_forces_ = !fl.energy_only;
+    ran_vatom_ = fl.vatom && !fl.energy_only;
+    if (ran_vatom_) {
+      vatom_.ensure(std::max<size_t>((size_t) 6 * n_nodes_, 1) * sizeof(double));
+      HIP_CHECK(hipMemsetAsync(vatom_.p, 0, (size_t) 6 * n_nodes_ * sizeof(double), stream_));
+    }
     ran_eatom_ = fl.eatom;
     ran_uq_ = false;    // set by the engine that evaluates a UQ head
     if (fl.uq && !has_uq_head_) throw InvalidArgument(who_ + ": the model has no usable UQ head (" + uq_why_ + ")");
@@ -1273,6 +1297,9 @@ class EngineBase : public Engine, protected BufRegistry {
   // uploaded structure
   int n_nodes_ = 0;           // central atoms and ghosts (= n_ without ghosts)
   uint64_t upload_serial_ = 0;
+  DevBuf vatom_;              // per-atom virials [n_nodes][6] of a pass with the vatom flag
+  bool ran_vatom_ = false;
+  double *vatom_ptr() { return ran_vatom_ ? vatom_.as<double>() : nullptr; }
   ExchangeCallbacks exchange_{};
   DevBuf comm_list_, comm_buf_;    // staging of the host forms of the row movers
   int n_ = 0, n_peak_ = 0;    // atoms of the uploaded structure; of the largest pass since the work buffers were released

@@ -257,6 +257,16 @@ static __global__ void k_add_results(const int *atom, int nf, int ne, const doub
   if (eatom && q < ne) eatom[i] += ee[q];
 }
 
+// dst[atom[q]][k] += src[q][k], k < 6 (atom null: row q)
+static __global__ void k_add_rows6(const int *atom, int n, const double *src, double *dst)
+{
+  const long long t = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (t >= 6ll * n) return;
+  const long long q = t / 6;
+  const int k = (int) (t % 6);
+  dst[6 * (atom ? (long long) atom[q] : q) + k] += src[t];
+}
+
 struct Edges {
   int *ei, *ej, *emu;         // central atom, neighbour, neighbour element
   double *rh;                 // [E][3] unit vectors
@@ -1378,6 +1388,7 @@ template<class T> struct BondBwdArgs {
   double *f;                  // [n][3]  (+=, atomics)
   double *virial;             // [6]     (+=, atomics); with sid: record 8 sid[i] of the atom's structure
   const int *sid;             // [n] structure of each atom, or null
+  double *vatom;              // [n][6] per-atom virial (+=, atomics), or null: half of a bond's (-r rhat) (x) fv to each of its atoms
   int a0;
   int C, nl, nlm, noutp;
   int drow[16];               // accumulator row of (lane / 16, register)
@@ -1485,6 +1496,11 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
       const double ddx = -u0 * br, ddy = -u1 * br, ddz = -u2 * br;
       vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
       vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
+      if (a.vatom) {    // the neighbour's half (add_vatom, libgrace/include/grace/fused_cpu.h:1075-1087); the atom's own below
+        double *vj = a.vatom + 6 * (long long) jj;
+        atomicAdd(vj, 0.5 * ddx * fv[0]); atomicAdd(vj + 1, 0.5 * ddy * fv[1]); atomicAdd(vj + 2, 0.5 * ddz * fv[2]);
+        atomicAdd(vj + 3, 0.5 * ddx * fv[1]); atomicAdd(vj + 4, 0.5 * ddx * fv[2]); atomicAdd(vj + 5, 0.5 * ddy * fv[2]);
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -1500,7 +1516,10 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
     const double s = red[0][t] + red[1][t] + red[2][t] + red[3][t];
     if (e1 > e0) {
       if (t < 3) atomicAdd(&a.f[3 * (long long) i + t], s);
-      else atomicAdd(&a.virial[(a.sid ? 8 * a.sid[i] : 0) + t - 3], s);
+      else {
+        atomicAdd(&a.virial[(a.sid ? 8 * a.sid[i] : 0) + t - 3], s);
+        if (a.vatom) atomicAdd(&a.vatom[6 * (long long) i + t - 3], 0.5 * s);
+      }
     }
   }
 }

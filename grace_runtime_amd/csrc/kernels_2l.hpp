@@ -206,7 +206,8 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
                            const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
                            const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
                            T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
-                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms, int a0)
+                           int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms, int a0,
+                           double *__restrict__ vatom)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   __shared__ double bsum[kPairChunk][4];
@@ -276,6 +277,11 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
       const double ddx = -u[0] * r, ddy = -u[1] * r, ddz = -u[2] * r;
       vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
       vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
+      if (vatom) {    // per-atom virial: the neighbour's half of this bond (fused_cpu.h:1075-1087 of the reference)
+        double *vj = vatom + 6 * (long long) jj;
+        atomicAdd(vj, 0.5 * ddx * fv[0]); atomicAdd(vj + 1, 0.5 * ddy * fv[1]); atomicAdd(vj + 2, 0.5 * ddz * fv[2]);
+        atomicAdd(vj + 3, 0.5 * ddx * fv[1]); atomicAdd(vj + 4, 0.5 * ddx * fv[2]); atomicAdd(vj + 5, 0.5 * ddy * fv[2]);
+      }
     }
   }
   // the finishing threads t < kPairChunk sit in wave 0
@@ -287,6 +293,8 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
     if (lane == 0 && e1 > e0) {
       for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) (a0 + i) + k], vsum[k]);
       for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[a0 + i] : 0) + k], vsum[3 + k]);
+      if (vatom)
+        for (int k = 0; k < 6; k++) atomicAdd(&vatom[6 * (long long) (a0 + i) + k], 0.5 * vsum[3 + k]);
     }
   }
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive

@@ -313,10 +313,11 @@ class Engine:
         return n, (types, offset, j, rij, positions, image, shifts), nimg
 
     def compute_lammps(self, nlocal, types, x, ilist, numneigh, firstneigh, owner=None, neighmask=0x1FFFFFFF, energies=False,
-                       energy_only=False, forces=None, eatom=None):
+                       energy_only=False, forces=None, eatom=None, vatom=None):
         """The call of a LAMMPS pair style (gr_compute_lammps): owned + ghost atoms `x[nall, 3]`, `types[nall]`, the full
         neighbour list as `numneigh[nlocal]` and a list of index arrays `firstneigh[i]`, `owner[nall]` the owned atom of every
-        ghost.  Forces are ADDED to `forces[nall, 3]` (zeros when not given), per-atom energies to `eatom[nall]`."""
+        ghost.  Forces are ADDED to `forces[nall, 3]` (zeros when not given), per-atom energies to `eatom[nall]`, per-atom
+        virials to `vatom[nall, 6]` when given."""
         types = as_array(types, np.int32)
         x = as_array(x, np.float64, 3)
         nall = types.shape[0]
@@ -328,11 +329,14 @@ class Engine:
         f = np.zeros((nall, 3)) if forces is None else forces
         ea = (np.zeros(nall) if eatom is None else eatom) if energies else None
         e, v = C.c_double(), np.zeros(6)
-        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (_lib.FLAG_VATOM if vatom is not None else 0)
         check(_lib.lib().gr_compute_lammps(self._h, int(nlocal), nall, ptr(types), ptr(x), ilist.shape[0], ptr(ilist), ptr(numneigh), fn,
                                            int(neighmask), ptr(own) if own is not None else None, flags, C.byref(e),
                                            None if energy_only else ptr(f), ptr(v), ptr(ea) if ea is not None else None))
         out = {"energy": e.value}
+        if vatom is not None:
+            check(_lib.lib().gr_lammps_add_vatom(self._h, nall, ptr(vatom)))
+            out["vatom"] = vatom
         if not energy_only:
             out["forces"], out["virial"] = f, v
         if energies:
@@ -340,7 +344,7 @@ class Engine:
         return out
 
     def compute_lammps_device(self, nlocal, types, x, ilist, numneigh, neighbors, owner=None, neighmask=0x1FFFFFFF, energy_only=False,
-                              forces=None, eatom=None, same_list=False):
+                              forces=None, eatom=None, same_list=False, vatom=None):
         """The call of a KOKKOS pair style (gr_compute_lammps_device): every array is a device array of the module's GPU
         (torch tensors): `types[nall]` int32, `x[nall, 3]`, `ilist[inum]`, `numneigh[nlocal]`, the 2-d neighbour view
         `neighbors[nlocal, maxneigh]` in either layout, `owner[nall]`.  Forces are ADDED to `forces[nall, 3]` and per-atom
@@ -359,10 +363,14 @@ class Engine:
         p_f = _device_pointer(forces, "forces", (nall, 3), "float64") if forces is not None else None
         p_ea = _device_pointer(eatom, "eatom", (nall,), "float64") if eatom is not None else None
         e, v = C.c_double(), np.zeros(6)
-        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if eatom is not None else 0) | (_lib.FLAG_SAME_LIST if same_list else 0)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if eatom is not None else 0) | (_lib.FLAG_SAME_LIST if same_list else 0) | \
+            (_lib.FLAG_VATOM if vatom is not None else 0)
+        p_va = _device_pointer(vatom, "vatom", (nall, 6), "float64") if vatom is not None else None
         check(_lib.lib().gr_compute_lammps_device(self._h, int(nlocal), nall, len(self.species), p_t, p_x, inum, p_il, p_nn,
                                                   C.c_void_p(neighbors.data_ptr()), int(neighbors.stride(0)), int(neighbors.stride(1)),
                                                   int(neighmask), p_own, flags, C.byref(e), None if energy_only else p_f, ptr(v), p_ea))
+        if vatom is not None:
+            check(_lib.lib().gr_lammps_add_vatom_device(self._h, nall, p_va))
         out = {"energy": e.value}
         if not energy_only:
             out["virial"] = v
@@ -395,9 +403,17 @@ class Engine:
         check(_lib.lib().gr_engine_upload(self._h, n, *[ptr(a) for a in arrs], nimg))
         self._n = n
 
-    def run(self, energies=False, energy_only=False, uq=False):
-        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (FLAG_UQ if uq else 0)
+    def run(self, energies=False, energy_only=False, uq=False, virials=False):
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (FLAG_UQ if uq else 0) | \
+            (_lib.FLAG_VATOM if virials else 0)
         check(_lib.lib().gr_engine_run(self._h, flags))
+
+    def fetch_vatom(self, rows=None):
+        """per-atom virials [rows, 6] = xx yy zz xy xz yz of the last run(virials=True), in the order of the uploaded list
+        (Outputs::vatom, libgrace/include/grace/system.h:71): half of every bond's virial to each of its two atoms"""
+        v = np.zeros((self._n if rows is None else int(rows), 6))
+        check(_lib.lib().gr_engine_fetch_vatom(self._h, ptr(v)))
+        return v
 
     def fetch_uq(self):
         """gamma, atomic_sigma, gmm_cluster [n] of the last run(uq=True), in the order of the uploaded list"""
@@ -613,9 +629,10 @@ class System:
         check(_lib.lib().gr_system_list_get(self._h, ptr(perm), ptr(offset), ptr(j), ptr(image), ptr(shifts)))
         return perm, offset, j, image, shifts
 
-    def compute(self, types, positions, cell, pbc, energies=False, uq=False, energy_only=False):
+    def compute(self, types, positions, cell, pbc, energies=False, uq=False, energy_only=False, virials=False):
         """energy, forces [n, 3], virial [6], energies [n]; with `uq` also gamma, atomic_sigma, gmm_cluster [n] of the
-        model's UQ head (ValueError when the model has none that can be evaluated)."""
+        model's UQ head (ValueError when the model has none that can be evaluated); with `virials` the per-atom virials
+        [n, 6] (the reference's vatom)."""
         types = as_array(types, np.int32)
         pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
         cell = np.ascontiguousarray(cell, dtype=np.float64).reshape(3, 3)
@@ -630,7 +647,8 @@ class System:
         forces = None if energy_only else np.empty((n, 3))
         virial = None if energy_only else np.empty(6)
         eat = np.empty(n) if energies else None
-        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (FLAG_UQ if uq else 0)
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (FLAG_UQ if uq else 0) | \
+            (_lib.FLAG_VATOM if virials and not energy_only else 0)
         check(_lib.lib().gr_system_compute(self._h, n, ptr(types), ptr(pos), ptr(cell), ptr(pb), flags, C.byref(e),
                                       ptr(forces) if forces is not None else None, ptr(virial) if virial is not None else None,
                                       ptr(eat) if eat is not None else None))
@@ -643,6 +661,10 @@ class System:
             g, sg, cl = np.empty(n), np.empty(n), np.empty(n)
             check(_lib.lib().gr_system_fetch_uq(self._h, ptr(g), ptr(sg), ptr(cl)))
             res["gamma"], res["atomic_sigma"], res["gmm_cluster"] = g, sg, cl
+        if virials and not energy_only:
+            va = np.zeros((n, 6))
+            check(_lib.lib().gr_system_fetch_vatom(self._h, ptr(va)))
+            res["virials"] = va
         return res
 
 

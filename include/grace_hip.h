@@ -34,6 +34,10 @@ enum {
   GR_FLAG_UQ = 4,          /* ComputeFlags::uq (system.h:117): the UQ head; gr_engine_run and gr_system_compute */
   GR_FLAG_ACCUMULATE = 8,  /* gr_compute_csr: energy, forces, virial and per-atom energies are ADDED to the caller's values, as
                               the reference's Outputs accumulate (system.h:66-75); without it they are overwritten */
+  GR_FLAG_VATOM = 32,      /* ComputeFlags::vflag_atom (system.h:115): per-atom virials, Outputs::vatom (system.h:71): every bond's
+                              virial (x_i - x_j) (x) f_i goes half to each of its two atoms (add_vatom, libgrace/include/grace/
+                              fused_cpu.h:1075-1087), so the rows add up to the total virial.  Needs forces.  The rows are read
+                              with gr_engine_fetch_vatom / gr_system_fetch_vatom / gr_lammps_add_vatom after the call */
   GR_FLAG_SAME_LIST = 16   /* gr_compute_lammps_device: atom counts, types, ilist, neighbour list and owner map are those of the
                               previous call on this engine and only x has changed (LAMMPS: neighbor->ago > 0, the steps between
                               two reneighbourings): the converted list is kept, only the bond vectors are renewed and no array
@@ -184,7 +188,13 @@ int gr_compute(gr_engine *e, int n, const int *types, const double *positions, c
 int gr_model_has_uq(const gr_model *m);
 int gr_model_validate_uq(const gr_model *m);
 int gr_engine_fetch_uq(gr_engine *e, double *gamma, double *sigma, double *cluster);
+/* Per-atom virials [atoms][6] = xx yy zz xy xz yz of the last pass with GR_FLAG_VATOM (gr_engine_run, gr_compute_csr):
+ * rows in the order of the uploaded list (with ghost atoms as nodes: all of them); Outputs::vatom of the reference
+ * (libgrace/include/grace/system.h:71).  GR_ERROR when that pass did not compute them. */
+int gr_engine_fetch_vatom(gr_engine *e, double *vatom);
 int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *cluster);
+/* Per-atom virials [n][6] of the last gr_system_compute with GR_FLAG_VATOM, in the caller's atom order. */
+int gr_system_fetch_vatom(gr_system *s, double *vatom);
 
 /* The call of a LAMMPS pair style on one MPI rank: owned and ghost atoms with LAMMPS' full neighbour list.  Replaces
  * Grace{1,2,3}LFused::compute<LammpsBonds>(inum, ilist, n_nodes, nmax_nodes, LammpsBonds{x, type, numneigh, firstneigh,
@@ -245,6 +255,13 @@ int gr_engine_unpack_reverse_host(gr_engine *e, int layer, int n, const int *sen
 int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, const int *type, const double *x, int inum, const int *ilist,
                              const int *numneigh, const int *neighbors, int64_t stride_i, int64_t stride_k, int neighmask, const int *owner,
                              unsigned flags, double *energy, double *f, double *virial, double *eatom);
+
+/* Adds the per-atom virials of the last gr_compute_lammps (host array) / gr_compute_lammps_device (device array) call
+ * that carried GR_FLAG_VATOM to vatom [nall][6] by LAMMPS atom index: RunInput::vatom of the reference's GPU engines
+ * (libgrace/include/grace/kk/grace_1l_kk.h:93,101).  With an owner map the halves of ghost atoms are on their owners'
+ * rows; without one (nodes) they stay on the ghosts for LAMMPS' reverse communication. */
+int gr_lammps_add_vatom(gr_engine *e, int nall, double *vatom);
+int gr_lammps_add_vatom_device(gr_engine *e, int nall, double *vatom);
 
 /* One structure resident on the device with a Verlet list at cutoff + skin: System of the reference's GPU module
  * (python/kk/kk_api.h:66-93, System::compute python/kk/kk_core.cpp:802-958; list policy python/grace_runtime/

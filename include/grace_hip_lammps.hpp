@@ -44,6 +44,8 @@ struct RunInput {
   bool energy_only = false;
   bool same_list = false;             // neighbor->ago > 0: the arrays are those of the previous run, only x has changed
   double *eatom = nullptr;            // [nall], per-atom energies are ADDED (with eflag_atom)
+  int vflag_atom = 0;
+  double *vatom = nullptr;            // [nall][6] xx yy zz xy xz yz, per-atom virials are ADDED (with vflag_atom)
 };
 struct RunOutput {
   double eng_vdwl = 0.0;
@@ -92,8 +94,11 @@ class Engine {
     if (in.energy_only) flags |= GR_FLAG_ENERGY_ONLY;
     if (in.eflag_atom && in.eatom) flags |= GR_FLAG_EATOM;
     if (in.same_list) flags |= GR_FLAG_SAME_LIST;
+    const bool vatom = in.vflag_atom && in.vatom && !in.energy_only;
+    if (vatom) flags |= GR_FLAG_VATOM;
     check(gr_compute_lammps_device(engine_, in.nlocal, in.nall, in.ntypes, in.type, in.x, in.inum, in.ilist, in.numneigh, in.neighbors,
                                    in.stride_i, in.stride_k, in.neighmask, in.owner, flags, &out.eng_vdwl, in.f, out.virial, in.eatom));
+    if (vatom) check(gr_lammps_add_vatom_device(engine_, in.nall, in.vatom));
     return out;
   }
 

@@ -450,6 +450,7 @@ def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=Tru
     energies = np.zeros(n)
     forces = np.zeros((n, 3))
     virial = np.zeros(6)
+    virials = np.zeros((n, 6))
     uqv = [np.zeros(n), np.zeros(n), np.zeros(n)] if uq else None
     feats = np.zeros((n, model.uq_D)) if uq else None
     for a0 in range(0, n, chunk):
@@ -502,12 +503,20 @@ def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=Tru
         np.add.at(forces, bi, fv)                                                # fused_cpu.h:1089-1095
         np.add.at(forces, bj, -fv)
         dl = -rh * r[:, None]                                                    # src/fused_1l.cpp:46-51
-        virial += np.array([(dl[:, 0] * fv[:, 0]).sum(), (dl[:, 1] * fv[:, 1]).sum(), (dl[:, 2] * fv[:, 2]).sum(),
-                            (dl[:, 0] * fv[:, 1]).sum(), (dl[:, 0] * fv[:, 2]).sum(), (dl[:, 1] * fv[:, 2]).sum()])
-    out = {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial}
+        v6 = bond_virials(dl, fv)
+        virial += v6.sum(0)
+        np.add.at(virials, bi, 0.5 * v6)                                         # add_vatom, fused_cpu.h:1075-1087: half to each atom
+        np.add.at(virials, bj, 0.5 * v6)
+    out = {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial, "virials": virials}
     if uq:
         out.update(gamma=uqv[0], atomic_sigma=uqv[1], gmm_cluster=uqv[2], uq_features=feats)
     return out
+
+
+def bond_virials(dl, fv):
+    """[nb, 6] = (xx yy zz xy xz yz) of dl (x) fv per bond, dl = x_i - x_j, fv = force on i (src/fused_1l.cpp:46-51)"""
+    return np.stack([dl[:, 0] * fv[:, 0], dl[:, 1] * fv[:, 1], dl[:, 2] * fv[:, 2], dl[:, 0] * fv[:, 1], dl[:, 0] * fv[:, 2],
+                     dl[:, 1] * fv[:, 2]], axis=1)
 
 
 def virial_to_stress(virial, volume):

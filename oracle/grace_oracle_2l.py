@@ -343,6 +343,15 @@ def _bond_force(dEdx, gY, G, rh, r, rc):
     return (dEdx / rc)[:, None] * rh + (gv - gr[:, None] * rh) / r[:, None]
 
 
+def _add_vatom(virials, bi, bj, rh, r, fv):
+    """add_vatom, libgrace/include/grace/fused_cpu.h:1075-1087: half of the bond's (x_i - x_j) (x) f_i to each of its atoms"""
+    dl = -rh * r[:, None]
+    v6 = 0.5 * np.stack([dl[:, 0] * fv[:, 0], dl[:, 1] * fv[:, 1], dl[:, 2] * fv[:, 2], dl[:, 0] * fv[:, 1], dl[:, 0] * fv[:, 2],
+                         dl[:, 1] * fv[:, 2]], axis=1)
+    np.add.at(virials, bi, v6)
+    np.add.at(virials, bj, v6)
+
+
 def _virial(rh, r, fv):
     dl = -rh * r[:, None]
     return np.array([(dl[:, 0] * fv[:, 0]).sum(), (dl[:, 1] * fv[:, 1]).sum(), (dl[:, 2] * fv[:, 2]).sum(),
@@ -366,6 +375,7 @@ def compute_2l(model: Model2L, mu, offset, j, rij, *, chunk=128, want_forces=Tru
     energies = np.zeros(n)
     forces = np.zeros((n, 3))
     virial = np.zeros(6)
+    virials = np.zeros((len(mu), 6))
 
     def bonds(a0, a1):
         b0, b1 = offset[a0], offset[a1]
@@ -443,6 +453,7 @@ def compute_2l(model: Model2L, mu, offset, j, rij, *, chunk=128, want_forces=Tru
         np.add.at(forces, bi, fv)
         np.add.at(forces, bj, -fv)
         virial += _virial(rh, r, fv)
+        _add_vatom(virials, bi, bj, rh, r, fv)                                         # src/fused_2l.cpp:778
     if want_forces:
         # ---- P5
         for (a0, a1), t in zip(chunks, state):
@@ -461,7 +472,8 @@ def compute_2l(model: Model2L, mu, offset, j, rij, *, chunk=128, want_forces=Tru
             np.add.at(forces, bi, fv)
             np.add.at(forces, bj, -fv)
             virial += _virial(rh, r, fv)
-    out = {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial}
+            _add_vatom(virials, bi, bj, rh, r, fv)                                     # src/fused_2l.cpp:539
+    out = {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial, "virials": virials}
     if uq:
         g, sg, cl = model.uq(mu, feats)
         out.update(gamma=g, atomic_sigma=sg, gmm_cluster=cl, uq_features=feats)

@@ -366,4 +366,13 @@ def compute_3l(model: Model3L, mu, offset, j, rij, *, want_forces=True, bond_chu
     out["forces"] = forces
     out["virial"] = np.array([(dl[:, 0] * g[:, 0]).sum(), (dl[:, 1] * g[:, 1]).sum(), (dl[:, 2] * g[:, 2]).sum(),
                               (dl[:, 0] * g[:, 1]).sum(), (dl[:, 0] * g[:, 2]).sum(), (dl[:, 1] * g[:, 2]).sum()])
+    # per-atom virials: half of each bond's (x_i - x_j) (x) f_i to each of its atoms (add_vatom, libgrace/include/grace/
+    # fused_cpu.h:1075-1087, called per layer in src/fused_3l.cpp:1424; the halves are linear in the bond force, so the
+    # total bond force g gives the sum over the layers)
+    v6 = 0.5 * np.stack([dl[:, 0] * g[:, 0], dl[:, 1] * g[:, 1], dl[:, 2] * g[:, 2], dl[:, 0] * g[:, 1], dl[:, 0] * g[:, 2],
+                         dl[:, 1] * g[:, 2]], axis=1)
+    virials = np.zeros((n, 6))
+    np.add.at(virials, bi[keep], v6)
+    np.add.at(virials, j_np[keep], v6)
+    out["virials"] = virials
     return out

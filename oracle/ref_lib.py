@@ -55,6 +55,8 @@ def _load():
     L.ref_cutoff.argtypes = [C.c_void_p, C.c_int, C.c_int]
     L.ref_compute.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 7 + [C.c_int, C.c_int] + [C.c_void_p] * 4
     L.ref_compute_uq.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 7 + [C.c_int] + [C.c_void_p] * 4
+    if hasattr(L, "ref_compute_vatom"):
+        L.ref_compute_vatom.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 4 + [C.c_int] + [C.c_void_p] * 4
     L.ref_close.argtypes = [C.c_void_p]
     L.ref_nl_build.restype = C.c_void_p
     L.ref_nl_build.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_double, C.c_int]
@@ -109,6 +111,20 @@ class RefModel:
         if rc:
             raise RuntimeError(self._L.ref_last_error().decode())
         return {"energy": e.value, "energies": eat, "forces": f, "virial": v}
+
+    def compute_vatom(self, types, offset, j, rij, nthreads=1):
+        """the call with ComputeFlags::vflag_atom: also virials [n, 6], the reference's Outputs::vatom"""
+        types = np.ascontiguousarray(types, dtype=np.int32)
+        offset = np.ascontiguousarray(offset, dtype=np.int64)
+        j = np.ascontiguousarray(j, dtype=np.int32)
+        rij = np.ascontiguousarray(rij, dtype=np.float64)
+        n = types.size
+        e = C.c_double(0.0)
+        f, v, va = np.zeros((n, 3)), np.zeros(6), np.zeros((n, 6))
+        rc = self._L.ref_compute_vatom(self._h, n, _p(types), _p(offset), _p(j), _p(rij), int(nthreads), C.addressof(e), _p(f), _p(v), _p(va))
+        if rc:
+            raise RuntimeError(self._L.ref_last_error().decode())
+        return {"energy": e.value, "forces": f, "virial": v, "virials": va}
 
     def compute_uq(self, types, offset, j, rij, nthreads=1):
         """GRACE-1L UQ head of the reference (forward only): energy, gamma, atomic_sigma, gmm_cluster per atom."""

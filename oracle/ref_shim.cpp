@@ -140,6 +140,40 @@ int ref_compute(void *hv, int n, const int *types, const int64_t *offset, const 
   }
 }
 
+// The same call with per-atom virials: vatom [n][6] is OVERWRITTEN (Outputs::vatom, ComputeFlags::vflag_atom).
+int ref_compute_vatom(void *hv, int n, const int *types, const int64_t *offset, const int *j, const double *rij, int nthreads, double *energy,
+                      double *f, double *virial, double *vatom)
+{
+  Ref *h = static_cast<Ref *>(hv);
+  try {
+    grace::CsrBonds src{types, offset, j, rij, nullptr, nullptr, nullptr};
+    grace::Outputs out;
+    std::memset(f, 0, sizeof(double) * 3 * (size_t) n);
+    std::memset(vatom, 0, sizeof(double) * 6 * (size_t) n);
+    std::vector<double *> rows((size_t) n);
+    for (int a = 0; a < n; a++) rows[(size_t) a] = vatom + 6 * (size_t) a;
+    out.f = f;
+    out.vatom = rows.data();
+    grace::ComputeFlags fl;
+    fl.virial = true;
+    fl.vflag_atom = true;
+    grace::NoExchange ex;
+    if (h->d1) h->d1->compute(n, nullptr, n, n, src, out, fl, nthreads);
+    else if (h->d2) h->d2->compute(n, nullptr, n, n, src, ex, out, fl, nthreads);
+    else if (h->d3) h->d3->compute(n, nullptr, n, n, src, ex, out, fl, nthreads);
+    else {
+      g_err = "setup_types not called";
+      return 1;
+    }
+    *energy = out.energy;
+    for (int k = 0; k < 6; k++) virial[k] = out.virial[k];
+    return 0;
+  } catch (const std::exception &e) {
+    g_err = e.what();
+    return 1;
+  }
+}
+
 // GRACE-1L / 2L / 3L with the UQ head (uqv6): forward only; gamma, sigma, cluster [n] per atom (Grace{1,2,3}LFused::enable_uq)
 int ref_compute_uq(void *hv, int n, const int *types, const int64_t *offset, const int *j, const double *rij, const double *x,
                    const int *image, const double *shifts, int nthreads, double *energy, double *gamma, double *sigma, double *cluster)

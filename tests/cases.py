@@ -218,6 +218,9 @@ E2E_CASES_2L = [("config3", "fcc108", None), ("l2mix", "alloy54", 5.5), ("l2mix"
 # reference fixture models (tests/golden/ref_fixtures) on the reference's fixture cells: goldens of the compiled reference
 E2E_CASES_3L = [("l3mix", "alloy54", 5.5), ("l3mix", "triclinic", None), ("l3mix", "slab", None), ("l3mix", "molecule", None),
                 ("l3wide", "fcc108", None), ("l3nat", "config1", None), ("l3el", "alloy54", None)]
+# cases with per-atom virials of the compiled reference among the goldens
+VATOM_CASES = [("mix2", "alloy54", 5.5), ("cut2", "slab", 6.0), ("l2mix", "triclinic", None), ("l2mix", "slab", None), ("l3mix", "alloy54", 5.5),
+               ("l3el", "alloy54", None)]
 UQ_CASES = [("uq2", "alloy54"), ("uq2", "triclinic"), ("uq2l", "alloy54"), ("uq2l", "triclinic"), ("uq3l", "alloy54"), ("uq3l", "triclinic")]
 FIXTURE_CASES_2L = [(m, c) for m in ("grace_2l_small", "grace_2l_l3", "legacy_2l_small", "legacy_2l_wide") for c in ("W54", "WMo54")]
 

@@ -58,6 +58,23 @@ def main():
         for k in ("energy", "energies", "forces", "virial"):
             out[f"{tag}/{k}"] = np.asarray(r[k])
         print(tag, key, "bonds", len(nl["j"]), "E", r["energy"], "max|F|", np.abs(r["forces"]).max())
+    # per-atom virials (ComputeFlags::vflag_atom) of a 1L, 2L and 3L case each, on the golden list of the structure
+    for model, struct, rc_list in cases.VATOM_CASES:
+        tag = f"e2e/{model}/{struct}"
+        if f"{tag}/virials" in out:
+            continue
+        path = cases.write_model(model, tmp)
+        nel = int(cases.MODELS[model]()["n_elements"][0])
+        ref = ref_lib.RefModel(path, list(range(nel)))
+        pos, cell, pbc, types = cases.STRUCTURES[struct]()
+        types = np.minimum(types, nel).astype(np.int32)
+        key = f"{struct}@{float(out[tag + '/rc_list']):g}"
+        nl = {k: out[f"nl/{key}/{k}"] for k in ("perm", "offset", "j", "image", "shifts")}
+        rij = cases.bond_vectors(pos, nl["perm"], nl["offset"], nl["j"], nl["image"], nl["shifts"])
+        r = ref.compute_vatom(types[nl["perm"]], nl["offset"], nl["j"], rij, nthreads=2)
+        assert abs(r["energy"] - float(out[tag + "/energy"])) < 1e-9 * max(1.0, abs(r["energy"]))
+        out[f"{tag}/virials"] = r["virials"]                     # rows in the order of the list (perm)
+        print(tag, "virials: sum - virial", np.abs(r["virials"].sum(0) - r["virial"]).max())
     # the reference's own 2L fixture models without TF goldens, on its fixture cells (CSR bonds as stored there)
     for model, cell in cases.FIXTURE_CASES_2L:
         if f"fixture/{model}/{cell}/energy" in out:

@@ -55,11 +55,12 @@ def device_call(eng, me, **kw):
     for i, r in enumerate(me["rows"]):
         nbh[i, :len(r)] = r
     f, ea = torch.zeros((nall, 3), dtype=torch.float64, device=dev), torch.zeros(nall, dtype=torch.float64, device=dev)
+    va = torch.zeros((nall, 6), dtype=torch.float64, device=dev)
     out = eng.compute_lammps_device(nl, torch.as_tensor(me["type"], device=dev), torch.as_tensor(me["x"], device=dev),
                                     torch.arange(nl, dtype=torch.int32, device=dev),
                                     torch.as_tensor(np.array([len(r) for r in me["rows"]], np.int32), device=dev),
-                                    torch.as_tensor(nbh, device=dev), owner=None, forces=f, eatom=ea, **kw)
-    out["forces"], out["energies"] = f.cpu().numpy(), ea.cpu().numpy()
+                                    torch.as_tensor(nbh, device=dev), owner=None, forces=f, eatom=ea, vatom=va, **kw)
+    out["forces"], out["energies"], out["vatom"] = f.cpu().numpy(), ea.cpu().numpy(), va.cpu().numpy()
     return out
 
 
@@ -68,7 +69,7 @@ def device_call(eng, me, **kw):
 def test_two_ranks_with_an_exchange_equal_one_engine(model_dir, model, rc, arrays):
     pos, cell, pbc, types = cases.structure_alloy54()
     m = kk.Model(cases.model_file(model_dir, model))
-    ref = kk.System(m, ["Mo", "W"], skin=0.0).compute(types, pos, cell, pbc, energies=True)
+    ref = kk.System(m, ["Mo", "W"], skin=0.0).compute(types, pos, cell, pbc, energies=True, virials=True)
     ranks, rank_of = two_ranks(pos, cell, pbc, types, rc)
     engines = [kk.Engine(m, ["Mo", "W"], 64) for _ in ranks]
     assert engines[0].comm_layers == {"l2mix": 1, "l3mix": 2, "mix2": 0}[model]
@@ -117,7 +118,7 @@ def test_two_ranks_with_an_exchange_equal_one_engine(model_dir, model, rc, array
                 out[r] = device_call(engines[r], me)
             else:
                 out[r] = engines[r].compute_lammps(me["nlocal"], me["type"], me["x"], np.arange(me["nlocal"], dtype=np.int32), numneigh,
-                                                   me["rows"], owner=None, energies=True)
+                                                   me["rows"], owner=None, energies=True, vatom=np.zeros((me["nall"], 6)))
         except Exception as e:      # noqa: BLE001
             err[r] = e
             barrier.abort()
@@ -132,18 +133,21 @@ def test_two_ranks_with_an_exchange_equal_one_engine(model_dir, model, rc, array
     want = [("f", k) for k in range(1, layers + 1)] + [("r", k) for k in range(layers, 0, -1)]
     assert calls[0] == want and calls[1] == want
     n = len(pos)
-    f, ea = np.zeros((n, 3)), np.zeros(n)
+    f, ea, va = np.zeros((n, 3)), np.zeros(n), np.zeros((n, 6))
     for r in (0, 1):
         me = ranks[r]
         f[me["owned"]] += out[r]["forces"][:me["nlocal"]]
         ea[me["owned"]] += out[r]["energies"][:me["nlocal"]]
-        for g, (atom, _) in enumerate(me["ghosts"]):            # LAMMPS' reverse communication of f
+        va[me["owned"]] += out[r]["vatom"][:me["nlocal"]]
+        for g, (atom, _) in enumerate(me["ghosts"]):            # LAMMPS' reverse communication of f (and of vatom)
             f[atom] += out[r]["forces"][me["nlocal"] + g]
+            va[atom] += out[r]["vatom"][me["nlocal"] + g]
     fs = max(1.0, np.abs(ref["forces"]).max())
     assert abs(out[0]["energy"] + out[1]["energy"] - ref["energy"]) / n < 1e-10 * fs
     assert np.abs(f - ref["forces"]).max() < 1e-9 * fs
     assert np.abs(ea - ref["energies"]).max() < 1e-10 * fs
     assert np.abs(out[0]["virial"] + out[1]["virial"] - ref["virial"]).max() < 1e-8 * fs
+    assert np.abs(va - ref["virials"]).max() < 1e-9 * max(1.0, np.abs(ref["virials"]).max())
 
 
 def test_device_row_movers_equal_the_host_forms(model_dir):
