@@ -490,6 +490,9 @@ template<class T> void Engine3L<T>::build_layer(int k)
     // the specialised straight-line kernels pay off (and compile in seconds) for the shorter term lists
     if (h.terms.size() <= 1500)
       jit_compile_product((c.name + "_cp").c_str(), h.terms, nfl, nfr, c.nfunc, false, P.rankP, sizeof(T) == 4, arch_, P.cp.jit, P.cp.jit_note);
+    else
+      jit_compile_blocked((c.name + "_cp").c_str(), h.terms, c.group_left, c.group_right, nfl, nfr, c.nfunc, P.rankP, sizeof(T) == 4, arch_, P.cp.jit,
+                          P.cp.jit_note);
     P.jit = P.cp.jit.ok();
     {
       std::vector<int> tl, tr, to;
