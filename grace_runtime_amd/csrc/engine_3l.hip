@@ -95,11 +95,12 @@ template<class T> struct DevContract {
 // sparse matrix in CSR form on the device (k_lincomb)
 struct DevCsr {
   DevBuf off, idx, rowof, val;
-  int nrow = 0, ncol = 0;
+  int nrow = 0, ncol = 0, rows = 8;    // rows: output rows per wave
   void build(int nrow_, int ncol_, const std::vector<int> &row, const std::vector<int> &col, const std::vector<double> &v)
   {
     nrow = nrow_;
     ncol = ncol_;
+    rows = lincomb_rows((int) row.size(), nrow_);
     std::vector<int> o(nrow + 1, 0), ix(row.size()), rw(row.size());
     std::vector<double> vv(row.size());
     for (int r : row) o[r + 1]++;
@@ -133,6 +134,7 @@ template<class T> struct ProdStage {
   CoupleDev cd{};
   int nfunc = 0, rankP = 0;
   bool jit = false;
+  bool jit_sets = false;    // the specialised reverse kernel writes every row of both adjoints: nothing to clear before it
 };
 
 template<class T> struct FcStage {
@@ -491,8 +493,8 @@ template<class T> void Engine3L<T>::build_layer(int k)
     if (h.terms.size() <= 1500)
       jit_compile_product((c.name + "_cp").c_str(), h.terms, nfl, nfr, c.nfunc, false, P.rankP, sizeof(T) == 4, arch_, P.cp.jit, P.cp.jit_note);
     else
-      jit_compile_blocked((c.name + "_cp").c_str(), h.terms, c.group_left, c.group_right, nfl, nfr, c.nfunc, P.rankP, sizeof(T) == 4, arch_, P.cp.jit,
-                          P.cp.jit_note);
+      P.jit_sets = jit_compile_blocked((c.name + "_cp").c_str(), h.terms, c.group_left, c.group_right, nfl, nfr, c.nfunc, P.rankP, sizeof(T) == 4,
+                                       arch_, P.cp.jit, P.cp.jit_note);
     P.jit = P.cp.jit.ok();
     {
       std::vector<int> tl, tr, to;
@@ -603,11 +605,11 @@ template<class T> void Engine3L<T>::couple_fwd(ProdStage<T> &p, const T *Lp, int
   hipLaunchKernelGGL(k_prod_fwd<T>, dim3(p.cp.d.nout * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, p.cp.d, Lp, Rp, out, n, KP, nfl, nfr);
 }
 
-// gL, gR are accumulated into (zeroed by the caller)
+// gL, gR are accumulated into (zeroed by the caller), or set when the stage says jit_sets
 template<class T> void Engine3L<T>::couple_bwd(ProdStage<T> &p, const T *Lp, int nfl, const T *Rp, int nfr, const T *g, T *gL, T *gR)
 {
   const int n = cn_, KP = p.rankP;
-  int one = 1, nat = n, acc = 1;
+  int one = 1, nat = n, acc = p.jit_sets ? 0 : 1;
   if (p.jit) {
     void *args[] = {(void *) &Lp, (void *) &Rp, (void *) &g, (void *) &gL, (void *) &gR, (void *) &acc, (void *) &acc, (void *) &nat, (void *) &one};
     const long long cols = (long long) n * KP;
@@ -706,9 +708,9 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw, bo
     });
     stage(tg(k, "couple_YI").c_str(), [&] {
       const int AT = 64 / L.CP;
-      hipLaunchKernelGGL(k_lincomb<T>, dim3((n + AT - 1) / AT, (L.nfA + 4 * kLincombRows - 1) / (4 * kLincombRows)), dim3(256), 0, stream_,
+      hipLaunchKernelGGL(k_lincomb<T>, dim3((n + AT - 1) / AT, (L.nfA + 4 * L.cg.rows - 1) / (4 * L.cg.rows)), dim3(256), 0, stream_,
                          L.cg.off.template as<int>(), L.cg.idx.template as<int>(), L.cg.rowof.template as<int>(), L.cg.val.template as<double>(),
-                         (const T *) pairP_.as<T>(), A_.as<T>(), npf, L.nfA, L.CP, n);
+                         (const T *) pairP_.as<T>(), A_.as<T>(), npf, L.nfA, L.CP, n, L.cg.rows);
     });
     stage(tg(k, "reduce_A").c_str(), [&] { cfwd_set(L.redA, A_.as<T>(), X); });
   }
@@ -856,8 +858,10 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
     const T *lp = Lp.buf.template as<T>(), *rp = Rp.buf.template as<T>();
     stage(tg(k, (std::string("reduce_") + name + "_bwd").c_str()).c_str(), [&] { cbwd_set(p.red, gR, gP); });
     stage(tg(k, (std::string("couple_") + name + "_bwd").c_str()).c_str(), [&] {
-      zero(gLp, Lp.bytes(nn, s));
-      zero(gRp, Rp.bytes(nn, s));
+      if (!p.jit_sets) {
+        zero(gLp, Lp.bytes(nn, s));
+        zero(gRp, Rp.bytes(nn, s));
+      }
       couple_bwd(p, lp, Lp.nf, rp, Rp.nf, gP, gLp, gRp);
     });
     stage(tg(k, (std::string("proj_") + name + "_bwd").c_str()).c_str(), [&] {
@@ -891,9 +895,9 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   stage(tg(k, "reduce_A_bwd").c_str(), [&] { cbwd_set(L.redA, gX, gA_.as<T>()); });
   stage(tg(k, "couple_YI_bwd").c_str(), [&] {
     const int AT = 64 / L.CP;
-    hipLaunchKernelGGL(k_lincomb<T>, dim3((n + AT - 1) / AT, (npf + 4 * kLincombRows - 1) / (4 * kLincombRows)), dim3(256), 0, stream_,
+    hipLaunchKernelGGL(k_lincomb<T>, dim3((n + AT - 1) / AT, (npf + 4 * L.cgt.rows - 1) / (4 * L.cgt.rows)), dim3(256), 0, stream_,
                        L.cgt.off.template as<int>(), L.cgt.idx.template as<int>(), L.cgt.rowof.template as<int>(), L.cgt.val.template as<double>(),
-                       (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP, n);
+                       (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP, n, L.cgt.rows);
   });
   const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
   stage(tg(k, "pair_bwd").c_str(), [&] {
