@@ -627,6 +627,8 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   gI2_.ensure(na * nrho_ * sizeof(double));
   T *P = P_.as<T>(), *B = B_.as<T>();
   const int pthreads = round_up(nslot_ * CRP_, 64);
+  // the pair kernels copy rows of CRP_ values and of noutp values to LDS 16 bytes at a time
+  if ((CRP_ * sizeof(T)) % 16 || (radR1_.noutp * sizeof(T)) % 16) throw Error("GRACE-2L: pair kernels need rows that are multiples of 16 bytes");
   if (forces) {
     gP_.ensure(na * npf * CRP_ * sizeof(T));
     gM_.ensure(nnodes * nI_ * CRP_ * sizeof(T));
@@ -649,6 +651,24 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     case 6: GR_PAIR1(K_, 36, __VA_ARGS__) break;             \
     default: GR_PAIR1(K_, 49, __VA_ARGS__) break;            \
   }
+// the reverse kernel with asynchronous staging and chunks of CH_ bonds
+#define GR_PAIR_ASYNC1(N_, CH_, grid_, block_, lds_, ...)                                                                \
+  {                                                                                                                      \
+    auto kern = k_pair_bwd_async<T, N_, CH_>;                                                                            \
+    if (lds_ > 48 * 1024)                                                                                                \
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_)); \
+    hipLaunchKernelGGL(kern, grid_, block_, lds_, __VA_ARGS__);                                                          \
+  }
+#define GR_PAIR_ASYNC(CH_, ...)                              \
+  switch (nl_) {                                             \
+    case 1: GR_PAIR_ASYNC1(1, CH_, __VA_ARGS__) break;       \
+    case 2: GR_PAIR_ASYNC1(4, CH_, __VA_ARGS__) break;       \
+    case 3: GR_PAIR_ASYNC1(9, CH_, __VA_ARGS__) break;       \
+    case 4: GR_PAIR_ASYNC1(16, CH_, __VA_ARGS__) break;      \
+    case 5: GR_PAIR_ASYNC1(25, CH_, __VA_ARGS__) break;      \
+    case 6: GR_PAIR_ASYNC1(36, CH_, __VA_ARGS__) break;      \
+    default: GR_PAIR_ASYNC1(49, CH_, __VA_ARGS__) break;     \
+  }
   for (int q = 0; q < nchunks; q++) {
     set_chunk(q);
     const int nc = cn_;
@@ -657,9 +677,9 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     T *R1 = moved_back(R1_.as<T>(), eb * radR1_.noutp), *dR1 = moved_back(dR1_.as<T>(), eb * radR1_.noutp);
     stage("radial_R1", [&] { radR1_.launch(stream_, ncu_, ones_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), R1, dR1, n_edges); });
     stage("pair_fwd", [&] {
-      const size_t lds = (size_t) kPairChunk * (nslot_ * CRP_ + radR1_.noutp) * sizeof(T);
-      GR_PAIR(k_pair_fwd, dim3(nc), dim3(nslot_ * CRP_), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) M, P, nslot_, CRP_,
-              nl_, radR1_.noutp, yw, sink_.as<T>(), 0, nc);
+      const size_t lds = (size_t) 2 * kAsyncChunkFwd * (pthreads + radR1_.noutp) * sizeof(T);
+      GR_PAIR(k_pair_fwd, dim3(nc), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) M, P, nslot_, CRP_,
+              nl_, radR1_.noutp, yw, sink_.as<T>(), 0, nc, nslot_);
     });
     stage("reduce_B", [&] { gemm(jB_, CRP_ / 16, C2P_ / 16, P, npf, B, nB_, 0); });
     chain_forward(c2_, "_L2", B);
@@ -691,12 +711,27 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     chain_backward(c2_, "_L2", B, [&] { stage("reduce_I2_bwd_X_XX", [&] { reduce_bwd(redI2_, c2_, gI2_.as<double>(), false); }); });
     stage("reduce_B_bwd", [&] { gemm(jBb_, C2P_ / 16, CRP_ / 16, c2_.gX.template as<T>(), nB_, gP_.as<T>(), npf, 0); });    // gP: every row is written
     stage("pair_bwd", [&] {
-      const size_t lds = (size_t) kPairChunk * (pthreads + 2 * radR1_.noutp) * sizeof(T);
-      GR_PAIR(k_pair_bwd, dim3(nc), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) dR1, (const T *) M,
-              (const T *) gP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(), scal_.as<double>() + 1,
-              nslot_, nI_, CRP_, nl_, radR1_.noutp, sink_.as<T>(), 1, sid_ptr(), nslot_, 0, nc, a0_, vatom_ptr());
+      // fp32: the next chunk is copied to a second LDS buffer while this one is worked on (chunks of 8 bonds in the large
+      // blocks that fill a CU alone, of 4 otherwise); fp64 runs faster with one chunk staged through registers
+      const size_t row = (size_t) (pthreads + 2 * radR1_.noutp) * sizeof(T);
+      const int ch = sizeof(T) != 4 ? 0 : (pthreads >= 512 && 16 * row <= kPairLdsMax) ? 8 : 8 * row <= kPairLdsMax ? 4 : 0;
+      const size_t lds = ch ? 2 * ch * row : kPairChunk * row;
+#define GR_ARGS                                                                                                                         \
+  dim3(nc), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) dR1, (const T *) M, (const T *) gP_.as<T>(),        \
+      rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(), scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, \
+      sink_.as<T>(), 1, sid_ptr(), nslot_, 0, nc, a0_, vatom_ptr()
+      if (ch == 8) {
+        GR_PAIR_ASYNC(8, GR_ARGS)
+      } else if (ch == 4) {
+        GR_PAIR_ASYNC(4, GR_ARGS)
+      } else {
+        GR_PAIR(k_pair_bwd, GR_ARGS)
+      }
+#undef GR_ARGS
     });
   }
+#undef GR_PAIR_ASYNC
+#undef GR_PAIR_ASYNC1
 #undef GR_PAIR
 #undef GR_PAIR1
   if (!forces) {

@@ -656,6 +656,24 @@ static int slots_per_block(int nslot, int CP)
     case 6: GR_PAIR1(K_, 36, __VA_ARGS__) break;             \
     default: GR_PAIR1(K_, 49, __VA_ARGS__) break;            \
   }
+// the reverse kernel with asynchronous staging and chunks of CH_ bonds
+#define GR_PAIR_ASYNC1(N_, CH_, grid_, block_, lds_, ...)                                                                \
+  {                                                                                                                      \
+    auto kern = k_pair_bwd_async<T, N_, CH_>;                                                                            \
+    if (lds_ > 48 * 1024)                                                                                                \
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_)); \
+    hipLaunchKernelGGL(kern, grid_, block_, lds_, __VA_ARGS__);                                                          \
+  }
+#define GR_PAIR_ASYNC(CH_, ...)                              \
+  switch (nl_) {                                             \
+    case 1: GR_PAIR_ASYNC1(1, CH_, __VA_ARGS__) break;       \
+    case 2: GR_PAIR_ASYNC1(4, CH_, __VA_ARGS__) break;       \
+    case 3: GR_PAIR_ASYNC1(9, CH_, __VA_ARGS__) break;       \
+    case 4: GR_PAIR_ASYNC1(16, CH_, __VA_ARGS__) break;      \
+    case 5: GR_PAIR_ASYNC1(25, CH_, __VA_ARGS__) break;      \
+    case 6: GR_PAIR_ASYNC1(36, CH_, __VA_ARGS__) break;      \
+    default: GR_PAIR_ASYNC1(49, CH_, __VA_ARGS__) break;     \
+  }
 
 // The message layer k gathers, for every atom and ghost: the normalised output of the layer below plus the species term
 // (once per layer, before the chunks of its forward pass and again before those of its reverse: M_ is shared scratch).
@@ -702,9 +720,12 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw, bo
     A_.ensure(na * L.nfA * L.CP * s);
     const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb;
     stage(tg(k, "pair_fwd").c_str(), [&] {
-      const size_t lds = (size_t) kPairChunk * (spb * L.CP + L.rad.noutp) * s;
-      GR_PAIR(k_pair_fwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(spb * L.CP), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl,
-              (const T *) M_.as<T>(), pairP_.as<T>(), L.nlmi, L.CP, nl_, L.rad.noutp, yw, sink_.as<T>(), ngrp, n);
+      const int pt = round_up(spb * L.CP, 64);
+      // rows of CP values and of noutp values go to LDS 16 bytes at a time
+      if ((L.CP * s) % 16 || (L.rad.noutp * s) % 16) throw Error("GRACE-3L: pair kernels need rows that are multiples of 16 bytes");
+      const size_t lds = (size_t) 2 * kAsyncChunkFwd * (pt + L.rad.noutp) * s;
+      GR_PAIR(k_pair_fwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pt), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl,
+              (const T *) M_.as<T>(), pairP_.as<T>(), L.nlmi, L.CP, nl_, L.rad.noutp, yw, sink_.as<T>(), ngrp, n, spb);
     });
     stage(tg(k, "couple_YI").c_str(), [&] {
       const int AT = 64 / L.CP;
@@ -901,10 +922,23 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   });
   const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
   stage(tg(k, "pair_bwd").c_str(), [&] {
-    const size_t lds = (size_t) kPairChunk * (pthreads + 2 * L.rad.noutp) * s;
-    GR_PAIR(k_pair_bwd, dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl,
-            (const T *) dRl, (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(),
-            f_.as<double>(), scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_, vatom_ptr());
+    // fp32: the next chunk is copied to a second LDS buffer while this one is worked on (chunks of 8 bonds in the large
+    // blocks that fill a CU alone, of 4 otherwise); fp64 runs faster with one chunk staged through registers
+    const size_t row = (size_t) (pthreads + 2 * L.rad.noutp) * s;
+    const int ch = s != 4 ? 0 : (pthreads >= 512 && 16 * row <= kPairLdsMax) ? 8 : 8 * row <= kPairLdsMax ? 4 : 0;
+    const size_t lds = ch ? 2 * ch * row : kPairChunk * row;
+#define GR_ARGS                                                                                                                          \
+  dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl, (const T *) dRl,     \
+      (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),   \
+      scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_, vatom_ptr()
+    if (ch == 8) {
+      GR_PAIR_ASYNC(8, GR_ARGS)
+    } else if (ch == 4) {
+      GR_PAIR_ASYNC(4, GR_ARGS)
+    } else {
+      GR_PAIR(k_pair_bwd, GR_ARGS)
+    }
+#undef GR_ARGS
   });
   (void) yw;
 }
@@ -1035,6 +1069,8 @@ template<class T> void Engine3L<T>::run(const RunFlags &fl)
   set_chunk(0);
 }
 
+#undef GR_PAIR_ASYNC
+#undef GR_PAIR_ASYNC1
 #undef GR_PAIR
 #undef GR_PAIR1
 

@@ -5,7 +5,7 @@
 //   k_pair_fwd     P[slot][lm][n] = sum_b Y_lm(b) R1_l(b)[n] M_jb[slot][n]: the neighbour gather of the messages
 //                  (slots 0 .. nI-1: the equivariant message I_j; slot nI: zB0, which gives B0)
 //                  (atom_yi / atom_scatter, libgrace/include/grace/fused_cpu.h:947-1025)
-//   k_pair_bwd     its reverse: per-bond force of layer 2, dE/dI_j added to the neighbour's row
+//   k_pair_bwd[_async]  its reverse: per-bond force of layer 2, dE/dI_j added to the neighbour's row
 //                  (bond_yi_bwd_g, bond_yi_commit, bond_scatter_bwd_t, bond_force: fused_cpu.h:836-942,1027-1050)
 //   k_energy_2l    readout with the two RMSNorms, fp64 (libgrace/src/fused_2l.cpp:548-615)
 //
@@ -80,7 +80,8 @@ template<class S, class D> __global__ void k_convert(const S *src, D *dst, long 
   if (q < count) dst[q] = (D) src[q];
 }
 
-constexpr int kPairChunk = 8;    // bonds staged in LDS at a time by the pair kernels
+constexpr int kPairChunk = 8;    // bonds staged in LDS at a time by the pair kernel that stages through registers
+constexpr size_t kPairLdsMax = 158 * 1024;    // dynamic LDS a pair kernel may ask for
 
 // Block -> (atom, slot group).  ngrp == 0: a (atoms, groups) grid.  ngrp > 0: a 1-d grid of 8 ceil(atoms / 8) ngrp
 // blocks laid out so that the groups of one atom are blocks b, b + 8, b + 16 ...: workgroups go to the 8 XCDs in turn,
@@ -126,52 +127,6 @@ __device__ inline T pair_stage(const int *__restrict__ ej, const T *__restrict__
 #pragma unroll
   for (int b = 0; b < kPairChunk; b++) Msh[b * NT + t] = mv[b];
   return touch;
-}
-
-// grid: (atoms, slot groups); block: spb * C threads, spb slots per block (slot = blockIdx.y * spb + t / C, n = t % C);
-// dynamic LDS: kPairChunk * (NT + nl * C) values.  NLM = nl * nl exactly.
-template<class T, int NLM>
-__global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ Y,
-                           const T *__restrict__ R1, const T *__restrict__ M, T *__restrict__ P, int nslot, int C, int nl, int noutp,
-                           int ystride, T *__restrict__ sink, int ngrp, int natoms)
-{
-  extern __shared__ __align__(16) unsigned char smem_raw[];
-  int i, grp;
-  if (!pair_block(ngrp, natoms, i, grp)) return;
-  const int t = threadIdx.x, NT = blockDim.x;
-  T *Msh = reinterpret_cast<T *>(smem_raw), *Rsh = Msh + kPairChunk * NT;
-  const int slot_raw = grp * (NT / C) + t / C, n = t % C;
-  const bool active = slot_raw < nslot;
-  const int slot = active ? slot_raw : 0;
-  const int nlm = nl * nl;
-  const long long e0 = eoff[i], e1 = eoff[i + 1];
-  T acc[NLM];
-#pragma unroll
-  for (int q = 0; q < NLM; q++) acc[q] = (T) 0;
-  T touch = (T) 0;
-  for (long long base = e0; base < e1; base += kPairChunk) {
-    const int nb = (int) (e1 - base < kPairChunk ? e1 - base : kPairChunk);
-    __syncthreads();
-    touch += pair_stage<T>(ej, M, R1, nullptr, Y, ystride, nlm, base, nb, nslot, C, noutp, active, slot, n, Msh, Rsh, nullptr, NT);
-    __syncthreads();
-    for (int b = 0; b < nb; b++) {
-      const T m = Msh[b * NT + t];
-      const T *r = Rsh + b * noutp + n;
-      const T *y = Y + (base + b) * ystride;
-#pragma unroll
-      for (int l = 0; l <= kKernMaxL; l++)
-        if (l * l < NLM) {
-          const T rm = r[l * C] * m;
-#pragma unroll
-          for (int mm = 0; mm < 2 * l + 1; mm++) acc[l * l + mm] += y[l * l + mm] * rm;
-        }
-    }
-  }
-  T *o = P + ((long long) i * nslot + slot) * nlm * C + n;
-#pragma unroll
-  for (int q = 0; q < NLM; q++)
-    if (active && q < nlm) o[(long long) q * C] = acc[q];
-  if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
 }
 
 // sums of 4 values per lane over the wave with 7 exchanges: afterwards lanes 0, 1, 2, 3 hold the totals of
@@ -285,6 +240,233 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
     }
   }
   // the finishing threads t < kPairChunk sit in wave 0
+  if (wave == 0) {
+    double vsum[9] = {fi[0], fi[1], fi[2], vir[0], vir[1], vir[2], vir[3], vir[4], vir[5]};
+#pragma unroll
+    for (int k = 0; k < 9; k++)
+      for (int o = 32; o > 0; o >>= 1) vsum[k] += __shfl_xor(vsum[k], o, 64);
+    if (lane == 0 && e1 > e0) {
+      for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) (a0 + i) + k], vsum[k]);
+      for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[a0 + i] : 0) + k], vsum[3 + k]);
+      if (vatom)
+        for (int k = 0; k < 6; k++) atomicAdd(&vatom[6 * (long long) (a0 + i) + k], 0.5 * vsum[3 + k]);
+    }
+  }
+  if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
+}
+
+// ---- the pair kernels with asynchronous staging
+// The chunk after the one being worked on is copied from global memory straight into a second LDS buffer while the
+// waves compute (global_load_lds: no registers, no wait until the end of the chunk), so the memory latency of the
+// neighbour rows no longer stands between two chunks.
+constexpr int kAsyncChunkFwd = 4;    // bonds per chunk of the gather; two chunks are resident
+
+__device__ inline void lds_load_word(const void *src, void *lds_wave_base)
+{
+  __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *) src, (void __attribute__((address_space(3))) *) lds_wave_base, 4, 0, 0);
+}
+
+// The waves of a block copy nbytes (a multiple of 16, both ends 16-byte aligned) from global memory to LDS: pieces of
+// 1 kB are dealt to the waves, a lane moves 16 bytes; the data lands at dst in the order it has at src.
+__device__ inline void block_copy_async(const void *src, void *dst, int nbytes, int wave, int nw, int lane)
+{
+  for (int p = wave; p * 1024 < nbytes; p += nw) {
+    const int q = p * 64 + lane;
+    if (q * 16 < nbytes)
+      __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *) (reinterpret_cast<const char *>(src) + 16 * (size_t) q),
+                                       (void __attribute__((address_space(3))) *) (reinterpret_cast<char *>(dst) + 1024 * (size_t) p), 16, 0, 0);
+  }
+}
+
+__device__ inline void wait_async_loads() { __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// The neighbour gather: spb slots per block, spb C threads rounded up to whole waves (a copy is the work
+// of all 64 lanes of a wave).  dynamic LDS: 2 kAsyncChunkFwd (NT + noutp) values.
+template<class T, int NLM>
+__global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ Y,
+                           const T *__restrict__ R1, const T *__restrict__ M, T *__restrict__ P, int nslot, int C, int nl, int noutp,
+                           int ystride, T *__restrict__ sink, int ngrp, int natoms, int spb)
+{
+  constexpr int CH = kAsyncChunkFwd;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  int i, grp;
+  if (!pair_block(ngrp, natoms, i, grp)) return;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, NT = blockDim.x, nw = NT >> 6;
+  T *Msh = reinterpret_cast<T *>(smem_raw), *Rsh = Msh + 2 * CH * NT;
+  const int slot_raw = grp * spb + t / C, n = t % C;
+  const bool active = t < spb * C && slot_raw < nslot;
+  const int slot = active ? slot_raw : 0;
+  const int nlm = nl * nl;
+  const int nact = (nslot - grp * spb < spb ? nslot - grp * spb : spb) * C;
+  const long long e0 = eoff[i], e1 = eoff[i + 1];
+  const int nchunk = (int) ((e1 - e0 + CH - 1) / CH);
+  T acc[NLM];
+#pragma unroll
+  for (int q = 0; q < NLM; q++) acc[q] = (T) 0;
+  for (int q = t; q < 2 * CH * NT; q += NT) Msh[q] = (T) 0;
+  __syncthreads();
+  auto stage = [&](int c) {
+    const long long base = e0 + (long long) c * CH;
+    const int nb = (int) (e1 - base < CH ? e1 - base : CH), buf = c & 1;
+    // the rows of the block's slots are contiguous in M_j and in the buffer: nact values per bond
+    for (int b = 0; b < nb; b++)
+      block_copy_async(M + ((long long) ej[base + b] * nslot + grp * spb) * C, Msh + (size_t) (buf * CH + b) * NT, nact * (int) sizeof(T), (wave + b) % nw,
+                       nw, lane);
+    block_copy_async(R1 + base * noutp, Rsh + (size_t) buf * CH * noutp, nb * noutp * (int) sizeof(T), wave, nw, lane);
+  };
+  T touch = (T) 0;
+  // round c stages chunk c + 1 and works on chunk c (round -1 only stages)
+  for (int c = -1; c < nchunk; c++) {
+    const long long base = e0 + (long long) c * CH;
+    const int nb = c < 0 ? 0 : (int) (e1 - base < CH ? e1 - base : CH), buf = c & 1;
+    T tv = (T) 0;
+    if (c + 1 < nchunk) {
+      stage(c + 1);
+      const long long nbase = base + CH;
+      const int nnb = (int) (e1 - nbase < CH ? e1 - nbase : CH), per = (nlm + 7) / 8;
+      if (t < nnb * per) tv = Y[(nbase + t / per) * ystride + (t % per) * 8];
+    }
+    for (int b = 0; b < nb; b++) {
+      const T m = Msh[(size_t) (buf * CH + b) * NT + t];
+      const T *r = Rsh + (size_t) (buf * CH + b) * noutp + n;
+      const T *y = Y + (base + b) * ystride;
+#pragma unroll
+      for (int l = 0; l <= kKernMaxL; l++)
+        if (l * l < NLM) {
+          const T rm = r[l * C] * m;
+#pragma unroll
+          for (int mm = 0; mm < 2 * l + 1; mm++) acc[l * l + mm] += y[l * l + mm] * rm;
+        }
+    }
+    touch += tv;
+    wait_async_loads();
+    __syncthreads();
+  }
+  T *o = P + ((long long) i * nslot + slot) * nlm * C + n;
+#pragma unroll
+  for (int q = 0; q < NLM; q++)
+    if (active && q < nlm) o[(long long) q * C] = acc[q];
+  if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
+}
+
+// k_pair_bwd with asynchronous staging and chunks of CH bonds; same arguments, grid and block.
+// dynamic LDS: 2 CH (NT + 2 noutp) values.
+template<class T, int NLM, int CH>
+__global__ void k_pair_bwd_async(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ YG,
+                                 const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
+                                 const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
+                                 T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
+                                 int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms, int a0,
+                                 double *__restrict__ vatom)
+{
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  __shared__ double bsum[2][CH][4];
+  __shared__ __align__(16) double g_rh[2][CH * 3], g_r[2][CH], g_rc[2][CH];
+  __shared__ __align__(16) int g_j[2][CH];
+  int i, grp;
+  if (!pair_block(ngrp, natoms, i, grp)) return;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, NT = blockDim.x, nw = NT >> 6;
+  T *Msh = reinterpret_cast<T *>(smem_raw), *Rsh = Msh + 2 * CH * NT, *dRsh = Rsh + 2 * CH * noutp;
+  const int slot_raw = grp * spb + t / C;
+  const bool active = t < spb * C && slot_raw < nslot;
+  const int slot = active ? slot_raw : 0, n = t % C;
+  const int nlm = nl * nl;
+  // threads of the block with a slot: the first nact (slots grp spb .. of the atom's rows, C values each)
+  const int nact = (nslot - grp * spb < spb ? nslot - grp * spb : spb) * C;
+  const long long e0 = eoff[i], e1 = eoff[i + 1];
+  const int nchunk = (int) ((e1 - e0 + CH - 1) / CH);
+  T g[NLM];
+  {
+    const T *gp = gP + ((long long) i * nslot + slot) * nlm * C + n;
+#pragma unroll
+    for (int q = 0; q < NLM; q++) g[q] = (active && q < nlm) ? gp[(long long) q * C] : (T) 0;
+  }
+  for (int q = t; q < 2 * CH * NT; q += NT) Msh[q] = (T) 0;
+  if (t < 2 * CH * 4) (&bsum[0][0][0])[t] = 0.0;
+  __syncthreads();
+  // stage(c): everything chunk c needs, into buffer c & 1
+  auto stage = [&](int c) {
+    const long long base = e0 + (long long) c * CH;
+    const int nb = (int) (e1 - base < CH ? e1 - base : CH), buf = c & 1;
+    // the rows of the block's slots are contiguous in M_j and in the buffer: nact values per bond
+    for (int b = 0; b < nb; b++)
+      block_copy_async(M + ((long long) ej[base + b] * nslot + grp * spb) * C, Msh + (size_t) (buf * CH + b) * NT, nact * (int) sizeof(T), (wave + b) % nw,
+                       nw, lane);
+    block_copy_async(R1 + base * noutp, Rsh + (size_t) buf * CH * noutp, nb * noutp * (int) sizeof(T), (wave + 1) % nw, nw, lane);
+    block_copy_async(dR1 + base * noutp, dRsh + (size_t) buf * CH * noutp, nb * noutp * (int) sizeof(T), (wave + 2) % nw, nw, lane);
+    if (wave == 0) {
+      if (lane < nb * 6) lds_load_word(reinterpret_cast<const char *>(rh + 3 * base) + 4 * lane, &g_rh[buf][0]);
+      if (lane < nb * 2) lds_load_word(reinterpret_cast<const char *>(rlen + base) + 4 * lane, &g_r[buf][0]);
+      if (lane < nb * 2) lds_load_word(reinterpret_cast<const char *>(rcut + base) + 4 * lane, &g_rc[buf][0]);
+      if (lane < nb) lds_load_word(reinterpret_cast<const char *>(ej + base) + 4 * lane, &g_j[buf][0]);
+    }
+  };
+  double fi[3] = {0, 0, 0}, vir[6] = {0, 0, 0, 0, 0, 0};
+  T touch = (T) 0;
+  // round c stages chunk c + 1 and works on chunk c (round -1 only stages)
+  for (int c = -1; c < nchunk; c++) {
+    const long long base = e0 + (long long) c * CH;
+    const int nb = c < 0 ? 0 : (int) (e1 - base < CH ? e1 - base : CH), buf = c & 1;
+    T tv = (T) 0;
+    if (c + 1 < nchunk) {
+      stage(c + 1);
+      // the harmonics of the next chunk, one 64-byte piece per thread, so that its uniform reads find them in the L2
+      const long long nbase = base + CH;
+      const int nnb = (int) (e1 - nbase < CH ? e1 - nbase : CH), per = (nlm * 3 + 7) / 8;
+      if (t < nnb * per) tv = YG[(nbase + t / per) * nlm * 3 + (t % per) * 8];
+    }
+    for (int b = 0; b < nb; b++) {
+      const long long e = base + b;
+      const T m = Msh[(size_t) (buf * CH + b) * NT + t];
+      const T *r = Rsh + (size_t) (buf * CH + b) * noutp + n, *dr = dRsh + (size_t) (buf * CH + b) * noutp + n;
+      const T *yg = YG + e * nlm * 3;
+      T sI = (T) 0, dE = (T) 0, t1 = (T) 0, t2 = (T) 0;
+#pragma unroll
+      for (int l = 0; l <= kKernMaxL; l++)
+        if (l * l < NLM) for (int it = 0; it < one; it++) {
+          T S = (T) 0, a1 = (T) 0, a2 = (T) 0;
+#pragma unroll
+          for (int mm = 0; mm < 2 * l + 1; mm++) {
+            const T gv = g[l * l + mm];
+            S += yg[l * l + mm] * gv; a1 += yg[nlm + l * l + mm] * gv; a2 += yg[2 * nlm + l * l + mm] * gv;
+          }
+          const T rl = r[l * C], drl = dr[l * C];
+          sI += rl * S;
+          dE += drl * S;
+          t1 += rl * a1; t2 += rl * a2;
+        }
+      if (active && slot < nI) atomicAdd(&gM[((long long) g_j[buf][b] * nI + slot) * C + n], sI);
+      const double cs = wave_sum4((double) (dE * m), (double) (t1 * m), (double) (t2 * m), 0.0, lane);
+      if (lane < 3) atomicAdd(&bsum[buf][b][lane], cs);    // lanes 0..2: dE/dx, g . e2, g . e1  (order v0, v2, v1, v3)
+    }
+    touch += tv;
+    wait_async_loads();
+    __syncthreads();
+    // the forces of the chunk: threads 0 .. nb - 1 while the other waves go on; bsum[buf] is clear again before the
+    // chunk after the next adds to it (a barrier lies between)
+    if (t < nb) {
+      const double *u = &g_rh[buf][3 * t];
+      const double r = g_r[buf][t], rc = g_rc[buf][t];
+      const double dEdr = bsum[buf][t][0] / rc, g1 = bsum[buf][t][2] / r, g2 = bsum[buf][t][1] / r;
+      bsum[buf][t][0] = bsum[buf][t][1] = bsum[buf][t][2] = 0.0;
+      double e1v[3], e2v[3], fv[3];
+      tangent_basis(u, e1v, e2v);
+      for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + g1 * e1v[d] + g2 * e2v[d];
+      const int jj = g_j[buf][t];
+      for (int d = 0; d < 3; d++) {
+        fi[d] += fv[d];
+        atomicAdd(&f[3 * (long long) jj + d], -fv[d]);
+      }
+      const double ddx = -u[0] * r, ddy = -u[1] * r, ddz = -u[2] * r;
+      vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
+      vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
+      if (vatom) {    // per-atom virial: the neighbour's half of this bond (fused_cpu.h:1075-1087 of the reference)
+        double *vj = vatom + 6 * (long long) jj;
+        atomicAdd(vj, 0.5 * ddx * fv[0]); atomicAdd(vj + 1, 0.5 * ddy * fv[1]); atomicAdd(vj + 2, 0.5 * ddz * fv[2]);
+        atomicAdd(vj + 3, 0.5 * ddx * fv[1]); atomicAdd(vj + 4, 0.5 * ddx * fv[2]); atomicAdd(vj + 5, 0.5 * ddy * fv[2]);
+      }
+    }
+  }
   if (wave == 0) {
     double vsum[9] = {fi[0], fi[1], fi[2], vir[0], vir[1], vir[2], vir[3], vir[4], vir[5]};
 #pragma unroll
