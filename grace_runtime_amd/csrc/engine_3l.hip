@@ -729,9 +729,10 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw, bo
     });
     stage(tg(k, "couple_YI").c_str(), [&] {
       const int AT = 64 / L.CP;
-      hipLaunchKernelGGL(k_lincomb<T>, dim3((n + AT - 1) / AT, (L.nfA + 4 * L.cg.rows - 1) / (4 * L.cg.rows)), dim3(256), 0, stream_,
+      const int ngrp = (L.nfA + 4 * L.cg.rows - 1) / (4 * L.cg.rows);
+      hipLaunchKernelGGL(k_lincomb<T>, dim3((unsigned) (((n + AT - 1) / AT + 7) / 8 * 8 * ngrp)), dim3(256), 0, stream_,
                          L.cg.off.template as<int>(), L.cg.idx.template as<int>(), L.cg.rowof.template as<int>(), L.cg.val.template as<double>(),
-                         (const T *) pairP_.as<T>(), A_.as<T>(), npf, L.nfA, L.CP, n, L.cg.rows);
+                         (const T *) pairP_.as<T>(), A_.as<T>(), npf, L.nfA, L.CP, n, L.cg.rows, ngrp);
     });
     stage(tg(k, "reduce_A").c_str(), [&] { cfwd_set(L.redA, A_.as<T>(), X); });
   }
@@ -916,9 +917,10 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   stage(tg(k, "reduce_A_bwd").c_str(), [&] { cbwd_set(L.redA, gX, gA_.as<T>()); });
   stage(tg(k, "couple_YI_bwd").c_str(), [&] {
     const int AT = 64 / L.CP;
-    hipLaunchKernelGGL(k_lincomb<T>, dim3((n + AT - 1) / AT, (npf + 4 * L.cgt.rows - 1) / (4 * L.cgt.rows)), dim3(256), 0, stream_,
+    const int ngrp = (npf + 4 * L.cgt.rows - 1) / (4 * L.cgt.rows);
+    hipLaunchKernelGGL(k_lincomb<T>, dim3((unsigned) (((n + AT - 1) / AT + 7) / 8 * 8 * ngrp)), dim3(256), 0, stream_,
                        L.cgt.off.template as<int>(), L.cgt.idx.template as<int>(), L.cgt.rowof.template as<int>(), L.cgt.val.template as<double>(),
-                       (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP, n, L.cgt.rows);
+                       (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP, n, L.cgt.rows, ngrp);
   });
   const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
   stage(tg(k, "pair_bwd").c_str(), [&] {

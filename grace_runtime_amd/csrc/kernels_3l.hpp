@@ -44,7 +44,9 @@ __global__ void k_message(const T *I, const int *mu, const T *zproj, const T *ma
 // row: terms [off[f], off[f + 1]), row[t] = f.  A wave spans the channels of AT = 64 / C atoms and takes `rows`
 // consecutive output rows (lincomb_rows: about 64 terms per wave); it reads its terms 64 at a time, one per lane, and
 // walks them with lane reads, the source rows of 8 terms requested before the first is used.
-// grid: (ceil(atoms / AT), ceil(nout / (4 rows))); block 256.
+// grid: 8 ceil(ceil(atoms / AT) / 8) ngrp blocks, ngrp = ceil(nout / (4 rows)), in the order of pair_block: the row groups
+// of one atom run on one XCD shortly after each other, so a source row that several groups read comes from HBM once.
+// block 256.
 inline int lincomb_rows(int nterms, int nout)
 {
   const int per = nout > 0 ? (nterms + nout - 1) / nout : 1;
@@ -55,12 +57,14 @@ inline int lincomb_rows(int nterms, int nout)
 template<class T>
 __global__ __launch_bounds__(256) void k_lincomb(const int *__restrict__ off, const int *__restrict__ idx, const int *__restrict__ row,
                                                  const double *__restrict__ val, const T *__restrict__ in, T *__restrict__ out, int nin, int nout,
-                                                 int C, int natoms, int rows)
+                                                 int C, int natoms, int rows, int ngrp)
 {
   const int AT = 64 / C, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int a0 = blockIdx.x * AT, sub = lane / C, n = lane % C;
+  int ab, grp;
+  if (!pair_block(ngrp, (natoms + AT - 1) / AT, ab, grp)) return;
+  const int a0 = ab * AT, sub = lane / C, n = lane % C;
   const bool live = a0 + sub < natoms;
-  const int r0 = (blockIdx.y * 4 + wave) * rows, r1 = r0 + rows < nout ? r0 + rows : nout;
+  const int r0 = (grp * 4 + wave) * rows, r1 = r0 + rows < nout ? r0 + rows : nout;
   if (r0 >= nout) return;
   const T *src = in + (long long) (a0 + (live ? sub : 0)) * nin * C + n;
   T *dst = out + (long long) (a0 + (live ? sub : 0)) * nout * C + n;
