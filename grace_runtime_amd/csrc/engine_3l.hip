@@ -489,8 +489,15 @@ template<class T> void Engine3L<T>::build_layer(int k)
     P.rankP = P.U.kout;
     const HostProd h = grhip::build_prod(c.cg, std::vector<char>(c.nfunc, 1), nfl, nfr);
     P.cp.build(h);
-    // the specialised straight-line kernels pay off (and compile in seconds) for the shorter term lists
-    if (h.terms.size() <= 1500)
+    // The shorter term lists run with the operands of both sides in registers (that generator writes only outputs with
+    // terms, so it needs a list that feeds every output), the longer ones block by block.
+    bool every_output = true;
+    {
+      std::vector<char> fed(c.nfunc, 0);
+      for (const ProdTerm &t : h.terms) fed[t.o] = 1;
+      for (char x : fed) every_output = every_output && x;
+    }
+    if (h.terms.size() <= 1500 && every_output)
       jit_compile_product((c.name + "_cp").c_str(), h.terms, nfl, nfr, c.nfunc, false, P.rankP, sizeof(T) == 4, arch_, P.cp.jit, P.cp.jit_note);
     else
       P.jit_sets = jit_compile_blocked((c.name + "_cp").c_str(), h.terms, c.group_left, c.group_right, nfl, nfr, c.nfunc, P.rankP, sizeof(T) == 4,
