@@ -51,7 +51,7 @@ DENSE_TRAFFIC = {"config2": 6.5e9}
 DENSE_PREFIXES = ("fc_", "prod_", "reduce_", "energy_mlp", "zero_grads", "chain_")
 
 
-def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4, radial_flops=59392.0, slots=None):
+def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4, radial_flops=59392.0, slots=None, stream_bytes=None):
     """Roofline entry of one stage: algorithmic work / measured time."""
     base = name.rsplit("_L", 1)[0] if slots else name     # GRACE-3L stages carry their layer: pair_fwd_L2, radial_L1 ...
     if slots and base in ("pair_fwd", "pair_bwd"):
@@ -83,7 +83,28 @@ def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4,
     if name in dense_flops:
         fl = dense_flops[name]
         return {"bound": "mfma", "achieved": fl / (ms * 1e-3) / 1e12, "peak": PEAK[prec], "unit": "TFLOP/s", "work": fl}
+    if stream_bytes and name in stream_bytes:
+        by = stream_bytes[name]
+        return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
     return None
+
+
+def couple_stream_bytes(md, N, s):
+    """Algorithmic bytes of the cp_l couples and of the sparse Clebsch-Gordan map of a GRACE-3L model, per stage name:
+    every operand row, output row and adjoint row once (forward: both projections in, the product out; reverse: the
+    projections and the product's adjoint in, both projection adjoints out)."""
+    out = {}
+    for layer in (1, 2, 3):
+        for q in ("2", "3", "4"):
+            P = f"A{layer}_{q}"
+            nfl, nfr, nout, rank = len(md[P + "_group_left"]), len(md[P + "_group_right"]), int(md[P + "_nfunc"][0]), int(md[P + "_rank"][0])
+            out[f"couple_{q}_L{layer}"] = N * rank * s * (nfl + nfr + nout)
+            out[f"couple_{q}_bwd_L{layer}"] = N * rank * s * (nfl + nfr + nout + nfl + nfr)
+        if layer > 1:
+            npair, nfa = md[f"A{layer}_cg_W"].shape
+            width = int(md[f"A{layer}_n_rad_max"][0])
+            out[f"couple_YI_L{layer}"] = out[f"couple_YI_bwd_L{layer}"] = N * width * s * (npair + nfa)
+    return out
 
 
 def main():
@@ -236,7 +257,8 @@ def main():
 
     C, nl, nlm, s = (64, 6, 36, a.precision // 8) if three else (32, 5, 25, a.precision // 8)
     # GRACE-3L: message functions gathered by the pair kernels of layers 2 and 3; radial MLP 8-128-128-384, value + tangent
-    extra = dict(radial_flops=4.0 * (8 * 128 + 128 * 128 + 128 * 384), slots={"2": 36, "3": 72}) if three else {}
+    extra = dict(radial_flops=4.0 * (8 * 128 + 128 * 128 + 128 * 384), slots={"2": 36, "3": 72},
+                 stream_bytes=couple_stream_bytes(workloads.model_config4(), N, s)) if three else {}
     # FC / reduce tile GEMMs: flops of the live functions as the engine counts them
     dense_flops = dict(gemm_flops)
     roof = {}
