@@ -445,7 +445,7 @@ template<class T> struct DevRadial {
     for (int q = 0; q < 16; q++) ra.drow[q] = drow[q];
     ra.emi = emi; ra.bias_i = bias_i.as<T>(); ra.bias_j = bias_j.as<T>(); ra.bias1 = bias1.as<T>();
     if (mode == 1 && !emi) throw Error("radial kernel: the species form needs the central element of every edge");
-    const int threads = hb == 4 ? 512 : 256;
+    const int threads = radial_threads(hb, mode, w2_in_lds != 0);
     // <T, 16-row blocks of the hidden width, activation, species form, layer-2 weights in LDS>
     void (*kern)(RadialArgs<T>);
     if (w2_in_lds)

@@ -399,7 +399,11 @@ __device__ inline double ipow(double x, int n)
 // Every k-step feeds all row blocks of the value and the tangent stream (2 HB independent accumulator chains).
 // ACT: 0 SiLU, 1 tanh (compile-time: the fp64 tanh is large, and both activations inlined 32 times overflow the
 // instruction cache).
-template<class T, int HB, int ACT, int MODE, bool W2L> __global__ __launch_bounds__(HB <= 4 ? 512 : 256) void k_radial(RadialArgs<T> a)
+// Threads of a block: hidden width 64 with every weight in LDS runs three waves per SIMD (168 registers; two waves at 180
+// were 2 % slower in fp64, 6 % in fp32), the other forms would spill at that size; width 128 runs one wave per SIMD.
+constexpr int radial_threads(int hb, int mode, bool w2l) { return hb <= 4 ? (w2l && mode == 0 ? 768 : 512) : 256; }
+
+template<class T, int HB, int ACT, int MODE, bool W2L> __global__ __launch_bounds__((radial_threads(HB, MODE, W2L))) void k_radial(RadialArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
   extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -539,15 +543,16 @@ template<class T, int HB, int ACT, int MODE, bool W2L> __global__ __launch_bound
     // single dependent accumulator chain keeps the matrix pipe full, and one block's weights are all that is in flight)
     // The z values of a column block are requested one block ahead and the inputs of the next tile before the first
     // store of this one: no load is issued behind a store whose completion it would then wait for.
-    const T *zrow[4];
-    long long row_v[4];
+    // rows of the tile as 32-bit offsets from its first row (the tile is wave-uniform), -1: no such edge
+    T *const Rt = a.Rz + (a.e_begin + tile * 16) * a.noutp, *const dRt = a.dRz + (a.e_begin + tile * 16) * a.noutp;
+    int zrow[4], row_v[4];
     T env_v[4], denv_v[4], zc[4];
 #pragma unroll
     for (int v = 0; v < 4; v++) {
-      const long long el = tile * 16 + a.drow[g * 4 + v];
-      row_v[v] = el < cnt ? (a.e_begin + el) * a.noutp : -1;
-      zrow[v] = a.z + emu_n[v] * a.C + c;
-      zc[v] = zrow[v][0];
+      const int rl = a.drow[g * 4 + v];
+      row_v[v] = tile * 16 + rl < cnt ? rl * a.noutp : -1;
+      zrow[v] = emu_n[v] * a.C + c;
+      zc[v] = a.z[zrow[v]];
       if (MODE == 1) {
         const double xpm = ipow(xv[v], p - 1), xp = xpm * xv[v], xp1 = xp * xv[v], xp2 = xp1 * xv[v];
         env_v[v] = (T) (1.0 - cf0 * xp + cf1 * xp1 - cf2 * xp2);
@@ -569,7 +574,7 @@ template<class T, int HB, int ACT, int MODE, bool W2L> __global__ __launch_bound
       T zn[4];
       const int kn = ((cb + 1) & (KZ - 1)) * 16;       // column n = c + 16 k of z in the next block
 #pragma unroll
-      for (int v = 0; v < 4; v++) zn[v] = zrow[v][kn];
+      for (int v = 0; v < 4; v++) zn[v] = a.z[zrow[v] + kn];
       v4 acc = {0, 0, 0, 0}, dacc = {0, 0, 0, 0};
       const T *wc = wl + (long long) cb * NQ * 64;
 #pragma unroll
@@ -586,11 +591,11 @@ template<class T, int HB, int ACT, int MODE, bool W2L> __global__ __launch_bound
       for (int v = 0; v < 4; v++) {
         if (row_v[v] >= 0) {
           if (MODE == 1) {
-            a.Rz[row_v[v] + col] = acc[v] * env_v[v] * zc[v];
-            a.dRz[row_v[v] + col] = (dacc[v] * env_v[v] + acc[v] * denv_v[v]) * zc[v];
+            Rt[row_v[v] + col] = acc[v] * env_v[v] * zc[v];
+            dRt[row_v[v] + col] = (dacc[v] * env_v[v] + acc[v] * denv_v[v]) * zc[v];
           } else {
-            a.Rz[row_v[v] + col] = acc[v] * zc[v];
-            a.dRz[row_v[v] + col] = dacc[v] * zc[v];
+            Rt[row_v[v] + col] = acc[v] * zc[v];
+            dRt[row_v[v] + col] = dacc[v] * zc[v];
           }
         }
         zc[v] = zn[v];
