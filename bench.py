@@ -244,6 +244,19 @@ def main():
             del sysm
     upload()
 
+    # the same passes with ordered (atomic-free) sums of forces, virial and energy (GRACE-1L engines): reported beside
+    ordered_ms = None
+    if not (two or three or batch):
+        eng.set_ordered_sums(True)
+        eng.run()
+        eng.sync()
+        t1 = time.perf_counter()
+        for _ in range(a.steps):
+            eng.run()
+        eng.sync()
+        ordered_ms = (time.perf_counter() - t1) / a.steps * 1e3
+        eng.set_ordered_sums(False)
+
     # per-stage durations: HIP events around every launch on the engine's stream, averaged over the same K steps
     eng.set_profile(True)
     acc = {}
@@ -346,6 +359,7 @@ def main():
         "ms_per_call_host_buffers": round(host_ms, 3) if host_ms is not None else None,
         "ms_per_calculator_call": batch_ms if batch else {"neighbour_list_rebuilt": round(list_ms["rebuilt"], 3),
                                                           "neighbour_list_kept": round(list_ms["kept"], 3)},
+        "ms_per_step_ordered_sums": round(ordered_ms, 4) if ordered_ms is not None else None,
         "engine_create_s": round(create_s, 3),
         "chunksize": eng.chunksize,              # atoms per engine pass the timed steps ran with (0: the whole structure in one pass)
         "device_memory_GB": round(mem_gb, 3),

@@ -37,6 +37,7 @@ struct gr_engine {
   bool has_exchange = false;                           // an exchange is installed: ghosts of the LAMMPS call stay atoms of their own
   grhip::ExchangeCallbacks exchange;                   // kept for the engine a reset makes
   int chunk_request = -1;                              // the caller's chunk size, kept for the engine a reset makes
+  bool ordered = false;                                // ordered sums requested, kept for the engine a reset makes
   std::vector<int> lmp_rows;                           // gr_compute_lammps: LAMMPS index of engine row q (empty: rows are LAMMPS indices)
   int lmp_nall = -1;                                   // atoms of the last gr_compute_lammps[_device] call
   uint64_t lmp_serial = 0;                             // the engine's upload count at that call: its list is still the one held
@@ -56,6 +57,7 @@ struct gr_engine {
     make();
     if (has_exchange) eng->set_exchange(exchange);
     eng->set_chunksize(chunk_request);
+    if (ordered) eng->set_ordered_sums(true);
   }
   std::vector<grhip::StageTime> times;
   std::unique_ptr<grhip::BatchDeviceNeighbors> bnl;    // lists of gr_compute_batch_device (buffers kept between calls)
@@ -1064,6 +1066,16 @@ int gr_engine_set_chunksize(gr_engine *e, int atoms)
 }
 
 int gr_engine_chunksize(const gr_engine *e) { return e && e->eng ? e->eng->chunksize_used() : 0; }
+
+int gr_engine_set_ordered_sums(gr_engine *e, int on)
+{
+  return guarded([&] {
+    live(e).set_ordered_sums(on != 0);
+    e->ordered = on != 0;
+  });
+}
+
+int gr_engine_ordered_sums(const gr_engine *e) { return e && e->eng && e->eng->ordered_sums() ? 1 : 0; }
 
 int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *cluster)
 {

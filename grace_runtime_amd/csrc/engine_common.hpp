@@ -575,6 +575,11 @@ class EngineBase : public Engine, protected BufRegistry {
     chunk_request_ = atoms;
   }
   int chunksize_used() const override { return chunk_used_; }
+  void set_ordered_sums(bool on) override
+  {
+    if (on) throw InvalidArgument(who_ + ": ordered (atomic-free) sums are available for GRACE-1L engines only");
+  }
+  bool ordered_sums() const override { return false; }
   void set_exchange(const ExchangeCallbacks &cb) override { exchange_ = cb; }
   int comm_layers() const override { return 0; }
   int comm_width(int) const override { return 0; }
@@ -699,6 +704,7 @@ class EngineBase : public Engine, protected BufRegistry {
     nb_ = nb;
     nstruct_ = in.sid ? in.nstruct : 1;
     have_sid_ = in.sid != nullptr;
+    sid_sorted_ = !in.sid || std::is_sorted(in.sid, in.sid + n);
     scal_.ensure((size_t) 8 * nstruct_ * sizeof(double));
     have_rij_ = in.rij != nullptr;
     auto put = [&](DevBuf &b, const void *src, size_t bytes) {
@@ -748,6 +754,7 @@ class EngineBase : public Engine, protected BufRegistry {
     nb_ = in.nb;
     nstruct_ = in.sid ? in.nstruct : 1;
     have_sid_ = in.sid != nullptr;
+    sid_sorted_ = !in.sid || std::is_sorted(in.sid, in.sid + n);
     have_rij_ = in.rij != nullptr;
     scal_.ensure((size_t) 8 * nstruct_ * sizeof(double));
     auto put = [&](DevBuf &b, const void *src, size_t bytes, hipMemcpyKind kind) {
@@ -1310,7 +1317,7 @@ class EngineBase : public Engine, protected BufRegistry {
   DevBuf cut_, mu_, sid_, offset_, j_, rij_, x_, image_, shifts_, tiles_;
   int ntiles_ = 0, nstruct_ = 1;
   std::vector<int> tile_el_;    // [nel + 1] tile range of every element
-  bool have_sid_ = false;
+  bool have_sid_ = false, sid_sorted_ = true;    // sid_sorted_: the atoms of every structure are one range of rows
   const int *sid_ptr() const { return have_sid_ ? sid_.as<int>() : nullptr; }
   // edges of the pass and its outputs (scal: energy, virial[6])
   DevBuf count_, eoff_, zero_, ei_, ej_, emu_, rh_, r_, xr_, rc_, f_, eatom_, scal_;

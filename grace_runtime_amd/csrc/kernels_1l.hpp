@@ -1170,7 +1170,8 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
     const double Ei = (act(M.nlay, 0) + r[0]) * M.out_scale + M.shift[mu[a0 + at]];
     if (lane == 0) {
       if (eatom_chunk) eatom_chunk[at] = Ei;
-      if (sid) atomicAdd(energy + 8 * sid[a0 + at], Ei);    // one (energy, virial[6]) record of 8 doubles per structure
+      if (!energy) {}    // ordered mode: the records are summed from the per-atom energies afterwards
+      else if (sid) atomicAdd(energy + 8 * sid[a0 + at], Ei);    // one (energy, virial[6]) record of 8 doubles per structure
       else esum += Ei;
     }
     if (!want_grad) continue;
@@ -1223,7 +1224,7 @@ static __global__ __launch_bounds__(256) void k_energy(EnergyDev M, const int *m
     if (lane == 0) g[0] = M.out_scale;
     for (int k = lane; k < n0; k += 64) g[k + 1] = gbuf(cur, k);
   }
-  if (!sid) {    // one atomic per block (every wave leaves the loop above and arrives here)
+  if (!sid && energy) {    // one atomic per block (every wave leaves the loop above and arrives here)
     __shared__ double eblk[4];
     if (lane == 0) eblk[wave] = esum;
     __syncthreads();
@@ -1394,6 +1395,9 @@ template<class T> struct BondBwdArgs {
   double *virial;             // [6]     (+=, atomics); with sid: record 8 sid[i] of the atom's structure
   const int *sid;             // [n] structure of each atom, or null
   double *vatom;              // [n][6] per-atom virial (+=, atomics), or null: half of a bond's (-r rhat) (x) fv to each of its atoms
+  // ordered mode (both set, no atomics, vatom null): fedge[e][3] = force of bond e on its central atom; fcen[i][9] = sum of
+  // these over the bonds of atom i, then the six virial sums of its bonds; k_ordered_forces / k_ordered_records finish
+  double *fedge, *fcen;
   int a0;
   int C, nl, nlm, noutp;
   int drow[16];               // accumulator row of (lane / 16, register)
@@ -1496,7 +1500,8 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
       const double fv[3] = {dEdr * u0 + (p0 - gr * u0) / br, dEdr * u1 + (p1 - gr * u1) / br, dEdr * u2 + (p2 - gr * u2) / br};
       for (int d = 0; d < 3; d++) {
         fi[d] += fv[d];
-        atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
+        if (a.fedge) a.fedge[3 * (eb + lane) + d] = fv[d];
+        else atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
       }
       const double ddx = -u0 * br, ddy = -u1 * br, ddz = -u2 * br;
       vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
@@ -1519,7 +1524,8 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
   __syncthreads();
   if (t < 9) {
     const double s = red[0][t] + red[1][t] + red[2][t] + red[3][t];
-    if (e1 > e0) {
+    if (a.fcen) a.fcen[9 * (long long) i + t] = s;
+    else if (e1 > e0) {
       if (t < 3) atomicAdd(&a.f[3 * (long long) i + t], s);
       else {
         atomicAdd(&a.virial[(a.sid ? 8 * a.sid[i] : 0) + t - 3], s);
@@ -1527,6 +1533,97 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
       }
     }
   }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// ordered (atomic-free) sums of the forces, the virial and the energy: same bits on every run
+// ---------------------------------------------------------------------------------------------------------------
+// bonds per neighbour atom: count[ej[e]] += 1 (integer atomics: the result does not depend on their order)
+static __global__ void k_tlist_count(const long long *n_edges, const int *ej, int *count)
+{
+  const long long e = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (e < *n_edges) atomicAdd(&count[ej[e]], 1);
+}
+// bond numbers by neighbour atom, in arrival order (k_tlist_sort orders every row)
+static __global__ void k_tlist_fill(const long long *n_edges, const int *ej, const long long *toff, int *cursor, int *raw)
+{
+  const long long e = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (e < *n_edges) {
+    const int j = ej[e];
+    raw[toff[j] + atomicAdd(&cursor[j], 1)] = (int) e;
+  }
+}
+// One wave per atom k (owned atoms, then ghosts): its row of bond numbers in ascending order, by counting for every
+// entry the entries below it (a row is a few hundred entries at most).
+static __global__ void k_tlist_sort(int n_nodes, const long long *toff, const int *raw, int *sorted)
+{
+  const int lane = threadIdx.x & 63;
+  const int k = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (k >= n_nodes) return;
+  const long long t0 = toff[k];
+  const int *row = raw + t0;
+  const int len = (int) (toff[k + 1] - t0);
+  for (int p = lane; p < len; p += 64) {
+    const int mine = row[p];
+    int rank = 0;
+    for (int q = 0; q < len; q++) rank += row[q] < mine;
+    sorted[t0 + rank] = mine;
+  }
+}
+// One wave per atom k: f[k] = fcen[k] (owned atoms) - sum of fedge over the bonds that have k as their neighbour, the
+// sorted row taken by the lanes in turn and the lane sums added in a fixed tree.
+static __global__ void k_ordered_forces(int n_nodes, int n, const long long *toff, const int *sorted, const double *fedge, const double *fcen, double *f)
+{
+  const int lane = threadIdx.x & 63;
+  const int k = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (k >= n_nodes) return;
+  const long long t0 = toff[k];
+  const int len = (int) (toff[k + 1] - t0);
+  double s[3] = {0, 0, 0};
+  for (int p = lane; p < len; p += 64) {
+    const double *fe = fedge + 3 * (long long) sorted[t0 + p];
+    s[0] += fe[0]; s[1] += fe[1]; s[2] += fe[2];
+  }
+#pragma unroll
+  for (int d = 0; d < 3; d++)
+    for (int o = 32; o > 0; o >>= 1) s[d] += __shfl_xor(s[d], o, 64);
+  if (lane < 3) f[3 * (long long) k + lane] = (k < n ? fcen[9 * (long long) k + lane] : 0.0) - s[lane];
+}
+// One block per structure: record (energy, virial[6]) = sums of eatom[i] and fcen[i][3 .. 9] over its atoms, which are
+// the range [lower_bound(s), lower_bound(s + 1)) of the non-decreasing sid (null: one structure, all atoms); every
+// thread adds its atoms in ascending order, the thread sums are added in a fixed tree.
+static __global__ __launch_bounds__(256) void k_ordered_records(int n, const int *sid, const double *eatom, const double *fcen, int with_virial, double *rec)
+{
+  __shared__ double part[256][7];
+  const int s = blockIdx.x, t = threadIdx.x;
+  int lo = 0, hi = n;
+  if (sid) {
+    auto lower = [&](int key) {
+      int a = 0, b = n;
+      while (a < b) {
+        const int m = (a + b) >> 1;
+        if (sid[m] < key) a = m + 1;
+        else b = m;
+      }
+      return a;
+    };
+    lo = lower(s);
+    hi = lower(s + 1);
+  }
+  double v[7] = {0, 0, 0, 0, 0, 0, 0};
+  for (int i = lo + t; i < hi; i += 256) {
+    v[0] += eatom[i];
+    if (with_virial)
+      for (int k = 0; k < 6; k++) v[1 + k] += fcen[9 * (long long) i + 3 + k];
+  }
+  for (int k = 0; k < 7; k++) part[t][k] = v[k];
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if (t < o)
+      for (int k = 0; k < 7; k++) part[t][k] += part[t + o][k];
+    __syncthreads();
+  }
+  if (t < 7) rec[8 * (long long) s + t] = part[0][t];
 }
 
 }    // namespace grhip

@@ -268,6 +268,15 @@ class Engine:
     def chunksize(self) -> int:
         return int(_lib.lib().gr_engine_chunksize(self._h))
 
+    def set_ordered_sums(self, on: bool = True):
+        """forces, virial and energy added in a fixed order instead of with floating-point atomics: the same bits on every
+        call with the same input.  GRACE-1L engines only (ValueError otherwise); no per-atom virials in this mode."""
+        check(_lib.lib().gr_engine_set_ordered_sums(self._h, 1 if on else 0))
+
+    @property
+    def ordered_sums(self) -> bool:
+        return bool(_lib.lib().gr_engine_ordered_sums(self._h))
+
     def release_buffers(self):
         """frees the work buffers and the uploaded structure; weights, tables and compiled kernels stay"""
         check(_lib.lib().gr_engine_release_buffers(self._h))

@@ -292,6 +292,16 @@ int gr_engine_set_chunksize(gr_engine *e, int atoms);
 int gr_engine_chunksize(const gr_engine *e);
 int gr_system_set_chunksize(gr_system *s, int atoms);
 int gr_system_chunksize(const gr_system *s);
+
+/* Ordered sums: with on != 0 the engine adds forces, virial and energy in a fixed order instead of with floating-point
+ * atomics, so that two calls on the same input return the same bits.  The forces on the neighbours are gathered through
+ * the bonds listed by neighbour atom (rebuilt every pass), the energy and virial of every structure are summed over its
+ * atoms in ascending order.  The reference's GPU engines have no such mode: they document last-bit variation from run to
+ * run (python/tests/test_gpu_several_calculators.py).  GRACE-1L engines only: GR_INVALID with on != 0 for a GRACE-2L or
+ * GRACE-3L engine (their message adjoints are summed with atomics).  With ordered sums a run with GR_FLAG_VATOM gives
+ * GR_INVALID, and so does a batch whose atoms are not grouped by structure.  gr_engine_ordered_sums: 1 when on. */
+int gr_engine_set_ordered_sums(gr_engine *e, int on);
+int gr_engine_ordered_sums(const gr_engine *e);
 int gr_system_rebuilds(const gr_system *s);
 int gr_system_list_on_device(const gr_system *s);
 int gr_system_list_sizes(gr_system *s, int64_t *nbonds, int64_t *nimages);

@@ -66,6 +66,9 @@ class Engine {
   int precision = 64, device = 0;
   // atoms per pass: > 0 fixed, 0 one pass, -1 from the free device memory (kk/grace_1l_kk.h: chunksize)
   int chunksize = -1;
+  // forces, virial and energy added in a fixed order (same bits on every run) instead of with floating-point atomics;
+  // GRACE-1L models only, no per-atom virials (gr_engine_set_ordered_sums)
+  bool ordered_sums = false;
 
   void set_model(const std::string &npz_path, const std::vector<int> &type2mu)
   {
@@ -81,6 +84,7 @@ class Engine {
     engine_ = nullptr;
     check(gr_engine_create(model_, (int) type2mu_.size() - 1, type2mu_.data(), precision, device, &engine_));
     check(gr_engine_set_chunksize(engine_, chunksize));
+    if (ordered_sums) check(gr_engine_set_ordered_sums(engine_, 1));
     if (exchange_) install_exchange();
   }
   double cutoff(int type_i, int type_j) const { return engine_ ? gr_engine_cutoff(engine_, type_i, type_j) : 0.0; }
