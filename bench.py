@@ -244,9 +244,10 @@ def main():
             del sysm
     upload()
 
-    # the same passes with ordered (atomic-free) sums of forces, virial and energy (GRACE-1L engines): reported beside
+    # the same passes with ordered (atomic-free) sums of forces, virial, energy and message adjoints (GRACE-1L and 2L
+    # engines): reported beside
     ordered_ms = None
-    if not (two or three or batch):
+    if not three:
         eng.set_ordered_sums(True)
         eng.run()
         eng.sync()

@@ -127,9 +127,9 @@ class Engine {
   // passes with it (the reference sizes the first pass from the free memory: libgrace/include/grace/kk/support.h:425-450)
   virtual int64_t atoms_that_fit() = 0;
   virtual void set_chunksize(int atoms) = 0;
-  // ordered sums: forces, virial and energy are added in a fixed order instead of with floating-point atomics, so that two
-  // runs on the same input give the same bits (the reference's GPU engines accept last-bit variation from run to run:
-  // python/tests/test_gpu_several_calculators.py).  GRACE-1L engines only; the others refuse `on`.
+  // ordered sums: forces, virial, energy and message adjoints are added in a fixed order instead of with floating-point
+  // atomics, so that two runs on the same input give the same bits (the reference's GPU engines accept last-bit variation
+  // from run to run: python/tests/test_gpu_several_calculators.py).  GRACE-1L and 2L engines; GRACE-3L engines refuse `on`.
   virtual void set_ordered_sums(bool on) = 0;
   virtual bool ordered_sums() const = 0;
   virtual int chunksize_used() const = 0;

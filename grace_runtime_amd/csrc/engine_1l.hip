@@ -74,6 +74,7 @@ template<class T> class Engine1L final : public EngineBase {
   {
     this->template probe_mfma<T>();
     chunks_ = true;
+    ordered_ok_ = true;
     build();
     scratch_dev_ = scratch_of_device(device);    // set-up: the device is current (EngineBase)
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
@@ -83,16 +84,8 @@ template<class T> class Engine1L final : public EngineBase {
   void run(const RunFlags &fl) override;
   void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) override;
   void radial_noalloc(int m, const double *x, const int *mu_j, double *Rz, double *dRz) override;
-  void set_ordered_sums(bool on) override { ordered_ = on; }
-  bool ordered_sums() const override { return ordered_; }
 
  private:
-  // ordered sums: the bond reverse stores the force of every bond and the sums over each atom's own bonds; the forces on
-  // the neighbours are then gathered through the bonds listed by neighbour atom (rebuilt every pass: the bonds inside the
-  // cutoff change with the positions), energy and virial records are summed per structure in a fixed order
-  bool ordered_ = false;
-  DevBuf fedge_, fcen_, tcount_, toff_, traw_, tsorted_;
-  void finish_ordered(const RunFlags &fl);
   unsigned char *scratch_dev_ = nullptr;    // this device's copy of the fixed array (hipGetSymbolAddress)
   std::shared_ptr<const Model1L> model_;
   bool jit_all_ = false;
@@ -315,16 +308,9 @@ void Engine1L<T>::launch_radial(long long e_begin, long long e_count, const doub
 template<class T> void Engine1L<T>::run(const RunFlags &fl)
 {
   const int n = n_;
-  if (ordered_) {
-    if (fl.vatom && !fl.energy_only) throw InvalidArgument("GRACE-1L: per-atom virials are not available with ordered sums");
-    if (!sid_sorted_) throw InvalidArgument("GRACE-1L: ordered sums need the atoms of every structure in one range of rows");
-    if (nb_ >= INT32_MAX) throw InvalidArgument("GRACE-1L: ordered sums number the bonds with 32 bits");
-  }
+  ordered_check(fl);
   if (!begin_pass(fl)) return;
-  if (ordered_ && !fl.energy_only) {
-    fedge_.ensure((size_t) 3 * std::max<int64_t>(nb_, 1) * sizeof(double));
-    fcen_.ensure((size_t) 9 * n * sizeof(double));
-  }
+  if (ordered_ && !fl.energy_only) ordered_begin();
 
   // ---- chunks of atoms: every stage after the bond filter acts on the atoms of a chunk and on their bonds only, so the
   // radial rows and the per-atom tensors are sized for one chunk; forces, per-atom energies and the compact bonds are
@@ -385,33 +371,7 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
       run_chunk(fl, a0, nc, ebound[(size_t) k], ebound[(size_t) k + 1] - ebound[(size_t) k]);
     }
   }
-  if (ordered_) finish_ordered(fl);
-}
-
-template<class T> void Engine1L<T>::finish_ordered(const RunFlags &fl)
-{
-  const int n = n_, nn = n_nodes_;
-  stage("ordered_sums", [&] {
-    if (!fl.energy_only) {
-      const size_t ne = (size_t) std::max<int64_t>(nb_, 1);
-      tcount_.ensure((size_t) 2 * nn * sizeof(int));    // bonds per neighbour atom, then the fill cursors
-      toff_.ensure(((size_t) nn + 1) * sizeof(long long));
-      traw_.ensure(ne * sizeof(int));
-      tsorted_.ensure(ne * sizeof(int));
-      HIP_CHECK(hipMemsetAsync(tcount_.p, 0, (size_t) 2 * nn * sizeof(int), stream_));
-      const long long *n_edges = eoff_.as<long long>() + n;
-      const dim3 egrid((unsigned) ((ne + 255) / 256)), agrid((unsigned) ((nn + 3) / 4));
-      hipLaunchKernelGGL(k_tlist_count, egrid, dim3(256), 0, stream_, n_edges, ej_.as<int>(), tcount_.as<int>());
-      hipLaunchKernelGGL(k_scan, dim3(1), dim3(1024), 0, stream_, tcount_.as<int>(), nn, toff_.as<long long>());
-      hipLaunchKernelGGL(k_tlist_fill, egrid, dim3(256), 0, stream_, n_edges, ej_.as<int>(), toff_.as<long long>(), tcount_.as<int>() + nn,
-                         traw_.as<int>());
-      hipLaunchKernelGGL(k_tlist_sort, agrid, dim3(256), 0, stream_, nn, toff_.as<long long>(), traw_.as<int>(), tsorted_.as<int>());
-      hipLaunchKernelGGL(k_ordered_forces, agrid, dim3(256), 0, stream_, nn, n, toff_.as<long long>(), tsorted_.as<int>(), fedge_.as<double>(),
-                         fcen_.as<double>(), f_.as<double>());
-    }
-    hipLaunchKernelGGL(k_ordered_records, dim3((unsigned) nstruct_), dim3(256), 0, stream_, n, sid_ptr(), eatom_.as<double>(), fcen_.as<double>(),
-                       fl.energy_only ? 0 : 1, scal_.as<double>());
-  });
+  if (ordered_) ordered_finish(fl);
 }
 
 // One chunk: atoms [a0, a0 + nc) and their bonds [e_begin, e_begin + e_count) (e_count < 0: all bonds, counted on the

@@ -37,6 +37,7 @@ template<class T> class Engine2L final : public EngineBase {
     build();
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
     chunks_ = true;
+    ordered_ok_ = true;
   }
   int layers() const override { return 2; }
   void run(const RunFlags &fl) override;
@@ -71,6 +72,7 @@ template<class T> class Engine2L final : public EngineBase {
   Energy2Dev en_{};
   // pass buffers
   DevBuf sink_, Rz_, dRz_, R1_, dR1_, YG_, A_, rho_, grho_, I1_, gI1_, I1t_, gI1t_, M_, gM_, P_, gP_, B_, I2_, gI2_;
+  DevBuf gMe_;    // ordered sums: the message adjoints of a chunk's bonds, [bond][nI][CRP]
   // the chunk of atoms the chain and reduce functions act on: cn_ atoms from a0_, the chunk's element tiles (atoms counted
   // from a0_), the capacity the chunk buffers are sized for
   int cn_ = 0, a0_ = 0;
@@ -506,10 +508,12 @@ template<class T> void Engine2L<T>::reduce_bwd(DevReduce<T> &R, const Chain<T> &
 template<class T> void Engine2L<T>::run(const RunFlags &fl)
 {
   const int n = n_;
+  ordered_check(fl);
   if (!begin_pass(fl)) return;
   const size_t ecap_all = (size_t) std::max<int64_t>(nb_, 1);
   const long long *n_edges = eoff_.as<long long>() + n;
   const bool forces = !fl.energy_only;
+  if (ordered_ && forces) ordered_begin();
   const int yw = forces ? 3 * nlm_ : nlm_;    // row of an edge: Y[nlm] and, for forces, the two tangential gradients D1[nlm], D2[nlm]
   YG_.ensure(ecap_all * yw * sizeof(T));
   stage("sh_edges", [&] {
@@ -632,6 +636,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   if (forces) {
     gP_.ensure(na * npf * CRP_ * sizeof(T));
     gM_.ensure(nnodes * nI_ * CRP_ * sizeof(T));
+    if (ordered_) gMe_.ensure(ecap * nI_ * CRP_ * sizeof(T));
     stage("zero_gM", [&] { HIP_CHECK(hipMemsetAsync(gM_.p, 0, nnodes * nI_ * CRP_ * sizeof(T), stream_)); });
   }
 #define GR_PAIR1(K_, N_, grid_, block_, lds_, ...)                                                                       \
@@ -650,6 +655,24 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     case 5: GR_PAIR1(K_, 25, __VA_ARGS__) break;             \
     case 6: GR_PAIR1(K_, 36, __VA_ARGS__) break;             \
     default: GR_PAIR1(K_, 49, __VA_ARGS__) break;            \
+  }
+// the staged reverse kernel in its form without floating-point atomics
+#define GR_PAIR_ORD1(N_, grid_, block_, lds_, ...)                                                                       \
+  {                                                                                                                      \
+    auto kern = k_pair_bwd<T, N_, true>;                                                                                 \
+    if (lds_ > 48 * 1024)                                                                                                \
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_)); \
+    hipLaunchKernelGGL(kern, grid_, block_, lds_, __VA_ARGS__);                                                          \
+  }
+#define GR_PAIR_ORD(...)                                     \
+  switch (nl_) {                                             \
+    case 1: GR_PAIR_ORD1(1, __VA_ARGS__) break;              \
+    case 2: GR_PAIR_ORD1(4, __VA_ARGS__) break;              \
+    case 3: GR_PAIR_ORD1(9, __VA_ARGS__) break;              \
+    case 4: GR_PAIR_ORD1(16, __VA_ARGS__) break;             \
+    case 5: GR_PAIR_ORD1(25, __VA_ARGS__) break;             \
+    case 6: GR_PAIR_ORD1(36, __VA_ARGS__) break;             \
+    default: GR_PAIR_ORD1(49, __VA_ARGS__) break;            \
   }
 // the reverse kernel with asynchronous staging and chunks of CH_ bonds
 #define GR_PAIR_ASYNC1(N_, CH_, grid_, block_, lds_, ...)                                                                \
@@ -701,8 +724,8 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     stage("energy_mlp", [&] {
       hipLaunchKernelGGL(k_energy_2l, dim3(nc), dim3(64), (size_t) (2 * en_.nlay + 4) * en_.width * sizeof(double), stream_, en_, mu, nc,
                          (const double *) rho_.as<double>() + (size_t) a0_ * nrho_, (const double *) I2_.as<double>(),
-                         grho_.as<double>() + (size_t) a0_ * nrho_, gI2_.as<double>(), fl.eatom ? eatom_.as<double>() + a0_ : nullptr,
-                         scal_.as<double>(), forces ? 1 : 0, sid_ptr() ? sid_ptr() + a0_ : nullptr);
+                         grho_.as<double>() + (size_t) a0_ * nrho_, gI2_.as<double>(), fl.eatom || ordered_ ? eatom_.as<double>() + a0_ : nullptr,
+                         ordered_ ? nullptr : scal_.as<double>(), forces ? 1 : 0, sid_ptr() ? sid_ptr() + a0_ : nullptr);
     });
     if (!forces) continue;
     // layer 2 reverse: dE/dB -> dE/dP -> bond forces of layer 2 and dE/dI of the neighbours
@@ -715,27 +738,44 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
       // blocks that fill a CU alone, of 4 otherwise); fp64 runs faster with one chunk staged through registers
       const size_t row = (size_t) (pthreads + 2 * radR1_.noutp) * sizeof(T);
       const int ch = sizeof(T) != 4 ? 0 : (pthreads >= 512 && 16 * row <= kPairLdsMax) ? 8 : 8 * row <= kPairLdsMax ? 4 : 0;
-      const size_t lds = ch ? 2 * ch * row : kPairChunk * row;
-#define GR_ARGS                                                                                                                         \
+      const size_t lds = ch && !ordered_ ? 2 * ch * row : kPairChunk * row;
+#define GR_ARGS_ASYNC                                                                                                                   \
   dim3(nc), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) dR1, (const T *) M, (const T *) gP_.as<T>(),        \
       rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(), scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, \
       sink_.as<T>(), 1, sid_ptr(), nslot_, 0, nc, a0_, vatom_ptr()
-      if (ch == 8) {
-        GR_PAIR_ASYNC(8, GR_ARGS)
+#define GR_ARGS GR_ARGS_ASYNC, po
+      // ordered sums: the staged kernel without atomics; the message adjoints of the chunk's bonds are gathered afterwards
+      PairOrdered<T> po{};
+      if (ordered_) {
+        po.gMe = gMe_.as<T>(); po.fedge = fedge_.as<double>(); po.fcen = fcen_.as<double>(); po.e_base = eb;
+      }
+      if (ordered_) {
+        GR_PAIR_ORD(GR_ARGS)
+      } else if (ch == 8) {
+        GR_PAIR_ASYNC(8, GR_ARGS_ASYNC)
       } else if (ch == 4) {
-        GR_PAIR_ASYNC(4, GR_ARGS)
+        GR_PAIR_ASYNC(4, GR_ARGS_ASYNC)
       } else {
         GR_PAIR(k_pair_bwd, GR_ARGS)
       }
 #undef GR_ARGS
+#undef GR_ARGS_ASYNC
     });
+    if (ordered_)
+      stage("ordered_gM", [&] {
+        hipLaunchKernelGGL(k_ordered_gm<T>, dim3((unsigned) n_nodes_), dim3(std::min(1024, round_up(nI_ * CRP_, 64))), 0, stream_, toff_.as<long long>(),
+                           tsorted_.as<int>(), (const T *) gMe_.as<T>(), eb, n_edges, ecnt, nI_ * CRP_, gM_.as<T>());
+      });
   }
 #undef GR_PAIR_ASYNC
 #undef GR_PAIR_ASYNC1
+#undef GR_PAIR_ORD
+#undef GR_PAIR_ORD1
 #undef GR_PAIR
 #undef GR_PAIR1
   if (!forces) {
     set_chunk(0);
+    if (ordered_) ordered_finish(fl);
     return;
   }
   exchange_reverse(1);
@@ -773,9 +813,13 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     ba.Rz = moved_back(Rz_.as<T>(), eb * radR_.noutp); ba.dRz = moved_back(dRz_.as<T>(), eb * radR_.noutp); ba.gA = c1_.gX.template as<T>();
     ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr(); ba.vatom = vatom_ptr();
     ba.a0 = a0_; ba.C = C1P_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = radR_.noutp; ba.sh = sh_;
+    if (ordered_) {    // added to what the pair kernel of layer 2 stored for the same bonds and atoms
+      ba.fedge = fedge_.as<double>(); ba.fcen = fcen_.as<double>(); ba.ordered_add = 1;
+    }
     stage("bond_bwd", [&] { launch_bond_bwd<T>(ba, cn_); });
   }
   set_chunk(0);
+  if (ordered_) ordered_finish(fl);
 }
 
 }    // namespace

@@ -945,7 +945,7 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
     } else if (ch == 4) {
       GR_PAIR_ASYNC(4, GR_ARGS)
     } else {
-      GR_PAIR(k_pair_bwd, GR_ARGS)
+      GR_PAIR(k_pair_bwd, GR_ARGS, PairOrdered<T>{})
     }
 #undef GR_ARGS
   });

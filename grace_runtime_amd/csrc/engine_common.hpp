@@ -577,9 +577,10 @@ class EngineBase : public Engine, protected BufRegistry {
   int chunksize_used() const override { return chunk_used_; }
   void set_ordered_sums(bool on) override
   {
-    if (on) throw InvalidArgument(who_ + ": ordered (atomic-free) sums are available for GRACE-1L engines only");
+    if (on && !ordered_ok_) throw InvalidArgument(who_ + ": ordered (atomic-free) sums are available for GRACE-1L and GRACE-2L engines only");
+    ordered_ = on;
   }
-  bool ordered_sums() const override { return false; }
+  bool ordered_sums() const override { return ordered_; }
   void set_exchange(const ExchangeCallbacks &cb) override { exchange_ = cb; }
   int comm_layers() const override { return 0; }
   int comm_width(int) const override { return 0; }
@@ -1318,6 +1319,57 @@ class EngineBase : public Engine, protected BufRegistry {
   int ntiles_ = 0, nstruct_ = 1;
   std::vector<int> tile_el_;    // [nel + 1] tile range of every element
   bool have_sid_ = false, sid_sorted_ = true;    // sid_sorted_: the atoms of every structure are one range of rows
+
+  // ---- ordered sums (engines that set ordered_ok_): the reverse kernels store the force of every bond on its central atom
+  // (fedge_[e][3]) and, per atom, the sums over its own bonds (fcen_[i][9]: force, then the six virial sums) instead of
+  // adding with atomics; the forces on the neighbours are gathered through the bonds listed by neighbour atom (rebuilt every
+  // pass: the bonds inside the cutoff change with the positions); energy and virial records are summed per structure in a
+  // fixed order from the per-atom energies and fcen_
+  bool ordered_ok_ = false, ordered_ = false;
+  DevBuf fedge_, fcen_, tcount_, toff_, traw_, tsorted_;
+  // before begin_pass(): what the mode cannot do
+  void ordered_check(const RunFlags &fl) const
+  {
+    if (!ordered_) return;
+    if (fl.vatom && !fl.energy_only) throw InvalidArgument(who_ + ": per-atom virials are not available with ordered sums");
+    if (!sid_sorted_) throw InvalidArgument(who_ + ": ordered sums need the atoms of every structure in one range of rows");
+    if (nb_ >= INT32_MAX) throw InvalidArgument(who_ + ": ordered sums number the bonds with 32 bits");
+  }
+  // after begin_pass() of a pass with forces: the per-bond and per-atom stores, and the bonds by neighbour atom, each row
+  // in ascending order
+  void ordered_begin()
+  {
+    const int n = n_, nn = n_nodes_;
+    const size_t ne = (size_t) std::max<int64_t>(nb_, 1);
+    fedge_.ensure(3 * ne * sizeof(double));
+    fcen_.ensure((size_t) 9 * std::max(n, 1) * sizeof(double));
+    tcount_.ensure((size_t) 2 * nn * sizeof(int));    // bonds per neighbour atom, then the fill cursors
+    toff_.ensure(((size_t) nn + 1) * sizeof(long long));
+    traw_.ensure(ne * sizeof(int));
+    tsorted_.ensure(ne * sizeof(int));
+    stage("ordered_list", [&] {
+      HIP_CHECK(hipMemsetAsync(tcount_.p, 0, (size_t) 2 * nn * sizeof(int), stream_));
+      const long long *n_edges = eoff_.as<long long>() + n;
+      const dim3 egrid((unsigned) ((ne + 255) / 256)), agrid((unsigned) ((nn + 3) / 4));
+      hipLaunchKernelGGL(k_tlist_count, egrid, dim3(256), 0, stream_, n_edges, ej_.as<int>(), tcount_.as<int>());
+      hipLaunchKernelGGL(k_scan, dim3(1), dim3(1024), 0, stream_, tcount_.as<int>(), nn, toff_.as<long long>());
+      hipLaunchKernelGGL(k_tlist_fill, egrid, dim3(256), 0, stream_, n_edges, ej_.as<int>(), toff_.as<long long>(), tcount_.as<int>() + nn,
+                         traw_.as<int>());
+      hipLaunchKernelGGL(k_tlist_sort, agrid, dim3(256), 0, stream_, nn, toff_.as<long long>(), traw_.as<int>(), tsorted_.as<int>());
+    });
+  }
+  // end of the pass: forces of all rows (ghosts included) and the records of the structures
+  void ordered_finish(const RunFlags &fl)
+  {
+    const int n = n_, nn = n_nodes_;
+    stage("ordered_sums", [&] {
+      if (!fl.energy_only)
+        hipLaunchKernelGGL(k_ordered_forces, dim3((unsigned) ((nn + 3) / 4)), dim3(256), 0, stream_, nn, n, toff_.as<long long>(), tsorted_.as<int>(),
+                           fedge_.as<double>(), fcen_.as<double>(), f_.as<double>());
+      hipLaunchKernelGGL(k_ordered_records, dim3((unsigned) nstruct_), dim3(256), 0, stream_, n, sid_ptr(), eatom_.as<double>(), fcen_.as<double>(),
+                         fl.energy_only ? 0 : 1, scal_.as<double>());
+    });
+  }
   const int *sid_ptr() const { return have_sid_ ? sid_.as<int>() : nullptr; }
   // edges of the pass and its outputs (scal: energy, virial[6])
   DevBuf count_, eoff_, zero_, ei_, ej_, emu_, rh_, r_, xr_, rc_, f_, eatom_, scal_;

@@ -1398,6 +1398,7 @@ template<class T> struct BondBwdArgs {
   // ordered mode (both set, no atomics, vatom null): fedge[e][3] = force of bond e on its central atom; fcen[i][9] = sum of
   // these over the bonds of atom i, then the six virial sums of its bonds; k_ordered_forces / k_ordered_records finish
   double *fedge, *fcen;
+  int ordered_add;            // ordered mode: add to what fedge / fcen hold (a later layer of the same pass) instead of storing
   int a0;
   int C, nl, nlm, noutp;
   int drow[16];               // accumulator row of (lane / 16, register)
@@ -1500,7 +1501,7 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
       const double fv[3] = {dEdr * u0 + (p0 - gr * u0) / br, dEdr * u1 + (p1 - gr * u1) / br, dEdr * u2 + (p2 - gr * u2) / br};
       for (int d = 0; d < 3; d++) {
         fi[d] += fv[d];
-        if (a.fedge) a.fedge[3 * (eb + lane) + d] = fv[d];
+        if (a.fedge) a.fedge[3 * (eb + lane) + d] = (a.ordered_add ? a.fedge[3 * (eb + lane) + d] : 0.0) + fv[d];
         else atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
       }
       const double ddx = -u0 * br, ddy = -u1 * br, ddz = -u2 * br;
@@ -1524,7 +1525,7 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
   __syncthreads();
   if (t < 9) {
     const double s = red[0][t] + red[1][t] + red[2][t] + red[3][t];
-    if (a.fcen) a.fcen[9 * (long long) i + t] = s;
+    if (a.fcen) a.fcen[9 * (long long) i + t] = (a.ordered_add ? a.fcen[9 * (long long) i + t] : 0.0) + s;
     else if (e1 > e0) {
       if (t < 3) atomicAdd(&a.f[3 * (long long) i + t], s);
       else {

@@ -156,16 +156,25 @@ __device__ inline double wave_sum4(double v0, double v1, double v2, double v3, i
 //   dE/dx = sum_{slot,n,l} S_l dR1_l M_j,   g_k = sum_{slot,n,l} T_l,k R1_l M_j
 //   fv = dE/dx / rc rhat + (g_1 e1 + g_2 e2) / r  (= the reference's dE/dx / rc rhat + (g - (g . rhat) rhat) / r with
 //   g the Cartesian sum);  f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv
-template<class T, int NLM>
+// ORD (ordered sums, one slot group): no floating-point atomics.  The message adjoint of bond e goes to
+// ord.gMe[e - ord.e_base][slot][n], the bond's force to ord.fedge[e][3], the sums over the atom's bonds to
+// ord.fcen[a0 + i][9]; the sums over the waves of a block are added in the order of the waves.
+template<class T> struct PairOrdered {
+  T *gMe;
+  double *fedge, *fcen;
+  long long e_base;
+};
+template<class T, int NLM, bool ORD = false>
 __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ YG,
                            const T *__restrict__ R1, const T *__restrict__ dR1, const T *__restrict__ M, const T *__restrict__ gP,
                            const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
                            T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
                            int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms, int a0,
-                           double *__restrict__ vatom)
+                           double *__restrict__ vatom, PairOrdered<T> ord)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   __shared__ double bsum[kPairChunk][4];
+  __shared__ double bwave[ORD ? kPairChunk : 1][ORD ? 16 : 1][4];    // ORD: the sums of every wave (at most 16 waves)
   int i, grp;
   if (!pair_block(ngrp, natoms, i, grp)) return;
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6, NT = blockDim.x;
@@ -211,11 +220,23 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
           dE += drl * S;
           t1 += rl * a1; t2 += rl * a2;
         }
-      if (active && slot < nI) atomicAdd(&gM[((long long) ej[e] * nI + slot) * C + n], sI);
+      if (active && slot < nI) {
+        if (ORD) ord.gMe[((e - ord.e_base) * nI + slot) * C + n] = sI;
+        else atomicAdd(&gM[((long long) ej[e] * nI + slot) * C + n], sI);
+      }
       const double c = wave_sum4((double) (dE * m), (double) (t1 * m), (double) (t2 * m), 0.0, lane);
-      if (lane < 3) atomicAdd(&bsum[b][lane], c);    // lanes 0..2: dE/dx, g . e2, g . e1  (order v0, v2, v1, v3)
+      if (lane < 3) {    // lanes 0..2: dE/dx, g . e2, g . e1  (order v0, v2, v1, v3)
+        if (ORD) bwave[b][wave][lane] = c;
+        else atomicAdd(&bsum[b][lane], c);
+      }
     }
     __syncthreads();
+    if (ORD && t < nb)
+      for (int k = 0; k < 3; k++) {
+        double sw = 0.0;
+        for (int w = 0; w < (NT >> 6); w++) sw += bwave[t][w][k];
+        bsum[t][k] = sw;
+      }
     if (t < nb) {
       const long long e = base + t;
       const double *u = rh + 3 * e;
@@ -227,12 +248,13 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
       const int jj = ej[e];
       for (int d = 0; d < 3; d++) {
         fi[d] += fv[d];
-        atomicAdd(&f[3 * (long long) jj + d], -fv[d]);
+        if (ORD) ord.fedge[3 * e + d] = fv[d];
+        else atomicAdd(&f[3 * (long long) jj + d], -fv[d]);
       }
       const double ddx = -u[0] * r, ddy = -u[1] * r, ddz = -u[2] * r;
       vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
       vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
-      if (vatom) {    // per-atom virial: the neighbour's half of this bond (fused_cpu.h:1075-1087 of the reference)
+      if (!ORD && vatom) {    // per-atom virial: the neighbour's half of this bond (fused_cpu.h:1075-1087 of the reference)
         double *vj = vatom + 6 * (long long) jj;
         atomicAdd(vj, 0.5 * ddx * fv[0]); atomicAdd(vj + 1, 0.5 * ddy * fv[1]); atomicAdd(vj + 2, 0.5 * ddz * fv[2]);
         atomicAdd(vj + 3, 0.5 * ddx * fv[1]); atomicAdd(vj + 4, 0.5 * ddx * fv[2]); atomicAdd(vj + 5, 0.5 * ddy * fv[2]);
@@ -245,7 +267,10 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
 #pragma unroll
     for (int k = 0; k < 9; k++)
       for (int o = 32; o > 0; o >>= 1) vsum[k] += __shfl_xor(vsum[k], o, 64);
-    if (lane == 0 && e1 > e0) {
+    if (ORD) {
+      if (lane == 0)
+        for (int k = 0; k < 9; k++) ord.fcen[9 * (long long) (a0 + i) + k] = vsum[k];
+    } else if (lane == 0 && e1 > e0) {
       for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) (a0 + i) + k], vsum[k]);
       for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[a0 + i] : 0) + k], vsum[3 + k]);
       if (vatom)
@@ -253,6 +278,26 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
     }
   }
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
+}
+
+// Ordered sums: gM[j][slot][n] += sum of gMe[e - e_base][slot][n] over the bonds e in [e_base, e_end) that have j as their
+// neighbour, in ascending order of e (sorted: the bonds by neighbour atom, each row ascending; ncol = nI C columns).
+// One block per atom j; a thread owns columns, so no two threads add to one value.
+template<class T>
+__global__ void k_ordered_gm(const long long *__restrict__ toff, const int *__restrict__ sorted, const T *__restrict__ gMe, long long e_base,
+                             const long long *__restrict__ e_end_dev, long long e_count, int ncol, T *__restrict__ gM)
+{
+  const int j = blockIdx.x;
+  const long long t0 = toff[j], t1 = toff[j + 1];
+  const long long e_end = e_count >= 0 ? e_base + e_count : *e_end_dev;
+  for (int col = threadIdx.x; col < ncol; col += blockDim.x) {
+    T s = (T) 0;
+    for (long long p = t0; p < t1; p++) {
+      const long long e = sorted[p];
+      if (e >= e_base && e < e_end) s += gMe[(e - e_base) * ncol + col];
+    }
+    gM[(long long) j * ncol + col] += s;
+  }
 }
 
 // ---- the pair kernels with asynchronous staging
@@ -554,7 +599,7 @@ static __global__ void k_energy_2l(Energy2Dev M, const int *mu, int natoms, cons
   const double Ei = (act(M.nlay, 0) + r[0] + i2[0] / s0 * M.ln0[0]) * M.out_scale + M.shift[mu[at]];
   if (lane == 0) {
     if (eatom) eatom[at] = Ei;
-    atomicAdd(energy + (sid ? 8 * sid[at] : 0), Ei);
+    if (energy) atomicAdd(energy + (sid ? 8 * sid[at] : 0), Ei);    // null: ordered sums, the records are added from eatom afterwards
   }
   if (!want_grad) return;
   int cur = 0;

@@ -1,5 +1,5 @@
-"""Ordered (atomic-free) sums of the GRACE-1L engines (gr_engine_set_ordered_sums): forces, virial and energy added in a
-fixed order.  The reference's GPU engines have no such mode and document last-bit variation from run to run
+"""Ordered (atomic-free) sums of the GRACE-1L and GRACE-2L engines (gr_engine_set_ordered_sums): forces, virial, energy
+and, for 2L, the message adjoints added in a fixed order.  The reference's GPU engines have no such mode and document last-bit variation from run to run
 (python/tests/test_gpu_several_calculators.py); the tests hold the ordered mode to the atomic mode at the parity bounds of
 the other GPU tests (1e-10 eV/atom, 1e-9 eV/A) and to ITSELF bit for bit: repeated calls, a fresh engine, chunked passes."""
 import numpy as np
@@ -30,7 +30,8 @@ def _close(a, b, n, tol):
 
 
 @pytest.mark.parametrize("precision", [64, 32])
-@pytest.mark.parametrize("model,struct,species", [("mix2", "alloy54", ["Mo", "W"]), ("cut2", "slab", ["Al", "Ni"]), ("config1", "config1", ["W"])])
+@pytest.mark.parametrize("model,struct,species", [("mix2", "alloy54", ["Mo", "W"]), ("cut2", "slab", ["Al", "Ni"]), ("config1", "config1", ["W"]),
+                                                  ("l2mix", "alloy54", ["Mo", "W"]), ("l2mix", "slab", ["Mo", "W"]), ("config3", "fcc108", ["Al", "Co", "Ni", "Ti"])])
 def test_ordered_sums_equal_atomic_sums_and_repeat_bit_for_bit(model_dir, model, struct, species, precision):
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     types = np.minimum(types, len(species)).astype(np.int32)
@@ -50,23 +51,32 @@ def test_ordered_sums_equal_atomic_sums_and_repeat_bit_for_bit(model_dir, model,
     fresh = kk.System(m, species, skin=0.0, chunksize=0, precision=precision)
     fresh.engine.set_ordered_sums(True)
     _same_bits(fresh.compute(types, pos, cell, pbc, energies=True), out)
-    # chunks change neither a bond's force nor the order of the sums
+    # GRACE-1L: chunks change neither a bond's force nor the order of the sums.  GRACE-2L: a neighbour's message adjoint is
+    # added chunk by chunk, so a chunked pass equals the one-pass result to rounding, and itself bit for bit
+    one_layer = m.layers == 1
     for cs in (7, 16, n - 1):
         c = kk.System(m, species, skin=0.0, chunksize=cs, precision=precision)
         c.engine.set_ordered_sums(True)
-        _same_bits(c.compute(types, pos, cell, pbc, energies=True), out)
+        first = c.compute(types, pos, cell, pbc, energies=True)
+        if one_layer:
+            _same_bits(first, out)
+        else:
+            _close(first, out, n, 1e-10 if precision == 64 else 2e-6)
+            c.compute(types, pos + 1e-2, cell, pbc)
+            _same_bits(c.compute(types, pos, cell, pbc, energies=True), first)
     eo = s.compute(types, pos, cell, pbc, energy_only=True)
     assert eo["energy"] == out["energy"]
     s.engine.set_ordered_sums(False)                            # and back: the atomic sums again
     _close(s.compute(types, pos, cell, pbc, energies=True), ref, n, 1e-10 if precision == 64 else 2e-6)
 
 
-def test_ordered_sums_of_a_batch(model_dir):
+@pytest.mark.parametrize("model", ["mix2", "l2mix"])
+def test_ordered_sums_of_a_batch(model_dir, model):
     """several structures in one list: a record per structure, summed over its rows in ascending order"""
     structs = workloads.structures_config5(6)
     natoms, types, pos, cells, pbc = workloads.batch_arrays(structs)
     types = np.minimum(types, 2).astype(np.int32)
-    m = kk.Model(cases.model_file(model_dir, "mix2"))
+    m = kk.Model(cases.model_file(model_dir, model))
     ref = kk.Batch(m, ["Mo", "W"], chunksize=0).compute(natoms, types, pos, cells, pbc, energies=True)
     b = kk.Batch(m, ["Mo", "W"], chunksize=0)
     b.engine.set_ordered_sums(True)
@@ -76,7 +86,7 @@ def test_ordered_sums_of_a_batch(model_dir):
     assert np.abs(out["forces"] - ref["forces"]).max() < 1e-9 * fs
     assert np.abs(out["virial"] - ref["virial"]).max() < 1e-8 * fs
     assert np.abs(out["energies"] - ref["energies"]).max() < 1e-9 * fs
-    for cs in (0, 50):
+    for cs in (0, 50) if model == "mix2" else (0,):
         c = kk.Batch(m, ["Mo", "W"], chunksize=cs)
         c.engine.set_ordered_sums(True)
         again = c.compute(natoms, types, pos, cells, pbc, energies=True)
@@ -84,10 +94,11 @@ def test_ordered_sums_of_a_batch(model_dir):
             assert np.array_equal(again[k], out[k]), (cs, k)
 
 
-def test_ordered_sums_with_ghost_atoms(model_dir):
+@pytest.mark.parametrize("model,struct", [("mix2", "alloy54"), ("l2mix", "triclinic")])
+def test_ordered_sums_with_ghost_atoms(model_dir, model, struct):
     """the LAMMPS call: the neighbours of a bond are ghost rows, whose forces are folded onto their owners afterwards"""
-    eng = kk.Engine(kk.Model(cases.model_file(model_dir, "mix2")), ["Mo", "W"], 64)
-    pos, cell, pbc, types = cases.structure_alloy54()
+    eng = kk.Engine(kk.Model(cases.model_file(model_dir, model)), ["Mo", "W"], 64)
+    pos, cell, pbc, types = cases.STRUCTURES[struct]()
     n = len(pos)
     rc = max(eng.cutoff(a, b) for a in (1, 2) for b in (1, 2))
     x, t, owner, rows = lammps_inputs(pos, cell, types, rc + 0.7)
@@ -105,10 +116,35 @@ def test_ordered_sums_with_ghost_atoms(model_dir):
         eng.compute_lammps(*args, owner=owner, vatom=np.zeros((len(x), 6)))
 
 
-def test_only_grace_1l_engines_have_ordered_sums(model_dir):
-    for name in ("l2mix", "l3mix"):
-        eng = kk.Engine(kk.Model(cases.model_file(model_dir, name)), ["Mo", "W"], 64)
-        with pytest.raises(ValueError, match="GRACE-1L engines only"):
-            eng.set_ordered_sums(True)
-        eng.set_ordered_sums(False)
-        assert not eng.ordered_sums
+def test_grace_3l_engines_have_no_ordered_sums(model_dir):
+    eng = kk.Engine(kk.Model(cases.model_file(model_dir, "l3mix")), ["Mo", "W"], 64)
+    with pytest.raises(ValueError, match="GRACE-1L and GRACE-2L engines only"):
+        eng.set_ordered_sums(True)
+    eng.set_ordered_sums(False)
+    assert not eng.ordered_sums
+
+
+@pytest.mark.parametrize("name", ["config2", "config3"])
+def test_full_size_passes_repeat_bit_for_bit(name, tmp_path):
+    """benchmark configurations 2 (GRACE-1L, 8192 atoms) and 3 (GRACE-2L, 32000 atoms, 2.5 M bonds): at this size the atomic
+    sums of two engines rarely agree in every bit; the ordered sums of two engines do, and agree with the atomic ones"""
+    if name == "config2":
+        pos, cell, pbc, types = workloads.structure_config2()
+        path, species = workloads.write_model("config1", str(tmp_path)), ["W"]
+    else:
+        pos, cell, pbc, types = workloads.structure_config3()
+        path, species = workloads.write_model("config3", str(tmp_path)), ["Al", "Co", "Ni", "Ti"]
+    m = kk.Model(path)
+    n = len(pos)
+    ref = kk.System(m, species, skin=0.0, precision=64).compute(types, pos, cell, pbc, energies=True)
+    outs = []
+    for _ in range(2):
+        s = kk.System(m, species, skin=0.0, precision=64)
+        s.engine.set_ordered_sums(True)
+        outs.append(s.compute(types, pos, cell, pbc, energies=True))
+        outs.append(s.compute(types, pos, cell, pbc, energies=True))
+        del s
+    for o in outs[1:]:
+        _same_bits(o, outs[0])
+    _close(outs[0], ref, n, 1e-10)
+    assert np.abs(outs[0]["forces"].sum(axis=0)).max() < 1e-8 * max(1.0, np.abs(ref["forces"]).max()) * np.sqrt(n)
