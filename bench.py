@@ -244,10 +244,9 @@ def main():
             del sysm
     upload()
 
-    # the same passes with ordered (atomic-free) sums of forces, virial, energy and message adjoints (GRACE-1L and 2L
-    # engines): reported beside
+    # the same passes with ordered (atomic-free) sums of forces, virial, energy and message adjoints: reported beside
     ordered_ms = None
-    if not three:
+    if True:
         eng.set_ordered_sums(True)
         eng.run()
         eng.sync()

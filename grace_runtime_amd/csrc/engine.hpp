@@ -129,7 +129,7 @@ class Engine {
   virtual void set_chunksize(int atoms) = 0;
   // ordered sums: forces, virial, energy and message adjoints are added in a fixed order instead of with floating-point
   // atomics, so that two runs on the same input give the same bits (the reference's GPU engines accept last-bit variation
-  // from run to run: python/tests/test_gpu_several_calculators.py).  GRACE-1L and 2L engines; GRACE-3L engines refuse `on`.
+  // from run to run: python/tests/test_gpu_several_calculators.py).
   virtual void set_ordered_sums(bool on) = 0;
   virtual bool ordered_sums() const = 0;
   virtual int chunksize_used() const = 0;

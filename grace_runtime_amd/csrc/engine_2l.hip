@@ -747,7 +747,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
       // ordered sums: the staged kernel without atomics; the message adjoints of the chunk's bonds are gathered afterwards
       PairOrdered<T> po{};
       if (ordered_) {
-        po.gMe = gMe_.as<T>(); po.fedge = fedge_.as<double>(); po.fcen = fcen_.as<double>(); po.e_base = eb;
+        po.gMe = gMe_.as<T>(); po.fedge = fedge_.as<double>(); po.fcen = fcen_.as<double>(); po.e_base = eb; po.ngrp = 1;
       }
       if (ordered_) {
         GR_PAIR_ORD(GR_ARGS)

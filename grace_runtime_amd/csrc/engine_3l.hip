@@ -179,6 +179,7 @@ template<class T> class Engine3L final : public EngineBase {
     build();
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
     chunks_ = true;
+    ordered_ok_ = true;
   }
   int layers() const override { return 3; }
   void run(const RunFlags &fl) override;
@@ -214,6 +215,10 @@ template<class T> class Engine3L final : public EngineBase {
   int comm_reverse_layer_ = 0;    // the message whose adjoint rows gM_ holds while its reverse exchange runs
   // scratch shared by the layers (largest size over the layers): temporaries of the forward pass and all adjoints
   DevBuf M_, gM_, pairP_, gpairP_, A_, gA_, P_, gP_, R2_, R3_, R4_, FA_, FB_, gX_, gR2_, gR3_, gR4_, gFA_, gFB_, gLp_, gRp_, gEQ_;
+  // ordered sums: the message adjoints of a chunk's bonds [bond][nlmi][CP]; the forces and per-atom sums of the slot groups
+  // of a pair kernel, [bond][group][3] and [atom][group][9]; ordered_first_: no layer of this pass has stored its bond forces yet
+  DevBuf gMe_, fpart_, cpart_;
+  bool ordered_first_ = true;
   DevBuf gMin_;    // adjoint of the message the layer in reverse SENT (filled by the layer above); gM_: of the one it gathers
   // the chunk of atoms the layer functions act on: atoms [a0_, a0_ + cn_), their bonds [eb_, eb_ + ecnt_) (ecnt_ < 0: all
   // bonds), the capacities the chunk buffers are sized for, the chunk's element tiles (atoms counted from a0_)
@@ -625,7 +630,7 @@ template<class T> void Engine3L<T>::couple_bwd(ProdStage<T> &p, const T *Lp, int
   }
   const int ATl = 64 / KP;
   const size_t lds = (size_t) ATl * (nfl + nfr) * KP * (sizeof(T) + sizeof(double));
-  if (lds <= kCoupleLdsMax && p.cd.nterms > 0) {
+  if (!ordered_ && lds <= kCoupleLdsMax && p.cd.nterms > 0) {    // ordered sums: the gather form below has no atomics
     auto kern = k_couple_bwd_lds<T>;
     if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
     hipLaunchKernelGGL(kern, dim3((n + ATl - 1) / ATl), dim3(p.cd.nout >= 256 ? 1024 : 256), lds, stream_, p.cd, Lp, Rp, g, gL, gR, KP, nfl, nfr, n);
@@ -662,6 +667,24 @@ static int slots_per_block(int nslot, int CP)
     case 5: GR_PAIR1(K_, 25, __VA_ARGS__) break;             \
     case 6: GR_PAIR1(K_, 36, __VA_ARGS__) break;             \
     default: GR_PAIR1(K_, 49, __VA_ARGS__) break;            \
+  }
+// the staged reverse kernel in its form without floating-point atomics
+#define GR_PAIR_ORD1(N_, grid_, block_, lds_, ...)                                                                       \
+  {                                                                                                                      \
+    auto kern = k_pair_bwd<T, N_, true>;                                                                                 \
+    if (lds_ > 48 * 1024)                                                                                                \
+      HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds_)); \
+    hipLaunchKernelGGL(kern, grid_, block_, lds_, __VA_ARGS__);                                                          \
+  }
+#define GR_PAIR_ORD(...)                                     \
+  switch (nl_) {                                             \
+    case 1: GR_PAIR_ORD1(1, __VA_ARGS__) break;              \
+    case 2: GR_PAIR_ORD1(4, __VA_ARGS__) break;              \
+    case 3: GR_PAIR_ORD1(9, __VA_ARGS__) break;              \
+    case 4: GR_PAIR_ORD1(16, __VA_ARGS__) break;             \
+    case 5: GR_PAIR_ORD1(25, __VA_ARGS__) break;             \
+    case 6: GR_PAIR_ORD1(36, __VA_ARGS__) break;             \
+    default: GR_PAIR_ORD1(49, __VA_ARGS__) break;            \
   }
 // the reverse kernel with asynchronous staging and chunks of CH_ bonds
 #define GR_PAIR_ASYNC1(N_, CH_, grid_, block_, lds_, ...)                                                                \
@@ -915,6 +938,9 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
     ba.Rz = Rl; ba.dRz = dRl; ba.gA = gX;
     ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr(); ba.vatom = vatom_ptr();
     ba.a0 = a0_; ba.C = L.CP; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = L.rad.noutp; ba.sh = sh_;
+    if (ordered_) {
+      ba.fedge = fedge_.as<double>(); ba.fcen = fcen_.as<double>(); ba.ordered_add = ordered_first_ ? 0 : 1;
+    }
     stage(tg(k, "bond_bwd").c_str(), [&] { launch_bond_bwd<T>(ba, n); });
     return;
   }
@@ -935,17 +961,34 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
     // blocks that fill a CU alone, of 4 otherwise); fp64 runs faster with one chunk staged through registers
     const size_t row = (size_t) (pthreads + 2 * L.rad.noutp) * s;
     const int ch = s != 4 ? 0 : (pthreads >= 512 && 16 * row <= kPairLdsMax) ? 8 : 8 * row <= kPairLdsMax ? 4 : 0;
-    const size_t lds = ch ? 2 * ch * row : kPairChunk * row;
+    const size_t lds = ch && !ordered_ ? 2 * ch * row : kPairChunk * row;
+    // ordered sums: the staged kernel without atomics; per slot group the bond forces and the per-atom sums, added in the
+    // order of the groups afterwards; the message adjoints of the chunk's bonds gathered by neighbour atom afterwards
+    PairOrdered<T> po{};
+    if (ordered_) {
+      gMe_.ensure(ecap_ * L.nlmi * L.CP * s);
+      fpart_.ensure((size_t) 3 * std::max<int64_t>(nb_, 1) * ngrp * sizeof(double));
+      cpart_.ensure((size_t) 9 * n_ * ngrp * sizeof(double));
+      po.gMe = gMe_.as<T>(); po.fedge = fpart_.as<double>(); po.fcen = cpart_.as<double>(); po.e_base = eb_; po.ngrp = ngrp;
+    }
 #define GR_ARGS                                                                                                                          \
   dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl, (const T *) dRl,     \
       (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),   \
       scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_, vatom_ptr()
-    if (ch == 8) {
+    if (ordered_) {
+      GR_PAIR_ORD(GR_ARGS, po)
+      const long long nwork = 3 * (long long) (ecnt_ >= 0 ? ecnt_ : std::max<int64_t>(nb_, 1)) + 9ll * n;
+      hipLaunchKernelGGL(k_ordered_combine, dim3((unsigned) ((nwork + 255) / 256)), dim3(256), 0, stream_, (const double *) fpart_.as<double>(),
+                         (const double *) cpart_.as<double>(), ngrp, eb_, (const long long *) (eoff_.as<long long>() + n_), ecnt_, a0_, n, ordered_first_ ? 0 : 1, fedge_.as<double>(),
+                         fcen_.as<double>());
+      hipLaunchKernelGGL(k_ordered_gm<T>, dim3((unsigned) n_nodes_), dim3(std::min(1024, round_up(L.nlmi * L.CP, 64))), 0, stream_,
+                         toff_.as<long long>(), tsorted_.as<int>(), (const T *) gMe_.as<T>(), eb_, (const long long *) (eoff_.as<long long>() + n_), ecnt_, L.nlmi * L.CP, gM_.as<T>());
+    } else if (ch == 8) {
       GR_PAIR_ASYNC(8, GR_ARGS)
     } else if (ch == 4) {
       GR_PAIR_ASYNC(4, GR_ARGS)
     } else {
-      GR_PAIR(k_pair_bwd, GR_ARGS, PairOrdered<T>{})
+      GR_PAIR(k_pair_bwd, GR_ARGS, po)
     }
 #undef GR_ARGS
   });
@@ -972,16 +1015,24 @@ template<class T> double Engine3L<T>::chunk_bytes_per_atom() const
     shared = std::max(shared, spbf + 2.0 * maxP + 2.0 * maxLp + X + 2.0 * R + 2.0 * F + (L.has_eq ? (double) L.EQ.nf * L.EQ.w : 0.0));
     kept += X + proj + eq / 2.0 + 2.0 * bonds * L.rad.noutp;    // every layer keeps its own inputs of the reverse
   }
+  if (ordered_) {    // ordered sums: the message adjoints of the chunk's bonds, widest layer
+    double rows = 0.0;
+    for (int k = 0; k < 3; k++)
+      if (L_[k].equiv) rows = std::max(rows, (double) L_[k].nlmi * L_[k].CP);
+    shared += bonds * rows;
+  }
   return (shared + kept) * sizeof(T);
 }
 
 template<class T> void Engine3L<T>::run(const RunFlags &fl)
 {
   const int n = n_;
+  ordered_check(fl);
   if (!begin_pass(fl)) return;
   const size_t ecap = (size_t) std::max<int64_t>(nb_, 1);
   const long long *n_edges = eoff_.as<long long>() + n;
   const bool forces = !fl.energy_only;
+  if (ordered_ && forces) ordered_begin();
   emi_.ensure(ecap * sizeof(int));
   stage("edge_center", [&] { hipLaunchKernelGGL(k_edge_center, dim3(n), dim3(64), 0, stream_, eoff_.as<long long>(), mu_.as<int>(), emi_.as<int>()); });
   const int yw = forces ? 3 * nlm_ : nlm_;    // row of an edge: Y[nlm] and, for forces, the two tangential gradients D1[nlm], D2[nlm]
@@ -1052,9 +1103,14 @@ template<class T> void Engine3L<T>::run(const RunFlags &fl)
     hipLaunchKernelGGL(k_energy_3l, dim3(n), dim3(64), (size_t) (nrho_ + 2 * en_.nh) * sizeof(double), stream_, en_, mu_.as<int>(),
                        (const double *) L_[0].rho_raw.template as<double>(), (const double *) L_[1].rho_raw.template as<double>(),
                        (const double *) L_[2].rho_raw.template as<double>(), L_[0].grho.template as<double>(), L_[1].grho.template as<double>(),
-                       L_[2].grho.template as<double>(), fl.eatom ? eatom_.as<double>() : nullptr, scal_.as<double>(), forces ? 1 : 0, sid_ptr());
+                       L_[2].grho.template as<double>(), fl.eatom || ordered_ ? eatom_.as<double>() : nullptr, ordered_ ? nullptr : scal_.as<double>(),
+                       forces ? 1 : 0, sid_ptr());
   });
-  if (!forces) return;
+  if (!forces) {
+    if (ordered_) ordered_finish(fl);
+    return;
+  }
+  ordered_first_ = true;
   for (int k = 2; k >= 0; k--) {
     Layer3<T> &L = L_[k];
     if (L.equiv) {
@@ -1067,6 +1123,7 @@ template<class T> void Engine3L<T>::run(const RunFlags &fl)
       if (nchunks > 1) layer_forward(k, forces, yw, true);
       layer_backward(k, yw);
     }
+    ordered_first_ = false;    // the layers below add to the bond forces this one stored
     if (L.equiv) {
       comm_reverse_layer_ = k;
       exchange_reverse(k);    // the ghosts' adjoint rows of the message of layer k go to their owners
@@ -1076,10 +1133,13 @@ template<class T> void Engine3L<T>::run(const RunFlags &fl)
     }
   }
   set_chunk(0);
+  if (ordered_) ordered_finish(fl);
 }
 
 #undef GR_PAIR_ASYNC
 #undef GR_PAIR_ASYNC1
+#undef GR_PAIR_ORD
+#undef GR_PAIR_ORD1
 #undef GR_PAIR
 #undef GR_PAIR1
 

@@ -577,7 +577,7 @@ class EngineBase : public Engine, protected BufRegistry {
   int chunksize_used() const override { return chunk_used_; }
   void set_ordered_sums(bool on) override
   {
-    if (on && !ordered_ok_) throw InvalidArgument(who_ + ": ordered (atomic-free) sums are available for GRACE-1L and GRACE-2L engines only");
+    if (on && !ordered_ok_) throw InvalidArgument(who_ + ": this engine has no ordered (atomic-free) sums");
     ordered_ = on;
   }
   bool ordered_sums() const override { return ordered_; }

@@ -156,13 +156,15 @@ __device__ inline double wave_sum4(double v0, double v1, double v2, double v3, i
 //   dE/dx = sum_{slot,n,l} S_l dR1_l M_j,   g_k = sum_{slot,n,l} T_l,k R1_l M_j
 //   fv = dE/dx / rc rhat + (g_1 e1 + g_2 e2) / r  (= the reference's dE/dx / rc rhat + (g - (g . rhat) rhat) / r with
 //   g the Cartesian sum);  f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv
-// ORD (ordered sums, one slot group): no floating-point atomics.  The message adjoint of bond e goes to
-// ord.gMe[e - ord.e_base][slot][n], the bond's force to ord.fedge[e][3], the sums over the atom's bonds to
-// ord.fcen[a0 + i][9]; the sums over the waves of a block are added in the order of the waves.
+// ORD (ordered sums): no floating-point atomics.  The message adjoint of bond e goes to ord.gMe[e - ord.e_base][slot][n],
+// the force that the block's slot group gives the bond to ord.fedge[e][group][3], the sums over the atom's bonds to
+// ord.fcen[a0 + i][group][9] (ord.ngrp groups: with one group these are the engine's per-bond and per-atom stores, with
+// several k_ordered_combine adds the groups in turn); the sums over the waves of a block are added in the order of the waves.
 template<class T> struct PairOrdered {
   T *gMe;
   double *fedge, *fcen;
   long long e_base;
+  int ngrp;
 };
 template<class T, int NLM, bool ORD = false>
 __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__restrict__ ej, const T *__restrict__ YG,
@@ -248,7 +250,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
       const int jj = ej[e];
       for (int d = 0; d < 3; d++) {
         fi[d] += fv[d];
-        if (ORD) ord.fedge[3 * e + d] = fv[d];
+        if (ORD) ord.fedge[3 * (e * ord.ngrp + grp) + d] = fv[d];
         else atomicAdd(&f[3 * (long long) jj + d], -fv[d]);
       }
       const double ddx = -u[0] * r, ddy = -u[1] * r, ddz = -u[2] * r;
@@ -269,7 +271,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
       for (int o = 32; o > 0; o >>= 1) vsum[k] += __shfl_xor(vsum[k], o, 64);
     if (ORD) {
       if (lane == 0)
-        for (int k = 0; k < 9; k++) ord.fcen[9 * (long long) (a0 + i) + k] = vsum[k];
+        for (int k = 0; k < 9; k++) ord.fcen[9 * ((long long) (a0 + i) * ord.ngrp + grp) + k] = vsum[k];
     } else if (lane == 0 && e1 > e0) {
       for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) (a0 + i) + k], vsum[k]);
       for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[a0 + i] : 0) + k], vsum[3 + k]);
@@ -278,6 +280,29 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
     }
   }
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
+}
+
+// Ordered sums with several slot groups per atom: fedge[e][3] (=, or += with add) the sum over the groups, in their order, of
+// fpart[e][group][3] for the bonds [e_base, e_end), and fcen[i][9] likewise of cpart[i][group][9] for the atoms [a0, a0 + natoms).
+static __global__ void k_ordered_combine(const double *__restrict__ fpart, const double *__restrict__ cpart, int ngrp, long long e_base,
+                                         const long long *__restrict__ e_end_dev, long long e_count, int a0, int natoms, int add,
+                                         double *__restrict__ fedge, double *__restrict__ fcen)
+{
+  const long long e_end = e_count >= 0 ? e_base + e_count : *e_end_dev;
+  const long long ne3 = 3 * (e_end - e_base), t = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (t < ne3) {
+    const long long e = e_base + t / 3;
+    const int d = (int) (t % 3);
+    double s = add ? fedge[3 * e + d] : 0.0;
+    for (int g = 0; g < ngrp; g++) s += fpart[3 * (e * ngrp + g) + d];
+    fedge[3 * e + d] = s;
+  } else if (t < ne3 + 9ll * natoms) {
+    const long long q = t - ne3, i = a0 + q / 9;
+    const int k = (int) (q % 9);
+    double s = add ? fcen[9 * i + k] : 0.0;
+    for (int g = 0; g < ngrp; g++) s += cpart[9 * (i * ngrp + g) + k];
+    fcen[9 * i + k] = s;
+  }
 }
 
 // Ordered sums: gM[j][slot][n] += sum of gMe[e - e_base][slot][n] over the bonds e in [e_base, e_end) that have j as their

@@ -360,7 +360,7 @@ static __global__ void k_energy_3l(Energy3Dev M, const int *mu, const double *rh
   const double Ei = (e * M.norm1 + h[0]) * M.out_scale + M.shift[mu[at]];
   if (lane == 0) {
     if (eatom) eatom[at] = Ei;
-    atomicAdd(energy + (sid ? 8 * sid[at] : 0), Ei);
+    if (energy) atomicAdd(energy + (sid ? 8 * sid[at] : 0), Ei);    // null: ordered sums, the records are added from eatom afterwards
   }
   if (!want_grad) return;
   for (int j = lane; j < M.nh; j += 64) {

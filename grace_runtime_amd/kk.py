@@ -270,8 +270,7 @@ class Engine:
 
     def set_ordered_sums(self, on: bool = True):
         """forces, virial, energy and message adjoints added in a fixed order instead of with floating-point atomics: the
-        same bits on every call with the same input.  GRACE-1L and 2L engines (ValueError for 3L); no per-atom virials in
-        this mode."""
+        same bits on every call with the same input; no per-atom virials in this mode."""
         check(_lib.lib().gr_engine_set_ordered_sums(self._h, 1 if on else 0))
 
     @property

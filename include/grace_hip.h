@@ -293,15 +293,16 @@ int gr_engine_chunksize(const gr_engine *e);
 int gr_system_set_chunksize(gr_system *s, int atoms);
 int gr_system_chunksize(const gr_system *s);
 
-/* Ordered sums: with on != 0 the engine adds forces, virial, energy and (GRACE-2L) the message adjoints in a fixed order
- * instead of with floating-point atomics, so that two calls on the same input return the same bits.  The reverse kernels
- * store every bond's contribution; the forces and message adjoints of the neighbours are gathered through the bonds
- * listed by neighbour atom (rebuilt every pass, each row in ascending order), the energy and virial of every structure
- * are summed over its atoms in ascending order.  The reference's GPU engines have no such mode: they document last-bit
- * variation from run to run (python/tests/test_gpu_several_calculators.py).  GRACE-1L and GRACE-2L engines; GR_INVALID
- * with on != 0 for a GRACE-3L engine.  A GRACE-1L result does not depend on the chunk size; a GRACE-2L result is the
- * same for the same chunk size.  With ordered sums a run with GR_FLAG_VATOM gives GR_INVALID, and so does a batch whose
- * atoms are not grouped by structure.  About 3-5 % slower.  gr_engine_ordered_sums: 1 when on. */
+/* Ordered sums: with on != 0 the engine adds forces, virial, energy and (GRACE-2L / 3L) the message adjoints in a fixed
+ * order instead of with floating-point atomics, so that two calls on the same input return the same bits.  The reverse
+ * kernels store every bond's contribution; the forces and message adjoints of the neighbours are gathered through the
+ * bonds listed by neighbour atom (rebuilt every pass, each row in ascending order), the energy and virial of every
+ * structure are summed over its atoms in ascending order.  The reference's GPU engines have no such mode: they document
+ * last-bit variation from run to run (python/tests/test_gpu_several_calculators.py).  A GRACE-1L result does not depend
+ * on the chunk size; a GRACE-2L / 3L result is the same for the same chunk size.  With ordered sums a run with
+ * GR_FLAG_VATOM gives GR_INVALID, and so does a batch whose atoms are not grouped by structure.  A few per cent slower;
+ * the multi-layer engines hold one more array of nI x channels values per bond of a chunk.  gr_engine_ordered_sums: 1
+ * when on. */
 int gr_engine_set_ordered_sums(gr_engine *e, int on);
 int gr_engine_ordered_sums(const gr_engine *e);
 int gr_system_rebuilds(const gr_system *s);

@@ -67,7 +67,7 @@ class Engine {
   // atoms per pass: > 0 fixed, 0 one pass, -1 from the free device memory (kk/grace_1l_kk.h: chunksize)
   int chunksize = -1;
   // forces, virial and energy added in a fixed order (same bits on every run) instead of with floating-point atomics;
-  // GRACE-1L and 2L models, no per-atom virials (gr_engine_set_ordered_sums)
+  // no per-atom virials in this mode (gr_engine_set_ordered_sums)
   bool ordered_sums = false;
 
   void set_model(const std::string &npz_path, const std::vector<int> &type2mu)

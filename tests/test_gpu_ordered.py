@@ -1,5 +1,5 @@
-"""Ordered (atomic-free) sums of the GRACE-1L and GRACE-2L engines (gr_engine_set_ordered_sums): forces, virial, energy
-and, for 2L, the message adjoints added in a fixed order.  The reference's GPU engines have no such mode and document last-bit variation from run to run
+"""Ordered (atomic-free) sums of the engines (gr_engine_set_ordered_sums): forces, virial, energy and, for GRACE-2L and
+3L, the message adjoints added in a fixed order.  The reference's GPU engines have no such mode and document last-bit variation from run to run
 (python/tests/test_gpu_several_calculators.py); the tests hold the ordered mode to the atomic mode at the parity bounds of
 the other GPU tests (1e-10 eV/atom, 1e-9 eV/A) and to ITSELF bit for bit: repeated calls, a fresh engine, chunked passes."""
 import numpy as np
@@ -31,7 +31,8 @@ def _close(a, b, n, tol):
 
 @pytest.mark.parametrize("precision", [64, 32])
 @pytest.mark.parametrize("model,struct,species", [("mix2", "alloy54", ["Mo", "W"]), ("cut2", "slab", ["Al", "Ni"]), ("config1", "config1", ["W"]),
-                                                  ("l2mix", "alloy54", ["Mo", "W"]), ("l2mix", "slab", ["Mo", "W"]), ("config3", "fcc108", ["Al", "Co", "Ni", "Ti"])])
+                                                  ("l2mix", "alloy54", ["Mo", "W"]), ("l2mix", "slab", ["Mo", "W"]), ("config3", "fcc108", ["Al", "Co", "Ni", "Ti"]),
+                                                  ("l3mix", "alloy54", ["Mo", "W"]), ("l3wide", "fcc108", ["Al", "Ni"]), ("l3el", "alloy54", ["Mo", "W"])])
 def test_ordered_sums_equal_atomic_sums_and_repeat_bit_for_bit(model_dir, model, struct, species, precision):
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     types = np.minimum(types, len(species)).astype(np.int32)
@@ -51,8 +52,8 @@ def test_ordered_sums_equal_atomic_sums_and_repeat_bit_for_bit(model_dir, model,
     fresh = kk.System(m, species, skin=0.0, chunksize=0, precision=precision)
     fresh.engine.set_ordered_sums(True)
     _same_bits(fresh.compute(types, pos, cell, pbc, energies=True), out)
-    # GRACE-1L: chunks change neither a bond's force nor the order of the sums.  GRACE-2L: a neighbour's message adjoint is
-    # added chunk by chunk, so a chunked pass equals the one-pass result to rounding, and itself bit for bit
+    # GRACE-1L: chunks change neither a bond's force nor the order of the sums.  GRACE-2L / 3L: a neighbour's message adjoint
+    # is added chunk by chunk, so a chunked pass equals the one-pass result to rounding, and itself bit for bit
     one_layer = m.layers == 1
     for cs in (7, 16, n - 1):
         c = kk.System(m, species, skin=0.0, chunksize=cs, precision=precision)
@@ -70,7 +71,7 @@ def test_ordered_sums_equal_atomic_sums_and_repeat_bit_for_bit(model_dir, model,
     _close(s.compute(types, pos, cell, pbc, energies=True), ref, n, 1e-10 if precision == 64 else 2e-6)
 
 
-@pytest.mark.parametrize("model", ["mix2", "l2mix"])
+@pytest.mark.parametrize("model", ["mix2", "l2mix", "l3mix"])
 def test_ordered_sums_of_a_batch(model_dir, model):
     """several structures in one list: a record per structure, summed over its rows in ascending order"""
     structs = workloads.structures_config5(6)
@@ -94,7 +95,7 @@ def test_ordered_sums_of_a_batch(model_dir, model):
             assert np.array_equal(again[k], out[k]), (cs, k)
 
 
-@pytest.mark.parametrize("model,struct", [("mix2", "alloy54"), ("l2mix", "triclinic")])
+@pytest.mark.parametrize("model,struct", [("mix2", "alloy54"), ("l2mix", "triclinic"), ("l3mix", "alloy54")])
 def test_ordered_sums_with_ghost_atoms(model_dir, model, struct):
     """the LAMMPS call: the neighbours of a bond are ghost rows, whose forces are folded onto their owners afterwards"""
     eng = kk.Engine(kk.Model(cases.model_file(model_dir, model)), ["Mo", "W"], 64)
@@ -116,24 +117,21 @@ def test_ordered_sums_with_ghost_atoms(model_dir, model, struct):
         eng.compute_lammps(*args, owner=owner, vatom=np.zeros((len(x), 6)))
 
 
-def test_grace_3l_engines_have_no_ordered_sums(model_dir):
-    eng = kk.Engine(kk.Model(cases.model_file(model_dir, "l3mix")), ["Mo", "W"], 64)
-    with pytest.raises(ValueError, match="GRACE-1L and GRACE-2L engines only"):
-        eng.set_ordered_sums(True)
-    eng.set_ordered_sums(False)
-    assert not eng.ordered_sums
-
-
-@pytest.mark.parametrize("name", ["config2", "config3"])
+@pytest.mark.parametrize("name", ["config2", "config3", "config4"])
 def test_full_size_passes_repeat_bit_for_bit(name, tmp_path):
-    """benchmark configurations 2 (GRACE-1L, 8192 atoms) and 3 (GRACE-2L, 32000 atoms, 2.5 M bonds): at this size the atomic
-    sums of two engines rarely agree in every bit; the ordered sums of two engines do, and agree with the atomic ones"""
+    """benchmark configurations 2 (GRACE-1L, 8192 atoms), 3 (GRACE-2L, 32000 atoms, 2.5 M bonds) and the model of 4 (GRACE-3L,
+    lmax 5, 64 channels) on 2000 atoms: at this size the atomic sums of two engines rarely agree in every bit; the ordered
+    sums of two engines do, and agree with the atomic ones"""
     if name == "config2":
         pos, cell, pbc, types = workloads.structure_config2()
         path, species = workloads.write_model("config1", str(tmp_path)), ["W"]
-    else:
+    elif name == "config3":
         pos, cell, pbc, types = workloads.structure_config3()
         path, species = workloads.write_model("config3", str(tmp_path)), ["Al", "Co", "Ni", "Ti"]
+    else:
+        pos, cell, pbc, t89 = workloads.structure_config4(natoms=2000)
+        path = workloads.write_model("config4", str(tmp_path))
+        species, types = workloads.config4_species(kk.Model(path).element_names), workloads.config4_types(t89)
     m = kk.Model(path)
     n = len(pos)
     ref = kk.System(m, species, skin=0.0, precision=64).compute(types, pos, cell, pbc, energies=True)
