@@ -27,7 +27,8 @@ SYMBOLS = [
     "gr_system_create", "gr_system_free", "gr_system_compute", "gr_system_rebuilds", "gr_system_list_on_device",
     "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_batch_uq", "gr_compute_batch_device_uq", "gr_engine_reset", "gr_engine_release_buffers", "gr_set_memory_limit", "gr_memory_in_use", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
     "gr_system_fetch_uq", "gr_engine_atoms_that_fit", "gr_engine_set_exchange", "gr_engine_comm_layers", "gr_engine_comm_width", "gr_engine_pack_forward", "gr_engine_unpack_forward", "gr_engine_pack_reverse", "gr_engine_unpack_reverse", "gr_engine_pack_forward_host", "gr_engine_unpack_forward_host", "gr_engine_pack_reverse_host", "gr_engine_unpack_reverse_host", "gr_engine_set_chunksize", "gr_engine_chunksize", "gr_system_set_chunksize", "gr_system_chunksize",
-    "gr_engine_set_ordered_sums", "gr_engine_ordered_sums",
+    "gr_engine_set_ordered_sums", "gr_engine_ordered_sums", "gr_engine_fetch_cvatom", "gr_system_fetch_cvatom", "gr_lammps_add_cvatom",
+    "gr_lammps_add_cvatom_device",
 ]
 
 
@@ -111,6 +112,10 @@ def lib():
     L.gr_system_fetch_vatom.argtypes = [vp, vp]
     L.gr_lammps_add_vatom.argtypes = [vp, i32, vp]
     L.gr_lammps_add_vatom_device.argtypes = [vp, i32, vp]
+    L.gr_engine_fetch_cvatom.argtypes = [vp, vp]
+    L.gr_system_fetch_cvatom.argtypes = [vp, vp]
+    L.gr_lammps_add_cvatom.argtypes = [vp, i32, vp]
+    L.gr_lammps_add_cvatom_device.argtypes = [vp, i32, vp]
     L.gr_neighbor_build.argtypes = [i64, vp, vp, vp, dbl, i32, C.POINTER(vp)]
     L.gr_nlist_nbonds.restype = i64
     L.gr_nlist_nbonds.argtypes = [vp]

@@ -331,6 +331,14 @@ int gr_engine_fetch_vatom(gr_engine *e, double *vatom)
   });
 }
 
+int gr_engine_fetch_cvatom(gr_engine *e, double *cvatom)
+{
+  return guarded([&] {
+    if (!e || !cvatom) throw grhip::InvalidArgument("null argument");
+    live(e).fetch_vatom(cvatom, 9);
+  });
+}
+
 int gr_model_has_uq(const gr_model *m)
 {
   return m && ((m->m1 && m->m1->uq.has_uq) || (m->m2 && m->m2->uq.has_uq) || (m->m3 && m->m3->uq.has_uq)) ? 1 : 0;
@@ -862,33 +870,46 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
   });
 }
 
+namespace {
+// rows of ncomp components (6: vatom, 9: cvatom) of the last LAMMPS call added to the caller's array
+void lammps_add_virials(gr_engine *e, int nall, double *vatom, int ncomp, bool device)
+{
+  if (!e || !vatom) throw grhip::InvalidArgument("null argument");
+  grhip::Engine &eng = live(e);
+  if (device) {
+    if (e->lmp_nall != nall || !e->lmp_on_device || e->lmp_serial != eng.upload_serial() || !e->lmp)
+      throw grhip::Error("the per-atom virials of the device call follow a gr_compute_lammps_device call with GR_FLAG_VATOM on the same atoms");
+    eng.add_vatom_device(e->lmp->nodes ? nullptr : e->lmp->atom.as<int>(), vatom, ncomp);
+    return;
+  }
+  if (e->lmp_nall != nall || e->lmp_on_device || e->lmp_serial != eng.upload_serial())
+    throw grhip::Error("the per-atom virials follow a gr_compute_lammps call with GR_FLAG_VATOM on the same atoms");
+  const bool nodes = e->lmp_rows.empty();
+  const size_t rows = nodes ? (size_t) nall : e->lmp_rows.size();
+  std::vector<double> v((size_t) ncomp * std::max<size_t>(rows, 1));
+  eng.fetch_vatom(v.data(), ncomp);
+  for (size_t q = 0; q < rows; q++) {
+    const size_t a = nodes ? q : (size_t) e->lmp_rows[q];
+    for (int k = 0; k < ncomp; k++) vatom[(size_t) ncomp * a + k] += v[(size_t) ncomp * q + k];
+  }
+}
+}    // namespace
+
 int gr_lammps_add_vatom(gr_engine *e, int nall, double *vatom)
 {
-  return guarded([&] {
-    if (!e || !vatom) throw grhip::InvalidArgument("null argument");
-    grhip::Engine &eng = live(e);
-    if (e->lmp_nall != nall || e->lmp_on_device || e->lmp_serial != eng.upload_serial())
-      throw grhip::Error("gr_lammps_add_vatom follows a gr_compute_lammps call with GR_FLAG_VATOM on the same atoms");
-    const bool nodes = e->lmp_rows.empty();
-    const size_t rows = nodes ? (size_t) nall : e->lmp_rows.size();
-    std::vector<double> v(6 * std::max<size_t>(rows, 1));
-    eng.fetch_vatom(v.data());
-    for (size_t q = 0; q < rows; q++) {
-      const size_t a = nodes ? q : (size_t) e->lmp_rows[q];
-      for (int k = 0; k < 6; k++) vatom[6 * a + k] += v[6 * q + k];
-    }
-  });
+  return guarded([&] { lammps_add_virials(e, nall, vatom, 6, false); });
 }
-
+int gr_lammps_add_cvatom(gr_engine *e, int nall, double *cvatom)
+{
+  return guarded([&] { lammps_add_virials(e, nall, cvatom, 9, false); });
+}
 int gr_lammps_add_vatom_device(gr_engine *e, int nall, double *vatom)
 {
-  return guarded([&] {
-    if (!e || !vatom) throw grhip::InvalidArgument("null argument");
-    grhip::Engine &eng = live(e);
-    if (e->lmp_nall != nall || !e->lmp_on_device || e->lmp_serial != eng.upload_serial() || !e->lmp)
-      throw grhip::Error("gr_lammps_add_vatom_device follows a gr_compute_lammps_device call with GR_FLAG_VATOM on the same atoms");
-    eng.add_vatom_device(e->lmp->nodes ? nullptr : e->lmp->atom.as<int>(), vatom);
-  });
+  return guarded([&] { lammps_add_virials(e, nall, vatom, 6, true); });
+}
+int gr_lammps_add_cvatom_device(gr_engine *e, int nall, double *cvatom)
+{
+  return guarded([&] { lammps_add_virials(e, nall, cvatom, 9, true); });
 }
 
 int gr_system_create(gr_engine *e, double skin, gr_system **out)
@@ -1093,17 +1114,26 @@ int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *clust
   });
 }
 
+namespace {
+void system_fetch_virials(gr_system *s, double *vatom, int ncomp)
+{
+  if (!s || !s->have) throw grhip::Error("the per-atom virials of a system: no structure has been computed");
+  if (!vatom) throw grhip::InvalidArgument("null argument");
+  const int n = s->n;
+  std::vector<double> v((size_t) ncomp * n);
+  live(s->eng).fetch_vatom(v.data(), ncomp);
+  for (int q = 0; q < n; q++)
+    for (int k = 0; k < ncomp; k++) vatom[(size_t) ncomp * s->perm[q] + k] = v[(size_t) ncomp * q + k];
+}
+}    // namespace
+
 int gr_system_fetch_vatom(gr_system *s, double *vatom)
 {
-  return guarded([&] {
-    if (!s || !s->have) throw grhip::Error("gr_system_fetch_vatom: no structure has been computed");
-    if (!vatom) throw grhip::InvalidArgument("null argument");
-    const int n = s->n;
-    std::vector<double> v((size_t) 6 * n);
-    live(s->eng).fetch_vatom(v.data());
-    for (int q = 0; q < n; q++)
-      for (int k = 0; k < 6; k++) vatom[6 * s->perm[q] + k] = v[6 * (size_t) q + k];
-  });
+  return guarded([&] { system_fetch_virials(s, vatom, 6); });
+}
+int gr_system_fetch_cvatom(gr_system *s, double *cvatom)
+{
+  return guarded([&] { system_fetch_virials(s, cvatom, 9); });
 }
 
 // the list of the last rebuild: sizes, then the arrays (perm [n], offset [n + 1], j [nb], image [nb], shifts [nimages][3])

@@ -105,9 +105,10 @@ class Engine {
   virtual void fetch_add_device(const int *atom, double *energy, double *forces, double *virial, double *eatom) = 0;
   // UQ outputs of the last run with RunFlags::uq, [n] each in the order of the uploaded list (null pointers are skipped)
   // per-atom virials [n_nodes][6] (xx yy zz xy xz yz) of a run with the vatom flag, in the order of the uploaded list; host memory
-  virtual void fetch_vatom(double *vatom) = 0;
+  // ncomp 9: the centroid form, the six components followed by yx zx zy (cvatom of kk/grace_1l_kk.h:94)
+  virtual void fetch_vatom(double *vatom, int ncomp = 6) = 0;
   // the same rows added to a device array: row q of the list goes to row atom[q] (null: row q) of vatom
-  virtual void add_vatom_device(const int *atom, double *vatom) = 0;
+  virtual void add_vatom_device(const int *atom, double *vatom, int ncomp = 6) = 0;
   virtual void fetch_uq(double *gamma, double *sigma, double *cluster) = 0;
   // atoms per engine pass (python/kk/kk_api.h:72-75): 0 all atoms in one pass, < 0 chosen from the free device memory
   // (one pass while it fits, else the largest power of two >= 512 that fits), > 0 as given.  chunksize_used(): atoms per

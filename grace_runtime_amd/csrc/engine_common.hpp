@@ -887,23 +887,31 @@ class EngineBase : public Engine, protected BufRegistry {
     if (virial && ran_forces_)
       for (int k = 0; k < 6; k++) virial[k] = s[1 + k];
   }
-  void fetch_vatom(double *vatom) override
+  void fetch_vatom(double *vatom, int ncomp) override
   {
     HIP_CHECK(hipSetDevice(device_));
+    if (ncomp != 6 && ncomp != 9) throw InvalidArgument("per-atom virials have 6 or 9 components");
     if (!ran_ || !ran_vatom_) throw Error("fetch_vatom() needs a run with the per-atom virial flag (and forces)");
     HIP_CHECK(hipStreamSynchronize(stream_));
     check_zero_bond();
-    if (vatom && n_nodes_ > 0) HIP_CHECK(hipMemcpy(vatom, vatom_.p, sizeof(double) * 6 * n_nodes_, hipMemcpyDeviceToHost));
+    if (!vatom || n_nodes_ <= 0) return;
+    std::vector<double> rows((size_t) 9 * n_nodes_);
+    HIP_CHECK(hipMemcpy(rows.data(), vatom_.p, sizeof(double) * rows.size(), hipMemcpyDeviceToHost));
+    for (size_t q = 0; q < (size_t) n_nodes_; q++)
+      for (int k = 0; k < ncomp; k++) vatom[(size_t) ncomp * q + k] = rows[9 * q + k];
   }
-  void add_vatom_device(const int *atom, double *vatom) override
+  void add_vatom_device(const int *atom, double *vatom, int ncomp) override
   {
+    if (ncomp != 6 && ncomp != 9) throw InvalidArgument("per-atom virials have 6 or 9 components");
     HIP_CHECK(hipSetDevice(device_));
     if (!ran_ || !ran_vatom_) throw Error("per-atom virials need a run with the per-atom virial flag (and forces)");
     if (n_nodes_ > n_ && atom) throw Error("add_vatom_device: a list with ghost atoms keeps the caller's atom order");
     HIP_CHECK(hipStreamSynchronize(stream_));
     check_zero_bond();
-    const long long tot = 6ll * n_nodes_;
-    if (tot > 0) hipLaunchKernelGGL(k_add_rows6, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, atom, n_nodes_, vatom_.as<double>(), vatom);
+    const long long tot = (long long) ncomp * n_nodes_;
+    if (tot > 0)
+      hipLaunchKernelGGL(k_add_rows, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream_, atom, n_nodes_, (const double *) vatom_.as<double>(), 9,
+                         ncomp, vatom);
     HIP_CHECK(hipStreamSynchronize(stream_));
   }
   void fetch_uq(double *gamma, double *sigma, double *cluster) override
@@ -961,8 +969,8 @@ class EngineBase : public Engine, protected BufRegistry {
     ran_forces_ = !fl.energy_only;
     ran_vatom_ = fl.vatom && !fl.energy_only;
     if (ran_vatom_) {
-      vatom_.ensure(std::max<size_t>((size_t) 6 * n_nodes_, 1) * sizeof(double));
-      HIP_CHECK(hipMemsetAsync(vatom_.p, 0, (size_t) 6 * n_nodes_ * sizeof(double), stream_));
+      vatom_.ensure(std::max<size_t>((size_t) 9 * n_nodes_, 1) * sizeof(double));
+      HIP_CHECK(hipMemsetAsync(vatom_.p, 0, (size_t) 9 * n_nodes_ * sizeof(double), stream_));
     }
     ran_eatom_ = fl.eatom;
     ran_uq_ = false;    // set by the engine that evaluates a UQ head
@@ -1307,7 +1315,7 @@ class EngineBase : public Engine, protected BufRegistry {
   // uploaded structure
   int n_nodes_ = 0;           // central atoms and ghosts (= n_ without ghosts)
   uint64_t upload_serial_ = 0;
-  DevBuf vatom_;              // per-atom virials [n_nodes][6] of a pass with the vatom flag
+  DevBuf vatom_;              // per-atom virials [n_nodes][9] (xx yy zz xy xz yz yx zx zy) of a pass with the vatom flag
   bool ran_vatom_ = false;
   double *vatom_ptr() { return ran_vatom_ ? vatom_.as<double>() : nullptr; }
   ExchangeCallbacks exchange_{};

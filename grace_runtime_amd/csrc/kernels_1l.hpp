@@ -257,14 +257,14 @@ static __global__ void k_add_results(const int *atom, int nf, int ne, const doub
   if (eatom && q < ne) eatom[i] += ee[q];
 }
 
-// dst[atom[q]][k] += src[q][k], k < 6 (atom null: row q)
-static __global__ void k_add_rows6(const int *atom, int n, const double *src, double *dst)
+// dst[atom[q]][k] += src[q][k], k < ncomp, for rows of sstride values in src and ncomp values in dst (atom null: row q)
+static __global__ void k_add_rows(const int *atom, int n, const double *src, int sstride, int ncomp, double *dst)
 {
   const long long t = blockIdx.x * (long long) blockDim.x + threadIdx.x;
-  if (t >= 6ll * n) return;
-  const long long q = t / 6;
-  const int k = (int) (t % 6);
-  dst[6 * (atom ? (long long) atom[q] : q) + k] += src[t];
+  if (t >= (long long) ncomp * n) return;
+  const long long q = t / ncomp;
+  const int k = (int) (t % ncomp);
+  dst[ncomp * (atom ? (long long) atom[q] : q) + k] += src[sstride * q + k];
 }
 
 struct Edges {
@@ -1394,7 +1394,7 @@ template<class T> struct BondBwdArgs {
   double *f;                  // [n][3]  (+=, atomics)
   double *virial;             // [6]     (+=, atomics); with sid: record 8 sid[i] of the atom's structure
   const int *sid;             // [n] structure of each atom, or null
-  double *vatom;              // [n][6] per-atom virial (+=, atomics), or null: half of a bond's (-r rhat) (x) fv to each of its atoms
+  double *vatom;              // [n][9] per-atom virial xx yy zz xy xz yz yx zx zy (+=, atomics), or null: half of a bond's (-r rhat) (x) fv to each of its atoms
   // ordered mode (both set, no atomics, vatom null): fedge[e][3] = force of bond e on its central atom; fcen[i][9] = sum of
   // these over the bonds of atom i, then the six virial sums of its bonds; k_ordered_forces / k_ordered_records finish
   double *fedge, *fcen;
@@ -1508,9 +1508,14 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
       vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
       vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
       if (a.vatom) {    // the neighbour's half (add_vatom, libgrace/include/grace/fused_cpu.h:1075-1087); the atom's own below
-        double *vj = a.vatom + 6 * (long long) jj;
+        double *vj = a.vatom + 9 * (long long) jj;
         atomicAdd(vj, 0.5 * ddx * fv[0]); atomicAdd(vj + 1, 0.5 * ddy * fv[1]); atomicAdd(vj + 2, 0.5 * ddz * fv[2]);
         atomicAdd(vj + 3, 0.5 * ddx * fv[1]); atomicAdd(vj + 4, 0.5 * ddx * fv[2]); atomicAdd(vj + 5, 0.5 * ddy * fv[2]);
+        // the components below the diagonal (the centroid form, kk/grace_1l_kk_impl.h:1344-1349), for both atoms of the bond
+        double *vi = a.vatom + 9 * (long long) i;
+        const double yx = 0.5 * ddy * fv[0], zx = 0.5 * ddz * fv[0], zy = 0.5 * ddz * fv[1];
+        atomicAdd(vj + 6, yx); atomicAdd(vj + 7, zx); atomicAdd(vj + 8, zy);
+        atomicAdd(vi + 6, yx); atomicAdd(vi + 7, zx); atomicAdd(vi + 8, zy);
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -1530,7 +1535,7 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
       if (t < 3) atomicAdd(&a.f[3 * (long long) i + t], s);
       else {
         atomicAdd(&a.virial[(a.sid ? 8 * a.sid[i] : 0) + t - 3], s);
-        if (a.vatom) atomicAdd(&a.vatom[6 * (long long) i + t - 3], 0.5 * s);
+        if (a.vatom) atomicAdd(&a.vatom[9 * (long long) i + t - 3], 0.5 * s);
       }
     }
   }

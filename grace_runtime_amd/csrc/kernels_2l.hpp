@@ -257,9 +257,14 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
       vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
       vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
       if (!ORD && vatom) {    // per-atom virial: the neighbour's half of this bond (fused_cpu.h:1075-1087 of the reference)
-        double *vj = vatom + 6 * (long long) jj;
+        double *vj = vatom + 9 * (long long) jj;
         atomicAdd(vj, 0.5 * ddx * fv[0]); atomicAdd(vj + 1, 0.5 * ddy * fv[1]); atomicAdd(vj + 2, 0.5 * ddz * fv[2]);
         atomicAdd(vj + 3, 0.5 * ddx * fv[1]); atomicAdd(vj + 4, 0.5 * ddx * fv[2]); atomicAdd(vj + 5, 0.5 * ddy * fv[2]);
+        // the components below the diagonal (the centroid form, kk/grace_1l_kk_impl.h:1344-1349), for both atoms of the bond
+        double *vi = vatom + 9 * (long long) (a0 + i);
+        const double yx = 0.5 * ddy * fv[0], zx = 0.5 * ddz * fv[0], zy = 0.5 * ddz * fv[1];
+        atomicAdd(vj + 6, yx); atomicAdd(vj + 7, zx); atomicAdd(vj + 8, zy);
+        atomicAdd(vi + 6, yx); atomicAdd(vi + 7, zx); atomicAdd(vi + 8, zy);
       }
     }
   }
@@ -276,7 +281,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
       for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) (a0 + i) + k], vsum[k]);
       for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[a0 + i] : 0) + k], vsum[3 + k]);
       if (vatom)
-        for (int k = 0; k < 6; k++) atomicAdd(&vatom[6 * (long long) (a0 + i) + k], 0.5 * vsum[3 + k]);
+        for (int k = 0; k < 6; k++) atomicAdd(&vatom[9 * (long long) (a0 + i) + k], 0.5 * vsum[3 + k]);
     }
   }
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
@@ -531,9 +536,14 @@ __global__ void k_pair_bwd_async(const long long *__restrict__ eoff, const int *
       vir[0] += ddx * fv[0]; vir[1] += ddy * fv[1]; vir[2] += ddz * fv[2];
       vir[3] += ddx * fv[1]; vir[4] += ddx * fv[2]; vir[5] += ddy * fv[2];
       if (vatom) {    // per-atom virial: the neighbour's half of this bond (fused_cpu.h:1075-1087 of the reference)
-        double *vj = vatom + 6 * (long long) jj;
+        double *vj = vatom + 9 * (long long) jj;
         atomicAdd(vj, 0.5 * ddx * fv[0]); atomicAdd(vj + 1, 0.5 * ddy * fv[1]); atomicAdd(vj + 2, 0.5 * ddz * fv[2]);
         atomicAdd(vj + 3, 0.5 * ddx * fv[1]); atomicAdd(vj + 4, 0.5 * ddx * fv[2]); atomicAdd(vj + 5, 0.5 * ddy * fv[2]);
+        // the components below the diagonal (the centroid form, kk/grace_1l_kk_impl.h:1344-1349), for both atoms of the bond
+        double *vi = vatom + 9 * (long long) (a0 + i);
+        const double yx = 0.5 * ddy * fv[0], zx = 0.5 * ddz * fv[0], zy = 0.5 * ddz * fv[1];
+        atomicAdd(vj + 6, yx); atomicAdd(vj + 7, zx); atomicAdd(vj + 8, zy);
+        atomicAdd(vi + 6, yx); atomicAdd(vi + 7, zx); atomicAdd(vi + 8, zy);
       }
     }
   }
@@ -546,7 +556,7 @@ __global__ void k_pair_bwd_async(const long long *__restrict__ eoff, const int *
       for (int k = 0; k < 3; k++) atomicAdd(&f[3 * (long long) (a0 + i) + k], vsum[k]);
       for (int k = 0; k < 6; k++) atomicAdd(&virial[(sid ? 8 * sid[a0 + i] : 0) + k], vsum[3 + k]);
       if (vatom)
-        for (int k = 0; k < 6; k++) atomicAdd(&vatom[6 * (long long) (a0 + i) + k], 0.5 * vsum[3 + k]);
+        for (int k = 0; k < 6; k++) atomicAdd(&vatom[9 * (long long) (a0 + i) + k], 0.5 * vsum[3 + k]);
     }
   }
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive

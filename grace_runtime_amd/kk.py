@@ -322,11 +322,11 @@ class Engine:
         return n, (types, offset, j, rij, positions, image, shifts), nimg
 
     def compute_lammps(self, nlocal, types, x, ilist, numneigh, firstneigh, owner=None, neighmask=0x1FFFFFFF, energies=False,
-                       energy_only=False, forces=None, eatom=None, vatom=None):
+                       energy_only=False, forces=None, eatom=None, vatom=None, cvatom=None):
         """The call of a LAMMPS pair style (gr_compute_lammps): owned + ghost atoms `x[nall, 3]`, `types[nall]`, the full
         neighbour list as `numneigh[nlocal]` and a list of index arrays `firstneigh[i]`, `owner[nall]` the owned atom of every
         ghost.  Forces are ADDED to `forces[nall, 3]` (zeros when not given), per-atom energies to `eatom[nall]`, per-atom
-        virials to `vatom[nall, 6]` when given."""
+        virials to `vatom[nall, 6]` and, in the centroid form xx yy zz xy xz yz yx zx zy, to `cvatom[nall, 9]` when given."""
         types = as_array(types, np.int32)
         x = as_array(x, np.float64, 3)
         nall = types.shape[0]
@@ -338,7 +338,8 @@ class Engine:
         f = np.zeros((nall, 3)) if forces is None else forces
         ea = (np.zeros(nall) if eatom is None else eatom) if energies else None
         e, v = C.c_double(), np.zeros(6)
-        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (_lib.FLAG_VATOM if vatom is not None else 0)
+        want_v = vatom is not None or cvatom is not None
+        flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if energies else 0) | (_lib.FLAG_VATOM if want_v else 0)
         check(_lib.lib().gr_compute_lammps(self._h, int(nlocal), nall, ptr(types), ptr(x), ilist.shape[0], ptr(ilist), ptr(numneigh), fn,
                                            int(neighmask), ptr(own) if own is not None else None, flags, C.byref(e),
                                            None if energy_only else ptr(f), ptr(v), ptr(ea) if ea is not None else None))
@@ -346,6 +347,9 @@ class Engine:
         if vatom is not None:
             check(_lib.lib().gr_lammps_add_vatom(self._h, nall, ptr(vatom)))
             out["vatom"] = vatom
+        if cvatom is not None:
+            check(_lib.lib().gr_lammps_add_cvatom(self._h, nall, ptr(cvatom)))
+            out["cvatom"] = cvatom
         if not energy_only:
             out["forces"], out["virial"] = f, v
         if energies:
@@ -353,7 +357,7 @@ class Engine:
         return out
 
     def compute_lammps_device(self, nlocal, types, x, ilist, numneigh, neighbors, owner=None, neighmask=0x1FFFFFFF, energy_only=False,
-                              forces=None, eatom=None, same_list=False, vatom=None):
+                              forces=None, eatom=None, same_list=False, vatom=None, cvatom=None):
         """The call of a KOKKOS pair style (gr_compute_lammps_device): every array is a device array of the module's GPU
         (torch tensors): `types[nall]` int32, `x[nall, 3]`, `ilist[inum]`, `numneigh[nlocal]`, the 2-d neighbour view
         `neighbors[nlocal, maxneigh]` in either layout, `owner[nall]`.  Forces are ADDED to `forces[nall, 3]` and per-atom
@@ -373,13 +377,16 @@ class Engine:
         p_ea = _device_pointer(eatom, "eatom", (nall,), "float64") if eatom is not None else None
         e, v = C.c_double(), np.zeros(6)
         flags = (FLAG_ENERGY_ONLY if energy_only else 0) | (FLAG_EATOM if eatom is not None else 0) | (_lib.FLAG_SAME_LIST if same_list else 0) | \
-            (_lib.FLAG_VATOM if vatom is not None else 0)
+            (_lib.FLAG_VATOM if vatom is not None or cvatom is not None else 0)
         p_va = _device_pointer(vatom, "vatom", (nall, 6), "float64") if vatom is not None else None
+        p_cva = _device_pointer(cvatom, "cvatom", (nall, 9), "float64") if cvatom is not None else None
         check(_lib.lib().gr_compute_lammps_device(self._h, int(nlocal), nall, len(self.species), p_t, p_x, inum, p_il, p_nn,
                                                   C.c_void_p(neighbors.data_ptr()), int(neighbors.stride(0)), int(neighbors.stride(1)),
                                                   int(neighmask), p_own, flags, C.byref(e), None if energy_only else p_f, ptr(v), p_ea))
         if vatom is not None:
             check(_lib.lib().gr_lammps_add_vatom_device(self._h, nall, p_va))
+        if cvatom is not None:
+            check(_lib.lib().gr_lammps_add_cvatom_device(self._h, nall, p_cva))
         out = {"energy": e.value}
         if not energy_only:
             out["virial"] = v
@@ -422,6 +429,13 @@ class Engine:
         (Outputs::vatom, libgrace/include/grace/system.h:71): half of every bond's virial to each of its two atoms"""
         v = np.zeros((self._n if rows is None else int(rows), 6))
         check(_lib.lib().gr_engine_fetch_vatom(self._h, ptr(v)))
+        return v
+
+    def fetch_cvatom(self, rows=None):
+        """the same rows in the centroid form [rows, 9] = xx yy zz xy xz yz yx zx zy (cvatom of the reference's GPU engines,
+        libgrace/include/grace/kk/grace_1l_kk.h:94)"""
+        v = np.zeros((self._n if rows is None else int(rows), 9))
+        check(_lib.lib().gr_engine_fetch_cvatom(self._h, ptr(v)))
         return v
 
     def fetch_uq(self):
@@ -641,7 +655,7 @@ class System:
     def compute(self, types, positions, cell, pbc, energies=False, uq=False, energy_only=False, virials=False):
         """energy, forces [n, 3], virial [6], energies [n]; with `uq` also gamma, atomic_sigma, gmm_cluster [n] of the
         model's UQ head (ValueError when the model has none that can be evaluated); with `virials` the per-atom virials
-        [n, 6] (the reference's vatom)."""
+        [n, 6] (the reference's vatom) and `centroid_virials` [n, 9] = xx yy zz xy xz yz yx zx zy (its cvatom)."""
         types = as_array(types, np.int32)
         pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
         cell = np.ascontiguousarray(cell, dtype=np.float64).reshape(3, 3)
@@ -674,6 +688,9 @@ class System:
             va = np.zeros((n, 6))
             check(_lib.lib().gr_system_fetch_vatom(self._h, ptr(va)))
             res["virials"] = va
+            cva = np.zeros((n, 9))
+            check(_lib.lib().gr_system_fetch_cvatom(self._h, ptr(cva)))
+            res["centroid_virials"] = cva
         return res
 
 

@@ -37,7 +37,8 @@ enum {
   GR_FLAG_VATOM = 32,      /* ComputeFlags::vflag_atom (system.h:115): per-atom virials, Outputs::vatom (system.h:71): every bond's
                               virial (x_i - x_j) (x) f_i goes half to each of its two atoms (add_vatom, libgrace/include/grace/
                               fused_cpu.h:1075-1087), so the rows add up to the total virial.  Needs forces.  The rows are read
-                              with gr_engine_fetch_vatom / gr_system_fetch_vatom / gr_lammps_add_vatom after the call */
+                              with gr_engine_fetch_vatom / gr_system_fetch_vatom / gr_lammps_add_vatom after the call, or in
+                              the nine-component centroid form with the _cvatom calls */
   GR_FLAG_SAME_LIST = 16   /* gr_compute_lammps_device: atom counts, types, ilist, neighbour list and owner map are those of the
                               previous call on this engine and only x has changed (LAMMPS: neighbor->ago > 0, the steps between
                               two reneighbourings): the converted list is kept, only the bond vectors are renewed and no array
@@ -192,9 +193,16 @@ int gr_engine_fetch_uq(gr_engine *e, double *gamma, double *sigma, double *clust
  * rows in the order of the uploaded list (with ghost atoms as nodes: all of them); Outputs::vatom of the reference
  * (libgrace/include/grace/system.h:71).  GR_ERROR when that pass did not compute them. */
 int gr_engine_fetch_vatom(gr_engine *e, double *vatom);
+/* The same pass in the centroid form [atoms][9] = xx yy zz xy xz yz yx zx zy: the tensor (x_i - x_j) (x) f_i of every
+ * bond is not symmetric, and this form keeps the components below the diagonal as well (RunInput::cvatom of the
+ * reference's GPU engines, libgrace/include/grace/kk/grace_1l_kk.h:94, accumulated in kk/grace_1l_kk_impl.h:1344-1362).
+ * The first six columns are those of gr_engine_fetch_vatom. */
+int gr_engine_fetch_cvatom(gr_engine *e, double *cvatom);
 int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *cluster);
 /* Per-atom virials [n][6] of the last gr_system_compute with GR_FLAG_VATOM, in the caller's atom order. */
 int gr_system_fetch_vatom(gr_system *s, double *vatom);
+/* The same in the centroid form [n][9] (gr_engine_fetch_cvatom). */
+int gr_system_fetch_cvatom(gr_system *s, double *cvatom);
 
 /* The call of a LAMMPS pair style on one MPI rank: owned and ghost atoms with LAMMPS' full neighbour list.  Replaces
  * Grace{1,2,3}LFused::compute<LammpsBonds>(inum, ilist, n_nodes, nmax_nodes, LammpsBonds{x, type, numneigh, firstneigh,
@@ -262,6 +270,10 @@ int gr_compute_lammps_device(gr_engine *e, int nlocal, int nall, int ntypes, con
  * rows; without one (nodes) they stay on the ghosts for LAMMPS' reverse communication. */
 int gr_lammps_add_vatom(gr_engine *e, int nall, double *vatom);
 int gr_lammps_add_vatom_device(gr_engine *e, int nall, double *vatom);
+/* The same for the centroid form, cvatom [nall][9] = xx yy zz xy xz yz yx zx zy (RunInput::cvatom,
+ * libgrace/include/grace/kk/grace_1l_kk.h:94): host array / device array. */
+int gr_lammps_add_cvatom(gr_engine *e, int nall, double *cvatom);
+int gr_lammps_add_cvatom_device(gr_engine *e, int nall, double *cvatom);
 
 /* One structure resident on the device with a Verlet list at cutoff + skin: System of the reference's GPU module
  * (python/kk/kk_api.h:66-93, System::compute python/kk/kk_core.cpp:802-958; list policy python/grace_runtime/

@@ -46,6 +46,8 @@ struct RunInput {
   double *eatom = nullptr;            // [nall], per-atom energies are ADDED (with eflag_atom)
   int vflag_atom = 0;
   double *vatom = nullptr;            // [nall][6] xx yy zz xy xz yz, per-atom virials are ADDED (with vflag_atom)
+  int cvflag_atom = 0;
+  double *cvatom = nullptr;           // [nall][9] xx yy zz xy xz yz yx zx zy, centroid form, ADDED (with cvflag_atom)
 };
 struct RunOutput {
   double eng_vdwl = 0.0;
@@ -98,11 +100,12 @@ class Engine {
     if (in.energy_only) flags |= GR_FLAG_ENERGY_ONLY;
     if (in.eflag_atom && in.eatom) flags |= GR_FLAG_EATOM;
     if (in.same_list) flags |= GR_FLAG_SAME_LIST;
-    const bool vatom = in.vflag_atom && in.vatom && !in.energy_only;
-    if (vatom) flags |= GR_FLAG_VATOM;
+    const bool vatom = in.vflag_atom && in.vatom && !in.energy_only, cvatom = in.cvflag_atom && in.cvatom && !in.energy_only;
+    if (vatom || cvatom) flags |= GR_FLAG_VATOM;
     check(gr_compute_lammps_device(engine_, in.nlocal, in.nall, in.ntypes, in.type, in.x, in.inum, in.ilist, in.numneigh, in.neighbors,
                                    in.stride_i, in.stride_k, in.neighmask, in.owner, flags, &out.eng_vdwl, in.f, out.virial, in.eatom));
     if (vatom) check(gr_lammps_add_vatom_device(engine_, in.nall, in.vatom));
+    if (cvatom) check(gr_lammps_add_cvatom_device(engine_, in.nall, in.cvatom));
     return out;
   }
 

@@ -451,6 +451,7 @@ def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=Tru
     forces = np.zeros((n, 3))
     virial = np.zeros(6)
     virials = np.zeros((n, 6))
+    lower = np.zeros((n, 3))    # yx zx zy of the centroid form (cvatom of the GPU engines: kk/grace_1l_kk_impl.h:1344-1362)
     uqv = [np.zeros(n), np.zeros(n), np.zeros(n)] if uq else None
     feats = np.zeros((n, model.uq_D)) if uq else None
     for a0 in range(0, n, chunk):
@@ -507,7 +508,11 @@ def compute_1l(model: Model1L, mu, offset, j, rij, *, chunk=512, want_forces=Tru
         virial += v6.sum(0)
         np.add.at(virials, bi, 0.5 * v6)                                         # add_vatom, fused_cpu.h:1075-1087: half to each atom
         np.add.at(virials, bj, 0.5 * v6)
-    out = {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial, "virials": virials}
+        l3 = 0.5 * np.stack([dl[:, 1] * fv[:, 0], dl[:, 2] * fv[:, 0], dl[:, 2] * fv[:, 1]], axis=1)    # v6 v7 v8 of kk/grace_1l_kk_impl.h:1346
+        np.add.at(lower, bi, l3)
+        np.add.at(lower, bj, l3)
+    out = {"energy": float(energies.sum()), "energies": energies, "forces": forces, "virial": virial, "virials": virials,
+           "centroid_virials": np.concatenate([virials, lower], axis=1)}
     if uq:
         out.update(gamma=uqv[0], atomic_sigma=uqv[1], gmm_cluster=uqv[2], uq_features=feats)
     return out

@@ -65,7 +65,7 @@ def test_virials_of_a_system_in_chunks_and_through_the_lammps_calls(model_dir, m
     out = eng.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows, owner=owner, vatom=v0.copy())
     assert np.abs(out["vatom"][:n] - v0[:n] - va).max() < 1e-9 * max(1.0, np.abs(va).max())
     assert np.array_equal(out["vatom"][n:], v0[n:])
-    with pytest.raises(RuntimeError, match="follows a gr_compute_lammps"):
+    with pytest.raises(RuntimeError, match="follow a gr_compute_lammps_device call"):
         kk._lib.check(kk._lib.lib().gr_lammps_add_vatom_device(eng._h, len(x), v0.ctypes.data))
     # device arrays
     dev = torch.device("cuda", 0)
@@ -79,3 +79,66 @@ def test_virials_of_a_system_in_chunks_and_through_the_lammps_calls(model_dir, m
                               owner=torch.as_tensor(owner, device=dev), forces=f, vatom=vd)
     assert np.abs(vd.cpu().numpy()[:n] - v0[:n] - va).max() < 1e-9 * max(1.0, np.abs(va).max())
     assert np.array_equal(vd.cpu().numpy()[n:], v0[n:])
+
+
+@pytest.mark.parametrize("precision", [64, 32])
+@pytest.mark.parametrize("model", ["mix2", "l2mix", "l3mix"])
+def test_centroid_form(model_dir, model, precision):
+    """cvatom of the reference's GPU engines (kk/grace_1l_kk.h:94; kk/grace_1l_kk_impl.h:1344-1362): the six components of
+    vatom followed by yx zx zy.  The lower three are held to the upper three of the same structure with its axes exchanged
+    (the upper three are pinned by the reference's vatom), to the 1L oracle's centroid rows, and to the symmetric total."""
+    from test_vatom import permuted_centroid
+    mdl = kk.Model(cases.model_file(model_dir, model))
+    pos, cell, pbc, types = cases.structure_alloy54()
+    n = len(pos)
+    tol = 1e-9 if precision == 64 else 2e-5
+    s = kk.System(mdl, ["Mo", "W"], skin=0.0, chunksize=0, precision=precision)
+    one = s.compute(types, pos, cell, pbc, virials=True)
+    cv = one["centroid_virials"]
+    scale = max(1.0, np.abs(cv).max())
+    assert cv.shape == (n, 9) and np.array_equal(cv[:, :6], one["virials"])
+    assert np.abs(cv[:, 6:] - cv[:, 3:6]).max() > 1e-6
+    tot = cv.sum(0)
+    assert np.abs(tot[6:] - tot[3:6]).max() < tol * max(1.0, np.abs(tot).max()) * 10
+    for p in ([1, 0, 2], [1, 2, 0]):
+        outp = s.compute(types, pos[:, p], cell[:, p], pbc, virials=True)
+        assert abs(outp["energy"] - one["energy"]) < tol * max(1.0, abs(one["energy"]))
+        assert np.abs(outp["centroid_virials"] - permuted_centroid(cv, p)).max() < tol * scale
+    chunked = kk.System(mdl, ["Mo", "W"], skin=0.0, chunksize=13, precision=precision).compute(types, pos, cell, pbc, virials=True)
+    assert np.abs(chunked["centroid_virials"] - cv).max() < tol * scale
+    s.compute(types, pos, cell, pbc)                                       # the list of the structure as given again
+    if model == "mix2":
+        m, compute = _oracle(model_dir, model)
+        perm, offset, j, image, shifts = s.neighbor_list()
+        rij = cases.bond_vectors(pos, perm, offset, j, image, shifts)
+        want = compute(m, types[perm] - 1, offset, j, rij)["centroid_virials"]
+        assert np.abs(cv[perm] - want).max() < tol * scale
+    # the LAMMPS calls: rows are ADDED, ghosts' halves on their owners
+    eng = kk.Engine(mdl, ["Mo", "W"], precision)
+    rcut = max(eng.cutoff(a, b) for a in (1, 2) for b in (1, 2))
+    x, t, owner, rows = lammps_inputs(pos, cell, types, rcut + 0.4)
+    v0 = np.random.default_rng(5).standard_normal((len(x), 9))
+    out = eng.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows, owner=owner, cvatom=v0.copy())
+    assert np.abs(out["cvatom"][:n] - v0[:n] - cv).max() < tol * scale
+    assert np.array_equal(out["cvatom"][n:], v0[n:])
+    import torch
+    dev = torch.device("cuda", 0)
+    nbh = np.zeros((n, max(len(r) for r in rows)), np.int32)
+    for i, r in enumerate(rows):
+        nbh[i, :len(r)] = r
+    vd = torch.as_tensor(v0.copy(), device=dev)
+    f = torch.zeros((len(x), 3), dtype=torch.float64, device=dev)
+    eng.compute_lammps_device(n, torch.as_tensor(t, device=dev), torch.as_tensor(x, device=dev), torch.arange(n, dtype=torch.int32, device=dev),
+                              torch.as_tensor(np.array([len(r) for r in rows], np.int32), device=dev), torch.as_tensor(nbh, device=dev),
+                              owner=torch.as_tensor(owner, device=dev), forces=f, cvatom=vd)
+    assert np.abs(vd.cpu().numpy()[:n] - v0[:n] - cv).max() < tol * scale
+    assert np.array_equal(vd.cpu().numpy()[n:], v0[n:])
+    # the rows of the engine call
+    eng.upload(*_csr(s, types, pos))
+    eng.run(virials=True)
+    assert np.abs(eng.fetch_cvatom()[np.argsort(s.neighbor_list()[0])] - cv).max() < tol * scale
+
+
+def _csr(system, types, pos):
+    perm, offset, j, image, shifts = system.neighbor_list()
+    return types[perm], offset, j, cases.bond_vectors(pos, perm, offset, j, image, shifts)

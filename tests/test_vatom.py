@@ -75,3 +75,39 @@ def test_virials_from_bond_forces_by_differences(model_dir):
     np.add.at(rows, j, v6)
     assert np.abs(rows).max() > 1e-3
     assert np.abs(rows - out["virials"]).max() < 1e-12 * max(1.0, np.abs(rows).max())
+
+
+# index of component (a, b) in the centroid form xx yy zz xy xz yz yx zx zy (cvatom, kk/grace_1l_kk_impl.h:1344-1362)
+CENTROID = {(0, 0): 0, (1, 1): 1, (2, 2): 2, (0, 1): 3, (0, 2): 4, (1, 2): 5, (1, 0): 6, (2, 0): 7, (2, 1): 8}
+
+
+def permuted_centroid(cv, p):
+    """the centroid rows of the structure with axes x'_a = x_p[a]: W'_ab = W_p[a]p[b]"""
+    out = np.empty_like(cv)
+    for (a, b), k in CENTROID.items():
+        out[:, k] = cv[:, CENTROID[(p[a], p[b])]]
+    return out
+
+
+def test_centroid_form_of_the_1l_oracle(model_dir, gold):
+    """the three components below the diagonal: equal to those above it of the structure with its axes exchanged (the model
+    is invariant under any permutation of the axes), and the nine columns add up to the full tensor sum dl (x) f"""
+    model, struct = "mix2", "alloy54"
+    m, compute = _oracle(model_dir, model)
+    pos, cell, pbc, types = cases.STRUCTURES[struct]()
+    tag = f"e2e/{model}/{struct}"
+    key = f"nl/{struct}@{float(gold[tag + '/rc_list']):g}"
+    perm, offset, j, image, shifts = (gold[f"{key}/{k}"] for k in ("perm", "offset", "j", "image", "shifts"))
+    rij = cases.bond_vectors(pos, perm, offset, j, image, shifts)
+    out = compute(m, types[perm] - 1, offset, j, rij)
+    cv = out["centroid_virials"]
+    assert cv.shape == (len(pos), 9) and np.array_equal(cv[:, :6], out["virials"])
+    assert np.abs(cv[:, 6:] - cv[:, 3:6]).max() > 1e-6          # a bond's tensor is not symmetric: the lower half says something
+    scale = max(1.0, np.abs(cv).max())
+    for p in ([1, 0, 2], [1, 2, 0], [2, 1, 0]):
+        outp = compute(m, types[perm] - 1, offset, j, rij[:, p])
+        assert abs(outp["energy"] - out["energy"]) < 1e-10 * max(1.0, abs(out["energy"]))
+        assert np.abs(outp["centroid_virials"] - permuted_centroid(cv, p)).max() < 1e-10 * scale
+    # the total tensor is symmetric (rotational invariance of the energy) although the rows are not
+    tot = cv.sum(0)
+    assert np.abs(tot[6:] - tot[3:6]).max() < 1e-9 * max(1.0, np.abs(tot).max())
