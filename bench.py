@@ -70,6 +70,10 @@ def stage_model(name, ms, E, N, C, nl, nlm, s, prec, dense_flops, nslot=5, nI=4,
         # geometry, forces
         by = E * (2 * s * C * nl + 3 * s * nlm + nslot * C * s + 2 * nI * C * s + 28 + 24) + N * (nslot * nlm * C * s + 24)
         return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
+    if name in ("radial_mlp", "radial_R", "radial_R1") and radial_flops == 0.0:
+        # radial tables: per edge x and the neighbour element read, one row of values and one of derivatives written
+        by = E * (12 + 2 * s * C * nl)
+        return {"bound": "hbm", "achieved": by / (ms * 1e-3) / 1e9, "peak": HBM_PEAK, "unit": "GB/s", "work": by}
     if name in ("radial_mlp", "radial_R", "radial_R1"):
         # value + tangent through the 3 layers: 2 * 2 * E * sum n_in n_out
         fl = radial_flops * E
@@ -117,6 +121,8 @@ def main():
     ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5"])
     ap.add_argument("--reps", type=int, default=0, help="supercell repetitions (default: 16 bcc cells / 20 fcc cells per edge)")
     ap.add_argument("--atoms", type=int, default=10000, help="atoms of the amorphous cube of config4")
+    ap.add_argument("--spline", type=int, default=0, help="intervals of the radial tables of the GRACE-1L / 2L engines (the reference's engines "
+                                                            "use 1024); 0: the radial MLP is evaluated for every bond")
     ap.add_argument("--chunksize", type=int, default=-1, help="atoms per engine pass: -1 chosen from the free device memory (one pass when "
                                                               "the structure fits), 0 one pass, > 0 fixed")
     a = ap.parse_args()
@@ -166,6 +172,7 @@ def main():
     eng = kk.Engine(model, species, precision=a.precision)
     create_s = time.perf_counter() - t1        # includes the run-time compilation of the model-specialised product kernels
     eng.set_chunksize(a.chunksize)
+    eng.set_spline(a.spline)
     if batch:
         def upload():
             eng.upload_batch(structs, 6.0)
@@ -257,6 +264,19 @@ def main():
         ordered_ms = (time.perf_counter() - t1) / a.steps * 1e3
         eng.set_ordered_sums(False)
 
+    # the same passes with the radial functions from tables of 1024 intervals, as the reference's engines take them (1L / 2L)
+    spline_ms = None
+    if not three and a.spline == 0:
+        eng.set_spline(1024)
+        eng.run()
+        eng.sync()
+        t1 = time.perf_counter()
+        for _ in range(a.steps):
+            eng.run()
+        eng.sync()
+        spline_ms = (time.perf_counter() - t1) / a.steps * 1e3
+        eng.set_spline(0)
+
     # per-stage durations: HIP events around every launch on the engine's stream, averaged over the same K steps
     eng.set_profile(True)
     acc = {}
@@ -272,6 +292,8 @@ def main():
     # GRACE-3L: message functions gathered by the pair kernels of layers 2 and 3; radial MLP 8-128-128-384, value + tangent
     extra = dict(radial_flops=4.0 * (8 * 128 + 128 * 128 + 128 * 384), slots={"2": 36, "3": 72},
                  stream_bytes=couple_stream_bytes(workloads.model_config4(), N, s)) if three else {}
+    if a.spline > 0 and not three:
+        extra = dict(radial_flops=0.0)    # the radial stages are table look-ups: a stream, not a GEMM
     # FC / reduce tile GEMMs: flops of the live functions as the engine counts them
     dense_flops = dict(gemm_flops)
     roof = {}
@@ -295,7 +317,7 @@ def main():
     d = modelled[dom]
     roofline = {"kernel": dom, "bound": d["bound"], "achieved": round(d["achieved"], 3), "peak": d["peak"],
                 "unit": d["unit"], "frac": round(d["frac"], 4),
-                "traffic": MEASURED_TRAFFIC.get((a.workload, dom)) if reps == (20 if two else 16) and a.atoms == 10000 and a.precision == 64 else None,
+                "traffic": MEASURED_TRAFFIC.get((a.workload, dom)) if reps == (20 if two else 16) and a.atoms == 10000 and a.precision == 64 and a.spline == 0 else None,
                 "avg_ms": round(d["ms"], 4), "algorithmic_work": d["work"]}
 
     cpu = None
@@ -360,6 +382,8 @@ def main():
         "ms_per_calculator_call": batch_ms if batch else {"neighbour_list_rebuilt": round(list_ms["rebuilt"], 3),
                                                           "neighbour_list_kept": round(list_ms["kept"], 3)},
         "ms_per_step_ordered_sums": round(ordered_ms, 4) if ordered_ms is not None else None,
+        "ms_per_step_radial_tables_1024": round(spline_ms, 4) if spline_ms is not None else None,
+        "spline": a.spline,
         "engine_create_s": round(create_s, 3),
         "chunksize": eng.chunksize,              # atoms per engine pass the timed steps ran with (0: the whole structure in one pass)
         "device_memory_GB": round(mem_gb, 3),

@@ -28,7 +28,7 @@ SYMBOLS = [
     "gr_system_list_sizes", "gr_system_list_get", "gr_compute_lammps", "gr_compute_batch_device", "gr_compute_batch_uq", "gr_compute_batch_device_uq", "gr_engine_reset", "gr_engine_release_buffers", "gr_set_memory_limit", "gr_memory_in_use", "gr_compute_lammps_device", "gr_model_has_uq", "gr_model_validate_uq", "gr_engine_fetch_uq",
     "gr_system_fetch_uq", "gr_engine_atoms_that_fit", "gr_engine_set_exchange", "gr_engine_comm_layers", "gr_engine_comm_width", "gr_engine_pack_forward", "gr_engine_unpack_forward", "gr_engine_pack_reverse", "gr_engine_unpack_reverse", "gr_engine_pack_forward_host", "gr_engine_unpack_forward_host", "gr_engine_pack_reverse_host", "gr_engine_unpack_reverse_host", "gr_engine_set_chunksize", "gr_engine_chunksize", "gr_system_set_chunksize", "gr_system_chunksize",
     "gr_engine_set_ordered_sums", "gr_engine_ordered_sums", "gr_engine_fetch_cvatom", "gr_system_fetch_cvatom", "gr_lammps_add_cvatom",
-    "gr_lammps_add_cvatom_device",
+    "gr_lammps_add_cvatom_device", "gr_engine_set_spline", "gr_engine_spline",
 ]
 
 
@@ -103,6 +103,8 @@ def lib():
     L.gr_engine_chunksize.argtypes = [vp]
     L.gr_engine_set_ordered_sums.argtypes = [vp, i32]
     L.gr_engine_ordered_sums.argtypes = [vp]
+    L.gr_engine_set_spline.argtypes = [vp, i32]
+    L.gr_engine_spline.argtypes = [vp]
     L.gr_system_set_chunksize.argtypes = [vp, i32]
     L.gr_system_chunksize.argtypes = [vp]
     L.gr_engine_radial_noalloc.argtypes = [vp, i32, vp, vp, vp, vp]

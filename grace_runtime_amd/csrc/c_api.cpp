@@ -38,6 +38,7 @@ struct gr_engine {
   grhip::ExchangeCallbacks exchange;                   // kept for the engine a reset makes
   int chunk_request = -1;                              // the caller's chunk size, kept for the engine a reset makes
   bool ordered = false;                                // ordered sums requested, kept for the engine a reset makes
+  int spline = 0;                                      // radial-table intervals requested, kept for the engine a reset makes
   std::vector<int> lmp_rows;                           // gr_compute_lammps: LAMMPS index of engine row q (empty: rows are LAMMPS indices)
   int lmp_nall = -1;                                   // atoms of the last gr_compute_lammps[_device] call
   uint64_t lmp_serial = 0;                             // the engine's upload count at that call: its list is still the one held
@@ -58,6 +59,7 @@ struct gr_engine {
     if (has_exchange) eng->set_exchange(exchange);
     eng->set_chunksize(chunk_request);
     if (ordered) eng->set_ordered_sums(true);
+    if (spline > 0) eng->set_spline(spline);
   }
   std::vector<grhip::StageTime> times;
   std::unique_ptr<grhip::BatchDeviceNeighbors> bnl;    // lists of gr_compute_batch_device (buffers kept between calls)
@@ -1097,6 +1099,16 @@ int gr_engine_set_ordered_sums(gr_engine *e, int on)
 }
 
 int gr_engine_ordered_sums(const gr_engine *e) { return e && e->eng && e->eng->ordered_sums() ? 1 : 0; }
+
+int gr_engine_set_spline(gr_engine *e, int intervals)
+{
+  return guarded([&] {
+    live(e).set_spline(intervals);
+    e->spline = intervals;
+  });
+}
+
+int gr_engine_spline(const gr_engine *e) { return e && e->eng ? e->eng->spline() : 0; }
 
 int gr_system_fetch_uq(gr_system *s, double *gamma, double *sigma, double *cluster)
 {

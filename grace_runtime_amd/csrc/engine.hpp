@@ -128,6 +128,11 @@ class Engine {
   // passes with it (the reference sizes the first pass from the free memory: libgrace/include/grace/kk/support.h:425-450)
   virtual int64_t atoms_that_fit() = 0;
   virtual void set_chunksize(int atoms) = 0;
+  // radial tables (spline_n of the reference's engines, libgrace/include/grace/system.h:78; `spline` of Model / System /
+  // Batch, python/kk/kk_api.h:53,75): n > 0: the radial functions of GRACE-1L and 2L engines come from cubic tables of n
+  // intervals, as in the reference; 0 (the engines' default): the radial MLP is evaluated for every bond
+  virtual void set_spline(int n) = 0;
+  virtual int spline() const = 0;
   // ordered sums: forces, virial, energy and message adjoints are added in a fixed order instead of with floating-point
   // atomics, so that two runs on the same input give the same bits (the reference's GPU engines accept last-bit variation
   // from run to run: python/tests/test_gpu_several_calculators.py).

@@ -72,7 +72,7 @@ template<class T> class Engine1L final : public EngineBase {
   Engine1L(std::shared_ptr<const Model1L> m, int ntypes, const std::vector<int> &type2mu, int device) :
       EngineBase(device, "GRACE-1L", ntypes, type2mu, m->n_elements), model_(std::move(m))
   {
-    this->template probe_mfma<T>();
+    this->template probe_mfma_both<T>();
     chunks_ = true;
     ordered_ok_ = true;
     build();
@@ -123,7 +123,8 @@ template<class T> class Engine1L final : public EngineBase {
     EngineBase::launch_gemm<T>(J, kb0, kb1, nb, X0, nf0, X1, nf1, out, nfo, accumulate, cur_tiles_, cur_ntiles_);
   }
   void launch_radial(long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
-                     const long long *n_edges);
+                     const long long *n_edges, bool tables = false);
+  void apply_spline(int n) override { rad_.spline_n = n; }
 };
 
 template<class T> void Engine1L<T>::build()
@@ -182,6 +183,7 @@ template<class T> void Engine1L<T>::build()
 
   // ---- radial MLP in MFMA fragment order
   rad_.build(m.mlp_rad, m.nradbase, m.radial_basis_p, m.radial_activation, C_, CP_, nl_, nel_, drow_, "GRACE-1L");
+  rad_.build_double(m.mlp_rad, m.nradbase, m.radial_basis_p, m.radial_activation, C_, CP_, nl_, nel_, drow64_, "GRACE-1L");
   noutp_ = rad_.noutp;
 
   // ---- liveness, products, FCs (fused_1l.cpp:176-216)
@@ -300,9 +302,9 @@ template<class T> void Engine1L<T>::build()
 
 template<class T>
 void Engine1L<T>::launch_radial(long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
-                                const long long *n_edges)
+                                const long long *n_edges, bool tables)
 {
-  rad_.launch(stream_, ncu_, z_.as<T>(), e_begin, e_count, x, emu, Rz, dRz, n_edges);
+  rad_.launch(stream_, ncu_, z_.as<T>(), e_begin, e_count, x, emu, Rz, dRz, n_edges, nullptr, tables);
 }
 
 template<class T> void Engine1L<T>::run(const RunFlags &fl)
@@ -386,7 +388,7 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
   // the radial rows of the chunk start at row 0 of Rz_ / dRz_; the kernels index them by the bond's number in the structure
   T *Rz = moved_back(Rz_.as<T>(), e_begin * noutp_), *dRz = moved_back(dRz_.as<T>(), e_begin * noutp_);
 
-  stage("radial_mlp", [&] { launch_radial(e_begin, e_count, xr_.as<double>(), emu_.as<int>(), Rz, dRz, eoff_.as<long long>() + n_); });
+  stage("radial_mlp", [&] { launch_radial(e_begin, e_count, xr_.as<double>(), emu_.as<int>(), Rz, dRz, eoff_.as<long long>() + n_, true); });
 
   ScatterArgs<T> sa{};
   sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz; sa.A = A_.as<T>();

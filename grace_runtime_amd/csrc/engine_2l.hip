@@ -33,13 +33,14 @@ template<class T> class Engine2L final : public EngineBase {
   Engine2L(std::shared_ptr<const Model2L> m, int ntypes, const std::vector<int> &type2mu, int device) :
       EngineBase(device, "GRACE-2L", ntypes, type2mu, m->n_elements), model_(std::move(m))
   {
-    this->template probe_mfma<T>();
+    this->template probe_mfma_both<T>();
     build();
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
     chunks_ = true;
     ordered_ok_ = true;
   }
   int layers() const override { return 2; }
+  void apply_spline(int n) override { radR_.spline_n = radR1_.spline_n = n; }
   void run(const RunFlags &fl) override;
   void debug_radial(int, const double *, const int *, double *, double *) override
   {
@@ -201,6 +202,8 @@ template<class T> void Engine2L<T>::build()
   sink_.ensure(64);
   radR_.build(m.mlp_R, m.nradbase, m.radial_basis_p, m.radial_activation, m.C1, C1P_, nl_, nel_, drow_, "GRACE-2L");
   radR1_.build(m.mlp_R1, m.nradbase, m.radial_basis_p, m.radial_activation, m.CR, CRP_, nl_, nel_, drow_, "GRACE-2L");
+  radR_.build_double(m.mlp_R, m.nradbase, m.radial_basis_p, m.radial_activation, m.C1, C1P_, nl_, nel_, drow64_, "GRACE-2L");
+  radR1_.build_double(m.mlp_R1, m.nradbase, m.radial_basis_p, m.radial_activation, m.CR, CRP_, nl_, nel_, drow64_, "GRACE-2L");
 
   // ---- the two dense chains
   const int ns = m.nsrc();
@@ -590,7 +593,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   // in the structure)
   auto layer1_chain = [&] {
     T *Rz = moved_back(Rz_.as<T>(), eb * radR_.noutp), *dRz = moved_back(dRz_.as<T>(), eb * radR_.noutp);
-    stage("radial_R", [&] { radR_.launch(stream_, ncu_, zA_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), Rz, dRz, n_edges); });
+    stage("radial_R", [&] { radR_.launch(stream_, ncu_, zA_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), Rz, dRz, n_edges, nullptr, true); });
     ScatterArgs<T> sa{};
     sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz; sa.A = A;
     sa.a0 = a0_; sa.C = C1P_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = radR_.noutp; sa.sh = sh_;
@@ -698,7 +701,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     const long long *eoff = eoff_.as<long long>() + a0_;
     const int *mu = mu_.as<int>() + a0_;
     T *R1 = moved_back(R1_.as<T>(), eb * radR1_.noutp), *dR1 = moved_back(dR1_.as<T>(), eb * radR1_.noutp);
-    stage("radial_R1", [&] { radR1_.launch(stream_, ncu_, ones_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), R1, dR1, n_edges); });
+    stage("radial_R1", [&] { radR1_.launch(stream_, ncu_, ones_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), R1, dR1, n_edges, nullptr, true); });
     stage("pair_fwd", [&] {
       const size_t lds = (size_t) 2 * kAsyncChunkFwd * (pthreads + radR1_.noutp) * sizeof(T);
       GR_PAIR(k_pair_fwd, dim3(nc), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) M, P, nslot_, CRP_,

@@ -342,6 +342,19 @@ template<class T> struct DevFcPairBwd {
 // R_{n,l}(x) z[mu_j][n] (file order of the last layer: o = n nl + l, libgrace/src/fused_1l.cpp:123).
 template<class T> struct DevRadial {
   DevBuf w0, w1, w2, bias_i, bias_j, bias1;
+  // radial tables (the reference's spline_n, libgrace/include/grace/system.h:78): intervals asked for (0: the MLP itself is
+  // evaluated for every bond) and the table that exists: value and d/dx at the knots, [N + 1][noutp] each
+  int spline_n = 0, table_n = 0;
+  DevBuf tabF, tabD, knots, knot_mu, unit_z, knotF, knotD;
+  // fp32 engines: the same MLP in fp64, which evaluates the knots of the tables (build_double)
+  std::unique_ptr<DevRadial<double>> dbl;
+  template<class... A> void build_double(A &&...a)
+  {
+    if constexpr (sizeof(T) == 4) {
+      dbl = std::make_unique<DevRadial<double>>();
+      dbl->build(std::forward<A>(a)...);
+    }
+  }
   int mode = 0;    // 1: species form (build_species)
   int hb = 4, ks0 = 2, nob = 0, noutp = 0, w2_in_lds = 1, nrb = 0, p = 0, act = 0, CP = 0, nel = 0;
   size_t lds = 0;
@@ -426,9 +439,45 @@ template<class T> struct DevRadial {
   }
   // z: [nel][CP] species weights of the neighbour; e_count < 0: the edge count is read from *n_edges on the device;
   // emi: element of the central atom of every edge (species form only)
+  // tables: use the radial tables when the engine was asked for them (the plain form only); otherwise, and for the debug
+  // entry points, the MLP is evaluated for every bond
   void launch(hipStream_t stream, int ncu, const T *z, long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
-              const long long *n_edges, const int *emi = nullptr)
+              const long long *n_edges, const int *emi = nullptr, bool tables = false)
   {
+    if (tables && spline_n > 0 && mode == 0) {
+      const int N = spline_n;
+      if (table_n != N || !tabF.p || (sizeof(T) == 8 && !tabD.p)) {    // the MLP at the knots x = k / N, unit species weights (again after release_buffers)
+        std::vector<double> xs((size_t) N + 1);
+        for (int k = 0; k <= N; k++) xs[(size_t) k] = (double) k / N;
+        upload_vec(knots, xs);
+        upload_vec(knot_mu, std::vector<int>((size_t) N + 1, 0));
+        const size_t rows = ((size_t) N + 1) * noutp;
+        if constexpr (sizeof(T) == 8) {
+          upload_vec(unit_z, std::vector<T>((size_t) CP, (T) 1));
+          tabF.ensure(rows * sizeof(T));
+          tabD.ensure(rows * sizeof(T));
+          launch(stream, ncu, unit_z.template as<T>(), 0, (long long) N + 1, knots.as<double>(), knot_mu.as<int>(), tabF.template as<T>(),
+                 tabD.template as<T>(), nullptr);
+        } else {
+          if (!dbl) throw Error("radial tables of an fp32 engine need the fp64 form of its radial MLP");
+          upload_vec(unit_z, std::vector<double>((size_t) CP, 1.0));
+          knotF.ensure(rows * sizeof(double));
+          knotD.ensure(rows * sizeof(double));
+          tabF.ensure((size_t) N * 4 * noutp * sizeof(T));
+          dbl->launch(stream, ncu, unit_z.as<double>(), 0, (long long) N + 1, knots.as<double>(), knot_mu.as<int>(), knotF.as<double>(),
+                      knotD.as<double>(), nullptr);
+          const long long tot = (long long) N * noutp;
+          hipLaunchKernelGGL(k_spline_coef, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream, (const double *) knotF.as<double>(),
+                             (const double *) knotD.as<double>(), N, noutp, tabF.as<float>());
+        }
+        table_n = N;
+      }
+      const long long bound = e_count >= 0 ? e_count : (long long) 1 << 40;
+      const unsigned grid = (unsigned) std::max<long long>(1, std::min<long long>(bound, (long long) ncu * 32));
+      hipLaunchKernelGGL((k_radial_spline<T, sizeof(T) == 4>), dim3(grid), dim3(round_up(noutp, 64)), 0, stream, n_edges, e_begin, e_count, x, emu,
+                         (const T *) tabF.template as<T>(), (const T *) tabD.template as<T>(), table_n, z, CP, noutp, Rz, dRz);
+      return;
+    }
     RadialArgs<T> ra{};
     ra.n_edges = n_edges;
     ra.e_begin = e_begin;
@@ -575,6 +624,13 @@ class EngineBase : public Engine, protected BufRegistry {
     chunk_request_ = atoms;
   }
   int chunksize_used() const override { return chunk_used_; }
+  void set_spline(int n) override
+  {
+    if (n < 0 || (n > 0 && n < 16) || n > (1 << 20)) throw InvalidArgument(who_ + ": spline must be 0 (the radial MLP itself) or 16 .. 1048576 intervals");
+    apply_spline(n);
+    spline_n_ = n;
+  }
+  int spline() const override { return spline_n_; }
   void set_ordered_sums(bool on) override
   {
     if (on && !ordered_ok_) throw InvalidArgument(who_ + ": this engine has no ordered (atomic-free) sums");
@@ -1334,6 +1390,12 @@ class EngineBase : public Engine, protected BufRegistry {
   // pass: the bonds inside the cutoff change with the positions); energy and virial records are summed per structure in a
   // fixed order from the per-atom energies and fcen_
   bool ordered_ok_ = false, ordered_ = false;
+  int spline_n_ = 0;
+  // the engine's radial kernels take the setting (engines without radial tables say so and stay exact)
+  virtual void apply_spline(int n)
+  {
+    if (n > 0) log_message(0, who_ + ": radial tables are not used by this engine; the radial MLPs are evaluated for every bond");
+  }
   DevBuf fedge_, fcen_, tcount_, toff_, traw_, tsorted_;
   // before begin_pass(): what the mode cannot do
   void ordered_check(const RunFlags &fl) const
@@ -1394,6 +1456,18 @@ class EngineBase : public Engine, protected BufRegistry {
   size_t ev_used_ = 0;
   std::vector<StageTime> times_;
   int drow_[16];
+  int drow64_[16];    // fp32 engines: the accumulator rows of the fp64 MFMA (the fp64 radial MLP that fills the radial tables)
+  // probes the MFMA accumulator layout of the engine's precision; an fp32 engine probes the fp64 one first and keeps it
+  template<class T> void probe_mfma_both()
+  {
+    if constexpr (sizeof(T) == 4) {
+      probe_mfma<double>();
+      for (int q = 0; q < 16; q++) drow64_[q] = drow_[q];
+    }
+    probe_mfma<T>();
+    if constexpr (sizeof(T) == 8)
+      for (int q = 0; q < 16; q++) drow64_[q] = drow_[q];
+  }
 };
 
 }    // namespace grhip

@@ -399,6 +399,77 @@ __device__ inline double ipow(double x, int n)
 // Every k-step feeds all row blocks of the value and the tangent stream (2 HB independent accumulator chains).
 // ACT: 0 SiLU, 1 tanh (compile-time: the fp64 tanh is large, and both activations inlined 32 times overflow the
 // instruction cache).
+// Radial functions from tables, as the reference's engines evaluate them (spline_eval, libgrace/include/grace/fused_cpu.h:
+// 1052-1074; tables of Grace1LFused::build_splines, libgrace/src/fused_1l.cpp:102-129): N intervals over x = r / rc in
+// [0, 1], per interval the cubic through the values and derivatives of the radial MLP at its two ends,
+//   R(t) = f0 + t (d0 + t (c2 + t c3)),  c2 = -3 f0 - 2 d0 + 3 f1 - d1,  c3 = 2 f0 + d0 - 2 f1 + d1,  d = f' / N,
+//   dR/dx = N (d0 + t (2 c2 + 3 c3 t)),  k = min(int(x N), N - 1),  t = x N - k.
+// COEF false (fp64): F, D are [N + 1][noutp] value and d/dx at the knots (what k_radial returns for x = k / N and unit
+// species weights) and the cubic's coefficients are formed per use, so the table is half the size of stored coefficients
+// and stays in the L2.  COEF true (fp32): F is [N][4][noutp] coefficients formed in fp64 by k_spline_coef (c2 and c3 are
+// differences of nearly equal values: formed in fp32 they would cost four digits of dR/dx), D unused.
+// One block = noutp threads rounded up to a wave, a thread per column, blocks stride over the edges; rows as k_radial.
+template<class T, bool COEF>
+__global__ void k_radial_spline(const long long *__restrict__ n_edges, long long e_begin, long long e_count, const double *__restrict__ x,
+                                const int *__restrict__ emu, const T *__restrict__ F, const T *__restrict__ D, int N, const T *__restrict__ z, int C,
+                                int noutp, T *__restrict__ Rz, T *__restrict__ dRz)
+{
+  const long long cnt = e_count >= 0 ? e_count : *n_edges - e_begin;
+  const int col = threadIdx.x;
+  if (col >= noutp) return;
+  const int n = col % C;
+  const T h = (T) (1.0 / N);
+  constexpr int U = 4;    // edges of one step: their table reads are in flight together
+  for (long long el0 = (long long) blockIdx.x * U; el0 < cnt; el0 += (long long) gridDim.x * U) {
+    T c0[U], c1[U], c2[U], c3[U], t[U], zc[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const long long e = e_begin + (el0 + u < cnt ? el0 + u : cnt - 1);
+      const double sx = x[e] * N;
+      int k = (int) sx;
+      k = k > N - 1 ? N - 1 : (k < 0 ? 0 : k);
+      t[u] = (T) (sx - k);
+      zc[u] = z[emu[e] * C + n];
+      if (COEF) {
+        const T *c = F + (long long) k * 4 * noutp + col;
+        c0[u] = c[0]; c1[u] = c[noutp]; c2[u] = c[2 * noutp]; c3[u] = c[3 * noutp];
+      } else {
+        const T *f = F + (long long) k * noutp + col, *d = D + (long long) k * noutp + col;
+        c0[u] = f[0]; c1[u] = d[0]; c2[u] = f[noutp]; c3[u] = d[noutp];    // f0, f0', f1, f1'
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      if (el0 + u >= cnt) break;
+      const long long e = e_begin + el0 + u;
+      T a0 = c0[u], a1 = c1[u], a2 = c2[u], a3 = c3[u];
+      if (!COEF) {
+        const T f1 = a2, d1 = a3 * h;
+        a1 *= h;
+        a2 = (T) -3 * a0 - (T) 2 * a1 + (T) 3 * f1 - d1;
+        a3 = (T) 2 * a0 + a1 - (T) 2 * f1 + d1;
+      }
+      const T tt = t[u];
+      Rz[e * noutp + col] = (a0 + tt * (a1 + tt * (a2 + tt * a3))) * zc[u];
+      dRz[e * noutp + col] = (a1 + tt * ((T) 2 * a2 + tt * (T) 3 * a3)) * (T) N * zc[u];
+    }
+  }
+}
+// coefficients [N][4][noutp] of the cubics in fp32 from the knot values and derivatives in fp64
+static __global__ void k_spline_coef(const double *__restrict__ F, const double *__restrict__ D, int N, int noutp, float *__restrict__ coef)
+{
+  const long long q = blockIdx.x * (long long) blockDim.x + threadIdx.x;
+  if (q >= (long long) N * noutp) return;
+  const long long k = q / noutp;
+  const int col = (int) (q % noutp);
+  const double f0 = F[k * noutp + col], f1 = F[(k + 1) * noutp + col], d0 = D[k * noutp + col] / N, d1 = D[(k + 1) * noutp + col] / N;
+  float *c = coef + k * 4 * noutp + col;
+  c[0] = (float) f0;
+  c[noutp] = (float) d0;
+  c[2 * noutp] = (float) (-3.0 * f0 - 2.0 * d0 + 3.0 * f1 - d1);
+  c[3 * noutp] = (float) (2.0 * f0 + d0 - 2.0 * f1 + d1);
+}
+
 // Threads of a block: hidden width 64 with every weight in LDS runs three waves per SIMD (168 registers; two waves at 180
 // were 2 % slower in fp64, 6 % in fp32), the other forms would spill at that size; width 128 runs one wave per SIMD.
 constexpr int radial_threads(int hb, int mode, bool w2l) { return hb <= 4 ? (w2l && mode == 0 ? 768 : 512) : 256; }

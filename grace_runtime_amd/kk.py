@@ -132,8 +132,9 @@ def neighbor_search(positions, cell, pbc, cutoff, num_threads: int = 0):
 
 
 class Model:
-    """A loaded kokkos.npz (host side).  `Model(path, spline=1024, asi="")`: python/kk/kk_api.h:51-64; `spline` is
-    accepted for interface compatibility (this engine evaluates the radial MLP exactly, without tables)."""
+    """A loaded kokkos.npz (host side).  `Model(path, spline=1024, asi="")`: python/kk/kk_api.h:51-64; `spline` is kept as
+    the attribute of that name, which the reference's calculator hands to System / Batch (python/grace_runtime/
+    calculator.py:358)."""
 
     def __init__(self, path, spline: int = 1024, asi: str = ""):
         L = _lib.lib()
@@ -144,6 +145,7 @@ class Model:
         info = _lib.ModelInfo()
         check(L.gr_model_get_info(self._h, C.byref(info)))
         self.path = str(path)
+        self.spline = int(spline)
         self.layers = info.layers
         self.lmax, self.n_radial, self.rcut, self.max_order = info.lmax, info.n_radial, info.rcut, info.max_order
         self.n_elements = info.n_elements
@@ -267,6 +269,15 @@ class Engine:
     @property
     def chunksize(self) -> int:
         return int(_lib.lib().gr_engine_chunksize(self._h))
+
+    def set_spline(self, intervals: int):
+        """radial tables of `intervals` cubic pieces for GRACE-1L / 2L engines, as the reference's engines use (0: the radial
+        MLP is evaluated for every bond; GRACE-3L engines keep their MLPs)"""
+        check(_lib.lib().gr_engine_set_spline(self._h, int(intervals)))
+
+    @property
+    def spline(self) -> int:
+        return int(_lib.lib().gr_engine_spline(self._h))
 
     def set_ordered_sums(self, on: bool = True):
         """forces, virial, energy and message adjoints added in a fixed order instead of with floating-point atomics: the
@@ -601,12 +612,16 @@ class System:
     neighbors.py:68-89).  The list lives on the device (gr_system_*): its pair search runs there, and calls between
     rebuilds send positions only."""
 
-    def __init__(self, model: Model, species, skin: float = 0.5, spline: int = 1024, chunksize: int = -1,
+    def __init__(self, model: Model, species, skin: float = 0.5, spline: int = 0, chunksize: int = -1,
                  precision: int = 64):
+        """spline: intervals of the radial tables of GRACE-1L / 2L engines (the reference's engines always use tables,
+        1024 intervals unless told otherwise: docs/advanced.md:34); 0, the default HERE: the radial MLP is evaluated for
+        every bond, without interpolation error.  The reference's calculator passes its model's spline (1024)."""
         skin = float(skin)
         if not (np.isfinite(skin) and skin >= 0.0):
             raise ValueError(f"skin must be a finite number >= 0, got {skin!r}")
         self.engine = Engine(model, species, precision)
+        self.engine.set_spline(int(spline))
         self.skin = skin
         self.cutoff = float(self.engine.cutoff_matrix().max()) if len(species) else 0.0
         self._h = C.c_void_p()
@@ -698,8 +713,10 @@ class Batch:
     """Many structures per call (python/kk/kk_api.h:116-156): energy [S], virial [S, 6], forces [N, 3] in input
     order.  All structures are packed into one atom list and evaluated in one engine pass."""
 
-    def __init__(self, model: Model, species, spline: int = 1024, chunksize: int = -1, precision: int = 64):
+    def __init__(self, model: Model, species, spline: int = 0, chunksize: int = -1, precision: int = 64):
+        """spline: as for System (0: the radial MLP itself; n: radial tables of n intervals, the reference's default is 1024)"""
         self.engine = Engine(model, species, precision)
+        self.engine.set_spline(int(spline))
         self.cutoff = float(self.engine.cutoff_matrix().max()) if len(species) else 0.0
         self.passes = 0
         self.keep_buffers = False

@@ -317,6 +317,18 @@ int gr_system_chunksize(const gr_system *s);
  * when on. */
 int gr_engine_set_ordered_sums(gr_engine *e, int on);
 int gr_engine_ordered_sums(const gr_engine *e);
+
+/* Radial tables: intervals > 0 makes a GRACE-1L or 2L engine take its radial functions from cubic tables of that many
+ * intervals over r / rc in [0, 1] (per interval the cubic through the values and derivatives of the radial MLP at its two
+ * ends), which is how the reference's CPU and GPU engines evaluate them: FusedSettings::spline_n, default 1024
+ * (libgrace/include/grace/system.h:78), `spline` of Model / System / Batch (python/kk/kk_api.h:53,75), tables of
+ * Grace1LFused::build_splines (libgrace/src/fused_1l.cpp:102-129), evaluation spline_eval (fused_cpu.h:1052-1074); the
+ * tables here hold the engine's precision where the reference's hold fp32.  0, the default of gr_engine_create: the
+ * radial MLP itself is evaluated for every bond (no interpolation error).  16 .. 1048576, else GR_INVALID.  GRACE-3L
+ * engines accept the call, say so through the logger and keep evaluating their radial MLPs (their tables would be per pair
+ * of species).  gr_engine_spline: the value set. */
+int gr_engine_set_spline(gr_engine *e, int intervals);
+int gr_engine_spline(const gr_engine *e);
 int gr_system_rebuilds(const gr_system *s);
 int gr_system_list_on_device(const gr_system *s);
 int gr_system_list_sizes(gr_system *s, int64_t *nbonds, int64_t *nimages);

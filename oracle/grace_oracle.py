@@ -421,11 +421,37 @@ class Model1L:
         grho[:, 1:] = g
         return E, grho
 
+    spline = 0    # > 0: the radial functions from cubic tables of that many intervals, as the reference's engines take them
+
+    def radial_exact(self, x):
+        g, dg = radial_basis(x, self.p, self.nrb)
+        return mlp_value_tangent(self.rad, g, dg, self.rad_act)
+
     def radial(self, x):
         """R[nb, C, nl], dR/dx  (MLP output index o = n nl + l: src/fused_1l.cpp:123)."""
-        g, dg = radial_basis(x, self.p, self.nrb)
-        R, dR = mlp_value_tangent(self.rad, g, dg, self.rad_act)
+        R, dR = self.radial_exact(x) if self.spline <= 0 else spline_radial(self, "_tab", self.radial_exact, self.spline, x)
         return R.reshape(-1, self.C, self.nl), dR.reshape(-1, self.C, self.nl)
+
+
+def spline_radial(owner, slot, exact, N, x):
+    """Radial functions and d/dx from the reference's tables, in fp64 (the reference stores fp32 coefficients): N intervals
+    over x in [0, 1], per interval the cubic through value and derivative of the MLP at both ends
+    (Grace1LFused::build_splines, src/fused_1l.cpp:102-129: c = {f0, d0, -3 f0 - 2 d0 + 3 f1 - d1, 2 f0 + d0 - 2 f1 + d1}
+    with d = f' / N), evaluated as spline_eval (libgrace/include/grace/fused_cpu.h:1052-1074): k = min(int(x N), N - 1),
+    t = x N - k, R = c0 + t (c1 + t (c2 + t c3)), dR/dx = N (c1 + t (2 c2 + 3 c3 t)).  The table is kept on `owner`."""
+    tab = getattr(owner, slot, None)
+    if tab is None or tab[0] != N:
+        F, D = exact(np.arange(N + 1) / N)
+        tab = (N, F, D / N)
+        setattr(owner, slot, tab)
+    _, F, Dh = tab
+    s = np.asarray(x, dtype=np.float64) * N
+    k = np.clip(s.astype(np.int64), 0, N - 1)
+    t = (s - k)[:, None]
+    f0, f1, d0, d1 = F[k], F[k + 1], Dh[k], Dh[k + 1]
+    c2 = -3.0 * f0 - 2.0 * d0 + 3.0 * f1 - d1
+    c3 = 2.0 * f0 + d0 - 2.0 * f1 + d1
+    return f0 + t * (d0 + t * (c2 + t * c3)), (d0 + t * (2.0 * c2 + t * 3.0 * c3)) * N
 
 
 class ZeroBondError(ValueError):

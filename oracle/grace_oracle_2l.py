@@ -29,7 +29,7 @@ from __future__ import annotations
 
 import numpy as np
 
-from .grace_oracle import (ZeroBondError, _FC, _Prod, _scalar, load_npz, mlp_value_tangent, radial_basis, real_sh)
+from .grace_oracle import (ZeroBondError, _FC, _Prod, _scalar, load_npz, mlp_value_tangent, radial_basis, real_sh, spline_radial)
 
 __all__ = ["Model2L", "compute_2l"]
 
@@ -194,10 +194,15 @@ class Model2L:
             cluster[a] = k
         return gamma, sigma, cluster
 
+    spline = 0    # > 0: the radial functions of both layers from cubic tables of that many intervals (grace_oracle.spline_radial)
+
     def radial(self, which, x):
         layers, C = (self.rad1, self.C1) if which == 1 else (self.rad2, self.CR)
-        g, dg = radial_basis(x, self.p, self.nrb)
-        R, dR = mlp_value_tangent(layers, g, dg, self.rad_act)
+
+        def exact(xs):
+            g, dg = radial_basis(xs, self.p, self.nrb)
+            return mlp_value_tangent(layers, g, dg, self.rad_act)
+        R, dR = exact(x) if self.spline <= 0 else spline_radial(self, f"_tab{which}", exact, self.spline, x)
         return R.reshape(-1, C, self.nl), dR.reshape(-1, C, self.nl)
 
     # ---- layer 1 dense chain: fused_2l.cpp:404-452 ------------------------------------------------------------
