@@ -450,8 +450,8 @@ __global__ void k_radial_spline(const long long *__restrict__ n_edges, long long
         a3 = (T) 2 * a0 + a1 - (T) 2 * f1 + d1;
       }
       const T tt = t[u];
-      Rz[e * noutp + col] = (a0 + tt * (a1 + tt * (a2 + tt * a3))) * zc[u];
-      dRz[e * noutp + col] = (a1 + tt * ((T) 2 * a2 + tt * (T) 3 * a3)) * (T) N * zc[u];
+      __builtin_nontemporal_store((a0 + tt * (a1 + tt * (a2 + tt * a3))) * zc[u], &Rz[e * noutp + col]);
+      __builtin_nontemporal_store((a1 + tt * ((T) 2 * a2 + tt * (T) 3 * a3)) * (T) N * zc[u], &dRz[e * noutp + col]);
     }
   }
 }
@@ -661,12 +661,13 @@ template<class T, int HB, int ACT, int MODE, bool W2L> __global__ __launch_bound
 #pragma unroll
       for (int v = 0; v < 4; v++) {
         if (row_v[v] >= 0) {
+          // streaming stores: the rows are read by other kernels after the whole array has been written
           if (MODE == 1) {
-            Rt[row_v[v] + col] = acc[v] * env_v[v] * zc[v];
-            dRt[row_v[v] + col] = (dacc[v] * env_v[v] + acc[v] * denv_v[v]) * zc[v];
+            __builtin_nontemporal_store((T) (acc[v] * env_v[v] * zc[v]), &Rt[row_v[v] + col]);
+            __builtin_nontemporal_store((T) ((dacc[v] * env_v[v] + acc[v] * denv_v[v]) * zc[v]), &dRt[row_v[v] + col]);
           } else {
-            Rt[row_v[v] + col] = acc[v] * zc[v];
-            dRt[row_v[v] + col] = dacc[v] * zc[v];
+            __builtin_nontemporal_store((T) (acc[v] * zc[v]), &Rt[row_v[v] + col]);
+            __builtin_nontemporal_store((T) (dacc[v] * zc[v]), &dRt[row_v[v] + col]);
           }
         }
         zc[v] = zn[v];
