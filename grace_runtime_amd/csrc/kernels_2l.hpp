@@ -420,7 +420,7 @@ __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__rest
   T *o = P + ((long long) i * nslot + slot) * nlm * C + n;
 #pragma unroll
   for (int q = 0; q < NLM; q++)
-    if (active && q < nlm) o[(long long) q * C] = acc[q];
+    if (active && q < nlm) __builtin_nontemporal_store(acc[q], &o[(long long) q * C]);
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
 }
 
