@@ -221,7 +221,7 @@ template<class T> void Engine1L<T>::build()
       if (order4_) jit_compile_product("prod_AAAA", hAAAA.terms, nAA_, nAA_, nAAAA_, true, CFP_, f32, arch_, pAAAA_.jit, pAAAA_.jit_note);
       jit_all_ = pAA_.jit.ok() && pAAA_.jit.ok() && (!order4_ || pAAAA_.jit.ok());
     }
-    fcA1_.build(m.fc_A1, liveA1, nlm_, CP_, CP_, CFP_, drow_);
+    fcA1_.build(m.fc_A1, liveA1, nlm_, CP_, CP_, CFP_, drow_, false, true);    // both inputs are A: one reverse launch
     fcAA1_.build(m.fc_AA1, liveAA1, nlm_, CFP_, CP_, CFP_, drow_);
     if (order4_) {
       fcAA2_.build(m.fc_AA2, liveAA2, nlm_, CFP_, CP_, CFP_, drow_);
@@ -500,6 +500,10 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
   // FC reverse: left input (same functions as the output), then right input (functions of A)
   auto fc_bwd = [&](const char *name, DevFc<T> &F, const T *g, T *gXl, T *gXr, int nfl, int kl) {
     stage(name, [&] {
+      if (F.have_lr && gXl == gXr && kl == ka && nfl == nlm_) {
+        launch_gemm(F.bwd_lr, kf, kf, ka, g, nfl, g, nfl, gXl, nlm_, 1);
+        return;
+      }
       launch_gemm(F.bwd_l, kf, kf, kl, g, nfl, g, nfl, gXl, nfl, 1);
       launch_gemm(F.bwd_r, kf, kf, ka, g, nfl, g, nfl, gXr, nlm_, 1);
     });

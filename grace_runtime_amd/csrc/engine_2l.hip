@@ -135,7 +135,7 @@ void Engine2L<T>::build_chain(Chain<T> &c, const char *tag, int nf, int KP, cons
   jit_compile_product(("prod3" + t).c_str(), h3.terms, c.nXX, nf, c.nXXX, false, KP, f32, arch_, c.p3.jit, c.p3.jit_note);
   if (order4_) jit_compile_product(("prod4" + t).c_str(), h4.terms, c.nXX, c.nXX, c.nXXXX, true, KP, f32, arch_, c.p4.jit, c.p4.jit_note);
   c.jit_all = c.p2.jit.ok() && c.p3.jit.ok() && (!order4_ || c.p4.jit.ok());
-  c.fc1.build(*fc[0], live1, nf, KP, KP, KP, drow_);
+  c.fc1.build(*fc[0], live1, nf, KP, KP, KP, drow_, false, true);    // both inputs are X: one reverse launch
   // the reverse of fc2 (with the fourth-order stage: of fc2 and fc3 in one pass) WRITES the adjoint of XX: a job per function
   c.fc2.build(*fc[1], live2, nf, KP, KP, KP, drow_, true);
   if (order4_) {
@@ -461,6 +461,10 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
   };
   auto fc_bwd = [&](const std::string &name, DevFc<T> &F, const T *g, T *gXl, T *gXr, int nfl, int acc_left) {
     stage(name.c_str(), [&] {
+      if (F.have_lr && gXl == gXr && nfl == c.nf && acc_left) {
+        launch_gemm<T>(F.bwd_lr, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXl, nfl, 1, cur_tiles_, cur_ntiles_);
+        return;
+      }
       launch_gemm<T>(F.bwd_l, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXl, nfl, acc_left, cur_tiles_, cur_ntiles_);
       launch_gemm<T>(F.bwd_r, c.kb, c.kb, c.kb, g, nfl, g, nfl, gXr, c.nf, 1, cur_tiles_, cur_ntiles_);
     });

@@ -234,12 +234,17 @@ template<class T> struct DevJobs {
 template<class T> struct DevFc {
   DevBuf WlF, WrF, WlTF, WrTF;
   DevJobs<T> fwd, bwd_l, bwd_r;
+  // the reverse of a layer whose two inputs are ONE tensor (A1 = FC(A, A)): a job per input function that takes the left
+  // segment and the right segments together (source 0: left weights, source 1: right weights; both sources are the output
+  // adjoint), one launch and one read-add-write of the input adjoint instead of two; empty unless build() was asked for it
+  DevJobs<T> bwd_lr;
+  bool have_lr = false;
   int nil = 0, nir = 0, no = 0;    // padded widths
   // nfr: functions of the right-input tensor; livef: outputs that are computed; cover_left: the reverse into the left
   // input has a job for EVERY function (without segments for outputs that are not computed), so that a launch that
   // overwrites instead of accumulating leaves no row of the adjoint unwritten
   void build(const FCWeights &w, const std::vector<char> &livef, int nfr, int nil_p, int nir_p, int no_p, const int *drow,
-             bool cover_left = false)
+             bool cover_left = false, bool same_input = false)
   {
     nil = nil_p; nir = nir_p; no = no_p;
     const int nt = w.tiles_left;
@@ -293,6 +298,19 @@ template<class T> struct DevFc {
     bwd_l.build(hl, WlTF.as<T>(), WlTF.as<T>());
     bwd_r.build(hr, WrTF.as<T>(), WrTF.as<T>());
     fwd.set_rows(drow); bwd_l.set_rows(drow); bwd_r.set_rows(drow);
+    have_lr = same_input && nil == nir && nfr == w.n_funcs;
+    if (have_lr) {
+      typename DevJobs<T>::Host hlr;
+      for (int r = 0; r < nfr; r++) {
+        if (!livef[r] && conn_from[r].empty()) continue;
+        hlr.job(r, 1.0);
+        if (livef[r]) hlr.seg(0, r, w.w_tile_left[r], w.norm_out_factor[r]);
+        for (int c : conn_from[r]) hlr.seg(1, w.collect_to[c], w.w_tile_right[c], w.norm_out_factor[w.collect_to[c]]);
+        hlr.end_job();
+      }
+      bwd_lr.build(hlr, WlTF.as<T>(), WrTF.as<T>());
+      bwd_lr.set_rows(drow);
+    }
   }
 };
 
