@@ -41,10 +41,10 @@ HBM_PEAK = 8000.0                 # GB/s
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs of this
 # script, counters scaled by what they read for the 1 GiB copy kernel; summaries under profiles/): (workload, kernel)
 MEASURED_TRAFFIC = {
-    ("config2", "radial_mlp"): 7.0e6 + 1216.3e6,        # fetch + write of k_radial<double,4,0,0,true>
-    ("config3", "pair_bwd"): 11234.9e6 + 2773.0e6,      # fetch + write of k_pair_bwd<double,25>
+    ("config2", "radial_mlp"): 14.9e6 + 1224.4e6,       # fetch + write of k_radial<double,4,0,0,true> (its launches on the full edge list)
+    ("config3", "pair_bwd"): 11240.9e6 + 2773.0e6,      # fetch + write of k_pair_bwd<double,25>
     ("config4", "pair_bwd_L3"): 48727e6 + 30596e6,      # the layer-3 launches of k_pair_bwd<double,36> (layer 2: 25.6 + 15.2 GB)
-    ("config5", "pair_bwd"): 9811.7e6 + 2477.6e6,       # fetch + write of k_pair_bwd<double,25> over the ragged batch
+    ("config5", "pair_bwd"): 9842.0e6 + 2477.7e6,       # fetch + write of k_pair_bwd<double,25> over the ragged batch
 }
 # the per-atom dense chain of configuration 2 (every FC, product, reduce and readout launch of a pass), same counters
 DENSE_TRAFFIC = {"config2": 6.5e9}
