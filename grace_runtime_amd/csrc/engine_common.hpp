@@ -114,6 +114,36 @@ struct DevBuf {
   template<class U> U *as() const { return static_cast<U *>(p); }
 };
 
+// pinned host memory of the engine (allocated, never registered): staging of the small per-call transfers, so that they are
+// asynchronous copies on the engine's stream with one wait instead of one blocking copy each
+struct PinnedBuf {
+  void *p = nullptr;
+  size_t bytes = 0;
+  PinnedBuf() = default;
+  PinnedBuf(const PinnedBuf &) = delete;
+  PinnedBuf &operator=(const PinnedBuf &) = delete;
+  ~PinnedBuf() { release(); }
+  void release()
+  {
+    if (p) (void) hipHostFree(p);
+    p = nullptr;
+    bytes = 0;
+  }
+  void ensure(size_t need)
+  {
+    if (need <= bytes && p) return;
+    release();
+    const size_t want = std::max<size_t>(need + need / 8, 4096);
+    if (hipHostMalloc(&p, want, hipHostMallocDefault) != hipSuccess) {
+      p = nullptr;
+      (void) hipGetLastError();
+      throw std::bad_alloc();
+    }
+    bytes = want;
+  }
+  template<class U> U *as() const { return static_cast<U *>(p); }
+};
+
 template<class U> void upload_vec(DevBuf &b, const std::vector<U> &v)
 {
   b.ensure(std::max<size_t>(v.size(), 1) * sizeof(U));
@@ -859,9 +889,13 @@ class EngineBase : public Engine, protected BufRegistry {
   {
     HIP_CHECK(hipSetDevice(device_));
     if (have_rij_) throw Error("update_positions: the uploaded list holds bond vectors, not positions");
-    HIP_CHECK(hipStreamSynchronize(stream_));
-    if (n_ > 0) HIP_CHECK(hipMemcpyAsync(x_.p, x, sizeof(double) * 3 * n_, hipMemcpyHostToDevice, stream_));
-    HIP_CHECK(hipStreamSynchronize(stream_));
+    HIP_CHECK(hipStreamSynchronize(stream_));    // no pass of the stream still reads the staging memory or x_
+    if (n_ > 0) {
+      const size_t bytes = sizeof(double) * 3 * (size_t) n_;
+      pin_in_.ensure(bytes);
+      std::memcpy(pin_in_.p, x, bytes);
+      HIP_CHECK(hipMemcpyAsync(x_.p, pin_in_.p, bytes, hipMemcpyHostToDevice, stream_));    // ordered before the pass on the same stream
+    }
     ran_ = false;
   }
   double *bond_vectors_device() override
@@ -907,17 +941,29 @@ class EngineBase : public Engine, protected BufRegistry {
     HIP_CHECK(hipSetDevice(device_));
     if (!ran_) throw Error("fetch() before run()");
     if (nstruct != nstruct_) throw InvalidArgument("fetch_batch: the uploaded list holds " + std::to_string(nstruct_) + " structures");
+    // everything the call returns goes to pinned memory as asynchronous copies behind the pass, with one wait:
+    // [zero-bond flag (2 ints, padded to 16 bytes)][records 8 nstruct][forces 3 n_nodes][per-atom energies n]
+    const bool wf = forces && ran_forces_ && n_nodes_ > 0, we = eatom && ran_eatom_ && n_ > 0;
+    const size_t nrec = (size_t) 8 * nstruct_, nf = wf ? (size_t) 3 * n_nodes_ : 0, ne = we ? (size_t) n_ : 0;
+    pin_out_.ensure(16 + (nrec + nf + ne) * sizeof(double));
+    int *zb = pin_out_.as<int>();
+    double *rec = reinterpret_cast<double *>(pin_out_.as<unsigned char>() + 16), *pf = rec + nrec, *pe = pf + nf;
+    zb[0] = zb[1] = -1;
+    if (n_ > 0) HIP_CHECK(hipMemcpyAsync(zb, zero_.p, 2 * sizeof(int), hipMemcpyDeviceToHost, stream_));
+    HIP_CHECK(hipMemcpyAsync(rec, scal_.p, nrec * sizeof(double), hipMemcpyDeviceToHost, stream_));
+    if (wf) HIP_CHECK(hipMemcpyAsync(pf, f_.p, nf * sizeof(double), hipMemcpyDeviceToHost, stream_));
+    if (we) HIP_CHECK(hipMemcpyAsync(pe, eatom_.p, ne * sizeof(double), hipMemcpyDeviceToHost, stream_));
     HIP_CHECK(hipStreamSynchronize(stream_));
-    check_zero_bond();
-    std::vector<double> s((size_t) 8 * nstruct_);
-    HIP_CHECK(hipMemcpy(s.data(), scal_.p, s.size() * sizeof(double), hipMemcpyDeviceToHost));
+    if (zb[0] >= 0)
+      throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " + std::to_string(zb[1]) +
+                  " of the neighbour list): not a physical structure");
     for (int q = 0; q < nstruct_; q++) {
-      if (energy) energy[q] = s[8 * (size_t) q];
+      if (energy) energy[q] = rec[8 * (size_t) q];
       if (virial && ran_forces_)
-        for (int k = 0; k < 6; k++) virial[6 * (size_t) q + k] = s[8 * (size_t) q + 1 + k];
+        for (int k = 0; k < 6; k++) virial[6 * (size_t) q + k] = rec[8 * (size_t) q + 1 + k];
     }
-    if (forces && ran_forces_ && n_nodes_ > 0) HIP_CHECK(hipMemcpy(forces, f_.p, sizeof(double) * 3 * n_nodes_, hipMemcpyDeviceToHost));
-    if (eatom && ran_eatom_ && n_ > 0) HIP_CHECK(hipMemcpy(eatom, eatom_.p, sizeof(double) * n_, hipMemcpyDeviceToHost));
+    if (wf) std::memcpy(forces, pf, nf * sizeof(double));
+    if (we) std::memcpy(eatom, pe, ne * sizeof(double));
   }
   void fetch_batch_device(int nstruct, double *energy, double *forces, double *virial, double *eatom) override
   {
@@ -1389,6 +1435,7 @@ class EngineBase : public Engine, protected BufRegistry {
   // uploaded structure
   int n_nodes_ = 0;           // central atoms and ghosts (= n_ without ghosts)
   uint64_t upload_serial_ = 0;
+  PinnedBuf pin_in_, pin_out_;    // staging of the positions of a call and of what a call returns
   DevBuf vatom_;              // per-atom virials [n_nodes][9] (xx yy zz xy xz yz yx zx zy) of a pass with the vatom flag
   bool ran_vatom_ = false;
   double *vatom_ptr() { return ran_vatom_ ? vatom_.as<double>() : nullptr; }
