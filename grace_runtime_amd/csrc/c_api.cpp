@@ -39,6 +39,7 @@ struct gr_engine {
   int chunk_request = -1;                              // the caller's chunk size, kept for the engine a reset makes
   bool ordered = false;                                // ordered sums requested, kept for the engine a reset makes
   int spline = 0;                                      // radial-table intervals requested, kept for the engine a reset makes
+  grhip::PinnedBuf pin_types;                          // gr_compute_batch_device: the atom types of a pass on their way to the host
   std::vector<int> lmp_rows;                           // gr_compute_lammps: LAMMPS index of engine row q (empty: rows are LAMMPS indices)
   int lmp_nall = -1;                                   // atoms of the last gr_compute_lammps[_device] call
   uint64_t lmp_serial = 0;                             // the engine's upload count at that call: its list is still the one held
@@ -1440,10 +1441,12 @@ int gr_compute_batch_device_uq(gr_engine *e, int nstruct, const int *natoms, con
         const int64_t a0 = start[g0], na = start[g1] - a0;
         nl.build(ns, natoms + g0, positions + 3 * a0, cells + 9 * (size_t) g0, pbc + 3 * (size_t) g0, rc, e->bnl_stream);
         // atom types: 4 bytes per atom to the host, where the element tiles of the tile GEMMs are laid out
-        std::vector<int> ty((size_t) na);
-        if (na > 0 && hipMemcpyAsync(ty.data(), types + a0, sizeof(int) * (size_t) na, hipMemcpyDeviceToHost, e->bnl_stream) != hipSuccess)
+        e->pin_types.ensure(sizeof(int) * (size_t) std::max<int64_t>(na, 1));    // pinned: the copy is a DMA, not a staged one
+        int *ty_pinned = e->pin_types.as<int>();
+        if (na > 0 && hipMemcpyAsync(ty_pinned, types + a0, sizeof(int) * (size_t) na, hipMemcpyDeviceToHost, e->bnl_stream) != hipSuccess)
           throw grhip::Error("copy of the atom types failed");
         if (hipStreamSynchronize(e->bnl_stream) != hipSuccess) throw grhip::Error("the device neighbour search failed");
+        const std::vector<int> ty(ty_pinned, ty_pinned + na);
         grhip::DeviceCsr in;
         in.n = (int) na;
         in.types = ty.data();

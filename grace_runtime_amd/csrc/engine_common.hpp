@@ -916,19 +916,19 @@ class EngineBase : public Engine, protected BufRegistry {
   // el_off[e] .. el_off[e + 1]: the tiles of element e
   static std::vector<int> element_tiles(const std::vector<int> &mu, int nel, std::vector<int> &el_off)
   {
+    // a counting pass per element (the elements are few): atoms per element, the tiles each element needs, then every atom
+    // to the next free slot of its element, in atom order
     const int n = (int) mu.size();
-    std::vector<int> tiles, ord(n);
-    std::iota(ord.begin(), ord.end(), 0);
-    std::stable_sort(ord.begin(), ord.end(), [&](int a, int b) { return mu[a] < mu[b]; });
-    el_off.assign(nel + 1, 0);
-    for (int q = 0; q < n;) {
-      int cnt = 0;
-      const int m0 = mu[ord[q]];
-      while (cnt < 16 && q < n && mu[ord[q]] == m0) { tiles.push_back(ord[q]); q++; cnt++; }
-      while (cnt < 16) { tiles.push_back(-1); cnt++; }
-      el_off[m0 + 1]++;
+    std::vector<int> count((size_t) nel, 0);
+    for (int a = 0; a < n; a++) {
+      if (mu[a] < 0 || mu[a] >= nel) throw Error("element of a central atom out of range");
+      count[(size_t) mu[a]]++;
     }
-    for (int e = 0; e < nel; e++) el_off[e + 1] += el_off[e];
+    el_off.assign(nel + 1, 0);
+    for (int e = 0; e < nel; e++) el_off[e + 1] = el_off[e] + (count[(size_t) e] + 15) / 16;
+    std::vector<int> tiles((size_t) 16 * el_off[nel], -1), next((size_t) nel);
+    for (int e = 0; e < nel; e++) next[(size_t) e] = 16 * el_off[e];
+    for (int a = 0; a < n; a++) tiles[(size_t) next[(size_t) mu[a]]++] = a;
     return tiles;
   }
   void fetch(double *energy, double *forces, double *virial, double *eatom) override
