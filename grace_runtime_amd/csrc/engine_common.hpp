@@ -1098,10 +1098,7 @@ class EngineBase : public Engine, protected BufRegistry {
     if (n == 0) return false;
     count_.ensure(sizeof(int) * n);
     eoff_.ensure(sizeof(long long) * (n + 1));
-    {
-      const int init[2] = {-1, -1};
-      HIP_CHECK(hipMemcpyAsync(zero_.p, init, sizeof(init), hipMemcpyHostToDevice, stream_));
-    }
+    HIP_CHECK(hipMemsetAsync(zero_.p, 0xFF, 2 * sizeof(int), stream_));    // (-1, -1): no bond of length zero seen
     BondSrc src{};
     src.mu = mu_.as<int>(); src.offset = offset_.as<long long>(); src.j = j_.as<int>();
     src.rij = have_rij_ ? rij_.as<double>() : nullptr;
