@@ -949,14 +949,11 @@ class EngineBase : public Engine, protected BufRegistry {
     int *zb = pin_out_.as<int>();
     double *rec = reinterpret_cast<double *>(pin_out_.as<unsigned char>() + 16), *pf = rec + nrec, *pe = pf + nf;
     zb[0] = zb[1] = -1;
-    if (n_ > 0) HIP_CHECK(hipMemcpyAsync(zb, zero_.p, 2 * sizeof(int), hipMemcpyDeviceToHost, stream_));
     HIP_CHECK(hipMemcpyAsync(rec, scal_.p, nrec * sizeof(double), hipMemcpyDeviceToHost, stream_));
     if (wf) HIP_CHECK(hipMemcpyAsync(pf, f_.p, nf * sizeof(double), hipMemcpyDeviceToHost, stream_));
     if (we) HIP_CHECK(hipMemcpyAsync(pe, eatom_.p, ne * sizeof(double), hipMemcpyDeviceToHost, stream_));
     HIP_CHECK(hipStreamSynchronize(stream_));
-    if (zb[0] >= 0)
-      throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " + std::to_string(zb[1]) +
-                  " of the neighbour list): not a physical structure");
+    check_zero_bond();
     for (int q = 0; q < nstruct_; q++) {
       if (energy) energy[q] = rec[8 * (size_t) q];
       if (virial && ran_forces_)
@@ -982,8 +979,9 @@ class EngineBase : public Engine, protected BufRegistry {
   void check_zero_bond()
   {
     if (n_ == 0) return;
-    int zb[2];
-    HIP_CHECK(hipMemcpy(zb, zero_.p, sizeof(zb), hipMemcpyDeviceToHost));
+    // the pass sent the flag to pinned memory right after its bond filter; every caller has waited for the stream
+    const int *zb = pin_flag_.as<int>();
+    if (!zb) return;
     if (zb[0] >= 0)
       throw Error("two atoms at the same position (a bond of length 0 between atoms " + std::to_string(zb[0]) + " and " + std::to_string(zb[1]) +
                   " of the neighbour list): not a physical structure");
@@ -1115,6 +1113,8 @@ class EngineBase : public Engine, protected BufRegistry {
     stage("edge_count", [&] { hipLaunchKernelGGL(k_edge_count, dim3((n + wpb - 1) / wpb), dim3(64 * wpb), 0, stream_, src, n, count_.as<int>(), zero_.as<int>()); });
     stage("edge_scan", [&] { hipLaunchKernelGGL(k_scan, dim3(1), dim3(1024), 0, stream_, count_.as<int>(), n, eoff_.as<long long>()); });
     stage("edge_fill", [&] { hipLaunchKernelGGL(k_edge_fill, dim3((n + wpb - 1) / wpb), dim3(64 * wpb), 0, stream_, src, n, eoff_.as<long long>(), ed); });
+    pin_flag_.ensure(2 * sizeof(int));
+    HIP_CHECK(hipMemcpyAsync(pin_flag_.p, zero_.p, 2 * sizeof(int), hipMemcpyDeviceToHost, stream_));    // read by check_zero_bond()
     return true;
   }
   EngineBase(int device, const char *who, int ntypes, const std::vector<int> &type2mu, int n_elements) :
@@ -1433,6 +1433,7 @@ class EngineBase : public Engine, protected BufRegistry {
   int n_nodes_ = 0;           // central atoms and ghosts (= n_ without ghosts)
   uint64_t upload_serial_ = 0;
   PinnedBuf pin_in_, pin_out_;    // staging of the positions of a call and of what a call returns
+  PinnedBuf pin_flag_;            // the zero-bond flag of the last pass (two ints)
   DevBuf vatom_;              // per-atom virials [n_nodes][9] (xx yy zz xy xz yz yx zx zy) of a pass with the vatom flag
   bool ran_vatom_ = false;
   double *vatom_ptr() { return ran_vatom_ ? vatom_.as<double>() : nullptr; }
