@@ -44,6 +44,15 @@ struct gr_engine {
   int lmp_nall = -1;                                   // atoms of the last gr_compute_lammps[_device] call
   uint64_t lmp_serial = 0;                             // the engine's upload count at that call: its list is still the one held
   bool lmp_on_device = false;                          // that call was the device form (its row map is lmp->atom)
+  // the state of the last LAMMPS call names rows of a structure the engine no longer holds (the new engine of a reset
+  // counts its uploads from zero again, so the old count could match a later, unrelated upload)
+  void forget_lammps_call()
+  {
+    lmp_rows.clear();
+    lmp_nall = -1;
+    lmp_serial = 0;
+    lmp_on_device = false;
+  }
   void make()
   {
     if (m1) eng = grhip::make_engine_1l(m1, ntypes, type2mu, precision, device);
@@ -54,6 +63,7 @@ struct gr_engine {
   {
     bnl.reset();
     lmp.reset();
+    forget_lammps_call();
     eng.reset();    // frees every device buffer of the engine before the new one allocates
     generation++;
     make();
@@ -276,6 +286,7 @@ int gr_engine_release_buffers(gr_engine *e)
     if (!e) throw grhip::InvalidArgument("null engine");
     e->bnl.reset();
     e->lmp.reset();
+    e->forget_lammps_call();
     live(e).release_buffers();
     e->generation++;    // a gr_system on this engine uploads its structure again
   });
@@ -890,7 +901,7 @@ void lammps_add_virials(gr_engine *e, int nall, double *vatom, int ncomp, bool d
   const bool nodes = e->lmp_rows.empty();
   const size_t rows = nodes ? (size_t) nall : e->lmp_rows.size();
   std::vector<double> v((size_t) ncomp * std::max<size_t>(rows, 1));
-  eng.fetch_vatom(v.data(), ncomp);
+  eng.fetch_vatom(v.data(), ncomp, (long long) rows);
   for (size_t q = 0; q < rows; q++) {
     const size_t a = nodes ? q : (size_t) e->lmp_rows[q];
     for (int k = 0; k < ncomp; k++) vatom[(size_t) ncomp * a + k] += v[(size_t) ncomp * q + k];

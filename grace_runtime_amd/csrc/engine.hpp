@@ -106,7 +106,8 @@ class Engine {
   // UQ outputs of the last run with RunFlags::uq, [n] each in the order of the uploaded list (null pointers are skipped)
   // per-atom virials [n_nodes][6] (xx yy zz xy xz yz) of a run with the vatom flag, in the order of the uploaded list; host memory
   // ncomp 9: the centroid form, the six components followed by yx zx zy (cvatom of kk/grace_1l_kk.h:94)
-  virtual void fetch_vatom(double *vatom, int ncomp = 6) = 0;
+  // expect_rows >= 0: the rows the caller's buffer holds; a different count held by the engine is an error
+  virtual void fetch_vatom(double *vatom, int ncomp = 6, long long expect_rows = -1) = 0;
   // the same rows added to a device array: row q of the list goes to row atom[q] (null: row q) of vatom
   virtual void add_vatom_device(const int *atom, double *vatom, int ncomp = 6) = 0;
   virtual void fetch_uq(double *gamma, double *sigma, double *cluster) = 0;

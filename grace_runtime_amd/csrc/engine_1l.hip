@@ -23,6 +23,8 @@ constexpr int kScratchMaxDevices = 64;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 static void *scratch_ptr[kScratchMaxDevices] = {};
 static std::mutex scratch_mutex;
+// one call at a time per GPU uses the array: held by radial_noalloc from its first launch until its results are written
+static std::mutex scratch_in_use[kScratchMaxDevices];
 
 // address of the current device's copy of `scratch`
 static unsigned char *scratch_of_device(int device)
@@ -563,7 +565,10 @@ template<class T> void Engine1L<T>::debug_radial(int m, const double *x, const i
 }
 
 // The radial functions of debug_radial for device arrays, without any device allocation: the staging rows live in the
-// fixed array.  Calls on one GPU share that array (also calls of different engines): they must not overlap.
+// fixed array.  Calls on one GPU share that array (also calls of different engines and of different threads): a mutex per
+// GPU lets one call at a time use it.  The caller's arrays may still be in flight on another stream (x written by a
+// kernel of the caller's library just before the call), so the call first waits for the device, as the other entry
+// points that take device arrays do.
 template<class T> void Engine1L<T>::radial_noalloc(int m, const double *x, const int *mu_j, double *Rz, double *dRz)
 {
   HIP_CHECK(hipSetDevice(device_));
@@ -586,6 +591,8 @@ template<class T> void Engine1L<T>::radial_noalloc(int m, const double *x, const
                           " bytes of the fixed " + std::to_string(kScratchBytes) + "-byte device array (at most " +
                           std::to_string((kScratchBytes - kScratchHeader - 768) / per) + " arguments for this model and precision)");
   }
+  std::lock_guard<std::mutex> in_use(scratch_in_use[device_]);
+  HIP_CHECK(hipDeviceSynchronize());
   unsigned char *base = scratch_dev_;
   int *bad = reinterpret_cast<int *>(base);
   long long *nedges = reinterpret_cast<long long *>(base + 8);    // not read: the count is passed by value

@@ -942,13 +942,11 @@ class EngineBase : public Engine, protected BufRegistry {
     if (!ran_) throw Error("fetch() before run()");
     if (nstruct != nstruct_) throw InvalidArgument("fetch_batch: the uploaded list holds " + std::to_string(nstruct_) + " structures");
     // everything the call returns goes to pinned memory as asynchronous copies behind the pass, with one wait:
-    // [zero-bond flag (2 ints, padded to 16 bytes)][records 8 nstruct][forces 3 n_nodes][per-atom energies n]
+    // [records 8 nstruct][forces 3 n_nodes][per-atom energies n]; the zero-bond flag of the pass is in pin_flag_ already
     const bool wf = forces && ran_forces_ && n_nodes_ > 0, we = eatom && ran_eatom_ && n_ > 0;
     const size_t nrec = (size_t) 8 * nstruct_, nf = wf ? (size_t) 3 * n_nodes_ : 0, ne = we ? (size_t) n_ : 0;
-    pin_out_.ensure(16 + (nrec + nf + ne) * sizeof(double));
-    int *zb = pin_out_.as<int>();
-    double *rec = reinterpret_cast<double *>(pin_out_.as<unsigned char>() + 16), *pf = rec + nrec, *pe = pf + nf;
-    zb[0] = zb[1] = -1;
+    pin_out_.ensure((nrec + nf + ne) * sizeof(double));
+    double *rec = pin_out_.as<double>(), *pf = rec + nrec, *pe = pf + nf;
     HIP_CHECK(hipMemcpyAsync(rec, scal_.p, nrec * sizeof(double), hipMemcpyDeviceToHost, stream_));
     if (wf) HIP_CHECK(hipMemcpyAsync(pf, f_.p, nf * sizeof(double), hipMemcpyDeviceToHost, stream_));
     if (we) HIP_CHECK(hipMemcpyAsync(pe, eatom_.p, ne * sizeof(double), hipMemcpyDeviceToHost, stream_));
@@ -1005,11 +1003,13 @@ class EngineBase : public Engine, protected BufRegistry {
     if (virial && ran_forces_)
       for (int k = 0; k < 6; k++) virial[k] = s[1 + k];
   }
-  void fetch_vatom(double *vatom, int ncomp) override
+  void fetch_vatom(double *vatom, int ncomp, long long expect_rows = -1) override
   {
     HIP_CHECK(hipSetDevice(device_));
     if (ncomp != 6 && ncomp != 9) throw InvalidArgument("per-atom virials have 6 or 9 components");
     if (!ran_ || !ran_vatom_) throw Error("fetch_vatom() needs a run with the per-atom virial flag (and forces)");
+    if (expect_rows >= 0 && expect_rows != n_nodes_)
+      throw Error("fetch_vatom(): the engine holds " + std::to_string(n_nodes_) + " rows, the caller expects " + std::to_string(expect_rows));
     HIP_CHECK(hipStreamSynchronize(stream_));
     check_zero_bond();
     if (!vatom || n_nodes_ <= 0) return;
@@ -1076,6 +1076,8 @@ class EngineBase : public Engine, protected BufRegistry {
   bool begin_pass(const RunFlags &fl)
   {
     HIP_CHECK(hipSetDevice(device_));
+    // argument checks first: a refused call leaves the state of the last good run (fetch() after it returns that run)
+    if (fl.uq && !has_uq_head_) throw InvalidArgument(who_ + ": the model has no usable UQ head (" + uq_why_ + ")");
     ev_used_ = 0;
     const int n = n_;
     f_.ensure(std::max<size_t>((size_t) 3 * n_nodes_, 1) * sizeof(double));
@@ -1092,7 +1094,6 @@ class EngineBase : public Engine, protected BufRegistry {
     }
     ran_eatom_ = fl.eatom;
     ran_uq_ = false;    // set by the engine that evaluates a UQ head
-    if (fl.uq && !has_uq_head_) throw InvalidArgument(who_ + ": the model has no usable UQ head (" + uq_why_ + ")");
     if (n == 0) return false;
     count_.ensure(sizeof(int) * n);
     eoff_.ensure(sizeof(long long) * (n + 1));

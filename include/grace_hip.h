@@ -140,14 +140,16 @@ int gr_engine_stage_flops(gr_engine *e, int k, double *flops);
  * Test hook for the radial-MLP kernel (the reference's counterpart is radial_x.h:29-60 evaluated on the host). */
 int gr_engine_debug_radial(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz);
 
-/* gr_engine_debug_radial for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  x [m], mu_j [m], Rz and dRz [m][lmax+1]
+/* gr_engine_debug_radial for callers that cannot allocate device memory (tight serving loops, harnesses that forbid
+ * hipMalloc, code that runs between the captures of a HIP graph and must leave the allocator alone).  No counterpart in
+ * the reference.  The call itself synchronises (it waits for the device on entry, so arrays that another stream is
+ * still writing are complete, and for its own stream before it returns): it cannot be recorded INTO a graph.  x [m], mu_j [m], Rz and dRz [m][lmax+1]
  * [n_radial] are DEVICE arrays of the engine's GPU.  The staging rows of the radial kernel live in a fixed 32 MiB
  * device array of the library (one per GPU, held until the process ends), so the call makes no hipMalloc / hipFree:
  * m is bounded by 256 + 4 m + 2 m nl CP s <= 32 MiB (CP = n_radial padded to 16 / 32 / 64, s = 8 or 4 bytes; 13 000
  * arguments for a 32-channel lmax-4 model in fp64), a larger m gives GR_INVALID with the limit in the message.
- * GRACE-1L engines only.  The call returns when Rz and dRz are written.  All calls on one GPU share the array: calls
- * that overlap on one GPU (two threads, two engines) race. */
+ * GRACE-1L engines only.  The call returns when Rz and dRz are written.  All calls on one GPU share the array: the
+ * library serialises them with one lock per GPU (calls of two threads or two engines wait for each other). */
 int gr_engine_radial_noalloc(gr_engine *e, int m, const double *x, const int *mu_j, double *Rz, double *dRz);
 
 /* Runs a plain device-to-device copy kernel (k_copy_calibration) over `bytes` bytes: the known-size kernel that the
@@ -293,8 +295,8 @@ int gr_system_compute(gr_system *s, int n, const int *types, const double *posit
  * choice libgrace/include/grace/kk/support.h:425-450).  atoms = 0: all atoms in one pass; < 0 (the default): chosen from
  * the free device memory: one pass while the work buffers fit 70 % of it, else the largest power of two >= 512 that
  * fits, and halved (down to 512) when an allocation still fails; > 0: as given.  gr_*_chunksize: atoms per pass of the last
- * call, 0 for one pass.  GRACE-1L engines evaluate chunks; the GRACE-2L and GRACE-3L engines evaluate a structure in one
- * pass and give GR_INVALID for atoms > 0. */
+ * call, 0 for one pass.  All three engine kinds evaluate chunks: GRACE-1L chunk after chunk; GRACE-2L and GRACE-3L sweep
+ * layer by layer over the chunks and repeat a layer's forward pass for a chunk before its reverse. */
 /* Atoms of one pass whose work buffers fit 70 % of the device memory the library may use, from the bytes per atom the
  * last pass held (before any pass: 262144 / 131072 / 16384 atoms for GRACE-1L / 2L / 3L).  The batch entry points bound
  * their passes by it, as the reference sizes a batch pass from the free memory (libgrace/include/grace/kk/support.h:425-450,

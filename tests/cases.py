@@ -228,3 +228,52 @@ FIXTURE_CASES_2L = [(m, c) for m in ("grace_2l_small", "grace_2l_l3", "legacy_2l
 def bond_vectors(pos, perm, offset, j, image, shifts):
     x = pos[perm]
     return x[j] - np.repeat(x, np.diff(offset), axis=0) + (shifts[image] if len(shifts) else 0.0)
+
+
+def oracle_reference(model_dir, model, pos, cell, pbc, types):
+    """Energy, forces, virial, per-atom energies and per-atom virials of the CPU oracle for a structure on its own
+    neighbour list (searched at the model's largest cutoff), in the caller's atom order.  `types` are 1-based indices
+    into the model's element list.  The independent second source the call-level GPU tests compare with (the reference
+    checks its LAMMPS bond source against its CSR source in the same way, tests/test_bonds.cpp:2-91)."""
+    from grace_runtime_amd import kk
+    from oracle import grace_oracle as g1
+    from oracle import grace_oracle_2l as g2
+    from oracle import grace_oracle_3l as g3
+    make, compute = {1: (g1.Model1L, g1.compute_1l), 2: (g2.Model2L, g2.compute_2l), 3: (g3.Model3L, g3.compute_3l)}[LAYERS[model]]
+    om = make(model_file(model_dir, model))
+    rc = float(np.max(om.cut))
+    pcell, shift = kk._padded_cell_arrays(cell, pos, rc, pbc)
+    perm, offset, j, image, shifts = kk.neighbor_search(pos + shift, pcell, pbc, rc)
+    out = compute(om, np.asarray(types)[perm] - 1, offset, j, bond_vectors(pos, perm, offset, j, image, shifts))
+    res = {"energy": float(out["energy"]), "virial": np.asarray(out["virial"])}
+    for key in ("forces", "energies", "virials"):
+        if key in out:
+            a = np.empty_like(out[key])
+            a[perm] = out[key]
+            res[key] = a
+    return res
+
+
+def golden_reference(gold, model, struct):
+    """The committed outputs of the compiled reference for an e2e case, in the caller's atom order (the goldens are stored in
+    the order of the reference's neighbour list)."""
+    tag = f"e2e/{model}/{struct}"
+    perm = gold[f"nl/{struct}@{float(gold[tag + '/rc_list']):g}/perm"]
+    res = {"energy": float(gold[tag + "/energy"]), "virial": gold[tag + "/virial"]}
+    for key in ("forces", "energies", "virials"):
+        if f"{tag}/{key}" in gold:
+            a = np.empty_like(gold[f"{tag}/{key}"])
+            a[perm] = gold[f"{tag}/{key}"]
+            res[key] = a
+    return res
+
+
+def check_against(out, ref, n, tol_e, tol_f, tol_ea, tol_v):
+    """out (energy, forces [n..], virial, energies) against ref to the given bounds, forces and per-atom energies scaled by
+    the largest reference force where that exceeds 1 eV/A"""
+    fs = max(1.0, np.abs(ref["forces"]).max())
+    assert abs(out["energy"] - ref["energy"]) / n < tol_e * fs
+    assert np.abs(np.asarray(out["forces"])[:n] - ref["forces"]).max() < tol_f * fs
+    assert np.abs(out["virial"] - ref["virial"]).max() < tol_v * max(1.0, np.abs(ref["virial"]).max())
+    if "energies" in out and "energies" in ref:
+        assert np.abs(np.asarray(out["energies"])[:n] - ref["energies"]).max() < tol_ea * fs

@@ -2,8 +2,8 @@
 kk/grace_2l_kk.h:141-157, kk/grace_3l_kk.h:313-324) on one GPU: a periodic structure is cut into two "ranks", each with its owned
 atoms and the ghosts its bonds reach (images of its own atoms and atoms of the other rank).  Two engines run the LAMMPS call
 side by side in two host threads; their exchange callbacks move the message rows and the adjoint rows through host buffers, as
-MPI would.  The energies of the ranks add up to, and the forces folded back onto their atoms equal, the single-engine result
-(itself checked against the oracle in the other GPU tests)."""
+MPI would.  The energies of the ranks add up to, and the forces folded back onto their atoms equal, the single-engine result,
+the fp64 CPU oracle on the uncut structure and the committed outputs of the compiled reference."""
 import threading
 
 import numpy as np
@@ -66,7 +66,7 @@ def device_call(eng, me, **kw):
 
 @pytest.mark.parametrize("arrays", ["host", "device"])
 @pytest.mark.parametrize("model,rc", [("l2mix", 5.0), ("l3mix", 5.0), ("mix2", 5.0)])
-def test_two_ranks_with_an_exchange_equal_one_engine(model_dir, model, rc, arrays):
+def test_two_ranks_with_an_exchange_equal_one_engine(model_dir, gold, model, rc, arrays):
     pos, cell, pbc, types = cases.structure_alloy54()
     m = kk.Model(cases.model_file(model_dir, model))
     ref = kk.System(m, ["Mo", "W"], skin=0.0).compute(types, pos, cell, pbc, energies=True, virials=True)
@@ -148,6 +148,16 @@ def test_two_ranks_with_an_exchange_equal_one_engine(model_dir, model, rc, array
     assert np.abs(ea - ref["energies"]).max() < 1e-10 * fs
     assert np.abs(out[0]["virial"] + out[1]["virial"] - ref["virial"]).max() < 1e-8 * fs
     assert np.abs(va - ref["virials"]).max() < 1e-9 * max(1.0, np.abs(ref["virials"]).max())
+    # and against the independent sources: the fp64 oracle on the uncut structure's own list, and (5.0 A is the cutoff of these
+    # models, so the ranks' lists hold the bonds of the reference's list) the compiled reference's committed outputs
+    two = {"energy": out[0]["energy"] + out[1]["energy"], "virial": out[0]["virial"] + out[1]["virial"], "forces": f, "energies": ea}
+    orc = cases.oracle_reference(model_dir, model, pos, cell, pbc, types)
+    cases.check_against(two, orc, n, 1e-10, 1e-9, 1e-10, 1e-8)
+    assert np.abs(va - orc["virials"]).max() < 1e-9 * max(1.0, np.abs(orc["virials"]).max())
+    gref = cases.golden_reference(gold, model, "alloy54")
+    cases.check_against(two, gref, n, 1e-6, 2e-5, 1e-5, 1e-5)
+    if "virials" in gref:
+        assert np.abs(va - gref["virials"]).max() < 2e-5 * max(1.0, np.abs(gref["virials"]).max())
 
 
 def test_device_row_movers_equal_the_host_forms(model_dir):

@@ -46,11 +46,14 @@ def lammps_inputs(pos, cell, types, reach, seed=0):
 
 @pytest.mark.parametrize("model,species,struct", [("mix2", ["Mo", "W"], "alloy54"), ("l2mix", ["Mo", "W"], "triclinic"),
                                                   ("l3mix", ["Mo", "W"], "alloy54")])
-def test_lammps_call_equals_csr_call(model_dir, model, species, struct):
+def test_lammps_call_equals_csr_call(model_dir, gold, model, species, struct):
     eng = kk.Engine(kk.Model(cases.model_file(model_dir, model)), species, 64)
     pos, cell, pbc, types = cases.STRUCTURES[struct]()
     n = len(pos)
     ref = kk.System(eng.model, species, skin=0.0).compute(types, pos, cell, pbc, energies=True)
+    # the independent sources: the fp64 oracle on the structure's own list and the compiled reference's committed outputs
+    orc = cases.oracle_reference(model_dir, model, pos, cell, pbc, types)
+    gref = cases.golden_reference(gold, model, struct)
     rc = max(eng.cutoff(a, b) for a in (1, 2) for b in (1, 2))
     x, t, owner, rows = lammps_inputs(pos, cell, types, rc + 0.7)
     f0 = np.random.default_rng(1).standard_normal((len(x), 3))              # forces are added to what the array holds
@@ -61,8 +64,18 @@ def test_lammps_call_equals_csr_call(model_dir, model, species, struct):
     assert np.array_equal(out["forces"][n:], f0[n:])                        # nothing is left on the ghosts
     assert np.abs(out["virial"] - ref["virial"]).max() < 1e-9 * max(1.0, np.abs(ref["virial"]).max())
     assert np.abs(out["energies"][:n] - ref["energies"]).max() < 1e-10 * fs and np.all(out["energies"][n:] == 0)
+    mine = dict(out, forces=out["forces"][:n] - f0[:n])
+    cases.check_against(mine, orc, n, 1e-10, 1e-9, 1e-10, 1e-9)                 # fp64 oracle
+    cases.check_against(mine, gref, n, 1e-6, 2e-5, 1e-5, 1e-5)                  # compiled reference (fp32 + tables): its gate
     eo = eng.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows, owner=owner, energy_only=True)
     assert abs(eo["energy"] - ref["energy"]) < 1e-10 * max(1.0, abs(ref["energy"])) and "forces" not in eo
+    assert abs(eo["energy"] - orc["energy"]) / n < 1e-10 * fs
+    # ghosts as atoms of their own (no owner map; GRACE-1L has no message to exchange): forces folded onto the owners
+    if eng.comm_layers == 0:
+        loose = eng.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows, energies=True)
+        folded = loose["forces"][:n].copy()
+        np.add.at(folded, owner[n:], loose["forces"][n:])
+        cases.check_against(dict(loose, forces=folded), orc, n, 1e-10, 1e-9, 1e-10, 1e-9)
 
 
 @pytest.mark.parametrize("layout", ["right", "left"])
@@ -96,6 +109,9 @@ def test_device_arrays_equal_host_arrays(model_dir, model, species, struct, layo
     assert np.abs(f.cpu().numpy() - ref["forces"]).max() < 1e-9 * fs
     assert np.abs(out["virial"] - ref["virial"]).max() < 1e-9 * max(1.0, np.abs(ref["virial"]).max())
     assert np.abs(ea.cpu().numpy() - ref["energies"]).max() < 1e-10 * fs
+    orc = cases.oracle_reference(model_dir, model, pos, cell, pbc, types)
+    cases.check_against({"energy": out["energy"], "virial": out["virial"], "forces": f.cpu().numpy()[:n] - f0[:n],
+                         "energies": ea.cpu().numpy()}, orc, n, 1e-10, 1e-9, 1e-10, 1e-9)
     eo = eng.compute_lammps_device(n, td, xd, il, nn, nb, owner=od, energy_only=True)
     assert abs(eo["energy"] - ref["energy"]) < 1e-10 * max(1.0, abs(ref["energy"]))
     if eng.comm_layers:                                                     # a message needs the map or an exchange
@@ -150,6 +166,10 @@ def test_same_list_renews_only_the_bond_vectors(model_dir, model, species, struc
         assert abs(got[0] - want[0]) < 1e-11 * max(1.0, abs(want[0])) and abs(got[0] - e0) > 1e-6
         for a, b in zip(got[1:], want[1:]):                  # sums by atomic adds: equal up to their order
             assert np.abs(a - b).max() < 1e-11 * max(1.0, np.abs(b).max())
+        # the same_list step against the oracle on the moved atoms (its own list, searched anew)
+        moved = xd[:n].cpu().numpy()
+        orc = cases.oracle_reference(model_dir, model, moved, cell, pbc, types)
+        cases.check_against({"energy": got[0], "virial": got[1], "forces": got[2][:n], "energies": got[3]}, orc, n, 1e-10, 1e-9, 1e-10, 1e-9)
     # another list on the engine in between: the hint is dropped and the list converted again
     eng.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows, owner=owner)
     got, want = call(eng, True), call(fresh, False)

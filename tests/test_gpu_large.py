@@ -57,7 +57,11 @@ def test_full_size_configuration_equals_the_compiled_reference(name, large, benc
     assert len(j) == int(large[f"{name}/nbonds"])
     for key, arr in (("perm", perm), ("offset", offset), ("j", j), ("image", image)):
         assert np.array_equal(sha(arr), large[f"{name}/nl_sha256_{key}"]), key
-    assert np.abs(shifts - large[f"{name}/nl_shifts"]).max() < 1e-12
+    # the shift vectors S cell: equal up to the reference's own FMA contraction (about one unit in the last place of the
+    # largest entry), the same bound as for the small structures
+    ref_shifts = large[f"{name}/nl_shifts"]
+    assert shifts.shape == ref_shifts.shape
+    assert np.abs(shifts - ref_shifts).max() <= 4e-16 * max(1.0, np.abs(ref_shifts).max())
     # energy, virial, sampled forces and per-atom energies at the reference's fp32 gate
     idx = large[f"{name}/atoms"]
     fmax = float(large[f"{name}/max_abs_force"])

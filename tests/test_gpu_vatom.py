@@ -51,6 +51,9 @@ def test_virials_of_a_system_in_chunks_and_through_the_lammps_calls(model_dir, m
     n = len(pos)
     one = kk.System(mdl, ["Mo", "W"], skin=0.0, chunksize=0).compute(types, pos, cell, pbc, virials=True)
     va = one["virials"]                                                    # in the caller's atom order
+    # the rows every path below is compared with are the oracle's rows (the independent source)
+    orc = cases.oracle_reference(model_dir, model, pos, cell, pbc, types)
+    assert np.abs(va - orc["virials"]).max() < 1e-10 * max(1.0, np.abs(orc["virials"]).max())
     assert va.shape == (n, 6) and np.abs(va.sum(0) - one["virial"]).max() < 1e-10 * max(1.0, np.abs(one["virial"]).max())
     chunked = kk.System(mdl, ["Mo", "W"], skin=0.0, chunksize=13).compute(types, pos, cell, pbc, virials=True)
     assert np.abs(chunked["virials"] - va).max() < 1e-10 * max(1.0, np.abs(va).max())
@@ -64,6 +67,7 @@ def test_virials_of_a_system_in_chunks_and_through_the_lammps_calls(model_dir, m
     v0 = np.random.default_rng(3).standard_normal((len(x), 6))            # rows are ADDED
     out = eng.compute_lammps(n, t, x, np.arange(n), [len(r) for r in rows], rows, owner=owner, vatom=v0.copy())
     assert np.abs(out["vatom"][:n] - v0[:n] - va).max() < 1e-9 * max(1.0, np.abs(va).max())
+    assert np.abs(out["vatom"][:n] - v0[:n] - orc["virials"]).max() < 1e-9 * max(1.0, np.abs(va).max())
     assert np.array_equal(out["vatom"][n:], v0[n:])
     with pytest.raises(RuntimeError, match="follow a gr_compute_lammps_device call"):
         kk._lib.check(kk._lib.lib().gr_lammps_add_vatom_device(eng._h, len(x), v0.ctypes.data))
@@ -78,6 +82,7 @@ def test_virials_of_a_system_in_chunks_and_through_the_lammps_calls(model_dir, m
                               torch.as_tensor(np.array([len(r) for r in rows], np.int32), device=dev), torch.as_tensor(nbh, device=dev),
                               owner=torch.as_tensor(owner, device=dev), forces=f, vatom=vd)
     assert np.abs(vd.cpu().numpy()[:n] - v0[:n] - va).max() < 1e-9 * max(1.0, np.abs(va).max())
+    assert np.abs(vd.cpu().numpy()[:n] - v0[:n] - orc["virials"]).max() < 1e-9 * max(1.0, np.abs(va).max())
     assert np.array_equal(vd.cpu().numpy()[n:], v0[n:])
 
 

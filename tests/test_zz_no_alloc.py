@@ -38,12 +38,76 @@ def test_no_alloc_radial_equals_debug_radial_on_consecutive_calls(model_path, pr
         xd, mud = torch.tensor(x, device=dev), torch.tensor(mu, device=dev)
         R = torch.full((m, nl, Cn), float("nan"), dtype=torch.float64, device=dev)
         dR = torch.full((m, nl, Cn), float("nan"), dtype=torch.float64, device=dev)
-        torch.cuda.synchronize()
+        # no synchronisation here: the fills above are still queued on torch's stream when the call starts
         eng.radial_noalloc(xd, mud, R, dR)
         assert np.array_equal(R.cpu().numpy(), R_ref), (precision, m)
         assert np.array_equal(dR.cpu().numpy(), dR_ref), (precision, m)
     assert _lib.lib().gr_memory_in_use() == used    # the library's own allocations did not change
     eng.close()
+
+
+def test_no_alloc_radial_waits_for_arguments_written_on_another_stream(model_path):
+    """x is produced on torch's stream right before the call, behind a long queue of work, with no synchronisation by
+    the caller: the entry point itself waits for the device before its kernels read x."""
+    import torch
+    model = kk.Model(model_path)
+    eng = kk.Engine(model, ["Mo", "W"], 64)
+    nl, Cn, nel = model.lmax + 1, model.n_radial, len(model.element_names)
+    dev = torch.device("cuda", 0)
+    m = 2048
+    x, mu = _args(m, nel, 21)
+    R_ref, dR_ref = eng.debug_radial(x, mu)
+    mud = torch.tensor(mu, device=dev)
+    R = torch.empty((m, nl, Cn), dtype=torch.float64, device=dev)
+    dR = torch.empty_like(R)
+    xh = torch.tensor(x).pin_memory()
+    big = torch.ones((4096, 4096), dtype=torch.float64, device=dev)
+    torch.cuda.synchronize()
+    for _ in range(4):
+        big = big @ big * 1e-4                   # a few hundred milliseconds of queued work in front of x
+    xd = torch.full((m,), 0.5, dtype=torch.float64, device=dev)
+    xd.copy_(xh, non_blocking=True)              # x arrives last on torch's stream
+    eng.radial_noalloc(xd, mud, R, dR)
+    assert np.array_equal(R.cpu().numpy(), R_ref) and np.array_equal(dR.cpu().numpy(), dR_ref)
+    eng.close()
+
+
+def test_no_alloc_radial_calls_of_two_threads_and_two_engines_do_not_mix(model_path):
+    """Two engines called from two threads share the one fixed array of the GPU: the library serialises the calls, so
+    each gets its own values."""
+    import threading
+
+    import torch
+    model = kk.Model(model_path)
+    nl, Cn, nel = model.lmax + 1, model.n_radial, len(model.element_names)
+    dev = torch.device("cuda", 0)
+    engines = [kk.Engine(model, ["Mo", "W"], 64), kk.Engine(model, ["Mo", "W"], 64)]
+    jobs = []
+    for t in range(2):
+        m = 1500 + 700 * t
+        x, mu = _args(m, nel, 31 + t)
+        jobs.append((m, x, mu, engines[t].debug_radial(x, mu)))
+    bad = []
+
+    def work(t):
+        m, x, mu, (R_ref, dR_ref) = jobs[t]
+        xd, mud = torch.tensor(x, device=dev), torch.tensor(mu, device=dev)
+        R = torch.empty((m, nl, Cn), dtype=torch.float64, device=dev)
+        dR = torch.empty_like(R)
+        for _ in range(20):
+            engines[t].radial_noalloc(xd, mud, R, dR)
+            if not (np.array_equal(R.cpu().numpy(), R_ref) and np.array_equal(dR.cpu().numpy(), dR_ref)):
+                bad.append(t)
+                return
+
+    th = [threading.Thread(target=work, args=(t,)) for t in range(2)]
+    for t in th:
+        t.start()
+    for t in th:
+        t.join()
+    assert not bad
+    for e in engines:
+        e.close()
 
 
 def test_no_alloc_radial_limits_and_errors(model_path):
