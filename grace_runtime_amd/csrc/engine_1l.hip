@@ -3,6 +3,7 @@
 // and the staged GPU pipeline of libgrace/include/grace/kk/grace_1l_kk.h:449-454; liveness pruning of FC outputs and
 // CG terms after libgrace/src/fused_1l.cpp:176-216.
 #include "engine_common.hpp"
+#include "jit_chain.hpp"
 
 #include <mutex>
 
@@ -82,6 +83,7 @@ template<class T> class Engine1L final : public EngineBase {
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
   }
 
+  ~Engine1L() override { chain_.release(); }
   int layers() const override { return 1; }
   void run(const RunFlags &fl) override;
   void debug_radial(int m, const double *x, const int *mu_j, double *Rz, double *dRz) override;
@@ -105,6 +107,12 @@ template<class T> class Engine1L final : public EngineBase {
   DevFc<T> fcA1_, fcAA1_, fcAA2_;
   DevFcPairBwd<T> fcAA12_;    // reverse of fc_AA1 and fc_AA2 in one pass over their shared inputs (models with the AAAA stage)
   DevProd pAA_, pAAA_, pAAAA_;
+  // the whole chain A -> A1 -> AA -> AA1 / AA2 -> AAA / AAAA as one generated kernel per direction (jit_chain.hpp); not
+  // ok(): the stage-by-stage kernels above run
+  ChainKernels chain_;
+  DevBuf chainW_;
+  std::string chain_note_;
+  bool red_writes_ = false;    // the reverse of the rho reduce may overwrite the adjoints (every function collected at most once)
   DevReduce<T> redrho_;
   UqDev<T> uq_{};             // UQ head (models that carry a valid one)
   DevBuf uqR_, uqCen_, uqIcov_, uqNcl_, uqThr_, uqCi_[4];
@@ -222,6 +230,40 @@ template<class T> void Engine1L<T>::build()
         jit_compile_product("prod_AAA", hAAA.terms, nAA_, nlm_, nAAA_, false, CFP_, f32, arch_, pAAA_.jit, pAAA_.jit_note);
       if (order4_) jit_compile_product("prod_AAAA", hAAAA.terms, nAA_, nAA_, nAAAA_, true, CFP_, f32, arch_, pAAAA_.jit, pAAAA_.jit_note);
       jit_all_ = pAA_.jit.ok() && pAAA_.jit.ok() && (!order4_ || pAAAA_.jit.ok());
+    }
+    // ---- the fused chain (same liveness, same pruned term lists)
+    if (CP_ == CFP_ && !(aaa_a_ && CP_ != CFP_)) {
+      ChainSpec sp;
+      sp.C = CFP_;
+      sp.f32 = sizeof(T) == 4;
+      sp.nf0 = nlm_;
+      sp.fc1 = chain_fc_spec(m.fc_A1, liveA1, nlm_);
+      sp.nP2 = nAA_;
+      sp.prod2 = hAA.terms;
+      sp.fc21 = chain_fc_spec(m.fc_AA1, liveAA1, nlm_);
+      sp.have22 = order4_;
+      if (order4_) sp.fc22 = chain_fc_spec(m.fc_AA2, liveAA2, nlm_);
+      sp.nP3 = nAAA_;
+      sp.prod3 = hAAA.terms;
+      sp.prod3_right_x0 = aaa_a_;
+      sp.nP4 = nAAAA_;
+      if (order4_) sp.prod4 = hAAAA.terms;
+      sp.keepP2 = collected(m.red_AA, nAA_);
+      sp.keepX0 = collected(m.red_A, nlm_);
+      for (int q = 0; q < 16; q++) sp.drow[q] = drow_[q];
+      std::vector<double> w;
+      if (jit_compile_chain("chain_1l", sp, arch_, chain_, w, chain_note_)) {
+        std::vector<T> wt(w.begin(), w.end());
+        upload_vec(chainW_, wt);
+      } else {
+        log_message(1, "GRACE-1L: the dense chain runs stage by stage (" + chain_note_ + ")");
+      }
+      // the reverse of the rho reduce may write its rows instead of adding to cleared ones when no function is collected twice
+      red_writes_ = true;
+      for (const ReduceWeights *rw : {&m.red_A, &m.red_AA, &m.red_AAA, &m.red_AAAA}) {
+        std::set<int> seen;
+        for (int c : rw->collect_ind) red_writes_ = red_writes_ && seen.insert(c).second;
+      }
     }
     fcA1_.build(m.fc_A1, liveA1, nlm_, CP_, CP_, CFP_, drow_, false, true);    // both inputs are A: one reverse launch
     fcAA1_.build(m.fc_AA1, liveAA1, nlm_, CFP_, CP_, CFP_, drow_);
@@ -416,13 +458,26 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
   T *A = A_.as<T>(), *A1 = A1_.as<T>(), *AA = AA_.as<T>(), *AA1 = AA1_.as<T>(), *AA2 = AA2_.as<T>(), *AAA = AAA_.as<T>(),
     *AAAA = AAAA_.as<T>();
   const T *Ar = aaa_a_ ? A : A1;
-  stage("fc_A1", [&] { launch_gemm(fcA1_.fwd, ka, ka, kf, A, nlm_, A, nlm_, A1, nlm_, 0); });
-  prod_fwd("prod_AA", pAA_, A1, A1, AA, nlm_, nlm_);
-  stage("fc_AA1", [&] { launch_gemm(fcAA1_.fwd, kf, ka, kf, AA, nAA_, A, nlm_, AA1, nAA_, 0); });
-  prod_fwd("prod_AAA", pAAA_, AA1, Ar, AAA, nAA_, nlm_);
-  if (order4_) {
-    stage("fc_AA2", [&] { launch_gemm(fcAA2_.fwd, kf, ka, kf, AA, nAA_, A, nlm_, AA2, nAA_, 0); });
-    prod_fwd("prod_AAAA", pAAAA_, AA2, AA2, AAAA, nAA_, nAA_);
+  const bool fused = chain_.ok();
+  const T *chainW = chainW_.as<T>();
+  const unsigned chain_blocks = fused ? (unsigned) ((n + chain_.atoms_per_block - 1) / chain_.atoms_per_block) : 0;
+  if (fused) {
+    // A -> A1 -> AA -> AA1 / AA2 -> AAA / AAAA in one kernel: AA is written for the functions the rho reduce collects only
+    stage("chain_fwd", [&] {
+      const T *x0 = A;
+      void *args[] = {(void *) &x0, (void *) &A1, (void *) &AA, (void *) &AA1, (void *) &AA2, (void *) &AAA, (void *) &AAAA, (void *) &chainW, (void *) &nat,
+                      (void *) &one};
+      HIP_CHECK(hipModuleLaunchKernel(chain_.fwd, chain_blocks, 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+    });
+  } else {
+    stage("fc_A1", [&] { launch_gemm(fcA1_.fwd, ka, ka, kf, A, nlm_, A, nlm_, A1, nlm_, 0); });
+    prod_fwd("prod_AA", pAA_, A1, A1, AA, nlm_, nlm_);
+    stage("fc_AA1", [&] { launch_gemm(fcAA1_.fwd, kf, ka, kf, AA, nAA_, A, nlm_, AA1, nAA_, 0); });
+    prod_fwd("prod_AAA", pAAA_, AA1, Ar, AAA, nAA_, nlm_);
+    if (order4_) {
+      stage("fc_AA2", [&] { launch_gemm(fcAA2_.fwd, kf, ka, kf, AA, nAA_, A, nlm_, AA2, nAA_, 0); });
+      prod_fwd("prod_AAAA", pAAAA_, AA2, AA2, AAAA, nAA_, nAA_);
+    }
   }
   stage("reduce_rho", [&] {
 #define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(ntiles), dim3(256), 0, stream_, redrho_.d, mu, tiles, \
@@ -462,6 +517,29 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
   // ---- reverse
   T *gA = gA_.as<T>(), *gA1 = gA1_.as<T>(), *gAA = gAA_.as<T>(), *gAA1 = gAA1_.as<T>(), *gAA2 = gAA2_.as<T>(),
     *gAAA = gAAA_.as<T>(), *gAAAA = gAAAA_.as<T>();
+  if (fused) {
+    // the reverse of the rho reduce leaves the adjoints of AAA, AAAA and of the collected functions of A and AA; the chain
+    // kernel takes them to the adjoint of A.  Rows the reduce does not visit are not read by it, so nothing is cleared
+    // when the reduce may write its rows.
+    if (!red_writes_)
+      stage("zero_grads", [&] {
+        HIP_CHECK(hipMemsetAsync(gA, 0, na * nlm_ * CP_ * sizeof(T), stream_));
+        HIP_CHECK(hipMemsetAsync(gAA, 0, na * nAA_ * CFP_ * sizeof(T), stream_));
+        HIP_CHECK(hipMemsetAsync(gAAA, 0, na * nAAA_ * CFP_ * sizeof(T), stream_));
+        if (order4_) HIP_CHECK(hipMemsetAsync(gAAAA, 0, na * nAAAA_ * CFP_ * sizeof(T), stream_));
+      });
+    stage("reduce_rho_bwd", [&] {
+      if (redrho_.njobs > 0)
+        hipLaunchKernelGGL(k_reduce_bwd<T>, dim3(ntiles, redrho_.njobs), dim3(64), 0, stream_, redrho_.d, mu, tiles, grho_.as<double>(), gA, gAA,
+                           gAAA, gAAAA, 0, red_writes_ ? 1 : 0);
+    });
+    stage("chain_bwd", [&] {
+      const T *x0 = A, *x1 = A1, *p21 = AA1, *p22 = AA2, *g2 = gAA, *g3 = gAAA, *g4 = gAAAA;
+      void *args[] = {(void *) &x0, (void *) &x1, (void *) &p21, (void *) &p22, (void *) &g2, (void *) &g3, (void *) &g4, (void *) &gA, (void *) &chainW,
+                      (void *) &nat, (void *) &one};
+      HIP_CHECK(hipModuleLaunchKernel(chain_.bwd, chain_blocks, 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+    });
+  } else {
   stage("zero_grads", [&] {
     HIP_CHECK(hipMemsetAsync(gA, 0, na * nlm_ * CP_ * sizeof(T), stream_));
     HIP_CHECK(hipMemsetAsync(gA1, 0, na * nlm_ * CFP_ * sizeof(T), stream_));
@@ -528,6 +606,7 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
   }
   prod_bwd("prod_AA_bwd", pAA_, A1, A1, gAA, gA1, gA1, nlm_, nlm_, 1, 1);
   fc_bwd("fc_A1_bwd", fcA1_, gA1, gA, gA, nlm_, ka);
+  }
 
   BondBwdArgs<T> ba{};
   ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();

@@ -388,7 +388,7 @@ inline std::string generate_blocked(const std::vector<ProdTerm> &terms, const st
 // when hiprtc cannot be used; the caller then keeps the table-driven kernels.  GRACE_HIP_JIT=0 switches the
 // specialisation off, GRACE_HIP_JIT_DUMP=<dir> writes the generated sources there.
 inline bool jit_compile_source(const char *name, const std::string &src, bool f32, const std::string &arch, JitKernels &out, std::string &why,
-                               bool in_order = false)
+                               bool in_order = false, const char *fwd_name = "prod_fwd", const char *bwd_name = "prod_bwd")
 {
   const char *sw = std::getenv("GRACE_HIP_JIT");
   if (sw && sw[0] == '0') {
@@ -452,7 +452,7 @@ inline bool jit_compile_source(const char *name, const std::string &src, bool f3
     why = "hipModuleLoadData failed";
     return false;
   }
-  if (hipModuleGetFunction(&out.fwd, out.mod, "prod_fwd") != hipSuccess || hipModuleGetFunction(&out.bwd, out.mod, "prod_bwd") != hipSuccess) {
+  if (hipModuleGetFunction(&out.fwd, out.mod, fwd_name) != hipSuccess || hipModuleGetFunction(&out.bwd, out.mod, bwd_name) != hipSuccess) {
     (void) hipGetLastError();
     out.release();
     why = "kernel not found in the compiled module";

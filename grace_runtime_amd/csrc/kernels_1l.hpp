@@ -1099,10 +1099,11 @@ __global__ __launch_bounds__(256) void k_reduce_fwd(ReduceDev<T> R, const int *m
 }
 
 // gX_s[atom][fn c][n] += sum_k grho[atom][k] W_s[mu][c][n][k]: grid (tiles, jobs), one wave per block; the jobs are all
-// (s, c) in the order of the sources, this launch takes those from job_first on
+// (s, c) in the order of the sources, this launch takes those from job_first on.  overwrite: the rows are written, not
+// added to (for callers that know every row is visited once and read no row that is not visited)
 template<class T>
 __global__ __launch_bounds__(64) void k_reduce_bwd(ReduceDev<T> R, const int *mu, const int *tile_atoms, const double *grho, T *G0, T *G1,
-                                                   T *G2, T *G3, int job_first = 0)
+                                                   T *G2, T *G3, int job_first = 0, int overwrite = 0)
 {
   typedef typename Mfma<T>::v4 v4;
   const int tile = blockIdx.x;
@@ -1129,7 +1130,10 @@ __global__ __launch_bounds__(64) void k_reduce_bwd(ReduceDev<T> R, const int *mu
 #pragma unroll
     for (int v = 0; v < 4; v++) {
       const int at = tile_atoms[tile * 16 + R.drow[4 * g + v]];
-      if (at >= 0) G[s][((long long) at * R.stride[s] + fn) * R.nin[s] + cb * 16 + c] += acc[v];
+      if (at >= 0) {
+        T *out = &G[s][((long long) at * R.stride[s] + fn) * R.nin[s] + cb * 16 + c];
+        *out = overwrite ? acc[v] : *out + acc[v];
+      }
     }
   }
 }
