@@ -375,7 +375,9 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
     ecap = 1;
     for (int k = 0; k < nchunks; k++) ecap = std::max(ecap, (size_t) (ebound[(size_t) k + 1] - ebound[(size_t) k]));
   }
-  const size_t na = (size_t) cs;
+  // rows of the per-atom tensors: the generated chain kernels run whole blocks of atoms and neither guard their loads nor
+  // their stores, so the tensors hold rows up to the end of the last block
+  const size_t na = (size_t) round_up(cs, 16);
   Rz_.ensure(ecap * noutp_ * sizeof(T));
   dRz_.ensure(ecap * noutp_ * sizeof(T));
   A_.ensure(na * nlm_ * CP_ * sizeof(T));

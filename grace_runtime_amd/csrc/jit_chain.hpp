@@ -370,8 +370,13 @@ inline bool generate_chain(const ChainSpec &sp, ChainCode &out)
   std::ostringstream s;
   s << "typedef " << (f32 ? "float" : "double") << " T;\n";
   s << "typedef T v4 __attribute__((ext_vector_type(4)));\n";
+  s << "#define ST(dst, val) dst = val\n";
+  s << "#define LDW(p, q) (p)[(q) * 64]\n";
   s << "#define MMA(a, b, c) " << (f32 ? "__builtin_amdgcn_mfma_f32_16x16x4f32" : "__builtin_amdgcn_mfma_f64_16x16x4f64") << "(a, b, c, 0, 0, 0)\n";
   s << "#define C " << C << "\n#define NA " << NA << "\n#define S " << S << "\n#define KS " << KS << "\n";
+  // The barrier between the column phase and the matrix phase of a path orders LDS traffic only: the weight requests of the
+  // next step and the stores of the results to global memory stay in flight across it (__syncthreads would wait for them).
+  s << "#define SYNC() __asm__ volatile(\"s_waitcnt lgkmcnt(0)\\n\\ts_barrier\" ::: \"memory\")\n";
   s << "__device__ const int DROW[16] = {";
   for (int q = 0; q < 16; q++) s << (q ? ", " : "") << sp.drow[q];
   s << "};\n";
@@ -379,28 +384,80 @@ inline bool generate_chain(const ChainSpec &sp, ChainCode &out)
   // items in column blocks of 16 from cb0 in steps of cbstep.  wf: the weight fragments of the segments (KS each); B0 / B1 /
   // Y: LDS rows of item 0; acc: add to the row instead of writing it.
   s << R"(
-template<int NSEG>
-__device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * KS], const T *B0, const T *B1, T *Y, int nitems, int cb0, int cbstep, int rb,
-                                        int acc, int lane)
+// One wave, one 16-row block of the output: D[row][item] = sum over the segments of W_seg (16 x C) B_seg (C x items), items
+// in column blocks of 16 from cb0 in steps of CBSTEP.  wf: the weight fragments of the segments (KS each); B0 / B1 / Y: LDS
+// rows of item 0; acc: add to the row instead of writing it.  wn / wq / NNEXT: the buffer, the lane's source pointer and the
+// count of the NEXT step's weight fragments, requested one per matrix instruction of the first column block: the
+// vector-memory pipe of the CU takes 8 cycles per request, and 16 requests per wave issued in one burst (next to the burst
+// of stores of the column phase) hold the issuing waves up.
+template<int NSEG, int NITEMS, int CBSTEP, int NNEXT, int PIPE>
+__device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * KS], T (&wn)[2 * KS], const T *wq, const T *B0, const T *B1, T *Y, int cb0,
+                                                              int rb, int acc, int lane)
 {
+  constexpr int NCB = (NITEMS + 15) / 16, MAXT = (NCB + CBSTEP - 1) / CBSTEP, NK = NSEG * KS;
   const int g = lane >> 4, c = lane & 15;
-  const int ncb = (nitems + 15) >> 4;
   const int d0 = DROW[4 * g], d1 = DROW[4 * g + 1], d2 = DROW[4 * g + 2], d3 = DROW[4 * g + 3];
-  for (int cb = cb0; cb < ncb; cb += cbstep) {
-    const int item = cb * 16 + c, it = item < nitems ? item : nitems - 1;
-    v4 d = {0, 0, 0, 0};
-    const T *b0 = B0 + it * S + g;
+  // PIPE: the B fragments of a column block and (acc) the old values of its output rows are requested while the matrix
+  // instructions of the block before it run, so that nothing but arithmetic and writes is left for the end of a block (the
+  // reverse kernel, whose output rows are read, added to and written); else at the start of the block itself (fewer registers)
+  T b[2][NK], o[2][4];
+  auto request = [&](int cb, T (&dst)[NK], T (&old)[4]) {
+    const int item = cb * 16 + c, it = item < NITEMS ? item : NITEMS - 1;
+    const T *p0 = B0 + it * S + g;
 #pragma unroll
-    for (int q = 0; q < KS; q++) d = MMA(wf[q], b0[4 * q], d);
+    for (int q = 0; q < KS; q++) dst[q] = p0[4 * q];
     if (NSEG == 2) {
-      const T *b1 = B1 + it * S + g;
+      const T *p1 = B1 + it * S + g;
 #pragma unroll
-      for (int q = 0; q < KS; q++) d = MMA(wf[KS + q], b1[4 * q], d);
+      for (int q = 0; q < KS; q++) dst[KS + q] = p1[4 * q];
     }
-    if (item < nitems) {
-      T *y = Y + it * S + rb * 16;
-      if (acc) { y[d0] += d[0]; y[d1] += d[1]; y[d2] += d[2]; y[d3] += d[3]; }
-      else { y[d0] = d[0]; y[d1] = d[1]; y[d2] = d[2]; y[d3] = d[3]; }
+    if (acc) {
+      const T *y = Y + it * S + rb * 16;
+      old[0] = y[d0]; old[1] = y[d1]; old[2] = y[d2]; old[3] = y[d3];
+    } else {
+      old[0] = old[1] = old[2] = old[3] = (T) 0;
+    }
+  };
+  if (cb0 >= NCB) {    // a wave without a column block in this step
+#pragma unroll
+    for (int q = 0; q < NNEXT; q++) wn[q] = LDW(wq, q);
+  } else if (PIPE) {
+    request(cb0, b[0], o[0]);
+  }
+#pragma unroll
+  for (int t = 0; t < MAXT; t++) {
+    const int cb = cb0 + t * CBSTEP;
+    if (cb < NCB) {
+      if (PIPE) {
+        if (t + 1 < MAXT && cb + CBSTEP < NCB) request(cb + CBSTEP, b[(t + 1) & 1], o[(t + 1) & 1]);
+      } else {
+        request(cb, b[t & 1], o[t & 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      v4 d = {0, 0, 0, 0};
+      if (t == 0) {
+#pragma unroll
+        for (int q = 0; q < NK; q++) {
+          d = MMA(wf[q], b[0][q], d);    // t == 0
+          if (q < NNEXT) wn[q] = LDW(wq, q);
+        }
+#pragma unroll
+        for (int q = NK; q < NNEXT; q++) wn[q] = LDW(wq, q);
+#pragma unroll
+        for (int q = 0; q < NK; q++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+      } else {
+#pragma unroll
+        for (int q = 0; q < NK; q++) d = MMA(wf[q], b[t & 1][q], d);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const int item = cb * 16 + c;
+      if (item < NITEMS) {
+        T *y = Y + item * S + rb * 16;
+        y[d0] = o[t & 1][0] + d[0]; y[d1] = o[t & 1][1] + d[1]; y[d2] = o[t & 1][2] + d[2]; y[d3] = o[t & 1][3] + d[3];
+      }
     }
   }
 }
@@ -410,19 +467,40 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
     o << "(wave == 0 ? " << u.off[0] << "LL : wave == 1 ? " << u.off[1] << "LL : wave == 2 ? " << u.off[2] << "LL : " << u.off[3] << "LL)";
     return o.str();
   };
-  auto load_wf = [&](const WaveUnits &u) {
+  // The weight fragments of a step (one path's FC phase) are requested one step ahead, into the buffer the current step
+  // does not use: a request issued right before its barrier is answered after ~2 us, longer than the products of a path take.
+  std::vector<const WaveUnits *> steps;    // the steps of the kernel being written, in execution order
+  size_t step = 0;
+  // the first step's fragments are requested at the start of the kernel; every step requests the next one's
+  auto request_wf = [&](size_t k) {
+    if (k >= steps.size()) return;
+    const WaveUnits &u = *steps[k];
     s << "    { const T *wq = W + " << woff(u) << " + lane;\n";
-    s << "#pragma unroll\n      for (int q = 0; q < " << u.nseg * KS << "; q++) wf[q] = wq[q * 64]; }\n";
+    s << "#pragma unroll\n      for (int q = 0; q < " << u.nseg * KS << "; q++) wf" << (k & 1) << "[q] = LDW(wq, q); }\n";
+  };
+  // begin_step: template and call arguments of fc_rows that name this step's buffer and the next step's request
+  struct StepArgs { std::string nnext, bufs; };
+  auto begin_step = [&]() {
+    StepArgs a;
+    const bool more = step + 1 < steps.size();
+    a.nnext = std::to_string(more ? steps[step + 1]->nseg * KS : 0);
+    const std::string cur = (step & 1) ? "wf1" : "wf0", nxt = (step & 1) ? "wf0" : "wf1";
+    a.bufs = cur + ", " + nxt + ", W + " + (more ? woff(*steps[step + 1]) : std::string("0")) + " + lane";
+    step++;
+    return a;
   };
   auto common_head = [&](const char *lds_decl) {
     s << "  " << lds_decl << "\n";
     s << "  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);\n";
     s << "  const int a = tid / C, n = tid % C;\n";
-    s << "  const long long at_raw = (long long) blockIdx.x * NA + a;\n";
-    s << "  const bool on = at_raw < natoms;\n";
-    s << "  const long long at = on ? at_raw : (long long) natoms - 1;\n";
+    // every tensor holds rows for a whole number of blocks (the caller pads the atom count to a multiple of NA): the
+    // columns of the atoms past the end compute on whatever those rows hold and write rows nobody reads, so no load or
+    // store is guarded and the column phases are branch-free (a guarded store ends a scheduling region: the LDS reads of
+    // a phase then wait for each other)
+    s << "  const long long at = (long long) blockIdx.x * NA + a;\n";
+    s << "  (void) natoms;\n";
     s << "  const int col = a * S + n;    // this thread's element of row 0 of a buffer whose rows are (function, atom)\n";
-    s << "  T wf[2 * KS];\n";
+    s << "  T wf0[2 * KS], wf1[2 * KS];\n";
   };
   auto sum_terms = [&](const std::vector<const ProdTerm *> &ts, const std::function<std::string(const ProdTerm *)> &f) {
     std::ostringstream o;
@@ -448,22 +526,30 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
   }
   s << "  X0 += at * " << nf0 << " * C + n; X1 += at * " << nf0 << " * C + n; P2 += at * " << nP2 << " * C + n; P21 += at * " << nP2
     << " * C + n; P22 += at * " << nP2 << " * C + n; P3 += at * " << std::max(nP3, 1) << " * C + n; P4 += at * " << std::max(nP4, 1) << " * C + n;\n";
-  for (int f = 0; f < nf0; f++) s << "  L0[" << f * NA * S << " + col] = on ? X0[" << f << " * C] : (T) 0;\n";
+  for (int f = 0; f < nf0; f++) s << "  L0[" << f * NA * S << " + col] = X0[" << f << " * C];\n";
   if (sp.prod3_right_x0)
     for (int f = 0; f < nf0; f++) s << "  const T x0_" << f << " = L0[" << f * NA * S << " + col];\n";
   for (int f = 0; f < nf0; f++) s << "  T " << x1(f) << ";\n";
   for (int o = 0; o < nP3; o++) s << "  T p3_" << o << " = (T) 0;\n";
+  // the steps of the forward kernel: FC1 paths, then the paths of P2 with an FC phase, group by group
+  steps.clear();
+  step = 0;
+  for (size_t q = 0; q < f1.size(); q++) steps.push_back(&wu_f1[q]);
+  for (const auto &g : order)
+    for (int q : g)
+      if (paths[q].any && (paths[q].l21 || paths[q].l22)) steps.push_back(&wu_p[q]);
+  request_wf(0);
   // FC1
   for (size_t q = 0; q < f1.size(); q++) {
     const Fc1Path &p = f1[q];
     s << "  {    // FC1, functions " << p.f0 << " .. " << p.f0 + p.M - 1 << "\n";
-    load_wf(wu_f1[q]);
-    s << "    __syncthreads();\n";
-    s << "    fc_rows<2>(wf, L0 + " << p.f0 * NA * S << ", L0 + " << p.r0 * NA * S << ", LY1, " << p.M * NA << ", wave >> 1, 2, wave & 1, 0, lane);\n";
-    s << "    __syncthreads();\n";
+    const StepArgs wf = begin_step();
+    s << "    SYNC();\n";
+    s << "    fc_rows<2, " << p.M * NA << ", 2, " << wf.nnext << ", 0>(" << wf.bufs << ", L0 + " << p.f0 * NA * S << ", L0 + " << p.r0 * NA * S << ", LY1, wave >> 1, wave & 1, 0, lane);\n";
+    s << "    SYNC();\n";
     for (int i = 0; i < p.M; i++) {
       const int f = p.f0 + i;
-      s << "    " << x1(f) << " = (T) " << lit(sp.fc1.nof[f], f32) << " * LY1[" << i * NA * S << " + col]; if (on) X1[" << f << " * C] = " << x1(f) << ";\n";
+      s << "    " << x1(f) << " = (T) " << lit(sp.fc1.nof[f], f32) << " * LY1[" << i * NA * S << " + col]; X1[" << f << " * C] = " << x1(f) << ";\n";
     }
     s << "  }\n";
   }
@@ -484,7 +570,7 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
       if (!p.any) continue;
       const bool gemm = p.l21 || p.l22;
       s << "    {    // path " << q << ": functions " << p.f0 << " .. " << p.f0 + p.M - 1 << "\n";
-      if (gemm) load_wf(wu_p[q]);
+      const StepArgs wf = gemm ? begin_step() : StepArgs();
       for (int i = 0; i < p.M; i++) {
         const int f = p.f0 + i;
         const auto it = p2_by_o.find(f);
@@ -492,30 +578,30 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
                                         [&](const ProdTerm *t) { return x1(t->l) + " * " + x1(t->r); });
         s << "      { const T v = " << e << ";";
         if (gemm) s << " LX[" << i * NA * S << " + col] = v;";
-        if (keep2[f]) s << " if (on) P2[" << f << " * C] = v;";
+        if (keep2[f]) s << " ST(P2[" << f << " * C], v);";
         s << " }\n";
       }
       if (gemm) {
-        s << "      __syncthreads();\n";
+        s << "      SYNC();\n";
         if (p.l21 && p.l22)
-          s << "      fc_rows<2>(wf, LX, L0 + (wave < 2 ? " << p.r21 * NA * S << " : " << p.r22 * NA * S << "), wave < 2 ? LY1 : LY2, " << p.M * NA
-            << ", 0, 1, wave & 1, 0, lane);\n";
+          s << "      fc_rows<2, " << p.M * NA << ", 1, " << wf.nnext << ", 0>(" << wf.bufs << ", LX, L0 + (wave < 2 ? " << p.r21 * NA * S << " : " << p.r22 * NA * S
+            << "), wave < 2 ? LY1 : LY2, 0, wave & 1, 0, lane);\n";
         else
-          s << "      fc_rows<2>(wf, LX, L0 + " << (p.l22 ? p.r22 : p.r21) * NA * S << ", " << (p.l22 ? "LY2" : "LY1") << ", " << p.M * NA
-            << ", wave >> 1, 2, wave & 1, 0, lane);\n";
-        s << "      __syncthreads();\n";
+          s << "      fc_rows<2, " << p.M * NA << ", 2, " << wf.nnext << ", 0>(" << wf.bufs << ", LX, L0 + " << (p.l22 ? p.r22 : p.r21) * NA * S << ", " << (p.l22 ? "LY2" : "LY1")
+            << ", wave >> 1, wave & 1, 0, lane);\n";
+        s << "      SYNC();\n";
         for (int i = 0; i < p.M; i++) {
           const int f = p.f0 + i;
           if (live21[f]) {
-            s << "      { const T v = (T) " << lit(sp.fc21.nof[f], f32) << " * LY1[" << i * NA * S << " + col]; if (on) P21[" << f << " * C] = v;";
+            s << "      { const T v = (T) " << lit(sp.fc21.nof[f], f32) << " * LY1[" << i * NA * S << " + col]; ST(P21[" << f << " * C], v);";
             const auto it = p3_by_l.find(f);
             if (it != p3_by_l.end())
               for (const ProdTerm *t : it->second) s << " p3_" << t->o << " += (T) " << lit(t->c, f32) << " * v * " << xr(t->r) << ";";
             s << " }\n";
           }
           if (live22[f]) {
-            s << "      " << v2(f) << " = (T) " << lit(sp.fc22.nof[f], f32) << " * LY2[" << i * NA * S << " + col]; if (on) P22[" << f << " * C] = " << v2(f)
-              << ";\n";
+            s << "      " << v2(f) << " = (T) " << lit(sp.fc22.nof[f], f32) << " * LY2[" << i * NA * S << " + col]; ST(P22[" << f << " * C], " << v2(f)
+              << ");\n";
             for (const auto *m : {&p4_by_l, &p4_by_r}) {
               const auto it = m->find(f);
               if (it != m->end())
@@ -527,14 +613,14 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
       s << "    }\n";
     }
     if (!outs4.empty()) {
-      s << "    if (on) {\n";
+      s << "    {\n";
       for (int o : outs4)
-        s << "      P4[" << o << " * C] = " << sum_terms(p4_by_o[o], [&](const ProdTerm *t) { return v2(t->l) + " * " + v2(t->r); }) << ";\n";
+        s << "      ST(P4[" << o << " * C], " << sum_terms(p4_by_o[o], [&](const ProdTerm *t) { return v2(t->l) + " * " + v2(t->r); }) << ");\n";
       s << "    }\n";
     }
     s << "  }\n";
   }
-  s << "  if (on) {\n";
+  s << "  {\n";
   for (int o = 0; o < nP3; o++) s << "    P3[" << o << " * C] = p3_" << o << ";\n";
   for (int o = 0; o < nP4; o++)
     if (!p4_by_o.count(o)) s << "    P4[" << o << " * C] = (T) 0;\n";
@@ -559,6 +645,55 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
   for (int f = 0; f < nf0; f++) s << "  T g1_" << f << " = (T) 0;\n";
   for (int o = 0; o < nP3; o++) s << "  const T g3_" << o << " = gP3[" << o << " * C];\n";
   auto gr = [&](int f) { return (sp.prod3_right_x0 ? "gx0_" : "g1_") + std::to_string(f); };
+  // the reverse of P3 with respect to its right operand needs P21 only here: all of it up front, with every load in flight
+  // at once, instead of a load per path whose latency nothing hides (one wave per SIMD)
+  s << "  {\n";
+  for (const auto &kv : p3_by_l) s << "    const T p_" << kv.first << " = P21[" << kv.first << " * C];\n";
+  for (const auto &kv : p3_by_l)
+    for (const ProdTerm *t : kv.second) s << "    " << gr(t->r) << " += (T) " << lit(t->c, f32) << " * g3_" << t->o << " * p_" << kv.first << ";\n";
+  s << "  }\n";
+  for (int f = 0; f < nP2; f++)
+    if (keep2[f] && p2_by_o.count(f)) s << "  const T gk_" << f << " = gP2[" << f << " * C];\n";
+  // the P22 rows and the P4 adjoints of a group are requested one path ahead of the group (behind the column phase of the
+  // last path of the group before it, whose own rows are dead by then), so that they arrive during that path's matrix phase
+  for (int f = 0; f < nP2; f++)
+    if (live22[f]) s << "  T " << v2(f) << ";\n";
+  for (int o = 0; o < nP4; o++)
+    if (p4_by_o.count(o)) s << "  T g4_" << o << ";\n";
+  std::vector<size_t> live_groups;
+  for (size_t gi = 0; gi < order.size(); gi++) {
+    bool any = false;
+    for (int q : order[gi]) any = any || paths[q].any;
+    if (any) live_groups.push_back(gi);
+  }
+  auto group_loads = [&](size_t gi, const char *p22, const char *g4p, const char *indent) {
+    std::set<int> outs4;
+    for (int q : order[gi])
+      if (paths[q].l22)
+        for (int i = 0; i < paths[q].M; i++) {
+          const int f = paths[q].f0 + i;
+          s << indent << v2(f) << " = " << p22 << "[" << f << " * C];\n";
+          for (const auto *m : {&p4_by_l, &p4_by_r}) {
+            const auto it = m->find(f);
+            if (it != m->end())
+              for (const ProdTerm *t : it->second) outs4.insert(t->o);
+          }
+        }
+    for (int o : outs4) s << indent << "g4_" << o << " = " << g4p << "[" << o << " * C];\n";
+  };
+  if (!live_groups.empty()) {
+    s << "  for (int it = 0; it < one; it++) {\n    const T *P22v = P22 + it, *gP4v = gP4 + it;\n";
+    group_loads(live_groups[0], "P22v", "gP4v", "    ");
+    s << "  }\n";
+  }
+  // the steps of the reverse kernel: the paths of P2 with an FC phase, group by group, then the FC1 paths
+  steps.clear();
+  step = 0;
+  for (const auto &g : order)
+    for (int q : g)
+      if (paths[q].any && (paths[q].l21 || paths[q].l22)) steps.push_back(&wu_pb[q]);
+  for (size_t q = 0; q < f1.size(); q++) steps.push_back(&wu_f1b[q]);
+  request_wf(0);
   for (const auto &g : order) {
     bool any = false;
     for (int q : g) any = any || paths[q].any;
@@ -569,28 +704,23 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
     s << "  for (int it = 0; it < one; it++) {    // group of paths";
     for (int q : g) s << " " << q;
     s << "\n";
-    s << "    const T *P21v = P21 + it, *P22v = P22 + it, *gP2v = gP2 + it, *gP4v = gP4 + it;\n";
-    std::set<int> outs4;
+    s << "    const T *P22v = P22 + it, *gP4v = gP4 + it;\n";
+    // the last path of this group with a matrix phase requests the next group's rows
+    int last_gemm = -1;
     for (int q : g)
-      if (paths[q].l22)
-        for (int i = 0; i < paths[q].M; i++) {
-          const int f = paths[q].f0 + i;
-          s << "    const T " << v2(f) << " = P22v[" << f << " * C];\n";
-          for (const auto *m : {&p4_by_l, &p4_by_r}) {
-            const auto it = m->find(f);
-            if (it != m->end())
-              for (const ProdTerm *t : it->second) outs4.insert(t->o);
-          }
-        }
-    for (int o : outs4) s << "    const T g4_" << o << " = gP4v[" << o << " * C];\n";
+      if (paths[q].any && (paths[q].l21 || paths[q].l22)) last_gemm = q;
+    size_t next_group = order.size();
+    for (size_t k = 0; k + 1 < live_groups.size(); k++)
+      if (&order[live_groups[k]] == &g) next_group = live_groups[k + 1];
+    bool next_requested = false;
     for (int q : g) {
       const Path &p = paths[q];
       if (!p.any) continue;
       const bool gemm = p.l21 || p.l22;
       s << "    for (int ip = 0; ip < one; ip++) {    // path " << q << ": functions " << p.f0 << " .. " << p.f0 + p.M - 1 << "\n";
-      s << "      const T *P21w = P21v + ip, *gP2w = gP2v + ip;\n";
+      s << "      const T *P22w = P22v + ip, *gP4w = gP4v + ip;\n";
+      const StepArgs wf = gemm ? begin_step() : StepArgs();
       if (gemm) {
-        load_wf(wu_pb[q]);
         for (int i = 0; i < p.M; i++) {
           const int f = p.f0 + i;
           if (p.l21) {
@@ -598,10 +728,8 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
               const auto it = p3_by_l.find(f);
               const std::vector<const ProdTerm *> none;
               const auto &ts = it == p3_by_l.end() ? none : it->second;
-              s << "      { const T p = P21w[" << f << " * C];";
-              for (const ProdTerm *t : ts) s << " " << gr(t->r) << " += (T) " << lit(t->c, f32) << " * g3_" << t->o << " * p;";
-              s << " LX1[" << i * NA * S << " + col] = (T) " << lit(sp.fc21.nof[f], f32) << " * ("
-                << sum_terms(ts, [&](const ProdTerm *t) { return "g3_" + std::to_string(t->o) + " * " + xr(t->r); }) << "); }\n";
+              s << "      LX1[" << i * NA * S << " + col] = (T) " << lit(sp.fc21.nof[f], f32) << " * ("
+                << sum_terms(ts, [&](const ProdTerm *t) { return "g3_" + std::to_string(t->o) + " * " + xr(t->r); }) << ");\n";
             } else {
               s << "      LX1[" << i * NA * S << " + col] = (T) 0;\n";
             }
@@ -628,14 +756,18 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
             }
           }
         }
-        s << "      __syncthreads();\n";
+        if (q == last_gemm && next_group < order.size()) {
+          group_loads(next_group, "P22w", "gP4w", "      ");
+          next_requested = true;
+        }
+        s << "      SYNC();\n";
         // waves 0, 1: adjoint of P2 (left weights) into LY; waves 2, 3: adjoint of X0 (right weights) added to its rows
         const char *b0 = p.l21 ? "LX1" : "LX2";
         const int rr = p.l21 ? p.r21 : p.r22;
         if (p.l21 && p.l22 && p.r21 != p.r22) { out.why = "the two layers of a path read different right inputs"; return false; }
-        s << "      fc_rows<" << wu_pb[q].nseg << ">(wf, " << b0 << ", LX2, wave < 2 ? LY : LG + " << rr * NA * S << ", " << p.M * NA
-          << ", 0, 1, wave & 1, wave >> 1, lane);\n";
-        s << "      __syncthreads();\n";
+        s << "      fc_rows<" << wu_pb[q].nseg << ", " << p.M * NA << ", 1, " << wf.nnext << ", 1>(" << wf.bufs << ", " << b0 << ", LX2, wave < 2 ? LY : LG + " << rr * NA * S
+          << ", 0, wave & 1, wave >> 1, lane);\n";
+        s << "      SYNC();\n";
       }
       for (int i = 0; i < p.M; i++) {
         const int f = p.f0 + i;
@@ -645,7 +777,7 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
         s << "      { const T g = ";
         if (gemm) s << "LY[" << i * NA * S << " + col]";
         if (gemm && keep2[f]) s << " + ";
-        if (keep2[f]) s << "gP2w[" << f << " * C]";
+        if (keep2[f]) s << "gk_" << f;
         s << ";";
         for (const ProdTerm *t : it->second) {
           s << " { const T cg = (T) " << lit(t->c, f32) << " * g; g1_" << t->l << " += cg * " << x1(t->r) << "; g1_" << t->r << " += cg * " << x1(t->l)
@@ -655,6 +787,7 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
       }
       s << "    }\n";
     }
+    if (!next_requested && next_group < order.size()) group_loads(next_group, "P22v", "gP4v", "    ");
     s << "  }\n";
   }
   // reverse of FC1
@@ -662,24 +795,24 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
     const Fc1Path &p = f1[q];
     const bool same = p.r0 == p.f0;
     s << "  {    // FC1 reverse, functions " << p.f0 << " .. " << p.f0 + p.M - 1 << "\n";
-    load_wf(wu_f1b[q]);
+    const StepArgs wf = begin_step();
     for (int i = 0; i < p.M; i++) {
       const int f = p.f0 + i;
       s << "    LX1[" << i * NA * S << " + col] = (T) " << lit(sp.fc1.nof[f], f32) << " * g1_" << f << ";\n";
     }
-    s << "    __syncthreads();\n";
+    s << "    SYNC();\n";
     if (same)
-      s << "    fc_rows<2>(wf, LX1, LX1, LG + " << p.f0 * NA * S << ", " << p.M * NA << ", wave >> 1, 2, wave & 1, 1, lane);\n";
+      s << "    fc_rows<2, " << p.M * NA << ", 2, " << wf.nnext << ", 1>(" << wf.bufs << ", LX1, LX1, LG + " << p.f0 * NA * S << ", wave >> 1, wave & 1, 1, lane);\n";
     else
-      s << "    fc_rows<1>(wf, LX1, LX1, LG + (wave < 2 ? " << p.f0 * NA * S << " : " << p.r0 * NA * S << "), " << p.M * NA << ", 0, 1, wave & 1, 1, lane);\n";
-    s << "    __syncthreads();\n";
+      s << "    fc_rows<1, " << p.M * NA << ", 1, " << wf.nnext << ", 1>(" << wf.bufs << ", LX1, LX1, LG + (wave < 2 ? " << p.f0 * NA * S << " : " << p.r0 * NA * S << "), 0, wave & 1, 1, lane);\n";
+    s << "    SYNC();\n";
     s << "  }\n";
   }
   // when left and right rows of FC1 differ, two waves may add to one row in the same phase only if the rows of a path's two
   // sides are disjoint
   for (const Fc1Path &p : f1)
     if (p.r0 != p.f0 && p.r0 < p.f0 + p.M && p.f0 < p.r0 + p.M) { out.why = "fc1: left and right rows of a path overlap"; return false; }
-  s << "  if (on) {\n";
+  s << "  {\n";
   std::vector<char> keep0 = sp.keepX0;
   keep0.resize(nf0, 0);
   for (int f = 0; f < nf0; f++) {

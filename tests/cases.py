@@ -33,6 +33,30 @@ def model_cut2():
     return d
 
 
+def model_ch20():
+    """two elements, lmax 3, 20 channels in every stage (padded to 32 on the device: the widths the fused dense chain
+    covers), with the AAAA stage"""
+    return synth.random_model_1l(lmax=3, n_elements=2, element_names=("Mo", "W"), embedding_size=12, nradbase=8,
+                                 nradmax=20, hidden=32, rho_n_out=9, energy_hidden=16, rcut=5.0,
+                                 inv_avg_n_neigh=1.0 / 26.0, seed=31)
+
+
+def model_ch3():
+    """two elements, lmax 2, 32 channels, max_order 3 (no AA2 / AAAA stage)"""
+    return synth.random_model_1l(lmax=2, n_elements=2, element_names=("Mo", "W"), embedding_size=8, nradbase=8,
+                                 nradmax=32, hidden=32, rho_n_out=7, energy_hidden=16, rcut=5.0, order4=False,
+                                 inv_avg_n_neigh=1.0 / 26.0, seed=32)
+
+
+def model_chleg():
+    """two elements, lmax 2, 24 channels, the legacy product AAA = AA1 x A (right operand A instead of A1)"""
+    d = synth.random_model_1l(lmax=2, n_elements=2, element_names=("Mo", "W"), embedding_size=8, nradbase=8,
+                              nradmax=24, hidden=32, rho_n_out=7, energy_hidden=16, rcut=5.0,
+                              inv_avg_n_neigh=1.0 / 26.0, seed=33)
+    d["AAA_right_A"] = np.array([1], dtype=np.int64)
+    return d
+
+
 def model_l2mix():
     """GRACE-2L, two elements with pair-specific cutoffs, lmax 2, different (unpadded) widths in every stage"""
     d = synth.random_model_2l(lmax=2, n_elements=2, element_names=("Mo", "W"), embedding_size=8, nradbase=10, c1=20, cr=12,
@@ -152,8 +176,8 @@ def model_uq3l():
     return d
 
 
-MODELS = {"uq3l": model_uq3l, "uq2l": model_uq2l, "uq2": model_uq2, "l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3el": model_l3el, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
-LAYERS = {"uq3l": 3, "uq2l": 2, "uq2": 1, "l3mix": 3, "l3wide": 3, "l3pad": 3, "l3el": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
+MODELS = {"ch20": model_ch20, "ch3": model_ch3, "chleg": model_chleg, "uq3l": model_uq3l, "uq2l": model_uq2l, "uq2": model_uq2, "l3mix": model_l3mix, "l3wide": model_l3wide, "l3pad": model_l3pad, "l3el": model_l3el, "l3nat": model_l3nat, "config4": model_config4, "config5": model_config5, "config1": model_config1, "mix2": model_mix2, "cut2": model_cut2, "config3": model_config3, "l2mix": model_l2mix}
+LAYERS = {"ch20": 1, "ch3": 1, "chleg": 1, "uq3l": 3, "uq2l": 2, "uq2": 1, "l3mix": 3, "l3wide": 3, "l3pad": 3, "l3el": 3, "l3nat": 3, "config4": 3, "config5": 2, "config1": 1, "mix2": 1, "cut2": 1, "config3": 2, "l2mix": 2}
 
 
 def write_model(name, directory):
