@@ -470,6 +470,7 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
       void *args[] = {(void *) &x0, (void *) &A1, (void *) &AA, (void *) &AA1, (void *) &AA2, (void *) &AAA, (void *) &AAAA, (void *) &chainW, (void *) &nat,
                       (void *) &one};
       HIP_CHECK(hipModuleLaunchKernel(chain_.fwd, chain_blocks, 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+      cur_flops_ += chain_.flops_per_atom * n;
     });
   } else {
     stage("fc_A1", [&] { launch_gemm(fcA1_.fwd, ka, ka, kf, A, nlm_, A, nlm_, A1, nlm_, 0); });
@@ -536,10 +537,12 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
                            gAAA, gAAAA, 0, red_writes_ ? 1 : 0);
     });
     stage("chain_bwd", [&] {
-      const T *x0 = A, *x1 = A1, *p21 = AA1, *p22 = AA2, *g2 = gAA, *g3 = gAAA, *g4 = gAAAA;
-      void *args[] = {(void *) &x0, (void *) &x1, (void *) &p21, (void *) &p22, (void *) &g2, (void *) &g3, (void *) &g4, (void *) &gA, (void *) &chainW,
+      const T *x0 = A, *x1 = A1, *p21 = AA1, *p22 = AA2, *g2 = gAA, *g3 = gAAA, *g4 = gAAAA, *g21 = nullptr;    // P3 is inside the kernel
+      void *args[] = {(void *) &x0, (void *) &x1, (void *) &p21, (void *) &p22, (void *) &g2, (void *) &g3, (void *) &g4, (void *) &g21, (void *) &gA,
+                      (void *) &chainW,
                       (void *) &nat, (void *) &one};
       HIP_CHECK(hipModuleLaunchKernel(chain_.bwd, chain_blocks, 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+      cur_flops_ += chain_.flops_per_atom * n;
     });
   } else {
   stage("zero_grads", [&] {

@@ -4,6 +4,7 @@
 // layer-1 recompute: the layer-1 tensors of all atoms stay in device memory between P1 and P5.
 // Dense chains (FC, CG products, reduces) reuse the GRACE-1L kernels; liveness pruning after fused_2l.cpp:296-345.
 #include "engine_common.hpp"
+#include "jit_chain.hpp"
 #include "kernels_2l.hpp"
 #include "model_2l.hpp"
 
@@ -19,6 +20,13 @@ template<class T> struct Chain {
   DevFc<T> fc1, fc2, fc3;
   DevFcPairBwd<T> fc23;    // reverse of fc2 and fc3 in one pass over their shared inputs (order 4)
   DevProd p2, p3, p4;
+  // the whole chain as one generated kernel per direction (jit_chain.hpp); not ok(): the stage-by-stage kernels run
+  ChainKernels fused;
+  DevBuf fusedW, keepXX;    // fragment-ordered weights; the functions of XX the reduces collect (their adjoint rows are cleared)
+  int nkeepXX = 0;
+  bool fuse3 = true;        // P3 = XX1 x X inside the chain kernels (few outputs) or as the product kernels below (many)
+  std::string fused_note;
+  ~Chain() { fused.release(); }
   DevBuf X1, XX, XX1, XXX, XX2, XXXX, gX, gX1, gXX, gXX1, gXXX, gXX2, gXXXX;
   const T *src(int s, const T *X) const
   {
@@ -135,6 +143,45 @@ void Engine2L<T>::build_chain(Chain<T> &c, const char *tag, int nf, int KP, cons
   jit_compile_product(("prod3" + t).c_str(), h3.terms, c.nXX, nf, c.nXXX, false, KP, f32, arch_, c.p3.jit, c.p3.jit_note);
   if (order4_) jit_compile_product(("prod4" + t).c_str(), h4.terms, c.nXX, c.nXX, c.nXXXX, true, KP, f32, arch_, c.p4.jit, c.p4.jit_note);
   c.jit_all = c.p2.jit.ok() && c.p3.jit.ok() && (!order4_ || c.p4.jit.ok());
+  {
+    // the fused chain: same liveness, same pruned term lists; P3 = XX1 x X (the right operand is the chain's input)
+    ChainSpec sp;
+    sp.C = KP;
+    sp.f32 = f32;
+    sp.nf0 = nf;
+    sp.fc1 = chain_fc_spec(*fc[0], live1, nf);
+    sp.nP2 = c.nXX;
+    sp.prod2 = h2.terms;
+    sp.fc21 = chain_fc_spec(*fc[1], live2, nf);
+    sp.have22 = order4_;
+    if (order4_) sp.fc22 = chain_fc_spec(*fc[2], live3, nf);
+    sp.nP3 = c.nXXX;
+    sp.prod3 = h3.terms;
+    sp.prod3_right_x0 = true;
+    {
+      std::set<int> outs;
+      for (const ProdTerm &q : h3.terms) outs.insert(q.o);
+      c.fuse3 = sp.fuse3 = outs.size() <= 24;    // the outputs of a fused P3 are accumulated in registers
+    }
+    sp.nP4 = c.nXXXX;
+    if (order4_) sp.prod4 = h4.terms;
+    sp.keepP2 = collected(1, c.nXX);
+    sp.keepX0 = collected(0, nf);
+    for (int q = 0; q < 16; q++) sp.drow[q] = drow_[q];
+    std::vector<double> w;
+    if (jit_compile_chain(("chain" + t).c_str(), sp, arch_, c.fused, w, c.fused_note)) {
+      std::vector<T> wt(w.begin(), w.end());
+      upload_vec(c.fusedW, wt);
+      std::vector<int> keep;
+      for (int q = 0; q < c.nXX; q++)
+        if (sp.keepP2[q]) keep.push_back(q);
+      c.nkeepXX = (int) keep.size();
+      if (keep.empty()) keep.push_back(0);
+      upload_vec(c.keepXX, keep);
+    } else {
+      log_message(1, std::string("GRACE-2L: the dense chain") + tag + " runs stage by stage (" + c.fused_note + ")");
+    }
+  }
   c.fc1.build(*fc[0], live1, nf, KP, KP, KP, drow_, false, true);    // both inputs are X: one reverse launch
   // the reverse of fc2 (with the fourth-order stage: of fc2 and fc3 in one pass) WRITES the adjoint of XX: a job per function
   c.fc2.build(*fc[1], live2, nf, KP, KP, KP, drow_, true);
@@ -400,6 +447,19 @@ template<class T> void Engine2L<T>::chain_forward(Chain<T> &c, const char *tag, 
   };
   T *X1 = c.X1.template as<T>(), *XX = c.XX.template as<T>(), *XX1 = c.XX1.template as<T>(), *XXX = c.XXX.template as<T>(),
     *XX2 = c.XX2.template as<T>(), *XXXX = c.XXXX.template as<T>();
+  if (c.fused.ok()) {
+    // X -> X1 -> XX -> XX1 / XX2 -> XXX / XXXX in one kernel; XX is written for the functions the reduces collect only
+    stage(tagged(tag, "chain_fwd").c_str(), [&] {
+      const T *w = c.fusedW.template as<T>();
+      void *args[] = {(void *) &X, (void *) &X1, (void *) &XX, (void *) &XX1, (void *) &XX2, (void *) &XXX, (void *) &XXXX, (void *) &w, (void *) &nat,
+                      (void *) &one};
+      const unsigned blocks = (unsigned) ((n + c.fused.atoms_per_block - 1) / c.fused.atoms_per_block);
+      HIP_CHECK(hipModuleLaunchKernel(c.fused.fwd, blocks, 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+      cur_flops_ += c.fused.flops_per_atom * n;
+    });
+    if (!c.fuse3) prod(tagged(tag, "prod_3"), c.p3, XX1, X, XXX, c.nXX, c.nf);
+    return;
+  }
   stage(tagged(tag, "fc_1").c_str(), [&] { launch_gemm<T>(c.fc1.fwd, c.kb, c.kb, c.kb, X, c.nf, X, c.nf, X1, c.nf, 0, cur_tiles_, cur_ntiles_); });
   prod(tagged(tag, "prod_2"), c.p2, X1, X1, XX, c.nf, c.nf);
   stage(tagged(tag, "fc_2").c_str(), [&] { launch_gemm<T>(c.fc2.fwd, c.kb, c.kb, c.kb, XX, c.nXX, X, c.nf, XX1, c.nXX, 0, cur_tiles_, cur_ntiles_); });
@@ -413,6 +473,27 @@ template<class T> void Engine2L<T>::chain_forward(Chain<T> &c, const char *tag, 
 template<class T> void Engine2L<T>::chain_zero(Chain<T> &c, const char *tag)
 {
   const size_t nc = cap_, KP = c.kb * 16;
+  if (c.fused.ok()) {
+    // the reduces add their adjoints to gX, gXXX, gXXXX and to the collected rows of gXX; the chain kernel reads those rows
+    // only and writes gX
+    c.gX.ensure(nc * c.nf * KP * sizeof(T));
+    c.gXX.ensure(nc * c.nXX * KP * sizeof(T));
+    c.gXXX.ensure(nc * c.nXXX * KP * sizeof(T));
+    if (c.order4) c.gXXXX.ensure(nc * std::max(c.nXXXX, 1) * KP * sizeof(T));
+    if (!c.fuse3) c.gXX1.ensure(nc * c.nXX * KP * sizeof(T));
+    const size_t na = (size_t) cn_;
+    stage(tagged(tag, "zero_grads").c_str(), [&] {
+      HIP_CHECK(hipMemsetAsync(c.gX.p, 0, na * c.nf * KP * sizeof(T), stream_));
+      if (!c.fuse3 && !c.jit_all) HIP_CHECK(hipMemsetAsync(c.gXX1.p, 0, na * c.nXX * KP * sizeof(T), stream_));
+      HIP_CHECK(hipMemsetAsync(c.gXXX.p, 0, na * c.nXXX * KP * sizeof(T), stream_));
+      if (c.order4) HIP_CHECK(hipMemsetAsync(c.gXXXX.p, 0, na * std::max(c.nXXXX, 1) * KP * sizeof(T), stream_));
+      const long long total = (long long) na * c.nkeepXX * (long long) KP;
+      if (total > 0)
+        hipLaunchKernelGGL(k_clear_functions<T>, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, stream_, c.gXX.template as<T>(), c.nXX, (int) KP,
+                           c.keepXX.template as<int>(), c.nkeepXX, total);
+    });
+    return;
+  }
   c.gX.ensure(nc * c.nf * KP * sizeof(T));
   c.gX1.ensure(nc * c.nf * KP * sizeof(T));
   c.gXX.ensure(nc * c.nXX * KP * sizeof(T));
@@ -472,6 +553,19 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
   const T *X1 = c.X1.template as<T>(), *XX1 = c.XX1.template as<T>(), *XX2 = c.XX2.template as<T>();
   T *gX = c.gX.template as<T>(), *gX1 = c.gX1.template as<T>(), *gXX = c.gXX.template as<T>(), *gXX1 = c.gXX1.template as<T>(),
     *gXXX = c.gXXX.template as<T>(), *gXX2 = c.gXX2.template as<T>(), *gXXXX = c.gXXXX.template as<T>();
+  if (c.fused.ok()) {
+    reduces_x_xx();    // the adjoints the reduces leave on X and on the collected functions of XX come first
+    if (!c.fuse3) prod_bwd(tagged(tag, "prod_3_bwd"), c.p3, XX1, X, gXXX, gXX1, gX, c.nXX, c.nf, 0, 1);
+    stage(tagged(tag, "chain_bwd").c_str(), [&] {
+      const T *w = c.fusedW.template as<T>(), *g2 = gXX, *g3 = gXXX, *g4 = gXXXX, *g21 = gXX1;
+      void *args[] = {(void *) &X, (void *) &X1, (void *) &XX1, (void *) &XX2, (void *) &g2, (void *) &g3, (void *) &g4, (void *) &g21, (void *) &gX,
+                      (void *) &w, (void *) &nat, (void *) &one};
+      const unsigned blocks = (unsigned) ((n + c.fused.atoms_per_block - 1) / c.fused.atoms_per_block);
+      HIP_CHECK(hipModuleLaunchKernel(c.fused.bwd, blocks, 1, 1, 256, 1, 1, 0, stream_, args, nullptr));
+      cur_flops_ += c.fused.flops_per_atom * n;
+    });
+    return;
+  }
   if (c.order4) prod_bwd(tagged(tag, "prod_4_bwd"), c.p4, XX2, XX2, gXXXX, gXX2, gXX2, c.nXX, c.nXX, 0, 0);
   prod_bwd(tagged(tag, "prod_3_bwd"), c.p3, XX1, X, gXXX, gXX1, gX, c.nXX, c.nf, 0, 1);
   if (c.order4) {
@@ -551,7 +645,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   chunk_used_ = nchunks > 1 ? cs : 0;
   std::vector<long long> ebound;
   size_t ecap = ecap_all;
-  cap_ = (size_t) cs;
+  cap_ = (size_t) round_up(cs, 16);    // the generated chain kernels run whole blocks of atoms: rows up to the end of the last block
   if (nchunks > 1) {
     layout_chunks(cs);
     ebound = chunk_edge_bounds(cs);

@@ -63,6 +63,10 @@ struct ChainSpec {
   int nP3 = 0;
   std::vector<ProdTerm> prod3;
   bool prod3_right_x0 = false;
+  // P3 inside the kernels (its outputs are accumulated in registers: for the few scalar outputs of a readout chain) or left to
+  // the product kernels of the caller (many outputs): the forward kernel then only writes P21, the reverse kernel reads the
+  // adjoint of P21 from gP21, and the adjoint of X0 that the reverse of P3 leaves in gX0 is added to, for every function
+  bool fuse3 = true;
   int nP4 = 0;
   std::vector<ProdTerm> prod4;
   std::vector<char> keepP2;     // P2 functions read outside the chain (reduce, UQ): written forward, adjoint read in the reverse
@@ -75,12 +79,14 @@ struct ChainCode {
   std::vector<double> weights;    // fragment-ordered weight units of both kernels
   std::string why;
   int atoms_per_block = 0;
+  double flops_per_atom = 0.0;    // of the FC layers of one direction (live functions, padded widths; 2 per multiply-add)
 };
 
 struct ChainKernels {
   hipModule_t mod = nullptr;
   hipFunction_t fwd = nullptr, bwd = nullptr;
   int atoms_per_block = 0;
+  double flops_per_atom = 0.0;
   bool ok() const { return mod != nullptr; }
   void release()
   {
@@ -186,6 +192,7 @@ inline bool generate_chain(const ChainSpec &sp, ChainCode &out)
   std::map<int, std::vector<const ProdTerm *>> p2_by_o, p3_by_o, p3_by_l, p4_by_o, p4_by_l, p4_by_r;
   for (const auto &t : sp.prod2) {
     if (t.o < 0 || t.o >= nP2 || t.l < 0 || t.l >= nf0 || t.r < 0 || t.r >= nf0) { out.why = "prod2 term out of range"; return false; }
+    if (!sp.fc1.live[t.l] || !sp.fc1.live[t.r]) { out.why = "prod2 reads a function fc1 does not compute"; return false; }
     p2_by_o[t.o].push_back(&t);
   }
   for (const auto &t : sp.prod3) {
@@ -266,8 +273,8 @@ inline bool generate_chain(const ChainSpec &sp, ChainCode &out)
   // ---- paths of FC1
   std::vector<Fc1Path> f1;
   for (int f = 0; f < nf0; f++) {
-    if (!sp.fc1.live[f]) { out.why = "fc1 leaves a function out"; return false; }
-    const bool fresh = f1.empty() || f1.back().M >= maxM || sp.fc1.tile_l[f] != f1.back().tl || sp.fc1.tile_r[f] != f1.back().tr ||
+    if (!sp.fc1.live[f]) continue;    // a function no product reads: not computed, its adjoint is zero
+    const bool fresh = f1.empty() || f1.back().f0 + f1.back().M != f || f1.back().M >= maxM || sp.fc1.tile_l[f] != f1.back().tl || sp.fc1.tile_r[f] != f1.back().tr ||
                        sp.fc1.from[f] != f1.back().r0 + f1.back().M;
     if (fresh) {
       Fc1Path p;
@@ -527,10 +534,9 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
   s << "  X0 += at * " << nf0 << " * C + n; X1 += at * " << nf0 << " * C + n; P2 += at * " << nP2 << " * C + n; P21 += at * " << nP2
     << " * C + n; P22 += at * " << nP2 << " * C + n; P3 += at * " << std::max(nP3, 1) << " * C + n; P4 += at * " << std::max(nP4, 1) << " * C + n;\n";
   for (int f = 0; f < nf0; f++) s << "  L0[" << f * NA * S << " + col] = X0[" << f << " * C];\n";
-  if (sp.prod3_right_x0)
-    for (int f = 0; f < nf0; f++) s << "  const T x0_" << f << " = L0[" << f * NA * S << " + col];\n";
   for (int f = 0; f < nf0; f++) s << "  T " << x1(f) << ";\n";
-  for (int o = 0; o < nP3; o++) s << "  T p3_" << o << " = (T) 0;\n";
+  if (sp.fuse3)
+    for (int o = 0; o < nP3; o++) s << "  T p3_" << o << " = (T) 0;\n";
   // the steps of the forward kernel: FC1 paths, then the paths of P2 with an FC phase, group by group
   steps.clear();
   step = 0;
@@ -595,8 +601,10 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
           if (live21[f]) {
             s << "      { const T v = (T) " << lit(sp.fc21.nof[f], f32) << " * LY1[" << i * NA * S << " + col]; ST(P21[" << f << " * C], v);";
             const auto it = p3_by_l.find(f);
-            if (it != p3_by_l.end())
-              for (const ProdTerm *t : it->second) s << " p3_" << t->o << " += (T) " << lit(t->c, f32) << " * v * " << xr(t->r) << ";";
+            if (sp.fuse3 && it != p3_by_l.end())
+              for (const ProdTerm *t : it->second)
+                s << " p3_" << t->o << " += (T) " << lit(t->c, f32) << " * v * "
+                  << (sp.prod3_right_x0 ? "L0[" + std::to_string(t->r * NA * S) + " + col]" : x1(t->r)) << ";";    // X0 is resident in LDS
             s << " }\n";
           }
           if (live22[f]) {
@@ -621,14 +629,16 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
     s << "  }\n";
   }
   s << "  {\n";
-  for (int o = 0; o < nP3; o++) s << "    P3[" << o << " * C] = p3_" << o << ";\n";
+  if (sp.fuse3)
+    for (int o = 0; o < nP3; o++) s << "    P3[" << o << " * C] = p3_" << o << ";\n";
   for (int o = 0; o < nP4; o++)
     if (!p4_by_o.count(o)) s << "    P4[" << o << " * C] = (T) 0;\n";
   s << "  }\n}\n\n";
 
   // =========================================================== reverse
   s << "extern \"C\" __global__ __launch_bounds__(256) void chain_bwd(const T *__restrict__ X0, const T *__restrict__ X1, const T *__restrict__ P21, "
-       "const T *__restrict__ P22, const T *__restrict__ gP2, const T *__restrict__ gP3, const T *__restrict__ gP4, T *__restrict__ gX0, "
+       "const T *__restrict__ P22, const T *__restrict__ gP2, const T *__restrict__ gP3, const T *__restrict__ gP4, const T *__restrict__ gP21, "
+       "T *__restrict__ gX0, "
        "const T *__restrict__ W, int natoms, int one)\n{\n";
   {
     std::ostringstream d;
@@ -637,23 +647,30 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
   }
   s << "  X0 += at * " << nf0 << " * C + n; X1 += at * " << nf0 << " * C + n; P21 += at * " << nP2 << " * C + n; P22 += at * " << nP2
     << " * C + n; gP2 += at * " << nP2 << " * C + n; gP3 += at * " << std::max(nP3, 1) << " * C + n; gP4 += at * " << std::max(nP4, 1)
-    << " * C + n; gX0 += at * " << nf0 << " * C + n;\n";
-  for (int f = 0; f < nf0; f++) s << "  LG[" << f * NA * S << " + col] = (T) 0;\n";
-  for (int f = 0; f < nf0; f++) s << "  const T " << x1(f) << " = X1[" << f << " * C];\n";
-  if (sp.prod3_right_x0)
-    for (int f = 0; f < nf0; f++) s << "  const T x0_" << f << " = X0[" << f << " * C]; T gx0_" << f << " = (T) 0;\n";
+    << " * C + n; gX0 += at * " << nf0 << " * C + n; gP21 += at * " << nP2 << " * C + n;\n";
+
+  for (int f = 0; f < nf0; f++)
+    if (sp.fc1.live[f]) s << "  const T " << x1(f) << " = X1[" << f << " * C];\n";
+  if (sp.prod3_right_x0 && sp.fuse3)
+    for (int f = 0; f < nf0; f++) s << "  const T x0_" << f << " = X0[" << f << " * C];\n";
   for (int f = 0; f < nf0; f++) s << "  T g1_" << f << " = (T) 0;\n";
-  for (int o = 0; o < nP3; o++) s << "  const T g3_" << o << " = gP3[" << o << " * C];\n";
+  if (sp.fuse3)
+    for (int o = 0; o < nP3; o++) s << "  const T g3_" << o << " = gP3[" << o << " * C];\n";
   auto gr = [&](int f) { return (sp.prod3_right_x0 ? "gx0_" : "g1_") + std::to_string(f); };
   // the reverse of P3 with respect to its right operand needs P21 only here: all of it up front, with every load in flight
   // at once, instead of a load per path whose latency nothing hides (one wave per SIMD)
+  // (when the right operand is X0 the sums are the initial values of the LDS rows in which the adjoint of X0 is gathered)
   s << "  {\n";
-  for (const auto &kv : p3_by_l) s << "    const T p_" << kv.first << " = P21[" << kv.first << " * C];\n";
-  for (const auto &kv : p3_by_l)
-    for (const ProdTerm *t : kv.second) s << "    " << gr(t->r) << " += (T) " << lit(t->c, f32) << " * g3_" << t->o << " * p_" << kv.first << ";\n";
+  if (sp.fuse3) {
+    if (sp.prod3_right_x0)
+      for (int f = 0; f < nf0; f++) s << "    T gx0_" << f << " = (T) 0;\n";
+    for (const auto &kv : p3_by_l) s << "    const T p_" << kv.first << " = P21[" << kv.first << " * C];\n";
+    for (const auto &kv : p3_by_l)
+      for (const ProdTerm *t : kv.second) s << "    " << gr(t->r) << " += (T) " << lit(t->c, f32) << " * g3_" << t->o << " * p_" << kv.first << ";\n";
+  }
+  for (int f = 0; f < nf0; f++)
+    s << "    LG[" << f * NA * S << " + col] = " << (sp.prod3_right_x0 && sp.fuse3 ? "gx0_" + std::to_string(f) : std::string("(T) 0")) << ";\n";
   s << "  }\n";
-  for (int f = 0; f < nP2; f++)
-    if (keep2[f] && p2_by_o.count(f)) s << "  const T gk_" << f << " = gP2[" << f << " * C];\n";
   // the P22 rows and the P4 adjoints of a group are requested one path ahead of the group (behind the column phase of the
   // last path of the group before it, whose own rows are dead by then), so that they arrive during that path's matrix phase
   for (int f = 0; f < nP2; f++)
@@ -718,7 +735,10 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
       if (!p.any) continue;
       const bool gemm = p.l21 || p.l22;
       s << "    for (int ip = 0; ip < one; ip++) {    // path " << q << ": functions " << p.f0 << " .. " << p.f0 + p.M - 1 << "\n";
-      s << "      const T *P22w = P22v + ip, *gP4w = gP4v + ip;\n";
+      s << "      const T *P22w = P22v + ip, *gP4w = gP4v + ip, *gP2w = gP2 + it + ip, *gP21w = gP21 + it + ip;\n";
+      // the adjoints that the reduces left on this path's functions: requested here, used behind the matrix phase
+      for (int i = 0; i < p.M; i++)
+        if (keep2[p.f0 + i] && p2_by_o.count(p.f0 + i)) s << "      const T gk_" << p.f0 + i << " = gP2w[" << p.f0 + i << " * C];\n";
       const StepArgs wf = gemm ? begin_step() : StepArgs();
       if (gemm) {
         for (int i = 0; i < p.M; i++) {
@@ -728,8 +748,11 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
               const auto it = p3_by_l.find(f);
               const std::vector<const ProdTerm *> none;
               const auto &ts = it == p3_by_l.end() ? none : it->second;
-              s << "      LX1[" << i * NA * S << " + col] = (T) " << lit(sp.fc21.nof[f], f32) << " * ("
-                << sum_terms(ts, [&](const ProdTerm *t) { return "g3_" + std::to_string(t->o) + " * " + xr(t->r); }) << ");\n";
+              if (sp.fuse3)
+                s << "      LX1[" << i * NA * S << " + col] = (T) " << lit(sp.fc21.nof[f], f32) << " * ("
+                  << sum_terms(ts, [&](const ProdTerm *t) { return "g3_" + std::to_string(t->o) + " * " + xr(t->r); }) << ");\n";
+              else
+                s << "      LX1[" << i * NA * S << " + col] = (T) " << lit(sp.fc21.nof[f], f32) << " * gP21w[" << f << " * C];\n";
             } else {
               s << "      LX1[" << i * NA * S << " + col] = (T) 0;\n";
             }
@@ -817,13 +840,18 @@ __device__ inline __attribute__((always_inline)) void fc_rows(const T (&wf)[2 * 
   keep0.resize(nf0, 0);
   for (int f = 0; f < nf0; f++) {
     s << "    gX0[" << f << " * C] = LG[" << f * NA * S << " + col]";
-    if (keep0[f]) s << " + gX0[" << f << " * C]";
-    if (sp.prod3_right_x0) s << " + gx0_" << f;
+    if (keep0[f] || !sp.fuse3) s << " + gX0[" << f << " * C]";
     s << ";\n";
   }
   s << "  }\n}\n";
   out.src = s.str();
   out.atoms_per_block = NA;
+  {
+    double nfun = 0.0;    // live output functions, each with a left and a right segment of C x C
+    for (int f = 0; f < nf0; f++) nfun += sp.fc1.live[f] ? 1.0 : 0.0;
+    for (int f = 0; f < nP2; f++) nfun += (live21[f] ? 1.0 : 0.0) + (live22[f] ? 1.0 : 0.0);
+    out.flops_per_atom = nfun * 2.0 * 2.0 * C * C;
+  }
   return true;
 }
 
@@ -848,6 +876,7 @@ inline bool jit_compile_chain(const char *name, const ChainSpec &sp, const std::
   k.fwd = jk.fwd;
   k.bwd = jk.bwd;
   k.atoms_per_block = code.atoms_per_block;
+  k.flops_per_atom = code.flops_per_atom;
   weights = std::move(code.weights);
   return true;
 }

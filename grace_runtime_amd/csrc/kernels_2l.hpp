@@ -18,6 +18,17 @@
 
 namespace grhip {
 
+// rows (atom, listed function) of a per-atom tensor [atom][nfun][KP] set to zero; total = atoms x listed functions x KP
+template<class T> __global__ void k_clear_functions(T *G, int nfun, int KP, const int *list, int nlist, long long total)
+{
+  const long long i = (long long) blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int n = (int) (i % KP), q = (int) ((i / KP) % nlist);
+  const long long a = i / ((long long) KP * nlist);
+  G[(a * nfun + list[q]) * KP + n] = (T) 0;
+}
+
+
 // Two unit vectors that span the plane normal to the unit vector u: e1 = a x u / |a x u| with a the coordinate axis on
 // which u has its smallest component, e2 = u x e1.  A pure function of u: the kernel that stores tangential gradients
 // and the kernel that turns their adjoints into a force compute the same pair.
