@@ -15,6 +15,9 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <sys/stat.h>
+#include <unistd.h>
+
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -382,6 +385,67 @@ inline std::string generate_blocked(const std::vector<ProdTerm> &terms, const st
   return s.str();
 }
 
+// ---- code objects on disk
+inline std::string cache_dir()
+{
+  const char *e = std::getenv("GRACE_HIP_CACHE");
+  if (e && e[0] == '0' && e[1] == 0) return "";
+  if (e && e[0]) return e;
+  const char *x = std::getenv("XDG_CACHE_HOME");
+  if (x && x[0]) return std::string(x) + "/grace_hip";
+  const char *h = std::getenv("HOME");
+  if (h && h[0]) return std::string(h) + "/.cache/grace_hip";
+  return "";
+}
+// file of the code object of `key` (architecture, options and source): two independent 64-bit FNV-1a digests of the key
+// and of the compiler's version in its name; "" when there is no cache directory
+inline std::string cache_file(const std::string &key)
+{
+  const std::string dir = cache_dir();
+  if (dir.empty()) return "";
+  int major = 0, minor = 0;
+  (void) hiprtcVersion(&major, &minor);
+  const std::string full = "hiprtc " + std::to_string(major) + "." + std::to_string(minor) + "\n" + key;
+  unsigned long long h1 = 1469598103934665603ULL, h2 = 0x9E3779B97F4A7C15ULL;
+  for (unsigned char ch : full) {
+    h1 = (h1 ^ ch) * 1099511628211ULL;
+    h2 = (h2 ^ (ch + 0x5bULL)) * 0x100000001B3ULL + (h2 >> 29);
+  }
+  char name[64];
+  std::snprintf(name, sizeof name, "%016llx%016llx_%zu.co", h1, h2, full.size());
+  return dir + "/" + name;
+}
+inline bool read_file(const std::string &path, std::vector<char> &out)
+{
+  FILE *f = std::fopen(path.c_str(), "rb");
+  if (!f) return false;
+  std::fseek(f, 0, SEEK_END);
+  const long n = std::ftell(f);
+  std::fseek(f, 0, SEEK_SET);
+  bool ok = n > 0;
+  if (ok) {
+    out.resize((size_t) n);
+    ok = std::fread(out.data(), 1, (size_t) n, f) == (size_t) n;
+  }
+  std::fclose(f);
+  return ok;
+}
+// written under a temporary name and renamed: a reader never sees half a file, two writers of the same key write the same bytes
+inline void write_file_atomically(const std::string &path, const std::vector<char> &data)
+{
+  const size_t slash = path.rfind('/');
+  if (slash != std::string::npos) {
+    std::string dir = path.substr(0, slash), cmd;
+    for (size_t q = 1; q <= dir.size(); q++)    // the directories on the way, one by one
+      if (q == dir.size() || dir[q] == '/') (void) ::mkdir(dir.substr(0, q).c_str(), 0700);
+  }
+  const std::string tmp = path + ".tmp" + std::to_string((long long) ::getpid());
+  FILE *f = std::fopen(tmp.c_str(), "wb");
+  if (!f) return;
+  const bool ok = std::fwrite(data.data(), 1, data.size(), f) == data.size();
+  if (std::fclose(f) != 0 || !ok || std::rename(tmp.c_str(), path.c_str()) != 0) (void) std::remove(tmp.c_str());
+}
+
 }    // namespace jit_detail
 
 // Compiles the two kernels of a generated source for the current device.  Returns false (with the reason in `why`)
@@ -417,6 +481,19 @@ inline bool jit_compile_source(const char *name, const std::string &src, bool f3
     auto it = cache.find(key);
     if (it != cache.end()) obj = it->second;
   }
+  // and across processes: a directory of code objects keyed by a digest of (architecture, compiler version, options, source);
+  // the reference ships its product tables compiled (libgrace/include/grace/kk/cg_tables.h), here the second process that
+  // loads a model finds its kernels on disk.  GRACE_HIP_CACHE=<dir> names the directory (default ~/.cache/grace_hip),
+  // GRACE_HIP_CACHE=0 switches the disk cache off.
+  const std::string disk = jit_detail::cache_file(key);
+  if (!obj && !disk.empty()) {
+    std::vector<char> code;
+    if (jit_detail::read_file(disk, code) && code.size() > 64) {
+      obj = std::make_shared<const std::vector<char>>(std::move(code));
+      std::lock_guard<std::mutex> lk(cache_mu);
+      cache[key] = obj;
+    }
+  }
   if (!obj) {
     hiprtcProgram prog;
     if (hiprtcCreateProgram(&prog, src.c_str(), name, 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
@@ -443,6 +520,7 @@ inline bool jit_compile_source(const char *name, const std::string &src, bool f3
     hiprtcGetCode(prog, code.data());
     hiprtcDestroyProgram(&prog);
     obj = std::make_shared<const std::vector<char>>(std::move(code));
+    if (!disk.empty()) jit_detail::write_file_atomically(disk, *obj);
     std::lock_guard<std::mutex> lk(cache_mu);
     cache[key] = obj;
   }

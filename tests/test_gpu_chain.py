@@ -95,3 +95,40 @@ def test_models_outside_the_generator_keep_the_staged_chain(model_dir):
         names = _stages(eng)
         assert "chain_fwd" not in names and "fc_A1" in names
         eng.close()
+
+
+def test_compiled_kernels_are_kept_on_disk_for_the_next_process(model_dir, tmp_path):
+    """GRACE_HIP_CACHE: the first process compiles the generated kernels and leaves their code objects in the directory, the
+    second one loads them (no compiler run: engine creation in a fraction of the time) and computes the same numbers"""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    path = cases.model_file(model_dir, "ch20")
+    code = (
+        "import sys, time, numpy as np\n"
+        f"sys.path.insert(0, {root!r}); sys.path.insert(0, {os.path.join(root, 'tests')!r})\n"
+        "import cases\n"
+        "from grace_runtime_amd import kk\n"
+        "t = time.perf_counter()\n"
+        f"eng = kk.Engine(kk.Model({path!r}), ['Mo', 'W'], 64)\n"
+        "dt = time.perf_counter() - t\n"
+        "pos, cell, pbc, types = cases.structure_alloy54()\n"
+        "perm, offset, j, image, shifts = kk.neighbor_search(pos, cell, pbc, 5.0)\n"
+        "out = eng.compute(types[perm], offset, j, positions=pos[perm], image=image, shifts=shifts)\n"
+        "print(dt, repr(out['energy']), repr(float(np.abs(out['forces']).sum())))\n")
+    env = dict(os.environ, GRACE_HIP_CACHE=str(tmp_path / "cache"))
+    runs = []
+    for _ in range(2):
+        res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
+        assert res.returncode == 0, res.stderr
+        runs.append(res.stdout.strip().split("\n")[-1].split())
+    files = os.listdir(tmp_path / "cache")
+    assert len(files) >= 3 and all(f.endswith(".co") for f in files)          # three products and the chain
+    assert float(runs[1][0]) < 0.5 * float(runs[0][0])
+    assert abs(float(runs[0][1]) - float(runs[1][1])) < 1e-9 * abs(float(runs[0][1]))
+    assert abs(float(runs[0][2]) - float(runs[1][2])) < 1e-9 * abs(float(runs[0][2]))
+    # switched off: nothing is written
+    env0 = dict(os.environ, GRACE_HIP_CACHE="0", HOME=str(tmp_path / "home"))
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env0, timeout=300)
+    assert res.returncode == 0, res.stderr
+    assert not os.path.exists(tmp_path / "home" / ".cache" / "grace_hip")
