@@ -1239,7 +1239,7 @@ class EngineBase : public Engine, protected BufRegistry {
   {
     for (int q = 0; q < 16; q++) ba.drow[q] = drow_[q];
     const int kb = ba.C / 16;
-    const size_t lds = ((size_t) ba.nlm * (ba.C + 2) + (size_t) 4 * 16 * ba.nlm * 4) * sizeof(T);
+    const size_t lds = ((size_t) ba.nlm * (ba.C + 2) + (size_t) 4 * 16 * ba.nlm * 3) * sizeof(T);
     if (kb != 1 && kb != 2 && kb != 4) throw Error("bond backward: channel width must be 16, 32 or 64");
 #define GR_BB(KB, NL) hipLaunchKernelGGL((k_bond_bwd<T, KB, NL>), dim3(n), dim3(256), lds, stream_, ba)
 #define GR_BB_NL(NL) case NL: if (kb == 1) GR_BB(1, NL); else if (kb == 2) GR_BB(2, NL); else GR_BB(4, NL); break

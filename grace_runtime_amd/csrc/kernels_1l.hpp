@@ -1458,6 +1458,22 @@ __global__ __launch_bounds__(256) void k_uq(UqDev<T> U, const int *mu, int natom
   }
 }
 
+// Two unit vectors that span the plane normal to the unit vector u: e1 = a x u / |a x u| with a the coordinate axis on
+// which u has its smallest component, e2 = u x e1.  A pure function of u: the kernel that stores tangential gradients
+// and the kernel that turns their adjoints into a force compute the same pair.
+__device__ inline void tangent_basis(const double *u, double *e1, double *e2)
+{
+  const double ax = fabs(u[0]), ay = fabs(u[1]), az = fabs(u[2]);
+  double a[3] = {0.0, 0.0, 0.0};
+  if (ax <= ay && ax <= az) a[0] = 1.0;
+  else if (ay <= az) a[1] = 1.0;
+  else a[2] = 1.0;
+  const double c0 = a[1] * u[2] - a[2] * u[1], c1 = a[2] * u[0] - a[0] * u[2], c2 = a[0] * u[1] - a[1] * u[0];
+  const double inv = 1.0 / sqrt(c0 * c0 + c1 * c1 + c2 * c2);
+  e1[0] = c0 * inv; e1[1] = c1 * inv; e1[2] = c2 * inv;
+  e2[0] = u[1] * e1[2] - u[2] * e1[1]; e2[1] = u[2] * e1[0] - u[0] * e1[2]; e2[2] = u[0] * e1[1] - u[1] * e1[0];
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // bond backward: forces and virial
 // ---------------------------------------------------------------------------------------------------------------
@@ -1488,9 +1504,12 @@ template<class T> struct BondBwdArgs {
 // the harmonics of bond c and holds its geometry in registers -- finishes the bond:
 //   g_d = sum_lm G[b][lm][d] P[lm][b],  dE/dx = sum_lm Y[b][lm] Q[lm][b],
 //   fv = dE/dx / rc rhat + (g - (g . rhat) rhat) / r;  f_i += fv, f_j -= fv, virial += (-r rhat) (x) fv
-// (fused_cpu.h:836-860,1027-1050; fused_1l.cpp:46-51 of the reference).  gA of the atom sits in LDS as [lm][C + 2]
+// (fused_cpu.h:836-860,1027-1050; fused_1l.cpp:46-51 of the reference).  Only the part of g normal to the bond enters,
+// g - (g . rhat) rhat = (g . e1) e1 + (g . e2) e2 for an orthonormal pair e1, e2 normal to the bond (tangent_basis), so
+// the harmonics' gradients are kept as their two components along e1 and e2: two sums per bond instead of three, and a
+// third less LDS per block (three blocks per CU instead of two).  gA of the atom sits in LDS as [lm][C + 2]
 // (the pad spreads the rows over the banks); the radial rows of l + 1 are requested before the products of l.
-// KB = channels / 16, NL = lmax + 1.  dynamic LDS: nlm (C + 2) + 4 waves x 16 bonds x 4 nlm values.
+// KB = channels / 16, NL = lmax + 1.  dynamic LDS: nlm (C + 2) + 4 waves x 16 bonds x 3 nlm values.
 template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_bwd(BondBwdArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
@@ -1498,7 +1517,7 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *gAl = reinterpret_cast<T *>(smem_raw);                          // [NLM][CS]
   T *Ysh = gAl + NLM * CS;                                           // [4 waves][16][NLM]
-  T *Gsh = Ysh + 4 * 16 * NLM;                                       // [4 waves][16][NLM][3]
+  T *Gsh = Ysh + 4 * 16 * NLM;                                       // [4 waves][16][2][NLM]: gradient . e1, gradient . e2
   __shared__ double red[4][9];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int c = lane & 15, g = lane >> 4;
@@ -1509,7 +1528,7 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
     for (int q = t; q < NLM * C; q += 256) gAl[(q / C) * CS + q % C] = gAi[q];
   }
   __syncthreads();
-  T *Yw = Ysh + wave * 16 * NLM, *Gw = Gsh + wave * 16 * 3 * NLM;
+  T *Yw = Ysh + wave * 16 * NLM, *Gw = Gsh + wave * 16 * 2 * NLM;
   int mrow[4];
 #pragma unroll
   for (int v = 0; v < 4; v++) mrow[v] = a.drow[4 * g + v];
@@ -1526,18 +1545,21 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
     for (int s = 0; s < KS; s++) { x[0][s] = rp[s]; dx[0][s] = dp[s]; }
     // geometry of bond `lane` (lanes below nb), kept for the end of the tile
     double u0 = 0, u1 = 0, u2 = 1, br = 1, brc = 1;
+    double e1[3] = {1, 0, 0}, e2[3] = {0, 1, 0};
     int jj = 0;
     if (lane < nb) {
       const long long e = eb + lane;
       u0 = a.rh[3 * e]; u1 = a.rh[3 * e + 1]; u2 = a.rh[3 * e + 2];
       br = a.r[e]; brc = a.rc[e]; jj = a.ej[e];
-      sh_eval<true, T, NL - 1>(a.sh, u0, u1, u2, Yw + lane * NLM, Gw + lane * 3 * NLM);
+      const double u[3] = {u0, u1, u2};
+      tangent_basis(u, e1, e2);
+      sh_eval<true, T, NL - 1>(a.sh, u0, u1, u2, Yw + lane * NLM, Gw + lane * 2 * NLM, e1, e2, Gw + lane * 2 * NLM + NLM);
     }
     // LDS writes of this wave visible to its other lanes (the Y / G region is private to the wave)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    double px = 0, p0 = 0, p1 = 0, p2 = 0;
+    double px = 0, p1 = 0, p2 = 0;
 #pragma unroll
     for (int l = 0; l < NL; l++) {
       const int cur = l & 1, nxt = cur ^ 1;
@@ -1559,22 +1581,20 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
         for (int v = 0; v < 4; v++) {
           if (mrow[v] < 2 * l + 1) {
             const int lm = l * l + mrow[v];
-            const T *G = Gw + (c * NLM + lm) * 3;
+            const T *G = Gw + c * 2 * NLM + lm;
             px += (double) (Yw[c * NLM + lm] * aQ[v]);
-            p0 += (double) (G[0] * aP[v]);
-            p1 += (double) (G[1] * aP[v]);
-            p2 += (double) (G[2] * aP[v]);
+            p1 += (double) (G[0] * aP[v]);
+            p2 += (double) (G[NLM] * aP[v]);
           }
         }
       }
     }
     // sum over the four lane groups (the rows m of a bond are spread over them)
-    px += __shfl_xor(px, 16, 64); p0 += __shfl_xor(p0, 16, 64); p1 += __shfl_xor(p1, 16, 64); p2 += __shfl_xor(p2, 16, 64);
-    px += __shfl_xor(px, 32, 64); p0 += __shfl_xor(p0, 32, 64); p1 += __shfl_xor(p1, 32, 64); p2 += __shfl_xor(p2, 32, 64);
+    px += __shfl_xor(px, 16, 64); p1 += __shfl_xor(p1, 16, 64); p2 += __shfl_xor(p2, 16, 64);
+    px += __shfl_xor(px, 32, 64); p1 += __shfl_xor(p1, 32, 64); p2 += __shfl_xor(p2, 32, 64);
     if (lane < nb) {
-      const double dEdr = px / brc;
-      const double gr = p0 * u0 + p1 * u1 + p2 * u2;
-      const double fv[3] = {dEdr * u0 + (p0 - gr * u0) / br, dEdr * u1 + (p1 - gr * u1) / br, dEdr * u2 + (p2 - gr * u2) / br};
+      const double dEdr = px / brc, t1 = p1 / br, t2 = p2 / br;
+      const double fv[3] = {dEdr * u0 + t1 * e1[0] + t2 * e2[0], dEdr * u1 + t1 * e1[1] + t2 * e2[1], dEdr * u2 + t1 * e1[2] + t2 * e2[2]};
       for (int d = 0; d < 3; d++) {
         fi[d] += fv[d];
         if (a.fedge) a.fedge[3 * (eb + lane) + d] = (a.ordered_add ? a.fedge[3 * (eb + lane) + d] : 0.0) + fv[d];

@@ -29,22 +29,6 @@ template<class T> __global__ void k_clear_functions(T *G, int nfun, int KP, cons
 }
 
 
-// Two unit vectors that span the plane normal to the unit vector u: e1 = a x u / |a x u| with a the coordinate axis on
-// which u has its smallest component, e2 = u x e1.  A pure function of u: the kernel that stores tangential gradients
-// and the kernel that turns their adjoints into a force compute the same pair.
-__device__ inline void tangent_basis(const double *u, double *e1, double *e2)
-{
-  const double ax = fabs(u[0]), ay = fabs(u[1]), az = fabs(u[2]);
-  double a[3] = {0.0, 0.0, 0.0};
-  if (ax <= ay && ax <= az) a[0] = 1.0;
-  else if (ay <= az) a[1] = 1.0;
-  else a[2] = 1.0;
-  const double c0 = a[1] * u[2] - a[2] * u[1], c1 = a[2] * u[0] - a[0] * u[2], c2 = a[0] * u[1] - a[1] * u[0];
-  const double inv = 1.0 / sqrt(c0 * c0 + c1 * c1 + c2 * c2);
-  e1[0] = c0 * inv; e1[1] = c1 * inv; e1[2] = c2 * inv;
-  e2[0] = u[1] * e1[2] - u[2] * e1[1]; e2[1] = u[2] * e1[0] - u[0] * e1[2]; e2[2] = u[0] * e1[1] - u[1] * e1[0];
-}
-
 // One thread per edge: YG[e] = (Y[nlm], D1[nlm], D2[nlm]) (row width W = 3 nlm), or Y[nlm] alone (W = nlm, no
 // gradients).  D1 = G . e1, D2 = G . e2 are the components of the gradient G of the polynomial extension of Y along the
 // tangent vectors of the bond (tangent_basis): the bond force only uses the part of sum_lm gY_lm G_lm normal to the bond,
