@@ -118,7 +118,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--precision", type=int, default=64, choices=[64, 32])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5"])
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config4", "config5", "sizes"])
     ap.add_argument("--reps", type=int, default=0, help="supercell repetitions (default: 16 bcc cells / 20 fcc cells per edge)")
     ap.add_argument("--atoms", type=int, default=10000, help="atoms of the amorphous cube of config4")
     ap.add_argument("--spline", type=int, default=0, help="intervals of the radial tables of the GRACE-1L / 2L engines (the reference's engines "
@@ -130,6 +130,9 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (no collectives in the path); run with --gpus 1")
+    if a.workload == "sizes":
+        print(json.dumps(run_sizes(a)))
+        return
     res = run_workload(a)
     if a.workload == "config2" and a.precision == 64 and not a.no_others and a.reps == 0 and a.spline == 0 and a.chunksize == -1:
         # the other benchmark configurations, a few steps each, in the same run (the same code path as --workload <name>)
@@ -150,6 +153,66 @@ def main():
                                "cpu_baseline": r["cpu_baseline"]}
         res["other_workloads"] = others
     print(json.dumps(res))
+
+
+def run_sizes(a):
+    """The calculator-level call (kk.System.compute: positions in, device neighbour list kept between calls, results out; the
+    reference's protocol, docs/benchmarks.md:9-20) over a range of structure sizes: the GRACE-1L model from 128 atoms to a
+    bcc 128^3 supercell, and one structure per model kind well past the benchmark size, evaluated in the chunks the engine
+    chooses from the free device memory (the reference's "largest system" column, docs/benchmarks.md:17, is the same
+    mechanism pushed to the limit of a 64 GB device; here the sizes are fixed and chosen to fit).  Prints atoms, bonds per
+    atom, ms per call, us/atom, atoms per engine pass and the device memory the library holds."""
+    import torch
+
+    from grace_runtime_amd import kk, synth, workloads
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    tmp = tempfile.mkdtemp()
+    pbc = [True, True, True]
+    out = []
+
+    def measure(label, model, species, types, pos, cell, calls):
+        t0 = time.perf_counter()
+        sysm = kk.System(model, species, skin=0.5, precision=a.precision)
+        create_s = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        r = sysm.compute(types, pos, cell, pbc)
+        first_s = time.perf_counter() - t0
+        ts = []
+        for _ in range(calls):
+            t0 = time.perf_counter()
+            r = sysm.compute(types, pos, cell, pbc)
+            ts.append(time.perf_counter() - t0)
+        n = len(pos)
+        ms = float(np.median(ts)) * 1e3
+        e = {"structure": label, "atoms": n, "edges": int(sysm.engine.edge_count()), "ms_per_call_list_kept": round(ms, 3),
+             "us_per_atom": round(ms * 1e3 / n, 5), "first_call_s_with_list_build": round(first_s, 3), "atoms_per_engine_pass": sysm.chunksize or n,
+             "device_memory_GB": round(kk.memory_in_use() / 1e9, 3), "engine_create_s": round(create_s, 2), "energy_per_atom": r["energy"] / n,
+             "net_force": float(np.abs(r["forces"].sum(0)).max())}
+        print(json.dumps(e), file=sys.stderr, flush=True)
+        out.append(e)
+        del sysm
+
+    m1 = kk.Model(workloads.write_model("config1", tmp))
+    for reps in (4, 8, 10, 16, 32, 64, 128):
+        pos, cell = synth.bcc_supercell(3.165, reps)
+        pos = synth.jitter(pos, 0.05, 2)
+        measure(f"GRACE-1L, bcc W {reps}^3", m1, ["W"], np.ones(len(pos), np.int32), pos, cell, 5 if reps <= 32 else 3)
+    m2 = kk.Model(workloads.write_model("config3", tmp))
+    pos, cell = synth.fcc_supercell(3.6, 63)
+    pos = synth.jitter(pos, 0.08, 3)
+    measure("GRACE-2L, 4-species fcc alloy 63^3", m2, ["Al", "Co", "Ni", "Ti"], np.random.default_rng(3).integers(1, 5, size=len(pos)).astype(np.int32),
+            pos, cell, 3)
+    mp = workloads.write_model("config4", tmp)
+    with np.load(mp) as z:
+        names = [x.decode() for x in z["element_names"]]
+    p0, c0, _, t89 = workloads.structure_config4(natoms=10000)
+    # the amorphous cube of configuration 4 repeated 3 x 3 x 3 (a periodic structure again) with its own jitter: 270 000 atoms
+    shifts = np.array([[i, j, k] for i in range(3) for j in range(3) for k in range(3)], float) @ c0
+    pos = (p0[None, :, :] + shifts[:, None, :]).reshape(-1, 3) + np.random.default_rng(9).normal(0.0, 0.02, (27 * len(p0), 3))
+    measure("GRACE-3L, amorphous cube of configuration 4 repeated 3x3x3", kk.Model(mp), workloads.config4_species(names),
+            np.tile(workloads.config4_types(t89), 27), pos, 3.0 * c0, 2)
+    return {"workload": "size range, calculator-level call with the neighbour list kept", "dtype": "f64" if a.precision == 64 else "f32", "entries": out}
 
 
 def run_workload(a, light=False):

@@ -78,6 +78,7 @@ template<class T> class Engine1L final : public EngineBase {
     this->template probe_mfma_both<T>();
     chunks_ = true;
     ordered_ok_ = true;
+    if (const char *e = std::getenv("GRACE_HIP_TABLE_ROWS")) tables_inside_ = !(e[0] == '1');
     build();
     scratch_dev_ = scratch_of_device(device);    // set-up: the device is current (EngineBase)
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
@@ -112,6 +113,7 @@ template<class T> class Engine1L final : public EngineBase {
   ChainKernels chain_;
   DevBuf chainW_;
   std::string chain_note_;
+  bool tables_inside_ = true;  // radial tables evaluated by the kernels that use the radial functions
   bool red_writes_ = false;    // the reverse of the rho reduce may overwrite the adjoints (every function collected at most once)
   DevReduce<T> redrho_;
   UqDev<T> uq_{};             // UQ head (models that carry a valid one)
@@ -378,8 +380,10 @@ template<class T> void Engine1L<T>::run(const RunFlags &fl)
   // rows of the per-atom tensors: the generated chain kernels run whole blocks of atoms and neither guard their loads nor
   // their stores, so the tensors hold rows up to the end of the last block
   const size_t na = (size_t) round_up(cs, 16);
-  Rz_.ensure(ecap * noutp_ * sizeof(T));
-  dRz_.ensure(ecap * noutp_ * sizeof(T));
+  if (!(rad_.has_tables() && tables_inside_)) {    // with tables evaluated inside the kernels the rows do not exist
+    Rz_.ensure(ecap * noutp_ * sizeof(T));
+    dRz_.ensure(ecap * noutp_ * sizeof(T));
+  }
   A_.ensure(na * nlm_ * CP_ * sizeof(T));
   A1_.ensure(na * nlm_ * CFP_ * sizeof(T));
   AA_.ensure(na * nAA_ * CFP_ * sizeof(T));
@@ -434,9 +438,15 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
   // the radial rows of the chunk start at row 0 of Rz_ / dRz_; the kernels index them by the bond's number in the structure
   T *Rz = moved_back(Rz_.as<T>(), e_begin * noutp_), *dRz = moved_back(dRz_.as<T>(), e_begin * noutp_);
 
-  stage("radial_mlp", [&] { launch_radial(e_begin, e_count, xr_.as<double>(), emu_.as<int>(), Rz, dRz, eoff_.as<long long>() + n_, true); });
+  // radial tables asked for: the A basis and the bond reverse evaluate them themselves, no radial row is written or read
+  // (GRACE_HIP_TABLE_ROWS=1: the rows are written by the table kernel and read back, as without tables)
+  const bool tab_inside = rad_.has_tables() && tables_inside_ && (nl_ * (CP_ / 16) <= 10 || (nl_ <= 7 && CP_ == 16));
+  RadialTable<T> tb{};
+  if (tab_inside) tb = rad_.table(stream_, ncu_, xr_.as<double>(), emu_.as<int>(), z_.as<T>());
+  else stage("radial_mlp", [&] { launch_radial(e_begin, e_count, xr_.as<double>(), emu_.as<int>(), Rz, dRz, eoff_.as<long long>() + n_, true); });
 
   ScatterArgs<T> sa{};
+  sa.tb = tb;
   sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz; sa.A = A_.as<T>();
   sa.a0 = a0; sa.C = CP_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = noutp_; sa.sh = sh_;
   stage("scatter_A", [&] { launch_scatter<T>(sa, n, lmax_); });
@@ -616,6 +626,7 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
   BondBwdArgs<T> ba{};
   ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
   ba.Rz = Rz; ba.dRz = dRz; ba.gA = gA;
+  ba.tb = tb;
   ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr(); ba.vatom = vatom_ptr();
   ba.fedge = ordered_ ? fedge_.as<double>() : nullptr; ba.fcen = ordered_ ? fcen_.as<double>() : nullptr;
   ba.a0 = a0; ba.C = CP_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = noutp_; ba.sh = sh_;

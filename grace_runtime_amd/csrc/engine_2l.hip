@@ -677,8 +677,17 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     uq_gamma_.ensure((size_t) n * sizeof(double)); uq_sigma_.ensure((size_t) n * sizeof(double)); uq_cluster_.ensure((size_t) n * sizeof(double));
   }
   // buffers of a chunk
-  Rz_.ensure(ecap * radR_.noutp * sizeof(T));
-  dRz_.ensure(ecap * radR_.noutp * sizeof(T));
+  // radial tables asked for: the A basis and the bond reverse of layer 1 evaluate them themselves, and the rows of R are
+  // neither written nor read (GRACE_HIP_TABLE_ROWS=1: rows from the table kernel, as without tables).  The pair kernels of
+  // layer 2 read the rows of R1 in either case.
+  const char *rows_env = std::getenv("GRACE_HIP_TABLE_ROWS");
+  const bool tab_inside = radR_.has_tables() && !(rows_env && rows_env[0] == '1') && nl_ * (C1P_ / 16) <= 10;
+  if (!tab_inside) {
+    Rz_.ensure(ecap * radR_.noutp * sizeof(T));
+    dRz_.ensure(ecap * radR_.noutp * sizeof(T));
+  }
+  RadialTable<T> tbR{};
+  if (tab_inside) tbR = radR_.table(stream_, ncu_, xr_.as<double>(), emu_.as<int>(), zA_.as<T>());
   A_.ensure(na * nlm_ * C1P_ * sizeof(T));
   T *A = A_.as<T>();
   if (I1_.bytes < na * nI1_ * PI1_ * sizeof(double)) {
@@ -691,8 +700,10 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   // in the structure)
   auto layer1_chain = [&] {
     T *Rz = moved_back(Rz_.as<T>(), eb * radR_.noutp), *dRz = moved_back(dRz_.as<T>(), eb * radR_.noutp);
-    stage("radial_R", [&] { radR_.launch(stream_, ncu_, zA_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), Rz, dRz, n_edges, nullptr, true); });
+    if (!tab_inside)
+      stage("radial_R", [&] { radR_.launch(stream_, ncu_, zA_.as<T>(), eb, ecnt, xr_.as<double>(), emu_.as<int>(), Rz, dRz, n_edges, nullptr, true); });
     ScatterArgs<T> sa{};
+    sa.tb = tbR;
     sa.eoff = eoff_.as<long long>(); sa.rh = rh_.as<double>(); sa.Rz = Rz; sa.A = A;
     sa.a0 = a0_; sa.C = C1P_; sa.nl = nl_; sa.nlm = nlm_; sa.noutp = radR_.noutp; sa.sh = sh_;
     stage("scatter_A", [&] { launch_scatter<T>(sa, cn_, lmax_); });
@@ -913,6 +924,7 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
     ba.eoff = eoff_.as<long long>(); ba.ej = ej_.as<int>(); ba.rh = rh_.as<double>(); ba.r = r_.as<double>(); ba.rc = rc_.as<double>();
     ba.Rz = moved_back(Rz_.as<T>(), eb * radR_.noutp); ba.dRz = moved_back(dRz_.as<T>(), eb * radR_.noutp); ba.gA = c1_.gX.template as<T>();
     ba.f = f_.as<double>(); ba.virial = scal_.as<double>() + 1; ba.sid = sid_ptr(); ba.vatom = vatom_ptr();
+    ba.tb = tbR;
     ba.a0 = a0_; ba.C = C1P_; ba.nl = nl_; ba.nlm = nlm_; ba.noutp = radR_.noutp; ba.sh = sh_;
     if (ordered_) {    // added to what the pair kernel of layer 2 stored for the same bonds and atoms
       ba.fedge = fedge_.as<double>(); ba.fcen = fcen_.as<double>(); ba.ordered_add = 1;

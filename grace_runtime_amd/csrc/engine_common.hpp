@@ -493,6 +493,33 @@ template<class T> struct DevRadial {
               const long long *n_edges, const int *emi = nullptr, bool tables = false)
   {
     if (tables && spline_n > 0 && mode == 0) {
+      ensure_tables(stream, ncu);
+      const long long bound = e_count >= 0 ? e_count : (long long) 1 << 40;
+      const unsigned grid = (unsigned) std::max<long long>(1, std::min<long long>(bound, (long long) ncu * 32));
+      hipLaunchKernelGGL((k_radial_spline<T, sizeof(T) == 4>), dim3(grid), dim3(round_up(noutp, 64)), 0, stream, n_edges, e_begin, e_count, x, emu,
+                         (const T *) tabF.template as<T>(), (const T *) tabD.template as<T>(), table_n, z, CP, noutp, Rz, dRz);
+      return;
+    }
+    launch_mlp(stream, ncu, z, e_begin, e_count, x, emu, Rz, dRz, n_edges, emi);
+  }
+  // tables requested (spline_n > 0) for a form of the MLP that has them
+  bool has_tables() const { return spline_n > 0 && mode == 0; }
+  // the tables as the kernels that evaluate them take them (built on first use and again after release_buffers)
+  RadialTable<T> table(hipStream_t stream, int ncu, const double *x, const int *emu, const T *z)
+  {
+    ensure_tables(stream, ncu);
+    RadialTable<T> t{};
+    t.F = tabF.template as<T>();
+    t.D = tabD.template as<T>();
+    t.N = table_n;
+    t.x = x;
+    t.emu = emu;
+    t.z = z;
+    return t;
+  }
+  void ensure_tables(hipStream_t stream, int ncu)
+  {
+    {
       const int N = spline_n;
       if (table_n != N || !tabF.p || (sizeof(T) == 8 && !tabD.p)) {    // the MLP at the knots x = k / N, unit species weights (again after release_buffers)
         std::vector<double> xs((size_t) N + 1);
@@ -504,28 +531,28 @@ template<class T> struct DevRadial {
           upload_vec(unit_z, std::vector<T>((size_t) CP, (T) 1));
           tabF.ensure(rows * sizeof(T));
           tabD.ensure(rows * sizeof(T));
-          launch(stream, ncu, unit_z.template as<T>(), 0, (long long) N + 1, knots.as<double>(), knot_mu.as<int>(), tabF.template as<T>(),
-                 tabD.template as<T>(), nullptr);
+          launch_mlp(stream, ncu, unit_z.template as<T>(), 0, (long long) N + 1, knots.as<double>(), knot_mu.as<int>(), tabF.template as<T>(),
+                     tabD.template as<T>(), nullptr, nullptr);
         } else {
           if (!dbl) throw Error("radial tables of an fp32 engine need the fp64 form of its radial MLP");
           upload_vec(unit_z, std::vector<double>((size_t) CP, 1.0));
           knotF.ensure(rows * sizeof(double));
           knotD.ensure(rows * sizeof(double));
           tabF.ensure((size_t) N * 4 * noutp * sizeof(T));
-          dbl->launch(stream, ncu, unit_z.as<double>(), 0, (long long) N + 1, knots.as<double>(), knot_mu.as<int>(), knotF.as<double>(),
-                      knotD.as<double>(), nullptr);
+          dbl->launch_mlp(stream, ncu, unit_z.as<double>(), 0, (long long) N + 1, knots.as<double>(), knot_mu.as<int>(), knotF.as<double>(),
+                          knotD.as<double>(), nullptr, nullptr);
           const long long tot = (long long) N * noutp;
           hipLaunchKernelGGL(k_spline_coef, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream, (const double *) knotF.as<double>(),
                              (const double *) knotD.as<double>(), N, noutp, tabF.as<float>());
         }
         table_n = N;
       }
-      const long long bound = e_count >= 0 ? e_count : (long long) 1 << 40;
-      const unsigned grid = (unsigned) std::max<long long>(1, std::min<long long>(bound, (long long) ncu * 32));
-      hipLaunchKernelGGL((k_radial_spline<T, sizeof(T) == 4>), dim3(grid), dim3(round_up(noutp, 64)), 0, stream, n_edges, e_begin, e_count, x, emu,
-                         (const T *) tabF.template as<T>(), (const T *) tabD.template as<T>(), table_n, z, CP, noutp, Rz, dRz);
-      return;
     }
+  }
+  // the radial MLP itself for every edge of the range
+  void launch_mlp(hipStream_t stream, int ncu, const T *z, long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
+                  const long long *n_edges, const int *emi)
+  {
     RadialArgs<T> ra{};
     ra.n_edges = n_edges;
     ra.e_begin = e_begin;
@@ -1219,7 +1246,11 @@ class EngineBase : public Engine, protected BufRegistry {
     const int kb = sa.C / 16;
     const size_t lds = (size_t) 4 * 16 * sa.nlm * sizeof(T);
     const dim3 grid((n + 3) / 4), block(256);
-#define GR_SCAT(NL_, KB_) hipLaunchKernelGGL((k_scatter_a_mfma<T, NL_, KB_>), grid, block, lds, stream_, sa)
+#define GR_SCAT(NL_, KB_)                                                                       \
+  do {                                                                                          \
+    if (sa.tb.F) hipLaunchKernelGGL((k_scatter_a_tab<T, NL_, KB_>), grid, block, lds, stream_, sa); \
+    else hipLaunchKernelGGL((k_scatter_a_mfma<T, NL_, KB_>), grid, block, lds, stream_, sa);    \
+  } while (0)
     const int key = sa.nl * 10 + kb;    // register tiles of the kernel: nl * kb <= 10
     if (key == 11) GR_SCAT(1, 1); else if (key == 12) GR_SCAT(1, 2); else if (key == 14) GR_SCAT(1, 4);
     else if (key == 21) GR_SCAT(2, 1); else if (key == 22) GR_SCAT(2, 2); else if (key == 24) GR_SCAT(2, 4);
@@ -1229,6 +1260,7 @@ class EngineBase : public Engine, protected BufRegistry {
     else if (key == 61) GR_SCAT(6, 1); else if (key == 71) GR_SCAT(7, 1);
 #undef GR_SCAT
     else {
+      if (sa.tb.F) throw Error("A basis from radial tables: the channel widths of this model have no matrix-core kernel");
       const int sthreads = round_up(sa.nl * sa.C, 64);
       if (lmax <= 4) hipLaunchKernelGGL((k_scatter_a<T, 9>), dim3(n), dim3(sthreads), 0, stream_, sa);
       else hipLaunchKernelGGL((k_scatter_a<T, 13>), dim3(n), dim3(sthreads), 0, stream_, sa);
@@ -1241,7 +1273,11 @@ class EngineBase : public Engine, protected BufRegistry {
     const int kb = ba.C / 16;
     const size_t lds = ((size_t) ba.nlm * (ba.C + 2) + (size_t) 4 * 16 * ba.nlm * 3) * sizeof(T);
     if (kb != 1 && kb != 2 && kb != 4) throw Error("bond backward: channel width must be 16, 32 or 64");
-#define GR_BB(KB, NL) hipLaunchKernelGGL((k_bond_bwd<T, KB, NL>), dim3(n), dim3(256), lds, stream_, ba)
+#define GR_BB(KB, NL)                                                                                  \
+  do {                                                                                                 \
+    if (ba.tb.F) hipLaunchKernelGGL((k_bond_bwd<T, KB, NL, true>), dim3(n), dim3(256), lds, stream_, ba); \
+    else hipLaunchKernelGGL((k_bond_bwd<T, KB, NL, false>), dim3(n), dim3(256), lds, stream_, ba);     \
+  } while (0)
 #define GR_BB_NL(NL) case NL: if (kb == 1) GR_BB(1, NL); else if (kb == 2) GR_BB(2, NL); else GR_BB(4, NL); break
     switch (ba.nl) {
       GR_BB_NL(1); GR_BB_NL(2); GR_BB_NL(3); GR_BB_NL(4); GR_BB_NL(5); GR_BB_NL(6); GR_BB_NL(7);

@@ -679,10 +679,56 @@ template<class T, int HB, int ACT, int MODE, bool W2L> __global__ __launch_bound
 // ---------------------------------------------------------------------------------------------------------------
 // A basis
 // ---------------------------------------------------------------------------------------------------------------
+// The radial tables for kernels that evaluate them themselves instead of reading rows another kernel wrote (the bond
+// loops of the reference's fused GPU engines read their table in the same place, libgrace/include/grace/kk/
+// grace_1l_fused_kk_impl.h:405-440; CPU: spline_eval, libgrace/include/grace/fused_cpu.h:1052-1074).  F == nullptr: no
+// tables, the kernel reads rows.  Layouts and formulas are those of k_radial_spline.
+template<class T> struct RadialTable {
+  const T *F, *D;     // fp64: value and d/dx at the knots, [N + 1][noutp] each; fp32: F = coefficients [N][4][noutp], D unused
+  int N;              // intervals over x = r / rc in [0, 1]
+  const double *x;    // [E] r / rc
+  const int *emu;     // [E] neighbour element
+  const T *z;         // [nel][C] species weights (all ones where the rows carry none)
+};
+// interval and offset of x in a table of N intervals
+__device__ inline int table_interval(double x, int N, double &t)
+{
+  const double sx = x * N;
+  int k = (int) sx;
+  k = k > N - 1 ? N - 1 : (k < 0 ? 0 : k);
+  t = sx - k;
+  return k;
+}
+// the four table entries of column col in interval k (requested here, used by table_value)
+template<class T> __device__ inline void table_request(const RadialTable<T> &tb, int k, int col, int noutp, T (&raw)[4])
+{
+  if constexpr (sizeof(T) == 4) {
+    const T *c = tb.F + (long long) k * 4 * noutp + col;
+    raw[0] = c[0]; raw[1] = c[noutp]; raw[2] = c[2 * noutp]; raw[3] = c[3 * noutp];
+  } else {
+    const T *f = tb.F + (long long) k * noutp + col, *d = tb.D + (long long) k * noutp + col;
+    raw[0] = f[0]; raw[1] = d[0]; raw[2] = f[noutp]; raw[3] = d[noutp];    // f0, f0', f1, f1'
+  }
+}
+// R(t) and, with DERIV, dR/dx of the cubic of the interval
+template<class T, bool DERIV> __device__ inline void table_value(const T (&raw)[4], T t, T h, T fN, T &R, T &dR)
+{
+  T a0 = raw[0], a1 = raw[1], a2 = raw[2], a3 = raw[3];
+  if constexpr (sizeof(T) == 8) {
+    const T f1 = a2, d1 = a3 * h;
+    a1 *= h;
+    a2 = (T) -3 * a0 - (T) 2 * a1 + (T) 3 * f1 - d1;
+    a3 = (T) 2 * a0 + a1 - (T) 2 * f1 + d1;
+  }
+  R = a0 + t * (a1 + t * (a2 + t * a3));
+  if (DERIV) dR = (a1 + t * ((T) 2 * a2 + t * (T) 3 * a3)) * fN;
+}
+
 template<class T> struct ScatterArgs {
   const long long *eoff;      // [n + 1]
   const double *rh;           // [E][3]
   const T *Rz;                // [E][noutp]
+  RadialTable<T> tb;          // tb.F set: the radial functions come from the tables, Rz is not read
   T *A;                       // [chunk atoms][nlm][C]
   int a0, natoms;             // first atom of the chunk, atoms in it
   int C, nl, nlm, noutp;
@@ -824,6 +870,109 @@ template<class T, int NL, int KB> __global__ __launch_bounds__(256) __attribute_
       }
       if (more) request(eb + 16, h);
     }
+  }
+  T *Ai = a.A + (long long) ia * a.nlm * C;
+#pragma unroll
+  for (int l = 0; l < NL; l++) {
+#pragma unroll
+      for (int v = 0; v < 4; v++) {
+        const int m = a.drow[4 * g + v];
+        if (m < 2 * l + 1) {
+#pragma unroll
+          for (int cb = 0; cb < KB; cb++) Ai[(l * l + m) * C + cb * 16 + c] = acc[l][cb][v];
+        }
+      }
+  }
+}
+
+// k_scatter_a_mfma with the B operand formed from the radial tables: lane (g, c) supplies, in step s, the columns
+// l C + cb 16 + c of bond 4 s + g, i.e. per (l, cb) four table entries of the bond's interval (16 lanes read 128
+// consecutive bytes of a table row; the 2.6 MB table of a 32-channel lmax-4 model stays in the L2), the cubic in t, times
+// the species weight.  The entries of step s + 1 are requested when those of step s have been turned into operands, and
+// arrive while the matrix instructions of step s run; x and the element of the lane's four bonds of the NEXT tile are
+// requested a tile ahead.  No radial row is read: the rows need not exist.
+template<class T, int NL, int KB> __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_scatter_a_tab(ScatterArgs<T> a)
+{
+  typedef typename Mfma<T>::v4 v4;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  T *Yw = reinterpret_cast<T *>(smem_raw) + wave * 16 * a.nlm;     // [16 bonds][nlm]
+  const int ia = a.natoms - 1 - (blockIdx.x * 4 + wave);
+  if (ia < 0) return;
+  const int i = a.a0 + ia;
+  const long long w0 = a.eoff[i], w1 = a.eoff[i + 1];
+  const int C = a.C;
+  const RadialTable<T> tb = a.tb;
+  const T h = (T) (1.0 / tb.N), fN = (T) tb.N;
+  v4 acc[NL][KB];
+#pragma unroll
+  for (int l = 0; l < NL; l++)
+#pragma unroll
+    for (int cb = 0; cb < KB; cb++) acc[l][cb] = v4{0, 0, 0, 0};
+  double xs[4], xn[4] = {0, 0, 0, 0};
+  int ms[4], mn[4] = {0, 0, 0, 0};
+  auto geometry = [&](long long eb, double (&x)[4], int (&m)[4]) {
+    const int nb = (int) (w1 - eb < 16 ? w1 - eb : 16);
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      const int b = 4 * s + g;
+      const long long e = eb + (b < nb ? b : 0);
+      x[s] = tb.x[e];
+      m[s] = tb.emu[e];
+    }
+  };
+  // one (step, 16-column block) at a time: NL x 4 entries in flight per lane
+  T raw[NL][4], zc = (T) 0, tt = (T) 0;
+  auto request = [&](int q) {    // q = s KB + cb
+    const int s = q / KB, cb = q % KB;
+    double t;
+    const int k = table_interval(xs[s], tb.N, t);
+    tt = (T) t;
+    zc = tb.z[ms[s] * C + cb * 16 + c];
+#pragma unroll
+    for (int l = 0; l < NL; l++) table_request(tb, k, l * C + cb * 16 + c, a.noutp, raw[l]);
+  };
+  if (w0 < w1) geometry(w0, xs, ms);
+  for (long long eb = w0; eb < w1; eb += 16) {
+    const int nb = (int) (w1 - eb < 16 ? w1 - eb : 16);
+    request(0);
+    const bool more = eb + 16 < w1;
+    if (more) geometry(eb + 16, xn, mn);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (lane < 16) {
+      if (lane < nb) {
+        const double *u = a.rh + 3 * (eb + lane);
+        sh_eval<false, T, NL - 1>(a.sh, u[0], u[1], u[2], Yw + lane * a.nlm, nullptr);
+      } else {
+        for (int q = 0; q < a.nlm; q++) Yw[lane * a.nlm + q] = (T) 0;
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int q = 0; q < 4 * KB; q++) {
+      const int s = q / KB, cb = q % KB;
+      if (4 * s >= nb) continue;                      // a step with no bond: neither evaluated nor multiplied
+      T bv[NL];
+#pragma unroll
+      for (int l = 0; l < NL; l++) {
+        T R, dR;
+        table_value<T, false>(raw[l], tt, h, fN, R, dR);
+        bv[l] = R * zc;
+      }
+      if (q + 1 < 4 * KB && 4 * ((q + 1) / KB) < nb) request(q + 1);
+      const T *yb = Yw + (4 * s + g) * a.nlm;
+#pragma unroll
+      for (int l = 0; l < NL; l++) {
+        const T y = c < 2 * l + 1 ? yb[l * l + c] : (T) 0;       // A operand: row m = c
+        acc[l][cb] = Mfma<T>::mma(y, bv[l], acc[l][cb]);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < 4; s++) { xs[s] = xn[s]; ms[s] = mn[s]; }
   }
   T *Ai = a.A + (long long) ia * a.nlm * C;
 #pragma unroll
@@ -1482,6 +1631,7 @@ template<class T> struct BondBwdArgs {
   const int *ej;
   const double *rh, *r, *rc;
   const T *Rz, *dRz;          // [E][noutp]
+  RadialTable<T> tb;          // tb.F set: value and derivative of the radial functions come from the tables, Rz / dRz are not read
   const T *gA;                // [chunk atoms][nlm][C]
   double *f;                  // [n][3]  (+=, atomics)
   double *virial;             // [6]     (+=, atomics); with sid: record 8 sid[i] of the atom's structure
@@ -1510,7 +1660,9 @@ template<class T> struct BondBwdArgs {
 // third less LDS per block (three blocks per CU instead of two).  gA of the atom sits in LDS as [lm][C + 2]
 // (the pad spreads the rows over the banks); the radial rows of l + 1 are requested before the products of l.
 // KB = channels / 16, NL = lmax + 1.  dynamic LDS: nlm (C + 2) + 4 waves x 16 bonds x 3 nlm values.
-template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_bwd(BondBwdArgs<T> a)
+// TAB: the B operands are formed from the radial tables (lane (g, c): the eight columns l C + 8 g + s of bond c, four table
+// entries each, value and derivative from the same four; requested for l + 1 before the products of l).
+template<class T, int KB, int NL, bool TAB> __global__ __launch_bounds__(256) void k_bond_bwd(BondBwdArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
   constexpr int KS = KB * 4, C = KB * 16, CS = C + 2, NLM = NL * NL;
@@ -1541,8 +1693,24 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
     const T *rp = a.Rz + (eb + (colok ? c : 0)) * a.noutp + g * KS;
     const T *dp = a.dRz + (eb + (colok ? c : 0)) * a.noutp + g * KS;
     T x[2][KS], dx[2][KS];
+    // tables: interval, offset and species weights of bond c, and the entries of l = 0
+    // (four columns at a time: the entries of the next four are requested before the products of these four)
+    constexpr int KH = 4;
+    T raw[TAB ? KH : 1][4], zc[TAB ? KS : 1], tt = (T) 0;
+    int tk = 0;
+    const T th = TAB ? (T) (1.0 / a.tb.N) : (T) 0, tN = TAB ? (T) a.tb.N : (T) 0;
+    if constexpr (TAB) {
+      const long long e = eb + (colok ? c : 0);
+      double t;
+      tk = table_interval(a.tb.x[e], a.tb.N, t);
+      tt = (T) t;
+      const int mu = a.tb.emu[e];
 #pragma unroll
-    for (int s = 0; s < KS; s++) { x[0][s] = rp[s]; dx[0][s] = dp[s]; }
+      for (int s = 0; s < KS; s++) zc[s] = a.tb.z[mu * C + g * KS + s];
+    } else {
+#pragma unroll
+      for (int s = 0; s < KS; s++) { x[0][s] = rp[s]; dx[0][s] = dp[s]; }
+    }
     // geometry of bond `lane` (lanes below nb), kept for the end of the tile
     double u0 = 0, u1 = 0, u2 = 1, br = 1, brc = 1;
     double e1[3] = {1, 0, 0}, e2[3] = {0, 1, 0};
@@ -1555,6 +1723,10 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
       tangent_basis(u, e1, e2);
       sh_eval<true, T, NL - 1>(a.sh, u0, u1, u2, Yw + lane * NLM, Gw + lane * 2 * NLM, e1, e2, Gw + lane * 2 * NLM + NLM);
     }
+    if constexpr (TAB) {
+#pragma unroll
+      for (int s = 0; s < KH; s++) table_request(a.tb, tk, g * KS + s, a.noutp, raw[s]);
+    }
     // LDS writes of this wave visible to its other lanes (the Y / G region is private to the wave)
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -1562,19 +1734,49 @@ template<class T, int KB, int NL> __global__ __launch_bounds__(256) void k_bond_
     double px = 0, p1 = 0, p2 = 0;
 #pragma unroll
     for (int l = 0; l < NL; l++) {
-      const int cur = l & 1, nxt = cur ^ 1;
-      if (l + 1 < NL) {
+      const int cur = TAB ? 0 : (l & 1), nxt = cur ^ 1;
+      if constexpr (!TAB) {
+        if (l + 1 < NL) {
 #pragma unroll
-        for (int s = 0; s < KS; s++) { x[nxt][s] = rp[(l + 1) * C + s]; dx[nxt][s] = dp[(l + 1) * C + s]; }
+          for (int s = 0; s < KS; s++) { x[nxt][s] = rp[(l + 1) * C + s]; dx[nxt][s] = dp[(l + 1) * C + s]; }
+        }
       }
       v4 aP = {0, 0, 0, 0}, aQ = {0, 0, 0, 0};
       // A operand: row m = c of gA_l^T, k = g KS + s
       const T *ga = gAl + (l * l + (c < 2 * l + 1 ? c : 0)) * CS + g * KS;
+      if constexpr (TAB) {
 #pragma unroll
-      for (int s = 0; s < KS; s++) {
-        const T w = c < 2 * l + 1 ? ga[s] : (T) 0;
-        aP = Mfma<T>::mma(w, x[cur][s], aP);
-        aQ = Mfma<T>::mma(w, dx[cur][s], aQ);
+        for (int hb = 0; hb < KS; hb += KH) {
+          T xv[KH], dxv[KH];
+#pragma unroll
+          for (int s = 0; s < KH; s++) {
+            T R, dR;
+            table_value<T, true>(raw[s], tt, th, tN, R, dR);
+            xv[s] = R * zc[hb + s];
+            dxv[s] = dR * zc[hb + s];
+          }
+          // the next four columns: of this l, or the first four of l + 1
+          if (hb + KH < KS) {
+#pragma unroll
+            for (int s = 0; s < KH; s++) table_request(a.tb, tk, l * C + g * KS + hb + KH + s, a.noutp, raw[s]);
+          } else if (l + 1 < NL) {
+#pragma unroll
+            for (int s = 0; s < KH; s++) table_request(a.tb, tk, (l + 1) * C + g * KS + s, a.noutp, raw[s]);
+          }
+#pragma unroll
+          for (int s = 0; s < KH; s++) {
+            const T w = c < 2 * l + 1 ? ga[hb + s] : (T) 0;
+            aP = Mfma<T>::mma(w, xv[s], aP);
+            aQ = Mfma<T>::mma(w, dxv[s], aQ);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+          const T w = c < 2 * l + 1 ? ga[s] : (T) 0;
+          aP = Mfma<T>::mma(w, x[cur][s], aP);
+          aQ = Mfma<T>::mma(w, dx[cur][s], aQ);
+        }
       }
       if (colok) {
 #pragma unroll
