@@ -175,13 +175,34 @@ template<class T> class Engine3L final : public EngineBase {
   Engine3L(std::shared_ptr<const Model3L> m, int ntypes, const std::vector<int> &type2mu, int device) :
       EngineBase(device, "GRACE-3L", ntypes, type2mu, m->n_elements), model_(std::move(m))
   {
-    this->template probe_mfma<T>();
+    this->template probe_mfma_both<T>();
     build();
     end_build();    // buffers allocated from here on are work buffers (release_buffers)
     chunks_ = true;
     ordered_ok_ = true;
   }
   int layers() const override { return 3; }
+  // radial tables per ordered pair of species and per layer: n / 2 intervals for layers 1 and 2 (at least 16), n for layer 3
+  // (spline_n_3l, libgrace/include/grace/system.h:95-103); tables that would exceed the memory they may take are not built
+  // and the MLPs stay (the reference's spline_mb, libgrace/src/fused_3l.cpp:405-418)
+  void apply_spline(int n) override
+  {
+    double total = 0.0;
+    for (int k = 0; k < 3; k++) {
+      L_[k].rad.spline_n = n > 0 ? (k < 2 ? std::max(16, n / 2) : n) : 0;
+      total += L_[k].rad.table_bytes(L_[k].rad.spline_n);
+    }
+    // the three layers' tables together against the limit (2048 MB as Grace3LKK::spline_mb, libgrace/include/grace/kk/
+    // grace_3l_kk.h:1264; GRACE_HIP_TABLE_MB sets another)
+    double limit_mb = 2048.0;
+    if (const char *e = std::getenv("GRACE_HIP_TABLE_MB")) limit_mb = std::atof(e);
+    const bool fits = total <= limit_mb * 1048576.0;
+    for (int k = 0; k < 3; k++) L_[k].rad.tables_allowed = fits;
+    if (n > 0 && !fits)
+      log_message(0, who_ + ": the radial MLPs are evaluated for every bond: tables for " + std::to_string(L_[0].rad.species_mu.size() *
+                         L_[0].rad.species_mu.size()) + " species pairs would need " + std::to_string((long long) (total / 1048576.0)) +
+                         " MB > " + std::to_string((long long) limit_mb) + " MB");
+  }
   void run(const RunFlags &fl) override;
   void debug_radial(int, const double *, const int *, double *, double *) override
   {
@@ -411,6 +432,16 @@ template<class T> void Engine3L<T>::build_layer(int k)
   // ---- radial MLP; fac[mu_j][n] = inv_avg (z_tr[mu_j][n] in layer 1): fused_3l.cpp:441-460
   const int ne = m.embedding_size;
   L.rad.build_species(sp.mlp.layers, sp.mlp.bias, m.chem_embedding, ne, m.nradbase, sp.p, L.C, L.CP, nl_, nel_, drow_, "GRACE-3L");
+  L.rad.build_species_double(sp.mlp.layers, sp.mlp.bias, m.chem_embedding, ne, m.nradbase, sp.p, L.C, L.CP, nl_, nel_, drow64_, "GRACE-3L");
+  {
+    // the species of this engine: the elements its atom types map to (tables per ordered pair of them, fused_3l.cpp:381-398)
+    std::vector<int> present;
+    for (int t = 1; t <= ntypes_; t++) {
+      const int mu = type2mu_[(size_t) t];
+      if (mu >= 0 && std::find(present.begin(), present.end(), mu) == present.end()) present.push_back(mu);
+    }
+    L.rad.set_species(present, nel_, "GRACE-3L layer " + std::to_string(k + 1));
+  }
   auto species_table = [&](const std::vector<double> &W, double norm) {
     std::vector<double> z((size_t) nel_ * L.C);
     for (int mu = 0; mu < nel_; mu++)
@@ -735,7 +766,7 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw, bo
   L.dR.ensure(ecap_ * L.rad.noutp * s);
   T *Rl = moved_back(L.R.template as<T>(), eb_ * L.rad.noutp), *dRl = moved_back(L.dR.template as<T>(), eb_ * L.rad.noutp);
   stage(tg(k, "radial").c_str(), [&] {
-    L.rad.launch(stream_, ncu_, L.fac.template as<T>(), eb_, ecnt_, xr_.as<double>(), emu_.as<int>(), Rl, dRl, n_edges, emi_.as<int>());
+    L.rad.launch(stream_, ncu_, L.fac.template as<T>(), eb_, ecnt_, xr_.as<double>(), emu_.as<int>(), Rl, dRl, n_edges, emi_.as<int>(), true);
   });
   L.X.buf.ensure(L.X.bytes(na, s));
   T *X = L.X.buf.template as<T>();

@@ -393,7 +393,27 @@ template<class T> struct DevRadial {
   // radial tables (the reference's spline_n, libgrace/include/grace/system.h:78): intervals asked for (0: the MLP itself is
   // evaluated for every bond) and the table that exists: value and d/dx at the knots, [N + 1][noutp] each
   int spline_n = 0, table_n = 0;
-  DevBuf tabF, tabD, knots, knot_mu, unit_z, knotF, knotD;
+  DevBuf tabF, tabD, knots, knot_mu, knot_mi, unit_z, knotF, knotD;
+  // species form: the species of the engine (elements that atom types map to), element -> species, and the memory the pair
+  // tables may take (the reference's spline_mb, libgrace/include/grace/system.h:85: beyond it the MLP itself is evaluated)
+  std::vector<int> species_mu;
+  DevBuf sp_of_mu;
+  bool tables_allowed = true;
+  std::string who_tables = "radial tables";
+  void set_species(const std::vector<int> &present_mu, int n_elements, const std::string &who)
+  {
+    species_mu = present_mu;
+    std::vector<int> map((size_t) n_elements, 0);
+    for (size_t q = 0; q < species_mu.size(); q++) map[(size_t) species_mu[q]] = (int) q;
+    upload_vec(sp_of_mu, map);
+    who_tables = who;
+  }
+  // bytes of the tables of `n` intervals for the engine's species pairs
+  double table_bytes(int n) const
+  {
+    const double pairs = mode == 1 ? (double) species_mu.size() * species_mu.size() : 1.0;
+    return sizeof(T) == 8 ? pairs * (n + 1.0) * noutp * 16.0 : pairs * n * 4.0 * noutp * 4.0;
+  }
   // fp32 engines: the same MLP in fp64, which evaluates the knots of the tables (build_double)
   std::unique_ptr<DevRadial<double>> dbl;
   template<class... A> void build_double(A &&...a)
@@ -401,6 +421,13 @@ template<class T> struct DevRadial {
     if constexpr (sizeof(T) == 4) {
       dbl = std::make_unique<DevRadial<double>>();
       dbl->build(std::forward<A>(a)...);
+    }
+  }
+  template<class... A> void build_species_double(A &&...a)
+  {
+    if constexpr (sizeof(T) == 4) {
+      dbl = std::make_unique<DevRadial<double>>();
+      dbl->build_species(std::forward<A>(a)...);
     }
   }
   int mode = 0;    // 1: species form (build_species)
@@ -492,18 +519,25 @@ template<class T> struct DevRadial {
   void launch(hipStream_t stream, int ncu, const T *z, long long e_begin, long long e_count, const double *x, const int *emu, T *Rz, T *dRz,
               const long long *n_edges, const int *emi = nullptr, bool tables = false)
   {
-    if (tables && spline_n > 0 && mode == 0) {
+    if (tables && has_tables()) {
       ensure_tables(stream, ncu);
       const long long bound = e_count >= 0 ? e_count : (long long) 1 << 40;
       const unsigned grid = (unsigned) std::max<long long>(1, std::min<long long>(bound, (long long) ncu * 32));
       hipLaunchKernelGGL((k_radial_spline<T, sizeof(T) == 4>), dim3(grid), dim3(round_up(noutp, 64)), 0, stream, n_edges, e_begin, e_count, x, emu,
-                         (const T *) tabF.template as<T>(), (const T *) tabD.template as<T>(), table_n, z, CP, noutp, Rz, dRz);
+                         (const T *) tabF.template as<T>(), (const T *) tabD.template as<T>(), table_n, z, CP, noutp, Rz, dRz,
+                         mode == 1 ? emi : (const int *) nullptr, (const int *) sp_of_mu.as<int>(), (int) species_mu.size());
       return;
     }
     launch_mlp(stream, ncu, z, e_begin, e_count, x, emu, Rz, dRz, n_edges, emi);
   }
-  // tables requested (spline_n > 0) for a form of the MLP that has them
-  bool has_tables() const { return spline_n > 0 && mode == 0; }
+  // tables requested (spline_n > 0) and, in the species form, within the memory they may take
+  bool has_tables()
+  {
+    if (spline_n <= 0) return false;
+    if (mode == 0) return true;
+    if (species_mu.empty()) return false;
+    return tables_allowed;
+  }
   // the tables as the kernels that evaluate them take them (built on first use and again after release_buffers)
   RadialTable<T> table(hipStream_t stream, int ncu, const double *x, const int *emu, const T *z)
   {
@@ -522,28 +556,43 @@ template<class T> struct DevRadial {
     {
       const int N = spline_n;
       if (table_n != N || !tabF.p || (sizeof(T) == 8 && !tabD.p)) {    // the MLP at the knots x = k / N, unit species weights (again after release_buffers)
-        std::vector<double> xs((size_t) N + 1);
-        for (int k = 0; k <= N; k++) xs[(size_t) k] = (double) k / N;
+        // species form: the knots of every ordered pair of species, pair after pair
+        const size_t nsp = mode == 1 ? species_mu.size() : 1, npair = nsp * nsp;
+        std::vector<double> xs(((size_t) N + 1) * npair);
+        std::vector<int> kmi(xs.size(), 0), kmj(xs.size(), 0);
+        for (size_t pr = 0; pr < npair; pr++)
+          for (int k = 0; k <= N; k++) {
+            const size_t q = pr * ((size_t) N + 1) + k;
+            xs[q] = (double) k / N;
+            if (mode == 1) { kmi[q] = species_mu[pr / nsp]; kmj[q] = species_mu[pr % nsp]; }
+          }
         upload_vec(knots, xs);
-        upload_vec(knot_mu, std::vector<int>((size_t) N + 1, 0));
-        const size_t rows = ((size_t) N + 1) * noutp;
+        upload_vec(knot_mu, kmj);
+        upload_vec(knot_mi, kmi);
+        const long long nknots = (long long) xs.size();
+        const size_t rows = xs.size() * noutp;
         if constexpr (sizeof(T) == 8) {
-          upload_vec(unit_z, std::vector<T>((size_t) CP, (T) 1));
+          upload_vec(unit_z, std::vector<T>((size_t) CP * std::max(nel, 1), (T) 1));
           tabF.ensure(rows * sizeof(T));
           tabD.ensure(rows * sizeof(T));
-          launch_mlp(stream, ncu, unit_z.template as<T>(), 0, (long long) N + 1, knots.as<double>(), knot_mu.as<int>(), tabF.template as<T>(),
-                     tabD.template as<T>(), nullptr, nullptr);
+          launch_mlp(stream, ncu, unit_z.template as<T>(), 0, nknots, knots.as<double>(), knot_mu.as<int>(), tabF.template as<T>(),
+                     tabD.template as<T>(), nullptr, mode == 1 ? knot_mi.as<int>() : nullptr);
         } else {
           if (!dbl) throw Error("radial tables of an fp32 engine need the fp64 form of its radial MLP");
-          upload_vec(unit_z, std::vector<double>((size_t) CP, 1.0));
+          upload_vec(unit_z, std::vector<double>((size_t) CP * std::max(nel, 1), 1.0));
           knotF.ensure(rows * sizeof(double));
           knotD.ensure(rows * sizeof(double));
-          tabF.ensure((size_t) N * 4 * noutp * sizeof(T));
-          dbl->launch_mlp(stream, ncu, unit_z.as<double>(), 0, (long long) N + 1, knots.as<double>(), knot_mu.as<int>(), knotF.as<double>(),
-                          knotD.as<double>(), nullptr, nullptr);
+          tabF.ensure(npair * (size_t) N * 4 * noutp * sizeof(T));
+          dbl->launch_mlp(stream, ncu, unit_z.as<double>(), 0, nknots, knots.as<double>(), knot_mu.as<int>(), knotF.as<double>(),
+                          knotD.as<double>(), nullptr, mode == 1 ? knot_mi.as<int>() : nullptr);
           const long long tot = (long long) N * noutp;
-          hipLaunchKernelGGL(k_spline_coef, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream, (const double *) knotF.as<double>(),
-                             (const double *) knotD.as<double>(), N, noutp, tabF.as<float>());
+          for (size_t pr = 0; pr < npair; pr++)
+            hipLaunchKernelGGL(k_spline_coef, dim3((unsigned) ((tot + 255) / 256)), dim3(256), 0, stream,
+                               (const double *) knotF.as<double>() + pr * ((size_t) N + 1) * noutp,
+                               (const double *) knotD.as<double>() + pr * ((size_t) N + 1) * noutp, N, noutp,
+                               tabF.as<float>() + pr * (size_t) N * 4 * noutp);
+          knotF.release();    // the fp64 knots are needed for the coefficients only
+          knotD.release();
         }
         table_n = N;
       }

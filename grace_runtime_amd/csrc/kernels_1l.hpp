@@ -409,10 +409,14 @@ __device__ inline double ipow(double x, int n)
 // and stays in the L2.  COEF true (fp32): F is [N][4][noutp] coefficients formed in fp64 by k_spline_coef (c2 and c3 are
 // differences of nearly equal values: formed in fp32 they would cost four digits of dR/dx), D unused.
 // One block = noutp threads rounded up to a wave, a thread per column, blocks stride over the edges; rows as k_radial.
+// Species form (GRACE-3L: the MLP takes the embeddings of both atoms of the bond; per-pair tables of the reference,
+// libgrace/src/fused_3l.cpp:487-520): emi set: one table per ordered pair of species, table number sp[emi[e]] nsp +
+// sp[emu[e]] (sp: element -> species of the engine), the tables one after the other in F and D.
 template<class T, bool COEF>
 __global__ void k_radial_spline(const long long *__restrict__ n_edges, long long e_begin, long long e_count, const double *__restrict__ x,
                                 const int *__restrict__ emu, const T *__restrict__ F, const T *__restrict__ D, int N, const T *__restrict__ z, int C,
-                                int noutp, T *__restrict__ Rz, T *__restrict__ dRz)
+                                int noutp, T *__restrict__ Rz, T *__restrict__ dRz, const int *__restrict__ emi = nullptr,
+                                const int *__restrict__ sp = nullptr, int nsp = 1)
 {
   const long long cnt = e_count >= 0 ? e_count : *n_edges - e_begin;
   const int col = threadIdx.x;
@@ -430,11 +434,12 @@ __global__ void k_radial_spline(const long long *__restrict__ n_edges, long long
       k = k > N - 1 ? N - 1 : (k < 0 ? 0 : k);
       t[u] = (T) (sx - k);
       zc[u] = z[emu[e] * C + n];
+      const long long pair = emi ? (long long) sp[emi[e]] * nsp + sp[emu[e]] : 0;
       if (COEF) {
-        const T *c = F + (long long) k * 4 * noutp + col;
+        const T *c = F + (pair * N + k) * 4 * noutp + col;
         c0[u] = c[0]; c1[u] = c[noutp]; c2[u] = c[2 * noutp]; c3[u] = c[3 * noutp];
       } else {
-        const T *f = F + (long long) k * noutp + col, *d = D + (long long) k * noutp + col;
+        const T *f = F + (pair * (N + 1) + k) * noutp + col, *d = D + (pair * (N + 1) + k) * noutp + col;
         c0[u] = f[0]; c1[u] = d[0]; c2[u] = f[noutp]; c3[u] = d[noutp];    // f0, f0', f1, f1'
       }
     }

@@ -239,8 +239,42 @@ class Model3L:
             cluster[a] = k
         return gamma, sigma, cluster, f
 
-    # ---- radial functions R[b, l, c] of layer k: MLP([T_1..T_nrb(2x - 1), emb_i, emb_j]) env(x) fac[mu_j]
+    # ---- radial functions from the reference's tables (libgrace/src/fused_3l.cpp:491-533, evaluated as
+    # spline_eval, libgrace/include/grace/fused_cpu.h:1052-1074), in fp64 (the reference stores fp32 coefficients): one table
+    # per ordered pair of species and per layer, N_k intervals over x in [0, 1] (spline_n_3l, libgrace/include/grace/
+    # system.h:95-103: spline / 2 for layers 1 and 2, at least 16; spline for layer 3), per interval the cubic through value
+    # and derivative of the exact function at both ends.  self.spline = 0 (the default): the exact function.
+    spline = 0
+
     def radial(self, L, x, mi, mj):
+        if not self.spline:
+            return self.radial_exact(L, x, mi, mj)
+        k = self.layers.index(L)
+        N = max(16, self.spline // 2) if k < 2 else self.spline
+        R = torch.zeros((x.shape[0], self.nl, L["C"]), dtype=torch.float64)
+        pairs = torch.unique(torch.stack([mi, mj], 1), dim=0) if x.shape[0] else []
+        for a, b in [(int(p[0]), int(p[1])) for p in pairs]:
+            key = (k, N, a, b)
+            tabs = self.__dict__.setdefault("_tables", {})
+            if key not in tabs:
+                knots = torch.arange(N + 1, dtype=torch.float64) / N
+                ia, ib = torch.full((N + 1,), a, dtype=torch.int64), torch.full((N + 1,), b, dtype=torch.int64)
+                # every row of the exact function depends on its own x only: the tangent along (1, 1, ...) is d/dx row by row
+                F, D = torch.func.jvp(lambda xx: self.radial_exact(L, xx, ia, ib), (knots,), (torch.ones_like(knots),))
+                tabs[key] = (F.detach(), D.detach() / N)
+            F, Dh = tabs[key]
+            sel = torch.nonzero((mi == a) & (mj == b))[:, 0]
+            sx = x[sel] * N
+            kk = torch.clamp(sx.detach().to(torch.int64), 0, N - 1)
+            t = (sx - kk)[:, None, None]
+            f0, f1, d0, d1 = F[kk], F[kk + 1], Dh[kk], Dh[kk + 1]
+            c2 = -3.0 * f0 - 2.0 * d0 + 3.0 * f1 - d1
+            c3 = 2.0 * f0 + d0 - 2.0 * f1 + d1
+            R = R.index_add(0, sel, f0 + t * (d0 + t * (c2 + t * c3)))
+        return R
+
+    # ---- radial functions R[b, l, c] of layer k: MLP([T_1..T_nrb(2x - 1), emb_i, emb_j]) env(x) fac[mu_j]
+    def radial_exact(self, L, x, mi, mj):
         t = 2.0 * x - 1.0
         Tp, Tc, cols = torch.ones_like(t), t, []
         for _ in range(self.nrb):
