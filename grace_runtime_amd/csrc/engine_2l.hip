@@ -615,14 +615,15 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
   const long long *n_edges = eoff_.as<long long>() + n;
   const bool forces = !fl.energy_only;
   if (ordered_ && forces) ordered_begin();
-  const int yw = forces ? 3 * nlm_ : nlm_;    // row of an edge: Y[nlm] and, for forces, the two tangential gradients D1[nlm], D2[nlm]
+  // row of an edge: Y[nlm] and, for forces, the two tangential gradients D1[nlm], D2[nlm] and padding (pair_row_stride)
+  const int yw = forces ? pair_row_stride(nlm_, sizeof(T)) : nlm_;
   YG_.ensure(ecap_all * yw * sizeof(T));
   stage("sh_edges", [&] {
-    const size_t lds = (size_t) 64 * (yw + 1) * sizeof(T);
+    const size_t lds = (size_t) 64 * ((forces ? 3 * nlm_ : nlm_) + 1) * sizeof(T);
     auto kern = k_sh_edges<T>;
     if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
     hipLaunchKernelGGL(kern, dim3((unsigned) ((ecap_all + 63) / 64)), dim3(64), lds, stream_, sh_, rh_.as<double>(), n_edges, nlm_, forces ? 1 : 0,
-                       YG_.as<T>());
+                       YG_.as<T>(), yw);
   });
 
   // ---- chunks of atoms.  Layer 2 gathers the messages of ALL atoms, so the pass is three sweeps over the chunks: layer 1
@@ -854,14 +855,23 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
 #define GR_ARGS_ASYNC                                                                                                                   \
   dim3(nc), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) R1, (const T *) dR1, (const T *) M, (const T *) gP_.as<T>(),        \
       rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(), scal_.as<double>() + 1, nslot_, nI_, CRP_, nl_, radR1_.noutp, \
-      sink_.as<T>(), 1, sid_ptr(), nslot_, 0, nc, a0_, vatom_ptr()
+      sink_.as<T>(), 1, sid_ptr(), nslot_, 0, nc, a0_, vatom_ptr(), yw
 #define GR_ARGS GR_ARGS_ASYNC, po
       // ordered sums: the staged kernel without atomics; the message adjoints of the chunk's bonds are gathered afterwards
       PairOrdered<T> po{};
       if (ordered_) {
         po.gMe = gMe_.as<T>(); po.fedge = fedge_.as<double>(); po.fcen = fcen_.as<double>(); po.e_base = eb; po.ngrp = 1;
       }
-      if (ordered_) {
+      const PairMfmaPlan mp = pair_mfma_plan(nslot_, CRP_, nl_, sizeof(T), pair_waves_);
+      if (!ordered_ && mp.ok && (pair_mfma_ > 0 || (pair_mfma_ < 0 && pair_mfma_pays(nslot_, CRP_, sizeof(T))))) {
+        PairMfmaArgs<T> pa{};
+        pa.eoff = eoff; pa.ej = ej_.as<int>(); pa.YG = YG_.as<T>(); pa.R1 = R1; pa.dR1 = dR1; pa.M = M; pa.gP = gP_.as<T>();
+        pa.rh = rh_.as<double>(); pa.rlen = r_.as<double>(); pa.rcut = rc_.as<double>();
+        pa.gM = gM_.as<T>(); pa.f = f_.as<double>(); pa.virial = scal_.as<double>() + 1; pa.vatom = vatom_ptr(); pa.sid = sid_ptr();
+        pa.nslot = nslot_; pa.nI = nI_; pa.C = CRP_; pa.noutp = radR1_.noutp; pa.natoms = nc; pa.a0 = a0_;
+        for (int q = 0; q < 16; q++) pa.drow[q] = drow_[q];
+        launch_pair_bwd_mfma(mp, pa, nl_, stream_);
+      } else if (ordered_) {
         GR_PAIR_ORD(GR_ARGS)
       } else if (ch == 8) {
         GR_PAIR_ASYNC(8, GR_ARGS_ASYNC)

@@ -1005,8 +1005,17 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
 #define GR_ARGS                                                                                                                          \
   dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl, (const T *) dRl,     \
       (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),   \
-      scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_, vatom_ptr()
-    if (ordered_) {
+      scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_, vatom_ptr(), yw
+    const PairMfmaPlan mp = pair_mfma_plan(L.nlmi, L.CP, nl_, s, pair_waves_);
+    if (!ordered_ && mp.ok && (pair_mfma_ > 0 || (pair_mfma_ < 0 && pair_mfma_pays(L.nlmi, L.CP, s)))) {
+      PairMfmaArgs<T> pa{};
+      pa.eoff = eoff; pa.ej = ej_.as<int>(); pa.YG = YG_.as<T>(); pa.R1 = Rl; pa.dR1 = dRl; pa.M = M_.as<T>(); pa.gP = gpairP_.as<T>();
+      pa.rh = rh_.as<double>(); pa.rlen = r_.as<double>(); pa.rcut = rc_.as<double>();
+      pa.gM = gM_.as<T>(); pa.f = f_.as<double>(); pa.virial = scal_.as<double>() + 1; pa.vatom = vatom_ptr(); pa.sid = sid_ptr();
+      pa.nslot = pa.nI = L.nlmi; pa.C = L.CP; pa.noutp = L.rad.noutp; pa.natoms = n; pa.a0 = a0_;
+      for (int q = 0; q < 16; q++) pa.drow[q] = drow_[q];
+      launch_pair_bwd_mfma(mp, pa, nl_, stream_);
+    } else if (ordered_) {
       GR_PAIR_ORD(GR_ARGS, po)
       const long long nwork = 3 * (long long) (ecnt_ >= 0 ? ecnt_ : std::max<int64_t>(nb_, 1)) + 9ll * n;
       hipLaunchKernelGGL(k_ordered_combine, dim3((unsigned) ((nwork + 255) / 256)), dim3(256), 0, stream_, (const double *) fpart_.as<double>(),
@@ -1023,7 +1032,6 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
     }
 #undef GR_ARGS
   });
-  (void) yw;
 }
 
 // bytes of chunk-sized work buffers per atom of a chunk (per-atom tensors of the forward and the reverse pass and, per bond
@@ -1066,14 +1074,15 @@ template<class T> void Engine3L<T>::run(const RunFlags &fl)
   if (ordered_ && forces) ordered_begin();
   emi_.ensure(ecap * sizeof(int));
   stage("edge_center", [&] { hipLaunchKernelGGL(k_edge_center, dim3(n), dim3(64), 0, stream_, eoff_.as<long long>(), mu_.as<int>(), emi_.as<int>()); });
-  const int yw = forces ? 3 * nlm_ : nlm_;    // row of an edge: Y[nlm] and, for forces, the two tangential gradients D1[nlm], D2[nlm]
+  // row of an edge: Y[nlm] and, for forces, the two tangential gradients D1[nlm], D2[nlm] and padding (pair_row_stride)
+  const int yw = forces ? pair_row_stride(nlm_, sizeof(T)) : nlm_;
   YG_.ensure(ecap * yw * sizeof(T));
   stage("sh_edges", [&] {
-    const size_t lds = (size_t) 64 * (yw + 1) * sizeof(T);
+    const size_t lds = (size_t) 64 * ((forces ? 3 * nlm_ : nlm_) + 1) * sizeof(T);
     auto kern = k_sh_edges<T>;
     if (lds > 48 * 1024) HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds));
     hipLaunchKernelGGL(kern, dim3((unsigned) ((ecap + 63) / 64)), dim3(64), lds, stream_, sh_, rh_.as<double>(), n_edges, nlm_, forces ? 1 : 0,
-                       YG_.as<T>());
+                       YG_.as<T>(), yw);
   });
   uq_on_ = fl.uq;
   if (fl.uq) {

@@ -30,12 +30,12 @@ template<class T> __global__ void k_clear_functions(T *G, int nfun, int KP, cons
 
 
 // One thread per edge: YG[e] = (Y[nlm], D1[nlm], D2[nlm]) (row width W = 3 nlm), or Y[nlm] alone (W = nlm, no
-// gradients).  D1 = G . e1, D2 = G . e2 are the components of the gradient G of the polynomial extension of Y along the
+// gradients), in rows of `stride` >= W values, the rest of a row zero.  D1 = G . e1, D2 = G . e2 are the components of the gradient G of the polynomial extension of Y along the
 // tangent vectors of the bond (tangent_basis): the bond force only uses the part of sum_lm gY_lm G_lm normal to the bond,
 // g - (g . rhat) rhat = (g . e1) e1 + (g . e2) e2, so two components per harmonic carry all of it.
 // The lanes write their rows into an LDS tile, the block copies the tile out in consecutive addresses.
 // block: 64 threads; dynamic LDS: 64 * (W + 1) values.
-template<class T> __global__ void k_sh_edges(ShCoef sh, const double *rh, const long long *n_edges, int nlm, int grad, T *YG)
+template<class T> __global__ void k_sh_edges(ShCoef sh, const double *rh, const long long *n_edges, int nlm, int grad, T *YG, int stride)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   T *tile = reinterpret_cast<T *>(smem_raw);
@@ -55,8 +55,11 @@ template<class T> __global__ void k_sh_edges(ShCoef sh, const double *rh, const 
   }
   __syncthreads();
   const int rows = (int) (ne - e0 < 64 ? ne - e0 : 64);
-  T *out = YG + e0 * W;
-  for (int q = t; q < rows * W; q += 64) out[q] = tile[(q / W) * (W + 1) + q % W];
+  T *out = YG + e0 * stride;
+  for (int q = t; q < rows * stride; q += 64) {
+    const int r = q / stride, col = q % stride;
+    out[q] = col < W ? tile[r * (W + 1) + col] : (T) 0;
+  }
 }
 
 // M[atom][slot][n] = z[mu_atom][n]
@@ -167,7 +170,7 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
                            const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
                            T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
                            int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms, int a0,
-                           double *__restrict__ vatom, PairOrdered<T> ord)
+                           double *__restrict__ vatom, int ystr, PairOrdered<T> ord)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   __shared__ double bsum[kPairChunk][4];
@@ -192,14 +195,14 @@ __global__ void k_pair_bwd(const long long *__restrict__ eoff, const int *__rest
   for (long long base = e0; base < e1; base += kPairChunk) {
     const int nb = (int) (e1 - base < kPairChunk ? e1 - base : kPairChunk);
     __syncthreads();
-    touch += pair_stage<T>(ej, M, R1, dR1, YG, nlm * 3, nlm * 3, base, nb, nslot, C, noutp, active, slot, n, Msh, Rsh, dRsh, NT);
+    touch += pair_stage<T>(ej, M, R1, dR1, YG, ystr, nlm * 3, base, nb, nslot, C, noutp, active, slot, n, Msh, Rsh, dRsh, NT);
     if (t < kPairChunk * 4) bsum[t >> 2][t & 3] = 0.0;
     __syncthreads();
     for (int b = 0; b < nb; b++) {
       const long long e = base + b;
       const T m = Msh[b * NT + t];
       const T *r = Rsh + b * noutp + n, *dr = dRsh + b * noutp + n;
-      const T *yg = YG + e * nlm * 3;
+      const T *yg = YG + e * ystr;
       T sI = (T) 0, dE = (T) 0, t1 = (T) 0, t2 = (T) 0;
       // every l is the body of a loop that runs `one` (= 1, a kernel argument) times: its uniform loads then stay inside
       // it (all harmonics of a bond at once need more scalar registers than there are)
@@ -427,7 +430,7 @@ __global__ void k_pair_bwd_async(const long long *__restrict__ eoff, const int *
                                  const double *__restrict__ rh, const double *__restrict__ rlen, const double *__restrict__ rcut,
                                  T *__restrict__ gM, double *__restrict__ f, double *__restrict__ virial, int nslot, int nI, int C, int nl,
                                  int noutp, T *__restrict__ sink, int one, const int *__restrict__ sid, int spb, int ngrp, int natoms, int a0,
-                                 double *__restrict__ vatom)
+                                 double *__restrict__ vatom, int ystr)
 {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   __shared__ double bsum[2][CH][4];
@@ -483,13 +486,13 @@ __global__ void k_pair_bwd_async(const long long *__restrict__ eoff, const int *
       // the harmonics of the next chunk, one 64-byte piece per thread, so that its uniform reads find them in the L2
       const long long nbase = base + CH;
       const int nnb = (int) (e1 - nbase < CH ? e1 - nbase : CH), per = (nlm * 3 + 7) / 8;
-      if (t < nnb * per) tv = YG[(nbase + t / per) * nlm * 3 + (t % per) * 8];
+      if (t < nnb * per) tv = YG[(nbase + t / per) * ystr + (t % per) * 8];
     }
     for (int b = 0; b < nb; b++) {
       const long long e = base + b;
       const T m = Msh[(size_t) (buf * CH + b) * NT + t];
       const T *r = Rsh + (size_t) (buf * CH + b) * noutp + n, *dr = dRsh + (size_t) (buf * CH + b) * noutp + n;
-      const T *yg = YG + e * nlm * 3;
+      const T *yg = YG + e * ystr;
       T sI = (T) 0, dE = (T) 0, t1 = (T) 0, t2 = (T) 0;
 #pragma unroll
       for (int l = 0; l <= kKernMaxL; l++)
@@ -555,6 +558,337 @@ __global__ void k_pair_bwd_async(const long long *__restrict__ eoff, const int *
     }
   }
   if (touch == (T) 1.2345e300) sink[0] = touch;    // keeps the touching loads alive
+}
+
+// ---- the reverse pair kernel on the matrix cores
+// For one atom the adjoints gP[slot][lm][n] are fixed while the bonds change, so per l the three sums over m
+//   S_l, T_l,1, T_l,2 [bond][column] = sum_m (Y, D1, D2)[bond][l, m] gP[l, m][column],   column = (slot, n),
+// are products of a [16 bonds][2l + 1] tile of the harmonics with a [2l + 1][16 columns] tile of the adjoints: MFMA
+// 16x16x4 with the bonds as rows, K = 2l + 1 in steps of 4 (the unused k of the last step are zero in the adjoint
+// tile).  A wave owns 16 channels (n0 .. n0 + 15) of TPW slots: its adjoint tiles stay in registers for all bonds of
+// the atom.  The harmonics of a chunk of 16 bonds (rows padded to `ystr` values in memory, so that a chunk is one range
+// of 16-byte pieces and its LDS rows fall into different banks) and the neighbours' message rows are copied to LDS
+// asynchronously one chunk ahead, a thread issuing a few 16-byte pieces; the neighbour indices of the chunk after that
+// wait in registers.  The radial rows come from memory, 16 lanes reading 128 consecutive bytes of a bond's row.
+// Per accumulator value (bond, column, l) four multiply-adds remain for the vector unit:
+//   sI += R_l S_l;  U_l += S_l m,  V_l,k += T_l,k m  (m = the neighbour's message value; summed over the wave's slots)
+// and per (bond, n, l) three:  dE/dx += dR_l U_l,  g_k += R_l V_l,k.
+// Blocks are small (at most 4 waves by default, 16 tiles of 16 columns) so that two or three of them share a CU and the
+// copies, barriers and force sums of one overlap the matrix work of another.
+// grid: as k_pair_bwd (pair_block); block: 64 (C / 16) ceil(spb / TPW) threads;
+// dynamic LDS: 2 * 16 * (spb C + ystr) values.
+template<class T> struct PairMfmaArgs {
+  const long long *eoff;
+  const int *ej;
+  const T *YG, *R1, *dR1, *M, *gP;
+  const double *rh, *rlen, *rcut;
+  T *gM;
+  double *f, *virial, *vatom;
+  const int *sid;
+  int nslot, nI, C, noutp, spb, ngrp, natoms, a0, ystr;
+  int one;         // 1
+  int drow[16];    // accumulator row of (lane / 16, register)
+};
+
+constexpr int pair_mfma_steps(int l) { return (2 * l + 1 + 3) / 4; }
+constexpr int pair_mfma_step0(int l) { return l == 0 ? 0 : pair_mfma_step0(l - 1) + pair_mfma_steps(l - 1); }
+constexpr int kPairMfmaPieces = 4;    // 16-byte pieces of the neighbour rows of a chunk that one thread may have to copy
+
+// nwords 4-byte words from global memory to LDS, in order: pieces of 64 words dealt to the waves
+__device__ inline void block_copy_async_words(const void *src, void *dst, int nwords, int wave, int nw, int lane)
+{
+  for (int p = wave; p * 64 < nwords; p += nw)
+    if (p * 64 + lane < nwords)
+      lds_load_word(reinterpret_cast<const char *>(src) + 4 * (size_t) (p * 64 + lane), reinterpret_cast<char *>(dst) + 256 * (size_t) p);
+}
+// one 16-byte piece per lane: lane's source address, the wave's destination (the lanes' pieces land one after another)
+__device__ inline void lds_load_piece(const void *src, void *lds_wave_base)
+{
+  __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *) src, (void __attribute__((address_space(3))) *) lds_wave_base, 16, 0, 0);
+}
+
+template<class T, int NL, int TPW>
+__global__ __launch_bounds__(512) void k_pair_bwd_mfma(PairMfmaArgs<T> a)
+{
+  typedef typename Mfma<T>::v4 v4;
+  constexpr int NLM = NL * NL, STEPS = pair_mfma_step0(NL), VPP = 16 / (int) sizeof(T);    // VPP: values per 16-byte piece
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  __shared__ double bsum[2][16][4], fsum[16][9];    // fsum: what thread t < 16 has summed over its bonds (3 force, 6 virial)
+  __shared__ __align__(16) double g_rh[2][48], g_r[2][16], g_rc[2][16];
+  __shared__ __align__(16) int g_j[2][16];
+  int i, grp;
+  if (!pair_block(a.ngrp, a.natoms, i, grp)) return;
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6, NT = blockDim.x;
+  const int c = lane & 15, g = lane >> 4;
+  const int C = a.C, nbk = C >> 4, mrow = a.spb * C;
+  T *Msh = reinterpret_cast<T *>(smem_raw), *Ysh = Msh + 2 * 16 * mrow;
+  const int n0 = (wave % nbk) * 16, ls0 = (wave / nbk) * TPW;       // channels and first local slot of the wave
+  const int nloc = a.nslot - grp * a.spb < a.spb ? a.nslot - grp * a.spb : a.spb;    // slots of this block
+  const long long e0 = a.eoff[i], e1 = a.eoff[i + 1];
+  const int nchunk = (int) ((e1 - e0 + 15) / 16);
+  // the pieces of the neighbour rows that this thread copies: piece id = t + k NT of the chunk, ppr pieces per row
+  const int ppr = nloc * C / VPP;
+  int prow[kPairMfmaPieces], poff[kPairMfmaPieces], jn[kPairMfmaPieces];
+#pragma unroll
+  for (int k = 0; k < kPairMfmaPieces; k++) {
+    const int id = t + k * NT;
+    prow[k] = ppr > 0 ? id / ppr : 16;
+    poff[k] = ppr > 0 ? (id % ppr) * VPP : 0;
+  }
+  auto neighbours = [&](int ch) {      // of the rows this thread copies in chunk ch
+    const long long base = e0 + (long long) ch * 16;
+#pragma unroll
+    for (int k = 0; k < kPairMfmaPieces; k++) jn[k] = (prow[k] < 16 && base + prow[k] < e1) ? a.ej[base + prow[k]] : -1;
+  };
+  if (nchunk > 0) neighbours(0);
+  int rows[4];
+#pragma unroll
+  for (int v = 0; v < 4; v++) rows[v] = a.drow[4 * g + v];
+  // the adjoint tiles of the wave: B operand, lane (g, c) holds k = 4 s + g of column c
+  T B[TPW][STEPS];
+  bool any = false;
+#pragma unroll
+  for (int q = 0; q < TPW; q++) {
+    const bool ok = ls0 + q < nloc;
+    any = any || ok;
+    const T *gp = a.gP + ((long long) i * a.nslot + grp * a.spb + (ok ? ls0 + q : 0)) * NLM * C + n0 + c;
+#pragma unroll
+    for (int l = 0; l < NL; l++)
+#pragma unroll
+      for (int s = 0; s < pair_mfma_steps(l); s++) {
+        const int kk = 4 * s + g;
+        B[q][pair_mfma_step0(l) + s] = (ok && kk < 2 * l + 1) ? gp[(long long) (l * l + kk) * C] : (T) 0;
+      }
+  }
+  for (int q = t; q < 2 * 16 * 4; q += NT) (&bsum[0][0][0])[q] = 0.0;
+  for (int q = t; q < 16 * 9; q += NT) (&fsum[0][0])[q] = 0.0;
+  __syncthreads();
+  // stage(ch): the copies of chunk ch into buffer ch & 1 (jn: its neighbours), then the neighbours of chunk ch + 1
+  auto stage = [&](int ch) {
+    const long long base = e0 + (long long) ch * 16;
+    const int nb = (int) (e1 - base < 16 ? e1 - base : 16), buf = ch & 1;
+    char *mdst = reinterpret_cast<char *>(Msh + (size_t) buf * 16 * mrow) + 16 * (size_t) (t & ~63);
+#pragma unroll
+    for (int k = 0; k < kPairMfmaPieces; k++)
+      if (jn[k] >= 0) lds_load_piece(a.M + ((long long) jn[k] * a.nslot + grp * a.spb) * C + poff[k], mdst + 16 * (size_t) k * NT);
+    // the rows of the harmonics: one range of memory, rows of ystr values here as there
+    const int ypieces = nb * a.ystr / VPP;
+    const char *ysrc = reinterpret_cast<const char *>(a.YG + base * a.ystr);
+    char *ydst = reinterpret_cast<char *>(Ysh + (size_t) buf * 16 * a.ystr);
+    for (int id0 = t & ~63; id0 < ypieces; id0 += NT)
+      if (id0 + lane < ypieces) lds_load_piece(ysrc + 16 * (size_t) (id0 + lane), ydst + 16 * (size_t) id0);
+    if (wave == 0) {    // the wave that reads them for the forces of the chunk before: its reads come first
+      block_copy_async_words(a.rh + 3 * base, &g_rh[buf][0], nb * 6, 0, 1, lane);
+      if (lane < nb * 2) lds_load_word(reinterpret_cast<const char *>(a.rlen + base) + 4 * lane, &g_r[buf][0]);
+      if (lane < nb * 2) lds_load_word(reinterpret_cast<const char *>(a.rcut + base) + 4 * lane, &g_rc[buf][0]);
+      if (lane < nb) lds_load_word(reinterpret_cast<const char *>(a.ej + base) + 4 * lane, &g_j[buf][0]);
+    }
+    if (ch + 1 < nchunk) neighbours(ch + 1);
+  };
+  // round ch stages chunk ch + 1 and works on chunk ch (round -1 only stages)
+  for (int ch = -1; ch < nchunk; ch++) {
+    const long long base = e0 + (long long) ch * 16;
+    const int nb = ch < 0 ? 0 : (int) (e1 - base < 16 ? e1 - base : 16), buf = ch & 1;
+    if (ch + 1 < nchunk) stage(ch + 1);
+    if (nb > 0 && any) {
+      const T *Yc = Ysh + (size_t) (buf * 16 + c) * a.ystr + g;          // A operand: row = bond c of the chunk, k = 4 s + g
+      const T *Mc = Msh + (size_t) buf * 16 * mrow + n0 + c;
+      // the radial rows of the lane's four bonds (rows beyond the chunk: its last bond; their results are not used)
+      int ro[4];
+#pragma unroll
+      for (int v = 0; v < 4; v++) ro[v] = (int) ((rows[v] < nb ? rows[v] : nb - 1) * a.noutp) + n0 + c;
+      const T *Rb = a.R1 + base * a.noutp, *dRb = a.dR1 + base * a.noutp;
+      T sI[TPW][4], pE[4], p1[4], p2[4];
+      // the message values of the lane's bonds: rows of nloc C values, as copied (a row beyond the chunk: its last bond;
+      // what it gives is not used)
+      int mo[4];
+#pragma unroll
+      for (int v = 0; v < 4; v++) mo[v] = (rows[v] < nb ? rows[v] : nb - 1) * (nloc * C) + (ls0 < nloc ? ls0 : 0) * C;
+#pragma unroll
+      for (int q = 0; q < TPW; q++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) sI[q][v] = (T) 0;
+#pragma unroll
+      for (int v = 0; v < 4; v++) pE[v] = p1[v] = p2[v] = (T) 0;
+      // every l is the body of a loop that runs `one` (= 1, a kernel argument) times, so that its loads stay inside it
+#pragma unroll
+      for (int l = 0; l < NL; l++)
+        for (int it = 0; it < a.one; it++) {
+          T rc[4], dc[4];
+#pragma unroll
+          for (int v = 0; v < 4; v++) { rc[v] = Rb[ro[v] + l * C]; dc[v] = dRb[ro[v] + l * C]; }
+          T aS[3], a1[3], a2[3];
+#pragma unroll
+          for (int s = 0; s < pair_mfma_steps(l); s++) {
+            aS[s] = Yc[l * l + 4 * s];
+            a1[s] = Yc[NLM + l * l + 4 * s];
+            a2[s] = Yc[2 * NLM + l * l + 4 * s];
+          }
+          // the matrix products of all tiles of the wave first (a tile without a slot: its adjoint tile is zero), then
+          // the vector work on their results: while that runs, the matrix unit works for the other wave of the SIMD
+          v4 accS[TPW], acc1[TPW], acc2[TPW];
+#pragma unroll
+          for (int q = 0; q < TPW; q++) accS[q] = acc1[q] = acc2[q] = v4{0, 0, 0, 0};
+#pragma unroll
+          for (int s = 0; s < pair_mfma_steps(l); s++)
+#pragma unroll
+            for (int q = 0; q < TPW; q++) {
+              const T b = B[q][pair_mfma_step0(l) + s];
+              accS[q] = Mfma<T>::mma(aS[s], b, accS[q]);
+              acc1[q] = Mfma<T>::mma(a1[s], b, acc1[q]);
+              acc2[q] = Mfma<T>::mma(a2[s], b, acc2[q]);
+            }
+          T U[4] = {0, 0, 0, 0}, V1[4] = {0, 0, 0, 0}, V2[4] = {0, 0, 0, 0};
+#pragma unroll
+          for (int q = 0; q < TPW; q++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+              const T m = ls0 + q < nloc ? Mc[mo[v] + q * C] : (T) 0;
+              sI[q][v] += rc[v] * accS[q][v];
+              U[v] += accS[q][v] * m;
+              V1[v] += acc1[q][v] * m;
+              V2[v] += acc2[q][v] * m;
+            }
+#pragma unroll
+          for (int v = 0; v < 4; v++) {
+            pE[v] += dc[v] * U[v];
+            p1[v] += rc[v] * V1[v];
+            p2[v] += rc[v] * V2[v];
+          }
+        }
+      // dE/dI of the neighbours
+#pragma unroll
+      for (int q = 0; q < TPW; q++) {
+        const int slot = grp * a.spb + ls0 + q;
+        if (ls0 + q < nloc && slot < a.nI) {
+#pragma unroll
+          for (int v = 0; v < 4; v++)
+            if (rows[v] < nb) atomicAdd(&a.gM[((long long) g_j[buf][rows[v]] * a.nI + slot) * C + n0 + c], sI[q][v]);
+        }
+      }
+      // the three sums of the lane's four bonds over the 16 columns: 12 values, halved twice while exchanged, so that
+      // lane c holds the sums of register v = c % 4
+      double w[12];
+#pragma unroll
+      for (int v = 0; v < 4; v++) { w[v] = (double) pE[v]; w[4 + v] = (double) p1[v]; w[8 + v] = (double) p2[v]; }
+      const bool b0 = c & 1, b1 = c & 2;
+      double h[6];
+#pragma unroll
+      for (int q = 0; q < 6; q++) {
+        const double keep = b0 ? w[2 * q + 1] : w[2 * q], give = b0 ? w[2 * q] : w[2 * q + 1];
+        h[q] = keep + __shfl_xor(give, 1, 64);
+      }
+      double z[3];
+#pragma unroll
+      for (int q = 0; q < 3; q++) {
+        const double keep = b1 ? h[2 * q + 1] : h[2 * q], give = b1 ? h[2 * q] : h[2 * q + 1];
+        z[q] = keep + __shfl_xor(give, 2, 64);
+        z[q] += __shfl_xor(z[q], 4, 64);
+        z[q] += __shfl_xor(z[q], 8, 64);
+      }
+      if (c < 4) {
+        const int row = a.drow[4 * g + c];
+        if (row < nb) {
+#pragma unroll
+          for (int q = 0; q < 3; q++) atomicAdd(&bsum[buf][row][q], z[q]);
+        }
+      }
+    }
+    wait_async_loads();
+    __syncthreads();
+    // the forces of the chunk: threads 0 .. nb - 1 while the other waves go on; bsum[buf] is clear again before the
+    // chunk after the next adds to it (a barrier lies between)
+    if (t < nb) {
+      const double *u = &g_rh[buf][3 * t];
+      const double r = g_r[buf][t], rcv = g_rc[buf][t];
+      const double dEdr = bsum[buf][t][0] / rcv, g1 = bsum[buf][t][1] / r, g2 = bsum[buf][t][2] / r;
+      bsum[buf][t][0] = bsum[buf][t][1] = bsum[buf][t][2] = 0.0;
+      double e1v[3], e2v[3], fv[3];
+      tangent_basis(u, e1v, e2v);
+      for (int d = 0; d < 3; d++) fv[d] = dEdr * u[d] + g1 * e1v[d] + g2 * e2v[d];
+      const int jj = g_j[buf][t];
+      double *fs = fsum[t];
+      for (int d = 0; d < 3; d++) {
+        fs[d] += fv[d];
+        atomicAdd(&a.f[3 * (long long) jj + d], -fv[d]);
+      }
+      const double ddx = -u[0] * r, ddy = -u[1] * r, ddz = -u[2] * r;
+      fs[3] += ddx * fv[0]; fs[4] += ddy * fv[1]; fs[5] += ddz * fv[2];
+      fs[6] += ddx * fv[1]; fs[7] += ddx * fv[2]; fs[8] += ddy * fv[2];
+      if (a.vatom) {    // per-atom virial, as k_pair_bwd
+        double *vj = a.vatom + 9 * (long long) jj;
+        atomicAdd(vj, 0.5 * ddx * fv[0]); atomicAdd(vj + 1, 0.5 * ddy * fv[1]); atomicAdd(vj + 2, 0.5 * ddz * fv[2]);
+        atomicAdd(vj + 3, 0.5 * ddx * fv[1]); atomicAdd(vj + 4, 0.5 * ddx * fv[2]); atomicAdd(vj + 5, 0.5 * ddy * fv[2]);
+        double *vi = a.vatom + 9 * (long long) (a.a0 + i);
+        const double yx = 0.5 * ddy * fv[0], zx = 0.5 * ddz * fv[0], zy = 0.5 * ddz * fv[1];
+        atomicAdd(vj + 6, yx); atomicAdd(vj + 7, zx); atomicAdd(vj + 8, zy);
+        atomicAdd(vi + 6, yx); atomicAdd(vi + 7, zx); atomicAdd(vi + 8, zy);
+      }
+    }
+  }
+  if (t < 9 && e1 > e0) {
+    double sum = 0.0;
+    for (int q = 0; q < 16; q++) sum += fsum[q][t];      // written by threads of this wave
+    if (t < 3) atomicAdd(&a.f[3 * (long long) (a.a0 + i) + t], sum);
+    else {
+      atomicAdd(&a.virial[(a.sid ? 8 * a.sid[a.a0 + i] : 0) + t - 3], sum);
+      if (a.vatom) atomicAdd(&a.vatom[9 * (long long) (a.a0 + i) + t - 3], 0.5 * sum);
+    }
+  }
+}
+
+// Values per row of the harmonics and their two gradient components in memory: at least 3 nlm + 3 (the last MFMA step of
+// the largest l reads up to three values past the row's third part: zeros), a whole number of 16-byte pieces, and 16
+// consecutive rows in different LDS banks (fp64: rows 2 (mod 4) values apart, fp32: 4 (mod 8))
+inline int pair_row_stride(int nlm, size_t value_bytes)
+{
+  int v = 3 * nlm + 3;
+  if (value_bytes == 8) while (v % 4 != 2) v++;
+  else while (v % 8 != 4) v++;
+  return v;
+}
+
+// Shape of a k_pair_bwd_mfma launch for nslot message functions of C channels (TPW = 2) in blocks of at most `waves`
+// waves: ok = false where the kernel does not apply (channels not in blocks of 16 or more of them than 16 waves' worth,
+// lmax above 6, a thread would copy more than kPairMfmaPieces pieces of the neighbour rows)
+struct PairMfmaPlan {
+  bool ok = false;
+  int spb = 0, ngrp = 0, threads = 0, ystr = 0;
+  size_t lds = 0;
+};
+inline PairMfmaPlan pair_mfma_plan(int nslot, int C, int nl, size_t value_bytes, int waves)
+{
+  PairMfmaPlan p;
+  if (C % 16 != 0 || nl > 7 || nslot < 1) return p;
+  const int nbk = C / 16, wsmax = waves / nbk;
+  if (wsmax < 1) return p;
+  const int spbmax = wsmax * 2;
+  p.ngrp = (nslot + spbmax - 1) / spbmax;
+  p.spb = (nslot + p.ngrp - 1) / p.ngrp;
+  p.threads = 64 * nbk * ((p.spb + 1) / 2);
+  p.ystr = pair_row_stride(nl * nl, value_bytes);
+  p.lds = (size_t) 2 * 16 * (p.spb * C + p.ystr) * value_bytes;
+  const int pieces = 16 * (p.spb * C * (int) value_bytes / 16);
+  p.ok = p.lds <= kPairLdsMax && p.threads <= 512 && pieces <= kPairMfmaPieces * p.threads;
+  return p;
+}
+// Where the matrix-core kernel is the faster one of the reverse pair kernels (measured, fp64 / fp32, vector kernel ->
+// this one): 72 slots x 64 channels 43.6 -> 37.2 ms / 31.8 -> 25.7 ms; 36 x 64: 24.5 -> 18.9 / 16.6 -> 13.0; 5 x 32:
+// 6.9 -> 5.3 / 4.0 -> 4.3.  fp32 with few columns per atom stays with the vector kernel that copies asynchronously.
+inline bool pair_mfma_pays(int nslot, int C, size_t value_bytes) { return value_bytes == 8 || nslot * C >= 1024; }
+
+template<class T> inline void launch_pair_bwd_mfma(const PairMfmaPlan &p, PairMfmaArgs<T> a, int nl, hipStream_t stream)
+{
+  void (*kern)(PairMfmaArgs<T>) = nl == 1 ? k_pair_bwd_mfma<T, 1, 2> : nl == 2 ? k_pair_bwd_mfma<T, 2, 2> : nl == 3 ? k_pair_bwd_mfma<T, 3, 2>
+                                : nl == 4 ? k_pair_bwd_mfma<T, 4, 2> : nl == 5 ? k_pair_bwd_mfma<T, 5, 2> : nl == 6 ? k_pair_bwd_mfma<T, 6, 2>
+                                                                                                            : k_pair_bwd_mfma<T, 7, 2>;
+  if (p.lds > 48 * 1024)
+    HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int) p.lds));
+  a.spb = p.spb;
+  a.ngrp = p.ngrp;
+  a.ystr = p.ystr;
+  a.one = 1;
+  hipLaunchKernelGGL(kern, dim3((unsigned) ((a.natoms + 7) / 8 * 8 * p.ngrp)), dim3(p.threads), p.lds, stream, a);
 }
 
 struct Energy2Dev {
