@@ -41,13 +41,14 @@ HBM_PEAK = 8000.0                 # GB/s
 # HBM bytes per launch of the dominant kernel measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs of this
 # script, counters scaled by what they read for the 1 GiB copy kernel; summaries under profiles/): (workload, kernel)
 MEASURED_TRAFFIC = {
-    ("config2", "radial_mlp"): 14.9e6 + 1224.4e6,       # fetch + write of k_radial<double,4,0,0,true> (its launches on the full edge list)
-    ("config3", "pair_bwd"): 11240.9e6 + 2773.0e6,      # fetch + write of k_pair_bwd<double,25>
-    ("config4", "pair_bwd_L3"): 48727e6 + 30596e6,      # the layer-3 launches of k_pair_bwd<double,36> (layer 2: 25.6 + 15.2 GB)
-    ("config5", "pair_bwd"): 9842.0e6 + 2477.7e6,       # fetch + write of k_pair_bwd<double,25> over the ragged batch
+    ("config2", "radial_mlp"): 14.3e6 + 1175.4e6,       # fetch + write of k_radial<double,4,0,0,true> (its launches on the full edge list)
+    ("config3", "pair_bwd"): 10754.5e6 + 2764.4e6,      # fetch + write of k_pair_bwd_mfma<double,5,2>
+    ("config4", "pair_bwd_L3"): 44870e6 + 31121e6,      # the layer-3 launches of k_pair_bwd_mfma<double,6,2> (layer 2: 24.5 + 15.6 GB)
+    ("config5", "pair_bwd"): 8993.2e6 + 2467.7e6,       # fetch + write of k_pair_bwd_mfma<double,5,2> over the ragged batch
 }
-# the per-atom dense chain of configuration 2 (every FC, product, reduce and readout launch of a pass), same counters
-DENSE_TRAFFIC = {"config2": 6.5e9}
+# the per-atom dense chain of configuration 2 (chain_fwd 0.72 GB, k_reduce_fwd 0.19, k_energy < 0.01, k_reduce_bwd 0.19, chain_bwd
+# 0.79 GB: every launch between the A basis and the bond reverse), same counters
+DENSE_TRAFFIC = {"config2": 1.90e9}
 DENSE_PREFIXES = ("fc_", "prod_", "reduce_", "energy_mlp", "zero_grads", "chain_")
 
 

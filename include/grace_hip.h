@@ -320,15 +320,18 @@ int gr_system_chunksize(const gr_system *s);
 int gr_engine_set_ordered_sums(gr_engine *e, int on);
 int gr_engine_ordered_sums(const gr_engine *e);
 
-/* Radial tables: intervals > 0 makes a GRACE-1L or 2L engine take its radial functions from cubic tables of that many
+/* Radial tables: intervals > 0 makes an engine take its radial functions from cubic tables of that many
  * intervals over r / rc in [0, 1] (per interval the cubic through the values and derivatives of the radial MLP at its two
  * ends), which is how the reference's CPU and GPU engines evaluate them: FusedSettings::spline_n, default 1024
  * (libgrace/include/grace/system.h:78), `spline` of Model / System / Batch (python/kk/kk_api.h:53,75), tables of
  * Grace1LFused::build_splines (libgrace/src/fused_1l.cpp:102-129), evaluation spline_eval (fused_cpu.h:1052-1074); the
  * tables here hold the engine's precision where the reference's hold fp32.  0, the default of gr_engine_create: the
  * radial MLP itself is evaluated for every bond (no interpolation error).  16 .. 1048576, else GR_INVALID.  GRACE-3L
- * engines accept the call, say so through the logger and keep evaluating their radial MLPs (their tables would be per pair
- * of species).  gr_engine_spline: the value set. */
+ * engines hold one table per ordered pair of the engine's species and per layer, of intervals / 2 (at least 16) for
+ * layers 1 and 2 and of `intervals` for layer 3 (libgrace/src/fused_3l.cpp:491-533, spline_n_3l of libgrace/include/
+ * grace/system.h:95-103); tables of the three layers that together exceed 2048 MB (Grace3LKK::spline_mb, libgrace/
+ * include/grace/kk/grace_3l_kk.h:1264) are not built: the engine says so through the logger and keeps evaluating its
+ * radial MLPs.  gr_engine_spline: the value set. */
 int gr_engine_set_spline(gr_engine *e, int intervals);
 int gr_engine_spline(const gr_engine *e);
 int gr_system_rebuilds(const gr_system *s);
