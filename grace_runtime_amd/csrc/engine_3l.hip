@@ -672,12 +672,14 @@ template<class T> void Engine3L<T>::couple_bwd(ProdStage<T> &p, const T *Lp, int
   hipLaunchKernelGGL(k_prod_bwd<T>, dim3(p.cp.d.nright * 8 * (((n + AT - 1) / AT + 7) / 8)), dim3(KP * AT), 0, stream_, p.cp.d, 1, Lp, g, gR, n, KP, nfl, nfr);
 }
 
-// Slots (message functions) of one block of the pair kernels: blocks of at most 1024 threads; when spreading the slots
-// evenly over the same number of groups saves whole rounds of waves on the four SIMDs (36 slots of 64 channels: 3 x 12
-// instead of 16 + 16 + 4), the even split, else the full blocks (72 slots: 4 x 16 + 8 ran faster than 5 x 15).
-static int slots_per_block(int nslot, int CP)
+// Slots (message functions) of one block of the pair kernels, in blocks of at most max_threads threads; when spreading the
+// slots evenly over the same number of groups saves whole rounds of waves on the four SIMDs (36 slots of 64 channels: 3 x 12
+// instead of 16 + 16 + 4), the even split, else the full blocks (72 slots: 4 x 16 + 8 ran faster than 5 x 15).  The forward
+// kernel runs in blocks of 512 threads (config 4, layers 2 / 3: 6.3 / 11.3 ms against 7.2 / 13.2 with 1024; fp32 3.8 / 6.8
+// against 3.6 / 9.9; 256 threads 6.0 / 11.7), the vector reverse kernels in blocks of 1024.
+static int slots_per_block(int nslot, int CP, int max_threads)
 {
-  const int smax = std::max(1, std::min(nslot, 1024 / CP)), ngrp = (nslot + smax - 1) / smax, even = (nslot + ngrp - 1) / ngrp;
+  const int smax = std::max(1, std::min(nslot, max_threads / CP)), ngrp = (nslot + smax - 1) / smax, even = (nslot + ngrp - 1) / ngrp;
   auto rounds = [&](int spb) { return (spb * CP / 64 + 3) / 4; };
   return rounds(even) < rounds(smax) ? even : smax;
 }
@@ -779,7 +781,7 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw, bo
     const int npf = L.nlmi * nlm_;
     pairP_.ensure(na * npf * L.CP * s);
     A_.ensure(na * L.nfA * L.CP * s);
-    const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb;
+    const int spb = slots_per_block(L.nlmi, L.CP, 512), ngrp = (L.nlmi + spb - 1) / spb;
     stage(tg(k, "pair_fwd").c_str(), [&] {
       const int pt = round_up(spb * L.CP, 64);
       // rows of CP values and of noutp values go to LDS 16 bytes at a time
@@ -986,7 +988,7 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
                        L.cgt.off.template as<int>(), L.cgt.idx.template as<int>(), L.cgt.rowof.template as<int>(), L.cgt.val.template as<double>(),
                        (const T *) gA_.as<T>(), gpairP_.as<T>(), L.nfA, npf, L.CP, n, L.cgt.rows, ngrp);
   });
-  const int spb = slots_per_block(L.nlmi, L.CP), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
+  const int spb = slots_per_block(L.nlmi, L.CP, 1024), ngrp = (L.nlmi + spb - 1) / spb, pthreads = round_up(spb * L.CP, 64);
   stage(tg(k, "pair_bwd").c_str(), [&] {
     // fp32: the next chunk is copied to a second LDS buffer while this one is worked on (chunks of 8 bonds in the large
     // blocks that fill a CU alone, of 4 otherwise); fp64 runs faster with one chunk staged through registers

@@ -388,6 +388,7 @@ __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__rest
     block_copy_async(R1 + base * noutp, Rsh + (size_t) buf * CH * noutp, nb * noutp * (int) sizeof(T), wave, nw, lane);
   };
   T touch = (T) 0;
+  const bool works = __ballot(active) != 0;      // a wave without a slot (the last group of an atom) only copies
   // round c stages chunk c + 1 and works on chunk c (round -1 only stages)
   for (int c = -1; c < nchunk; c++) {
     const long long base = e0 + (long long) c * CH;
@@ -399,7 +400,7 @@ __global__ void k_pair_fwd(const long long *__restrict__ eoff, const int *__rest
       const int nnb = (int) (e1 - nbase < CH ? e1 - nbase : CH), per = (nlm + 7) / 8;
       if (t < nnb * per) tv = Y[(nbase + t / per) * ystride + (t % per) * 8];
     }
-    for (int b = 0; b < nb; b++) {
+    for (int b = 0; b < (works ? nb : 0); b++) {
       const T m = Msh[(size_t) (buf * CH + b) * NT + t];
       const T *r = Rsh + (size_t) (buf * CH + b) * noutp + n;
       const T *y = Y + (base + b) * ystride;
