@@ -493,7 +493,7 @@ template<class T> void Engine1L<T>::run_chunk(const RunFlags &fl, int a0, int nc
     }
   }
   stage("reduce_rho", [&] {
-#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(ntiles), dim3(256), 0, stream_, redrho_.d, mu, tiles, \
+#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(ntiles), dim3(64 * kReduceWaves), 0, stream_, redrho_.d, mu, tiles, \
                                           (const T *) A, (const T *) AA, (const T *) AAA, (const T *) AAAA, rho_.as<double>())
     switch (ka * 10 + kf) {
       case 11: GR_RED(1, 1); break; case 12: GR_RED(1, 2); break; case 14: GR_RED(1, 4); break;

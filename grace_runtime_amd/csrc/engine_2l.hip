@@ -585,7 +585,7 @@ template<class T> void Engine2L<T>::chain_backward(Chain<T> &c, const char *tag,
 template<class T> void Engine2L<T>::reduce_fwd(DevReduce<T> &R, int kb, const Chain<T> &c, const T *X, double *out)
 {
   const int *tiles = cur_tiles_;
-#define GR_RED(KA) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KA>), dim3(cur_ntiles_), dim3(256), 0, stream_, R.d, mu_.as<int>() + a0_, tiles, \
+#define GR_RED(KA) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KA>), dim3(cur_ntiles_), dim3(64 * kReduceWaves), 0, stream_, R.d, mu_.as<int>() + a0_, tiles, \
                                       c.src(0, X), c.src(1, X), c.src(2, X), c.src(3, X), out)
   switch (kb) {
     case 1: GR_RED(1); break;

@@ -852,7 +852,7 @@ template<class T> void Engine3L<T>::layer_forward(int k, bool forces, int yw, bo
   if (again) return;    // the densities, the energy and the UQ rows come from the first forward pass
   stage(tg(k, "reduce_rho").c_str(), [&] {
     const int *tiles = cur_tiles_;
-#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(cur_ntiles_), dim3(256), 0, stream_, L.rho.d, mu, tiles, srcs[0], srcs[1], \
+#define GR_RED(KA, KF) hipLaunchKernelGGL((k_reduce_fwd<T, KA, KF>), dim3(cur_ntiles_), dim3(64 * kReduceWaves), 0, stream_, L.rho.d, mu, tiles, srcs[0], srcs[1], \
                                           srcs[2], srcs[3], L.rho_raw.template as<double>() + (size_t) a0_ * nrho_)
     switch ((wX / 16) * 10 + wR / 16) {
       case 11: GR_RED(1, 1); break;

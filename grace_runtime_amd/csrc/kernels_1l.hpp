@@ -1197,14 +1197,15 @@ template<class T> struct ReduceDev {
 };
 
 // rho[atom][k] = sum_s sum_c sum_n W_s[mu][c][n][k] X_s[atom][fn c][n] on the matrix cores: one block per tile of
-// 16 atoms, its 4 waves split the (s, c) list, partial tiles summed through LDS.  KBA / KBF: 16-channel blocks of
+// 16 atoms, its kReduceWaves waves split the (s, c) list, partial tiles summed through LDS.  KBA / KBF: 16-channel blocks of
 // source 0 (A) and of the other sources.
+constexpr int kReduceWaves = 8;    // waves of a k_reduce_fwd block: each takes every eighth collected function
 template<class T, int KBA, int KBF>
-__global__ __launch_bounds__(256) void k_reduce_fwd(ReduceDev<T> R, const int *mu, const int *tile_atoms, const T *X0, const T *X1,
+__global__ __launch_bounds__(64 * kReduceWaves) void k_reduce_fwd(ReduceDev<T> R, const int *mu, const int *tile_atoms, const T *X0, const T *X1,
                                                     const T *X2, const T *X3, double *rho)
 {
   typedef typename Mfma<T>::v4 v4;
-  __shared__ double part[4][2][16][17];
+  __shared__ double part[kReduceWaves][2][16][17];
   const int tile = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, g = lane >> 4;
@@ -1217,7 +1218,7 @@ __global__ __launch_bounds__(256) void k_reduce_fwd(ReduceDev<T> R, const int *m
   for (int s = 0; s < R.nsrc; s++) {
     const int ks = (s == 0 ? KBA : KBF) * 4, K = ks * 4;
     for (int cc = 0; cc < R.ncol[s]; cc++, job++) {
-      if ((job & 3) != wave) continue;
+      if (job % kReduceWaves != wave) continue;
       const T *wf = R.WF[s] + ((long long) m * R.ncol[s] + cc) * R.nbr * ks * 64 + lane;
       T x[(KBA > KBF ? KBA : KBF) * 4];
       if (arow >= 0) {
@@ -1242,12 +1243,12 @@ __global__ __launch_bounds__(256) void k_reduce_fwd(ReduceDev<T> R, const int *m
 #pragma unroll
     for (int v = 0; v < 4; v++) part[wave][cb][R.drow[4 * g + v]][c] = (double) acc[cb][v];
   __syncthreads();
-  for (int e = threadIdx.x; e < 16 * R.nrho; e += 256) {
+  for (int e = threadIdx.x; e < 16 * R.nrho; e += 64 * kReduceWaves) {
     const int r = e / R.nrho, k = e % R.nrho;
     const int at = tile_atoms[tile * 16 + r];
     if (at < 0) continue;
     double v = 0.0;
-    for (int w = 0; w < 4; w++) v += part[w][k >> 4][r][k & 15];
+    for (int w = 0; w < kReduceWaves; w++) v += part[w][k >> 4][r][k & 15];
     rho[(long long) at * R.ostride + R.ooff + k] = v;
   }
 }
