@@ -5,11 +5,12 @@
 //   k_pair_fwd     P[slot][lm][n] = sum_b Y_lm(b) R1_l(b)[n] M_jb[slot][n]: the neighbour gather of the messages
 //                  (slots 0 .. nI-1: the equivariant message I_j; slot nI: zB0, which gives B0)
 //                  (atom_yi / atom_scatter, libgrace/include/grace/fused_cpu.h:947-1025)
-//   k_pair_bwd[_async]  its reverse: per-bond force of layer 2, dE/dI_j added to the neighbour's row
-//                  (bond_yi_bwd_g, bond_yi_commit, bond_scatter_bwd_t, bond_force: fused_cpu.h:836-942,1027-1050)
+//   k_pair_bwd_mfma, k_pair_bwd[_async]  its reverse: per-bond force of layer 2, dE/dI_j added to the neighbour's row
+//                  (bond_yi_bwd_g, bond_yi_commit, bond_scatter_bwd_t, bond_force: fused_cpu.h:836-942,1027-1050); the first
+//                  forms the sums over m on the matrix cores, the others on the vector unit
 //   k_energy_2l    readout with the two RMSNorms, fp64 (libgrace/src/fused_2l.cpp:548-615)
 //
-// The gather kernels run one block per atom with one thread per (slot, channel): a thread keeps its 2l+1 .. nlm
+// The vector gather kernels run one block per atom with one thread per (slot, channel): a thread keeps its 2l+1 .. nlm
 // accumulators (or adjoints) in registers and walks the atom's bonds; everything that is the same for the whole block
 // (neighbour index, Y, G of the bond) is read through uniform addresses.
 #pragma once
