@@ -862,8 +862,8 @@ template<class T> void Engine2L<T>::run(const RunFlags &fl)
       if (ordered_) {
         po.gMe = gMe_.as<T>(); po.fedge = fedge_.as<double>(); po.fcen = fcen_.as<double>(); po.e_base = eb; po.ngrp = 1;
       }
-      const PairMfmaPlan mp = pair_mfma_plan(nslot_, CRP_, nl_, sizeof(T), pair_waves_);
-      if (!ordered_ && mp.ok && (pair_mfma_ > 0 || (pair_mfma_ < 0 && pair_mfma_pays(nslot_, CRP_, sizeof(T))))) {
+      const PairMfmaPlan mp = pair_mfma_plan(nslot_, CRP_, nl_, sizeof(T), pair_mfma_waves(sizeof(T), pair_waves_));
+      if (!ordered_ && mp.ok && pair_mfma_ != 0) {
         PairMfmaArgs<T> pa{};
         pa.eoff = eoff; pa.ej = ej_.as<int>(); pa.YG = YG_.as<T>(); pa.R1 = R1; pa.dR1 = dR1; pa.M = M; pa.gP = gP_.as<T>();
         pa.rh = rh_.as<double>(); pa.rlen = r_.as<double>(); pa.rcut = rc_.as<double>();

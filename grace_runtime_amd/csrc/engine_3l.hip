@@ -1008,8 +1008,8 @@ template<class T> void Engine3L<T>::layer_backward(int k, int yw)
   dim3((unsigned) ((n + 7) / 8 * 8 * ngrp)), dim3(pthreads), lds, stream_, eoff, ej_.as<int>(), YG_.as<T>(), (const T *) Rl, (const T *) dRl,     \
       (const T *) M_.as<T>(), (const T *) gpairP_.as<T>(), rh_.as<double>(), r_.as<double>(), rc_.as<double>(), gM_.as<T>(), f_.as<double>(),   \
       scal_.as<double>() + 1, L.nlmi, L.nlmi, L.CP, nl_, L.rad.noutp, sink_.as<T>(), 1, sid_ptr(), spb, ngrp, n, a0_, vatom_ptr(), yw
-    const PairMfmaPlan mp = pair_mfma_plan(L.nlmi, L.CP, nl_, s, pair_waves_);
-    if (!ordered_ && mp.ok && (pair_mfma_ > 0 || (pair_mfma_ < 0 && pair_mfma_pays(L.nlmi, L.CP, s)))) {
+    const PairMfmaPlan mp = pair_mfma_plan(L.nlmi, L.CP, nl_, s, pair_mfma_waves(s, pair_waves_));
+    if (!ordered_ && mp.ok && pair_mfma_ != 0) {
       PairMfmaArgs<T> pa{};
       pa.eoff = eoff; pa.ej = ej_.as<int>(); pa.YG = YG_.as<T>(); pa.R1 = Rl; pa.dR1 = dRl; pa.M = M_.as<T>(); pa.gP = gpairP_.as<T>();
       pa.rh = rh_.as<double>(); pa.rlen = r_.as<double>(); pa.rcut = rc_.as<double>();

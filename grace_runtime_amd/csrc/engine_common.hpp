@@ -1604,20 +1604,19 @@ class EngineBase : public Engine, protected BufRegistry {
   double cur_flops_ = 0.0;
   size_t ev_used_ = 0;
   std::vector<StageTime> times_;
-  // the reverse pair kernel on the matrix cores: -1 where it is the faster one (pair_mfma_pays), GRACE_HIP_PAIR_MFMA=0 never
-  // (the vector kernels), =1 wherever it applies
+  // the reverse pair kernel on the matrix cores wherever it applies; GRACE_HIP_PAIR_MFMA=0: the vector kernels
   int pair_mfma_ = pair_mfma_switch();
   static int pair_mfma_switch()
   {
     const char *e = std::getenv("GRACE_HIP_PAIR_MFMA");
-    return !e ? -1 : e[0] == '0' ? 0 : 1;
+    return e && e[0] == '0' ? 0 : 1;
   }
-  int pair_waves_ = pair_waves_switch();    // waves of a block of that kernel
+  int pair_waves_ = pair_waves_switch();    // waves of a block of that kernel; 0: 8 in fp64, 4 in fp32 (pair_mfma_waves)
   static int pair_waves_switch()
   {
     const char *e = std::getenv("GRACE_HIP_PAIR_WAVES");
-    const int w = e ? std::atoi(e) : 8;
-    return w >= 1 && w <= 8 ? w : 8;
+    const int w = e ? std::atoi(e) : 0;
+    return w >= 1 && w <= 8 ? w : 0;
   }
   int drow_[16];
   int drow64_[16];    // fp32 engines: the accumulator rows of the fp64 MFMA (the fp64 radial MLP that fills the radial tables)

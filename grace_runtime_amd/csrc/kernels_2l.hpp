@@ -610,7 +610,7 @@ __device__ inline void lds_load_piece(const void *src, void *lds_wave_base)
 }
 
 template<class T, int NL, int TPW>
-__global__ __launch_bounds__(512) void k_pair_bwd_mfma(PairMfmaArgs<T> a)
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(sizeof(T) == 4 ? 3 : 2))) void k_pair_bwd_mfma(PairMfmaArgs<T> a)
 {
   typedef typename Mfma<T>::v4 v4;
   constexpr int NLM = NL * NL, STEPS = pair_mfma_step0(NL), VPP = 16 / (int) sizeof(T);    // VPP: values per 16-byte piece
@@ -875,9 +875,11 @@ inline PairMfmaPlan pair_mfma_plan(int nslot, int C, int nl, size_t value_bytes,
   return p;
 }
 // Where the matrix-core kernel is the faster one of the reverse pair kernels (measured, fp64 / fp32, vector kernel ->
-// this one): 72 slots x 64 channels 43.6 -> 37.2 ms / 31.8 -> 25.7 ms; 36 x 64: 24.5 -> 18.9 / 16.6 -> 13.0; 5 x 32:
-// 6.9 -> 5.3 / 4.0 -> 4.3.  fp32 with few columns per atom stays with the vector kernel that copies asynchronously.
-inline bool pair_mfma_pays(int nslot, int C, size_t value_bytes) { return value_bytes == 8 || nslot * C >= 1024; }
+// this one): 72 slots x 64 channels 43.6 -> 37.2 ms / 31.8 -> 24.8 ms; 36 x 64: 24.5 -> 18.9 / 16.6 -> 12.4; 5 x 32:
+// 6.9 -> 5.3 / 4.0 -> 3.4: everywhere it applies.  Waves of a block: 8 in fp64 (250 registers: two waves per SIMD, one
+// block per CU; blocks of 4 were 5 % slower), 4 in fp32, where the kernel is compiled for three waves per SIMD (168
+// registers, 8 of them spilled) and three blocks share a CU (blocks of 8: 27.2 / 13.8 / 4.3 ms).
+inline int pair_mfma_waves(size_t value_bytes, int asked) { return asked > 0 ? asked : value_bytes == 4 ? 4 : 8; }
 
 template<class T> inline void launch_pair_bwd_mfma(const PairMfmaPlan &p, PairMfmaArgs<T> a, int nl, hipStream_t stream)
 {
