@@ -153,10 +153,13 @@ def main():
                                "stages_ms": r["stages_ms"], "engine_create_s": r["engine_create_s"], "device_memory_GB": r["device_memory_GB"],
                                "cpu_baseline": r["cpu_baseline"]}
         res["other_workloads"] = others
+        # us/atom of the calculator-level call from 128 to 65 536 atoms (GRACE-1L; --workload sizes goes on to millions)
+        res["size_range"] = [{k: e[k] for k in ("structure", "atoms", "edges", "ms_per_call_list_kept", "us_per_atom", "device_memory_GB")}
+                             for e in run_sizes(a, short=True)["entries"]]
     print(json.dumps(res))
 
 
-def run_sizes(a):
+def run_sizes(a, short=False):
     """The calculator-level call (kk.System.compute: positions in, device neighbour list kept between calls, results out; the
     reference's protocol, docs/benchmarks.md:9-20) over a range of structure sizes: the GRACE-1L model from 128 atoms to a
     bcc 128^3 supercell, and one structure per model kind well past the benchmark size, evaluated in the chunks the engine
@@ -195,10 +198,12 @@ def run_sizes(a):
         del sysm
 
     m1 = kk.Model(workloads.write_model("config1", tmp))
-    for reps in (4, 8, 10, 16, 32, 64, 128):
+    for reps in ((4, 8, 10, 16, 32) if short else (4, 8, 10, 16, 32, 64, 128)):
         pos, cell = synth.bcc_supercell(3.165, reps)
         pos = synth.jitter(pos, 0.05, 2)
         measure(f"GRACE-1L, bcc W {reps}^3", m1, ["W"], np.ones(len(pos), np.int32), pos, cell, 5 if reps <= 32 else 3)
+    if short:    # the default run: the GRACE-1L sizes from 128 to 65 536 atoms only
+        return {"workload": "size range, calculator-level call with the neighbour list kept", "dtype": "f64" if a.precision == 64 else "f32", "entries": out}
     m2 = kk.Model(workloads.write_model("config3", tmp))
     pos, cell = synth.fcc_supercell(3.6, 63)
     pos = synth.jitter(pos, 0.08, 3)
