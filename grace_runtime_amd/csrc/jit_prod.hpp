@@ -15,6 +15,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <cstring>
 #include <sys/stat.h>
 #include <unistd.h>
 
@@ -415,6 +416,32 @@ inline std::string cache_file(const std::string &key)
   std::snprintf(name, sizeof name, "%016llx%016llx_%zu.co", h1, h2, full.size());
   return dir + "/" + name;
 }
+// A cache file is the code object followed by 24 bytes: a tag, the length of the code object and an FNV-1a digest of its
+// bytes.  A file without them (cut short, damaged, of another layout) is not handed to the driver.
+constexpr unsigned long long kCacheTag = 0x4f43504948524721ULL;
+inline unsigned long long bytes_digest(const char *p, size_t n)
+{
+  unsigned long long h = 1469598103934665603ULL;
+  for (size_t q = 0; q < n; q++) h = (h ^ (unsigned char) p[q]) * 1099511628211ULL;
+  return h;
+}
+inline void seal(std::vector<char> &data)
+{
+  const unsigned long long t[3] = {kCacheTag, (unsigned long long) data.size(), bytes_digest(data.data(), data.size())};
+  const char *b = reinterpret_cast<const char *>(t);
+  data.insert(data.end(), b, b + sizeof t);
+}
+// true and the trailer removed when `data` is a whole sealed file
+inline bool unseal(std::vector<char> &data)
+{
+  unsigned long long t[3];
+  if (data.size() < sizeof t + 64) return false;
+  std::memcpy(t, data.data() + data.size() - sizeof t, sizeof t);
+  const size_t n = data.size() - sizeof t;
+  if (t[0] != kCacheTag || t[1] != n || t[2] != bytes_digest(data.data(), n)) return false;
+  data.resize(n);
+  return true;
+}
 inline bool read_file(const std::string &path, std::vector<char> &out)
 {
   FILE *f = std::fopen(path.c_str(), "rb");
@@ -475,6 +502,7 @@ inline bool jit_compile_source(const char *name, const std::string &src, bool f3
   static std::mutex cache_mu;
   static std::map<std::string, std::shared_ptr<const std::vector<char>>> cache;
   const std::string key = arch + (in_order ? "\nin order\n" : "\n") + src;
+  out.release();
   std::shared_ptr<const std::vector<char>> obj;
   {
     std::lock_guard<std::mutex> lk(cache_mu);
@@ -486,12 +514,28 @@ inline bool jit_compile_source(const char *name, const std::string &src, bool f3
   // loads a model finds its kernels on disk.  GRACE_HIP_CACHE=<dir> names the directory (default ~/.cache/grace_hip),
   // GRACE_HIP_CACHE=0 switches the disk cache off.
   const std::string disk = jit_detail::cache_file(key);
+  bool from_disk = false;
   if (!obj && !disk.empty()) {
     std::vector<char> code;
-    if (jit_detail::read_file(disk, code) && code.size() > 64) {
-      obj = std::make_shared<const std::vector<char>>(std::move(code));
+    if (jit_detail::read_file(disk, code)) {
+      if (jit_detail::unseal(code)) {
+        obj = std::make_shared<const std::vector<char>>(std::move(code));
+        from_disk = true;
+      } else {
+        (void) std::remove(disk.c_str());    // cut short or damaged: compiled again below and written anew
+      }
+    }
+  }
+  // a whole file that the driver does not load (written for another driver) is dropped as well and the source compiled
+  if (from_disk) {
+    if (hipModuleLoadData(&out.mod, obj->data()) == hipSuccess) {
       std::lock_guard<std::mutex> lk(cache_mu);
       cache[key] = obj;
+    } else {
+      (void) hipGetLastError();
+      out.mod = nullptr;
+      obj.reset();
+      (void) std::remove(disk.c_str());
     }
   }
   if (!obj) {
@@ -520,11 +564,15 @@ inline bool jit_compile_source(const char *name, const std::string &src, bool f3
     hiprtcGetCode(prog, code.data());
     hiprtcDestroyProgram(&prog);
     obj = std::make_shared<const std::vector<char>>(std::move(code));
-    if (!disk.empty()) jit_detail::write_file_atomically(disk, *obj);
+    if (!disk.empty()) {
+      std::vector<char> sealed(*obj);
+      jit_detail::seal(sealed);
+      jit_detail::write_file_atomically(disk, sealed);
+    }
     std::lock_guard<std::mutex> lk(cache_mu);
     cache[key] = obj;
   }
-  if (hipModuleLoadData(&out.mod, obj->data()) != hipSuccess) {
+  if (!out.mod && hipModuleLoadData(&out.mod, obj->data()) != hipSuccess) {
     (void) hipGetLastError();
     out.mod = nullptr;
     why = "hipModuleLoadData failed";

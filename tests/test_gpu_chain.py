@@ -127,6 +127,16 @@ def test_compiled_kernels_are_kept_on_disk_for_the_next_process(model_dir, tmp_p
     assert float(runs[1][0]) < 0.5 * float(runs[0][0])
     assert abs(float(runs[0][1]) - float(runs[1][1])) < 1e-9 * abs(float(runs[0][1]))
     assert abs(float(runs[0][2]) - float(runs[1][2])) < 1e-9 * abs(float(runs[0][2]))
+    # a file that the driver does not load (cut short here) is dropped, its source compiled again and the file replaced
+    sizes = {f: os.path.getsize(tmp_path / "cache" / f) for f in files}
+    for f in files:
+        with open(tmp_path / "cache" / f, "r+b") as fh:
+            fh.truncate(200)
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
+    assert res.returncode == 0, res.stderr
+    third = res.stdout.strip().split("\n")[-1].split()
+    assert abs(float(third[1]) - float(runs[0][1])) < 1e-9 * abs(float(runs[0][1]))
+    assert {f: os.path.getsize(tmp_path / "cache" / f) for f in os.listdir(tmp_path / "cache")} == sizes
     # switched off: nothing is written
     env0 = dict(os.environ, GRACE_HIP_CACHE="0", HOME=str(tmp_path / "home"))
     res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env0, timeout=300)
