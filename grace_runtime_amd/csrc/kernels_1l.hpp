@@ -1696,8 +1696,11 @@ template<class T, int KB, int NL, bool TAB> __global__ __launch_bounds__(256) vo
     const long long eb = e0 + (long long) tile * 16;
     const int nb = (int) (e1 - eb < 16 ? e1 - eb : 16);
     const bool colok = c < nb;                      // B operand column = bond c of the tile
-    const T *rp = a.Rz + (eb + (colok ? c : 0)) * a.noutp + g * KS;
-    const T *dp = a.dRz + (eb + (colok ? c : 0)) * a.noutp + g * KS;
+    // rows read by this lane: without tables step s of lane group g is channel 8 (s / 2) + 2 g + s % 2 (CH), so that the
+    // four lane groups read 64 consecutive bytes of a bond's row in one instruction; with tables channel g KS + s
+    const T *rp = a.Rz + (eb + (colok ? c : 0)) * a.noutp + (TAB ? g * KS : 2 * g);
+    const T *dp = a.dRz + (eb + (colok ? c : 0)) * a.noutp + (TAB ? g * KS : 2 * g);
+#define CH(s_) (TAB ? (s_) : 8 * ((s_) >> 1) + ((s_) & 1))
     T x[2][KS], dx[2][KS];
     // tables: interval, offset and species weights of bond c, and the entries of l = 0
     // (four columns at a time: the entries of the next four are requested before the products of these four)
@@ -1715,7 +1718,7 @@ template<class T, int KB, int NL, bool TAB> __global__ __launch_bounds__(256) vo
       for (int s = 0; s < KS; s++) zc[s] = a.tb.z[mu * C + g * KS + s];
     } else {
 #pragma unroll
-      for (int s = 0; s < KS; s++) { x[0][s] = rp[s]; dx[0][s] = dp[s]; }
+      for (int s = 0; s < KS; s++) { x[0][s] = rp[CH(s)]; dx[0][s] = dp[CH(s)]; }
     }
     // geometry of bond `lane` (lanes below nb), kept for the end of the tile
     double u0 = 0, u1 = 0, u2 = 1, br = 1, brc = 1;
@@ -1744,12 +1747,12 @@ template<class T, int KB, int NL, bool TAB> __global__ __launch_bounds__(256) vo
       if constexpr (!TAB) {
         if (l + 1 < NL) {
 #pragma unroll
-          for (int s = 0; s < KS; s++) { x[nxt][s] = rp[(l + 1) * C + s]; dx[nxt][s] = dp[(l + 1) * C + s]; }
+          for (int s = 0; s < KS; s++) { x[nxt][s] = rp[(l + 1) * C + CH(s)]; dx[nxt][s] = dp[(l + 1) * C + CH(s)]; }
         }
       }
       v4 aP = {0, 0, 0, 0}, aQ = {0, 0, 0, 0};
       // A operand: row m = c of gA_l^T, k = g KS + s
-      const T *ga = gAl + (l * l + (c < 2 * l + 1 ? c : 0)) * CS + g * KS;
+      const T *ga = gAl + (l * l + (c < 2 * l + 1 ? c : 0)) * CS + (TAB ? g * KS : 2 * g);
       if constexpr (TAB) {
 #pragma unroll
         for (int hb = 0; hb < KS; hb += KH) {
@@ -1779,7 +1782,7 @@ template<class T, int KB, int NL, bool TAB> __global__ __launch_bounds__(256) vo
       } else {
 #pragma unroll
         for (int s = 0; s < KS; s++) {
-          const T w = c < 2 * l + 1 ? ga[s] : (T) 0;
+          const T w = c < 2 * l + 1 ? ga[CH(s)] : (T) 0;
           aP = Mfma<T>::mma(w, x[cur][s], aP);
           aQ = Mfma<T>::mma(w, dx[cur][s], aQ);
         }
@@ -1844,6 +1847,7 @@ template<class T, int KB, int NL, bool TAB> __global__ __launch_bounds__(256) vo
     }
   }
 }
+#undef CH
 
 // ---------------------------------------------------------------------------------------------------------------
 // ordered (atomic-free) sums of the forces, the virial and the energy: same bits on every run
